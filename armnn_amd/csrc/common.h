@@ -1,0 +1,56 @@
+// Internal helpers shared by the device library's translation units (not part of the C ABI).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include <cstdarg>
+#include <cstdint>
+#include <cstdio>
+#include <cstring>
+
+#include "armnn_mi355x.h"
+
+namespace mi355x
+{
+
+// thread-local message behind mi355x_last_error()
+char* ErrorBuffer();
+int SetError(int code, const char* fmt, ...);
+
+inline int HipFail(hipError_t e, const char* what)
+{
+    return SetError(static_cast<int>(e), "%s: %s", what, hipGetErrorString(e));
+}
+
+#define MI355X_HIP(expr)                                             \
+    do {                                                             \
+        hipError_t e_ = (expr);                                      \
+        if (e_ != hipSuccess) return ::mi355x::HipFail(e_, #expr);   \
+    } while (0)
+
+inline hipStream_t ToHip(mi355x_stream_t s) { return reinterpret_cast<hipStream_t>(s); }
+
+inline bool IsActivationDtype(int32_t d) { return d == MI355X_QASYMM_S8 || d == MI355X_QASYMM_U8; }
+
+// armnn::Quantize (src/armnn/TypesUtils.cpp:29-45) on the host, used to turn activation bounds into codes
+int32_t QuantizeHost(float value, float scale, int32_t offset, int32_t dtype);
+
+// Integer clamp equivalent to an Activation layer that follows a layer with the same output quantization:
+// q2 = clamp(q1, Quantize(b), Quantize(a)) for BoundedReLu, clamp(q1, Quantize(0), type max) for ReLu.
+void ActivationClamp(int32_t activation, float a, float b, const mi355x_quant& out, int32_t* lo, int32_t* hi);
+
+// Parameters of the shared requantization epilogue
+struct Requant
+{
+    float   out_scale;
+    float   out_offset_f;   // float(offset)
+    float   type_min_f;     // float(lowest) of the output type
+    float   type_max_f;
+    int32_t act_lo;         // fused activation clamp in the quantized domain (already within the type range)
+    int32_t act_hi;
+    int32_t out_is_u8;
+};
+
+Requant MakeRequant(const mi355x_quant& out, int32_t activation, float a, float b);
+
+} // namespace mi355x

@@ -1,0 +1,375 @@
+// Convolution2d / DepthwiseConvolution2d / FullyConnected entry points of the C ABI: plan creation
+// (constant re-layout, per-channel requantization constants, kernel selection) and launches.
+#include "common.h"
+#include "conv_kernels.h"
+
+#include <cmath>
+#include <cstdlib>
+#include <string>
+#include <vector>
+
+using namespace mi355x;
+
+struct mi355x_conv2d_s
+{
+    mi355x_conv2d_desc d{};
+    int32_t algo = MI355X_ALGO_DIRECT;
+    ConvGeom geom{};
+    Requant rq{};
+    // device constants
+    uint8_t* w_direct = nullptr;   // [Kh][Kw][Ci][Co] / depthwise [Kh][Kw][Co], raw codes
+    int8_t*  w_mfma   = nullptr;   // [Co_pad][K_pad] signed, zero padded
+    float*   mult     = nullptr;   // [Co_pad]  s_in * s_w[c]
+    float*   biasf    = nullptr;   // [Co_pad]  float(bias[c]) * s_b[c]
+    int32_t* corr     = nullptr;   // [Co_pad]  -zx' * sum_k w[c][k]
+    int K = 0, K_pad = 0, Co_pad = 0;
+    int bm = 0, bn = 0;
+    uint32_t xor_mask = 0, pad_word = 0;
+    std::string info;
+
+    ~mi355x_conv2d_s()
+    {
+        (void)hipFree(w_direct);
+        (void)hipFree(w_mfma);
+        (void)hipFree(mult);
+        (void)hipFree(biasf);
+        (void)hipFree(corr);
+    }
+};
+
+struct mi355x_fc_s
+{
+    mi355x_conv2d_s* conv = nullptr;
+    ~mi355x_fc_s() { delete conv; }
+};
+
+namespace
+{
+
+int Upload(void** dst, const void* src, size_t bytes)
+{
+    MI355X_HIP(hipMalloc(dst, bytes));
+    MI355X_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
+    return 0;
+}
+
+int ValidateQuant(const mi355x_quant& q, const char* what)
+{
+    if (!IsActivationDtype(q.dtype)) return SetError(MI355X_ERR_UNSUPPORTED, "%s: data type %d is not QAsymmS8/QAsymmU8", what, q.dtype);
+    if (!(q.scale > 0.0f) || !std::isfinite(q.scale)) return SetError(MI355X_ERR_INVALID_ARGUMENT, "%s: scale must be positive and finite", what);
+    return 0;
+}
+
+// `weights` in the reference layout: conv [Co][Kh][Kw][Ci]; depthwise [1][Kh][Kw][Co].
+int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355x_const_quant* wq,
+              const int32_t* bias_host, const mi355x_const_quant* bq, mi355x_conv2d_s* p)
+{
+    if (!weights_host || !wq) return SetError(MI355X_ERR_INVALID_ARGUMENT, "weights / weight quantization missing");
+    if (d.in_h == 0 || d.in_w == 0 || d.in_c == 0 || d.out_h == 0 || d.out_w == 0 || d.out_c == 0 || d.kernel_h == 0 ||
+        d.kernel_w == 0 || d.stride_x == 0 || d.stride_y == 0 || d.dilation_x == 0 || d.dilation_y == 0)
+        return SetError(MI355X_ERR_INVALID_ARGUMENT, "zero extent / stride / dilation in convolution descriptor");
+    if (int rc = ValidateQuant(d.input, "input")) return rc;
+    if (int rc = ValidateQuant(d.output, "output")) return rc;
+    if (wq->dtype != MI355X_QSYMM_S8 && wq->dtype != MI355X_QASYMM_S8 && wq->dtype != MI355X_QASYMM_U8)
+        return SetError(MI355X_ERR_UNSUPPORTED, "weights data type %d is not an 8-bit quantized type", wq->dtype);
+    if (wq->n_scales != 1 && wq->n_scales != d.out_c)
+        return SetError(MI355X_ERR_INVALID_ARGUMENT, "weights carry %u scales; expected 1 or %u", wq->n_scales, d.out_c);
+    if (!wq->scales) return SetError(MI355X_ERR_INVALID_ARGUMENT, "weight scales missing");
+    if (wq->n_scales > 1 && wq->offset != 0)
+        return SetError(MI355X_ERR_INVALID_ARGUMENT, "per-axis weights must have offset 0");
+    if (d.bias_enabled)
+    {
+        if (!bias_host || !bq || !bq->scales) return SetError(MI355X_ERR_INVALID_ARGUMENT, "bias enabled but bias data / quantization missing");
+        if (bq->dtype != MI355X_SIGNED32) return SetError(MI355X_ERR_UNSUPPORTED, "bias must be Signed32");
+        if (bq->n_scales != 1 && bq->n_scales != d.out_c)
+            return SetError(MI355X_ERR_INVALID_ARGUMENT, "bias carries %u scales; expected 1 or %u", bq->n_scales, d.out_c);
+        if (bq->offset != 0) return SetError(MI355X_ERR_INVALID_ARGUMENT, "bias offset must be 0");
+    }
+    if (d.depthwise && (d.out_c % d.in_c) != 0)
+        return SetError(MI355X_ERR_INVALID_ARGUMENT, "depthwise: out_c %u is not a multiple of in_c %u", d.out_c, d.in_c);
+    if (d.activation < MI355X_ACT_NONE || d.activation > MI355X_ACT_BOUNDED_RELU)
+        return SetError(MI355X_ERR_UNSUPPORTED, "activation %d cannot be fused", d.activation);
+    // the output extent must be consistent with the window walk (bottom/right padding is implied, never negative reach)
+    {
+        const long long need_h = static_cast<long long>(d.out_h - 1) * d.stride_y + static_cast<long long>(d.kernel_h - 1) * d.dilation_y;
+        const long long need_w = static_cast<long long>(d.out_w - 1) * d.stride_x + static_cast<long long>(d.kernel_w - 1) * d.dilation_x;
+        if (need_h > 2ll * 1000000 || need_w > 2ll * 1000000) return SetError(MI355X_ERR_INVALID_ARGUMENT, "unreasonable geometry");
+    }
+
+    p->d = d;
+    const int Co = static_cast<int>(d.out_c), Ci = static_cast<int>(d.in_c);
+    const int Kh = static_cast<int>(d.kernel_h), Kw = static_cast<int>(d.kernel_w);
+    ConvGeom& g = p->geom;
+    g.H = d.in_h; g.W = d.in_w; g.Ci = Ci; g.Ho = d.out_h; g.Wo = d.out_w; g.Co = Co;
+    g.Kh = Kh; g.Kw = Kw;
+    g.pad_top = d.pad_top; g.pad_left = d.pad_left; g.stride_x = d.stride_x; g.stride_y = d.stride_y;
+    g.dil_x = d.dilation_x; g.dil_y = d.dilation_y;
+    g.depth_mult = d.depthwise ? Co / Ci : 1;
+    g.zx = d.input.offset; g.zw = wq->offset;
+    g.in_u8 = d.input.dtype == MI355X_QASYMM_U8;
+    g.w_u8 = wq->dtype == MI355X_QASYMM_U8;
+    p->rq = MakeRequant(d.output, d.activation, d.activation_a, d.activation_b);
+
+    p->K = d.depthwise ? Kh * Kw : Kh * Kw * Ci;
+    p->Co_pad = (Co + 127) / 128 * 128;
+    p->K_pad = (p->K + kIgemmBK - 1) / kIgemmBK * kIgemmBK;
+
+    // ---- per-channel requantization constants, in fp32 exactly as the reference's decoders produce them ----
+    std::vector<float> mult(p->Co_pad, 0.0f), biasf(p->Co_pad, 0.0f);
+    for (int c = 0; c < Co; ++c)
+    {
+        const float sw = wq->n_scales == 1 ? wq->scales[0] : wq->scales[c];
+        mult[c] = d.input.scale * sw;
+        if (d.bias_enabled)
+        {
+            if (bq->n_scales == 1)
+            {
+                // ScaledInt32Decoder, or Int32Decoder when no scale is set (Decoders.hpp:40-55)
+                const float sb = bq->scales[0];
+                biasf[c] = sb == 0.0f ? static_cast<float>(bias_host[c]) : static_cast<float>(bias_host[c]) * sb;
+            }
+            else
+            {
+                biasf[c] = static_cast<float>(bias_host[c]) * bq->scales[c];   // ScaledInt32PerAxisDecoder
+            }
+        }
+    }
+    if (int rc = Upload(reinterpret_cast<void**>(&p->mult), mult.data(), mult.size() * sizeof(float))) return rc;
+    if (int rc = Upload(reinterpret_cast<void**>(&p->biasf), biasf.data(), biasf.size() * sizeof(float))) return rc;
+
+    // ---- kernel selection ----------------------------------------------------------------------------------
+    const int zx_shift = g.in_u8 ? g.zx - 128 : g.zx;
+    const bool mfma_ok = !d.depthwise && g.zw == 0 && !g.w_u8 && (Ci % 16) == 0 && zx_shift >= -128 && zx_shift <= 127 &&
+                         p->K <= 100000;
+    const bool dw_ok = d.depthwise && g.depth_mult == 1 && (Co % 4) == 0;
+    int32_t algo = d.algo;
+    if (algo == MI355X_ALGO_AUTO) algo = mfma_ok ? MI355X_ALGO_MFMA : dw_ok ? MI355X_ALGO_DEPTHWISE : MI355X_ALGO_DIRECT;
+    if (algo == MI355X_ALGO_MFMA && !mfma_ok)
+        return SetError(MI355X_ERR_UNSUPPORTED, "MFMA kernel needs a non-depthwise layer, symmetric int8 weights and in_c %% 16 == 0");
+    if (algo == MI355X_ALGO_DEPTHWISE && !dw_ok)
+        return SetError(MI355X_ERR_UNSUPPORTED, "depthwise kernel needs multiplier 1 and channels %% 4 == 0");
+    if (algo < MI355X_ALGO_DIRECT || algo > MI355X_ALGO_DEPTHWISE) return SetError(MI355X_ERR_INVALID_ARGUMENT, "unknown algo %d", algo);
+    p->algo = algo;
+
+    const uint8_t* wsrc = static_cast<const uint8_t*>(weights_host);
+    if (algo == MI355X_ALGO_MFMA)
+    {
+        std::vector<int8_t> wp(static_cast<size_t>(p->Co_pad) * p->K_pad, 0);
+        std::vector<int32_t> corr(p->Co_pad, 0);
+        for (int c = 0; c < Co; ++c)
+        {
+            long long sum = 0;
+            const int8_t* src = reinterpret_cast<const int8_t*>(wsrc) + static_cast<size_t>(c) * p->K;
+            int8_t* dst = wp.data() + static_cast<size_t>(c) * p->K_pad;
+            for (int k = 0; k < p->K; ++k) { dst[k] = src[k]; sum += src[k]; }
+            corr[c] = static_cast<int32_t>(-static_cast<long long>(zx_shift) * sum);
+        }
+        if (int rc = Upload(reinterpret_cast<void**>(&p->w_mfma), wp.data(), wp.size())) return rc;
+        if (int rc = Upload(reinterpret_cast<void**>(&p->corr), corr.data(), corr.size() * sizeof(int32_t))) return rc;
+        p->xor_mask = g.in_u8 ? 0x80808080u : 0u;
+        const uint32_t zb = static_cast<uint32_t>(zx_shift) & 0xffu;
+        p->pad_word = zb | (zb << 8) | (zb << 16) | (zb << 24);
+        p->bm = 128;
+        p->bn = (Co <= 64) ? 64 : 128;
+        char buf[96];
+        snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 tile %dx%dx%d K=%d", p->bm, p->bn, kIgemmBK, p->K);
+        p->info = buf;
+    }
+    else if (algo == MI355X_ALGO_DEPTHWISE)
+    {
+        if (int rc = Upload(reinterpret_cast<void**>(&p->w_direct), wsrc, static_cast<size_t>(Kh) * Kw * Co)) return rc;
+        p->info = "depthwise_c4_valu";
+    }
+    else
+    {
+        if (d.depthwise)
+        {
+            if (int rc = Upload(reinterpret_cast<void**>(&p->w_direct), wsrc, static_cast<size_t>(Kh) * Kw * Co)) return rc;
+        }
+        else
+        {
+            // [Co][Kh][Kw][Ci] -> [Kh][Kw][Ci][Co]
+            std::vector<uint8_t> wt(static_cast<size_t>(Co) * p->K);
+            const size_t taps = static_cast<size_t>(Kh) * Kw * Ci;
+            for (int c = 0; c < Co; ++c)
+                for (size_t k = 0; k < taps; ++k) wt[k * Co + c] = wsrc[static_cast<size_t>(c) * taps + k];
+            if (int rc = Upload(reinterpret_cast<void**>(&p->w_direct), wt.data(), wt.size())) return rc;
+        }
+        p->info = d.depthwise ? "direct_depthwise" : "direct_conv";
+    }
+    return 0;
+}
+
+template <int BM, int BN, int WM, int WN>
+int LaunchIgemm(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    const ConvGeom& g = p->geom;
+    IgemmArgs a;
+    a.x = static_cast<const uint8_t*>(x);
+    a.w = p->w_mfma;
+    a.mult = p->mult;
+    a.biasf = p->biasf;
+    a.corr = p->corr;
+    a.y = static_cast<uint8_t*>(y);
+    const long long M = static_cast<long long>(batch) * g.Ho * g.Wo;
+    if (M > 0x7fffffffll / 2) return SetError(MI355X_ERR_UNSUPPORTED, "too many output pixels for one launch (%lld)", M);
+    a.M = static_cast<int>(M);
+    a.H = g.H; a.W = g.W; a.Ci = g.Ci; a.Ho = g.Ho; a.Wo = g.Wo; a.Co = g.Co;
+    a.Kh = g.Kh; a.Kw = g.Kw;
+    a.pad_top = g.pad_top; a.pad_left = g.pad_left; a.stride_x = g.stride_x; a.stride_y = g.stride_y;
+    a.dil_x = g.dil_x; a.dil_y = g.dil_y;
+    a.K_pad = p->K_pad;
+    a.tiles_m = static_cast<int>((M + BM - 1) / BM);
+    a.tiles_n = (g.Co + BN - 1) / BN;
+    a.xor_mask = p->xor_mask;
+    a.pad_word = p->pad_word;
+    a.rq = p->rq;
+    const int nblocks = a.tiles_m * a.tiles_n;
+    const int grid = (nblocks + 7) / 8 * 8;
+    hipLaunchKernelGGL((IgemmKernel<BM, BN, WM, WN>), dim3(grid), dim3(256), 0, stream, a);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    if (!p) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
+    if (batch == 0) return 0;
+    if (!x || !y) return SetError(MI355X_ERR_INVALID_ARGUMENT, "input / output pointer is null");
+    const ConvGeom& g = p->geom;
+    const long long total = static_cast<long long>(batch) * g.Ho * g.Wo * g.Co;
+    const uint8_t* xin = static_cast<const uint8_t*>(x);
+    uint8_t* yout = static_cast<uint8_t*>(y);
+    switch (p->algo)
+    {
+    case MI355X_ALGO_MFMA:
+        if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || ((g.Co & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) != 0))
+            return SetError(MI355X_ERR_INVALID_ARGUMENT, "MFMA kernel needs 16-byte aligned tensors");
+        if (p->bn == 64) return LaunchIgemm<128, 64, 2, 2>(p, batch, x, y, stream);
+        return LaunchIgemm<128, 128, 2, 2>(p, batch, x, y, stream);
+    case MI355X_ALGO_DEPTHWISE:
+    {
+        if ((reinterpret_cast<uintptr_t>(x) & 3) != 0 || (reinterpret_cast<uintptr_t>(y) & 3) != 0)
+            return SetError(MI355X_ERR_INVALID_ARGUMENT, "depthwise kernel needs 4-byte aligned tensors");
+        const long long total4 = total / 4;
+        const unsigned blocks = static_cast<unsigned>((total4 + 255) / 256);
+        if (g.in_u8 && !g.w_u8)
+            hipLaunchKernelGGL((DepthwiseC4Kernel<true, false>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total4);
+        else if (!g.in_u8 && !g.w_u8)
+            hipLaunchKernelGGL((DepthwiseC4Kernel<false, false>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total4);
+        else if (g.in_u8 && g.w_u8)
+            hipLaunchKernelGGL((DepthwiseC4Kernel<true, true>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total4);
+        else
+            hipLaunchKernelGGL((DepthwiseC4Kernel<false, true>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total4);
+        MI355X_HIP(hipGetLastError());
+        return 0;
+    }
+    default:
+    {
+        const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
+        if (p->d.depthwise)
+            hipLaunchKernelGGL((ConvDirectKernel<true>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total);
+        else
+            hipLaunchKernelGGL((ConvDirectKernel<false>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total);
+        MI355X_HIP(hipGetLastError());
+        return 0;
+    }
+    }
+}
+
+} // namespace
+
+extern "C" {
+
+int mi355x_conv2d_create(const mi355x_conv2d_desc* desc, const void* weights_host, const mi355x_const_quant* weights_quant,
+                         const int32_t* bias_host, const mi355x_const_quant* bias_quant, mi355x_conv2d_t* plan)
+{
+    if (!desc || !plan) return SetError(MI355X_ERR_INVALID_ARGUMENT, "descriptor / plan pointer is null");
+    *plan = nullptr;
+    auto* p = new mi355x_conv2d_s;
+    int rc = BuildPlan(*desc, weights_host, weights_quant, bias_host, bias_quant, p);
+    if (rc != 0) { delete p; return rc; }
+    *plan = p;
+    return 0;
+}
+
+int mi355x_conv2d_run(mi355x_conv2d_t plan, uint32_t batch, const void* input_dev, void* output_dev, mi355x_stream_t stream)
+{
+    return RunPlan(plan, batch, input_dev, output_dev, ToHip(stream));
+}
+
+int mi355x_conv2d_destroy(mi355x_conv2d_t plan)
+{
+    delete plan;
+    return 0;
+}
+
+int mi355x_conv2d_algo(mi355x_conv2d_t plan, int32_t* algo, char* desc_buf, size_t desc_len)
+{
+    if (!plan) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
+    if (algo) *algo = plan->algo;
+    if (desc_buf && desc_len) snprintf(desc_buf, desc_len, "%s", plan->info.c_str());
+    return 0;
+}
+
+// FullyConnected = 1x1 convolution over a 1x1 image with in_c = K: row n of the input is pixel n.
+int mi355x_fc_create(const mi355x_fc_desc* desc, const void* weights_host, const mi355x_const_quant* weights_quant,
+                     const int32_t* bias_host, const mi355x_const_quant* bias_quant, mi355x_fc_t* plan)
+{
+    if (!desc || !plan) return SetError(MI355X_ERR_INVALID_ARGUMENT, "descriptor / plan pointer is null");
+    *plan = nullptr;
+    if (desc->k == 0 || desc->out_features == 0) return SetError(MI355X_ERR_INVALID_ARGUMENT, "zero-sized FullyConnected");
+    if (!weights_host) return SetError(MI355X_ERR_INVALID_ARGUMENT, "weights missing");
+    mi355x_conv2d_desc c{};
+    c.in_h = c.in_w = c.out_h = c.out_w = 1;
+    c.in_c = desc->k;
+    c.out_c = desc->out_features;
+    c.kernel_h = c.kernel_w = 1;
+    c.stride_x = c.stride_y = c.dilation_x = c.dilation_y = 1;
+    c.bias_enabled = desc->bias_enabled;
+    c.input = desc->input;
+    c.output = desc->output;
+    c.activation = desc->activation;
+    c.activation_a = desc->activation_a;
+    c.activation_b = desc->activation_b;
+    c.algo = desc->algo;
+
+    const uint8_t* w = static_cast<const uint8_t*>(weights_host);
+    std::vector<uint8_t> wt;
+    if (!desc->transpose_weights)
+    {
+        // [K][O] -> [O][K]
+        const size_t K = desc->k, O = desc->out_features;
+        wt.resize(K * O);
+        for (size_t k = 0; k < K; ++k)
+            for (size_t o = 0; o < O; ++o) wt[o * K + k] = w[k * O + o];
+        w = wt.data();
+    }
+    auto* cp = new mi355x_conv2d_s;
+    int rc = BuildPlan(c, w, weights_quant, bias_host, bias_quant, cp);
+    if (rc != 0) { delete cp; return rc; }
+    auto* p = new mi355x_fc_s;
+    p->conv = cp;
+    *plan = p;
+    return 0;
+}
+
+int mi355x_fc_run(mi355x_fc_t plan, uint32_t batch, const void* input_dev, void* output_dev, mi355x_stream_t stream)
+{
+    if (!plan) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
+    return RunPlan(plan->conv, batch, input_dev, output_dev, ToHip(stream));
+}
+
+int mi355x_fc_destroy(mi355x_fc_t plan)
+{
+    delete plan;
+    return 0;
+}
+
+int mi355x_fc_algo(mi355x_fc_t plan, int32_t* algo, char* desc_buf, size_t desc_len)
+{
+    if (!plan) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
+    return mi355x_conv2d_algo(plan->conv, algo, desc_buf, desc_len);
+}
+
+} // extern "C"

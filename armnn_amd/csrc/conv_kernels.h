@@ -1,0 +1,427 @@
+// Device kernels for quantized Convolution2d / DepthwiseConvolution2d / FullyConnected on gfx950.
+//
+//   ConvDirectKernel      one thread per output element; every configuration the library accepts.
+//   DepthwiseC4Kernel     depthwise, multiplier 1, channels % 4 == 0: one thread per (pixel, 4 channels).
+//   IgemmKernel<BM,BN,..> implicit GEMM on v_mfma_i32_32x32x32_i8, NHWC tiles staged in LDS, exact int32
+//                         accumulation, fused requantize/clamp epilogue, output tile staged in LDS and stored
+//                         with 16-byte coalesced writes.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "device_math.h"
+
+namespace mi355x
+{
+
+typedef int v4i __attribute__((ext_vector_type(4)));
+typedef int v16i __attribute__((ext_vector_type(16)));
+
+struct ConvGeom
+{
+    int H, W, Ci, Ho, Wo, Co;
+    int Kh, Kw;
+    int pad_top, pad_left, stride_x, stride_y, dil_x, dil_y;
+    int depth_mult;     // depthwise only
+    int zx, zw;         // zero points of input and weights (in their own domain)
+    int in_u8, w_u8;
+};
+
+// ---------------------------------------------------------------------------------------------------------
+// Direct kernel.  Weights are laid out [Kh][Kw][Ci][Co] (conv) or [Kh][Kw][Co] (depthwise) so that
+// neighbouring threads (neighbouring output channels) read neighbouring bytes.
+// ---------------------------------------------------------------------------------------------------------
+template <bool DEPTHWISE>
+__global__ __launch_bounds__(256) void ConvDirectKernel(ConvGeom g, Requant rq, const uint8_t* __restrict__ x,
+                                                        const uint8_t* __restrict__ w,
+                                                        const float* __restrict__ mult,
+                                                        const float* __restrict__ biasf, uint8_t* __restrict__ y,
+                                                        long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int co = static_cast<int>(idx % g.Co);
+    long long pix = idx / g.Co;
+    const int ox = static_cast<int>(pix % g.Wo);
+    pix /= g.Wo;
+    const int oy = static_cast<int>(pix % g.Ho);
+    const long long n = pix / g.Ho;
+
+    const uint8_t* xn = x + n * g.H * g.W * g.Ci;
+    int acc = 0;
+    for (int ky = 0; ky < g.Kh; ++ky)
+    {
+        const int iy = oy * g.stride_y + ky * g.dil_y - g.pad_top;
+        if (iy < 0 || iy >= g.H) continue;
+        for (int kx = 0; kx < g.Kw; ++kx)
+        {
+            const int ix = ox * g.stride_x + kx * g.dil_x - g.pad_left;
+            if (ix < 0 || ix >= g.W) continue;
+            const uint8_t* xp = xn + (static_cast<long long>(iy) * g.W + ix) * g.Ci;
+            if (DEPTHWISE)
+            {
+                const int ci = co / g.depth_mult;
+                const int xv = g.in_u8 ? static_cast<int>(xp[ci]) : static_cast<int>(static_cast<int8_t>(xp[ci]));
+                const uint8_t wb = w[(ky * g.Kw + kx) * g.Co + co];
+                const int wv = g.w_u8 ? static_cast<int>(wb) : static_cast<int>(static_cast<int8_t>(wb));
+                acc += (xv - g.zx) * (wv - g.zw);
+            }
+            else
+            {
+                const uint8_t* wp = w + static_cast<long long>(ky * g.Kw + kx) * g.Ci * g.Co + co;
+                for (int ci = 0; ci < g.Ci; ++ci)
+                {
+                    const int xv = g.in_u8 ? static_cast<int>(xp[ci]) : static_cast<int>(static_cast<int8_t>(xp[ci]));
+                    const uint8_t wb = wp[static_cast<long long>(ci) * g.Co];
+                    const int wv = g.w_u8 ? static_cast<int>(wb) : static_cast<int>(static_cast<int8_t>(wb));
+                    acc += (xv - g.zx) * (wv - g.zw);
+                }
+            }
+        }
+    }
+    y[idx] = static_cast<uint8_t>(RequantDev(acc, mult[co], biasf[co], rq));
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Depthwise, multiplier 1, C % 4 == 0.  Weights stay in the reference layout [Kh][Kw][C].
+// ---------------------------------------------------------------------------------------------------------
+template <bool IN_U8, bool W_U8>
+__device__ __forceinline__ void DwMac4(uint32_t xw, uint32_t ww, int zx, int zw, int acc[4])
+{
+#pragma unroll
+    for (int b = 0; b < 4; ++b)
+    {
+        const int xv = IN_U8 ? static_cast<int>((xw >> (8 * b)) & 0xffu)
+                             : static_cast<int>(static_cast<int8_t>((xw >> (8 * b)) & 0xffu));
+        const int wv = W_U8 ? static_cast<int>((ww >> (8 * b)) & 0xffu)
+                            : static_cast<int>(static_cast<int8_t>((ww >> (8 * b)) & 0xffu));
+        acc[b] += (xv - zx) * (wv - zw);
+    }
+}
+
+template <bool IN_U8, bool W_U8>
+__global__ __launch_bounds__(256) void DepthwiseC4Kernel(ConvGeom g, Requant rq, const uint8_t* __restrict__ x,
+                                                         const uint8_t* __restrict__ w,
+                                                         const float* __restrict__ mult,
+                                                         const float* __restrict__ biasf,
+                                                         uint8_t* __restrict__ y, long long total_c4)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total_c4) return;
+    const int C4 = g.Co >> 2;
+    const int c = static_cast<int>(idx % C4) * 4;
+    long long pix = idx / C4;
+    const int ox = static_cast<int>(pix % g.Wo);
+    pix /= g.Wo;
+    const int oy = static_cast<int>(pix % g.Ho);
+    const long long n = pix / g.Ho;
+
+    const uint8_t* xn = x + n * g.H * g.W * g.Ci + c;
+    int acc[4] = {0, 0, 0, 0};
+    for (int ky = 0; ky < g.Kh; ++ky)
+    {
+        const int iy = oy * g.stride_y + ky * g.dil_y - g.pad_top;
+        if (iy < 0 || iy >= g.H) continue;
+        for (int kx = 0; kx < g.Kw; ++kx)
+        {
+            const int ix = ox * g.stride_x + kx * g.dil_x - g.pad_left;
+            if (ix < 0 || ix >= g.W) continue;
+            const uint32_t xw = *reinterpret_cast<const uint32_t*>(xn + (static_cast<long long>(iy) * g.W + ix) * g.Ci);
+            const uint32_t ww = *reinterpret_cast<const uint32_t*>(w + (ky * g.Kw + kx) * g.Co + c);
+            DwMac4<IN_U8, W_U8>(xw, ww, g.zx, g.zw, acc);
+        }
+    }
+    const float4 m4 = *reinterpret_cast<const float4*>(mult + c);
+    const float4 b4 = *reinterpret_cast<const float4*>(biasf + c);
+    uint32_t out = static_cast<uint32_t>(RequantDev(acc[0], m4.x, b4.x, rq) & 0xff);
+    out |= static_cast<uint32_t>(RequantDev(acc[1], m4.y, b4.y, rq) & 0xff) << 8;
+    out |= static_cast<uint32_t>(RequantDev(acc[2], m4.z, b4.z, rq) & 0xff) << 16;
+    out |= static_cast<uint32_t>(RequantDev(acc[3], m4.w, b4.w, rq) & 0xff) << 24;
+    *reinterpret_cast<uint32_t*>(y + idx * 4) = out;
+}
+
+// ---------------------------------------------------------------------------------------------------------
+// Implicit GEMM on MFMA.
+//
+//   GEMM view: rows m = (n, oy, ox) output pixels, columns = output channels, K = (ky, kx, ci) with ci
+//   fastest -- which is the memory order of both the NHWC input (per tap) and the [Co][Kh][Kw][Ci] weights, so
+//   both operands are read in 16-byte pieces that are contiguous in K.  Requires Ci % 16 == 0.
+//
+//   Inputs are brought to signed int8 on the fly (uint8: x ^ 0x80, i.e. x - 128, zero point shifted likewise);
+//   padding taps are filled with the (shifted) zero point, so acc = sum x'w - zx' * sum_k w, and the second
+//   term is a per-channel constant that initialises the accumulators (`corr`).  Weights must be symmetric
+//   (offset 0).
+//
+//   Block = 256 threads = 4 waves arranged WM x WN; each wave owns (BM/WM) x (BN/WN) outputs as 32x32 MFMA
+//   tiles.  The MFMA "A" operand is the weight fragment (row = channel) and "B" the activation fragment
+//   (column = pixel), so a lane ends up with 4 consecutive channels of one pixel per accumulator quad: the
+//   epilogue packs them into one dword, stages the BM x BN byte tile in LDS, and the block writes it out
+//   in 16-byte row-contiguous stores.
+// ---------------------------------------------------------------------------------------------------------
+struct IgemmArgs
+{
+    const uint8_t* x;
+    const int8_t*  w;       // [Co_pad][K_pad], zero padded
+    const float*   mult;    // [Co_pad]
+    const float*   biasf;   // [Co_pad]
+    const int32_t* corr;    // [Co_pad]
+    uint8_t*       y;
+    int M;                  // batch * Ho * Wo
+    int H, W, Ci, Ho, Wo, Co;
+    int Kh, Kw;
+    int pad_top, pad_left, stride_x, stride_y, dil_x, dil_y;
+    int K_pad;
+    int tiles_m, tiles_n;
+    uint32_t xor_mask;      // 0x80808080 for uint8 input, else 0
+    uint32_t pad_word;      // shifted input zero point replicated in 4 bytes
+    Requant rq;
+};
+
+constexpr int kIgemmBK  = 64;
+constexpr int kIgemmLDK = kIgemmBK + 16;   // LDS row stride in bytes: 80 keeps ds_read_b128 conflict-free
+
+template <int BM, int BN>
+constexpr int IgemmSmemBytes()
+{
+    constexpr int stage = (BM + BN) * kIgemmLDK;
+    constexpr int out = BM * (BN + 16);
+    return 2 * stage > out ? 2 * stage : out;
+}
+
+template <int BM, int BN, int WM, int WN>
+__global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
+{
+    static_assert(WM * WN == 4, "4 waves per block");
+    static_assert(BM % 64 == 0 && BN % 64 == 0, "tile sizes are multiples of 64");
+    constexpr int BK = kIgemmBK;
+    constexpr int LDK = kIgemmLDK;
+    constexpr int RA = BM / 64;                 // activation rows loaded per thread per k-tile
+    constexpr int RB = BN / 64;                 // weight rows loaded per thread per k-tile
+    constexpr int WTM = BM / WM;                // wave tile (pixels)
+    constexpr int WTN = BN / WN;                // wave tile (channels)
+    constexpr int TP = WTM / 32;                // 32-pixel sub-tiles per wave
+    constexpr int TC = WTN / 32;                // 32-channel sub-tiles per wave
+    constexpr int STAGE = (BM + BN) * LDK;
+    constexpr int LDO = BN + 16;
+
+    __shared__ __attribute__((aligned(16))) uint8_t smem[IgemmSmemBytes<BM, BN>()];
+
+    // XCD-aware tile order: consecutive block ids land on different XCDs, so give each XCD a contiguous run
+    // of tiles (tiles that share activation rows then share that XCD's L2).
+    const int nblocks = a.tiles_m * a.tiles_n;
+    const int per_xcd = (nblocks + 7) >> 3;
+    const int tile = static_cast<int>(blockIdx.x & 7) * per_xcd + static_cast<int>(blockIdx.x >> 3);
+    if (tile >= nblocks) return;
+    const int tn = tile % a.tiles_n;
+    const int tm = tile / a.tiles_n;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WN;
+    const int wn = wave % WN;
+
+    // ---- global -> LDS load assignment: 16-byte chunk `lc` of row `lr (+64 j)` -------------------------
+    const int lc = tid & 3;
+    const int lr = tid >> 2;
+
+    const uint8_t* xrow[RA];
+    int iy0[RA], ix0[RA];
+    bool mvalid[RA];
+#pragma unroll
+    for (int j = 0; j < RA; ++j)
+    {
+        const int m = tm * BM + lr + 64 * j;
+        mvalid[j] = m < a.M;
+        const int mm = mvalid[j] ? m : 0;
+        const int ox = mm % a.Wo;
+        const int t = mm / a.Wo;
+        const int oy = t % a.Ho;
+        const int n = t / a.Ho;
+        iy0[j] = oy * a.stride_y - a.pad_top;
+        ix0[j] = ox * a.stride_x - a.pad_left;
+        xrow[j] = a.x + static_cast<long long>(n) * a.H * a.W * a.Ci;
+    }
+    // position of this thread's chunk inside K: (ky, kx, ci), advanced by BK every k-tile
+    int ci, kx, ky;
+    {
+        const int k0 = lc * 16;
+        const int tap = k0 / a.Ci;
+        ci = k0 - tap * a.Ci;
+        ky = tap / a.Kw;
+        kx = tap - ky * a.Kw;
+    }
+    const int8_t* wrow = a.w + static_cast<long long>(tn * BN + lr) * a.K_pad + lc * 16;
+
+    v4i ra[RA], rb[RB];
+    const v4i padv = {static_cast<int>(a.pad_word), static_cast<int>(a.pad_word), static_cast<int>(a.pad_word),
+                      static_cast<int>(a.pad_word)};
+    const int xm = static_cast<int>(a.xor_mask);
+
+    auto load_tile = [&](int kt) {
+        const bool kvalid = ky < a.Kh;
+#pragma unroll
+        for (int j = 0; j < RA; ++j)
+        {
+            const int iy = iy0[j] + ky * a.dil_y;
+            const int ix = ix0[j] + kx * a.dil_x;
+            const bool ok = mvalid[j] && kvalid && static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) &&
+                            static_cast<unsigned>(ix) < static_cast<unsigned>(a.W);
+            if (ok)
+            {
+                v4i v = *reinterpret_cast<const v4i*>(xrow[j] + (static_cast<long long>(iy) * a.W + ix) * a.Ci + ci);
+                ra[j] = v ^ xm;
+            }
+            else
+            {
+                ra[j] = padv;
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < RB; ++j)
+        {
+            rb[j] = *reinterpret_cast<const v4i*>(wrow + static_cast<long long>(64 * j) * a.K_pad + kt * BK);
+        }
+        // advance (ky, kx, ci) by one k-tile
+        ci += BK;
+        while (ci >= a.Ci)
+        {
+            ci -= a.Ci;
+            if (++kx == a.Kw) { kx = 0; ++ky; }
+        }
+    };
+
+    auto store_tile = [&](int buf) {
+        uint8_t* As = smem + buf * STAGE;
+        uint8_t* Bs = As + BM * LDK;
+#pragma unroll
+        for (int j = 0; j < RA; ++j) *reinterpret_cast<v4i*>(As + (lr + 64 * j) * LDK + lc * 16) = ra[j];
+#pragma unroll
+        for (int j = 0; j < RB; ++j) *reinterpret_cast<v4i*>(Bs + (lr + 64 * j) * LDK + lc * 16) = rb[j];
+    };
+
+    // ---- accumulators, initialised with the zero-point correction -------------------------------------
+    // lane owns pixel (lane & 31) of each pixel sub-tile and channels 8*(v/4) + 4*(lane/32) + v%4 of each
+    // channel sub-tile.
+    const int lane_c = 4 * (lane >> 5);
+    const int cbase = tn * BN + wn * WTN;
+    v16i acc[TC][TP];
+#pragma unroll
+    for (int tc = 0; tc < TC; ++tc)
+    {
+        v16i init;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const v4i c4 = *reinterpret_cast<const v4i*>(a.corr + cbase + tc * 32 + 8 * q + lane_c);
+            init[4 * q + 0] = c4[0];
+            init[4 * q + 1] = c4[1];
+            init[4 * q + 2] = c4[2];
+            init[4 * q + 3] = c4[3];
+        }
+#pragma unroll
+        for (int tp = 0; tp < TP; ++tp) acc[tc][tp] = init;
+    }
+
+    const int nk = a.K_pad / BK;
+    load_tile(0);
+    store_tile(0);
+    __syncthreads();
+
+    const int frag_row = lane & 31;
+    const int frag_k = (lane >> 5) * 16;
+
+    for (int kt = 0; kt < nk; ++kt)
+    {
+        const int buf = kt & 1;
+        if (kt + 1 < nk) load_tile(kt + 1);
+
+        const uint8_t* As = smem + buf * STAGE;
+        const uint8_t* Bs = As + BM * LDK;
+#pragma unroll
+        for (int ks = 0; ks < BK / 32; ++ks)
+        {
+            v4i fa[TP], fw[TC];
+#pragma unroll
+            for (int tp = 0; tp < TP; ++tp)
+                fa[tp] = *reinterpret_cast<const v4i*>(As + (wm * WTM + tp * 32 + frag_row) * LDK + ks * 32 + frag_k);
+#pragma unroll
+            for (int tc = 0; tc < TC; ++tc)
+                fw[tc] = *reinterpret_cast<const v4i*>(Bs + (wn * WTN + tc * 32 + frag_row) * LDK + ks * 32 + frag_k);
+#pragma unroll
+            for (int tc = 0; tc < TC; ++tc)
+#pragma unroll
+                for (int tp = 0; tp < TP; ++tp)
+                    acc[tc][tp] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[tc], fa[tp], acc[tc][tp], 0, 0, 0);
+        }
+
+        if (kt + 1 < nk) store_tile(buf ^ 1);
+        __syncthreads();
+    }
+
+    // ---- epilogue: requantize, pack 4 channels per dword, stage the byte tile in LDS ---------------------
+    uint8_t* Os = smem;   // all reads of the stage buffers are behind the loop's final barrier
+#pragma unroll
+    for (int tc = 0; tc < TC; ++tc)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const int cl = wn * WTN + tc * 32 + 8 * q + lane_c;           // channel within the block tile
+            const float4 m4 = *reinterpret_cast<const float4*>(a.mult + tn * BN + cl);
+            const float4 b4 = *reinterpret_cast<const float4*>(a.biasf + tn * BN + cl);
+#pragma unroll
+            for (int tp = 0; tp < TP; ++tp)
+            {
+                const v16i& c = acc[tc][tp];
+                uint32_t out = static_cast<uint32_t>(RequantDev(c[4 * q + 0], m4.x, b4.x, a.rq) & 0xff);
+                out |= static_cast<uint32_t>(RequantDev(c[4 * q + 1], m4.y, b4.y, a.rq) & 0xff) << 8;
+                out |= static_cast<uint32_t>(RequantDev(c[4 * q + 2], m4.z, b4.z, a.rq) & 0xff) << 16;
+                out |= static_cast<uint32_t>(RequantDev(c[4 * q + 3], m4.w, b4.w, a.rq) & 0xff) << 24;
+                const int pl = wm * WTM + tp * 32 + (lane & 31);          // pixel within the block tile
+                *reinterpret_cast<uint32_t*>(Os + pl * LDO + cl) = out;
+            }
+        }
+    }
+    __syncthreads();
+
+    // ---- coalesced write-out ----------------------------------------------------------------------------
+    constexpr int CHUNKS = BN / 16;             // 16-byte chunks per tile row
+    constexpr int ROWS_PER_PASS = 256 / CHUNKS;
+    const int oc = tid % CHUNKS;
+    const int orow = tid / CHUNKS;
+    const int c0 = tn * BN + oc * 16;
+    if ((a.Co & 15) == 0)
+    {
+        if (c0 < a.Co)
+        {
+#pragma unroll
+            for (int r = orow; r < BM; r += ROWS_PER_PASS)
+            {
+                const int m = tm * BM + r;
+                if (m < a.M)
+                {
+                    const v4i v = *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16);
+                    *reinterpret_cast<v4i*>(a.y + static_cast<long long>(m) * a.Co + c0) = v;
+                }
+            }
+        }
+    }
+    else
+    {
+        // ragged channel count (e.g. 1001 classes): rows are not 16-byte aligned, store byte by byte
+        for (int r = orow; r < BM; r += ROWS_PER_PASS)
+        {
+            const int m = tm * BM + r;
+            if (m >= a.M) continue;
+            for (int b = 0; b < 16; ++b)
+            {
+                const int c = c0 + b;
+                if (c < a.Co) a.y[static_cast<long long>(m) * a.Co + c] = Os[r * LDO + oc * 16 + b];
+            }
+        }
+    }
+}
+
+} // namespace mi355x

@@ -1,0 +1,239 @@
+// Bandwidth-bound layers that keep a network resident on the device between the convolutions:
+// Activation, Pooling2d, ElementwiseBinary Add, Softmax.  All follow the reference's float formulation
+// (dequantize -> float op -> armnn::Quantize) element for element.
+#include "common.h"
+#include "device_math.h"
+
+#include <cfloat>
+#include <cmath>
+
+using namespace mi355x;
+
+namespace
+{
+
+struct QIn
+{
+    float scale;
+    int   offset;
+    int   is_u8;
+};
+
+__device__ __forceinline__ float DequantDev(uint8_t code, const QIn& q)
+{
+    const int v = q.is_u8 ? static_cast<int>(code) : static_cast<int>(static_cast<int8_t>(code));
+    return __fmul_rn(static_cast<float>(v - q.offset), q.scale);   // armnn::Dequantize, TypesUtils.cpp:47-56
+}
+
+__device__ __forceinline__ float ActivationDev(float in, int fn, float a, float b)
+{
+    if (fn == MI355X_ACT_RELU) return fmaxf(0.0f, in);
+    if (fn == MI355X_ACT_BOUNDED_RELU) return fminf(a, fmaxf(b, in));
+    return in;
+}
+
+QIn MakeQIn(const mi355x_quant& q)
+{
+    QIn r;
+    r.scale = q.scale;
+    r.offset = q.offset;
+    r.is_u8 = q.dtype == MI355X_QASYMM_U8;
+    return r;
+}
+
+// A per-element function of one 8-bit code: build the 256-entry table once per block, then stream.
+__global__ __launch_bounds__(256) void ActivationKernel(QIn qin, Requant rq, int fn, float a, float b,
+                                                        const uint8_t* __restrict__ x, uint8_t* __restrict__ y, size_t n)
+{
+    __shared__ uint8_t lut[256];
+    lut[threadIdx.x] = static_cast<uint8_t>(QuantizeDev(ActivationDev(DequantDev(static_cast<uint8_t>(threadIdx.x), qin), fn, a, b), rq));
+    __syncthreads();
+    size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (; i < n; i += stride) y[i] = lut[x[i]];
+}
+
+struct PoolArgs
+{
+    int H, W, C, Ho, Wo;
+    int pool_w, pool_h, stride_x, stride_y;
+    int pad_left, pad_right, pad_top, pad_bottom;
+    int is_max, exclude;
+};
+
+// One thread per output element; same window clamping and divisor rules as Pooling2d.cpp:186-300.
+__global__ __launch_bounds__(256) void Pool2dKernel(PoolArgs p, QIn qin, Requant rq, const uint8_t* __restrict__ x,
+                                                    uint8_t* __restrict__ y, long long total)
+{
+    long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total) return;
+    const int c = static_cast<int>(idx % p.C);
+    long long pix = idx / p.C;
+    const int ox = static_cast<int>(pix % p.Wo);
+    pix /= p.Wo;
+    const int oy = static_cast<int>(pix % p.Ho);
+    const long long n = pix / p.Ho;
+
+    int hstart = oy * p.stride_y - p.pad_top;
+    int hend = min(hstart + p.pool_h, p.H + p.pad_bottom);
+    const int height = hend - hstart;
+    bool clamped = hstart < 0 || hend > p.H;
+    hstart = min(max(hstart, 0), p.H);
+    hend = min(max(hend, 0), p.H);
+    int wstart = ox * p.stride_x - p.pad_left;
+    int wend = min(wstart + p.pool_w, p.W + p.pad_right);
+    float area = static_cast<float>(height * (wend - wstart));
+    float result;
+    if (hend <= 0 || hstart > p.H || wend <= 0 || wstart > p.W)
+    {
+        result = 0.0f;      // window covers padding only
+    }
+    else
+    {
+        clamped = clamped || wstart < 0 || wend > p.W;
+        wstart = min(max(wstart, 0), p.W);
+        wend = min(max(wend, 0), p.W);
+        // The reference's clamp flag carries along a row, but with Exclude the divisor it selects equals
+        // the unclamped one whenever this window itself is unclamped, so the per-window flag is equivalent.
+        if (clamped && p.exclude) area = static_cast<float>((hend - hstart) * (wend - wstart));
+        result = p.is_max ? -FLT_MAX : 0.0f;
+        const uint8_t* xn = x + n * p.H * p.W * p.C + c;
+        for (int iy = hstart; iy < hend; ++iy)
+            for (int ix = wstart; ix < wend; ++ix)
+            {
+                const float v = DequantDev(xn[(static_cast<long long>(iy) * p.W + ix) * p.C], qin);
+                if (p.is_max) { if (v > result) result = v; }
+                else result = __fadd_rn(result, v);
+            }
+        if (!p.is_max) result = __fdiv_rn(result, area);
+    }
+    y[idx] = static_cast<uint8_t>(QuantizeDev(result, rq));
+}
+
+__global__ __launch_bounds__(256) void AddKernel(QIn q0, QIn q1, Requant rq, int fn, float a, float b,
+                                                 const uint8_t* __restrict__ x0, const uint8_t* __restrict__ x1,
+                                                 uint8_t* __restrict__ y, size_t n)
+{
+    size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (; i < n; i += stride)
+    {
+        const float s = __fadd_rn(DequantDev(x0[i], q0), DequantDev(x1[i], q1));
+        int q = QuantizeDev(s, rq);   // rq carries the fused activation as an integer clamp
+        y[i] = static_cast<uint8_t>(q);
+    }
+    (void)fn; (void)a; (void)b;
+}
+
+// One wave per row. exp((x - max) * beta) / sum, Softmax.cpp:41-64.
+__global__ __launch_bounds__(64) void SoftmaxKernel(int cols, float beta, QIn qin, Requant rq,
+                                                    const uint8_t* __restrict__ x, uint8_t* __restrict__ y)
+{
+    const uint8_t* xr = x + static_cast<long long>(blockIdx.x) * cols;
+    uint8_t* yr = y + static_cast<long long>(blockIdx.x) * cols;
+    const int lane = threadIdx.x;
+    float mx = -FLT_MAX;
+    for (int i = lane; i < cols; i += 64) mx = fmaxf(mx, DequantDev(xr[i], qin));
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    float sum = 0.0f;
+    for (int i = lane; i < cols; i += 64) sum += expf(__fmul_rn(__fsub_rn(DequantDev(xr[i], qin), mx), beta));
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    for (int i = lane; i < cols; i += 64)
+    {
+        const float e = expf(__fmul_rn(__fsub_rn(DequantDev(xr[i], qin), mx), beta));
+        yr[i] = static_cast<uint8_t>(QuantizeDev(__fdiv_rn(e, sum), rq));
+    }
+}
+
+int CheckQ(const mi355x_quant* q, const char* what)
+{
+    if (!q) return SetError(MI355X_ERR_INVALID_ARGUMENT, "%s quantization is null", what);
+    if (!IsActivationDtype(q->dtype)) return SetError(MI355X_ERR_UNSUPPORTED, "%s: data type %d is not QAsymmS8/QAsymmU8", what, q->dtype);
+    if (!(q->scale > 0.0f) || !std::isfinite(q->scale)) return SetError(MI355X_ERR_INVALID_ARGUMENT, "%s: scale must be positive and finite", what);
+    return 0;
+}
+
+unsigned GridFor(size_t n)
+{
+    size_t b = (n + 255) / 256;
+    return static_cast<unsigned>(b > 16384 ? 16384 : b);
+}
+
+} // namespace
+
+extern "C" {
+
+int mi355x_activation_run(size_t n, const mi355x_quant* in_q, const mi355x_quant* out_q, int32_t activation, float a,
+                          float b, const void* input_dev, void* output_dev, mi355x_stream_t stream)
+{
+    if (int rc = CheckQ(in_q, "input")) return rc;
+    if (int rc = CheckQ(out_q, "output")) return rc;
+    if (activation < MI355X_ACT_NONE || activation > MI355X_ACT_BOUNDED_RELU) return SetError(MI355X_ERR_UNSUPPORTED, "activation %d", activation);
+    if (n == 0) return 0;
+    if (!input_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "null tensor pointer");
+    Requant rq = MakeRequant(*out_q, MI355X_ACT_NONE, 0.0f, 0.0f);
+    hipLaunchKernelGGL(ActivationKernel, dim3(GridFor(n)), dim3(256), 0, ToHip(stream), MakeQIn(*in_q), rq, activation, a, b,
+                       static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), n);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+int mi355x_pool2d_run(const mi355x_pool2d_desc* d, uint32_t batch, const void* input_dev, void* output_dev,
+                      mi355x_stream_t stream)
+{
+    if (!d) return SetError(MI355X_ERR_INVALID_ARGUMENT, "descriptor is null");
+    if (int rc = CheckQ(&d->input, "input")) return rc;
+    if (int rc = CheckQ(&d->output, "output")) return rc;
+    if (d->pool_type != 0 && d->pool_type != 1) return SetError(MI355X_ERR_UNSUPPORTED, "Unsupported pooling algorithm %d", d->pool_type);
+    if (d->padding_method != 0 && d->padding_method != 1) return SetError(MI355X_ERR_UNSUPPORTED, "Unsupported padding type %d", d->padding_method);
+    if (d->pool_w == 0 || d->pool_h == 0 || d->stride_x == 0 || d->stride_y == 0 || d->channels == 0)
+        return SetError(MI355X_ERR_INVALID_ARGUMENT, "zero pool size / stride / channels");
+    if (batch == 0 || d->out_h == 0 || d->out_w == 0) return 0;
+    if (!input_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "null tensor pointer");
+    PoolArgs p;
+    p.H = d->in_h; p.W = d->in_w; p.C = d->channels; p.Ho = d->out_h; p.Wo = d->out_w;
+    p.pool_w = d->pool_w; p.pool_h = d->pool_h; p.stride_x = d->stride_x; p.stride_y = d->stride_y;
+    p.pad_left = d->pad_left; p.pad_right = d->pad_right; p.pad_top = d->pad_top; p.pad_bottom = d->pad_bottom;
+    p.is_max = d->pool_type == 0;
+    p.exclude = d->padding_method == 1;
+    Requant rq = MakeRequant(d->output, MI355X_ACT_NONE, 0.0f, 0.0f);
+    const long long total = static_cast<long long>(batch) * p.Ho * p.Wo * p.C;
+    hipLaunchKernelGGL(Pool2dKernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, ToHip(stream), p,
+                       MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), total);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+int mi355x_add_run(size_t n, const mi355x_quant* in0_q, const mi355x_quant* in1_q, const mi355x_quant* out_q,
+                   int32_t activation, float a, float b, const void* input0_dev, const void* input1_dev,
+                   void* output_dev, mi355x_stream_t stream)
+{
+    if (int rc = CheckQ(in0_q, "input0")) return rc;
+    if (int rc = CheckQ(in1_q, "input1")) return rc;
+    if (int rc = CheckQ(out_q, "output")) return rc;
+    if (activation < MI355X_ACT_NONE || activation > MI355X_ACT_BOUNDED_RELU) return SetError(MI355X_ERR_UNSUPPORTED, "activation %d", activation);
+    if (n == 0) return 0;
+    if (!input0_dev || !input1_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "null tensor pointer");
+    Requant rq = MakeRequant(*out_q, activation, a, b);
+    hipLaunchKernelGGL(AddKernel, dim3(GridFor(n)), dim3(256), 0, ToHip(stream), MakeQIn(*in0_q), MakeQIn(*in1_q), rq,
+                       activation, a, b, static_cast<const uint8_t*>(input0_dev), static_cast<const uint8_t*>(input1_dev),
+                       static_cast<uint8_t*>(output_dev), n);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+int mi355x_softmax_run(uint32_t rows, uint32_t cols, float beta, const mi355x_quant* in_q, const mi355x_quant* out_q,
+                       const void* input_dev, void* output_dev, mi355x_stream_t stream)
+{
+    if (int rc = CheckQ(in_q, "input")) return rc;
+    if (int rc = CheckQ(out_q, "output")) return rc;
+    if (rows == 0 || cols == 0) return 0;
+    if (!input_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "null tensor pointer");
+    Requant rq = MakeRequant(*out_q, MI355X_ACT_NONE, 0.0f, 0.0f);
+    hipLaunchKernelGGL(SoftmaxKernel, dim3(rows), dim3(64), 0, ToHip(stream), static_cast<int>(cols), beta, MakeQIn(*in_q), rq,
+                       static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev));
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+} // extern "C"

@@ -1,0 +1,234 @@
+/*
+ * armnn_mi355x.h -- C ABI of the MI355X (gfx950) device library behind the Arm NN "Mi355x" backend.
+ *
+ * This is the only door to the GPU: the C++17 backend (IBackendInternal / IWorkloadFactory / ITensorHandle /
+ * IMemoryManager implementations) calls nothing but these functions, and so can any other host
+ * (ctypes, JNI, cgo ...).  Plain pointers, sizes and POD structs only; no C++ or framework types.
+ *
+ * Conventions
+ *   - every function returns 0 on success, otherwise a non-zero code (a hipError_t value when the
+ *     failure came from HIP, MI355X_ERR_* otherwise); mi355x_last_error() returns a thread-local message.
+ *     Nothing throws across this boundary.
+ *   - pointers named *_dev are device pointers obtained from mi355x_malloc(); *_host are host pointers.
+ *   - tensors are dense NHWC (Convolution2d / DepthwiseConvolution2d / Pooling2d) or row-major [M,K]
+ *     (FullyConnected), 8-bit quantized, exactly as the reference's workloads see them.
+ *   - a "plan" owns device copies of the constant operands (weights re-laid-out for the kernel, per-channel
+ *     requantization multipliers, bias, zero-point corrections).  Plans are immutable after creation and may
+ *     be run concurrently on different streams.
+ *   - results equal the reference's CpuRef workloads to within 1 LSB (the accumulation is exact int32 where
+ *     the reference accumulates in fp32); the requantization uses the reference's float formula.
+ *
+ * Reference interfaces each entry point stands in for (paths relative to the Arm NN 35.0.0 tree) are cited
+ * at each declaration.
+ */
+#ifndef ARMNN_MI355X_H
+#define ARMNN_MI355X_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define MI355X_ABI_VERSION 1
+
+/* error codes outside the hipError_t range */
+#define MI355X_ERR_INVALID_ARGUMENT 10001
+#define MI355X_ERR_UNSUPPORTED      10002
+#define MI355X_ERR_NO_DEVICE        10003
+#define MI355X_ERR_OUT_OF_MEMORY    10004
+
+/* armnn::DataType subset (include/armnn/Types.hpp:48-64) */
+typedef enum {
+    MI355X_QASYMM_S8 = 0,
+    MI355X_QASYMM_U8 = 1,
+    MI355X_QSYMM_S8  = 2,
+    MI355X_SIGNED32  = 3
+} mi355x_dtype;
+
+/* armnn::ActivationFunction subset that the backend fuses (include/armnn/Types.hpp:86-101) */
+typedef enum {
+    MI355X_ACT_NONE         = 0,
+    MI355X_ACT_RELU         = 1,   /* max(0, x)            */
+    MI355X_ACT_BOUNDED_RELU = 2    /* min(a, max(b, x))    */
+} mi355x_activation;
+
+/* kernel selection; AUTO picks the fastest kernel whose preconditions hold */
+typedef enum {
+    MI355X_ALGO_AUTO      = 0,
+    MI355X_ALGO_DIRECT    = 1,   /* one thread per output element; accepts every supported configuration      */
+    MI355X_ALGO_MFMA      = 2,   /* implicit-GEMM on v_mfma_i32_32x32x32_i8 (conv / FC; symmetric int8 weights) */
+    MI355X_ALGO_DEPTHWISE = 3    /* channel-vectorised VALU kernel (depthwise, multiplier 1)                   */
+} mi355x_algo;
+
+typedef struct mi355x_stream_s* mi355x_stream_t;   /* NULL = the default stream */
+typedef struct mi355x_event_s*  mi355x_event_t;
+typedef struct mi355x_graph_s*  mi355x_graph_t;
+typedef struct mi355x_conv2d_s* mi355x_conv2d_t;
+typedef struct mi355x_fc_s*     mi355x_fc_t;
+
+/* Quantization of one activation tensor: armnn::TensorInfo scale/offset (include/armnn/Tensor.hpp:203-217). */
+typedef struct {
+    int32_t dtype;      /* MI355X_QASYMM_S8 or MI355X_QASYMM_U8 */
+    float   scale;
+    int32_t offset;
+} mi355x_quant;
+
+/* Quantization of a constant tensor: per-tensor (n_scales == 1) or per-axis (one scale per output channel). */
+typedef struct {
+    int32_t      dtype;      /* weights: QSYMM_S8 / QASYMM_S8 / QASYMM_U8 ; bias: SIGNED32 */
+    int32_t      offset;     /* must be 0 for per-axis weights and for bias (WorkloadData.cpp:180-205,353-393) */
+    uint32_t     n_scales;   /* 1 or the number of output channels */
+    const float* scales;     /* host pointer, n_scales entries */
+} mi355x_const_quant;
+
+/* ------------------------------------------------------------------------------------------------------
+ * Runtime: device, memory, streams, events, graphs.
+ * Used by the backend's IBackendContext / IMemoryManager / ITensorHandle implementations; the CpuRef
+ * counterparts are RefMemoryManager (src/backends/reference/RefMemoryManager.cpp:20-101) and
+ * RefTensorHandle::Map/CopyInFrom/CopyOutTo (src/backends/reference/RefTensorHandle.cpp:45-133).
+ * ---------------------------------------------------------------------------------------------------- */
+const char* mi355x_last_error(void);
+int  mi355x_abi_version(void);
+int  mi355x_device_count(int* count);                 /* 0 devices is success with *count == 0 */
+int  mi355x_init(int device);                         /* select + warm up the device; idempotent */
+int  mi355x_device_name(char* buf, size_t buf_len);   /* e.g. "gfx950:sramecc+:xnack-" */
+int  mi355x_device_props(int* compute_units, int* clock_khz, size_t* total_mem, size_t* lds_per_cu);
+
+int  mi355x_malloc(void** ptr_dev, size_t bytes);
+int  mi355x_free(void* ptr_dev);
+int  mi355x_host_alloc(void** ptr_host, size_t bytes);          /* pinned host memory (hipHostMalloc) */
+int  mi355x_host_free(void* ptr_host);
+int  mi355x_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes, mi355x_stream_t stream);
+int  mi355x_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, mi355x_stream_t stream);
+int  mi355x_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, mi355x_stream_t stream);
+int  mi355x_fill_u8(void* dst_dev, uint8_t value, size_t bytes, mi355x_stream_t stream);  /* fill kernel, graph-safe */
+
+int  mi355x_stream_create(mi355x_stream_t* stream);
+int  mi355x_stream_destroy(mi355x_stream_t stream);
+int  mi355x_stream_synchronize(mi355x_stream_t stream);
+int  mi355x_device_synchronize(void);
+
+int  mi355x_event_create(mi355x_event_t* event);
+int  mi355x_event_destroy(mi355x_event_t event);
+int  mi355x_event_record(mi355x_event_t event, mi355x_stream_t stream);
+int  mi355x_event_synchronize(mi355x_event_t event);
+int  mi355x_event_elapsed_ms(mi355x_event_t start, mi355x_event_t stop, float* ms);
+
+/* Capture everything launched on `stream` between begin and end into an executable graph, then replay it
+ * with one launch (removes per-kernel launch latency from a network's steady-state loop). */
+int  mi355x_graph_capture_begin(mi355x_stream_t stream);
+int  mi355x_graph_capture_end(mi355x_stream_t stream, mi355x_graph_t* graph);
+int  mi355x_graph_launch(mi355x_graph_t graph, mi355x_stream_t stream);
+int  mi355x_graph_destroy(mi355x_graph_t graph);
+
+/* ------------------------------------------------------------------------------------------------------
+ * Convolution2d / DepthwiseConvolution2d
+ *
+ * Stands in for RefConvolution2dWorkload::Execute (workloads/RefConvolution2dWorkload.cpp:38-58) and
+ * RefDepthwiseConvolution2dWorkload::Execute (workloads/RefDepthwiseConvolution2dWorkload.cpp:38-62), i.e.
+ * Convolve() (workloads/ConvImpl.cpp:68-233) between MakeDecoder/MakeEncoder (Decoders.hpp:63-126,
+ * Encoders.hpp:19-91), optionally followed by the Activation layer the backend fused into it
+ * (workloads/Activation.cpp:33-42 via RefActivationWorkload.cpp:23-36).
+ *
+ * Fields mirror armnn::Convolution2dDescriptor / DepthwiseConvolution2dDescriptor
+ * (include/armnn/Descriptors.hpp:534-585,659-711) and the tensor infos in WorkloadInfo.  As in Convolve(),
+ * only pad_top / pad_left are inputs; bottom / right padding is implied by the output shape.
+ * ---------------------------------------------------------------------------------------------------- */
+typedef struct {
+    uint32_t in_h, in_w, in_c;            /* input  [N, in_h, in_w, in_c]                      */
+    uint32_t out_h, out_w, out_c;         /* output [N, out_h, out_w, out_c]                   */
+    uint32_t kernel_h, kernel_w;
+    uint32_t pad_top, pad_left;
+    uint32_t stride_x, stride_y;
+    uint32_t dilation_x, dilation_y;
+    uint32_t depthwise;                   /* 0: weights [out_c, kh, kw, in_c]; 1: weights [1, kh, kw, out_c], out_c = in_c * M */
+    uint32_t bias_enabled;
+    mi355x_quant input;
+    mi355x_quant output;
+    int32_t  activation;                  /* mi355x_activation */
+    float    activation_a, activation_b;  /* ActivationDescriptor::m_A / m_B */
+    int32_t  algo;                        /* mi355x_algo */
+} mi355x_conv2d_desc;
+
+/* weights_host / bias_host are read once and may be released after the call returns.
+ * Weight scales index the OUTPUT channel (quantization dim 0 for conv, 3 for depthwise); bias scales index
+ * the output channel; with n_scales == 1 the single scale applies to all channels.  bias quantization is
+ * NOT assumed to equal input_scale * weight_scale. */
+int mi355x_conv2d_create(const mi355x_conv2d_desc* desc,
+                         const void* weights_host, const mi355x_const_quant* weights_quant,
+                         const int32_t* bias_host, const mi355x_const_quant* bias_quant,
+                         mi355x_conv2d_t* plan);
+int mi355x_conv2d_run(mi355x_conv2d_t plan, uint32_t batch, const void* input_dev, void* output_dev,
+                      mi355x_stream_t stream);
+int mi355x_conv2d_destroy(mi355x_conv2d_t plan);
+/* which kernel a plan resolved to (mi355x_algo) and its tile configuration, for logs and tests */
+int mi355x_conv2d_algo(mi355x_conv2d_t plan, int32_t* algo, char* desc_buf, size_t desc_len);
+
+/* ------------------------------------------------------------------------------------------------------
+ * FullyConnected
+ *
+ * Stands in for RefFullyConnectedWorkload::Execute (workloads/RefFullyConnectedWorkload.cpp:39-67) ->
+ * FullyConnected() (workloads/FullyConnected.cpp:13-65).  K is the product of the input's dimensions after
+ * the first (GetNumActivations, RefFullyConnectedWorkload.cpp:16-24).
+ * Fields mirror armnn::FullyConnectedDescriptor (include/armnn/Descriptors.hpp:507-531).
+ * ---------------------------------------------------------------------------------------------------- */
+typedef struct {
+    uint32_t k;                           /* inputs per row                                        */
+    uint32_t out_features;                /* outputs per row                                       */
+    uint32_t transpose_weights;           /* 1: weights [out_features, k]; 0: weights [k, out_features] */
+    uint32_t bias_enabled;
+    mi355x_quant input;
+    mi355x_quant output;
+    int32_t  activation;
+    float    activation_a, activation_b;
+    int32_t  algo;
+} mi355x_fc_desc;
+
+int mi355x_fc_create(const mi355x_fc_desc* desc,
+                     const void* weights_host, const mi355x_const_quant* weights_quant,
+                     const int32_t* bias_host, const mi355x_const_quant* bias_quant,
+                     mi355x_fc_t* plan);
+int mi355x_fc_run(mi355x_fc_t plan, uint32_t batch, const void* input_dev, void* output_dev,
+                  mi355x_stream_t stream);
+int mi355x_fc_destroy(mi355x_fc_t plan);
+int mi355x_fc_algo(mi355x_fc_t plan, int32_t* algo, char* desc_buf, size_t desc_len);
+
+/* ------------------------------------------------------------------------------------------------------
+ * Bandwidth-bound layers that keep a whole network on the device (no bounce through CpuRef).
+ * ---------------------------------------------------------------------------------------------------- */
+
+/* Standalone Activation layer, ReLu / BoundedReLu, same quantization in and out or different:
+ * RefActivationWorkload::Execute (workloads/RefActivationWorkload.cpp:23-36). */
+int mi355x_activation_run(size_t n_elements, const mi355x_quant* in_q, const mi355x_quant* out_q,
+                          int32_t activation, float a, float b,
+                          const void* input_dev, void* output_dev, mi355x_stream_t stream);
+
+/* Pooling2d, NHWC: Pooling2d() (workloads/Pooling2d.cpp:142-303).  Fields mirror armnn::Pooling2dDescriptor
+ * (include/armnn/Descriptors.hpp:371-418). pool_type: 0 Max, 1 Average.  padding_method: 0 IgnoreValue, 1 Exclude. */
+typedef struct {
+    uint32_t in_h, in_w, channels, out_h, out_w;
+    uint32_t pool_w, pool_h, stride_x, stride_y;
+    uint32_t pad_left, pad_right, pad_top, pad_bottom;
+    int32_t  pool_type, padding_method;
+    mi355x_quant input, output;
+} mi355x_pool2d_desc;
+int mi355x_pool2d_run(const mi355x_pool2d_desc* desc, uint32_t batch, const void* input_dev, void* output_dev,
+                      mi355x_stream_t stream);
+
+/* ElementwiseBinary Add of two equally-shaped tensors (dequantize, add, requantize) with an optional fused
+ * ReLu / BoundedReLu: RefElementwiseBinaryWorkload (workloads/RefElementwiseBinaryWorkload.cpp:27-107). */
+int mi355x_add_run(size_t n_elements, const mi355x_quant* in0_q, const mi355x_quant* in1_q,
+                   const mi355x_quant* out_q, int32_t activation, float a, float b,
+                   const void* input0_dev, const void* input1_dev, void* output_dev, mi355x_stream_t stream);
+
+/* Softmax over the last axis of a [rows, cols] tensor: Softmax() (workloads/Softmax.cpp:16-69). */
+int mi355x_softmax_run(uint32_t rows, uint32_t cols, float beta, const mi355x_quant* in_q,
+                       const mi355x_quant* out_q, const void* input_dev, void* output_dev,
+                       mi355x_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* ARMNN_MI355X_H */

@@ -1,0 +1,133 @@
+"""HIP kernels vs the CPU checker through the C ABI, on seeded inputs (needs an MI355X).
+
+Bar: every quantized output within 1 LSB of CpuRef's float-accumulated result (the reference's own tolerance for
+quantized layer tests, include/armnnTestUtils/TensorHelpers.hpp:24-31); the exact-match fraction is printed and
+asserted to stay high.  Kernels that share the integer accumulation (direct / MFMA / depthwise) must agree with
+each other bit for bit.
+"""
+import numpy as np
+import pytest
+
+from armnn_amd import shim
+from armnn_amd.tensor import DataType
+from tests import cases
+from tests.helpers import load_json, tensor_from_json, lsb_diff
+
+pytestmark = pytest.mark.gpu
+
+CONV = cases.small_conv_cases()
+FC = cases.small_fc_cases()
+LIT = load_json("reference_literals.json")
+
+
+def _oracle_conv(port, c):
+    y = port.conv2d(c.x, c.w, c.b, c.out_info, **c.params)
+    fn, a, b = c.act
+    return port.activation(y, c.out_info, fn, a, b) if fn else y
+
+
+def _gpu_conv(c, algo):
+    fn, a, b = c.act
+    return shim.conv2d(c.x, c.w, c.b, c.out_info, activation=fn, act_a=a, act_b=b, algo=algo, **c.params)
+
+
+@pytest.mark.parametrize("case", CONV, ids=[c.name for c in CONV])
+def test_conv_cases(port, case):
+    print(f"case={case.name} x={case.x.info.shape} w={case.w.info.shape}", flush=True)
+    want = _oracle_conv(port, case)
+    direct = _gpu_conv(case, shim.ALGO_DIRECT)
+    mx, exact = lsb_diff(direct.data, want.data)
+    print(f"  direct: max|d|={mx} exact={exact:.5f}", flush=True)
+    assert mx <= 1 and exact >= 0.99
+    auto = _gpu_conv(case, shim.ALGO_AUTO)
+    np.testing.assert_array_equal(auto.data, direct.data)
+
+
+@pytest.mark.parametrize("case", FC, ids=[c.name for c in FC])
+def test_fc_cases(port, case):
+    print(f"case={case.name} x={case.x.info.shape} w={case.w.info.shape}", flush=True)
+    fn, a, b = case.act
+    want = port.fully_connected(case.x, case.w, case.b, case.out_info, transpose_weights=case.transpose_weights)
+    if fn:
+        want = port.activation(want, case.out_info, fn, a, b)
+    kw = dict(transpose_weights=case.transpose_weights, activation=fn, act_a=a, act_b=b)
+    direct = shim.fully_connected(case.x, case.w, case.b, case.out_info, algo=shim.ALGO_DIRECT, **kw)
+    mx, exact = lsb_diff(direct.data, want.data)
+    print(f"  direct: max|d|={mx} exact={exact:.5f}", flush=True)
+    assert mx <= 1 and exact >= 0.99
+    auto = shim.fully_connected(case.x, case.w, case.b, case.out_info, algo=shim.ALGO_AUTO, **kw)
+    np.testing.assert_array_equal(auto.data, direct.data)
+
+
+@pytest.mark.parametrize("case", [c for c in LIT["cases"] if c["params"].get("layout", "NHWC") == "NHWC"],
+                         ids=lambda c: c["name"])
+def test_reference_literals_on_gpu(case):
+    x, w, b = (tensor_from_json(case[k]) for k in ("input", "weights", "bias"))
+    exp = tensor_from_json(case["output"])
+    act = case.get("activation")
+    fn = {"ReLu": 1, "BoundedReLu": 2}[act["function"]] if act else 0
+    a, bb = (act["a"], act["b"]) if act else (0.0, 0.0)
+    if case["op"] == "conv2d":
+        p = {k: v for k, v in case["params"].items() if k != "layout"}
+        y = shim.conv2d(x, w, b, exp.info, activation=fn, act_a=a, act_b=bb, **p)
+    else:
+        y = shim.fully_connected(x, w, b, exp.info, transpose_weights=case["params"]["transpose_weights"])
+    mx, _ = lsb_diff(y.data, exp.data)
+    assert mx <= case["tolerance"]
+
+
+def test_algo_selection():
+    c = cases.make_conv_case("sel", 1, ci=16, co=16)
+    plan = shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params)
+    assert plan.algo()[0] == shim.ALGO_MFMA
+    c = cases.make_conv_case("sel", 1, ci=3, co=16)
+    assert shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()[0] == shim.ALGO_DIRECT
+    c = cases.make_conv_case("sel", 1, ci=16, depthwise=True)
+    assert shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()[0] == shim.ALGO_DEPTHWISE
+    with pytest.raises(shim.ShimError):
+        c = cases.make_conv_case("sel", 1, ci=3, co=16)
+        shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, algo=shim.ALGO_MFMA, **c.params)
+
+
+def test_config_c1_full_size(port):
+    """BASELINE config 1: 1x56x56x64 -> 64, 3x3 SAME, per-channel, ReLU6; expected code range [-128, -8]."""
+    c = cases.make_conv_case("C1", 20250101, h=56, w=56, ci=64, co=64, act=cases.RELU6)
+    want = _oracle_conv(port, c)
+    got = _gpu_conv(c, shim.ALGO_AUTO)
+    mx, exact = lsb_diff(got.data, want.data)
+    print(f"C1: max|d|={mx} exact={exact:.6f} range=[{got.data.min()},{got.data.max()}]", flush=True)
+    assert mx <= 1 and exact >= 0.999
+    assert got.data.min() == -128 and got.data.max() == -8
+    np.testing.assert_array_equal(_gpu_conv(c, shim.ALGO_DIRECT).data, got.data)
+
+
+def test_config_c2_block(port):
+    """BASELINE config 2: depthwise 3x3 + pointwise 32->64 on 1x112x112x32 QAsymmU8, ReLU6 after each."""
+    U8 = DataType.QAsymmU8
+    dw = cases.make_conv_case("C2dw", 20250102, h=112, w=112, ci=32, depthwise=True, in_dtype=U8, in_scale=0.0235,
+                              in_offset=128, out_scale=0.0235, out_offset=0, act=cases.RELU6, w_scale_range=(0.01, 0.05))
+    want1 = _oracle_conv(port, dw)
+    got1 = _gpu_conv(dw, shim.ALGO_AUTO)
+    mx, exact = lsb_diff(got1.data, want1.data)
+    print(f"C2 dw: max|d|={mx} exact={exact:.6f}", flush=True)
+    assert mx <= 1 and exact >= 0.999
+    pw = cases.make_conv_case("C2pw", 20250103, h=112, w=112, ci=32, co=64, kh=1, kw=1, in_dtype=U8, in_scale=0.0235,
+                              in_offset=0, out_scale=0.0235, out_offset=0, act=cases.RELU6)
+    pw.x.data = want1.data          # feed the oracle's intermediate so the two stages are judged independently
+    want2 = _oracle_conv(port, pw)
+    got2 = _gpu_conv(pw, shim.ALGO_AUTO)
+    mx, exact = lsb_diff(got2.data, want2.data)
+    print(f"C2 pw: max|d|={mx} exact={exact:.6f} max code={got2.data.max()}", flush=True)
+    assert mx <= 1 and exact >= 0.999
+
+
+@pytest.mark.parametrize("m", [1, 256])
+def test_config_c4_fc(port, m):
+    """BASELINE config 4: [M,4096] x [4096,4096] per-channel, fused requantize (output scale 1.0, zp 0)."""
+    c = cases.make_fc_case("C4", 20250104, m=m, k=4096, o=4096, in_offset=0, out_scale=1.0, out_offset=0)
+    want = port.fully_connected(c.x, c.w, c.b, c.out_info)
+    got = shim.fully_connected(c.x, c.w, c.b, c.out_info)
+    mx, exact = lsb_diff(got.data, want.data)
+    sat = float(((got.data == 127) | (got.data == -128)).mean())
+    print(f"C4 M={m}: max|d|={mx} exact={exact:.6f} saturated={sat:.4f}", flush=True)
+    assert mx <= 1 and exact >= 0.995 and sat < 0.05
