@@ -1,0 +1,144 @@
+"""Runs a nets.Network on the device through the C ABI: one plan per layer, all activations resident in HBM,
+the whole forward pass optionally captured into a HIP graph and replayed with one launch."""
+from __future__ import annotations
+
+import ctypes as C
+from typing import Dict, List, Optional
+
+import numpy as np
+
+from . import shim
+from .nets import Network
+from .tensor import QTensor, numpy_dtype
+
+
+class DeviceNetwork:
+    def __init__(self, net: Network, batch: int, algo_overrides: Optional[Dict[str, int]] = None, use_graph: bool = True):
+        self.net, self.batch = net, batch
+        self.dev = shim.Device()
+        self.lib = shim.load_library()
+        self.stream = self.dev.stream()
+        self.buffers: Dict[str, shim.DeviceBuffer] = {}
+        self.steps: List = []          # (layer, callable(stream))
+        self.plans = []
+        self.graph = None
+        self.use_graph = use_graph
+        algo_overrides = algo_overrides or {}
+
+        def buf(name):
+            if name not in self.buffers:
+                self.buffers[name] = shim.DeviceBuffer(net.info(name, batch).num_elements)
+            return self.buffers[name]
+
+        buf(net.input)
+        for l in net.layers:
+            xin = [net.info(i, batch) for i in l.inputs]
+            yout = net.info(l.output, batch)
+            if l.op == "reshape":
+                self.buffers[l.output] = self.buffers[l.inputs[0]]      # same bytes, new shape
+                continue
+            xb = [buf(i) for i in l.inputs]
+            yb = buf(l.output)
+            if l.op in ("conv", "depthwise"):
+                p = {k: v for k, v in l.params.items() if not k.startswith("_")}
+                plan = shim.Conv2dPlan(xin[0], l.weights, l.bias, yout, activation=l.act[0], act_a=l.act[1],
+                                       act_b=l.act[2], algo=algo_overrides.get(l.name, shim.ALGO_AUTO), **p)
+                self.plans.append(plan)
+                self.steps.append((l, self._conv_step(plan, xb[0].ptr, yb.ptr)))
+            elif l.op == "fc":
+                plan = shim.FullyConnectedPlan(xin[0], l.weights, l.bias, yout, transpose_weights=l.params["transpose_weights"],
+                                               activation=l.act[0], act_a=l.act[1], act_b=l.act[2],
+                                               algo=algo_overrides.get(l.name, shim.ALGO_AUTO))
+                self.plans.append(plan)
+                self.steps.append((l, self._conv_step(plan, xb[0].ptr, yb.ptr)))
+            elif l.op == "pool":
+                _, h, w, c = xin[0].shape
+                _, ho, wo, _ = yout.shape
+                p = l.params
+                d = shim.Pool2dDesc(h, w, c, ho, wo, p["pool_w"], p["pool_h"], p["stride_x"], p["stride_y"], p["pad_left"],
+                                    p["pad_right"], p["pad_top"], p["pad_bottom"], p["pool_type"], p["padding_method"],
+                                    shim._quant(xin[0]), shim._quant(yout))
+                self.steps.append((l, self._pool_step(d, xb[0].ptr, yb.ptr)))
+            elif l.op == "add":
+                q0, q1, qo = shim._quant(xin[0]), shim._quant(xin[1]), shim._quant(yout)
+                self.steps.append((l, self._add_step(yout.num_elements, q0, q1, qo, l.act, xb[0].ptr, xb[1].ptr, yb.ptr)))
+            elif l.op == "softmax":
+                rows, cols = yout.shape
+                qi, qo = shim._quant(xin[0]), shim._quant(yout)
+                self.steps.append((l, self._softmax_step(rows, cols, l.params["beta"], qi, qo, xb[0].ptr, yb.ptr)))
+            else:
+                raise ValueError(l.op)
+
+    # each step keeps its ctypes structs alive through the closure
+    def _conv_step(self, plan, x, y):
+        batch = self.batch
+        return lambda s: plan.run(batch, x, y, s)
+
+    def _pool_step(self, d, x, y):
+        batch, lib = self.batch, self.lib
+        return lambda s: shim._chk(lib.mi355x_pool2d_run(C.byref(d), batch, x, y, s))
+
+    def _add_step(self, n, q0, q1, qo, act, x0, x1, y):
+        lib = self.lib
+        return lambda s: shim._chk(lib.mi355x_add_run(n, C.byref(q0), C.byref(q1), C.byref(qo), act[0], act[1], act[2], x0, x1, y, s))
+
+    def _softmax_step(self, rows, cols, beta, qi, qo, x, y):
+        lib = self.lib
+        return lambda s: shim._chk(lib.mi355x_softmax_run(rows, cols, beta, C.byref(qi), C.byref(qo), x, y, s))
+
+    # ---------------------------------------------------------------------------------------------------------
+    def upload_input(self, x: QTensor):
+        assert x.info.shape == self.net.info(self.net.input, self.batch).shape
+        self.buffers[self.net.input].upload(x.data, self.stream)
+
+    def enqueue(self):
+        """One forward pass on self.stream (asynchronous)."""
+        if self.use_graph:
+            if self.graph is None:
+                self.dev.graph_begin(self.stream)
+                for _, fn in self.steps:
+                    fn(self.stream)
+                self.graph = self.dev.graph_end(self.stream)
+            self.dev.graph_launch(self.graph, self.stream)
+        else:
+            for _, fn in self.steps:
+                fn(self.stream)
+
+    def synchronize(self):
+        self.dev.stream_sync(self.stream)
+
+    def download(self, name: Optional[str] = None) -> QTensor:
+        name = name or self.net.output
+        info = self.net.info(name, self.batch)
+        self.synchronize()
+        return QTensor(info, self.buffers[name].download(info.shape, numpy_dtype(info.dtype), self.stream))
+
+    def run(self, x: QTensor) -> QTensor:
+        self.upload_input(x)
+        self.enqueue()
+        return self.download()
+
+    def time_layers(self, iters: int = 20, warmup: int = 3):
+        """Per-layer device time in ms (HIP events on the launch stream), eager launches."""
+        e0, e1 = self.dev.event(), self.dev.event()
+        out = []
+        for l, fn in self.steps:
+            for _ in range(warmup):
+                fn(self.stream)
+            self.dev.event_record(e0, self.stream)
+            for _ in range(iters):
+                fn(self.stream)
+            self.dev.event_record(e1, self.stream)
+            self.dev.event_sync(e1)
+            out.append((l, self.dev.elapsed_ms(e0, e1) / iters))
+        return out
+
+    def close(self):
+        if self.graph is not None:
+            self.dev.graph_destroy(self.graph)
+            self.graph = None
+        for p in self.plans:
+            p.destroy()
+        for b in set(self.buffers.values()):
+            b.free()
+        self.dev.stream_destroy(self.stream)

@@ -1,0 +1,58 @@
+"""Whole networks on the device vs the CPU checker (needs an MI355X)."""
+import numpy as np
+import pytest
+
+from armnn_amd import nets, shim
+from armnn_amd.executor import DeviceNetwork
+from armnn_amd.tensor import numpy_dtype
+from oracle import netref
+from tests.helpers import lsb_diff
+
+pytestmark = pytest.mark.gpu
+
+
+def _layerwise(port, net, batch):
+    """Each device layer is fed the checker's own input for that layer, so every layer is judged at <= 1 LSB
+    independently of drift upstream.  Returns the end-to-end device output as well."""
+    x = nets.synthetic_input(net, batch)
+    ref = netref.run_network(port, net, x, keep=True)
+    dn = DeviceNetwork(net, batch, use_graph=False)
+    worst = 0
+    for l, fn in dn.steps:
+        for name in l.inputs:
+            dn.buffers[name].upload(ref[name].data, dn.stream)
+        fn(dn.stream)
+        got = dn.download(l.output)
+        mx, exact = lsb_diff(got.data, ref[l.output].data)
+        print(f"{net.name} b{batch} {l.name:>10s} {l.op:>9s}: max|d|={mx} exact={exact:.6f}", flush=True)
+        assert mx <= 1, l.name
+        if l.op != "softmax":
+            assert exact >= 0.995, l.name
+        worst = max(worst, mx)
+    # end to end (drift allowed to accumulate): graph replay must equal eager launches bit for bit
+    eager = dn.run(x)
+    dn.close()
+    dg = DeviceNetwork(net, batch, use_graph=True)
+    g1 = dg.run(x)
+    dg.enqueue()
+    g2 = dg.download()
+    dg.close()
+    np.testing.assert_array_equal(g1.data, eager.data)
+    np.testing.assert_array_equal(g2.data, eager.data)
+    mx, exact = lsb_diff(eager.data, ref[net.output].data)
+    top1 = float((eager.data.argmax(-1) == ref[net.output].data.argmax(-1)).mean())
+    print(f"{net.name} b{batch} end-to-end: max|d|={mx} exact={exact:.6f} top1-agree={top1:.3f}", flush=True)
+    return worst
+
+
+def test_mobilenet_v1_batch2(port):
+    _layerwise(port, nets.mobilenet_v1(), 2)
+
+
+def test_mobilenet_v1_small_odd_resolution(port):
+    # odd spatial sizes exercise the SAME-padding edges of every stride-2 layer
+    _layerwise(port, nets.mobilenet_v1(resolution=97, classes=37), 3)
+
+
+def test_resnet50_batch1(port):
+    _layerwise(port, nets.resnet50(resolution=96), 1)
