@@ -49,8 +49,20 @@ struct Requant
     int32_t act_lo;         // fused activation clamp in the quantized domain (already within the type range)
     int32_t act_hi;
     int32_t out_is_u8;
+    // fast path: multiply by fl(1/scale) instead of dividing; exact division is redone only for values that land
+    // within kTieWindow of a rounding tie, so the result is bit-identical to the division everywhere
+    float   inv_scale;
+    float   act_lo_f, act_hi_f;
+    int32_t fast_ok;
 };
 
 Requant MakeRequant(const mi355x_quant& out, int32_t activation, float a, float b);
+
+// process-wide options set through mi355x_set_option()
+struct Options
+{
+    int exact_division_epilogue = 0;   // 1: every output takes the fp32 division (no reciprocal fast path)
+};
+Options& GlobalOptions();
 
 } // namespace mi355x

@@ -2,6 +2,7 @@
 // (constant re-layout, per-channel requantization constants, kernel selection) and launches.
 #include "common.h"
 #include "conv_kernels.h"
+#include "dw_stem_kernels.h"
 
 #include <cmath>
 #include <cstdlib>
@@ -19,6 +20,9 @@ struct mi355x_conv2d_s
     // device constants
     uint8_t* w_direct = nullptr;   // [Kh][Kw][Ci][Co] / depthwise [Kh][Kw][Co], raw codes
     int8_t*  w_mfma   = nullptr;   // [Co_pad][K_pad] signed, zero padded
+    uint32_t* w_dot4  = nullptr;   // depthwise 3x3: [C][4] dwords; small-Ci conv: [Co][Kh][RD] dwords
+    int variant = 0;               // kernel variant within an algo (see RunPlan)
+    int row_dwords = 0;            // small-Ci conv: dwords per filter row
     float*   mult     = nullptr;   // [Co_pad]  s_in * s_w[c]
     float*   biasf    = nullptr;   // [Co_pad]  float(bias[c]) * s_b[c]
     int32_t* corr     = nullptr;   // [Co_pad]  -zx' * sum_k w[c][k]
@@ -31,6 +35,7 @@ struct mi355x_conv2d_s
     {
         (void)hipFree(w_direct);
         (void)hipFree(w_mfma);
+        (void)hipFree(w_dot4);
         (void)hipFree(mult);
         (void)hipFree(biasf);
         (void)hipFree(corr);
@@ -142,13 +147,27 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     const bool mfma_ok = !d.depthwise && g.zw == 0 && !g.w_u8 && (Ci % 16) == 0 && zx_shift >= -128 && zx_shift <= 127 &&
                          p->K <= 100000;
     const bool dw_ok = d.depthwise && g.depth_mult == 1 && (Co % 4) == 0;
+    const bool sym_s8 = g.zw == 0 && !g.w_u8 && zx_shift >= -128 && zx_shift <= 127;
+    // depthwise 3x3 on v_dot4 with an LDS halo tile
+    const bool dw3_ok = dw_ok && sym_s8 && Kh == 3 && Kw == 3 && (Co % 32) == 0 && d.dilation_x == 1 && d.dilation_y == 1 &&
+                        d.stride_x == d.stride_y && (d.stride_x == 1 || d.stride_x == 2);
+    // stems: <= 4 input channels, rows of Kw*Ci bytes walked with v_dot4
+    const int row_bytes = Kw * Ci;
+    const bool stem_ok = !d.depthwise && sym_s8 && Ci <= 4 && (Co % 4) == 0 && d.dilation_x == 1 && d.dilation_y == 1 &&
+                         d.stride_x == d.stride_y && (d.stride_x == 1 || d.stride_x == 2) &&
+                         ((Kh == 3 && row_bytes <= 12) || (Kh == 7 && row_bytes <= 24) || (Kh == 1 && row_bytes <= 4) ||
+                          (Kh == 5 && row_bytes <= 20));
     int32_t algo = d.algo;
-    if (algo == MI355X_ALGO_AUTO) algo = mfma_ok ? MI355X_ALGO_MFMA : dw_ok ? MI355X_ALGO_DEPTHWISE : MI355X_ALGO_DIRECT;
+    if (algo == MI355X_ALGO_AUTO)
+        algo = mfma_ok ? MI355X_ALGO_MFMA : dw_ok ? MI355X_ALGO_DEPTHWISE : stem_ok ? MI355X_ALGO_DOT4 : MI355X_ALGO_DIRECT;
+    if (algo == MI355X_ALGO_DOT4 && !stem_ok)
+        return SetError(MI355X_ERR_UNSUPPORTED, "dot4 kernel needs <= 4 input channels, symmetric int8 weights, stride 1 or 2, "
+                                                "no dilation and a 1/3/5/7-row filter");
     if (algo == MI355X_ALGO_MFMA && !mfma_ok)
         return SetError(MI355X_ERR_UNSUPPORTED, "MFMA kernel needs a non-depthwise layer, symmetric int8 weights and in_c %% 16 == 0");
     if (algo == MI355X_ALGO_DEPTHWISE && !dw_ok)
         return SetError(MI355X_ERR_UNSUPPORTED, "depthwise kernel needs multiplier 1 and channels %% 4 == 0");
-    if (algo < MI355X_ALGO_DIRECT || algo > MI355X_ALGO_DEPTHWISE) return SetError(MI355X_ERR_INVALID_ARGUMENT, "unknown algo %d", algo);
+    if (algo < MI355X_ALGO_DIRECT || algo > MI355X_ALGO_DOT4) return SetError(MI355X_ERR_INVALID_ARGUMENT, "unknown algo %d", algo);
     p->algo = algo;
 
     const uint8_t* wsrc = static_cast<const uint8_t*>(weights_host);
@@ -175,10 +194,67 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 tile %dx%dx%d K=%d", p->bm, p->bn, kIgemmBK, p->K);
         p->info = buf;
     }
+    else if (algo == MI355X_ALGO_DEPTHWISE && dw3_ok)
+    {
+        // [1][3][3][C] -> per channel 4 dwords, dword r = { w[r][0], w[r][1], w[r][2], 0 }
+        const int8_t* ws = reinterpret_cast<const int8_t*>(wsrc);
+        std::vector<uint32_t> wp(static_cast<size_t>(Co) * 4, 0u);
+        std::vector<int32_t> corr(Co, 0);
+        for (int c = 0; c < Co; ++c)
+        {
+            long long sum = 0;
+            for (int r = 0; r < 3; ++r)
+            {
+                uint32_t dw = 0;
+                for (int kx = 0; kx < 3; ++kx)
+                {
+                    const int8_t v = ws[(r * 3 + kx) * Co + c];
+                    dw |= static_cast<uint32_t>(static_cast<uint8_t>(v)) << (8 * kx);
+                    sum += v;
+                }
+                wp[static_cast<size_t>(c) * 4 + r] = dw;
+            }
+            corr[c] = static_cast<int32_t>(-static_cast<long long>(zx_shift) * sum);
+        }
+        if (int rc = Upload(reinterpret_cast<void**>(&p->w_dot4), wp.data(), wp.size() * sizeof(uint32_t))) return rc;
+        if (int rc = Upload(reinterpret_cast<void**>(&p->corr), corr.data(), corr.size() * sizeof(int32_t))) return rc;
+        p->xor_mask = g.in_u8 ? 0x80808080u : 0u;
+        const uint32_t zb = static_cast<uint32_t>(zx_shift) & 0xffu;
+        p->pad_word = zb | (zb << 8) | (zb << 16) | (zb << 24);
+        p->variant = 1;
+        p->info = d.stride_x == 1 ? "depthwise3x3_dot4_lds stride 1, tile 8x16x32" : "depthwise3x3_dot4_lds stride 2, tile 8x8x32";
+    }
     else if (algo == MI355X_ALGO_DEPTHWISE)
     {
         if (int rc = Upload(reinterpret_cast<void**>(&p->w_direct), wsrc, static_cast<size_t>(Kh) * Kw * Co)) return rc;
         p->info = "depthwise_c4_valu";
+    }
+    else if (algo == MI355X_ALGO_DOT4)
+    {
+        const int RD = Kh == 3 ? 3 : Kh == 7 ? 6 : Kh == 5 ? 5 : 1;
+        const int8_t* ws = reinterpret_cast<const int8_t*>(wsrc);
+        std::vector<uint32_t> wp(static_cast<size_t>(Co) * Kh * RD, 0u);
+        std::vector<int32_t> corr(Co, 0);
+        for (int c = 0; c < Co; ++c)
+        {
+            long long sum = 0;
+            for (int r = 0; r < Kh; ++r)
+                for (int bidx = 0; bidx < row_bytes; ++bidx)
+                {
+                    const int8_t v = ws[(static_cast<size_t>(c) * Kh + r) * row_bytes + bidx];
+                    wp[(static_cast<size_t>(c) * Kh + r) * RD + bidx / 4] |= static_cast<uint32_t>(static_cast<uint8_t>(v)) << (8 * (bidx % 4));
+                    sum += v;
+                }
+            corr[c] = static_cast<int32_t>(-static_cast<long long>(zx_shift) * sum);
+        }
+        if (int rc = Upload(reinterpret_cast<void**>(&p->w_dot4), wp.data(), wp.size() * sizeof(uint32_t))) return rc;
+        if (int rc = Upload(reinterpret_cast<void**>(&p->corr), corr.data(), corr.size() * sizeof(int32_t))) return rc;
+        p->xor_mask = g.in_u8 ? 0x80u : 0u;
+        p->pad_word = static_cast<uint32_t>(zx_shift) & 0xffu;
+        p->row_dwords = RD;
+        char buf[96];
+        snprintf(buf, sizeof(buf), "smallci_dot4_lds %dx%dx%d stride %u, tile 16x16", Kh, Kw, Ci, d.stride_x);
+        p->info = buf;
     }
     else
     {
@@ -247,8 +323,47 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             return SetError(MI355X_ERR_INVALID_ARGUMENT, "MFMA kernel needs 16-byte aligned tensors");
         if (p->bn == 64) return LaunchIgemm<128, 64, 2, 2>(p, batch, x, y, stream);
         return LaunchIgemm<128, 128, 2, 2>(p, batch, x, y, stream);
+    case MI355X_ALGO_DOT4:
+    {
+        if ((reinterpret_cast<uintptr_t>(y) & 3) != 0) return SetError(MI355X_ERR_INVALID_ARGUMENT, "dot4 kernel needs a 4-byte aligned output");
+        SmallCiArgs a;
+        a.x = xin; a.wpack = p->w_dot4; a.mult = p->mult; a.biasf = p->biasf; a.corr = p->corr; a.y = yout;
+        a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.Ci = g.Ci; a.Ho = g.Ho; a.Wo = g.Wo; a.Co = g.Co;
+        a.Kw = g.Kw; a.stride = g.stride_x; a.pad_top = g.pad_top; a.pad_left = g.pad_left;
+        a.tiles_x = (g.Wo + 15) / 16; a.tiles_y = (g.Ho + 15) / 16;
+        a.xor_mask = p->xor_mask; a.pad_byte = p->pad_word;
+        a.ci_recip = (65536u + static_cast<uint32_t>(g.Ci) - 1u) / static_cast<uint32_t>(g.Ci);
+        a.rq = p->rq;
+        const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
+        if (nb > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
+        const dim3 grid(static_cast<unsigned>(nb));
+        if (g.Kh == 3) hipLaunchKernelGGL((SmallCiConvKernel<3, 3>), grid, dim3(256), 0, stream, a);
+        else if (g.Kh == 7) hipLaunchKernelGGL((SmallCiConvKernel<7, 6>), grid, dim3(256), 0, stream, a);
+        else if (g.Kh == 5) hipLaunchKernelGGL((SmallCiConvKernel<5, 5>), grid, dim3(256), 0, stream, a);
+        else hipLaunchKernelGGL((SmallCiConvKernel<1, 1>), grid, dim3(256), 0, stream, a);
+        MI355X_HIP(hipGetLastError());
+        return 0;
+    }
     case MI355X_ALGO_DEPTHWISE:
     {
+        if (p->variant == 1)
+        {
+            if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 3) != 0)
+                return SetError(MI355X_ERR_INVALID_ARGUMENT, "depthwise 3x3 kernel needs a 16-byte aligned input and 4-byte aligned output");
+            Dw3x3Args a;
+            a.x = xin; a.wpack = p->w_dot4; a.mult = p->mult; a.biasf = p->biasf; a.corr = p->corr; a.y = yout;
+            a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.C = g.Co; a.Ho = g.Ho; a.Wo = g.Wo;
+            a.pad_top = g.pad_top; a.pad_left = g.pad_left;
+            const int tw = g.stride_x == 1 ? 16 : 8;
+            a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + 7) / 8; a.cblocks = g.Co / 32;
+            a.xor_mask = p->xor_mask; a.pad_word = p->pad_word; a.rq = p->rq;
+            const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y * a.cblocks;
+            if (nb > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
+            if (g.stride_x == 1) hipLaunchKernelGGL((Depthwise3x3Kernel<1>), dim3(static_cast<unsigned>(nb)), dim3(256), 0, stream, a);
+            else hipLaunchKernelGGL((Depthwise3x3Kernel<2>), dim3(static_cast<unsigned>(nb)), dim3(256), 0, stream, a);
+            MI355X_HIP(hipGetLastError());
+            return 0;
+        }
         if ((reinterpret_cast<uintptr_t>(x) & 3) != 0 || (reinterpret_cast<uintptr_t>(y) & 3) != 0)
             return SetError(MI355X_ERR_INVALID_ARGUMENT, "depthwise kernel needs 4-byte aligned tensors");
         const long long total4 = total / 4;

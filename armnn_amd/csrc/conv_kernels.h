@@ -39,14 +39,16 @@ __global__ __launch_bounds__(256) void ConvDirectKernel(ConvGeom g, Requant rq, 
                                                         const float* __restrict__ biasf, uint8_t* __restrict__ y,
                                                         long long total)
 {
-    long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+    const long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
     if (idx >= total) return;
-    const int co = static_cast<int>(idx % g.Co);
-    long long pix = idx / g.Co;
-    const int ox = static_cast<int>(pix % g.Wo);
-    pix /= g.Wo;
-    const int oy = static_cast<int>(pix % g.Ho);
-    const long long n = pix / g.Ho;
+    // one 64-bit division to split off the batch index, 32-bit arithmetic below it
+    const unsigned per_image = static_cast<unsigned>(g.Ho) * g.Wo * g.Co;
+    const long long n = idx / per_image;
+    unsigned rem = static_cast<unsigned>(idx - n * per_image);
+    const int co = static_cast<int>(rem % g.Co);
+    rem /= g.Co;
+    const int ox = static_cast<int>(rem % g.Wo);
+    const int oy = static_cast<int>(rem / g.Wo);
 
     const uint8_t* xn = x + n * g.H * g.W * g.Ci;
     int acc = 0;
@@ -107,15 +109,16 @@ __global__ __launch_bounds__(256) void DepthwiseC4Kernel(ConvGeom g, Requant rq,
                                                          const float* __restrict__ biasf,
                                                          uint8_t* __restrict__ y, long long total_c4)
 {
-    long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+    const long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
     if (idx >= total_c4) return;
-    const int C4 = g.Co >> 2;
-    const int c = static_cast<int>(idx % C4) * 4;
-    long long pix = idx / C4;
-    const int ox = static_cast<int>(pix % g.Wo);
-    pix /= g.Wo;
-    const int oy = static_cast<int>(pix % g.Ho);
-    const long long n = pix / g.Ho;
+    const unsigned C4 = static_cast<unsigned>(g.Co) >> 2;
+    const unsigned per_image = static_cast<unsigned>(g.Ho) * g.Wo * C4;
+    const long long n = idx / per_image;
+    unsigned rem = static_cast<unsigned>(idx - n * per_image);
+    const int c = static_cast<int>(rem % C4) * 4;
+    rem /= C4;
+    const int ox = static_cast<int>(rem % g.Wo);
+    const int oy = static_cast<int>(rem / g.Wo);
 
     const uint8_t* xn = x + n * g.H * g.W * g.Ci + c;
     int acc[4] = {0, 0, 0, 0};
@@ -134,11 +137,9 @@ __global__ __launch_bounds__(256) void DepthwiseC4Kernel(ConvGeom g, Requant rq,
     }
     const float4 m4 = *reinterpret_cast<const float4*>(mult + c);
     const float4 b4 = *reinterpret_cast<const float4*>(biasf + c);
-    uint32_t out = static_cast<uint32_t>(RequantDev(acc[0], m4.x, b4.x, rq) & 0xff);
-    out |= static_cast<uint32_t>(RequantDev(acc[1], m4.y, b4.y, rq) & 0xff) << 8;
-    out |= static_cast<uint32_t>(RequantDev(acc[2], m4.z, b4.z, rq) & 0xff) << 16;
-    out |= static_cast<uint32_t>(RequantDev(acc[3], m4.w, b4.w, rq) & 0xff) << 24;
-    *reinterpret_cast<uint32_t*>(y + idx * 4) = out;
+    *reinterpret_cast<uint32_t*>(y + idx * 4) =
+        Pack4(RequantDev(acc[0], m4.x, b4.x, rq), RequantDev(acc[1], m4.y, b4.y, rq), RequantDev(acc[2], m4.z, b4.z, rq),
+              RequantDev(acc[3], m4.w, b4.w, rq));
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -375,10 +376,8 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
             for (int tp = 0; tp < TP; ++tp)
             {
                 const v16i& c = acc[tc][tp];
-                uint32_t out = static_cast<uint32_t>(RequantDev(c[4 * q + 0], m4.x, b4.x, a.rq) & 0xff);
-                out |= static_cast<uint32_t>(RequantDev(c[4 * q + 1], m4.y, b4.y, a.rq) & 0xff) << 8;
-                out |= static_cast<uint32_t>(RequantDev(c[4 * q + 2], m4.z, b4.z, a.rq) & 0xff) << 16;
-                out |= static_cast<uint32_t>(RequantDev(c[4 * q + 3], m4.w, b4.w, a.rq) & 0xff) << 24;
+                const uint32_t out = Pack4(RequantDev(c[4 * q + 0], m4.x, b4.x, a.rq), RequantDev(c[4 * q + 1], m4.y, b4.y, a.rq),
+                                           RequantDev(c[4 * q + 2], m4.z, b4.z, a.rq), RequantDev(c[4 * q + 3], m4.w, b4.w, a.rq));
                 const int pl = wm * WTM + tp * 32 + (lane & 31);          // pixel within the block tile
                 *reinterpret_cast<uint32_t*>(Os + pl * LDO + cl) = out;
             }

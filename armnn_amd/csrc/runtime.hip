@@ -22,6 +22,12 @@ int SetError(int code, const char* fmt, ...)
     return code;
 }
 
+Options& GlobalOptions()
+{
+    static Options o;
+    return o;
+}
+
 int32_t QuantizeHost(float value, float scale, int32_t offset, int32_t dtype)
 {
     const float lo = dtype == MI355X_QASYMM_U8 ? 0.0f : -128.0f;
@@ -60,6 +66,13 @@ Requant MakeRequant(const mi355x_quant& out, int32_t activation, float a, float 
     rq.type_max_f   = out.dtype == MI355X_QASYMM_U8 ? 255.0f : 127.0f;
     rq.out_is_u8    = out.dtype == MI355X_QASYMM_U8;
     ActivationClamp(activation, a, b, out, &rq.act_lo, &rq.act_hi);
+    rq.inv_scale = 1.0f / out.scale;
+    rq.act_lo_f  = static_cast<float>(rq.act_lo);
+    rq.act_hi_f  = static_cast<float>(rq.act_hi);
+    // The tie window argument needs |offset| <= 255 (so that |value/scale| > 512 always clamps) and a normal,
+    // finite reciprocal.
+    rq.fast_ok = !GlobalOptions().exact_division_epilogue && std::isnormal(rq.inv_scale) && std::isnormal(out.scale) && out.offset >= -255 && out.offset <= 255 &&
+                 rq.act_lo <= rq.act_hi;
     return rq;
 }
 
@@ -79,6 +92,13 @@ extern "C" {
 const char* mi355x_last_error(void) { return ErrorBuffer(); }
 
 int mi355x_abi_version(void) { return MI355X_ABI_VERSION; }
+
+int mi355x_set_option(const char* name, int value)
+{
+    if (!name) return SetError(MI355X_ERR_INVALID_ARGUMENT, "option name is null");
+    if (std::strcmp(name, "exact_division_epilogue") == 0) { GlobalOptions().exact_division_epilogue = value != 0; return 0; }
+    return SetError(MI355X_ERR_INVALID_ARGUMENT, "unknown option '%s'", name);
+}
 
 int mi355x_device_count(int* count)
 {

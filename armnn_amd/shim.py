@@ -16,12 +16,12 @@ from .tensor import DataType, QTensor, TensorInfo, numpy_dtype
 _HERE = os.path.dirname(os.path.abspath(__file__))
 LIB_PATH = os.path.join(_HERE, "lib", "libarmnn_mi355x.so")
 
-ALGO_AUTO, ALGO_DIRECT, ALGO_MFMA, ALGO_DEPTHWISE = 0, 1, 2, 3
+ALGO_AUTO, ALGO_DIRECT, ALGO_MFMA, ALGO_DEPTHWISE, ALGO_DOT4 = 0, 1, 2, 3, 4
 ACT_NONE, ACT_RELU, ACT_BOUNDED_RELU = 0, 1, 2
 
 #: every symbol include/armnn_mi355x.h declares
 EXPORTS = [
-    "mi355x_last_error", "mi355x_abi_version", "mi355x_device_count", "mi355x_init", "mi355x_device_name",
+    "mi355x_last_error", "mi355x_abi_version", "mi355x_set_option", "mi355x_device_count", "mi355x_init", "mi355x_device_name",
     "mi355x_device_props", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc", "mi355x_host_free",
     "mi355x_memcpy_h2d", "mi355x_memcpy_d2h", "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_synchronize", "mi355x_device_synchronize", "mi355x_event_create",
@@ -110,6 +110,7 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
                                C.c_float, V, V, V, V],
             "mi355x_softmax_run": [C.c_uint32, C.c_uint32, C.c_float, C.POINTER(Quant), C.POINTER(Quant), V, V, V],
             "mi355x_device_count": [C.POINTER(C.c_int)], "mi355x_init": [C.c_int],
+            "mi355x_set_option": [C.c_char_p, C.c_int],
             "mi355x_device_name": [C.c_char_p, C.c_size_t],
             "mi355x_device_props": [C.POINTER(C.c_int), C.POINTER(C.c_int), C.POINTER(C.c_size_t), C.POINTER(C.c_size_t)],
         }
@@ -127,6 +128,10 @@ def _chk(rc):
 
 def _quant(info: TensorInfo) -> Quant:
     return Quant(int(info.dtype), float(np.float32(info.scale)), int(info.offset))
+
+
+def set_option(name: str, value: int):
+    _chk(load_library().mi355x_set_option(name.encode(), int(value)))
 
 
 class DeviceBuffer:

@@ -59,7 +59,8 @@ typedef enum {
     MI355X_ALGO_AUTO      = 0,
     MI355X_ALGO_DIRECT    = 1,   /* one thread per output element; accepts every supported configuration      */
     MI355X_ALGO_MFMA      = 2,   /* implicit-GEMM on v_mfma_i32_32x32x32_i8 (conv / FC; symmetric int8 weights) */
-    MI355X_ALGO_DEPTHWISE = 3    /* channel-vectorised VALU kernel (depthwise, multiplier 1)                   */
+    MI355X_ALGO_DEPTHWISE = 3,   /* channel-vectorised VALU kernels (depthwise, multiplier 1); 3x3 uses v_dot4 + LDS halo */
+    MI355X_ALGO_DOT4      = 4    /* v_dot4 kernel with an LDS halo tile for layers with <= 4 input channels (stems) */
 } mi355x_algo;
 
 typedef struct mi355x_stream_s* mi355x_stream_t;   /* NULL = the default stream */
@@ -91,6 +92,11 @@ typedef struct {
  * ---------------------------------------------------------------------------------------------------- */
 const char* mi355x_last_error(void);
 int  mi355x_abi_version(void);
+/* Process-wide switches, read when a plan or a layer call is set up.
+ *   "exact_division_epilogue" = 1: requantize every output with the fp32 division of armnn::Quantize
+ *   (src/armnn/TypesUtils.cpp:40) instead of the reciprocal fast path that falls back to the division near
+ *   rounding ties.  Both give identical bytes; the switch exists so that tests can prove it. */
+int  mi355x_set_option(const char* name, int value);
 int  mi355x_device_count(int* count);                 /* 0 devices is success with *count == 0 */
 int  mi355x_init(int device);                         /* select + warm up the device; idempotent */
 int  mi355x_device_name(char* buf, size_t buf_len);   /* e.g. "gfx950:sramecc+:xnack-" */

@@ -168,6 +168,25 @@ def small_conv_cases():
     c.append(make_conv_case("dw_s8_per_tensor", 204, ci=8, depthwise=True, per_axis=False, w_scale_range=(0.01, 0.05)))
     c.append(make_conv_case("dw_s8_dilated", 205, h=12, w=12, ci=8, depthwise=True, dilation=(2, 2),
                             w_scale_range=(0.01, 0.05)))
+    # the v_dot4 + LDS-halo depthwise kernel (channels % 32 == 0, 3x3, stride 1/2) incl. ragged tile edges
+    c.append(make_conv_case("dw3_u8_c32_s1", 210, h=19, w=21, ci=32, depthwise=True, in_dtype=U8, in_scale=0.0235, in_offset=128,
+                            out_scale=0.0235, out_offset=0, act=RELU6, w_scale_range=(0.01, 0.05)))
+    c.append(make_conv_case("dw3_u8_c64_s2_even", 211, n=2, h=20, w=18, ci=64, depthwise=True, stride=(2, 2), in_dtype=U8,
+                            in_scale=0.0235, in_offset=3, out_scale=0.0235, out_offset=0, act=RELU6, w_scale_range=(0.01, 0.05)))
+    c.append(make_conv_case("dw3_s8_c32_s2_odd", 212, h=17, w=23, ci=32, depthwise=True, stride=(2, 2),
+                            w_scale_range=(0.01, 0.05)))
+    c.append(make_conv_case("dw3_s8_c96_s1_valid", 213, h=9, w=37, ci=96, depthwise=True, padding="valid",
+                            w_scale_range=(0.01, 0.05)))
+    c.append(make_conv_case("dw3_s8_c32_pad2", 214, h=10, w=10, ci=32, depthwise=True, padding=(2, 2, 2, 2),
+                            w_scale_range=(0.01, 0.05)))
+    # stems on the small-Ci v_dot4 kernel
+    c.append(make_conv_case("stem_u8_3x3_s2_224", 220, n=2, h=47, w=45, ci=3, co=32, stride=(2, 2), in_dtype=U8, in_offset=128,
+                            in_scale=0.0078, out_scale=0.0235, out_offset=0, act=RELU6, w_scale_range=(0.005, 0.02)))
+    c.append(make_conv_case("stem_s8_7x7_s2", 221, h=45, w=50, ci=3, co=64, kh=7, kw=7, stride=(2, 2), in_scale=0.0078,
+                            in_offset=0, act=RELU, w_scale_range=(0.002, 0.008)))
+    c.append(make_conv_case("stem_s8_3x3_s1_ci1", 222, h=20, w=33, ci=1, co=8, in_offset=-100))
+    c.append(make_conv_case("stem_s8_5x5_ci4", 223, h=21, w=18, ci=4, co=12, kh=5, kw=5, padding=(1, 2, 0, 3)))
+    c.append(make_conv_case("stem_s8_1x1_ci4", 224, h=9, w=9, ci=4, co=16, kh=1, kw=1))
     c.append(make_conv_case("dw_u8_5x5_c20", 206, h=9, w=9, ci=20, depthwise=True, kh=5, kw=5, in_dtype=U8,
                             in_offset=100, out_offset=3, w_scale_range=(0.005, 0.02)))
     return c

@@ -81,12 +81,40 @@ def test_algo_selection():
     plan = shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params)
     assert plan.algo()[0] == shim.ALGO_MFMA
     c = cases.make_conv_case("sel", 1, ci=3, co=16)
+    assert shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()[0] == shim.ALGO_DOT4
+    c = cases.make_conv_case("sel", 1, ci=3, co=15)
     assert shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()[0] == shim.ALGO_DIRECT
     c = cases.make_conv_case("sel", 1, ci=16, depthwise=True)
-    assert shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()[0] == shim.ALGO_DEPTHWISE
+    a, info = shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()
+    assert a == shim.ALGO_DEPTHWISE and "c4" in info
+    c = cases.make_conv_case("sel", 1, ci=64, depthwise=True)
+    a, info = shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()
+    assert a == shim.ALGO_DEPTHWISE and "dot4" in info
     with pytest.raises(shim.ShimError):
         c = cases.make_conv_case("sel", 1, ci=3, co=16)
         shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, algo=shim.ALGO_MFMA, **c.params)
+
+
+def test_fast_epilogue_equals_exact_division():
+    """The reciprocal fast path (with its fallback near rounding ties) must give the same bytes as dividing every
+    output, on tensors large enough to hit many near-tie values."""
+    cs = [cases.make_conv_case("epi_conv", 501, n=4, h=56, w=56, ci=32, co=64, kh=1, kw=1, in_dtype=cases.U8, in_scale=0.0235,
+                               in_offset=0, out_scale=0.0235, out_offset=0, act=cases.RELU6),
+          cases.make_conv_case("epi_conv_s8", 502, n=2, h=40, w=40, ci=16, co=32, out_scale=0.11, out_offset=17),
+          cases.make_conv_case("epi_dw", 503, n=4, h=56, w=56, ci=64, depthwise=True, in_dtype=cases.U8, in_scale=0.0235,
+                               in_offset=128, out_scale=0.0235, out_offset=0, act=cases.RELU6, w_scale_range=(0.01, 0.05)),
+          cases.make_conv_case("epi_stem", 504, n=4, h=64, w=64, ci=3, co=32, stride=(2, 2), in_dtype=cases.U8,
+                               in_scale=0.0078, in_offset=128, out_scale=0.0235, out_offset=0, act=cases.RELU6,
+                               w_scale_range=(0.005, 0.02))]
+    fast = [_gpu_conv(c, shim.ALGO_AUTO) for c in cs]
+    shim.set_option("exact_division_epilogue", 1)
+    try:
+        exact = [_gpu_conv(c, shim.ALGO_AUTO) for c in cs]
+    finally:
+        shim.set_option("exact_division_epilogue", 0)
+    for c, f, e in zip(cs, fast, exact):
+        print(f"{c.name}: {f.data.size} outputs, distinct codes {len(np.unique(f.data))}", flush=True)
+        np.testing.assert_array_equal(f.data, e.data)
 
 
 def test_config_c1_full_size(port):
