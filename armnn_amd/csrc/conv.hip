@@ -3,6 +3,7 @@
 #include "common.h"
 #include "conv_kernels.h"
 #include "dw_stem_kernels.h"
+#include "pw_gemm_kernel.h"
 
 #include <cmath>
 #include <cstdlib>
@@ -23,11 +24,12 @@ struct mi355x_conv2d_s
     uint32_t* w_dot4  = nullptr;   // depthwise 3x3: [C][4] dwords; small-Ci conv: [Co][Kh][RD] dwords
     int variant = 0;               // kernel variant within an algo (see RunPlan)
     int row_dwords = 0;            // small-Ci conv: dwords per filter row
-    float*   mult     = nullptr;   // [Co_pad]  s_in * s_w[c]
-    float*   biasf    = nullptr;   // [Co_pad]  float(bias[c]) * s_b[c]
+    float*   chan     = nullptr;   // [5][Co_pad] per-channel requantization constants (rows: see ChanTab)
     int32_t* corr     = nullptr;   // [Co_pad]  -zx' * sum_k w[c][k]
     int K = 0, K_pad = 0, Co_pad = 0;
-    int bm = 0, bn = 0;
+    std::vector<float> chan_host;  // host copy, completed with the corr-folded rows once corr is known
+    int pw_bn = 0, pw_ks = 0;      // pointwise GEMM kernel configuration (0: not applicable)
+    int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 128: force (MI355X_IGEMM_TILE, for experiments)
     uint32_t xor_mask = 0, pad_word = 0;
     std::string info;
 
@@ -36,8 +38,7 @@ struct mi355x_conv2d_s
         (void)hipFree(w_direct);
         (void)hipFree(w_mfma);
         (void)hipFree(w_dot4);
-        (void)hipFree(mult);
-        (void)hipFree(biasf);
+        (void)hipFree(chan);
         (void)hipFree(corr);
     }
 };
@@ -50,6 +51,9 @@ struct mi355x_fc_s
 
 namespace
 {
+
+void FoldCorrIntoTable(mi355x_conv2d_s* p, const std::vector<int32_t>& corr, int Co);
+void ChoosePointwiseConfig(mi355x_conv2d_s* p);
 
 int Upload(void** dst, const void* src, size_t bytes)
 {
@@ -139,8 +143,37 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             }
         }
     }
-    if (int rc = Upload(reinterpret_cast<void**>(&p->mult), mult.data(), mult.size() * sizeof(float))) return rc;
-    if (int rc = Upload(reinterpret_cast<void**>(&p->biasf), biasf.data(), biasf.size() * sizeof(float))) return rc;
+    // fast-path coefficients: r' = fma(float(acc), fm, fb) ~ f / s_out + offset, with the per-channel tie window
+    // inside which the value is recomputed exactly (device_math.h).  thr = -1 sends every value to the exact path.
+    {
+        const int CP = p->Co_pad;
+        std::vector<float> tab(static_cast<size_t>(7) * CP, 0.0f);
+        const float inv = 1.0f / d.output.scale;
+        const float zp_f = static_cast<float>(d.output.offset);
+        const double max_acc = static_cast<double>(p->K) * 65025.0;
+        const bool base_ok = !GlobalOptions().exact_division_epilogue && std::isnormal(inv) && std::isnormal(d.output.scale) &&
+                             d.output.offset >= -255 && d.output.offset <= 255;
+        for (int c = 0; c < CP; ++c)
+        {
+            tab[c] = mult[c];
+            tab[CP + c] = biasf[c];
+            tab[4 * CP + c] = -1.0f;
+            tab[6 * CP + c] = -1.0f;
+            if (c >= Co || !base_ok) continue;
+            const float fm = mult[c] * inv;
+            const float fb = biasf[c] * inv + zp_f;
+            const float bq = std::fabs(biasf[c]) * inv;
+            // |r' - (reference quotient + offset)| <= 2^-24 * (5400 + 7 |biasf/s_out|) for in-range results; 1.5x margin
+            const float win = (8192.0f + 11.0f * bq) * (1.0f / 16777216.0f);
+            const bool ok = std::isfinite(fm) && std::isfinite(fb) && std::isfinite(win) && win < 0.25f &&
+                            max_acc * std::fabs(static_cast<double>(fm)) < 268435456.0;
+            if (!ok) continue;
+            tab[2 * CP + c] = fm;
+            tab[3 * CP + c] = fb;
+            tab[4 * CP + c] = 0.5f - win;
+        }
+        p->chan_host = tab;
+    }
 
     // ---- kernel selection ----------------------------------------------------------------------------------
     const int zx_shift = g.in_u8 ? g.zx - 128 : g.zx;
@@ -188,10 +221,15 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         p->xor_mask = g.in_u8 ? 0x80808080u : 0u;
         const uint32_t zb = static_cast<uint32_t>(zx_shift) & 0xffu;
         p->pad_word = zb | (zb << 8) | (zb << 16) | (zb << 24);
-        p->bm = 128;
-        p->bn = (Co <= 64) ? 64 : 128;
-        char buf[96];
-        snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 tile %dx%dx%d K=%d", p->bm, p->bn, kIgemmBK, p->K);
+        if (const char* t = std::getenv("MI355X_IGEMM_TILE")) p->tile_override = std::atoi(t);
+        FoldCorrIntoTable(p, corr, Co);
+        ChoosePointwiseConfig(p);
+        if (p->tile_override != 0) p->pw_bn = 0;     // experiments: force the LDS-tiled implicit GEMM
+        char buf[128];
+        if (p->pw_bn)
+            snprintf(buf, sizeof(buf), "pointwise_gemm_mfma_i8_32x32x32 weight-stationary slab %dxK=%d, chunk %d k-steps", p->pw_bn, p->K, p->pw_ks);
+        else
+            snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 tiles 128x128|128x64|64x64 x%d K=%d", kIgemmBK, p->K);
         p->info = buf;
     }
     else if (algo == MI355X_ALGO_DEPTHWISE && dw3_ok)
@@ -273,7 +311,98 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         }
         p->info = d.depthwise ? "direct_depthwise" : "direct_conv";
     }
+    if (int rc = Upload(reinterpret_cast<void**>(&p->chan), p->chan_host.data(), p->chan_host.size() * sizeof(float))) return rc;
+    p->chan_host.clear();
+    p->chan_host.shrink_to_fit();
     return 0;
+}
+
+// Rows 5/6 of the channel table: the fast-path constants with the zero-point correction folded in,
+//   fb' = fb + corr * fm,   window' = 2^-24 * (8192 + 11 (|biasf/s_out| + |corr * fm|))
+// (the accumulator then starts at zero and only the rare exact path adds corr as an integer).
+void FoldCorrIntoTable(mi355x_conv2d_s* p, const std::vector<int32_t>& corr, int Co)
+{
+    const int CP = p->Co_pad;
+    std::vector<float>& tab = p->chan_host;
+    for (int c = 0; c < Co; ++c)
+    {
+        if (tab[4 * CP + c] < 0.0f) continue;         // fast path disabled for this channel
+        const float fm = tab[2 * CP + c];
+        const float cq = static_cast<float>(corr[c]) * fm;
+        const float fbc = tab[3 * CP + c] + cq;
+        const float win = (0.5f - tab[4 * CP + c]) + 11.0f * std::fabs(cq) * (1.0f / 16777216.0f);
+        if (!std::isfinite(fbc) || !(win < 0.25f) || std::fabs(static_cast<double>(corr[c])) >= 16777216.0) continue;
+        tab[5 * CP + c] = fbc;
+        tab[6 * CP + c] = 0.5f - win;
+    }
+}
+
+// Configuration of the weight-stationary pointwise GEMM kernel, or bn == 0 when it does not apply.
+void ChoosePointwiseConfig(mi355x_conv2d_s* p)
+{
+    const mi355x_conv2d_desc& d = p->d;
+    p->pw_bn = 0;
+    const bool pointwise = !d.depthwise && d.kernel_h == 1 && d.kernel_w == 1 && d.stride_x == 1 && d.stride_y == 1 &&
+                           d.pad_top == 0 && d.pad_left == 0 && d.out_h == d.in_h && d.out_w == d.in_w;
+    const int K = static_cast<int>(d.in_c), N = static_cast<int>(d.out_c);
+    if (!pointwise || (K % 32) != 0) return;
+    const int budget = 80 * 1024;
+    int bn = 0;
+    if (N > 64 && PwSmemBytes<128>(K) <= budget) bn = 128;
+    else if (N > 32 && PwSmemBytes<64>(K) <= budget) bn = 64;
+    else if (PwSmemBytes<32>(K) <= budget) bn = 32;
+    if (bn == 0) return;
+    const int steps = K / 32;
+    p->pw_bn = bn;
+    p->pw_ks = (steps % 8) == 0 ? 8 : (steps % 4) == 0 ? 4 : (steps % 2) == 0 ? 2 : 1;
+}
+
+template <int BN, int KS>
+int LaunchPw(const mi355x_conv2d_s* p, long long M, const void* x, void* y, hipStream_t stream)
+{
+    const ConvGeom& g = p->geom;
+    PwArgs a;
+    a.x = static_cast<const uint8_t*>(x);
+    a.w = p->w_mfma;
+    a.ct = ChanTab{p->chan, p->Co_pad};
+    a.corr = p->corr;
+    a.y = static_cast<uint8_t*>(y);
+    a.M = static_cast<int>(M);
+    a.K = g.Ci;
+    a.N = g.Co;
+    a.w_stride = p->K_pad;
+    a.n_slabs = (g.Co + BN - 1) / BN;
+    a.xor_mask = p->xor_mask;
+    a.rq = p->rq;
+    const int smem = PwSmemBytes<BN>(g.Ci);
+    const int per_cu = std::max(1, std::min(4, (160 * 1024) / smem));
+    const long long groups = ((M + 31) / 32 + 3) / 4;
+    long long gm = (256ll * per_cu) / a.n_slabs;
+    if (gm < 1) gm = 1;
+    if (gm > groups) gm = groups;
+    a.gm = static_cast<int>(gm);
+    auto kernel = PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2)>;
+    static bool attr_set = false;       // one flag per instantiation
+    if (!attr_set)
+    {
+        MI355X_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+        attr_set = true;
+    }
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(a.n_slabs * gm)), dim3(256), smem, stream, a);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+template <int BN>
+int LaunchPwKs(const mi355x_conv2d_s* p, long long M, const void* x, void* y, hipStream_t stream)
+{
+    switch (p->pw_ks)
+    {
+    case 8: return LaunchPw<BN, 8>(p, M, x, y, stream);
+    case 4: return LaunchPw<BN, 4>(p, M, x, y, stream);
+    case 2: return LaunchPw<BN, 2>(p, M, x, y, stream);
+    default: return LaunchPw<BN, 1>(p, M, x, y, stream);
+    }
 }
 
 template <int BM, int BN, int WM, int WN>
@@ -283,8 +412,7 @@ int LaunchIgemm(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y
     IgemmArgs a;
     a.x = static_cast<const uint8_t*>(x);
     a.w = p->w_mfma;
-    a.mult = p->mult;
-    a.biasf = p->biasf;
+    a.ct = ChanTab{p->chan, p->Co_pad};
     a.corr = p->corr;
     a.y = static_cast<uint8_t*>(y);
     const long long M = static_cast<long long>(batch) * g.Ho * g.Wo;
@@ -321,13 +449,29 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
     case MI355X_ALGO_MFMA:
         if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || ((g.Co & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) != 0))
             return SetError(MI355X_ERR_INVALID_ARGUMENT, "MFMA kernel needs 16-byte aligned tensors");
-        if (p->bn == 64) return LaunchIgemm<128, 64, 2, 2>(p, batch, x, y, stream);
+    {
+        if (p->pw_bn)
+        {
+            const long long Mrows = static_cast<long long>(batch) * g.Ho * g.Wo;
+            if (Mrows > 0x7fffffffll / 2) return SetError(MI355X_ERR_UNSUPPORTED, "too many rows for one launch (%lld)", Mrows);
+            if (p->pw_bn == 128) return LaunchPwKs<128>(p, Mrows, x, y, stream);
+            if (p->pw_bn == 64) return LaunchPwKs<64>(p, Mrows, x, y, stream);
+            return LaunchPwKs<32>(p, Mrows, x, y, stream);
+        }
+        // Tile choice: the large tile has the best MFMA : LDS-traffic ratio, but a launch needs several blocks per CU
+        // in flight to hide global-load latency, so problems that would yield few large tiles take 64x64 tiles
+        // (4x the blocks, 8 waves/SIMD).
+        const long long M = static_cast<long long>(batch) * g.Ho * g.Wo;
+        const long long big = ((M + 127) / 128) * ((g.Co + 127) / 128);
+        if (p->tile_override == 64 || (p->tile_override == 0 && big < 1024)) return LaunchIgemm<64, 64, 2, 2>(p, batch, x, y, stream);
+        if (g.Co <= 64) return LaunchIgemm<128, 64, 2, 2>(p, batch, x, y, stream);
         return LaunchIgemm<128, 128, 2, 2>(p, batch, x, y, stream);
+    }
     case MI355X_ALGO_DOT4:
     {
         if ((reinterpret_cast<uintptr_t>(y) & 3) != 0) return SetError(MI355X_ERR_INVALID_ARGUMENT, "dot4 kernel needs a 4-byte aligned output");
         SmallCiArgs a;
-        a.x = xin; a.wpack = p->w_dot4; a.mult = p->mult; a.biasf = p->biasf; a.corr = p->corr; a.y = yout;
+        a.x = xin; a.wpack = p->w_dot4; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
         a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.Ci = g.Ci; a.Ho = g.Ho; a.Wo = g.Wo; a.Co = g.Co;
         a.Kw = g.Kw; a.stride = g.stride_x; a.pad_top = g.pad_top; a.pad_left = g.pad_left;
         a.tiles_x = (g.Wo + 15) / 16; a.tiles_y = (g.Ho + 15) / 16;
@@ -351,7 +495,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 3) != 0)
                 return SetError(MI355X_ERR_INVALID_ARGUMENT, "depthwise 3x3 kernel needs a 16-byte aligned input and 4-byte aligned output");
             Dw3x3Args a;
-            a.x = xin; a.wpack = p->w_dot4; a.mult = p->mult; a.biasf = p->biasf; a.corr = p->corr; a.y = yout;
+            a.x = xin; a.wpack = p->w_dot4; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
             a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.C = g.Co; a.Ho = g.Ho; a.Wo = g.Wo;
             a.pad_top = g.pad_top; a.pad_left = g.pad_left;
             const int tw = g.stride_x == 1 ? 16 : 8;
@@ -369,13 +513,13 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const long long total4 = total / 4;
         const unsigned blocks = static_cast<unsigned>((total4 + 255) / 256);
         if (g.in_u8 && !g.w_u8)
-            hipLaunchKernelGGL((DepthwiseC4Kernel<true, false>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total4);
+            hipLaunchKernelGGL((DepthwiseC4Kernel<true, false>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, ChanTab{p->chan, p->Co_pad}, yout, total4);
         else if (!g.in_u8 && !g.w_u8)
-            hipLaunchKernelGGL((DepthwiseC4Kernel<false, false>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total4);
+            hipLaunchKernelGGL((DepthwiseC4Kernel<false, false>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, ChanTab{p->chan, p->Co_pad}, yout, total4);
         else if (g.in_u8 && g.w_u8)
-            hipLaunchKernelGGL((DepthwiseC4Kernel<true, true>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total4);
+            hipLaunchKernelGGL((DepthwiseC4Kernel<true, true>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, ChanTab{p->chan, p->Co_pad}, yout, total4);
         else
-            hipLaunchKernelGGL((DepthwiseC4Kernel<false, true>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total4);
+            hipLaunchKernelGGL((DepthwiseC4Kernel<false, true>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, ChanTab{p->chan, p->Co_pad}, yout, total4);
         MI355X_HIP(hipGetLastError());
         return 0;
     }
@@ -383,9 +527,9 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
     {
         const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
         if (p->d.depthwise)
-            hipLaunchKernelGGL((ConvDirectKernel<true>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total);
+            hipLaunchKernelGGL((ConvDirectKernel<true>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, ChanTab{p->chan, p->Co_pad}, yout, total);
         else
-            hipLaunchKernelGGL((ConvDirectKernel<false>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, p->mult, p->biasf, yout, total);
+            hipLaunchKernelGGL((ConvDirectKernel<false>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, ChanTab{p->chan, p->Co_pad}, yout, total);
         MI355X_HIP(hipGetLastError());
         return 0;
     }

@@ -34,10 +34,8 @@ struct ConvGeom
 // ---------------------------------------------------------------------------------------------------------
 template <bool DEPTHWISE>
 __global__ __launch_bounds__(256) void ConvDirectKernel(ConvGeom g, Requant rq, const uint8_t* __restrict__ x,
-                                                        const uint8_t* __restrict__ w,
-                                                        const float* __restrict__ mult,
-                                                        const float* __restrict__ biasf, uint8_t* __restrict__ y,
-                                                        long long total)
+                                                        const uint8_t* __restrict__ w, ChanTab ct,
+                                                        uint8_t* __restrict__ y, long long total)
 {
     const long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
     if (idx >= total) return;
@@ -82,7 +80,7 @@ __global__ __launch_bounds__(256) void ConvDirectKernel(ConvGeom g, Requant rq, 
             }
         }
     }
-    y[idx] = static_cast<uint8_t>(RequantDev(acc, mult[co], biasf[co], rq));
+    y[idx] = static_cast<uint8_t>(Requant1Dev(acc, ct, co, rq));
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -104,9 +102,7 @@ __device__ __forceinline__ void DwMac4(uint32_t xw, uint32_t ww, int zx, int zw,
 
 template <bool IN_U8, bool W_U8>
 __global__ __launch_bounds__(256) void DepthwiseC4Kernel(ConvGeom g, Requant rq, const uint8_t* __restrict__ x,
-                                                         const uint8_t* __restrict__ w,
-                                                         const float* __restrict__ mult,
-                                                         const float* __restrict__ biasf,
+                                                         const uint8_t* __restrict__ w, ChanTab ct,
                                                          uint8_t* __restrict__ y, long long total_c4)
 {
     const long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
@@ -135,11 +131,8 @@ __global__ __launch_bounds__(256) void DepthwiseC4Kernel(ConvGeom g, Requant rq,
             DwMac4<IN_U8, W_U8>(xw, ww, g.zx, g.zw, acc);
         }
     }
-    const float4 m4 = *reinterpret_cast<const float4*>(mult + c);
-    const float4 b4 = *reinterpret_cast<const float4*>(biasf + c);
-    *reinterpret_cast<uint32_t*>(y + idx * 4) =
-        Pack4(RequantDev(acc[0], m4.x, b4.x, rq), RequantDev(acc[1], m4.y, b4.y, rq), RequantDev(acc[2], m4.z, b4.z, rq),
-              RequantDev(acc[3], m4.w, b4.w, rq));
+    const Fast4 f4 = LoadFast4(ct, c);
+    *reinterpret_cast<uint32_t*>(y + idx * 4) = Requant4Dev(acc[0], acc[1], acc[2], acc[3], f4, ct, c, rq);
 }
 
 // ---------------------------------------------------------------------------------------------------------
@@ -164,8 +157,7 @@ struct IgemmArgs
 {
     const uint8_t* x;
     const int8_t*  w;       // [Co_pad][K_pad], zero padded
-    const float*   mult;    // [Co_pad]
-    const float*   biasf;   // [Co_pad]
+    ChanTab        ct;      // per-channel requantization constants, rows of Co_pad floats
     const int32_t* corr;    // [Co_pad]
     uint8_t*       y;
     int M;                  // batch * Ho * Wo
@@ -370,14 +362,12 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
         for (int q = 0; q < 4; ++q)
         {
             const int cl = wn * WTN + tc * 32 + 8 * q + lane_c;           // channel within the block tile
-            const float4 m4 = *reinterpret_cast<const float4*>(a.mult + tn * BN + cl);
-            const float4 b4 = *reinterpret_cast<const float4*>(a.biasf + tn * BN + cl);
+            const Fast4 f4 = LoadFast4(a.ct, tn * BN + cl);
 #pragma unroll
             for (int tp = 0; tp < TP; ++tp)
             {
                 const v16i& c = acc[tc][tp];
-                const uint32_t out = Pack4(RequantDev(c[4 * q + 0], m4.x, b4.x, a.rq), RequantDev(c[4 * q + 1], m4.y, b4.y, a.rq),
-                                           RequantDev(c[4 * q + 2], m4.z, b4.z, a.rq), RequantDev(c[4 * q + 3], m4.w, b4.w, a.rq));
+                const uint32_t out = Requant4Dev(c[4 * q + 0], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], f4, a.ct, tn * BN + cl, a.rq);
                 const int pl = wm * WTM + tp * 32 + (lane & 31);          // pixel within the block tile
                 *reinterpret_cast<uint32_t*>(Os + pl * LDO + cl) = out;
             }

@@ -23,40 +23,137 @@ __device__ __forceinline__ int QuantizeDev(float f, const Requant& rq)
     return r;
 }
 
-// Same result as QuantizeDev, cheaper on average (9 VALU instructions + pack instead of ~30).
-//   r' = fma(f, fl(1/scale), offset) differs from fl(f/scale) + offset by less than 2^-12 whenever |f/scale| <= 512
-//   (reciprocal and fma rounding: (|r| + |r'|) * 2^-24; the correctly rounded quotient: |r| * 2^-24), so the two can
-//   round to different integers only when r' lies within 2^-12 of a half-integer.  Those values (kTieWindow = 2^-11
-//   either side: about 1 in 1000) take the exact division instead.  For |f/scale| > 512 both results are beyond the
-//   8-bit range whatever the offset (|offset| <= 255, checked on the host) and clamp alike.
-//   Round-half-even (v_rndne) serves on the fast path: it differs from round-half-away only at exact ties, which
-//   are inside the window.
+// int32 accumulator of sum (x - zx)(w - zw) -> output code, the reference's way:
+//   f = float(acc) * (s_in * s_w[c]) + float(bias[c]) * s_b[c]      (separate multiply and add, no FMA)
+// `mult` and `biasf` are prepared on the host in fp32 exactly as the reference's decoders would produce them.
+__device__ __forceinline__ int RequantExactDev(int acc, float mult, float biasf, const Requant& rq)
+{
+    return QuantizeDev(__fadd_rn(__fmul_rn(static_cast<float>(acc), mult), biasf), rq);
+}
+
+// Per-channel constants, five rows of `stride` floats (see ChannelTable on the host side):
+//   row 0 mult   s_in * s_w[c]                      row 1 biasf  float(bias[c]) * s_b[c]
+//   row 2 fm     fl(mult * fl(1/s_out))             row 3 fb     fl(fl(biasf * fl(1/s_out)) + offset)
+//   row 4 thr    0.5 - window[c]   (negative: channel always takes the exact path)
+struct ChanTab
+{
+    const float* p;
+    int stride;
+};
+
+// Fast path with an exact fallback.  r' = fma(float(acc), fm, fb) approximates f/s_out + offset with an absolute
+// error below window[c] = 2^-19 * (|biasf/s_out| + 1024) whenever the exact result is within the 8-bit range
+// (three roundings of the reference, the coefficient roundings and the fma rounding, each 2^-24 relative to
+// magnitudes bounded by |biasf/s_out| + 767).  So r' and the reference can round to different integers only when
+// r' is within window[c] of a half-integer; exactly those values are recomputed the reference's way.
+// Results beyond the 8-bit range clamp alike on both paths.  Round-half-even (v_rndne) serves on the fast path:
+// it differs from round-half-away only at exact ties, which are inside the window.
+__device__ __forceinline__ uint32_t Pack4(int q0, int q1, int q2, int q3)
+{
+    // four codes -> one dword (byte 0 = q0), three v_perm_b32
+    const uint32_t t0 = __builtin_amdgcn_perm(static_cast<uint32_t>(q1), static_cast<uint32_t>(q0), 0x0c0c0400u);
+    const uint32_t t1 = __builtin_amdgcn_perm(static_cast<uint32_t>(q3), static_cast<uint32_t>(q2), 0x0c0c0400u);
+    return __builtin_amdgcn_perm(t1, t0, 0x05040100u);
+}
+
+struct Fast4
+{
+    float4 m, b, t;
+};
+
+__device__ __forceinline__ Fast4 LoadFast4(const ChanTab& ct, int c)
+{
+    Fast4 f;
+    f.m = *reinterpret_cast<const float4*>(ct.p + 2 * ct.stride + c);
+    f.b = *reinterpret_cast<const float4*>(ct.p + 3 * ct.stride + c);
+    f.t = *reinterpret_cast<const float4*>(ct.p + 4 * ct.stride + c);
+    return f;
+}
+
+#define MI355X_FAST1(ACC, M, B, K, E)                                   \
+    {                                                                   \
+        const float r_ = __fmaf_rn(static_cast<float>(ACC), M, B);      \
+        K = __builtin_rintf(r_);                                        \
+        E = __fsub_rn(r_, K);                                           \
+    }
+
+// Four consecutive channels c..c+3 of one pixel -> packed dword.
+//   `corr` (may be null) is an integer added to the accumulator on the exact path only: kernels that start their
+//   accumulators at zero use channel-table rows whose fast-path constants already contain corr * fm.
+// The fast path is branch-free (7 VALU instructions per value); the four flags are combined as wave masks, and
+// only when some lane of the wave has a value inside its tie window does the wave enter the fix-up loop, which
+// evaluates one flagged value per lane and pass.
+__device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const float4& fm, const float4& fb,
+                                                const float4& thr, const ChanTab& ct, const int32_t* corr, int c,
+                                                const Requant& rq)
+{
+    float k0, k1, k2, k3, e0, e1, e2, e3;
+    MI355X_FAST1(a0, fm.x, fb.x, k0, e0)
+    MI355X_FAST1(a1, fm.y, fb.y, k1, e1)
+    MI355X_FAST1(a2, fm.z, fb.z, k2, e2)
+    MI355X_FAST1(a3, fm.w, fb.w, k3, e3)
+    int q0 = static_cast<int>(__builtin_amdgcn_fmed3f(k0, rq.act_lo_f, rq.act_hi_f));
+    int q1 = static_cast<int>(__builtin_amdgcn_fmed3f(k1, rq.act_lo_f, rq.act_hi_f));
+    int q2 = static_cast<int>(__builtin_amdgcn_fmed3f(k2, rq.act_lo_f, rq.act_hi_f));
+    int q3 = static_cast<int>(__builtin_amdgcn_fmed3f(k3, rq.act_lo_f, rq.act_hi_f));
+    // "not (|e| <= thr)" also sends NaN to the exact path
+    const bool s0 = !(fabsf(e0) <= thr.x), s1 = !(fabsf(e1) <= thr.y), s2 = !(fabsf(e2) <= thr.z), s3 = !(fabsf(e3) <= thr.w);
+    const unsigned long long any = __builtin_amdgcn_ballot_w64(s0) | __builtin_amdgcn_ballot_w64(s1) |
+                                   __builtin_amdgcn_ballot_w64(s2) | __builtin_amdgcn_ballot_w64(s3);
+    if (__builtin_expect(any != 0, 0))
+    {
+        const float4 m = *reinterpret_cast<const float4*>(ct.p + c);
+        const float4 b = *reinterpret_cast<const float4*>(ct.p + ct.stride + c);
+        int4 cr = {0, 0, 0, 0};
+        if (corr) cr = *reinterpret_cast<const int4*>(corr + c);
+        unsigned fl = (s0 ? 1u : 0u) | (s1 ? 2u : 0u) | (s2 ? 4u : 0u) | (s3 ? 8u : 0u);
+        while (__builtin_amdgcn_ballot_w64(fl != 0) != 0)
+        {
+            const int which = __builtin_ctz(fl | 16u);     // 4 when the lane has nothing left
+            const int av = which == 0 ? a0 + cr.x : which == 1 ? a1 + cr.y : which == 2 ? a2 + cr.z : a3 + cr.w;
+            const float mv = which == 0 ? m.x : which == 1 ? m.y : which == 2 ? m.z : m.w;
+            const float bv = which == 0 ? b.x : which == 1 ? b.y : which == 2 ? b.z : b.w;
+            const int qe = RequantExactDev(av, mv, bv, rq);
+            if (which == 0) q0 = qe;
+            if (which == 1) q1 = qe;
+            if (which == 2) q2 = qe;
+            if (which == 3) q3 = qe;
+            fl &= fl - 1u;
+        }
+    }
+    return Pack4(q0, q1, q2, q3);
+}
+
+// constants of rows 2,3,4 (accumulator already contains the zero-point correction)
+__device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const Fast4& f, const ChanTab& ct, int c,
+                                                const Requant& rq)
+{
+    return Requant4Dev(a0, a1, a2, a3, f.m, f.b, f.t, ct, nullptr, c, rq);
+}
+
+// one channel (scalar kernels)
+__device__ __forceinline__ int Requant1Dev(int acc, const ChanTab& ct, int c, const Requant& rq)
+{
+    float k, e;
+    MI355X_FAST1(acc, ct.p[2 * ct.stride + c], ct.p[3 * ct.stride + c], k, e)
+    if (__builtin_expect(!(fabsf(e) <= ct.p[4 * ct.stride + c]), 0))
+        return RequantExactDev(acc, ct.p[c], ct.p[ct.stride + c], rq);
+    return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.act_lo_f, rq.act_hi_f));
+}
+
+// value already in float (pooling, add, ...): reciprocal fast path with the exact fallback near ties.
+//   r' = fma(f, fl(1/scale), offset) is within (|r| + |r'|) * 2^-24 of f/scale + offset; for |f/scale| <= 512 that is
+//   below 2^-12, and beyond it both paths clamp alike (|offset| <= 255 is checked on the host, else fast_ok = 0).
 constexpr float kTieWindow = 1.0f / 2048.0f;
 
 __device__ __forceinline__ int QuantizeFastDev(float f, const Requant& rq)
 {
+    if (!rq.fast_ok) return QuantizeDev(f, rq);
     const float r = __fmaf_rn(f, rq.inv_scale, rq.out_offset_f);
     const float k = __builtin_rintf(r);
     const float e = __fsub_rn(r, k);
-    if (__builtin_expect(fabsf(e) > 0.5f - kTieWindow, 0)) return QuantizeDev(f, rq);
+    if (__builtin_expect(!(fabsf(e) <= 0.5f - kTieWindow), 0)) return QuantizeDev(f, rq);
     return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.act_lo_f, rq.act_hi_f));
-}
-
-// int32 accumulator of sum (x - zx)(w - zw)  ->  output code.
-//   f = float(acc) * (s_in * s_w[c]) + float(bias[c]) * s_b[c]      (separate multiply and add, no FMA)
-// `mult` and `biasf` are prepared on the host in fp32 exactly as the reference's decoders would produce them.
-__device__ __forceinline__ int RequantDev(int acc, float mult, float biasf, const Requant& rq)
-{
-    const float f = __fadd_rn(__fmul_rn(static_cast<float>(acc), mult), biasf);
-    return rq.fast_ok ? QuantizeFastDev(f, rq) : QuantizeDev(f, rq);
-}
-
-// four codes -> one dword (byte 0 = q0), three v_perm_b32
-__device__ __forceinline__ uint32_t Pack4(int q0, int q1, int q2, int q3)
-{
-    const uint32_t t0 = __builtin_amdgcn_perm(static_cast<uint32_t>(q1), static_cast<uint32_t>(q0), 0x0c0c0400u);
-    const uint32_t t1 = __builtin_amdgcn_perm(static_cast<uint32_t>(q3), static_cast<uint32_t>(q2), 0x0c0c0400u);
-    return __builtin_amdgcn_perm(t1, t0, 0x05040100u);
 }
 
 } // namespace mi355x

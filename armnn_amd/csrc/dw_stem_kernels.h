@@ -21,8 +21,7 @@ struct Dw3x3Args
 {
     const uint8_t*  x;
     const uint32_t* wpack;    // [C][4] dwords; dword r (r < 3) = bytes { w[r][0][c], w[r][1][c], w[r][2][c], 0 }
-    const float*    mult;
-    const float*    biasf;
+    ChanTab         ct;
     const int32_t*  corr;     // [C]  -zx' * sum of the 9 taps
     uint8_t*        y;
     int N, H, W, C, Ho, Wo;
@@ -140,8 +139,7 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
     // ---- epilogue ------------------------------------------------------------------------------------------------
     const int oy = ty * TH + row;
     if (oy >= a.Ho) return;
-    const float4 m4 = *reinterpret_cast<const float4*>(a.mult + c);
-    const float4 b4 = *reinterpret_cast<const float4*>(a.biasf + c);
+    const Fast4 f4 = LoadFast4(a.ct, c);
     uint8_t* yrow = a.y + (static_cast<long long>(n) * a.Ho + oy) * a.Wo * a.C + c;
 #pragma unroll
     for (int j = 0; j < P; ++j)
@@ -150,8 +148,7 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
         if (ox < a.Wo)
         {
             *reinterpret_cast<uint32_t*>(yrow + static_cast<long long>(ox) * a.C) =
-                Pack4(RequantDev(acc[j][0], m4.x, b4.x, a.rq), RequantDev(acc[j][1], m4.y, b4.y, a.rq),
-                      RequantDev(acc[j][2], m4.z, b4.z, a.rq), RequantDev(acc[j][3], m4.w, b4.w, a.rq));
+                Requant4Dev(acc[j][0], acc[j][1], acc[j][2], acc[j][3], f4, a.ct, c, a.rq);
         }
     }
 }
@@ -161,8 +158,7 @@ struct SmallCiArgs
 {
     const uint8_t*  x;
     const uint32_t* wpack;    // [Co][KH][RD] dwords: row r of filter co as consecutive (kx, ci) bytes, zero padded
-    const float*    mult;
-    const float*    biasf;
+    ChanTab         ct;
     const int32_t*  corr;     // [Co]
     uint8_t*        y;
     int N, H, W, Ci, Ho, Wo, Co;
@@ -238,6 +234,7 @@ __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
     for (int co = 0; co < a.Co; co += 4)
     {
         int q[4];
+        const Fast4 f4 = LoadFast4(a.ct, co);
 #pragma unroll
         for (int u = 0; u < 4; ++u)
         {
@@ -248,9 +245,9 @@ __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
 #pragma unroll
                 for (int i = 0; i < RD; ++i)
                     acc = __builtin_amdgcn_sdot4(static_cast<int>(xr[r][i]), static_cast<int>(w[r * RD + i]), acc, false);
-            q[u] = RequantDev(acc, a.mult[co + u], a.biasf[co + u], a.rq);
+            q[u] = acc;
         }
-        *reinterpret_cast<uint32_t*>(yp + co) = Pack4(q[0], q[1], q[2], q[3]);
+        *reinterpret_cast<uint32_t*>(yp + co) = Requant4Dev(q[0], q[1], q[2], q[3], f4, a.ct, co, a.rq);
     }
 }
 

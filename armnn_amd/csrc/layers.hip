@@ -107,7 +107,7 @@ __global__ __launch_bounds__(256) void Pool2dKernel(PoolArgs p, QIn qin, Requant
             }
         if (!p.is_max) result = __fdiv_rn(result, area);
     }
-    y[idx] = static_cast<uint8_t>(QuantizeDev(result, rq));
+    y[idx] = static_cast<uint8_t>(QuantizeFastDev(result, rq));
 }
 
 __global__ __launch_bounds__(256) void AddKernel(QIn q0, QIn q1, Requant rq, int fn, float a, float b,
@@ -119,7 +119,7 @@ __global__ __launch_bounds__(256) void AddKernel(QIn q0, QIn q1, Requant rq, int
     for (; i < n; i += stride)
     {
         const float s = __fadd_rn(DequantDev(x0[i], q0), DequantDev(x1[i], q1));
-        int q = QuantizeDev(s, rq);   // rq carries the fused activation as an integer clamp
+        int q = QuantizeFastDev(s, rq);   // rq carries the fused activation as an integer clamp
         y[i] = static_cast<uint8_t>(q);
     }
     (void)fn; (void)a; (void)b;

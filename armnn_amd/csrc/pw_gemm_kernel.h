@@ -1,0 +1,214 @@
+// Pointwise (1x1, stride 1, unpadded) Convolution2d and FullyConnected as a weight-stationary GEMM on MFMA.
+//
+//   out[m][n] = requant( sum_k A[m][k] * W[n][k] ),  A = activations [M][K] (NHWC rows are pixels), W = [N][K].
+//
+//   A block keeps its BN x K weight slab in LDS for its whole life and walks over 32-row tiles of A.  Each wave owns
+//   whole tiles: it reads its MFMA "B" fragments (lane = pixel row, 16 contiguous K bytes) straight from global
+//   memory into registers -- NHWC makes them contiguous -- NB-1 register chunks ahead of the MFMAs, so there is no
+//   LDS staging of activations, no block barrier after the prologue, and many 16-byte loads in flight per lane.
+//   The epilogue requantizes 4 channels at a time, stages the 32 x BN byte tile in the wave's private LDS area and
+//   writes it with 16-byte row-contiguous stores.
+//
+//   Zero points: uint8 activations are xor-ed with 0x80 in registers; acc = sum x' w, and the per-channel constant
+//   corr[n] = -zx' * sum_k w[n][k] is folded into the requantization constants (rows 5/6 of the channel table) on
+//   the fast path and added to the accumulator on the exact path.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "conv_kernels.h"
+#include "device_math.h"
+
+namespace mi355x
+{
+
+struct PwArgs
+{
+    const uint8_t* x;
+    const int8_t*  w;        // [>= n_slabs*BN][w_stride], rows zero padded
+    ChanTab        ct;       // rows 0,1 exact; rows 2,5,6: fm, fb + corr*fm, threshold for the corr-folded form
+    const int32_t* corr;
+    uint8_t*       y;
+    int M, K, N;
+    int w_stride;
+    int n_slabs, gm;         // grid = n_slabs * gm blocks; block (slab, g) takes tile groups g, g+gm, ...
+    uint32_t xor_mask;
+    Requant rq;
+};
+
+template <int BN>
+constexpr int PwSmemBytes(int K)
+{
+    return BN * (K + 16) + 4 * 32 * (BN + 16) + 3 * BN * 4;
+}
+
+// KS = MFMA k-steps (of 32) per register chunk, K % (32 * KS) == 0;  NB = register chunks per wave (NB-1 in flight).
+template <int BN, int KS, int NB>
+__global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
+{
+    constexpr int TC = BN / 32;
+    constexpr int LDO = BN + 16;
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
+    const int LDW = a.K + 16;
+    uint8_t* slab = smem;
+    float* cst = reinterpret_cast<float*>(smem + BN * LDW);                 // [3][BN]: fm, fb(folded), thr(folded)
+    uint8_t* ostage_all = smem + BN * LDW + 3 * BN * 4;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int slab_id = blockIdx.x % a.n_slabs;
+    const int g = blockIdx.x / a.n_slabs;
+    const int n0 = slab_id * BN;
+
+    // ---- prologue: weight slab and epilogue constants into LDS (loads batched per column of chunks) ---------
+    {
+        const int chunks = a.K >> 4;
+        const int8_t* src = a.w + static_cast<long long>(n0 + (tid >> 4)) * a.w_stride;
+        for (int c = tid & 15; c < chunks; c += 16)
+        {
+            v4i t[BN / 16];
+#pragma unroll
+            for (int i = 0; i < BN / 16; ++i) t[i] = *reinterpret_cast<const v4i*>(src + static_cast<long long>(16 * i) * a.w_stride + c * 16);
+#pragma unroll
+            for (int i = 0; i < BN / 16; ++i) *reinterpret_cast<v4i*>(slab + ((tid >> 4) + 16 * i) * LDW + c * 16) = t[i];
+        }
+        for (int i = tid; i < 3 * BN; i += 256)
+        {
+            const int row = i / BN, c = i - row * BN;
+            const int src_row = row == 0 ? 2 : row == 1 ? 5 : 6;
+            cst[i] = a.ct.p[src_row * a.ct.stride + n0 + c];
+        }
+    }
+    __syncthreads();
+
+    uint8_t* ostage = ostage_all + wave * 32 * LDO;
+    const int n_tiles = (a.M + 31) >> 5;
+    const int nch = a.K / (32 * KS);
+    const int frag_row = lane & 31;
+    const int frag_k = (lane >> 5) * 16;
+    const int xm = static_cast<int>(a.xor_mask);
+    const int tile_step = a.gm * 4;
+    const int tile0 = g * 4 + wave;              // first tile of this wave
+    if (tile0 >= n_tiles) return;
+
+    v16i acc[TC];
+#pragma unroll
+    for (int tc = 0; tc < TC; ++tc)
+#pragma unroll
+        for (int v = 0; v < 16; ++v) acc[tc][v] = 0;
+
+    auto load_chunk = [&](v4i (&buf)[KS], int t, int ch) {
+        const int row = t * 32 + frag_row;
+        if (row < a.M)
+        {
+            const uint8_t* p = a.x + static_cast<long long>(row) * a.K + ch * (32 * KS) + frag_k;
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) buf[ks] = *reinterpret_cast<const v4i*>(p + ks * 32);
+        }
+        else
+        {
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) buf[ks] = v4i{0, 0, 0, 0};
+        }
+    };
+
+    auto compute_chunk = [&](v4i (&buf)[KS], int ch) {
+        const uint8_t* wbase = slab + frag_row * LDW + ch * (32 * KS) + frag_k;
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+        {
+            const v4i av = buf[ks] ^ xm;
+#pragma unroll
+            for (int tc = 0; tc < TC; ++tc)
+            {
+                const v4i wv = *reinterpret_cast<const v4i*>(wbase + tc * 32 * LDW + ks * 32);
+                acc[tc] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wv, av, acc[tc], 0, 0, 0);
+            }
+        }
+    };
+
+    auto epilogue = [&](int t) {
+        const int lane_c = 4 * (lane >> 5);
+#pragma unroll
+        for (int tc = 0; tc < TC; ++tc)
+        {
+#pragma unroll
+            for (int q = 0; q < 4; ++q)
+            {
+                const int cl = tc * 32 + 8 * q + lane_c;
+                const float4 fm = *reinterpret_cast<const float4*>(cst + cl);
+                const float4 fb = *reinterpret_cast<const float4*>(cst + BN + cl);
+                const float4 th = *reinterpret_cast<const float4*>(cst + 2 * BN + cl);
+                const uint32_t out = Requant4Dev(acc[tc][4 * q + 0], acc[tc][4 * q + 1], acc[tc][4 * q + 2], acc[tc][4 * q + 3],
+                                                 fm, fb, th, a.ct, a.corr, n0 + cl, a.rq);
+                *reinterpret_cast<uint32_t*>(ostage + frag_row * LDO + cl) = out;
+            }
+#pragma unroll
+            for (int v = 0; v < 16; ++v) acc[tc][v] = 0;
+        }
+        // the wave reads back what its own lanes wrote: LDS operations of one wave complete in order; the fences keep
+        // the compiler from moving the reads above the writes (different lanes, so no dependency it can see)
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+        __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+        constexpr int CH = BN / 16;                 // 16-byte chunks per row
+        if ((a.N & 15) == 0)
+        {
+#pragma unroll
+            for (int j = lane; j < 32 * CH; j += 64)
+            {
+                const int r = j / CH, cc = j % CH;
+                const int row = t * 32 + r;
+                const int c0 = n0 + cc * 16;
+                if (row < a.M && c0 < a.N)
+                    *reinterpret_cast<v4i*>(a.y + static_cast<long long>(row) * a.N + c0) =
+                        *reinterpret_cast<const v4i*>(ostage + r * LDO + cc * 16);
+            }
+        }
+        else
+        {
+            for (int j = lane; j < 32 * BN; j += 64)
+            {
+                const int r = j / BN, c = j % BN;
+                const int row = t * 32 + r;
+                if (row < a.M && n0 + c < a.N) a.y[static_cast<long long>(row) * a.N + n0 + c] = ostage[r * LDO + c];
+            }
+        }
+        // and the next tile's staging writes must stay behind these reads
+        __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+        __builtin_amdgcn_wave_barrier();
+    };
+
+    // ---- software pipeline over (tile, chunk): NB-1 chunks are in flight while one feeds the MFMAs --------------
+    v4i buf[NB][KS];
+    int t_cur = tile0, c_cur = 0;                // chunk being computed
+    int t_nxt = tile0, c_nxt = 0;                // next chunk to load
+    auto advance = [&](int& t, int& c) {
+        if (++c == nch) { c = 0; t += tile_step; }
+    };
+#pragma unroll
+    for (int j = 0; j < NB - 1; ++j)
+    {
+        if (t_nxt < n_tiles) { load_chunk(buf[j], t_nxt, c_nxt); advance(t_nxt, c_nxt); }
+    }
+    bool done = false;
+    while (!done)
+    {
+#pragma unroll
+        for (int j = 0; j < NB; ++j)
+        {
+            if (!done)
+            {
+                if (t_nxt < n_tiles) { load_chunk(buf[(j + NB - 1) % NB], t_nxt, c_nxt); advance(t_nxt, c_nxt); }
+                compute_chunk(buf[j], c_cur);
+                if (c_cur == nch - 1) epilogue(t_cur);
+                advance(t_cur, c_cur);
+                done = t_cur >= n_tiles;
+            }
+        }
+    }
+}
+
+} // namespace mi355x

@@ -1,0 +1,108 @@
+"""Time one quantized layer on the device through the C ABI and price it against its roofline.
+
+  python -m armnn_amd.layerbench conv --n 64 --h 14 --w 14 --ci 512 --co 512 --k 1
+  python -m armnn_amd.layerbench dw   --n 64 --h 112 --w 112 --c 32 --stride 1
+  python -m armnn_amd.layerbench fc   --m 2048 --k 4096 --o 4096
+
+Prints one JSON line: kernel chosen, average launch time (HIP events on the launch stream), algorithmic
+ops and bytes, and the fraction of the int8 MFMA peak (5.0 POP/s) or of the HBM peak (8 TB/s).
+Inputs are seeded synthetic data; nothing is checked here (parity lives in tests/).
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import sys
+
+import numpy as np
+
+from . import shim, synth
+from .tensor import DataType, QTensor, TensorInfo
+
+INT8_PEAK = 5.0e15
+HBM_PEAK = 8.0e12
+
+
+def _same(in_size, k, stride):
+    out = (in_size + stride - 1) // stride
+    total = max((out - 1) * stride + k - in_size, 0)
+    return out, total // 2
+
+
+def main(argv=None):
+    ap = argparse.ArgumentParser()
+    ap.add_argument("op", choices=["conv", "dw", "fc"])
+    ap.add_argument("--n", type=int, default=64)
+    ap.add_argument("--h", type=int, default=56)
+    ap.add_argument("--w", type=int, default=56)
+    ap.add_argument("--ci", type=int, default=64)
+    ap.add_argument("--co", type=int, default=64)
+    ap.add_argument("--c", type=int, default=32)
+    ap.add_argument("--k", type=int, default=3, help="kernel size (conv/dw) or K (fc)")
+    ap.add_argument("--stride", type=int, default=1)
+    ap.add_argument("--m", type=int, default=256)
+    ap.add_argument("--o", type=int, default=4096)
+    ap.add_argument("--u8", action="store_true", help="QAsymmU8 activations (default QAsymmS8)")
+    ap.add_argument("--algo", type=int, default=0)
+    ap.add_argument("--iters", type=int, default=50)
+    ap.add_argument("--warmup", type=int, default=5)
+    a = ap.parse_args(argv)
+
+    dev = shim.Device()
+    adt = DataType.QAsymmU8 if a.u8 else DataType.QAsymmS8
+    zp = 128 if a.u8 else -3
+    act = (shim.ACT_BOUNDED_RELU, 6.0, 0.0)
+    if a.op == "fc":
+        k, o, m = a.k if a.k > 3 else 4096, a.o, a.m
+        xin = TensorInfo((m, k), adt, (0.02,), zp)
+        yout = TensorInfo((m, o), adt, (1.0,), 0)
+        ws = synth.scales(3, o)
+        w = QTensor(TensorInfo((o, k), DataType.QSymmS8, tuple(ws), 0, 0), synth.int8_weights(2, (o, k)))
+        b = QTensor(TensorInfo((o,), DataType.Signed32, tuple(np.float32(0.02) * ws), 0, 0), synth.int32_bias(4, o))
+        plan = shim.FullyConnectedPlan(xin, w, b, yout, algo=a.algo)
+        batch, macs = m, m * k * o
+        nbytes = m * k + m * o + k * o + 8 * o
+        desc = f"fc M={m} K={k} O={o}"
+    else:
+        dw = a.op == "dw"
+        ci = a.c if dw else a.ci
+        co = a.c if dw else a.co
+        ho, pt = _same(a.h, a.k, a.stride)
+        wo, pl = _same(a.w, a.k, a.stride)
+        xin = TensorInfo((a.n, a.h, a.w, ci), adt, (0.0235,), zp)
+        yout = TensorInfo((a.n, ho, wo, co), adt, (0.0235,), 0 if a.u8 else -128)
+        wshape = (1, a.k, a.k, co) if dw else (co, a.k, a.k, ci)
+        taps = a.k * a.k * (1 if dw else ci)
+        ws = synth.scales(3, co) / np.float32(np.sqrt(taps) / 3.0)
+        w = QTensor(TensorInfo(wshape, DataType.QSymmS8, tuple(ws), 0, 3 if dw else 0), synth.int8_weights(2, wshape))
+        b = QTensor(TensorInfo((co,), DataType.Signed32, tuple(np.float32(0.0235) * ws), 0, 0), synth.int32_bias(4, co))
+        plan = shim.Conv2dPlan(xin, w, b, yout, pad_top=pt, pad_left=pl, stride_x=a.stride, stride_y=a.stride,
+                               depthwise=dw, activation=act[0], act_a=act[1], act_b=act[2], algo=a.algo)
+        batch, macs = a.n, a.n * ho * wo * co * taps
+        nbytes = xin.num_elements + yout.num_elements + w.info.num_elements + 8 * co
+        desc = f"{a.op} N={a.n} {a.h}x{a.w}x{ci}->{co} k{a.k} s{a.stride}"
+
+    lo, hi = (0, 255) if a.u8 else (-128, 127)
+    xd = shim.DeviceBuffer(xin.num_elements).upload(synth.uniform_int(1, xin.shape, lo, hi, np.uint8 if a.u8 else np.int8))
+    yd = shim.DeviceBuffer(yout.num_elements)
+    stream = dev.stream()
+    for _ in range(a.warmup):
+        plan.run(batch, xd.ptr, yd.ptr, stream)
+    e0, e1 = dev.event(), dev.event()
+    dev.event_record(e0, stream)
+    for _ in range(a.iters):
+        plan.run(batch, xd.ptr, yd.ptr, stream)
+    dev.event_record(e1, stream)
+    dev.event_sync(e1)
+    ms = dev.elapsed_ms(e0, e1) / a.iters
+    ops = 2.0 * macs
+    out = {"layer": desc, "kernel": plan.algo()[1], "us": ms * 1e3, "TOPS": ops / (ms * 1e-3) / 1e12,
+           "GBps": nbytes / (ms * 1e-3) / 1e9, "frac_mfma_peak": ops / (ms * 1e-3) / INT8_PEAK,
+           "frac_hbm_peak": nbytes / (ms * 1e-3) / HBM_PEAK, "ops": ops, "bytes": nbytes,
+           "arithmetic_intensity": ops / nbytes}
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -157,6 +157,17 @@ def small_conv_cases():
                             in_scale=0.0235, out_scale=0.0235, out_offset=0, act=RELU6))
     c.append(make_conv_case("s8_wide_64x64", 117, h=6, w=6, ci=64, co=64, act=RELU6))
     c.append(make_conv_case("s8_1x1_k128_n96", 118, h=5, w=5, ci=128, co=96, kh=1, kw=1))
+    # weight-stationary pointwise GEMM kernel: several tiles per wave, ragged M, every chunk depth
+    c.append(make_conv_case("pw_u8_k64_n128_m3200", 120, n=2, h=40, w=40, ci=64, co=128, kh=1, kw=1, in_dtype=U8, in_scale=0.0235,
+                            in_offset=0, out_scale=0.0235, out_offset=0, act=RELU6))
+    c.append(make_conv_case("pw_u8_k256_n512_m189", 121, n=3, h=9, w=7, ci=256, co=512, kh=1, kw=1, in_dtype=U8, in_scale=0.0235,
+                            in_offset=0, out_scale=0.0235, out_offset=0, act=RELU6))
+    c.append(make_conv_case("pw_s8_k32_n64_m12544", 122, n=1, h=112, w=112, ci=32, co=64, kh=1, kw=1, act=RELU6))
+    c.append(make_conv_case("pw_s8_k96_n48", 123, n=1, h=13, w=11, ci=96, co=48, kh=1, kw=1))
+    c.append(make_conv_case("pw_s8_k512_n32", 124, n=2, h=14, w=14, ci=512, co=32, kh=1, kw=1, in_offset=-128))
+    c.append(make_conv_case("pw_u8_k1024_n1024", 125, n=1, h=7, w=7, ci=1024, co=1024, kh=1, kw=1, in_dtype=U8, in_scale=0.0235,
+                            in_offset=0, out_scale=0.0235, out_offset=0, act=RELU6))
+    c.append(make_conv_case("pw_s8_stride2_not_pointwise", 126, n=1, h=14, w=14, ci=64, co=64, kh=1, kw=1, stride=(2, 2)))
     # depthwise
     c.append(make_conv_case("dw_u8_3x3_m1", 200, ci=16, depthwise=True, in_dtype=U8, in_scale=0.0235, in_offset=128,
                             out_scale=0.0235, out_offset=0, act=RELU6, w_scale_range=(0.01, 0.05)))
