@@ -163,8 +163,9 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             const float fm = mult[c] * inv;
             const float fb = biasf[c] * inv + zp_f;
             const float bq = std::fabs(biasf[c]) * inv;
-            // |r' - (reference quotient + offset)| <= 2^-24 * (5400 + 7 |biasf/s_out|) for in-range results; 1.5x margin
-            const float win = (8192.0f + 11.0f * bq) * (1.0f / 16777216.0f);
+            // constant part of the tie window (device_math.h): 1.5 * 2^-24 * (9 |offset| + 9 |biasf/s_out| + 64);
+            // the part proportional to |r'| is applied per value on the device
+            const float win = 1.5f * (9.0f * std::fabs(zp_f) + 9.0f * bq + 64.0f) * (1.0f / 16777216.0f);
             const bool ok = std::isfinite(fm) && std::isfinite(fb) && std::isfinite(win) && win < 0.25f &&
                             max_acc * std::fabs(static_cast<double>(fm)) < 268435456.0;
             if (!ok) continue;
@@ -330,7 +331,7 @@ void FoldCorrIntoTable(mi355x_conv2d_s* p, const std::vector<int32_t>& corr, int
         const float fm = tab[2 * CP + c];
         const float cq = static_cast<float>(corr[c]) * fm;
         const float fbc = tab[3 * CP + c] + cq;
-        const float win = (0.5f - tab[4 * CP + c]) + 11.0f * std::fabs(cq) * (1.0f / 16777216.0f);
+        const float win = (0.5f - tab[4 * CP + c]) + 1.5f * 7.0f * std::fabs(cq) * (1.0f / 16777216.0f);
         if (!std::isfinite(fbc) || !(win < 0.25f) || std::fabs(static_cast<double>(corr[c])) >= 16777216.0) continue;
         tab[5 * CP + c] = fbc;
         tab[6 * CP + c] = 0.5f - win;
@@ -375,19 +376,26 @@ int LaunchPw(const mi355x_conv2d_s* p, long long M, const void* x, void* y, hipS
     a.xor_mask = p->xor_mask;
     a.rq = p->rq;
     const int smem = PwSmemBytes<BN>(g.Ci);
-    const int per_cu = std::max(1, std::min(4, (160 * 1024) / smem));
-    const long long groups = ((M + 31) / 32 + 3) / 4;
-    long long gm = (256ll * per_cu) / a.n_slabs;
-    if (gm < 1) gm = 1;
-    if (gm > groups) gm = groups;
-    a.gm = static_cast<int>(gm);
     auto kernel = PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2)>;
-    static bool attr_set = false;       // one flag per instantiation
-    if (!attr_set)
+    // one residency query per instantiation and K: how many blocks a CU holds at once (registers and LDS)
+    static int cached_k = -1, cached_per_cu = 1, n_cu = 256;
+    if (cached_k != g.Ci)
     {
         MI355X_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-        attr_set = true;
+        int per_cu = 1, dev = 0;
+        MI355X_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, smem));
+        MI355X_HIP(hipGetDevice(&dev));
+        MI355X_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+        cached_per_cu = std::max(1, per_cu);
+        cached_k = g.Ci;
     }
+    // exactly one resident wave of blocks: every block walks its share of the row tiles
+    const long long groups = ((M + 31) / 32 + 3) / 4;
+    long long gm = (static_cast<long long>(n_cu) * cached_per_cu) / a.n_slabs;
+    gm = gm / 8 * 8;                // the kernel deals groups out to the 8 XCDs
+    if (gm < 8) gm = 8;
+    if (gm > (groups + 7) / 8 * 8) gm = (groups + 7) / 8 * 8;
+    a.gm = static_cast<int>(gm);
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(a.n_slabs * gm)), dim3(256), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;

@@ -31,23 +31,32 @@ __device__ __forceinline__ int RequantExactDev(int acc, float mult, float biasf,
     return QuantizeDev(__fadd_rn(__fmul_rn(static_cast<float>(acc), mult), biasf), rq);
 }
 
-// Per-channel constants, five rows of `stride` floats (see ChannelTable on the host side):
+// Per-channel constants, seven rows of `stride` floats, built on the host (conv.hip):
 //   row 0 mult   s_in * s_w[c]                      row 1 biasf  float(bias[c]) * s_b[c]
 //   row 2 fm     fl(mult * fl(1/s_out))             row 3 fb     fl(fl(biasf * fl(1/s_out)) + offset)
-//   row 4 thr    0.5 - window[c]   (negative: channel always takes the exact path)
+//   row 4 thr    tie threshold for rows 2/3 (negative: the channel always takes the exact path)
+//   row 5 fbc    fb + corr * fm                     row 6 thrc   tie threshold for rows 2/5
+// Rows 5/6 serve kernels whose accumulators start at zero: the zero-point correction corr[c] is then part of the
+// fast-path constant, and only the exact path adds it to the accumulator as an integer.
 struct ChanTab
 {
     const float* p;
     int stride;
 };
 
-// Fast path with an exact fallback.  r' = fma(float(acc), fm, fb) approximates f/s_out + offset with an absolute
-// error below window[c] = 2^-19 * (|biasf/s_out| + 1024) whenever the exact result is within the 8-bit range
-// (three roundings of the reference, the coefficient roundings and the fma rounding, each 2^-24 relative to
-// magnitudes bounded by |biasf/s_out| + 767).  So r' and the reference can round to different integers only when
-// r' is within window[c] of a half-integer; exactly those values are recomputed the reference's way.
-// Results beyond the 8-bit range clamp alike on both paths.  Round-half-even (v_rndne) serves on the fast path:
-// it differs from round-half-away only at exact ties, which are inside the window.
+// Fast path with an exact fallback.
+//   r' = fma(float(acc), fm, fb) approximates  t = f/s_out + offset  (f = the reference's fp32 value).  Counting every
+//   rounding on both sides (three in the reference; the reciprocal, two coefficient products, the offset add and the
+//   fma on ours), each relative 2^-24 to a magnitude bounded through |r'|, one gets
+//       |r' - (fl(f/s_out) + offset)|  <=  2^-24 * (8 |r'| + 9 |offset| + 9 |biasf/s_out| + 7 |corr*fm|)
+//   (this includes the int32 -> fp32 conversion of accumulators beyond 2^24 on either path).
+//   The two can therefore round to different integers only when r' lies that close to a half-integer.  The test
+//       |r' - rint(r')|  <=  thr[c] - kTieSlope * |r'|,    thr[c] = 0.5 - 1.5 * 2^-24 * (9|offset| + 9|biasf/s_out| + 7|corr*fm| + 64)
+//   (1.5x margin on every term) passes everything else; values that fail it -- a few in 10^4 -- are recomputed with
+//   the reference's own sequence.  Results beyond the 8-bit range clamp alike on both paths.  Round-half-even
+//   (v_rndne) serves on the fast path: it differs from round-half-away only at exact ties, which fail the test.
+constexpr float kTieSlope = 12.0f / 16777216.0f;
+
 __device__ __forceinline__ uint32_t Pack4(int q0, int q1, int q2, int q3)
 {
     // four codes -> one dword (byte 0 = q0), three v_perm_b32
@@ -70,34 +79,34 @@ __device__ __forceinline__ Fast4 LoadFast4(const ChanTab& ct, int c)
     return f;
 }
 
-#define MI355X_FAST1(ACC, M, B, K, E)                                   \
-    {                                                                   \
-        const float r_ = __fmaf_rn(static_cast<float>(ACC), M, B);      \
-        K = __builtin_rintf(r_);                                        \
-        E = __fsub_rn(r_, K);                                           \
+// K = rint(r'), SLOW = the value needs the exact path ("not <=" also catches NaN)
+#define MI355X_FAST1(ACC, M, B, T, K, SLOW)                                   \
+    {                                                                         \
+        const float r_ = __fmaf_rn(static_cast<float>(ACC), M, B);            \
+        K = __builtin_rintf(r_);                                              \
+        const float e_ = __fsub_rn(r_, K);                                    \
+        SLOW = !(fabsf(e_) <= __fmaf_rn(fabsf(r_), -kTieSlope, T));           \
     }
 
 // Four consecutive channels c..c+3 of one pixel -> packed dword.
-//   `corr` (may be null) is an integer added to the accumulator on the exact path only: kernels that start their
-//   accumulators at zero use channel-table rows whose fast-path constants already contain corr * fm.
-// The fast path is branch-free (7 VALU instructions per value); the four flags are combined as wave masks, and
-// only when some lane of the wave has a value inside its tie window does the wave enter the fix-up loop, which
-// evaluates one flagged value per lane and pass.
+//   `corr` (may be null) is an integer added to the accumulator on the exact path only (rows 5/6, see ChanTab).
+// The fast path is branch-free (8 VALU instructions per value); the four flags are combined as wave masks, and
+// only when some lane of the wave has a flagged value does the wave enter the fix-up loop, which evaluates one
+// flagged value per lane and pass.
 __device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const float4& fm, const float4& fb,
                                                 const float4& thr, const ChanTab& ct, const int32_t* corr, int c,
                                                 const Requant& rq)
 {
-    float k0, k1, k2, k3, e0, e1, e2, e3;
-    MI355X_FAST1(a0, fm.x, fb.x, k0, e0)
-    MI355X_FAST1(a1, fm.y, fb.y, k1, e1)
-    MI355X_FAST1(a2, fm.z, fb.z, k2, e2)
-    MI355X_FAST1(a3, fm.w, fb.w, k3, e3)
+    float k0, k1, k2, k3;
+    bool s0, s1, s2, s3;
+    MI355X_FAST1(a0, fm.x, fb.x, thr.x, k0, s0)
+    MI355X_FAST1(a1, fm.y, fb.y, thr.y, k1, s1)
+    MI355X_FAST1(a2, fm.z, fb.z, thr.z, k2, s2)
+    MI355X_FAST1(a3, fm.w, fb.w, thr.w, k3, s3)
     int q0 = static_cast<int>(__builtin_amdgcn_fmed3f(k0, rq.act_lo_f, rq.act_hi_f));
     int q1 = static_cast<int>(__builtin_amdgcn_fmed3f(k1, rq.act_lo_f, rq.act_hi_f));
     int q2 = static_cast<int>(__builtin_amdgcn_fmed3f(k2, rq.act_lo_f, rq.act_hi_f));
     int q3 = static_cast<int>(__builtin_amdgcn_fmed3f(k3, rq.act_lo_f, rq.act_hi_f));
-    // "not (|e| <= thr)" also sends NaN to the exact path
-    const bool s0 = !(fabsf(e0) <= thr.x), s1 = !(fabsf(e1) <= thr.y), s2 = !(fabsf(e2) <= thr.z), s3 = !(fabsf(e3) <= thr.w);
     const unsigned long long any = __builtin_amdgcn_ballot_w64(s0) | __builtin_amdgcn_ballot_w64(s1) |
                                    __builtin_amdgcn_ballot_w64(s2) | __builtin_amdgcn_ballot_w64(s3);
     if (__builtin_expect(any != 0, 0))
@@ -134,25 +143,25 @@ __device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, 
 // one channel (scalar kernels)
 __device__ __forceinline__ int Requant1Dev(int acc, const ChanTab& ct, int c, const Requant& rq)
 {
-    float k, e;
-    MI355X_FAST1(acc, ct.p[2 * ct.stride + c], ct.p[3 * ct.stride + c], k, e)
-    if (__builtin_expect(!(fabsf(e) <= ct.p[4 * ct.stride + c]), 0))
-        return RequantExactDev(acc, ct.p[c], ct.p[ct.stride + c], rq);
+    float k;
+    bool slow;
+    MI355X_FAST1(acc, ct.p[2 * ct.stride + c], ct.p[3 * ct.stride + c], ct.p[4 * ct.stride + c], k, slow)
+    if (__builtin_expect(slow, 0)) return RequantExactDev(acc, ct.p[c], ct.p[ct.stride + c], rq);
     return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.act_lo_f, rq.act_hi_f));
 }
 
 // value already in float (pooling, add, ...): reciprocal fast path with the exact fallback near ties.
-//   r' = fma(f, fl(1/scale), offset) is within (|r| + |r'|) * 2^-24 of f/scale + offset; for |f/scale| <= 512 that is
-//   below 2^-12, and beyond it both paths clamp alike (|offset| <= 255 is checked on the host, else fast_ok = 0).
-constexpr float kTieWindow = 1.0f / 2048.0f;
-
+//   r' = fma(f, fl(1/scale), offset) is within 2^-24 * (|f/scale| + |r'|) of f/scale + offset and the correctly rounded
+//   quotient within 2^-24 * |f/scale|; |offset| <= 255 is checked on the host (else fast_ok = 0).
 __device__ __forceinline__ int QuantizeFastDev(float f, const Requant& rq)
 {
     if (!rq.fast_ok) return QuantizeDev(f, rq);
     const float r = __fmaf_rn(f, rq.inv_scale, rq.out_offset_f);
     const float k = __builtin_rintf(r);
     const float e = __fsub_rn(r, k);
-    if (__builtin_expect(!(fabsf(e) <= 0.5f - kTieWindow), 0)) return QuantizeDev(f, rq);
+    // 3 |r'| + 2 |offset| <= 3 |r'| + 510, with the same 1.5x margin as above
+    if (__builtin_expect(!(fabsf(e) <= __fmaf_rn(fabsf(r), -4.5f / 16777216.0f, 0.5f - 1024.0f / 16777216.0f)), 0))
+        return QuantizeDev(f, rq);
     return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.act_lo_f, rq.act_hi_f));
 }
 

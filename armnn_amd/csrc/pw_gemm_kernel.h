@@ -16,6 +16,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "conv_kernels.h"
 #include "device_math.h"
@@ -58,30 +60,14 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
     const int tid = threadIdx.x;
     const int lane = tid & 63;
     const int wave = tid >> 6;
-    const int slab_id = blockIdx.x % a.n_slabs;
-    const int g = blockIdx.x / a.n_slabs;
+    // Consecutive block ids land on different XCDs (8 per device, each with its own L2).  All slabs of one group of
+    // activation rows are given to the same XCD, so those rows cross the fabric once and are then served from that
+    // XCD's L2; the (small) weight slabs are what gets replicated.
+    const int xcd = blockIdx.x & 7;
+    const int local = blockIdx.x >> 3;
+    const int slab_id = local % a.n_slabs;
+    const int g = (local / a.n_slabs) * 8 + xcd;
     const int n0 = slab_id * BN;
-
-    // ---- prologue: weight slab and epilogue constants into LDS (loads batched per column of chunks) ---------
-    {
-        const int chunks = a.K >> 4;
-        const int8_t* src = a.w + static_cast<long long>(n0 + (tid >> 4)) * a.w_stride;
-        for (int c = tid & 15; c < chunks; c += 16)
-        {
-            v4i t[BN / 16];
-#pragma unroll
-            for (int i = 0; i < BN / 16; ++i) t[i] = *reinterpret_cast<const v4i*>(src + static_cast<long long>(16 * i) * a.w_stride + c * 16);
-#pragma unroll
-            for (int i = 0; i < BN / 16; ++i) *reinterpret_cast<v4i*>(slab + ((tid >> 4) + 16 * i) * LDW + c * 16) = t[i];
-        }
-        for (int i = tid; i < 3 * BN; i += 256)
-        {
-            const int row = i / BN, c = i - row * BN;
-            const int src_row = row == 0 ? 2 : row == 1 ? 5 : 6;
-            cst[i] = a.ct.p[src_row * a.ct.stride + n0 + c];
-        }
-    }
-    __syncthreads();
 
     uint8_t* ostage = ostage_all + wave * 32 * LDO;
     const int n_tiles = (a.M + 31) >> 5;
@@ -91,7 +77,6 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
     const int xm = static_cast<int>(a.xor_mask);
     const int tile_step = a.gm * 4;
     const int tile0 = g * 4 + wave;              // first tile of this wave
-    if (tile0 >= n_tiles) return;
 
     v16i acc[TC];
 #pragma unroll
@@ -182,6 +167,7 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
     };
 
     // ---- software pipeline over (tile, chunk): NB-1 chunks are in flight while one feeds the MFMAs --------------
+    // The first activation loads are issued before the weight slab is fetched, so both latencies overlap.
     v4i buf[NB][KS];
     int t_cur = tile0, c_cur = 0;                // chunk being computed
     int t_nxt = tile0, c_nxt = 0;                // next chunk to load
@@ -193,21 +179,52 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
     {
         if (t_nxt < n_tiles) { load_chunk(buf[j], t_nxt, c_nxt); advance(t_nxt, c_nxt); }
     }
-    bool done = false;
-    while (!done)
+
+    // ---- prologue: weight slab and epilogue constants into LDS (loads batched per column of chunks) ---------
     {
-#pragma unroll
-        for (int j = 0; j < NB; ++j)
+        const int chunks = a.K >> 4;
+        const int8_t* src = a.w + static_cast<long long>(n0 + (tid >> 4)) * a.w_stride;
+        for (int c = tid & 15; c < chunks; c += 16)
         {
-            if (!done)
-            {
-                if (t_nxt < n_tiles) { load_chunk(buf[(j + NB - 1) % NB], t_nxt, c_nxt); advance(t_nxt, c_nxt); }
-                compute_chunk(buf[j], c_cur);
-                if (c_cur == nch - 1) epilogue(t_cur);
-                advance(t_cur, c_cur);
-                done = t_cur >= n_tiles;
-            }
+            v4i t[BN / 16];
+#pragma unroll
+            for (int i = 0; i < BN / 16; ++i) t[i] = *reinterpret_cast<const v4i*>(src + static_cast<long long>(16 * i) * a.w_stride + c * 16);
+#pragma unroll
+            for (int i = 0; i < BN / 16; ++i) *reinterpret_cast<v4i*>(slab + ((tid >> 4) + 16 * i) * LDW + c * 16) = t[i];
         }
+        for (int i = tid; i < 3 * BN; i += 256)
+        {
+            const int row = i / BN, c = i - row * BN;
+            const int src_row = row == 0 ? 2 : row == 1 ? 5 : 6;
+            cst[i] = a.ct.p[src_row * a.ct.stride + n0 + c];
+        }
+    }
+    __syncthreads();
+    if (tile0 >= n_tiles) return;
+
+    // One loop iteration = one chunk.  The buffer index is wave-uniform; dispatching on it keeps every register
+    // index static while the epilogue appears only once in the code.
+    static_assert(NB == 2 || NB == 4, "2 or 4 register chunks");
+    int j = 0;
+    while (t_cur < n_tiles)
+    {
+        const bool more = t_nxt < n_tiles;
+        auto step = [&](auto jc) {
+            constexpr int J = decltype(jc)::value;
+            if (more) load_chunk(buf[(J + NB - 1) % NB], t_nxt, c_nxt);
+            compute_chunk(buf[J], c_cur);
+        };
+        if (j == 0) step(std::integral_constant<int, 0>{});
+        else if (j == 1) step(std::integral_constant<int, 1>{});
+        else if constexpr (NB == 4)
+        {
+            if (j == 2) step(std::integral_constant<int, 2>{});
+            else step(std::integral_constant<int, 3>{});
+        }
+        if (more) advance(t_nxt, c_nxt);
+        j = (j + 1 == NB) ? 0 : j + 1;
+        if (c_cur == nch - 1) epilogue(t_cur);
+        advance(t_cur, c_cur);
     }
 }
 
