@@ -1,0 +1,86 @@
+// Minimal host core: layer descriptors with the member names of include/armnn/Descriptors.hpp.
+#pragma once
+#include "Tensor.hpp"
+#include "Types.hpp"
+
+namespace armnn
+{
+struct BaseDescriptor
+{
+    virtual bool IsNull() const { return false; }
+    virtual ~BaseDescriptor() = default;
+};
+struct NullDescriptor : BaseDescriptor
+{
+    bool IsNull() const override { return true; }
+};
+
+struct ActivationDescriptor : BaseDescriptor
+{
+    ActivationDescriptor() = default;
+    ActivationDescriptor(ActivationFunction fn, float a = 0, float b = 0) : m_Function(fn), m_A(a), m_B(b) {}
+    bool operator==(const ActivationDescriptor& rhs) const { return m_Function == rhs.m_Function && m_A == rhs.m_A && m_B == rhs.m_B; }
+    ActivationFunction m_Function = ActivationFunction::Sigmoid;
+    float m_A = 0;   ///< upper bound for BoundedReLu
+    float m_B = 0;   ///< lower bound for BoundedReLu
+};
+
+struct Convolution2dDescriptor : BaseDescriptor
+{
+    uint32_t GetNumInputs() const { return m_BiasEnabled ? 3u : 2u; }
+    uint32_t m_PadLeft = 0, m_PadRight = 0, m_PadTop = 0, m_PadBottom = 0;
+    uint32_t m_StrideX = 1, m_StrideY = 1;
+    uint32_t m_DilationX = 1, m_DilationY = 1;
+    bool m_BiasEnabled = false;
+    DataLayout m_DataLayout = DataLayout::NCHW;
+};
+
+struct DepthwiseConvolution2dDescriptor : BaseDescriptor
+{
+    uint32_t GetNumInputs() const { return m_BiasEnabled ? 3u : 2u; }
+    uint32_t m_PadLeft = 0, m_PadRight = 0, m_PadTop = 0, m_PadBottom = 0;
+    uint32_t m_StrideX = 1, m_StrideY = 1;
+    uint32_t m_DilationX = 1, m_DilationY = 1;
+    bool m_BiasEnabled = false;
+    DataLayout m_DataLayout = DataLayout::NCHW;
+};
+
+struct FullyConnectedDescriptor : BaseDescriptor
+{
+    uint32_t GetNumInputs() const { return m_BiasEnabled ? 3u : 2u; }
+    bool m_BiasEnabled = false;
+    bool m_TransposeWeightMatrix = false;
+    bool m_ConstantWeights = true;
+};
+
+struct Pooling2dDescriptor : BaseDescriptor
+{
+    PoolingAlgorithm m_PoolType = PoolingAlgorithm::Max;
+    uint32_t m_PadLeft = 0, m_PadRight = 0, m_PadTop = 0, m_PadBottom = 0;
+    uint32_t m_PoolWidth = 0, m_PoolHeight = 0;
+    uint32_t m_StrideX = 0, m_StrideY = 0;
+    OutputShapeRounding m_OutputShapeRounding = OutputShapeRounding::Floor;
+    PaddingMethod m_PaddingMethod = PaddingMethod::Exclude;
+    DataLayout m_DataLayout = DataLayout::NCHW;
+};
+
+struct SoftmaxDescriptor : BaseDescriptor
+{
+    float m_Beta = 1.0f;
+    int m_Axis = -1;
+};
+
+struct ElementwiseBinaryDescriptor : BaseDescriptor
+{
+    ElementwiseBinaryDescriptor() = default;
+    ElementwiseBinaryDescriptor(BinaryOperation op) : m_Operation(op) {}
+    BinaryOperation m_Operation = BinaryOperation::Add;
+};
+
+struct ReshapeDescriptor : BaseDescriptor
+{
+    ReshapeDescriptor() = default;
+    ReshapeDescriptor(const TensorShape& shape) : m_TargetShape(shape) {}
+    TensorShape m_TargetShape;
+};
+} // namespace armnn

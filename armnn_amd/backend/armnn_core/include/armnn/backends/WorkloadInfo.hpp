@@ -1,0 +1,15 @@
+// Minimal host core: include/armnn/backends/WorkloadInfo.hpp:16-36.
+#pragma once
+#include "../Optional.hpp"
+#include "../Tensor.hpp"
+#include <string>
+#include <vector>
+namespace armnn
+{
+struct WorkloadInfo
+{
+    std::vector<TensorInfo> m_InputTensorInfos;
+    std::vector<TensorInfo> m_OutputTensorInfos;
+    std::string m_Name;
+};
+} // namespace armnn

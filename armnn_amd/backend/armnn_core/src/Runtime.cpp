@@ -1,0 +1,359 @@
+// Minimal host core: IRuntime -- backend discovery, LoadNetwork (tensor handles, workloads, constants), and
+// EnqueueWorkload (src/armnn/Runtime.cpp:301-574, src/armnn/LoadedNetwork.cpp:82-360 and :845-1100).
+#include <Layer.hpp>
+#include <armnn/BackendRegistry.hpp>
+#include <armnn/IRuntime.hpp>
+#include <armnn/backends/DynamicBackend.hpp>
+#include <armnn/backends/IBackendInternal.hpp>
+#include <armnn/backends/TensorHandleFactoryRegistry.hpp>
+#include <armnn/backends/WorkloadFactory.hpp>
+
+#include <cstring>
+#include <iostream>
+#include <map>
+#include <mutex>
+
+namespace armnn
+{
+namespace
+{
+class DeviceSpec final : public IDeviceSpec
+{
+public:
+    const BackendIdSet& GetSupportedBackends() const override { return m_Supported; }
+    BackendIdSet m_Supported;
+    BackendIdSet m_Dynamic;
+};
+
+struct BackendSlot
+{
+    IBackendInternalUniquePtr backend;
+    IBackendInternal::IWorkloadFactoryPtr factory;
+    ITensorHandleFactory* handleFactory = nullptr;   // preferred tensor handle factory, null: use the workload factory
+};
+
+class LoadedNetwork
+{
+public:
+    LoadedNetwork(IOptimizedNetworkPtr net) : m_Net(std::move(net))
+    {
+        Graph& graph = m_Net->GetGraph();
+        m_Order = graph.TopologicalSort();
+
+        // one backend object, handle factory and workload factory per backend in use (LoadedNetwork.cpp:169-260)
+        for (Layer* l : m_Order)
+        {
+            const BackendId& id = l->GetBackendId();
+            if (m_Backends.count(id)) continue;
+            BackendSlot slot;
+            slot.backend = BackendRegistryInstance().GetFactory(id)();
+            if (slot.backend->SupportsTensorAllocatorAPI())
+            {
+                slot.backend->RegisterTensorHandleFactories(m_Registry);
+                slot.factory = slot.backend->CreateWorkloadFactory(m_Registry, m_Net->GetModelOptions());
+                slot.handleFactory = m_Registry.GetFactory(slot.backend->GetHandleFactoryPreferences().front());
+            }
+            else
+            {
+                IBackendInternal::IMemoryManagerSharedPtr mm = slot.backend->CreateMemoryManager();
+                if (mm) m_Registry.RegisterMemoryManager(mm);
+                slot.factory = slot.backend->CreateWorkloadFactory(mm, m_Net->GetModelOptions());
+            }
+            if (!slot.factory) throw RuntimeException("backend " + id.Get() + " returned no workload factory");
+            m_Backends.emplace(id, std::move(slot));
+        }
+
+        // Tensor handles in execution order.  Manage() opens a tensor's lifetime when its producer is reached and
+        // Allocate() closes it after its last consumer, so a pooling memory manager can overlap tensors whose
+        // lifetimes do not (LoadedNetwork.cpp:262-330, Layer::CreateTensorHandles).  Constants and network inputs
+        // live for the whole network and are not managed.
+        std::map<const OutputSlot*, unsigned int> remaining;
+        for (Layer* l : m_Order)
+        {
+            BackendSlot& slot = m_Backends.at(l->GetBackendId());
+            const bool managed = l->GetType() != LayerType::Constant && l->GetType() != LayerType::Input;
+            for (unsigned int o = 0; o < l->GetNumOutputSlots(); ++o)
+            {
+                OutputSlot& out = l->Out(o);
+                std::unique_ptr<ITensorHandle> h = slot.handleFactory ? slot.handleFactory->CreateTensorHandle(out.GetTensorInfo(), managed)
+                                                                      : slot.factory->CreateTensorHandle(out.GetTensorInfo(), managed);
+                if (!h) throw RuntimeException(std::string("no tensor handle for layer ") + l->GetName());
+                // a tensor read by a network output must survive until the caller has copied it out
+                bool pinned = !managed;
+                for (InputSlot* c : out.GetConnections()) pinned |= c->GetOwningLayer().GetType() == LayerType::Output;
+                if (managed) h->Manage();
+                out.SetTensorHandle(std::move(h));
+                remaining[&out] = pinned ? ~0u : out.GetNumConnections();
+                if (!managed || out.GetNumConnections() == 0 || pinned) m_AllocateLast.push_back(out.GetTensorHandle());
+            }
+            CreateWorkloadFor(*l, slot);
+            for (unsigned int i = 0; i < l->GetNumInputSlots(); ++i)
+            {
+                const OutputSlot* src = l->In(i).GetConnectedOutputSlot();
+                unsigned int& r = remaining[src];
+                if (r != ~0u && --r == 0) src->GetTensorHandle()->Allocate();
+            }
+        }
+        for (ITensorHandle* h : m_AllocateLast) h->Allocate();
+        m_AllocateLast.clear();
+
+        m_Registry.AquireMemory();
+        for (auto& w : m_Constants) w->PostAllocationConfigure();
+        for (auto& w : m_Workloads) w->PostAllocationConfigure();
+        for (auto& b : m_Backends) b.second.factory->AfterWorkloadsCreated();
+        // constant layers produce their output once (LoadedNetwork.cpp:342-357)
+        for (auto& w : m_Constants) w->Execute();
+    }
+
+    ~LoadedNetwork()
+    {
+        m_Constants.clear();
+        m_Workloads.clear();
+        m_Registry.ReleaseMemory();
+    }
+
+    const Layer* FindBinding(LayerType type, LayerBindingId id) const
+    {
+        for (const Layer* l : m_Order)
+            if (l->GetType() == type && l->GetBindingId() == id) return l;
+        return nullptr;
+    }
+
+    TensorInfo GetInputTensorInfo(LayerBindingId id) const
+    {
+        const Layer* l = FindBinding(LayerType::Input, id);
+        if (!l) throw InvalidArgumentException("No input layer is associated with id " + std::to_string(id));
+        return l->Out(0).GetTensorInfo();
+    }
+    TensorInfo GetOutputTensorInfo(LayerBindingId id) const
+    {
+        const Layer* l = FindBinding(LayerType::Output, id);
+        if (!l) throw InvalidArgumentException("No output layer is associated with id " + std::to_string(id));
+        return l->In(0).GetConnectedOutputSlot()->GetTensorInfo();
+    }
+
+    Status Enqueue(const InputTensors& inputs, const OutputTensors& outputs)
+    {
+        if (inputs.size() != m_Net->GetNumInputs()) throw InvalidArgumentException("Number of inputs provided does not match network.");
+        if (outputs.size() != m_Net->GetNumOutputs()) throw InvalidArgumentException("Number of outputs provided does not match network.");
+        std::lock_guard<std::mutex> lock(m_Mutex);
+        for (const auto& in : inputs)
+        {
+            const Layer* l = FindBinding(LayerType::Input, in.first);
+            if (!l) throw InvalidArgumentException("No input layer is associated with id " + std::to_string(in.first));
+            const TensorInfo& info = l->Out(0).GetTensorInfo();
+            if (in.second.GetNumBytes() != info.GetNumBytes()) throw InvalidArgumentException("Input tensor size does not match the network's");
+            ITensorHandle* h = l->Out(0).GetTensorHandle();
+            void* dst = h->Map();
+            std::memcpy(dst, in.second.GetMemoryArea(), info.GetNumBytes());
+            h->Unmap();
+        }
+        for (auto& w : m_Workloads) w->Execute();
+        for (const auto& out : outputs)
+        {
+            const Layer* l = FindBinding(LayerType::Output, out.first);
+            if (!l) throw InvalidArgumentException("No output layer is associated with id " + std::to_string(out.first));
+            const OutputSlot* src = l->In(0).GetConnectedOutputSlot();
+            if (out.second.GetNumBytes() != src->GetTensorInfo().GetNumBytes()) throw InvalidArgumentException("Output tensor size does not match the network's");
+            const ITensorHandle* h = src->GetTensorHandle();
+            const void* p = h->Map();
+            std::memcpy(out.second.GetMemoryArea(), p, src->GetTensorInfo().GetNumBytes());
+            h->Unmap();
+        }
+        return Status::Success;
+    }
+
+private:
+    template <typename Desc>
+    void Fill(Desc& d, WorkloadInfo& info, Layer& l)
+    {
+        for (unsigned int i = 0; i < l.GetNumInputSlots(); ++i)
+        {
+            const OutputSlot* src = l.In(i).GetConnectedOutputSlot();
+            d.m_Inputs.push_back(src->GetTensorHandle());
+            info.m_InputTensorInfos.push_back(src->GetTensorInfo());
+        }
+        for (unsigned int o = 0; o < l.GetNumOutputSlots(); ++o)
+        {
+            d.m_Outputs.push_back(l.Out(o).GetTensorHandle());
+            info.m_OutputTensorInfos.push_back(l.Out(o).GetTensorInfo());
+        }
+        d.m_AdditionalInfoObject = l.GetAdditionalInformation<void>().get();
+        info.m_Name = l.GetNameStr();
+    }
+
+    template <typename Desc, typename Params>
+    std::unique_ptr<IWorkload> Make(Layer& l, BackendSlot& slot)
+    {
+        Desc d;
+        WorkloadInfo info;
+        Fill(d, info, l);
+        d.m_Parameters = static_cast<const Params&>(l.GetParameters());
+        return slot.factory->CreateWorkload(l.GetType(), d, info);
+    }
+
+    void CreateWorkloadFor(Layer& l, BackendSlot& slot)
+    {
+        std::unique_ptr<IWorkload> w;
+        switch (l.GetType())
+        {
+            case LayerType::Input:
+            case LayerType::Output:
+                return;   // the runtime itself moves data between caller memory and the bound tensor handles
+            case LayerType::Constant:
+            {
+                ConstantQueueDescriptor d;
+                WorkloadInfo info;
+                Fill(d, info, l);
+                d.m_LayerOutput = l.m_LayerOutput.get();
+                w = slot.factory->CreateWorkload(LayerType::Constant, d, info);
+                if (!w) throw RuntimeException(std::string("No workload created for layer (name: '") + l.GetName() + "' type: 'Constant')");
+                m_Constants.push_back(std::move(w));
+                return;
+            }
+            case LayerType::MemCopy:
+            {
+                MemCopyQueueDescriptor d;
+                WorkloadInfo info;
+                Fill(d, info, l);
+                w = slot.factory->CreateWorkload(LayerType::MemCopy, d, info);
+                break;
+            }
+            case LayerType::Convolution2d: w = Make<Convolution2dQueueDescriptor, Convolution2dDescriptor>(l, slot); break;
+            case LayerType::DepthwiseConvolution2d: w = Make<DepthwiseConvolution2dQueueDescriptor, DepthwiseConvolution2dDescriptor>(l, slot); break;
+            case LayerType::FullyConnected: w = Make<FullyConnectedQueueDescriptor, FullyConnectedDescriptor>(l, slot); break;
+            case LayerType::Activation: w = Make<ActivationQueueDescriptor, ActivationDescriptor>(l, slot); break;
+            case LayerType::Pooling2d: w = Make<Pooling2dQueueDescriptor, Pooling2dDescriptor>(l, slot); break;
+            case LayerType::Softmax: w = Make<SoftmaxQueueDescriptor, SoftmaxDescriptor>(l, slot); break;
+            case LayerType::ElementwiseBinary: w = Make<ElementwiseBinaryQueueDescriptor, ElementwiseBinaryDescriptor>(l, slot); break;
+            case LayerType::Reshape: w = Make<ReshapeQueueDescriptor, ReshapeDescriptor>(l, slot); break;
+        }
+        if (!w)
+            throw RuntimeException(std::string("No workload created for layer (name: '") + l.GetName() + "' type: '" +
+                                   GetLayerTypeAsCString(l.GetType()) + "' backend: '" + l.GetBackendId().Get() + "')");
+        m_Workloads.push_back(std::move(w));
+    }
+
+    IOptimizedNetworkPtr m_Net;
+    std::vector<Layer*> m_Order;
+    TensorHandleFactoryRegistry m_Registry;
+    std::map<BackendId, BackendSlot> m_Backends;
+    std::vector<std::unique_ptr<IWorkload>> m_Constants;
+    std::vector<std::unique_ptr<IWorkload>> m_Workloads;
+    std::vector<ITensorHandle*> m_AllocateLast;
+    std::mutex m_Mutex;
+};
+} // namespace
+
+class RuntimeImpl
+{
+public:
+    explicit RuntimeImpl(const IRuntime::CreationOptions& options)
+    {
+        // dynamic backends first, so they are part of the registry scan (Runtime.cpp:655-676)
+        if (!options.m_DynamicBackendsPath.empty())
+            m_DeviceSpec.m_Dynamic = DynamicBackendUtils::RegisterDynamicBackends(DynamicBackendUtils::GetSharedObjects(options.m_DynamicBackendsPath));
+        // a backend whose context cannot be created is not offered to Optimize (Runtime.cpp:377-470)
+        for (const BackendId& id : BackendRegistryInstance().GetBackendIds())
+        {
+            try
+            {
+                auto backend = BackendRegistryInstance().GetFactory(id)();
+                auto context = backend->CreateBackendContext(options);
+                if (context) m_Contexts.emplace(id, std::move(context));
+                m_DeviceSpec.m_Supported.insert(id);
+            }
+            catch (const BackendUnavailableException& e)
+            {
+                std::cerr << "armnn: backend " << id << " is unavailable and ignored: " << e.what() << "\n";
+            }
+        }
+    }
+
+    ~RuntimeImpl()
+    {
+        m_Networks.clear();
+        m_Contexts.clear();
+        for (const BackendId& id : m_DeviceSpec.m_Dynamic) BackendRegistryInstance().Deregister(id);
+    }
+
+    Status LoadNetwork(NetworkId& idOut, IOptimizedNetworkPtr network, std::string& error)
+    {
+        const NetworkId id = m_NextId++;
+        idOut = id;
+        for (auto& c : m_Contexts) c.second->BeforeLoadNetwork(id);
+        try
+        {
+            m_Networks[id] = std::make_unique<LoadedNetwork>(std::move(network));
+        }
+        catch (const Exception& e)
+        {
+            error = e.what();
+            m_Networks.erase(id);
+            return Status::Failure;
+        }
+        for (auto& c : m_Contexts) c.second->AfterLoadNetwork(id);
+        return Status::Success;
+    }
+
+    LoadedNetwork& Get(NetworkId id) const
+    {
+        auto it = m_Networks.find(id);
+        if (it == m_Networks.end()) throw InvalidArgumentException("Unknown network id " + std::to_string(id));
+        return *it->second;
+    }
+
+    Status Enqueue(NetworkId id, const InputTensors& in, const OutputTensors& out)
+    {
+        LoadedNetwork& net = Get(id);
+        Status s = Status::Failure;
+        try
+        {
+            s = net.Enqueue(in, out);
+        }
+        catch (const RuntimeException& e)
+        {
+            // a failing workload ends the inference, not the process (LoadedNetwork.cpp:1088-1100)
+            std::cerr << "armnn: an error occurred attempting to execute a workload: " << e.what() << "\n";
+            return Status::Failure;
+        }
+        for (auto& c : m_Contexts) c.second->AfterEnqueueWorkload(id);
+        return s;
+    }
+
+    Status Unload(NetworkId id)
+    {
+        for (auto& c : m_Contexts) c.second->BeforeUnloadNetwork(id);
+        const bool erased = m_Networks.erase(id) != 0;
+        for (auto& c : m_Contexts) c.second->AfterUnloadNetwork(id);
+        return erased ? Status::Success : Status::Failure;
+    }
+
+    DeviceSpec m_DeviceSpec;
+private:
+    std::map<BackendId, IBackendInternal::IBackendContextPtr> m_Contexts;
+    std::map<NetworkId, std::unique_ptr<LoadedNetwork>> m_Networks;
+    NetworkId m_NextId = 0;
+};
+
+IRuntime::IRuntime(const CreationOptions& options) : pRuntimeImpl(new RuntimeImpl(options)) {}
+IRuntime::~IRuntime() = default;
+IRuntime* IRuntime::CreateRaw(const CreationOptions& options) { return new IRuntime(options); }
+IRuntimePtr IRuntime::Create(const CreationOptions& options) { return IRuntimePtr(CreateRaw(options), &IRuntime::Destroy); }
+void IRuntime::Destroy(IRuntime* runtime) { delete runtime; }
+Status IRuntime::LoadNetwork(NetworkId& id, IOptimizedNetworkPtr network)
+{
+    std::string ignored;
+    return pRuntimeImpl->LoadNetwork(id, std::move(network), ignored);
+}
+Status IRuntime::LoadNetwork(NetworkId& id, IOptimizedNetworkPtr network, std::string& error) { return pRuntimeImpl->LoadNetwork(id, std::move(network), error); }
+Status IRuntime::LoadNetwork(NetworkId& id, IOptimizedNetworkPtr network, std::string& error, const INetworkProperties&)
+{
+    return pRuntimeImpl->LoadNetwork(id, std::move(network), error);
+}
+TensorInfo IRuntime::GetInputTensorInfo(NetworkId id, LayerBindingId layerId) const { return pRuntimeImpl->Get(id).GetInputTensorInfo(layerId); }
+TensorInfo IRuntime::GetOutputTensorInfo(NetworkId id, LayerBindingId layerId) const { return pRuntimeImpl->Get(id).GetOutputTensorInfo(layerId); }
+Status IRuntime::EnqueueWorkload(NetworkId id, const InputTensors& in, const OutputTensors& out) { return pRuntimeImpl->Enqueue(id, in, out); }
+Status IRuntime::UnloadNetwork(NetworkId id) { return pRuntimeImpl->Unload(id); }
+const IDeviceSpec& IRuntime::GetDeviceSpec() const { return pRuntimeImpl->m_DeviceSpec; }
+} // namespace armnn

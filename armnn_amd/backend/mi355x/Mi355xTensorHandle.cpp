@@ -1,0 +1,135 @@
+#include "Mi355xTensorHandle.hpp"
+#include "Mi355xDevice.hpp"
+
+#include <armnn/backends/TensorHandle.hpp>
+
+#include <cstring>
+
+namespace armnn
+{
+Mi355xTensorHandle::Mi355xTensorHandle(const TensorInfo& info, std::shared_ptr<Mi355xMemoryManager> memoryManager, bool managed)
+    : m_Info(info), m_MemoryManager(std::move(memoryManager)), m_Managed(managed && m_MemoryManager)
+{
+}
+
+Mi355xTensorHandle::~Mi355xTensorHandle()
+{
+    if (m_Owned) mi355x_free(m_Owned);
+    if (m_Staging) mi355x_host_free(m_Staging);
+}
+
+void Mi355xTensorHandle::Manage()
+{
+    if (!m_Managed) return;
+    if (m_Reserved) throw InvalidArgumentException("Mi355xTensorHandle::Manage() called twice");
+    m_Offset = m_MemoryManager->Reserve(m_Info.GetNumBytes());
+    m_Reserved = true;
+}
+
+void Mi355xTensorHandle::Allocate()
+{
+    if (m_Managed)
+    {
+        if (!m_Reserved) throw InvalidArgumentException("Mi355xTensorHandle::Allocate() called before Manage()");
+        if (m_Retired) throw InvalidArgumentException("Mi355xTensorHandle::Allocate() called twice");
+        m_MemoryManager->Retire(m_Offset, m_Info.GetNumBytes());
+        m_Retired = true;
+        return;
+    }
+    if (m_Owned) throw InvalidArgumentException("Mi355xTensorHandle::Allocate() called on a tensor that already has memory");
+    mi355x::EnsureDevice();
+    const size_t bytes = m_Info.GetNumBytes() ? m_Info.GetNumBytes() : 1;
+    mi355x::Check(mi355x_malloc(&m_Owned, bytes), "mi355x_malloc");
+}
+
+void* Mi355xTensorHandle::GetDevicePointer() const
+{
+    if (m_Managed)
+    {
+        if (!m_Reserved) throw NullPointerException("Mi355xTensorHandle: managed tensor was never given a lifetime (Manage)");
+        return m_MemoryManager->Resolve(m_Offset);
+    }
+    if (!m_Owned) throw NullPointerException("Mi355xTensorHandle: tensor has no memory (Allocate was not called)");
+    return m_Owned;
+}
+
+TensorShape Mi355xTensorHandle::GetStrides() const { return GetUnpaddedTensorStrides(m_Info); }
+
+const void* Mi355xTensorHandle::Map(bool /*blocking*/) const
+{
+    void* dev = GetDevicePointer();
+    const size_t bytes = m_Info.GetNumBytes();
+    if (!m_Staging) mi355x::Check(mi355x_host_alloc(&m_Staging, bytes ? bytes : 1), "mi355x_host_alloc");
+    if (m_MapCount == 0 && m_UploadInFlight)
+    {
+        // the host is about to touch the staging copy again: the previous upload must have left it
+        mi355x::Synchronize();
+        m_UploadInFlight = false;
+    }
+    if (m_MapCount++ == 0 && m_DeviceNewer && bytes)
+    {
+        mi355x::Check(mi355x_memcpy_d2h(m_Staging, dev, bytes, mi355x::Stream()), "mi355x_memcpy_d2h");
+        mi355x::Synchronize();
+        m_DeviceNewer = false;
+    }
+    return m_Staging;
+}
+
+void Mi355xTensorHandle::Unmap() const
+{
+    if (m_MapCount == 0) return;
+    if (--m_MapCount != 0) return;
+    const size_t bytes = m_Info.GetNumBytes();
+    if (!bytes) return;
+    // the pinned copy stays alive with the handle, so the upload may complete asynchronously in stream order
+    mi355x::Check(mi355x_memcpy_h2d(GetDevicePointer(), m_Staging, bytes, mi355x::Stream()), "mi355x_memcpy_h2d");
+    m_UploadInFlight = true;
+}
+
+void Mi355xTensorHandle::CopyOutTo(void* memory) const
+{
+    const void* p = Map(true);
+    std::memcpy(memory, p, m_Info.GetNumBytes());
+    // nothing was modified: skip the upload Unmap() would do
+    --m_MapCount;
+}
+
+void Mi355xTensorHandle::CopyInFrom(const void* memory)
+{
+    const size_t bytes = m_Info.GetNumBytes();
+    if (!m_Staging) mi355x::Check(mi355x_host_alloc(&m_Staging, bytes ? bytes : 1), "mi355x_host_alloc");
+    if (m_UploadInFlight) mi355x::Synchronize();
+    std::memcpy(m_Staging, memory, bytes);
+    if (bytes) mi355x::Check(mi355x_memcpy_h2d(GetDevicePointer(), m_Staging, bytes, mi355x::Stream()), "mi355x_memcpy_h2d");
+    m_UploadInFlight = bytes != 0;
+    m_DeviceNewer = false;
+}
+
+// ---- factory ---------------------------------------------------------------------------------------------------------
+const ITensorHandleFactory::FactoryId& Mi355xTensorHandleFactory::GetIdStatic()
+{
+    static const FactoryId id(Mi355xTensorHandleFactoryId());
+    return id;
+}
+
+std::unique_ptr<ITensorHandle> Mi355xTensorHandleFactory::CreateSubTensorHandle(ITensorHandle&, TensorShape const&, unsigned int const*) const
+{
+    return nullptr;
+}
+std::unique_ptr<ITensorHandle> Mi355xTensorHandleFactory::CreateTensorHandle(const TensorInfo& info) const
+{
+    return std::make_unique<Mi355xTensorHandle>(info, m_MemoryManager, true);
+}
+std::unique_ptr<ITensorHandle> Mi355xTensorHandleFactory::CreateTensorHandle(const TensorInfo& info, DataLayout) const
+{
+    return std::make_unique<Mi355xTensorHandle>(info, m_MemoryManager, true);
+}
+std::unique_ptr<ITensorHandle> Mi355xTensorHandleFactory::CreateTensorHandle(const TensorInfo& info, const bool managed) const
+{
+    return std::make_unique<Mi355xTensorHandle>(info, m_MemoryManager, managed);
+}
+std::unique_ptr<ITensorHandle> Mi355xTensorHandleFactory::CreateTensorHandle(const TensorInfo& info, DataLayout, const bool managed) const
+{
+    return std::make_unique<Mi355xTensorHandle>(info, m_MemoryManager, managed);
+}
+} // namespace armnn

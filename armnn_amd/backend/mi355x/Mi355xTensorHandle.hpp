@@ -1,0 +1,78 @@
+// ITensorHandle / ITensorHandleFactory of the Mi355x backend: dense device tensors.
+//
+//   managed handles   live in the memory manager's arena (Manage() reserves, Allocate() ends the lifetime);
+//   unmanaged handles (constants, network inputs) own a device allocation made by Allocate().
+//
+// Map() gives the host a pinned staging copy: it downloads the tensor if kernels may have written it since the
+// last upload, and Unmap() uploads the staging copy again -- so the Map/memcpy/Unmap sequence of
+// CopyMemGenericWorkload and of the runtime's input/output binding works unchanged
+// (RefTensorHandle::Map/CopyInFrom/CopyOutTo, src/backends/reference/RefTensorHandle.cpp:45-133, are the host-memory
+// counterparts).  Workloads call MarkDeviceWritten() on their outputs.
+#pragma once
+#include "Mi355xBackendId.hpp"
+#include "Mi355xMemoryManager.hpp"
+
+#include <armnn/backends/ITensorHandle.hpp>
+#include <armnn/backends/ITensorHandleFactory.hpp>
+
+#include <memory>
+
+namespace armnn
+{
+class Mi355xTensorHandle : public ITensorHandle
+{
+public:
+    Mi355xTensorHandle(const TensorInfo& info, std::shared_ptr<Mi355xMemoryManager> memoryManager, bool managed);
+    ~Mi355xTensorHandle() override;
+
+    void Manage() override;
+    void Allocate() override;
+    ITensorHandle* GetParent() const override { return nullptr; }
+    const void* Map(bool blocking = true) const override;
+    void Unmap() const override;
+    TensorShape GetStrides() const override;
+    TensorShape GetShape() const override { return m_Info.GetShape(); }
+    void CopyOutTo(void* memory) const override;
+    void CopyInFrom(const void* memory) override;
+
+    const TensorInfo& GetTensorInfo() const { return m_Info; }
+    /// device address; throws NullPointerException when the tensor has no memory yet
+    void* GetDevicePointer() const;
+    void MarkDeviceWritten() const { m_DeviceNewer = true; }
+    bool IsManaged() const { return m_Managed; }
+
+private:
+    TensorInfo m_Info;
+    std::shared_ptr<Mi355xMemoryManager> m_MemoryManager;
+    const bool m_Managed;
+    bool m_Reserved = false;
+    bool m_Retired = false;
+    size_t m_Offset = 0;
+    void* m_Owned = nullptr;            // unmanaged handles
+    mutable void* m_Staging = nullptr;  // pinned host copy, created by the first Map()
+    mutable bool m_DeviceNewer = false;
+    mutable bool m_UploadInFlight = false;
+    mutable int m_MapCount = 0;
+};
+
+class Mi355xTensorHandleFactory : public ITensorHandleFactory
+{
+public:
+    explicit Mi355xTensorHandleFactory(std::shared_ptr<Mi355xMemoryManager> mgr) : m_MemoryManager(std::move(mgr)) {}
+    std::unique_ptr<ITensorHandle> CreateSubTensorHandle(ITensorHandle& parent, TensorShape const& subTensorShape,
+                                                         unsigned int const* subTensorOrigin) const override;
+    std::unique_ptr<ITensorHandle> CreateTensorHandle(const TensorInfo& tensorInfo) const override;
+    std::unique_ptr<ITensorHandle> CreateTensorHandle(const TensorInfo& tensorInfo, DataLayout dataLayout) const override;
+    std::unique_ptr<ITensorHandle> CreateTensorHandle(const TensorInfo& tensorInfo, const bool IsMemoryManaged) const override;
+    std::unique_ptr<ITensorHandle> CreateTensorHandle(const TensorInfo& tensorInfo, DataLayout dataLayout,
+                                                      const bool IsMemoryManaged) const override;
+    static const FactoryId& GetIdStatic();
+    const FactoryId& GetId() const override { return GetIdStatic(); }
+    bool SupportsSubTensors() const override { return false; }
+    MemorySourceFlags GetExportFlags() const override { return 0; }
+    MemorySourceFlags GetImportFlags() const override { return 0; }
+    const std::shared_ptr<Mi355xMemoryManager>& GetMemoryManager() const { return m_MemoryManager; }
+private:
+    std::shared_ptr<Mi355xMemoryManager> m_MemoryManager;
+};
+} // namespace armnn

@@ -1,0 +1,70 @@
+#include "Mi355xWorkloadFactory.hpp"
+#include "Mi355xBackendId.hpp"
+#include "Mi355xTensorHandle.hpp"
+#include "Mi355xWorkloads.hpp"
+
+#include <armnn/backends/MemCopyWorkload.hpp>
+#include <armnn/utility/PolymorphicDowncast.hpp>
+
+namespace armnn
+{
+namespace
+{
+const BackendId s_Id{Mi355xBackendId()};
+}
+
+Mi355xWorkloadFactory::Mi355xWorkloadFactory(const std::shared_ptr<Mi355xMemoryManager>& memoryManager) : m_MemoryManager(memoryManager) {}
+Mi355xWorkloadFactory::Mi355xWorkloadFactory() : m_MemoryManager(new Mi355xMemoryManager()) {}
+
+const BackendId& Mi355xWorkloadFactory::GetBackendId() const { return s_Id; }
+
+bool Mi355xWorkloadFactory::IsLayerSupported(const IConnectableLayer& layer, Optional<DataType> dataType, std::string& outReasonIfUnsupported)
+{
+    return IWorkloadFactory::IsLayerSupported(s_Id, layer, dataType, outReasonIfUnsupported);
+}
+
+std::unique_ptr<ITensorHandle> Mi355xWorkloadFactory::CreateTensorHandle(const TensorInfo& info, const bool managed) const
+{
+    return std::make_unique<Mi355xTensorHandle>(info, m_MemoryManager, managed);
+}
+std::unique_ptr<ITensorHandle> Mi355xWorkloadFactory::CreateTensorHandle(const TensorInfo& info, DataLayout, const bool managed) const
+{
+    return std::make_unique<Mi355xTensorHandle>(info, m_MemoryManager, managed);
+}
+
+std::unique_ptr<IWorkload> Mi355xWorkloadFactory::CreateWorkload(LayerType type, const QueueDescriptor& descriptor, const WorkloadInfo& info) const
+{
+    switch (type)
+    {
+        case LayerType::Convolution2d:
+            return std::make_unique<Mi355xConvolution2dWorkload>(*PolymorphicDowncast<const Convolution2dQueueDescriptor*>(&descriptor), info);
+        case LayerType::DepthwiseConvolution2d:
+            return std::make_unique<Mi355xDepthwiseConvolution2dWorkload>(*PolymorphicDowncast<const DepthwiseConvolution2dQueueDescriptor*>(&descriptor), info);
+        case LayerType::FullyConnected:
+            return std::make_unique<Mi355xFullyConnectedWorkload>(*PolymorphicDowncast<const FullyConnectedQueueDescriptor*>(&descriptor), info);
+        case LayerType::Activation:
+            return std::make_unique<Mi355xActivationWorkload>(*PolymorphicDowncast<const ActivationQueueDescriptor*>(&descriptor), info);
+        case LayerType::Pooling2d:
+            return std::make_unique<Mi355xPooling2dWorkload>(*PolymorphicDowncast<const Pooling2dQueueDescriptor*>(&descriptor), info);
+        case LayerType::Softmax:
+            return std::make_unique<Mi355xSoftmaxWorkload>(*PolymorphicDowncast<const SoftmaxQueueDescriptor*>(&descriptor), info);
+        case LayerType::ElementwiseBinary:
+            return std::make_unique<Mi355xAdditionWorkload>(*PolymorphicDowncast<const ElementwiseBinaryQueueDescriptor*>(&descriptor), info);
+        case LayerType::Reshape:
+            return std::make_unique<Mi355xReshapeWorkload>(*PolymorphicDowncast<const ReshapeQueueDescriptor*>(&descriptor), info);
+        case LayerType::Constant:
+            return std::make_unique<Mi355xConstantWorkload>(*PolymorphicDowncast<const ConstantQueueDescriptor*>(&descriptor), info);
+        case LayerType::Input:
+        case LayerType::Output:
+        case LayerType::MemCopy:
+        {
+            // Map / memcpy / Unmap between any two handle types; the device handle's Map() and Unmap() do the transfers
+            const auto* d = PolymorphicDowncast<const MemCopyQueueDescriptor*>(&descriptor);
+            if (d->m_Inputs.empty() || !d->m_Inputs[0]) throw InvalidArgumentException("Mi355xWorkloadFactory: copy workload without an input handle");
+            return std::make_unique<CopyMemGenericWorkload>(*d, info);
+        }
+        default:
+            return nullptr;
+    }
+}
+} // namespace armnn

@@ -1,0 +1,334 @@
+#include "Mi355xWorkloads.hpp"
+#include "Mi355xTensorHandle.hpp"
+
+#include <armnn/backends/TensorHandle.hpp>
+#include <armnn/utility/PolymorphicDowncast.hpp>
+
+#include <cstring>
+
+namespace armnn
+{
+namespace
+{
+// Device address of a workload operand.  Every operand of a workload this backend creates was made by this backend's
+// tensor handle factory; anything else reaches it through a MemCopy layer.
+const Mi355xTensorHandle& Dev(const ITensorHandle* h)
+{
+    const auto* d = dynamic_cast<const Mi355xTensorHandle*>(h);
+    if (!d) throw InvalidArgumentException("Mi355x workload: operand is not a device tensor handle");
+    return *d;
+}
+const void* In(const ITensorHandle* h) { return Dev(h).GetDevicePointer(); }
+void* Out(ITensorHandle* h)
+{
+    const Mi355xTensorHandle& d = Dev(h);
+    d.MarkDeviceWritten();
+    return d.GetDevicePointer();
+}
+
+// Host copy of a constant operand plus its quantization in C-ABI form.  The copy is taken through Map(), so it
+// works for any handle type a constant may arrive in.
+struct HostConstant
+{
+    std::vector<unsigned char> data;
+    std::vector<float> scales;
+    mi355x_const_quant quant{};
+
+    HostConstant(const ITensorHandle* handle, const TensorInfo& info)
+    {
+        data.resize(info.GetNumBytes());
+        const void* p = handle->Map(true);
+        if (!p) throw NullPointerException("Mi355x workload: constant operand has no data");
+        std::memcpy(data.data(), p, data.size());
+        handle->Unmap();
+        scales = info.GetQuantizationScales();
+        if (scales.empty()) scales.push_back(1.0f);
+        quant.dtype = mi355x::ToDType(info.GetDataType());
+        quant.offset = info.GetQuantizationOffset();
+        quant.n_scales = static_cast<uint32_t>(scales.size());
+        quant.scales = scales.data();
+    }
+};
+} // namespace
+
+Mi355xFusedActivation Mi355xFusedActivation::From(const ActivationDescriptor* d)
+{
+    Mi355xFusedActivation f;
+    if (!d) return f;
+    switch (d->m_Function)
+    {
+        case ActivationFunction::ReLu: f.function = MI355X_ACT_RELU; break;
+        case ActivationFunction::BoundedReLu: f.function = MI355X_ACT_BOUNDED_RELU; f.a = d->m_A; f.b = d->m_B; break;
+        default: throw InvalidArgumentException("Mi355x: only ReLu / BoundedReLu can be fused into a layer");
+    }
+    return f;
+}
+
+// ---- Convolution2d ---------------------------------------------------------------------------------------------------
+Mi355xConvolution2dWorkload::Mi355xConvolution2dWorkload(const Convolution2dQueueDescriptor& descriptor, const WorkloadInfo& info)
+    : BaseWorkload<Convolution2dQueueDescriptor>(descriptor, info), m_Info(info)
+{
+    if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xConvolution2dWorkload: NHWC only");
+    Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());   // validates early
+}
+
+Mi355xConvolution2dWorkload::~Mi355xConvolution2dWorkload()
+{
+    if (m_Plan) mi355x_conv2d_destroy(m_Plan);
+}
+
+void Mi355xConvolution2dWorkload::BuildPlan() const
+{
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& w = m_Info.m_InputTensorInfos[1];
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const Convolution2dDescriptor& p = m_Data.m_Parameters;
+    const Mi355xFusedActivation act = Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
+
+    mi355x_conv2d_desc d{};
+    d.in_h = in.GetShape()[1]; d.in_w = in.GetShape()[2]; d.in_c = in.GetShape()[3];
+    d.out_h = out.GetShape()[1]; d.out_w = out.GetShape()[2]; d.out_c = out.GetShape()[3];
+    d.kernel_h = w.GetShape()[1]; d.kernel_w = w.GetShape()[2];
+    d.pad_top = p.m_PadTop; d.pad_left = p.m_PadLeft;
+    d.stride_x = p.m_StrideX; d.stride_y = p.m_StrideY;
+    d.dilation_x = p.m_DilationX; d.dilation_y = p.m_DilationY;
+    d.depthwise = 0;
+    d.bias_enabled = p.m_BiasEnabled ? 1u : 0u;
+    d.input = mi355x::ToQuant(in);
+    d.output = mi355x::ToQuant(out);
+    d.activation = act.function; d.activation_a = act.a; d.activation_b = act.b;
+    d.algo = MI355X_ALGO_AUTO;
+
+    HostConstant weights(m_Data.m_Inputs[1], w);
+    std::unique_ptr<HostConstant> bias;
+    if (p.m_BiasEnabled) bias = std::make_unique<HostConstant>(m_Data.m_Inputs[2], m_Info.m_InputTensorInfos[2]);
+    mi355x::EnsureDevice();
+    mi355x::Check(mi355x_conv2d_create(&d, weights.data.data(), &weights.quant,
+                                       bias ? reinterpret_cast<const int32_t*>(bias->data.data()) : nullptr,
+                                       bias ? &bias->quant : nullptr, &m_Plan),
+                  "mi355x_conv2d_create");
+}
+
+void Mi355xConvolution2dWorkload::Execute() const
+{
+    std::call_once(m_Once, [this] { BuildPlan(); });
+    if (!m_Plan) throw RuntimeException("Mi355xConvolution2dWorkload: no device plan (its creation failed earlier)");
+    const uint32_t batch = m_Info.m_InputTensorInfos[0].GetShape()[0];
+    mi355x::Check(mi355x_conv2d_run(m_Plan, batch, In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()), "mi355x_conv2d_run");
+}
+
+std::string Mi355xConvolution2dWorkload::GetKernelDescription() const
+{
+    if (!m_Plan) return std::string();
+    int32_t algo = 0;
+    char buf[256] = {0};
+    mi355x_conv2d_algo(m_Plan, &algo, buf, sizeof(buf));
+    return buf;
+}
+
+// ---- DepthwiseConvolution2d ------------------------------------------------------------------------------------------
+Mi355xDepthwiseConvolution2dWorkload::Mi355xDepthwiseConvolution2dWorkload(const DepthwiseConvolution2dQueueDescriptor& descriptor, const WorkloadInfo& info)
+    : BaseWorkload<DepthwiseConvolution2dQueueDescriptor>(descriptor, info), m_Info(info)
+{
+    if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xDepthwiseConvolution2dWorkload: NHWC only");
+    Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
+}
+
+Mi355xDepthwiseConvolution2dWorkload::~Mi355xDepthwiseConvolution2dWorkload()
+{
+    if (m_Plan) mi355x_conv2d_destroy(m_Plan);
+}
+
+void Mi355xDepthwiseConvolution2dWorkload::BuildPlan() const
+{
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& w = m_Info.m_InputTensorInfos[1];   // [1, H, W, O]
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const DepthwiseConvolution2dDescriptor& p = m_Data.m_Parameters;
+    const Mi355xFusedActivation act = Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
+
+    mi355x_conv2d_desc d{};
+    d.in_h = in.GetShape()[1]; d.in_w = in.GetShape()[2]; d.in_c = in.GetShape()[3];
+    d.out_h = out.GetShape()[1]; d.out_w = out.GetShape()[2]; d.out_c = out.GetShape()[3];
+    d.kernel_h = w.GetShape()[1]; d.kernel_w = w.GetShape()[2];
+    d.pad_top = p.m_PadTop; d.pad_left = p.m_PadLeft;
+    d.stride_x = p.m_StrideX; d.stride_y = p.m_StrideY;
+    d.dilation_x = p.m_DilationX; d.dilation_y = p.m_DilationY;
+    d.depthwise = 1;
+    d.bias_enabled = p.m_BiasEnabled ? 1u : 0u;
+    d.input = mi355x::ToQuant(in);
+    d.output = mi355x::ToQuant(out);
+    d.activation = act.function; d.activation_a = act.a; d.activation_b = act.b;
+    d.algo = MI355X_ALGO_AUTO;
+
+    HostConstant weights(m_Data.m_Inputs[1], w);
+    std::unique_ptr<HostConstant> bias;
+    if (p.m_BiasEnabled) bias = std::make_unique<HostConstant>(m_Data.m_Inputs[2], m_Info.m_InputTensorInfos[2]);
+    mi355x::EnsureDevice();
+    mi355x::Check(mi355x_conv2d_create(&d, weights.data.data(), &weights.quant,
+                                       bias ? reinterpret_cast<const int32_t*>(bias->data.data()) : nullptr,
+                                       bias ? &bias->quant : nullptr, &m_Plan),
+                  "mi355x_conv2d_create(depthwise)");
+}
+
+void Mi355xDepthwiseConvolution2dWorkload::Execute() const
+{
+    std::call_once(m_Once, [this] { BuildPlan(); });
+    if (!m_Plan) throw RuntimeException("Mi355xDepthwiseConvolution2dWorkload: no device plan (its creation failed earlier)");
+    const uint32_t batch = m_Info.m_InputTensorInfos[0].GetShape()[0];
+    mi355x::Check(mi355x_conv2d_run(m_Plan, batch, In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()), "mi355x_conv2d_run(depthwise)");
+}
+
+// ---- FullyConnected --------------------------------------------------------------------------------------------------
+Mi355xFullyConnectedWorkload::Mi355xFullyConnectedWorkload(const FullyConnectedQueueDescriptor& descriptor, const WorkloadInfo& info)
+    : BaseWorkload<FullyConnectedQueueDescriptor>(descriptor, info), m_Info(info)
+{
+    Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
+}
+
+Mi355xFullyConnectedWorkload::~Mi355xFullyConnectedWorkload()
+{
+    if (m_Plan) mi355x_fc_destroy(m_Plan);
+}
+
+void Mi355xFullyConnectedWorkload::BuildPlan() const
+{
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& w = m_Info.m_InputTensorInfos[1];
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const FullyConnectedDescriptor& p = m_Data.m_Parameters;
+    const Mi355xFusedActivation act = Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
+
+    mi355x_fc_desc d{};
+    d.k = in.GetNumElements() / in.GetShape()[0];       // GetNumActivations, RefFullyConnectedWorkload.cpp:16-24
+    d.out_features = out.GetShape()[1];
+    d.transpose_weights = p.m_TransposeWeightMatrix ? 1u : 0u;
+    d.bias_enabled = p.m_BiasEnabled ? 1u : 0u;
+    d.input = mi355x::ToQuant(in);
+    d.output = mi355x::ToQuant(out);
+    d.activation = act.function; d.activation_a = act.a; d.activation_b = act.b;
+    d.algo = MI355X_ALGO_AUTO;
+
+    HostConstant weights(m_Data.m_Inputs[1], w);
+    std::unique_ptr<HostConstant> bias;
+    if (p.m_BiasEnabled) bias = std::make_unique<HostConstant>(m_Data.m_Inputs[2], m_Info.m_InputTensorInfos[2]);
+    mi355x::EnsureDevice();
+    mi355x::Check(mi355x_fc_create(&d, weights.data.data(), &weights.quant,
+                                   bias ? reinterpret_cast<const int32_t*>(bias->data.data()) : nullptr,
+                                   bias ? &bias->quant : nullptr, &m_Plan),
+                  "mi355x_fc_create");
+}
+
+void Mi355xFullyConnectedWorkload::Execute() const
+{
+    std::call_once(m_Once, [this] { BuildPlan(); });
+    if (!m_Plan) throw RuntimeException("Mi355xFullyConnectedWorkload: no device plan (its creation failed earlier)");
+    const uint32_t batch = m_Info.m_InputTensorInfos[0].GetShape()[0];
+    mi355x::Check(mi355x_fc_run(m_Plan, batch, In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()), "mi355x_fc_run");
+}
+
+// ---- Activation ------------------------------------------------------------------------------------------------------
+Mi355xActivationWorkload::Mi355xActivationWorkload(const ActivationQueueDescriptor& descriptor, const WorkloadInfo& info)
+    : BaseWorkload<ActivationQueueDescriptor>(descriptor, info), m_Info(info)
+{
+    Mi355xFusedActivation::From(&m_Data.m_Parameters);
+}
+
+void Mi355xActivationWorkload::Execute() const
+{
+    const Mi355xFusedActivation act = Mi355xFusedActivation::From(&m_Data.m_Parameters);
+    const mi355x_quant qi = mi355x::ToQuant(m_Info.m_InputTensorInfos[0]);
+    const mi355x_quant qo = mi355x::ToQuant(m_Info.m_OutputTensorInfos[0]);
+    mi355x::Check(mi355x_activation_run(m_Info.m_InputTensorInfos[0].GetNumElements(), &qi, &qo, act.function, act.a, act.b,
+                                        In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()),
+                  "mi355x_activation_run");
+}
+
+// ---- Pooling2d -------------------------------------------------------------------------------------------------------
+Mi355xPooling2dWorkload::Mi355xPooling2dWorkload(const Pooling2dQueueDescriptor& descriptor, const WorkloadInfo& info)
+    : BaseWorkload<Pooling2dQueueDescriptor>(descriptor, info), m_Info(info)
+{
+    if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xPooling2dWorkload: NHWC only");
+}
+
+void Mi355xPooling2dWorkload::Execute() const
+{
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const Pooling2dDescriptor& p = m_Data.m_Parameters;
+    mi355x_pool2d_desc d{};
+    d.in_h = in.GetShape()[1]; d.in_w = in.GetShape()[2]; d.channels = in.GetShape()[3];
+    d.out_h = out.GetShape()[1]; d.out_w = out.GetShape()[2];
+    d.pool_w = p.m_PoolWidth; d.pool_h = p.m_PoolHeight; d.stride_x = p.m_StrideX; d.stride_y = p.m_StrideY;
+    d.pad_left = p.m_PadLeft; d.pad_right = p.m_PadRight; d.pad_top = p.m_PadTop; d.pad_bottom = p.m_PadBottom;
+    d.pool_type = p.m_PoolType == PoolingAlgorithm::Max ? 0 : 1;
+    d.padding_method = p.m_PaddingMethod == PaddingMethod::IgnoreValue ? 0 : 1;
+    d.input = mi355x::ToQuant(in);
+    d.output = mi355x::ToQuant(out);
+    mi355x::Check(mi355x_pool2d_run(&d, in.GetShape()[0], In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()), "mi355x_pool2d_run");
+}
+
+// ---- Softmax ---------------------------------------------------------------------------------------------------------
+Mi355xSoftmaxWorkload::Mi355xSoftmaxWorkload(const SoftmaxQueueDescriptor& descriptor, const WorkloadInfo& info)
+    : BaseWorkload<SoftmaxQueueDescriptor>(descriptor, info), m_Info(info)
+{
+}
+
+void Mi355xSoftmaxWorkload::Execute() const
+{
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const unsigned int rank = in.GetNumDimensions();
+    const uint32_t cols = in.GetShape()[rank - 1];
+    const uint32_t rows = cols ? in.GetNumElements() / cols : 0;
+    const mi355x_quant qi = mi355x::ToQuant(in);
+    const mi355x_quant qo = mi355x::ToQuant(m_Info.m_OutputTensorInfos[0]);
+    mi355x::Check(mi355x_softmax_run(rows, cols, m_Data.m_Parameters.m_Beta, &qi, &qo, In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()),
+                  "mi355x_softmax_run");
+}
+
+// ---- Add -------------------------------------------------------------------------------------------------------------
+Mi355xAdditionWorkload::Mi355xAdditionWorkload(const ElementwiseBinaryQueueDescriptor& descriptor, const WorkloadInfo& info)
+    : BaseWorkload<ElementwiseBinaryQueueDescriptor>(descriptor, info), m_Info(info)
+{
+    if (m_Data.m_Parameters.m_Operation != BinaryOperation::Add) throw InvalidArgumentException("Mi355xAdditionWorkload: Add only");
+    Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
+}
+
+void Mi355xAdditionWorkload::Execute() const
+{
+    const Mi355xFusedActivation act = Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
+    const mi355x_quant q0 = mi355x::ToQuant(m_Info.m_InputTensorInfos[0]);
+    const mi355x_quant q1 = mi355x::ToQuant(m_Info.m_InputTensorInfos[1]);
+    const mi355x_quant qo = mi355x::ToQuant(m_Info.m_OutputTensorInfos[0]);
+    mi355x::Check(mi355x_add_run(m_Info.m_OutputTensorInfos[0].GetNumElements(), &q0, &q1, &qo, act.function, act.a, act.b,
+                                 In(m_Data.m_Inputs[0]), In(m_Data.m_Inputs[1]), Out(m_Data.m_Outputs[0]), mi355x::Stream()),
+                  "mi355x_add_run");
+}
+
+// ---- Reshape ---------------------------------------------------------------------------------------------------------
+Mi355xReshapeWorkload::Mi355xReshapeWorkload(const ReshapeQueueDescriptor& descriptor, const WorkloadInfo& info)
+    : BaseWorkload<ReshapeQueueDescriptor>(descriptor, info), m_Info(info)
+{
+}
+
+void Mi355xReshapeWorkload::Execute() const
+{
+    const size_t bytes = m_Info.m_InputTensorInfos[0].GetNumBytes();
+    if (!bytes) return;
+    mi355x::Check(mi355x_memcpy_d2d(Out(m_Data.m_Outputs[0]), In(m_Data.m_Inputs[0]), bytes, mi355x::Stream()), "mi355x_memcpy_d2d");
+}
+
+// ---- Constant --------------------------------------------------------------------------------------------------------
+Mi355xConstantWorkload::Mi355xConstantWorkload(const ConstantQueueDescriptor& descriptor, const WorkloadInfo& info)
+    : BaseWorkload<ConstantQueueDescriptor>(descriptor, info)
+{
+}
+
+void Mi355xConstantWorkload::Execute() const
+{
+    const void* src = m_Data.m_LayerOutput->Map(true);
+    if (!src) throw NullPointerException("Mi355xConstantWorkload: layer has no data");
+    m_Data.m_Outputs[0]->CopyInFrom(src);
+    m_Data.m_LayerOutput->Unmap();
+}
+} // namespace armnn

@@ -1,0 +1,126 @@
+// Workloads of the Mi355x backend.  Each one is the device counterpart of a CpuRef workload and does its GPU work through
+// the C ABI only.  Convolution2d / DepthwiseConvolution2d / FullyConnected build their device plan (weights re-laid-out
+// for the kernel, per-channel requantization constants) on the first Execute(), when the constant inputs have been
+// produced -- the point at which RefConvolution2dWorkload::PostAllocationConfigure builds its decoders
+// (src/backends/reference/workloads/RefConvolution2dWorkload.cpp:24-36).
+#pragma once
+#include "Mi355xDevice.hpp"
+
+#include <armnn/backends/Workload.hpp>
+#include <armnn/backends/WorkloadData.hpp>
+
+#include <mutex>
+#include <vector>
+
+namespace armnn
+{
+/// the fused activation a layer carries as its "additional info" object, translated for the C ABI
+struct Mi355xFusedActivation
+{
+    int32_t function = MI355X_ACT_NONE;
+    float a = 0.0f, b = 0.0f;
+    static Mi355xFusedActivation From(const ActivationDescriptor* descriptor);
+};
+
+/// counterpart of RefConvolution2dWorkload (RefConvolution2dWorkload.cpp:38-58)
+class Mi355xConvolution2dWorkload : public BaseWorkload<Convolution2dQueueDescriptor>
+{
+public:
+    Mi355xConvolution2dWorkload(const Convolution2dQueueDescriptor& descriptor, const WorkloadInfo& info);
+    ~Mi355xConvolution2dWorkload() override;
+    void Execute() const override;
+    /// kernel the plan resolved to; empty before the first Execute()
+    std::string GetKernelDescription() const;
+private:
+    void BuildPlan() const;
+    WorkloadInfo m_Info;
+    mutable mi355x_conv2d_t m_Plan = nullptr;
+    mutable std::once_flag m_Once;
+};
+
+/// counterpart of RefDepthwiseConvolution2dWorkload (RefDepthwiseConvolution2dWorkload.cpp:38-62)
+class Mi355xDepthwiseConvolution2dWorkload : public BaseWorkload<DepthwiseConvolution2dQueueDescriptor>
+{
+public:
+    Mi355xDepthwiseConvolution2dWorkload(const DepthwiseConvolution2dQueueDescriptor& descriptor, const WorkloadInfo& info);
+    ~Mi355xDepthwiseConvolution2dWorkload() override;
+    void Execute() const override;
+private:
+    void BuildPlan() const;
+    WorkloadInfo m_Info;
+    mutable mi355x_conv2d_t m_Plan = nullptr;
+    mutable std::once_flag m_Once;
+};
+
+/// counterpart of RefFullyConnectedWorkload (RefFullyConnectedWorkload.cpp:39-67)
+class Mi355xFullyConnectedWorkload : public BaseWorkload<FullyConnectedQueueDescriptor>
+{
+public:
+    Mi355xFullyConnectedWorkload(const FullyConnectedQueueDescriptor& descriptor, const WorkloadInfo& info);
+    ~Mi355xFullyConnectedWorkload() override;
+    void Execute() const override;
+private:
+    void BuildPlan() const;
+    WorkloadInfo m_Info;
+    mutable mi355x_fc_t m_Plan = nullptr;
+    mutable std::once_flag m_Once;
+};
+
+/// counterpart of RefActivationWorkload (RefActivationWorkload.cpp:23-36)
+class Mi355xActivationWorkload : public BaseWorkload<ActivationQueueDescriptor>
+{
+public:
+    Mi355xActivationWorkload(const ActivationQueueDescriptor& descriptor, const WorkloadInfo& info);
+    void Execute() const override;
+private:
+    WorkloadInfo m_Info;
+};
+
+/// counterpart of RefPooling2dWorkload (RefPooling2dWorkload.cpp:17-40)
+class Mi355xPooling2dWorkload : public BaseWorkload<Pooling2dQueueDescriptor>
+{
+public:
+    Mi355xPooling2dWorkload(const Pooling2dQueueDescriptor& descriptor, const WorkloadInfo& info);
+    void Execute() const override;
+private:
+    WorkloadInfo m_Info;
+};
+
+/// counterpart of RefSoftmaxWorkload (RefSoftmaxWorkload.cpp:21-43)
+class Mi355xSoftmaxWorkload : public BaseWorkload<SoftmaxQueueDescriptor>
+{
+public:
+    Mi355xSoftmaxWorkload(const SoftmaxQueueDescriptor& descriptor, const WorkloadInfo& info);
+    void Execute() const override;
+private:
+    WorkloadInfo m_Info;
+};
+
+/// counterpart of RefElementwiseBinaryWorkload for BinaryOperation::Add (RefElementwiseBinaryWorkload.cpp:27-107)
+class Mi355xAdditionWorkload : public BaseWorkload<ElementwiseBinaryQueueDescriptor>
+{
+public:
+    Mi355xAdditionWorkload(const ElementwiseBinaryQueueDescriptor& descriptor, const WorkloadInfo& info);
+    void Execute() const override;
+private:
+    WorkloadInfo m_Info;
+};
+
+/// counterpart of RefReshapeWorkload (RefReshapeWorkload.cpp:14-31): a device-to-device copy
+class Mi355xReshapeWorkload : public BaseWorkload<ReshapeQueueDescriptor>
+{
+public:
+    Mi355xReshapeWorkload(const ReshapeQueueDescriptor& descriptor, const WorkloadInfo& info);
+    void Execute() const override;
+private:
+    WorkloadInfo m_Info;
+};
+
+/// counterpart of RefConstantWorkload (RefConstantWorkload.cpp:22-47): uploads the layer's data once
+class Mi355xConstantWorkload : public BaseWorkload<ConstantQueueDescriptor>
+{
+public:
+    Mi355xConstantWorkload(const ConstantQueueDescriptor& descriptor, const WorkloadInfo& info);
+    void Execute() const override;
+};
+} // namespace armnn

@@ -1,0 +1,682 @@
+// Tests of the Mi355x backend through the Arm NN backend interfaces.
+//   tag "cpu": host logic only -- registry, layer-support envelope, descriptor validation, sub-graph fusion, the arena
+//              planner, behaviour when the process sees no device.  These never launch a kernel.
+//   tag "gpu": INetwork -> Optimize -> LoadNetwork -> EnqueueWorkload on the device, checked against the CPU oracle
+//              (every output byte within 1 LSB of CpuRef's) and against the C ABI called directly (identical bytes).
+#include "MiniTest.hpp"
+#include "HostTestBackend.hpp"
+#include "TestUtils.hpp"
+
+#include "../mi355x/Mi355xBackend.hpp"
+#include "../mi355x/Mi355xBackendId.hpp"
+#include "../mi355x/Mi355xDevice.hpp"
+#include "../mi355x/Mi355xLayerSupport.hpp"
+#include "../mi355x/Mi355xMemoryManager.hpp"
+#include "../mi355x/Mi355xTensorHandle.hpp"
+#include "../mi355x/Mi355xWorkloadFactory.hpp"
+
+#include <armnn/backends/TensorHandleFactoryRegistry.hpp>
+#include <armnn/backends/WorkloadData.hpp>
+
+using namespace armnn;
+using namespace tu;
+
+namespace
+{
+const BackendId kMi355x{Mi355xBackendId()};
+
+// Input -> layer(s) -> Output
+struct SingleLayerNet
+{
+    INetworkPtr net = INetwork::Create();
+    SingleLayerNet(const QLayer& l)
+    {
+        IConnectableLayer* in = net->AddInputLayer(0, "input");
+        in->GetOutputSlot(0).SetTensorInfo(l.in);
+        IOutputSlot& out = AddToNetwork(*net, in->GetOutputSlot(0), l, "layer");
+        IConnectableLayer* o = net->AddOutputLayer(0, "output");
+        out.Connect(o->GetInputSlot(0));
+    }
+};
+
+std::vector<uint8_t> RunOnRuntime(IRuntime& rt, const INetwork& net, const std::vector<BackendId>& prefs, const TensorInfo& inInfo,
+                                  const std::vector<uint8_t>& input, const TensorInfo& outInfo, int repeats = 1)
+{
+    IOptimizedNetworkPtr opt = Optimize(net, prefs, rt.GetDeviceSpec());
+    NetworkId id = -1;
+    std::string err;
+    if (rt.LoadNetwork(id, std::move(opt), err) != Status::Success) throw std::runtime_error("LoadNetwork failed: " + err);
+    std::vector<uint8_t> out(outInfo.GetNumBytes());
+    TensorInfo constIn = inInfo;
+    constIn.SetConstant(true);
+    for (int i = 0; i < repeats; ++i)
+    {
+        std::fill(out.begin(), out.end(), 0xA5);
+        InputTensors ins{{0, ConstTensor(constIn, input.data())}};
+        OutputTensors outs{{0, Tensor(outInfo, out.data())}};
+        if (rt.EnqueueWorkload(id, ins, outs) != Status::Success) throw std::runtime_error("EnqueueWorkload failed");
+    }
+    rt.UnloadNetwork(id);
+    return out;
+}
+} // namespace
+
+// ---------------------------------------------------------------------------------------------------------------------
+// cpu
+// ---------------------------------------------------------------------------------------------------------------------
+TEST_CASE("registry: Mi355x is registered by the static initializer", "cpu")
+{
+    CHECK(BackendRegistryInstance().IsBackendRegistered(kMi355x));
+    CHECK(BackendRegistryInstance().GetBackendIdsAsString().find("Mi355x") != std::string::npos);
+    auto backend = BackendRegistryInstance().GetFactory(kMi355x)();
+    REQUIRE(backend != nullptr);
+    CHECK(backend->GetId() == kMi355x);
+    CHECK(backend->SupportsTensorAllocatorAPI());
+    CHECK(backend->GetHandleFactoryPreferences().front() == std::string(Mi355xTensorHandleFactoryId()));
+    CHECK_THROWS_AS(BackendRegistryInstance().Register(kMi355x, [] { return IBackendInternalUniquePtr(); }), InvalidArgumentException);
+    CHECK(!HasCapability("Nonexistent", backend->GetCapabilities()));
+    CHECK(HasCapability("ConstantTensorsAsInputs", backend->GetCapabilities()));
+}
+
+TEST_CASE("layer support: the accepted envelope and the reasons outside it", "cpu")
+{
+    Mi355xLayerSupport ls;
+    std::string why;
+    Optional<std::string&> reason(why);
+    const TensorInfo in = ActInfo({1, 8, 8, 16}, DataType::QAsymmS8, 0.05f, -3);
+    QLayer l = MakeConv(QLayer::Conv, in, 32, 3, 1, 0.1f, 5, false, true, 1);
+    Convolution2dDescriptor d;
+    d.m_DataLayout = DataLayout::NHWC;
+    d.m_BiasEnabled = true;
+    d.m_PadLeft = d.m_PadRight = d.m_PadTop = d.m_PadBottom = 1;
+    CHECK(ls.IsLayerSupported(LayerType::Convolution2d, {l.in, l.out, l.w, l.b}, d, EmptyOptional(), EmptyOptional(), reason));
+
+    Convolution2dDescriptor nchw = d;
+    nchw.m_DataLayout = DataLayout::NCHW;
+    CHECK(!ls.IsLayerSupported(LayerType::Convolution2d, {l.in, l.out, l.w, l.b}, nchw, EmptyOptional(), EmptyOptional(), reason));
+    CHECK(why.find("NHWC") != std::string::npos);
+
+    TensorInfo f32in = l.in;
+    f32in.SetDataType(DataType::Float32);
+    CHECK(!ls.IsLayerSupported(LayerType::Convolution2d, {f32in, l.out, l.w, l.b}, d, EmptyOptional(), EmptyOptional(), reason));
+    CHECK(why.find("Float32") != std::string::npos);
+
+    TensorInfo dynW = l.w;
+    dynW.SetConstant(false);
+    CHECK(!ls.IsLayerSupported(LayerType::Convolution2d, {l.in, l.out, dynW, l.b}, d, EmptyOptional(), EmptyOptional(), reason));
+    CHECK(why.find("constant") != std::string::npos);
+
+    TensorInfo badBias = l.b;
+    badBias.SetQuantizationOffset(1);
+    CHECK(!ls.IsLayerSupported(LayerType::Convolution2d, {l.in, l.out, l.w, badBias}, d, EmptyOptional(), EmptyOptional(), reason));
+
+    TensorInfo u8out = l.out;
+    u8out.SetDataType(DataType::QAsymmU8);
+    CHECK(!ls.IsLayerSupported(LayerType::Convolution2d, {l.in, u8out, l.w, l.b}, d, EmptyOptional(), EmptyOptional(), reason));
+
+    // depthwise: [1,H,W,O] weights quantized along dimension 3
+    QLayer dw = MakeConv(QLayer::Depthwise, in, 16, 3, 2, 0.1f, 5, false, true, 2);
+    DepthwiseConvolution2dDescriptor dd;
+    dd.m_DataLayout = DataLayout::NHWC;
+    dd.m_BiasEnabled = true;
+    dd.m_StrideX = dd.m_StrideY = 2;
+    CHECK(ls.IsLayerSupported(LayerType::DepthwiseConvolution2d, {dw.in, dw.out, dw.w, dw.b}, dd, EmptyOptional(), EmptyOptional(), reason));
+    TensorInfo wrongDim = dw.w;
+    wrongDim.SetQuantizationDim(Optional<unsigned int>(0u));
+    CHECK(!ls.IsLayerSupported(LayerType::DepthwiseConvolution2d, {dw.in, dw.out, wrongDim, dw.b}, dd, EmptyOptional(), EmptyOptional(), reason));
+
+    // activations
+    CHECK(ls.IsLayerSupported(LayerType::Activation, {in, in}, ActivationDescriptor(ActivationFunction::ReLu), EmptyOptional(), EmptyOptional(), reason));
+    CHECK(ls.IsLayerSupported(LayerType::Activation, {in, in}, ActivationDescriptor(ActivationFunction::BoundedReLu, 6.f, 0.f), EmptyOptional(), EmptyOptional(), reason));
+    CHECK(!ls.IsLayerSupported(LayerType::Activation, {in, in}, ActivationDescriptor(ActivationFunction::TanH), EmptyOptional(), EmptyOptional(), reason));
+    CHECK(why.find("ReLu") != std::string::npos);
+
+    // pooling / add / softmax / reshape
+    Pooling2dDescriptor pd;
+    pd.m_DataLayout = DataLayout::NHWC;
+    pd.m_PoolType = PoolingAlgorithm::Average;
+    pd.m_PoolWidth = pd.m_PoolHeight = 8;
+    pd.m_StrideX = pd.m_StrideY = 1;
+    const TensorInfo pooled = ActInfo({1, 1, 1, 16}, DataType::QAsymmS8, 0.05f, -3);
+    CHECK(ls.IsLayerSupported(LayerType::Pooling2d, {in, pooled}, pd, EmptyOptional(), EmptyOptional(), reason));
+    pd.m_PoolType = PoolingAlgorithm::L2;
+    CHECK(!ls.IsLayerSupported(LayerType::Pooling2d, {in, pooled}, pd, EmptyOptional(), EmptyOptional(), reason));
+    CHECK(ls.IsLayerSupported(LayerType::ElementwiseBinary, {in, in, in}, ElementwiseBinaryDescriptor(BinaryOperation::Add), EmptyOptional(), EmptyOptional(), reason));
+    CHECK(!ls.IsLayerSupported(LayerType::ElementwiseBinary, {in, in, in}, ElementwiseBinaryDescriptor(BinaryOperation::Mul), EmptyOptional(), EmptyOptional(), reason));
+    CHECK(!ls.IsLayerSupported(LayerType::ElementwiseBinary, {in, pooled, in}, ElementwiseBinaryDescriptor(BinaryOperation::Add), EmptyOptional(), EmptyOptional(), reason));
+    SoftmaxDescriptor sd;
+    const TensorInfo logits = ActInfo({4, 10}, DataType::QAsymmU8, 0.1f, 128);
+    const TensorInfo probs = ActInfo({4, 10}, DataType::QAsymmU8, 1.0f / 256.0f, 0);
+    CHECK(ls.IsLayerSupported(LayerType::Softmax, {logits, probs}, sd, EmptyOptional(), EmptyOptional(), reason));
+    sd.m_Axis = 0;
+    CHECK(!ls.IsLayerSupported(LayerType::Softmax, {logits, probs}, sd, EmptyOptional(), EmptyOptional(), reason));
+    CHECK(ls.IsLayerSupported(LayerType::Reshape, {pooled, ActInfo({1, 16}, DataType::QAsymmS8, 0.05f, -3)}, ReshapeDescriptor(TensorShape({1, 16})), EmptyOptional(), EmptyOptional(), reason));
+}
+
+TEST_CASE("queue descriptors: Validate enforces the quantized conv rules", "cpu")
+{
+    const TensorInfo in = ActInfo({1, 8, 8, 16}, DataType::QAsymmS8, 0.05f, -3);
+    QLayer l = MakeConv(QLayer::Conv, in, 32, 3, 1, 0.1f, 5, false, true, 3);
+    Convolution2dQueueDescriptor q;
+    q.m_Parameters.m_BiasEnabled = true;
+    q.m_Parameters.m_DataLayout = DataLayout::NHWC;
+    WorkloadInfo info;
+    info.m_InputTensorInfos = {l.in, l.w, l.b};
+    info.m_OutputTensorInfos = {l.out};
+    CHECK_NOTHROW(q.Validate(info));
+
+    WorkloadInfo bad = info;
+    bad.m_InputTensorInfos[2].SetQuantizationOffset(7);                       // bias offset must be 0
+    CHECK_THROWS_AS(q.Validate(bad), InvalidArgumentException);
+    bad = info;
+    bad.m_InputTensorInfos[2] = TensorInfo(TensorShape({32}), DataType::Signed32, 0.001f, 0, true);   // per-axis weights need per-axis bias
+    CHECK_THROWS_AS(q.Validate(bad), InvalidArgumentException);
+    bad = info;
+    bad.m_InputTensorInfos[1].SetDataType(DataType::QAsymmU8);                // per-axis weights must be QSymmS8
+    CHECK_THROWS_AS(q.Validate(bad), InvalidArgumentException);
+    bad = info;
+    bad.m_OutputTensorInfos[0].SetDataType(DataType::QAsymmU8);               // input and output types must match
+    CHECK_THROWS_AS(q.Validate(bad), InvalidArgumentException);
+    bad = info;
+    bad.m_InputTensorInfos.pop_back();                                          // bias enabled means three inputs
+    CHECK_THROWS_AS(q.Validate(bad), InvalidArgumentException);
+    Convolution2dQueueDescriptor zeroStride = q;
+    zeroStride.m_Parameters.m_StrideX = 0;
+    CHECK_THROWS_AS(zeroStride.Validate(info), InvalidArgumentException);
+
+    QLayer dw = MakeConv(QLayer::Depthwise, in, 16, 3, 1, 0.1f, 5, false, true, 4);
+    DepthwiseConvolution2dQueueDescriptor dq;
+    dq.m_Parameters.m_BiasEnabled = true;
+    dq.m_Parameters.m_DataLayout = DataLayout::NHWC;
+    WorkloadInfo dinfo;
+    dinfo.m_InputTensorInfos = {dw.in, dw.w, dw.b};
+    dinfo.m_OutputTensorInfos = {dw.out};
+    CHECK_NOTHROW(dq.Validate(dinfo));
+    WorkloadInfo dbad = dinfo;
+    dbad.m_InputTensorInfos[1].SetShape(TensorShape({2, 3, 3, 8}));           // weights must be [1,H,W,O]
+    CHECK_THROWS_AS(dq.Validate(dbad), InvalidArgumentException);
+    DepthwiseConvolution2dQueueDescriptor dil = dq;
+    dil.m_Parameters.m_DilationX = 0;
+    CHECK_THROWS_AS(dil.Validate(dinfo), InvalidArgumentException);
+
+    QLayer fc = MakeFc(ActInfo({2, 64}, DataType::QAsymmS8, 0.05f, 0), 10, 0.2f, 0, false, 5);
+    FullyConnectedQueueDescriptor fq;
+    fq.m_Parameters.m_BiasEnabled = true;
+    fq.m_Parameters.m_TransposeWeightMatrix = true;
+    WorkloadInfo finfo;
+    finfo.m_InputTensorInfos = {fc.in, fc.w, fc.b};
+    finfo.m_OutputTensorInfos = {fc.out};
+    CHECK_NOTHROW(fq.Validate(finfo));
+    WorkloadInfo fbad = finfo;
+    fbad.m_InputTensorInfos[2].SetDataType(DataType::Float32);                // bias of a quantized layer is Signed32
+    CHECK_THROWS_AS(fq.Validate(fbad), InvalidArgumentException);
+}
+
+TEST_CASE("arena planner: lifetimes that do not overlap share addresses", "cpu")
+{
+    Mi355xMemoryManager mm;
+    const size_t a = mm.Reserve(1000);      // 1024
+    const size_t b = mm.Reserve(5000);      // 5120
+    CHECK(a == 0);
+    CHECK(b == 1024);
+    mm.Retire(a, 1000);
+    const size_t c = mm.Reserve(512);       // fits in a's hole
+    CHECK(c == 0);
+    const size_t d = mm.Reserve(512);       // second half of a's hole
+    CHECK(d == 512);
+    mm.Retire(b, 5000);
+    mm.Retire(c, 512);
+    mm.Retire(d, 512);                      // everything free again and coalesced
+    const size_t e = mm.Reserve(6144);
+    CHECK(e == 0);
+    CHECK(mm.ArenaBytes() == 6144);
+    const size_t f = mm.Reserve(100);       // grows past the end
+    CHECK(f == 6144);
+    mm.Retire(f, 100);
+    const size_t g = mm.Reserve(300);       // the free tail is extended, not left behind
+    CHECK(g == 6144);
+    CHECK(mm.ArenaBytes() == 6144 + 512);
+    CHECK(mm.ReservedTotal() > mm.ArenaBytes());
+    CHECK_THROWS_AS(mm.Resolve(0), MemoryValidationException);   // nothing acquired yet
+}
+
+TEST_CASE("tensor handle: lifecycle errors are reported, not ignored", "cpu")
+{
+    auto mm = std::make_shared<Mi355xMemoryManager>();
+    const TensorInfo info = ActInfo({1, 4, 4, 8}, DataType::QAsymmS8, 0.1f, 0);
+    Mi355xTensorHandle managed(info, mm, true);
+    CHECK(managed.IsManaged());
+    CHECK_THROWS_AS(managed.Allocate(), InvalidArgumentException);          // before Manage()
+    CHECK_THROWS_AS(managed.GetDevicePointer(), NullPointerException);
+    managed.Manage();
+    CHECK_THROWS_AS(managed.Manage(), InvalidArgumentException);
+    CHECK_THROWS_AS(managed.GetDevicePointer(), MemoryValidationException);  // arena not acquired
+    managed.Allocate();
+    CHECK_THROWS_AS(managed.Allocate(), InvalidArgumentException);
+    CHECK(managed.GetShape() == info.GetShape());
+    CHECK(managed.GetStrides()[3] == 1);
+    CHECK(managed.GetStrides()[0] == 4 * 4 * 8);
+    Mi355xTensorHandle unmanaged(info, mm, false);
+    CHECK(!unmanaged.IsManaged());
+    CHECK_THROWS_AS(unmanaged.GetDevicePointer(), NullPointerException);     // Allocate() not called
+}
+
+namespace
+{
+INetworkPtr ConvReluNet(bool sameQuant, bool secondConsumer)
+{
+    INetworkPtr net = INetwork::Create();
+    const TensorInfo in = ActInfo({1, 8, 8, 16}, DataType::QAsymmS8, 0.05f, -3);
+    QLayer l = MakeConv(QLayer::Conv, in, 32, 3, 1, 0.1f, -128, false, true, 11);
+    IConnectableLayer* input = net->AddInputLayer(0, "input");
+    input->GetOutputSlot(0).SetTensorInfo(in);
+    IOutputSlot& convOut = AddToNetwork(*net, input->GetOutputSlot(0), l, "conv");
+    IConnectableLayer* act = net->AddActivationLayer(ActivationDescriptor(ActivationFunction::BoundedReLu, 6.0f, 0.0f), "relu6");
+    convOut.Connect(act->GetInputSlot(0));
+    TensorInfo actOut = l.out;
+    if (!sameQuant) actOut.SetQuantizationScale(0.05f);
+    act->GetOutputSlot(0).SetTensorInfo(actOut);
+    IConnectableLayer* out = net->AddOutputLayer(0, "output");
+    act->GetOutputSlot(0).Connect(out->GetInputSlot(0));
+    if (secondConsumer)
+    {
+        IConnectableLayer* out2 = net->AddOutputLayer(1, "output2");
+        convOut.Connect(out2->GetInputSlot(0));
+    }
+    return net;
+}
+} // namespace
+
+TEST_CASE("optimize: BoundedReLu is folded into the convolution only when that changes no byte", "cpu")
+{
+    FixedDeviceSpec spec{kMi355x};
+    {
+        INetworkPtr net = ConvReluNet(true, false);
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, spec);
+        const Graph& g = opt->GetGraph();
+        CHECK(CountLayers(g, LayerType::Activation) == 0);
+        CHECK(CountLayers(g, LayerType::Convolution2d) == 1);
+        const Layer* fused = FindLayer(g, "fused-");
+        REQUIRE(fused != nullptr);
+        auto ad = fused->GetAdditionalInformation<ActivationDescriptor>();
+        REQUIRE(ad != nullptr);
+        CHECK(ad->m_Function == ActivationFunction::BoundedReLu);
+        CHECK(ad->m_A == 6.0f);
+        CHECK(fused->GetBackendId() == kMi355x);
+        CHECK(fused->GetNumInputSlots() == 3);
+        CHECK(fused->In(1).GetConnectedOutputSlot()->GetOwningLayer().GetType() == LayerType::Constant);
+        CHECK(fused->Out(0).GetConnections()[0]->GetOwningLayer().GetType() == LayerType::Output);
+        CHECK(CountLayers(g, LayerType::MemCopy) == 0);
+    }
+    {
+        INetworkPtr net = ConvReluNet(false, false);       // the activation re-quantizes: it stays a layer
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, spec);
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Activation) == 1);
+        CHECK(FindLayer(opt->GetGraph(), "fused-") == nullptr);
+    }
+    {
+        INetworkPtr net = ConvReluNet(true, true);         // the pre-activation tensor is also a network output
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, spec);
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Activation) == 1);
+    }
+}
+
+TEST_CASE("optimize: unsupported layers fall back along the preference list, with copies between backends", "cpu")
+{
+    testhost::Register();
+    INetworkPtr net = INetwork::Create();
+    const TensorInfo in = ActInfo({1, 8, 8, 16}, DataType::QAsymmS8, 0.05f, -3);
+    QLayer c1 = MakeConv(QLayer::Conv, in, 16, 1, 1, 0.05f, -3, false, true, 21);
+    QLayer c2 = MakeConv(QLayer::Conv, c1.out, 8, 1, 1, 0.05f, -3, false, true, 22);
+    IConnectableLayer* input = net->AddInputLayer(0, "input");
+    input->GetOutputSlot(0).SetTensorInfo(in);
+    IOutputSlot& s1 = AddToNetwork(*net, input->GetOutputSlot(0), c1, "conv1");
+    IConnectableLayer* lin = net->AddActivationLayer(ActivationDescriptor(ActivationFunction::Linear, 1.0f, 0.0f), "identity");
+    s1.Connect(lin->GetInputSlot(0));
+    lin->GetOutputSlot(0).SetTensorInfo(c1.out);
+    IOutputSlot& s2 = AddToNetwork(*net, lin->GetOutputSlot(0), c2, "conv2");
+    IConnectableLayer* out = net->AddOutputLayer(0, "output");
+    s2.Connect(out->GetInputSlot(0));
+
+    FixedDeviceSpec both{kMi355x, testhost::Id()};
+    std::vector<std::string> messages;
+    IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x, testhost::Id()}, both, OptimizerOptionsOpaque(), Optional<std::vector<std::string>&>(messages));
+    const Graph& g = opt->GetGraph();
+    CHECK(FindLayer(g, "identity")->GetBackendId() == testhost::Id());
+    CHECK(FindLayer(g, "conv1")->GetBackendId() == kMi355x);
+    CHECK(CountLayers(g, LayerType::MemCopy) == 2);
+    bool warned = false;
+    for (const auto& m : messages) warned |= m.find("Activation") != std::string::npos && m.find("falling back") != std::string::npos;
+    CHECK(warned);
+
+    // no backend takes the convolution: Optimize refuses
+    FixedDeviceSpec hostOnly{testhost::Id()};
+    CHECK_THROWS_AS(Optimize(*net, {kMi355x, testhost::Id()}, hostOnly), InvalidArgumentException);
+    // no preferred backend is present at all
+    FixedDeviceSpec none{};
+    CHECK_THROWS_AS(Optimize(*net, {kMi355x}, none), InvalidArgumentException);
+    CHECK_THROWS_AS(Optimize(*net, {}, both), InvalidArgumentException);
+}
+
+TEST_CASE("runtime: without a device the backend is left out and nothing runs on a substitute", "cpu")
+{
+    if (mi355x::DeviceCount() > 0)
+    {
+        std::printf("    (a device is present: the no-device path is covered where there is none)\n");
+        return;
+    }
+    Mi355xBackend backend;
+    CHECK_THROWS_AS(backend.CreateBackendContext(IRuntime::CreationOptions()), BackendUnavailableException);
+    IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+    CHECK(rt->GetDeviceSpec().GetSupportedBackends().count(kMi355x) == 0);
+    QLayer l = MakeConv(QLayer::Conv, ActInfo({1, 8, 8, 16}, DataType::QAsymmS8, 0.05f, -3), 32, 3, 1, 0.1f, 5, true, true, 31);
+    SingleLayerNet n(l);
+    CHECK_THROWS_AS(Optimize(*n.net, {kMi355x}, rt->GetDeviceSpec()), InvalidArgumentException);
+    // workloads exist without a device, but executing one fails loudly
+    FixedDeviceSpec pretend{kMi355x};
+    IOptimizedNetworkPtr opt = Optimize(*n.net, {kMi355x}, pretend);
+    NetworkId id = -1;
+    std::string err;
+    CHECK(rt->LoadNetwork(id, std::move(opt), err) == Status::Failure);
+    CHECK_MSG(err.find("unavailable") != std::string::npos || err.find("failed") != std::string::npos, err);
+}
+
+// ---------------------------------------------------------------------------------------------------------------------
+// gpu
+// ---------------------------------------------------------------------------------------------------------------------
+namespace
+{
+void CheckSingleLayer(const QLayer& l, uint64_t seed, const char* what)
+{
+    IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+    REQUIRE(rt->GetDeviceSpec().GetSupportedBackends().count(kMi355x) == 1);
+    SingleLayerNet n(l);
+    const std::vector<uint8_t> input = RandomActivations(l.in, seed);
+    const std::vector<uint8_t> got = RunOnRuntime(*rt, *n.net, {kMi355x}, l.in, input, l.out, 2);
+    const std::vector<uint8_t> want = OracleRun(l, input);
+    const Diff d = Compare(got, want, l.out.GetDataType());
+    std::printf("    %s: %zu outputs, max |diff| %d LSB, exact %.5f\n", what, d.n, d.maxAbs, 1.0 - static_cast<double>(d.mismatches) / static_cast<double>(d.n));
+    CHECK(d.maxAbs <= 1);
+    CHECK(static_cast<double>(d.mismatches) <= 0.002 * static_cast<double>(d.n));
+    // not a constant answer
+    size_t distinct = 0;
+    bool seen[256] = {false};
+    for (uint8_t v : got) if (!seen[v]) { seen[v] = true; ++distinct; }
+    CHECK(distinct > 8);
+}
+} // namespace
+
+TEST_CASE("runtime: Convolution2d 3x3 s2, per-axis QSymmS8 weights, QAsymmS8, fused BoundedReLu", "gpu")
+{
+    CheckSingleLayer(MakeConv(QLayer::Conv, ActInfo({2, 23, 19, 16}, DataType::QAsymmS8, 0.0235f, -7), 48, 3, 2, 0.0235f, -128, true, true, 101), 1, "conv3x3");
+}
+
+TEST_CASE("runtime: pointwise Convolution2d, per-tensor weights, QAsymmU8", "gpu")
+{
+    CheckSingleLayer(MakeConv(QLayer::Conv, ActInfo({3, 14, 14, 64}, DataType::QAsymmU8, 0.0235f, 120), 128, 1, 1, 0.03f, 110, false, false, 102), 2, "conv1x1-u8");
+}
+
+TEST_CASE("runtime: stem Convolution2d with 3 input channels", "gpu")
+{
+    CheckSingleLayer(MakeConv(QLayer::Conv, ActInfo({2, 32, 32, 3}, DataType::QAsymmS8, 0.0078f, 0), 32, 3, 2, 0.0235f, -128, true, true, 103), 3, "stem");
+}
+
+TEST_CASE("runtime: DepthwiseConvolution2d 3x3, per-axis weights, fused BoundedReLu", "gpu")
+{
+    CheckSingleLayer(MakeConv(QLayer::Depthwise, ActInfo({2, 28, 28, 64}, DataType::QAsymmS8, 0.0235f, -128), 64, 3, 1, 0.0235f, -128, true, true, 104), 4, "dw3x3");
+    CheckSingleLayer(MakeConv(QLayer::Depthwise, ActInfo({1, 15, 15, 24}, DataType::QAsymmU8, 0.0235f, 3), 24, 3, 2, 0.0235f, 0, true, true, 105), 5, "dw3x3-s2-u8");
+}
+
+TEST_CASE("runtime: FullyConnected, per-axis weights", "gpu")
+{
+    CheckSingleLayer(MakeFc(ActInfo({5, 1, 1, 256}, DataType::QAsymmS8, 0.02f, -128), 100, 0.09f, -20, true, 106), 6, "fc");
+}
+
+namespace
+{
+// stem conv -> dw -> pw -> dw s2 -> pw -> global average pool -> FC -> softmax, relu6 everywhere it belongs
+struct MiniMobileNet
+{
+    std::vector<QLayer> layers;
+    TensorInfo in, pooled, logits, probs;
+    MiniMobileNet(unsigned int batch, DataType t)
+    {
+        const int zp = t == DataType::QAsymmU8 ? 0 : -128;
+        in = ActInfo({batch, 32, 32, 3}, t, 0.0078f, t == DataType::QAsymmU8 ? 128 : 0);
+        layers.push_back(MakeConv(QLayer::Conv, in, 32, 3, 2, 0.0235f, zp, true, true, 201));
+        layers.push_back(MakeConv(QLayer::Depthwise, layers.back().out, 32, 3, 1, 0.0235f, zp, true, true, 202));
+        layers.push_back(MakeConv(QLayer::Conv, layers.back().out, 64, 1, 1, 0.0235f, zp, true, true, 203));
+        layers.push_back(MakeConv(QLayer::Depthwise, layers.back().out, 64, 3, 2, 0.0235f, zp, true, true, 204));
+        layers.push_back(MakeConv(QLayer::Conv, layers.back().out, 128, 1, 1, 0.0235f, zp, true, true, 205));
+        const TensorInfo& last = layers.back().out;
+        pooled = TensorInfo(TensorShape({batch, 1, 1, 128}), t, 0.0235f, zp);
+        (void)last;
+        layers.push_back(MakeFc(pooled, 10, 0.1f, t == DataType::QAsymmU8 ? 128 : 0, true, 206));
+        logits = layers.back().out;
+        probs = TensorInfo(TensorShape({batch, 10}), t, 1.0f / 256.0f, zp);
+    }
+
+    INetworkPtr Build() const
+    {
+        INetworkPtr net = INetwork::Create();
+        IConnectableLayer* input = net->AddInputLayer(0, "input");
+        input->GetOutputSlot(0).SetTensorInfo(in);
+        IOutputSlot* slot = &input->GetOutputSlot(0);
+        for (size_t i = 0; i < 5; ++i) slot = &AddToNetwork(*net, *slot, layers[i], "l" + std::to_string(i));
+        Pooling2dDescriptor pd;
+        pd.m_DataLayout = DataLayout::NHWC;
+        pd.m_PoolType = PoolingAlgorithm::Average;
+        pd.m_PoolWidth = layers[4].out.GetShape()[2];
+        pd.m_PoolHeight = layers[4].out.GetShape()[1];
+        pd.m_StrideX = pd.m_StrideY = 1;
+        IConnectableLayer* pool = net->AddPooling2dLayer(pd, "avgpool");
+        slot->Connect(pool->GetInputSlot(0));
+        pool->GetOutputSlot(0).SetTensorInfo(pooled);
+        slot = &AddToNetwork(*net, pool->GetOutputSlot(0), layers[5], "logits");
+        IConnectableLayer* sm = net->AddSoftmaxLayer(SoftmaxDescriptor(), "softmax");
+        slot->Connect(sm->GetInputSlot(0));
+        sm->GetOutputSlot(0).SetTensorInfo(probs);
+        IConnectableLayer* out = net->AddOutputLayer(0, "output");
+        sm->GetOutputSlot(0).Connect(out->GetInputSlot(0));
+        return net;
+    }
+
+    // the same layers through the C ABI, one call after the other, every tensor in a buffer of its own
+    std::vector<uint8_t> RunDirect(const std::vector<uint8_t>& input) const
+    {
+        auto check = [](int rc, const char* what) { if (rc) throw std::runtime_error(std::string(what) + ": " + mi355x_last_error()); };
+        const unsigned int batch = in.GetShape()[0];
+        std::vector<void*> bufs;
+        auto alloc = [&](size_t n) { void* p = nullptr; check(mi355x_malloc(&p, n), "malloc"); bufs.push_back(p); return p; };
+        void* cur = alloc(input.size());
+        check(mi355x_memcpy_h2d(cur, input.data(), input.size(), nullptr), "h2d");
+        for (size_t i = 0; i < layers.size(); ++i)
+        {
+            const QLayer& l = layers[i];
+            mi355x_const_quant wq{MI355X_QSYMM_S8, 0, static_cast<uint32_t>(l.wScales.size()), l.wScales.data()};
+            mi355x_const_quant bq{MI355X_SIGNED32, 0, static_cast<uint32_t>(l.bScales.size()), l.bScales.data()};
+            if (i == 5)
+            {
+                mi355x_pool2d_desc pd{};
+                pd.in_h = layers[4].out.GetShape()[1]; pd.in_w = layers[4].out.GetShape()[2]; pd.channels = 128; pd.out_h = pd.out_w = 1;
+                pd.pool_w = pd.in_w; pd.pool_h = pd.in_h; pd.stride_x = pd.stride_y = 1;
+                pd.pool_type = 1; pd.padding_method = 1;
+                pd.input = mi355x::ToQuant(layers[4].out); pd.output = mi355x::ToQuant(pooled);
+                void* next = alloc(pooled.GetNumBytes());
+                check(mi355x_pool2d_run(&pd, batch, cur, next, nullptr), "pool");
+                cur = next;
+                mi355x_fc_desc fd{};
+                fd.k = 128; fd.out_features = 10; fd.transpose_weights = 1; fd.bias_enabled = 1;
+                fd.input = mi355x::ToQuant(l.in); fd.output = mi355x::ToQuant(l.out);
+                mi355x_fc_t plan = nullptr;
+                check(mi355x_fc_create(&fd, l.weights.data(), &wq, l.bias.data(), &bq, &plan), "fc_create");
+                next = alloc(l.out.GetNumBytes());
+                check(mi355x_fc_run(plan, batch, cur, next, nullptr), "fc_run");
+                check(mi355x_device_synchronize(), "sync");
+                mi355x_fc_destroy(plan);
+                cur = next;
+                continue;
+            }
+            mi355x_conv2d_desc d{};
+            d.in_h = l.in.GetShape()[1]; d.in_w = l.in.GetShape()[2]; d.in_c = l.in.GetShape()[3];
+            d.out_h = l.out.GetShape()[1]; d.out_w = l.out.GetShape()[2]; d.out_c = l.out.GetShape()[3];
+            d.kernel_h = l.w.GetShape()[1]; d.kernel_w = l.w.GetShape()[2];
+            d.pad_top = l.padTop; d.pad_left = l.padLeft; d.stride_x = d.stride_y = l.stride; d.dilation_x = d.dilation_y = 1;
+            d.depthwise = l.kind == QLayer::Depthwise; d.bias_enabled = 1;
+            d.input = mi355x::ToQuant(l.in); d.output = mi355x::ToQuant(l.out);
+            d.activation = MI355X_ACT_BOUNDED_RELU; d.activation_a = 6.0f; d.activation_b = 0.0f;
+            mi355x_conv2d_t plan = nullptr;
+            check(mi355x_conv2d_create(&d, l.weights.data(), &wq, l.bias.data(), &bq, &plan), "conv_create");
+            void* next = alloc(l.out.GetNumBytes());
+            check(mi355x_conv2d_run(plan, batch, cur, next, nullptr), "conv_run");
+            check(mi355x_device_synchronize(), "sync");
+            mi355x_conv2d_destroy(plan);
+            cur = next;
+        }
+        const mi355x_quant qi = mi355x::ToQuant(logits), qo = mi355x::ToQuant(probs);
+        void* sm = alloc(probs.GetNumBytes());
+        check(mi355x_softmax_run(batch, 10, 1.0f, &qi, &qo, cur, sm, nullptr), "softmax");
+        std::vector<uint8_t> out(probs.GetNumBytes());
+        check(mi355x_memcpy_d2h(out.data(), sm, out.size(), nullptr), "d2h");
+        check(mi355x_device_synchronize(), "sync");
+        for (void* p : bufs) mi355x_free(p);
+        return out;
+    }
+};
+} // namespace
+
+TEST_CASE("runtime: a small MobileNet gives the bytes of the same C-ABI calls made one by one", "gpu")
+{
+    for (DataType t : {DataType::QAsymmS8, DataType::QAsymmU8})
+    {
+        MiniMobileNet m(4, t);
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        INetworkPtr net = m.Build();
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, rt->GetDeviceSpec());
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Activation) == 0);       // all five relu6 folded
+        CHECK(CountLayers(opt->GetGraph(), LayerType::MemCopy) == 0);
+        opt.reset();
+        const std::vector<uint8_t> input = RandomActivations(m.in, 77);
+        const std::vector<uint8_t> got = RunOnRuntime(*rt, *net, {kMi355x}, m.in, input, m.probs, 3);
+        const std::vector<uint8_t> want = m.RunDirect(input);
+        const Diff d = Compare(got, want, t);
+        std::printf("    %s: %zu outputs, %zu differ\n", GetDataTypeName(t), d.n, d.mismatches);
+        CHECK(d.mismatches == 0);
+        // probabilities of a row sum to about 1 (256 codes)
+        for (unsigned int r = 0; r < 4; ++r)
+        {
+            int sum = 0;
+            for (unsigned int c = 0; c < 10; ++c) sum += t == DataType::QAsymmU8 ? got[r * 10 + c] : static_cast<int8_t>(got[r * 10 + c]) + 128;
+            CHECK(std::abs(sum - 256) <= 10);
+        }
+    }
+}
+
+TEST_CASE("runtime: intermediate tensors share an arena smaller than their sum", "gpu")
+{
+    MiniMobileNet m(4, DataType::QAsymmS8);
+    INetworkPtr net = m.Build();
+    FixedDeviceSpec spec{kMi355x};
+    IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, spec);
+    // replay the runtime's handle protocol by hand against one backend instance
+    Mi355xBackend backend;
+    TensorHandleFactoryRegistry registry;
+    backend.RegisterTensorHandleFactories(registry);
+    auto factory = backend.CreateWorkloadFactory(registry);
+    auto* hf = dynamic_cast<Mi355xTensorHandleFactory*>(registry.GetFactory(Mi355xTensorHandleFactory::GetIdStatic()));
+    REQUIRE(hf != nullptr);
+    std::vector<std::unique_ptr<ITensorHandle>> handles;
+    size_t total = 0;
+    const std::vector<Layer*> order = opt->GetGraph().TopologicalSort();
+    ITensorHandle* previous = nullptr;
+    for (Layer* l : order)
+    {
+        if (l->GetType() == LayerType::Constant || l->GetType() == LayerType::Input || l->GetNumOutputSlots() == 0) continue;
+        handles.push_back(hf->CreateTensorHandle(l->Out(0).GetTensorInfo(), true));
+        handles.back()->Manage();
+        total += l->Out(0).GetTensorInfo().GetNumBytes();
+        if (previous) previous->Allocate();      // a chain: the producer's input dies once the layer is placed
+        previous = handles.back().get();
+    }
+    if (previous) previous->Allocate();
+    const size_t arena = hf->GetMemoryManager()->ArenaBytes();
+    std::printf("    sum of intermediates %zu bytes, arena %zu bytes\n", total, arena);
+    CHECK(arena < total);
+    CHECK(arena >= 2 * 4 * 16 * 16 * 32u);      // the two largest neighbours must both fit
+    CHECK_NOTHROW(registry.AquireMemory());
+    CHECK(dynamic_cast<Mi355xTensorHandle*>(handles[0].get())->GetDevicePointer() != nullptr);
+    registry.ReleaseMemory();
+    (void)factory;
+}
+
+TEST_CASE("runtime: a layer the device lacks runs on the next backend and the copies preserve the data", "gpu")
+{
+    testhost::Register();
+    const TensorInfo in = ActInfo({2, 12, 12, 32}, DataType::QAsymmS8, 0.0235f, -128);
+    QLayer c1 = MakeConv(QLayer::Conv, in, 32, 1, 1, 0.0235f, -128, true, true, 301);
+    QLayer c2 = MakeConv(QLayer::Conv, c1.out, 64, 3, 1, 0.0235f, -128, true, true, 302);
+    auto build = [&](bool withIdentity) {
+        INetworkPtr net = INetwork::Create();
+        IConnectableLayer* input = net->AddInputLayer(0, "input");
+        input->GetOutputSlot(0).SetTensorInfo(in);
+        IOutputSlot* s = &AddToNetwork(*net, input->GetOutputSlot(0), c1, "conv1");
+        if (withIdentity)
+        {
+            IConnectableLayer* lin = net->AddActivationLayer(ActivationDescriptor(ActivationFunction::Linear, 1.0f, 0.0f), "identity");
+            s->Connect(lin->GetInputSlot(0));
+            lin->GetOutputSlot(0).SetTensorInfo(c1.out);
+            s = &lin->GetOutputSlot(0);
+        }
+        s = &AddToNetwork(*net, *s, c2, "conv2");
+        IConnectableLayer* out = net->AddOutputLayer(0, "output");
+        s->Connect(out->GetInputSlot(0));
+        return net;
+    };
+    IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+    REQUIRE(rt->GetDeviceSpec().GetSupportedBackends().count(testhost::Id()) == 1);
+    const std::vector<uint8_t> input = RandomActivations(in, 9);
+    const int before = testhost::CopyActivationWorkload::Executions();
+    INetworkPtr split = build(true), whole = build(false);
+    const std::vector<uint8_t> a = RunOnRuntime(*rt, *split, {kMi355x, testhost::Id()}, in, input, c2.out);
+    CHECK(testhost::CopyActivationWorkload::Executions() == before + 1);
+    const std::vector<uint8_t> b = RunOnRuntime(*rt, *whole, {kMi355x}, in, input, c2.out);
+    CHECK(Compare(a, b, DataType::QAsymmS8).mismatches == 0);
+    const std::vector<uint8_t> want = OracleRun(c2, OracleRun(c1, input));
+    // two layers deep, a 1-LSB difference after the first layer may move a few second-layer outputs by more; the
+    // bound that holds per layer is checked by the single-layer cases above
+    const Diff d = Compare(a, want, DataType::QAsymmS8);
+    std::printf("    two layers vs oracle: max |diff| %d, exact %.5f\n", d.maxAbs, 1.0 - static_cast<double>(d.mismatches) / static_cast<double>(d.n));
+    CHECK(d.maxAbs <= 2);
+    CHECK(static_cast<double>(d.mismatches) <= 0.01 * static_cast<double>(d.n));
+}
+
+TEST_CASE("runtime: new inputs give new outputs, bad bindings are refused, a failing plan fails the load or the inference", "gpu")
+{
+    IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+    QLayer l = MakeConv(QLayer::Conv, ActInfo({1, 16, 16, 16}, DataType::QAsymmS8, 0.0235f, -5), 32, 3, 1, 0.0235f, -128, true, true, 401);
+    SingleLayerNet n(l);
+    IOptimizedNetworkPtr opt = Optimize(*n.net, {kMi355x}, rt->GetDeviceSpec());
+    NetworkId id = -1;
+    std::string err;
+    REQUIRE(rt->LoadNetwork(id, std::move(opt), err) == Status::Success);
+    CHECK(rt->GetInputTensorInfo(id, 0) == l.in);
+    CHECK(rt->GetOutputTensorInfo(id, 0) == l.out);
+    CHECK_THROWS_AS(rt->GetInputTensorInfo(id, 5), InvalidArgumentException);
+    TensorInfo cin = l.in;
+    cin.SetConstant(true);
+    for (uint64_t seed : {1u, 2u, 3u})
+    {
+        const std::vector<uint8_t> input = RandomActivations(l.in, seed);
+        std::vector<uint8_t> out(l.out.GetNumBytes());
+        CHECK(rt->EnqueueWorkload(id, {{0, ConstTensor(cin, input.data())}}, {{0, Tensor(l.out, out.data())}}) == Status::Success);
+        CHECK(Compare(out, OracleRun(l, input), DataType::QAsymmS8).maxAbs <= 1);
+    }
+    std::vector<uint8_t> small(8), out(l.out.GetNumBytes());
+    TensorInfo wrong = ActInfo({1, 1, 1, 8}, DataType::QAsymmS8, 0.0235f, -5);
+    wrong.SetConstant(true);
+    CHECK_THROWS_AS(rt->EnqueueWorkload(id, {{0, ConstTensor(wrong, small.data())}}, {{0, Tensor(l.out, out.data())}}), InvalidArgumentException);
+    CHECK_THROWS_AS(rt->EnqueueWorkload(id, {}, {{0, Tensor(l.out, out.data())}}), InvalidArgumentException);
+    CHECK(rt->UnloadNetwork(id) == Status::Success);
+    CHECK(rt->UnloadNetwork(id) == Status::Failure);
+    CHECK_THROWS_AS(rt->EnqueueWorkload(id, {}, {}), InvalidArgumentException);
+}
