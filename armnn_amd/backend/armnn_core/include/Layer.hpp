@@ -74,10 +74,11 @@ public:
     const std::string& GetNameStr() const { return m_Name; }
     unsigned int GetNumInputSlots() const override { return static_cast<unsigned int>(m_InputSlots.size()); }
     unsigned int GetNumOutputSlots() const override { return static_cast<unsigned int>(m_OutputSlots.size()); }
-    const IInputSlot& GetInputSlot(unsigned int index) const override { return *m_InputSlots.at(index); }
-    IInputSlot& GetInputSlot(unsigned int index) override { return *m_InputSlots.at(index); }
-    const IOutputSlot& GetOutputSlot(unsigned int index) const override { return *m_OutputSlots.at(index); }
-    IOutputSlot& GetOutputSlot(unsigned int index) override { return *m_OutputSlots.at(index); }
+    // covariant returns, as in src/armnn/Layer.hpp:339-342: code holding a Layer gets the concrete slot types
+    const InputSlot& GetInputSlot(unsigned int index) const override { return *m_InputSlots.at(index); }
+    InputSlot& GetInputSlot(unsigned int index) override { return *m_InputSlots.at(index); }
+    const OutputSlot& GetOutputSlot(unsigned int index = 0) const override { return *m_OutputSlots.at(index); }
+    OutputSlot& GetOutputSlot(unsigned int index = 0) override { return *m_OutputSlots.at(index); }
     InputSlot& In(unsigned int i) { return *m_InputSlots.at(i); }
     OutputSlot& Out(unsigned int i) { return *m_OutputSlots.at(i); }
     const InputSlot& In(unsigned int i) const { return *m_InputSlots.at(i); }

@@ -1,7 +1,7 @@
 // Minimal host core: src/backends/backendsCommon/TensorHandleFactoryRegistry.hpp:23-67.
 #pragma once
-#include "IMemoryManager.hpp"
-#include "ITensorHandleFactory.hpp"
+#include <armnn/backends/IMemoryManager.hpp>
+#include <armnn/backends/ITensorHandleFactory.hpp>
 #include <map>
 #include <memory>
 #include <vector>

@@ -5,7 +5,7 @@
 #include <armnn/backends/DynamicBackend.hpp>
 #include <armnn/backends/IBackendInternal.hpp>
 #include <armnn/backends/MemCopyWorkload.hpp>
-#include <armnn/backends/TensorHandleFactoryRegistry.hpp>
+#include <backendsCommon/TensorHandleFactoryRegistry.hpp>
 #include <armnn/backends/WorkloadData.hpp>
 #include <armnn/backends/WorkloadFactory.hpp>
 

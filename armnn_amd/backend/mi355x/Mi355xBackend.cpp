@@ -8,7 +8,7 @@
 #include <Layer.hpp>
 #include <armnn/BackendRegistry.hpp>
 #include <armnn/backends/IBackendContext.hpp>
-#include <armnn/backends/TensorHandleFactoryRegistry.hpp>
+#include <backendsCommon/TensorHandleFactoryRegistry.hpp>
 
 #include <set>
 
@@ -117,21 +117,22 @@ BackendCapabilities Mi355xBackend::GetCapabilities() const
 OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgraph, const ModelOptions& modelOptions) const
 {
     OptimizationViews views(modelOptions);
-    std::set<const IConnectableLayer*> members(subgraph.begin(), subgraph.end());
+    const SubgraphView::IConnectableLayers& layers = subgraph.GetIConnectableLayers();
+    std::set<const IConnectableLayer*> members(layers.begin(), layers.end());
     std::set<const IConnectableLayer*> consumed;
 
-    for (IConnectableLayer* il : subgraph)
+    for (IConnectableLayer* il : layers)
     {
         if (consumed.count(il)) continue;
         Layer* base = PolymorphicDowncast<Layer*>(il);
         if (!Fusable(*base) || base->GetAdditionalInformation<ActivationDescriptor>() != nullptr) continue;
-        OutputSlot& out = base->Out(0);
+        OutputSlot& out = base->GetOutputSlot(0);
         if (out.GetNumConnections() != 1) continue;
         Layer* act = &out.GetConnections()[0]->GetOwningLayer();
         if (act->GetType() != LayerType::Activation || !members.count(act) || consumed.count(act)) continue;
         const auto& ad = static_cast<const ActivationDescriptor&>(act->GetParameters());
         if (ad.m_Function != ActivationFunction::ReLu && ad.m_Function != ActivationFunction::BoundedReLu) continue;
-        if (!SameQuantization(out.GetTensorInfo(), act->Out(0).GetTensorInfo())) continue;
+        if (!SameQuantization(out.GetTensorInfo(), act->GetOutputSlot(0).GetTensorInfo())) continue;
 
         const std::string name = std::string("fused-") + act->GetName() + "-into-" + base->GetName();
         INetwork& net = views.GetINetworkRef();
@@ -151,7 +152,7 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
                 replacement = net.AddElementwiseBinaryLayer(static_cast<const ElementwiseBinaryDescriptor&>(base->GetParameters()), name.c_str());
                 break;
         }
-        replacement->GetOutputSlot(0).SetTensorInfo(act->Out(0).GetTensorInfo());
+        replacement->GetOutputSlot(0).SetTensorInfo(act->GetOutputSlot(0).GetTensorInfo());
         PolymorphicDowncast<Layer*>(replacement)->SetAdditionalInfoForObject(std::make_shared<ActivationDescriptor>(ad));
 
         SubgraphView::IInputSlots ins;
@@ -163,7 +164,7 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
         consumed.insert(act);
     }
 
-    for (IConnectableLayer* il : subgraph)
+    for (IConnectableLayer* il : layers)
         if (!consumed.count(il)) views.AddUntouchedSubgraph(SubgraphView(il));
     return views;
 }

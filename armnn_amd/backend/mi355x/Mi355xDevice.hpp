@@ -1,6 +1,7 @@
 // Process-wide device state of the backend: which GPU, the stream every workload launches on, and the translation
 // of C-ABI status codes into Arm NN exceptions.  All GPU work goes through include/armnn_mi355x.h.
 #pragma once
+#include <armnn/TypesUtils.hpp>
 #include <armnn/Exceptions.hpp>
 #include <armnn/Tensor.hpp>
 

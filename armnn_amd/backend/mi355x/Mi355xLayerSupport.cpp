@@ -1,5 +1,6 @@
 #include "Mi355xLayerSupport.hpp"
 
+#include <armnn/TypesUtils.hpp>
 #include <armnn/utility/PolymorphicDowncast.hpp>
 
 #include <cmath>

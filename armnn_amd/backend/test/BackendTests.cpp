@@ -15,7 +15,7 @@
 #include "../mi355x/Mi355xTensorHandle.hpp"
 #include "../mi355x/Mi355xWorkloadFactory.hpp"
 
-#include <armnn/backends/TensorHandleFactoryRegistry.hpp>
+#include <backendsCommon/TensorHandleFactoryRegistry.hpp>
 #include <armnn/backends/WorkloadData.hpp>
 
 using namespace armnn;

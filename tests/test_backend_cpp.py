@@ -54,3 +54,10 @@ def test_backend_networks_on_device():
 @pytest.mark.gpu
 def test_backend_dynamic_on_device():
     _run("dynamic_tests", "gpu", 300)
+
+
+@pytest.mark.skipif(not os.path.isdir("/root/reference/include/armnn"), reason="needs an Arm NN source tree")
+def test_backend_sources_compile_against_real_armnn_headers():
+    """-fsyntax-only against the reference's own headers: the backend uses no name the real API lacks."""
+    proc = subprocess.run(["make", "-C", BACKEND, "conformance"], capture_output=True, text=True, timeout=600)
+    assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
