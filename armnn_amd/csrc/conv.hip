@@ -291,8 +291,9 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         p->xor_mask = g.in_u8 ? 0x80u : 0u;
         p->pad_word = static_cast<uint32_t>(zx_shift) & 0xffu;
         p->row_dwords = RD;
+        FoldCorrIntoTable(p, corr, Co);
         char buf[96];
-        snprintf(buf, sizeof(buf), "smallci_dot4_lds %dx%dx%d stride %u, tile 16x16", Kh, Kw, Ci, d.stride_x);
+        snprintf(buf, sizeof(buf), "smallci_dot4_lds %dx%dx%d stride %u, tile 32x16", Kh, Kw, Ci, d.stride_x);
         p->info = buf;
     }
     else
@@ -482,9 +483,14 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         a.x = xin; a.wpack = p->w_dot4; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
         a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.Ci = g.Ci; a.Ho = g.Ho; a.Wo = g.Wo; a.Co = g.Co;
         a.Kw = g.Kw; a.stride = g.stride_x; a.pad_top = g.pad_top; a.pad_left = g.pad_left;
-        a.tiles_x = (g.Wo + 15) / 16; a.tiles_y = (g.Ho + 15) / 16;
+        a.tiles_x = (g.Wo + 31) / 32; a.tiles_y = (g.Ho + 15) / 16;
         a.xor_mask = p->xor_mask; a.pad_byte = p->pad_word;
-        a.ci_recip = (65536u + static_cast<uint32_t>(g.Ci) - 1u) / static_cast<uint32_t>(g.Ci);
+        // LDS row: up to 3 bytes of misalignment, 31 pixel steps, one pixel's row of RD dwords, one spare dword
+        a.lp = ((3 + 31 * g.stride_x * g.Ci + 4 * p->row_dwords + 3) & ~3) + 8;
+        a.ndw_recip = static_cast<uint32_t>((0x100000000ull + static_cast<unsigned long long>(a.lp / 4) - 1ull) / static_cast<unsigned long long>(a.lp / 4));
+        a.vec16 = ((reinterpret_cast<uintptr_t>(y) & 15) == 0 && (g.Co % 16) == 0) ? 1 : 0;
+        if (a.lp > 288) return SetError(MI355X_ERR_UNSUPPORTED, "dot4 kernel: halo row of %d bytes does not fit", a.lp);
+        if (static_cast<long long>(g.H) * g.W * g.Ci >= (1ll << 30)) return SetError(MI355X_ERR_UNSUPPORTED, "dot4 kernel: image too large for 32-bit offsets");
         a.rq = p->rq;
         const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
         if (nb > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
@@ -510,9 +516,12 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + 7) / 8; a.cblocks = g.Co / 32;
             a.xor_mask = p->xor_mask; a.pad_word = p->pad_word; a.rq = p->rq;
             const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y * a.cblocks;
-            if (nb > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
-            if (g.stride_x == 1) hipLaunchKernelGGL((Depthwise3x3Kernel<1>), dim3(static_cast<unsigned>(nb)), dim3(256), 0, stream, a);
-            else hipLaunchKernelGGL((Depthwise3x3Kernel<2>), dim3(static_cast<unsigned>(nb)), dim3(256), 0, stream, a);
+            if (nb > 0x7fffffffll - 8) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
+            a.total_blocks = static_cast<int>(nb);
+            a.xcd_chunk = static_cast<int>((nb + 7) / 8);
+            const dim3 grid(static_cast<unsigned>(a.xcd_chunk) * 8u);
+            if (g.stride_x == 1) hipLaunchKernelGGL((Depthwise3x3Kernel<1>), grid, dim3(256), 0, stream, a);
+            else hipLaunchKernelGGL((Depthwise3x3Kernel<2>), grid, dim3(256), 0, stream, a);
             MI355X_HIP(hipGetLastError());
             return 0;
         }

@@ -27,9 +27,18 @@ struct Dw3x3Args
     int N, H, W, C, Ho, Wo;
     int pad_top, pad_left;
     int tiles_x, tiles_y, cblocks;
+    int total_blocks, xcd_chunk;   // work items, and ceil(work items / 8): the grid is 8 * xcd_chunk blocks
     uint32_t xor_mask, pad_word;
     Requant rq;
 };
+
+// Consecutive block ids are dealt round-robin to the 8 XCDs, each with its own L2.  Giving XCD x the contiguous range
+// [x * chunk, (x + 1) * chunk) of work items makes blocks that run together on one XCD neighbours in the work order,
+// so the channel blocks of one pixel tile -- which read different 32-byte parts of the same cache lines -- share an L2.
+__device__ __forceinline__ int XcdContiguousWorkItem(int block, int chunk)
+{
+    return (block & 7) * chunk + (block >> 3);
+}
 
 // Block: 8 output rows x (4 groups of P pixels) x 32 channels; thread = (4 channels, P pixels of one row).
 // A thread reads 6 consecutive input pixels per kernel row (one dword = 4 channels each), transposes them with
@@ -48,7 +57,8 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
     constexpr int PITCH = 48;                    // bytes per pixel in LDS: 32 used; 48 spreads dword reads over banks
     __shared__ __attribute__((aligned(16))) uint8_t tile[HR * HC * PITCH];
 
-    int b = blockIdx.x;
+    int b = XcdContiguousWorkItem(blockIdx.x, a.xcd_chunk);
+    if ((static_cast<int>(blockIdx.x) >> 3) >= a.xcd_chunk || b >= a.total_blocks) return;
     const int cb = b % a.cblocks; b /= a.cblocks;
     const int tx = b % a.tiles_x; b /= a.tiles_x;
     const int ty = b % a.tiles_y;
@@ -154,31 +164,47 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
 }
 
 // ---------------------------------------------------------------------------------------------------------------
+// Constant address space: a wave-uniform load through such a pointer is a scalar load, whatever stores the kernel
+// makes elsewhere.  Only memory that no kernel writes while this one runs (plan constants) may be read this way.
+#define MI355X_CONST_AS __attribute__((address_space(4)))
+
+template <typename T>
+__device__ __forceinline__ const T MI355X_CONST_AS* AsConstant(const T* p)
+{
+    return (const T MI355X_CONST_AS*)p;
+}
+
 struct SmallCiArgs
 {
     const uint8_t*  x;
     const uint32_t* wpack;    // [Co][KH][RD] dwords: row r of filter co as consecutive (kx, ci) bytes, zero padded
-    ChanTab         ct;
+    ChanTab         ct;       // rows 2, 5, 6 on the fast path (accumulators start at zero), rows 0, 1 on the exact path
     const int32_t*  corr;     // [Co]
     uint8_t*        y;
     int N, H, W, Ci, Ho, Wo, Co;
     int Kw, stride, pad_top, pad_left;
     int tiles_x, tiles_y;
+    int lp;                   // LDS row pitch in bytes (multiple of 4)
+    uint32_t ndw_recip;       // ceil(2^32 / (lp / 4))
     uint32_t xor_mask, pad_byte;
-    uint32_t ci_recip;        // ceil(65536 / Ci): (b * ci_recip) >> 16 == b / Ci for the small b used here
+    int vec16;                // output rows allow 16-byte stores (y 16-byte aligned, Co % 16 == 0)
     Requant rq;
 };
 
-// Block: 16 x 16 output pixels; thread = one pixel, all output channels.  The input halo is staged byte by byte
-// (rows start at arbitrary byte addresses when Ci is 3), each thread then reads its KH rows of Kw*Ci contiguous
-// bytes as aligned dwords + v_alignbyte, and walks the output channels with wave-uniform (scalar-loaded) weights.
+// Block: 32 x 16 output pixels; thread = two horizontally adjacent pixels, all output channels.
+//   Staging: each halo row is copied as ALIGNED dwords (rows start at arbitrary byte addresses when Ci is 3, so the
+//   LDS row keeps the global misalignment and readers add it back); only dwords that straddle an image edge are
+//   assembled byte by byte, and positions outside the image hold the shifted zero point.
+//   Compute: a thread reads its KH rows of Kw*Ci contiguous bytes as aligned dwords + v_alignbyte, then walks the
+//   output channels; weights and requantization constants are wave-uniform scalar loads, so a v_dot4 takes its
+//   weight operand from an SGPR.  16 channels of a pixel leave as one 16-byte store.
 template <int KH, int RD>
 __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
 {
-    constexpr int TW = 16, TH = 16;
+    constexpr int P = 2, TW = 16 * P, TH = 16;
     constexpr int HRMAX = (TH - 1) * 2 + KH;
-    constexpr int LP = (TW - 1) * 2 * 4 + RD * 4 + 8;       // LDS row pitch in bytes (multiple of 4)
-    __shared__ __attribute__((aligned(16))) uint8_t tile[HRMAX * LP + 16];
+    constexpr int LPMAX = 288;                               // >= 3 + (TW-1)*2*4 + 4*6 rounded up, + 8
+    __shared__ __attribute__((aligned(16))) uint32_t tile[HRMAX * LPMAX / 4];
 
     int b = blockIdx.x;
     const int tx = b % a.tiles_x; b /= a.tiles_x;
@@ -187,67 +213,147 @@ __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
     const int tid = threadIdx.x;
     const int S = a.stride;
     const int HR = (TH - 1) * S + KH;
-    const int RB = ((TW - 1) * S + a.Kw) * a.Ci;            // bytes per halo row that carry data
+    const int NDW = a.lp >> 2;
 
     const int iy_org = ty * TH * S - a.pad_top;
     const int ix_org = tx * TW * S - a.pad_left;
     const uint8_t* xn = a.x + static_cast<long long>(n) * a.H * a.W * a.Ci;
-    const uint8_t xm = static_cast<uint8_t>(a.xor_mask);
-    for (int row = tid >> 6; row < HR; row += 4)
+    const int mis = static_cast<int>(reinterpret_cast<uintptr_t>(xn) & 3);
+    const uint8_t* xal = xn - mis;                           // 4-byte aligned
+    const uint32_t xm = a.xor_mask & 0xffu;
+    const uint32_t xm4 = xm * 0x01010101u;
+    const uint32_t pad4 = (a.pad_byte & 0xffu) * 0x01010101u;
+    // columns of the halo that lie inside the image, as byte offsets from the halo's first column
+    const int vb0 = max(0, -ix_org) * a.Ci;
+    const int vb1 = min((TW - 1) * S + a.Kw, a.W - ix_org) * a.Ci;
+    // Two passes so that all of a thread's global loads are in flight together: pass 1 issues the aligned dword
+    // loads, pass 2 assembles the few dwords that straddle an image edge and writes everything to LDS.
+    constexpr int MAXIT = (HRMAX * (LPMAX / 4) + 255) / 256;
+    const int total = HR * NDW;
+    uint32_t sv[MAXIT];
+    // loads are unconditional (a dword that is not wholly inside the image reads a harmless in-tensor address and
+    // is discarded), so that none of them waits for another
+    const long long safe = reinterpret_cast<const uint8_t*>((reinterpret_cast<uintptr_t>(a.x) + 3) & ~static_cast<uintptr_t>(3)) - xal;
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k)
     {
+        const int i = min(tid + k * 256, total - 1);
+        const int row = static_cast<int>(__umulhi(static_cast<uint32_t>(i), a.ndw_recip));
+        const int j = i - row * NDW;
         const int iy = iy_org + row;
-        const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(a.H);
-        const uint8_t* xrow = xn + static_cast<long long>(iy) * a.W * a.Ci;
-        for (int bcol = tid & 63; bcol < LP; bcol += 64)
+        const int A = (iy * a.W + ix_org) * a.Ci + mis;      // halo row start as a byte offset from xal (may be < 0)
+        const int lo = (A & ~3) + 4 * j;
+        const bool inside = static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && lo >= A + vb0 && lo + 4 <= A + vb1;
+        const uint32_t ld = *reinterpret_cast<const uint32_t*>(xal + (inside ? static_cast<long long>(lo) : safe));
+        sv[k] = inside ? (ld ^ xm4) : pad4;
+    }
+#pragma unroll
+    for (int k = 0; k < MAXIT; ++k)
+    {
+        const int i = tid + k * 256;
+        if (i < total)
         {
-            uint8_t v = static_cast<uint8_t>(a.pad_byte);
-            if (row_ok && bcol < RB)
+            const int row = static_cast<int>(__umulhi(static_cast<uint32_t>(i), a.ndw_recip));
+            const int j = i - row * NDW;
+            const int iy = iy_org + row;
+            const int A = (iy * a.W + ix_org) * a.Ci + mis;
+            const int lo = (A & ~3) + 4 * j;
+            const int vbeg = A + vb0, vend = A + vb1;
+            uint32_t v = sv[k];
+            const bool inside = lo >= vbeg && lo + 4 <= vend;
+            if (static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && !inside && lo + 4 > vbeg && lo < vend)
             {
-                const int pix = static_cast<int>((static_cast<uint32_t>(bcol) * a.ci_recip) >> 16);
-                const int ix = ix_org + pix;
-                if (static_cast<unsigned>(ix) < static_cast<unsigned>(a.W))
-                    v = xrow[ix_org * a.Ci + bcol] ^ xm;
+                v = 0;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                {
+                    const int o = lo + q;
+                    uint32_t byte = a.pad_byte & 0xffu;
+                    if (o >= vbeg && o < vend) byte = static_cast<uint32_t>(xal[o]) ^ xm;
+                    v |= byte << (8 * q);
+                }
             }
-            tile[row * LP + bcol] = v;
+            tile[i] = v;
         }
     }
     __syncthreads();
 
     const int lx = tid & 15, ly = tid >> 4;
-    uint32_t xr[KH][RD];
+    uint32_t xr[P][KH][RD];
 #pragma unroll
     for (int r = 0; r < KH; ++r)
     {
-        const int off = (ly * S + r) * LP + lx * S * a.Ci;
-        const uint32_t* p = reinterpret_cast<const uint32_t*>(tile + (off & ~3));
-        const int sh = off & 3;
-        uint32_t d[RD + 1];
+        const int row = ly * S + r;
+        const int sh_row = ((((iy_org + row) * a.W + ix_org) * a.Ci + mis) & 3);
 #pragma unroll
-        for (int i = 0; i <= RD; ++i) d[i] = p[i];
+        for (int p = 0; p < P; ++p)
+        {
+            const int off = row * a.lp + sh_row + (lx * P + p) * S * a.Ci;
+            const uint32_t* q = tile + (off >> 2);
+            const int sh = off & 3;
+            uint32_t d[RD + 1];
 #pragma unroll
-        for (int i = 0; i < RD; ++i) xr[r][i] = __builtin_amdgcn_alignbyte(d[i + 1], d[i], sh);
+            for (int i = 0; i <= RD; ++i) d[i] = q[i];
+#pragma unroll
+            for (int i = 0; i < RD; ++i) xr[p][r][i] = __builtin_amdgcn_alignbyte(d[i + 1], d[i], sh);
+        }
     }
 
-    const int oy = ty * TH + ly, ox = tx * TW + lx;
-    if (oy >= a.Ho || ox >= a.Wo) return;
-    uint8_t* yp = a.y + ((static_cast<long long>(n) * a.Ho + oy) * a.Wo + ox) * a.Co;
-    for (int co = 0; co < a.Co; co += 4)
+    const int oy = ty * TH + ly, ox0 = tx * TW + lx * P;
+    if (oy >= a.Ho || ox0 >= a.Wo) return;
+    const bool second = ox0 + 1 < a.Wo;
+    uint8_t* yp = a.y + ((static_cast<long long>(n) * a.Ho + oy) * a.Wo + ox0) * a.Co;
+    const uint32_t MI355X_CONST_AS* wc = AsConstant(a.wpack);
+    const float MI355X_CONST_AS* tab = AsConstant(a.ct.p);
+    const int ts = a.ct.stride;
+    for (int co = 0; co < a.Co; co += 16)
     {
-        int q[4];
-        const Fast4 f4 = LoadFast4(a.ct, co);
+        const int groups = min(4, (a.Co - co) >> 2);
+        uint32_t o[P][4];
 #pragma unroll
-        for (int u = 0; u < 4; ++u)
+        for (int g4 = 0; g4 < 4; ++g4)
         {
-            const uint32_t* w = a.wpack + static_cast<long long>(co + u) * KH * RD;
-            int acc = a.corr[co + u];
+            if (g4 >= groups) continue;
+            const int c = co + 4 * g4;
+            int acc[P][4];
 #pragma unroll
-            for (int r = 0; r < KH; ++r)
+            for (int u = 0; u < 4; ++u)
+            {
+                const uint32_t MI355X_CONST_AS* w = wc + (c + u) * (KH * RD);
 #pragma unroll
-                for (int i = 0; i < RD; ++i)
-                    acc = __builtin_amdgcn_sdot4(static_cast<int>(xr[r][i]), static_cast<int>(w[r * RD + i]), acc, false);
-            q[u] = acc;
+                for (int p = 0; p < P; ++p) acc[p][u] = 0;
+#pragma unroll
+                for (int r = 0; r < KH; ++r)
+#pragma unroll
+                    for (int i = 0; i < RD; ++i)
+                    {
+                        const int wv = static_cast<int>(w[r * RD + i]);
+#pragma unroll
+                        for (int p = 0; p < P; ++p) acc[p][u] = __builtin_amdgcn_sdot4(static_cast<int>(xr[p][r][i]), wv, acc[p][u], false);
+                    }
+            }
+            const float4 fm = {tab[2 * ts + c], tab[2 * ts + c + 1], tab[2 * ts + c + 2], tab[2 * ts + c + 3]};
+            const float4 fb = {tab[5 * ts + c], tab[5 * ts + c + 1], tab[5 * ts + c + 2], tab[5 * ts + c + 3]};
+            const float4 th = {tab[6 * ts + c], tab[6 * ts + c + 1], tab[6 * ts + c + 2], tab[6 * ts + c + 3]};
+#pragma unroll
+            for (int p = 0; p < P; ++p)
+                o[p][g4] = Requant4Dev(acc[p][0], acc[p][1], acc[p][2], acc[p][3], fm, fb, th, a.ct, a.corr, c, a.rq);
         }
-        *reinterpret_cast<uint32_t*>(yp + co) = Requant4Dev(q[0], q[1], q[2], q[3], f4, a.ct, co, a.rq);
+        if (groups == 4 && a.vec16)
+        {
+            *reinterpret_cast<uint4*>(yp + co) = uint4{o[0][0], o[0][1], o[0][2], o[0][3]};
+            if (second) *reinterpret_cast<uint4*>(yp + a.Co + co) = uint4{o[1][0], o[1][1], o[1][2], o[1][3]};
+        }
+        else
+        {
+#pragma unroll
+            for (int g4 = 0; g4 < 4; ++g4)
+            {
+                if (g4 >= groups) continue;
+                *reinterpret_cast<uint32_t*>(yp + co + 4 * g4) = o[0][g4];
+                if (second) *reinterpret_cast<uint32_t*>(yp + a.Co + co + 4 * g4) = o[1][g4];
+            }
+        }
     }
 }
 

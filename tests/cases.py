@@ -198,6 +198,10 @@ def small_conv_cases():
     c.append(make_conv_case("stem_s8_3x3_s1_ci1", 222, h=20, w=33, ci=1, co=8, in_offset=-100))
     c.append(make_conv_case("stem_s8_5x5_ci4", 223, h=21, w=18, ci=4, co=12, kh=5, kw=5, padding=(1, 2, 0, 3)))
     c.append(make_conv_case("stem_s8_1x1_ci4", 224, h=9, w=9, ci=4, co=16, kh=1, kw=1))
+    # several tiles in x and y, rows and images that start at odd byte addresses, a lone last column
+    c.append(make_conv_case("stem_u8_3x3_s1_ci3_wide", 225, n=3, h=37, w=71, ci=3, co=20, in_dtype=U8, in_offset=77,
+                            out_offset=3))
+    c.append(make_conv_case("stem_s8_3x3_s2_ci2", 226, n=2, h=35, w=131, ci=2, co=48, stride=(2, 2), in_offset=5))
     c.append(make_conv_case("dw_u8_5x5_c20", 206, h=9, w=9, ci=20, depthwise=True, kh=5, kw=5, in_dtype=U8,
                             in_offset=100, out_offset=3, w_scale_range=(0.005, 0.02)))
     return c
