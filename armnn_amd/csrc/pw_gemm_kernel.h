@@ -79,10 +79,6 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
     const int tile0 = g * 4 + wave;              // first tile of this wave
 
     v16i acc[TC];
-#pragma unroll
-    for (int tc = 0; tc < TC; ++tc)
-#pragma unroll
-        for (int v = 0; v < 16; ++v) acc[tc][v] = 0;
 
     auto load_chunk = [&](v4i (&buf)[KS], int t, int ch) {
         const int row = t * 32 + frag_row;
@@ -99,8 +95,11 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
         }
     };
 
-    auto compute_chunk = [&](v4i (&buf)[KS], int ch) {
+    // FIRST: the chunk opens a tile; its first MFMA takes a zero C operand instead of cleared registers
+    auto compute_chunk = [&](v4i (&buf)[KS], int ch, auto first) {
+        constexpr bool FIRST = decltype(first)::value;
         const uint8_t* wbase = slab + frag_row * LDW + ch * (32 * KS) + frag_k;
+        const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
 #pragma unroll
         for (int ks = 0; ks < KS; ++ks)
         {
@@ -109,7 +108,7 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
             for (int tc = 0; tc < TC; ++tc)
             {
                 const v4i wv = *reinterpret_cast<const v4i*>(wbase + tc * 32 * LDW + ks * 32);
-                acc[tc] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wv, av, acc[tc], 0, 0, 0);
+                acc[tc] = __builtin_amdgcn_mfma_i32_32x32x32_i8(wv, av, (FIRST && ks == 0) ? zero : acc[tc], 0, 0, 0);
             }
         }
     };
@@ -130,8 +129,6 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
                                                  fm, fb, th, a.ct, a.corr, n0 + cl, a.rq);
                 *reinterpret_cast<uint32_t*>(ostage + frag_row * LDO + cl) = out;
             }
-#pragma unroll
-            for (int v = 0; v < 16; ++v) acc[tc][v] = 0;
         }
         // the wave reads back what its own lanes wrote: LDS operations of one wave complete in order; the fences keep
         // the compiler from moving the reads above the writes (different lanes, so no dependency it can see)
@@ -212,7 +209,8 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
         auto step = [&](auto jc) {
             constexpr int J = decltype(jc)::value;
             if (more) load_chunk(buf[(J + NB - 1) % NB], t_nxt, c_nxt);
-            compute_chunk(buf[J], c_cur);
+            if (c_cur == 0) compute_chunk(buf[J], 0, std::true_type{});
+            else compute_chunk(buf[J], c_cur, std::false_type{});
         };
         if (j == 0) step(std::integral_constant<int, 0>{});
         else if (j == 1) step(std::integral_constant<int, 1>{});
