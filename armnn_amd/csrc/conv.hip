@@ -21,6 +21,7 @@ struct mi355x_conv2d_s
     // device constants
     uint8_t* w_direct = nullptr;   // [Kh][Kw][Ci][Co] / depthwise [Kh][Kw][Co], raw codes
     int8_t*  w_mfma   = nullptr;   // [Co_pad][K_pad] signed, zero padded
+    uint8_t* pad16    = nullptr;   // 16 bytes that turn into the padding value under the kernel's input xor
     uint32_t* w_dot4  = nullptr;   // depthwise 3x3: [C][4] dwords; small-Ci conv: [Co][Kh][RD] dwords
     int variant = 0;               // kernel variant within an algo (see RunPlan)
     int row_dwords = 0;            // small-Ci conv: dwords per filter row
@@ -29,6 +30,7 @@ struct mi355x_conv2d_s
     int K = 0, K_pad = 0, Co_pad = 0;
     std::vector<float> chan_host;  // host copy, completed with the corr-folded rows once corr is known
     int pw_bn = 0, pw_ks = 0;      // pointwise GEMM kernel configuration (0: not applicable)
+    bool bk128 = false;            // implicit GEMM walks K in 128-byte tiles
     int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 128: force (MI355X_IGEMM_TILE, for experiments)
     uint32_t xor_mask = 0, pad_word = 0;
     std::string info;
@@ -37,6 +39,7 @@ struct mi355x_conv2d_s
     {
         (void)hipFree(w_direct);
         (void)hipFree(w_mfma);
+        (void)hipFree(pad16);
         (void)hipFree(w_dot4);
         (void)hipFree(chan);
         (void)hipFree(corr);
@@ -121,7 +124,11 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
 
     p->K = d.depthwise ? Kh * Kw : Kh * Kw * Ci;
     p->Co_pad = (Co + 127) / 128 * 128;
-    p->K_pad = (p->K + kIgemmBK - 1) / kIgemmBK * kIgemmBK;
+    // K is padded to the implicit GEMM's k-tile.  128-byte tiles pay when a row chunk is one whole cache line, i.e. when
+    // 128 consecutive K bytes are contiguous in memory (input channels a multiple of 128) and K needs no extra padding
+    // for it; otherwise 64.
+    p->K_pad = (p->K + 63) / 64 * 64;
+    p->bk128 = (d.in_c % 128) == 0 && (p->K % 128) == 0;
 
     // ---- per-channel requantization constants, in fp32 exactly as the reference's decoders produce them ----
     std::vector<float> mult(p->Co_pad, 0.0f), biasf(p->Co_pad, 0.0f);
@@ -222,6 +229,10 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         p->xor_mask = g.in_u8 ? 0x80808080u : 0u;
         const uint32_t zb = static_cast<uint32_t>(zx_shift) & 0xffu;
         p->pad_word = zb | (zb << 8) | (zb << 16) | (zb << 24);
+        {
+            const std::vector<uint8_t> padbytes(16, static_cast<uint8_t>((zb ^ (g.in_u8 ? 0x80u : 0u)) & 0xffu));
+            if (int rc = Upload(reinterpret_cast<void**>(&p->pad16), padbytes.data(), padbytes.size())) return rc;
+        }
         if (const char* t = std::getenv("MI355X_IGEMM_TILE")) p->tile_override = std::atoi(t);
         FoldCorrIntoTable(p, corr, Co);
         ChoosePointwiseConfig(p);
@@ -230,7 +241,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         if (p->pw_bn)
             snprintf(buf, sizeof(buf), "pointwise_gemm_mfma_i8_32x32x32 weight-stationary slab %dxK=%d, chunk %d k-steps", p->pw_bn, p->K, p->pw_ks);
         else
-            snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 tiles 128x128|128x64|64x64 x%d K=%d", kIgemmBK, p->K);
+            snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 tiles 128x128|128x64|64x64 x%d K=%d", p->bk128 ? 128 : 64, p->K);
         p->info = buf;
     }
     else if (algo == MI355X_ALGO_DEPTHWISE && dw3_ok)
@@ -347,7 +358,9 @@ void ChoosePointwiseConfig(mi355x_conv2d_s* p)
     const bool pointwise = !d.depthwise && d.kernel_h == 1 && d.kernel_w == 1 && d.stride_x == 1 && d.stride_y == 1 &&
                            d.pad_top == 0 && d.pad_left == 0 && d.out_h == d.in_h && d.out_w == d.in_w;
     const int K = static_cast<int>(d.in_c), N = static_cast<int>(d.out_c);
-    if (!pointwise || (K % 32) != 0) return;
+    // with K beyond 128 the LDS-tiled implicit GEMM is the faster kernel (its k-tiles keep more loads in flight than a
+    // wave's register chunks can); the weight-stationary kernel is for the shallow, wide-M layers
+    if (!pointwise || (K % 32) != 0 || K > 128) return;
     const int budget = 80 * 1024;
     int bn = 0;
     if (N > 64 && PwSmemBytes<128>(K) <= budget) bn = 128;
@@ -414,12 +427,13 @@ int LaunchPwKs(const mi355x_conv2d_s* p, long long M, const void* x, void* y, hi
     }
 }
 
-template <int BM, int BN, int WM, int WN>
+template <int BM, int BN, int WM, int WN, int D, int BK>
 int LaunchIgemm(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
 {
     const ConvGeom& g = p->geom;
     IgemmArgs a;
     a.x = static_cast<const uint8_t*>(x);
+    a.pad16 = p->pad16;
     a.w = p->w_mfma;
     a.ct = ChanTab{p->chan, p->Co_pad};
     a.corr = p->corr;
@@ -439,7 +453,11 @@ int LaunchIgemm(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y
     a.rq = p->rq;
     const int nblocks = a.tiles_m * a.tiles_n;
     const int grid = (nblocks + 7) / 8 * 8;
-    hipLaunchKernelGGL((IgemmKernel<BM, BN, WM, WN>), dim3(grid), dim3(256), 0, stream, a);
+    constexpr int smem = IgemmSmemBytes<BM, BN, BK>();
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmKernel<BM, BN, WM, WN, D, BK>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    MI355X_HIP(attr);
+    hipLaunchKernelGGL((IgemmKernel<BM, BN, WM, WN, D, BK>), dim3(grid), dim3(256), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;
 }
@@ -472,9 +490,12 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         // (4x the blocks, 8 waves/SIMD).
         const long long M = static_cast<long long>(batch) * g.Ho * g.Wo;
         const long long big = ((M + 127) / 128) * ((g.Co + 127) / 128);
-        if (p->tile_override == 64 || (p->tile_override == 0 && big < 1024)) return LaunchIgemm<64, 64, 2, 2>(p, batch, x, y, stream);
-        if (g.Co <= 64) return LaunchIgemm<128, 64, 2, 2>(p, batch, x, y, stream);
-        return LaunchIgemm<128, 128, 2, 2>(p, batch, x, y, stream);
+        // tile: 64x64 while the 128-wide tiling would leave CUs idle; k-tile: 128 bytes whenever K was padded to it
+        const bool bk128 = p->bk128;
+        const int tile = p->tile_override ? p->tile_override : big < 400 ? 64 : 128;
+        if (tile == 64) return bk128 ? LaunchIgemm<64, 64, 2, 2, 2, 128>(p, batch, x, y, stream) : LaunchIgemm<64, 64, 2, 2, 2, 64>(p, batch, x, y, stream);
+        if (g.Co <= 64) return bk128 ? LaunchIgemm<128, 64, 2, 2, 2, 128>(p, batch, x, y, stream) : LaunchIgemm<128, 64, 2, 2, 2, 64>(p, batch, x, y, stream);
+        return bk128 ? LaunchIgemm<128, 128, 2, 2, 2, 128>(p, batch, x, y, stream) : LaunchIgemm<128, 128, 2, 2, 2, 64>(p, batch, x, y, stream);
     }
     case MI355X_ALGO_DOT4:
     {

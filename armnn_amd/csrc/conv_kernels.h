@@ -9,6 +9,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <type_traits>
+
 #include "common.h"
 #include "device_math.h"
 
@@ -156,6 +158,7 @@ __global__ __launch_bounds__(256) void DepthwiseC4Kernel(ConvGeom g, Requant rq,
 struct IgemmArgs
 {
     const uint8_t* x;
+    const uint8_t* pad16;   // 16 bytes of (padding value ^ input xor): what a chunk outside the image loads
     const int8_t*  w;       // [Co_pad][K_pad], zero padded
     ChanTab        ct;      // per-channel requantization constants, rows of Co_pad floats
     const int32_t* corr;    // [Co_pad]
@@ -171,26 +174,31 @@ struct IgemmArgs
     Requant rq;
 };
 
-constexpr int kIgemmBK  = 64;
-constexpr int kIgemmLDK = kIgemmBK + 16;   // LDS row stride in bytes: 80 keeps ds_read_b128 conflict-free
-
-template <int BM, int BN>
+// K is walked in tiles of BK bytes per GEMM row.  BK = 128 makes every row chunk a whole 128-byte cache line: with 64-byte
+// chunks half of each line fetched from L2 is thrown away, and the L2-to-CU path (not MFMA, not HBM) becomes the limit.
+// LDS rows are BK + 16 bytes apart (80 or 144), which keeps the ds_read_b128 fragment reads free of bank conflicts.
+template <int BM, int BN, int BK>
 constexpr int IgemmSmemBytes()
 {
-    constexpr int stage = (BM + BN) * kIgemmLDK;
+    constexpr int stage = (BM + BN) * (BK + 16);
     constexpr int out = BM * (BN + 16);
     return 2 * stage > out ? 2 * stage : out;
 }
 
-template <int BM, int BN, int WM, int WN>
+// D = register slots for k-tiles on their way from global memory to LDS: the loads of tile kt + D - 1 are issued while
+// tile kt is multiplied, so D - 1 tiles are in flight and an iteration no longer has to last a whole memory round trip.
+template <int BM, int BN, int WM, int WN, int D, int BK>
 __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
 {
     static_assert(WM * WN == 4, "4 waves per block");
+    static_assert(D >= 2 && D <= 4, "2 to 4 register slots");
     static_assert(BM % 64 == 0 && BN % 64 == 0, "tile sizes are multiples of 64");
-    constexpr int BK = kIgemmBK;
-    constexpr int LDK = kIgemmLDK;
-    constexpr int RA = BM / 64;                 // activation rows loaded per thread per k-tile
-    constexpr int RB = BN / 64;                 // weight rows loaded per thread per k-tile
+    static_assert(BK == 64 || BK == 128, "k-tiles of 64 or 128 bytes");
+    constexpr int LDK = BK + 16;
+    constexpr int CPR = BK / 16;                // 16-byte chunks per row of a k-tile
+    constexpr int RP = 256 / CPR;               // rows covered by one pass of the block's threads
+    constexpr int RA = BM / RP;                 // activation rows loaded per thread per k-tile
+    constexpr int RB = BN / RP;                 // weight rows loaded per thread per k-tile
     constexpr int WTM = BM / WM;                // wave tile (pixels)
     constexpr int WTN = BN / WN;                // wave tile (channels)
     constexpr int TP = WTM / 32;                // 32-pixel sub-tiles per wave
@@ -198,7 +206,7 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
     constexpr int STAGE = (BM + BN) * LDK;
     constexpr int LDO = BN + 16;
 
-    __shared__ __attribute__((aligned(16))) uint8_t smem[IgemmSmemBytes<BM, BN>()];
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];   // IgemmSmemBytes<BM, BN, BK>()
 
     // XCD-aware tile order: consecutive block ids land on different XCDs, so give each XCD a contiguous run
     // of tiles (tiles that share activation rows then share that XCD's L2).
@@ -216,8 +224,8 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
     const int wn = wave % WN;
 
     // ---- global -> LDS load assignment: 16-byte chunk `lc` of row `lr (+64 j)` -------------------------
-    const int lc = tid & 3;
-    const int lr = tid >> 2;
+    const int lc = tid % CPR;
+    const int lr = tid / CPR;
 
     const uint8_t* xrow[RA];
     int iy0[RA], ix0[RA];
@@ -225,7 +233,7 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
 #pragma unroll
     for (int j = 0; j < RA; ++j)
     {
-        const int m = tm * BM + lr + 64 * j;
+        const int m = tm * BM + lr + RP * j;
         mvalid[j] = m < a.M;
         const int mm = mvalid[j] ? m : 0;
         const int ox = mm % a.Wo;
@@ -247,12 +255,11 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
     }
     const int8_t* wrow = a.w + static_cast<long long>(tn * BN + lr) * a.K_pad + lc * 16;
 
-    v4i ra[RA], rb[RB];
-    const v4i padv = {static_cast<int>(a.pad_word), static_cast<int>(a.pad_word), static_cast<int>(a.pad_word),
-                      static_cast<int>(a.pad_word)};
+    v4i ra[D][RA], rb[D][RB];
     const int xm = static_cast<int>(a.xor_mask);
 
-    auto load_tile = [&](int kt) {
+    auto load_tile = [&](int kt, auto slot) {
+        constexpr int SL = decltype(slot)::value;
         const bool kvalid = ky < a.Kh;
 #pragma unroll
         for (int j = 0; j < RA; ++j)
@@ -261,20 +268,16 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
             const int ix = ix0[j] + kx * a.dil_x;
             const bool ok = mvalid[j] && kvalid && static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) &&
                             static_cast<unsigned>(ix) < static_cast<unsigned>(a.W);
-            if (ok)
-            {
-                v4i v = *reinterpret_cast<const v4i*>(xrow[j] + (static_cast<long long>(iy) * a.W + ix) * a.Ci + ci);
-                ra[j] = v ^ xm;
-            }
-            else
-            {
-                ra[j] = padv;
-            }
+            // A chunk outside the image loads 16 prepared padding bytes instead: every load is unconditional and its
+            // value is used as it is, so the compiler has no branch to put it in (a load inside a divergent branch is
+            // waited for on the spot, which would serialise the prefetch).
+            const uint8_t* src = ok ? xrow[j] + ((static_cast<long long>(iy) * a.W + ix) * a.Ci + ci) : a.pad16;
+            ra[SL][j] = *reinterpret_cast<const v4i*>(src);   // the xor waits until the value goes to LDS
         }
 #pragma unroll
         for (int j = 0; j < RB; ++j)
         {
-            rb[j] = *reinterpret_cast<const v4i*>(wrow + static_cast<long long>(64 * j) * a.K_pad + kt * BK);
+            rb[SL][j] = *reinterpret_cast<const v4i*>(wrow + static_cast<long long>(RP * j) * a.K_pad + kt * BK);
         }
         // advance (ky, kx, ci) by one k-tile
         ci += BK;
@@ -285,13 +288,14 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
         }
     };
 
-    auto store_tile = [&](int buf) {
+    auto store_tile = [&](int buf, auto slot) {
+        constexpr int SL = decltype(slot)::value;
         uint8_t* As = smem + buf * STAGE;
         uint8_t* Bs = As + BM * LDK;
 #pragma unroll
-        for (int j = 0; j < RA; ++j) *reinterpret_cast<v4i*>(As + (lr + 64 * j) * LDK + lc * 16) = ra[j];
+        for (int j = 0; j < RA; ++j) *reinterpret_cast<v4i*>(As + (lr + RP * j) * LDK + lc * 16) = ra[SL][j] ^ xm;
 #pragma unroll
-        for (int j = 0; j < RB; ++j) *reinterpret_cast<v4i*>(Bs + (lr + 64 * j) * LDK + lc * 16) = rb[j];
+        for (int j = 0; j < RB; ++j) *reinterpret_cast<v4i*>(Bs + (lr + RP * j) * LDK + lc * 16) = rb[SL][j];
     };
 
     // ---- accumulators, initialised with the zero-point correction -------------------------------------
@@ -318,18 +322,11 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
     }
 
     const int nk = a.K_pad / BK;
-    load_tile(0);
-    store_tile(0);
-    __syncthreads();
-
     const int frag_row = lane & 31;
     const int frag_k = (lane >> 5) * 16;
+    using std::integral_constant;
 
-    for (int kt = 0; kt < nk; ++kt)
-    {
-        const int buf = kt & 1;
-        if (kt + 1 < nk) load_tile(kt + 1);
-
+    auto compute = [&](int buf) {
         const uint8_t* As = smem + buf * STAGE;
         const uint8_t* Bs = As + BM * LDK;
 #pragma unroll
@@ -348,9 +345,30 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
                 for (int tp = 0; tp < TP; ++tp)
                     acc[tc][tp] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[tc], fa[tp], acc[tc][tp], 0, 0, 0);
         }
+    };
 
-        if (kt + 1 < nk) store_tile(buf ^ 1);
+    // prologue: tiles 0 .. D-2 go on their way, tile 0 lands in LDS
+    load_tile(0, integral_constant<int, 0>{});
+    if constexpr (D > 2) { if (1 < nk) load_tile(1, integral_constant<int, 1>{}); }
+    if constexpr (D > 3) { if (2 < nk) load_tile(2, integral_constant<int, 2>{}); }
+    store_tile(0, integral_constant<int, 0>{});
+    __syncthreads();
+
+    // iteration kt (kt % D == J): issue tile kt+D-1 into the slot tile kt-1 left, multiply tile kt, move tile kt+1
+    // from its slot to the other LDS buffer
+    auto step = [&](int kt, auto jc) {
+        constexpr int J = decltype(jc)::value;
+        if (kt + D - 1 < nk) load_tile(kt + D - 1, integral_constant<int, (J + D - 1) % D>{});
+        compute(kt & 1);
+        if (kt + 1 < nk) store_tile((kt + 1) & 1, integral_constant<int, (J + 1) % D>{});
         __syncthreads();
+    };
+    for (int kt = 0; kt < nk; kt += D)
+    {
+        step(kt, integral_constant<int, 0>{});
+        if (kt + 1 < nk) step(kt + 1, integral_constant<int, 1>{});
+        if constexpr (D > 2) { if (kt + 2 < nk) step(kt + 2, integral_constant<int, 2>{}); }
+        if constexpr (D > 3) { if (kt + 3 < nk) step(kt + 3, integral_constant<int, 3>{}); }
     }
 
     // ---- epilogue: requantize, pack 4 channels per dword, stage the byte tile in LDS ---------------------

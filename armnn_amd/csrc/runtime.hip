@@ -24,7 +24,15 @@ int SetError(int code, const char* fmt, ...)
 
 Options& GlobalOptions()
 {
-    static Options o;
+    static Options o = [] {
+        Options init;
+        if (const char* e = std::getenv("MI355X_IGEMM_DEPTH"))     // experiments
+        {
+            const int v = std::atoi(e);
+            if (v >= 2 && v <= 4) init.igemm_depth = v;
+        }
+        return init;
+    }();
     return o;
 }
 
@@ -97,6 +105,12 @@ int mi355x_set_option(const char* name, int value)
 {
     if (!name) return SetError(MI355X_ERR_INVALID_ARGUMENT, "option name is null");
     if (std::strcmp(name, "exact_division_epilogue") == 0) { GlobalOptions().exact_division_epilogue = value != 0; return 0; }
+    if (std::strcmp(name, "igemm_depth") == 0)
+    {
+        if (value < 2 || value > 4) return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_depth must be 2, 3 or 4");
+        GlobalOptions().igemm_depth = value;
+        return 0;
+    }
     return SetError(MI355X_ERR_INVALID_ARGUMENT, "unknown option '%s'", name);
 }
 
