@@ -3,6 +3,7 @@
 #include "common.h"
 #include "conv_kernels.h"
 #include "dw_stem_kernels.h"
+#include "dwpw_kernel.h"
 #include "pw_gemm_kernel.h"
 
 #include <cmath>
@@ -22,6 +23,7 @@ struct mi355x_conv2d_s
     uint8_t* w_direct = nullptr;   // [Kh][Kw][Ci][Co] / depthwise [Kh][Kw][Co], raw codes
     int8_t*  w_mfma   = nullptr;   // [Co_pad][K_pad] signed, zero padded
     uint8_t* pad16    = nullptr;   // 16 bytes that turn into the padding value under the kernel's input xor
+    uint32_t* dw_grp  = nullptr;   // depthwise 3x3: constants per group of 4 channels for the fused dw+pw kernel
     uint32_t* w_dot4  = nullptr;   // depthwise 3x3: [C][4] dwords; small-Ci conv: [Co][Kh][RD] dwords
     int variant = 0;               // kernel variant within an algo (see RunPlan)
     int row_dwords = 0;            // small-Ci conv: dwords per filter row
@@ -40,6 +42,7 @@ struct mi355x_conv2d_s
         (void)hipFree(w_direct);
         (void)hipFree(w_mfma);
         (void)hipFree(pad16);
+        (void)hipFree(dw_grp);
         (void)hipFree(w_dot4);
         (void)hipFree(chan);
         (void)hipFree(corr);
@@ -272,6 +275,21 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         const uint32_t zb = static_cast<uint32_t>(zx_shift) & 0xffu;
         p->pad_word = zb | (zb << 8) | (zb << 16) | (zb << 24);
         p->variant = 1;
+        {
+            // [C/4][8][4] dwords: weight rows 0..2, corr, fm, fb, thr (rows 2..4 of the channel table), 0
+            const int CP = p->Co_pad;
+            std::vector<uint32_t> grp(static_cast<size_t>(Co / 4) * 32, 0u);
+            for (int c = 0; c < Co; ++c)
+            {
+                uint32_t* gdst = grp.data() + static_cast<size_t>(c / 4) * 32 + (c % 4);
+                for (int r = 0; r < 3; ++r) gdst[r * 4] = wp[static_cast<size_t>(c) * 4 + r];
+                gdst[3 * 4] = static_cast<uint32_t>(corr[c]);
+                for (int r = 0; r < 3; ++r) std::memcpy(&gdst[(4 + r) * 4], &p->chan_host[static_cast<size_t>(2 + r) * CP + c], 4);
+            }
+            if (int rc = Upload(reinterpret_cast<void**>(&p->dw_grp), grp.data(), grp.size() * sizeof(uint32_t))) return rc;
+            const std::vector<uint8_t> padbytes(16, static_cast<uint8_t>((zb ^ (g.in_u8 ? 0x80u : 0u)) & 0xffu));
+            if (int rc = Upload(reinterpret_cast<void**>(&p->pad16), padbytes.data(), padbytes.size())) return rc;
+        }
         p->info = d.stride_x == 1 ? "depthwise3x3_dot4_lds stride 1, tile 8x16x32" : "depthwise3x3_dot4_lds stride 2, tile 8x8x32";
     }
     else if (algo == MI355X_ALGO_DEPTHWISE)
@@ -494,7 +512,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const bool bk128 = p->bk128;
         const int tile = p->tile_override ? p->tile_override : big < 400 ? 64 : 128;
         if (tile == 64) return bk128 ? LaunchIgemm<64, 64, 2, 2, 2, 128>(p, batch, x, y, stream) : LaunchIgemm<64, 64, 2, 2, 2, 64>(p, batch, x, y, stream);
-        if (g.Co <= 64) return bk128 ? LaunchIgemm<128, 64, 2, 2, 2, 128>(p, batch, x, y, stream) : LaunchIgemm<128, 64, 2, 2, 2, 64>(p, batch, x, y, stream);
+        if (g.Co <= 64 || tile == 96) return bk128 ? LaunchIgemm<128, 64, 2, 2, 2, 128>(p, batch, x, y, stream) : LaunchIgemm<128, 64, 2, 2, 2, 64>(p, batch, x, y, stream);
         return bk128 ? LaunchIgemm<128, 128, 2, 2, 2, 128>(p, batch, x, y, stream) : LaunchIgemm<128, 128, 2, 2, 2, 64>(p, batch, x, y, stream);
     }
     case MI355X_ALGO_DOT4:
@@ -576,6 +594,34 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
 
 } // namespace
 
+namespace
+{
+template <int S, int P>
+int LaunchDwPw(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    using G = DwPwGeom<S, P>;
+    constexpr int D = 4;
+    const ConvGeom& g = dw->geom;
+    DwPwArgs a;
+    a.x = static_cast<const uint8_t*>(x); a.pad16 = dw->pad16; a.dw_grp = dw->dw_grp; a.dw_ct = ChanTab{dw->chan, dw->Co_pad};
+    a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.C = g.Co; a.Ho = g.Ho; a.Wo = g.Wo;
+    a.pad_top = g.pad_top; a.pad_left = g.pad_left;
+    a.tiles_x = (g.Wo + G::TW - 1) / G::TW; a.tiles_y = (g.Ho + G::TH - 1) / G::TH;
+    const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
+    if (nb > 0x7fffffffll - 8) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
+    a.total_blocks = static_cast<int>(nb); a.xcd_chunk = static_cast<int>((nb + 7) / 8);
+    a.dw_xor = dw->xor_mask; a.dw_rq = dw->rq;
+    a.pw_w = pw->w_mfma; a.pw_wstride = pw->K_pad; a.pw_ct = ChanTab{pw->chan, pw->Co_pad}; a.pw_corr = pw->corr;
+    a.y = static_cast<uint8_t*>(y); a.Co = pw->geom.Co; a.mid_xor = pw->xor_mask; a.pw_rq = pw->rq;
+    const int smem = DwPwSmemBytes<S, P>(g.Co);
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&DwPwKernel<S, P, D>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    MI355X_HIP(attr);
+    hipLaunchKernelGGL((DwPwKernel<S, P, D>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(256), smem, stream, a);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+} // namespace
+
 extern "C" {
 
 int mi355x_conv2d_create(const mi355x_conv2d_desc* desc, const void* weights_host, const mi355x_const_quant* weights_quant,
@@ -593,6 +639,42 @@ int mi355x_conv2d_create(const mi355x_conv2d_desc* desc, const void* weights_hos
 int mi355x_conv2d_run(mi355x_conv2d_t plan, uint32_t batch, const void* input_dev, void* output_dev, mi355x_stream_t stream)
 {
     return RunPlan(plan, batch, input_dev, output_dev, ToHip(stream));
+}
+
+int mi355x_conv2d_fusable(mi355x_conv2d_t dw, mi355x_conv2d_t pw)
+{
+    if (!dw || !pw) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
+    const mi355x_conv2d_desc& a = dw->d;
+    const mi355x_conv2d_desc& b = pw->d;
+    if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || !dw->dw_grp)
+        return SetError(MI355X_ERR_UNSUPPORTED, "first plan is not a 3x3 depthwise layer on the v_dot4 kernel");
+    const bool pointwise = pw->algo == MI355X_ALGO_MFMA && !b.depthwise && b.kernel_h == 1 && b.kernel_w == 1 && b.stride_x == 1 &&
+                           b.stride_y == 1 && b.pad_top == 0 && b.pad_left == 0 && b.out_h == b.in_h && b.out_w == b.in_w;
+    if (!pointwise) return SetError(MI355X_ERR_UNSUPPORTED, "second plan is not an unpadded 1x1 stride-1 convolution on the MFMA kernel");
+    if (a.out_c != b.in_c || a.out_h != b.in_h || a.out_w != b.in_w) return SetError(MI355X_ERR_INVALID_ARGUMENT, "the layers' shapes do not chain");
+    if (a.output.dtype != b.input.dtype || a.output.scale != b.input.scale || a.output.offset != b.input.offset)
+        return SetError(MI355X_ERR_INVALID_ARGUMENT, "the first layer's output quantization is not the second layer's input quantization");
+    if ((b.out_c % 64) != 0) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel needs output channels %% 64 == 0");
+    const int smem = a.stride_x == 1 ? DwPwSmemBytes<1, 2>(static_cast<int>(a.out_c)) : DwPwSmemBytes<2, 2>(static_cast<int>(a.out_c));
+    if (smem > 160 * 1024) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel: %d channels need %d bytes of LDS", a.out_c, smem);
+    if (static_cast<long long>(a.in_h) * a.in_w * a.in_c >= (1ll << 31)) return SetError(MI355X_ERR_UNSUPPORTED, "image too large for 32-bit offsets");
+    return 0;
+}
+
+int mi355x_conv2d_run_fused(mi355x_conv2d_t dw, mi355x_conv2d_t pw, uint32_t batch, const void* input_dev, void* output_dev,
+                            mi355x_stream_t stream)
+{
+    if (int rc = mi355x_conv2d_fusable(dw, pw)) return rc;
+    if (batch == 0) return 0;
+    if (!input_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "input / output pointer is null");
+    if ((reinterpret_cast<uintptr_t>(input_dev) & 15) != 0 || (reinterpret_cast<uintptr_t>(output_dev) & 15) != 0)
+        return SetError(MI355X_ERR_INVALID_ARGUMENT, "fused kernel needs 16-byte aligned tensors");
+    if (dw->d.stride_x == 2) return LaunchDwPw<2, 2>(dw, pw, batch, input_dev, output_dev, ToHip(stream));
+    // stride 1: the wide tile (8 x 16 pixels) while it still yields two blocks per CU, else the narrow one (8 x 8)
+    const long long wide = static_cast<long long>(batch) * ((dw->d.out_w + 15) / 16) * ((dw->d.out_h + 7) / 8);
+    if (wide >= 512 && DwPwSmemBytes<1, 4>(static_cast<int>(dw->d.out_c)) <= 160 * 1024)
+        return LaunchDwPw<1, 4>(dw, pw, batch, input_dev, output_dev, ToHip(stream));
+    return LaunchDwPw<1, 2>(dw, pw, batch, input_dev, output_dev, ToHip(stream));
 }
 
 int mi355x_conv2d_destroy(mi355x_conv2d_t plan)

@@ -3,7 +3,8 @@ the whole forward pass optionally captured into a HIP graph and replayed with on
 from __future__ import annotations
 
 import ctypes as C
-from typing import Dict, List, Optional
+from dataclasses import dataclass
+from typing import Dict, List, Optional, Tuple
 
 import numpy as np
 
@@ -12,14 +13,36 @@ from .nets import Network
 from .tensor import QTensor, numpy_dtype
 
 
+@dataclass
+class FusedPair:
+    """A depthwise layer and the pointwise convolution consuming it, launched as one kernel."""
+    name: str
+    parts: Tuple                       # (depthwise Layer, pointwise Layer)
+    op: str = "dwpw"
+
+    @property
+    def inputs(self):
+        return self.parts[0].inputs
+
+    @property
+    def output(self):
+        return self.parts[1].output
+
+    @property
+    def macs_per_image(self):
+        return self.parts[0].macs_per_image + self.parts[1].macs_per_image
+
+
 class DeviceNetwork:
-    def __init__(self, net: Network, batch: int, algo_overrides: Optional[Dict[str, int]] = None, use_graph: bool = True):
+    def __init__(self, net: Network, batch: int, algo_overrides: Optional[Dict[str, int]] = None, use_graph: bool = True,
+                 fuse: bool = False):
         self.net, self.batch = net, batch
         self.dev = shim.Device()
         self.lib = shim.load_library()
         self.stream = self.dev.stream()
         self.buffers: Dict[str, shim.DeviceBuffer] = {}
         self.steps: List = []          # (layer, callable(stream))
+        self._step_plans: List = []    # plan of each step (None for plan-less layers), parallel to self.steps
         self.plans = []
         self.graph = None
         self.use_graph = use_graph
@@ -45,12 +68,14 @@ class DeviceNetwork:
                                        act_b=l.act[2], algo=algo_overrides.get(l.name, shim.ALGO_AUTO), **p)
                 self.plans.append(plan)
                 self.steps.append((l, self._conv_step(plan, xb[0].ptr, yb.ptr)))
+                self._step_plans.append(plan)
             elif l.op == "fc":
                 plan = shim.FullyConnectedPlan(xin[0], l.weights, l.bias, yout, transpose_weights=l.params["transpose_weights"],
                                                activation=l.act[0], act_a=l.act[1], act_b=l.act[2],
                                                algo=algo_overrides.get(l.name, shim.ALGO_AUTO))
                 self.plans.append(plan)
                 self.steps.append((l, self._conv_step(plan, xb[0].ptr, yb.ptr)))
+                self._step_plans.append(plan)
             elif l.op == "pool":
                 _, h, w, c = xin[0].shape
                 _, ho, wo, _ = yout.shape
@@ -59,15 +84,47 @@ class DeviceNetwork:
                                     p["pad_right"], p["pad_top"], p["pad_bottom"], p["pool_type"], p["padding_method"],
                                     shim._quant(xin[0]), shim._quant(yout))
                 self.steps.append((l, self._pool_step(d, xb[0].ptr, yb.ptr)))
+                self._step_plans.append(None)
             elif l.op == "add":
                 q0, q1, qo = shim._quant(xin[0]), shim._quant(xin[1]), shim._quant(yout)
                 self.steps.append((l, self._add_step(yout.num_elements, q0, q1, qo, l.act, xb[0].ptr, xb[1].ptr, yb.ptr)))
+                self._step_plans.append(None)
             elif l.op == "softmax":
                 rows, cols = yout.shape
                 qi, qo = shim._quant(xin[0]), shim._quant(yout)
                 self.steps.append((l, self._softmax_step(rows, cols, l.params["beta"], qi, qo, xb[0].ptr, yb.ptr)))
+                self._step_plans.append(None)
             else:
                 raise ValueError(l.op)
+        if fuse:
+            self._fuse_depthwise_pointwise()
+
+    def _fuse_depthwise_pointwise(self):
+        """Replace (depthwise 3x3, 1x1 convolution) neighbours by one fused launch where the library accepts the pair
+        and nothing else reads the tensor between them."""
+        net = self.net
+        consumers: Dict[str, int] = {}
+        for l in net.layers:
+            for i in l.inputs:
+                consumers[i] = consumers.get(i, 0) + 1
+        plan_of = {id(l): pl for (l, _), pl in zip(self.steps, self._step_plans)}
+        fused, k = [], 0
+        while k < len(self.steps):
+            l, fn = self.steps[k]
+            nxt = self.steps[k + 1][0] if k + 1 < len(self.steps) else None
+            if (l.op == "depthwise" and nxt is not None and nxt.op == "conv" and nxt.inputs[0] == l.output and
+                    consumers.get(l.output, 0) == 1 and l.output != net.output and
+                    plan_of[id(l)].fusable_with(plan_of[id(nxt)])):
+                pdw, ppw = plan_of[id(l)], plan_of[id(nxt)]
+                x, y = self.buffers[l.inputs[0]].ptr, self.buffers[nxt.output].ptr
+                batch = self.batch
+                fused.append((FusedPair(f"{l.name}+{nxt.name}", (l, nxt)),
+                              (lambda pdw, ppw, x, y: lambda s: pdw.run_fused(ppw, batch, x, y, s))(pdw, ppw, x, y)))
+                k += 2
+            else:
+                fused.append((l, fn))
+                k += 1
+        self.steps = fused
 
     # each step keeps its ctypes structs alive through the closure
     def _conv_step(self, plan, x, y):

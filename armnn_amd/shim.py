@@ -28,6 +28,7 @@ EXPORTS = [
     "mi355x_event_destroy", "mi355x_event_record", "mi355x_event_synchronize", "mi355x_event_elapsed_ms",
     "mi355x_graph_capture_begin", "mi355x_graph_capture_end", "mi355x_graph_launch", "mi355x_graph_destroy",
     "mi355x_conv2d_create", "mi355x_conv2d_run", "mi355x_conv2d_destroy", "mi355x_conv2d_algo",
+    "mi355x_conv2d_fusable", "mi355x_conv2d_run_fused",
     "mi355x_fc_create", "mi355x_fc_run", "mi355x_fc_destroy", "mi355x_fc_algo",
     "mi355x_activation_run", "mi355x_pool2d_run", "mi355x_add_run", "mi355x_softmax_run",
 ]
@@ -101,6 +102,7 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
             "mi355x_conv2d_create": [C.POINTER(Conv2dDesc), V, C.POINTER(ConstQuant), V, C.POINTER(ConstQuant), C.POINTER(V)],
             "mi355x_conv2d_run": [V, C.c_uint32, V, V, V], "mi355x_conv2d_destroy": [V],
             "mi355x_conv2d_algo": [V, C.POINTER(C.c_int32), C.c_char_p, C.c_size_t],
+            "mi355x_conv2d_fusable": [V, V], "mi355x_conv2d_run_fused": [V, V, C.c_uint32, V, V, V],
             "mi355x_fc_create": [C.POINTER(FcDesc), V, C.POINTER(ConstQuant), V, C.POINTER(ConstQuant), C.POINTER(V)],
             "mi355x_fc_run": [V, C.c_uint32, V, V, V], "mi355x_fc_destroy": [V],
             "mi355x_fc_algo": [V, C.POINTER(C.c_int32), C.c_char_p, C.c_size_t],
@@ -276,6 +278,14 @@ class Conv2dPlan:
 
     def run(self, batch: int, x_dev: int, y_dev: int, stream=None):
         _chk(self.lib.mi355x_conv2d_run(self.plan, batch, x_dev, y_dev, stream))
+
+    def fusable_with(self, pointwise: "Conv2dPlan") -> bool:
+        """True when this 3x3 depthwise plan and `pointwise` (the 1x1 convolution consuming it) can run as one kernel."""
+        return self.lib.mi355x_conv2d_fusable(self.plan, pointwise.plan) == 0
+
+    def run_fused(self, pointwise: "Conv2dPlan", batch: int, x_dev: int, y_dev: int, stream=None):
+        """depthwise -> pointwise without the intermediate tensor; bytes equal run() + pointwise.run()."""
+        _chk(self.lib.mi355x_conv2d_run_fused(self.plan, pointwise.plan, batch, x_dev, y_dev, stream))
 
     def destroy(self):
         if self.plan:

@@ -32,6 +32,14 @@ def layer_work(net, l, batch):
     """(kind, algorithmic work per launch): conv/fc -> ops = 2*MACs; others -> bytes, each tensor once."""
     if l.op in ("conv", "fc"):
         return "mfma", 2.0 * l.macs_per_image * batch
+    if l.op == "dwpw":
+        # fused depthwise + pointwise: the tensor between them never exists, so the unit's algorithmic bytes are its
+        # input, its output and both layers' constants; priced against HBM like the depthwise layer it absorbs
+        dw, pw = l.parts
+        nbytes = (net.tensors[dw.inputs[0]].num_elements + net.tensors[pw.output].num_elements) * batch
+        for part in (dw, pw):
+            nbytes += part.weights.info.num_elements + 8 * net.tensors[part.output].shape[-1]
+        return "hbm", float(nbytes)
     nbytes = sum(net.tensors[i].num_elements for i in l.inputs) + net.tensors[l.output].num_elements
     nbytes *= batch
     if l.weights is not None:
@@ -70,6 +78,8 @@ def main():
     ap.add_argument("--net", default="mobilenet_v1", choices=["mobilenet_v1", "resnet50"])
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--fuse", action="store_true",
+                    help="run depthwise + pointwise pairs as one kernel (same bytes; slower than two launches at present)")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -82,7 +92,7 @@ def main():
 
     net = nets.mobilenet_v1() if args.net == "mobilenet_v1" else nets.resnet50()
     batch = args.batch
-    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph)
+    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev
 
@@ -128,7 +138,7 @@ def main():
         return {"ms": t * 1e3, "achieved": w / t, "frac": w / t / peak} if t > 0 else None
 
     g_conv = group(("conv", "fc"), INT8_MFMA_PEAK_OPS)
-    g_dw = group(("depthwise",), HBM_PEAK_BYTES)
+    g_dw = group(("depthwise", "dwpw"), HBM_PEAK_BYTES)
     groups = {
         "conv_fc": {"ms": g_conv["ms"], "TOPS": g_conv["achieved"] / 1e12, "frac_of_int8_mfma_peak": g_conv["frac"]},
     }
@@ -142,7 +152,7 @@ def main():
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"{net.name} int8 (QAsymm activations, per-channel QSymmS8 weights), batch {batch}, "
                                f"random-init, whole forward pass incl. avgpool/FC/softmax, input resident in HBM",
-                   "batch": batch, "graph_replay": not args.no_graph,
+                   "batch": batch, "graph_replay": not args.no_graph, "fused_depthwise_pointwise": args.fuse,
                    "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12},
         "roofline": roof, "groups": groups,
     }

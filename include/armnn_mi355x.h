@@ -169,6 +169,17 @@ int mi355x_conv2d_create(const mi355x_conv2d_desc* desc,
 int mi355x_conv2d_run(mi355x_conv2d_t plan, uint32_t batch, const void* input_dev, void* output_dev,
                       mi355x_stream_t stream);
 int mi355x_conv2d_destroy(mi355x_conv2d_t plan);
+/* A 3x3 depthwise plan and the plan of the unpadded 1x1 stride-1 Convolution2d that consumes its output, run as one
+ * kernel: the depthwise result is requantized to its own int8 codes in on-chip memory and fed to the pointwise GEMM
+ * there, so the intermediate tensor is never written.  The bytes produced equal mi355x_conv2d_run(depthwise) followed
+ * by mi355x_conv2d_run(pointwise) -- in the reference these are two workloads in sequence
+ * (RefDepthwiseConvolution2dWorkload.cpp:38-62, then RefConvolution2dWorkload.cpp:38-58).
+ * mi355x_conv2d_fusable returns 0 when the pair qualifies (3x3 depthwise with channels % 32 == 0, multiplier 1,
+ * stride 1 or 2; pointwise with output channels % 64 == 0; chaining shapes and identical quantization of the shared
+ * tensor), else MI355X_ERR_UNSUPPORTED / MI355X_ERR_INVALID_ARGUMENT with the reason in mi355x_last_error(). */
+int mi355x_conv2d_fusable(mi355x_conv2d_t depthwise, mi355x_conv2d_t pointwise);
+int mi355x_conv2d_run_fused(mi355x_conv2d_t depthwise, mi355x_conv2d_t pointwise, uint32_t batch,
+                            const void* input_dev, void* output_dev, mi355x_stream_t stream);
 /* which kernel a plan resolved to (mi355x_algo) and its tile configuration, for logs and tests */
 int mi355x_conv2d_algo(mi355x_conv2d_t plan, int32_t* algo, char* desc_buf, size_t desc_len);
 

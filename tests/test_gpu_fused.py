@@ -1,0 +1,98 @@
+"""Depthwise 3x3 + pointwise 1x1 as one kernel: bytes must equal the two layers run one after the other, and the pair
+must stay within 1 LSB of the oracle per layer (the second layer judged on the first layer's actual output)."""
+import numpy as np
+import pytest
+
+from armnn_amd import shim
+from armnn_amd.tensor import DataType, QTensor, numpy_dtype
+from tests import cases
+from tests.helpers import lsb_diff
+
+pytestmark = pytest.mark.gpu
+
+S8, U8 = DataType.QAsymmS8, DataType.QAsymmU8
+
+# (name, n, h, w, c, co, stride, dtype, act after dw, act after pw)
+PAIRS = [
+    ("s1_c32_co64_u8", 2, 37, 45, 32, 64, 1, U8, cases.RELU6, cases.RELU6),
+    ("s2_c64_co128_s8", 3, 41, 30, 64, 128, 2, S8, cases.RELU6, cases.RELU6),
+    ("s1_c128_co128_s8", 1, 19, 23, 128, 128, 1, S8, cases.RELU6, (0, 0.0, 0.0)),
+    ("s2_c128_co256_u8", 2, 28, 28, 128, 256, 2, U8, cases.RELU, cases.RELU6),
+    ("s1_c256_co256_s8", 2, 14, 14, 256, 256, 1, S8, (0, 0.0, 0.0), cases.RELU6),
+    ("s1_c512_co512_s8", 2, 14, 14, 512, 512, 1, S8, cases.RELU6, cases.RELU6),
+    ("s1_c96_co192_s8_tiny", 1, 5, 3, 96, 192, 1, S8, cases.RELU6, cases.RELU6),
+]
+
+
+def _make(name, n, h, w, c, co, stride, dt, act_dw, act_pw):
+    zp_in = 120 if dt == U8 else -8
+    zp_mid = 0 if dt == U8 else -128
+    dw = cases.make_conv_case(name + "_dw", 900 + c, n=n, h=h, w=w, ci=c, depthwise=True, stride=(stride, stride), in_dtype=dt,
+                              in_scale=0.0235, in_offset=zp_in, out_scale=0.0235, out_offset=zp_mid, act=act_dw,
+                              w_scale_range=(0.01, 0.05))
+    ho, wo = dw.out_info.shape[1], dw.out_info.shape[2]
+    pw = cases.make_conv_case(name + "_pw", 901 + co, n=n, h=ho, w=wo, ci=c, co=co, kh=1, kw=1, in_dtype=dt, in_scale=0.0235,
+                              in_offset=zp_mid, out_scale=0.03, out_offset=zp_mid + 5, act=act_pw)
+    return dw, pw
+
+
+def _plan(c):
+    fn, a, b = c.act
+    return shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, activation=fn, act_a=a, act_b=b, **c.params)
+
+
+@pytest.mark.parametrize("pair", PAIRS, ids=[p[0] for p in PAIRS])
+def test_fused_equals_two_layers(port, pair):
+    print("pair", pair, flush=True)
+    shim.Device()
+    dw, pw = _make(*pair)
+    pdw, ppw = _plan(dw), _plan(pw)
+    assert pdw.fusable_with(ppw), shim.load_library().mi355x_last_error().decode()
+    n = dw.x.info.shape[0]
+    xd = shim.DeviceBuffer(dw.x.data.nbytes).upload(dw.x.data)
+    mid = shim.DeviceBuffer(dw.out_info.num_elements)
+    y2 = shim.DeviceBuffer(pw.out_info.num_elements)
+    yf = shim.DeviceBuffer(pw.out_info.num_elements)
+    pdw.run(n, xd.ptr, mid.ptr)
+    ppw.run(n, mid.ptr, y2.ptr)
+    pdw.run_fused(ppw, n, xd.ptr, yf.ptr)
+    mid_h = mid.download(dw.out_info.shape, numpy_dtype(dw.out_info.dtype))
+    two = y2.download(pw.out_info.shape, numpy_dtype(pw.out_info.dtype))
+    fused = yf.download(pw.out_info.shape, numpy_dtype(pw.out_info.dtype))
+    np.testing.assert_array_equal(fused, two)
+    assert len(np.unique(fused)) > 8
+    # and the two layers themselves against the oracle
+    fn, a, b = dw.act
+    want_mid = port.activation(port.conv2d(dw.x, dw.w, dw.b, dw.out_info, **dw.params), dw.out_info, fn, a, b) if fn else \
+        port.conv2d(dw.x, dw.w, dw.b, dw.out_info, **dw.params)
+    mx, exact = lsb_diff(mid_h, want_mid.data)
+    assert mx <= 1 and exact >= 0.99
+    pw.x = QTensor(pw.x.info, mid_h)
+    fn, a, b = pw.act
+    want = port.conv2d(pw.x, pw.w, pw.b, pw.out_info, **pw.params)
+    if fn:
+        want = port.activation(want, pw.out_info, fn, a, b)
+    mx, exact = lsb_diff(fused, want.data)
+    print(f"  fused vs oracle on the device's intermediate: max|d|={mx} exact={exact:.5f}", flush=True)
+    assert mx <= 1 and exact >= 0.99
+
+
+def test_unfusable_pairs_are_refused():
+    shim.Device()
+    dw, pw = _make("x", 1, 9, 9, 32, 64, 1, S8, cases.RELU6, cases.RELU6)
+    pdw, ppw = _plan(dw), _plan(pw)
+    assert pdw.fusable_with(ppw)
+    assert not ppw.fusable_with(pdw)                      # wrong order
+    # the shared tensor's quantization differs
+    pw2 = cases.make_conv_case("x_pw2", 5, n=1, h=9, w=9, ci=32, co=64, kh=1, kw=1, in_scale=0.05, in_offset=-128)
+    assert not pdw.fusable_with(_plan(pw2))
+    # channel counts do not chain
+    pw3 = cases.make_conv_case("x_pw3", 6, n=1, h=9, w=9, ci=64, co=64, kh=1, kw=1, in_scale=0.0235, in_offset=-128)
+    assert not pdw.fusable_with(_plan(pw3))
+    # 3x3 consumer is not pointwise
+    c3 = cases.make_conv_case("x_c3", 7, n=1, h=9, w=9, ci=32, co=64, in_scale=0.0235, in_offset=-128)
+    assert not pdw.fusable_with(_plan(c3))
+    with pytest.raises(shim.ShimError):
+        xd = shim.DeviceBuffer(dw.x.data.nbytes).upload(dw.x.data)
+        yd = shim.DeviceBuffer(c3.out_info.num_elements)
+        pdw.run_fused(_plan(c3), 1, xd.ptr, yd.ptr)

@@ -16,7 +16,7 @@ def _layerwise(port, net, batch):
     independently of drift upstream.  Returns the end-to-end device output as well."""
     x = nets.synthetic_input(net, batch)
     ref = netref.run_network(port, net, x, keep=True)
-    dn = DeviceNetwork(net, batch, use_graph=False)
+    dn = DeviceNetwork(net, batch, use_graph=False, fuse=False)
     worst = 0
     for l, fn in dn.steps:
         for name in l.inputs:
@@ -32,7 +32,14 @@ def _layerwise(port, net, batch):
     # end to end (drift allowed to accumulate): graph replay must equal eager launches bit for bit
     eager = dn.run(x)
     dn.close()
-    dg = DeviceNetwork(net, batch, use_graph=True)
+    # depthwise + pointwise pairs as one kernel: same bytes, fewer launches
+    df = DeviceNetwork(net, batch, use_graph=False, fuse=True)
+    n_fused = sum(1 for l, _ in df.steps if l.op == "dwpw")
+    fused = df.run(x)
+    df.close()
+    print(f"{net.name} b{batch}: {n_fused} fused depthwise+pointwise pairs", flush=True)
+    np.testing.assert_array_equal(fused.data, eager.data)
+    dg = DeviceNetwork(net, batch, use_graph=True, fuse=False)
     g1 = dg.run(x)
     dg.enqueue()
     g2 = dg.download()
