@@ -98,13 +98,43 @@ __global__ __launch_bounds__(256) void Pool2dKernel(PoolArgs p, QIn qin, Requant
         if (clamped && p.exclude) area = static_cast<float>((hend - hstart) * (wend - wstart));
         result = p.is_max ? -FLT_MAX : 0.0f;
         const uint8_t* xn = x + n * p.H * p.W * p.C + c;
-        for (int iy = hstart; iy < hend; ++iy)
-            for (int ix = wstart; ix < wend; ++ix)
-            {
-                const float v = DequantDev(xn[(static_cast<long long>(iy) * p.W + ix) * p.C], qin);
-                if (p.is_max) { if (v > result) result = v; }
-                else result = __fadd_rn(result, v);
-            }
+        if (hend - hstart <= 8 && wend - wstart <= 8)
+        {
+            // up to 8 x 8 taps: all loads are issued before the first one is used (an element outside the window reads
+            // the window's first element and is ignored), then accumulated in the reference's row-major order
+            uint8_t raw[64];
+            const long long first = (static_cast<long long>(hstart) * p.W + wstart) * p.C;
+#pragma unroll
+            for (int dy = 0; dy < 8; ++dy)
+#pragma unroll
+                for (int dx = 0; dx < 8; ++dx)
+                {
+                    const bool in = hstart + dy < hend && wstart + dx < wend;
+                    raw[dy * 8 + dx] = xn[in ? (static_cast<long long>(hstart + dy) * p.W + wstart + dx) * p.C : first];
+                }
+#pragma unroll
+            for (int dy = 0; dy < 8; ++dy)
+#pragma unroll
+                for (int dx = 0; dx < 8; ++dx)
+                {
+                    if (hstart + dy < hend && wstart + dx < wend)
+                    {
+                        const float v = DequantDev(raw[dy * 8 + dx], qin);
+                        if (p.is_max) { if (v > result) result = v; }
+                        else result = __fadd_rn(result, v);
+                    }
+                }
+        }
+        else
+        {
+            for (int iy = hstart; iy < hend; ++iy)
+                for (int ix = wstart; ix < wend; ++ix)
+                {
+                    const float v = DequantDev(xn[(static_cast<long long>(iy) * p.W + ix) * p.C], qin);
+                    if (p.is_max) { if (v > result) result = v; }
+                    else result = __fadd_rn(result, v);
+                }
+        }
         if (!p.is_max) result = __fdiv_rn(result, area);
     }
     y[idx] = static_cast<uint8_t>(QuantizeFastDev(result, rq));
@@ -143,6 +173,46 @@ __global__ __launch_bounds__(64) void SoftmaxKernel(int cols, float beta, QIn qi
         const float e = expf(__fmul_rn(__fsub_rn(DequantDev(xr[i], qin), mx), beta));
         yr[i] = static_cast<uint8_t>(QuantizeDev(__fdiv_rn(e, sum), rq));
     }
+}
+
+// One block per row, the row held in registers (cols <= 256 * V): one pass over memory, one exp per element.
+template <int V>
+__global__ __launch_bounds__(256) void SoftmaxRowKernel(int cols, float beta, QIn qin, Requant rq,
+                                                         const uint8_t* __restrict__ x, uint8_t* __restrict__ y)
+{
+    __shared__ float red[8];
+    const uint8_t* xr = x + static_cast<long long>(blockIdx.x) * cols;
+    uint8_t* yr = y + static_cast<long long>(blockIdx.x) * cols;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    uint8_t raw[V];
+#pragma unroll
+    for (int k = 0; k < V; ++k) raw[k] = xr[min(tid + 256 * k, cols - 1)];
+    float v[V];
+    float mx = -FLT_MAX;
+#pragma unroll
+    for (int k = 0; k < V; ++k)
+    {
+        v[k] = DequantDev(raw[k], qin);
+        if (tid + 256 * k < cols) mx = fmaxf(mx, v[k]);
+    }
+    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
+    if (lane == 0) red[wave] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    float sum = 0.0f;
+#pragma unroll
+    for (int k = 0; k < V; ++k)
+    {
+        v[k] = tid + 256 * k < cols ? expf(__fmul_rn(__fsub_rn(v[k], mx), beta)) : 0.0f;
+        sum += v[k];
+    }
+    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
+    if (lane == 0) red[4 + wave] = sum;
+    __syncthreads();
+    sum = (red[4] + red[5]) + (red[6] + red[7]);
+#pragma unroll
+    for (int k = 0; k < V; ++k)
+        if (tid + 256 * k < cols) yr[tid + 256 * k] = static_cast<uint8_t>(QuantizeDev(__fdiv_rn(v[k], sum), rq));
 }
 
 int CheckQ(const mi355x_quant* q, const char* what)
@@ -230,8 +300,14 @@ int mi355x_softmax_run(uint32_t rows, uint32_t cols, float beta, const mi355x_qu
     if (rows == 0 || cols == 0) return 0;
     if (!input_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "null tensor pointer");
     Requant rq = MakeRequant(*out_q, MI355X_ACT_NONE, 0.0f, 0.0f);
-    hipLaunchKernelGGL(SoftmaxKernel, dim3(rows), dim3(64), 0, ToHip(stream), static_cast<int>(cols), beta, MakeQIn(*in_q), rq,
-                       static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev));
+    const uint8_t* xin = static_cast<const uint8_t*>(input_dev);
+    uint8_t* yout = static_cast<uint8_t*>(output_dev);
+    if (cols <= 1024)
+        hipLaunchKernelGGL(SoftmaxRowKernel<4>, dim3(rows), dim3(256), 0, ToHip(stream), static_cast<int>(cols), beta, MakeQIn(*in_q), rq, xin, yout);
+    else if (cols <= 2048)
+        hipLaunchKernelGGL(SoftmaxRowKernel<8>, dim3(rows), dim3(256), 0, ToHip(stream), static_cast<int>(cols), beta, MakeQIn(*in_q), rq, xin, yout);
+    else
+        hipLaunchKernelGGL(SoftmaxKernel, dim3(rows), dim3(64), 0, ToHip(stream), static_cast<int>(cols), beta, MakeQIn(*in_q), rq, xin, yout);
     MI355X_HIP(hipGetLastError());
     return 0;
 }
