@@ -495,6 +495,27 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || ((g.Co & 15) == 0 && (reinterpret_cast<uintptr_t>(y) & 15) != 0))
             return SetError(MI355X_ERR_INVALID_ARGUMENT, "MFMA kernel needs 16-byte aligned tensors");
     {
+        const mi355x_conv2d_desc& dd = p->d;
+        const long long rows = static_cast<long long>(batch) * g.Ho * g.Wo;
+        const bool unit = dd.kernel_h == 1 && dd.kernel_w == 1 && dd.stride_x == 1 && dd.stride_y == 1 && dd.pad_top == 0 &&
+                          dd.pad_left == 0 && dd.out_h == dd.in_h && dd.out_w == dd.in_w;
+        if (unit && rows <= 4 && (g.Ci % 16) == 0 && p->tile_override == 0)
+        {
+            // a handful of rows: stream the weights once, no tiles
+            GemvArgs a;
+            a.x = xin; a.w = p->w_mfma; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
+            a.M = static_cast<int>(rows); a.K = g.Ci; a.N = g.Co; a.w_stride = p->K_pad; a.xor_mask = p->xor_mask; a.rq = p->rq;
+            const dim3 grid(static_cast<unsigned>((g.Co + 15) / 16));
+            switch (a.M)
+            {
+                case 1: hipLaunchKernelGGL(GemvKernel<1>, grid, dim3(256), 0, stream, a); break;
+                case 2: hipLaunchKernelGGL(GemvKernel<2>, grid, dim3(256), 0, stream, a); break;
+                case 3: hipLaunchKernelGGL(GemvKernel<3>, grid, dim3(256), 0, stream, a); break;
+                default: hipLaunchKernelGGL(GemvKernel<4>, grid, dim3(256), 0, stream, a); break;
+            }
+            MI355X_HIP(hipGetLastError());
+            return 0;
+        }
         if (p->pw_bn)
         {
             const long long Mrows = static_cast<long long>(batch) * g.Ho * g.Wo;

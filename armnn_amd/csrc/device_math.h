@@ -150,6 +150,16 @@ __device__ __forceinline__ int Requant1Dev(int acc, const ChanTab& ct, int c, co
     return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.act_lo_f, rq.act_hi_f));
 }
 
+// one channel, accumulator started at zero: rows 2/5/6 on the fast path, `corr[c]` joins the accumulator on the exact path
+__device__ __forceinline__ int Requant1FoldedDev(int acc, const ChanTab& ct, const int32_t* corr, int c, const Requant& rq)
+{
+    float k;
+    bool slow;
+    MI355X_FAST1(acc, ct.p[2 * ct.stride + c], ct.p[5 * ct.stride + c], ct.p[6 * ct.stride + c], k, slow)
+    if (__builtin_expect(slow, 0)) return RequantExactDev(acc + corr[c], ct.p[c], ct.p[ct.stride + c], rq);
+    return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.act_lo_f, rq.act_hi_f));
+}
+
 // value already in float (pooling, add, ...): reciprocal fast path with the exact fallback near ties.
 //   r' = fma(f, fl(1/scale), offset) is within 2^-24 * (|f/scale| + |r'|) of f/scale + offset and the correctly rounded
 //   quotient within 2^-24 * |f/scale|; |offset| <= 255 is checked on the host (else fast_ok = 0).

@@ -226,4 +226,64 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
     }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// FullyConnected / pointwise layers with at most 4 GEMM rows (batch-1 inference): a matrix-vector product bound by
+// streaming the weights once from HBM.  A wave owns 4 output channels at a time; its 64 lanes split K in 16-byte
+// chunks (one coalesced 1 KB load per weight row and step), multiply with v_dot4 and reduce across the wave.
+struct GemvArgs
+{
+    const uint8_t* x;        // [M][K]
+    const int8_t*  w;        // [>= N rounded up to 4][w_stride], rows zero padded
+    ChanTab        ct;
+    const int32_t* corr;
+    uint8_t*       y;        // [M][N]
+    int M, K, N, w_stride;
+    uint32_t xor_mask;
+    Requant rq;
+};
+
+template <int MR>
+__global__ __launch_bounds__(256) void GemvKernel(GemvArgs a)
+{
+    constexpr int R = 4;
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n0 = (static_cast<int>(blockIdx.x) * 4 + wave) * R;
+    if (n0 >= a.N) return;
+    const int xm = static_cast<int>(a.xor_mask);
+    int acc[R][MR];
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m) acc[r][m] = 0;
+    const int chunks = a.K >> 4;
+    const int8_t* wrow = a.w + static_cast<long long>(n0) * a.w_stride;
+#pragma unroll 4
+    for (int j = lane; j < chunks; j += 64)
+    {
+        v4i xv[MR];
+#pragma unroll
+        for (int m = 0; m < MR; ++m) xv[m] = *reinterpret_cast<const v4i*>(a.x + static_cast<long long>(m) * a.K + j * 16) ^ xm;
+#pragma unroll
+        for (int r = 0; r < R; ++r)
+        {
+            const v4i wv = *reinterpret_cast<const v4i*>(wrow + static_cast<long long>(r) * a.w_stride + j * 16);
+#pragma unroll
+            for (int m = 0; m < MR; ++m)
+#pragma unroll
+                for (int d = 0; d < 4; ++d) acc[r][m] = __builtin_amdgcn_sdot4(xv[m][d], wv[d], acc[r][m], false);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < R; ++r)
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+        {
+            int v = acc[r][m];
+            for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o);
+            if (lane == 0 && n0 + r < a.N)
+                a.y[static_cast<long long>(m) * a.N + n0 + r] = static_cast<uint8_t>(Requant1FoldedDev(v, a.ct, a.corr, n0 + r, a.rq));
+        }
+}
+
 } // namespace mi355x

@@ -219,4 +219,8 @@ def small_fc_cases():
     c.append(make_fc_case("fc_s8_m1_k1024_o1001", 306, m=1, k=1024, o=1001))
     c.append(make_fc_case("fc_s8_k4096", 307, m=3, k=4096, o=40))
     c.append(make_fc_case("fc_s8_relu", 308, m=5, k=100, o=33, act=RELU))
+    # few rows: the weight-streaming matrix-vector kernel (1..4 rows, K % 16 == 0), ragged output counts
+    c.append(make_fc_case("fc_u8_m2_k80_o10", 309, m=2, k=80, o=10, in_dtype=U8, in_offset=131, out_offset=7, act=RELU6))
+    c.append(make_fc_case("fc_s8_m4_k2048_o203", 310, m=4, k=2048, o=203))
+    c.append(make_fc_case("fc_s8_m1_k48_o5_not_transposed", 311, m=1, k=48, o=5, transpose=False, bias=False))
     return c
