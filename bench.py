@@ -26,6 +26,46 @@ sys.path.insert(0, ROOT)
 
 INT8_MFMA_PEAK_OPS = 5.0e15      # MI355X dense int8, ops/s
 HBM_PEAK_BYTES = 8.0e12          # MI355X HBM3E, B/s
+RIDGE_OPS_PER_BYTE = INT8_MFMA_PEAK_OPS / HBM_PEAK_BYTES
+
+# HBM bytes per launch (read + written) of each MobileNetV1 layer at batch 64, from two rocprofv3 --pmc passes
+# (FETCH_SIZE, then WRITE_SIZE) over `python3 bench.py --profile-pass --no-graph`, each scaled by what the same counter
+# reads for the 64 MiB calibration copy of that pass (FETCH_SIZE counts 2 KiB units on this device: factor 1.999;
+# WRITE_SIZE 1 KiB units: factor 1.000).  Summary: profiles/mobilenet_v1_b64_hbm_traffic.md.
+MEASURED_HBM_TRAFFIC = {
+    ("mobilenet_v1_1.0_224", 64): {
+        "stem": 43143792,
+        "dw1": 51482293,
+        "pw1": 77282791,
+        "dw2": 64298192,
+        "pw2": 38912815,
+        "dw3": 51513126,
+        "pw3": 51807254,
+        "dw4": 32217414,
+        "pw4": 19858707,
+        "dw5": 25869979,
+        "pw5": 26564936,
+        "dw6": 16205108,
+        "pw6": 10982215,
+        "dw7": 13107001,
+        "pw7": 15305224,
+        "dw8": 13106106,
+        "pw8": 15305736,
+        "dw9": 13104059,
+        "pw9": 15306376,
+        "dw10": 13104187,
+        "pw10": 15305608,
+        "dw11": 13104827,
+        "pw11": 15306120,
+        "dw12": 8241622,
+        "pw12": 9543656,
+        "dw13": 6807456,
+        "pw13": 15567723,
+        "avgpool": 3581259,
+        "logits": 1801463,
+        "softmax": 194497
+    },
+}
 
 
 def layer_work(net, l, batch):
@@ -46,6 +86,14 @@ def layer_work(net, l, batch):
         co = net.tensors[l.output].shape[-1]
         nbytes += l.weights.info.num_elements + 8 * co     # + bias 4 B + per-channel scale 4 B
     return "hbm", float(nbytes)
+
+
+def algorithmic_bytes(net, l, batch):
+    """input(s) + output + weights + 8 B per output channel (bias, scale), each once, 1 B per 8-bit element."""
+    n = (sum(net.tensors[i].num_elements for i in l.inputs) + net.tensors[l.output].num_elements) * batch
+    if getattr(l, "weights", None) is not None:
+        n += l.weights.info.num_elements + 8 * net.tensors[l.output].shape[-1]
+    return n
 
 
 def cpu_baseline(net, seconds_budget=25.0):
@@ -81,6 +129,9 @@ def main():
     ap.add_argument("--fuse", action="store_true",
                     help="run depthwise + pointwise pairs as one kernel (same bytes; slower than two launches at present)")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
+    ap.add_argument("--profile-pass", action="store_true",
+                    help="for rocprofv3 --pmc: one 64 MiB calibration copy (1 B read + 1 B written per element), then ONE "
+                         "eager forward pass, one kernel per layer in network order; prints the dispatch order as JSON")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
@@ -95,6 +146,22 @@ def main():
     dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev
+
+    if args.profile_pass:
+        import ctypes as C
+        n = 64 << 20
+        a, b = shim.DeviceBuffer(n), shim.DeviceBuffer(n)
+        q = shim.Quant(0, 1.0, 0)
+        shim._chk(dn.lib.mi355x_fill_u8(a.ptr, 1, n, dn.stream))
+        dev.stream_sync(dn.stream)
+        shim._chk(dn.lib.mi355x_activation_run(n, C.byref(q), C.byref(q), shim.ACT_BOUNDED_RELU, 1000.0, -1000.0, a.ptr, b.ptr, dn.stream))
+        for _, fn in dn.steps:
+            fn(dn.stream)
+        dev.stream_sync(dn.stream)
+        print(json.dumps({"dispatch_order": ["fill (setup)", f"calibration copy {n} B in + {n} B out"] + [l.name for l, _ in dn.steps],
+                          "batch": batch, "net": net.name}))
+        dn.close()
+        return 0
 
     for _ in range(args.warmup):
         dn.enqueue()
@@ -113,22 +180,33 @@ def main():
     for l, ms in per_layer:
         kind, work = layer_work(net, l, batch)
         peak = INT8_MFMA_PEAK_OPS if kind == "mfma" else HBM_PEAK_BYTES
-        rows.append({"layer": l.name, "op": l.op, "ms": ms, "bound": kind, "work": work, "frac": work / (ms * 1e-3) / peak})
+        row = {"layer": l.name, "op": l.op, "ms": ms, "bound": kind, "work": work, "frac": work / (ms * 1e-3) / peak}
+        if kind == "mfma":
+            # the roof that binds a conv / FC layer depends on its arithmetic intensity: below the ridge
+            # (peak ops / peak bytes = 625 ops/B) the HBM roof is the lower one
+            nbytes = float(algorithmic_bytes(net, l, batch))
+            row["bytes"] = nbytes
+            row["binding"] = "mfma" if work / nbytes >= RIDGE_OPS_PER_BYTE else "hbm"
+        else:
+            row["bytes"] = work
+            row["binding"] = "hbm"
+        rows.append(row)
     total_ms = sum(r["ms"] for r in rows)
     dom = max(rows, key=lambda r: r["ms"])
     if args.layers:
         for r in rows:
-            print(f"{r['layer']:>10s} {r['op']:>9s} {r['ms']*1e3:9.1f} us  {r['bound']:>4s}  {100*r['frac']:6.2f}% of peak",
-                  file=sys.stderr)
+            hbm = r["bytes"] / (r["ms"] * 1e-3) / HBM_PEAK_BYTES
+            print(f"{r['layer']:>10s} {r['op']:>9s} {r['ms']*1e3:9.1f} us  {r['bound']:>4s} {100*r['frac']:6.2f}% of peak"
+                  f"   binding roof {r['binding']:>4s}, {100*hbm:5.1f}% of HBM peak on algorithmic bytes", file=sys.stderr)
         print(f"sum of kernels {total_ms:.3f} ms; graph step {ms_per_step:.3f} ms", file=sys.stderr)
-    if dom["bound"] == "mfma":
+    if dom["binding"] == "mfma":
         roof = {"bound": "mfma", "achieved": dom["work"] / (dom["ms"] * 1e-3) / 1e12, "peak": INT8_MFMA_PEAK_OPS / 1e12,
                 "unit": "TOP/s"}
     else:
-        roof = {"bound": "hbm", "achieved": dom["work"] / (dom["ms"] * 1e-3) / 1e9, "peak": HBM_PEAK_BYTES / 1e9,
+        roof = {"bound": "hbm", "achieved": dom["bytes"] / (dom["ms"] * 1e-3) / 1e9, "peak": HBM_PEAK_BYTES / 1e9,
                 "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = None
+    roof["traffic"] = MEASURED_HBM_TRAFFIC.get((net.name, batch), {}).get(dom["layer"])
     roof["kernel"] = f"{dom['layer']} ({dom['op']}), {dom['ms']*1e3:.1f} us of {total_ms*1e3:.1f} us"
 
     def group(ops, peak):
