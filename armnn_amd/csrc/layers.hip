@@ -5,9 +5,12 @@
 #include "device_math.h"
 
 #include <cfloat>
+#include <climits>
 #include <cmath>
 
 using namespace mi355x;
+
+typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 
 namespace
 {
@@ -140,6 +143,106 @@ __global__ __launch_bounds__(256) void Pool2dKernel(PoolArgs p, QIn qin, Requant
     y[idx] = static_cast<uint8_t>(QuantizeFastDev(result, rq));
 }
 
+// Four channels per thread (one dword per tap), windows of at most WB x WB taps with all loads issued up front.
+// Max pooling compares the raw codes: dequantization is strictly increasing, so the largest code is the largest value.
+template <int WB>
+__global__ __launch_bounds__(256) void Pool2dC4Kernel(PoolArgs p, QIn qin, Requant rq, const uint8_t* __restrict__ x,
+                                                      uint8_t* __restrict__ y, long long total4)
+{
+    const long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total4) return;
+    const int C4 = p.C >> 2;
+    const int c = static_cast<int>(idx % C4) * 4;
+    long long pix = idx / C4;
+    const int ox = static_cast<int>(pix % p.Wo);
+    pix /= p.Wo;
+    const int oy = static_cast<int>(pix % p.Ho);
+    const long long n = pix / p.Ho;
+
+    int hstart = oy * p.stride_y - p.pad_top;
+    int hend = min(hstart + p.pool_h, p.H + p.pad_bottom);
+    const int height = hend - hstart;
+    bool clamped = hstart < 0 || hend > p.H;
+    hstart = min(max(hstart, 0), p.H);
+    hend = min(max(hend, 0), p.H);
+    int wstart = ox * p.stride_x - p.pad_left;
+    int wend = min(wstart + p.pool_w, p.W + p.pad_right);
+    float area = static_cast<float>(height * (wend - wstart));
+    float res[4] = {0.0f, 0.0f, 0.0f, 0.0f};
+    if (!(hend <= 0 || hstart > p.H || wend <= 0 || wstart > p.W))
+    {
+        clamped = clamped || wstart < 0 || wend > p.W;
+        wstart = min(max(wstart, 0), p.W);
+        wend = min(max(wend, 0), p.W);
+        if (clamped && p.exclude) area = static_cast<float>((hend - hstart) * (wend - wstart));
+        const uint8_t* xn = x + n * p.H * p.W * p.C + c;
+        uint32_t raw[WB * WB];
+        const long long first = (static_cast<long long>(hstart) * p.W + wstart) * p.C;
+#pragma unroll
+        for (int dy = 0; dy < WB; ++dy)
+#pragma unroll
+            for (int dx = 0; dx < WB; ++dx)
+            {
+                const bool in = hstart + dy < hend && wstart + dx < wend;
+                raw[dy * WB + dx] = *reinterpret_cast<const uint32_t*>(xn + (in ? (static_cast<long long>(hstart + dy) * p.W + wstart + dx) * p.C : first));
+            }
+        int best[4] = {INT_MIN, INT_MIN, INT_MIN, INT_MIN};
+#pragma unroll
+        for (int dy = 0; dy < WB; ++dy)
+#pragma unroll
+            for (int dx = 0; dx < WB; ++dx)
+            {
+                if (hstart + dy < hend && wstart + dx < wend)
+                {
+                    const uint32_t w = raw[dy * WB + dx];
+#pragma unroll
+                    for (int ch = 0; ch < 4; ++ch)
+                    {
+                        const int code = qin.is_u8 ? static_cast<int>((w >> (8 * ch)) & 0xffu)
+                                                   : static_cast<int>(static_cast<int8_t>((w >> (8 * ch)) & 0xffu));
+                        if (p.is_max) best[ch] = max(best[ch], code);
+                        else res[ch] = __fadd_rn(res[ch], __fmul_rn(static_cast<float>(code - qin.offset), qin.scale));
+                    }
+                }
+            }
+#pragma unroll
+        for (int ch = 0; ch < 4; ++ch)
+        {
+            if (p.is_max) res[ch] = best[ch] == INT_MIN ? -FLT_MAX : __fmul_rn(static_cast<float>(best[ch] - qin.offset), qin.scale);
+            else res[ch] = __fdiv_rn(res[ch], area);
+        }
+    }
+    *reinterpret_cast<uint32_t*>(y + idx * 4) = Pack4(QuantizeFastDev(res[0], rq), QuantizeFastDev(res[1], rq),
+                                                      QuantizeFastDev(res[2], rq), QuantizeFastDev(res[3], rq));
+}
+
+// 16 elements per thread, 16-byte loads and stores
+__global__ __launch_bounds__(256) void AddVec16Kernel(QIn q0, QIn q1, Requant rq, const v4u* __restrict__ x0,
+                                                      const v4u* __restrict__ x1, v4u* __restrict__ y, size_t n16)
+{
+    size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
+    const size_t stride = static_cast<size_t>(gridDim.x) * 256;
+    for (; i < n16; i += stride)
+    {
+        const v4u a = x0[i], b = x1[i];
+        v4u o;
+#pragma unroll
+        for (int d = 0; d < 4; ++d)
+        {
+            int q[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k)
+            {
+                const float s = __fadd_rn(DequantDev(static_cast<uint8_t>((a[d] >> (8 * k)) & 0xffu), q0),
+                                          DequantDev(static_cast<uint8_t>((b[d] >> (8 * k)) & 0xffu), q1));
+                q[k] = QuantizeFastDev(s, rq);
+            }
+            o[d] = Pack4(q[0], q[1], q[2], q[3]);
+        }
+        y[i] = o;
+    }
+}
+
 __global__ __launch_bounds__(256) void AddKernel(QIn q0, QIn q1, Requant rq, int fn, float a, float b,
                                                  const uint8_t* __restrict__ x0, const uint8_t* __restrict__ x1,
                                                  uint8_t* __restrict__ y, size_t n)
@@ -268,8 +371,16 @@ int mi355x_pool2d_run(const mi355x_pool2d_desc* d, uint32_t batch, const void* i
     p.exclude = d->padding_method == 1;
     Requant rq = MakeRequant(d->output, MI355X_ACT_NONE, 0.0f, 0.0f);
     const long long total = static_cast<long long>(batch) * p.Ho * p.Wo * p.C;
-    hipLaunchKernelGGL(Pool2dKernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, ToHip(stream), p,
-                       MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), total);
+    const bool vec4 = (p.C % 4) == 0 && (reinterpret_cast<uintptr_t>(input_dev) & 3) == 0 && (reinterpret_cast<uintptr_t>(output_dev) & 3) == 0;
+    if (vec4 && p.pool_w <= 3 && p.pool_h <= 3)
+        hipLaunchKernelGGL(Pool2dC4Kernel<3>, dim3(static_cast<unsigned>((total / 4 + 255) / 256)), dim3(256), 0, ToHip(stream), p,
+                           MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), total / 4);
+    else if (vec4 && p.pool_w <= 8 && p.pool_h <= 8)
+        hipLaunchKernelGGL(Pool2dC4Kernel<8>, dim3(static_cast<unsigned>((total / 4 + 255) / 256)), dim3(256), 0, ToHip(stream), p,
+                           MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), total / 4);
+    else
+        hipLaunchKernelGGL(Pool2dKernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, ToHip(stream), p,
+                           MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), total);
     MI355X_HIP(hipGetLastError());
     return 0;
 }
@@ -285,9 +396,15 @@ int mi355x_add_run(size_t n, const mi355x_quant* in0_q, const mi355x_quant* in1_
     if (n == 0) return 0;
     if (!input0_dev || !input1_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "null tensor pointer");
     Requant rq = MakeRequant(*out_q, activation, a, b);
-    hipLaunchKernelGGL(AddKernel, dim3(GridFor(n)), dim3(256), 0, ToHip(stream), MakeQIn(*in0_q), MakeQIn(*in1_q), rq,
-                       activation, a, b, static_cast<const uint8_t*>(input0_dev), static_cast<const uint8_t*>(input1_dev),
-                       static_cast<uint8_t*>(output_dev), n);
+    const bool vec16 = (n % 16) == 0 && ((reinterpret_cast<uintptr_t>(input0_dev) | reinterpret_cast<uintptr_t>(input1_dev) |
+                                           reinterpret_cast<uintptr_t>(output_dev)) & 15) == 0;
+    if (vec16)
+        hipLaunchKernelGGL(AddVec16Kernel, dim3(GridFor(n / 16)), dim3(256), 0, ToHip(stream), MakeQIn(*in0_q), MakeQIn(*in1_q), rq,
+                           static_cast<const v4u*>(input0_dev), static_cast<const v4u*>(input1_dev), static_cast<v4u*>(output_dev), n / 16);
+    else
+        hipLaunchKernelGGL(AddKernel, dim3(GridFor(n)), dim3(256), 0, ToHip(stream), MakeQIn(*in0_q), MakeQIn(*in1_q), rq,
+                           activation, a, b, static_cast<const uint8_t*>(input0_dev), static_cast<const uint8_t*>(input1_dev),
+                           static_cast<uint8_t*>(output_dev), n);
     MI355X_HIP(hipGetLastError());
     return 0;
 }
