@@ -23,6 +23,8 @@ struct mi355x_conv2d_s
     uint8_t* w_direct = nullptr;   // [Kh][Kw][Ci][Co] / depthwise [Kh][Kw][Co], raw codes
     int8_t*  w_mfma   = nullptr;   // [Co_pad][K_pad] signed, zero padded
     uint8_t* pad16    = nullptr;   // 16 bytes that turn into the padding value under the kernel's input xor
+    int8_t*  w_stem   = nullptr;   // small-Ci conv on MFMA: [Co rounded up to 32][stem_kp]
+    int      stem_kp  = 0;
     uint32_t* dw_grp  = nullptr;   // depthwise 3x3: constants per group of 4 channels for the fused dw+pw kernel
     uint32_t* w_dot4  = nullptr;   // depthwise 3x3: [C][4] dwords; small-Ci conv: [Co][Kh][RD] dwords
     int variant = 0;               // kernel variant within an algo (see RunPlan)
@@ -43,6 +45,7 @@ struct mi355x_conv2d_s
         (void)hipFree(w_mfma);
         (void)hipFree(pad16);
         (void)hipFree(dw_grp);
+        (void)hipFree(w_stem);
         (void)hipFree(w_dot4);
         (void)hipFree(chan);
         (void)hipFree(corr);
@@ -320,6 +323,16 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         p->xor_mask = g.in_u8 ? 0x80u : 0u;
         p->pad_word = static_cast<uint32_t>(zx_shift) & 0xffu;
         p->row_dwords = RD;
+        if (Co == 32 || Co == 64)
+        {
+            // the same rows, end to end, as the K vector of the MFMA variant
+            const int kp = (Kh * RD * 4 + 31) / 32 * 32;
+            const int rows = (Co + 31) / 32 * 32;
+            std::vector<int8_t> wm(static_cast<size_t>(rows) * kp, 0);
+            for (int c = 0; c < Co; ++c) std::memcpy(wm.data() + static_cast<size_t>(c) * kp, wp.data() + static_cast<size_t>(c) * Kh * RD, static_cast<size_t>(Kh) * RD * 4);
+            if (int rc = Upload(reinterpret_cast<void**>(&p->w_stem), wm.data(), wm.size())) return rc;
+            p->stem_kp = kp;
+        }
         FoldCorrIntoTable(p, corr, Co);
         char buf[96];
         snprintf(buf, sizeof(buf), "smallci_dot4_lds %dx%dx%d stride %u, tile 32x16", Kh, Kw, Ci, d.stride_x);
@@ -555,6 +568,16 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
         if (nb > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
         const dim3 grid(static_cast<unsigned>(nb));
+        a.w_mfma = p->w_stem; a.kp = p->stem_kp;
+        if (p->w_stem && !GlobalOptions().stem_dot4 && (g.Kh == 3 || g.Kh == 7))
+        {
+            if (g.Kh == 3 && g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 1>), grid, dim3(256), 0, stream, a);
+            else if (g.Kh == 3) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 2>), grid, dim3(256), 0, stream, a);
+            else if (g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 1>), grid, dim3(256), 0, stream, a);
+            else hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 2>), grid, dim3(256), 0, stream, a);
+            MI355X_HIP(hipGetLastError());
+            return 0;
+        }
         if (g.Kh == 3) hipLaunchKernelGGL((SmallCiConvKernel<3, 3>), grid, dim3(256), 0, stream, a);
         else if (g.Kh == 7) hipLaunchKernelGGL((SmallCiConvKernel<7, 6>), grid, dim3(256), 0, stream, a);
         else if (g.Kh == 5) hipLaunchKernelGGL((SmallCiConvKernel<5, 5>), grid, dim3(256), 0, stream, a);

@@ -188,6 +188,8 @@ struct SmallCiArgs
     uint32_t ndw_recip;       // ceil(2^32 / (lp / 4))
     uint32_t xor_mask, pad_byte;
     int vec16;                // output rows allow 16-byte stores (y 16-byte aligned, Co % 16 == 0)
+    const int8_t* w_mfma;     // MFMA variant: [Co rounded up to 32][kp] bytes, a filter's rows as RD dwords each, zero padded
+    int kp;                   // bytes per weight row of w_mfma (multiple of 32)
     Requant rq;
 };
 
@@ -198,27 +200,34 @@ struct SmallCiArgs
 //   Compute: a thread reads its KH rows of Kw*Ci contiguous bytes as aligned dwords + v_alignbyte, then walks the
 //   output channels; weights and requantization constants are wave-uniform scalar loads, so a v_dot4 takes its
 //   weight operand from an SGPR.  16 channels of a pixel leave as one 16-byte store.
-template <int KH, int RD>
-__global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
+// Geometry of the small-Ci kernels' block tile: 32 x 16 output pixels and its input halo in LDS.
+template <int KH>
+struct SmallCiTile
 {
-    constexpr int P = 2, TW = 16 * P, TH = 16;
-    constexpr int HRMAX = (TH - 1) * 2 + KH;
-    constexpr int LPMAX = 288;                               // >= 3 + (TW-1)*2*4 + 4*6 rounded up, + 8
-    __shared__ __attribute__((aligned(16))) uint32_t tile[HRMAX * LPMAX / 4];
+    static constexpr int TW = 32, TH = 16;
+    static constexpr int HRMAX = (TH - 1) * 2 + KH;
+    static constexpr int LPMAX = 288;                        // >= 3 + (TW-1)*2*4 + 4*6 rounded up, + 8
+    static constexpr int DWORDS = HRMAX * LPMAX / 4;
+};
 
-    int b = blockIdx.x;
-    const int tx = b % a.tiles_x; b /= a.tiles_x;
-    const int ty = b % a.tiles_y;
-    const int n = b / a.tiles_y;
-    const int tid = threadIdx.x;
+// Copies the halo of output tile (tx, ty) of image n into `tile` (LDS row pitch a.lp bytes).
+//   Each halo row is copied as ALIGNED dwords (rows start at arbitrary byte addresses when Ci is 3, so the LDS row keeps
+//   the global misalignment and readers add it back: row r starts at byte (A_r & 3) of its LDS row, A_r being the row's
+//   byte offset from the aligned image base); only dwords that straddle an image edge are assembled byte by byte, and
+//   positions outside the image hold the shifted zero point.  Returns through the references what readers need.
+template <int KH>
+__device__ __forceinline__ void StageSmallCiHalo(const SmallCiArgs& a, uint32_t* tile, int tx, int ty, int n, int tid,
+                                                 int& iy_org, int& ix_org, int& mis)
+{
+    constexpr int TW = SmallCiTile<KH>::TW, TH = SmallCiTile<KH>::TH;
+    constexpr int HRMAX = SmallCiTile<KH>::HRMAX, LPMAX = SmallCiTile<KH>::LPMAX;
     const int S = a.stride;
     const int HR = (TH - 1) * S + KH;
     const int NDW = a.lp >> 2;
-
-    const int iy_org = ty * TH * S - a.pad_top;
-    const int ix_org = tx * TW * S - a.pad_left;
+    iy_org = ty * TH * S - a.pad_top;
+    ix_org = tx * TW * S - a.pad_left;
     const uint8_t* xn = a.x + static_cast<long long>(n) * a.H * a.W * a.Ci;
-    const int mis = static_cast<int>(reinterpret_cast<uintptr_t>(xn) & 3);
+    mis = static_cast<int>(reinterpret_cast<uintptr_t>(xn) & 3);
     const uint8_t* xal = xn - mis;                           // 4-byte aligned
     const uint32_t xm = a.xor_mask & 0xffu;
     const uint32_t xm4 = xm * 0x01010101u;
@@ -276,6 +285,22 @@ __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
             tile[i] = v;
         }
     }
+}
+
+template <int KH, int RD>
+__global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
+{
+    constexpr int P = 2, TW = 16 * P, TH = 16;
+    __shared__ __attribute__((aligned(16))) uint32_t tile[SmallCiTile<KH>::DWORDS];
+
+    int b = blockIdx.x;
+    const int tx = b % a.tiles_x; b /= a.tiles_x;
+    const int ty = b % a.tiles_y;
+    const int n = b / a.tiles_y;
+    const int tid = threadIdx.x;
+    const int S = a.stride;
+    int iy_org, ix_org, mis;
+    StageSmallCiHalo<KH>(a, tile, tx, ty, n, tid, iy_org, ix_org, mis);
     __syncthreads();
 
     const int lx = tid & 15, ly = tid >> 4;
@@ -352,6 +377,97 @@ __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
                 if (g4 >= groups) continue;
                 *reinterpret_cast<uint32_t*>(yp + co + 4 * g4) = o[0][g4];
                 if (second) *reinterpret_cast<uint32_t*>(yp + a.Co + co + 4 * g4) = o[1][g4];
+            }
+        }
+    }
+}
+
+// The same layers on the matrix cores.  A filter row of Kw*Ci bytes, padded to RD dwords, is how the dot4 kernel already
+// holds a pixel's inputs in registers; laid end to end, the KH rows are a K vector of KH*RD*4 bytes (zero weights under
+// the padding), and 32 pixels x 32 output channels become ceil(KH*RD/8) MFMA steps instead of 32*KH*RD dot products per
+// pixel.  Both lanes of a pixel (lane, lane + 32) gather the pixel's rows from the LDS halo and keep the half of each
+// 32-byte k-step that the MFMA B operand assigns them.  A wave takes 4 of the tile's 16 rows; NT = output channels / 32.
+template <int KH, int RD, int NT>
+__global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
+{
+    constexpr int TW = 32, TH = 16;
+    constexpr int NDWP = KH * RD;                 // patch dwords per pixel
+    constexpr int KST = (NDWP + 7) / 8;           // MFMA k-steps of 32 bytes
+    __shared__ __attribute__((aligned(16))) uint32_t tile[SmallCiTile<KH>::DWORDS];
+    __shared__ __attribute__((aligned(16))) float cst[3][NT * 32];
+
+    int b = blockIdx.x;
+    const int tx = b % a.tiles_x; b /= a.tiles_x;
+    const int ty = b % a.tiles_y;
+    const int n = b / a.tiles_y;
+    const int tid = threadIdx.x;
+    const int S = a.stride;
+    int iy_org, ix_org, mis;
+    StageSmallCiHalo<KH>(a, tile, tx, ty, n, tid, iy_org, ix_org, mis);
+    for (int i = tid; i < 3 * NT * 32; i += 256)
+    {
+        const int row = i / (NT * 32), c = i - row * (NT * 32);
+        cst[row][c] = a.ct.p[(row == 0 ? 2 : row == 1 ? 5 : 6) * a.ct.stride + c];
+    }
+
+    const int lane = tid & 63, wave = tid >> 6;
+    const int px = lane & 31, half = lane >> 5;
+    // weight fragments of every channel tile and k-step stay in registers
+    v4i wfrag[NT][KST];
+#pragma unroll
+    for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+        for (int t = 0; t < KST; ++t)
+            wfrag[ct][t] = *reinterpret_cast<const v4i*>(a.w_mfma + static_cast<long long>(ct * 32 + px) * a.kp + t * 32 + half * 16);
+    __syncthreads();
+
+    const int ox = tx * TW + px;
+#pragma unroll 1
+    for (int rr = 0; rr < 4; ++rr)
+    {
+        const int ly = wave * 4 + rr;
+        const int oy = ty * TH + ly;
+        if (oy >= a.Ho) break;                    // wave-uniform
+        uint32_t flat[KST * 8];
+#pragma unroll
+        for (int i = NDWP; i < KST * 8; ++i) flat[i] = 0u;
+#pragma unroll
+        for (int r = 0; r < KH; ++r)
+        {
+            const int row = ly * S + r;
+            const int sh_row = ((((iy_org + row) * a.W + ix_org) * a.Ci + mis) & 3);
+            const int off = row * a.lp + sh_row + px * S * a.Ci;
+            const uint32_t* q = tile + (off >> 2);
+            const int sh = off & 3;
+            uint32_t d[RD + 1];
+#pragma unroll
+            for (int i = 0; i <= RD; ++i) d[i] = q[i];
+#pragma unroll
+            for (int i = 0; i < RD; ++i) flat[r * RD + i] = __builtin_amdgcn_alignbyte(d[i + 1], d[i], sh);
+        }
+        v4i bfrag[KST];
+#pragma unroll
+        for (int t = 0; t < KST; ++t)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) bfrag[t][j] = static_cast<int>(half ? flat[8 * t + 4 + j] : flat[8 * t + j]);
+
+        uint8_t* yp = a.y + ((static_cast<long long>(n) * a.Ho + oy) * a.Wo + ox) * a.Co;
+#pragma unroll
+        for (int ct = 0; ct < NT; ++ct)
+        {
+            const v16i zero = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+            v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wfrag[ct][0], bfrag[0], zero, 0, 0, 0);
+#pragma unroll
+            for (int t = 1; t < KST; ++t) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wfrag[ct][t], bfrag[t], acc, 0, 0, 0);
+#pragma unroll
+            for (int qd = 0; qd < 4; ++qd)
+            {
+                const int cl = ct * 32 + 8 * qd + 4 * half;
+                const float4 fm = *reinterpret_cast<const float4*>(&cst[0][cl]);
+                const float4 fb = *reinterpret_cast<const float4*>(&cst[1][cl]);
+                const float4 th = *reinterpret_cast<const float4*>(&cst[2][cl]);
+                const uint32_t out = Requant4Dev(acc[4 * qd + 0], acc[4 * qd + 1], acc[4 * qd + 2], acc[4 * qd + 3], fm, fb, th, a.ct, a.corr, cl, a.rq);
+                if (ox < a.Wo) *reinterpret_cast<uint32_t*>(yp + cl) = out;
             }
         }
     }

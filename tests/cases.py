@@ -202,6 +202,11 @@ def small_conv_cases():
     c.append(make_conv_case("stem_u8_3x3_s1_ci3_wide", 225, n=3, h=37, w=71, ci=3, co=20, in_dtype=U8, in_offset=77,
                             out_offset=3))
     c.append(make_conv_case("stem_s8_3x3_s2_ci2", 226, n=2, h=35, w=131, ci=2, co=48, stride=(2, 2), in_offset=5))
+    # 32 or 64 output channels: the matrix-core variant (the other counts above stay on v_dot4)
+    c.append(make_conv_case("stem_s8_3x3_s1_ci3_co64", 227, n=2, h=33, w=70, ci=3, co=64, in_offset=-20, act=RELU6))
+    c.append(make_conv_case("stem_u8_7x7_s2_ci3_co32", 228, n=2, h=39, w=45, ci=3, co=32, kh=7, kw=7, stride=(2, 2), in_dtype=U8,
+                            in_offset=111, out_offset=9, w_scale_range=(0.002, 0.008)))
+    c.append(make_conv_case("stem_s8_3x3_s2_ci4_co32", 229, n=1, h=18, w=40, ci=4, co=32, stride=(2, 2)))
     c.append(make_conv_case("dw_u8_5x5_c20", 206, h=9, w=9, ci=20, depthwise=True, kh=5, kw=5, in_dtype=U8,
                             in_offset=100, out_offset=3, w_scale_range=(0.005, 0.02)))
     return c

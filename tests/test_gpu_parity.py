@@ -117,6 +117,21 @@ def test_fast_epilogue_equals_exact_division():
         np.testing.assert_array_equal(f.data, e.data)
 
 
+def test_stem_mfma_equals_stem_dot4():
+    """Small-Ci convolutions: the matrix-core kernel and the v_dot4 kernel produce the same bytes."""
+    for c in CONV:
+        if not c.name.startswith("stem_") or c.out_info.shape[-1] not in (32, 64) or c.w.info.shape[1] not in (3, 7):
+            continue
+        print("case", c.name, flush=True)
+        mfma = _gpu_conv(c, shim.ALGO_AUTO)
+        shim.set_option("stem_dot4", 1)
+        try:
+            dot4 = _gpu_conv(c, shim.ALGO_AUTO)
+        finally:
+            shim.set_option("stem_dot4", 0)
+        np.testing.assert_array_equal(mfma.data, dot4.data)
+
+
 def test_config_c1_full_size(port):
     """BASELINE config 1: 1x56x56x64 -> 64, 3x3 SAME, per-channel, ReLU6; expected code range [-128, -8]."""
     c = cases.make_conv_case("C1", 20250101, h=56, w=56, ci=64, co=64, act=cases.RELU6)
