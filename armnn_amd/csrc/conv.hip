@@ -565,19 +565,22 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         if (a.lp > 288) return SetError(MI355X_ERR_UNSUPPORTED, "dot4 kernel: halo row of %d bytes does not fit", a.lp);
         if (static_cast<long long>(g.H) * g.W * g.Ci >= (1ll << 30)) return SetError(MI355X_ERR_UNSUPPORTED, "dot4 kernel: image too large for 32-bit offsets");
         a.rq = p->rq;
-        const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
-        if (nb > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
-        const dim3 grid(static_cast<unsigned>(nb));
         a.w_mfma = p->w_stem; a.kp = p->stem_kp;
         if (p->w_stem && !GlobalOptions().stem_dot4 && (g.Kh == 3 || g.Kh == 7))
         {
-            if (g.Kh == 3 && g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 1>), grid, dim3(256), 0, stream, a);
-            else if (g.Kh == 3) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 2>), grid, dim3(256), 0, stream, a);
-            else if (g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 1>), grid, dim3(256), 0, stream, a);
-            else hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 2>), grid, dim3(256), 0, stream, a);
+            const long long nbm = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
+            if (nbm > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
+            const dim3 gridm(static_cast<unsigned>(nbm));
+            if (g.Kh == 3 && g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 1, 16>), gridm, dim3(256), 0, stream, a);
+            else if (g.Kh == 3) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 2, 16>), gridm, dim3(256), 0, stream, a);
+            else if (g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 1, 16>), gridm, dim3(256), 0, stream, a);
+            else hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 2, 16>), gridm, dim3(256), 0, stream, a);
             MI355X_HIP(hipGetLastError());
             return 0;
         }
+        const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
+        if (nb > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
+        const dim3 grid(static_cast<unsigned>(nb));
         if (g.Kh == 3) hipLaunchKernelGGL((SmallCiConvKernel<3, 3>), grid, dim3(256), 0, stream, a);
         else if (g.Kh == 7) hipLaunchKernelGGL((SmallCiConvKernel<7, 6>), grid, dim3(256), 0, stream, a);
         else if (g.Kh == 5) hipLaunchKernelGGL((SmallCiConvKernel<5, 5>), grid, dim3(256), 0, stream, a);

@@ -201,10 +201,10 @@ struct SmallCiArgs
 //   output channels; weights and requantization constants are wave-uniform scalar loads, so a v_dot4 takes its
 //   weight operand from an SGPR.  16 channels of a pixel leave as one 16-byte store.
 // Geometry of the small-Ci kernels' block tile: 32 x 16 output pixels and its input halo in LDS.
-template <int KH>
+template <int KH, int TH_ = 16>
 struct SmallCiTile
 {
-    static constexpr int TW = 32, TH = 16;
+    static constexpr int TW = 32, TH = TH_;
     static constexpr int HRMAX = (TH - 1) * 2 + KH;
     static constexpr int LPMAX = 288;                        // >= 3 + (TW-1)*2*4 + 4*6 rounded up, + 8
     static constexpr int DWORDS = HRMAX * LPMAX / 4;
@@ -215,12 +215,12 @@ struct SmallCiTile
 //   the global misalignment and readers add it back: row r starts at byte (A_r & 3) of its LDS row, A_r being the row's
 //   byte offset from the aligned image base); only dwords that straddle an image edge are assembled byte by byte, and
 //   positions outside the image hold the shifted zero point.  Returns through the references what readers need.
-template <int KH>
+template <int KH, int TH_ = 16>
 __device__ __forceinline__ void StageSmallCiHalo(const SmallCiArgs& a, uint32_t* tile, int tx, int ty, int n, int tid,
                                                  int& iy_org, int& ix_org, int& mis)
 {
-    constexpr int TW = SmallCiTile<KH>::TW, TH = SmallCiTile<KH>::TH;
-    constexpr int HRMAX = SmallCiTile<KH>::HRMAX, LPMAX = SmallCiTile<KH>::LPMAX;
+    constexpr int TW = SmallCiTile<KH, TH_>::TW, TH = SmallCiTile<KH, TH_>::TH;
+    constexpr int HRMAX = SmallCiTile<KH, TH_>::HRMAX, LPMAX = SmallCiTile<KH, TH_>::LPMAX;
     const int S = a.stride;
     const int HR = (TH - 1) * S + KH;
     const int NDW = a.lp >> 2;
@@ -239,39 +239,46 @@ __device__ __forceinline__ void StageSmallCiHalo(const SmallCiArgs& a, uint32_t*
     // loads, pass 2 assembles the few dwords that straddle an image edge and writes everything to LDS.
     constexpr int MAXIT = (HRMAX * (LPMAX / 4) + 255) / 256;
     const int total = HR * NDW;
+    const int nit = (total + 255) >> 8;                      // passes this tile really needs (block-uniform)
     uint32_t sv[MAXIT];
+    int slo[MAXIT];                                          // dword offset from xal; bit 0: straddles an image edge
     // loads are unconditional (a dword that is not wholly inside the image reads a harmless in-tensor address and
     // is discarded), so that none of them waits for another
     const long long safe = reinterpret_cast<const uint8_t*>((reinterpret_cast<uintptr_t>(a.x) + 3) & ~static_cast<uintptr_t>(3)) - xal;
 #pragma unroll
     for (int k = 0; k < MAXIT; ++k)
     {
-        const int i = min(tid + k * 256, total - 1);
-        const int row = static_cast<int>(__umulhi(static_cast<uint32_t>(i), a.ndw_recip));
-        const int j = i - row * NDW;
-        const int iy = iy_org + row;
-        const int A = (iy * a.W + ix_org) * a.Ci + mis;      // halo row start as a byte offset from xal (may be < 0)
-        const int lo = (A & ~3) + 4 * j;
-        const bool inside = static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && lo >= A + vb0 && lo + 4 <= A + vb1;
-        const uint32_t ld = *reinterpret_cast<const uint32_t*>(xal + (inside ? static_cast<long long>(lo) : safe));
-        sv[k] = inside ? (ld ^ xm4) : pad4;
+        if (k < nit)
+        {
+            const int i = min(tid + k * 256, total - 1);
+            const int row = static_cast<int>(__umulhi(static_cast<uint32_t>(i), a.ndw_recip));
+            const int j = i - row * NDW;
+            const int iy = iy_org + row;
+            const int A = (iy * a.W + ix_org) * a.Ci + mis;  // halo row start as a byte offset from xal (may be < 0)
+            const int lo = (A & ~3) + 4 * j;
+            const int vbeg = A + vb0, vend = A + vb1;
+            const bool row_ok = static_cast<unsigned>(iy) < static_cast<unsigned>(a.H);
+            const bool inside = row_ok && lo >= vbeg && lo + 4 <= vend;
+            const bool edge = row_ok && !inside && lo + 4 > vbeg && lo < vend;
+            const uint32_t ld = *reinterpret_cast<const uint32_t*>(xal + (inside ? static_cast<long long>(lo) : safe));
+            sv[k] = inside ? (ld ^ xm4) : pad4;
+            slo[k] = lo | (edge ? 1 : 0);
+        }
     }
 #pragma unroll
     for (int k = 0; k < MAXIT; ++k)
     {
         const int i = tid + k * 256;
-        if (i < total)
+        if (k < nit && i < total)
         {
-            const int row = static_cast<int>(__umulhi(static_cast<uint32_t>(i), a.ndw_recip));
-            const int j = i - row * NDW;
-            const int iy = iy_org + row;
-            const int A = (iy * a.W + ix_org) * a.Ci + mis;
-            const int lo = (A & ~3) + 4 * j;
-            const int vbeg = A + vb0, vend = A + vb1;
             uint32_t v = sv[k];
-            const bool inside = lo >= vbeg && lo + 4 <= vend;
-            if (static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && !inside && lo + 4 > vbeg && lo < vend)
+            if (slo[k] & 1)
             {
+                // rare: rebuild the dword byte by byte against this row's valid range
+                const int lo = slo[k] & ~3;
+                const int row = static_cast<int>(__umulhi(static_cast<uint32_t>(i), a.ndw_recip));
+                const int A = ((iy_org + row) * a.W + ix_org) * a.Ci + mis;
+                const int vbeg = A + vb0, vend = A + vb1;
                 v = 0;
 #pragma unroll
                 for (int q = 0; q < 4; ++q)
@@ -387,13 +394,14 @@ __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
 // the padding), and 32 pixels x 32 output channels become ceil(KH*RD/8) MFMA steps instead of 32*KH*RD dot products per
 // pixel.  Both lanes of a pixel (lane, lane + 32) gather the pixel's rows from the LDS halo and keep the half of each
 // 32-byte k-step that the MFMA B operand assigns them.  A wave takes 4 of the tile's 16 rows; NT = output channels / 32.
-template <int KH, int RD, int NT>
+template <int KH, int RD, int NT, int TH>
 __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
 {
-    constexpr int TW = 32, TH = 16;
+    constexpr int TW = 32;
+    constexpr int RPW = TH / 4;                   // tile rows per wave
     constexpr int NDWP = KH * RD;                 // patch dwords per pixel
     constexpr int KST = (NDWP + 7) / 8;           // MFMA k-steps of 32 bytes
-    __shared__ __attribute__((aligned(16))) uint32_t tile[SmallCiTile<KH>::DWORDS];
+    __shared__ __attribute__((aligned(16))) uint32_t tile[SmallCiTile<KH, TH>::DWORDS];
     __shared__ __attribute__((aligned(16))) float cst[3][NT * 32];
 
     int b = blockIdx.x;
@@ -403,7 +411,7 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
     const int tid = threadIdx.x;
     const int S = a.stride;
     int iy_org, ix_org, mis;
-    StageSmallCiHalo<KH>(a, tile, tx, ty, n, tid, iy_org, ix_org, mis);
+    StageSmallCiHalo<KH, TH>(a, tile, tx, ty, n, tid, iy_org, ix_org, mis);
     for (int i = tid; i < 3 * NT * 32; i += 256)
     {
         const int row = i / (NT * 32), c = i - row * (NT * 32);
@@ -423,9 +431,9 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
 
     const int ox = tx * TW + px;
 #pragma unroll 1
-    for (int rr = 0; rr < 4; ++rr)
+    for (int rr = 0; rr < RPW; ++rr)
     {
-        const int ly = wave * 4 + rr;
+        const int ly = wave * RPW + rr;
         const int oy = ty * TH + ly;
         if (oy >= a.Ho) break;                    // wave-uniform
         uint32_t flat[KST * 8];
@@ -459,6 +467,7 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
             v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wfrag[ct][0], bfrag[0], zero, 0, 0, 0);
 #pragma unroll
             for (int t = 1; t < KST; ++t) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wfrag[ct][t], bfrag[t], acc, 0, 0, 0);
+            uint32_t o[4];
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd)
             {
@@ -466,8 +475,21 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
                 const float4 fm = *reinterpret_cast<const float4*>(&cst[0][cl]);
                 const float4 fb = *reinterpret_cast<const float4*>(&cst[1][cl]);
                 const float4 th = *reinterpret_cast<const float4*>(&cst[2][cl]);
-                const uint32_t out = Requant4Dev(acc[4 * qd + 0], acc[4 * qd + 1], acc[4 * qd + 2], acc[4 * qd + 3], fm, fb, th, a.ct, a.corr, cl, a.rq);
-                if (ox < a.Wo) *reinterpret_cast<uint32_t*>(yp + cl) = out;
+                o[qd] = Requant4Dev(acc[4 * qd + 0], acc[4 * qd + 1], acc[4 * qd + 2], acc[4 * qd + 3], fm, fb, th, a.ct, a.corr, cl, a.rq);
+            }
+            // lane and lane + 32 hold interleaved 4-channel groups of one pixel; trading two dwords gives each of them
+            // 16 contiguous channels (the low lane 0..15, the high lane 16..31) and one 16-byte store
+            const uint32_t r0 = __shfl_xor(half ? o[0] : o[2], 32);
+            const uint32_t r1 = __shfl_xor(half ? o[1] : o[3], 32);
+            const uint4 v = half ? uint4{r0, o[2], r1, o[3]} : uint4{o[0], r0, o[1], r1};
+            if (ox < a.Wo)
+            {
+                if (a.vec16) *reinterpret_cast<uint4*>(yp + ct * 32 + 16 * half) = v;
+                else
+                {
+                    uint32_t* dst = reinterpret_cast<uint32_t*>(yp + ct * 32 + 16 * half);
+                    dst[0] = v.x; dst[1] = v.y; dst[2] = v.z; dst[3] = v.w;
+                }
             }
         }
     }
