@@ -595,7 +595,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 3) != 0)
                 return SetError(MI355X_ERR_INVALID_ARGUMENT, "depthwise 3x3 kernel needs a 16-byte aligned input and 4-byte aligned output");
             Dw3x3Args a;
-            a.x = xin; a.wpack = p->w_dot4; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
+            a.x = xin; a.pad16 = p->pad16; a.wpack = p->w_dot4; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
             a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.C = g.Co; a.Ho = g.Ho; a.Wo = g.Wo;
             a.pad_top = g.pad_top; a.pad_left = g.pad_left;
             const int tw = g.stride_x == 1 ? 16 : 8;

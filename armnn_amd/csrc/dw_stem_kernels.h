@@ -20,6 +20,7 @@ namespace mi355x
 struct Dw3x3Args
 {
     const uint8_t*  x;
+    const uint8_t*  pad16;    // 16 bytes of (padding value ^ input xor)
     const uint32_t* wpack;    // [C][4] dwords; dword r (r < 3) = bytes { w[r][0][c], w[r][1][c], w[r][2][c], 0 }
     ChanTab         ct;
     const int32_t*  corr;     // [C]  -zx' * sum of the 9 taps
@@ -69,20 +70,29 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
     const int iy_org = ty * TH * S - a.pad_top;
     const int ix_org = tx * TW * S - a.pad_left;
     const uint8_t* xn = a.x + static_cast<long long>(n) * a.H * a.W * a.C + cb * CB;
-    const v4i padv = {static_cast<int>(a.pad_word), static_cast<int>(a.pad_word), static_cast<int>(a.pad_word),
-                      static_cast<int>(a.pad_word)};
     const int xm = static_cast<int>(a.xor_mask);
-    for (int i = tid; i < HR * HC * 2; i += 256)
+    // all of a thread's staging loads are issued before the first is used; a chunk outside the image reads 16 prepared
+    // bytes that become the padding value under the xor, so no load sits in a divergent branch
+    constexpr int NST = (HR * HC * 2 + 255) / 256;
+    v4i st[NST];
+#pragma unroll
+    for (int k = 0; k < NST; ++k)
     {
+        const int i = min(tid + k * 256, HR * HC * 2 - 1);
         const int half = i & 1;
         const int pix = i >> 1;
         const int col = pix % HC;
         const int row = pix / HC;
         const int iy = iy_org + row, ix = ix_org + col;
-        v4i v = padv;
-        if (static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && static_cast<unsigned>(ix) < static_cast<unsigned>(a.W))
-            v = *reinterpret_cast<const v4i*>(xn + (static_cast<long long>(iy) * a.W + ix) * a.C + half * 16) ^ xm;
-        *reinterpret_cast<v4i*>(tile + pix * PITCH + half * 16) = v;
+        const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && static_cast<unsigned>(ix) < static_cast<unsigned>(a.W);
+        const uint8_t* src = ok ? xn + (static_cast<long long>(iy) * a.W + ix) * a.C + half * 16 : a.pad16;
+        st[k] = *reinterpret_cast<const v4i*>(src);
+    }
+#pragma unroll
+    for (int k = 0; k < NST; ++k)
+    {
+        const int i = tid + k * 256;
+        if (i < HR * HC * 2) *reinterpret_cast<v4i*>(tile + (i >> 1) * PITCH + (i & 1) * 16) = st[k] ^ xm;
     }
 
     // ---- per-thread constants ---------------------------------------------------------------------------------
