@@ -81,18 +81,11 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
     v16i acc[TC];
 
     auto load_chunk = [&](v4i (&buf)[KS], int t, int ch) {
-        const int row = t * 32 + frag_row;
-        if (row < a.M)
-        {
-            const uint8_t* p = a.x + static_cast<long long>(row) * a.K + ch * (32 * KS) + frag_k;
+        // rows past the end re-read the last row (their results are never stored): no load depends on a branch
+        const int row = min(t * 32 + frag_row, a.M - 1);
+        const uint8_t* p = a.x + static_cast<long long>(row) * a.K + ch * (32 * KS) + frag_k;
 #pragma unroll
-            for (int ks = 0; ks < KS; ++ks) buf[ks] = *reinterpret_cast<const v4i*>(p + ks * 32);
-        }
-        else
-        {
-#pragma unroll
-            for (int ks = 0; ks < KS; ++ks) buf[ks] = v4i{0, 0, 0, 0};
-        }
+        for (int ks = 0; ks < KS; ++ks) buf[ks] = *reinterpret_cast<const v4i*>(p + ks * 32);
     };
 
     // FIRST: the chunk opens a tile; its first MFMA takes a zero C operand instead of cleared registers
