@@ -283,6 +283,12 @@ int mi355x_event_record(mi355x_event_t event, mi355x_stream_t stream)
     return 0;
 }
 
+int mi355x_stream_wait_event(mi355x_stream_t stream, mi355x_event_t event)
+{
+    MI355X_HIP(hipStreamWaitEvent(ToHip(stream), reinterpret_cast<hipEvent_t>(event), 0));
+    return 0;
+}
+
 int mi355x_event_synchronize(mi355x_event_t event)
 {
     MI355X_HIP(hipEventSynchronize(reinterpret_cast<hipEvent_t>(event)));

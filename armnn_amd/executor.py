@@ -35,11 +35,20 @@ class FusedPair:
 
 class DeviceNetwork:
     def __init__(self, net: Network, batch: int, algo_overrides: Optional[Dict[str, int]] = None, use_graph: bool = True,
-                 fuse: bool = False):
+                 fuse: bool = False, lanes: int = 1):
+        """lanes > 1 splits the batch into that many contiguous slices; each slice runs the whole network on a stream of
+        its own (the same plans, pointers offset to the slice), so one slice's kernels fill the ramp-up, tail and
+        launch gaps of the others. Results do not depend on the split: every image is computed independently."""
+        if lanes < 1 or batch % lanes != 0:
+            raise ValueError("lanes must divide the batch")
         self.net, self.batch = net, batch
+        self.lanes = lanes
         self.dev = shim.Device()
         self.lib = shim.load_library()
         self.stream = self.dev.stream()
+        self.side_streams = [self.dev.stream() for _ in range(lanes - 1)]
+        self.fork_event = self.dev.event() if lanes > 1 else None
+        self.join_events = [self.dev.event() for _ in range(lanes - 1)]
         self.buffers: Dict[str, shim.DeviceBuffer] = {}
         self.steps: List = []          # (layer, callable(stream))
         self._step_plans: List = []    # plan of each step (None for plan-less layers), parallel to self.steps
@@ -67,14 +76,14 @@ class DeviceNetwork:
                 plan = shim.Conv2dPlan(xin[0], l.weights, l.bias, yout, activation=l.act[0], act_a=l.act[1],
                                        act_b=l.act[2], algo=algo_overrides.get(l.name, shim.ALGO_AUTO), **p)
                 self.plans.append(plan)
-                self.steps.append((l, self._conv_step(plan, xb[0].ptr, yb.ptr)))
+                self.steps.append((l, self._conv_step(plan, xb[0].ptr, yb.ptr, xin[0].num_elements, yout.num_elements)))
                 self._step_plans.append(plan)
             elif l.op == "fc":
                 plan = shim.FullyConnectedPlan(xin[0], l.weights, l.bias, yout, transpose_weights=l.params["transpose_weights"],
                                                activation=l.act[0], act_a=l.act[1], act_b=l.act[2],
                                                algo=algo_overrides.get(l.name, shim.ALGO_AUTO))
                 self.plans.append(plan)
-                self.steps.append((l, self._conv_step(plan, xb[0].ptr, yb.ptr)))
+                self.steps.append((l, self._conv_step(plan, xb[0].ptr, yb.ptr, xin[0].num_elements, yout.num_elements)))
                 self._step_plans.append(plan)
             elif l.op == "pool":
                 _, h, w, c = xin[0].shape
@@ -83,7 +92,7 @@ class DeviceNetwork:
                 d = shim.Pool2dDesc(h, w, c, ho, wo, p["pool_w"], p["pool_h"], p["stride_x"], p["stride_y"], p["pad_left"],
                                     p["pad_right"], p["pad_top"], p["pad_bottom"], p["pool_type"], p["padding_method"],
                                     shim._quant(xin[0]), shim._quant(yout))
-                self.steps.append((l, self._pool_step(d, xb[0].ptr, yb.ptr)))
+                self.steps.append((l, self._pool_step(d, xb[0].ptr, yb.ptr, xin[0].num_elements, yout.num_elements)))
                 self._step_plans.append(None)
             elif l.op == "add":
                 q0, q1, qo = shim._quant(xin[0]), shim._quant(xin[1]), shim._quant(yout)
@@ -117,9 +126,11 @@ class DeviceNetwork:
                     plan_of[id(l)].fusable_with(plan_of[id(nxt)])):
                 pdw, ppw = plan_of[id(l)], plan_of[id(nxt)]
                 x, y = self.buffers[l.inputs[0]].ptr, self.buffers[nxt.output].ptr
+                nx, ny = net.info(l.inputs[0], self.batch).num_elements, net.info(nxt.output, self.batch).num_elements
                 batch = self.batch
                 fused.append((FusedPair(f"{l.name}+{nxt.name}", (l, nxt)),
-                              (lambda pdw, ppw, x, y: lambda s: pdw.run_fused(ppw, batch, x, y, s))(pdw, ppw, x, y)))
+                              (lambda pdw, ppw, x, y, nx, ny: lambda s, lane=0, lanes=1: pdw.run_fused(
+                                  ppw, batch // lanes, x + lane * (nx // lanes), y + lane * (ny // lanes), s))(pdw, ppw, x, y, nx, ny)))
                 k += 2
             else:
                 fused.append((l, fn))
@@ -127,39 +138,61 @@ class DeviceNetwork:
         self.steps = fused
 
     # each step keeps its ctypes structs alive through the closure
-    def _conv_step(self, plan, x, y):
+    # A step is callable(stream, lane=0, lanes=1): lane k of n works on images [k*batch/n, (k+1)*batch/n) of every buffer.
+    def _conv_step(self, plan, x, y, nx, ny):
         batch = self.batch
-        return lambda s: plan.run(batch, x, y, s)
+        return lambda s, lane=0, lanes=1: plan.run(batch // lanes, x + lane * (nx // lanes), y + lane * (ny // lanes), s)
 
-    def _pool_step(self, d, x, y):
+    def _pool_step(self, d, x, y, nx, ny):
         batch, lib = self.batch, self.lib
-        return lambda s: shim._chk(lib.mi355x_pool2d_run(C.byref(d), batch, x, y, s))
+        return lambda s, lane=0, lanes=1: shim._chk(lib.mi355x_pool2d_run(C.byref(d), batch // lanes, x + lane * (nx // lanes),
+                                                                          y + lane * (ny // lanes), s))
 
     def _add_step(self, n, q0, q1, qo, act, x0, x1, y):
         lib = self.lib
-        return lambda s: shim._chk(lib.mi355x_add_run(n, C.byref(q0), C.byref(q1), C.byref(qo), act[0], act[1], act[2], x0, x1, y, s))
+        return lambda s, lane=0, lanes=1: shim._chk(lib.mi355x_add_run(
+            n // lanes, C.byref(q0), C.byref(q1), C.byref(qo), act[0], act[1], act[2], x0 + lane * (n // lanes),
+            x1 + lane * (n // lanes), y + lane * (n // lanes), s))
 
     def _softmax_step(self, rows, cols, beta, qi, qo, x, y):
         lib = self.lib
-        return lambda s: shim._chk(lib.mi355x_softmax_run(rows, cols, beta, C.byref(qi), C.byref(qo), x, y, s))
+        return lambda s, lane=0, lanes=1: shim._chk(lib.mi355x_softmax_run(
+            rows // lanes, cols, beta, C.byref(qi), C.byref(qo), x + lane * (rows // lanes) * cols,
+            y + lane * (rows // lanes) * cols, s))
 
     # ---------------------------------------------------------------------------------------------------------
     def upload_input(self, x: QTensor):
         assert x.info.shape == self.net.info(self.net.input, self.batch).shape
         self.buffers[self.net.input].upload(x.data, self.stream)
 
+    def _enqueue_lanes(self):
+        """Every lane's chain of launches: lane 0 on self.stream, the others on streams forked from it and joined back."""
+        if self.lanes == 1:
+            for _, fn in self.steps:
+                fn(self.stream)
+            return
+        self.dev.event_record(self.fork_event, self.stream)
+        for side in self.side_streams:
+            self.dev.stream_wait_event(side, self.fork_event)
+        # lanes interleaved layer by layer, so launches next to each other in submission order can overlap
+        for _, fn in self.steps:
+            fn(self.stream, 0, self.lanes)
+            for k, side in enumerate(self.side_streams, start=1):
+                fn(side, k, self.lanes)
+        for k, side in enumerate(self.side_streams, start=1):
+            self.dev.event_record(self.join_events[k - 1], side)
+            self.dev.stream_wait_event(self.stream, self.join_events[k - 1])
+
     def enqueue(self):
         """One forward pass on self.stream (asynchronous)."""
         if self.use_graph:
             if self.graph is None:
                 self.dev.graph_begin(self.stream)
-                for _, fn in self.steps:
-                    fn(self.stream)
+                self._enqueue_lanes()
                 self.graph = self.dev.graph_end(self.stream)
             self.dev.graph_launch(self.graph, self.stream)
         else:
-            for _, fn in self.steps:
-                fn(self.stream)
+            self._enqueue_lanes()
 
     def synchronize(self):
         self.dev.stream_sync(self.stream)
@@ -176,15 +209,16 @@ class DeviceNetwork:
         return self.download()
 
     def time_layers(self, iters: int = 20, warmup: int = 3):
-        """Per-layer device time in ms (HIP events on the launch stream), eager launches."""
+        """Device time in ms of one launch of every step, as launched by enqueue() (lane 0's slice of the batch when
+        the network runs in lanes), alone on the launch stream, timed with HIP events on that stream."""
         e0, e1 = self.dev.event(), self.dev.event()
         out = []
         for l, fn in self.steps:
             for _ in range(warmup):
-                fn(self.stream)
+                fn(self.stream, 0, self.lanes)
             self.dev.event_record(e0, self.stream)
             for _ in range(iters):
-                fn(self.stream)
+                fn(self.stream, 0, self.lanes)
             self.dev.event_record(e1, self.stream)
             self.dev.event_sync(e1)
             out.append((l, self.dev.elapsed_ms(e0, e1) / iters))
@@ -198,4 +232,6 @@ class DeviceNetwork:
             p.destroy()
         for b in set(self.buffers.values()):
             b.free()
+        for side in self.side_streams:
+            self.dev.stream_destroy(side)
         self.dev.stream_destroy(self.stream)

@@ -25,7 +25,7 @@ EXPORTS = [
     "mi355x_device_props", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc", "mi355x_host_free",
     "mi355x_memcpy_h2d", "mi355x_memcpy_d2h", "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_synchronize", "mi355x_device_synchronize", "mi355x_event_create",
-    "mi355x_event_destroy", "mi355x_event_record", "mi355x_event_synchronize", "mi355x_event_elapsed_ms",
+    "mi355x_event_destroy", "mi355x_event_record", "mi355x_stream_wait_event", "mi355x_event_synchronize", "mi355x_event_elapsed_ms",
     "mi355x_graph_capture_begin", "mi355x_graph_capture_end", "mi355x_graph_launch", "mi355x_graph_destroy",
     "mi355x_conv2d_create", "mi355x_conv2d_run", "mi355x_conv2d_destroy", "mi355x_conv2d_algo",
     "mi355x_conv2d_fusable", "mi355x_conv2d_run_fused",
@@ -96,6 +96,7 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
             "mi355x_memcpy_d2d": [V, V, C.c_size_t, V], "mi355x_fill_u8": [V, C.c_uint8, C.c_size_t, V],
             "mi355x_stream_create": [C.POINTER(V)], "mi355x_stream_destroy": [V], "mi355x_stream_synchronize": [V],
             "mi355x_event_create": [C.POINTER(V)], "mi355x_event_destroy": [V], "mi355x_event_record": [V, V],
+            "mi355x_stream_wait_event": [V, V],
             "mi355x_event_synchronize": [V], "mi355x_event_elapsed_ms": [V, V, C.POINTER(C.c_float)],
             "mi355x_graph_capture_begin": [V], "mi355x_graph_capture_end": [V, C.POINTER(V)],
             "mi355x_graph_launch": [V, V], "mi355x_graph_destroy": [V],
@@ -218,6 +219,9 @@ class Device:
 
     def event_record(self, e, stream=None):
         _chk(self.lib.mi355x_event_record(e, stream))
+
+    def stream_wait_event(self, stream, e):
+        _chk(self.lib.mi355x_stream_wait_event(stream, e))
 
     def event_sync(self, e):
         _chk(self.lib.mi355x_event_synchronize(e))

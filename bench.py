@@ -128,6 +128,8 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--fuse", action="store_true",
                     help="run depthwise + pointwise pairs as one kernel (same bytes; slower than two launches at present)")
+    ap.add_argument("--lanes", type=int, default=2,
+                    help="split the batch into this many slices, each running the network on a stream of its own")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
     ap.add_argument("--profile-pass", action="store_true",
                     help="for rocprofv3 --pmc: one 64 MiB calibration copy (1 B read + 1 B written per element), then ONE "
@@ -143,7 +145,7 @@ def main():
 
     net = nets.mobilenet_v1() if args.net == "mobilenet_v1" else nets.resnet50()
     batch = args.batch
-    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse)
+    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse, lanes=args.lanes)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev
 
@@ -156,10 +158,10 @@ def main():
         dev.stream_sync(dn.stream)
         shim._chk(dn.lib.mi355x_activation_run(n, C.byref(q), C.byref(q), shim.ACT_BOUNDED_RELU, 1000.0, -1000.0, a.ptr, b.ptr, dn.stream))
         for _, fn in dn.steps:
-            fn(dn.stream)
+            fn(dn.stream, 0, args.lanes)                 # lane 0's launch of every layer, as the timed region launches it
         dev.stream_sync(dn.stream)
         print(json.dumps({"dispatch_order": ["fill (setup)", f"calibration copy {n} B in + {n} B out"] + [l.name for l, _ in dn.steps],
-                          "batch": batch, "net": net.name}))
+                          "batch": batch, "launch_batch": batch // args.lanes, "net": net.name}))
         dn.close()
         return 0
 
@@ -175,16 +177,19 @@ def main():
     images_per_s = batch * args.steps / (t1 - t0)
 
     # ---- per-kernel timing on the launch stream, for the roofline object ------------------------------------
+    # (one launch = one layer over one lane's slice of the batch; in the timed region `lanes` such launches of a layer
+    # run side by side on their own streams)
+    launch_batch = batch // args.lanes
     per_layer = dn.time_layers(iters=20, warmup=3)
     rows = []
     for l, ms in per_layer:
-        kind, work = layer_work(net, l, batch)
+        kind, work = layer_work(net, l, launch_batch)
         peak = INT8_MFMA_PEAK_OPS if kind == "mfma" else HBM_PEAK_BYTES
         row = {"layer": l.name, "op": l.op, "ms": ms, "bound": kind, "work": work, "frac": work / (ms * 1e-3) / peak}
         if kind == "mfma":
             # the roof that binds a conv / FC layer depends on its arithmetic intensity: below the ridge
             # (peak ops / peak bytes = 625 ops/B) the HBM roof is the lower one
-            nbytes = float(algorithmic_bytes(net, l, batch))
+            nbytes = float(algorithmic_bytes(net, l, launch_batch))
             row["bytes"] = nbytes
             row["binding"] = "mfma" if work / nbytes >= RIDGE_OPS_PER_BYTE else "hbm"
         else:
@@ -198,7 +203,8 @@ def main():
             hbm = r["bytes"] / (r["ms"] * 1e-3) / HBM_PEAK_BYTES
             print(f"{r['layer']:>10s} {r['op']:>9s} {r['ms']*1e3:9.1f} us  {r['bound']:>4s} {100*r['frac']:6.2f}% of peak"
                   f"   binding roof {r['binding']:>4s}, {100*hbm:5.1f}% of HBM peak on algorithmic bytes", file=sys.stderr)
-        print(f"sum of kernels {total_ms:.3f} ms; graph step {ms_per_step:.3f} ms", file=sys.stderr)
+        print(f"launches of {launch_batch} images; sum of one lane's launches {total_ms:.3f} ms; step of {args.lanes} lane(s) "
+              f"{ms_per_step:.3f} ms", file=sys.stderr)
     if dom["binding"] == "mfma":
         roof = {"bound": "mfma", "achieved": dom["work"] / (dom["ms"] * 1e-3) / 1e12, "peak": INT8_MFMA_PEAK_OPS / 1e12,
                 "unit": "TOP/s"}
@@ -206,8 +212,9 @@ def main():
         roof = {"bound": "hbm", "achieved": dom["bytes"] / (dom["ms"] * 1e-3) / 1e9, "peak": HBM_PEAK_BYTES / 1e9,
                 "unit": "GB/s"}
     roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = MEASURED_HBM_TRAFFIC.get((net.name, batch), {}).get(dom["layer"])
-    roof["kernel"] = f"{dom['layer']} ({dom['op']}), {dom['ms']*1e3:.1f} us of {total_ms*1e3:.1f} us"
+    roof["traffic"] = MEASURED_HBM_TRAFFIC.get((net.name, launch_batch), {}).get(dom["layer"])
+    roof["kernel"] = (f"{dom['layer']} ({dom['op']}), one launch over {launch_batch} images: {dom['ms']*1e3:.1f} us of "
+                      f"{total_ms*1e3:.1f} us for all layers")
 
     def group(ops, peak):
         sel = [r for r in rows if r["op"] in ops]
@@ -230,7 +237,7 @@ def main():
         "dtype": "int8", "data": "synthetic",
         "config": {"workload": f"{net.name} int8 (QAsymm activations, per-channel QSymmS8 weights), batch {batch}, "
                                f"random-init, whole forward pass incl. avgpool/FC/softmax, input resident in HBM",
-                   "batch": batch, "graph_replay": not args.no_graph, "fused_depthwise_pointwise": args.fuse,
+                   "batch": batch, "graph_replay": not args.no_graph, "fused_depthwise_pointwise": args.fuse, "lanes": args.lanes,
                    "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12},
         "roofline": roof, "groups": groups,
     }

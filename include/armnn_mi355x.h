@@ -119,6 +119,9 @@ int  mi355x_device_synchronize(void);
 int  mi355x_event_create(mi355x_event_t* event);
 int  mi355x_event_destroy(mi355x_event_t event);
 int  mi355x_event_record(mi355x_event_t event, mi355x_stream_t stream);
+/* Work queued on `stream` after this call starts only when the work recorded by `event` is done. Inside a graph
+ * capture this is how a second stream joins the capture (fork) and how its work is joined back. */
+int  mi355x_stream_wait_event(mi355x_stream_t stream, mi355x_event_t event);
 int  mi355x_event_synchronize(mi355x_event_t event);
 int  mi355x_event_elapsed_ms(mi355x_event_t start, mi355x_event_t stop, float* ms);
 

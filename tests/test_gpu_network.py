@@ -46,6 +46,16 @@ def _layerwise(port, net, batch):
     dg.close()
     np.testing.assert_array_equal(g1.data, eager.data)
     np.testing.assert_array_equal(g2.data, eager.data)
+    # the batch split into slices that run side by side on forked streams (eager, then as a replayed graph)
+    for lanes in sorted({n for n in (2, 3, 4) if batch % n == 0}):
+        for use_graph in (False, True):
+            dl = DeviceNetwork(net, batch, use_graph=use_graph, lanes=lanes)
+            l1 = dl.run(x)
+            dl.enqueue()
+            l2 = dl.download()
+            dl.close()
+            np.testing.assert_array_equal(l1.data, eager.data)
+            np.testing.assert_array_equal(l2.data, eager.data)
     mx, exact = lsb_diff(eager.data, ref[net.output].data)
     top1 = float((eager.data.argmax(-1) == ref[net.output].data.argmax(-1)).mean())
     print(f"{net.name} b{batch} end-to-end: max|d|={mx} exact={exact:.6f} top1-agree={top1:.3f}", flush=True)
@@ -63,3 +73,8 @@ def test_mobilenet_v1_small_odd_resolution(port):
 
 def test_resnet50_batch1(port):
     _layerwise(port, nets.resnet50(resolution=96), 1)
+
+
+def test_resnet50_batch4_in_lanes(port):
+    # the residual adds and the pooling layers split by image like the convolutions
+    _layerwise(port, nets.resnet50(resolution=64), 4)
