@@ -216,6 +216,54 @@ __global__ __launch_bounds__(256) void Pool2dC4Kernel(PoolArgs p, QIn qin, Requa
                                                       QuantizeFastDev(res[2], rq), QuantizeFastDev(res[3], rq));
 }
 
+// The window is the whole image (global pooling): a block owns 256 channels of one image.  All threads fetch the
+// image's taps as dwords into LDS at once; then thread c walks channel c's taps in the reference's order (row by row),
+// so the fp32 sum is the reference's sum.  `taps` = H * W, at most kGlobalPoolMaxTaps.
+constexpr int kGlobalPoolMaxTaps = 196;
+__global__ __launch_bounds__(256) void GlobalPoolKernel(PoolArgs p, QIn qin, Requant rq, const uint8_t* __restrict__ x,
+                                                        uint8_t* __restrict__ y)
+{
+    __shared__ uint32_t raw[kGlobalPoolMaxTaps * 64];
+    const int taps = p.H * p.W;
+    const int groups = (p.C + 255) >> 8;
+    const long long n = blockIdx.x / groups;
+    const int c0 = static_cast<int>(blockIdx.x % groups) * 256;
+    const int quads = min(64, (p.C - c0) >> 2);
+    const uint8_t* xn = x + n * taps * p.C + c0;
+    for (int i = threadIdx.x; i < taps * 64; i += 256)
+    {
+        const int tap = i >> 6, q = i & 63;
+        if (q < quads) raw[i] = *reinterpret_cast<const uint32_t*>(xn + static_cast<long long>(tap) * p.C + q * 4);
+    }
+    __syncthreads();
+    const int c = threadIdx.x;
+    if (c0 + c >= p.C) return;
+    const uint8_t* col = reinterpret_cast<const uint8_t*>(raw) + c;
+    float res;
+    if (p.is_max)
+    {
+        int best = INT_MIN;
+        for (int t = 0; t < taps; ++t)
+        {
+            const int code = qin.is_u8 ? static_cast<int>(col[t * 256]) : static_cast<int>(static_cast<int8_t>(col[t * 256]));
+            best = max(best, code);
+        }
+        res = __fmul_rn(static_cast<float>(best - qin.offset), qin.scale);
+    }
+    else
+    {
+        float sum = 0.0f;
+#pragma unroll 7
+        for (int t = 0; t < taps; ++t)
+        {
+            const int code = qin.is_u8 ? static_cast<int>(col[t * 256]) : static_cast<int>(static_cast<int8_t>(col[t * 256]));
+            sum = __fadd_rn(sum, __fmul_rn(static_cast<float>(code - qin.offset), qin.scale));
+        }
+        res = __fdiv_rn(sum, static_cast<float>(taps));
+    }
+    y[n * p.C + c0 + c] = static_cast<uint8_t>(QuantizeFastDev(res, rq));
+}
+
 // 16 elements per thread, 16-byte loads and stores
 __global__ __launch_bounds__(256) void AddVec16Kernel(QIn q0, QIn q1, Requant rq, const v4u* __restrict__ x0,
                                                       const v4u* __restrict__ x1, v4u* __restrict__ y, size_t n16)
@@ -372,7 +420,12 @@ int mi355x_pool2d_run(const mi355x_pool2d_desc* d, uint32_t batch, const void* i
     Requant rq = MakeRequant(d->output, MI355X_ACT_NONE, 0.0f, 0.0f);
     const long long total = static_cast<long long>(batch) * p.Ho * p.Wo * p.C;
     const bool vec4 = (p.C % 4) == 0 && (reinterpret_cast<uintptr_t>(input_dev) & 3) == 0 && (reinterpret_cast<uintptr_t>(output_dev) & 3) == 0;
-    if (vec4 && p.pool_w <= 3 && p.pool_h <= 3)
+    const bool global = p.Ho == 1 && p.Wo == 1 && p.pad_top == 0 && p.pad_left == 0 && p.pool_h == p.H && p.pool_w == p.W &&
+                        p.H * p.W <= kGlobalPoolMaxTaps;
+    if (vec4 && global)
+        hipLaunchKernelGGL(GlobalPoolKernel, dim3(static_cast<unsigned>(batch * ((p.C + 255) / 256))), dim3(256), 0, ToHip(stream), p,
+                           MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev));
+    else if (vec4 && p.pool_w <= 3 && p.pool_h <= 3)
         hipLaunchKernelGGL(Pool2dC4Kernel<3>, dim3(static_cast<unsigned>((total / 4 + 255) / 256)), dim3(256), 0, ToHip(stream), p,
                            MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), total / 4);
     else if (vec4 && p.pool_w <= 8 && p.pool_h <= 8)

@@ -279,4 +279,71 @@ __global__ __launch_bounds__(256) void GemvKernel(GemvArgs a)
         }
 }
 
+// ---------------------------------------------------------------------------------------------------------------
+// A few dozen rows (the classifier of a network at its batch size): too many for the vector kernel above, too few to
+// fill LDS-tiled blocks.  A block owns 32 rows x 32 channels; its four waves split K (wave w takes the 32-byte
+// k-steps w, w+4, ...), each issues the loads of UN steps at once and feeds them to v_mfma_i32_32x32x32_i8, and the
+// four partial tiles meet in LDS, where wave g requantizes accumulator group g.  K must be a multiple of 16.
+template <int UN>
+__global__ __launch_bounds__(256) void SmallMGemmKernel(GemvArgs a)
+{
+    __shared__ int part[4][16][64];
+    const int lane = threadIdx.x & 63;
+    const int wave = threadIdx.x >> 6;
+    const int n0 = static_cast<int>(blockIdx.x) * 32;
+    const int m0 = static_cast<int>(blockIdx.y) * 32;
+    const int frag_row = lane & 31;
+    const int frag_k = (lane >> 5) * 16;
+    const int xm = static_cast<int>(a.xor_mask);
+    const int steps = (a.K + 31) >> 5;
+    // rows past the end re-read the last row (never stored); a lane's 16 bytes past K re-read the row's last 16 bytes
+    // against weights that are zero there: no load depends on a branch
+    const uint8_t* xp = a.x + static_cast<long long>(min(m0 + frag_row, a.M - 1)) * a.K;
+    const int8_t* wp = a.w + static_cast<long long>(n0 + frag_row) * a.w_stride + frag_k;
+    v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    for (int s0 = wave; s0 < steps; s0 += 4 * UN)
+    {
+        v4i xv[UN], wv[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+        {
+            const int s = min(s0 + 4 * u, steps - 1);
+            xv[u] = *reinterpret_cast<const v4i*>(xp + min(s * 32 + frag_k, a.K - 16));
+            wv[u] = *reinterpret_cast<const v4i*>(wp + s * 32);
+        }
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+        {
+            const v4i zero = {0, 0, 0, 0};
+            const v4i wu = (s0 + 4 * u < steps) ? wv[u] : zero;      // steps past the end (clamped above) add nothing
+            acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wu, xv[u] ^ xm, acc, 0, 0, 0);
+        }
+    }
+#pragma unroll
+    for (int i = 0; i < 16; ++i) part[wave][i][lane] = acc[i];
+    __syncthreads();
+    int v[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+        v[i] = part[0][4 * wave + i][lane] + part[1][4 * wave + i][lane] + part[2][4 * wave + i][lane] + part[3][4 * wave + i][lane];
+    // accumulator group g of the 32x32 tile: channels 8 g + 4 (lane / 32) + 0..3 of row lane % 32
+    const int c = n0 + 8 * wave + 4 * (lane >> 5);
+    const int row = m0 + frag_row;
+    const float4 fm = *reinterpret_cast<const float4*>(a.ct.p + 2 * a.ct.stride + c);
+    const float4 fb = *reinterpret_cast<const float4*>(a.ct.p + 5 * a.ct.stride + c);
+    const float4 th = *reinterpret_cast<const float4*>(a.ct.p + 6 * a.ct.stride + c);
+    const uint32_t out = Requant4Dev(v[0], v[1], v[2], v[3], fm, fb, th, a.ct, a.corr, c, a.rq);
+    if (row < a.M)
+    {
+        uint8_t* dst = a.y + static_cast<long long>(row) * a.N + c;
+        if ((a.N & 3) == 0 && c + 3 < a.N) *reinterpret_cast<uint32_t*>(dst) = out;
+        else
+        {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+                if (c + i < a.N) dst[i] = static_cast<uint8_t>(out >> (8 * i));
+        }
+    }
+}
+
 } // namespace mi355x

@@ -228,4 +228,9 @@ def small_fc_cases():
     c.append(make_fc_case("fc_u8_m2_k80_o10", 309, m=2, k=80, o=10, in_dtype=U8, in_offset=131, out_offset=7, act=RELU6))
     c.append(make_fc_case("fc_s8_m4_k2048_o203", 310, m=4, k=2048, o=203))
     c.append(make_fc_case("fc_s8_m1_k48_o5_not_transposed", 311, m=1, k=48, o=5, transpose=False, bias=False))
+    # a few dozen rows: 32x32 tiles with K split over the waves (5..64 rows, K % 16 == 0, K >= 128)
+    c.append(make_fc_case("fc_s8_m32_k1024_o1001", 312, m=32, k=1024, o=1001))
+    c.append(make_fc_case("fc_u8_m33_k144_o36", 313, m=33, k=144, o=36, in_dtype=U8, in_offset=120, out_offset=3, act=RELU6))
+    c.append(make_fc_case("fc_s8_m64_k2048_o100", 314, m=64, k=2048, o=100, per_axis=False))
+    c.append(make_fc_case("fc_s8_m5_k128_o7_no_bias", 315, m=5, k=128, o=7, bias=False))
     return c

@@ -23,6 +23,8 @@ POOLS = [
     ("max3x3s2_c64", (2, 23, 21, 64), cpuref.POOL_MAX, 3, 3, 2, 2, (1, 1, 1, 1)),
     ("max3x3s2_c5", (1, 11, 13, 5), cpuref.POOL_MAX, 3, 3, 2, 2, (1, 1, 1, 1)),
     ("avg7x7_global_c1024", (3, 7, 7, 1024), cpuref.POOL_AVERAGE, 7, 7, 1, 1, (0, 0, 0, 0)),
+    ("max14x14_global_c300", (2, 14, 14, 300), cpuref.POOL_MAX, 14, 14, 1, 1, (0, 0, 0, 0)),
+    ("avg3x5_global_c8", (5, 5, 3, 8), cpuref.POOL_AVERAGE, 3, 5, 2, 2, (0, 0, 0, 0)),
     ("avg3x2_pad_c12", (1, 9, 10, 12), cpuref.POOL_AVERAGE, 3, 2, 2, 1, (1, 1, 1, 0)),
     ("avg2x2_c8", (2, 8, 8, 8), cpuref.POOL_AVERAGE, 2, 2, 2, 2, (0, 0, 0, 0)),
     ("max9x9_big_window_c8", (1, 12, 12, 8), cpuref.POOL_MAX, 9, 9, 3, 3, (4, 4, 4, 4)),
