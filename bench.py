@@ -28,13 +28,45 @@ INT8_MFMA_PEAK_OPS = 5.0e15      # MI355X dense int8, ops/s
 HBM_PEAK_BYTES = 8.0e12          # MI355X HBM3E, B/s
 RIDGE_OPS_PER_BYTE = INT8_MFMA_PEAK_OPS / HBM_PEAK_BYTES
 
-# HBM bytes per launch (read + written) of each MobileNetV1 layer at batch 64, from two rocprofv3 --pmc passes
-# (FETCH_SIZE, then WRITE_SIZE) over `python3 bench.py --profile-pass --no-graph`, each scaled by what the same counter
+# HBM bytes per launch (read + written) of each MobileNetV1 layer, keyed by the images one launch covers (32 = one of
+# the two lanes of the default run), from two rocprofv3 --pmc passes (FETCH_SIZE, then WRITE_SIZE) over
+# `python3 bench.py --profile-pass --no-graph` (batch-64 entries: `--lanes 1`), each scaled by what the same counter
 # reads for the 64 MiB calibration copy of that pass (FETCH_SIZE counts 2 KiB units on this device: factor 1.999;
 # WRITE_SIZE 1 KiB units: factor 1.000).  Summary: profiles/mobilenet_v1_b64_hbm_traffic.md.
 MEASURED_HBM_TRAFFIC = {
+    ("mobilenet_v1_1.0_224", 32): {
+        "stem": 21553091,
+        "dw1": 25801624,
+        "pw1": 38745575,
+        "dw2": 32204273,
+        "pw2": 19641072,
+        "dw3": 25832073,
+        "pw3": 26122490,
+        "dw4": 16173845,
+        "pw4": 10208825,
+        "dw5": 13030988,
+        "pw5": 13554890,
+        "dw6": 8182875,
+        "pw6": 6195140,
+        "dw7": 6682452,
+        "pw7": 8948984,
+        "dw8": 6680533,
+        "pw8": 8944763,
+        "dw9": 6682708,
+        "pw9": 8946682,
+        "dw10": 6681045,
+        "pw10": 8946554,
+        "dw11": 6678870,
+        "pw11": 8946937,
+        "dw12": 4231529,
+        "pw12": 7120742,
+        "dw13": 3576246,
+        "pw13": 12342237,
+        "avgpool": 1687762,
+        "logits": 1437820,
+        "softmax": 127442
+    },
     ("mobilenet_v1_1.0_224", 64): {
-        "stem": 43143792,
         "dw1": 51482293,
         "pw1": 77282791,
         "dw2": 64298192,
@@ -61,8 +93,6 @@ MEASURED_HBM_TRAFFIC = {
         "pw12": 9543656,
         "dw13": 6807456,
         "pw13": 15567723,
-        "avgpool": 3581259,
-        "logits": 1801463,
         "softmax": 194497
     },
 }
