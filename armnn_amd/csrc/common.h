@@ -63,7 +63,6 @@ struct Options
 {
     int exact_division_epilogue = 0;   // 1: every output takes the fp32 division (no reciprocal fast path)
     int stem_dot4 = 0;                 // 1: small-Ci convolutions stay on the v_dot4 kernel (tests compare it with the MFMA one)
-    int igemm_depth = 3;               // register slots of the implicit-GEMM prefetch pipeline (2..4)
 };
 Options& GlobalOptions();
 

@@ -24,15 +24,7 @@ int SetError(int code, const char* fmt, ...)
 
 Options& GlobalOptions()
 {
-    static Options o = [] {
-        Options init;
-        if (const char* e = std::getenv("MI355X_IGEMM_DEPTH"))     // experiments
-        {
-            const int v = std::atoi(e);
-            if (v >= 2 && v <= 4) init.igemm_depth = v;
-        }
-        return init;
-    }();
+    static Options o;
     return o;
 }
 
@@ -106,12 +98,6 @@ int mi355x_set_option(const char* name, int value)
     if (!name) return SetError(MI355X_ERR_INVALID_ARGUMENT, "option name is null");
     if (std::strcmp(name, "exact_division_epilogue") == 0) { GlobalOptions().exact_division_epilogue = value != 0; return 0; }
     if (std::strcmp(name, "stem_dot4") == 0) { GlobalOptions().stem_dot4 = value != 0; return 0; }
-    if (std::strcmp(name, "igemm_depth") == 0)
-    {
-        if (value < 2 || value > 4) return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_depth must be 2, 3 or 4");
-        GlobalOptions().igemm_depth = value;
-        return 0;
-    }
     return SetError(MI355X_ERR_INVALID_ARGUMENT, "unknown option '%s'", name);
 }
 

@@ -95,7 +95,10 @@ int  mi355x_abi_version(void);
 /* Process-wide switches, read when a plan or a layer call is set up.
  *   "exact_division_epilogue" = 1: requantize every output with the fp32 division of armnn::Quantize
  *   (src/armnn/TypesUtils.cpp:40) instead of the reciprocal fast path that falls back to the division near
- *   rounding ties.  Both give identical bytes; the switch exists so that tests can prove it. */
+ *   rounding ties.  Both give identical bytes; the switch exists so that tests can prove it.
+ *   "stem_dot4" = 1: convolutions with at most 4 input channels run on the v_dot4 kernel instead of the MFMA one
+ *   (identical bytes; lets tests compare the two).
+ * Unknown names return MI355X_ERR_INVALID_ARGUMENT. */
 int  mi355x_set_option(const char* name, int value);
 int  mi355x_device_count(int* count);                 /* 0 devices is success with *count == 0 */
 int  mi355x_init(int device);                         /* select + warm up the device; idempotent */
