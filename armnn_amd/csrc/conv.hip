@@ -458,8 +458,19 @@ int LaunchPwKs(const mi355x_conv2d_s* p, long long M, const void* x, void* y, hi
     }
 }
 
+template <int BM, int BN, int WM, int WN, int D, int BK, bool UT>
+int LaunchIgemmT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream);
+
+// uniform-tap variant whenever a k-tile cannot straddle two filter taps
 template <int BM, int BN, int WM, int WN, int D, int BK>
 int LaunchIgemm(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    if ((p->geom.Ci % BK) == 0) return LaunchIgemmT<BM, BN, WM, WN, D, BK, true>(p, batch, x, y, stream);
+    return LaunchIgemmT<BM, BN, WM, WN, D, BK, false>(p, batch, x, y, stream);
+}
+
+template <int BM, int BN, int WM, int WN, int D, int BK, bool UT>
+int LaunchIgemmT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
 {
     const ConvGeom& g = p->geom;
     IgemmArgs a;
@@ -485,10 +496,10 @@ int LaunchIgemm(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y
     const int nblocks = a.tiles_m * a.tiles_n;
     const int grid = (nblocks + 7) / 8 * 8;
     constexpr int smem = IgemmSmemBytes<BM, BN, BK>();
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmKernel<BM, BN, WM, WN, D, BK>),
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmKernel<BM, BN, WM, WN, D, BK, UT>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);
-    hipLaunchKernelGGL((IgemmKernel<BM, BN, WM, WN, D, BK>), dim3(grid), dim3(256), smem, stream, a);
+    hipLaunchKernelGGL((IgemmKernel<BM, BN, WM, WN, D, BK, UT>), dim3(grid), dim3(256), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;
 }

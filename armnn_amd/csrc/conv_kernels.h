@@ -187,7 +187,10 @@ constexpr int IgemmSmemBytes()
 
 // D = register slots for k-tiles on their way from global memory to LDS: the loads of tile kt + D - 1 are issued while
 // tile kt is multiplied, so D - 1 tiles are in flight and an iteration no longer has to last a whole memory round trip.
-template <int BM, int BN, int WM, int WN, int D, int BK>
+// UT ("uniform tap"): Ci is a multiple of BK, so a k-tile never straddles two filter taps.  The walk over (ky, kx, ci) is
+// then the same for every thread (scalar registers), and a thread's address is a fixed per-row pointer plus a scalar
+// tap offset: no per-load multiplications.
+template <int BM, int BN, int WM, int WN, int D, int BK, bool UT>
 __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
 {
     static_assert(WM * WN == 4, "4 waves per block");
@@ -243,9 +246,14 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
         iy0[j] = oy * a.stride_y - a.pad_top;
         ix0[j] = ox * a.stride_x - a.pad_left;
         xrow[j] = a.x + static_cast<long long>(n) * a.H * a.W * a.Ci;
+        // UT: the chunk this thread would load for tap (0, 0), channel 0 (outside the tensor when the tap is padding;
+        // such an address is never dereferenced)
+        if constexpr (UT) xrow[j] += (static_cast<long long>(iy0[j]) * a.W + ix0[j]) * a.Ci + lc * 16;
     }
     // position of this thread's chunk inside K: (ky, kx, ci), advanced by BK every k-tile
     int ci, kx, ky;
+    if constexpr (UT) { ci = 0; kx = 0; ky = 0; }       // of the k-tile: identical in every thread
+    else
     {
         const int k0 = lc * 16;
         const int tap = k0 / a.Ci;
@@ -261,17 +269,20 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
     auto load_tile = [&](int kt, auto slot) {
         constexpr int SL = decltype(slot)::value;
         const bool kvalid = ky < a.Kh;
+        const int dy = ky * a.dil_y, dx = kx * a.dil_x;
+        const long long tap_off = (static_cast<long long>(dy) * a.W + dx) * a.Ci + ci;      // UT: scalar
 #pragma unroll
         for (int j = 0; j < RA; ++j)
         {
-            const int iy = iy0[j] + ky * a.dil_y;
-            const int ix = ix0[j] + kx * a.dil_x;
+            const int iy = iy0[j] + dy;
+            const int ix = ix0[j] + dx;
             const bool ok = mvalid[j] && kvalid && static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) &&
                             static_cast<unsigned>(ix) < static_cast<unsigned>(a.W);
             // A chunk outside the image loads 16 prepared padding bytes instead: every load is unconditional and its
             // value is used as it is, so the compiler has no branch to put it in (a load inside a divergent branch is
             // waited for on the spot, which would serialise the prefetch).
-            const uint8_t* src = ok ? xrow[j] + ((static_cast<long long>(iy) * a.W + ix) * a.Ci + ci) : a.pad16;
+            const uint8_t* in = UT ? xrow[j] + tap_off : xrow[j] + ((static_cast<long long>(iy) * a.W + ix) * a.Ci + ci);
+            const uint8_t* src = ok ? in : a.pad16;
             ra[SL][j] = *reinterpret_cast<const v4i*>(src);   // the xor waits until the value goes to LDS
         }
 #pragma unroll
