@@ -15,6 +15,7 @@
 #include "../mi355x/Mi355xTensorHandle.hpp"
 #include "../mi355x/Mi355xWorkloadFactory.hpp"
 
+#include <chrono>
 #include <backendsCommon/TensorHandleFactoryRegistry.hpp>
 #include <armnn/backends/WorkloadData.hpp>
 
@@ -434,26 +435,33 @@ TEST_CASE("runtime: FullyConnected, per-axis weights", "gpu")
 
 namespace
 {
-// stem conv -> dw -> pw -> dw s2 -> pw -> global average pool -> FC -> softmax, relu6 everywhere it belongs
+// stem conv -> (dw -> pw)* -> global average pool -> FC -> softmax, relu6 everywhere it belongs.
+// The default is two depthwise-separable blocks on a 32x32 image; `full` is MobileNetV1-1.0 (13 blocks, 1001 classes).
 struct MiniMobileNet
 {
-    std::vector<QLayer> layers;
+    std::vector<QLayer> layers;        // convolutions, then the FullyConnected layer last
     TensorInfo in, pooled, logits, probs;
-    MiniMobileNet(unsigned int batch, DataType t)
+    unsigned int classes = 10;
+    MiniMobileNet(unsigned int batch, DataType t, unsigned int resolution = 32, bool full = false)
     {
         const int zp = t == DataType::QAsymmU8 ? 0 : -128;
-        in = ActInfo({batch, 32, 32, 3}, t, 0.0078f, t == DataType::QAsymmU8 ? 128 : 0);
+        in = ActInfo({batch, resolution, resolution, 3}, t, 0.0078f, t == DataType::QAsymmU8 ? 128 : 0);
         layers.push_back(MakeConv(QLayer::Conv, in, 32, 3, 2, 0.0235f, zp, true, true, 201));
-        layers.push_back(MakeConv(QLayer::Depthwise, layers.back().out, 32, 3, 1, 0.0235f, zp, true, true, 202));
-        layers.push_back(MakeConv(QLayer::Conv, layers.back().out, 64, 1, 1, 0.0235f, zp, true, true, 203));
-        layers.push_back(MakeConv(QLayer::Depthwise, layers.back().out, 64, 3, 2, 0.0235f, zp, true, true, 204));
-        layers.push_back(MakeConv(QLayer::Conv, layers.back().out, 128, 1, 1, 0.0235f, zp, true, true, 205));
-        const TensorInfo& last = layers.back().out;
-        pooled = TensorInfo(TensorShape({batch, 1, 1, 128}), t, 0.0235f, zp);
-        (void)last;
-        layers.push_back(MakeFc(pooled, 10, 0.1f, t == DataType::QAsymmU8 ? 128 : 0, true, 206));
+        std::vector<std::pair<unsigned int, unsigned int>> blocks = {{1, 64}, {2, 128}};     // (depthwise stride, pointwise channels)
+        if (full) blocks = {{1, 64}, {2, 128}, {1, 128}, {2, 256}, {1, 256}, {2, 512}, {1, 512}, {1, 512}, {1, 512}, {1, 512}, {1, 512}, {2, 1024}, {1, 1024}};
+        uint64_t seed = 202;
+        for (const auto& blk : blocks)
+        {
+            const unsigned int c = layers.back().out.GetShape()[3];
+            layers.push_back(MakeConv(QLayer::Depthwise, layers.back().out, c, 3, blk.first, 0.0235f, zp, true, true, seed++));
+            layers.push_back(MakeConv(QLayer::Conv, layers.back().out, blk.second, 1, 1, 0.0235f, zp, true, true, seed++));
+        }
+        const unsigned int channels = layers.back().out.GetShape()[3];
+        classes = full ? 1001 : 10;
+        pooled = TensorInfo(TensorShape({batch, 1, 1, channels}), t, 0.0235f, zp);
+        layers.push_back(MakeFc(pooled, classes, 0.1f, t == DataType::QAsymmU8 ? 128 : 0, true, seed++));
         logits = layers.back().out;
-        probs = TensorInfo(TensorShape({batch, 10}), t, 1.0f / 256.0f, zp);
+        probs = TensorInfo(TensorShape({batch, classes}), t, 1.0f / 256.0f, zp);
     }
 
     INetworkPtr Build() const
@@ -462,17 +470,18 @@ struct MiniMobileNet
         IConnectableLayer* input = net->AddInputLayer(0, "input");
         input->GetOutputSlot(0).SetTensorInfo(in);
         IOutputSlot* slot = &input->GetOutputSlot(0);
-        for (size_t i = 0; i < 5; ++i) slot = &AddToNetwork(*net, *slot, layers[i], "l" + std::to_string(i));
+        const size_t nConv = layers.size() - 1;
+        for (size_t i = 0; i < nConv; ++i) slot = &AddToNetwork(*net, *slot, layers[i], "l" + std::to_string(i));
         Pooling2dDescriptor pd;
         pd.m_DataLayout = DataLayout::NHWC;
         pd.m_PoolType = PoolingAlgorithm::Average;
-        pd.m_PoolWidth = layers[4].out.GetShape()[2];
-        pd.m_PoolHeight = layers[4].out.GetShape()[1];
+        pd.m_PoolWidth = layers[nConv - 1].out.GetShape()[2];
+        pd.m_PoolHeight = layers[nConv - 1].out.GetShape()[1];
         pd.m_StrideX = pd.m_StrideY = 1;
         IConnectableLayer* pool = net->AddPooling2dLayer(pd, "avgpool");
         slot->Connect(pool->GetInputSlot(0));
         pool->GetOutputSlot(0).SetTensorInfo(pooled);
-        slot = &AddToNetwork(*net, pool->GetOutputSlot(0), layers[5], "logits");
+        slot = &AddToNetwork(*net, pool->GetOutputSlot(0), layers[nConv], "logits");
         IConnectableLayer* sm = net->AddSoftmaxLayer(SoftmaxDescriptor(), "softmax");
         slot->Connect(sm->GetInputSlot(0));
         sm->GetOutputSlot(0).SetTensorInfo(probs);
@@ -495,18 +504,19 @@ struct MiniMobileNet
             const QLayer& l = layers[i];
             mi355x_const_quant wq{MI355X_QSYMM_S8, 0, static_cast<uint32_t>(l.wScales.size()), l.wScales.data()};
             mi355x_const_quant bq{MI355X_SIGNED32, 0, static_cast<uint32_t>(l.bScales.size()), l.bScales.data()};
-            if (i == 5)
+            if (i + 1 == layers.size())
             {
+                const TensorInfo& last = layers[i - 1].out;
                 mi355x_pool2d_desc pd{};
-                pd.in_h = layers[4].out.GetShape()[1]; pd.in_w = layers[4].out.GetShape()[2]; pd.channels = 128; pd.out_h = pd.out_w = 1;
+                pd.in_h = last.GetShape()[1]; pd.in_w = last.GetShape()[2]; pd.channels = last.GetShape()[3]; pd.out_h = pd.out_w = 1;
                 pd.pool_w = pd.in_w; pd.pool_h = pd.in_h; pd.stride_x = pd.stride_y = 1;
                 pd.pool_type = 1; pd.padding_method = 1;
-                pd.input = mi355x::ToQuant(layers[4].out); pd.output = mi355x::ToQuant(pooled);
+                pd.input = mi355x::ToQuant(last); pd.output = mi355x::ToQuant(pooled);
                 void* next = alloc(pooled.GetNumBytes());
                 check(mi355x_pool2d_run(&pd, batch, cur, next, nullptr), "pool");
                 cur = next;
                 mi355x_fc_desc fd{};
-                fd.k = 128; fd.out_features = 10; fd.transpose_weights = 1; fd.bias_enabled = 1;
+                fd.k = last.GetShape()[3]; fd.out_features = classes; fd.transpose_weights = 1; fd.bias_enabled = 1;
                 fd.input = mi355x::ToQuant(l.in); fd.output = mi355x::ToQuant(l.out);
                 mi355x_fc_t plan = nullptr;
                 check(mi355x_fc_create(&fd, l.weights.data(), &wq, l.bias.data(), &bq, &plan), "fc_create");
@@ -535,7 +545,7 @@ struct MiniMobileNet
         }
         const mi355x_quant qi = mi355x::ToQuant(logits), qo = mi355x::ToQuant(probs);
         void* sm = alloc(probs.GetNumBytes());
-        check(mi355x_softmax_run(batch, 10, 1.0f, &qi, &qo, cur, sm, nullptr), "softmax");
+        check(mi355x_softmax_run(batch, classes, 1.0f, &qi, &qo, cur, sm, nullptr), "softmax");
         std::vector<uint8_t> out(probs.GetNumBytes());
         check(mi355x_memcpy_d2h(out.data(), sm, out.size(), nullptr), "d2h");
         check(mi355x_device_synchronize(), "sync");
@@ -570,6 +580,37 @@ TEST_CASE("runtime: a small MobileNet gives the bytes of the same C-ABI calls ma
             CHECK(std::abs(sum - 256) <= 10);
         }
     }
+}
+
+TEST_CASE("runtime: MobileNetV1-224 batch 64 through EnqueueWorkload equals the C-ABI calls; host-to-host images/s printed", "gpu")
+{
+    MiniMobileNet m(64, DataType::QAsymmS8, 224, true);
+    IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+    INetworkPtr net = m.Build();
+    IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, rt->GetDeviceSpec());
+    CHECK(CountLayers(opt->GetGraph(), LayerType::Activation) == 0);
+    CHECK(CountLayers(opt->GetGraph(), LayerType::MemCopy) == 0);
+    NetworkId id = -1;
+    std::string err;
+    REQUIRE(rt->LoadNetwork(id, std::move(opt), err) == Status::Success);
+    const std::vector<uint8_t> input = RandomActivations(m.in, 78);
+    std::vector<uint8_t> got(m.probs.GetNumBytes());
+    TensorInfo constIn = m.in;
+    constIn.SetConstant(true);
+    InputTensors ins{{0, ConstTensor(constIn, input.data())}};
+    OutputTensors outs{{0, Tensor(m.probs, got.data())}};
+    for (int i = 0; i < 3; ++i) REQUIRE(rt->EnqueueWorkload(id, ins, outs) == Status::Success);      // plans are built on the first call
+    const int steps = 20;
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int i = 0; i < steps; ++i) REQUIRE(rt->EnqueueWorkload(id, ins, outs) == Status::Success);
+    const double sec = std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count();
+    std::printf("    EnqueueWorkload, pageable host buffers in and out (9.6 MB + 64 KB per call): %.3f ms per batch of 64 = %.0f images/s\n",
+                1e3 * sec / steps, 64.0 * steps / sec);
+    rt->UnloadNetwork(id);
+    const std::vector<uint8_t> want = m.RunDirect(input);
+    const Diff d = Compare(got, want, DataType::QAsymmS8);
+    std::printf("    %zu outputs, %zu differ from the one-by-one C-ABI calls\n", d.n, d.mismatches);
+    CHECK(d.mismatches == 0);
 }
 
 TEST_CASE("runtime: intermediate tensors share an arena smaller than their sum", "gpu")
