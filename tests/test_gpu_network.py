@@ -4,7 +4,7 @@ import pytest
 
 from armnn_amd import nets, shim
 from armnn_amd.executor import DeviceNetwork
-from armnn_amd.tensor import numpy_dtype
+from armnn_amd.tensor import QTensor, numpy_dtype
 from oracle import netref
 from tests.helpers import lsb_diff
 
@@ -78,3 +78,28 @@ def test_resnet50_batch1(port):
 def test_resnet50_batch4_in_lanes(port):
     # the residual adds and the pooling layers split by image like the convolutions
     _layerwise(port, nets.resnet50(resolution=64), 4)
+
+
+def _rows_equal_small_batch_runs(net, batch, picks, lanes):
+    """Full-size property: image i of a large batch gives the bytes it gives in a batch of two (images are independent,
+    whatever tiles, lanes or kernels the batch size selects); the batch of two is what the layerwise tests tie to the
+    CPU checker."""
+    x = nets.synthetic_input(net, batch)
+    big = DeviceNetwork(net, batch, use_graph=True, lanes=lanes)
+    y = big.run(x)
+    big.close()
+    small = DeviceNetwork(net, 2, use_graph=False)
+    for i in picks:
+        xi = QTensor(net.info(net.input, 2), np.ascontiguousarray(x.data[i:i + 2]))
+        yi = small.run(xi)
+        np.testing.assert_array_equal(yi.data, y.data[i:i + 2], err_msg=f"{net.name} images {i},{i + 1} of {batch}")
+    small.close()
+    assert y.data.max() > y.data.min()                    # not one constant value
+
+
+def test_mobilenet_v1_batch64_rows_equal_batch2_runs():
+    _rows_equal_small_batch_runs(nets.mobilenet_v1(), 64, (0, 31, 62), lanes=2)
+
+
+def test_resnet50_batch32_rows_equal_batch2_runs():
+    _rows_equal_small_batch_runs(nets.resnet50(), 32, (0, 15, 30), lanes=2)
