@@ -271,6 +271,9 @@ def main():
                    "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12},
         "roofline": roof, "groups": groups,
     }
+    # what the device itself delivers on register-only MFMA chains and on a plain copy, next to the published peaks
+    from armnn_amd import peaks
+    line["measured_peaks"] = peaks.measure()
     if not args.no_cpu_baseline:
         line["cpu_baseline"] = cpu_baseline(net)
     dn.close()
