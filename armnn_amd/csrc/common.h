@@ -62,6 +62,7 @@ Requant MakeRequant(const mi355x_quant& out, int32_t activation, float a, float 
 struct Options
 {
     int exact_division_epilogue = 0;   // 1: every output takes the fp32 division (no reciprocal fast path)
+    int igemm_tile = 0;                // 0: automatic; 64, 96 (128x64) or 128: every MFMA plan created meanwhile uses that implicit-GEMM tile
     int stem_dot4 = 0;                 // 1: small-Ci convolutions stay on the v_dot4 kernel (tests compare it with the MFMA one)
 };
 Options& GlobalOptions();

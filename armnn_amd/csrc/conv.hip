@@ -32,10 +32,11 @@ struct mi355x_conv2d_s
     float*   chan     = nullptr;   // [5][Co_pad] per-channel requantization constants (rows: see ChanTab)
     int32_t* corr     = nullptr;   // [Co_pad]  -zx' * sum_k w[c][k]
     int K = 0, K_pad = 0, Co_pad = 0;
+    int pw_blocks_per_cu = 1, pw_n_cu = 256;     // weight-stationary kernel: blocks a CU holds at once, CUs of the device
     std::vector<float> chan_host;  // host copy, completed with the corr-folded rows once corr is known
     int pw_bn = 0, pw_ks = 0;      // pointwise GEMM kernel configuration (0: not applicable)
     bool bk128 = false;            // implicit GEMM walks K in 128-byte tiles
-    int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 128: force (MI355X_IGEMM_TILE, for experiments)
+    int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 96 (= 128x64) / 128: the "igemm_tile" option at plan creation
     uint32_t xor_mask = 0, pad_word = 0;
     std::string info;
 
@@ -63,6 +64,7 @@ namespace
 
 void FoldCorrIntoTable(mi355x_conv2d_s* p, const std::vector<int32_t>& corr, int Co);
 void ChoosePointwiseConfig(mi355x_conv2d_s* p);
+int PreparePointwise(mi355x_conv2d_s* p);
 
 int Upload(void** dst, const void* src, size_t bytes)
 {
@@ -239,10 +241,11 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             const std::vector<uint8_t> padbytes(16, static_cast<uint8_t>((zb ^ (g.in_u8 ? 0x80u : 0u)) & 0xffu));
             if (int rc = Upload(reinterpret_cast<void**>(&p->pad16), padbytes.data(), padbytes.size())) return rc;
         }
-        if (const char* t = std::getenv("MI355X_IGEMM_TILE")) p->tile_override = std::atoi(t);
+        p->tile_override = GlobalOptions().igemm_tile;
         FoldCorrIntoTable(p, corr, Co);
         ChoosePointwiseConfig(p);
-        if (p->tile_override != 0) p->pw_bn = 0;     // experiments: force the LDS-tiled implicit GEMM
+        if (p->tile_override != 0) p->pw_bn = 0;     // a forced tile also forces the LDS-tiled implicit GEMM
+        if (int rc = PreparePointwise(p)) return rc;
         char buf[128];
         if (p->pw_bn)
             snprintf(buf, sizeof(buf), "pointwise_gemm_mfma_i8_32x32x32 weight-stationary slab %dxK=%d, chunk %d k-steps", p->pw_bn, p->K, p->pw_ks);
@@ -403,6 +406,42 @@ void ChoosePointwiseConfig(mi355x_conv2d_s* p)
     p->pw_ks = (steps % 8) == 0 ? 8 : (steps % 4) == 0 ? 4 : (steps % 2) == 0 ? 2 : 1;
 }
 
+// Plan-time set-up of the weight-stationary kernel: allow its LDS slab and ask how many blocks a CU holds at once
+// (registers and LDS), so that a launch can size its grid to exactly one resident wave of blocks.
+template <int BN, int KS>
+int PreparePw(mi355x_conv2d_s* p)
+{
+    auto kernel = PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2)>;
+    MI355X_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
+    int per_cu = 1, dev = 0, n_cu = 256;
+    MI355X_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, PwSmemBytes<BN>(p->geom.Ci)));
+    MI355X_HIP(hipGetDevice(&dev));
+    MI355X_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
+    p->pw_blocks_per_cu = std::max(1, per_cu);
+    p->pw_n_cu = std::max(1, n_cu);
+    return 0;
+}
+
+template <int BN>
+int PreparePwKs(mi355x_conv2d_s* p)
+{
+    switch (p->pw_ks)
+    {
+    case 8: return PreparePw<BN, 8>(p);
+    case 4: return PreparePw<BN, 4>(p);
+    case 2: return PreparePw<BN, 2>(p);
+    default: return PreparePw<BN, 1>(p);
+    }
+}
+
+int PreparePointwise(mi355x_conv2d_s* p)
+{
+    if (p->pw_bn == 128) return PreparePwKs<128>(p);
+    if (p->pw_bn == 64) return PreparePwKs<64>(p);
+    if (p->pw_bn == 32) return PreparePwKs<32>(p);
+    return 0;
+}
+
 template <int BN, int KS>
 int LaunchPw(const mi355x_conv2d_s* p, long long M, const void* x, void* y, hipStream_t stream)
 {
@@ -422,18 +461,7 @@ int LaunchPw(const mi355x_conv2d_s* p, long long M, const void* x, void* y, hipS
     a.rq = p->rq;
     const int smem = PwSmemBytes<BN>(g.Ci);
     auto kernel = PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2)>;
-    // one residency query per instantiation and K: how many blocks a CU holds at once (registers and LDS)
-    static int cached_k = -1, cached_per_cu = 1, n_cu = 256;
-    if (cached_k != g.Ci)
-    {
-        MI355X_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
-        int per_cu = 1, dev = 0;
-        MI355X_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, smem));
-        MI355X_HIP(hipGetDevice(&dev));
-        MI355X_HIP(hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev));
-        cached_per_cu = std::max(1, per_cu);
-        cached_k = g.Ci;
-    }
+    const int n_cu = p->pw_n_cu, cached_per_cu = p->pw_blocks_per_cu;      // queried once, when the plan was built
     // exactly one resident wave of blocks: every block walks its share of the row tiles
     const long long groups = ((M + 31) / 32 + 3) / 4;
     long long gm = (static_cast<long long>(n_cu) * cached_per_cu) / a.n_slabs;

@@ -98,7 +98,9 @@ int  mi355x_abi_version(void);
  *   rounding ties.  Both give identical bytes; the switch exists so that tests can prove it.
  *   "stem_dot4" = 1: convolutions with at most 4 input channels run on the v_dot4 kernel instead of the MFMA one
  *   (identical bytes; lets tests compare the two).
- * Unknown names return MI355X_ERR_INVALID_ARGUMENT. */
+ *   "igemm_tile" = 0 | 64 | 96 | 128: plans created while it is set run on the LDS-tiled implicit-GEMM kernel with
+ *   64x64, 128x64 or 128x128 tiles instead of the automatic choice (identical bytes; tests and tuning).
+ * Unknown names and values outside these return MI355X_ERR_INVALID_ARGUMENT. */
 int  mi355x_set_option(const char* name, int value);
 int  mi355x_device_count(int* count);                 /* 0 devices is success with *count == 0 */
 int  mi355x_init(int device);                         /* select + warm up the device; idempotent */

@@ -132,6 +132,28 @@ def test_stem_mfma_equals_stem_dot4():
         np.testing.assert_array_equal(mfma.data, dot4.data)
 
 
+def test_every_igemm_tiling_gives_the_same_bytes():
+    """64x64, 128x64 and 128x128 tiles, 64- and 128-byte k-tiles, uniform-tap and per-thread tap walks: the automatic
+    choice depends on the problem size, so every variant is forced on each case and compared with the direct kernel."""
+    cs = [cases.make_conv_case("tile_3x3_c64", 601, n=2, h=30, w=28, ci=64, co=96, act=cases.RELU6),           # BK 64, uniform taps
+          cases.make_conv_case("tile_3x3_c128_s2", 602, n=2, h=29, w=31, ci=128, co=64, stride=(2, 2)),         # BK 128, uniform taps
+          cases.make_conv_case("tile_3x3_c48", 603, n=1, h=33, w=17, ci=48, co=40, in_dtype=cases.U8, in_offset=119),   # taps straddle k-tiles
+          cases.make_conv_case("tile_1x1_c256", 604, n=3, h=14, w=14, ci=256, co=512, kh=1, kw=1),              # pointwise, K > 128
+          cases.make_conv_case("tile_1x1_c32", 605, n=2, h=20, w=20, ci=32, co=64, kh=1, kw=1)]                 # pointwise, K <= 128 (weight-stationary by default)
+    for c in cs:
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        for tile in (0, 64, 96, 128):
+            shim.set_option("igemm_tile", tile)
+            try:
+                got = _gpu_conv(c, shim.ALGO_MFMA)
+            finally:
+                shim.set_option("igemm_tile", 0)
+            print(f"{c.name} tile {tile}: {got.data.size} outputs", flush=True)
+            np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} tile {tile}")
+    with pytest.raises(shim.ShimError):
+        shim.set_option("igemm_tile", 100)
+
+
 def test_config_c1_full_size(port):
     """BASELINE config 1: 1x56x56x64 -> 64, 3x3 SAME, per-channel, ReLU6; expected code range [-128, -8]."""
     c = cases.make_conv_case("C1", 20250101, h=56, w=56, ci=64, co=64, act=cases.RELU6)
