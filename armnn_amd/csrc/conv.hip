@@ -5,6 +5,7 @@
 #include "dw_stem_kernels.h"
 #include "dwpw_kernel.h"
 #include "pw_gemm_kernel.h"
+#include "igemm_lds_kernel.h"
 
 #include <cmath>
 #include <cstdlib>
@@ -249,6 +250,8 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         char buf[128];
         if (p->pw_bn)
             snprintf(buf, sizeof(buf), "pointwise_gemm_mfma_i8_32x32x32 weight-stationary slab %dxK=%d, chunk %d k-steps", p->pw_bn, p->K, p->pw_ks);
+        else if (p->bk128 && (Ci % 128) == 0)
+            snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 global_load_lds tiles 64x64..256x256 x128 K=%d", p->K);
         else
             snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 tiles 128x128|128x64|64x64 x%d K=%d", p->bk128 ? 128 : 64, p->K);
         p->info = buf;
@@ -532,6 +535,53 @@ int LaunchIgemmT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* 
     return 0;
 }
 
+template <int BM, int BN, int WM, int WN, int ST, bool U8>
+int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    const ConvGeom& g = p->geom;
+    IgemmArgs a;
+    a.x = static_cast<const uint8_t*>(x);
+    a.pad16 = p->pad16;
+    a.w = p->w_mfma;
+    a.ct = ChanTab{p->chan, p->Co_pad};
+    a.corr = p->corr;
+    a.y = static_cast<uint8_t*>(y);
+    const long long M = static_cast<long long>(batch) * g.Ho * g.Wo;
+    if (M > 0x7fffffffll / 2) return SetError(MI355X_ERR_UNSUPPORTED, "too many output pixels for one launch (%lld)", M);
+    a.M = static_cast<int>(M);
+    a.H = g.H; a.W = g.W; a.Ci = g.Ci; a.Ho = g.Ho; a.Wo = g.Wo; a.Co = g.Co;
+    a.Kh = g.Kh; a.Kw = g.Kw;
+    a.pad_top = g.pad_top; a.pad_left = g.pad_left; a.stride_x = g.stride_x; a.stride_y = g.stride_y;
+    a.dil_x = g.dil_x; a.dil_y = g.dil_y;
+    a.K_pad = p->K_pad;
+    a.tiles_m = static_cast<int>((M + BM - 1) / BM);
+    a.tiles_n = (g.Co + BN - 1) / BN;
+    a.xor_mask = p->xor_mask;
+    a.pad_word = p->pad_word;
+    a.rq = p->rq;
+    const int nblocks = a.tiles_m * a.tiles_n;
+    const int grid = (nblocks + 7) / 8 * 8;
+    constexpr int smem = IgemmLdsSmemBytes<BM, BN, ST>();
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmLdsKernel<BM, BN, WM, WN, ST, U8>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    MI355X_HIP(attr);
+    hipLaunchKernelGGL((IgemmLdsKernel<BM, BN, WM, WN, ST, U8>), dim3(grid), dim3(64 * WM * WN), smem, stream, a);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+template <int BM, int BN, int WM, int WN>
+int LaunchIgemmLds(const mi355x_conv2d_s* p, int stages, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    const bool u8 = p->xor_mask != 0;
+    if constexpr (3 * (BM + BN) * 128 <= 160 * 1024)
+    {
+        if (stages == 3)
+            return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 3, true>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 3, false>(p, batch, x, y, stream);
+    }
+    return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 2, true>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 2, false>(p, batch, x, y, stream);
+}
+
 int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
 {
     if (!p) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
@@ -596,7 +646,19 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const long long big = ((M + 127) / 128) * ((g.Co + 127) / 128);
         // tile: 64x64 while the 128-wide tiling would leave CUs idle; k-tile: 128 bytes whenever K was padded to it
         const bool bk128 = p->bk128;
-        const int tile = p->tile_override ? p->tile_override : big < 400 ? 64 : 128;
+        // 256x256 tiles (16 waves) halve the operand traffic per output once they alone fill three quarters of the CUs
+        const long long huge = ((M + 255) / 256) * ((g.Co + 255) / 256);
+        const int tile = p->tile_override ? p->tile_override : big < 400 ? 64 : (huge >= 192 && g.Co >= 256) ? 512 : 128;
+        // channel counts that are multiples of 128: k-tiles go from global memory straight into LDS
+        const int lds_stages = GlobalOptions().igemm_lds;
+        if (lds_stages != 0 && bk128 && (g.Ci % 128) == 0)
+        {
+            if (tile == 64) return LaunchIgemmLds<64, 64, 2, 2>(p, lds_stages, batch, x, y, stream);
+            if (g.Co <= 64 || tile == 96) return LaunchIgemmLds<128, 64, 2, 2>(p, lds_stages, batch, x, y, stream);
+            if (tile == 256) return LaunchIgemmLds<256, 128, 4, 2>(p, lds_stages, batch, x, y, stream);
+            if (tile == 512) return LaunchIgemmLds<256, 256, 4, 4>(p, lds_stages, batch, x, y, stream);
+            return LaunchIgemmLds<128, 128, 2, 2>(p, lds_stages, batch, x, y, stream);
+        }
         if (tile == 64) return bk128 ? LaunchIgemm<64, 64, 2, 2, 2, 128>(p, batch, x, y, stream) : LaunchIgemm<64, 64, 2, 2, 2, 64>(p, batch, x, y, stream);
         if (g.Co <= 64 || tile == 96) return bk128 ? LaunchIgemm<128, 64, 2, 2, 2, 128>(p, batch, x, y, stream) : LaunchIgemm<128, 64, 2, 2, 2, 64>(p, batch, x, y, stream);
         return bk128 ? LaunchIgemm<128, 128, 2, 2, 2, 128>(p, batch, x, y, stream) : LaunchIgemm<128, 128, 2, 2, 2, 64>(p, batch, x, y, stream);

@@ -1,0 +1,252 @@
+// Implicit GEMM whose k-tiles travel from global memory straight into LDS (global_load_lds_dwordx4): no staging
+// registers, no ds_write, and the loads of the next tiles stay in flight across the block barrier.
+//
+//   * For convolutions whose channel count is a multiple of 128: a k-tile is 128 bytes of ONE filter tap, so the walk over
+//     (ky, kx, ci) is scalar and a lane's address is a fixed per-row pointer plus a scalar tap offset.
+//   * A wave's load instruction moves 8 rows x 128 bytes; lane l delivers its 16 bytes to LDS slot l of that 1 KB, so
+//     the LDS image of a tile is dense (row pitch 128 bytes).  To keep the MFMA fragment reads (32 rows x 16 bytes)
+//     spread over all banks, lane l fetches chunk (l & 7) ^ (l >> 3) of row l >> 3: chunk c of row r lives at slot
+//     c ^ (r & 7), and readers apply the same xor.
+//   * uint8 activations become int8 by xor 0x80 on the fragment registers (template U8), weights are int8 already.
+//   * ST stages of LDS; tile kt + ST - 1 is requested right after the barrier that retires tile kt - 1.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#include "common.h"
+#include "conv_kernels.h"
+#include "device_math.h"
+
+namespace mi355x
+{
+
+template <int BM, int BN, int ST>
+constexpr int IgemmLdsSmemBytes()
+{
+    constexpr int stages = ST * (BM + BN) * 128;
+    constexpr int out = BM * (BN + 16);
+    return stages > out ? stages : out;
+}
+
+// s_waitcnt immediate that waits for all but the `n` youngest vector-memory operations and for nothing else
+constexpr int VmcntImm(int n)
+{
+    return (n & 0xF) | ((n >> 4) << 14) | (0x7 << 4) | (0xF << 8);
+}
+
+// WM x WN waves per block (4, 8 or 16), each with a (BM / WM) x (BN / WN) tile of the block tile.
+template <int BM, int BN, int WM, int WN, int ST, bool U8>
+__global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
+{
+    static_assert(ST == 2 || ST == 3, "2 or 3 LDS stages");
+    constexpr int BK = 128;
+    constexpr int NW = WM * WN;                 // waves
+    constexpr int NT = 64 * NW;                 // threads
+    constexpr int WTM = BM / WM, WTN = BN / WN; // wave tile
+    static_assert(WTM % 32 == 0 && WTN % 32 == 0, "wave tiles are multiples of 32");
+    static_assert(BM % (8 * NW) == 0 && BN % (8 * NW) == 0, "every wave loads whole 8-row groups");
+    constexpr int RA = BM / (8 * NW);           // load instructions per wave and k-tile: activations (8 rows each)
+    constexpr int RB = BN / (8 * NW);           //                                         weights
+    constexpr int TP = WTM / 32, TC = WTN / 32;
+    constexpr int STAGE = (BM + BN) * BK;
+    constexpr int LDO = BN + 16;
+    typedef __attribute__((address_space(3))) void* LdsPtr;
+    typedef const __attribute__((address_space(1))) void* GlobalPtr;
+
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];   // IgemmLdsSmemBytes<BM, BN, ST>()
+
+    const int nblocks = a.tiles_m * a.tiles_n;
+    const int per_xcd = (nblocks + 7) >> 3;
+    const int tile = static_cast<int>(blockIdx.x & 7) * per_xcd + static_cast<int>(blockIdx.x >> 3);
+    if (tile >= nblocks) return;
+    const int tn = tile % a.tiles_n;
+    const int tm = tile / a.tiles_n;
+
+    const int tid = threadIdx.x;
+    const int lane = tid & 63;
+    const int wave = tid >> 6;
+    const int wm = wave / WN, wn = wave % WN;
+
+    // ---- what this lane fetches: row (lane >> 3) of each 8-row group, 16-byte chunk (lane & 7) ^ (lane >> 3) ------
+    const int lrow = lane >> 3;
+    const int lchunk = (lane & 7) ^ lrow;
+    const uint8_t* xrow[RA];
+    int iy0[RA], ix0[RA];
+    bool mvalid[RA];
+#pragma unroll
+    for (int j = 0; j < RA; ++j)
+    {
+        const int m = tm * BM + wave * (BM / NW) + j * 8 + lrow;
+        mvalid[j] = m < a.M;
+        const int mm = mvalid[j] ? m : 0;
+        const int ox = mm % a.Wo;
+        const int t = mm / a.Wo;
+        const int oy = t % a.Ho;
+        const int n = t / a.Ho;
+        iy0[j] = oy * a.stride_y - a.pad_top;
+        ix0[j] = ox * a.stride_x - a.pad_left;
+        // the chunk this lane would fetch for tap (0, 0), channel 0 (outside the tensor when that tap is padding; such
+        // an address is never dereferenced)
+        xrow[j] = a.x + static_cast<long long>(n) * a.H * a.W * a.Ci + (static_cast<long long>(iy0[j]) * a.W + ix0[j]) * a.Ci + lchunk * 16;
+    }
+    const int8_t* wrow = a.w + static_cast<long long>(tn * BN + wave * (BN / NW) + lrow) * a.K_pad + lchunk * 16;
+    int ci = 0, kx = 0, ky = 0;                  // tap walk, identical in every thread
+
+    auto load_tile = [&](int kt, int stage) {
+        uint8_t* As = smem + stage * STAGE + wave * (BM / NW) * BK;
+        uint8_t* Bs = smem + stage * STAGE + BM * BK + wave * (BN / NW) * BK;
+        const int dy = ky * a.dil_y, dx = kx * a.dil_x;
+        const long long tap_off = (static_cast<long long>(dy) * a.W + dx) * a.Ci + ci;
+#pragma unroll
+        for (int j = 0; j < RA; ++j)
+        {
+            const int iy = iy0[j] + dy;
+            const int ix = ix0[j] + dx;
+            const bool ok = mvalid[j] && static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && static_cast<unsigned>(ix) < static_cast<unsigned>(a.W);
+            // padding and rows past the end fetch 16 prepared bytes instead: every lane always delivers its slot
+            const uint8_t* src = ok ? xrow[j] + tap_off : a.pad16;
+            __builtin_amdgcn_global_load_lds((GlobalPtr)(src), (LdsPtr)(As + j * 8 * BK), 16, 0, 0);
+        }
+#pragma unroll
+        for (int j = 0; j < RB; ++j)
+        {
+            const int8_t* src = wrow + static_cast<long long>(j * 8) * a.K_pad + kt * BK;
+            __builtin_amdgcn_global_load_lds((GlobalPtr)(src), (LdsPtr)(Bs + j * 8 * BK), 16, 0, 0);
+        }
+        ci += BK;
+        if (ci >= a.Ci)
+        {
+            ci = 0;
+            if (++kx == a.Kw) { kx = 0; ++ky; }
+        }
+    };
+
+    // ---- accumulators start at the zero-point correction ---------------------------------------------------------
+    const int lane_c = 4 * (lane >> 5);
+    const int cbase = tn * BN + wn * WTN;
+    v16i acc[TC][TP];
+#pragma unroll
+    for (int tc = 0; tc < TC; ++tc)
+    {
+        v16i init;
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const v4i c4 = *reinterpret_cast<const v4i*>(a.corr + cbase + tc * 32 + 8 * q + lane_c);
+            init[4 * q + 0] = c4[0];
+            init[4 * q + 1] = c4[1];
+            init[4 * q + 2] = c4[2];
+            init[4 * q + 3] = c4[3];
+        }
+#pragma unroll
+        for (int tp = 0; tp < TP; ++tp) acc[tc][tp] = init;
+    }
+
+    const int nk = a.K_pad / BK;
+    const int frag_row = lane & 31;
+    const int frag_half = lane >> 5;
+    const int xm = static_cast<int>(a.xor_mask);
+
+    auto compute = [&](int stage) {
+        const uint8_t* As = smem + stage * STAGE;
+        const uint8_t* Bs = As + BM * BK;
+#pragma unroll
+        for (int ks = 0; ks < BK / 32; ++ks)
+        {
+            // chunk ks*2 + half of row r sits at slot (chunk ^ (r & 7)); every fragment row here has r & 7 == frag_row & 7
+            const int slot = ((ks * 2 + frag_half) ^ (frag_row & 7)) * 16;
+            v4i fa[TP], fw[TC];
+#pragma unroll
+            for (int tp = 0; tp < TP; ++tp)
+            {
+                fa[tp] = *reinterpret_cast<const v4i*>(As + (wm * WTM + tp * 32 + frag_row) * BK + slot);
+                if (U8) fa[tp] ^= xm;
+            }
+#pragma unroll
+            for (int tc = 0; tc < TC; ++tc)
+                fw[tc] = *reinterpret_cast<const v4i*>(Bs + (wn * WTN + tc * 32 + frag_row) * BK + slot);
+#pragma unroll
+            for (int tc = 0; tc < TC; ++tc)
+#pragma unroll
+                for (int tp = 0; tp < TP; ++tp)
+                    acc[tc][tp] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[tc], fa[tp], acc[tc][tp], 0, 0, 0);
+        }
+    };
+
+    // ---- pipeline: ST - 1 tiles requested ahead ---------------------------------------------------------------------
+#pragma unroll
+    for (int s = 0; s < ST - 1; ++s)
+        if (s < nk) load_tile(s, s);
+    int stage = 0;
+    for (int kt = 0; kt < nk; ++kt)
+    {
+        // tile kt has landed when at most the younger requests are outstanding
+        if (ST == 3 && kt + 1 < nk) __builtin_amdgcn_s_waitcnt(VmcntImm(RA + RB));
+        else __builtin_amdgcn_s_waitcnt(VmcntImm(0));
+        __syncthreads();                         // every wave's part of tile kt is in LDS; tile kt - 1 is no longer read
+        if (kt + ST - 1 < nk)
+        {
+            int ls = stage + ST - 1;
+            if (ls >= ST) ls -= ST;
+            load_tile(kt + ST - 1, ls);
+        }
+        compute(stage);
+        if (++stage == ST) stage = 0;
+    }
+    __syncthreads();
+
+    // ---- epilogue: requantize, pack 4 channels per dword, stage the byte tile in LDS, coalesced write-out -----------
+    uint8_t* Os = smem;
+#pragma unroll
+    for (int tc = 0; tc < TC; ++tc)
+    {
+#pragma unroll
+        for (int q = 0; q < 4; ++q)
+        {
+            const int cl = wn * WTN + tc * 32 + 8 * q + lane_c;
+            const Fast4 f4 = LoadFast4(a.ct, tn * BN + cl);
+#pragma unroll
+            for (int tp = 0; tp < TP; ++tp)
+            {
+                const v16i& c = acc[tc][tp];
+                const uint32_t out = Requant4Dev(c[4 * q + 0], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], f4, a.ct, tn * BN + cl, a.rq);
+                const int pl = wm * WTM + tp * 32 + (lane & 31);
+                *reinterpret_cast<uint32_t*>(Os + pl * LDO + cl) = out;
+            }
+        }
+    }
+    __syncthreads();
+    constexpr int CHUNKS = BN / 16;
+    constexpr int ROWS_PER_PASS = NT / CHUNKS;
+    const int oc = tid % CHUNKS;
+    const int orow = tid / CHUNKS;
+    const int c0 = tn * BN + oc * 16;
+    if ((a.Co & 15) == 0)
+    {
+        if (c0 < a.Co)
+        {
+#pragma unroll
+            for (int r = orow; r < BM; r += ROWS_PER_PASS)
+            {
+                const int m = tm * BM + r;
+                if (m < a.M)
+                    *reinterpret_cast<v4i*>(a.y + static_cast<long long>(m) * a.Co + c0) = *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16);
+            }
+        }
+    }
+    else
+    {
+        for (int r = orow; r < BM; r += ROWS_PER_PASS)
+        {
+            const int m = tm * BM + r;
+            if (m >= a.M) continue;
+            for (int b = 0; b < 16; ++b)
+            {
+                const int c = c0 + b;
+                if (c < a.Co) a.y[static_cast<long long>(m) * a.Co + c] = Os[r * LDO + oc * 16 + b];
+            }
+        }
+    }
+}
+
+} // namespace mi355x

@@ -98,9 +98,16 @@ int mi355x_set_option(const char* name, int value)
     if (!name) return SetError(MI355X_ERR_INVALID_ARGUMENT, "option name is null");
     if (std::strcmp(name, "exact_division_epilogue") == 0) { GlobalOptions().exact_division_epilogue = value != 0; return 0; }
     if (std::strcmp(name, "stem_dot4") == 0) { GlobalOptions().stem_dot4 = value != 0; return 0; }
+    if (std::strcmp(name, "igemm_lds") == 0)
+    {
+        if (value != 0 && value != 2 && value != 3) return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_lds must be 0, 2 or 3");
+        GlobalOptions().igemm_lds = value;
+        return 0;
+    }
     if (std::strcmp(name, "igemm_tile") == 0)
     {
-        if (value != 0 && value != 64 && value != 96 && value != 128) return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_tile must be 0, 64, 96 or 128");
+        if (value != 0 && value != 64 && value != 96 && value != 128 && value != 256 && value != 512)
+            return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_tile must be 0, 64, 96, 128, 256 or 512");
         GlobalOptions().igemm_tile = value;
         return 0;
     }

@@ -46,7 +46,11 @@ def main(argv=None):
     ap.add_argument("--algo", type=int, default=0)
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE", help="mi355x_set_option before the plan is built")
     a = ap.parse_args(argv)
+    for item in a.opt:
+        name, value = item.split("=")
+        shim.set_option(name, int(value))
 
     dev = shim.Device()
     adt = DataType.QAsymmU8 if a.u8 else DataType.QAsymmS8

@@ -98,8 +98,11 @@ int  mi355x_abi_version(void);
  *   rounding ties.  Both give identical bytes; the switch exists so that tests can prove it.
  *   "stem_dot4" = 1: convolutions with at most 4 input channels run on the v_dot4 kernel instead of the MFMA one
  *   (identical bytes; lets tests compare the two).
- *   "igemm_tile" = 0 | 64 | 96 | 128: plans created while it is set run on the LDS-tiled implicit-GEMM kernel with
- *   64x64, 128x64 or 128x128 tiles instead of the automatic choice (identical bytes; tests and tuning).
+ *   "igemm_tile" = 0 | 64 | 96 | 128 | 256 | 512: plans created while it is set run on the LDS-tiled implicit-GEMM
+ *   kernel with 64x64, 128x64, 128x128, 256x128 or 256x256 tiles instead of the automatic choice (the two largest only
+ *   where the direct-to-LDS kernel applies; identical bytes; tests and tuning).
+ *   "igemm_lds" = 2 | 3 | 0: LDS stages of the implicit-GEMM kernel that loads its k-tiles from global memory straight
+ *   into LDS (input channels a multiple of 128); 0 selects the register-staged kernel instead (identical bytes).
  * Unknown names and values outside these return MI355X_ERR_INVALID_ARGUMENT. */
 int  mi355x_set_option(const char* name, int value);
 int  mi355x_device_count(int* count);                 /* 0 devices is success with *count == 0 */

@@ -140,16 +140,21 @@ def test_every_igemm_tiling_gives_the_same_bytes():
           cases.make_conv_case("tile_3x3_c48", 603, n=1, h=33, w=17, ci=48, co=40, in_dtype=cases.U8, in_offset=119),   # taps straddle k-tiles
           cases.make_conv_case("tile_1x1_c256", 604, n=3, h=14, w=14, ci=256, co=512, kh=1, kw=1),              # pointwise, K > 128
           cases.make_conv_case("tile_1x1_c32", 605, n=2, h=20, w=20, ci=32, co=64, kh=1, kw=1)]                 # pointwise, K <= 128 (weight-stationary by default)
+    cs.append(cases.make_conv_case("tile_3x3_c128_u8_dil2", 606, n=2, h=19, w=23, ci=128, co=192, dilation=(2, 2), in_dtype=cases.U8,
+                                   in_offset=131, out_offset=-100))                                            # direct-to-LDS, xor on fragments
     for c in cs:
         want = _gpu_conv(c, shim.ALGO_DIRECT)
-        for tile in (0, 64, 96, 128):
-            shim.set_option("igemm_tile", tile)
-            try:
-                got = _gpu_conv(c, shim.ALGO_MFMA)
-            finally:
-                shim.set_option("igemm_tile", 0)
-            print(f"{c.name} tile {tile}: {got.data.size} outputs", flush=True)
-            np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} tile {tile}")
+        for tile in (0, 64, 96, 128, 256, 512):
+            for lds in (0, 2, 3):              # register-staged kernel, direct-to-LDS kernel with 2 / 3 stages
+                shim.set_option("igemm_tile", tile)
+                shim.set_option("igemm_lds", lds)
+                try:
+                    got = _gpu_conv(c, shim.ALGO_MFMA)
+                finally:
+                    shim.set_option("igemm_tile", 0)
+                    shim.set_option("igemm_lds", 2)
+                print(f"{c.name} tile {tile} lds {lds}: {got.data.size} outputs", flush=True)
+                np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} tile {tile} lds {lds}")
     with pytest.raises(shim.ShimError):
         shim.set_option("igemm_tile", 100)
 
