@@ -4,9 +4,11 @@
 //   * For convolutions whose channel count is a multiple of 128: a k-tile is 128 bytes of ONE filter tap, so the walk over
 //     (ky, kx, ci) is scalar and a lane's address is a fixed per-row pointer plus a scalar tap offset.
 //   * A wave's load instruction moves 8 rows x 128 bytes; lane l delivers its 16 bytes to LDS slot l of that 1 KB, so
-//     the LDS image of a tile is dense (row pitch 128 bytes).  To keep the MFMA fragment reads (32 rows x 16 bytes)
-//     spread over all banks, lane l fetches chunk (l & 7) ^ (l >> 3) of row l >> 3: chunk c of row r lives at slot
-//     c ^ (r & 7), and readers apply the same xor.
+//     the LDS image of a tile is dense (row pitch 128 bytes = half of the 64 banks).  A ds_read_b128 serves 16 lanes
+//     per cycle; an MFMA fragment read takes the same chunk of 16 consecutive rows there, which must therefore sit in
+//     16 different 4-bank groups: chunk c of row r lives at slot c ^ ((r >> 1) & 7) (rows of equal parity share the
+//     bank half and get 8 different slots).  Lanes pick the global chunk that belongs in their slot; readers apply
+//     the same xor.
 //   * uint8 activations become int8 by xor 0x80 on the fragment registers (template U8), weights are int8 already.
 //   * ST stages of LDS; tile kt + ST - 1 is requested right after the barrier that retires tile kt - 1.
 #pragma once
@@ -67,9 +69,12 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
     const int wave = tid >> 6;
     const int wm = wave / WN, wn = wave % WN;
 
-    // ---- what this lane fetches: row (lane >> 3) of each 8-row group, 16-byte chunk (lane & 7) ^ (lane >> 3) ------
+    // ---- what this lane fetches: row (lane >> 3) of each 8-row group; the chunk whose slot is (lane & 7).  Row r of
+    // the tile is 8 * (group index) + lrow, and a wave's first row is a multiple of 16, so (r >> 1) & 7 is
+    // (lrow >> 1) + 4 * (group parity).
     const int lrow = lane >> 3;
-    const int lchunk = (lane & 7) ^ lrow;
+    const int lchunk_even = (lane & 7) ^ (lrow >> 1);            // groups j = 0, 2, ...
+    const int lchunk_odd = (lane & 7) ^ ((lrow >> 1) + 4);       // groups j = 1, 3, ...
     const uint8_t* xrow[RA];
     int iy0[RA], ix0[RA];
     bool mvalid[RA];
@@ -87,9 +92,11 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
         ix0[j] = ox * a.stride_x - a.pad_left;
         // the chunk this lane would fetch for tap (0, 0), channel 0 (outside the tensor when that tap is padding; such
         // an address is never dereferenced)
-        xrow[j] = a.x + static_cast<long long>(n) * a.H * a.W * a.Ci + (static_cast<long long>(iy0[j]) * a.W + ix0[j]) * a.Ci + lchunk * 16;
+        xrow[j] = a.x + static_cast<long long>(n) * a.H * a.W * a.Ci + (static_cast<long long>(iy0[j]) * a.W + ix0[j]) * a.Ci +
+                  ((j & 1) ? lchunk_odd : lchunk_even) * 16;
     }
-    const int8_t* wrow = a.w + static_cast<long long>(tn * BN + wave * (BN / NW) + lrow) * a.K_pad + lchunk * 16;
+    static_assert((BM / NW) % 16 == 0 && (BN / NW) % 16 == 0, "a wave's first row is a multiple of 16");
+    const int8_t* wrow = a.w + static_cast<long long>(tn * BN + wave * (BN / NW) + lrow) * a.K_pad;
     int ci = 0, kx = 0, ky = 0;                  // tap walk, identical in every thread
 
     auto load_tile = [&](int kt, int stage) {
@@ -110,7 +117,7 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
 #pragma unroll
         for (int j = 0; j < RB; ++j)
         {
-            const int8_t* src = wrow + static_cast<long long>(j * 8) * a.K_pad + kt * BK;
+            const int8_t* src = wrow + static_cast<long long>(j * 8) * a.K_pad + kt * BK + ((j & 1) ? lchunk_odd : lchunk_even) * 16;
             __builtin_amdgcn_global_load_lds((GlobalPtr)(src), (LdsPtr)(Bs + j * 8 * BK), 16, 0, 0);
         }
         ci += BK;
@@ -153,8 +160,8 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
 #pragma unroll
         for (int ks = 0; ks < BK / 32; ++ks)
         {
-            // chunk ks*2 + half of row r sits at slot (chunk ^ (r & 7)); every fragment row here has r & 7 == frag_row & 7
-            const int slot = ((ks * 2 + frag_half) ^ (frag_row & 7)) * 16;
+            // chunk ks*2 + half of row r sits at slot chunk ^ ((r >> 1) & 7); fragment rows start at multiples of 32
+            const int slot = ((ks * 2 + frag_half) ^ ((frag_row >> 1) & 7)) * 16;
             v4i fa[TP], fw[TC];
 #pragma unroll
             for (int tp = 0; tp < TP; ++tp)
