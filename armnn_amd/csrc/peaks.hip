@@ -1,5 +1,7 @@
-// Two micro-benchmarks that measure what this device delivers at its actual clocks, for reading roofline fractions:
+// Micro-benchmarks that measure what this device delivers at its actual clocks, for reading roofline fractions:
 //   * int8 MFMA issue rate: every wave runs independent v_mfma_i32_32x32x32_i8 chains on register operands only;
+//   * the same with the operands read from LDS every step (2 + 4 fragments per 8 MFMAs, as a GEMM wave tile does):
+//     the clock the device sustains with the matrix cores and LDS busy together is lower, and so is this rate;
 //   * HBM copy rate: 16-byte loads and stores over buffers far larger than the caches.
 // Measurement support for the benchmark scripts; not part of the inference ABI.
 #include <hip/hip_runtime.h>
@@ -32,6 +34,42 @@ __global__ __launch_bounds__(256) void MfmaPeakKernel(int iters, int* sink)
 }
 
 // four 16-byte loads in flight per thread, non-temporal both ways (the fastest of the variants tried on this device)
+// ops per wave and iteration: 8 MFMAs x 32*32*32 MACs x 2; 6 ds_read_b128 per iteration
+__global__ __launch_bounds__(256) void MfmaLdsFedKernel(int iters, int* sink)
+{
+    __shared__ __attribute__((aligned(16))) int lds[16384];
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    for (int i = threadIdx.x; i < 16384; i += 256) lds[i] = static_cast<int>(i * 2654435761u);
+    __syncthreads();
+    v16i c[2][4];
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j) c[i][j] = v16i{0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    const int base = wave * 4096 + lane * 4;
+    for (int it = 0; it < iters; ++it)
+    {
+        const int o = (it & 3) * 1024;
+        v4i fa[2], fb[4];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) fa[i] = *reinterpret_cast<const v4i*>(&lds[(base + o + 256 * i) & 16383]);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) fb[j] = *reinterpret_cast<const v4i*>(&lds[(base + o + 256 * (2 + j)) & 16383]);
+#pragma unroll
+        for (int i = 0; i < 2; ++i)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) c[i][j] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fa[i], fb[j], c[i][j], 0, 0, 0);
+    }
+    int t = 0;
+#pragma unroll
+    for (int i = 0; i < 2; ++i)
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+            for (int k = 0; k < 16; ++k) t += c[i][j][k];
+    if (t == 0x7fffffff) sink[0] = t;
+}
+
 __global__ __launch_bounds__(256) void CopyKernel(const v4i* __restrict__ src, v4i* __restrict__ dst, size_t n16)
 {
     size_t i = static_cast<size_t>(blockIdx.x) * 1024 + threadIdx.x;
@@ -99,6 +137,33 @@ int mi355x_peak_mfma_i8(int waves_per_simd, double* ops_per_s)
         float ms = 0.0f;
         if (hipEventSynchronize(ev.e1) != hipSuccess || hipEventElapsedTime(&ms, ev.e0, ev.e1) != hipSuccess || ms <= 0.0f) rc = 2;
         else *ops_per_s = static_cast<double>(grid.x) * 4.0 * iters * 4.0 * 65536.0 / (ms * 1e-3);
+    }
+    (void)hipFree(sink);
+    return rc;
+}
+
+// Dense int8 MFMA rate in ops/s when every operand fragment comes from LDS (two waves per SIMD).
+int mi355x_peak_mfma_i8_lds_fed(double* ops_per_s)
+{
+    if (!ops_per_s) return 1;
+    int dev = 0, n_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 2;
+    if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 2;
+    int* sink = nullptr;
+    if (hipMalloc(&sink, 64) != hipSuccess) return 2;
+    Events ev;
+    const int iters = 10000;
+    const dim3 grid(static_cast<unsigned>(n_cu * 2));
+    int rc = ev.ok ? 0 : 2;
+    if (rc == 0)
+    {
+        hipLaunchKernelGGL(MfmaLdsFedKernel, grid, dim3(256), 0, nullptr, 100, sink);
+        (void)hipEventRecord(ev.e0, nullptr);
+        hipLaunchKernelGGL(MfmaLdsFedKernel, grid, dim3(256), 0, nullptr, iters, sink);
+        (void)hipEventRecord(ev.e1, nullptr);
+        float ms = 0.0f;
+        if (hipEventSynchronize(ev.e1) != hipSuccess || hipEventElapsedTime(&ms, ev.e0, ev.e1) != hipSuccess || ms <= 0.0f) rc = 2;
+        else *ops_per_s = static_cast<double>(grid.x) * 4.0 * iters * 8.0 * 65536.0 / (ms * 1e-3);
     }
     (void)hipFree(sink);
     return rc;

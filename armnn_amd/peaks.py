@@ -25,6 +25,12 @@ def measure(copy_bytes: int = 1 << 30) -> dict:
             raise RuntimeError(f"mi355x_peak_mfma_i8 failed ({rc})")
         best = max(best, v.value)
     out["mfma_i8_TOPs"] = best / 1e12
+    lib.mi355x_peak_mfma_i8_lds_fed.argtypes = [C.POINTER(C.c_double)]
+    v = C.c_double()
+    rc = lib.mi355x_peak_mfma_i8_lds_fed(C.byref(v))
+    if rc != 0:
+        raise RuntimeError(f"mi355x_peak_mfma_i8_lds_fed failed ({rc})")
+    out["mfma_i8_lds_fed_TOPs"] = v.value / 1e12
     v = C.c_double()
     rc = lib.mi355x_peak_hbm_read(copy_bytes, C.byref(v))
     if rc != 0:
