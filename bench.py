@@ -35,36 +35,36 @@ RIDGE_OPS_PER_BYTE = INT8_MFMA_PEAK_OPS / HBM_PEAK_BYTES
 # WRITE_SIZE 1 KiB units: factor 1.000).  Summary: profiles/mobilenet_v1_b64_hbm_traffic.md.
 MEASURED_HBM_TRAFFIC = {
     ("mobilenet_v1_1.0_224", 32): {
-        "stem": 21553091,
-        "dw1": 25801624,
-        "pw1": 38745575,
-        "dw2": 32204273,
-        "pw2": 19641072,
-        "dw3": 25832073,
-        "pw3": 26122490,
-        "dw4": 16173845,
-        "pw4": 10208825,
-        "dw5": 13030988,
-        "pw5": 13554890,
-        "dw6": 8182875,
-        "pw6": 6195140,
-        "dw7": 6682452,
-        "pw7": 8948984,
-        "dw8": 6680533,
-        "pw8": 8944763,
-        "dw9": 6682708,
-        "pw9": 8946682,
-        "dw10": 6681045,
-        "pw10": 8946554,
-        "dw11": 6678870,
-        "pw11": 8946937,
-        "dw12": 4231529,
-        "pw12": 7120742,
-        "dw13": 3576246,
-        "pw13": 12342237,
-        "avgpool": 1687762,
-        "logits": 1437820,
-        "softmax": 127442
+        "stem": 21548852,
+        "dw1": 25794179,
+        "pw1": 38745806,
+        "dw2": 32200130,
+        "pw2": 19635813,
+        "dw3": 25824756,
+        "pw3": 26118499,
+        "dw4": 16169854,
+        "pw4": 10218157,
+        "dw5": 13023811,
+        "pw5": 13534535,
+        "dw6": 8179920,
+        "pw6": 6174280,
+        "dw7": 6675793,
+        "pw7": 8928376,
+        "dw8": 6671954,
+        "pw8": 8925689,
+        "dw9": 6675537,
+        "pw9": 8926201,
+        "dw10": 6674001,
+        "pw10": 8925561,
+        "dw11": 6672210,
+        "pw11": 8926457,
+        "dw12": 4227428,
+        "pw12": 7101541,
+        "dw13": 3582895,
+        "pw13": 12321746,
+        "avgpool": 1687758,
+        "logits": 1452018,
+        "softmax": 127441
     },
     ("mobilenet_v1_1.0_224", 64): {
         "dw1": 51482293,
