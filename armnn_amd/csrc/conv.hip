@@ -579,6 +579,7 @@ int LaunchIgemmLds(const mi355x_conv2d_s* p, int stages, uint32_t batch, const v
         if (stages == 3)
             return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 3, true>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 3, false>(p, batch, x, y, stream);
     }
+
     return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 2, true>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 2, false>(p, batch, x, y, stream);
 }
 
@@ -653,7 +654,12 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const int lds_stages = GlobalOptions().igemm_lds;
         if (lds_stages != 0 && bk128 && (g.Ci % 128) == 0)
         {
-            if (tile == 64) return LaunchIgemmLds<64, 64, 2, 2>(p, lds_stages, batch, x, y, stream);
+            if (tile == 64)
+            {
+                // at most one block per CU: nothing else hides a k-tile's round trip, so keep two tiles on their way
+                const long long blocks64 = ((M + 63) / 64) * ((g.Co + 63) / 64);
+                return LaunchIgemmLds<64, 64, 2, 2>(p, (lds_stages == 2 && blocks64 <= 256) ? 3 : lds_stages, batch, x, y, stream);
+            }
             if (g.Co <= 64 || tile == 96) return LaunchIgemmLds<128, 64, 2, 2>(p, lds_stages, batch, x, y, stream);
             if (tile == 256) return LaunchIgemmLds<256, 128, 4, 2>(p, lds_stages, batch, x, y, stream);
             if (tile == 512) return LaunchIgemmLds<256, 256, 4, 4>(p, lds_stages, batch, x, y, stream);

@@ -10,7 +10,9 @@
 //     bank half and get 8 different slots).  Lanes pick the global chunk that belongs in their slot; readers apply
 //     the same xor.
 //   * uint8 activations become int8 by xor 0x80 on the fragment registers (template U8), weights are int8 already.
-//   * ST stages of LDS; tile kt + ST - 1 is requested right after the barrier that retires tile kt - 1.
+//   * ST stages of LDS (2 to 8); tile kt + ST - 1 is requested right after the barrier that retires tile kt - 1, so
+//     ST - 1 tiles are on their way while one is multiplied: deep for the few-block problems whose k-loop would
+//     otherwise run at one memory round trip per tile.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -40,7 +42,8 @@ constexpr int VmcntImm(int n)
 template <int BM, int BN, int WM, int WN, int ST, bool U8>
 __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
 {
-    static_assert(ST == 2 || ST == 3, "2 or 3 LDS stages");
+    static_assert(ST >= 2 && ST <= 8, "2 to 8 LDS stages");
+    static_assert((ST - 2) * (BM + BN) / (8 * WM * WN) < 64, "outstanding loads must fit the vmcnt counter");
     constexpr int BK = 128;
     constexpr int NW = WM * WN;                 // waves
     constexpr int NT = 64 * NW;                 // threads
@@ -187,8 +190,14 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
     int stage = 0;
     for (int kt = 0; kt < nk; ++kt)
     {
-        // tile kt has landed when at most the younger requests are outstanding
-        if (ST == 3 && kt + 1 < nk) __builtin_amdgcn_s_waitcnt(VmcntImm(RA + RB));
+        // tile kt has landed when at most the requests of the younger tiles (up to ST - 2 of them) are outstanding
+        const int younger = min(ST - 2, nk - 1 - kt);
+        if (ST >= 8 && younger == 6) __builtin_amdgcn_s_waitcnt(VmcntImm(6 * (RA + RB)));
+        else if (ST >= 7 && younger == 5) __builtin_amdgcn_s_waitcnt(VmcntImm(5 * (RA + RB)));
+        else if (ST >= 6 && younger == 4) __builtin_amdgcn_s_waitcnt(VmcntImm(4 * (RA + RB)));
+        else if (ST >= 5 && younger == 3) __builtin_amdgcn_s_waitcnt(VmcntImm(3 * (RA + RB)));
+        else if (ST >= 4 && younger == 2) __builtin_amdgcn_s_waitcnt(VmcntImm(2 * (RA + RB)));
+        else if (ST >= 3 && younger == 1) __builtin_amdgcn_s_waitcnt(VmcntImm(RA + RB));
         else __builtin_amdgcn_s_waitcnt(VmcntImm(0));
         __syncthreads();                         // every wave's part of tile kt is in LDS; tile kt - 1 is no longer read
         if (kt + ST - 1 < nk)
