@@ -54,6 +54,13 @@ struct Requant
     float   inv_scale;
     float   act_lo_f, act_hi_f;
     int32_t fast_ok;
+    // Convolution / FullyConnected epilogue: codes are produced as unsigned bytes with v_cvt_pk_u8_f32 (converts,
+    // saturates to 0..255 and packs in one instruction).  Signed outputs are computed 128 higher (pk_bias is folded into
+    // the per-channel constant fb on the host) and the finished dword is xor-ed with 0x80808080.
+    int32_t  pk_bias;       // 128 for QAsymmS8 outputs, 0 for QAsymmU8
+    uint32_t pk_xor;        // 0x80808080 or 0
+    float    pk_lo_f, pk_hi_f;   // activation clamp in the biased domain
+    int32_t  pk_full;       // the clamp is 0..255: the instruction's own saturation does it
 };
 
 Requant MakeRequant(const mi355x_quant& out, int32_t activation, float a, float b);

@@ -165,10 +165,11 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         const int CP = p->Co_pad;
         std::vector<float> tab(static_cast<size_t>(7) * CP, 0.0f);
         const float inv = 1.0f / d.output.scale;
-        const float zp_f = static_cast<float>(d.output.offset);
+        // the fast path works 128 codes higher for signed outputs (Requant::pk_bias), so that is its offset
+        const float zp_f = static_cast<float>(d.output.offset + (d.output.dtype == MI355X_QASYMM_U8 ? 0 : 128));
         const double max_acc = static_cast<double>(p->K) * 65025.0;
         const bool base_ok = !GlobalOptions().exact_division_epilogue && std::isnormal(inv) && std::isnormal(d.output.scale) &&
-                             d.output.offset >= -255 && d.output.offset <= 255;
+                             d.output.offset >= -255 && d.output.offset <= 255 && p->rq.fast_ok;
         for (int c = 0; c < CP; ++c)
         {
             tab[c] = mult[c];

@@ -33,7 +33,8 @@ __device__ __forceinline__ int RequantExactDev(int acc, float mult, float biasf,
 
 // Per-channel constants, seven rows of `stride` floats, built on the host (conv.hip):
 //   row 0 mult   s_in * s_w[c]                      row 1 biasf  float(bias[c]) * s_b[c]
-//   row 2 fm     fl(mult * fl(1/s_out))             row 3 fb     fl(fl(biasf * fl(1/s_out)) + offset)
+//   row 2 fm     fl(mult * fl(1/s_out))             row 3 fb     fl(fl(biasf * fl(1/s_out)) + offset'),
+//                                                    offset' = offset + Requant::pk_bias (codes as unsigned bytes)
 //   row 4 thr    tie threshold for rows 2/3 (negative: the channel always takes the exact path)
 //   row 5 fbc    fb + corr * fm                     row 6 thrc   tie threshold for rows 2/5
 // Rows 5/6 serve kernels whose accumulators start at zero: the zero-point correction corr[c] is then part of the
@@ -90,7 +91,7 @@ __device__ __forceinline__ Fast4 LoadFast4(const ChanTab& ct, int c)
 
 // Four consecutive channels c..c+3 of one pixel -> packed dword.
 //   `corr` (may be null) is an integer added to the accumulator on the exact path only (rows 5/6, see ChanTab).
-// The fast path is branch-free (8 VALU instructions per value); the four flags are combined as wave masks, and
+// The fast path is branch-free (7 VALU instructions per value when the clamp is the whole byte range); the four flags are combined as wave masks, and
 // only when some lane of the wave has a flagged value does the wave enter the fix-up loop, which evaluates one
 // flagged value per lane and pass.
 __device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const float4& fm, const float4& fb,
@@ -103,10 +104,18 @@ __device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, 
     MI355X_FAST1(a1, fm.y, fb.y, thr.y, k1, s1)
     MI355X_FAST1(a2, fm.z, fb.z, thr.z, k2, s2)
     MI355X_FAST1(a3, fm.w, fb.w, thr.w, k3, s3)
-    int q0 = static_cast<int>(__builtin_amdgcn_fmed3f(k0, rq.act_lo_f, rq.act_hi_f));
-    int q1 = static_cast<int>(__builtin_amdgcn_fmed3f(k1, rq.act_lo_f, rq.act_hi_f));
-    int q2 = static_cast<int>(__builtin_amdgcn_fmed3f(k2, rq.act_lo_f, rq.act_hi_f));
-    int q3 = static_cast<int>(__builtin_amdgcn_fmed3f(k3, rq.act_lo_f, rq.act_hi_f));
+    if (!rq.pk_full)      // wave-uniform: a clamp narrower than 0..255 (the conversion below saturates to that by itself)
+    {
+        k0 = __builtin_amdgcn_fmed3f(k0, rq.pk_lo_f, rq.pk_hi_f);
+        k1 = __builtin_amdgcn_fmed3f(k1, rq.pk_lo_f, rq.pk_hi_f);
+        k2 = __builtin_amdgcn_fmed3f(k2, rq.pk_lo_f, rq.pk_hi_f);
+        k3 = __builtin_amdgcn_fmed3f(k3, rq.pk_lo_f, rq.pk_hi_f);
+    }
+    // integral floats -> saturated unsigned bytes, one instruction per value, packed as it goes
+    uint32_t out = __builtin_amdgcn_cvt_pk_u8_f32(k0, 0, 0u);
+    out = __builtin_amdgcn_cvt_pk_u8_f32(k1, 1, out);
+    out = __builtin_amdgcn_cvt_pk_u8_f32(k2, 2, out);
+    out = __builtin_amdgcn_cvt_pk_u8_f32(k3, 3, out);
     const unsigned long long any = __builtin_amdgcn_ballot_w64(s0) | __builtin_amdgcn_ballot_w64(s1) |
                                    __builtin_amdgcn_ballot_w64(s2) | __builtin_amdgcn_ballot_w64(s3);
     if (__builtin_expect(any != 0, 0))
@@ -122,15 +131,12 @@ __device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, 
             const int av = which == 0 ? a0 + cr.x : which == 1 ? a1 + cr.y : which == 2 ? a2 + cr.z : a3 + cr.w;
             const float mv = which == 0 ? m.x : which == 1 ? m.y : which == 2 ? m.z : m.w;
             const float bv = which == 0 ? b.x : which == 1 ? b.y : which == 2 ? b.z : b.w;
-            const int qe = RequantExactDev(av, mv, bv, rq);
-            if (which == 0) q0 = qe;
-            if (which == 1) q1 = qe;
-            if (which == 2) q2 = qe;
-            if (which == 3) q3 = qe;
+            const uint32_t qe = static_cast<uint32_t>(RequantExactDev(av, mv, bv, rq) + rq.pk_bias) & 0xffu;
+            if (which < 4) out = (out & ~(0xffu << (8 * which))) | (qe << (8 * which));
             fl &= fl - 1u;
         }
     }
-    return Pack4(q0, q1, q2, q3);
+    return out ^ rq.pk_xor;
 }
 
 // constants of rows 2,3,4 (accumulator already contains the zero-point correction)
@@ -147,7 +153,7 @@ __device__ __forceinline__ int Requant1Dev(int acc, const ChanTab& ct, int c, co
     bool slow;
     MI355X_FAST1(acc, ct.p[2 * ct.stride + c], ct.p[3 * ct.stride + c], ct.p[4 * ct.stride + c], k, slow)
     if (__builtin_expect(slow, 0)) return RequantExactDev(acc, ct.p[c], ct.p[ct.stride + c], rq);
-    return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.act_lo_f, rq.act_hi_f));
+    return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.pk_lo_f, rq.pk_hi_f)) - rq.pk_bias;
 }
 
 // one channel, accumulator started at zero: rows 2/5/6 on the fast path, `corr[c]` joins the accumulator on the exact path
@@ -157,7 +163,7 @@ __device__ __forceinline__ int Requant1FoldedDev(int acc, const ChanTab& ct, con
     bool slow;
     MI355X_FAST1(acc, ct.p[2 * ct.stride + c], ct.p[5 * ct.stride + c], ct.p[6 * ct.stride + c], k, slow)
     if (__builtin_expect(slow, 0)) return RequantExactDev(acc + corr[c], ct.p[c], ct.p[ct.stride + c], rq);
-    return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.act_lo_f, rq.act_hi_f));
+    return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.pk_lo_f, rq.pk_hi_f)) - rq.pk_bias;
 }
 
 // value already in float (pooling, add, ...): reciprocal fast path with the exact fallback near ties.

@@ -71,6 +71,11 @@ Requant MakeRequant(const mi355x_quant& out, int32_t activation, float a, float 
     rq.act_hi_f  = static_cast<float>(rq.act_hi);
     // The tie window argument needs |offset| <= 255 (so that |value/scale| > 512 always clamps) and a normal,
     // finite reciprocal.
+    rq.pk_bias = rq.out_is_u8 ? 0 : 128;
+    rq.pk_xor  = rq.out_is_u8 ? 0u : 0x80808080u;
+    rq.pk_lo_f = static_cast<float>(rq.act_lo + rq.pk_bias);
+    rq.pk_hi_f = static_cast<float>(rq.act_hi + rq.pk_bias);
+    rq.pk_full = (rq.act_lo + rq.pk_bias == 0 && rq.act_hi + rq.pk_bias == 255) ? 1 : 0;
     rq.fast_ok = !GlobalOptions().exact_division_epilogue && std::isnormal(rq.inv_scale) && std::isnormal(out.scale) && out.offset >= -255 && out.offset <= 255 &&
                  rq.act_lo <= rq.act_hi;
     return rq;
