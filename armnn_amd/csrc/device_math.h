@@ -181,4 +181,33 @@ __device__ __forceinline__ int QuantizeFastDev(float f, const Requant& rq)
     return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.act_lo_f, rq.act_hi_f));
 }
 
+// Four float values -> packed dword of output codes: QuantizeFastDev's test per value, then v_cvt_pk_u8_f32 (convert,
+// saturate, pack) in the biased domain of Requant::pk_bias.  |offset + pk_bias| <= 383 here, hence the wider constant.
+__device__ __forceinline__ uint32_t QuantizePack4Dev(float f0, float f1, float f2, float f3, const Requant& rq)
+{
+    if (!rq.fast_ok) return Pack4(QuantizeDev(f0, rq), QuantizeDev(f1, rq), QuantizeDev(f2, rq), QuantizeDev(f3, rq));
+    const float off = rq.out_offset_f + static_cast<float>(rq.pk_bias);
+    const float f[4] = {f0, f1, f2, f3};
+    uint32_t out = 0u;
+    unsigned slow = 0u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+    {
+        const float r = __fmaf_rn(f[i], rq.inv_scale, off);
+        float k = __builtin_rintf(r);
+        const float e = __fsub_rn(r, k);
+        if (!(fabsf(e) <= __fmaf_rn(fabsf(r), -4.5f / 16777216.0f, 0.5f - 1536.0f / 16777216.0f))) slow |= 1u << i;
+        if (!rq.pk_full) k = __builtin_amdgcn_fmed3f(k, rq.pk_lo_f, rq.pk_hi_f);
+        out = __builtin_amdgcn_cvt_pk_u8_f32(k, i, out);
+    }
+    if (__builtin_expect(slow != 0u, 0))
+    {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if (slow & (1u << i))
+                out = (out & ~(0xffu << (8 * i))) | ((static_cast<uint32_t>(QuantizeDev(f[i], rq) + rq.pk_bias) & 0xffu) << (8 * i));
+    }
+    return out ^ rq.pk_xor;
+}
+
 } // namespace mi355x

@@ -28,6 +28,19 @@ __device__ __forceinline__ float DequantDev(uint8_t code, const QIn& q)
     return __fmul_rn(static_cast<float>(v - q.offset), q.scale);   // armnn::Dequantize, TypesUtils.cpp:47-56
 }
 
+// The four codes of a dword -> float values: signed codes are made unsigned with one xor for the dword (offset moves by
+// 128 with them), then v_cvt_f32_ubyteN converts byte N directly; value - offset is an exact small integer either way,
+// so the single multiplication rounds exactly as in armnn::Dequantize.
+__device__ __forceinline__ void Dequant4Dev(uint32_t w, const QIn& q, float (&v)[4])
+{
+    const uint32_t u = q.is_u8 ? w : (w ^ 0x80808080u);
+    const float off = static_cast<float>(q.is_u8 ? q.offset : q.offset + 128);
+    v[0] = __fmul_rn(__fsub_rn(static_cast<float>(u & 0xffu), off), q.scale);
+    v[1] = __fmul_rn(__fsub_rn(static_cast<float>((u >> 8) & 0xffu), off), q.scale);
+    v[2] = __fmul_rn(__fsub_rn(static_cast<float>((u >> 16) & 0xffu), off), q.scale);
+    v[3] = __fmul_rn(__fsub_rn(static_cast<float>(u >> 24), off), q.scale);
+}
+
 __device__ __forceinline__ float ActivationDev(float in, int fn, float a, float b)
 {
     if (fn == MI355X_ACT_RELU) return fmaxf(0.0f, in);
@@ -212,8 +225,7 @@ __global__ __launch_bounds__(256) void Pool2dC4Kernel(PoolArgs p, QIn qin, Requa
             else res[ch] = __fdiv_rn(res[ch], area);
         }
     }
-    *reinterpret_cast<uint32_t*>(y + idx * 4) = Pack4(QuantizeFastDev(res[0], rq), QuantizeFastDev(res[1], rq),
-                                                      QuantizeFastDev(res[2], rq), QuantizeFastDev(res[3], rq));
+    *reinterpret_cast<uint32_t*>(y + idx * 4) = QuantizePack4Dev(res[0], res[1], res[2], res[3], rq);
 }
 
 // The window is the whole image (global pooling): a block owns 256 channels of one image.  All threads fetch the
@@ -277,15 +289,10 @@ __global__ __launch_bounds__(256) void AddVec16Kernel(QIn q0, QIn q1, Requant rq
 #pragma unroll
         for (int d = 0; d < 4; ++d)
         {
-            int q[4];
-#pragma unroll
-            for (int k = 0; k < 4; ++k)
-            {
-                const float s = __fadd_rn(DequantDev(static_cast<uint8_t>((a[d] >> (8 * k)) & 0xffu), q0),
-                                          DequantDev(static_cast<uint8_t>((b[d] >> (8 * k)) & 0xffu), q1));
-                q[k] = QuantizeFastDev(s, rq);
-            }
-            o[d] = Pack4(q[0], q[1], q[2], q[3]);
+            float va[4], vb[4];
+            Dequant4Dev(a[d], q0, va);
+            Dequant4Dev(b[d], q1, vb);
+            o[d] = QuantizePack4Dev(__fadd_rn(va[0], vb[0]), __fadd_rn(va[1], vb[1]), __fadd_rn(va[2], vb[2]), __fadd_rn(va[3], vb[3]), rq);
         }
         y[i] = o;
     }
