@@ -330,6 +330,10 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         p->xor_mask = g.in_u8 ? 0x80u : 0u;
         p->pad_word = static_cast<uint32_t>(zx_shift) & 0xffu;
         p->row_dwords = RD;
+        {
+            const std::vector<uint8_t> padbytes(16, static_cast<uint8_t>((p->pad_word ^ p->xor_mask) & 0xffu));
+            if (int rc = Upload(reinterpret_cast<void**>(&p->pad16), padbytes.data(), padbytes.size())) return rc;
+        }
         if (Co == 32 || Co == 64)
         {
             // the same rows, end to end, as the K vector of the MFMA variant
@@ -683,6 +687,12 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         a.lp = ((3 + 31 * g.stride_x * g.Ci + 4 * p->row_dwords + 3) & ~3) + 8;
         a.ndw_recip = static_cast<uint32_t>((0x100000000ull + static_cast<unsigned long long>(a.lp / 4) - 1ull) / static_cast<unsigned long long>(a.lp / 4));
         a.vec16 = ((reinterpret_cast<uintptr_t>(y) & 15) == 0 && (g.Co % 16) == 0) ? 1 : 0;
+        // 16-byte staging when every halo row starts on a 16-byte boundary and image rows are whole chunks
+        a.pad16 = p->pad16;
+        a.vec_stage = ((g.W * g.Ci) % 16 == 0 && (static_cast<long long>(g.H) * g.W * g.Ci) % 16 == 0 && g.pad_left == 0 &&
+                       (32 * g.stride_x * g.Ci) % 16 == 0 && (reinterpret_cast<uintptr_t>(x) & 15) == 0) ? 1 : 0;
+        if (a.vec_stage) a.lp = (31 * g.stride_x * g.Ci + 4 * p->row_dwords + 4 + 15) / 16 * 16;
+        a.nch_recip = static_cast<uint32_t>((0x100000000ull + static_cast<unsigned long long>(a.lp / 16) - 1ull) / static_cast<unsigned long long>(std::max(1, a.lp / 16)));
         if (a.lp > 288) return SetError(MI355X_ERR_UNSUPPORTED, "dot4 kernel: halo row of %d bytes does not fit", a.lp);
         if (static_cast<long long>(g.H) * g.W * g.Ci >= (1ll << 30)) return SetError(MI355X_ERR_UNSUPPORTED, "dot4 kernel: image too large for 32-bit offsets");
         a.rq = p->rq;

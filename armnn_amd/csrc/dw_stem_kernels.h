@@ -198,6 +198,10 @@ struct SmallCiArgs
     uint32_t ndw_recip;       // ceil(2^32 / (lp / 4))
     uint32_t xor_mask, pad_byte;
     int vec16;                // output rows allow 16-byte stores (y 16-byte aligned, Co % 16 == 0)
+    const uint8_t* pad16;     // 16 bytes of (padding value ^ input xor)
+    int vec_stage;            // every halo row starts 16-byte aligned and image rows are whole 16-byte chunks: stage with
+                              // 16-byte loads (lp is then a multiple of 16)
+    uint32_t nch_recip;       // ceil(2^32 / (lp / 16))
     const int8_t* w_mfma;     // MFMA variant: [Co rounded up to 32][kp] bytes, a filter's rows as RD dwords each, zero padded
     int kp;                   // bytes per weight row of w_mfma (multiple of 32)
     Requant rq;
@@ -242,6 +246,35 @@ __device__ __forceinline__ void StageSmallCiHalo(const SmallCiArgs& a, uint32_t*
     const uint32_t xm = a.xor_mask & 0xffu;
     const uint32_t xm4 = xm * 0x01010101u;
     const uint32_t pad4 = (a.pad_byte & 0xffu) * 0x01010101u;
+    if (a.vec_stage)          // block-uniform
+    {
+        // Aligned geometry: a 16-byte chunk lies wholly inside the image or wholly outside it; a chunk outside loads 16
+        // prepared bytes that become the padding value under the xor, so every load is unconditional and in flight at once.
+        constexpr int MAXV = (HRMAX * (LPMAX / 16) + 255) / 256;
+        const int nch = a.lp >> 4;
+        const int total = HR * nch;
+        const int row_bytes = a.W * a.Ci;
+        const int col0 = ix_org * a.Ci;
+        v4i sv[MAXV];
+#pragma unroll
+        for (int k = 0; k < MAXV; ++k)
+        {
+            const int i = min(tid + k * 256, total - 1);
+            const int row = static_cast<int>(__umulhi(static_cast<uint32_t>(i), a.nch_recip));
+            const int c = i - row * nch;
+            const int iy = iy_org + row;
+            const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && col0 + 16 * c + 16 <= row_bytes;
+            const uint8_t* src = ok ? xn + static_cast<long long>(iy) * row_bytes + col0 + 16 * c : a.pad16;
+            sv[k] = *reinterpret_cast<const v4i*>(src);
+        }
+#pragma unroll
+        for (int k = 0; k < MAXV; ++k)
+        {
+            const int i = tid + k * 256;
+            if (i < total) *reinterpret_cast<v4i*>(tile + i * 4) = sv[k] ^ static_cast<int>(xm4);
+        }
+        return;
+    }
     // columns of the halo that lie inside the image, as byte offsets from the halo's first column
     const int vb0 = max(0, -ix_org) * a.Ci;
     const int vb1 = min((TW - 1) * S + a.Kw, a.W - ix_org) * a.Ci;

@@ -207,6 +207,12 @@ def small_conv_cases():
     c.append(make_conv_case("stem_u8_7x7_s2_ci3_co32", 228, n=2, h=39, w=45, ci=3, co=32, kh=7, kw=7, stride=(2, 2), in_dtype=U8,
                             in_offset=111, out_offset=9, w_scale_range=(0.002, 0.008)))
     c.append(make_conv_case("stem_s8_3x3_s2_ci4_co32", 229, n=1, h=18, w=40, ci=4, co=32, stride=(2, 2)))
+    # aligned geometry (image rows whole 16-byte chunks, no left padding): the 16-byte staging path, with tiles that reach past
+    # the right and bottom edges, on both small-Ci kernels
+    c.append(make_conv_case("stem_u8_3x3_s2_ci3_aligned_co32", 230, n=3, h=50, w=80, ci=3, co=32, stride=(2, 2), in_dtype=U8,
+                            in_offset=120, out_offset=4, act=RELU6))
+    c.append(make_conv_case("stem_s8_3x3_s2_ci4_aligned_co24", 231, n=2, h=34, w=140, ci=4, co=24, stride=(2, 2), in_offset=-9))
+    c.append(make_conv_case("stem_s8_3x3_s1_ci4_nopad_co64", 232, n=2, h=21, w=36, ci=4, co=64, padding="valid"))
     c.append(make_conv_case("dw_u8_5x5_c20", 206, h=9, w=9, ci=20, depthwise=True, kh=5, kw=5, in_dtype=U8,
                             in_offset=100, out_offset=3, w_scale_range=(0.005, 0.02)))
     return c
