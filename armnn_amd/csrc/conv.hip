@@ -730,15 +730,21 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.C = g.Co; a.Ho = g.Ho; a.Wo = g.Wo;
             a.pad_top = g.pad_top; a.pad_left = g.pad_left;
             const int tw = g.stride_x == 1 ? 16 : 8;
-            a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + 7) / 8; a.cblocks = g.Co / 32;
+            // two output rows per thread (16-row tiles) unless that would leave much of a tile outside a small feature map
+            const int opt_r = GlobalOptions().dw_rows;
+            const int rows_per_thread = opt_r ? opt_r : ((g.Ho + 15) / 16 * 16 - g.Ho) * 4 <= g.Ho ? 2 : 1;
+            const int th = 8 * rows_per_thread;
+            a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + th - 1) / th; a.cblocks = g.Co / 32;
             a.xor_mask = p->xor_mask; a.pad_word = p->pad_word; a.rq = p->rq;
             const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y * a.cblocks;
             if (nb > 0x7fffffffll - 8) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
             a.total_blocks = static_cast<int>(nb);
             a.xcd_chunk = static_cast<int>((nb + 7) / 8);
             const dim3 grid(static_cast<unsigned>(a.xcd_chunk) * 8u);
-            if (g.stride_x == 1) hipLaunchKernelGGL((Depthwise3x3Kernel<1>), grid, dim3(256), 0, stream, a);
-            else hipLaunchKernelGGL((Depthwise3x3Kernel<2>), grid, dim3(256), 0, stream, a);
+            if (g.stride_x == 1 && rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2>), grid, dim3(256), 0, stream, a);
+            else if (g.stride_x == 1) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1>), grid, dim3(256), 0, stream, a);
+            else if (rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<2, 2>), grid, dim3(256), 0, stream, a);
+            else hipLaunchKernelGGL((Depthwise3x3Kernel<2, 1>), grid, dim3(256), 0, stream, a);
             MI355X_HIP(hipGetLastError());
             return 0;
         }

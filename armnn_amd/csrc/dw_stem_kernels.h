@@ -1,6 +1,6 @@
 // VALU kernels built on v_dot4_i32_i8 with LDS-staged halo tiles:
 //
-//   Depthwise3x3Kernel<S>   DepthwiseConvolution2d 3x3, multiplier 1, stride S in {1,2}, channels % 32 == 0.
+//   Depthwise3x3Kernel<S,R> DepthwiseConvolution2d 3x3, multiplier 1, stride S in {1,2}, channels % 32 == 0, R output rows per thread.
 //   SmallCiConvKernel<..>   Convolution2d with <= 4 input channels (network stems): too little K per tap for MFMA.
 //
 // Both bring the input to signed int8 while staging (uint8: x ^ 0x80) and fill out-of-image positions with the
@@ -41,20 +41,23 @@ __device__ __forceinline__ int XcdContiguousWorkItem(int block, int chunk)
     return (block & 7) * chunk + (block >> 3);
 }
 
-// Block: 8 output rows x (4 groups of P pixels) x 32 channels; thread = (4 channels, P pixels of one row).
-// A thread reads 6 consecutive input pixels per kernel row (one dword = 4 channels each), transposes them with
+// Block: 8 R output rows x (4 groups of P pixels) x 32 channels; thread = (4 channels, P pixels of R consecutive rows).
+// A thread reads 6 consecutive input pixels per input row (one dword = 4 channels each), transposes them with
 // v_perm_b32 into per-channel dwords of 4 consecutive pixels, and each such dword feeds
 //   stride 1: two outputs  (weights {w0,w1,w2,0} and {0,w0,w1,w2})
 //   stride 2: one output   (weights {w0,w1,w2,0})
-// through one v_dot4 per channel.
-template <int S>
+// through one v_dot4 per channel and output row that the input row belongs to.  With R = 2 the rows two outputs share
+// are read and transposed once, and the per-thread set-up (staging, constants, addresses) is spread over twice the
+// outputs; R = 1 keeps more blocks in flight for small feature maps.
+template <int S, int R>
 __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
 {
-    constexpr int CB = 32, TH = 8, XG = 4;
-    constexpr int P = S == 1 ? 4 : 2;            // outputs per thread
+    constexpr int CB = 32, TH = 8 * R, XG = 4;
+    constexpr int P = S == 1 ? 4 : 2;            // outputs per thread and row
     constexpr int TW = P * XG;                   // outputs per tile row
     constexpr int HR = TH * S + 2;               // halo rows held in LDS
     constexpr int HC = TW * S + 2;               // halo columns
+    constexpr int IR = (R - 1) * S + 3;          // input rows a thread walks
     constexpr int PITCH = 48;                    // bytes per pixel in LDS: 32 used; 48 spreads dword reads over banks
     __shared__ __attribute__((aligned(16))) uint8_t tile[HR * HC * PITCH];
 
@@ -98,7 +101,7 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
     // ---- per-thread constants ---------------------------------------------------------------------------------
     const int c4 = tid & 7;
     const int xg = (tid >> 3) & 3;
-    const int row = tid >> 5;
+    const int row = (tid >> 5) * R;              // first of this thread's output rows within the tile
     const int c = cb * CB + c4 * 4;
     uint32_t wA[3][4];
 #pragma unroll
@@ -108,18 +111,20 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
         wA[0][ch] = w4.x; wA[1][ch] = w4.y; wA[2][ch] = w4.z;
     }
     const v4i corr4 = *reinterpret_cast<const v4i*>(a.corr + c);
-    int acc[P][4];
+    int acc[R][P][4];
 #pragma unroll
-    for (int j = 0; j < P; ++j)
+    for (int o = 0; o < R; ++o)
 #pragma unroll
-        for (int ch = 0; ch < 4; ++ch) acc[j][ch] = corr4[ch];
+        for (int j = 0; j < P; ++j)
+#pragma unroll
+            for (int ch = 0; ch < 4; ++ch) acc[o][j][ch] = corr4[ch];
 
     __syncthreads();
 
 #pragma unroll
-    for (int r = 0; r < 3; ++r)
+    for (int ir = 0; ir < IR; ++ir)
     {
-        const uint8_t* base = tile + ((row * S + r) * HC + xg * P * S) * PITCH + c4 * 4;
+        const uint8_t* base = tile + ((row * S + ir) * HC + xg * P * S) * PITCH + c4 * 4;
         uint32_t px[6];
 #pragma unroll
         for (int j = 0; j < 6; ++j) px[j] = *reinterpret_cast<const uint32_t*>(base + j * PITCH);
@@ -140,35 +145,46 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
             chv[1] = __builtin_amdgcn_perm(lo[g + 1], lo[g], 0x07060302u);
             chv[2] = __builtin_amdgcn_perm(hi[g + 1], hi[g], 0x05040100u);
             chv[3] = __builtin_amdgcn_perm(hi[g + 1], hi[g], 0x07060302u);
+            // input row ir is filter row r = ir - o * S of output row o
 #pragma unroll
-            for (int ch = 0; ch < 4; ++ch)
+            for (int o = 0; o < R; ++o)
             {
-                if (S == 1)
+                const int r = ir - o * S;
+                if (r < 0 || r > 2) continue;
+#pragma unroll
+                for (int ch = 0; ch < 4; ++ch)
                 {
-                    acc[2 * g][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wA[r][ch]), acc[2 * g][ch], false);
-                    acc[2 * g + 1][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wA[r][ch] << 8), acc[2 * g + 1][ch], false);
-                }
-                else
-                {
-                    acc[g][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wA[r][ch]), acc[g][ch], false);
+                    if (S == 1)
+                    {
+                        acc[o][2 * g][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wA[r][ch]), acc[o][2 * g][ch], false);
+                        acc[o][2 * g + 1][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wA[r][ch] << 8), acc[o][2 * g + 1][ch], false);
+                    }
+                    else
+                    {
+                        acc[o][g][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wA[r][ch]), acc[o][g][ch], false);
+                    }
                 }
             }
         }
     }
 
     // ---- epilogue ------------------------------------------------------------------------------------------------
-    const int oy = ty * TH + row;
-    if (oy >= a.Ho) return;
     const Fast4 f4 = LoadFast4(a.ct, c);
-    uint8_t* yrow = a.y + (static_cast<long long>(n) * a.Ho + oy) * a.Wo * a.C + c;
 #pragma unroll
-    for (int j = 0; j < P; ++j)
+    for (int o = 0; o < R; ++o)
     {
-        const int ox = tx * TW + xg * P + j;
-        if (ox < a.Wo)
+        const int oy = ty * TH + row + o;
+        if (oy >= a.Ho) break;
+        uint8_t* yrow = a.y + (static_cast<long long>(n) * a.Ho + oy) * a.Wo * a.C + c;
+#pragma unroll
+        for (int j = 0; j < P; ++j)
         {
-            *reinterpret_cast<uint32_t*>(yrow + static_cast<long long>(ox) * a.C) =
-                Requant4Dev(acc[j][0], acc[j][1], acc[j][2], acc[j][3], f4, a.ct, c, a.rq);
+            const int ox = tx * TW + xg * P + j;
+            if (ox < a.Wo)
+            {
+                *reinterpret_cast<uint32_t*>(yrow + static_cast<long long>(ox) * a.C) =
+                    Requant4Dev(acc[o][j][0], acc[o][j][1], acc[o][j][2], acc[o][j][3], f4, a.ct, c, a.rq);
+            }
         }
     }
 }

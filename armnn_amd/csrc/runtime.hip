@@ -103,6 +103,12 @@ int mi355x_set_option(const char* name, int value)
     if (!name) return SetError(MI355X_ERR_INVALID_ARGUMENT, "option name is null");
     if (std::strcmp(name, "exact_division_epilogue") == 0) { GlobalOptions().exact_division_epilogue = value != 0; return 0; }
     if (std::strcmp(name, "stem_dot4") == 0) { GlobalOptions().stem_dot4 = value != 0; return 0; }
+    if (std::strcmp(name, "dw_rows") == 0)
+    {
+        if (value < 0 || value > 2) return SetError(MI355X_ERR_INVALID_ARGUMENT, "dw_rows must be 0, 1 or 2");
+        GlobalOptions().dw_rows = value;
+        return 0;
+    }
     if (std::strcmp(name, "igemm_lds") == 0)
     {
         if (value != 0 && value != 2 && value != 3) return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_lds must be 0, 2 or 3");

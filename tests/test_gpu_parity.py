@@ -159,6 +159,25 @@ def test_every_igemm_tiling_gives_the_same_bytes():
         shim.set_option("igemm_tile", 100)
 
 
+def test_depthwise_rows_per_thread_variants_give_the_same_bytes():
+    """The 3x3 depthwise kernel with one and with two output rows per thread (8- and 16-row tiles), forced on feature maps
+    of every parity of height, against the plain depthwise kernel."""
+    cs = [cases.make_conv_case("dwr_s1_h14", 701, n=2, h=14, w=14, ci=64, depthwise=True, act=cases.RELU6),
+          cases.make_conv_case("dwr_s1_h23", 702, n=1, h=23, w=37, ci=32, depthwise=True, in_dtype=cases.U8, in_offset=140, out_offset=5),
+          cases.make_conv_case("dwr_s2_h29", 703, n=2, h=29, w=31, ci=96, depthwise=True, stride=(2, 2)),
+          cases.make_conv_case("dwr_s2_h7", 704, n=3, h=7, w=7, ci=32, depthwise=True, stride=(2, 2), act=cases.RELU)]
+    for c in cs:
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        for rows in (0, 1, 2):
+            shim.set_option("dw_rows", rows)
+            try:
+                got = _gpu_conv(c, shim.ALGO_DEPTHWISE)
+            finally:
+                shim.set_option("dw_rows", 0)
+            print(f"{c.name} rows {rows}", flush=True)
+            np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} rows {rows}")
+
+
 def test_config_c1_full_size(port):
     """BASELINE config 1: 1x56x56x64 -> 64, 3x3 SAME, per-channel, ReLU6; expected code range [-128, -8]."""
     c = cases.make_conv_case("C1", 20250101, h=56, w=56, ci=64, co=64, act=cases.RELU6)
