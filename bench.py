@@ -35,36 +35,36 @@ RIDGE_OPS_PER_BYTE = INT8_MFMA_PEAK_OPS / HBM_PEAK_BYTES
 # WRITE_SIZE 1 KiB units: factor 1.000).  Summary: profiles/mobilenet_v1_b64_hbm_traffic.md.
 MEASURED_HBM_TRAFFIC = {
     ("mobilenet_v1_1.0_224", 32): {
-        "stem": 21548852,
-        "dw1": 25794179,
-        "pw1": 38745806,
-        "dw2": 32200130,
-        "pw2": 19635813,
-        "dw3": 25824756,
-        "pw3": 26118499,
-        "dw4": 16169854,
-        "pw4": 10218157,
-        "dw5": 13023811,
-        "pw5": 13534535,
-        "dw6": 8179920,
-        "pw6": 6174280,
-        "dw7": 6675793,
-        "pw7": 8928376,
-        "dw8": 6671954,
-        "pw8": 8925689,
-        "dw9": 6675537,
-        "pw9": 8926201,
-        "dw10": 6674001,
-        "pw10": 8925561,
-        "dw11": 6672210,
-        "pw11": 8926457,
-        "dw12": 4227428,
-        "pw12": 7101541,
-        "dw13": 3582895,
-        "pw13": 12321746,
-        "avgpool": 1687758,
-        "logits": 1452018,
-        "softmax": 127441
+        "stem": 21485289,
+        "dw1": 25858383,
+        "pw1": 38751390,
+        "dw2": 32236845,
+        "pw2": 19656450,
+        "dw3": 25886017,
+        "pw3": 26132677,
+        "dw4": 16206570,
+        "pw4": 10235764,
+        "dw5": 13085401,
+        "pw5": 13540596,
+        "dw6": 8216572,
+        "pw6": 6180643,
+        "dw7": 6736907,
+        "pw7": 8934584,
+        "dw8": 6733324,
+        "pw8": 8931769,
+        "dw9": 6733708,
+        "pw9": 8932281,
+        "dw10": 6734988,
+        "pw10": 8931641,
+        "dw11": 6732557,
+        "pw11": 8932537,
+        "dw12": 4223300,
+        "pw12": 7106219,
+        "dw13": 3586967,
+        "pw13": 12327782,
+        "avgpool": 1687743,
+        "logits": 1453028,
+        "softmax": 127440
     },
     ("mobilenet_v1_1.0_224", 64): {
         "dw1": 51482293,
