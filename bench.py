@@ -167,7 +167,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs on ONE GPU; --gpus N with N > 1 is not supported "
-              "(the path shards by batch with no exchange step, see DESIGN.md).", file=sys.stderr)
+              "(the path shards by batch with no exchange step: one process per GPU would run the same plans on its slice).", file=sys.stderr)
         return 2
 
     from armnn_amd import nets, shim
