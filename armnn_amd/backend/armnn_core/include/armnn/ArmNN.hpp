@@ -1,11 +1,12 @@
+// Everything a client of the public API needs, in dependency order.
 #pragma once
-#include "BackendId.hpp"
-#include "BackendOptions.hpp"
-#include "BackendRegistry.hpp"
-#include "Descriptors.hpp"
+#include "Types.hpp"
 #include "Exceptions.hpp"
-#include "INetwork.hpp"
-#include "IRuntime.hpp"
 #include "Optional.hpp"
 #include "Tensor.hpp"
-#include "Types.hpp"
+#include "Descriptors.hpp"
+#include "BackendId.hpp"
+#include "BackendOptions.hpp"
+#include "INetwork.hpp"
+#include "IRuntime.hpp"
+#include <hostcore/BackendLifecycle.hpp>

@@ -1,6 +1,2 @@
 #pragma once
-namespace armnn
-{
-template <typename... Ts>
-inline void IgnoreUnused(Ts&&...) {}
-} // namespace armnn
+#include <hostcore/Utility.hpp>   // IgnoreUnused
