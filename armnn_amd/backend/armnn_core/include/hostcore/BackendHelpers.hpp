@@ -14,41 +14,48 @@
 
 namespace armnn
 {
+// Result of IBackendInternal::OptimizeSubgraphView.  A backend sorts the layers of the view it was given into four bins;
+// replacement layers are created through the private network the object owns, so they outlive the call.
 class OptimizationViews
 {
 public:
-    OptimizationViews(const NetworkOptions& networkOptions = {}) : m_INetwork(INetwork::Create(networkOptions)) {}
-    OptimizationViews(const OptimizationViews&) = delete;
-    OptimizationViews& operator=(const OptimizationViews&) = delete;
-    OptimizationViews(OptimizationViews&&) = default;
-    OptimizationViews& operator=(OptimizationViews&&) = default;
-
+    /// layers of the original graph to take out, and the layers (made through GetINetwork()) that go in their place
     struct SubstitutionPair
     {
-        SubgraphView m_SubstitutableSubgraph;   ///< layers of the original graph to take out
-        SubgraphView m_ReplacementSubgraph;     ///< layers created through GetINetwork() to put in their place
+        SubgraphView m_SubstitutableSubgraph;
+        SubgraphView m_ReplacementSubgraph;
     };
-    using Subgraphs = std::vector<SubgraphView>;
     using Substitutions = std::vector<SubstitutionPair>;
+    using Subgraphs = std::vector<SubgraphView>;
 
-    void AddSubstitution(SubstitutionPair&& substitution) { m_SuccesfulOptimizations.emplace_back(std::move(substitution)); }
-    void AddFailedSubgraph(SubgraphView&& subgraph) { m_FailedOptimizations.emplace_back(std::move(subgraph)); }
-    void AddUntouchedSubgraph(SubgraphView&& subgraph) { m_UntouchedSubgraphs.emplace_back(std::move(subgraph)); }
-    void AddDeletedSubgraph(SubgraphView&& subgraph) { m_DeletedSubgraphs.emplace_back(std::move(subgraph)); }
-    const Substitutions& GetSubstitutions() const { return m_SuccesfulOptimizations; }
-    const Subgraphs& GetFailedSubgraphs() const { return m_FailedOptimizations; }
-    const Subgraphs& GetUntouchedSubgraphs() const { return m_UntouchedSubgraphs; }
-    const Subgraphs& GetDeletedSubgraphs() const { return m_DeletedSubgraphs; }
-    Substitutions& GetSubstitutions() { return m_SuccesfulOptimizations; }
+    explicit OptimizationViews(const NetworkOptions& networkOptions = {});
+    OptimizationViews(OptimizationViews&&) = default;
+    OptimizationViews& operator=(OptimizationViews&&) = default;
+    OptimizationViews(const OptimizationViews&) = delete;
+    OptimizationViews& operator=(const OptimizationViews&) = delete;
+
+    // the four bins
+    void AddSubstitution(SubstitutionPair&& substitution);
+    void AddFailedSubgraph(SubgraphView&& subgraph);
+    void AddUntouchedSubgraph(SubgraphView&& subgraph);
+    void AddDeletedSubgraph(SubgraphView&& subgraph);
+    Substitutions& GetSubstitutions();
+    const Substitutions& GetSubstitutions() const;
+    const Subgraphs& GetFailedSubgraphs() const;
+    const Subgraphs& GetUntouchedSubgraphs() const;
+    const Subgraphs& GetDeletedSubgraphs() const;
+
+    /// true when every layer of `originalSubgraph` sits in exactly one bin and every substitution keeps its slot counts
     bool Validate(const SubgraphView& originalSubgraph) const;
-    INetwork* GetINetwork() { return m_INetwork.get(); }
-    INetwork& GetINetworkRef() { return *m_INetwork; }
+
+    /// where replacement layers are created
+    INetwork* GetINetwork();
+    INetwork& GetINetworkRef();
+
 private:
+    INetworkPtr m_INetwork;
     Substitutions m_SuccesfulOptimizations;
-    Subgraphs m_FailedOptimizations;
-    Subgraphs m_UntouchedSubgraphs;
-    Subgraphs m_DeletedSubgraphs;
-    INetworkPtr m_INetwork = INetworkPtr(nullptr, &INetwork::Destroy);
+    Subgraphs m_FailedOptimizations, m_UntouchedSubgraphs, m_DeletedSubgraphs;
 };
 
 class CopyMemGenericWorkload : public BaseWorkload<MemCopyQueueDescriptor>

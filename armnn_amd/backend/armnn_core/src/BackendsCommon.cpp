@@ -377,6 +377,19 @@ bool IWorkloadFactory::IsLayerSupported(const BackendId& backendId, const IConne
 }
 
 // ---- OptimizationViews (backendsCommon/OptimizationViews.cpp:11-75) ---------------------------------------------
+OptimizationViews::OptimizationViews(const NetworkOptions& networkOptions) : m_INetwork(INetwork::Create(networkOptions)) {}
+void OptimizationViews::AddSubstitution(SubstitutionPair&& substitution) { m_SuccesfulOptimizations.emplace_back(std::move(substitution)); }
+void OptimizationViews::AddFailedSubgraph(SubgraphView&& subgraph) { m_FailedOptimizations.emplace_back(std::move(subgraph)); }
+void OptimizationViews::AddUntouchedSubgraph(SubgraphView&& subgraph) { m_UntouchedSubgraphs.emplace_back(std::move(subgraph)); }
+void OptimizationViews::AddDeletedSubgraph(SubgraphView&& subgraph) { m_DeletedSubgraphs.emplace_back(std::move(subgraph)); }
+OptimizationViews::Substitutions& OptimizationViews::GetSubstitutions() { return m_SuccesfulOptimizations; }
+const OptimizationViews::Substitutions& OptimizationViews::GetSubstitutions() const { return m_SuccesfulOptimizations; }
+const OptimizationViews::Subgraphs& OptimizationViews::GetFailedSubgraphs() const { return m_FailedOptimizations; }
+const OptimizationViews::Subgraphs& OptimizationViews::GetUntouchedSubgraphs() const { return m_UntouchedSubgraphs; }
+const OptimizationViews::Subgraphs& OptimizationViews::GetDeletedSubgraphs() const { return m_DeletedSubgraphs; }
+INetwork* OptimizationViews::GetINetwork() { return m_INetwork.get(); }
+INetwork& OptimizationViews::GetINetworkRef() { return *m_INetwork; }
+
 bool OptimizationViews::Validate(const SubgraphView& original) const
 {
     std::multiset<const IConnectableLayer*> seen;
