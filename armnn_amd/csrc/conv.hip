@@ -524,6 +524,9 @@ int LaunchIgemmT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* 
     a.pad_top = g.pad_top; a.pad_left = g.pad_left; a.stride_x = g.stride_x; a.stride_y = g.stride_y;
     a.dil_x = g.dil_x; a.dil_y = g.dil_y;
     a.K_pad = p->K_pad;
+    a.unit = (g.Kh == 1 && g.Kw == 1 && g.stride_x == 1 && g.stride_y == 1 && g.pad_top == 0 && g.pad_left == 0 && g.Ho == g.H &&
+              g.Wo == g.W) ? 1 : 0;
+    if (a.unit) { a.H = 1; a.W = a.M; a.Ho = 1; a.Wo = a.M; }      // one row of M pixels
     a.tiles_m = static_cast<int>((M + BM - 1) / BM);
     a.tiles_n = (g.Co + BN - 1) / BN;
     a.xor_mask = p->xor_mask;
@@ -559,6 +562,9 @@ int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, voi
     a.pad_top = g.pad_top; a.pad_left = g.pad_left; a.stride_x = g.stride_x; a.stride_y = g.stride_y;
     a.dil_x = g.dil_x; a.dil_y = g.dil_y;
     a.K_pad = p->K_pad;
+    a.unit = (g.Kh == 1 && g.Kw == 1 && g.stride_x == 1 && g.stride_y == 1 && g.pad_top == 0 && g.pad_left == 0 && g.Ho == g.H &&
+              g.Wo == g.W) ? 1 : 0;
+    if (a.unit) { a.H = 1; a.W = a.M; a.Ho = 1; a.Wo = a.M; }      // one row of M pixels
     a.tiles_m = static_cast<int>((M + BM - 1) / BM);
     a.tiles_n = (g.Co + BN - 1) / BN;
     a.xor_mask = p->xor_mask;

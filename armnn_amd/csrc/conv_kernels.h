@@ -168,6 +168,7 @@ struct IgemmArgs
     int Kh, Kw;
     int pad_top, pad_left, stride_x, stride_y, dil_x, dil_y;
     int K_pad;
+    int unit;               // 1x1 kernel, stride 1, no padding: H = 1, W = M describe the input as one row of pixels
     int tiles_m, tiles_n;
     uint32_t xor_mask;      // 0x80808080 for uint8 input, else 0
     uint32_t pad_word;      // shifted input zero point replicated in 4 bytes
@@ -239,10 +240,20 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
         const int m = tm * BM + lr + RP * j;
         mvalid[j] = m < a.M;
         const int mm = mvalid[j] ? m : 0;
-        const int ox = mm % a.Wo;
-        const int t = mm / a.Wo;
-        const int oy = t % a.Ho;
-        const int n = t / a.Ho;
+        int n, oy, ox;
+        if (a.unit)
+        {
+            // 1x1, stride 1, no padding (and FullyConnected): output pixel m reads input pixel m, so the tensor is walked
+            // as one row of M pixels and the divisions below are not needed
+            n = 0; oy = 0; ox = mm;
+        }
+        else
+        {
+            ox = mm % a.Wo;
+            const int t = mm / a.Wo;
+            oy = t % a.Ho;
+            n = t / a.Ho;
+        }
         iy0[j] = oy * a.stride_y - a.pad_top;
         ix0[j] = ox * a.stride_x - a.pad_left;
         xrow[j] = a.x + static_cast<long long>(n) * a.H * a.W * a.Ci;

@@ -87,10 +87,20 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
         const int m = tm * BM + wave * (BM / NW) + j * 8 + lrow;
         mvalid[j] = m < a.M;
         const int mm = mvalid[j] ? m : 0;
-        const int ox = mm % a.Wo;
-        const int t = mm / a.Wo;
-        const int oy = t % a.Ho;
-        const int n = t / a.Ho;
+        int n, oy, ox;
+        if (a.unit)
+        {
+            // 1x1, stride 1, no padding (and FullyConnected): output pixel m reads input pixel m, so the tensor is walked
+            // as one row of M pixels and the divisions below are not needed
+            n = 0; oy = 0; ox = mm;
+        }
+        else
+        {
+            ox = mm % a.Wo;
+            const int t = mm / a.Wo;
+            oy = t % a.Ho;
+            n = t / a.Ho;
+        }
         iy0[j] = oy * a.stride_y - a.pad_top;
         ix0[j] = ox * a.stride_x - a.pad_left;
         // the chunk this lane would fetch for tap (0, 0), channel 0 (outside the tensor when that tap is padding; such
