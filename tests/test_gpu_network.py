@@ -103,3 +103,40 @@ def test_mobilenet_v1_batch64_rows_equal_batch2_runs():
 
 def test_resnet50_batch32_rows_equal_batch2_runs():
     _rows_equal_small_batch_runs(nets.resnet50(), 32, (0, 15, 30), lanes=2)
+
+
+def test_two_threads_run_two_networks_at_once():
+    """The library is re-entrant per stream: two host threads, each with its own network, plans, buffers and stream,
+    give the bytes they give when run one after the other."""
+    import threading
+
+    nets_and_batches = [(nets.mobilenet_v1(resolution=96, classes=50), 4), (nets.resnet50(resolution=64), 2)]
+    inputs = [nets.synthetic_input(n, b, seed=21 + i) for i, (n, b) in enumerate(nets_and_batches)]
+    want = []
+    for (n, b), x in zip(nets_and_batches, inputs):
+        dn = DeviceNetwork(n, b, use_graph=False)
+        want.append(dn.run(x).data.copy())
+        dn.close()
+    got, errors = [None, None], []
+
+    def worker(k):
+        try:
+            n, b = nets_and_batches[k]
+            dn = DeviceNetwork(n, b, use_graph=(k == 0), lanes=2)
+            for _ in range(5):
+                out = dn.run(inputs[k]).data.copy()
+                np.testing.assert_array_equal(out, want[k])
+            got[k] = out
+            dn.close()
+        except Exception as e:      # reported by the main thread
+            errors.append((k, repr(e)))
+
+    threads = [threading.Thread(target=worker, args=(k,)) for k in range(2)]
+    for t in threads:
+        t.start()
+    for t in threads:
+        t.join(timeout=240)
+    assert not errors, errors
+    assert all(not t.is_alive() for t in threads)
+    for k in range(2):
+        np.testing.assert_array_equal(got[k], want[k])
