@@ -6,6 +6,7 @@
 #include "Types.hpp"
 #include <memory>
 #include <string>
+#include <vector>
 
 namespace armnn
 {
@@ -46,7 +47,20 @@ public:
                        const INetworkProperties& networkProperties);
     TensorInfo GetInputTensorInfo(NetworkId networkId, LayerBindingId layerId) const;
     TensorInfo GetOutputTensorInfo(NetworkId networkId, LayerBindingId layerId) const;
-    Status EnqueueWorkload(NetworkId networkId, const InputTensors& inputTensors, const OutputTensors& outputTensors);
+    /// Lets the tensor handles bound to the given inputs / outputs adopt the caller's memory once, for use in any number
+    /// of EnqueueWorkload calls.  Returns the indices (in the order of the network's input / output layers) that were
+    /// adopted; a tensor the backend cannot adopt is left out, not reported as an error.  MemorySource::Undefined throws
+    /// MemoryImportException.
+    std::vector<ImportedInputId> ImportInputs(NetworkId networkId, const InputTensors& inputTensors,
+                                              MemorySource forceImportMemorySource = MemorySource::Undefined);
+    std::vector<ImportedOutputId> ImportOutputs(NetworkId networkId, const OutputTensors& outputTensors,
+                                                MemorySource forceImportMemorySource = MemorySource::Undefined);
+    void ClearImportedInputs(NetworkId networkId, const std::vector<ImportedInputId> inputIds);
+    void ClearImportedOutputs(NetworkId networkId, const std::vector<ImportedOutputId> outputIds);
+    /// inputs / outputs named in the pre-imported id lists are not passed again in the tensor lists
+    Status EnqueueWorkload(NetworkId networkId, const InputTensors& inputTensors, const OutputTensors& outputTensors,
+                           std::vector<ImportedInputId> preImportedInputIds = {},
+                           std::vector<ImportedOutputId> preImportedOutputIds = {});
     Status UnloadNetwork(NetworkId networkId);
     const IDeviceSpec& GetDeviceSpec() const;
     ~IRuntime();

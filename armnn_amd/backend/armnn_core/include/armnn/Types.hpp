@@ -43,6 +43,8 @@ enum class LayerType
 const char* GetLayerTypeAsCString(LayerType type);
 
 using NetworkId = int;
+using ImportedInputId = unsigned int;
+using ImportedOutputId = unsigned int;
 using LayerBindingId = int;
 using LayerGuid = uint64_t;
 

@@ -1,5 +1,6 @@
 // Minimal host core: IRuntime -- backend discovery, LoadNetwork (tensor handles, workloads, constants), and
 // EnqueueWorkload (src/armnn/Runtime.cpp:301-574, src/armnn/LoadedNetwork.cpp:82-360 and :845-1100).
+#include <algorithm>
 #include <Layer.hpp>
 #include <armnn/BackendRegistry.hpp>
 #include <armnn/IRuntime.hpp>
@@ -103,6 +104,13 @@ public:
         for (auto& b : m_Backends) b.second.factory->AfterWorkloadsCreated();
         // constant layers produce their output once (LoadedNetwork.cpp:342-357)
         for (auto& w : m_Constants) w->Execute();
+        for (Layer* l : m_Order)
+        {
+            Binding b;
+            b.layer = l;
+            if (l->GetType() == LayerType::Input) { b.slot = &l->Out(0); m_Inputs.push_back(std::move(b)); }
+            else if (l->GetType() == LayerType::Output) { b.slot = const_cast<OutputSlot*>(l->In(0).GetConnectedOutputSlot()); m_Outputs.push_back(std::move(b)); }
+        }
     }
 
     ~LoadedNetwork()
@@ -132,11 +140,20 @@ public:
         return l->In(0).GetConnectedOutputSlot()->GetTensorInfo();
     }
 
-    Status Enqueue(const InputTensors& inputs, const OutputTensors& outputs)
+    Status Enqueue(const InputTensors& inputs, const OutputTensors& outputs, const std::vector<ImportedInputId>& preIn = {},
+                   const std::vector<ImportedOutputId>& preOut = {})
     {
-        if (inputs.size() != m_Net->GetNumInputs()) throw InvalidArgumentException("Number of inputs provided does not match network.");
-        if (outputs.size() != m_Net->GetNumOutputs()) throw InvalidArgumentException("Number of outputs provided does not match network.");
+        // a tensor comes either in the list or pre-imported; together they must cover the network (LoadedNetwork.cpp:800-806)
+        if (inputs.size() + preIn.size() != m_Net->GetNumInputs()) throw InvalidArgumentException("Number of inputs provided does not match network.");
+        if (outputs.size() + preOut.size() != m_Net->GetNumOutputs()) throw InvalidArgumentException("Number of outputs provided does not match network.");
         std::lock_guard<std::mutex> lock(m_Mutex);
+        for (ImportedInputId id : preIn)
+            if (id >= m_Inputs.size() || !m_Inputs[id].adopted) throw InvalidArgumentException("EnqueueWorkload: input " + std::to_string(id) + " was not imported");
+        for (ImportedOutputId id : preOut)
+            if (id >= m_Outputs.size() || !m_Outputs[id].adopted) throw InvalidArgumentException("EnqueueWorkload: output " + std::to_string(id) + " was not imported");
+        // workloads read adopted memory for the ids named in this call and the network's own tensors for the rest
+        for (unsigned int i = 0; i < m_Inputs.size(); ++i) Point(m_Inputs[i], std::find(preIn.begin(), preIn.end(), i) != preIn.end());
+        for (unsigned int i = 0; i < m_Outputs.size(); ++i) Point(m_Outputs[i], std::find(preOut.begin(), preOut.end(), i) != preOut.end());
         for (const auto& in : inputs)
         {
             const Layer* l = FindBinding(LayerType::Input, in.first);
@@ -159,6 +176,13 @@ public:
             const void* p = h->Map();
             std::memcpy(out.second.GetMemoryArea(), p, src->GetTensorInfo().GetNumBytes());
             h->Unmap();
+        }
+        // an adopted output is complete once its handle has been mapped: that is where a device backend waits for its
+        // queue (the SyncMemGeneric workload of LoadedNetwork.cpp:905-918)
+        for (ImportedOutputId id : preOut)
+        {
+            m_Outputs[id].imported->Map(true);
+            m_Outputs[id].imported->Unmap();
         }
         return Status::Success;
     }
@@ -231,8 +255,127 @@ private:
         if (!w)
             throw RuntimeException(std::string("No workload created for layer (name: '") + l.GetName() + "' type: '" +
                                    GetLayerTypeAsCString(l.GetType()) + "' backend: '" + l.GetBackendId().Get() + "')");
+        m_WorkloadOf[&l] = m_Workloads.size();
         m_Workloads.push_back(std::move(w));
     }
+
+    // ---- pre-imported inputs and outputs (LoadedNetwork.cpp:1402-1560 and :796-960) ---------------------------------
+    struct Binding
+    {
+        Layer* layer = nullptr;                               // the Input / Output layer
+        OutputSlot* slot = nullptr;                           // the tensor it binds
+        std::unique_ptr<ITensorHandle> imported;              // handle that adopts caller memory (created on first use)
+        bool adopted = false;                                 // Import() succeeded and has not been cleared
+        bool inUse = false;                                   // the workloads currently point at `imported`
+    };
+
+    // workloads (with the slot index) that read / write `slot`
+    std::vector<std::pair<IWorkload*, unsigned int>> Readers(const OutputSlot& slot) const
+    {
+        std::vector<std::pair<IWorkload*, unsigned int>> r;
+        for (InputSlot* c : slot.GetConnections())
+        {
+            auto it = m_WorkloadOf.find(&c->GetOwningLayer());
+            if (it != m_WorkloadOf.end()) r.emplace_back(m_Workloads[it->second].get(), c->GetSlotIndex());
+        }
+        return r;
+    }
+    std::pair<IWorkload*, unsigned int> Writer(const OutputSlot& slot) const
+    {
+        auto it = m_WorkloadOf.find(&slot.GetOwningLayer());
+        if (it == m_WorkloadOf.end()) return {nullptr, 0u};
+        return {m_Workloads[it->second].get(), slot.CalculateIndexOnOwner()};
+    }
+
+    void Point(Binding& b, bool toImported)
+    {
+        if (b.inUse == toImported) return;
+        ITensorHandle* h = toImported ? b.imported.get() : b.slot->GetTensorHandle();
+        if (b.layer->GetType() == LayerType::Output)
+        {
+            const auto w = Writer(*b.slot);
+            if (w.first) w.first->ReplaceOutputTensorHandle(h, w.second);
+        }
+        for (const auto& r : Readers(*b.slot)) r.first->ReplaceInputTensorHandle(h, r.second);
+        b.inUse = toImported;
+    }
+
+    bool TryImport(Binding& b, void* memory, MemorySource source)
+    {
+        // the tensor must be produced and consumed by workloads that accept another handle
+        const bool isOutput = b.layer->GetType() == LayerType::Output;
+        if (isOutput)
+        {
+            const auto w = Writer(*b.slot);
+            if (!w.first || !w.first->SupportsTensorHandleReplacement()) return false;
+        }
+        for (const auto& r : Readers(*b.slot))
+            if (!r.first->SupportsTensorHandleReplacement()) return false;
+        if (!b.imported)
+        {
+            const Layer& owner = isOutput ? b.slot->GetOwningLayer() : b.slot->GetConnections().empty() ? *b.layer : b.slot->GetConnections().front()->GetOwningLayer();
+            BackendSlot& bs = m_Backends.at(owner.GetBackendId());
+            if (!bs.handleFactory || (bs.handleFactory->GetImportFlags() & static_cast<MemorySourceFlags>(source)) == 0) return false;
+            b.imported = bs.handleFactory->CreateTensorHandle(b.slot->GetTensorInfo(), false);
+            if (!b.imported) return false;
+        }
+        try
+        {
+            if (b.adopted) { Point(b, false); b.imported->Unimport(); b.adopted = false; }
+            if (b.imported->CanBeImported(memory, source) && b.imported->Import(memory, source)) b.adopted = true;
+        }
+        catch (const MemoryImportException& e)
+        {
+            std::cerr << "armnn: an error occurred attempting to import a tensor: " << e.what() << "\n";
+        }
+        return b.adopted;
+    }
+
+public:
+    std::vector<ImportedInputId> ImportInputs(const InputTensors& inputs, MemorySource source)
+    {
+        if (source == MemorySource::Undefined) throw MemoryImportException("ImportInputs: Memory Import failed, no memory source given");
+        if (inputs.size() > m_Inputs.size()) throw MemoryImportException("ImportInputs: The number of tensors provided exceeds the number of inputs.");
+        std::lock_guard<std::mutex> lock(m_Mutex);
+        std::vector<ImportedInputId> ids;
+        for (unsigned int i = 0; i < m_Inputs.size(); ++i)
+            for (const auto& t : inputs)
+                if (t.first == m_Inputs[i].layer->GetBindingId() && t.second.GetNumBytes() == m_Inputs[i].slot->GetTensorInfo().GetNumBytes() &&
+                    TryImport(m_Inputs[i], const_cast<void*>(t.second.GetMemoryArea()), source))
+                    ids.push_back(i);
+        return ids;
+    }
+
+    std::vector<ImportedOutputId> ImportOutputs(const OutputTensors& outputs, MemorySource source)
+    {
+        if (source == MemorySource::Undefined) throw MemoryImportException("ImportOutputs: Memory Import failed, no memory source given");
+        if (outputs.size() > m_Outputs.size()) throw MemoryImportException("ImportOutputs: The number of tensors provided exceeds the number of outputs.");
+        std::lock_guard<std::mutex> lock(m_Mutex);
+        std::vector<ImportedOutputId> ids;
+        for (unsigned int i = 0; i < m_Outputs.size(); ++i)
+            for (const auto& t : outputs)
+                if (t.first == m_Outputs[i].layer->GetBindingId() && t.second.GetNumBytes() == m_Outputs[i].slot->GetTensorInfo().GetNumBytes() &&
+                    TryImport(m_Outputs[i], t.second.GetMemoryArea(), source))
+                    ids.push_back(i);
+        return ids;
+    }
+
+    void ClearImported(bool inputs, const std::vector<unsigned int>& ids)
+    {
+        std::lock_guard<std::mutex> lock(m_Mutex);
+        std::vector<Binding>& all = inputs ? m_Inputs : m_Outputs;
+        for (unsigned int id : ids)
+        {
+            if (id >= all.size() || !all[id].adopted) throw InvalidArgumentException("ClearImported: id " + std::to_string(id) + " is not an imported tensor");
+            Point(all[id], false);
+            all[id].imported->Unimport();
+            all[id].adopted = false;
+        }
+    }
+
+private:
+    std::vector<Binding> m_Inputs, m_Outputs;                 // in the order of the network's Input / Output layers
+    std::map<const Layer*, size_t> m_WorkloadOf;
 
     IOptimizedNetworkPtr m_Net;
     std::vector<Layer*> m_Order;
@@ -303,13 +446,14 @@ public:
         return *it->second;
     }
 
-    Status Enqueue(NetworkId id, const InputTensors& in, const OutputTensors& out)
+    Status Enqueue(NetworkId id, const InputTensors& in, const OutputTensors& out, const std::vector<ImportedInputId>& preIn = {},
+                   const std::vector<ImportedOutputId>& preOut = {})
     {
         LoadedNetwork& net = Get(id);
         Status s = Status::Failure;
         try
         {
-            s = net.Enqueue(in, out);
+            s = net.Enqueue(in, out, preIn, preOut);
         }
         catch (const RuntimeException& e)
         {
@@ -353,7 +497,15 @@ Status IRuntime::LoadNetwork(NetworkId& id, IOptimizedNetworkPtr network, std::s
 }
 TensorInfo IRuntime::GetInputTensorInfo(NetworkId id, LayerBindingId layerId) const { return pRuntimeImpl->Get(id).GetInputTensorInfo(layerId); }
 TensorInfo IRuntime::GetOutputTensorInfo(NetworkId id, LayerBindingId layerId) const { return pRuntimeImpl->Get(id).GetOutputTensorInfo(layerId); }
-Status IRuntime::EnqueueWorkload(NetworkId id, const InputTensors& in, const OutputTensors& out) { return pRuntimeImpl->Enqueue(id, in, out); }
+Status IRuntime::EnqueueWorkload(NetworkId id, const InputTensors& in, const OutputTensors& out, std::vector<ImportedInputId> preIn,
+                                 std::vector<ImportedOutputId> preOut)
+{
+    return pRuntimeImpl->Enqueue(id, in, out, preIn, preOut);
+}
+std::vector<ImportedInputId> IRuntime::ImportInputs(NetworkId id, const InputTensors& in, MemorySource source) { return pRuntimeImpl->Get(id).ImportInputs(in, source); }
+std::vector<ImportedOutputId> IRuntime::ImportOutputs(NetworkId id, const OutputTensors& out, MemorySource source) { return pRuntimeImpl->Get(id).ImportOutputs(out, source); }
+void IRuntime::ClearImportedInputs(NetworkId id, const std::vector<ImportedInputId> ids) { pRuntimeImpl->Get(id).ClearImported(true, ids); }
+void IRuntime::ClearImportedOutputs(NetworkId id, const std::vector<ImportedOutputId> ids) { pRuntimeImpl->Get(id).ClearImported(false, ids); }
 Status IRuntime::UnloadNetwork(NetworkId id) { return pRuntimeImpl->Unload(id); }
 const IDeviceSpec& IRuntime::GetDeviceSpec() const { return pRuntimeImpl->m_DeviceSpec; }
 } // namespace armnn

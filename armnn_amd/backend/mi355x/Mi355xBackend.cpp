@@ -103,7 +103,7 @@ BackendCapabilities Mi355xBackend::GetCapabilities() const
                                                    {"AsyncExecution", false},
                                                    {"ProtectedContentAllocation", false},
                                                    {"ConstantTensorsAsInputs", true},
-                                                   {"PreImportIOTensors", false},
+                                                   {"PreImportIOTensors", true},
                                                    {"ExternallyManagedMemory", false},
                                                    {"MultiAxisPacking", false},
                                                    {"SingleAxisPacking", false}});

@@ -3,6 +3,7 @@
 
 #include <armnn/backends/TensorHandle.hpp>
 
+#include <cstdint>
 #include <cstring>
 
 namespace armnn
@@ -42,8 +43,55 @@ void Mi355xTensorHandle::Allocate()
     mi355x::Check(mi355x_malloc(&m_Owned, bytes), "mi355x_malloc");
 }
 
+bool Mi355xTensorHandle::CanBeImported(void* memory, MemorySource source)
+{
+    if (source != MemorySource::Malloc || m_Managed || !memory) return false;
+    if (reinterpret_cast<uintptr_t>(memory) % 16 != 0) return false;          // the kernels' vector loads and stores
+    if (mi355x::DeviceCount() == 0) return false;
+    void* device = nullptr;
+    int isDevice = 0;
+    return mi355x_host_device_pointer(memory, &device, &isDevice) == 0 && device != nullptr;
+}
+
+bool Mi355xTensorHandle::Import(void* memory, MemorySource source)
+{
+    if (m_Managed) throw MemoryImportException("Mi355xTensorHandle::Import: a tensor that lives in the arena cannot adopt caller memory");
+    if (source != MemorySource::Malloc) return false;
+    if (!memory) throw MemoryImportException("Mi355xTensorHandle::Import: null memory");
+    if (reinterpret_cast<uintptr_t>(memory) % 16 != 0) throw MemoryImportException("Mi355xTensorHandle::Import: memory is not 16-byte aligned");
+    mi355x::EnsureDevice();
+    void* device = nullptr;
+    int isDevice = 0;
+    if (mi355x_host_device_pointer(memory, &device, &isDevice) != 0 || !device) return false;
+    m_ImportedIsDeviceMemory = isDevice != 0;
+    if (!m_Owned && !m_ImportedIsDeviceMemory) mi355x::Check(mi355x_malloc(&m_Owned, m_Info.GetNumBytes() ? m_Info.GetNumBytes() : 1), "mi355x_malloc");
+    m_ImportedHost = memory;
+    m_ImportedDevice = device;
+    m_DeviceNewer = false;
+    return true;
+}
+
+void Mi355xTensorHandle::Unimport()
+{
+    if (m_ImportedDevice) mi355x::Synchronize();       // no kernel may still be using the caller's memory
+    m_ImportedHost = nullptr;
+    m_ImportedDevice = nullptr;
+    m_ImportedIsDeviceMemory = false;
+}
+
+const void* Mi355xTensorHandle::GetDevicePointerForRead() const
+{
+    void* dev = GetDevicePointer();
+    // adopted buffer, not written by a workload since the caller last saw it: it is an input, and whatever the caller
+    // has put there is what this inference reads
+    if (m_ImportedDevice && !m_ImportedIsDeviceMemory && !m_DeviceNewer && m_Info.GetNumBytes())
+        mi355x::Check(mi355x_memcpy_h2d(dev, m_ImportedDevice, m_Info.GetNumBytes(), mi355x::Stream()), "mi355x_memcpy_h2d (adopted buffer)");
+    return dev;
+}
+
 void* Mi355xTensorHandle::GetDevicePointer() const
 {
+    if (m_ImportedDevice && m_ImportedIsDeviceMemory) return m_ImportedDevice;
     if (m_Managed)
     {
         if (!m_Reserved) throw NullPointerException("Mi355xTensorHandle: managed tensor was never given a lifetime (Manage)");
@@ -57,6 +105,18 @@ TensorShape Mi355xTensorHandle::GetStrides() const { return GetUnpaddedTensorStr
 
 const void* Mi355xTensorHandle::Map(bool /*blocking*/) const
 {
+    if (m_ImportedDevice)
+    {
+        // results go straight into the caller's buffer; either way the host waits for what is queued
+        if (m_MapCount++ == 0)
+        {
+            if (m_DeviceNewer && !m_ImportedIsDeviceMemory && m_Info.GetNumBytes())
+                mi355x::Check(mi355x_memcpy_d2h(m_ImportedDevice, GetDevicePointer(), m_Info.GetNumBytes(), mi355x::Stream()), "mi355x_memcpy_d2h (adopted buffer)");
+            mi355x::Synchronize();
+            m_DeviceNewer = false;
+        }
+        return m_ImportedHost;
+    }
     void* dev = GetDevicePointer();
     const size_t bytes = m_Info.GetNumBytes();
     if (!m_Staging) mi355x::Check(mi355x_host_alloc(&m_Staging, bytes ? bytes : 1), "mi355x_host_alloc");
@@ -79,6 +139,7 @@ void Mi355xTensorHandle::Unmap() const
 {
     if (m_MapCount == 0) return;
     if (--m_MapCount != 0) return;
+    if (m_ImportedDevice) return;
     const size_t bytes = m_Info.GetNumBytes();
     if (!bytes) return;
     // the pinned copy stays alive with the handle, so the upload may complete asynchronously in stream order

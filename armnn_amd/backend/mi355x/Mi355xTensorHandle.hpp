@@ -8,6 +8,14 @@
 // CopyMemGenericWorkload and of the runtime's input/output binding works unchanged
 // (RefTensorHandle::Map/CopyInFrom/CopyOutTo, src/backends/reference/RefTensorHandle.cpp:45-133, are the host-memory
 // counterparts).  Workloads call MarkDeviceWritten() on their outputs.
+//
+// An unmanaged handle can instead adopt caller memory the copy engines reach directly -- pinned host memory or device
+// memory (Import with MemorySource::Malloc; pageable memory is refused).  The caller's buffer then takes the place of the
+// staging copy: a workload that reads the tensor before any workload wrote it gets the buffer's current contents by one
+// asynchronous transfer, and Map() brings results back into the buffer and waits -- no host-side memcpy on either side
+// (RefTensorHandle::Import, src/backends/reference/RefTensorHandle.cpp:135-165, is the host-memory counterpart).
+// Kernels do not read pinned host memory in place: a convolution reading its input across the bus proved slower than
+// the transfer.  Adopted device memory is used in place.
 #pragma once
 #include "Mi355xBackendId.hpp"
 #include "Mi355xMemoryManager.hpp"
@@ -34,10 +42,16 @@ public:
     TensorShape GetShape() const override { return m_Info.GetShape(); }
     void CopyOutTo(void* memory) const override;
     void CopyInFrom(const void* memory) override;
+    unsigned int GetImportFlags() const override { return static_cast<unsigned int>(MemorySource::Malloc); }
+    bool CanBeImported(void* memory, MemorySource source) override;
+    bool Import(void* memory, MemorySource source) override;
+    void Unimport() override;
 
     const TensorInfo& GetTensorInfo() const { return m_Info; }
     /// device address; throws NullPointerException when the tensor has no memory yet
     void* GetDevicePointer() const;
+    /// device address for a workload that reads the tensor: refreshes an adopted buffer's device copy first
+    const void* GetDevicePointerForRead() const;
     void MarkDeviceWritten() const { m_DeviceNewer = true; }
     bool IsManaged() const { return m_Managed; }
 
@@ -49,6 +63,9 @@ private:
     bool m_Retired = false;
     size_t m_Offset = 0;
     void* m_Owned = nullptr;            // unmanaged handles
+    void* m_ImportedHost = nullptr;     // caller memory adopted by Import(), as the caller addresses it ...
+    void* m_ImportedDevice = nullptr;   // ... and as the device does
+    bool m_ImportedIsDeviceMemory = false;   // adopted device memory is used in place, without transfers
     mutable void* m_Staging = nullptr;  // pinned host copy, created by the first Map()
     mutable bool m_DeviceNewer = false;
     mutable bool m_UploadInFlight = false;
@@ -69,8 +86,8 @@ public:
     static const FactoryId& GetIdStatic();
     const FactoryId& GetId() const override { return GetIdStatic(); }
     bool SupportsSubTensors() const override { return false; }
-    MemorySourceFlags GetExportFlags() const override { return 0; }
-    MemorySourceFlags GetImportFlags() const override { return 0; }
+    MemorySourceFlags GetExportFlags() const override { return static_cast<MemorySourceFlags>(MemorySource::Malloc); }
+    MemorySourceFlags GetImportFlags() const override { return static_cast<MemorySourceFlags>(MemorySource::Malloc); }
     const std::shared_ptr<Mi355xMemoryManager>& GetMemoryManager() const { return m_MemoryManager; }
 private:
     std::shared_ptr<Mi355xMemoryManager> m_MemoryManager;

@@ -18,7 +18,7 @@ const Mi355xTensorHandle& Dev(const ITensorHandle* h)
     if (!d) throw InvalidArgumentException("Mi355x workload: operand is not a device tensor handle");
     return *d;
 }
-const void* In(const ITensorHandle* h) { return Dev(h).GetDevicePointer(); }
+const void* In(const ITensorHandle* h) { return Dev(h).GetDevicePointerForRead(); }
 void* Out(ITensorHandle* h)
 {
     const Mi355xTensorHandle& d = Dev(h);
@@ -66,7 +66,7 @@ Mi355xFusedActivation Mi355xFusedActivation::From(const ActivationDescriptor* d)
 
 // ---- Convolution2d ---------------------------------------------------------------------------------------------------
 Mi355xConvolution2dWorkload::Mi355xConvolution2dWorkload(const Convolution2dQueueDescriptor& descriptor, const WorkloadInfo& info)
-    : BaseWorkload<Convolution2dQueueDescriptor>(descriptor, info), m_Info(info)
+    : Mi355xBaseWorkload<Convolution2dQueueDescriptor>(descriptor, info), m_Info(info)
 {
     if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xConvolution2dWorkload: NHWC only");
     Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());   // validates early
@@ -128,7 +128,7 @@ std::string Mi355xConvolution2dWorkload::GetKernelDescription() const
 
 // ---- DepthwiseConvolution2d ------------------------------------------------------------------------------------------
 Mi355xDepthwiseConvolution2dWorkload::Mi355xDepthwiseConvolution2dWorkload(const DepthwiseConvolution2dQueueDescriptor& descriptor, const WorkloadInfo& info)
-    : BaseWorkload<DepthwiseConvolution2dQueueDescriptor>(descriptor, info), m_Info(info)
+    : Mi355xBaseWorkload<DepthwiseConvolution2dQueueDescriptor>(descriptor, info), m_Info(info)
 {
     if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xDepthwiseConvolution2dWorkload: NHWC only");
     Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
@@ -181,7 +181,7 @@ void Mi355xDepthwiseConvolution2dWorkload::Execute() const
 
 // ---- FullyConnected --------------------------------------------------------------------------------------------------
 Mi355xFullyConnectedWorkload::Mi355xFullyConnectedWorkload(const FullyConnectedQueueDescriptor& descriptor, const WorkloadInfo& info)
-    : BaseWorkload<FullyConnectedQueueDescriptor>(descriptor, info), m_Info(info)
+    : Mi355xBaseWorkload<FullyConnectedQueueDescriptor>(descriptor, info), m_Info(info)
 {
     Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
 }
@@ -229,7 +229,7 @@ void Mi355xFullyConnectedWorkload::Execute() const
 
 // ---- Activation ------------------------------------------------------------------------------------------------------
 Mi355xActivationWorkload::Mi355xActivationWorkload(const ActivationQueueDescriptor& descriptor, const WorkloadInfo& info)
-    : BaseWorkload<ActivationQueueDescriptor>(descriptor, info), m_Info(info)
+    : Mi355xBaseWorkload<ActivationQueueDescriptor>(descriptor, info), m_Info(info)
 {
     Mi355xFusedActivation::From(&m_Data.m_Parameters);
 }
@@ -246,7 +246,7 @@ void Mi355xActivationWorkload::Execute() const
 
 // ---- Pooling2d -------------------------------------------------------------------------------------------------------
 Mi355xPooling2dWorkload::Mi355xPooling2dWorkload(const Pooling2dQueueDescriptor& descriptor, const WorkloadInfo& info)
-    : BaseWorkload<Pooling2dQueueDescriptor>(descriptor, info), m_Info(info)
+    : Mi355xBaseWorkload<Pooling2dQueueDescriptor>(descriptor, info), m_Info(info)
 {
     if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xPooling2dWorkload: NHWC only");
 }
@@ -270,7 +270,7 @@ void Mi355xPooling2dWorkload::Execute() const
 
 // ---- Softmax ---------------------------------------------------------------------------------------------------------
 Mi355xSoftmaxWorkload::Mi355xSoftmaxWorkload(const SoftmaxQueueDescriptor& descriptor, const WorkloadInfo& info)
-    : BaseWorkload<SoftmaxQueueDescriptor>(descriptor, info), m_Info(info)
+    : Mi355xBaseWorkload<SoftmaxQueueDescriptor>(descriptor, info), m_Info(info)
 {
 }
 
@@ -288,7 +288,7 @@ void Mi355xSoftmaxWorkload::Execute() const
 
 // ---- Add -------------------------------------------------------------------------------------------------------------
 Mi355xAdditionWorkload::Mi355xAdditionWorkload(const ElementwiseBinaryQueueDescriptor& descriptor, const WorkloadInfo& info)
-    : BaseWorkload<ElementwiseBinaryQueueDescriptor>(descriptor, info), m_Info(info)
+    : Mi355xBaseWorkload<ElementwiseBinaryQueueDescriptor>(descriptor, info), m_Info(info)
 {
     if (m_Data.m_Parameters.m_Operation != BinaryOperation::Add) throw InvalidArgumentException("Mi355xAdditionWorkload: Add only");
     Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
@@ -307,7 +307,7 @@ void Mi355xAdditionWorkload::Execute() const
 
 // ---- Reshape ---------------------------------------------------------------------------------------------------------
 Mi355xReshapeWorkload::Mi355xReshapeWorkload(const ReshapeQueueDescriptor& descriptor, const WorkloadInfo& info)
-    : BaseWorkload<ReshapeQueueDescriptor>(descriptor, info), m_Info(info)
+    : Mi355xBaseWorkload<ReshapeQueueDescriptor>(descriptor, info), m_Info(info)
 {
 }
 
@@ -320,7 +320,7 @@ void Mi355xReshapeWorkload::Execute() const
 
 // ---- Constant --------------------------------------------------------------------------------------------------------
 Mi355xConstantWorkload::Mi355xConstantWorkload(const ConstantQueueDescriptor& descriptor, const WorkloadInfo& info)
-    : BaseWorkload<ConstantQueueDescriptor>(descriptor, info)
+    : Mi355xBaseWorkload<ConstantQueueDescriptor>(descriptor, info)
 {
 }
 

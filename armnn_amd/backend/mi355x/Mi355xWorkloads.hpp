@@ -22,8 +22,20 @@ struct Mi355xFusedActivation
     static Mi355xFusedActivation From(const ActivationDescriptor* descriptor);
 };
 
+/// Every workload here reads its tensor handles when it executes, so the runtime may swap a handle for one that adopted
+/// caller memory (pre-imported inputs and outputs; RefBaseWorkload, src/backends/reference/workloads/RefBaseWorkload.hpp:13-35).
+template <typename QueueDescriptor>
+class Mi355xBaseWorkload : public BaseWorkload<QueueDescriptor>
+{
+public:
+    using BaseWorkload<QueueDescriptor>::BaseWorkload;
+    bool SupportsTensorHandleReplacement() const override { return true; }
+    void ReplaceInputTensorHandle(ITensorHandle* tensorHandle, unsigned int slot) override { this->m_Data.m_Inputs[slot] = tensorHandle; }
+    void ReplaceOutputTensorHandle(ITensorHandle* tensorHandle, unsigned int slot) override { this->m_Data.m_Outputs[slot] = tensorHandle; }
+};
+
 /// counterpart of RefConvolution2dWorkload (RefConvolution2dWorkload.cpp:38-58)
-class Mi355xConvolution2dWorkload : public BaseWorkload<Convolution2dQueueDescriptor>
+class Mi355xConvolution2dWorkload : public Mi355xBaseWorkload<Convolution2dQueueDescriptor>
 {
 public:
     Mi355xConvolution2dWorkload(const Convolution2dQueueDescriptor& descriptor, const WorkloadInfo& info);
@@ -39,7 +51,7 @@ private:
 };
 
 /// counterpart of RefDepthwiseConvolution2dWorkload (RefDepthwiseConvolution2dWorkload.cpp:38-62)
-class Mi355xDepthwiseConvolution2dWorkload : public BaseWorkload<DepthwiseConvolution2dQueueDescriptor>
+class Mi355xDepthwiseConvolution2dWorkload : public Mi355xBaseWorkload<DepthwiseConvolution2dQueueDescriptor>
 {
 public:
     Mi355xDepthwiseConvolution2dWorkload(const DepthwiseConvolution2dQueueDescriptor& descriptor, const WorkloadInfo& info);
@@ -53,7 +65,7 @@ private:
 };
 
 /// counterpart of RefFullyConnectedWorkload (RefFullyConnectedWorkload.cpp:39-67)
-class Mi355xFullyConnectedWorkload : public BaseWorkload<FullyConnectedQueueDescriptor>
+class Mi355xFullyConnectedWorkload : public Mi355xBaseWorkload<FullyConnectedQueueDescriptor>
 {
 public:
     Mi355xFullyConnectedWorkload(const FullyConnectedQueueDescriptor& descriptor, const WorkloadInfo& info);
@@ -67,7 +79,7 @@ private:
 };
 
 /// counterpart of RefActivationWorkload (RefActivationWorkload.cpp:23-36)
-class Mi355xActivationWorkload : public BaseWorkload<ActivationQueueDescriptor>
+class Mi355xActivationWorkload : public Mi355xBaseWorkload<ActivationQueueDescriptor>
 {
 public:
     Mi355xActivationWorkload(const ActivationQueueDescriptor& descriptor, const WorkloadInfo& info);
@@ -77,7 +89,7 @@ private:
 };
 
 /// counterpart of RefPooling2dWorkload (RefPooling2dWorkload.cpp:17-40)
-class Mi355xPooling2dWorkload : public BaseWorkload<Pooling2dQueueDescriptor>
+class Mi355xPooling2dWorkload : public Mi355xBaseWorkload<Pooling2dQueueDescriptor>
 {
 public:
     Mi355xPooling2dWorkload(const Pooling2dQueueDescriptor& descriptor, const WorkloadInfo& info);
@@ -87,7 +99,7 @@ private:
 };
 
 /// counterpart of RefSoftmaxWorkload (RefSoftmaxWorkload.cpp:21-43)
-class Mi355xSoftmaxWorkload : public BaseWorkload<SoftmaxQueueDescriptor>
+class Mi355xSoftmaxWorkload : public Mi355xBaseWorkload<SoftmaxQueueDescriptor>
 {
 public:
     Mi355xSoftmaxWorkload(const SoftmaxQueueDescriptor& descriptor, const WorkloadInfo& info);
@@ -97,7 +109,7 @@ private:
 };
 
 /// counterpart of RefElementwiseBinaryWorkload for BinaryOperation::Add (RefElementwiseBinaryWorkload.cpp:27-107)
-class Mi355xAdditionWorkload : public BaseWorkload<ElementwiseBinaryQueueDescriptor>
+class Mi355xAdditionWorkload : public Mi355xBaseWorkload<ElementwiseBinaryQueueDescriptor>
 {
 public:
     Mi355xAdditionWorkload(const ElementwiseBinaryQueueDescriptor& descriptor, const WorkloadInfo& info);
@@ -107,7 +119,7 @@ private:
 };
 
 /// counterpart of RefReshapeWorkload (RefReshapeWorkload.cpp:14-31): a device-to-device copy
-class Mi355xReshapeWorkload : public BaseWorkload<ReshapeQueueDescriptor>
+class Mi355xReshapeWorkload : public Mi355xBaseWorkload<ReshapeQueueDescriptor>
 {
 public:
     Mi355xReshapeWorkload(const ReshapeQueueDescriptor& descriptor, const WorkloadInfo& info);
@@ -117,7 +129,7 @@ private:
 };
 
 /// counterpart of RefConstantWorkload (RefConstantWorkload.cpp:22-47): uploads the layer's data once
-class Mi355xConstantWorkload : public BaseWorkload<ConstantQueueDescriptor>
+class Mi355xConstantWorkload : public Mi355xBaseWorkload<ConstantQueueDescriptor>
 {
 public:
     Mi355xConstantWorkload(const ConstantQueueDescriptor& descriptor, const WorkloadInfo& info);

@@ -207,6 +207,25 @@ int mi355x_host_alloc(void** ptr_host, size_t bytes)
     return 0;
 }
 
+int mi355x_host_device_pointer(const void* host_ptr, void** device_ptr, int* is_device_memory)
+{
+    if (!host_ptr || !device_ptr || !is_device_memory) return SetError(MI355X_ERR_INVALID_ARGUMENT, "null pointer");
+    *device_ptr = nullptr;
+    *is_device_memory = 0;
+    hipPointerAttribute_t attr;
+    const hipError_t e = hipPointerGetAttributes(&attr, host_ptr);
+    if (e != hipSuccess)
+    {
+        (void)hipGetLastError();      // an unknown (pageable) pointer is an answer here, not a sticky error
+        return SetError(MI355X_ERR_UNSUPPORTED, "pageable host memory is not reachable from the device; allocate it with mi355x_host_alloc");
+    }
+    if (attr.type == hipMemoryTypeDevice) { *device_ptr = const_cast<void*>(host_ptr); *is_device_memory = 1; return 0; }
+    if (attr.type != hipMemoryTypeHost || !attr.devicePointer)
+        return SetError(MI355X_ERR_UNSUPPORTED, "memory of this kind is not reachable from the device; allocate it with mi355x_host_alloc");
+    *device_ptr = attr.devicePointer;
+    return 0;
+}
+
 int mi355x_host_free(void* ptr_host)
 {
     if (!ptr_host) return 0;

@@ -115,6 +115,11 @@ int  mi355x_device_props(int* compute_units, int* clock_khz, size_t* total_mem, 
 int  mi355x_malloc(void** ptr_dev, size_t bytes);
 int  mi355x_free(void* ptr_dev);
 int  mi355x_host_alloc(void** ptr_host, size_t bytes);          /* pinned host memory (hipHostMalloc) */
+/* Device address of caller memory the device reaches directly: memory from mi355x_host_alloc (pinned; *is_device_memory
+ * = 0) or device memory itself (*is_device_memory = 1).  Fails with MI355X_ERR_UNSUPPORTED for pageable host memory.
+ * Lets a tensor handle adopt caller memory instead of copying it through a staging buffer (RefTensorHandle::CanBeImported /
+ * Import, src/backends/reference/RefTensorHandle.cpp:135-165). */
+int  mi355x_host_device_pointer(const void* ptr, void** device_ptr, int* is_device_memory);
 int  mi355x_host_free(void* ptr_host);
 int  mi355x_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes, mi355x_stream_t stream);
 int  mi355x_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, mi355x_stream_t stream);
