@@ -2,6 +2,8 @@
 #pragma once
 #include "Tensor.hpp"
 #include "Types.hpp"
+#include <utility>
+#include <vector>
 
 namespace armnn
 {
@@ -62,6 +64,23 @@ struct Pooling2dDescriptor : BaseDescriptor
     OutputShapeRounding m_OutputShapeRounding = OutputShapeRounding::Floor;
     PaddingMethod m_PaddingMethod = PaddingMethod::Exclude;
     DataLayout m_DataLayout = DataLayout::NCHW;
+};
+
+/// include/armnn/Descriptors.hpp:1196-1229: one (before, after) pair per dimension; for quantized tensors m_PadValue
+/// is the stored code itself, not a real number to be quantized (workloads/Pad.cpp:77-84)
+struct PadDescriptor : BaseDescriptor
+{
+    PadDescriptor() = default;
+    PadDescriptor(const std::vector<std::pair<unsigned int, unsigned int>>& padList, float padValue = 0,
+                  PaddingMode paddingMode = PaddingMode::Constant)
+        : m_PadList(padList), m_PadValue(padValue), m_PaddingMode(paddingMode) {}
+    bool operator==(const PadDescriptor& rhs) const
+    {
+        return m_PadList == rhs.m_PadList && m_PadValue == rhs.m_PadValue && m_PaddingMode == rhs.m_PaddingMode;
+    }
+    std::vector<std::pair<unsigned int, unsigned int>> m_PadList;
+    float m_PadValue = 0;
+    PaddingMode m_PaddingMode = PaddingMode::Constant;
 };
 
 struct SoftmaxDescriptor : BaseDescriptor

@@ -28,6 +28,7 @@ enum class ActivationFunction
 
 enum class PoolingAlgorithm { Max = 0, Average = 1, L2 = 2 };
 enum class PaddingMethod { IgnoreValue = 0, Exclude = 1 };
+enum class PaddingMode { Constant = 0, Reflect = 1, Symmetric = 2 };
 enum class OutputShapeRounding { Floor = 0, Ceiling = 1 };
 enum class BinaryOperation { Add = 0, Div = 1, Maximum = 2, Minimum = 3, Mul = 4, Sub = 5, SqDiff = 6, Power = 7, FloorDiv = 8 };
 
@@ -38,7 +39,7 @@ using MemorySourceFlags = unsigned int;
 enum class LayerType
 {
     Activation, Constant, Convolution2d, DepthwiseConvolution2d, ElementwiseBinary, FullyConnected, Input, MemCopy,
-    Output, Pooling2d, Reshape, Softmax
+    Output, Pad, Pooling2d, Reshape, Softmax
 };
 const char* GetLayerTypeAsCString(LayerType type);
 

@@ -284,6 +284,18 @@ void Pooling2dQueueDescriptor::Validate(const WorkloadInfo& info) const
     ValidateTypesMatch(info.m_InputTensorInfos[0], info.m_OutputTensorInfos[0], name, "input", "output");
 }
 
+// WorkloadData.cpp:2484-2504
+void PadQueueDescriptor::Validate(const WorkloadInfo& info) const
+{
+    const std::string name = "PadQueueDescriptor";
+    ValidateNumInputsOutputs(info, name, 1, 1);
+    const TensorInfo& in = info.m_InputTensorInfos[0];
+    ValidateDims(info.m_OutputTensorInfos[0], name, in.GetNumDimensions(), "output");
+    Require(m_Parameters.m_PadList.size() == in.GetNumDimensions(),
+            name + ": the pad list needs one entry per input dimension (" + std::to_string(in.GetNumDimensions()) +
+            "), not " + std::to_string(m_Parameters.m_PadList.size()));
+}
+
 void SoftmaxQueueDescriptor::Validate(const WorkloadInfo& info) const
 {
     const std::string name = "SoftmaxQueueDescriptor";

@@ -10,7 +10,10 @@
 #include <armnn/backends/IBackendContext.hpp>
 #include <backendsCommon/TensorHandleFactoryRegistry.hpp>
 
+#include <limits>
 #include <set>
+#include <string>
+#include <utility>
 
 namespace armnn
 {
@@ -43,6 +46,56 @@ bool Fusable(const Layer& base)
             return static_cast<const ElementwiseBinaryDescriptor&>(base.GetParameters()).m_Operation == BinaryOperation::Add;
         default: return false;
     }
+}
+// ---- Pad folding (src/armnn/optimizations/FoldPadIntoLayer2d.hpp:21-145) ---------------------------------------------
+// the stored value that stands for the real number 0 (:21-24)
+float ZeroElement(const TensorInfo& info) { return static_cast<float>(info.IsQuantized() ? info.GetQuantizationOffset() : 0); }
+
+// the smallest value the tensor's type can hold (:26-56: -infinity quantized, i.e. saturated)
+float LowestElement(const TensorInfo& info)
+{
+    switch (info.GetDataType())
+    {
+        case DataType::QAsymmU8: return 0.0f;
+        case DataType::QAsymmS8: case DataType::QSymmS8: return -128.0f;
+        default: return -std::numeric_limits<float>::infinity();
+    }
+}
+
+// height and width padding of `pad` added to the layer's own; batch and channels must be unpadded (:93-120)
+template <typename Descriptor>
+bool AddPadding(const PadDescriptor& pad, Descriptor& d)
+{
+    if (pad.m_PaddingMode != PaddingMode::Constant || pad.m_PadList.size() != 4) return false;
+    const bool nhwc = d.m_DataLayout == DataLayout::NHWC;
+    const unsigned int channels = nhwc ? 3 : 1, height = nhwc ? 1 : 2, width = nhwc ? 2 : 3;
+    const std::pair<unsigned int, unsigned int> none{0u, 0u};
+    if (pad.m_PadList[0] != none || pad.m_PadList[channels] != none) return false;
+    d.m_PadLeft += pad.m_PadList[width].first;
+    d.m_PadRight += pad.m_PadList[width].second;
+    d.m_PadTop += pad.m_PadList[height].first;
+    d.m_PadBottom += pad.m_PadList[height].second;
+    return true;
+}
+
+// convolutions skip padded taps, which equals multiplying by the zero element (:58-69)
+template <typename Descriptor>
+bool FoldPad(const PadDescriptor& pad, Descriptor& d, const TensorInfo& padded)
+{
+    return pad.m_PadValue == ZeroElement(padded) && AddPadding(pad, d);
+}
+
+// (:71-77, :122-145) max pooling ignores anything not above the lowest value; average pooling needs zeros that count in
+// the divisor, so it cannot keep padding of its own that is excluded from it
+bool FoldPadIntoPooling(const PadDescriptor& pad, Pooling2dDescriptor& d, const TensorInfo& padded)
+{
+    const bool isMax = d.m_PoolType == PoolingAlgorithm::Max;
+    const bool ownPadding = d.m_PadLeft || d.m_PadRight || d.m_PadTop || d.m_PadBottom;
+    if (!isMax && ownPadding && d.m_PaddingMethod == PaddingMethod::Exclude) return false;
+    if (isMax ? !(pad.m_PadValue <= LowestElement(padded)) : pad.m_PadValue != ZeroElement(padded)) return false;
+    if (!AddPadding(pad, d)) return false;
+    d.m_PaddingMethod = PaddingMethod::IgnoreValue;
+    return true;
 }
 } // namespace
 
@@ -109,11 +162,16 @@ BackendCapabilities Mi355xBackend::GetCapabilities() const
                                                    {"SingleAxisPacking", false}});
 }
 
-// A quantized ReLu / BoundedReLu whose input and output share one quantization is an integer clamp
-// (workloads/Activation.cpp:33-42 between a decoder and an encoder of the same scale and offset), which the device
-// kernels apply in their epilogue.  With different quantizations the Activation layer re-quantizes and stays a layer
-// of its own.  The replacement layer carries the ActivationDescriptor as its additional-info object, as the Neon and
-// CL backends do (src/backends/aclCommon/ArmComputeSubgraphUtils.hpp:60-109).
+// Two rewrites, alone or together on one layer:
+//
+// * A quantized ReLu / BoundedReLu whose input and output share one quantization is an integer clamp
+//   (workloads/Activation.cpp:33-42 between a decoder and an encoder of the same scale and offset), which the device
+//   kernels apply in their epilogue.  With different quantizations the Activation layer re-quantizes and stays a layer
+//   of its own.  The replacement layer carries the ActivationDescriptor as its additional-info object, as the Neon and
+//   CL backends do (src/backends/aclCommon/ArmComputeSubgraphUtils.hpp:60-109).
+// * A constant Pad of height and width in front of a Convolution2d, DepthwiseConvolution2d or Pooling2d moves into that
+//   layer's own padding when the padded value is the layer's neutral element, as CpuRef does
+//   (src/backends/reference/RefBackend.cpp:72-184 with the rules of src/armnn/optimizations/FoldPadIntoLayer2d.hpp:21-145).
 OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgraph, const ModelOptions& modelOptions) const
 {
     OptimizationViews views(modelOptions);
@@ -125,26 +183,57 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
     {
         if (consumed.count(il)) continue;
         Layer* base = PolymorphicDowncast<Layer*>(il);
-        if (!Fusable(*base) || base->GetAdditionalInformation<ActivationDescriptor>() != nullptr) continue;
-        OutputSlot& out = base->GetOutputSlot(0);
-        if (out.GetNumConnections() != 1) continue;
-        Layer* act = &out.GetConnections()[0]->GetOwningLayer();
-        if (act->GetType() != LayerType::Activation || !members.count(act) || consumed.count(act)) continue;
-        const auto& ad = static_cast<const ActivationDescriptor&>(act->GetParameters());
-        if (ad.m_Function != ActivationFunction::ReLu && ad.m_Function != ActivationFunction::BoundedReLu) continue;
-        if (!SameQuantization(out.GetTensorInfo(), act->GetOutputSlot(0).GetTensorInfo())) continue;
+        const LayerType type = base->GetType();
 
-        const std::string name = std::string("fused-") + act->GetName() + "-into-" + base->GetName();
+        // the descriptor the replacement would get; the Pad in front of the layer, if its padding fits into it
+        Convolution2dDescriptor conv;
+        DepthwiseConvolution2dDescriptor depthwise;
+        Pooling2dDescriptor pooling;
+        Layer* pad = nullptr;
+        if (type == LayerType::Convolution2d || type == LayerType::DepthwiseConvolution2d || type == LayerType::Pooling2d)
+        {
+            if (type == LayerType::Convolution2d) conv = static_cast<const Convolution2dDescriptor&>(base->GetParameters());
+            if (type == LayerType::DepthwiseConvolution2d) depthwise = static_cast<const DepthwiseConvolution2dDescriptor&>(base->GetParameters());
+            if (type == LayerType::Pooling2d) pooling = static_cast<const Pooling2dDescriptor&>(base->GetParameters());
+            OutputSlot* source = base->GetInputSlot(0).GetConnectedOutputSlot();
+            Layer* producer = source ? &source->GetOwningLayer() : nullptr;
+            if (producer && producer->GetType() == LayerType::Pad && members.count(producer) && !consumed.count(producer) &&
+                source->GetNumConnections() == 1 && producer->GetInputSlot(0).GetConnectedOutputSlot() != nullptr)
+            {
+                const auto& pd = static_cast<const PadDescriptor&>(producer->GetParameters());
+                const TensorInfo& padded = source->GetTensorInfo();
+                const bool folded = type == LayerType::Convolution2d ? FoldPad(pd, conv, padded)
+                                  : type == LayerType::DepthwiseConvolution2d ? FoldPad(pd, depthwise, padded)
+                                  : FoldPadIntoPooling(pd, pooling, padded);
+                if (folded) pad = producer;
+            }
+        }
+
+        // the Activation behind the layer, if it is a clamp in the layer's own output quantization
+        Layer* act = nullptr;
+        if (Fusable(*base) && base->GetAdditionalInformation<ActivationDescriptor>() == nullptr && base->GetOutputSlot(0).GetNumConnections() == 1)
+        {
+            Layer* next = &base->GetOutputSlot(0).GetConnections()[0]->GetOwningLayer();
+            if (next->GetType() == LayerType::Activation && members.count(next) && !consumed.count(next))
+            {
+                const auto& ad = static_cast<const ActivationDescriptor&>(next->GetParameters());
+                if ((ad.m_Function == ActivationFunction::ReLu || ad.m_Function == ActivationFunction::BoundedReLu) &&
+                    SameQuantization(base->GetOutputSlot(0).GetTensorInfo(), next->GetOutputSlot(0).GetTensorInfo()))
+                    act = next;
+            }
+        }
+        if (!pad && !act) continue;
+
+        std::string name = base->GetName();
+        if (pad) name = std::string("folded-") + pad->GetName() + "-into-" + name;
+        if (act) name = std::string("fused-") + act->GetName() + "-into-" + name;
         INetwork& net = views.GetINetworkRef();
         IConnectableLayer* replacement = nullptr;
-        switch (base->GetType())
+        switch (type)
         {
-            case LayerType::Convolution2d:
-                replacement = net.AddConvolution2dLayer(static_cast<const Convolution2dDescriptor&>(base->GetParameters()), name.c_str());
-                break;
-            case LayerType::DepthwiseConvolution2d:
-                replacement = net.AddDepthwiseConvolution2dLayer(static_cast<const DepthwiseConvolution2dDescriptor&>(base->GetParameters()), name.c_str());
-                break;
+            case LayerType::Convolution2d: replacement = net.AddConvolution2dLayer(conv, name.c_str()); break;
+            case LayerType::DepthwiseConvolution2d: replacement = net.AddDepthwiseConvolution2dLayer(depthwise, name.c_str()); break;
+            case LayerType::Pooling2d: replacement = net.AddPooling2dLayer(pooling, name.c_str()); break;
             case LayerType::FullyConnected:
                 replacement = net.AddFullyConnectedLayer(static_cast<const FullyConnectedDescriptor&>(base->GetParameters()), name.c_str());
                 break;
@@ -152,16 +241,26 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
                 replacement = net.AddElementwiseBinaryLayer(static_cast<const ElementwiseBinaryDescriptor&>(base->GetParameters()), name.c_str());
                 break;
         }
-        replacement->GetOutputSlot(0).SetTensorInfo(act->GetOutputSlot(0).GetTensorInfo());
-        PolymorphicDowncast<Layer*>(replacement)->SetAdditionalInfoForObject(std::make_shared<ActivationDescriptor>(ad));
+        Layer* last = act ? act : base;
+        replacement->GetOutputSlot(0).SetTensorInfo(last->GetOutputSlot(0).GetTensorInfo());
+        if (act)
+            PolymorphicDowncast<Layer*>(replacement)->SetAdditionalInfoForObject(
+                std::make_shared<ActivationDescriptor>(static_cast<const ActivationDescriptor&>(act->GetParameters())));
+        else if (auto carried = base->GetAdditionalInformation<ActivationDescriptor>())
+            PolymorphicDowncast<Layer*>(replacement)->SetAdditionalInfoForObject(carried);
 
+        SubgraphView::IConnectableLayers replaced;
         SubgraphView::IInputSlots ins;
-        for (unsigned int i = 0; i < base->GetNumInputSlots(); ++i) ins.push_back(&base->GetInputSlot(i));
-        SubgraphView::IOutputSlots outs{&act->GetOutputSlot(0)};
-        SubgraphView substitutable({base, act}, std::move(ins), std::move(outs));
+        if (pad) replaced.push_back(pad);
+        replaced.push_back(base);
+        if (act) replaced.push_back(act);
+        ins.push_back(pad ? &pad->GetInputSlot(0) : &base->GetInputSlot(0));
+        for (unsigned int i = 1; i < base->GetNumInputSlots(); ++i) ins.push_back(&base->GetInputSlot(i));
+        SubgraphView::IOutputSlots outs{&last->GetOutputSlot(0)};
+        SubgraphView substitutable(std::move(replaced), std::move(ins), std::move(outs));
         views.AddSubstitution({std::move(substitutable), SubgraphView(replacement)});
-        consumed.insert(base);
-        consumed.insert(act);
+        for (Layer* l : {pad, base, act})
+            if (l) consumed.insert(l);
     }
 
     for (IConnectableLayer* il : layers)

@@ -130,6 +130,20 @@ bool Mi355xLayerSupport::IsPooling2dSupported(const TensorInfo& input, const Ten
     return CheckActivations(input, output, reason);
 }
 
+bool Mi355xLayerSupport::IsPadSupported(const TensorInfo& input, const TensorInfo& output, const PadDescriptor& d,
+                                        Optional<std::string&> reason) const
+{
+    if (d.m_PaddingMode != PaddingMode::Constant) return No(reason, "only constant padding runs on the device");
+    const unsigned int rank = input.GetNumDimensions();
+    if (rank < 1 || rank > 4) return No(reason, "Pad runs on tensors of 1 to 4 dimensions");
+    if (output.GetNumDimensions() != rank || d.m_PadList.size() != rank) return No(reason, "Pad needs one (before, after) pair per dimension");
+    for (unsigned int k = 0; k < rank; ++k)
+        if (input.GetShape()[k] + d.m_PadList[k].first + d.m_PadList[k].second != output.GetShape()[k])
+            return No(reason, "output shape is not the input shape plus the padding");
+    if (std::isnan(d.m_PadValue)) return No(reason, "pad value is not a number");
+    return CheckActivations(input, output, reason);
+}
+
 bool Mi355xLayerSupport::IsSoftmaxSupported(const TensorInfo& input, const TensorInfo& output, const SoftmaxDescriptor& d,
                                             Optional<std::string&> reason) const
 {
@@ -206,6 +220,9 @@ bool Mi355xLayerSupport::IsLayerSupported(const LayerType& type, const std::vect
         case LayerType::Pooling2d:
             need(2);
             return IsPooling2dSupported(infos[0], infos[1], *PolymorphicDowncast<const Pooling2dDescriptor*>(&descriptor), reason);
+        case LayerType::Pad:
+            need(2);
+            return IsPadSupported(infos[0], infos[1], *PolymorphicDowncast<const PadDescriptor*>(&descriptor), reason);
         case LayerType::Softmax:
             need(2);
             return IsSoftmaxSupported(infos[0], infos[1], *PolymorphicDowncast<const SoftmaxDescriptor*>(&descriptor), reason);

@@ -24,6 +24,8 @@ public:
                                Optional<std::string&> reason) const;
     bool IsPooling2dSupported(const TensorInfo& input, const TensorInfo& output, const Pooling2dDescriptor& descriptor,
                               Optional<std::string&> reason) const;
+    bool IsPadSupported(const TensorInfo& input, const TensorInfo& output, const PadDescriptor& descriptor,
+                        Optional<std::string&> reasonIfUnsupported = EmptyOptional()) const;
     bool IsSoftmaxSupported(const TensorInfo& input, const TensorInfo& output, const SoftmaxDescriptor& descriptor,
                             Optional<std::string&> reason) const;
     bool IsElementwiseBinarySupported(const TensorInfo& input0, const TensorInfo& input1, const TensorInfo& output,

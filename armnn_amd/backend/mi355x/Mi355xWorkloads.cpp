@@ -268,6 +268,32 @@ void Mi355xPooling2dWorkload::Execute() const
     mi355x::Check(mi355x_pool2d_run(&d, in.GetShape()[0], In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()), "mi355x_pool2d_run");
 }
 
+// ---- Pad -------------------------------------------------------------------------------------------------------------
+Mi355xPadWorkload::Mi355xPadWorkload(const PadQueueDescriptor& descriptor, const WorkloadInfo& info)
+    : Mi355xBaseWorkload<PadQueueDescriptor>(descriptor, info), m_Info(info)
+{
+    if (m_Data.m_Parameters.m_PaddingMode != PaddingMode::Constant) throw InvalidArgumentException("Mi355xPadWorkload: constant padding only");
+    if (m_Info.m_InputTensorInfos[0].GetNumDimensions() > 4) throw InvalidArgumentException("Mi355xPadWorkload: at most 4 dimensions");
+}
+
+void Mi355xPadWorkload::Execute() const
+{
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const PadDescriptor& p = m_Data.m_Parameters;
+    mi355x_pad_desc d{};
+    d.rank = in.GetNumDimensions();
+    for (unsigned int k = 0; k < d.rank; ++k)
+    {
+        d.in_shape[k] = in.GetShape()[k];
+        d.pad_before[k] = p.m_PadList[k].first;
+        d.pad_after[k] = p.m_PadList[k].second;
+    }
+    d.pad_value = p.m_PadValue;
+    d.input = mi355x::ToQuant(in);
+    d.output = mi355x::ToQuant(m_Info.m_OutputTensorInfos[0]);
+    mi355x::Check(mi355x_pad_run(&d, In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()), "mi355x_pad_run");
+}
+
 // ---- Softmax ---------------------------------------------------------------------------------------------------------
 Mi355xSoftmaxWorkload::Mi355xSoftmaxWorkload(const SoftmaxQueueDescriptor& descriptor, const WorkloadInfo& info)
     : Mi355xBaseWorkload<SoftmaxQueueDescriptor>(descriptor, info), m_Info(info)

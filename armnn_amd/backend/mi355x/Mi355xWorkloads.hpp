@@ -98,6 +98,16 @@ private:
     WorkloadInfo m_Info;
 };
 
+/// counterpart of RefPadWorkload (RefPadWorkload.cpp:18-40)
+class Mi355xPadWorkload : public Mi355xBaseWorkload<PadQueueDescriptor>
+{
+public:
+    Mi355xPadWorkload(const PadQueueDescriptor& descriptor, const WorkloadInfo& info);
+    void Execute() const override;
+private:
+    WorkloadInfo m_Info;
+};
+
 /// counterpart of RefSoftmaxWorkload (RefSoftmaxWorkload.cpp:21-43)
 class Mi355xSoftmaxWorkload : public Mi355xBaseWorkload<SoftmaxQueueDescriptor>
 {

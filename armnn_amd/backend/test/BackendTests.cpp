@@ -152,6 +152,16 @@ TEST_CASE("layer support: the accepted envelope and the reasons outside it", "cp
     CHECK(ls.IsLayerSupported(LayerType::Softmax, {logits, probs}, sd, EmptyOptional(), EmptyOptional(), reason));
     sd.m_Axis = 0;
     CHECK(!ls.IsLayerSupported(LayerType::Softmax, {logits, probs}, sd, EmptyOptional(), EmptyOptional(), reason));
+
+    // Pad: constant mode, ranks 1..4, the output shape must be the padded input shape
+    PadDescriptor padDesc({{0, 0}, {1, 1}, {2, 0}, {0, 0}}, -3.0f);
+    const TensorInfo padIn = ActInfo({1, 8, 8, 16}, DataType::QAsymmS8, 0.05f, -3), padOut = ActInfo({1, 10, 10, 16}, DataType::QAsymmS8, 0.05f, -3);
+    CHECK(ls.IsLayerSupported(LayerType::Pad, {padIn, padOut}, padDesc, EmptyOptional(), EmptyOptional(), reason));
+    CHECK(!ls.IsLayerSupported(LayerType::Pad, {padIn, ActInfo({1, 10, 9, 16}, DataType::QAsymmS8, 0.05f, -3)}, padDesc, EmptyOptional(), EmptyOptional(), reason));
+    CHECK_MSG(why.find("output shape") != std::string::npos, why);
+    padDesc.m_PaddingMode = PaddingMode::Reflect;
+    CHECK(!ls.IsLayerSupported(LayerType::Pad, {padIn, padOut}, padDesc, EmptyOptional(), EmptyOptional(), reason));
+    CHECK_MSG(why.find("constant") != std::string::npos, why);
     CHECK(ls.IsLayerSupported(LayerType::Reshape, {pooled, ActInfo({1, 16}, DataType::QAsymmS8, 0.05f, -3)}, ReshapeDescriptor(TensorShape({1, 16})), EmptyOptional(), EmptyOptional(), reason));
 }
 
@@ -323,6 +333,145 @@ TEST_CASE("optimize: BoundedReLu is folded into the convolution only when that c
     }
 }
 
+namespace
+{
+using PadList = std::vector<std::pair<unsigned int, unsigned int>>;
+
+TensorInfo Padded(const TensorInfo& in, const PadList& pads)
+{
+    std::vector<unsigned int> dims;
+    for (unsigned int k = 0; k < in.GetNumDimensions(); ++k) dims.push_back(in.GetShape()[k] + pads[k].first + pads[k].second);
+    TensorInfo out = in;
+    out.SetShape(TensorShape(static_cast<unsigned int>(dims.size()), dims.data()));
+    return out;
+}
+
+// Input -> Pad -> conv / depthwise (+ BoundedReLu); `extraConsumer` makes the padded tensor a network output as well
+INetworkPtr PadConvNet(const TensorInfo& in, const PadList& pads, float padValue, const QLayer& conv, bool extraConsumer = false)
+{
+    INetworkPtr net = INetwork::Create();
+    IConnectableLayer* input = net->AddInputLayer(0, "input");
+    input->GetOutputSlot(0).SetTensorInfo(in);
+    IConnectableLayer* pad = net->AddPadLayer(PadDescriptor(pads, padValue), "pad");
+    input->GetOutputSlot(0).Connect(pad->GetInputSlot(0));
+    pad->GetOutputSlot(0).SetTensorInfo(Padded(in, pads));
+    IOutputSlot& out = AddToNetwork(*net, pad->GetOutputSlot(0), conv, "conv");
+    IConnectableLayer* o = net->AddOutputLayer(0, "output");
+    out.Connect(o->GetInputSlot(0));
+    if (extraConsumer)
+    {
+        IConnectableLayer* o2 = net->AddOutputLayer(1, "padded");
+        pad->GetOutputSlot(0).Connect(o2->GetInputSlot(0));
+    }
+    return net;
+}
+
+// Input -> Pad -> Pooling2d
+INetworkPtr PadPoolNet(const TensorInfo& in, const PadList& pads, float padValue, const Pooling2dDescriptor& pool, const TensorInfo& out)
+{
+    INetworkPtr net = INetwork::Create();
+    IConnectableLayer* input = net->AddInputLayer(0, "input");
+    input->GetOutputSlot(0).SetTensorInfo(in);
+    IConnectableLayer* pad = net->AddPadLayer(PadDescriptor(pads, padValue), "pad");
+    input->GetOutputSlot(0).Connect(pad->GetInputSlot(0));
+    pad->GetOutputSlot(0).SetTensorInfo(Padded(in, pads));
+    IConnectableLayer* p = net->AddPooling2dLayer(pool, "pool");
+    pad->GetOutputSlot(0).Connect(p->GetInputSlot(0));
+    p->GetOutputSlot(0).SetTensorInfo(out);
+    IConnectableLayer* o = net->AddOutputLayer(0, "output");
+    p->GetOutputSlot(0).Connect(o->GetInputSlot(0));
+    return net;
+}
+
+Pooling2dDescriptor Pool3x3s2(PoolingAlgorithm algo)
+{
+    Pooling2dDescriptor d;
+    d.m_PoolType = algo;
+    d.m_PoolWidth = d.m_PoolHeight = 3;
+    d.m_StrideX = d.m_StrideY = 2;
+    d.m_DataLayout = DataLayout::NHWC;
+    return d;
+}
+} // namespace
+
+TEST_CASE("optimize: a Pad of height and width moves into the layer behind it when the padded value is neutral there", "cpu")
+{
+    FixedDeviceSpec spec{kMi355x};
+    const TensorInfo in = ActInfo({2, 10, 12, 16}, DataType::QAsymmS8, 0.05f, -3);
+    const PadList hw{{0, 0}, {1, 2}, {3, 0}, {0, 0}};
+    const QLayer conv = MakeConv(QLayer::Conv, Padded(in, hw), 32, 3, 1, 0.1f, -128, true, true, 41);     // SAME: own padding 1
+    {
+        INetworkPtr net = PadConvNet(in, hw, -3.0f, conv);                  // the zero point: what a skipped tap contributes
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, spec);
+        const Graph& g = opt->GetGraph();
+        CHECK(CountLayers(g, LayerType::Pad) == 0);
+        CHECK(CountLayers(g, LayerType::Activation) == 0);
+        CHECK(CountLayers(g, LayerType::Convolution2d) == 1);
+        const Layer* folded = FindLayer(g, "folded-pad-into-conv");
+        REQUIRE(folded != nullptr);
+        CHECK(folded->GetNameStr().find("fused-") == 0);
+        const auto& d = static_cast<const Convolution2dDescriptor&>(folded->GetParameters());
+        CHECK(d.m_PadTop == 2); CHECK(d.m_PadBottom == 3); CHECK(d.m_PadLeft == 4); CHECK(d.m_PadRight == 1);
+        CHECK(folded->GetAdditionalInformation<ActivationDescriptor>() != nullptr);
+        CHECK(folded->In(0).GetConnectedOutputSlot()->GetOwningLayer().GetType() == LayerType::Input);
+        CHECK(folded->In(1).GetConnectedOutputSlot()->GetOwningLayer().GetType() == LayerType::Constant);
+        CHECK(folded->In(2).GetConnectedOutputSlot()->GetOwningLayer().GetType() == LayerType::Constant);
+        CHECK(folded->Out(0).GetTensorInfo().GetShape() == conv.out.GetShape());
+    }
+    {
+        INetworkPtr net = PadConvNet(in, hw, 0.0f, conv);                   // code 0 is the real number 0.15 here: not neutral
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, spec);
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Pad) == 1);
+        CHECK(FindLayer(opt->GetGraph(), "folded-") == nullptr);
+        CHECK(FindLayer(opt->GetGraph(), "fused-") != nullptr);             // the activation is still fused
+    }
+    {
+        const PadList withChannels{{0, 0}, {1, 1}, {1, 1}, {0, 16}};
+        QLayer c2 = MakeConv(QLayer::Conv, Padded(in, withChannels), 8, 1, 1, 0.1f, -128, false, true, 42);
+        IOptimizedNetworkPtr opt = Optimize(*PadConvNet(in, withChannels, -3.0f, c2), {kMi355x}, spec);
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Pad) == 1);
+    }
+    {
+        IOptimizedNetworkPtr opt = Optimize(*PadConvNet(in, hw, -3.0f, conv, true), {kMi355x}, spec);      // the padded tensor is read elsewhere
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Pad) == 1);
+    }
+    {
+        const QLayer dw = MakeConv(QLayer::Depthwise, Padded(in, hw), 16, 3, 2, 0.1f, -128, false, true, 43);
+        IOptimizedNetworkPtr opt = Optimize(*PadConvNet(in, hw, -3.0f, dw), {kMi355x}, spec);
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Pad) == 0);
+        REQUIRE(FindLayer(opt->GetGraph(), "folded-pad-into-conv") != nullptr);
+        CHECK(FindLayer(opt->GetGraph(), "folded-pad-into-conv")->GetType() == LayerType::DepthwiseConvolution2d);
+    }
+    // pooling: Max needs a value no element can undercut, Average needs zeros that count in the divisor
+    const TensorInfo padded = Padded(in, hw);
+    const TensorInfo pooled = ActInfo({2, (padded.GetShape()[1] - 3) / 2 + 1, (padded.GetShape()[2] - 3) / 2 + 1, 16}, DataType::QAsymmS8, 0.05f, -3);
+    {
+        IOptimizedNetworkPtr opt = Optimize(*PadPoolNet(in, hw, -128.0f, Pool3x3s2(PoolingAlgorithm::Max), pooled), {kMi355x}, spec);
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Pad) == 0);
+        const Layer* p = FindLayer(opt->GetGraph(), "folded-pad-into-pool");
+        REQUIRE(p != nullptr);
+        const auto& d = static_cast<const Pooling2dDescriptor&>(p->GetParameters());
+        CHECK(d.m_PaddingMethod == PaddingMethod::IgnoreValue);
+        CHECK(d.m_PadTop == 1); CHECK(d.m_PadBottom == 2); CHECK(d.m_PadLeft == 3); CHECK(d.m_PadRight == 0);
+    }
+    {
+        IOptimizedNetworkPtr opt = Optimize(*PadPoolNet(in, hw, -3.0f, Pool3x3s2(PoolingAlgorithm::Max), pooled), {kMi355x}, spec);
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Pad) == 1);           // an element below the zero point would lose to the padding
+    }
+    {
+        IOptimizedNetworkPtr opt = Optimize(*PadPoolNet(in, hw, -3.0f, Pool3x3s2(PoolingAlgorithm::Average), pooled), {kMi355x}, spec);
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Pad) == 0);
+    }
+    {
+        Pooling2dDescriptor own = Pool3x3s2(PoolingAlgorithm::Average);     // padding of its own, left out of the divisor
+        own.m_PadLeft = own.m_PadRight = 1;
+        own.m_PaddingMethod = PaddingMethod::Exclude;
+        const TensorInfo o2 = ActInfo({2, pooled.GetShape()[1], (padded.GetShape()[2] + 2 - 3) / 2 + 1, 16}, DataType::QAsymmS8, 0.05f, -3);
+        IOptimizedNetworkPtr opt = Optimize(*PadPoolNet(in, hw, -3.0f, own, o2), {kMi355x}, spec);
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Pad) == 1);
+    }
+}
+
 TEST_CASE("optimize: unsupported layers fall back along the preference list, with copies between backends", "cpu")
 {
     testhost::Register();
@@ -464,6 +613,106 @@ TEST_CASE("runtime: DepthwiseConvolution2d 3x3, per-axis weights, fused BoundedR
 {
     CheckSingleLayer(MakeConv(QLayer::Depthwise, ActInfo({2, 28, 28, 64}, DataType::QAsymmS8, 0.0235f, -128), 64, 3, 1, 0.0235f, -128, true, true, 104), 4, "dw3x3");
     CheckSingleLayer(MakeConv(QLayer::Depthwise, ActInfo({1, 15, 15, 24}, DataType::QAsymmU8, 0.0235f, 3), 24, 3, 2, 0.0235f, 0, true, true, 105), 5, "dw3x3-s2-u8");
+}
+
+namespace
+{
+std::vector<uint8_t> OraclePad(const TensorInfo& in, const std::vector<uint8_t>& input, const PadList& pads, float value)
+{
+    const TensorInfo outInfo = Padded(in, pads);
+    std::vector<uint8_t> out(outInfo.GetNumElements());
+    const std::vector<float> s{in.GetQuantizationScale()};
+    orc_tensor ti = Orc(in, input.data(), s), to = Orc(outInfo, out.data(), s);
+    std::vector<uint32_t> before;
+    for (const auto& p : pads) before.push_back(p.first);
+    if (orc_pad(&ti, &to, before.data(), value) != 0) throw std::runtime_error(std::string("oracle: ") + orc_last_error());
+    return out;
+}
+
+std::vector<uint8_t> OraclePool(const TensorInfo& in, const std::vector<uint8_t>& input, const Pooling2dDescriptor& d, const TensorInfo& outInfo)
+{
+    std::vector<uint8_t> out(outInfo.GetNumElements());
+    const std::vector<float> si{in.GetQuantizationScale()}, so{outInfo.GetQuantizationScale()};
+    orc_tensor ti = Orc(in, input.data(), si), to = Orc(outInfo, out.data(), so);
+    orc_pool_params p{};
+    p.pool_type = d.m_PoolType == PoolingAlgorithm::Max ? ORC_POOL_MAX : ORC_POOL_AVERAGE;
+    p.padding_method = d.m_PaddingMethod == PaddingMethod::Exclude ? ORC_PAD_EXCLUDE : ORC_PAD_IGNORE_VALUE;
+    p.pad_left = d.m_PadLeft; p.pad_right = d.m_PadRight; p.pad_top = d.m_PadTop; p.pad_bottom = d.m_PadBottom;
+    p.pool_w = d.m_PoolWidth; p.pool_h = d.m_PoolHeight; p.stride_x = d.m_StrideX; p.stride_y = d.m_StrideY;
+    if (orc_pooling2d(&ti, &to, &p, ORC_NHWC) != 0) throw std::runtime_error(std::string("oracle: ") + orc_last_error());
+    return out;
+}
+} // namespace
+
+TEST_CASE("runtime: Pad runs on the device; folded into the layer behind it, it gives the bytes of the two layers run apart", "gpu")
+{
+    IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+    REQUIRE(rt->GetDeviceSpec().GetSupportedBackends().count(kMi355x) == 1);
+    const TensorInfo in = ActInfo({2, 21, 19, 16}, DataType::QAsymmS8, 0.0235f, -7);
+    const PadList hw{{0, 0}, {1, 2}, {3, 0}, {0, 0}};
+    const TensorInfo padded = Padded(in, hw);
+    const std::vector<uint8_t> input = RandomActivations(in, 77);
+
+    // the layer on its own, with a value that is nobody's neutral element
+    auto padOnly = [&](float value) {
+        INetworkPtr net = INetwork::Create();
+        IConnectableLayer* i = net->AddInputLayer(0, "input");
+        i->GetOutputSlot(0).SetTensorInfo(in);
+        IConnectableLayer* p = net->AddPadLayer(PadDescriptor(hw, value), "pad");
+        i->GetOutputSlot(0).Connect(p->GetInputSlot(0));
+        p->GetOutputSlot(0).SetTensorInfo(padded);
+        IConnectableLayer* o = net->AddOutputLayer(0, "output");
+        p->GetOutputSlot(0).Connect(o->GetInputSlot(0));
+        return net;
+    };
+    CHECK(Compare(RunOnRuntime(*rt, *padOnly(11.0f), {kMi355x}, in, input, padded), OraclePad(in, input, hw, 11.0f), DataType::QAsymmS8).mismatches == 0);
+    const std::vector<uint8_t> paddedBytes = RunOnRuntime(*rt, *padOnly(-7.0f), {kMi355x}, in, input, padded);
+    CHECK(Compare(paddedBytes, OraclePad(in, input, hw, -7.0f), DataType::QAsymmS8).mismatches == 0);
+
+    for (QLayer::Kind kind : {QLayer::Conv, QLayer::Depthwise})
+    {
+        const QLayer conv = MakeConv(kind, padded, kind == QLayer::Conv ? 48 : 16, 3, kind == QLayer::Conv ? 1 : 2, 0.0235f, -128, true, true, 78);
+        INetworkPtr folded = PadConvNet(in, hw, -7.0f, conv);
+        {
+            IOptimizedNetworkPtr opt = Optimize(*folded, {kMi355x}, rt->GetDeviceSpec());
+            CHECK(CountLayers(opt->GetGraph(), LayerType::Pad) == 0);
+        }
+        const std::vector<uint8_t> got = RunOnRuntime(*rt, *folded, {kMi355x}, in, input, conv.out);
+        SingleLayerNet apart(conv);
+        const std::vector<uint8_t> twoSteps = RunOnRuntime(*rt, *apart.net, {kMi355x}, padded, paddedBytes, conv.out);
+        CHECK(Compare(got, twoSteps, DataType::QAsymmS8).mismatches == 0);
+        const Diff d = Compare(got, OracleRun(conv, paddedBytes), DataType::QAsymmS8);
+        std::printf("    pad folded into %s: max |diff| %d LSB vs oracle, exact %.5f\n", kind == QLayer::Conv ? "conv" : "depthwise", d.maxAbs,
+                    1.0 - static_cast<double>(d.mismatches) / static_cast<double>(d.n));
+        CHECK(d.maxAbs <= 1);
+    }
+
+    for (PoolingAlgorithm algo : {PoolingAlgorithm::Max, PoolingAlgorithm::Average})
+    {
+        const Pooling2dDescriptor pool = Pool3x3s2(algo);
+        const TensorInfo pooled = ActInfo({2, (padded.GetShape()[1] - 3) / 2 + 1, (padded.GetShape()[2] - 3) / 2 + 1, 16}, DataType::QAsymmS8, 0.03f, -20);
+        const float value = algo == PoolingAlgorithm::Max ? -128.0f : -7.0f;
+        INetworkPtr folded = PadPoolNet(in, hw, value, pool, pooled);
+        {
+            IOptimizedNetworkPtr opt = Optimize(*folded, {kMi355x}, rt->GetDeviceSpec());
+            CHECK(CountLayers(opt->GetGraph(), LayerType::Pad) == 0);
+        }
+        const std::vector<uint8_t> got = RunOnRuntime(*rt, *folded, {kMi355x}, in, input, pooled);
+        // CpuRef folds the same way (RefBackend.cpp:95-117) and then runs Pooling2d with the summed padding ignored
+        Pooling2dDescriptor summed = pool;
+        summed.m_PadTop = hw[1].first; summed.m_PadBottom = hw[1].second; summed.m_PadLeft = hw[2].first; summed.m_PadRight = hw[2].second;
+        summed.m_PaddingMethod = PaddingMethod::IgnoreValue;
+        CHECK(Compare(got, OraclePool(in, input, summed, pooled), DataType::QAsymmS8).mismatches == 0);
+        // The first window of every row lies wholly on the three padded columns.  Averaging gives the zero point either
+        // way; Max gives the reference's "nothing to pool" value 0.0 (Pooling2d.cpp:212-219) once folded, where the two
+        // layers run apart would give the lowest code -- so for Max only the other windows can be compared with that.
+        const std::vector<uint8_t> apart = OraclePool(padded, OraclePad(in, input, hw, value), pool, pooled);
+        size_t differing = 0;
+        const unsigned int wo = pooled.GetShape()[2], c = pooled.GetShape()[3];
+        for (size_t i = 0; i < got.size(); ++i)
+            if (got[i] != apart[i] && !(algo == PoolingAlgorithm::Max && (i / c) % wo == 0)) ++differing;
+        CHECK(differing == 0);
+    }
 }
 
 TEST_CASE("runtime: FullyConnected, per-axis weights", "gpu")

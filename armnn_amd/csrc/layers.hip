@@ -4,6 +4,7 @@
 #include "common.h"
 #include "device_math.h"
 
+#include <algorithm>
 #include <cfloat>
 #include <climits>
 #include <cmath>
@@ -373,6 +374,73 @@ __global__ __launch_bounds__(256) void SoftmaxRowKernel(int cols, float beta, QI
         if (tid + 256 * k < cols) yr[tid + 256 * k] = static_cast<uint8_t>(QuantizeDev(__fdiv_rn(v[k], sum), rq));
 }
 
+// Constant padding.  The host merges every unpadded dimension into the one outside it, so a row of the canonical
+// innermost dimension is one contiguous run of output bytes whose middle part is one contiguous run of input bytes.
+struct PadArgs
+{
+    uint32_t out[4], in[4], before[4];   // canonical shapes, right-aligned (leading extents 1)
+    uint32_t fill;                       // the pad code in all four bytes
+    int identity;                        // equal quantizations: elements are copied, not re-quantized
+};
+
+__device__ __forceinline__ uint32_t Recode4(uint32_t w, const uint8_t* lut)
+{
+    return static_cast<uint32_t>(lut[w & 0xffu]) | (static_cast<uint32_t>(lut[(w >> 8) & 0xffu]) << 8) |
+           (static_cast<uint32_t>(lut[(w >> 16) & 0xffu]) << 16) | (static_cast<uint32_t>(lut[w >> 24]) << 24);
+}
+
+// One block per 256 units of V bytes of one output row; V divides the innermost extents and the front padding, so a
+// unit lies either wholly inside the input or wholly in the padding.  grid.x = rows * chunks.
+template <int V>
+__global__ __launch_bounds__(256) void PadKernel(PadArgs p, QIn qin, Requant rq, uint32_t chunks,
+                                                 const uint8_t* __restrict__ x, uint8_t* __restrict__ y)
+{
+    __shared__ uint8_t lut[256];
+    if (!p.identity)
+    {
+        lut[threadIdx.x] = static_cast<uint8_t>(QuantizeDev(DequantDev(static_cast<uint8_t>(threadIdx.x), qin), rq));
+        __syncthreads();
+    }
+    const uint32_t row = blockIdx.x / chunks;
+    const uint32_t unit = (blockIdx.x - row * chunks) * 256 + threadIdx.x;
+    if (unit >= p.out[3] / V) return;
+    const uint32_t d2 = row % p.out[2];
+    const uint32_t r1 = row / p.out[2];
+    const uint32_t d1 = r1 % p.out[1];
+    const uint32_t d0 = r1 / p.out[1];
+    // unsigned wrap-around turns "in front of the input" into "beyond it"
+    const uint32_t s0 = d0 - p.before[0], s1 = d1 - p.before[1], s2 = d2 - p.before[2], s3 = unit * V - p.before[3];
+    const bool inside = s0 < p.in[0] && s1 < p.in[1] && s2 < p.in[2] && s3 < p.in[3];
+    const size_t src = ((static_cast<size_t>(s0) * p.in[1] + s1) * p.in[2] + s2) * p.in[3] + s3;
+    const size_t dst = static_cast<size_t>(row) * p.out[3] + static_cast<size_t>(unit) * V;
+    if constexpr (V == 1)
+    {
+        uint8_t v = static_cast<uint8_t>(p.fill);
+        if (inside) v = p.identity ? x[src] : lut[x[src]];
+        y[dst] = v;
+    }
+    else if constexpr (V == 4)
+    {
+        uint32_t w = p.fill;
+        if (inside)
+        {
+            w = *reinterpret_cast<const uint32_t*>(x + src);
+            if (!p.identity) w = Recode4(w, lut);
+        }
+        *reinterpret_cast<uint32_t*>(y + dst) = w;
+    }
+    else
+    {
+        v4u w = {p.fill, p.fill, p.fill, p.fill};
+        if (inside)
+        {
+            w = *reinterpret_cast<const v4u*>(x + src);
+            if (!p.identity) { w.x = Recode4(w.x, lut); w.y = Recode4(w.y, lut); w.z = Recode4(w.z, lut); w.w = Recode4(w.w, lut); }
+        }
+        *reinterpret_cast<v4u*>(y + dst) = w;
+    }
+}
+
 int CheckQ(const mi355x_quant* q, const char* what)
 {
     if (!q) return SetError(MI355X_ERR_INVALID_ARGUMENT, "%s quantization is null", what);
@@ -485,6 +553,74 @@ int mi355x_softmax_run(uint32_t rows, uint32_t cols, float beta, const mi355x_qu
         hipLaunchKernelGGL(SoftmaxRowKernel<8>, dim3(rows), dim3(256), 0, ToHip(stream), static_cast<int>(cols), beta, MakeQIn(*in_q), rq, xin, yout);
     else
         hipLaunchKernelGGL(SoftmaxKernel, dim3(rows), dim3(64), 0, ToHip(stream), static_cast<int>(cols), beta, MakeQIn(*in_q), rq, xin, yout);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+int mi355x_pad_run(const mi355x_pad_desc* d, const void* input_dev, void* output_dev, mi355x_stream_t stream)
+{
+    if (!d) return SetError(MI355X_ERR_INVALID_ARGUMENT, "descriptor is null");
+    if (d->rank < 1 || d->rank > 4) return SetError(MI355X_ERR_UNSUPPORTED, "Pad of rank %u (1..4 run on the device)", d->rank);
+    if (int rc = CheckQ(&d->input, "input")) return rc;
+    if (int rc = CheckQ(&d->output, "output")) return rc;
+    if (d->input.dtype != d->output.dtype) return SetError(MI355X_ERR_INVALID_ARGUMENT, "input and output data types differ");
+    if (std::isnan(d->pad_value)) return SetError(MI355X_ERR_INVALID_ARGUMENT, "pad value is not a number");
+
+    // merge every unpadded dimension into its outer neighbour
+    unsigned long long out[4], in[4], before[4];
+    int n = 0;
+    for (uint32_t k = 0; k < d->rank; ++k)
+    {
+        const unsigned long long o = static_cast<unsigned long long>(d->in_shape[k]) + d->pad_before[k] + d->pad_after[k];
+        const bool unpadded = d->pad_before[k] == 0 && d->pad_after[k] == 0;
+        if (n > 0 && unpadded)
+        {
+            out[n - 1] *= o; in[n - 1] *= o; before[n - 1] *= o;
+        }
+        else
+        {
+            out[n] = o; in[n] = d->in_shape[k]; before[n] = d->pad_before[k];
+            ++n;
+        }
+    }
+    unsigned long long total = 1, in_total = 1, rows = 1;
+    for (int k = 0; k < n; ++k) { total *= out[k]; in_total *= in[k]; }
+    if (total == 0) return 0;
+    if ((!input_dev && in_total != 0) || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "null tensor pointer");
+    PadArgs p;
+    for (int k = 0; k < 4; ++k) { p.out[k] = 1; p.in[k] = 1; p.before[k] = 0; }
+    for (int k = 0; k < n; ++k)
+    {
+        if (out[k] > 0xffffffffull) return SetError(MI355X_ERR_UNSUPPORTED, "Pad: a merged extent exceeds 32 bits");
+        p.out[4 - n + k] = static_cast<uint32_t>(out[k]);
+        p.in[4 - n + k] = static_cast<uint32_t>(in[k]);
+        p.before[4 - n + k] = static_cast<uint32_t>(before[k]);
+    }
+    for (int k = 0; k < 3; ++k) rows *= p.out[k];
+
+    // Quantize<T>(value, 1, 0): round half away from zero, then saturate (TypesUtils.cpp:29-45)
+    const bool u8 = d->output.dtype == MI355X_QASYMM_U8;
+    float code = std::round(d->pad_value);
+    code = std::min(std::max(code, u8 ? 0.0f : -128.0f), u8 ? 255.0f : 127.0f);
+    const uint32_t byte = static_cast<uint32_t>(static_cast<int>(code)) & 0xffu;
+    p.fill = byte * 0x01010101u;
+    p.identity = d->input.scale == d->output.scale && d->input.offset == d->output.offset;
+
+    const uintptr_t align = reinterpret_cast<uintptr_t>(input_dev) | reinterpret_cast<uintptr_t>(output_dev);
+    const uint32_t inner = p.out[3] | p.in[3] | p.before[3];
+    const int v = ((inner | align) & 15) == 0 ? 16 : ((inner | align) & 3) == 0 ? 4 : 1;
+    const unsigned long long chunks = (p.out[3] / v + 255) / 256;
+    if (rows * chunks > 0x7fffffffull) return SetError(MI355X_ERR_UNSUPPORTED, "Pad: tensor too large for one launch");
+    Requant rq = MakeRequant(d->output, MI355X_ACT_NONE, 0.0f, 0.0f);
+    const dim3 grid(static_cast<unsigned>(rows * chunks));
+    const uint8_t* xin = static_cast<const uint8_t*>(input_dev);
+    uint8_t* yout = static_cast<uint8_t*>(output_dev);
+    if (v == 16)
+        hipLaunchKernelGGL(PadKernel<16>, grid, dim3(256), 0, ToHip(stream), p, MakeQIn(d->input), rq, static_cast<uint32_t>(chunks), xin, yout);
+    else if (v == 4)
+        hipLaunchKernelGGL(PadKernel<4>, grid, dim3(256), 0, ToHip(stream), p, MakeQIn(d->input), rq, static_cast<uint32_t>(chunks), xin, yout);
+    else
+        hipLaunchKernelGGL(PadKernel<1>, grid, dim3(256), 0, ToHip(stream), p, MakeQIn(d->input), rq, static_cast<uint32_t>(chunks), xin, yout);
     MI355X_HIP(hipGetLastError());
     return 0;
 }

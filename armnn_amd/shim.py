@@ -30,7 +30,7 @@ EXPORTS = [
     "mi355x_conv2d_create", "mi355x_conv2d_run", "mi355x_conv2d_destroy", "mi355x_conv2d_algo",
     "mi355x_conv2d_fusable", "mi355x_conv2d_run_fused",
     "mi355x_fc_create", "mi355x_fc_run", "mi355x_fc_destroy", "mi355x_fc_algo",
-    "mi355x_activation_run", "mi355x_pool2d_run", "mi355x_add_run", "mi355x_softmax_run",
+    "mi355x_activation_run", "mi355x_pool2d_run", "mi355x_add_run", "mi355x_softmax_run", "mi355x_pad_run",
 ]
 
 
@@ -68,6 +68,11 @@ class Pool2dDesc(C.Structure):
                 ("stride_y", C.c_uint32), ("pad_left", C.c_uint32), ("pad_right", C.c_uint32),
                 ("pad_top", C.c_uint32), ("pad_bottom", C.c_uint32), ("pool_type", C.c_int32),
                 ("padding_method", C.c_int32), ("input", Quant), ("output", Quant)]
+
+
+class PadDesc(C.Structure):
+    _fields_ = [("rank", C.c_uint32), ("in_shape", C.c_uint32 * 4), ("pad_before", C.c_uint32 * 4),
+                ("pad_after", C.c_uint32 * 4), ("pad_value", C.c_float), ("input", Quant), ("output", Quant)]
 
 
 class ShimError(RuntimeError):
@@ -113,6 +118,7 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
             "mi355x_add_run": [C.c_size_t, C.POINTER(Quant), C.POINTER(Quant), C.POINTER(Quant), C.c_int32, C.c_float,
                                C.c_float, V, V, V, V],
             "mi355x_softmax_run": [C.c_uint32, C.c_uint32, C.c_float, C.POINTER(Quant), C.POINTER(Quant), V, V, V],
+            "mi355x_pad_run": [C.POINTER(PadDesc), V, V, V],
             "mi355x_device_count": [C.POINTER(C.c_int)], "mi355x_init": [C.c_int],
             "mi355x_set_option": [C.c_char_p, C.c_int],
             "mi355x_device_name": [C.c_char_p, C.c_size_t],
@@ -422,5 +428,28 @@ def softmax(x: QTensor, out_info: TensorInfo, beta=1.0) -> QTensor:
     yd = DeviceBuffer(y.data.nbytes)
     qi, qo = _quant(x.info), _quant(out_info)
     _chk(lib.mi355x_softmax_run(rows, cols, beta, C.byref(qi), C.byref(qo), xd.ptr, yd.ptr, None))
+    y.data = yd.download(out_info.shape, numpy_dtype(out_info.dtype))
+    return y
+
+
+def pad_desc(in_shape, pad_list, pad_value, in_info: TensorInfo, out_info: TensorInfo) -> PadDesc:
+    """pad_list holds one (before, after) pair per dimension, as armnn::PadDescriptor::m_PadList does."""
+    d = PadDesc()
+    d.rank = len(in_shape)
+    for k, (extent, (before, after)) in enumerate(zip(in_shape, pad_list)):
+        d.in_shape[k], d.pad_before[k], d.pad_after[k] = extent, before, after
+    d.pad_value = float(pad_value)
+    d.input, d.output = _quant(in_info), _quant(out_info)
+    return d
+
+
+def pad(x: QTensor, out_info: TensorInfo, pad_list, pad_value=0.0) -> QTensor:
+    Device()
+    lib = load_library()
+    d = pad_desc(x.info.shape, pad_list, pad_value, x.info, out_info)
+    xd = DeviceBuffer(max(x.data.nbytes, 1)).upload(x.data)
+    y = QTensor(out_info)
+    yd = DeviceBuffer(max(y.data.nbytes, 1))
+    _chk(lib.mi355x_pad_run(C.byref(d), xd.ptr, yd.ptr, None))
     y.data = yd.download(out_info.shape, numpy_dtype(out_info.dtype))
     return y

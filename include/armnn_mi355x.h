@@ -263,6 +263,21 @@ int mi355x_softmax_run(uint32_t rows, uint32_t cols, float beta, const mi355x_qu
                        const mi355x_quant* out_q, const void* input_dev, void* output_dev,
                        mi355x_stream_t stream);
 
+/* Pad with a constant, rank 1..4: Pad() (workloads/Pad.cpp:39-236) as RefPadWorkload::Execute calls it
+ * (workloads/RefPadWorkload.cpp:18-40).  Fields mirror armnn::PadDescriptor (include/armnn/Descriptors.hpp:1196-1229):
+ * pad_before[d] / pad_after[d] are m_PadList[d].first / .second.  pad_value is the stored code of the padding
+ * (rounded half away from zero and saturated to the type), not a real number: the reference encodes it with scale 1
+ * and offset 0 (Pad.cpp:77-84).  Elements of the input are decoded with `input` and encoded with `output`; with equal
+ * quantizations they are copied. */
+typedef struct {
+    uint32_t rank;
+    uint32_t in_shape[4];
+    uint32_t pad_before[4], pad_after[4];
+    float    pad_value;
+    mi355x_quant input, output;
+} mi355x_pad_desc;
+int mi355x_pad_run(const mi355x_pad_desc* desc, const void* input_dev, void* output_dev, mi355x_stream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

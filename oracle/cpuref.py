@@ -80,6 +80,7 @@ class Oracle:
         f("pooling2d", C.c_int, [TP, TP, C.POINTER(_PoolParams), C.c_int])
         f("softmax", C.c_int, [TP, TP, C.c_float, C.c_int])
         f("add", C.c_int, [TP, TP, TP])
+        f("pad", C.c_int, [TP, TP, C.POINTER(C.c_uint32), C.c_float])
         f("last_error", C.c_char_p, [])
 
     def _fn(self, name, restype, argtypes):
@@ -177,6 +178,15 @@ class Oracle:
         keep = []
         sx, sy = self._t(x, keep), self._t(y, keep)
         self._check(self._softmax(C.byref(sx), C.byref(sy), float(beta), int(axis)))
+        return y
+
+    def pad(self, x: QTensor, out_info: TensorInfo, pad_before, pad_value: float = 0.0) -> QTensor:
+        """Constant padding; what is added behind each dimension follows from out_info.shape."""
+        y = QTensor(out_info)
+        keep = []
+        sx, sy = self._t(x, keep), self._t(y, keep)
+        before = (C.c_uint32 * len(pad_before))(*[int(v) for v in pad_before])
+        self._check(self._pad(C.byref(sx), C.byref(sy), before, float(pad_value)))
         return y
 
     def add(self, a: QTensor, b: QTensor, out_info: TensorInfo) -> QTensor:

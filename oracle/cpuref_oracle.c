@@ -660,3 +660,51 @@ done:
     free(f0); free(f1); free(fo);
     return rc;
 }
+
+/* ------------------------------------------------------------------------------------------------
+ * Pad -- workloads/Pad.cpp:39-236.  The output is first filled with the pad value; for quantized
+ * outputs through an encoder of scale 1 and offset 0 (Pad.cpp:77-84), so the value is a code.  Then
+ * every input element is decoded with the input's quantization and encoded with the output's at
+ * its shifted position (Pad.cpp:93-233; the nested loops there are this one index walk).
+ * ---------------------------------------------------------------------------------------------- */
+int orc_pad(const orc_tensor* in, const orc_tensor* out, const uint32_t* pad_before, float pad_value)
+{
+    const uint32_t nd = in->ndim;
+    if (out->ndim != nd || nd == 0 || nd > 6) return fail("pad: ranks must match (1..6)");
+    for (uint32_t d = 0; d < nd; ++d)
+        if (pad_before[d] + in->shape[d] > out->shape[d]) return fail("pad: output too small");
+    const size_t n_in = num_elements(in), n_out = num_elements(out);
+    const size_t esz = out->dtype == ORC_FLOAT32 ? 4 : 1;
+    float* f = (float*)malloc(((n_in > n_out ? n_in : n_out) + 1) * sizeof(float));
+    uint8_t* packed = (uint8_t*)malloc(n_in * esz + 1);
+    int rc = -1;
+    if (!f || !packed) { fail("out of memory"); goto done; }
+    {
+        static const float one = 1.0f;
+        orc_tensor fill = *out;
+        if (out->dtype != ORC_FLOAT32) { fill.scales = &one; fill.n_scales = 1; fill.quant_dim = -1; fill.offset = 0; }
+        for (size_t i = 0; i < n_out; ++i) f[i] = pad_value;
+        if (orc_encode_tensor(f, n_out, &fill)) goto done;
+    }
+    if (orc_decode_tensor(in, 0, f)) goto done;
+    {
+        orc_tensor compact = *out;
+        compact.data = packed;
+        if (orc_encode_tensor(f, n_in, &compact)) goto done;
+    }
+    for (size_t i = 0; i < n_in; ++i)
+    {
+        size_t rem = i, o = 0, stride = 1;
+        for (int d = (int)nd - 1; d >= 0; --d)
+        {
+            size_t idx = rem % in->shape[d]; rem /= in->shape[d];
+            o += (idx + pad_before[d]) * stride;
+            stride *= out->shape[d];
+        }
+        memcpy((uint8_t*)out->data + o * esz, packed + i * esz, esz);
+    }
+    rc = 0;
+done:
+    free(f); free(packed);
+    return rc;
+}

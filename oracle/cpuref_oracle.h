@@ -113,6 +113,11 @@ int orc_softmax(const orc_tensor* in, const orc_tensor* out, float beta, int axi
 /* RefElementwiseBinaryWorkload.cpp:27-107 (BinaryOperation::Add, float path) with Broadcast.cpp:11-33 */
 int orc_add(const orc_tensor* in0, const orc_tensor* in1, const orc_tensor* out);
 
+/* workloads/Pad.cpp:39-236 (constant padding, any rank up to 6): pad_before[d] elements are added in front of
+ * dimension d; what is added behind follows from the output shape.  For quantized outputs pad_value is the
+ * stored code (rounded, saturated), not a real number. */
+int orc_pad(const orc_tensor* in, const orc_tensor* out, const uint32_t* pad_before, float pad_value);
+
 const char* orc_last_error(void);
 
 #ifdef __cplusplus

@@ -5,10 +5,10 @@
 // lie in the reference tree (see oracle/Makefile, target _ref), into oracle/_ref/libarmnn_cpuref_hotpath.so.
 // It does for each call what the reference workloads do in Execute(): build TensorInfos, make
 // decoders/encoders with MakeDecoder/MakeEncoder, and call Convolve / FullyConnected / Activation /
-// Pooling2d / Softmax / ElementwiseBinaryFunction (RefConvolution2dWorkload.cpp:38-58,
+// Pooling2d / Softmax / ElementwiseBinaryFunction / Pad (RefConvolution2dWorkload.cpp:38-58,
 // RefDepthwiseConvolution2dWorkload.cpp:38-62, RefFullyConnectedWorkload.cpp:39-67,
 // RefActivationWorkload.cpp:23-36, RefPooling2dWorkload.cpp, RefSoftmaxWorkload.cpp,
-// RefElementwiseBinaryWorkload.cpp:27-107).  It is used to validate the C restatement
+// RefElementwiseBinaryWorkload.cpp:27-107, RefPadWorkload.cpp:18-40).  It is used to validate the C restatement
 // (cpuref_oracle.c), to generate golden fixtures, and as the timed CPU baseline.
 //
 #include "cpuref_oracle.h"
@@ -19,12 +19,14 @@
 #include "Pooling2d.hpp"
 #include "Softmax.hpp"
 #include "ElementwiseFunction.hpp"
+#include "Pad.hpp"
 #include "Decoders.hpp"
 #include "Encoders.hpp"
 
 #include <armnn/Descriptors.hpp>
 #include <armnn/Tensor.hpp>
 #include <armnn/TypesUtils.hpp>
+#include <armnn/backends/ITensorHandle.hpp>
 
 #include <cstring>
 #include <functional>
@@ -64,6 +66,25 @@ TensorInfo ToInfo(const orc_tensor* t)
     info.SetQuantizationOffset(t->offset);
     return info;
 }
+
+// the caller's memory behind the tensor-handle interface Pad() reads and writes through
+class BorrowedHandle : public ITensorHandle
+{
+public:
+    BorrowedHandle(void* memory, const TensorShape& shape) : m_Memory(memory), m_Shape(shape) {}
+    void Manage() override {}
+    void Allocate() override {}
+    ITensorHandle* GetParent() const override { return nullptr; }
+    const void* Map(bool) const override { return m_Memory; }
+    void Unmap() const override {}
+    TensorShape GetStrides() const override { return m_Shape; }
+    TensorShape GetShape() const override { return m_Shape; }
+    void CopyOutTo(void*) const override {}
+    void CopyInFrom(const void*) override {}
+private:
+    void* m_Memory;
+    TensorShape m_Shape;
+};
 
 template <typename F>
 int Guard(F&& f)
@@ -184,6 +205,19 @@ int ref_add(const orc_tensor* in0, const orc_tensor* in1, const orc_tensor* out)
         auto d1 = MakeDecoder<float>(i1, in1->data);
         auto enc = MakeEncoder<float>(oi, out->data);
         ElementwiseBinaryFunction<std::plus<float>>(i0.GetShape(), i1.GetShape(), oi.GetShape(), *d0, *d1, *enc);
+    });
+}
+
+int ref_pad(const orc_tensor* in, const orc_tensor* out, const uint32_t* pad_before, float pad_value)
+{
+    return Guard([&] {
+        TensorInfo ii = ToInfo(in), oi = ToInfo(out);
+        PadQueueDescriptor q;
+        for (uint32_t d = 0; d < in->ndim; ++d)
+            q.m_Parameters.m_PadList.emplace_back(pad_before[d], out->shape[d] - in->shape[d] - pad_before[d]);
+        q.m_Parameters.m_PadValue = pad_value;
+        BorrowedHandle ih(in->data, ii.GetShape()), oh(out->data, oi.GetShape());
+        Pad(ii, oi, &ih, &oh, q);
     });
 }
 

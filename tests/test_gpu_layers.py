@@ -90,3 +90,79 @@ def test_activation_requantizing(port, dtype, act):
     want = port.activation(x, oi, *act)
     got = shim.activation(x, oi, *act)
     np.testing.assert_array_equal(got.data, want.data)
+
+
+PADS = [
+    # (name, input shape, (before, after) per dimension, pad value, output (scale, offset shift) or None)
+    ("nhwc_hw_c64_16B", (2, 14, 14, 64), ((0, 0), (1, 1), (1, 1), (0, 0)), None, None),      # 16-byte units
+    ("nhwc_same_s2_c32", (3, 112, 112, 32), ((0, 0), (0, 1), (0, 1), (0, 0)), None, None),
+    ("nhwc_hw_c12_4B", (2, 9, 7, 12), ((0, 0), (2, 1), (1, 3), (0, 0)), 5.0, None),          # 4-byte units
+    ("nhwc_hw_c3_1B", (1, 10, 11, 3), ((0, 0), (1, 2), (3, 0), (0, 0)), -2.5, None),         # byte units; rounds to -3
+    ("all_dims", (2, 4, 4, 3), ((1, 0), (1, 1), (1, 1), (2, 3)), 300.0, None),               # saturating code
+    ("requantized", (2, 6, 5, 16), ((0, 0), (1, 1), (2, 2), (0, 0)), 1.0, (0.07, 5)),
+    ("requantized_bytes", (3, 7), ((1, 0), (2, 3)), -300.0, (0.031, -2)),
+    ("rank1", (37,), ((2, 1),), 4.0, None),
+    ("rank3", (2, 3, 40), ((1, 0), (0, 1), (8, 0)), 0.0, None),
+    ("no_padding", (2, 5, 5, 8), ((0, 0), (0, 0), (0, 0), (0, 0)), 0.0, None),
+    ("batch_padded", (2, 3, 3, 16), ((1, 2), (0, 0), (0, 0), (0, 0)), 9.0, None),
+]
+
+
+@pytest.mark.parametrize("cfg", PADS, ids=[c[0] for c in PADS])
+@pytest.mark.parametrize("dtype", [S8, U8])
+def test_pad(port, cfg, dtype):
+    """Bytes are moved or re-coded one at a time: exact against the checker, and against numpy's constant padding
+    wherever input and output share one quantization."""
+    name, shape, pads, value, outq = cfg
+    print("pad", name, dtype, flush=True)
+    lo, hi = (0, 255) if dtype == U8 else (-128, 127)
+    zp = lo + 20
+    x = _rand(61, shape, dtype, 0.05, zp)
+    if value is None:
+        value = float(zp)                                   # the neutral element a folded convolution would use
+    oshape = tuple(s + b + a for s, (b, a) in zip(shape, pads))
+    oi = TensorInfo(oshape, dtype, (outq[0],), zp + outq[1]) if outq else TensorInfo(oshape, dtype, (0.05,), zp)
+    want = port.pad(x, oi, [b for b, _ in pads], value)
+    got = shim.pad(x, oi, pads, value)
+    np.testing.assert_array_equal(got.data, want.data)
+    if outq is None:
+        code = int(np.clip(np.sign(value) * np.floor(abs(value) + 0.5), lo, hi))
+        np.testing.assert_array_equal(got.data, np.pad(x.data, pads, constant_values=code))
+
+
+def test_pad_rejects_what_it_cannot_run():
+    with pytest.raises(shim.ShimError):
+        d = shim.PadDesc()
+        d.rank = 5
+        shim._chk(shim.load_library().mi355x_pad_run(shim.C.byref(d), None, None, None))
+    with pytest.raises(shim.ShimError):
+        shim.pad(_rand(63, (4,), S8, 0.05, 0), TensorInfo((6,), S8, (0.05,), 0), ((1, 1),), float("nan"))
+
+
+FOLDS = [
+    # (name, make_conv_case keywords): the layer's own padding is what a Pad layer in front of it would have added
+    ("conv3x3", dict(n=2, h=13, w=15, ci=16, co=32, padding=(1, 2, 2, 1))),
+    ("conv3x3_s2_u8", dict(n=1, h=14, w=14, ci=32, co=16, stride=(2, 2), padding=(0, 1, 0, 1), in_dtype=U8, in_offset=7, out_offset=0)),
+    ("depthwise3x3_s2", dict(n=2, h=28, w=28, ci=64, depthwise=True, stride=(2, 2), padding=(0, 1, 0, 1))),
+    ("depthwise3x3", dict(n=1, h=9, w=9, ci=24, depthwise=True, padding=(2, 2, 2, 2))),
+    ("conv1x1_padded", dict(n=1, h=6, w=6, ci=64, co=64, kh=1, kw=1, padding=(1, 1, 1, 1))),
+    ("stem7x7_s2", dict(n=2, h=32, w=32, ci=3, co=64, kh=7, kw=7, stride=(2, 2), padding=(3, 3, 3, 3))),
+]
+
+
+@pytest.mark.parametrize("cfg", FOLDS, ids=[c[0] for c in FOLDS])
+def test_padding_inside_the_convolution_equals_a_pad_layer_in_front_of_it(cfg):
+    """What folding a Pad layer into the convolution relies on: padding with the input's zero point and then running
+    the unpadded convolution gives the bytes of the convolution with that padding as its own."""
+    from tests.cases import make_conv_case
+    name, kw = cfg
+    print("fold", name, flush=True)
+    c = make_conv_case(name, 901, **kw)
+    pt, pb, pl, pr = kw["padding"]
+    folded = shim.conv2d(c.x, c.w, c.b, c.out_info, activation=c.act[0], act_a=c.act[1], act_b=c.act[2], **c.params)
+    n, h, w, ci = c.x.info.shape
+    pinfo = TensorInfo((n, h + pt + pb, w + pl + pr, ci), c.x.info.dtype, c.x.info.scales, c.x.info.offset)
+    padded = shim.pad(c.x, pinfo, ((0, 0), (pt, pb), (pl, pr), (0, 0)), float(c.x.info.offset))
+    params = dict(c.params, pad_top=0, pad_left=0)
+    apart = shim.conv2d(padded, c.w, c.b, c.out_info, activation=c.act[0], act_a=c.act[1], act_b=c.act[2], **params)
+    np.testing.assert_array_equal(folded.data, apart.data)

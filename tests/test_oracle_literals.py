@@ -55,3 +55,21 @@ def test_round_half_away_from_zero(port):
     assert port.quantize(-2.5, 1.0, 0, DataType.QAsymmS8) == -3
     assert port.quantize(1e9, 1.0, 0, DataType.QAsymmS8) == 127
     assert port.quantize(-1e9, 1.0, 0, DataType.QAsymmU8) == 0
+
+
+# PadQAsymmTestCommon (src/backends/backendsCommon/test/layerTests/PadTestImpl.cpp:491-565): a 3x3 tensor of raw codes
+# padded by 2 on every side; the expected border holds the pad value itself as a code, whatever scale and offset are.
+# PadInt8AsymmTest :758-765 (scale 2, offset 2, pad value 0) and PadInt8CustomPaddingAsymmTest :767-775 (scale 2,
+# offset 3, pad value 1).
+@pytest.mark.parametrize("scale,offset,value", [(2.0, 2, 0.0), (2.0, 3, 1.0)])
+@pytest.mark.parametrize("which", ["port", "reference"])
+def test_pad_qasymm_literals(request, which, scale, offset, value):
+    from armnn_amd.tensor import DataType, QTensor, TensorInfo
+    orc = request.getfixturevalue(which)
+    codes = np.array([[4, 8, 6], [7, 4, 4], [3, 2, 4]])
+    for dtype in (DataType.QAsymmS8, DataType.QAsymmU8):
+        x = QTensor(TensorInfo((3, 3), dtype, (scale,), offset), codes)
+        want = np.full((7, 7), int(value))
+        want[2:5, 2:5] = codes
+        got = orc.pad(x, TensorInfo((7, 7), dtype, (scale,), offset), [2, 2], value)
+        np.testing.assert_array_equal(got.data.astype(np.int32), want)

@@ -110,3 +110,31 @@ def test_softmax_and_add_bit_exact(port, reference, dtype):
     np.testing.assert_array_equal(port.add(a, b, oi).data, reference.add(a, b, oi).data)
     b1 = QTensor(TensorInfo((1, 1, 1, 16), dtype, (0.05,), lo + 90), synth.uniform_int(24, (1, 1, 1, 16), lo, hi, np.int64))
     np.testing.assert_array_equal(port.add(a, b1, oi).data, reference.add(a, b1, oi).data)
+
+
+PAD = [
+    # (input shape, (before, after) per dimension, pad value, output quantization or None for the input's)
+    ((2, 5, 6, 8), ((0, 0), (1, 2), (2, 1), (0, 0)), 3.0, None),
+    ((1, 9, 7, 16), ((0, 0), (0, 1), (0, 1), (0, 0)), -7.0, None),
+    ((2, 4, 4, 3), ((1, 0), (1, 1), (1, 1), (2, 3)), 2.5, None),          # every dimension padded; 2.5 rounds to 3
+    ((3, 7), ((1, 0), (2, 3)), -300.0, (0.07, 5)),                          # saturating pad code, re-quantized elements
+    ((4,), ((2, 1),), -3.5, None),
+    ((2, 3, 4), ((1, 0), (0, 1), (2, 0)), 1000.0, (0.031, -2)),
+]
+
+
+@pytest.mark.parametrize("cfg", PAD, ids=[str(c[0]) for c in PAD])
+@pytest.mark.parametrize("dtype", [DataType.QAsymmS8, DataType.QAsymmU8])
+def test_pad_bit_exact(port, reference, cfg, dtype):
+    shape, pads, value, outq = cfg
+    lo, hi = (0, 255) if dtype == DataType.QAsymmU8 else (-128, 127)
+    x = QTensor(TensorInfo(shape, dtype, (0.05,), lo + 20), synth.uniform_int(13, shape, lo, hi, np.int64))
+    oshape = tuple(s + b + a for s, (b, a) in zip(shape, pads))
+    oi = TensorInfo(oshape, dtype, (outq[0],), lo + 20 + outq[1]) if outq else TensorInfo(oshape, dtype, (0.05,), lo + 20)
+    before = [b for b, _ in pads]
+    p = port.pad(x, oi, before, value).data
+    np.testing.assert_array_equal(p, reference.pad(x, oi, before, value).data)
+    if outq is None:
+        # closed form: numpy's constant padding with the saturated, rounded code
+        code = int(np.clip(np.sign(value) * np.floor(abs(value) + 0.5), lo, hi))
+        np.testing.assert_array_equal(p, np.pad(x.data, pads, constant_values=code))
