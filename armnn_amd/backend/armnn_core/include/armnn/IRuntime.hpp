@@ -2,6 +2,7 @@
 #pragma once
 #include "BackendOptions.hpp"
 #include "INetwork.hpp"
+#include "IProfiler.hpp"
 #include "Tensor.hpp"
 #include "Types.hpp"
 #include <memory>
@@ -62,6 +63,9 @@ public:
                            std::vector<ImportedInputId> preImportedInputIds = {},
                            std::vector<ImportedOutputId> preImportedOutputIds = {});
     Status UnloadNetwork(NetworkId networkId);
+    /// the profiler of a loaded network; events are recorded while it is enabled (INetworkProperties::m_ProfilingEnabled
+    /// turns it on at load time)
+    const std::shared_ptr<IProfiler> GetProfiler(NetworkId networkId) const;
     const IDeviceSpec& GetDeviceSpec() const;
     ~IRuntime();
 protected:

@@ -11,5 +11,8 @@ struct WorkloadInfo
     std::vector<TensorInfo> m_InputTensorInfos;
     std::vector<TensorInfo> m_OutputTensorInfos;
     std::string m_Name;
+    Optional<TensorInfo> m_WeightsTensorInfo = EmptyOptional();
+    Optional<TensorInfo> m_BiasTensorInfo = EmptyOptional();
+    Optional<std::string> m_ConvolutionMethod = EmptyOptional();
 };
 } // namespace armnn

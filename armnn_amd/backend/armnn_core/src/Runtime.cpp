@@ -2,6 +2,7 @@
 // EnqueueWorkload (src/armnn/Runtime.cpp:301-574, src/armnn/LoadedNetwork.cpp:82-360 and :845-1100).
 #include <algorithm>
 #include <Layer.hpp>
+#include <Profiling.hpp>
 #include <armnn/BackendRegistry.hpp>
 #include <armnn/IRuntime.hpp>
 #include <armnn/backends/DynamicBackend.hpp>
@@ -33,11 +34,25 @@ struct BackendSlot
     ITensorHandleFactory* handleFactory = nullptr;   // preferred tensor handle factory, null: use the workload factory
 };
 
+// makes a profiler the calling thread's current one for a scope
+class CurrentProfiler
+{
+public:
+    explicit CurrentProfiler(IProfiler* profiler) : m_Previous(ProfilerManager::GetInstance().GetProfiler()) { ProfilerManager::GetInstance().RegisterProfiler(profiler); }
+    ~CurrentProfiler() { ProfilerManager::GetInstance().RegisterProfiler(m_Previous); }
+private:
+    IProfiler* m_Previous;
+};
+
 class LoadedNetwork
 {
 public:
-    LoadedNetwork(IOptimizedNetworkPtr net) : m_Net(std::move(net))
+    LoadedNetwork(IOptimizedNetworkPtr net, bool profilingEnabled = false) : m_Net(std::move(net)), m_Profiler(std::make_shared<IProfiler>())
     {
+        // the network's profiler is the thread's current one while its workloads are built and run
+        // (LoadedNetwork.cpp:131-136, :845-852)
+        m_Profiler->EnableProfiling(profilingEnabled);
+        CurrentProfiler current(m_Profiler.get());
         Graph& graph = m_Net->GetGraph();
         m_Order = graph.TopologicalSort();
 
@@ -120,6 +135,8 @@ public:
         m_Registry.ReleaseMemory();
     }
 
+    const std::shared_ptr<IProfiler>& GetProfiler() const { return m_Profiler; }
+
     const Layer* FindBinding(LayerType type, LayerBindingId id) const
     {
         for (const Layer* l : m_Order)
@@ -147,6 +164,8 @@ public:
         if (inputs.size() + preIn.size() != m_Net->GetNumInputs()) throw InvalidArgumentException("Number of inputs provided does not match network.");
         if (outputs.size() + preOut.size() != m_Net->GetNumOutputs()) throw InvalidArgumentException("Number of outputs provided does not match network.");
         std::lock_guard<std::mutex> lock(m_Mutex);
+        CurrentProfiler current(m_Profiler.get());
+        ARMNN_SCOPED_PROFILING_EVENT(BackendId(), "EnqueueWorkload");
         for (ImportedInputId id : preIn)
             if (id >= m_Inputs.size() || !m_Inputs[id].adopted) throw InvalidArgumentException("EnqueueWorkload: input " + std::to_string(id) + " was not imported");
         for (ImportedOutputId id : preOut)
@@ -165,7 +184,10 @@ public:
             std::memcpy(dst, in.second.GetMemoryArea(), info.GetNumBytes());
             h->Unmap();
         }
-        for (auto& w : m_Workloads) w->Execute();
+        {
+            ARMNN_SCOPED_PROFILING_EVENT(BackendId(), "Execute");
+            for (auto& w : m_Workloads) w->Execute();
+        }
         for (const auto& out : outputs)
         {
             const Layer* l = FindBinding(LayerType::Output, out.first);
@@ -379,6 +401,7 @@ private:
     std::map<const Layer*, size_t> m_WorkloadOf;
 
     IOptimizedNetworkPtr m_Net;
+    std::shared_ptr<IProfiler> m_Profiler;
     std::vector<Layer*> m_Order;
     TensorHandleFactoryRegistry m_Registry;
     std::map<BackendId, BackendSlot> m_Backends;
@@ -421,14 +444,14 @@ public:
         for (const BackendId& id : m_DeviceSpec.m_Dynamic) BackendRegistryInstance().Deregister(id);
     }
 
-    Status LoadNetwork(NetworkId& idOut, IOptimizedNetworkPtr network, std::string& error)
+    Status LoadNetwork(NetworkId& idOut, IOptimizedNetworkPtr network, std::string& error, bool profilingEnabled = false)
     {
         const NetworkId id = m_NextId++;
         idOut = id;
         for (auto& c : m_Contexts) c.second->BeforeLoadNetwork(id);
         try
         {
-            m_Networks[id] = std::make_unique<LoadedNetwork>(std::move(network));
+            m_Networks[id] = std::make_unique<LoadedNetwork>(std::move(network), profilingEnabled);
         }
         catch (const Exception& e)
         {
@@ -492,10 +515,11 @@ Status IRuntime::LoadNetwork(NetworkId& id, IOptimizedNetworkPtr network)
     return pRuntimeImpl->LoadNetwork(id, std::move(network), ignored);
 }
 Status IRuntime::LoadNetwork(NetworkId& id, IOptimizedNetworkPtr network, std::string& error) { return pRuntimeImpl->LoadNetwork(id, std::move(network), error); }
-Status IRuntime::LoadNetwork(NetworkId& id, IOptimizedNetworkPtr network, std::string& error, const INetworkProperties&)
+Status IRuntime::LoadNetwork(NetworkId& id, IOptimizedNetworkPtr network, std::string& error, const INetworkProperties& properties)
 {
-    return pRuntimeImpl->LoadNetwork(id, std::move(network), error);
+    return pRuntimeImpl->LoadNetwork(id, std::move(network), error, properties.m_ProfilingEnabled);
 }
+const std::shared_ptr<IProfiler> IRuntime::GetProfiler(NetworkId id) const { return pRuntimeImpl->Get(id).GetProfiler(); }
 TensorInfo IRuntime::GetInputTensorInfo(NetworkId id, LayerBindingId layerId) const { return pRuntimeImpl->Get(id).GetInputTensorInfo(layerId); }
 TensorInfo IRuntime::GetOutputTensorInfo(NetworkId id, LayerBindingId layerId) const { return pRuntimeImpl->Get(id).GetOutputTensorInfo(layerId); }
 Status IRuntime::EnqueueWorkload(NetworkId id, const InputTensors& in, const OutputTensors& out, std::vector<ImportedInputId> preIn,

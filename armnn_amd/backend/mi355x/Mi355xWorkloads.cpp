@@ -1,5 +1,9 @@
 #include "Mi355xWorkloads.hpp"
+#include "Mi355xBackendId.hpp"
 #include "Mi355xTensorHandle.hpp"
+#include "Mi355xTimer.hpp"
+
+#include <Profiling.hpp>
 
 #include <armnn/backends/TensorHandle.hpp>
 #include <armnn/utility/PolymorphicDowncast.hpp>
@@ -24,6 +28,20 @@ void* Out(ITensorHandle* h)
     const Mi355xTensorHandle& d = Dev(h);
     d.MarkDeviceWritten();
     return d.GetDevicePointer();
+}
+
+// the kernel a plan resolved to, for the profiler's details record
+std::string Describe(mi355x_conv2d_t plan)
+{
+    int32_t algo = 0;
+    char buf[256] = {0};
+    return mi355x_conv2d_algo(plan, &algo, buf, sizeof(buf)) == 0 ? std::string(buf) : std::string();
+}
+std::string Describe(mi355x_fc_t plan)
+{
+    int32_t algo = 0;
+    char buf[256] = {0};
+    return mi355x_fc_algo(plan, &algo, buf, sizeof(buf)) == 0 ? std::string(buf) : std::string();
 }
 
 // Host copy of a constant operand plus its quantization in C-ABI form.  The copy is taken through Map(), so it
@@ -68,6 +86,7 @@ Mi355xFusedActivation Mi355xFusedActivation::From(const ActivationDescriptor* d)
 Mi355xConvolution2dWorkload::Mi355xConvolution2dWorkload(const Convolution2dQueueDescriptor& descriptor, const WorkloadInfo& info)
     : Mi355xBaseWorkload<Convolution2dQueueDescriptor>(descriptor, info), m_Info(info)
 {
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xConvolution2dWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
     if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xConvolution2dWorkload: NHWC only");
     Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());   // validates early
 }
@@ -107,10 +126,14 @@ void Mi355xConvolution2dWorkload::BuildPlan() const
                                        bias ? reinterpret_cast<const int32_t*>(bias->data.data()) : nullptr,
                                        bias ? &bias->quant : nullptr, &m_Plan),
                   "mi355x_conv2d_create");
+    WorkloadInfo details = m_Info;
+    details.m_ConvolutionMethod = Optional<std::string>(Describe(m_Plan));
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xConvolution2dWorkload_Plan", m_Data.m_Parameters, details, this->GetGuid());
 }
 
 void Mi355xConvolution2dWorkload::Execute() const
 {
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xConvolution2dWorkload_Execute");
     std::call_once(m_Once, [this] { BuildPlan(); });
     if (!m_Plan) throw RuntimeException("Mi355xConvolution2dWorkload: no device plan (its creation failed earlier)");
     const uint32_t batch = m_Info.m_InputTensorInfos[0].GetShape()[0];
@@ -130,6 +153,7 @@ std::string Mi355xConvolution2dWorkload::GetKernelDescription() const
 Mi355xDepthwiseConvolution2dWorkload::Mi355xDepthwiseConvolution2dWorkload(const DepthwiseConvolution2dQueueDescriptor& descriptor, const WorkloadInfo& info)
     : Mi355xBaseWorkload<DepthwiseConvolution2dQueueDescriptor>(descriptor, info), m_Info(info)
 {
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xDepthwiseConvolution2dWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
     if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xDepthwiseConvolution2dWorkload: NHWC only");
     Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
 }
@@ -169,10 +193,14 @@ void Mi355xDepthwiseConvolution2dWorkload::BuildPlan() const
                                        bias ? reinterpret_cast<const int32_t*>(bias->data.data()) : nullptr,
                                        bias ? &bias->quant : nullptr, &m_Plan),
                   "mi355x_conv2d_create(depthwise)");
+    WorkloadInfo details = m_Info;
+    details.m_ConvolutionMethod = Optional<std::string>(Describe(m_Plan));
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xDepthwiseConvolution2dWorkload_Plan", m_Data.m_Parameters, details, this->GetGuid());
 }
 
 void Mi355xDepthwiseConvolution2dWorkload::Execute() const
 {
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xDepthwiseConvolution2dWorkload_Execute");
     std::call_once(m_Once, [this] { BuildPlan(); });
     if (!m_Plan) throw RuntimeException("Mi355xDepthwiseConvolution2dWorkload: no device plan (its creation failed earlier)");
     const uint32_t batch = m_Info.m_InputTensorInfos[0].GetShape()[0];
@@ -183,6 +211,7 @@ void Mi355xDepthwiseConvolution2dWorkload::Execute() const
 Mi355xFullyConnectedWorkload::Mi355xFullyConnectedWorkload(const FullyConnectedQueueDescriptor& descriptor, const WorkloadInfo& info)
     : Mi355xBaseWorkload<FullyConnectedQueueDescriptor>(descriptor, info), m_Info(info)
 {
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xFullyConnectedWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
     Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
 }
 
@@ -217,10 +246,14 @@ void Mi355xFullyConnectedWorkload::BuildPlan() const
                                    bias ? reinterpret_cast<const int32_t*>(bias->data.data()) : nullptr,
                                    bias ? &bias->quant : nullptr, &m_Plan),
                   "mi355x_fc_create");
+    WorkloadInfo details = m_Info;
+    details.m_ConvolutionMethod = Optional<std::string>(Describe(m_Plan));
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xFullyConnectedWorkload_Plan", m_Data.m_Parameters, details, this->GetGuid());
 }
 
 void Mi355xFullyConnectedWorkload::Execute() const
 {
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xFullyConnectedWorkload_Execute");
     std::call_once(m_Once, [this] { BuildPlan(); });
     if (!m_Plan) throw RuntimeException("Mi355xFullyConnectedWorkload: no device plan (its creation failed earlier)");
     const uint32_t batch = m_Info.m_InputTensorInfos[0].GetShape()[0];
@@ -231,11 +264,13 @@ void Mi355xFullyConnectedWorkload::Execute() const
 Mi355xActivationWorkload::Mi355xActivationWorkload(const ActivationQueueDescriptor& descriptor, const WorkloadInfo& info)
     : Mi355xBaseWorkload<ActivationQueueDescriptor>(descriptor, info), m_Info(info)
 {
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xActivationWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
     Mi355xFusedActivation::From(&m_Data.m_Parameters);
 }
 
 void Mi355xActivationWorkload::Execute() const
 {
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xActivationWorkload_Execute");
     const Mi355xFusedActivation act = Mi355xFusedActivation::From(&m_Data.m_Parameters);
     const mi355x_quant qi = mi355x::ToQuant(m_Info.m_InputTensorInfos[0]);
     const mi355x_quant qo = mi355x::ToQuant(m_Info.m_OutputTensorInfos[0]);
@@ -248,11 +283,13 @@ void Mi355xActivationWorkload::Execute() const
 Mi355xPooling2dWorkload::Mi355xPooling2dWorkload(const Pooling2dQueueDescriptor& descriptor, const WorkloadInfo& info)
     : Mi355xBaseWorkload<Pooling2dQueueDescriptor>(descriptor, info), m_Info(info)
 {
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xPooling2dWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
     if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xPooling2dWorkload: NHWC only");
 }
 
 void Mi355xPooling2dWorkload::Execute() const
 {
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xPooling2dWorkload_Execute");
     const TensorInfo& in = m_Info.m_InputTensorInfos[0];
     const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
     const Pooling2dDescriptor& p = m_Data.m_Parameters;
@@ -272,12 +309,14 @@ void Mi355xPooling2dWorkload::Execute() const
 Mi355xPadWorkload::Mi355xPadWorkload(const PadQueueDescriptor& descriptor, const WorkloadInfo& info)
     : Mi355xBaseWorkload<PadQueueDescriptor>(descriptor, info), m_Info(info)
 {
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xPadWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
     if (m_Data.m_Parameters.m_PaddingMode != PaddingMode::Constant) throw InvalidArgumentException("Mi355xPadWorkload: constant padding only");
     if (m_Info.m_InputTensorInfos[0].GetNumDimensions() > 4) throw InvalidArgumentException("Mi355xPadWorkload: at most 4 dimensions");
 }
 
 void Mi355xPadWorkload::Execute() const
 {
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xPadWorkload_Execute");
     const TensorInfo& in = m_Info.m_InputTensorInfos[0];
     const PadDescriptor& p = m_Data.m_Parameters;
     mi355x_pad_desc d{};
@@ -298,10 +337,12 @@ void Mi355xPadWorkload::Execute() const
 Mi355xSoftmaxWorkload::Mi355xSoftmaxWorkload(const SoftmaxQueueDescriptor& descriptor, const WorkloadInfo& info)
     : Mi355xBaseWorkload<SoftmaxQueueDescriptor>(descriptor, info), m_Info(info)
 {
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xSoftmaxWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
 }
 
 void Mi355xSoftmaxWorkload::Execute() const
 {
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xSoftmaxWorkload_Execute");
     const TensorInfo& in = m_Info.m_InputTensorInfos[0];
     const unsigned int rank = in.GetNumDimensions();
     const uint32_t cols = in.GetShape()[rank - 1];
@@ -316,12 +357,14 @@ void Mi355xSoftmaxWorkload::Execute() const
 Mi355xAdditionWorkload::Mi355xAdditionWorkload(const ElementwiseBinaryQueueDescriptor& descriptor, const WorkloadInfo& info)
     : Mi355xBaseWorkload<ElementwiseBinaryQueueDescriptor>(descriptor, info), m_Info(info)
 {
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xAdditionWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
     if (m_Data.m_Parameters.m_Operation != BinaryOperation::Add) throw InvalidArgumentException("Mi355xAdditionWorkload: Add only");
     Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
 }
 
 void Mi355xAdditionWorkload::Execute() const
 {
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xAdditionWorkload_Execute");
     const Mi355xFusedActivation act = Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
     const mi355x_quant q0 = mi355x::ToQuant(m_Info.m_InputTensorInfos[0]);
     const mi355x_quant q1 = mi355x::ToQuant(m_Info.m_InputTensorInfos[1]);
@@ -339,6 +382,7 @@ Mi355xReshapeWorkload::Mi355xReshapeWorkload(const ReshapeQueueDescriptor& descr
 
 void Mi355xReshapeWorkload::Execute() const
 {
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xReshapeWorkload_Execute");
     const size_t bytes = m_Info.m_InputTensorInfos[0].GetNumBytes();
     if (!bytes) return;
     mi355x::Check(mi355x_memcpy_d2d(Out(m_Data.m_Outputs[0]), In(m_Data.m_Inputs[0]), bytes, mi355x::Stream()), "mi355x_memcpy_d2d");
@@ -352,6 +396,7 @@ Mi355xConstantWorkload::Mi355xConstantWorkload(const ConstantQueueDescriptor& de
 
 void Mi355xConstantWorkload::Execute() const
 {
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xConstantWorkload_Execute");
     const void* src = m_Data.m_LayerOutput->Map(true);
     if (!src) throw NullPointerException("Mi355xConstantWorkload: layer has no data");
     m_Data.m_Outputs[0]->CopyInFrom(src);

@@ -15,7 +15,12 @@
 #include "../mi355x/Mi355xTensorHandle.hpp"
 #include "../mi355x/Mi355xWorkloadFactory.hpp"
 
+#include "../mi355x/Mi355xTimer.hpp"
+#include <Profiling.hpp>
+
 #include <chrono>
+#include <sstream>
+#include <thread>
 #include <cstring>
 #include <backendsCommon/TensorHandleFactoryRegistry.hpp>
 #include <armnn/backends/WorkloadData.hpp>
@@ -472,6 +477,63 @@ TEST_CASE("optimize: a Pad of height and width moves into the layer behind it wh
     }
 }
 
+TEST_CASE("profiling: events nest as their scopes do, exist only while the profiler is on, and print as JSON", "cpu")
+{
+    IProfiler profiler;
+    ProfilerManager::GetInstance().RegisterProfiler(&profiler);
+    {
+        // off: nothing is recorded, and the device timer handed to the macro is never started (no device is needed)
+        ARMNN_SCOPED_PROFILING_EVENT_WITH_INSTRUMENTS(kMi355x, EmptyOptional(), std::string("ignored"), Mi355xTimer(), WallClockTimer())
+    }
+    CHECK(profiler.GetEvents().empty());
+    profiler.EnableProfiling(true);
+    CHECK(profiler.IsProfilingEnabled());
+    {
+        ARMNN_SCOPED_PROFILING_EVENT(BackendId(), "outer");
+        {
+            ARMNN_SCOPED_PROFILING_EVENT_GUID(kMi355x, "inner \"quoted\"", arm::pipe::ProfilingGuid(42));
+            std::this_thread::sleep_for(std::chrono::milliseconds(2));
+        }
+        ARMNN_SCOPED_PROFILING_EVENT(kMi355x, "second inner");
+    }
+    WorkloadInfo info;
+    info.m_Name = "conv";
+    info.m_InputTensorInfos = {ActInfo({1, 8, 8, 16}, DataType::QAsymmS8, 0.05f, -3)};
+    info.m_ConvolutionMethod = Optional<std::string>("igemm 64x64");
+    Convolution2dDescriptor cd;
+    cd.m_PadLeft = 3;
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Conv_Construct", cd, info, arm::pipe::ProfilingGuid(7))
+    ProfilerManager::GetInstance().RegisterProfiler(nullptr);
+
+    const auto& events = profiler.GetEvents();
+    REQUIRE(events.size() == 3);
+    CHECK(events[0]->GetName() == "outer");
+    CHECK(events[0]->GetParentEvent() == nullptr);
+    CHECK(events[1]->GetParentEvent() == events[0].get());
+    CHECK(events[2]->GetParentEvent() == events[0].get());
+    const std::vector<Measurement> inner = events[1]->GetMeasurements();
+    REQUIRE(inner.size() == 1);
+    CHECK(inner[0].m_Unit == Measurement::TIME_US);
+    CHECK(inner[0].m_Value >= 2000.0);
+    CHECK(events[0]->GetMeasurements()[0].m_Value >= inner[0].m_Value);
+
+    std::ostringstream table, json;
+    profiler.AnalyzeEventsAndWriteResults(table);
+    CHECK(table.str().find("  second inner") != std::string::npos);
+    profiler.Print(json);
+    const std::string j = json.str();
+    CHECK(j.find("\"ArmNN\"") != std::string::npos);
+    CHECK(j.find("\"inner \\\"quoted\\\"_#1\"") != std::string::npos);
+    CHECK(j.find("\"GUID\": 42") != std::string::npos);
+    CHECK(j.find("\"ConvolutionMethod\": \"igemm 64x64\"") != std::string::npos);
+    CHECK(j.find("pad (l,r,t,b) 3,0,0,0") != std::string::npos);
+    CHECK(j.find("\"outer_#0\"") < j.find("\"second inner_#2\""));
+    size_t open = 0, close = 0;
+    for (char c : j) { open += c == '{'; close += c == '}'; }
+    CHECK(open == close);
+    CHECK(profiler.GetEvents().empty());       // printing starts a new recording
+}
+
 TEST_CASE("optimize: unsupported layers fall back along the preference list, with copies between backends", "cpu")
 {
     testhost::Register();
@@ -867,6 +929,63 @@ TEST_CASE("runtime: a small MobileNet gives the bytes of the same C-ABI calls ma
             CHECK(std::abs(sum - 256) <= 10);
         }
     }
+}
+
+TEST_CASE("profiling: every workload of a profiled network reports its device time, and its kernel in the details", "gpu")
+{
+    MiniMobileNet m(4, DataType::QAsymmS8);
+    IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+    INetworkPtr net = m.Build();
+    IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, rt->GetDeviceSpec());
+    NetworkId id = -1;
+    std::string err;
+    REQUIRE(rt->LoadNetwork(id, std::move(opt), err, INetworkProperties(false, MemorySource::Undefined, MemorySource::Undefined, true)) == Status::Success);
+    const std::shared_ptr<IProfiler> profiler = rt->GetProfiler(id);
+    REQUIRE(profiler != nullptr);
+    CHECK(profiler->IsProfilingEnabled());
+    const std::vector<uint8_t> input = RandomActivations(m.in, 5);
+    std::vector<uint8_t> out(m.probs.GetNumBytes());
+    TensorInfo constIn = m.in;
+    constIn.SetConstant(true);
+    auto run = [&] {
+        InputTensors ins{{0, ConstTensor(constIn, input.data())}};
+        OutputTensors outs{{0, Tensor(m.probs, out.data())}};
+        REQUIRE(rt->EnqueueWorkload(id, ins, outs) == Status::Success);
+    };
+    run();                                     // builds the plans
+    { std::ostringstream drop; profiler->Print(drop); }
+    run();
+    const std::vector<uint8_t> profiled = out;
+
+    size_t workloads = 0;
+    double deviceUs = 0.0, executeWallUs = 0.0;
+    for (const auto& e : profiler->GetEvents())
+    {
+        if (e->GetName() == "Execute") executeWallUs = e->GetMeasurements().at(0).m_Value;
+        if (e->GetBackendId() != kMi355x) continue;
+        ++workloads;
+        CHECK(e->GetParentEvent() != nullptr && e->GetParentEvent()->GetName() == "Execute");
+        bool hasDevice = false;
+        for (const Measurement& meas : e->GetMeasurements())
+            if (meas.m_Name == "Device time") { hasDevice = true; deviceUs += meas.m_Value; CHECK(meas.m_Value > 0.0); CHECK(meas.m_Value < 5000.0); }
+        CHECK(hasDevice);
+    }
+    CHECK(workloads == 8);                     // stem, 2 x (depthwise, pointwise), pool, fc, softmax; the activations are fused
+    std::ostringstream json;
+    profiler->Print(json);
+    const std::string j = json.str();
+    std::printf("    %zu device workloads, %.1f us on the device, Execute %.1f us on the host\n", workloads, deviceUs, executeWallUs);
+    CHECK(j.find("Mi355xConvolution2dWorkload_Execute") != std::string::npos);
+    CHECK(j.find("Mi355xDepthwiseConvolution2dWorkload_Plan") != std::string::npos);
+    CHECK(j.find("\"ConvolutionMethod\": \"") != std::string::npos);
+    CHECK(j.find("Device time_#0") != std::string::npos);
+
+    // the same bytes with the profiler off, and then no events
+    profiler->EnableProfiling(false);
+    run();
+    CHECK(out == profiled);
+    CHECK(profiler->GetEvents().empty());
+    rt->UnloadNetwork(id);
 }
 
 TEST_CASE("runtime: MobileNetV1-224 batch 64 through EnqueueWorkload equals the C-ABI calls; host-to-host images/s printed", "gpu")
