@@ -6,6 +6,7 @@
 #include "Mi355xWorkloadFactory.hpp"
 
 #include <Layer.hpp>
+#include <armnn/BackendOptions.hpp>
 #include <armnn/BackendRegistry.hpp>
 #include <armnn/backends/IBackendContext.hpp>
 #include <backendsCommon/TensorHandleFactoryRegistry.hpp>
@@ -23,7 +24,15 @@ namespace
 class Mi355xBackendContext : public IBackendContext
 {
 public:
-    explicit Mi355xBackendContext(const IRuntime::CreationOptions& options) : IBackendContext(options) { mi355x::EnsureDevice(); }
+    explicit Mi355xBackendContext(const IRuntime::CreationOptions& options) : IBackendContext(options)
+    {
+        mi355x::EnsureDevice();
+        // BackendOptions("Mi355x", {{"Lanes", n}}): into how many slices a batch is split (1 = one stream, addresses shared)
+        ParseOptions(options.m_BackendOptions, Mi355xBackendId(), [](const std::string& name, const BackendOptions::Var& value) {
+            if (name == "Lanes" && value.IsInt() && value.AsInt() >= 1 && value.AsInt() <= static_cast<int>(mi355x::kMaxLanes))
+                mi355x::SetLanes(static_cast<unsigned int>(value.AsInt()));
+        });
+    }
     bool BeforeLoadNetwork(NetworkId) override { return true; }
     bool AfterLoadNetwork(NetworkId) override { return true; }
     bool BeforeUnloadNetwork(NetworkId) override { mi355x::Synchronize(); return true; }
@@ -107,7 +116,7 @@ const BackendId& Mi355xBackend::GetIdStatic()
 
 IBackendInternal::IMemoryManagerUniquePtr Mi355xBackend::CreateMemoryManager() const
 {
-    return std::make_unique<Mi355xMemoryManager>();
+    return std::make_unique<Mi355xMemoryManager>(mi355x::Lanes() == 1);
 }
 
 IBackendInternal::IWorkloadFactoryPtr Mi355xBackend::CreateWorkloadFactory(const IBackendInternal::IMemoryManagerSharedPtr& memoryManager) const
@@ -120,7 +129,7 @@ IBackendInternal::IWorkloadFactoryPtr Mi355xBackend::CreateWorkloadFactory(Tenso
     // handles made by the registered tensor handle factory and by the workload factory share one arena
     if (auto* existing = dynamic_cast<Mi355xTensorHandleFactory*>(registry.GetFactory(Mi355xTensorHandleFactory::GetIdStatic())))
         return std::make_unique<Mi355xWorkloadFactory>(existing->GetMemoryManager());
-    auto memoryManager = std::make_shared<Mi355xMemoryManager>();
+    auto memoryManager = std::make_shared<Mi355xMemoryManager>(mi355x::Lanes() == 1);
     registry.RegisterMemoryManager(memoryManager);
     registry.RegisterFactory(std::make_unique<Mi355xTensorHandleFactory>(memoryManager));
     return std::make_unique<Mi355xWorkloadFactory>(memoryManager);
@@ -145,7 +154,7 @@ std::vector<ITensorHandleFactory::FactoryId> Mi355xBackend::GetHandleFactoryPref
 void Mi355xBackend::RegisterTensorHandleFactories(TensorHandleFactoryRegistry& registry)
 {
     if (registry.GetFactory(Mi355xTensorHandleFactory::GetIdStatic()) != nullptr) return;
-    auto memoryManager = std::make_shared<Mi355xMemoryManager>();
+    auto memoryManager = std::make_shared<Mi355xMemoryManager>(mi355x::Lanes() == 1);
     registry.RegisterMemoryManager(memoryManager);
     registry.RegisterFactory(std::make_unique<Mi355xTensorHandleFactory>(memoryManager));
 }

@@ -1,5 +1,7 @@
 #include "Mi355xDevice.hpp"
 
+#include <atomic>
+#include <cstdlib>
 #include <mutex>
 
 namespace armnn
@@ -9,9 +11,26 @@ namespace mi355x
 namespace
 {
 std::once_flag g_Once;
-mi355x_stream_t g_Stream = nullptr;
+mi355x_stream_t g_Streams[kMaxLanes] = {nullptr, nullptr, nullptr, nullptr};
+std::atomic<unsigned int> g_Lanes{0};          // 0: not decided yet
+std::atomic<int> g_SharingArenas{0};
 bool g_Ready = false;
 std::string g_Why;
+
+// per thread: whether its lanes are running apart, and the events it orders them with
+struct LaneState
+{
+    bool forked = false;
+    unsigned int count = 1;         // lanes running since the last Fork()
+    mi355x_event_t fork = nullptr;
+    mi355x_event_t lane[kMaxLanes] = {nullptr, nullptr, nullptr, nullptr};
+    mi355x_event_t Event(mi355x_event_t& e)
+    {
+        if (!e) Check(mi355x_event_create(&e), "mi355x_event_create");
+        return e;
+    }
+};
+thread_local LaneState t_Lanes;
 } // namespace
 
 int DeviceCount()
@@ -26,7 +45,8 @@ void EnsureDevice()
     std::call_once(g_Once, [] {
         if (DeviceCount() < 1) { g_Why = "no MI355X device is visible to this process"; return; }
         if (mi355x_init(0) != 0) { g_Why = std::string("device initialisation failed: ") + mi355x_last_error(); return; }
-        if (mi355x_stream_create(&g_Stream) != 0) { g_Why = std::string("stream creation failed: ") + mi355x_last_error(); return; }
+        for (mi355x_stream_t& s : g_Streams)
+            if (mi355x_stream_create(&s) != 0) { g_Why = std::string("stream creation failed: ") + mi355x_last_error(); return; }
         g_Ready = true;
     });
     if (!g_Ready) throw BackendUnavailableException("Mi355x backend unavailable: " + g_Why);
@@ -35,7 +55,98 @@ void EnsureDevice()
 mi355x_stream_t Stream()
 {
     EnsureDevice();
-    return g_Stream;
+    Join();
+    return g_Streams[0];
+}
+
+unsigned int Lanes()
+{
+    unsigned int n = g_Lanes.load();
+    if (n == 0)
+    {
+        n = 2;
+        if (const char* env = std::getenv("MI355X_LANES"))
+        {
+            const int v = std::atoi(env);
+            if (v >= 1 && v <= static_cast<int>(kMaxLanes)) n = static_cast<unsigned int>(v);
+        }
+        g_Lanes.store(n);
+    }
+    return n;
+}
+
+void SetLanes(unsigned int lanes)
+{
+    if (lanes < 1 || lanes > kMaxLanes) throw InvalidArgumentException("Mi355x: the number of lanes must be 1.." + std::to_string(kMaxLanes));
+    if (lanes > 1 && g_SharingArenas.load() > 0)
+        throw InvalidArgumentException("Mi355x: lanes cannot be turned on while a network loaded for one stream is alive");
+    if (g_Ready) Join();
+    g_Lanes.store(lanes);
+}
+
+void CountAddressSharingArena(int delta) { g_SharingArenas.fetch_add(delta); }
+
+unsigned int LanesFor(unsigned int batch)
+{
+    const unsigned int n = Lanes();
+    return (n > 1 && batch % n == 0 && batch / n >= kMinLaneBatch) ? n : 1u;
+}
+
+mi355x_stream_t LaneStream(unsigned int lane)
+{
+    EnsureDevice();
+    if (lane >= kMaxLanes) throw InvalidArgumentException("Mi355x: no such lane");
+    return g_Streams[lane];
+}
+
+void Fork()
+{
+    EnsureDevice();
+    LaneState& st = t_Lanes;
+    if (st.forked) return;
+    const unsigned int n = Lanes();
+    if (n > 1)
+    {
+        Check(mi355x_event_record(st.Event(st.fork), g_Streams[0]), "mi355x_event_record");
+        for (unsigned int k = 1; k < n; ++k) Check(mi355x_stream_wait_event(g_Streams[k], st.fork), "mi355x_stream_wait_event");
+    }
+    st.forked = true;
+    st.count = n;
+}
+
+void Join()
+{
+    LaneState& st = t_Lanes;
+    if (!st.forked) return;
+    for (unsigned int k = 1; k < st.count; ++k)
+    {
+        Check(mi355x_event_record(st.Event(st.lane[k]), g_Streams[k]), "mi355x_event_record");
+        Check(mi355x_stream_wait_event(g_Streams[0], st.lane[k]), "mi355x_stream_wait_event");
+    }
+    st.forked = false;
+}
+
+void UploadInLanes(void* dstDevice, const void* srcHost, size_t bytes, unsigned int lanes)
+{
+    if (lanes <= 1 || bytes % lanes != 0)
+    {
+        Check(mi355x_memcpy_h2d_async(dstDevice, srcHost, bytes, Stream()), "mi355x_memcpy_h2d_async");
+        return;
+    }
+    Fork();
+    LaneState& st = t_Lanes;
+    const size_t part = bytes / lanes;
+    mi355x_stream_t queue = g_Streams[lanes - 1];
+    for (unsigned int k = 0; k < lanes; ++k)
+    {
+        Check(mi355x_memcpy_h2d_async(static_cast<unsigned char*>(dstDevice) + k * part, static_cast<const unsigned char*>(srcHost) + k * part, part, queue),
+              "mi355x_memcpy_h2d");
+        if (k + 1 < lanes)
+        {
+            Check(mi355x_event_record(st.Event(st.lane[k]), queue), "mi355x_event_record");
+            Check(mi355x_stream_wait_event(g_Streams[k], st.lane[k]), "mi355x_stream_wait_event");
+        }
+    }
 }
 
 void Synchronize() { Check(mi355x_stream_synchronize(Stream()), "mi355x_stream_synchronize"); }

@@ -17,9 +17,38 @@ namespace mi355x
 int DeviceCount();
 /// selects device 0 on first use; throws BackendUnavailableException when there is no device
 void EnsureDevice();
-/// the stream all workloads and tensor-handle copies are ordered on
+/// The stream workloads and tensor-handle copies are ordered on.  If the calling thread has lanes running (see below) they
+/// are joined first, so whatever is queued through this stream comes after everything queued before it.
 mi355x_stream_t Stream();
+/// joins the lanes and waits for the stream
 void Synchronize();
+
+/// Lanes.  Every image of a batch is computed independently, so a workload may run its batch as Lanes() contiguous
+/// slices, slice k on LaneStream(k): one slice's launches then fill the ramp-up, tail and launch gaps of the others, and
+/// the input of a later slice crosses the bus while an earlier one computes.  Lane 0 is the stream of Stream().
+///   Fork()  the lanes continue, independently, after everything queued so far (no-op while forked)
+///   Join()  stream 0 continues after everything queued on every lane (no-op while joined)
+/// The forked/joined state belongs to the calling thread; a thread leaves EnqueueWorkload joined because reading a
+/// network output goes through Stream().
+constexpr unsigned int kMaxLanes = 4;
+unsigned int Lanes();
+/// 1 .. kMaxLanes; the initial value is 2, or what the environment variable MI355X_LANES says.  Raising it above 1 throws
+/// while a network loaded for one stream is alive: its tensors share addresses, which lanes must not.
+void SetLanes(unsigned int lanes);
+/// memory managers that let tensors share addresses announce themselves here (+1 when created, -1 when destroyed)
+void CountAddressSharingArena(int delta);
+/// the smallest slice worth a lane of its own: a batch splits only into slices of at least this many images
+constexpr unsigned int kMinLaneBatch = 8;
+/// number of slices a workload over `batch` images should run as: Lanes() if that divides the batch into slices of at
+/// least kMinLaneBatch, else 1
+unsigned int LanesFor(unsigned int batch);
+mi355x_stream_t LaneStream(unsigned int lane);
+void Fork();
+void Join();
+/// Host-to-device transfer from pinned memory (the staging copy of a tensor handle or an adopted buffer), queued without
+/// waiting for it: `bytes` in `lanes` equal parts queued back to back on one copy queue, so part k arrives
+/// at k+1 times a part's transfer time; lane k continues as soon as its part is there.  Leaves the lanes forked.
+void UploadInLanes(void* dstDevice, const void* srcHost, size_t bytes, unsigned int lanes);
 
 /// throws RuntimeException carrying mi355x_last_error() when `status` is non-zero
 void Check(int status, const char* what);

@@ -3,8 +3,14 @@
 
 namespace armnn
 {
+Mi355xMemoryManager::Mi355xMemoryManager(bool shareAddresses) : m_Share(shareAddresses)
+{
+    if (m_Share) mi355x::CountAddressSharingArena(+1);
+}
+
 Mi355xMemoryManager::~Mi355xMemoryManager()
 {
+    if (m_Share) mi355x::CountAddressSharingArena(-1);
     if (m_Arena) mi355x_free(m_Arena);
 }
 
@@ -38,6 +44,7 @@ size_t Mi355xMemoryManager::Reserve(size_t bytes)
 
 void Mi355xMemoryManager::Retire(size_t offset, size_t bytes)
 {
+    if (!m_Share) return;
     size_t len = Granules(bytes ? bytes : 1);
     auto next = m_Free.lower_bound(offset);
     if (next != m_Free.begin())

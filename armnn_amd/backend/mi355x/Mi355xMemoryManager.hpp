@@ -4,7 +4,8 @@
 // (ITensorHandle::Allocate, which the graph calls after the last consumer), so tensors whose lifetimes do not overlap
 // share addresses -- the same protocol RefMemoryManager implements with host pools
 // (src/backends/reference/RefMemoryManager.cpp:20-101).  Acquire() allocates the arena at its high-water size,
-// Release() returns it.  Kernels of one network run in order on one stream, which is what makes address reuse safe.
+// Release() returns it.  Address reuse is safe when the kernels of a network run in order on one stream; the backend turns
+// it off when networks run in lanes.
 #pragma once
 #include <armnn/backends/IMemoryManager.hpp>
 
@@ -16,7 +17,9 @@ namespace armnn
 class Mi355xMemoryManager : public IMemoryManager
 {
 public:
-    Mi355xMemoryManager() = default;
+    /// shareAddresses = false gives every tensor a range of its own.  That is what networks running in lanes need: the
+    /// lanes are at different layers at the same moment, so a tensor retired for one of them may still be read by another.
+    explicit Mi355xMemoryManager(bool shareAddresses = true);
     ~Mi355xMemoryManager() override;
 
     /// start of a lifetime: returns the offset of a free range of `bytes` (first fit, 256-byte granules)
@@ -34,6 +37,7 @@ public:
 
 private:
     static size_t Granules(size_t bytes) { return (bytes + 255) / 256 * 256; }
+    const bool m_Share;
     std::map<size_t, size_t> m_Free;     // offset -> length of free ranges below the high-water mark
     size_t m_HighWater = 0;
     size_t m_ReservedTotal = 0;

@@ -85,8 +85,16 @@ const void* Mi355xTensorHandle::GetDevicePointerForRead() const
     // adopted buffer, not written by a workload since the caller last saw it: it is an input, and whatever the caller
     // has put there is what this inference reads
     if (m_ImportedDevice && !m_ImportedIsDeviceMemory && !m_DeviceNewer && m_Info.GetNumBytes())
-        mi355x::Check(mi355x_memcpy_h2d(dev, m_ImportedDevice, m_Info.GetNumBytes(), mi355x::Stream()), "mi355x_memcpy_h2d (adopted buffer)");
+        mi355x::UploadInLanes(dev, m_ImportedDevice, m_Info.GetNumBytes(), UploadLanes());
     return dev;
+}
+
+// A batch of images large enough to be worth it goes up slice by slice, so that the first lane starts computing while
+// the later slices are still on the bus.
+unsigned int Mi355xTensorHandle::UploadLanes() const
+{
+    if (m_Info.IsConstant() || m_Info.GetNumDimensions() < 2 || m_Info.GetNumBytes() < (1u << 20)) return 1;
+    return mi355x::LanesFor(m_Info.GetShape()[0]);
 }
 
 void* Mi355xTensorHandle::GetDevicePointer() const
@@ -143,7 +151,7 @@ void Mi355xTensorHandle::Unmap() const
     const size_t bytes = m_Info.GetNumBytes();
     if (!bytes) return;
     // the pinned copy stays alive with the handle, so the upload may complete asynchronously in stream order
-    mi355x::Check(mi355x_memcpy_h2d(GetDevicePointer(), m_Staging, bytes, mi355x::Stream()), "mi355x_memcpy_h2d");
+    mi355x::UploadInLanes(GetDevicePointer(), m_Staging, bytes, UploadLanes());
     m_UploadInFlight = true;
 }
 
@@ -161,7 +169,7 @@ void Mi355xTensorHandle::CopyInFrom(const void* memory)
     if (!m_Staging) mi355x::Check(mi355x_host_alloc(&m_Staging, bytes ? bytes : 1), "mi355x_host_alloc");
     if (m_UploadInFlight) mi355x::Synchronize();
     std::memcpy(m_Staging, memory, bytes);
-    if (bytes) mi355x::Check(mi355x_memcpy_h2d(GetDevicePointer(), m_Staging, bytes, mi355x::Stream()), "mi355x_memcpy_h2d");
+    if (bytes) mi355x::UploadInLanes(GetDevicePointer(), m_Staging, bytes, UploadLanes());
     m_UploadInFlight = bytes != 0;
     m_DeviceNewer = false;
 }

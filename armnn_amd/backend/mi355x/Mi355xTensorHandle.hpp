@@ -56,6 +56,7 @@ public:
     bool IsManaged() const { return m_Managed; }
 
 private:
+    unsigned int UploadLanes() const;
     TensorInfo m_Info;
     std::shared_ptr<Mi355xMemoryManager> m_MemoryManager;
     const bool m_Managed;

@@ -30,6 +30,34 @@ void* Out(ITensorHandle* h)
     return d.GetDevicePointer();
 }
 
+// One slice of a batch and the stream it runs on.
+struct Lane
+{
+    mi355x_stream_t stream;
+    unsigned int index, count;
+    /// this lane's part of a dense tensor whose outermost dimension is the batch
+    const void* Of(const void* base, const TensorInfo& info) const { return static_cast<const unsigned char*>(base) + info.GetNumBytes() / count * index; }
+    void* Of(void* base, const TensorInfo& info) const { return static_cast<unsigned char*>(base) + info.GetNumBytes() / count * index; }
+};
+
+// Calls `launch` once per lane when `batch` splits into lanes, else once for the whole batch on the joined stream.
+// Operand addresses are taken before this (reading an adopted input may queue its transfer, lane by lane).
+template <typename Launch>
+void ForEachLane(unsigned int batch, Launch&& launch)
+{
+    const unsigned int lanes = mi355x::LanesFor(batch);
+    if (lanes == 1)
+    {
+        launch(Lane{mi355x::Stream(), 0u, 1u});
+        return;
+    }
+    mi355x::Fork();
+    for (unsigned int k = 0; k < lanes; ++k) launch(Lane{mi355x::LaneStream(k), k, lanes});
+}
+
+// batch of a tensor that has one: the outermost of at least two dimensions
+unsigned int BatchOf(const TensorInfo& info) { return info.GetNumDimensions() >= 2 ? info.GetShape()[0] : 1u; }
+
 // the kernel a plan resolved to, for the profiler's details record
 std::string Describe(mi355x_conv2d_t plan)
 {
@@ -136,8 +164,14 @@ void Mi355xConvolution2dWorkload::Execute() const
     ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xConvolution2dWorkload_Execute");
     std::call_once(m_Once, [this] { BuildPlan(); });
     if (!m_Plan) throw RuntimeException("Mi355xConvolution2dWorkload: no device plan (its creation failed earlier)");
-    const uint32_t batch = m_Info.m_InputTensorInfos[0].GetShape()[0];
-    mi355x::Check(mi355x_conv2d_run(m_Plan, batch, In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()), "mi355x_conv2d_run");
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const uint32_t batch = in.GetShape()[0];
+    const void* x = In(m_Data.m_Inputs[0]);
+    void* y = Out(m_Data.m_Outputs[0]);
+    ForEachLane(batch, [&](const Lane& l) {
+        mi355x::Check(mi355x_conv2d_run(m_Plan, batch / l.count, l.Of(x, in), l.Of(y, out), l.stream), "mi355x_conv2d_run");
+    });
 }
 
 std::string Mi355xConvolution2dWorkload::GetKernelDescription() const
@@ -203,8 +237,14 @@ void Mi355xDepthwiseConvolution2dWorkload::Execute() const
     ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xDepthwiseConvolution2dWorkload_Execute");
     std::call_once(m_Once, [this] { BuildPlan(); });
     if (!m_Plan) throw RuntimeException("Mi355xDepthwiseConvolution2dWorkload: no device plan (its creation failed earlier)");
-    const uint32_t batch = m_Info.m_InputTensorInfos[0].GetShape()[0];
-    mi355x::Check(mi355x_conv2d_run(m_Plan, batch, In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()), "mi355x_conv2d_run(depthwise)");
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const uint32_t batch = in.GetShape()[0];
+    const void* x = In(m_Data.m_Inputs[0]);
+    void* y = Out(m_Data.m_Outputs[0]);
+    ForEachLane(batch, [&](const Lane& l) {
+        mi355x::Check(mi355x_conv2d_run(m_Plan, batch / l.count, l.Of(x, in), l.Of(y, out), l.stream), "mi355x_conv2d_run(depthwise)");
+    });
 }
 
 // ---- FullyConnected --------------------------------------------------------------------------------------------------
@@ -256,8 +296,14 @@ void Mi355xFullyConnectedWorkload::Execute() const
     ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xFullyConnectedWorkload_Execute");
     std::call_once(m_Once, [this] { BuildPlan(); });
     if (!m_Plan) throw RuntimeException("Mi355xFullyConnectedWorkload: no device plan (its creation failed earlier)");
-    const uint32_t batch = m_Info.m_InputTensorInfos[0].GetShape()[0];
-    mi355x::Check(mi355x_fc_run(m_Plan, batch, In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()), "mi355x_fc_run");
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const uint32_t batch = in.GetShape()[0];
+    const void* x = In(m_Data.m_Inputs[0]);
+    void* y = Out(m_Data.m_Outputs[0]);
+    ForEachLane(batch, [&](const Lane& l) {
+        mi355x::Check(mi355x_fc_run(m_Plan, batch / l.count, l.Of(x, in), l.Of(y, out), l.stream), "mi355x_fc_run");
+    });
 }
 
 // ---- Activation ------------------------------------------------------------------------------------------------------
@@ -274,9 +320,14 @@ void Mi355xActivationWorkload::Execute() const
     const Mi355xFusedActivation act = Mi355xFusedActivation::From(&m_Data.m_Parameters);
     const mi355x_quant qi = mi355x::ToQuant(m_Info.m_InputTensorInfos[0]);
     const mi355x_quant qo = mi355x::ToQuant(m_Info.m_OutputTensorInfos[0]);
-    mi355x::Check(mi355x_activation_run(m_Info.m_InputTensorInfos[0].GetNumElements(), &qi, &qo, act.function, act.a, act.b,
-                                        In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()),
-                  "mi355x_activation_run");
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const void* x = In(m_Data.m_Inputs[0]);
+    void* y = Out(m_Data.m_Outputs[0]);
+    ForEachLane(BatchOf(in), [&](const Lane& l) {
+        mi355x::Check(mi355x_activation_run(in.GetNumElements() / l.count, &qi, &qo, act.function, act.a, act.b, l.Of(x, in), l.Of(y, out), l.stream),
+                      "mi355x_activation_run");
+    });
 }
 
 // ---- Pooling2d -------------------------------------------------------------------------------------------------------
@@ -302,7 +353,11 @@ void Mi355xPooling2dWorkload::Execute() const
     d.padding_method = p.m_PaddingMethod == PaddingMethod::IgnoreValue ? 0 : 1;
     d.input = mi355x::ToQuant(in);
     d.output = mi355x::ToQuant(out);
-    mi355x::Check(mi355x_pool2d_run(&d, in.GetShape()[0], In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()), "mi355x_pool2d_run");
+    const void* x = In(m_Data.m_Inputs[0]);
+    void* y = Out(m_Data.m_Outputs[0]);
+    ForEachLane(in.GetShape()[0], [&](const Lane& l) {
+        mi355x::Check(mi355x_pool2d_run(&d, in.GetShape()[0] / l.count, l.Of(x, in), l.Of(y, out), l.stream), "mi355x_pool2d_run");
+    });
 }
 
 // ---- Pad -------------------------------------------------------------------------------------------------------------
@@ -330,7 +385,16 @@ void Mi355xPadWorkload::Execute() const
     d.pad_value = p.m_PadValue;
     d.input = mi355x::ToQuant(in);
     d.output = mi355x::ToQuant(m_Info.m_OutputTensorInfos[0]);
-    mi355x::Check(mi355x_pad_run(&d, In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()), "mi355x_pad_run");
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const void* x = In(m_Data.m_Inputs[0]);
+    void* y = Out(m_Data.m_Outputs[0]);
+    // the batch splits only if nothing is added in front of or behind it
+    const bool batchPadded = p.m_PadList[0].first != 0 || p.m_PadList[0].second != 0;
+    ForEachLane(batchPadded ? 1u : BatchOf(in), [&](const Lane& l) {
+        mi355x_pad_desc slice = d;
+        slice.in_shape[0] = d.in_shape[0] / l.count;
+        mi355x::Check(mi355x_pad_run(&slice, l.Of(x, in), l.Of(y, out), l.stream), "mi355x_pad_run");
+    });
 }
 
 // ---- Softmax ---------------------------------------------------------------------------------------------------------
@@ -349,8 +413,12 @@ void Mi355xSoftmaxWorkload::Execute() const
     const uint32_t rows = cols ? in.GetNumElements() / cols : 0;
     const mi355x_quant qi = mi355x::ToQuant(in);
     const mi355x_quant qo = mi355x::ToQuant(m_Info.m_OutputTensorInfos[0]);
-    mi355x::Check(mi355x_softmax_run(rows, cols, m_Data.m_Parameters.m_Beta, &qi, &qo, In(m_Data.m_Inputs[0]), Out(m_Data.m_Outputs[0]), mi355x::Stream()),
-                  "mi355x_softmax_run");
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const void* x = In(m_Data.m_Inputs[0]);
+    void* y = Out(m_Data.m_Outputs[0]);
+    ForEachLane(BatchOf(in), [&](const Lane& l) {
+        mi355x::Check(mi355x_softmax_run(rows / l.count, cols, m_Data.m_Parameters.m_Beta, &qi, &qo, l.Of(x, in), l.Of(y, out), l.stream), "mi355x_softmax_run");
+    });
 }
 
 // ---- Add -------------------------------------------------------------------------------------------------------------
@@ -369,9 +437,15 @@ void Mi355xAdditionWorkload::Execute() const
     const mi355x_quant q0 = mi355x::ToQuant(m_Info.m_InputTensorInfos[0]);
     const mi355x_quant q1 = mi355x::ToQuant(m_Info.m_InputTensorInfos[1]);
     const mi355x_quant qo = mi355x::ToQuant(m_Info.m_OutputTensorInfos[0]);
-    mi355x::Check(mi355x_add_run(m_Info.m_OutputTensorInfos[0].GetNumElements(), &q0, &q1, &qo, act.function, act.a, act.b,
-                                 In(m_Data.m_Inputs[0]), In(m_Data.m_Inputs[1]), Out(m_Data.m_Outputs[0]), mi355x::Stream()),
-                  "mi355x_add_run");
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const void* x0 = In(m_Data.m_Inputs[0]);
+    const void* x1 = In(m_Data.m_Inputs[1]);
+    void* y = Out(m_Data.m_Outputs[0]);
+    ForEachLane(BatchOf(out), [&](const Lane& l) {
+        mi355x::Check(mi355x_add_run(out.GetNumElements() / l.count, &q0, &q1, &qo, act.function, act.a, act.b, l.Of(x0, m_Info.m_InputTensorInfos[0]),
+                                     l.Of(x1, m_Info.m_InputTensorInfos[1]), l.Of(y, out), l.stream),
+                      "mi355x_add_run");
+    });
 }
 
 // ---- Reshape ---------------------------------------------------------------------------------------------------------
@@ -385,7 +459,15 @@ void Mi355xReshapeWorkload::Execute() const
     ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xReshapeWorkload_Execute");
     const size_t bytes = m_Info.m_InputTensorInfos[0].GetNumBytes();
     if (!bytes) return;
-    mi355x::Check(mi355x_memcpy_d2d(Out(m_Data.m_Outputs[0]), In(m_Data.m_Inputs[0]), bytes, mi355x::Stream()), "mi355x_memcpy_d2d");
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const void* x = In(m_Data.m_Inputs[0]);
+    void* y = Out(m_Data.m_Outputs[0]);
+    // a reshape that keeps the batch outermost moves each image's bytes within its own slice
+    const bool keepsBatch = BatchOf(in) == BatchOf(out);
+    ForEachLane(keepsBatch ? BatchOf(in) : 1u, [&](const Lane& l) {
+        mi355x::Check(mi355x_memcpy_d2d(l.Of(y, out), l.Of(x, in), bytes / l.count, l.stream), "mi355x_memcpy_d2d");
+    });
 }
 
 // ---- Constant --------------------------------------------------------------------------------------------------------

@@ -1141,35 +1141,83 @@ TEST_CASE("runtime: intermediate tensors share an arena smaller than their sum",
     INetworkPtr net = m.Build();
     FixedDeviceSpec spec{kMi355x};
     IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, spec);
-    // replay the runtime's handle protocol by hand against one backend instance
-    Mi355xBackend backend;
-    TensorHandleFactoryRegistry registry;
-    backend.RegisterTensorHandleFactories(registry);
-    auto factory = backend.CreateWorkloadFactory(registry);
-    auto* hf = dynamic_cast<Mi355xTensorHandleFactory*>(registry.GetFactory(Mi355xTensorHandleFactory::GetIdStatic()));
-    REQUIRE(hf != nullptr);
-    std::vector<std::unique_ptr<ITensorHandle>> handles;
-    size_t total = 0;
-    const std::vector<Layer*> order = opt->GetGraph().TopologicalSort();
-    ITensorHandle* previous = nullptr;
-    for (Layer* l : order)
+    // replay the runtime's handle protocol by hand against one backend instance; addresses are shared only where
+    // everything runs on one stream
+    const unsigned int lanesBefore = mi355x::Lanes();
+    mi355x::SetLanes(1);
     {
-        if (l->GetType() == LayerType::Constant || l->GetType() == LayerType::Input || l->GetNumOutputSlots() == 0) continue;
-        handles.push_back(hf->CreateTensorHandle(l->Out(0).GetTensorInfo(), true));
-        handles.back()->Manage();
-        total += l->Out(0).GetTensorInfo().GetNumBytes();
-        if (previous) previous->Allocate();      // a chain: the producer's input dies once the layer is placed
-        previous = handles.back().get();
+        Mi355xBackend backend;
+        TensorHandleFactoryRegistry registry;
+        backend.RegisterTensorHandleFactories(registry);
+        auto factory = backend.CreateWorkloadFactory(registry);
+        auto* hf = dynamic_cast<Mi355xTensorHandleFactory*>(registry.GetFactory(Mi355xTensorHandleFactory::GetIdStatic()));
+        REQUIRE(hf != nullptr);
+        std::vector<std::unique_ptr<ITensorHandle>> handles;
+        size_t total = 0;
+        const std::vector<Layer*> order = opt->GetGraph().TopologicalSort();
+        ITensorHandle* previous = nullptr;
+        for (Layer* l : order)
+        {
+            if (l->GetType() == LayerType::Constant || l->GetType() == LayerType::Input || l->GetNumOutputSlots() == 0) continue;
+            handles.push_back(hf->CreateTensorHandle(l->Out(0).GetTensorInfo(), true));
+            handles.back()->Manage();
+            total += l->Out(0).GetTensorInfo().GetNumBytes();
+            if (previous) previous->Allocate();      // a chain: the producer's input dies once the layer is placed
+            previous = handles.back().get();
+        }
+        if (previous) previous->Allocate();
+        const size_t arena = hf->GetMemoryManager()->ArenaBytes();
+        std::printf("    sum of intermediates %zu bytes, arena %zu bytes\n", total, arena);
+        CHECK(arena < total);
+        CHECK(arena >= 2 * 4 * 16 * 16 * 32u);      // the two largest neighbours must both fit
+        CHECK_NOTHROW(registry.AquireMemory());
+        CHECK(dynamic_cast<Mi355xTensorHandle*>(handles[0].get())->GetDevicePointer() != nullptr);
+        registry.ReleaseMemory();
+        (void)factory;
     }
-    if (previous) previous->Allocate();
-    const size_t arena = hf->GetMemoryManager()->ArenaBytes();
-    std::printf("    sum of intermediates %zu bytes, arena %zu bytes\n", total, arena);
-    CHECK(arena < total);
-    CHECK(arena >= 2 * 4 * 16 * 16 * 32u);      // the two largest neighbours must both fit
-    CHECK_NOTHROW(registry.AquireMemory());
-    CHECK(dynamic_cast<Mi355xTensorHandle*>(handles[0].get())->GetDevicePointer() != nullptr);
-    registry.ReleaseMemory();
-    (void)factory;
+    mi355x::SetLanes(lanesBefore);
+}
+
+TEST_CASE("runtime: a batch run as two or four slices on streams of their own gives the bytes of the unsplit run", "gpu")
+{
+    const unsigned int lanesBefore = mi355x::Lanes();
+    MiniMobileNet m(32, DataType::QAsymmS8);
+    const std::vector<uint8_t> input = RandomActivations(m.in, 123);
+    std::vector<std::vector<uint8_t>> results;
+    for (unsigned int lanes : {1u, 2u, 4u})
+    {
+        mi355x::SetLanes(lanes);
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        INetworkPtr net = m.Build();
+        results.push_back(RunOnRuntime(*rt, *net, {kMi355x}, m.in, input, m.probs, 3));
+    }
+    CHECK(results[0] == m.RunDirect(input));
+    CHECK(results[1] == results[0]);
+    CHECK(results[2] == results[0]);
+
+    // a padded batch, a batch too small to split and a layer on another backend in the middle all fall back to joined
+    // execution without the caller noticing
+    mi355x::SetLanes(2);
+    {
+        MiniMobileNet small(4, DataType::QAsymmS8);
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        INetworkPtr net = small.Build();
+        const std::vector<uint8_t> in4 = RandomActivations(small.in, 124);
+        CHECK(RunOnRuntime(*rt, *net, {kMi355x}, small.in, in4, small.probs, 2) == small.RunDirect(in4));
+    }
+    {
+        // Input -> Pad (batch 16 -> 18: not splittable) -> Pooling2d (batch 18: splits into 9 + 9) -> Output
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        const TensorInfo in = ActInfo({16, 12, 12, 16}, DataType::QAsymmS8, 0.05f, -3);
+        const PadList pads{{1, 1}, {0, 0}, {0, 0}, {0, 0}};
+        const TensorInfo padded = Padded(in, pads);
+        const TensorInfo pooled = ActInfo({18, 5, 5, 16}, DataType::QAsymmS8, 0.05f, -3);
+        INetworkPtr net = PadPoolNet(in, pads, 9.0f, Pool3x3s2(PoolingAlgorithm::Max), pooled);
+        const std::vector<uint8_t> x = RandomActivations(in, 125);
+        const std::vector<uint8_t> got = RunOnRuntime(*rt, *net, {kMi355x}, in, x, pooled, 2);
+        CHECK(got == OraclePool(padded, OraclePad(in, x, pads, 9.0f), Pool3x3s2(PoolingAlgorithm::Max), pooled));
+    }
+    mi355x::SetLanes(lanesBefore);
 }
 
 TEST_CASE("runtime: a layer the device lacks runs on the next backend and the copies preserve the data", "gpu")

@@ -76,4 +76,8 @@ struct Options
 };
 Options& GlobalOptions();
 
+// Copies plan constants to the device and returns when they are there.  Uses a stream of the library's own, never the
+// legacy default stream: that one may not be touched while any thread captures a graph.
+int UploadNow(void* dst_dev, const void* src_host, size_t bytes);
+
 } // namespace mi355x

@@ -70,8 +70,7 @@ int PreparePointwise(mi355x_conv2d_s* p);
 int Upload(void** dst, const void* src, size_t bytes)
 {
     MI355X_HIP(hipMalloc(dst, bytes));
-    MI355X_HIP(hipMemcpy(*dst, src, bytes, hipMemcpyHostToDevice));
-    return 0;
+    return UploadNow(*dst, src, bytes);
 }
 
 int ValidateQuant(const mi355x_quant& q, const char* what)

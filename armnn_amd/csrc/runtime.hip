@@ -22,6 +22,21 @@ int SetError(int code, const char* fmt, ...)
     return code;
 }
 
+int UploadNow(void* dst_dev, const void* src_host, size_t bytes)
+{
+    // one stream per calling thread, so concurrent plan creations do not wait for each other
+    struct Own
+    {
+        hipStream_t s = nullptr;
+        ~Own() { if (s) (void)hipStreamDestroy(s); }
+    };
+    thread_local Own own;
+    if (!own.s) MI355X_HIP(hipStreamCreateWithFlags(&own.s, hipStreamNonBlocking));
+    MI355X_HIP(hipMemcpyAsync(dst_dev, src_host, bytes, hipMemcpyHostToDevice, own.s));
+    MI355X_HIP(hipStreamSynchronize(own.s));
+    return 0;
+}
+
 Options& GlobalOptions()
 {
     static Options o;
@@ -249,6 +264,19 @@ static int Copy(void* dst, const void* src, size_t bytes, hipMemcpyKind kind, mi
 int mi355x_memcpy_h2d(void* d, const void* s, size_t n, mi355x_stream_t st) { return Copy(d, s, n, hipMemcpyHostToDevice, st); }
 int mi355x_memcpy_d2h(void* d, const void* s, size_t n, mi355x_stream_t st) { return Copy(d, s, n, hipMemcpyDeviceToHost, st); }
 int mi355x_memcpy_d2d(void* d, const void* s, size_t n, mi355x_stream_t st) { return Copy(d, s, n, hipMemcpyDeviceToDevice, st); }
+
+static int CopyAsync(void* dst, const void* src, const void* host, size_t bytes, hipMemcpyKind kind, mi355x_stream_t stream)
+{
+    if (bytes == 0) return 0;
+    if (!dst || !src) return SetError(MI355X_ERR_INVALID_ARGUMENT, "null pointer in copy of %zu bytes", bytes);
+    void* device_alias = nullptr;
+    int is_device = 0;
+    if (int rc = mi355x_host_device_pointer(host, &device_alias, &is_device)) return rc;
+    MI355X_HIP(hipMemcpyAsync(dst, src, bytes, kind, ToHip(stream)));
+    return 0;
+}
+int mi355x_memcpy_h2d_async(void* d, const void* s, size_t n, mi355x_stream_t st) { return CopyAsync(d, s, s, n, hipMemcpyHostToDevice, st); }
+int mi355x_memcpy_d2h_async(void* d, const void* s, size_t n, mi355x_stream_t st) { return CopyAsync(d, s, d, n, hipMemcpyDeviceToHost, st); }
 
 int mi355x_fill_u8(void* dst_dev, uint8_t value, size_t bytes, mi355x_stream_t stream)
 {

@@ -23,7 +23,7 @@ ACT_NONE, ACT_RELU, ACT_BOUNDED_RELU = 0, 1, 2
 EXPORTS = [
     "mi355x_last_error", "mi355x_abi_version", "mi355x_set_option", "mi355x_device_count", "mi355x_init", "mi355x_device_name",
     "mi355x_device_props", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc", "mi355x_host_device_pointer", "mi355x_host_free",
-    "mi355x_memcpy_h2d", "mi355x_memcpy_d2h", "mi355x_memcpy_d2d", "mi355x_fill_u8", "mi355x_stream_create",
+    "mi355x_memcpy_h2d", "mi355x_memcpy_d2h", "mi355x_memcpy_d2d", "mi355x_memcpy_h2d_async", "mi355x_memcpy_d2h_async", "mi355x_fill_u8", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_synchronize", "mi355x_device_synchronize", "mi355x_event_create",
     "mi355x_event_destroy", "mi355x_event_record", "mi355x_stream_wait_event", "mi355x_event_synchronize", "mi355x_event_elapsed_ms",
     "mi355x_graph_capture_begin", "mi355x_graph_capture_end", "mi355x_graph_launch", "mi355x_graph_destroy",
@@ -99,7 +99,8 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
             "mi355x_host_alloc": [C.POINTER(V), C.c_size_t], "mi355x_host_free": [V],
             "mi355x_host_device_pointer": [V, C.POINTER(V), C.POINTER(C.c_int)],
             "mi355x_memcpy_h2d": [V, V, C.c_size_t, V], "mi355x_memcpy_d2h": [V, V, C.c_size_t, V],
-            "mi355x_memcpy_d2d": [V, V, C.c_size_t, V], "mi355x_fill_u8": [V, C.c_uint8, C.c_size_t, V],
+            "mi355x_memcpy_d2d": [V, V, C.c_size_t, V], "mi355x_memcpy_h2d_async": [V, V, C.c_size_t, V],
+            "mi355x_memcpy_d2h_async": [V, V, C.c_size_t, V], "mi355x_fill_u8": [V, C.c_uint8, C.c_size_t, V],
             "mi355x_stream_create": [C.POINTER(V)], "mi355x_stream_destroy": [V], "mi355x_stream_synchronize": [V],
             "mi355x_event_create": [C.POINTER(V)], "mi355x_event_destroy": [V], "mi355x_event_record": [V, V],
             "mi355x_stream_wait_event": [V, V],

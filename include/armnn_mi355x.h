@@ -123,6 +123,13 @@ int  mi355x_host_device_pointer(const void* ptr, void** device_ptr, int* is_devi
 int  mi355x_host_free(void* ptr_host);
 int  mi355x_memcpy_h2d(void* dst_dev, const void* src_host, size_t bytes, mi355x_stream_t stream);
 int  mi355x_memcpy_d2h(void* dst_host, const void* src_dev, size_t bytes, mi355x_stream_t stream);
+/* The two above return when the transfer is complete (the host buffer may be pageable and is the caller's again at
+ * once).  The _async forms only queue the transfer in stream order and return; the host buffer must be memory the
+ * device reaches directly (mi355x_host_alloc / what mi355x_host_device_pointer accepts) and must stay untouched
+ * (h2d) or unread (d2h) until the stream has passed the transfer.  Pageable memory is refused with
+ * MI355X_ERR_UNSUPPORTED. */
+int  mi355x_memcpy_h2d_async(void* dst_dev, const void* src_pinned, size_t bytes, mi355x_stream_t stream);
+int  mi355x_memcpy_d2h_async(void* dst_pinned, const void* src_dev, size_t bytes, mi355x_stream_t stream);
 int  mi355x_memcpy_d2d(void* dst_dev, const void* src_dev, size_t bytes, mi355x_stream_t stream);
 int  mi355x_fill_u8(void* dst_dev, uint8_t value, size_t bytes, mi355x_stream_t stream);  /* fill kernel, graph-safe */
 
