@@ -166,3 +166,32 @@ def test_padding_inside_the_convolution_equals_a_pad_layer_in_front_of_it(cfg):
     params = dict(c.params, pad_top=0, pad_left=0)
     apart = shim.conv2d(padded, c.w, c.b, c.out_info, activation=c.act[0], act_a=c.act[1], act_b=c.act[2], **params)
     np.testing.assert_array_equal(folded.data, apart.data)
+
+
+def test_async_copies_need_memory_the_device_reaches_and_keep_stream_order():
+    """mi355x_memcpy_h2d_async / _d2h_async: pinned memory goes up and comes back unchanged behind a kernel queued in
+    between; pageable memory is refused, not copied some slower way."""
+    import ctypes as C
+    lib = shim.load_library()
+    dev = shim.Device()
+    stream = dev.stream()
+    n = 1 << 20
+    src, dst = C.c_void_p(), C.c_void_p()
+    shim._chk(lib.mi355x_host_alloc(C.byref(src), n))
+    shim._chk(lib.mi355x_host_alloc(C.byref(dst), n))
+    data = np.random.default_rng(5).integers(0, 256, n, dtype=np.uint8)
+    C.memmove(src.value, data.ctypes.data, n)
+    a, b = shim.DeviceBuffer(n), shim.DeviceBuffer(n)
+    shim._chk(lib.mi355x_memcpy_h2d_async(a.ptr, src, n, stream))
+    shim._chk(lib.mi355x_memcpy_d2d(b.ptr, a.ptr, n, stream))
+    shim._chk(lib.mi355x_memcpy_d2h_async(dst, b.ptr, n, stream))
+    dev.stream_sync(stream)
+    back = np.ctypeslib.as_array(C.cast(dst.value, C.POINTER(C.c_uint8)), shape=(n,)).copy()
+    np.testing.assert_array_equal(back, data)
+    pageable = np.zeros(4096, dtype=np.uint8)
+    assert lib.mi355x_memcpy_h2d_async(a.ptr, pageable.ctypes.data, 4096, stream) != 0
+    assert lib.mi355x_memcpy_d2h_async(pageable.ctypes.data, a.ptr, 4096, stream) != 0
+    assert lib.mi355x_memcpy_h2d_async(a.ptr, src, 0, stream) == 0
+    a.free(); b.free()
+    shim._chk(lib.mi355x_host_free(src)); shim._chk(lib.mi355x_host_free(dst))
+    dev.stream_destroy(stream)
