@@ -98,6 +98,9 @@ class DeviceNetwork:
                 q0, q1, qo = shim._quant(xin[0]), shim._quant(xin[1]), shim._quant(yout)
                 self.steps.append((l, self._add_step(yout.num_elements, q0, q1, qo, l.act, xb[0].ptr, xb[1].ptr, yb.ptr)))
                 self._step_plans.append(None)
+            elif l.op == "pad":
+                self.steps.append((l, self._pad_step(xin[0], yout, l.params["pad_list"], l.params["pad_value"], xb[0].ptr, yb.ptr)))
+                self._step_plans.append(None)
             elif l.op == "softmax":
                 rows, cols = yout.shape
                 qi, qo = shim._quant(xin[0]), shim._quant(yout)
@@ -153,6 +156,21 @@ class DeviceNetwork:
         return lambda s, lane=0, lanes=1: shim._chk(lib.mi355x_add_run(
             n // lanes, C.byref(q0), C.byref(q1), C.byref(qo), act[0], act[1], act[2], x0 + lane * (n // lanes),
             x1 + lane * (n // lanes), y + lane * (n // lanes), s))
+
+    def _pad_step(self, xin, yout, pad_list, pad_value, x, y):
+        lib = self.lib
+        nx, ny = xin.num_elements, yout.num_elements
+        batch_padded = tuple(pad_list[0]) != (0, 0)
+        descs = {}
+
+        def run(s, lane=0, lanes=1):
+            if batch_padded and lanes > 1:
+                raise ValueError("a Pad layer that pads the batch cannot run in lanes")
+            if lanes not in descs:
+                shape = (xin.shape[0] // lanes,) + tuple(xin.shape[1:])
+                descs[lanes] = shim.pad_desc(shape, pad_list, pad_value, xin, yout)
+            shim._chk(lib.mi355x_pad_run(C.byref(descs[lanes]), x + lane * (nx // lanes), y + lane * (ny // lanes), s))
+        return run
 
     def _softmax_step(self, rows, cols, beta, qi, qo, x, y):
         lib = self.lib

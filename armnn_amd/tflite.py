@@ -1,0 +1,268 @@
+"""Reads a quantized .tflite model into a nets.Network, with the conventions of Arm NN's TfLite parser.
+
+Only what the device path runs is accepted: 8-bit quantized CONV_2D, DEPTHWISE_CONV_2D, FULLY_CONNECTED,
+AVERAGE_POOL_2D, MAX_POOL_2D, ADD, PAD, RESHAPE and SOFTMAX, one subgraph, one input, one output.  Anything else raises
+``UnsupportedModel`` naming the operator -- nothing is approximated or skipped.
+
+What is taken from the reference parser (src/armnnTfLiteParser/TfLiteParser.cpp):
+  * SAME padding, front = total // 2 (CalcPadding, :406-427); VALID = none;
+  * pooling excludes padding from the divisor and rounds output sizes down (ParsePool: PaddingMethod::Exclude, Floor);
+  * a fused activation becomes ReLu, BoundedReLu(6, 0) or BoundedReLu(1, -1) behind the layer, in the layer's own
+    output quantization (AddFusedActivationLayer, :5405-5464);
+  * FULLY_CONNECTED flattens an input of more than two dimensions to [elements / K, K] first (ParseFullyConnected);
+    TfLite keeps FC weights as [outputs, K], i.e. m_TransposeWeightMatrix = true;
+  * convolution weights are [O, H, W, I] and depthwise weights [1, H, W, I * multiplier], as the reference keeps them;
+  * per-channel weights carry their scales along quantized_dimension; the int32 bias keeps the scale the file states.
+
+The file format is FlatBuffers; the few accessors needed are written out here (the schema is tensorflow/lite/schema/
+schema.fbs, version 3: field numbers are cited where they are used).
+"""
+from __future__ import annotations
+
+import struct
+from typing import Dict, List, Optional, Tuple
+
+import numpy as np
+
+from .nets import Layer, Network, same_padding
+from .tensor import DataType, QTensor, TensorInfo
+
+
+class UnsupportedModel(ValueError):
+    pass
+
+
+# ---- FlatBuffers ---------------------------------------------------------------------------------------------------------
+class _Table:
+    """A FlatBuffers table: fields are looked up through the vtable the table points back to."""
+
+    def __init__(self, buf: bytes, pos: int):
+        self.buf, self.pos = buf, pos
+        self.vt = pos - struct.unpack_from("<i", buf, pos)[0]
+        self.vt_size = struct.unpack_from("<H", buf, self.vt)[0]
+
+    def _field(self, k: int) -> int:
+        off = 4 + 2 * k
+        if off >= self.vt_size:
+            return 0
+        rel = struct.unpack_from("<H", self.buf, self.vt + off)[0]
+        return self.pos + rel if rel else 0
+
+    def scalar(self, k: int, fmt: str, default=0):
+        p = self._field(k)
+        return struct.unpack_from("<" + fmt, self.buf, p)[0] if p else default
+
+    def table(self, k: int) -> Optional["_Table"]:
+        p = self._field(k)
+        return _Table(self.buf, p + struct.unpack_from("<I", self.buf, p)[0]) if p else None
+
+    def _vector(self, k: int) -> Tuple[int, int]:
+        p = self._field(k)
+        if not p:
+            return 0, 0
+        v = p + struct.unpack_from("<I", self.buf, p)[0]
+        return v + 4, struct.unpack_from("<I", self.buf, v)[0]
+
+    def string(self, k: int) -> str:
+        start, n = self._vector(k)
+        return self.buf[start:start + n].decode("utf-8", "replace") if start else ""
+
+    def numbers(self, k: int, dtype) -> np.ndarray:
+        start, n = self._vector(k)
+        return np.frombuffer(self.buf, dtype=dtype, count=n, offset=start).copy() if start else np.zeros(0, dtype)
+
+    def tables(self, k: int) -> List["_Table"]:
+        start, n = self._vector(k)
+        out = []
+        for i in range(n):
+            p = start + 4 * i
+            out.append(_Table(self.buf, p + struct.unpack_from("<I", self.buf, p)[0]))
+        return out
+
+
+# ---- schema constants ------------------------------------------------------------------------------------------------------
+_UINT8, _INT32, _INT8 = 3, 2, 9                                   # TensorType
+_OPS = {0: "ADD", 1: "AVERAGE_POOL_2D", 3: "CONV_2D", 4: "DEPTHWISE_CONV_2D", 9: "FULLY_CONNECTED", 17: "MAX_POOL_2D",
+        22: "RESHAPE", 25: "SOFTMAX", 34: "PAD"}                  # BuiltinOperator
+_ACT = {0: (0, 0.0, 0.0), 1: (1, 0.0, 0.0), 2: (2, 1.0, -1.0), 3: (2, 6.0, 0.0)}    # NONE, RELU, RELU_N1_TO_1, RELU6
+_SAME, _VALID = 0, 1
+
+
+def _pad(padding: int, size: int, k: int, stride: int, dilation: int = 1) -> Tuple[int, int]:
+    if padding == _VALID:
+        return 0, 0
+    _, front, back = same_padding(size, k, stride, dilation)
+    return front, back
+
+
+class _Model:
+    def __init__(self, data: bytes):
+        if len(data) < 8 or data[4:8] != b"TFL3":
+            raise UnsupportedModel("not a TfLite flatbuffer (file identifier TFL3 missing)")
+        self.buf = data
+        root = _Table(data, struct.unpack_from("<I", data, 0)[0])
+        self.opcodes = root.tables(1)                              # Model.operator_codes
+        graphs = root.tables(2)                                    # Model.subgraphs
+        if len(graphs) != 1:
+            raise UnsupportedModel(f"{len(graphs)} subgraphs (one is supported)")
+        self.graph = graphs[0]
+        self.buffers = root.tables(4)                              # Model.buffers
+        self.tensors = self.graph.tables(0)                        # SubGraph.tensors
+        self.description = root.string(3)
+
+    def opcode(self, op: _Table) -> int:
+        oc = self.opcodes[op.scalar(0, "I")]                      # Operator.opcode_index
+        # OperatorCode.builtin_code (3) superseded deprecated_builtin_code (0, a byte) for codes above 127
+        return max(oc.scalar(3, "i"), oc.scalar(0, "b"))
+
+    def info(self, index: int, constant: bool = False) -> TensorInfo:
+        t = self.tensors[index]
+        shape = tuple(int(v) for v in t.numbers(0, np.int32))     # Tensor.shape
+        ttype = t.scalar(1, "b")                                   # Tensor.type
+        q = t.table(4)                                             # Tensor.quantization
+        scales = q.numbers(2, np.float32) if q else np.zeros(0, np.float32)       # QuantizationParameters.scale
+        zeros = q.numbers(3, np.int64) if q else np.zeros(0, np.int64)            # .zero_point
+        qdim = q.scalar(6, "i") if q else 0                        # .quantized_dimension
+        name = t.string(3)
+        if ttype == _INT32:
+            dtype = DataType.Signed32
+        elif ttype == _UINT8:
+            dtype = DataType.QAsymmU8
+        elif ttype == _INT8:
+            # the reference maps per-channel int8 constants to QSymmS8 and everything else to QAsymmS8
+            dtype = DataType.QSymmS8 if (constant and len(scales) > 1) else DataType.QAsymmS8
+        else:
+            raise UnsupportedModel(f"tensor '{name}' has TensorType {ttype}; only UINT8, INT8 and INT32 run on the device")
+        if len(scales) == 0:
+            if dtype != DataType.Signed32:
+                raise UnsupportedModel(f"tensor '{name}' carries no quantization")
+            scales = np.ones(1, np.float32)
+        if len(scales) > 1:
+            if np.any(zeros != 0):
+                raise UnsupportedModel(f"tensor '{name}': per-channel quantization with non-zero zero points")
+            return TensorInfo(shape, dtype, tuple(float(s) for s in scales), 0, int(qdim))
+        return TensorInfo(shape, dtype, (float(scales[0]),), int(zeros[0]) if len(zeros) else 0)
+
+    def constant(self, index: int) -> Optional[QTensor]:
+        t = self.tensors[index]
+        b = self.buffers[t.scalar(2, "I")]                         # Tensor.buffer -> Buffer.data
+        info = self.info(index, constant=True)
+        np_dtype = {DataType.Signed32: np.int32, DataType.QAsymmU8: np.uint8}.get(info.dtype, np.int8)
+        raw = b.numbers(0, np.uint8)
+        if raw.size == 0:
+            return None
+        data = raw.view(np_dtype).reshape(info.shape)
+        return QTensor(info, data.astype(np.int64))
+
+
+def load(path: str) -> Network:
+    with open(path, "rb") as f:
+        return parse(f.read(), name=path.rsplit("/", 1)[-1])
+
+
+def parse(data: bytes, name: str = "tflite") -> Network:
+    m = _Model(data)
+    inputs = m.graph.numbers(1, np.int32)                          # SubGraph.inputs
+    outputs = m.graph.numbers(2, np.int32)                         # SubGraph.outputs
+    if len(inputs) != 1 or len(outputs) != 1:
+        raise UnsupportedModel(f"{len(inputs)} inputs and {len(outputs)} outputs (one of each is supported)")
+    tname = lambda i: f"t{i}:{m.tensors[i].string(3)}"
+    tensors: Dict[str, TensorInfo] = {}
+    layers: List[Layer] = []
+
+    def activation_tensor(i: int) -> str:
+        n = tname(i)
+        if n not in tensors:
+            tensors[n] = m.info(i)
+        return n
+
+    def need_constant(i: int, what: str, op: str) -> QTensor:
+        c = m.constant(i) if i >= 0 else None
+        if c is None:
+            raise UnsupportedModel(f"{op}: {what} must be a constant tensor")
+        return c
+
+    activation_tensor(int(inputs[0]))
+    for k, op in enumerate(m.graph.tables(3)):                     # SubGraph.operators
+        code = m.opcode(op)
+        kind = _OPS.get(code)
+        ins = [int(v) for v in op.numbers(1, np.int32)]            # Operator.inputs
+        outs = [int(v) for v in op.numbers(2, np.int32)]           # Operator.outputs
+        o = op.table(4)                                            # Operator.builtin_options
+        lname = f"op{k}:{kind}"
+        if kind is None:
+            raise UnsupportedModel(f"operator {k} has builtin code {code}, which the device path does not run")
+        x = activation_tensor(ins[0])
+        xi = tensors[x]
+        y = activation_tensor(outs[0])
+        yi = tensors[y]
+        if kind in ("CONV_2D", "DEPTHWISE_CONV_2D"):
+            dw = kind == "DEPTHWISE_CONV_2D"
+            w = need_constant(ins[1], "weights", kind)
+            b = need_constant(ins[2], "bias", kind) if len(ins) > 2 and ins[2] >= 0 else None
+            padding, sw, sh = o.scalar(0, "b"), o.scalar(1, "i"), o.scalar(2, "i")
+            act = _ACT[o.scalar(4 if dw else 3, "b")]
+            dwf, dhf = o.scalar(5 if dw else 4, "i", 1), o.scalar(6 if dw else 5, "i", 1)
+            _, h, wd, ci = xi.shape
+            kh, kw = w.info.shape[1], w.info.shape[2]
+            pt, _ = _pad(padding, h, kh, sh, dhf)
+            pl, _ = _pad(padding, wd, kw, sw, dwf)
+            if dw and w.info.shape[0] != 1:
+                raise UnsupportedModel("DEPTHWISE_CONV_2D weights must be [1, H, W, I * multiplier]")
+            if b is not None:
+                b = _bias_like_reference(b, xi, w.info)
+            taps = kh * kw if dw else kh * kw * ci
+            params = dict(pad_top=pt, pad_left=pl, stride_x=sw, stride_y=sh, dilation_x=dwf, dilation_y=dhf, depthwise=dw,
+                          _macs=yi.shape[1] * yi.shape[2] * yi.shape[3] * taps)
+            layers.append(Layer("depthwise" if dw else "conv", lname, (x,), y, w, b, params, act))
+        elif kind == "FULLY_CONNECTED":
+            w = need_constant(ins[1], "weights", kind)
+            b = need_constant(ins[2], "bias", kind) if len(ins) > 2 and ins[2] >= 0 else None
+            kdim = w.info.shape[1]
+            if len(xi.shape) > 2 or xi.shape[-1] != kdim:
+                flat = f"{x}:flat"
+                tensors[flat] = TensorInfo((xi.num_elements // kdim, kdim), xi.dtype, xi.scales, xi.offset)
+                layers.append(Layer("reshape", lname + ":flatten", (x,), flat))
+                x, xi = flat, tensors[flat]
+            if b is not None:
+                b = _bias_like_reference(b, xi, w.info)
+            if len(yi.shape) != 2:
+                tensors[y] = yi = TensorInfo((xi.shape[0], w.info.shape[0]), yi.dtype, yi.scales, yi.offset)
+            layers.append(Layer("fc", lname, (x,), y, w, b, dict(transpose_weights=True, _macs=kdim * w.info.shape[0]),
+                                _ACT[o.scalar(0, "b")] if o else _ACT[0]))
+        elif kind in ("AVERAGE_POOL_2D", "MAX_POOL_2D"):
+            padding, sw, sh, fw, fh = o.scalar(0, "b"), o.scalar(1, "i"), o.scalar(2, "i"), o.scalar(3, "i"), o.scalar(4, "i")
+            _, h, wd, _ = xi.shape
+            pt, pb = _pad(padding, h, fh, sh)
+            pl, pr = _pad(padding, wd, fw, sw)
+            params = dict(pool_type=0 if kind == "MAX_POOL_2D" else 1, pool_w=fw, pool_h=fh, stride_x=sw, stride_y=sh,
+                          pad_left=pl, pad_right=pr, pad_top=pt, pad_bottom=pb, padding_method=1)
+            layers.append(Layer("pool", lname, (x,), y, params=params, act=_ACT[o.scalar(5, "b")]))
+        elif kind == "ADD":
+            x1 = activation_tensor(ins[1])
+            if tensors[x1].shape != xi.shape:
+                raise UnsupportedModel("ADD with broadcasting")
+            layers.append(Layer("add", lname, (x, x1), y, act=_ACT[o.scalar(0, "b")] if o else _ACT[0]))
+        elif kind == "PAD":
+            p = need_constant(ins[1], "paddings", kind)
+            pads = tuple((int(a), int(b)) for a, b in p.data.reshape(-1, 2))
+            # TfLite pads with the real number 0, which is the zero point in the tensor's own code
+            layers.append(Layer("pad", lname, (x,), y, params=dict(pad_list=pads, pad_value=float(xi.offset))))
+        elif kind == "RESHAPE":
+            layers.append(Layer("reshape", lname, (x,), y))
+        elif kind == "SOFTMAX":
+            layers.append(Layer("softmax", lname, (x,), y, params=dict(beta=float(o.scalar(0, "f", 1.0)) if o else 1.0)))
+    return Network(name, tname(int(inputs[0])), tname(int(outputs[0])), tensors, layers)
+
+
+def _bias_like_reference(b: QTensor, x: TensorInfo, w: TensorInfo) -> QTensor:
+    """The bias keeps the scale(s) the file gives it, as the reference's decoder reads them; what the reference checks
+    (ValidateBiasTensorQuantization, src/backends/backendsCommon/WorkloadData.cpp) is checked here as well: Signed32,
+    zero point 0, as many scales as the weights have."""
+    if b.info.dtype != DataType.Signed32:
+        raise UnsupportedModel("bias is not INT32")
+    if b.info.offset != 0:
+        raise UnsupportedModel("bias zero point is not 0")
+    if len(b.info.scales) != len(w.scales):
+        raise UnsupportedModel("bias and weights differ in their number of quantization scales")
+    return b

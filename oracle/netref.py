@@ -30,6 +30,8 @@ def run_network(orc: Oracle, net: Network, x: QTensor, keep: bool = False, fast:
             y = orc.pooling2d(ins[0], out_info, **l.params)
         elif l.op == "add":
             y = orc.add(ins[0], ins[1], out_info)
+        elif l.op == "pad":
+            y = orc.pad(ins[0], out_info, [b for b, _ in l.params["pad_list"]], l.params["pad_value"])
         elif l.op == "softmax":
             y = orc.softmax(ins[0], out_info, l.params["beta"], -1)
         elif l.op == "reshape":

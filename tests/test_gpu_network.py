@@ -140,3 +140,22 @@ def test_two_threads_run_two_networks_at_once():
     assert all(not t.is_alive() for t in threads)
     for k in range(2):
         np.testing.assert_array_equal(got[k], want[k])
+
+
+def test_tflite_model_from_the_reference_test_data(port):
+    """delegate/python/test/test_data/mock_model.tflite (kept under tests/golden): uint8 with asymmetric per-tensor
+    weights, a depthwise layer of multiplier 32, max pooling, dense and softmax layers."""
+    import os
+    from armnn_amd import tflite
+    from tests.helpers import GOLDEN
+    net = tflite.load(os.path.join(GOLDEN, "mock_model.tflite"))
+    _layerwise(port, net, 1)
+    _layerwise(port, net, 8)
+
+
+def test_tflite_model_with_pad_per_channel_weights_and_fused_activations(port):
+    from armnn_amd import tflite
+    from tests.test_tflite import written_model
+    net = tflite.parse(written_model(), "written")
+    _layerwise(port, net, 1)
+    _layerwise(port, net, 6)
