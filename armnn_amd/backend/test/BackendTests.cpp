@@ -1178,6 +1178,33 @@ TEST_CASE("runtime: intermediate tensors share an arena smaller than their sum",
     mi355x::SetLanes(lanesBefore);
 }
 
+TEST_CASE("runtime: two host threads, each with a runtime and a network of its own, share the backend's streams", "gpu")
+{
+    // the forked / joined state of the lanes belongs to the calling thread; the streams are the process's
+    MiniMobileNet a(32, DataType::QAsymmS8), b(16, DataType::QAsymmU8);
+    const std::vector<uint8_t> inA = RandomActivations(a.in, 31), inB = RandomActivations(b.in, 32);
+    const std::vector<uint8_t> wantA = a.RunDirect(inA), wantB = b.RunDirect(inB);
+    std::vector<std::string> problems(2);
+    auto work = [&](int which) {
+        try
+        {
+            const MiniMobileNet& m = which == 0 ? a : b;
+            const std::vector<uint8_t>& in = which == 0 ? inA : inB;
+            const std::vector<uint8_t>& want = which == 0 ? wantA : wantB;
+            IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+            INetworkPtr net = m.Build();
+            for (int i = 0; i < 4; ++i)
+                if (RunOnRuntime(*rt, *net, {kMi355x}, m.in, in, m.probs, 3) != want) problems[which] = "bytes differ in round " + std::to_string(i);
+        }
+        catch (const std::exception& e) { problems[which] = e.what(); }
+    };
+    std::thread t0(work, 0), t1(work, 1);
+    t0.join();
+    t1.join();
+    CHECK_MSG(problems[0].empty(), problems[0]);
+    CHECK_MSG(problems[1].empty(), problems[1]);
+}
+
 TEST_CASE("runtime: a batch run as two or four slices on streams of their own gives the bytes of the unsplit run", "gpu")
 {
     const unsigned int lanesBefore = mi355x::Lanes();

@@ -3,6 +3,7 @@
   python -m armnn_amd.layerbench conv --n 64 --h 14 --w 14 --ci 512 --co 512 --k 1
   python -m armnn_amd.layerbench dw   --n 64 --h 112 --w 112 --c 32 --stride 1
   python -m armnn_amd.layerbench fc   --m 2048 --k 4096 --o 4096
+  python -m armnn_amd.layerbench pad  --n 64 --h 112 --w 112 --c 64        (one row and column on every side)
 
 Prints one JSON line: kernel chosen, average launch time (HIP events on the launch stream), algorithmic
 ops and bytes, and the fraction of the int8 MFMA peak (5.0 POP/s) or of the HBM peak (8 TB/s).
@@ -29,9 +30,36 @@ def _same(in_size, k, stride):
     return out, total // 2
 
 
+def _pad(dev, a, adt, zp):
+    """A constant Pad of one row and column on every side of an NHWC tensor: one byte read per input element, one
+    written per output element."""
+    import ctypes as C
+    xin = TensorInfo((a.n, a.h, a.w, a.c), adt, (0.0235,), zp)
+    yout = TensorInfo((a.n, a.h + 2, a.w + 2, a.c), adt, (0.0235,), zp)
+    d = shim.pad_desc(xin.shape, ((0, 0), (1, 1), (1, 1), (0, 0)), float(zp), xin, yout)
+    lib = shim.load_library()
+    xd = shim.DeviceBuffer(xin.num_elements).upload(synth.uniform_int(1, xin.shape, 0, 127, np.uint8))
+    yd = shim.DeviceBuffer(yout.num_elements)
+    stream = dev.stream()
+    run = lambda: shim._chk(lib.mi355x_pad_run(C.byref(d), xd.ptr, yd.ptr, stream))
+    for _ in range(a.warmup):
+        run()
+    e0, e1 = dev.event(), dev.event()
+    dev.event_record(e0, stream)
+    for _ in range(a.iters):
+        run()
+    dev.event_record(e1, stream)
+    dev.event_sync(e1)
+    ms = dev.elapsed_ms(e0, e1) / a.iters
+    nbytes = xin.num_elements + yout.num_elements
+    print(json.dumps({"layer": f"pad N={a.n} {a.h}x{a.w}x{a.c} by 1 on height and width", "kernel": "PadKernel", "us": ms * 1e3,
+                      "GBps": nbytes / (ms * 1e-3) / 1e9, "frac_hbm_peak": nbytes / (ms * 1e-3) / HBM_PEAK, "bytes": nbytes}))
+    return 0
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("op", choices=["conv", "dw", "fc"])
+    ap.add_argument("op", choices=["conv", "dw", "fc", "pad"])
     ap.add_argument("--n", type=int, default=64)
     ap.add_argument("--h", type=int, default=56)
     ap.add_argument("--w", type=int, default=56)
@@ -55,6 +83,8 @@ def main(argv=None):
     dev = shim.Device()
     adt = DataType.QAsymmU8 if a.u8 else DataType.QAsymmS8
     zp = 128 if a.u8 else -3
+    if a.op == "pad":
+        return _pad(dev, a, adt, zp)
     act = (shim.ACT_BOUNDED_RELU, 6.0, 0.0)
     if a.op == "fc":
         k, o, m = a.k if a.k > 3 else 4096, a.o, a.m
