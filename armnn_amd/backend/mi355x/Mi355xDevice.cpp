@@ -14,6 +14,7 @@ std::once_flag g_Once;
 mi355x_stream_t g_Streams[kMaxLanes] = {nullptr, nullptr, nullptr, nullptr};
 std::atomic<unsigned int> g_Lanes{0};          // 0: not decided yet
 std::atomic<int> g_SharingArenas{0};
+std::atomic<unsigned long long> g_Epoch{1};
 bool g_Ready = false;
 std::string g_Why;
 
@@ -149,7 +150,13 @@ void UploadInLanes(void* dstDevice, const void* srcHost, size_t bytes, unsigned 
     }
 }
 
-void Synchronize() { Check(mi355x_stream_synchronize(Stream()), "mi355x_stream_synchronize"); }
+void Synchronize()
+{
+    Check(mi355x_stream_synchronize(Stream()), "mi355x_stream_synchronize");
+    g_Epoch.fetch_add(1);
+}
+
+unsigned long long SyncEpoch() { return g_Epoch.load(); }
 
 void Check(int status, const char* what)
 {

@@ -22,6 +22,9 @@ void EnsureDevice();
 mi355x_stream_t Stream();
 /// joins the lanes and waits for the stream
 void Synchronize();
+/// how many times any thread has waited for the stream so far.  An inference ends with such a wait (the runtime maps the
+/// network's outputs), so a value that has not changed means "still the same inference".
+unsigned long long SyncEpoch();
 
 /// Lanes.  Every image of a batch is computed independently, so a workload may run its batch as Lanes() contiguous
 /// slices, slice k on LaneStream(k): one slice's launches then fill the ramp-up, tail and launch gaps of the others, and

@@ -68,6 +68,7 @@ bool Mi355xTensorHandle::Import(void* memory, MemorySource source)
     m_ImportedHost = memory;
     m_ImportedDevice = device;
     m_DeviceNewer = false;
+    m_FetchedInEpoch = 0;
     return true;
 }
 
@@ -83,9 +84,12 @@ const void* Mi355xTensorHandle::GetDevicePointerForRead() const
 {
     void* dev = GetDevicePointer();
     // adopted buffer, not written by a workload since the caller last saw it: it is an input, and whatever the caller
-    // has put there is what this inference reads
-    if (m_ImportedDevice && !m_ImportedIsDeviceMemory && !m_DeviceNewer && m_Info.GetNumBytes())
+    // has put there is what this inference reads -- fetched once per inference, however many workloads read the tensor
+    if (m_ImportedDevice && !m_ImportedIsDeviceMemory && !m_DeviceNewer && m_Info.GetNumBytes() && m_FetchedInEpoch != mi355x::SyncEpoch())
+    {
         mi355x::UploadInLanes(dev, m_ImportedDevice, m_Info.GetNumBytes(), UploadLanes());
+        m_FetchedInEpoch = mi355x::SyncEpoch();
+    }
     return dev;
 }
 

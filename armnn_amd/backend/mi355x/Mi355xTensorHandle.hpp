@@ -70,6 +70,7 @@ private:
     mutable void* m_Staging = nullptr;  // pinned host copy, created by the first Map()
     mutable bool m_DeviceNewer = false;
     mutable bool m_UploadInFlight = false;
+    mutable unsigned long long m_FetchedInEpoch = 0;   // mi355x::SyncEpoch() when an adopted input was last brought over
     mutable int m_MapCount = 0;
 };
 
