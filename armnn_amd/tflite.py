@@ -266,3 +266,42 @@ def _bias_like_reference(b: QTensor, x: TensorInfo, w: TensorInfo) -> QTensor:
     if len(b.info.scales) != len(w.scales):
         raise UnsupportedModel("bias and weights differ in their number of quantization scales")
     return b
+
+
+def main(argv=None) -> int:
+    """python -m armnn_amd.tflite model.tflite [--batch N] [--iterations K]: loads the model, runs it on the device on
+    seeded synthetic input and prints the layer list, the class distribution of the first image and the throughput
+    (what tests/ExecuteNetwork reports for a model in the reference: inference time over a number of iterations)."""
+    import argparse
+    import json
+    import time
+
+    from . import nets
+    from .executor import DeviceNetwork
+
+    ap = argparse.ArgumentParser()
+    ap.add_argument("model")
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--iterations", type=int, default=50)
+    ap.add_argument("--lanes", type=int, default=1)
+    a = ap.parse_args(argv)
+    net = load(a.model)
+    for l in net.layers:
+        print(f"{l.op:>9s} {l.name:<28s} {' '.join(str(net.tensors[i].shape) for i in l.inputs)} -> {net.tensors[l.output].shape}")
+    dn = DeviceNetwork(net, a.batch, lanes=a.lanes)
+    x = nets.synthetic_input(net, a.batch)
+    y = dn.run(x)
+    t0 = time.perf_counter()
+    for _ in range(a.iterations):
+        dn.enqueue()
+    dn.synchronize()
+    ms = (time.perf_counter() - t0) * 1e3 / a.iterations
+    dn.close()
+    print(json.dumps({"model": net.name, "batch": a.batch, "ms_per_inference": ms, "images_per_sec": a.batch / ms * 1e3,
+                      "first_image_output": [int(v) for v in y.data[0].ravel()[:16]]}))
+    return 0
+
+
+if __name__ == "__main__":
+    import sys
+    sys.exit(main())

@@ -179,7 +179,7 @@ def test_depthwise_rows_per_thread_variants_give_the_same_bytes():
 
 
 def test_config_c1_full_size(port):
-    """BASELINE config 1: 1x56x56x64 -> 64, 3x3 SAME, per-channel, ReLU6; expected code range [-128, -8]."""
+    """Benchmark configuration C1: 1x56x56x64 -> 64, 3x3 SAME, per-channel, ReLU6; expected code range [-128, -8]."""
     c = cases.make_conv_case("C1", 20250101, h=56, w=56, ci=64, co=64, act=cases.RELU6)
     want = _oracle_conv(port, c)
     got = _gpu_conv(c, shim.ALGO_AUTO)
@@ -191,7 +191,7 @@ def test_config_c1_full_size(port):
 
 
 def test_config_c2_block(port):
-    """BASELINE config 2: depthwise 3x3 + pointwise 32->64 on 1x112x112x32 QAsymmU8, ReLU6 after each."""
+    """Benchmark configuration C2: depthwise 3x3 + pointwise 32->64 on 1x112x112x32 QAsymmU8, ReLU6 after each."""
     U8 = DataType.QAsymmU8
     dw = cases.make_conv_case("C2dw", 20250102, h=112, w=112, ci=32, depthwise=True, in_dtype=U8, in_scale=0.0235,
                               in_offset=128, out_scale=0.0235, out_offset=0, act=cases.RELU6, w_scale_range=(0.01, 0.05))
@@ -212,7 +212,7 @@ def test_config_c2_block(port):
 
 @pytest.mark.parametrize("m", [1, 256])
 def test_config_c4_fc(port, m):
-    """BASELINE config 4: [M,4096] x [4096,4096] per-channel, fused requantize (output scale 1.0, zp 0)."""
+    """Benchmark configuration C4: [M,4096] x [4096,4096] per-channel, fused requantize (output scale 1.0, zp 0)."""
     c = cases.make_fc_case("C4", 20250104, m=m, k=4096, o=4096, in_offset=0, out_scale=1.0, out_offset=0)
     want = port.fully_connected(c.x, c.w, c.b, c.out_info)
     got = shim.fully_connected(c.x, c.w, c.b, c.out_info)
@@ -220,3 +220,126 @@ def test_config_c4_fc(port, m):
     sat = float(((got.data == 127) | (got.data == -128)).mean())
     print(f"C4 M={m}: max|d|={mx} exact={exact:.6f} saturated={sat:.4f}", flush=True)
     assert mx <= 1 and exact >= 0.995 and sat < 0.05
+
+
+def _random_conv_case(k):
+    """One seeded draw from the space of convolutions the library accepts: shapes, strides, dilations, paddings, data
+    types, per-channel or per-tensor (also asymmetric) weights, output quantizations from coarse to fine, activations."""
+    rng = np.random.default_rng(7000 + k)
+    pick = lambda xs: xs[int(rng.integers(len(xs)))]
+    depthwise = bool(rng.integers(4) == 0)
+    kh, kw = pick([1, 1, 2, 3, 3, 3, 5]), pick([1, 1, 2, 3, 3, 3, 5])
+    if rng.integers(3) != 0:
+        kw = kh
+    dil = (pick([1, 1, 1, 2]), pick([1, 1, 1, 2]))
+    h = int(rng.integers(max(1, (kh - 1) * dil[1] - 1), 24))
+    w = int(rng.integers(max(1, (kw - 1) * dil[0] - 1), 24))
+    ci = pick([1, 3, 4, 8, 16, 20, 32, 48, 64, 128, 256])
+    co = pick([1, 5, 8, 16, 32, 40, 64, 128, 256])
+    in_u8 = bool(rng.integers(2))
+    padding = pick(["same", "valid", (int(rng.integers(0, kh + 1)), int(rng.integers(0, kh + 1)), int(rng.integers(0, kw + 1)), int(rng.integers(0, kw + 1)))])
+    if padding == "valid" and (h < (kh - 1) * dil[1] + 1 or w < (kw - 1) * dil[0] + 1):
+        padding = "same"
+    w_kind = pick(["per_axis", "per_axis", "per_tensor", "asym_s8", "asym_u8"])
+    w_dtype = {"asym_s8": DataType.QAsymmS8, "asym_u8": DataType.QAsymmU8}.get(w_kind, DataType.QSymmS8)
+    w_offset = {"asym_s8": int(rng.integers(-20, 20)), "asym_u8": int(rng.integers(100, 150))}.get(w_kind, 0)
+    out_scale = float(np.exp(rng.uniform(np.log(0.004), np.log(0.5))))
+    lo = 0 if in_u8 else -128
+    act = pick([(0, 0.0, 0.0), (1, 0.0, 0.0), (2, 6.0, 0.0), (2, 1.0, -1.0)])
+    return cases.make_conv_case(
+        f"random{k}", 9000 + 11 * k, n=int(rng.integers(1, 4)), h=h, w=w, ci=ci, co=co, kh=kh, kw=kw,
+        stride=(pick([1, 1, 2, 3]), pick([1, 1, 2, 3])), dilation=dil, padding=padding, depthwise=depthwise,
+        mult=pick([1, 1, 1, 2]) if depthwise else 1, in_dtype=DataType.QAsymmU8 if in_u8 else DataType.QAsymmS8,
+        in_scale=float(rng.uniform(0.005, 0.05)), in_offset=lo + int(rng.integers(0, 256)), w_dtype=w_dtype,
+        per_axis=w_kind == "per_axis", w_offset=w_offset, bias=bool(rng.integers(4) != 0),
+        bias_scale_matches=bool(rng.integers(5) != 0), out_scale=out_scale, out_offset=lo + int(rng.integers(0, 256)), act=act)
+
+
+@pytest.mark.parametrize("chunk", range(8))
+def test_random_convolutions(port, chunk):
+    """240 seeded draws, 30 per test: whatever kernel AUTO picks must stay within 1 LSB of the checker and give the
+    bytes of the direct kernel."""
+    for k in range(30 * chunk, 30 * chunk + 30):
+        try:
+            case = _random_conv_case(k)
+        except ValueError:
+            continue                                   # a draw whose output would be empty
+        if 0 in case.out_info.shape:
+            continue
+        print(f"random case {k}: x={case.x.info.shape} w={case.w.info.shape} {case.w.info.dtype.name} params={case.params} "
+              f"act={case.act} out={case.out_info.scale:.4f}/{case.out_info.offset}", flush=True)
+        want = _oracle_conv(port, case)
+        auto = _gpu_conv(case, shim.ALGO_AUTO)
+        mx, exact = lsb_diff(auto.data, want.data)
+        assert mx <= 1, (k, mx)
+        assert exact >= 0.98 or auto.data.size < 200, (k, exact)
+        direct = _gpu_conv(case, shim.ALGO_DIRECT)
+        np.testing.assert_array_equal(auto.data, direct.data, err_msg=f"random case {k}")
+
+
+def _fast_path_case(k):
+    """A seeded draw from the shapes the specialised kernels take: pointwise and 3x3 convolutions with channel counts in
+    multiples of 16, 3x3 depthwise layers with channels in multiples of 32, stems with 1..4 input channels."""
+    rng = np.random.default_rng(17000 + k)
+    pick = lambda xs: xs[int(rng.integers(len(xs)))]
+    family = pick(["pointwise", "pointwise", "conv3x3", "conv3x3", "depthwise", "depthwise", "stem"])
+    in_u8 = bool(rng.integers(2))
+    lo = 0 if in_u8 else -128
+    kw = dict(n=int(rng.integers(1, 6)), h=int(rng.integers(3, 41)), w=int(rng.integers(3, 41)), per_axis=bool(rng.integers(4) != 0),
+              in_dtype=DataType.QAsymmU8 if in_u8 else DataType.QAsymmS8, in_scale=float(rng.uniform(0.005, 0.05)),
+              in_offset=lo + int(rng.integers(0, 256)), bias=bool(rng.integers(5) != 0),
+              out_scale=float(np.exp(rng.uniform(np.log(0.01), np.log(0.3)))), out_offset=lo + int(rng.integers(0, 256)),
+              act=pick([(0, 0.0, 0.0), (1, 0.0, 0.0), (2, 6.0, 0.0)]))
+    if family == "pointwise":
+        kw.update(ci=pick([16, 32, 64, 96, 128, 256, 512]), co=pick([16, 24, 32, 64, 128, 200, 256, 512]), kh=1, kw=1, padding="valid")
+    elif family == "conv3x3":
+        kw.update(ci=pick([16, 32, 64, 128, 256]), co=pick([16, 32, 64, 128, 256]), kh=3, kw=3, stride=pick([(1, 1), (1, 1), (2, 2)]),
+                  padding=pick(["same", "same", "valid", (1, 0, 2, 1)]))
+    elif family == "depthwise":
+        kw.update(ci=pick([32, 64, 96, 128, 256, 512]), kh=3, kw=3, depthwise=True, stride=pick([(1, 1), (2, 2)]), padding=pick(["same", "same", "valid"]))
+    else:
+        size = pick([3, 3, 7])
+        kw.update(ci=pick([1, 3, 3, 4]), co=pick([32, 64]), kh=size, kw=size, stride=pick([(1, 1), (2, 2), (2, 2)]), padding="same",
+                  h=int(rng.integers(8, 65)), w=int(rng.integers(8, 65)))
+    return cases.make_conv_case(f"fast{k}", 19000 + 13 * k, **kw)
+
+
+@pytest.mark.parametrize("chunk", range(6))
+def test_random_draws_from_the_specialised_kernels_shapes(port, chunk):
+    for k in range(30 * chunk, 30 * chunk + 30):
+        case = _fast_path_case(k)
+        print(f"fast-path case {k}: x={case.x.info.shape} w={case.w.info.shape} params={case.params} act={case.act} "
+              f"out={case.out_info.scale:.4f}/{case.out_info.offset}", flush=True)
+        want = _oracle_conv(port, case)
+        auto = _gpu_conv(case, shim.ALGO_AUTO)
+        mx, exact = lsb_diff(auto.data, want.data)
+        assert mx <= 1, (k, mx)
+        assert exact >= 0.98, (k, exact)
+        direct = _gpu_conv(case, shim.ALGO_DIRECT)
+        np.testing.assert_array_equal(auto.data, direct.data, err_msg=f"fast-path case {k}")
+
+
+@pytest.mark.parametrize("chunk", range(3))
+def test_random_fully_connected(port, chunk):
+    for k in range(20 * chunk, 20 * chunk + 20):
+        rng = np.random.default_rng(27000 + k)
+        in_u8 = bool(rng.integers(2))
+        lo = 0 if in_u8 else -128
+        m = int(rng.choice([1, 2, 3, 4, 5, 7, 16, 33, 64, 65, 130, 300]))
+        kdim = int(rng.choice([16, 48, 64, 100, 128, 256, 1000, 1024, 2048]))
+        o = int(rng.choice([1, 10, 16, 37, 64, 128, 1000, 1001]))
+        case = cases.make_fc_case(f"fc{k}", 29000 + 7 * k, m=m, k=kdim, o=o, in_dtype=DataType.QAsymmU8 if in_u8 else DataType.QAsymmS8,
+                                  in_scale=float(rng.uniform(0.005, 0.05)), in_offset=lo + int(rng.integers(0, 256)),
+                                  out_scale=float(np.exp(rng.uniform(np.log(0.01), np.log(0.5)))), out_offset=lo + int(rng.integers(0, 256)))
+        print(f"fc case {k}: m={m} k={kdim} o={o} u8={in_u8}", flush=True)
+        fn, a, b = case.act
+        want = port.fully_connected(case.x, case.w, case.b, case.out_info, transpose_weights=case.transpose_weights)
+        if fn:
+            want = port.activation(want, case.out_info, fn, a, b)
+        kw = dict(transpose_weights=case.transpose_weights, activation=fn, act_a=a, act_b=b)
+        auto = shim.fully_connected(case.x, case.w, case.b, case.out_info, algo=shim.ALGO_AUTO, **kw)
+        mx, exact = lsb_diff(auto.data, want.data)
+        assert mx <= 1, (k, mx)
+        assert exact >= 0.98 or auto.data.size < 200, (k, exact)
+        direct = shim.fully_connected(case.x, case.w, case.b, case.out_info, algo=shim.ALGO_DIRECT, **kw)
+        np.testing.assert_array_equal(auto.data, direct.data, err_msg=f"fc case {k}")
