@@ -195,3 +195,58 @@ def test_async_copies_need_memory_the_device_reaches_and_keep_stream_order():
     a.free(); b.free()
     shim._chk(lib.mi355x_host_free(src)); shim._chk(lib.mi355x_host_free(dst))
     dev.stream_destroy(stream)
+
+
+@pytest.mark.parametrize("chunk", range(4))
+def test_random_pooling_add_softmax_pad(port, chunk):
+    """Seeded draws over the bandwidth-bound layers: window, stride, padding (also wider than the window), padding method,
+    channel counts on and off the vector paths, quantizations, pad lists of every rank."""
+    for k in range(25 * chunk, 25 * chunk + 25):
+        rng = np.random.default_rng(37000 + k)
+        pick = lambda xs: xs[int(rng.integers(len(xs)))]
+        dtype = pick([S8, U8])
+        lo = 0 if dtype == U8 else -128
+        q = lambda: (float(np.exp(rng.uniform(np.log(0.01), np.log(0.2)))), lo + int(rng.integers(0, 256)))
+        kind = pick(["pool", "pool", "add", "softmax", "pad"])
+        print(f"layer case {k}: {kind} {dtype.name}", flush=True)
+        if kind == "pool":
+            n, h, w, c = int(rng.integers(1, 4)), int(rng.integers(1, 20)), int(rng.integers(1, 20)), pick([1, 3, 4, 8, 12, 16, 64, 100, 256])
+            pw, ph, sx, sy = int(rng.integers(1, 6)), int(rng.integers(1, 6)), int(rng.integers(1, 4)), int(rng.integers(1, 4))
+            pl, pr, pt, pb = (int(rng.integers(0, pw + 1)), int(rng.integers(0, pw + 1)), int(rng.integers(0, ph + 1)), int(rng.integers(0, ph + 1)))
+            if h + pt + pb < ph or w + pl + pr < pw:
+                continue
+            s, z = q()
+            x = _rand(38000 + k, (n, h, w, c), dtype, s, z)
+            so, zo = q()
+            oi = TensorInfo((n, (h + pt + pb - ph) // sy + 1, (w + pl + pr - pw) // sx + 1, c), dtype, (so,), zo)
+            kw = dict(pool_type=pick([cpuref.POOL_MAX, cpuref.POOL_AVERAGE]), pool_w=pw, pool_h=ph, stride_x=sx, stride_y=sy, pad_left=pl,
+                      pad_right=pr, pad_top=pt, pad_bottom=pb, padding_method=pick([cpuref.PAD_EXCLUDE, cpuref.PAD_IGNORE_VALUE]))
+            np.testing.assert_array_equal(shim.pooling2d(x, oi, **kw).data, port.pooling2d(x, oi, **kw).data, err_msg=f"case {k} {kw}")
+        elif kind == "add":
+            shape = tuple(int(rng.integers(1, 12)) for _ in range(3)) + (pick([1, 3, 8, 16, 50, 128]),)
+            (s0, z0), (s1, z1), (so, zo) = q(), q(), q()
+            a, b = _rand(39000 + k, shape, dtype, s0, z0), _rand(39500 + k, shape, dtype, s1, z1)
+            oi = TensorInfo(shape, dtype, (so,), zo)
+            act = pick([(0, 0.0, 0.0), (1, 0.0, 0.0), (2, 6.0, 0.0)])
+            want = port.add(a, b, oi)
+            if act[0]:
+                want = port.activation(want, oi, *act)
+            np.testing.assert_array_equal(shim.add(a, b, oi, activation=act[0], act_a=act[1], act_b=act[2]).data, want.data, err_msg=f"case {k}")
+        elif kind == "softmax":
+            rows, cols = int(rng.integers(1, 9)), pick([1, 2, 10, 100, 1000, 1001, 1025, 2048, 3000])
+            s, z = q()
+            x = _rand(40000 + k, (rows, cols), dtype, s, z)
+            oi = TensorInfo((rows, cols), dtype, (1.0 / 256,), lo)
+            beta = float(rng.uniform(0.5, 2.0))
+            mx, _ = lsb_diff(shim.softmax(x, oi, beta).data, port.softmax(x, oi, beta).data)
+            assert mx <= 1, k
+        else:
+            rank = int(rng.integers(1, 5))
+            shape = tuple(int(rng.integers(1, 10)) for _ in range(rank - 1)) + (pick([1, 4, 7, 16, 32]),)
+            pads = tuple((int(rng.integers(0, 3)), int(rng.integers(0, 3))) if rng.integers(2) else (0, 0) for _ in range(rank))
+            s, z = q()
+            x = _rand(41000 + k, shape, dtype, s, z)
+            so, zo = (s, z) if rng.integers(3) else q()
+            oi = TensorInfo(tuple(d + b + a for d, (b, a) in zip(shape, pads)), dtype, (so,), zo)
+            value = float(rng.integers(-300, 300)) + pick([0.0, 0.5])
+            np.testing.assert_array_equal(shim.pad(x, oi, pads, value).data, port.pad(x, oi, [b for b, _ in pads], value).data, err_msg=f"case {k}")
