@@ -88,6 +88,12 @@ _ACT = {0: (0, 0.0, 0.0), 1: (1, 0.0, 0.0), 2: (2, 1.0, -1.0), 3: (2, 6.0, 0.0)}
 _SAME, _VALID = 0, 1
 
 
+def _fused(code: int):
+    if code not in _ACT:
+        raise UnsupportedModel(f"fused activation {code} (NONE, RELU, RELU_N1_TO_1 and RELU6 are supported)")
+    return _ACT[code]
+
+
 def _pad(padding: int, size: int, k: int, stride: int, dilation: int = 1) -> Tuple[int, int]:
     if padding == _VALID:
         return 0, 0
@@ -161,6 +167,18 @@ def load(path: str) -> Network:
 
 
 def parse(data: bytes, name: str = "tflite") -> Network:
+    try:
+        return _parse(data, name)
+    except (struct.error, IndexError, OverflowError, KeyError, TypeError, AttributeError) as e:
+        # offsets that lead outside the buffer, vectors longer than the file, operator or tensor indices out of range
+        raise UnsupportedModel(f"malformed flatbuffer: {e}") from e
+    except ValueError as e:
+        if isinstance(e, UnsupportedModel):
+            raise
+        raise UnsupportedModel(f"malformed flatbuffer: {e}") from e
+
+
+def _parse(data: bytes, name: str) -> Network:
     m = _Model(data)
     inputs = m.graph.numbers(1, np.int32)                          # SubGraph.inputs
     outputs = m.graph.numbers(2, np.int32)                         # SubGraph.outputs
@@ -196,19 +214,33 @@ def parse(data: bytes, name: str = "tflite") -> Network:
         xi = tensors[x]
         y = activation_tensor(outs[0])
         yi = tensors[y]
+
+        def expect(shape, what=kind):
+            # buffers are sized from the file's shapes and kernels from the operator's arithmetic: they have to agree
+            if tuple(yi.shape) != tuple(shape):
+                raise UnsupportedModel(f"{what}: the file gives the output shape {yi.shape}, the operator produces {tuple(shape)}")
+
         if kind in ("CONV_2D", "DEPTHWISE_CONV_2D"):
             dw = kind == "DEPTHWISE_CONV_2D"
             w = need_constant(ins[1], "weights", kind)
             b = need_constant(ins[2], "bias", kind) if len(ins) > 2 and ins[2] >= 0 else None
             padding, sw, sh = o.scalar(0, "b"), o.scalar(1, "i"), o.scalar(2, "i")
-            act = _ACT[o.scalar(4 if dw else 3, "b")]
+            act = _fused(o.scalar(4 if dw else 3, "b"))
             dwf, dhf = o.scalar(5 if dw else 4, "i", 1), o.scalar(6 if dw else 5, "i", 1)
             _, h, wd, ci = xi.shape
             kh, kw = w.info.shape[1], w.info.shape[2]
             pt, _ = _pad(padding, h, kh, sh, dhf)
             pl, _ = _pad(padding, wd, kw, sw, dwf)
-            if dw and w.info.shape[0] != 1:
+            if len(xi.shape) != 4 or len(w.info.shape) != 4 or min(sw, sh, dwf, dhf) < 1:
+                raise UnsupportedModel(f"{kind}: needs 4-D tensors and positive strides and dilations")
+            if dw and (w.info.shape[0] != 1 or w.info.shape[3] % ci != 0):
                 raise UnsupportedModel("DEPTHWISE_CONV_2D weights must be [1, H, W, I * multiplier]")
+            if not dw and w.info.shape[3] != ci:
+                raise UnsupportedModel("CONV_2D weights must be [O, H, W, I]")
+            _, pb = _pad(padding, h, kh, sh, dhf)
+            _, pr = _pad(padding, wd, kw, sw, dwf)
+            expect((xi.shape[0], (h + pt + pb - (dhf * (kh - 1) + 1)) // sh + 1, (wd + pl + pr - (dwf * (kw - 1) + 1)) // sw + 1,
+                    w.info.shape[3] if dw else w.info.shape[0]))
             if b is not None:
                 b = _bias_like_reference(b, xi, w.info)
             taps = kh * kw if dw else kh * kw * ci
@@ -226,31 +258,47 @@ def parse(data: bytes, name: str = "tflite") -> Network:
                 x, xi = flat, tensors[flat]
             if b is not None:
                 b = _bias_like_reference(b, xi, w.info)
+            if len(w.info.shape) != 2 or xi.num_elements % kdim != 0:
+                raise UnsupportedModel("FULLY_CONNECTED: weights must be [outputs, K] with K dividing the input")
+            if yi.num_elements != xi.shape[0] * w.info.shape[0]:
+                expect((xi.shape[0], w.info.shape[0]))
             if len(yi.shape) != 2:
                 tensors[y] = yi = TensorInfo((xi.shape[0], w.info.shape[0]), yi.dtype, yi.scales, yi.offset)
             layers.append(Layer("fc", lname, (x,), y, w, b, dict(transpose_weights=True, _macs=kdim * w.info.shape[0]),
-                                _ACT[o.scalar(0, "b")] if o else _ACT[0]))
+                                _fused(o.scalar(0, "b")) if o else _fused(0)))
         elif kind in ("AVERAGE_POOL_2D", "MAX_POOL_2D"):
             padding, sw, sh, fw, fh = o.scalar(0, "b"), o.scalar(1, "i"), o.scalar(2, "i"), o.scalar(3, "i"), o.scalar(4, "i")
+            if len(xi.shape) != 4 or min(sw, sh, fw, fh) < 1:
+                raise UnsupportedModel(f"{kind}: needs a 4-D tensor and positive window and strides")
             _, h, wd, _ = xi.shape
             pt, pb = _pad(padding, h, fh, sh)
             pl, pr = _pad(padding, wd, fw, sw)
+            expect((xi.shape[0], (h + pt + pb - fh) // sh + 1, (wd + pl + pr - fw) // sw + 1, xi.shape[3]))
             params = dict(pool_type=0 if kind == "MAX_POOL_2D" else 1, pool_w=fw, pool_h=fh, stride_x=sw, stride_y=sh,
                           pad_left=pl, pad_right=pr, pad_top=pt, pad_bottom=pb, padding_method=1)
-            layers.append(Layer("pool", lname, (x,), y, params=params, act=_ACT[o.scalar(5, "b")]))
+            layers.append(Layer("pool", lname, (x,), y, params=params, act=_fused(o.scalar(5, "b"))))
         elif kind == "ADD":
             x1 = activation_tensor(ins[1])
             if tensors[x1].shape != xi.shape:
                 raise UnsupportedModel("ADD with broadcasting")
-            layers.append(Layer("add", lname, (x, x1), y, act=_ACT[o.scalar(0, "b")] if o else _ACT[0]))
+            expect(xi.shape)
+            layers.append(Layer("add", lname, (x, x1), y, act=_fused(o.scalar(0, "b")) if o else _fused(0)))
         elif kind == "PAD":
             p = need_constant(ins[1], "paddings", kind)
             pads = tuple((int(a), int(b)) for a, b in p.data.reshape(-1, 2))
+            if len(pads) != len(xi.shape) or len(pads) > 4 or any(a < 0 or b < 0 for a, b in pads):
+                raise UnsupportedModel("PAD: one non-negative (before, after) pair per dimension, at most 4 dimensions")
+            expect(tuple(d + a + b for d, (a, b) in zip(xi.shape, pads)))
             # TfLite pads with the real number 0, which is the zero point in the tensor's own code
             layers.append(Layer("pad", lname, (x,), y, params=dict(pad_list=pads, pad_value=float(xi.offset))))
         elif kind == "RESHAPE":
+            if yi.num_elements != xi.num_elements:
+                raise UnsupportedModel("RESHAPE: input and output differ in their number of elements")
             layers.append(Layer("reshape", lname, (x,), y))
         elif kind == "SOFTMAX":
+            expect(xi.shape)
+            if len(xi.shape) != 2:
+                raise UnsupportedModel("SOFTMAX: runs over the columns of a 2-D tensor")
             layers.append(Layer("softmax", lname, (x,), y, params=dict(beta=float(o.scalar(0, "f", 1.0)) if o else 1.0)))
     return Network(name, tname(int(inputs[0])), tname(int(outputs[0])), tensors, layers)
 

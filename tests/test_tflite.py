@@ -118,3 +118,43 @@ def test_port_and_reference_build_agree_on_the_models(port, reference, which):
     probs = a[net.output].data.astype(np.int64) - net.tensors[net.output].offset
     assert np.all(np.abs(probs.sum(axis=-1) - 256) <= 8)                     # a distribution over the 10 classes
     assert len(np.unique(a[net.output].data)) > 2
+
+
+def test_damaged_files_are_refused_not_misread():
+    """Truncations and overwritten offsets end in UnsupportedModel, never in another exception or a silently wrong net."""
+    data = open(os.path.join(GOLDEN, "mock_model.tflite"), "rb").read()
+    good = tflite.parse(data)
+    rng = np.random.default_rng(99)
+    refused = 0
+    for trial in range(300):
+        damaged = bytearray(data)
+        if trial % 3 == 0:
+            damaged = damaged[:int(rng.integers(8, len(data)))]
+        else:
+            at = int(rng.integers(8, 2200))            # tables, vtables and offsets live at the front of this file
+            damaged[at:at + 4] = rng.integers(0, 256, 4, dtype=np.uint8).tobytes()
+        try:
+            net = tflite.parse(bytes(damaged))
+        except tflite.UnsupportedModel:
+            refused += 1
+            continue
+        assert len(net.layers) <= len(good.layers) + 1            # still a network the reader understands
+    assert refused > 50
+
+
+def test_shapes_the_operator_cannot_produce_are_refused():
+    """Buffers are sized from the file, kernels from the operator: a PAD whose output tensor is smaller than input plus
+    padding, or a pooling output larger than the window arithmetic gives, must not reach the device."""
+    b = tw.ModelBuilder()
+    x = b.tensor("x", (1, 4, 4, 8), tw.UINT8, 0.1, 3)
+    pads = b.tensor("paddings", (4, 2), tw.INT32, data=np.array([[0, 0], [2, 2], [2, 2], [0, 0]], np.int32))
+    y = b.tensor("y", (1, 6, 6, 8), tw.UINT8, 0.1, 3)               # should be 8 x 8
+    b.op(tw.PAD, [x, pads], [y], tw.OPT_PAD, {})
+    with pytest.raises(tflite.UnsupportedModel, match="output shape"):
+        tflite.parse(b.finish([x], [y]))
+    b = tw.ModelBuilder()
+    x = b.tensor("x", (1, 8, 8, 4), tw.INT8, 0.1, 0)
+    y = b.tensor("y", (1, 5, 5, 4), tw.INT8, 0.1, 0)                # 2x2 stride 2 VALID gives 4 x 4
+    b.op(tw.MAX_POOL_2D, [x], [y], tw.OPT_POOL, {0: ("b", tw.VALID), 1: ("i", 2), 2: ("i", 2), 3: ("i", 2), 4: ("i", 2)})
+    with pytest.raises(tflite.UnsupportedModel, match="output shape"):
+        tflite.parse(b.finish([x], [y]))
