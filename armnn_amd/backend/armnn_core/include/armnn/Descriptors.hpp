@@ -66,6 +66,16 @@ struct Pooling2dDescriptor : BaseDescriptor
     DataLayout m_DataLayout = DataLayout::NCHW;
 };
 
+/// include/armnn/Descriptors.hpp:1172-1193: mean over the listed dimensions, which stay as extents of 1 if m_KeepDims
+struct MeanDescriptor : BaseDescriptor
+{
+    MeanDescriptor() = default;
+    MeanDescriptor(const std::vector<unsigned int>& axis, bool keepDims) : m_Axis(axis), m_KeepDims(keepDims) {}
+    bool operator==(const MeanDescriptor& rhs) const { return m_Axis == rhs.m_Axis && m_KeepDims == rhs.m_KeepDims; }
+    std::vector<unsigned int> m_Axis;
+    bool m_KeepDims = false;
+};
+
 /// include/armnn/Descriptors.hpp:1196-1229: one (before, after) pair per dimension; for quantized tensors m_PadValue
 /// is the stored code itself, not a real number to be quantized (workloads/Pad.cpp:77-84)
 struct PadDescriptor : BaseDescriptor

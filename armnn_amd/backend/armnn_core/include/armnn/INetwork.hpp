@@ -95,6 +95,7 @@ public:
     IConnectableLayer* AddFullyConnectedLayer(const FullyConnectedDescriptor& descriptor, const char* name = nullptr);
     IConnectableLayer* AddActivationLayer(const ActivationDescriptor& descriptor, const char* name = nullptr);
     IConnectableLayer* AddPooling2dLayer(const Pooling2dDescriptor& descriptor, const char* name = nullptr);
+    IConnectableLayer* AddMeanLayer(const MeanDescriptor& descriptor, const char* name = nullptr);
     IConnectableLayer* AddPadLayer(const PadDescriptor& descriptor, const char* name = nullptr);
     IConnectableLayer* AddSoftmaxLayer(const SoftmaxDescriptor& descriptor, const char* name = nullptr);
     IConnectableLayer* AddElementwiseBinaryLayer(const ElementwiseBinaryDescriptor& descriptor, const char* name = nullptr);

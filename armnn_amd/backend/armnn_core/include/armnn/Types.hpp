@@ -38,7 +38,7 @@ using MemorySourceFlags = unsigned int;
 // the layer kinds this core can hold (names as in include/armnn/Types.hpp:410-500)
 enum class LayerType
 {
-    Activation, Constant, Convolution2d, DepthwiseConvolution2d, ElementwiseBinary, FullyConnected, Input, MemCopy,
+    Activation, Constant, Convolution2d, DepthwiseConvolution2d, ElementwiseBinary, FullyConnected, Input, Mean, MemCopy,
     Output, Pad, Pooling2d, Reshape, Softmax
 };
 const char* GetLayerTypeAsCString(LayerType type);

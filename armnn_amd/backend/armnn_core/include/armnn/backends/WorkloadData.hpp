@@ -54,6 +54,7 @@ struct Convolution2dQueueDescriptor : QueueDescriptorWithParameters<Convolution2
 struct DepthwiseConvolution2dQueueDescriptor : QueueDescriptorWithParameters<DepthwiseConvolution2dDescriptor> { void Validate(const WorkloadInfo&) const; };
 struct FullyConnectedQueueDescriptor : QueueDescriptorWithParameters<FullyConnectedDescriptor> { void Validate(const WorkloadInfo&) const; };
 struct Pooling2dQueueDescriptor : QueueDescriptorWithParameters<Pooling2dDescriptor> { void Validate(const WorkloadInfo&) const; };
+struct MeanQueueDescriptor : QueueDescriptorWithParameters<MeanDescriptor> { void Validate(const WorkloadInfo&) const; };
 struct PadQueueDescriptor : QueueDescriptorWithParameters<PadDescriptor> { void Validate(const WorkloadInfo&) const; };
 struct SoftmaxQueueDescriptor : QueueDescriptorWithParameters<SoftmaxDescriptor> { void Validate(const WorkloadInfo&) const; };
 struct ElementwiseBinaryQueueDescriptor : QueueDescriptorWithParameters<ElementwiseBinaryDescriptor> { void Validate(const WorkloadInfo&) const; };

@@ -284,6 +284,20 @@ void Pooling2dQueueDescriptor::Validate(const WorkloadInfo& info) const
     ValidateTypesMatch(info.m_InputTensorInfos[0], info.m_OutputTensorInfos[0], name, "input", "output");
 }
 
+// WorkloadData.cpp:2439-2482
+void MeanQueueDescriptor::Validate(const WorkloadInfo& info) const
+{
+    const std::string name = "MeanQueueDescriptor";
+    ValidateNumInputsOutputs(info, name, 1, 1);
+    const TensorInfo& in = info.m_InputTensorInfos[0];
+    const TensorInfo& out = info.m_OutputTensorInfos[0];
+    ValidateTypesMatch(in, out, name, "input", "output");
+    const unsigned int rank = in.GetNumDimensions();
+    const unsigned int axes = static_cast<unsigned int>(m_Parameters.m_Axis.size());
+    const unsigned int expected = m_Parameters.m_KeepDims ? rank : m_Parameters.m_Axis.empty() ? 1u : (rank > axes ? rank - axes : 1u);
+    ValidateDims(out, name, expected, "output");
+}
+
 // WorkloadData.cpp:2484-2504
 void PadQueueDescriptor::Validate(const WorkloadInfo& info) const
 {

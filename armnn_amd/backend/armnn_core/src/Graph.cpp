@@ -203,6 +203,10 @@ IConnectableLayer* INetwork::AddPooling2dLayer(const Pooling2dDescriptor& d, con
 {
     return m_Graph->AddLayer(LayerType::Pooling2d, name, 1, 1, std::make_shared<Pooling2dDescriptor>(d));
 }
+IConnectableLayer* INetwork::AddMeanLayer(const MeanDescriptor& d, const char* name)
+{
+    return m_Graph->AddLayer(LayerType::Mean, name, 1, 1, std::make_shared<MeanDescriptor>(d));
+}
 IConnectableLayer* INetwork::AddPadLayer(const PadDescriptor& d, const char* name)
 {
     return m_Graph->AddLayer(LayerType::Pad, name, 1, 1, std::make_shared<PadDescriptor>(d));

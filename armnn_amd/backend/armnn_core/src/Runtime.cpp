@@ -270,6 +270,7 @@ private:
             case LayerType::FullyConnected: w = Make<FullyConnectedQueueDescriptor, FullyConnectedDescriptor>(l, slot); break;
             case LayerType::Activation: w = Make<ActivationQueueDescriptor, ActivationDescriptor>(l, slot); break;
             case LayerType::Pooling2d: w = Make<Pooling2dQueueDescriptor, Pooling2dDescriptor>(l, slot); break;
+            case LayerType::Mean: w = Make<MeanQueueDescriptor, MeanDescriptor>(l, slot); break;
             case LayerType::Pad: w = Make<PadQueueDescriptor, PadDescriptor>(l, slot); break;
             case LayerType::Softmax: w = Make<SoftmaxQueueDescriptor, SoftmaxDescriptor>(l, slot); break;
             case LayerType::ElementwiseBinary: w = Make<ElementwiseBinaryQueueDescriptor, ElementwiseBinaryDescriptor>(l, slot); break;

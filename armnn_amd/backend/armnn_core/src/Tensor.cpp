@@ -138,6 +138,7 @@ const char* GetLayerTypeAsCString(LayerType type)
         case LayerType::Output: return "Output";
         case LayerType::Pooling2d: return "Pooling2d";
         case LayerType::Reshape: return "Reshape";
+        case LayerType::Mean: return "Mean";
         case LayerType::Pad: return "Pad";
         case LayerType::Softmax: return "Softmax";
         default: return "Unknown";

@@ -3,7 +3,9 @@
 #include <armnn/TypesUtils.hpp>
 #include <armnn/utility/PolymorphicDowncast.hpp>
 
+#include <algorithm>
 #include <cmath>
+#include <vector>
 
 namespace armnn
 {
@@ -130,6 +132,22 @@ bool Mi355xLayerSupport::IsPooling2dSupported(const TensorInfo& input, const Ten
     return CheckActivations(input, output, reason);
 }
 
+bool Mi355xLayerSupport::IsMeanSupported(const TensorInfo& input, const TensorInfo& output, const MeanDescriptor& d,
+                                         Optional<std::string&> reason) const
+{
+    if (input.GetNumDimensions() != 4) return No(reason, "Mean runs on 4-D NHWC tensors");
+    std::vector<unsigned int> axes = d.m_Axis;
+    std::sort(axes.begin(), axes.end());
+    if (axes != std::vector<unsigned int>{1, 2}) return No(reason, "only the mean over height and width (axes 1 and 2) runs on the device");
+    const unsigned int n = input.GetShape()[0], c = input.GetShape()[3];
+    const bool shapeOk = d.m_KeepDims ? (output.GetNumDimensions() == 4 && output.GetShape()[0] == n && output.GetShape()[1] == 1 &&
+                                         output.GetShape()[2] == 1 && output.GetShape()[3] == c)
+                                      : (output.GetNumDimensions() == 2 && output.GetShape()[0] == n && output.GetShape()[1] == c);
+    if (!shapeOk) return No(reason, "output shape is not [N, 1, 1, C] (kept dimensions) or [N, C]");
+    if (input.GetShape()[1] == 0 || input.GetShape()[2] == 0) return No(reason, "empty feature map");
+    return CheckActivations(input, output, reason);
+}
+
 bool Mi355xLayerSupport::IsPadSupported(const TensorInfo& input, const TensorInfo& output, const PadDescriptor& d,
                                         Optional<std::string&> reason) const
 {
@@ -220,6 +238,9 @@ bool Mi355xLayerSupport::IsLayerSupported(const LayerType& type, const std::vect
         case LayerType::Pooling2d:
             need(2);
             return IsPooling2dSupported(infos[0], infos[1], *PolymorphicDowncast<const Pooling2dDescriptor*>(&descriptor), reason);
+        case LayerType::Mean:
+            need(2);
+            return IsMeanSupported(infos[0], infos[1], *PolymorphicDowncast<const MeanDescriptor*>(&descriptor), reason);
         case LayerType::Pad:
             need(2);
             return IsPadSupported(infos[0], infos[1], *PolymorphicDowncast<const PadDescriptor*>(&descriptor), reason);

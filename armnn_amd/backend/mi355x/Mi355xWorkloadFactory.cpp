@@ -46,6 +46,8 @@ std::unique_ptr<IWorkload> Mi355xWorkloadFactory::CreateWorkload(LayerType type,
             return std::make_unique<Mi355xActivationWorkload>(*PolymorphicDowncast<const ActivationQueueDescriptor*>(&descriptor), info);
         case LayerType::Pooling2d:
             return std::make_unique<Mi355xPooling2dWorkload>(*PolymorphicDowncast<const Pooling2dQueueDescriptor*>(&descriptor), info);
+        case LayerType::Mean:
+            return std::make_unique<Mi355xMeanWorkload>(*PolymorphicDowncast<const MeanQueueDescriptor*>(&descriptor), info);
         case LayerType::Pad:
             return std::make_unique<Mi355xPadWorkload>(*PolymorphicDowncast<const PadQueueDescriptor*>(&descriptor), info);
         case LayerType::Softmax:

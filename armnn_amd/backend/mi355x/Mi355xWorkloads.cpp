@@ -8,6 +8,7 @@
 #include <armnn/backends/TensorHandle.hpp>
 #include <armnn/utility/PolymorphicDowncast.hpp>
 
+#include <algorithm>
 #include <cstring>
 
 namespace armnn
@@ -357,6 +358,37 @@ void Mi355xPooling2dWorkload::Execute() const
     void* y = Out(m_Data.m_Outputs[0]);
     ForEachLane(in.GetShape()[0], [&](const Lane& l) {
         mi355x::Check(mi355x_pool2d_run(&d, in.GetShape()[0] / l.count, l.Of(x, in), l.Of(y, out), l.stream), "mi355x_pool2d_run");
+    });
+}
+
+// ---- Mean ------------------------------------------------------------------------------------------------------------
+Mi355xMeanWorkload::Mi355xMeanWorkload(const MeanQueueDescriptor& descriptor, const WorkloadInfo& info)
+    : Mi355xBaseWorkload<MeanQueueDescriptor>(descriptor, info), m_Info(info)
+{
+    ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xMeanWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
+    std::vector<unsigned int> axes = m_Data.m_Parameters.m_Axis;
+    std::sort(axes.begin(), axes.end());
+    if (m_Info.m_InputTensorInfos[0].GetNumDimensions() != 4 || axes != std::vector<unsigned int>{1, 2})
+        throw InvalidArgumentException("Mi355xMeanWorkload: the mean over height and width of a 4-D NHWC tensor only");
+}
+
+void Mi355xMeanWorkload::Execute() const
+{
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xMeanWorkload_Execute");
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    mi355x_pool2d_desc d{};
+    d.in_h = in.GetShape()[1]; d.in_w = in.GetShape()[2]; d.channels = in.GetShape()[3];
+    d.out_h = 1; d.out_w = 1;
+    d.pool_w = d.in_w; d.pool_h = d.in_h; d.stride_x = 1; d.stride_y = 1;
+    d.pool_type = 1;
+    d.padding_method = 1;
+    d.input = mi355x::ToQuant(in);
+    d.output = mi355x::ToQuant(out);
+    const void* x = In(m_Data.m_Inputs[0]);
+    void* y = Out(m_Data.m_Outputs[0]);
+    ForEachLane(in.GetShape()[0], [&](const Lane& l) {
+        mi355x::Check(mi355x_pool2d_run(&d, in.GetShape()[0] / l.count, l.Of(x, in), l.Of(y, out), l.stream), "mi355x_pool2d_run (mean)");
     });
 }
 

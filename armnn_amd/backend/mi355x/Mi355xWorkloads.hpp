@@ -98,6 +98,18 @@ private:
     WorkloadInfo m_Info;
 };
 
+/// counterpart of RefMeanWorkload (RefMeanWorkload.cpp:26-42) for the mean over height and width of an NHWC tensor: the
+/// float sum over the window in row order divided by the element count is what an average Pooling2d over the whole
+/// feature map computes, and that kernel is what runs
+class Mi355xMeanWorkload : public Mi355xBaseWorkload<MeanQueueDescriptor>
+{
+public:
+    Mi355xMeanWorkload(const MeanQueueDescriptor& descriptor, const WorkloadInfo& info);
+    void Execute() const override;
+private:
+    WorkloadInfo m_Info;
+};
+
 /// counterpart of RefPadWorkload (RefPadWorkload.cpp:18-40)
 class Mi355xPadWorkload : public Mi355xBaseWorkload<PadQueueDescriptor>
 {

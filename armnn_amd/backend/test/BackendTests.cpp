@@ -158,6 +158,14 @@ TEST_CASE("layer support: the accepted envelope and the reasons outside it", "cp
     sd.m_Axis = 0;
     CHECK(!ls.IsLayerSupported(LayerType::Softmax, {logits, probs}, sd, EmptyOptional(), EmptyOptional(), reason));
 
+    // Mean: over height and width only, kept dimensions or not
+    const TensorInfo meanIn = ActInfo({2, 7, 7, 64}, DataType::QAsymmS8, 0.05f, -3);
+    CHECK(ls.IsLayerSupported(LayerType::Mean, {meanIn, ActInfo({2, 1, 1, 64}, DataType::QAsymmS8, 0.05f, -3)}, MeanDescriptor({1, 2}, true), EmptyOptional(), EmptyOptional(), reason));
+    CHECK(ls.IsLayerSupported(LayerType::Mean, {meanIn, ActInfo({2, 64}, DataType::QAsymmS8, 0.04f, 5)}, MeanDescriptor({2, 1}, false), EmptyOptional(), EmptyOptional(), reason));
+    CHECK(!ls.IsLayerSupported(LayerType::Mean, {meanIn, ActInfo({2, 7, 7, 1}, DataType::QAsymmS8, 0.05f, -3)}, MeanDescriptor({3}, true), EmptyOptional(), EmptyOptional(), reason));
+    CHECK_MSG(why.find("height and width") != std::string::npos, why);
+    CHECK(!ls.IsLayerSupported(LayerType::Mean, {meanIn, ActInfo({2, 64, 1}, DataType::QAsymmS8, 0.05f, -3)}, MeanDescriptor({1, 2}, false), EmptyOptional(), EmptyOptional(), reason));
+
     // Pad: constant mode, ranks 1..4, the output shape must be the padded input shape
     PadDescriptor padDesc({{0, 0}, {1, 1}, {2, 0}, {0, 0}}, -3.0f);
     const TensorInfo padIn = ActInfo({1, 8, 8, 16}, DataType::QAsymmS8, 0.05f, -3), padOut = ActInfo({1, 10, 10, 16}, DataType::QAsymmS8, 0.05f, -3);
@@ -774,6 +782,32 @@ TEST_CASE("runtime: Pad runs on the device; folded into the layer behind it, it 
         for (size_t i = 0; i < got.size(); ++i)
             if (got[i] != apart[i] && !(algo == PoolingAlgorithm::Max && (i / c) % wo == 0)) ++differing;
         CHECK(differing == 0);
+    }
+}
+
+TEST_CASE("runtime: Mean over height and width gives the bytes of the global average pooling it runs as", "gpu")
+{
+    IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+    REQUIRE(rt->GetDeviceSpec().GetSupportedBackends().count(kMi355x) == 1);
+    for (bool keep : {true, false})
+    {
+        const TensorInfo in = ActInfo({16, 7, 5, 96}, DataType::QAsymmU8, 0.0235f, 3);
+        const TensorInfo out = keep ? ActInfo({16, 1, 1, 96}, DataType::QAsymmU8, 0.02f, 1) : ActInfo({16, 96}, DataType::QAsymmU8, 0.02f, 1);
+        INetworkPtr net = INetwork::Create();
+        IConnectableLayer* i = net->AddInputLayer(0, "input");
+        i->GetOutputSlot(0).SetTensorInfo(in);
+        IConnectableLayer* mean = net->AddMeanLayer(MeanDescriptor({1, 2}, keep), "mean");
+        i->GetOutputSlot(0).Connect(mean->GetInputSlot(0));
+        mean->GetOutputSlot(0).SetTensorInfo(out);
+        IConnectableLayer* o = net->AddOutputLayer(0, "output");
+        mean->GetOutputSlot(0).Connect(o->GetInputSlot(0));
+        const std::vector<uint8_t> x = RandomActivations(in, 321);
+        const std::vector<uint8_t> got = RunOnRuntime(*rt, *net, {kMi355x}, in, x, out, 2);
+        Pooling2dDescriptor whole;
+        whole.m_PoolType = PoolingAlgorithm::Average;
+        whole.m_PoolWidth = 5; whole.m_PoolHeight = 7; whole.m_StrideX = whole.m_StrideY = 1;
+        whole.m_DataLayout = DataLayout::NHWC;
+        CHECK(got == OraclePool(in, x, whole, ActInfo({16, 1, 1, 96}, DataType::QAsymmU8, 0.02f, 1)));
     }
 }
 

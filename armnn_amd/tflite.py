@@ -1,7 +1,7 @@
 """Reads a quantized .tflite model into a nets.Network, with the conventions of Arm NN's TfLite parser.
 
 Only what the device path runs is accepted: 8-bit quantized CONV_2D, DEPTHWISE_CONV_2D, FULLY_CONNECTED,
-AVERAGE_POOL_2D, MAX_POOL_2D, ADD, PAD, RESHAPE and SOFTMAX, one subgraph, one input, one output.  Anything else raises
+AVERAGE_POOL_2D, MAX_POOL_2D, ADD, PAD, MEAN (over height and width), RESHAPE and SOFTMAX, one subgraph, one input, one output.  Anything else raises
 ``UnsupportedModel`` naming the operator -- nothing is approximated or skipped.
 
 What is taken from the reference parser (src/armnnTfLiteParser/TfLiteParser.cpp):
@@ -12,6 +12,9 @@ What is taken from the reference parser (src/armnnTfLiteParser/TfLiteParser.cpp)
   * FULLY_CONNECTED flattens an input of more than two dimensions to [elements / K, K] first (ParseFullyConnected);
     TfLite keeps FC weights as [outputs, K], i.e. m_TransposeWeightMatrix = true;
   * convolution weights are [O, H, W, I] and depthwise weights [1, H, W, I * multiplier], as the reference keeps them;
+  * MEAN over the height and width of an NHWC tensor runs as an average pooling over the whole feature map: the
+    reference's Reduce (workloads/Reduce.cpp:69-173) adds the window up in the same order and divides by the same
+    count, and the two give the same bytes;
   * per-channel weights carry their scales along quantized_dimension; the int32 bias keeps the scale the file states.
 
 The file format is FlatBuffers; the few accessors needed are written out here (the schema is tensorflow/lite/schema/
@@ -83,7 +86,7 @@ class _Table:
 # ---- schema constants ------------------------------------------------------------------------------------------------------
 _UINT8, _INT32, _INT8 = 3, 2, 9                                   # TensorType
 _OPS = {0: "ADD", 1: "AVERAGE_POOL_2D", 3: "CONV_2D", 4: "DEPTHWISE_CONV_2D", 9: "FULLY_CONNECTED", 17: "MAX_POOL_2D",
-        22: "RESHAPE", 25: "SOFTMAX", 34: "PAD"}                  # BuiltinOperator
+        22: "RESHAPE", 25: "SOFTMAX", 34: "PAD", 40: "MEAN"}                  # BuiltinOperator
 _ACT = {0: (0, 0.0, 0.0), 1: (1, 0.0, 0.0), 2: (2, 1.0, -1.0), 3: (2, 6.0, 0.0)}    # NONE, RELU, RELU_N1_TO_1, RELU6
 _SAME, _VALID = 0, 1
 
@@ -291,6 +294,22 @@ def _parse(data: bytes, name: str) -> Network:
             expect(tuple(d + a + b for d, (a, b) in zip(xi.shape, pads)))
             # TfLite pads with the real number 0, which is the zero point in the tensor's own code
             layers.append(Layer("pad", lname, (x,), y, params=dict(pad_list=pads, pad_value=float(xi.offset))))
+        elif kind == "MEAN":
+            axes = sorted(int(v) % 4 for v in need_constant(ins[1], "axes", kind).data.ravel())
+            if len(xi.shape) != 4 or axes != [1, 2]:
+                raise UnsupportedModel("MEAN: only the mean over height and width of a 4-D tensor runs on the device")
+            n_, h, wd, c_ = xi.shape
+            keep = bool(o.scalar(0, "b")) if o else False                     # ReducerOptions.keep_dims
+            expect((n_, 1, 1, c_) if keep else (n_, c_))
+            pooled = y
+            if not keep:
+                pooled = f"{y}:pooled"
+                tensors[pooled] = TensorInfo((n_, 1, 1, c_), yi.dtype, yi.scales, yi.offset)
+            params = dict(pool_type=1, pool_w=wd, pool_h=h, stride_x=1, stride_y=1, pad_left=0, pad_right=0, pad_top=0, pad_bottom=0,
+                          padding_method=1)
+            layers.append(Layer("pool", lname, (x,), pooled, params=params))
+            if not keep:
+                layers.append(Layer("reshape", lname + ":squeeze", (pooled,), y))
         elif kind == "RESHAPE":
             if yi.num_elements != xi.num_elements:
                 raise UnsupportedModel("RESHAPE: input and output differ in their number of elements")

@@ -81,6 +81,8 @@ class Oracle:
         f("softmax", C.c_int, [TP, TP, C.c_float, C.c_int])
         f("add", C.c_int, [TP, TP, TP])
         f("pad", C.c_int, [TP, TP, C.POINTER(C.c_uint32), C.c_float])
+        if kind == "reference":
+            f("mean", C.c_int, [TP, TP, C.POINTER(C.c_uint32), C.c_uint32])
         f("last_error", C.c_char_p, [])
 
     def _fn(self, name, restype, argtypes):
@@ -187,6 +189,16 @@ class Oracle:
         sx, sy = self._t(x, keep), self._t(y, keep)
         before = (C.c_uint32 * len(pad_before))(*[int(v) for v in pad_before])
         self._check(self._pad(C.byref(sx), C.byref(sy), before, float(pad_value)))
+        return y
+
+    def mean(self, x: QTensor, out_info: TensorInfo, axes) -> QTensor:
+        """Mean over `axes` as the reference's Reduce computes it (reference build only; the restatement expresses the
+        spatial mean of an NHWC tensor as a global average pooling, which tests show to be the same bytes)."""
+        y = QTensor(out_info)
+        keep = []
+        sx, sy = self._t(x, keep), self._t(y, keep)
+        ax = (C.c_uint32 * len(axes))(*[int(a) for a in axes])
+        self._check(self._mean(C.byref(sx), C.byref(sy), ax, len(axes)))
         return y
 
     def add(self, a: QTensor, b: QTensor, out_info: TensorInfo) -> QTensor:

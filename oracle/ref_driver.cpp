@@ -20,6 +20,7 @@
 #include "Softmax.hpp"
 #include "ElementwiseFunction.hpp"
 #include "Pad.hpp"
+#include "Reduce.hpp"
 #include "Decoders.hpp"
 #include "Encoders.hpp"
 
@@ -218,6 +219,17 @@ int ref_pad(const orc_tensor* in, const orc_tensor* out, const uint32_t* pad_bef
         q.m_Parameters.m_PadValue = pad_value;
         BorrowedHandle ih(in->data, ii.GetShape()), oh(out->data, oi.GetShape());
         Pad(ii, oi, &ih, &oh, q);
+    });
+}
+
+// Mean over the given axes: RefMeanWorkload::Execute (workloads/RefMeanWorkload.cpp:26-42) -> Reduce(..., ReduceOperation::Mean)
+int ref_mean(const orc_tensor* in, const orc_tensor* out, const uint32_t* axes, uint32_t n_axes)
+{
+    return Guard([&] {
+        TensorInfo ii = ToInfo(in), oi = ToInfo(out);
+        auto dec = MakeDecoder<float>(ii, in->data);
+        auto enc = MakeEncoder<float>(oi, out->data);
+        Reduce(ii, oi, *dec, *enc, std::vector<uint32_t>(axes, axes + n_axes), ReduceOperation::Mean);
     });
 }
 

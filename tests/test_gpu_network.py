@@ -159,3 +159,12 @@ def test_tflite_model_with_pad_per_channel_weights_and_fused_activations(port):
     net = tflite.parse(written_model(), "written")
     _layerwise(port, net, 1)
     _layerwise(port, net, 6)
+
+
+@pytest.mark.parametrize("keep_dims", [True, False])
+def test_tflite_model_with_mean_over_height_and_width(port, keep_dims):
+    from armnn_amd import tflite
+    from tests.test_tflite import mean_model
+    net = tflite.parse(mean_model(keep_dims), "mean")
+    _layerwise(port, net, 1)
+    _layerwise(port, net, 16)

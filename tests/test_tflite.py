@@ -158,3 +158,50 @@ def test_shapes_the_operator_cannot_produce_are_refused():
     b.op(tw.MAX_POOL_2D, [x], [y], tw.OPT_POOL, {0: ("b", tw.VALID), 1: ("i", 2), 2: ("i", 2), 3: ("i", 2), 4: ("i", 2)})
     with pytest.raises(tflite.UnsupportedModel, match="output shape"):
         tflite.parse(b.finish([x], [y]))
+
+
+def mean_model(keep_dims):
+    """uint8: CONV_2D 1x1 (RELU6) -> MEAN over height and width -> FULLY_CONNECTED -> SOFTMAX, the tail of a ResNet."""
+    rng = np.random.default_rng(5)
+    b = tw.ModelBuilder()
+    x = b.tensor("input", (1, 7, 6, 16), tw.UINT8, 0.02, 120)
+    w = b.tensor("conv/w", (32, 1, 1, 16), tw.UINT8, 0.01, 128, rng.integers(60, 200, (32, 1, 1, 16)).astype(np.uint8))
+    bias = b.tensor("conv/b", (32,), tw.INT32, np.float32(0.02) * np.float32(0.01), 0, rng.integers(-200, 200, 32).astype(np.int32))
+    c = b.tensor("conv/out", (1, 7, 6, 32), tw.UINT8, 0.0235, 0)
+    b.op(tw.CONV_2D, [x, w, bias], [c], tw.OPT_CONV, {0: ("b", tw.VALID), 1: ("i", 1), 2: ("i", 1), 3: ("b", tw.ACT_RELU6)})
+    axes = b.tensor("axes", (2,), tw.INT32, data=np.array([1, 2], np.int32))
+    m = b.tensor("mean", (1, 1, 1, 32) if keep_dims else (1, 32), tw.UINT8, 0.02, 2)
+    b.op(tw.MEAN, [c, axes], [m], tw.OPT_REDUCER, {0: ("b", 1 if keep_dims else 0)})
+    wf = b.tensor("fc/w", (10, 32), tw.UINT8, 0.02, 128, rng.integers(60, 200, (10, 32)).astype(np.uint8))
+    bf = b.tensor("fc/b", (10,), tw.INT32, np.float32(0.02) * np.float32(0.02), 0, rng.integers(-50, 50, 10).astype(np.int32))
+    f = b.tensor("fc/out", (1, 10), tw.UINT8, 0.05, 100)
+    b.op(tw.FULLY_CONNECTED, [m, wf, bf], [f], tw.OPT_FC, {0: ("b", tw.ACT_NONE)})
+    y = b.tensor("probabilities", (1, 10), tw.UINT8, 1.0 / 256.0, 0)
+    b.op(tw.SOFTMAX, [f], [y], tw.OPT_SOFTMAX, {0: ("f", 1.0)})
+    return b.finish([x], [y])
+
+
+@pytest.mark.parametrize("keep_dims", [True, False])
+def test_mean_over_height_and_width_is_read_as_a_global_average_pooling(reference, port, keep_dims):
+    net = tflite.parse(mean_model(keep_dims), "mean")
+    ops = [l.op for l in net.layers]
+    assert ops == (["conv", "pool", "reshape", "fc", "softmax"] if keep_dims else ["conv", "pool", "reshape", "fc", "softmax"])
+    pool = net.layers[1]
+    assert pool.params["pool_type"] == 1 and (pool.params["pool_h"], pool.params["pool_w"]) == (7, 6)
+    # the pooling the reader substitutes gives the bytes of the reference's own Reduce
+    x = nets.synthetic_input(net, 3, seed=4)
+    vals = netref.run_network(port, net, x, keep=True)
+    conv_out = vals[net.layers[0].output]
+    pooled = vals[pool.output]
+    want = reference.mean(conv_out, pooled.info, [1, 2])
+    np.testing.assert_array_equal(pooled.data, want.data)
+
+
+def test_mean_over_other_axes_is_refused():
+    b = tw.ModelBuilder()
+    x = b.tensor("x", (1, 4, 4, 8), tw.UINT8, 0.1, 0)
+    axes = b.tensor("axes", (1,), tw.INT32, data=np.array([3], np.int32))
+    y = b.tensor("y", (1, 4, 4, 1), tw.UINT8, 0.1, 0)
+    b.op(tw.MEAN, [x, axes], [y], tw.OPT_REDUCER, {0: ("b", 1)})
+    with pytest.raises(tflite.UnsupportedModel, match="height and width"):
+        tflite.parse(b.finish([x], [y]))
