@@ -138,3 +138,17 @@ def test_pad_bit_exact(port, reference, cfg, dtype):
         # closed form: numpy's constant padding with the saturated, rounded code
         code = int(np.clip(np.sign(value) * np.floor(abs(value) + 0.5), lo, hi))
         np.testing.assert_array_equal(p, np.pad(x.data, pads, constant_values=code))
+
+
+@pytest.mark.parametrize("dtype", [DataType.QAsymmS8, DataType.QAsymmU8])
+@pytest.mark.parametrize("shape", [(2, 7, 7, 64), (3, 14, 14, 37), (1, 5, 3, 8), (2, 1, 1, 16), (1, 9, 9, 1024)])
+def test_mean_over_height_and_width_equals_global_average_pooling(port, reference, dtype, shape):
+    """What lets the device run the Mean layer on its pooling kernel: the reference's Reduce (Reduce.cpp:69-173) and an
+    average Pooling2d over the whole feature map give the same bytes, for any output quantization."""
+    lo = 0 if dtype == DataType.QAsymmU8 else -128
+    n, h, w, c = shape
+    x = QTensor(TensorInfo(shape, dtype, (0.05,), lo + 20), synth.uniform_int(100, shape, lo, lo + 255, np.int64))
+    for so, zo in ((0.05, lo + 3), (0.031, lo + 77), (0.2, lo + 250)):
+        oi = TensorInfo((n, 1, 1, c), dtype, (so,), zo)
+        pooled = port.pooling2d(x, oi, pool_type=cpuref.POOL_AVERAGE, pool_w=w, pool_h=h, stride_x=1, stride_y=1, padding_method=cpuref.PAD_EXCLUDE)
+        np.testing.assert_array_equal(pooled.data, reference.mean(x, oi, [1, 2]).data)
