@@ -98,6 +98,10 @@ class DeviceNetwork:
                 q0, q1, qo = shim._quant(xin[0]), shim._quant(xin[1]), shim._quant(yout)
                 self.steps.append((l, self._add_step(yout.num_elements, q0, q1, qo, l.act, xb[0].ptr, xb[1].ptr, yb.ptr)))
                 self._step_plans.append(None)
+            elif l.op == "activation":
+                qi, qo = shim._quant(xin[0]), shim._quant(yout)
+                self.steps.append((l, self._activation_step(yout.num_elements, qi, qo, l.act, xb[0].ptr, yb.ptr)))
+                self._step_plans.append(None)
             elif l.op == "pad":
                 self.steps.append((l, self._pad_step(xin[0], yout, l.params["pad_list"], l.params["pad_value"], xb[0].ptr, yb.ptr)))
                 self._step_plans.append(None)
@@ -156,6 +160,11 @@ class DeviceNetwork:
         return lambda s, lane=0, lanes=1: shim._chk(lib.mi355x_add_run(
             n // lanes, C.byref(q0), C.byref(q1), C.byref(qo), act[0], act[1], act[2], x0 + lane * (n // lanes),
             x1 + lane * (n // lanes), y + lane * (n // lanes), s))
+
+    def _activation_step(self, n, qi, qo, act, x, y):
+        lib = self.lib
+        return lambda s, lane=0, lanes=1: shim._chk(lib.mi355x_activation_run(
+            n // lanes, C.byref(qi), C.byref(qo), act[0], act[1], act[2], x + lane * (n // lanes), y + lane * (n // lanes), s))
 
     def _pad_step(self, xin, yout, pad_list, pad_value, x, y):
         lib = self.lib

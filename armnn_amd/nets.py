@@ -39,7 +39,7 @@ def same_padding(in_size, k, stride, dilation=1):
 
 @dataclass
 class Layer:
-    op: str                       # conv | depthwise | fc | pool | add | pad | softmax | reshape
+    op: str                       # conv | depthwise | fc | pool | add | pad | activation | softmax | reshape
     name: str
     inputs: Tuple[str, ...]
     output: str

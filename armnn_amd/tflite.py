@@ -1,7 +1,7 @@
 """Reads a quantized .tflite model into a nets.Network, with the conventions of Arm NN's TfLite parser.
 
 Only what the device path runs is accepted: 8-bit quantized CONV_2D, DEPTHWISE_CONV_2D, FULLY_CONNECTED,
-AVERAGE_POOL_2D, MAX_POOL_2D, ADD, PAD, MEAN (over height and width), RESHAPE and SOFTMAX, one subgraph, one input, one output.  Anything else raises
+AVERAGE_POOL_2D, MAX_POOL_2D, ADD, PAD, MEAN (over height and width), RELU, RELU_N1_TO_1, RELU6, RESHAPE and SOFTMAX, one subgraph, one input, one output.  Anything else raises
 ``UnsupportedModel`` naming the operator -- nothing is approximated or skipped.
 
 What is taken from the reference parser (src/armnnTfLiteParser/TfLiteParser.cpp):
@@ -86,7 +86,7 @@ class _Table:
 # ---- schema constants ------------------------------------------------------------------------------------------------------
 _UINT8, _INT32, _INT8 = 3, 2, 9                                   # TensorType
 _OPS = {0: "ADD", 1: "AVERAGE_POOL_2D", 3: "CONV_2D", 4: "DEPTHWISE_CONV_2D", 9: "FULLY_CONNECTED", 17: "MAX_POOL_2D",
-        22: "RESHAPE", 25: "SOFTMAX", 34: "PAD", 40: "MEAN"}                  # BuiltinOperator
+        19: "RELU", 20: "RELU_N1_TO_1", 21: "RELU6", 22: "RESHAPE", 25: "SOFTMAX", 34: "PAD", 40: "MEAN"}                  # BuiltinOperator
 _ACT = {0: (0, 0.0, 0.0), 1: (1, 0.0, 0.0), 2: (2, 1.0, -1.0), 3: (2, 6.0, 0.0)}    # NONE, RELU, RELU_N1_TO_1, RELU6
 _SAME, _VALID = 0, 1
 
@@ -310,6 +310,11 @@ def _parse(data: bytes, name: str) -> Network:
             layers.append(Layer("pool", lname, (x,), pooled, params=params))
             if not keep:
                 layers.append(Layer("reshape", lname + ":squeeze", (pooled,), y))
+        elif kind in ("RELU", "RELU_N1_TO_1", "RELU6"):
+            # an Activation layer of its own (ParseRelu / ParseReluN1To1 / ParseRelu6); it re-quantizes when the output
+            # tensor's quantization differs from the input's
+            expect(xi.shape)
+            layers.append(Layer("activation", lname, (x,), y, act=_fused({"RELU": 1, "RELU_N1_TO_1": 2, "RELU6": 3}[kind])))
         elif kind == "RESHAPE":
             if yi.num_elements != xi.num_elements:
                 raise UnsupportedModel("RESHAPE: input and output differ in their number of elements")

@@ -30,6 +30,8 @@ def run_network(orc: Oracle, net: Network, x: QTensor, keep: bool = False, fast:
             y = orc.pooling2d(ins[0], out_info, **l.params)
         elif l.op == "add":
             y = orc.add(ins[0], ins[1], out_info)
+        elif l.op == "activation":
+            y = orc.activation(ins[0], out_info, l.act[0], l.act[1], l.act[2])
         elif l.op == "pad":
             y = orc.pad(ins[0], out_info, [b for b, _ in l.params["pad_list"]], l.params["pad_value"])
         elif l.op == "softmax":
@@ -38,7 +40,7 @@ def run_network(orc: Oracle, net: Network, x: QTensor, keep: bool = False, fast:
             y = QTensor(out_info, ins[0].data.reshape(out_info.shape))
         else:
             raise ValueError(l.op)
-        if l.act[0]:
+        if l.act[0] and l.op != "activation":
             y = orc.activation(y, out_info, l.act[0], l.act[1], l.act[2])
         vals[l.output] = y
     return vals if keep else vals[net.output]

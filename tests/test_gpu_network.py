@@ -168,3 +168,11 @@ def test_tflite_model_with_mean_over_height_and_width(port, keep_dims):
     net = tflite.parse(mean_model(keep_dims), "mean")
     _layerwise(port, net, 1)
     _layerwise(port, net, 16)
+
+
+def test_tflite_model_with_standalone_activations(port):
+    from armnn_amd import tflite
+    from tests.test_tflite import relu_model
+    net = tflite.parse(relu_model(), "relu")
+    _layerwise(port, net, 1)
+    _layerwise(port, net, 32)

@@ -205,3 +205,31 @@ def test_mean_over_other_axes_is_refused():
     b.op(tw.MEAN, [x, axes], [y], tw.OPT_REDUCER, {0: ("b", 1)})
     with pytest.raises(tflite.UnsupportedModel, match="height and width"):
         tflite.parse(b.finish([x], [y]))
+
+
+def relu_model():
+    """int8: standalone RELU6 that re-quantizes, RELU_N1_TO_1 and RELU that keep the quantization, then SOFTMAX."""
+    b = tw.ModelBuilder()
+    x = b.tensor("input", (1, 48), tw.INT8, 0.1, -10)
+    a = b.tensor("relu6", (1, 48), tw.INT8, 6.0 / 255.0, -128)
+    b.op(tw.RELU6, [x], [a])
+    c = b.tensor("relu_n1_to_1", (1, 48), tw.INT8, 6.0 / 255.0, -128)
+    b.op(tw.RELU_N1_TO_1, [a], [c])
+    d = b.tensor("relu", (1, 48), tw.INT8, 0.01, -100)
+    b.op(tw.RELU, [c], [d])
+    y = b.tensor("probabilities", (1, 48), tw.INT8, 1.0 / 256.0, -128)
+    b.op(tw.SOFTMAX, [d], [y], tw.OPT_SOFTMAX, {0: ("f", 1.0)})
+    return b.finish([x], [y])
+
+
+def test_standalone_activations_become_layers_of_their_own(port, reference):
+    net = tflite.parse(relu_model(), "relu")
+    assert [l.op for l in net.layers] == ["activation", "activation", "activation", "softmax"]
+    assert [l.act for l in net.layers[:3]] == [(2, 6.0, 0.0), (2, 1.0, -1.0), (1, 0.0, 0.0)]
+    x = nets.synthetic_input(net, 5, seed=8)
+    a = netref.run_network(port, net, x, keep=True)
+    b = netref.run_network(reference, net, x, keep=True)
+    for name in a:
+        np.testing.assert_array_equal(a[name].data, b[name].data, err_msg=name)
+    first = a[net.layers[0].output].data
+    assert first.min() == -128 and first.max() == 127            # [0, 6] fills the re-quantized range
