@@ -5,6 +5,10 @@
 #include "IProfiler.hpp"
 #include "Tensor.hpp"
 #include "Types.hpp"
+#include "BackendId.hpp"
+#include "backends/ICustomAllocator.hpp"
+#include "backends/IMemoryOptimizerStrategy.hpp"
+#include <map>
 #include <memory>
 #include <string>
 #include <vector>
@@ -13,13 +17,19 @@ namespace armnn
 {
 struct INetworkProperties
 {
-    INetworkProperties(bool asyncEnabled = false, MemorySource inputSource = MemorySource::Undefined,
-                       MemorySource outputSource = MemorySource::Undefined, bool profilingEnabled = false)
-        : m_AsyncEnabled(asyncEnabled), m_InputSource(inputSource), m_OutputSource(outputSource), m_ProfilingEnabled(profilingEnabled) {}
-    const bool m_AsyncEnabled;
+    INetworkProperties(MemorySource inputSource, MemorySource outputSource, bool profilingEnabled = false,
+                       ProfilingDetailsMethod detailsMethod = ProfilingDetailsMethod::Undefined,
+                       bool externalMemoryManagementEnabled = false)
+        : m_ProfilingEnabled(profilingEnabled), m_OutputNetworkDetailsMethod(detailsMethod), m_InputSource(inputSource),
+          m_OutputSource(outputSource), m_ExternalMemoryManagementEnabled(externalMemoryManagementEnabled) {}
+    const bool m_ProfilingEnabled;
+    const ProfilingDetailsMethod m_OutputNetworkDetailsMethod;
     const MemorySource m_InputSource;
     const MemorySource m_OutputSource;
-    const bool m_ProfilingEnabled;
+    /// the runtime plans the memory of intermediate tensors itself (a strategy places them in buffers taken from the
+    /// backend's allocator) for every backend that lists the capability ExternallyManagedMemory
+    const bool m_ExternalMemoryManagementEnabled;
+    virtual ~INetworkProperties() {}
 };
 
 class IRuntime;
@@ -36,6 +46,10 @@ public:
         std::string m_DynamicBackendsPath;
         bool m_EnableGpuProfiling = false;
         std::vector<BackendOptions> m_BackendOptions;
+        /// per backend: the allocator the buffers of a caller-side memory plan come from (the backend must accept it)
+        std::map<BackendId, std::shared_ptr<ICustomAllocator>> m_CustomAllocatorMap;
+        /// per backend: the strategy that places tensors into those buffers (default: every tensor a buffer of its own)
+        std::map<BackendId, std::shared_ptr<IMemoryOptimizerStrategy>> m_MemoryOptimizerStrategyMap;
     };
 
     static IRuntime* CreateRaw(const CreationOptions& options);

@@ -34,6 +34,8 @@ enum class BinaryOperation { Add = 0, Div = 1, Maximum = 2, Minimum = 3, Mul = 4
 
 enum class MemorySource : uint32_t { Undefined = 0, Malloc = 1, DmaBuf = 2, DmaBufProtected = 4, Gralloc = 8 };
 using MemorySourceFlags = unsigned int;
+enum class MemBlockStrategyType { SingleAxisPacking = 0, MultiAxisPacking = 1 };
+enum class ProfilingDetailsMethod { Undefined = 0, DetailsWithEvents = 1, DetailsOnly = 2 };
 
 // the layer kinds this core can hold (names as in include/armnn/Types.hpp:410-500)
 enum class LayerType

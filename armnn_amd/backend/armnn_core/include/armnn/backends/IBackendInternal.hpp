@@ -1,6 +1,7 @@
 // Minimal host core: include/armnn/backends/IBackendInternal.hpp:75-208.
 #pragma once
 #include "IBackendContext.hpp"
+#include "ICustomAllocator.hpp"
 #include "ILayerSupport.hpp"
 #include "IMemoryManager.hpp"
 #include "ITensorHandleFactory.hpp"
@@ -100,6 +101,18 @@ public:
     }
     static constexpr BackendVersion GetApiVersion() { return BackendVersion(1, 0); }
     virtual BackendCapabilities GetCapabilities() const { return BackendCapabilities("IBackendInternal NullCapabilities"); }
+    /// the backend takes its memory from the caller's allocator from now on; false (with a reason) when it cannot
+    virtual bool UseCustomMemoryAllocator(std::shared_ptr<ICustomAllocator> allocator, armnn::Optional<std::string&> errMsg)
+    {
+        IgnoreUnused(allocator);
+        if (errMsg) errMsg.value() = "The backend " + GetId().Get() + " doesn't support using a custom allocator.";
+        return false;
+    }
+    /// the allocator a caller-side memory plan uses for this backend's tensors when the caller named none
+    virtual std::unique_ptr<ICustomAllocator> GetDefaultAllocator() const
+    {
+        throw armnn::Exception("GetDefaultAllocator: Function has not been implemented in backend.");
+    }
     virtual unsigned int GetNumberOfCacheFiles() const { return 0; }
 };
 using IBackendInternalUniquePtr = std::unique_ptr<IBackendInternal>;

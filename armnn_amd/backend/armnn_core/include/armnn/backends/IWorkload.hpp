@@ -1,6 +1,7 @@
 // Minimal host core: include/armnn/backends/IWorkload.hpp:14-43.
 #pragma once
 #include "ITensorHandle.hpp"
+#include "WorkloadInfo.hpp"
 #include <cstdint>
 #include <string>
 namespace arm { namespace pipe {
@@ -29,5 +30,6 @@ public:
     virtual void ReplaceInputTensorHandle(ITensorHandle*, unsigned int) = 0;
     virtual const std::string& GetName() const = 0;
     virtual void ReplaceOutputTensorHandle(ITensorHandle*, unsigned int) = 0;
+    virtual armnn::Optional<armnn::MemoryRequirements> GetMemoryRequirements() { return armnn::EmptyOptional(); }
 };
 } // namespace armnn

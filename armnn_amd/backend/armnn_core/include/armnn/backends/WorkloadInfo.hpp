@@ -15,4 +15,15 @@ struct WorkloadInfo
     Optional<TensorInfo> m_BiasTensorInfo = EmptyOptional();
     Optional<std::string> m_ConvolutionMethod = EmptyOptional();
 };
+/// scratch memory a workload needs besides its tensors, for a memory plan made outside the backend
+struct MemoryInfo
+{
+    unsigned int m_OutputSlotIndex;
+    size_t m_Size{0};
+    size_t m_Alignment{64};
+};
+struct MemoryRequirements
+{
+    Optional<std::vector<MemoryInfo>> m_IntraLayerTensors;
+};
 } // namespace armnn

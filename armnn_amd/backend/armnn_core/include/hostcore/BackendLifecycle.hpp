@@ -29,6 +29,13 @@ public:
     BackendIdSet GetBackendIds() const;
     std::string GetBackendIdsAsString() const;
     void Deregister(const BackendId& id);
+    /// allocators and memory optimizer strategies callers chose per backend (BackendRegistry.hpp:48-58)
+    void RegisterAllocator(const BackendId& id, std::shared_ptr<ICustomAllocator> alloc);
+    std::unordered_map<BackendId, std::shared_ptr<ICustomAllocator>> GetAllocators();
+    void DeregisterAllocator(const BackendId& id);
+    void RegisterMemoryOptimizerStrategy(const BackendId& id, std::shared_ptr<IMemoryOptimizerStrategy> strategy);
+    std::unordered_map<BackendId, std::shared_ptr<IMemoryOptimizerStrategy>> GetMemoryOptimizerStrategies();
+    void DeregisterMemoryOptimizerStrategy(const BackendId& id);
 
     BackendRegistry() {}
     virtual ~BackendRegistry() {}
@@ -44,6 +51,8 @@ private:
     BackendRegistry(const BackendRegistry&) = delete;
     BackendRegistry& operator=(const BackendRegistry&) = delete;
     std::unordered_map<BackendId, FactoryFunction> m_Factories;
+    std::unordered_map<BackendId, std::shared_ptr<ICustomAllocator>> m_CustomMemoryAllocatorMap;
+    std::unordered_map<BackendId, std::shared_ptr<IMemoryOptimizerStrategy>> m_MemoryOptimizerStrategyMap;
 };
 
 BackendRegistry& BackendRegistryInstance();

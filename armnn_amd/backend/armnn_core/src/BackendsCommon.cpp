@@ -69,6 +69,20 @@ std::string BackendRegistry::GetBackendIdsAsString() const
     return out + "]";
 }
 void BackendRegistry::Deregister(const BackendId& id) { m_Factories.erase(id); }
+void BackendRegistry::RegisterAllocator(const BackendId& id, std::shared_ptr<ICustomAllocator> alloc)
+{
+    if (m_CustomMemoryAllocatorMap.count(id)) throw InvalidArgumentException("Allocator for backend " + id.Get() + " already registered");
+    m_CustomMemoryAllocatorMap[id] = std::move(alloc);
+}
+std::unordered_map<BackendId, std::shared_ptr<ICustomAllocator>> BackendRegistry::GetAllocators() { return m_CustomMemoryAllocatorMap; }
+void BackendRegistry::DeregisterAllocator(const BackendId& id) { m_CustomMemoryAllocatorMap.erase(id); }
+void BackendRegistry::RegisterMemoryOptimizerStrategy(const BackendId& id, std::shared_ptr<IMemoryOptimizerStrategy> strategy)
+{
+    if (m_MemoryOptimizerStrategyMap.count(id)) throw InvalidArgumentException("Memory optimizer strategy for backend " + id.Get() + " already registered");
+    m_MemoryOptimizerStrategyMap[id] = std::move(strategy);
+}
+std::unordered_map<BackendId, std::shared_ptr<IMemoryOptimizerStrategy>> BackendRegistry::GetMemoryOptimizerStrategies() { return m_MemoryOptimizerStrategyMap; }
+void BackendRegistry::DeregisterMemoryOptimizerStrategy(const BackendId& id) { m_MemoryOptimizerStrategyMap.erase(id); }
 
 // ---- TensorHandleFactoryRegistry -----------------------------------------------------------------------------
 void TensorHandleFactoryRegistry::RegisterFactory(std::unique_ptr<ITensorHandleFactory> f)

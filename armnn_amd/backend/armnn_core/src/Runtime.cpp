@@ -32,6 +32,55 @@ struct BackendSlot
     IBackendInternalUniquePtr backend;
     IBackendInternal::IWorkloadFactoryPtr factory;
     ITensorHandleFactory* handleFactory = nullptr;   // preferred tensor handle factory, null: use the workload factory
+    bool external = false;                           // the runtime, not the backend, places this backend's tensors in memory
+};
+
+bool HasMatchingCapability(const BackendOptions::BackendOption& wanted, const BackendCapabilities& capabilities)
+{
+    for (size_t i = 0; i < capabilities.GetOptionCount(); ++i)
+    {
+        const auto& have = capabilities.GetOption(i);
+        if (have.GetName() != wanted.GetName()) continue;
+        if (wanted.GetValue().IsBool() && have.GetValue().IsBool()) return wanted.GetValue().AsBool() == have.GetValue().AsBool();
+        return false;
+    }
+    return false;
+}
+
+// every block a bin of its own, at offset 0 (ConstantMemoryStrategy,
+// src/backends/backendsCommon/memoryOptimizerStrategyLibrary/strategies/ConstantMemoryStrategy.cpp:22-38)
+class ConstantMemoryStrategy final : public IMemoryOptimizerStrategy
+{
+public:
+    std::string GetName() const override { return "ConstantMemoryStrategy"; }
+    MemBlockStrategyType GetMemBlockStrategyType() const override { return MemBlockStrategyType::SingleAxisPacking; }
+    std::vector<MemBin> Optimize(std::vector<MemBlock>& blocks) override
+    {
+        std::vector<MemBin> bins;
+        for (MemBlock& b : blocks)
+        {
+            b.m_Offset = 0;
+            MemBin bin;
+            bin.m_MemSize = b.m_MemSize;
+            bin.m_MemBlocks.push_back(b);
+            bins.push_back(std::move(bin));
+        }
+        return bins;
+    }
+};
+
+// the buffers of a memory plan and the tensors placed in them (src/backends/backendsCommon/MemoryManager.hpp:13-70)
+struct PlannedTensor
+{
+    ITensorHandle* handle = nullptr;
+    size_t offset = 0;
+};
+struct PlannedBuffer
+{
+    std::shared_ptr<ICustomAllocator> allocator;
+    size_t bytes = 0;
+    void* memory = nullptr;
+    std::vector<PlannedTensor> tensors;
 };
 
 // makes a profiler the calling thread's current one for a scope
@@ -47,8 +96,9 @@ private:
 class LoadedNetwork
 {
 public:
-    LoadedNetwork(IOptimizedNetworkPtr net, bool profilingEnabled = false) : m_Net(std::move(net)), m_Profiler(std::make_shared<IProfiler>())
+    LoadedNetwork(IOptimizedNetworkPtr net, const INetworkProperties& properties) : m_Net(std::move(net)), m_Profiler(std::make_shared<IProfiler>())
     {
+        const bool profilingEnabled = properties.m_ProfilingEnabled;
         // the network's profiler is the thread's current one while its workloads are built and run
         // (LoadedNetwork.cpp:131-136, :845-852)
         m_Profiler->EnableProfiling(profilingEnabled);
@@ -76,24 +126,52 @@ public:
                 slot.factory = slot.backend->CreateWorkloadFactory(mm, m_Net->GetModelOptions());
             }
             if (!slot.factory) throw RuntimeException("backend " + id.Get() + " returned no workload factory");
+            // LoadedNetwork.cpp:252-262
+            slot.external = properties.m_ExternalMemoryManagementEnabled &&
+                            HasMatchingCapability(BackendOptions::BackendOption{"ExternallyManagedMemory", true}, slot.backend->GetCapabilities());
             m_Backends.emplace(id, std::move(slot));
         }
 
         // Tensor handles in execution order.  Manage() opens a tensor's lifetime when its producer is reached and
         // Allocate() closes it after its last consumer, so a pooling memory manager can overlap tensors whose
-        // lifetimes do not (LoadedNetwork.cpp:262-330, Layer::CreateTensorHandles).  Constants and network inputs
-        // live for the whole network and are not managed.
+        // lifetimes do not (LoadedNetwork.cpp:262-330, Layer::CreateTensorHandles, Graph::AllocateDynamicBuffers).  The
+        // output of a Constant layer is created like the others but gets memory that lasts by an Allocate() without a
+        // lifetime (Graph.cpp:237-252).  Where the runtime plans the memory itself, the backend's tensors are created
+        // unmanaged, their lifetimes go into a memory profile (LoadedNetwork.cpp:1596-1718) and each is handed its place
+        // before the first inference.
         std::map<const OutputSlot*, unsigned int> remaining;
+        std::map<const OutputSlot*, size_t> blockOf;              // external tensors: index into `profile`
+        struct Lifetime { BackendId backend; ITensorHandle* handle; unsigned int start, end; size_t bytes; };
+        std::vector<Lifetime> profile;
+        unsigned int timestep = 0;
         for (Layer* l : m_Order)
         {
             BackendSlot& slot = m_Backends.at(l->GetBackendId());
-            const bool managed = l->GetType() != LayerType::Constant && l->GetType() != LayerType::Input;
+            const bool constant = l->GetType() == LayerType::Constant;
+            const bool external = slot.external && !constant;
+            const bool managed = !external;
             for (unsigned int o = 0; o < l->GetNumOutputSlots(); ++o)
             {
                 OutputSlot& out = l->Out(o);
                 std::unique_ptr<ITensorHandle> h = slot.handleFactory ? slot.handleFactory->CreateTensorHandle(out.GetTensorInfo(), managed)
                                                                       : slot.factory->CreateTensorHandle(out.GetTensorInfo(), managed);
                 if (!h) throw RuntimeException(std::string("no tensor handle for layer ") + l->GetName());
+                if (constant)
+                {
+                    h->Allocate();
+                    out.SetTensorHandle(std::move(h));
+                    remaining[&out] = ~0u;
+                    continue;
+                }
+                if (external)
+                {
+                    const size_t bytes = (out.GetTensorInfo().GetNumBytes() + 3) / 4 * 4;
+                    blockOf[&out] = profile.size();
+                    profile.push_back(Lifetime{l->GetBackendId(), h.get(), timestep, timestep, bytes});
+                    out.SetTensorHandle(std::move(h));
+                    remaining[&out] = ~0u;
+                    continue;
+                }
                 // a tensor read by a network output must survive until the caller has copied it out
                 bool pinned = !managed;
                 for (InputSlot* c : out.GetConnections()) pinned |= c->GetOwningLayer().GetType() == LayerType::Output;
@@ -106,12 +184,43 @@ public:
             for (unsigned int i = 0; i < l->GetNumInputSlots(); ++i)
             {
                 const OutputSlot* src = l->In(i).GetConnectedOutputSlot();
+                auto ext = blockOf.find(src);
+                // alive until its last consumer; what a network output reads, until the caller has copied it out
+                if (ext != blockOf.end())
+                    profile[ext->second].end = l->GetType() == LayerType::Output ? static_cast<unsigned int>(m_Order.size()) : std::max(profile[ext->second].end, timestep);
                 unsigned int& r = remaining[src];
                 if (r != ~0u && --r == 0) src->GetTensorHandle()->Allocate();
             }
+            ++timestep;
         }
         for (ITensorHandle* h : m_AllocateLast) h->Allocate();
         m_AllocateLast.clear();
+
+        // the memory plan: per backend, a strategy packs the blocks into bins; every bin becomes one buffer of the
+        // backend's allocator (LoadedNetwork.cpp:517-541 and :1722-1764)
+        {
+            std::map<BackendId, std::vector<MemBlock>> blocks;
+            for (size_t i = 0; i < profile.size(); ++i)
+                blocks[profile[i].backend].emplace_back(profile[i].start, profile[i].end, profile[i].bytes, 0, static_cast<unsigned int>(i));
+            auto strategies = BackendRegistryInstance().GetMemoryOptimizerStrategies();
+            auto allocators = BackendRegistryInstance().GetAllocators();
+            for (auto& perBackend : blocks)
+            {
+                const BackendId& id = perBackend.first;
+                ConstantMemoryStrategy constantStrategy;
+                IMemoryOptimizerStrategy* strategy = strategies.count(id) ? strategies[id].get() : &constantStrategy;
+                std::shared_ptr<ICustomAllocator> allocator = allocators.count(id) ? allocators[id]
+                                                                                   : std::shared_ptr<ICustomAllocator>(m_Backends.at(id).backend->GetDefaultAllocator());
+                for (const MemBin& bin : strategy->Optimize(perBackend.second))
+                {
+                    PlannedBuffer buffer;
+                    buffer.allocator = allocator;
+                    buffer.bytes = bin.m_MemSize;
+                    for (const MemBlock& b : bin.m_MemBlocks) buffer.tensors.push_back(PlannedTensor{profile.at(b.m_Index).handle, b.m_Offset});
+                    m_Plan.push_back(std::move(buffer));
+                }
+            }
+        }
 
         m_Registry.AquireMemory();
         for (auto& w : m_Constants) w->PostAllocationConfigure();
@@ -133,7 +242,15 @@ public:
         m_Constants.clear();
         m_Workloads.clear();
         m_Registry.ReleaseMemory();
+        // LoadedNetwork::FreeWorkingMemory, LoadedNetwork.cpp:1199-1225
+        for (PlannedBuffer& b : m_Plan)
+        {
+            for (PlannedTensor& t : b.tensors) t.handle->Unimport();
+            if (b.memory) b.allocator->free(b.memory);
+        }
     }
+
+    size_t GetNumPlannedBuffers() const { return m_Plan.size(); }
 
     const std::shared_ptr<IProfiler>& GetProfiler() const { return m_Profiler; }
 
@@ -166,6 +283,7 @@ public:
         std::lock_guard<std::mutex> lock(m_Mutex);
         CurrentProfiler current(m_Profiler.get());
         ARMNN_SCOPED_PROFILING_EVENT(BackendId(), "EnqueueWorkload");
+        AllocateWorkingMemory();
         for (ImportedInputId id : preIn)
             if (id >= m_Inputs.size() || !m_Inputs[id].adopted) throw InvalidArgumentException("EnqueueWorkload: input " + std::to_string(id) + " was not imported");
         for (ImportedOutputId id : preOut)
@@ -210,6 +328,20 @@ public:
     }
 
 private:
+    // the planned buffers come into being with the first inference; every tensor then adopts its place
+    // (LoadedNetwork::AllocateWorkingMemory, LoadedNetwork.cpp:1162-1197)
+    void AllocateWorkingMemory()
+    {
+        if (m_WorkingMemoryAllocated) return;
+        for (PlannedBuffer& b : m_Plan)
+        {
+            b.memory = b.allocator->allocate(b.bytes, 0);
+            for (PlannedTensor& t : b.tensors)
+                t.handle->Import(b.allocator->GetMemoryRegionAtOffset(b.memory, t.offset), b.allocator->GetMemorySourceType());
+        }
+        m_WorkingMemoryAllocated = true;
+    }
+
     template <typename Desc>
     void Fill(Desc& d, WorkloadInfo& info, Layer& l)
     {
@@ -409,6 +541,8 @@ private:
     std::vector<std::unique_ptr<IWorkload>> m_Constants;
     std::vector<std::unique_ptr<IWorkload>> m_Workloads;
     std::vector<ITensorHandle*> m_AllocateLast;
+    std::vector<PlannedBuffer> m_Plan;
+    bool m_WorkingMemoryAllocated = false;
     std::mutex m_Mutex;
 };
 } // namespace
@@ -428,6 +562,27 @@ public:
             {
                 auto backend = BackendRegistryInstance().GetFactory(id)();
                 auto context = backend->CreateBackendContext(options);
+                // a backend that cannot work with the allocator the caller chose for it is not used (Runtime.cpp:395-413)
+                auto allocator = options.m_CustomAllocatorMap.find(id);
+                if (allocator != options.m_CustomAllocatorMap.end())
+                {
+                    if (!allocator->second) throw Exception("Allocator associated with id " + id.Get() + " is null");
+                    std::string err;
+                    if (!backend->UseCustomMemoryAllocator(allocator->second, err))
+                    {
+                        std::cerr << "armnn: the backend " << id << " reported an error when trying to use the provided custom allocator."
+                                  << " Backend won't be used. ErrorMsg: " << err << "\n";
+                        continue;
+                    }
+                    BackendRegistryInstance().RegisterAllocator(id, allocator->second);
+                    m_AllocatorsAdded.insert(id);
+                }
+                auto strategy = options.m_MemoryOptimizerStrategyMap.find(id);
+                if (strategy != options.m_MemoryOptimizerStrategyMap.end() && strategy->second)
+                {
+                    BackendRegistryInstance().RegisterMemoryOptimizerStrategy(id, strategy->second);
+                    m_StrategiesAdded.insert(id);
+                }
                 if (context) m_Contexts.emplace(id, std::move(context));
                 m_DeviceSpec.m_Supported.insert(id);
             }
@@ -442,17 +597,20 @@ public:
     {
         m_Networks.clear();
         m_Contexts.clear();
+        for (const BackendId& id : m_AllocatorsAdded) BackendRegistryInstance().DeregisterAllocator(id);
+        for (const BackendId& id : m_StrategiesAdded) BackendRegistryInstance().DeregisterMemoryOptimizerStrategy(id);
         for (const BackendId& id : m_DeviceSpec.m_Dynamic) BackendRegistryInstance().Deregister(id);
     }
 
-    Status LoadNetwork(NetworkId& idOut, IOptimizedNetworkPtr network, std::string& error, bool profilingEnabled = false)
+    Status LoadNetwork(NetworkId& idOut, IOptimizedNetworkPtr network, std::string& error,
+                       const INetworkProperties& properties = INetworkProperties(MemorySource::Undefined, MemorySource::Undefined))
     {
         const NetworkId id = m_NextId++;
         idOut = id;
         for (auto& c : m_Contexts) c.second->BeforeLoadNetwork(id);
         try
         {
-            m_Networks[id] = std::make_unique<LoadedNetwork>(std::move(network), profilingEnabled);
+            m_Networks[id] = std::make_unique<LoadedNetwork>(std::move(network), properties);
         }
         catch (const Exception& e)
         {
@@ -502,6 +660,7 @@ public:
 private:
     std::map<BackendId, IBackendInternal::IBackendContextPtr> m_Contexts;
     std::map<NetworkId, std::unique_ptr<LoadedNetwork>> m_Networks;
+    BackendIdSet m_AllocatorsAdded, m_StrategiesAdded;
     NetworkId m_NextId = 0;
 };
 
@@ -518,7 +677,7 @@ Status IRuntime::LoadNetwork(NetworkId& id, IOptimizedNetworkPtr network)
 Status IRuntime::LoadNetwork(NetworkId& id, IOptimizedNetworkPtr network, std::string& error) { return pRuntimeImpl->LoadNetwork(id, std::move(network), error); }
 Status IRuntime::LoadNetwork(NetworkId& id, IOptimizedNetworkPtr network, std::string& error, const INetworkProperties& properties)
 {
-    return pRuntimeImpl->LoadNetwork(id, std::move(network), error, properties.m_ProfilingEnabled);
+    return pRuntimeImpl->LoadNetwork(id, std::move(network), error, properties);
 }
 const std::shared_ptr<IProfiler> IRuntime::GetProfiler(NetworkId id) const { return pRuntimeImpl->Get(id).GetProfiler(); }
 TensorInfo IRuntime::GetInputTensorInfo(NetworkId id, LayerBindingId layerId) const { return pRuntimeImpl->Get(id).GetInputTensorInfo(layerId); }

@@ -1,4 +1,5 @@
 #include "Mi355xBackend.hpp"
+#include "Mi355xDefaultAllocator.hpp"
 #include "Mi355xBackendId.hpp"
 #include "Mi355xDevice.hpp"
 #include "Mi355xLayerSupport.hpp"
@@ -159,6 +160,39 @@ void Mi355xBackend::RegisterTensorHandleFactories(TensorHandleFactoryRegistry& r
     registry.RegisterFactory(std::make_unique<Mi355xTensorHandleFactory>(memoryManager));
 }
 
+std::unique_ptr<ICustomAllocator> Mi355xBackend::GetDefaultAllocator() const
+{
+    return std::make_unique<Mi355xDefaultAllocator>();
+}
+
+bool Mi355xBackend::UseCustomMemoryAllocator(std::shared_ptr<ICustomAllocator> allocator, armnn::Optional<std::string&> errMsg)
+{
+    auto refuse = [&](const std::string& why)
+    {
+        if (errMsg) errMsg.value() = "Mi355x: " + why;
+        return false;
+    };
+    if (!allocator) return refuse("null allocator");
+    if (allocator->GetMemorySourceType() != MemorySource::Malloc) return refuse("only allocators of MemorySource::Malloc are supported");
+    if (mi355x::DeviceCount() == 0) return refuse("no device to check the allocator's memory against");
+    void* probe = nullptr;
+    try
+    {
+        mi355x::EnsureDevice();
+        probe = allocator->allocate(256, 16);
+    }
+    catch (const std::exception& e)
+    {
+        return refuse(std::string("the allocator's probe allocation failed: ") + e.what());
+    }
+    void* device = nullptr;
+    int isDevice = 0;
+    const bool reachable = probe && mi355x_host_device_pointer(probe, &device, &isDevice) == 0 && device != nullptr;
+    if (probe) allocator->free(probe);
+    if (!reachable) return refuse("the allocator returns memory the device cannot reach (pageable host memory); use device or pinned memory");
+    return true;
+}
+
 BackendCapabilities Mi355xBackend::GetCapabilities() const
 {
     return BackendCapabilities(Mi355xBackendId(), {{"NonConstWeights", false},
@@ -166,7 +200,7 @@ BackendCapabilities Mi355xBackend::GetCapabilities() const
                                                    {"ProtectedContentAllocation", false},
                                                    {"ConstantTensorsAsInputs", true},
                                                    {"PreImportIOTensors", true},
-                                                   {"ExternallyManagedMemory", false},
+                                                   {"ExternallyManagedMemory", true},
                                                    {"MultiAxisPacking", false},
                                                    {"SingleAxisPacking", false}});
 }

@@ -26,5 +26,11 @@ public:
     std::vector<ITensorHandleFactory::FactoryId> GetHandleFactoryPreferences() const override;
     void RegisterTensorHandleFactories(TensorHandleFactoryRegistry& registry) override;
     BackendCapabilities GetCapabilities() const override;
+    /// device memory for a memory plan made outside the backend (INetworkProperties::m_ExternalMemoryManagementEnabled)
+    std::unique_ptr<ICustomAllocator> GetDefaultAllocator() const override;
+    /// Accepts an allocator of MemorySource::Malloc whose memory the device reaches (device memory, or pinned host memory);
+    /// one probe allocation decides.  The runtime then takes the buffers of caller-side memory plans from it.  Weights and
+    /// other constants stay in memory the backend allocates itself.
+    bool UseCustomMemoryAllocator(std::shared_ptr<ICustomAllocator> allocator, armnn::Optional<std::string&> errMsg) override;
 };
 } // namespace armnn

@@ -1,7 +1,9 @@
 #include "Mi355xDevice.hpp"
 
 #include <atomic>
+#include <cstdint>
 #include <cstdlib>
+#include <map>
 #include <mutex>
 
 namespace armnn
@@ -87,9 +89,42 @@ void SetLanes(unsigned int lanes)
 
 void CountAddressSharingArena(int delta) { g_SharingArenas.fetch_add(delta); }
 
+namespace
+{
+std::mutex g_RangeMutex;
+std::multimap<uintptr_t, uintptr_t> g_Ranges;       // begin -> end of every adopted device range alive
+std::atomic<int> g_OverlappingRanges{0};
+}
+
+bool NoteAdoptedRange(const void* begin, size_t bytes)
+{
+    const uintptr_t b = reinterpret_cast<uintptr_t>(begin), e = b + (bytes ? bytes : 1);
+    std::lock_guard<std::mutex> lock(g_RangeMutex);
+    bool overlap = false;
+    for (const auto& r : g_Ranges)
+    {
+        if (r.first >= e) break;
+        if (r.second > b) { overlap = true; break; }
+    }
+    g_Ranges.emplace(b, e);
+    if (overlap) g_OverlappingRanges.fetch_add(1);
+    return overlap;
+}
+
+void ForgetAdoptedRange(const void* begin, size_t bytes, bool overlapped)
+{
+    const uintptr_t b = reinterpret_cast<uintptr_t>(begin), e = b + (bytes ? bytes : 1);
+    std::lock_guard<std::mutex> lock(g_RangeMutex);
+    auto range = g_Ranges.equal_range(b);
+    for (auto it = range.first; it != range.second; ++it)
+        if (it->second == e) { g_Ranges.erase(it); break; }
+    if (overlapped) g_OverlappingRanges.fetch_sub(1);
+}
+
 unsigned int LanesFor(unsigned int batch)
 {
     const unsigned int n = Lanes();
+    if (g_OverlappingRanges.load() != 0) return 1u;
     return (n > 1 && batch % n == 0 && batch / n >= kMinLaneBatch) ? n : 1u;
 }
 

@@ -40,10 +40,16 @@ unsigned int Lanes();
 void SetLanes(unsigned int lanes);
 /// memory managers that let tensors share addresses announce themselves here (+1 when created, -1 when destroyed)
 void CountAddressSharingArena(int delta);
+/// Device memory a tensor handle adopted announces its range here.  Two live ranges that overlap mean tensors share
+/// addresses (a caller's memory plan that reuses a buffer for tensors whose lifetimes do not meet): such tensors are only
+/// safe in launch order, so LanesFor() answers 1 while any overlap is alive.  NoteAdoptedRange returns true when the new
+/// range overlaps a live one; pass that to ForgetAdoptedRange when the handle lets go of the memory.
+bool NoteAdoptedRange(const void* begin, size_t bytes);
+void ForgetAdoptedRange(const void* begin, size_t bytes, bool overlapped);
 /// the smallest slice worth a lane of its own: a batch splits only into slices of at least this many images
 constexpr unsigned int kMinLaneBatch = 8;
 /// number of slices a workload over `batch` images should run as: Lanes() if that divides the batch into slices of at
-/// least kMinLaneBatch, else 1
+/// least kMinLaneBatch and no adopted ranges overlap, else 1
 unsigned int LanesFor(unsigned int batch);
 mi355x_stream_t LaneStream(unsigned int lane);
 void Fork();

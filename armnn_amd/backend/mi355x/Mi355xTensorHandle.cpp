@@ -15,6 +15,7 @@ Mi355xTensorHandle::Mi355xTensorHandle(const TensorInfo& info, std::shared_ptr<M
 
 Mi355xTensorHandle::~Mi355xTensorHandle()
 {
+    if (m_ImportedDevice && m_ImportedIsDeviceMemory) mi355x::ForgetAdoptedRange(m_ImportedDevice, m_Info.GetNumBytes(), m_ImportedOverlaps);
     if (m_Owned) mi355x_free(m_Owned);
     if (m_Staging) mi355x_host_free(m_Staging);
 }
@@ -29,9 +30,11 @@ void Mi355xTensorHandle::Manage()
 
 void Mi355xTensorHandle::Allocate()
 {
-    if (m_Managed)
+    // Allocate() without a lifetime opened by Manage() asks for memory that lasts: the runtime does that for the outputs
+    // of Constant layers (Graph::AllocateDynamicBuffers, src/armnn/Graph.cpp:237-252; RefTensorHandle::Allocate,
+    // src/backends/reference/RefTensorHandle.cpp:45-66, allocates directly in that case)
+    if (m_Managed && m_Reserved)
     {
-        if (!m_Reserved) throw InvalidArgumentException("Mi355xTensorHandle::Allocate() called before Manage()");
         if (m_Retired) throw InvalidArgumentException("Mi355xTensorHandle::Allocate() called twice");
         m_MemoryManager->Retire(m_Offset, m_Info.GetNumBytes());
         m_Retired = true;
@@ -63,7 +66,9 @@ bool Mi355xTensorHandle::Import(void* memory, MemorySource source)
     void* device = nullptr;
     int isDevice = 0;
     if (mi355x_host_device_pointer(memory, &device, &isDevice) != 0 || !device) return false;
+    if (m_ImportedDevice) Unimport();
     m_ImportedIsDeviceMemory = isDevice != 0;
+    m_ImportedOverlaps = m_ImportedIsDeviceMemory && mi355x::NoteAdoptedRange(device, m_Info.GetNumBytes());
     if (!m_Owned && !m_ImportedIsDeviceMemory) mi355x::Check(mi355x_malloc(&m_Owned, m_Info.GetNumBytes() ? m_Info.GetNumBytes() : 1), "mi355x_malloc");
     m_ImportedHost = memory;
     m_ImportedDevice = device;
@@ -75,6 +80,8 @@ bool Mi355xTensorHandle::Import(void* memory, MemorySource source)
 void Mi355xTensorHandle::Unimport()
 {
     if (m_ImportedDevice) mi355x::Synchronize();       // no kernel may still be using the caller's memory
+    if (m_ImportedDevice && m_ImportedIsDeviceMemory) mi355x::ForgetAdoptedRange(m_ImportedDevice, m_Info.GetNumBytes(), m_ImportedOverlaps);
+    m_ImportedOverlaps = false;
     m_ImportedHost = nullptr;
     m_ImportedDevice = nullptr;
     m_ImportedIsDeviceMemory = false;
@@ -104,11 +111,7 @@ unsigned int Mi355xTensorHandle::UploadLanes() const
 void* Mi355xTensorHandle::GetDevicePointer() const
 {
     if (m_ImportedDevice && m_ImportedIsDeviceMemory) return m_ImportedDevice;
-    if (m_Managed)
-    {
-        if (!m_Reserved) throw NullPointerException("Mi355xTensorHandle: managed tensor was never given a lifetime (Manage)");
-        return m_MemoryManager->Resolve(m_Offset);
-    }
+    if (m_Managed && m_Reserved) return m_MemoryManager->Resolve(m_Offset);
     if (!m_Owned) throw NullPointerException("Mi355xTensorHandle: tensor has no memory (Allocate was not called)");
     return m_Owned;
 }
@@ -117,7 +120,7 @@ TensorShape Mi355xTensorHandle::GetStrides() const { return GetUnpaddedTensorStr
 
 const void* Mi355xTensorHandle::Map(bool /*blocking*/) const
 {
-    if (m_ImportedDevice)
+    if (m_ImportedDevice && !m_ImportedIsDeviceMemory)
     {
         // results go straight into the caller's buffer; either way the host waits for what is queued
         if (m_MapCount++ == 0)
@@ -138,11 +141,22 @@ const void* Mi355xTensorHandle::Map(bool /*blocking*/) const
         mi355x::Synchronize();
         m_UploadInFlight = false;
     }
-    if (m_MapCount++ == 0 && m_DeviceNewer && bytes)
+    if (m_MapCount++ == 0)
     {
-        mi355x::Check(mi355x_memcpy_d2h(m_Staging, dev, bytes, mi355x::Stream()), "mi355x_memcpy_d2h");
-        mi355x::Synchronize();
-        m_DeviceNewer = false;
+        // A tensor has one producer.  If that is a kernel, the host maps the tensor to read it (a network output, a copy
+        // to another backend) and Unmap() has nothing to bring back; if it is the host, no kernel ever makes the device
+        // copy the newer one.
+        m_MappedToRead = m_DeviceNewer;
+        if (m_DeviceNewer && bytes)
+        {
+            mi355x::Check(mi355x_memcpy_d2h(m_Staging, dev, bytes, mi355x::Stream()), "mi355x_memcpy_d2h");
+            mi355x::Synchronize();
+            m_DeviceNewer = false;
+        }
+        else if (m_ImportedDevice)
+        {
+            mi355x::Synchronize();      // adopted device memory: mapping it is also how the runtime waits for the results
+        }
     }
     return m_Staging;
 }
@@ -151,9 +165,9 @@ void Mi355xTensorHandle::Unmap() const
 {
     if (m_MapCount == 0) return;
     if (--m_MapCount != 0) return;
-    if (m_ImportedDevice) return;
+    if (m_ImportedDevice && !m_ImportedIsDeviceMemory) return;
     const size_t bytes = m_Info.GetNumBytes();
-    if (!bytes) return;
+    if (!bytes || m_MappedToRead) return;
     // the pinned copy stays alive with the handle, so the upload may complete asynchronously in stream order
     mi355x::UploadInLanes(GetDevicePointer(), m_Staging, bytes, UploadLanes());
     m_UploadInFlight = true;

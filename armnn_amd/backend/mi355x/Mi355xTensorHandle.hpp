@@ -15,7 +15,10 @@
 // asynchronous transfer, and Map() brings results back into the buffer and waits -- no host-side memcpy on either side
 // (RefTensorHandle::Import, src/backends/reference/RefTensorHandle.cpp:135-165, is the host-memory counterpart).
 // Kernels do not read pinned host memory in place: a convolution reading its input across the bus proved slower than
-// the transfer.  Adopted device memory is used in place.
+// the transfer.  Adopted device memory is used in place: kernels read and write it, and Map() stages it through a pinned
+// copy like a tensor of the backend's own.  That is also how a caller-side memory plan reaches the backend: the runtime
+// creates every tensor unmanaged and hands each its place in a buffer from the backend's allocator
+// (LoadedNetwork.cpp:1176-1184 with ExternallyManagedMemory).
 #pragma once
 #include "Mi355xBackendId.hpp"
 #include "Mi355xMemoryManager.hpp"
@@ -67,6 +70,8 @@ private:
     void* m_ImportedHost = nullptr;     // caller memory adopted by Import(), as the caller addresses it ...
     void* m_ImportedDevice = nullptr;   // ... and as the device does
     bool m_ImportedIsDeviceMemory = false;   // adopted device memory is used in place, without transfers
+    bool m_ImportedOverlaps = false;         // ... and shares addresses with another adopted tensor
+    mutable bool m_MappedToRead = false;     // the current Map() downloaded the tensor: Unmap() has nothing to upload
     mutable void* m_Staging = nullptr;  // pinned host copy, created by the first Map()
     mutable bool m_DeviceNewer = false;
     mutable bool m_UploadInFlight = false;

@@ -19,6 +19,7 @@
 #include <Profiling.hpp>
 
 #include <chrono>
+#include <functional>
 #include <sstream>
 #include <thread>
 #include <cstring>
@@ -47,12 +48,14 @@ struct SingleLayerNet
 };
 
 std::vector<uint8_t> RunOnRuntime(IRuntime& rt, const INetwork& net, const std::vector<BackendId>& prefs, const TensorInfo& inInfo,
-                                  const std::vector<uint8_t>& input, const TensorInfo& outInfo, int repeats = 1)
+                                  const std::vector<uint8_t>& input, const TensorInfo& outInfo, int repeats = 1,
+                                  const INetworkProperties& properties = INetworkProperties(MemorySource::Undefined, MemorySource::Undefined),
+                                  const std::function<void()>& whileLoaded = nullptr)
 {
     IOptimizedNetworkPtr opt = Optimize(net, prefs, rt.GetDeviceSpec());
     NetworkId id = -1;
     std::string err;
-    if (rt.LoadNetwork(id, std::move(opt), err) != Status::Success) throw std::runtime_error("LoadNetwork failed: " + err);
+    if (rt.LoadNetwork(id, std::move(opt), err, properties) != Status::Success) throw std::runtime_error("LoadNetwork failed: " + err);
     std::vector<uint8_t> out(outInfo.GetNumBytes());
     TensorInfo constIn = inInfo;
     constIn.SetConstant(true);
@@ -63,6 +66,7 @@ std::vector<uint8_t> RunOnRuntime(IRuntime& rt, const INetwork& net, const std::
         OutputTensors outs{{0, Tensor(outInfo, out.data())}};
         if (rt.EnqueueWorkload(id, ins, outs) != Status::Success) throw std::runtime_error("EnqueueWorkload failed");
     }
+    if (whileLoaded) whileLoaded();
     rt.UnloadNetwork(id);
     return out;
 }
@@ -271,7 +275,6 @@ TEST_CASE("tensor handle: lifecycle errors are reported, not ignored", "cpu")
     const TensorInfo info = ActInfo({1, 4, 4, 8}, DataType::QAsymmS8, 0.1f, 0);
     Mi355xTensorHandle managed(info, mm, true);
     CHECK(managed.IsManaged());
-    CHECK_THROWS_AS(managed.Allocate(), InvalidArgumentException);          // before Manage()
     CHECK_THROWS_AS(managed.GetDevicePointer(), NullPointerException);
     managed.Manage();
     CHECK_THROWS_AS(managed.Manage(), InvalidArgumentException);
@@ -577,6 +580,148 @@ TEST_CASE("optimize: unsupported layers fall back along the preference list, wit
     FixedDeviceSpec none{};
     CHECK_THROWS_AS(Optimize(*net, {kMi355x}, none), InvalidArgumentException);
     CHECK_THROWS_AS(Optimize(*net, {}, both), InvalidArgumentException);
+}
+
+namespace
+{
+// Input -> identity x n -> Output on one backend
+INetworkPtr IdentityChain(const TensorInfo& info, int n)
+{
+    INetworkPtr net = INetwork::Create();
+    IConnectableLayer* input = net->AddInputLayer(0, "input");
+    input->GetOutputSlot(0).SetTensorInfo(info);
+    IOutputSlot* last = &input->GetOutputSlot(0);
+    for (int i = 0; i < n; ++i)
+    {
+        IConnectableLayer* l = net->AddActivationLayer(ActivationDescriptor(ActivationFunction::Linear, 1.0f, 0.0f), ("identity" + std::to_string(i)).c_str());
+        last->Connect(l->GetInputSlot(0));
+        l->GetOutputSlot(0).SetTensorInfo(info);
+        last = &l->GetOutputSlot(0);
+    }
+    IConnectableLayer* out = net->AddOutputLayer(0, "output");
+    last->Connect(out->GetInputSlot(0));
+    return net;
+}
+} // namespace
+
+TEST_CASE("memory plan: the runtime places the tensors of a backend that lets it, in buffers from that backend's allocator", "cpu")
+{
+    testhost::RegisterPlanned();
+    const BackendId planned = testhost::PlannedId();
+    const TensorInfo info = ActInfo({1, 5, 5, 10}, DataType::QAsymmS8, 0.05f, -3);     // 250 bytes -> blocks of 252
+    const std::vector<uint8_t> input = RandomActivations(info, 77);
+    const INetworkProperties external(MemorySource::Undefined, MemorySource::Undefined, false, ProfilingDetailsMethod::Undefined, true);
+    testhost::AllocatorLog& log = testhost::AllocatorLog::Default();
+
+    // not asked for: the backend's own tensors, no allocator call
+    {
+        log = testhost::AllocatorLog();
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        INetworkPtr net = IdentityChain(info, 3);
+        CHECK(RunOnRuntime(*rt, *net, {planned}, info, input, info, 2) == input);
+        CHECK(log.allocations == 0);
+    }
+    // asked for, no strategy named: every tensor (the input and the three layers' outputs) a buffer of its own, taken
+    // with the first inference and given back when the network goes
+    {
+        log = testhost::AllocatorLog();
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        INetworkPtr net = IdentityChain(info, 3);
+        IOptimizedNetworkPtr opt = Optimize(*net, {planned}, rt->GetDeviceSpec());
+        NetworkId id = -1;
+        std::string err;
+        REQUIRE(rt->LoadNetwork(id, std::move(opt), err, external) == Status::Success);
+        CHECK(log.allocations == 0);
+        std::vector<uint8_t> out(info.GetNumBytes());
+        TensorInfo constIn = info;
+        constIn.SetConstant(true);
+        for (int i = 0; i < 2; ++i)
+            CHECK(rt->EnqueueWorkload(id, {{0, ConstTensor(constIn, input.data())}}, {{0, Tensor(info, out.data())}}) == Status::Success);
+        CHECK(out == input);
+        CHECK(log.allocations == 4);
+        CHECK(log.bytes == 4 * 252u);
+        CHECK(log.frees == 0);
+        rt->UnloadNetwork(id);
+        CHECK(log.frees == 4);
+    }
+    // a strategy and an allocator of the caller's: one buffer; tensors whose lifetimes do not meet share addresses
+    {
+        log = testhost::AllocatorLog();
+        testhost::AllocatorLog mine;
+        IRuntime::CreationOptions options;
+        options.m_CustomAllocatorMap[planned] = std::make_shared<testhost::CountingAllocator>(mine);
+        options.m_MemoryOptimizerStrategyMap[planned] = std::make_shared<testhost::PackingStrategy>();
+        {
+            IRuntimePtr rt = IRuntime::Create(options);
+            INetworkPtr net = IdentityChain(info, 5);
+            CHECK(RunOnRuntime(*rt, *net, {planned}, info, input, info, 2, external) == input);
+            CHECK(log.allocations == 0);
+            CHECK(mine.allocations == 1);
+            CHECK(mine.frees == 1);
+            // input, then five outputs in a chain: two slots of 256 bytes alternate, and the network's output, alive to the
+            // end, needs no third one because it is the last tensor
+            CHECK(mine.bytes == 256u + 252u);
+        }
+        // the runtime took its registrations with it
+        CHECK(BackendRegistryInstance().GetAllocators().count(planned) == 0);
+        CHECK(BackendRegistryInstance().GetMemoryOptimizerStrategies().count(planned) == 0);
+    }
+    // an allocator the backend cannot work with: the backend is left out
+    {
+        testhost::AllocatorLog mine;
+        IRuntime::CreationOptions options;
+        options.m_CustomAllocatorMap[planned] = std::make_shared<testhost::CountingAllocator>(mine, MemorySource::DmaBuf);
+        IRuntimePtr rt = IRuntime::Create(options);
+        CHECK(rt->GetDeviceSpec().GetSupportedBackends().count(planned) == 0);
+        CHECK(BackendRegistryInstance().GetAllocators().count(planned) == 0);
+    }
+}
+
+TEST_CASE("memory plan: the backend lists the capability, hands out an allocator and refuses allocators it cannot check", "cpu")
+{
+    Mi355xBackend backend;
+    bool listed = false;
+    const BackendCapabilities caps = backend.GetCapabilities();
+    for (size_t i = 0; i < caps.GetOptionCount(); ++i)
+        if (caps.GetOption(i).GetName() == "ExternallyManagedMemory") listed = caps.GetOption(i).GetValue().AsBool();
+    CHECK(listed);
+    std::unique_ptr<ICustomAllocator> allocator = backend.GetDefaultAllocator();
+    REQUIRE(allocator != nullptr);
+    CHECK(allocator->GetMemorySourceType() == MemorySource::Malloc);
+    char buffer[8];
+    CHECK(allocator->GetMemoryRegionAtOffset(buffer, 5) == buffer + 5);
+    testhost::AllocatorLog log;
+    std::string why;
+    CHECK(!backend.UseCustomMemoryAllocator(nullptr, why));
+    CHECK(!backend.UseCustomMemoryAllocator(std::make_shared<testhost::CountingAllocator>(log, MemorySource::DmaBuf), why));
+    CHECK(why.find("Malloc") != std::string::npos);
+    if (mi355x::DeviceCount() == 0)
+    {
+        CHECK(!backend.UseCustomMemoryAllocator(std::make_shared<testhost::CountingAllocator>(log), why));
+        CHECK(why.find("no device") != std::string::npos);
+        CHECK(log.allocations == 0);
+    }
+    // adopted device ranges: an overlap turns the lanes off until the overlapping range goes
+    const unsigned int lanesBefore = mi355x::Lanes();
+    mi355x::SetLanes(2);
+    char* base = reinterpret_cast<char*>(uintptr_t(0x10000));
+    CHECK(mi355x::LanesFor(32) == 2);
+    const bool a = mi355x::NoteAdoptedRange(base, 1000);
+    const bool b = mi355x::NoteAdoptedRange(base + 1000, 1000);      // touching is not overlapping
+    CHECK(!a);
+    CHECK(!b);
+    CHECK(mi355x::LanesFor(32) == 2);
+    const bool c = mi355x::NoteAdoptedRange(base + 500, 100);
+    CHECK(c);
+    CHECK(mi355x::LanesFor(32) == 1);
+    mi355x::ForgetAdoptedRange(base + 500, 100, c);
+    CHECK(mi355x::LanesFor(32) == 2);
+    mi355x::ForgetAdoptedRange(base, 1000, a);
+    mi355x::ForgetAdoptedRange(base + 1000, 1000, b);
+    const bool d = mi355x::NoteAdoptedRange(base + 500, 100);        // nothing left to overlap with
+    CHECK(!d);
+    mi355x::ForgetAdoptedRange(base + 500, 100, d);
+    mi355x::SetLanes(lanesBefore);
 }
 
 TEST_CASE("runtime: importing is refused politely where a backend cannot adopt memory, and loudly when misused", "cpu")
@@ -973,7 +1118,7 @@ TEST_CASE("profiling: every workload of a profiled network reports its device ti
     IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, rt->GetDeviceSpec());
     NetworkId id = -1;
     std::string err;
-    REQUIRE(rt->LoadNetwork(id, std::move(opt), err, INetworkProperties(false, MemorySource::Undefined, MemorySource::Undefined, true)) == Status::Success);
+    REQUIRE(rt->LoadNetwork(id, std::move(opt), err, INetworkProperties(MemorySource::Undefined, MemorySource::Undefined, true)) == Status::Success);
     const std::shared_ptr<IProfiler> profiler = rt->GetProfiler(id);
     REQUIRE(profiler != nullptr);
     CHECK(profiler->IsProfilingEnabled());
@@ -1208,6 +1353,95 @@ TEST_CASE("runtime: intermediate tensors share an arena smaller than their sum",
         CHECK(dynamic_cast<Mi355xTensorHandle*>(handles[0].get())->GetDevicePointer() != nullptr);
         registry.ReleaseMemory();
         (void)factory;
+    }
+    mi355x::SetLanes(lanesBefore);
+}
+
+namespace
+{
+// pinned host memory: the device reaches it, so the backend accepts the allocator
+class PinnedAllocator : public ICustomAllocator
+{
+public:
+    void* allocate(size_t size, size_t) override
+    {
+        void* p = nullptr;
+        mi355x::Check(mi355x_host_alloc(&p, size ? size : 1), "mi355x_host_alloc");
+        ++allocations;
+        return p;
+    }
+    void free(void* p) override { mi355x::Synchronize(); mi355x_host_free(p); ++frees; }
+    MemorySource GetMemorySourceType() override { return MemorySource::Malloc; }
+    void* GetMemoryRegionAtOffset(void* buffer, size_t offset, size_t = 0) override { return static_cast<char*>(buffer) + offset; }
+    int allocations = 0, frees = 0;
+};
+} // namespace
+
+TEST_CASE("memory plan: tensors placed by the runtime give the same bytes; lanes run only while no two of them share addresses", "gpu")
+{
+    const unsigned int lanesBefore = mi355x::Lanes();
+    mi355x::SetLanes(2);
+    MiniMobileNet m(32, DataType::QAsymmS8);
+    const std::vector<uint8_t> input = RandomActivations(m.in, 321);
+    const std::vector<uint8_t> want = m.RunDirect(input);
+    const INetworkProperties external(MemorySource::Undefined, MemorySource::Undefined, false, ProfilingDetailsMethod::Undefined, true);
+
+    // the backend's allocator, every tensor a buffer of its own
+    {
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        INetworkPtr net = m.Build();
+        unsigned int lanesWhile = 0;
+        CHECK(RunOnRuntime(*rt, *net, {kMi355x}, m.in, input, m.probs, 3, external, [&] { lanesWhile = mi355x::LanesFor(32); }) == want);
+        CHECK(lanesWhile == 2);
+    }
+    // a strategy that lets tensors share addresses: the same bytes, on one stream
+    {
+        IRuntime::CreationOptions options;
+        options.m_MemoryOptimizerStrategyMap[kMi355x] = std::make_shared<testhost::PackingStrategy>();
+        IRuntimePtr rt = IRuntime::Create(options);
+        INetworkPtr net = m.Build();
+        unsigned int lanesWhile = 0;
+        CHECK(RunOnRuntime(*rt, *net, {kMi355x}, m.in, input, m.probs, 3, external, [&] { lanesWhile = mi355x::LanesFor(32); }) == want);
+        CHECK(lanesWhile == 1);
+        CHECK(mi355x::LanesFor(32) == 2);          // the network is gone, and its ranges with it
+    }
+    // the caller's allocator, pinned memory: accepted; tensors keep a device copy of their own
+    {
+        auto pinned = std::make_shared<PinnedAllocator>();
+        IRuntime::CreationOptions options;
+        options.m_CustomAllocatorMap[kMi355x] = pinned;
+        options.m_MemoryOptimizerStrategyMap[kMi355x] = std::make_shared<testhost::PackingStrategy>();
+        {
+            IRuntimePtr rt = IRuntime::Create(options);
+            REQUIRE(rt->GetDeviceSpec().GetSupportedBackends().count(kMi355x) == 1);
+            const int probes = pinned->allocations;
+            CHECK(probes == 1);
+            CHECK(pinned->frees == 1);
+            INetworkPtr net = m.Build();
+            unsigned int lanesWhile = 0;
+            CHECK(RunOnRuntime(*rt, *net, {kMi355x}, m.in, input, m.probs, 3, external, [&] { lanesWhile = mi355x::LanesFor(32); }) == want);
+            CHECK(lanesWhile == 2);
+            CHECK(pinned->allocations == probes + 1);
+            CHECK(pinned->frees == pinned->allocations);
+        }
+    }
+    // pageable memory: refused, and the backend is not offered
+    {
+        testhost::AllocatorLog log;
+        IRuntime::CreationOptions options;
+        options.m_CustomAllocatorMap[kMi355x] = std::make_shared<testhost::CountingAllocator>(log);
+        IRuntimePtr rt = IRuntime::Create(options);
+        CHECK(rt->GetDeviceSpec().GetSupportedBackends().count(kMi355x) == 0);
+        CHECK(log.allocations == 1);
+        CHECK(log.frees == 1);
+    }
+    // Allocate() without a lifetime, as the runtime does for the output of a Constant layer: memory of the tensor's own
+    {
+        auto mm = std::make_shared<Mi355xMemoryManager>(false);
+        Mi355xTensorHandle constant(ActInfo({1, 4, 4, 8}, DataType::QAsymmS8, 0.1f, 0), mm, true);
+        constant.Allocate();
+        CHECK(constant.GetDevicePointer() != nullptr);
+        CHECK_THROWS_AS(constant.Allocate(), InvalidArgumentException);
     }
     mi355x::SetLanes(lanesBefore);
 }

@@ -25,7 +25,17 @@ public:
     void Manage() override {}
     void Allocate() override { m_Data.resize(m_Info.GetNumBytes()); }
     ITensorHandle* GetParent() const override { return nullptr; }
-    const void* Map(bool) const override { if (m_Data.empty()) m_Data.resize(m_Info.GetNumBytes()); return m_Data.data(); }
+    const void* Map(bool) const override
+    {
+        if (m_Adopted) return m_Adopted;
+        if (m_Data.empty()) m_Data.resize(m_Info.GetNumBytes());
+        return m_Data.data();
+    }
+    unsigned int GetImportFlags() const override { return static_cast<unsigned int>(MemorySource::Malloc); }
+    bool CanBeImported(void* memory, MemorySource source) override { return memory && source == MemorySource::Malloc; }
+    bool Import(void* memory, MemorySource source) override { if (!CanBeImported(memory, source)) return false; m_Adopted = memory; return true; }
+    void Unimport() override { m_Adopted = nullptr; }
+    void* Adopted() const { return m_Adopted; }
     void Unmap() const override {}
     TensorShape GetStrides() const override { return GetUnpaddedTensorStrides(m_Info); }
     TensorShape GetShape() const override { return m_Info.GetShape(); }
@@ -34,6 +44,7 @@ public:
 private:
     TensorInfo m_Info;
     mutable std::vector<unsigned char> m_Data;
+    void* m_Adopted = nullptr;
 };
 
 class CopyActivationWorkload : public BaseWorkload<ActivationQueueDescriptor>
@@ -113,6 +124,85 @@ public:
     IWorkloadFactoryPtr CreateWorkloadFactory(const IMemoryManagerSharedPtr&) const override { return std::make_unique<Factory>(); }
     ILayerSupportSharedPtr GetLayerSupport() const override { static ILayerSupportSharedPtr s{new Support}; return s; }
 };
+
+// The same backend under a second id, with the capability that lets the runtime plan its tensors' memory; its default
+// allocator counts what it hands out.
+inline const BackendId& PlannedId() { static const BackendId id("TestHostPlanned"); return id; }
+struct AllocatorLog
+{
+    int allocations = 0, frees = 0;
+    size_t bytes = 0;
+    static AllocatorLog& Default() { static AllocatorLog log; return log; }
+};
+class CountingAllocator : public ICustomAllocator
+{
+public:
+    explicit CountingAllocator(AllocatorLog& log, MemorySource source = MemorySource::Malloc) : m_Log(log), m_Source(source) {}
+    void* allocate(size_t size, size_t) override { ++m_Log.allocations; m_Log.bytes += size; return ::operator new(size ? size : 1); }
+    void free(void* p) override { ++m_Log.frees; ::operator delete(p); }
+    MemorySource GetMemorySourceType() override { return m_Source; }
+    void* GetMemoryRegionAtOffset(void* buffer, size_t offset, size_t = 0) override { return static_cast<char*>(buffer) + offset; }
+private:
+    AllocatorLog& m_Log;
+    MemorySource m_Source;
+};
+class PlannedFactory : public Factory
+{
+public:
+    const BackendId& GetBackendId() const override { return PlannedId(); }
+};
+class PlannedBackend : public Backend
+{
+public:
+    const BackendId& GetId() const override { return PlannedId(); }
+    IWorkloadFactoryPtr CreateWorkloadFactory(const IMemoryManagerSharedPtr&) const override { return std::make_unique<PlannedFactory>(); }
+    BackendCapabilities GetCapabilities() const override { return BackendCapabilities(PlannedId(), {{"ExternallyManagedMemory", true}}); }
+    std::unique_ptr<ICustomAllocator> GetDefaultAllocator() const override { return std::make_unique<CountingAllocator>(AllocatorLog::Default()); }
+    bool UseCustomMemoryAllocator(std::shared_ptr<ICustomAllocator> allocator, armnn::Optional<std::string&> err) override
+    {
+        if (allocator->GetMemorySourceType() == MemorySource::Malloc) return true;
+        if (err) err.value() = "TestHostPlanned: only MemorySource::Malloc";
+        return false;
+    }
+};
+
+// Packs blocks into one bin: each block goes to the lowest 256-byte aligned offset where it meets no block placed
+// before it whose lifetime overlaps its own.
+class PackingStrategy : public IMemoryOptimizerStrategy
+{
+public:
+    std::string GetName() const override { return "TestPacking"; }
+    MemBlockStrategyType GetMemBlockStrategyType() const override { return MemBlockStrategyType::SingleAxisPacking; }
+    std::vector<MemBin> Optimize(std::vector<MemBlock>& blocks) override
+    {
+        MemBin bin;
+        bin.m_MemSize = 0;
+        for (MemBlock& b : blocks)
+        {
+            size_t offset = 0;
+            for (bool moved = true; moved;)
+            {
+                moved = false;
+                for (const MemBlock& placed : bin.m_MemBlocks)
+                {
+                    const bool alive = placed.m_StartOfLife <= b.m_EndOfLife && b.m_StartOfLife <= placed.m_EndOfLife;
+                    const bool meets = placed.m_Offset < offset + b.m_MemSize && offset < placed.m_Offset + placed.m_MemSize;
+                    if (alive && meets) { offset = (placed.m_Offset + placed.m_MemSize + 255) / 256 * 256; moved = true; }
+                }
+            }
+            b.m_Offset = offset;
+            bin.m_MemBlocks.push_back(b);
+            bin.m_MemSize = std::max(bin.m_MemSize, offset + b.m_MemSize);
+        }
+        return {bin};
+    }
+};
+
+inline void RegisterPlanned()
+{
+    if (!BackendRegistryInstance().IsBackendRegistered(PlannedId()))
+        BackendRegistryInstance().Register(PlannedId(), [] { return IBackendInternalUniquePtr(new PlannedBackend); });
+}
 
 inline void Register()
 {
