@@ -39,6 +39,7 @@ struct mi355x_conv2d_s
     bool bk128 = false;            // implicit GEMM walks K in 128-byte tiles
     int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 96 (= 128x64) / 128: the "igemm_tile" option at plan creation
     uint32_t xor_mask = 0, pad_word = 0;
+    int zw_neg = 0;                // MFMA plans: minus the zero point of the stored int8 weights (0: symmetric)
     std::string info;
 
     ~mi355x_conv2d_s()
@@ -194,7 +195,9 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
 
     // ---- kernel selection ----------------------------------------------------------------------------------
     const int zx_shift = g.in_u8 ? g.zx - 128 : g.zx;
-    const bool mfma_ok = !d.depthwise && g.zw == 0 && !g.w_u8 && (Ci % 16) == 0 && zx_shift >= -128 && zx_shift <= 127 &&
+    // weights as the MFMA kernels store them: int8, uint8 shifted by 128 like the activations; their zero point likewise
+    const int zw_shift = g.w_u8 ? g.zw - 128 : g.zw;
+    const bool mfma_ok = !d.depthwise && zw_shift >= -128 && zw_shift <= 127 && (Ci % 16) == 0 && zx_shift >= -128 && zx_shift <= 127 &&
                          p->K <= 100000;
     const bool dw_ok = d.depthwise && g.depth_mult == 1 && (Co % 4) == 0;
     const bool sym_s8 = g.zw == 0 && !g.w_u8 && zx_shift >= -128 && zx_shift <= 127;
@@ -214,7 +217,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         return SetError(MI355X_ERR_UNSUPPORTED, "dot4 kernel needs <= 4 input channels, symmetric int8 weights, stride 1 or 2, "
                                                 "no dilation and a 1/3/5/7-row filter");
     if (algo == MI355X_ALGO_MFMA && !mfma_ok)
-        return SetError(MI355X_ERR_UNSUPPORTED, "MFMA kernel needs a non-depthwise layer, symmetric int8 weights and in_c %% 16 == 0");
+        return SetError(MI355X_ERR_UNSUPPORTED, "MFMA kernel needs a non-depthwise layer and in_c %% 16 == 0");
     if (algo == MI355X_ALGO_DEPTHWISE && !dw_ok)
         return SetError(MI355X_ERR_UNSUPPORTED, "depthwise kernel needs multiplier 1 and channels %% 4 == 0");
     if (algo < MI355X_ALGO_DIRECT || algo > MI355X_ALGO_DOT4) return SetError(MI355X_ERR_INVALID_ARGUMENT, "unknown algo %d", algo);
@@ -230,9 +233,16 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             long long sum = 0;
             const int8_t* src = reinterpret_cast<const int8_t*>(wsrc) + static_cast<size_t>(c) * p->K;
             int8_t* dst = wp.data() + static_cast<size_t>(c) * p->K_pad;
-            for (int k = 0; k < p->K; ++k) { dst[k] = src[k]; sum += src[k]; }
-            corr[c] = static_cast<int32_t>(-static_cast<long long>(zx_shift) * sum);
+            for (int k = 0; k < p->K; ++k)
+            {
+                dst[k] = g.w_u8 ? static_cast<int8_t>(static_cast<uint8_t>(src[k]) ^ 0x80u) : src[k];
+                sum += dst[k];
+            }
+            // sum_k (x' - zx')(w - zw') = sum_k x'w - zx' sum_k w - zw' sum_k x' + K_pad zx' zw' over the padded row, whose bytes
+            // beyond K and outside the image are zx' against zero weights; the term with sum_k x' is the kernel's
+            corr[c] = static_cast<int32_t>(-static_cast<long long>(zx_shift) * sum + static_cast<long long>(zw_shift) * zx_shift * p->K_pad);
         }
+        p->zw_neg = -zw_shift;
         if (int rc = Upload(reinterpret_cast<void**>(&p->w_mfma), wp.data(), wp.size())) return rc;
         if (int rc = Upload(reinterpret_cast<void**>(&p->corr), corr.data(), corr.size() * sizeof(int32_t))) return rc;
         p->xor_mask = g.in_u8 ? 0x80808080u : 0u;
@@ -246,9 +256,12 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         FoldCorrIntoTable(p, corr, Co);
         ChoosePointwiseConfig(p);
         if (p->tile_override != 0) p->pw_bn = 0;     // a forced tile also forces the LDS-tiled implicit GEMM
+        if (p->zw_neg != 0) p->pw_bn = 0;            // only the implicit GEMM sums the activations a weight zero point needs
         if (int rc = PreparePointwise(p)) return rc;
         char buf[128];
-        if (p->pw_bn)
+        if (p->zw_neg != 0)
+            snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 tiles 128x128|128x64|64x64 x%d K=%d, weight zero point by row sums", p->bk128 ? 128 : 64, p->K);
+        else if (p->pw_bn)
             snprintf(buf, sizeof(buf), "pointwise_gemm_mfma_i8_32x32x32 weight-stationary slab %dxK=%d, chunk %d k-steps", p->pw_bn, p->K, p->pw_ks);
         else if (p->bk128 && (Ci % 128) == 0)
             snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 global_load_lds tiles 64x64..256x256 x128 K=%d", p->K);
@@ -493,18 +506,22 @@ int LaunchPwKs(const mi355x_conv2d_s* p, long long M, const void* x, void* y, hi
     }
 }
 
-template <int BM, int BN, int WM, int WN, int D, int BK, bool UT>
+template <int BM, int BN, int WM, int WN, int D, int BK, bool UT, bool AW>
 int LaunchIgemmT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream);
 
-// uniform-tap variant whenever a k-tile cannot straddle two filter taps
+// uniform-tap variant whenever a k-tile cannot straddle two filter taps; row sums when the weights have a zero point
 template <int BM, int BN, int WM, int WN, int D, int BK>
 int LaunchIgemm(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
 {
-    if ((p->geom.Ci % BK) == 0) return LaunchIgemmT<BM, BN, WM, WN, D, BK, true>(p, batch, x, y, stream);
-    return LaunchIgemmT<BM, BN, WM, WN, D, BK, false>(p, batch, x, y, stream);
+    const bool ut = (p->geom.Ci % BK) == 0;
+    if (p->zw_neg != 0)
+        return ut ? LaunchIgemmT<BM, BN, WM, WN, D, BK, true, true>(p, batch, x, y, stream)
+                  : LaunchIgemmT<BM, BN, WM, WN, D, BK, false, true>(p, batch, x, y, stream);
+    return ut ? LaunchIgemmT<BM, BN, WM, WN, D, BK, true, false>(p, batch, x, y, stream)
+              : LaunchIgemmT<BM, BN, WM, WN, D, BK, false, false>(p, batch, x, y, stream);
 }
 
-template <int BM, int BN, int WM, int WN, int D, int BK, bool UT>
+template <int BM, int BN, int WM, int WN, int D, int BK, bool UT, bool AW>
 int LaunchIgemmT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
 {
     const ConvGeom& g = p->geom;
@@ -530,14 +547,15 @@ int LaunchIgemmT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* 
     a.tiles_n = (g.Co + BN - 1) / BN;
     a.xor_mask = p->xor_mask;
     a.pad_word = p->pad_word;
+    a.zw_neg = p->zw_neg;
     a.rq = p->rq;
     const int nblocks = a.tiles_m * a.tiles_n;
     const int grid = (nblocks + 7) / 8 * 8;
     constexpr int smem = IgemmSmemBytes<BM, BN, BK>();
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmKernel<BM, BN, WM, WN, D, BK, UT>),
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmKernel<BM, BN, WM, WN, D, BK, UT, AW>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);
-    hipLaunchKernelGGL((IgemmKernel<BM, BN, WM, WN, D, BK, UT>), dim3(grid), dim3(256), smem, stream, a);
+    hipLaunchKernelGGL((IgemmKernel<BM, BN, WM, WN, D, BK, UT, AW>), dim3(grid), dim3(256), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;
 }
@@ -568,6 +586,7 @@ int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, voi
     a.tiles_n = (g.Co + BN - 1) / BN;
     a.xor_mask = p->xor_mask;
     a.pad_word = p->pad_word;
+    a.zw_neg = 0;
     a.rq = p->rq;
     const int nblocks = a.tiles_m * a.tiles_n;
     const int grid = (nblocks + 7) / 8 * 8;
@@ -612,7 +631,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const long long rows = static_cast<long long>(batch) * g.Ho * g.Wo;
         const bool unit = dd.kernel_h == 1 && dd.kernel_w == 1 && dd.stride_x == 1 && dd.stride_y == 1 && dd.pad_top == 0 &&
                           dd.pad_left == 0 && dd.out_h == dd.in_h && dd.out_w == dd.in_w;
-        if (unit && rows <= 4 && (g.Ci % 16) == 0 && p->tile_override == 0)
+        if (unit && rows <= 4 && (g.Ci % 16) == 0 && p->tile_override == 0 && p->zw_neg == 0)
         {
             // a handful of rows: stream the weights once, no tiles
             GemvArgs a;
@@ -629,7 +648,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             MI355X_HIP(hipGetLastError());
             return 0;
         }
-        if (unit && rows <= 64 && (g.Ci % 16) == 0 && g.Ci >= 128 && p->tile_override == 0 && p->Co_pad >= (g.Co + 31) / 32 * 32 &&
+        if (unit && rows <= 64 && (g.Ci % 16) == 0 && g.Ci >= 128 && p->tile_override == 0 && p->zw_neg == 0 && p->Co_pad >= (g.Co + 31) / 32 * 32 &&
             (reinterpret_cast<uintptr_t>(y) & 3) == 0)
         {
             // a few dozen rows: 32x32 tiles with K split over the block's waves
@@ -662,7 +681,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const int tile = p->tile_override ? p->tile_override : big < 400 ? 64 : (huge >= 192 && g.Co >= 256) ? 512 : 128;
         // channel counts that are multiples of 128: k-tiles go from global memory straight into LDS
         const int lds_stages = GlobalOptions().igemm_lds;
-        if (lds_stages != 0 && bk128 && (g.Ci % 128) == 0)
+        if (lds_stages != 0 && bk128 && (g.Ci % 128) == 0 && p->zw_neg == 0)
         {
             if (tile == 64)
             {
@@ -840,6 +859,7 @@ int mi355x_conv2d_fusable(mi355x_conv2d_t dw, mi355x_conv2d_t pw)
     const bool pointwise = pw->algo == MI355X_ALGO_MFMA && !b.depthwise && b.kernel_h == 1 && b.kernel_w == 1 && b.stride_x == 1 &&
                            b.stride_y == 1 && b.pad_top == 0 && b.pad_left == 0 && b.out_h == b.in_h && b.out_w == b.in_w;
     if (!pointwise) return SetError(MI355X_ERR_UNSUPPORTED, "second plan is not an unpadded 1x1 stride-1 convolution on the MFMA kernel");
+    if (pw->zw_neg != 0) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel needs pointwise weights without a zero point");
     if (a.out_c != b.in_c || a.out_h != b.in_h || a.out_w != b.in_w) return SetError(MI355X_ERR_INVALID_ARGUMENT, "the layers' shapes do not chain");
     if (a.output.dtype != b.input.dtype || a.output.scale != b.input.scale || a.output.offset != b.input.offset)
         return SetError(MI355X_ERR_INVALID_ARGUMENT, "the first layer's output quantization is not the second layer's input quantization");

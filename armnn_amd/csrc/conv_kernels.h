@@ -146,8 +146,13 @@ __global__ __launch_bounds__(256) void DepthwiseC4Kernel(ConvGeom g, Requant rq,
 //
 //   Inputs are brought to signed int8 on the fly (uint8: x ^ 0x80, i.e. x - 128, zero point shifted likewise);
 //   padding taps are filled with the (shifted) zero point, so acc = sum x'w - zx' * sum_k w, and the second
-//   term is a per-channel constant that initialises the accumulators (`corr`).  Weights must be symmetric
-//   (offset 0).
+//   term is a per-channel constant that initialises the accumulators (`corr`).
+//
+//   Weights with a zero point (template AW): w' = w - zw' with the stored int8 w, so
+//   sum (x' - zx')(w - zw') = sum x'w + corr[c] - zw' * S[m],  S[m] = sum_k x'[m][k] over the whole padded K row
+//   (bytes outside the image and beyond K are zx', which corr accounts for).  S[m] is summed with v_dot4 from the
+//   activation fragments a lane reads for the MFMA anyway -- the two lanes that hold the halves of a pixel's k-slice
+//   add up at the end -- and enters the accumulators just before they are requantized.
 //
 //   Block = 256 threads = 4 waves arranged WM x WN; each wave owns (BM/WM) x (BN/WN) outputs as 32x32 MFMA
 //   tiles.  The MFMA "A" operand is the weight fragment (row = channel) and "B" the activation fragment
@@ -172,6 +177,7 @@ struct IgemmArgs
     int tiles_m, tiles_n;
     uint32_t xor_mask;      // 0x80808080 for uint8 input, else 0
     uint32_t pad_word;      // shifted input zero point replicated in 4 bytes
+    int zw_neg;             // minus the zero point of the stored int8 weights (0: symmetric)
     Requant rq;
 };
 
@@ -191,7 +197,7 @@ constexpr int IgemmSmemBytes()
 // UT ("uniform tap"): Ci is a multiple of BK, so a k-tile never straddles two filter taps.  The walk over (ky, kx, ci) is
 // then the same for every thread (scalar registers), and a thread's address is a fixed per-row pointer plus a scalar
 // tap offset: no per-load multiplications.
-template <int BM, int BN, int WM, int WN, int D, int BK, bool UT>
+template <int BM, int BN, int WM, int WN, int D, int BK, bool UT, bool AW = false>
 __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
 {
     static_assert(WM * WN == 4, "4 waves per block");
@@ -347,6 +353,9 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
     const int frag_row = lane & 31;
     const int frag_k = (lane >> 5) * 16;
     using std::integral_constant;
+    int rowsum[TP];
+#pragma unroll
+    for (int tp = 0; tp < TP; ++tp) rowsum[tp] = 0;
 
     auto compute = [&](int buf) {
         const uint8_t* As = smem + buf * STAGE;
@@ -361,6 +370,13 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
 #pragma unroll
             for (int tc = 0; tc < TC; ++tc)
                 fw[tc] = *reinterpret_cast<const v4i*>(Bs + (wn * WTN + tc * 32 + frag_row) * LDK + ks * 32 + frag_k);
+            if constexpr (AW)
+            {
+#pragma unroll
+                for (int tp = 0; tp < TP; ++tp)
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) rowsum[tp] = __builtin_amdgcn_sdot4(fa[tp][i], 0x01010101, rowsum[tp], false);
+            }
 #pragma unroll
             for (int tc = 0; tc < TC; ++tc)
 #pragma unroll
@@ -395,6 +411,12 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
 
     // ---- epilogue: requantize, pack 4 channels per dword, stage the byte tile in LDS ---------------------
     uint8_t* Os = smem;   // all reads of the stage buffers are behind the loop's final barrier
+    if constexpr (AW)
+    {
+        // lanes l and l ^ 32 hold the two halves of every k-slice of pixel (l & 31)
+#pragma unroll
+        for (int tp = 0; tp < TP; ++tp) rowsum[tp] = (rowsum[tp] + __shfl_xor(rowsum[tp], 32)) * a.zw_neg;
+    }
 #pragma unroll
     for (int tc = 0; tc < TC; ++tc)
     {
@@ -407,7 +429,8 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
             for (int tp = 0; tp < TP; ++tp)
             {
                 const v16i& c = acc[tc][tp];
-                const uint32_t out = Requant4Dev(c[4 * q + 0], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], f4, a.ct, tn * BN + cl, a.rq);
+                const int rt = AW ? rowsum[tp] : 0;
+                const uint32_t out = Requant4Dev(c[4 * q + 0] + rt, c[4 * q + 1] + rt, c[4 * q + 2] + rt, c[4 * q + 3] + rt, f4, a.ct, tn * BN + cl, a.rq);
                 const int pl = wm * WTM + tp * 32 + (lane & 31);          // pixel within the block tile
                 *reinterpret_cast<uint32_t*>(Os + pl * LDO + cl) = out;
             }

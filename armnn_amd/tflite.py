@@ -1,7 +1,7 @@
 """Reads a quantized .tflite model into a nets.Network, with the conventions of Arm NN's TfLite parser.
 
 Only what the device path runs is accepted: 8-bit quantized CONV_2D, DEPTHWISE_CONV_2D, FULLY_CONNECTED,
-AVERAGE_POOL_2D, MAX_POOL_2D, ADD, PAD, MEAN (over height and width), RELU, RELU_N1_TO_1, RELU6, RESHAPE and SOFTMAX, one subgraph, one input, one output.  Anything else raises
+AVERAGE_POOL_2D, MAX_POOL_2D, ADD, PAD, MEAN (over height and width), RELU, RELU_N1_TO_1, RELU6, RESHAPE, SQUEEZE, QUANTIZE (between 8-bit quantizations) and SOFTMAX, one subgraph, one input, one output.  Anything else raises
 ``UnsupportedModel`` naming the operator -- nothing is approximated or skipped.
 
 What is taken from the reference parser (src/armnnTfLiteParser/TfLiteParser.cpp):
@@ -86,7 +86,8 @@ class _Table:
 # ---- schema constants ------------------------------------------------------------------------------------------------------
 _UINT8, _INT32, _INT8 = 3, 2, 9                                   # TensorType
 _OPS = {0: "ADD", 1: "AVERAGE_POOL_2D", 3: "CONV_2D", 4: "DEPTHWISE_CONV_2D", 9: "FULLY_CONNECTED", 17: "MAX_POOL_2D",
-        19: "RELU", 20: "RELU_N1_TO_1", 21: "RELU6", 22: "RESHAPE", 25: "SOFTMAX", 34: "PAD", 40: "MEAN"}                  # BuiltinOperator
+        19: "RELU", 20: "RELU_N1_TO_1", 21: "RELU6", 22: "RESHAPE", 25: "SOFTMAX", 34: "PAD", 40: "MEAN", 43: "SQUEEZE",
+        114: "QUANTIZE"}                  # BuiltinOperator
 _ACT = {0: (0, 0.0, 0.0), 1: (1, 0.0, 0.0), 2: (2, 1.0, -1.0), 3: (2, 6.0, 0.0)}    # NONE, RELU, RELU_N1_TO_1, RELU6
 _SAME, _VALID = 0, 1
 
@@ -315,9 +316,27 @@ def _parse(data: bytes, name: str) -> Network:
             # tensor's quantization differs from the input's
             expect(xi.shape)
             layers.append(Layer("activation", lname, (x,), y, act=_fused({"RELU": 1, "RELU_N1_TO_1": 2, "RELU6": 3}[kind])))
+        elif kind == "QUANTIZE":
+            # a Quantize layer (ParseQuantize); between two 8-bit quantizations it decodes and encodes every value
+            # (RefQuantizeWorkload.cpp), which is what an Activation layer without a function does
+            expect(xi.shape)
+            layers.append(Layer("activation", lname, (x,), y, act=(0, 0.0, 0.0)))
         elif kind == "RESHAPE":
             if yi.num_elements != xi.num_elements:
                 raise UnsupportedModel("RESHAPE: input and output differ in their number of elements")
+            layers.append(Layer("reshape", lname, (x,), y))
+        elif kind == "SQUEEZE":
+            # a Reshape layer (ParseSqueeze); the output keeps the input's dimensions except some of extent 1
+            kept = iter(yi.shape)
+            nxt = next(kept, None)
+            for extent in xi.shape:
+                if nxt is not None and extent == nxt:
+                    nxt = next(kept, None)
+                elif extent != 1:
+                    nxt = -1
+                    break
+            if nxt is not None:
+                raise UnsupportedModel(f"SQUEEZE: {tuple(yi.shape)} is not {tuple(xi.shape)} without some of its dimensions of extent 1")
             layers.append(Layer("reshape", lname, (x,), y))
         elif kind == "SOFTMAX":
             expect(xi.shape)

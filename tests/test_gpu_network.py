@@ -176,3 +176,10 @@ def test_tflite_model_with_standalone_activations(port):
     net = tflite.parse(relu_model(), "relu")
     _layerwise(port, net, 1)
     _layerwise(port, net, 32)
+
+
+def test_tflite_model_with_quantize_and_squeeze(port):
+    from armnn_amd import tflite
+    from tests.test_tflite import quantize_squeeze_model
+    net = tflite.parse(quantize_squeeze_model(), "qs")
+    _layerwise(port, net, 2)

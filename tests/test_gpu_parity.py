@@ -343,3 +343,58 @@ def test_random_fully_connected(port, chunk):
         assert exact >= 0.98 or auto.data.size < 200, (k, exact)
         direct = shim.fully_connected(case.x, case.w, case.b, case.out_info, algo=shim.ALGO_DIRECT, **kw)
         np.testing.assert_array_equal(auto.data, direct.data, err_msg=f"fc case {k}")
+
+
+_ZP_CONVS = [
+    # (name, conv kwargs): per-tensor weights with a zero point, shapes the MFMA implicit GEMM takes (in_c % 16 == 0)
+    ("u8_pointwise_c32", dict(n=3, h=14, w=14, ci=32, co=64, kh=1, kw=1, padding="valid", w_dtype=DataType.QAsymmU8, w_offset=93)),
+    ("u8_pointwise_c128_ragged_co", dict(n=2, h=9, w=11, ci=128, co=200, kh=1, kw=1, padding="valid", w_dtype=DataType.QAsymmU8, w_offset=151)),
+    ("u8_3x3_same_c64", dict(n=2, h=13, w=17, ci=64, co=128, kh=3, kw=3, padding="same", w_dtype=DataType.QAsymmU8, w_offset=120)),
+    ("u8_3x3_s2_c48", dict(n=2, h=15, w=15, ci=48, co=32, kh=3, kw=3, stride=(2, 2), padding="same", w_dtype=DataType.QAsymmU8, w_offset=3)),
+    ("u8_3x3_c128_uniform_tap", dict(n=1, h=12, w=12, ci=128, co=128, kh=3, kw=3, padding=(1, 0, 2, 1), w_dtype=DataType.QAsymmU8, w_offset=255)),
+    ("u8_5x5_dilated_c16", dict(n=1, h=20, w=18, ci=16, co=48, kh=5, kw=5, dilation=(2, 2), padding="same", w_dtype=DataType.QAsymmU8, w_offset=0)),
+    ("u8_zero_point_128_is_symmetric", dict(n=4, h=14, w=14, ci=64, co=64, kh=1, kw=1, padding="valid", w_dtype=DataType.QAsymmU8, w_offset=128)),
+    ("s8_pointwise_c256", dict(n=2, h=7, w=7, ci=256, co=512, kh=1, kw=1, padding="valid", w_dtype=DataType.QAsymmS8, w_offset=-17)),
+    ("s8_3x3_c32_big_batch", dict(n=16, h=28, w=28, ci=32, co=64, kh=3, kw=3, padding="same", w_dtype=DataType.QAsymmS8, w_offset=127)),
+    ("s8_3x3_lowest_zero_point", dict(n=1, h=8, w=8, ci=16, co=16, kh=3, kw=3, padding="same", w_dtype=DataType.QAsymmS8, w_offset=-128)),
+]
+
+
+@pytest.mark.parametrize("in_u8", [False, True], ids=["s8_in", "u8_in"])
+@pytest.mark.parametrize("name,kw", _ZP_CONVS, ids=[n for n, _ in _ZP_CONVS])
+def test_weights_with_a_zero_point_on_the_matrix_cores(port, name, kw, in_u8):
+    """Per-tensor QAsymmU8 / QAsymmS8 weights whose zero point is not 0: the implicit GEMM sums each pixel's activations
+    beside the products; the bytes must be the direct kernel's and within 1 LSB of the checker."""
+    seed = 31000 + 7 * [n for n, _ in _ZP_CONVS].index(name) + int(in_u8)
+    case = cases.make_conv_case(name, seed, per_axis=False, in_dtype=DataType.QAsymmU8 if in_u8 else DataType.QAsymmS8,
+                                in_offset=131 if in_u8 else -9, out_offset=100 if in_u8 else -20, act=(2, 6.0, 0.0), **kw)
+    print(f"{name}: x={case.x.info.shape} w={case.w.info.shape} zw={case.w.info.offset}", flush=True)
+    fn, a, b = case.act
+    plan = shim.Conv2dPlan(case.x.info, case.w, case.b, case.out_info, activation=fn, act_a=a, act_b=b, algo=shim.ALGO_AUTO, **case.params)
+    algo, desc = plan.algo()
+    plan.destroy()
+    print(f"  kernel: {desc}", flush=True)
+    assert algo == shim.ALGO_MFMA
+    assert ("weight zero point" in desc) == (case.w.info.offset != (128 if case.w.info.dtype == DataType.QAsymmU8 else 0))
+    want = _oracle_conv(port, case)
+    auto = _gpu_conv(case, shim.ALGO_AUTO)
+    mx, exact = lsb_diff(auto.data, want.data)
+    print(f"  max|d|={mx} exact={exact:.5f}", flush=True)
+    assert mx <= 1 and exact >= 0.99
+    np.testing.assert_array_equal(auto.data, _gpu_conv(case, shim.ALGO_DIRECT).data)
+
+
+@pytest.mark.parametrize("m", [1, 3, 40, 256])
+@pytest.mark.parametrize("w_dtype,w_offset", [(DataType.QAsymmU8, 93), (DataType.QAsymmS8, -30)])
+def test_fully_connected_weights_with_a_zero_point(port, m, w_dtype, w_offset):
+    case = cases.make_fc_case(f"fc_zp_m{m}", 32000 + m, m=m, k=512, o=320, in_dtype=DataType.QAsymmU8, in_offset=63, w_dtype=w_dtype,
+                              per_axis=False, w_offset=w_offset, out_offset=30)
+    print(f"fc m={m} {w_dtype.name} zw={w_offset}", flush=True)
+    kw = dict(transpose_weights=case.transpose_weights)
+    want = port.fully_connected(case.x, case.w, case.b, case.out_info, **kw)
+    auto = shim.fully_connected(case.x, case.w, case.b, case.out_info, algo=shim.ALGO_AUTO, **kw)
+    mx, exact = lsb_diff(auto.data, want.data)
+    print(f"  max|d|={mx} exact={exact:.5f}", flush=True)
+    assert mx <= 1 and exact >= 0.99
+    direct = shim.fully_connected(case.x, case.w, case.b, case.out_info, algo=shim.ALGO_DIRECT, **kw)
+    np.testing.assert_array_equal(auto.data, direct.data)

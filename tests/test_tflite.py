@@ -233,3 +233,33 @@ def test_standalone_activations_become_layers_of_their_own(port, reference):
         np.testing.assert_array_equal(a[name].data, b[name].data, err_msg=name)
     first = a[net.layers[0].output].data
     assert first.min() == -128 and first.max() == 127            # [0, 6] fills the re-quantized range
+
+
+def quantize_squeeze_model(squeezed=(2, 24)):
+    """uint8 input re-quantized to int8 (QUANTIZE), pooled to 1x1, squeezed to two dimensions, softmax."""
+    b = tw.ModelBuilder()
+    x = b.tensor("input", (2, 4, 4, 24), tw.UINT8, 0.05, 120)
+    q = b.tensor("as_int8", (2, 4, 4, 24), tw.INT8, 0.05, -8)
+    b.op(tw.QUANTIZE, [x], [q])
+    p = b.tensor("pooled", (2, 1, 1, 24), tw.INT8, 0.05, -8)
+    b.op(tw.AVERAGE_POOL_2D, [q], [p], tw.OPT_POOL, {0: ("b", tw.VALID), 1: ("i", 4), 2: ("i", 4), 3: ("i", 4), 4: ("i", 4)})
+    s = b.tensor("squeezed", squeezed, tw.INT8, 0.05, -8)
+    b.op(tw.SQUEEZE, [p], [s])
+    y = b.tensor("probabilities", squeezed, tw.INT8, 1.0 / 256.0, -128)
+    b.op(tw.SOFTMAX, [s], [y], tw.OPT_SOFTMAX, {0: ("f", 1.0)})
+    return b.finish([x], [y])
+
+
+def test_quantize_between_8_bit_types_and_squeeze(port, reference):
+    net = tflite.parse(quantize_squeeze_model(), "qs")
+    assert [l.op for l in net.layers] == ["activation", "pool", "reshape", "softmax"]
+    assert net.layers[0].act == (0, 0.0, 0.0)
+    x = nets.synthetic_input(net, 2, seed=9)
+    a = netref.run_network(port, net, x, keep=True)
+    b = netref.run_network(reference, net, x, keep=True)
+    for name in a:
+        np.testing.assert_array_equal(a[name].data, b[name].data, err_msg=name)
+    # same scale, zero points 128 apart: the int8 codes are the uint8 codes shifted
+    np.testing.assert_array_equal(a[net.layers[0].output].data.astype(np.int32), x.data.astype(np.int32) - 128)
+    with pytest.raises(tflite.UnsupportedModel, match="SQUEEZE"):
+        tflite.parse(quantize_squeeze_model(squeezed=(4, 12)), "bad")

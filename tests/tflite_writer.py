@@ -93,7 +93,7 @@ def build(root: dict) -> bytes:
 # ---- the TfLite schema, as far as the tests need it ----------------------------------------------------------------------
 FLOAT32, INT32, UINT8, INT8 = 0, 2, 3, 9
 ADD, AVERAGE_POOL_2D, CONV_2D, DEPTHWISE_CONV_2D, FULLY_CONNECTED, MAX_POOL_2D, RESHAPE, SOFTMAX, PAD, TANH, MEAN = 0, 1, 3, 4, 9, 17, 22, 25, 34, 28, 40
-RELU, RELU_N1_TO_1, RELU6 = 19, 20, 21
+RELU, RELU_N1_TO_1, RELU6, SQUEEZE, QUANTIZE = 19, 20, 21, 43, 114
 SAME, VALID = 0, 1
 ACT_NONE, ACT_RELU, ACT_RELU_N1_TO_1, ACT_RELU6 = 0, 1, 2, 3
 # BuiltinOptions union tags
