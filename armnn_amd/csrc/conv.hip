@@ -28,6 +28,7 @@ struct mi355x_conv2d_s
     int      stem_kp  = 0;
     uint32_t* dw_grp  = nullptr;   // depthwise 3x3: constants per group of 4 channels for the fused dw+pw kernel
     uint32_t* w_dot4  = nullptr;   // depthwise 3x3: [C][4] dwords; small-Ci conv: [Co][Kh][RD] dwords
+    uint32_t* w_dot4b = nullptr;   // depthwise 3x3 whose weight differences need two int8 halves: the second halves
     int variant = 0;               // kernel variant within an algo (see RunPlan)
     int row_dwords = 0;            // small-Ci conv: dwords per filter row
     float*   chan     = nullptr;   // [5][Co_pad] per-channel requantization constants (rows: see ChanTab)
@@ -50,6 +51,7 @@ struct mi355x_conv2d_s
         (void)hipFree(dw_grp);
         (void)hipFree(w_stem);
         (void)hipFree(w_dot4);
+        (void)hipFree(w_dot4b);
         (void)hipFree(chan);
         (void)hipFree(corr);
     }
@@ -202,8 +204,22 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     const bool dw_ok = d.depthwise && g.depth_mult == 1 && (Co % 4) == 0;
     const bool sym_s8 = g.zw == 0 && !g.w_u8 && zx_shift >= -128 && zx_shift <= 127;
     // depthwise 3x3 on v_dot4 with an LDS halo tile
-    const bool dw3_ok = dw_ok && sym_s8 && Kh == 3 && Kw == 3 && (Co % 32) == 0 && d.dilation_x == 1 && d.dilation_y == 1 &&
-                        d.stride_x == d.stride_y && (d.stride_x == 1 || d.stride_x == 2);
+    // It multiplies the activations with d = w - zw, one int8 when every d fits, else two int8 halves (floor(d / 2) and
+    // the rest); d = 255 has no such halves.
+    bool dw3_fits = true, dw3_halves = true;
+    if (dw_ok && Kh == 3 && Kw == 3 && zw_shift >= -128 && zw_shift <= 127)
+    {
+        const uint8_t* wb = static_cast<const uint8_t*>(weights_host);
+        for (int i = 0; i < 9 * Co; ++i)
+        {
+            const int dv = static_cast<int>(static_cast<int8_t>(g.w_u8 ? wb[i] ^ 0x80u : wb[i])) - zw_shift;
+            dw3_fits &= dv >= -128 && dv <= 127;
+            dw3_halves &= dv != 255;
+        }
+    }
+    const bool dw3_ok = dw_ok && zw_shift >= -128 && zw_shift <= 127 && zx_shift >= -128 && zx_shift <= 127 && dw3_halves && Kh == 3 &&
+                        Kw == 3 && (Co % 32) == 0 && d.dilation_x == 1 && d.dilation_y == 1 && d.stride_x == d.stride_y &&
+                        (d.stride_x == 1 || d.stride_x == 2);
     // stems: <= 4 input channels, rows of Kw*Ci bytes walked with v_dot4
     const int row_bytes = Kw * Ci;
     const bool stem_ok = !d.depthwise && sym_s8 && Ci <= 4 && (Co % 4) == 0 && d.dilation_x == 1 && d.dilation_y == 1 &&
@@ -272,26 +288,31 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     else if (algo == MI355X_ALGO_DEPTHWISE && dw3_ok)
     {
         // [1][3][3][C] -> per channel 4 dwords, dword r = { w[r][0], w[r][1], w[r][2], 0 }
-        const int8_t* ws = reinterpret_cast<const int8_t*>(wsrc);
-        std::vector<uint32_t> wp(static_cast<size_t>(Co) * 4, 0u);
+        std::vector<uint32_t> wp(static_cast<size_t>(Co) * 4, 0u), wp2(static_cast<size_t>(Co) * 4, 0u);
         std::vector<int32_t> corr(Co, 0);
         for (int c = 0; c < Co; ++c)
         {
             long long sum = 0;
             for (int r = 0; r < 3; ++r)
             {
-                uint32_t dw = 0;
+                uint32_t dw = 0, dw2 = 0;
                 for (int kx = 0; kx < 3; ++kx)
                 {
-                    const int8_t v = ws[(r * 3 + kx) * Co + c];
-                    dw |= static_cast<uint32_t>(static_cast<uint8_t>(v)) << (8 * kx);
-                    sum += v;
+                    const uint8_t raw = wsrc[(r * 3 + kx) * Co + c];
+                    const int dv = static_cast<int>(static_cast<int8_t>(g.w_u8 ? raw ^ 0x80u : raw)) - zw_shift;
+                    const int first = dw3_fits ? dv : dv >> 1;        // floor(d / 2): -128 .. 127
+                    dw |= static_cast<uint32_t>(static_cast<uint8_t>(first)) << (8 * kx);
+                    dw2 |= static_cast<uint32_t>(static_cast<uint8_t>(dv - first)) << (8 * kx);
+                    sum += dv;
                 }
                 wp[static_cast<size_t>(c) * 4 + r] = dw;
+                wp2[static_cast<size_t>(c) * 4 + r] = dw2;
             }
             corr[c] = static_cast<int32_t>(-static_cast<long long>(zx_shift) * sum);
         }
         if (int rc = Upload(reinterpret_cast<void**>(&p->w_dot4), wp.data(), wp.size() * sizeof(uint32_t))) return rc;
+        if (!dw3_fits)
+            if (int rc = Upload(reinterpret_cast<void**>(&p->w_dot4b), wp2.data(), wp2.size() * sizeof(uint32_t))) return rc;
         if (int rc = Upload(reinterpret_cast<void**>(&p->corr), corr.data(), corr.size() * sizeof(int32_t))) return rc;
         p->xor_mask = g.in_u8 ? 0x80808080u : 0u;
         const uint32_t zb = static_cast<uint32_t>(zx_shift) & 0xffu;
@@ -313,6 +334,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             if (int rc = Upload(reinterpret_cast<void**>(&p->pad16), padbytes.data(), padbytes.size())) return rc;
         }
         p->info = d.stride_x == 1 ? "depthwise3x3_dot4_lds stride 1, tile 8x16x32" : "depthwise3x3_dot4_lds stride 2, tile 8x8x32";
+        if (p->w_dot4b) p->info += ", weights minus their zero point as two int8 halves";
     }
     else if (algo == MI355X_ALGO_DEPTHWISE)
     {
@@ -765,7 +787,15 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             a.total_blocks = static_cast<int>(nb);
             a.xcd_chunk = static_cast<int>((nb + 7) / 8);
             const dim3 grid(static_cast<unsigned>(a.xcd_chunk) * 8u);
-            if (g.stride_x == 1 && rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2>), grid, dim3(256), 0, stream, a);
+            a.wpack2 = p->w_dot4b;
+            if (p->w_dot4b)
+            {
+                if (g.stride_x == 1 && rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2, true>), grid, dim3(256), 0, stream, a);
+                else if (g.stride_x == 1) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1, true>), grid, dim3(256), 0, stream, a);
+                else if (rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<2, 2, true>), grid, dim3(256), 0, stream, a);
+                else hipLaunchKernelGGL((Depthwise3x3Kernel<2, 1, true>), grid, dim3(256), 0, stream, a);
+            }
+            else if (g.stride_x == 1 && rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2>), grid, dim3(256), 0, stream, a);
             else if (g.stride_x == 1) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1>), grid, dim3(256), 0, stream, a);
             else if (rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<2, 2>), grid, dim3(256), 0, stream, a);
             else hipLaunchKernelGGL((Depthwise3x3Kernel<2, 1>), grid, dim3(256), 0, stream, a);
@@ -854,7 +884,7 @@ int mi355x_conv2d_fusable(mi355x_conv2d_t dw, mi355x_conv2d_t pw)
     if (!dw || !pw) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
     const mi355x_conv2d_desc& a = dw->d;
     const mi355x_conv2d_desc& b = pw->d;
-    if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || !dw->dw_grp)
+    if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || !dw->dw_grp || dw->w_dot4b)
         return SetError(MI355X_ERR_UNSUPPORTED, "first plan is not a 3x3 depthwise layer on the v_dot4 kernel");
     const bool pointwise = pw->algo == MI355X_ALGO_MFMA && !b.depthwise && b.kernel_h == 1 && b.kernel_w == 1 && b.stride_x == 1 &&
                            b.stride_y == 1 && b.pad_top == 0 && b.pad_left == 0 && b.out_h == b.in_h && b.out_w == b.in_w;

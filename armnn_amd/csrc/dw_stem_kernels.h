@@ -5,7 +5,10 @@
 //
 // Both bring the input to signed int8 while staging (uint8: x ^ 0x80) and fill out-of-image positions with the
 // shifted zero point, so that   sum (x - zx) w  =  sum x' w  -  zx' * sum_taps w ;   the second term is a
-// per-channel constant (`corr`) that initialises the accumulators.  Weights must be symmetric int8 (offset 0).
+// per-channel constant (`corr`) that initialises the accumulators.  The depthwise kernel takes as "w" the difference
+// d = w - zw between a weight and the weights' zero point; where some d does not fit int8 (it lies in -255 .. 254) it is
+// the sum of two int8 halves, each in a packed array of its own (template W2), and costs a second v_dot4.  The stem
+// kernel needs symmetric int8 weights (offset 0).
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -22,6 +25,7 @@ struct Dw3x3Args
     const uint8_t*  x;
     const uint8_t*  pad16;    // 16 bytes of (padding value ^ input xor)
     const uint32_t* wpack;    // [C][4] dwords; dword r (r < 3) = bytes { w[r][0][c], w[r][1][c], w[r][2][c], 0 }
+    const uint32_t* wpack2;   // W2: the second halves, same layout
     ChanTab         ct;
     const int32_t*  corr;     // [C]  -zx' * sum of the 9 taps
     uint8_t*        y;
@@ -49,7 +53,7 @@ __device__ __forceinline__ int XcdContiguousWorkItem(int block, int chunk)
 // through one v_dot4 per channel and output row that the input row belongs to.  With R = 2 the rows two outputs share
 // are read and transposed once, and the per-thread set-up (staging, constants, addresses) is spread over twice the
 // outputs; R = 1 keeps more blocks in flight for small feature maps.
-template <int S, int R>
+template <int S, int R, bool W2 = false>
 __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
 {
     constexpr int CB = 32, TH = 8 * R, XG = 4;
@@ -103,12 +107,21 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
     const int xg = (tid >> 3) & 3;
     const int row = (tid >> 5) * R;              // first of this thread's output rows within the tile
     const int c = cb * CB + c4 * 4;
-    uint32_t wA[3][4];
+    uint32_t wA[3][4], wB[3][4];
 #pragma unroll
     for (int ch = 0; ch < 4; ++ch)
     {
         const uint4 w4 = *reinterpret_cast<const uint4*>(a.wpack + (c + ch) * 4);
         wA[0][ch] = w4.x; wA[1][ch] = w4.y; wA[2][ch] = w4.z;
+        if constexpr (W2)
+        {
+            const uint4 v4 = *reinterpret_cast<const uint4*>(a.wpack2 + (c + ch) * 4);
+            wB[0][ch] = v4.x; wB[1][ch] = v4.y; wB[2][ch] = v4.z;
+        }
+        else
+        {
+            wB[0][ch] = wB[1][ch] = wB[2][ch] = 0u;
+        }
     }
     const v4i corr4 = *reinterpret_cast<const v4i*>(a.corr + c);
     int acc[R][P][4];
@@ -158,10 +171,16 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
                     {
                         acc[o][2 * g][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wA[r][ch]), acc[o][2 * g][ch], false);
                         acc[o][2 * g + 1][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wA[r][ch] << 8), acc[o][2 * g + 1][ch], false);
+                        if constexpr (W2)
+                        {
+                            acc[o][2 * g][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wB[r][ch]), acc[o][2 * g][ch], false);
+                            acc[o][2 * g + 1][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wB[r][ch] << 8), acc[o][2 * g + 1][ch], false);
+                        }
                     }
                     else
                     {
                         acc[o][g][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wA[r][ch]), acc[o][g][ch], false);
+                        if constexpr (W2) acc[o][g][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wB[r][ch]), acc[o][g][ch], false);
                     }
                 }
             }

@@ -72,7 +72,7 @@ def main(argv=None):
     ap.add_argument("--o", type=int, default=4096)
     ap.add_argument("--u8", action="store_true", help="QAsymmU8 activations (default QAsymmS8)")
     ap.add_argument("--wzp", type=int, default=None, metavar="ZERO_POINT",
-                    help="per-tensor QAsymmU8 weights with this zero point (default: per-channel QSymmS8); conv and fc")
+                    help="per-tensor QAsymmU8 weights with this zero point (default: per-channel QSymmS8)")
     ap.add_argument("--algo", type=int, default=0)
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
@@ -115,11 +115,11 @@ def main(argv=None):
         taps = a.k * a.k * (1 if dw else ci)
         ws = synth.scales(3, co) / np.float32(np.sqrt(taps) / 3.0)
         w = QTensor(TensorInfo(wshape, DataType.QSymmS8, tuple(ws), 0, 3 if dw else 0), synth.int8_weights(2, wshape))
-        if a.wzp is not None and not dw:
+        if a.wzp is not None:
             ws = ws[:1]
             w = QTensor(TensorInfo(wshape, DataType.QAsymmU8, tuple(ws), a.wzp, None),
                         np.clip(synth.int8_weights(2, wshape).astype(np.int32) + a.wzp, 0, 255).astype(np.uint8))
-        b = QTensor(TensorInfo((co,), DataType.Signed32, tuple(np.float32(0.0235) * ws), 0, 0 if a.wzp is None or dw else None), synth.int32_bias(4, co))
+        b = QTensor(TensorInfo((co,), DataType.Signed32, tuple(np.float32(0.0235) * ws), 0, 0 if a.wzp is None else None), synth.int32_bias(4, co))
         plan = shim.Conv2dPlan(xin, w, b, yout, pad_top=pt, pad_left=pl, stride_x=a.stride, stride_y=a.stride,
                                depthwise=dw, activation=act[0], act_a=act[1], act_b=act[2], algo=a.algo)
         batch, macs = a.n, a.n * ho * wo * co * taps

@@ -398,3 +398,51 @@ def test_fully_connected_weights_with_a_zero_point(port, m, w_dtype, w_offset):
     assert mx <= 1 and exact >= 0.99
     direct = shim.fully_connected(case.x, case.w, case.b, case.out_info, algo=shim.ALGO_DIRECT, **kw)
     np.testing.assert_array_equal(auto.data, direct.data)
+
+
+_ZP_DEPTHWISE = [
+    ("u8_zp128_fits_int8", dict(n=2, h=20, w=20, ci=32, stride=(1, 1), w_dtype=DataType.QAsymmU8, w_offset=128), False),
+    ("u8_zp93_two_halves", dict(n=3, h=19, w=23, ci=64, stride=(1, 1), w_dtype=DataType.QAsymmU8, w_offset=93), True),
+    ("u8_zp160_stride2", dict(n=2, h=28, w=28, ci=96, stride=(2, 2), w_dtype=DataType.QAsymmU8, w_offset=160), True),
+    ("u8_zp1_small_map", dict(n=5, h=7, w=7, ci=128, stride=(1, 1), w_dtype=DataType.QAsymmU8, w_offset=1), True),
+    ("s8_zp-40", dict(n=2, h=16, w=16, ci=32, stride=(2, 2), w_dtype=DataType.QAsymmS8, w_offset=-40), True),
+    ("s8_zp5_tall_batch", dict(n=16, h=56, w=56, ci=32, stride=(1, 1), w_dtype=DataType.QAsymmS8, w_offset=5), None),
+]
+
+
+@pytest.mark.parametrize("in_u8", [False, True], ids=["s8_in", "u8_in"])
+@pytest.mark.parametrize("name,kw,halves", _ZP_DEPTHWISE, ids=[n for n, _, _ in _ZP_DEPTHWISE])
+def test_depthwise_weights_with_a_zero_point(port, name, kw, halves, in_u8):
+    """3x3 depthwise layers whose per-tensor weights have a zero point run on the v_dot4 kernel with the weights minus
+    their zero point, as one int8 where that fits and as two halves otherwise."""
+    seed = 33000 + 5 * [n for n, _, _ in _ZP_DEPTHWISE].index(name) + int(in_u8)
+    case = cases.make_conv_case(name, seed, kh=3, kw=3, padding="same", depthwise=True, per_axis=False, w_std=60.0,
+                                in_dtype=DataType.QAsymmU8 if in_u8 else DataType.QAsymmS8, in_offset=140 if in_u8 else 11,
+                                out_offset=3 if in_u8 else -100, act=(2, 6.0, 0.0), **kw)
+    fn, a, b = case.act
+    plan = shim.Conv2dPlan(case.x.info, case.w, case.b, case.out_info, activation=fn, act_a=a, act_b=b, algo=shim.ALGO_AUTO, **case.params)
+    algo, desc = plan.algo()
+    plan.destroy()
+    print(f"{name}: x={case.x.info.shape} zw={case.w.info.offset} kernel: {desc}", flush=True)
+    assert "depthwise3x3_dot4" in desc
+    if halves is not None:
+        assert ("two int8 halves" in desc) == halves
+    want = _oracle_conv(port, case)
+    auto = _gpu_conv(case, shim.ALGO_AUTO)
+    mx, exact = lsb_diff(auto.data, want.data)
+    print(f"  max|d|={mx} exact={exact:.5f}", flush=True)
+    assert mx <= 1 and exact >= 0.99
+    np.testing.assert_array_equal(auto.data, _gpu_conv(case, shim.ALGO_DIRECT).data)
+
+
+def test_depthwise_weight_255_above_its_zero_point_takes_the_general_kernel(port):
+    case = cases.make_conv_case("dw_d255", 33900, n=1, h=9, w=9, ci=32, kh=3, kw=3, padding="same", depthwise=True, per_axis=False,
+                                in_dtype=DataType.QAsymmU8, in_offset=128, w_dtype=DataType.QAsymmU8, w_offset=0)
+    case.w.data.reshape(-1)[5] = 255
+    plan = shim.Conv2dPlan(case.x.info, case.w, case.b, case.out_info, algo=shim.ALGO_AUTO, **case.params)
+    desc = plan.algo()[1]
+    plan.destroy()
+    assert desc == "depthwise_c4_valu"
+    want = _oracle_conv(port, case)
+    got = _gpu_conv(case, shim.ALGO_AUTO)
+    assert lsb_diff(got.data, want.data)[0] <= 1
