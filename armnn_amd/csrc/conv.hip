@@ -28,7 +28,7 @@ struct mi355x_conv2d_s
     int      stem_kp  = 0;
     uint32_t* dw_grp  = nullptr;   // depthwise 3x3: constants per group of 4 channels for the fused dw+pw kernel
     uint32_t* w_dot4  = nullptr;   // depthwise 3x3: [C][4] dwords; small-Ci conv: [Co][Kh][RD] dwords
-    uint32_t* w_dot4b = nullptr;   // depthwise 3x3 whose weight differences need two int8 halves: the second halves
+    uint32_t* w_dot4b = nullptr;   // depthwise 3x3 / small-Ci conv whose weight differences need two int8 halves: the second halves
     int variant = 0;               // kernel variant within an algo (see RunPlan)
     int row_dwords = 0;            // small-Ci conv: dwords per filter row
     float*   chan     = nullptr;   // [5][Co_pad] per-channel requantization constants (rows: see ChanTab)
@@ -202,7 +202,6 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     const bool mfma_ok = !d.depthwise && zw_shift >= -128 && zw_shift <= 127 && (Ci % 16) == 0 && zx_shift >= -128 && zx_shift <= 127 &&
                          p->K <= 100000;
     const bool dw_ok = d.depthwise && g.depth_mult == 1 && (Co % 4) == 0;
-    const bool sym_s8 = g.zw == 0 && !g.w_u8 && zx_shift >= -128 && zx_shift <= 127;
     // depthwise 3x3 on v_dot4 with an LDS halo tile
     // It multiplies the activations with d = w - zw, one int8 when every d fits, else two int8 halves (floor(d / 2) and
     // the rest); d = 255 has no such halves.
@@ -222,7 +221,19 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
                         (d.stride_x == 1 || d.stride_x == 2);
     // stems: <= 4 input channels, rows of Kw*Ci bytes walked with v_dot4
     const int row_bytes = Kw * Ci;
-    const bool stem_ok = !d.depthwise && sym_s8 && Ci <= 4 && (Co % 4) == 0 && d.dilation_x == 1 && d.dilation_y == 1 &&
+    bool stem_fits = true, stem_halves = true;
+    if (!d.depthwise && Ci <= 4 && zw_shift >= -128 && zw_shift <= 127)
+    {
+        const uint8_t* wb = static_cast<const uint8_t*>(weights_host);
+        for (long long i = 0; i < static_cast<long long>(Co) * p->K; ++i)
+        {
+            const int dv = static_cast<int>(static_cast<int8_t>(g.w_u8 ? wb[i] ^ 0x80u : wb[i])) - zw_shift;
+            stem_fits &= dv >= -128 && dv <= 127;
+            stem_halves &= dv != 255;
+        }
+    }
+    const bool stem_ok = !d.depthwise && zw_shift >= -128 && zw_shift <= 127 && zx_shift >= -128 && zx_shift <= 127 && stem_halves &&
+                         Ci <= 4 && (Co % 4) == 0 && d.dilation_x == 1 && d.dilation_y == 1 &&
                          d.stride_x == d.stride_y && (d.stride_x == 1 || d.stride_x == 2) &&
                          ((Kh == 3 && row_bytes <= 12) || (Kh == 7 && row_bytes <= 24) || (Kh == 1 && row_bytes <= 4) ||
                           (Kh == 5 && row_bytes <= 20));
@@ -344,8 +355,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     else if (algo == MI355X_ALGO_DOT4)
     {
         const int RD = Kh == 3 ? 3 : Kh == 7 ? 6 : Kh == 5 ? 5 : 1;
-        const int8_t* ws = reinterpret_cast<const int8_t*>(wsrc);
-        std::vector<uint32_t> wp(static_cast<size_t>(Co) * Kh * RD, 0u);
+        std::vector<uint32_t> wp(static_cast<size_t>(Co) * Kh * RD, 0u), wp2(static_cast<size_t>(Co) * Kh * RD, 0u);
         std::vector<int32_t> corr(Co, 0);
         for (int c = 0; c < Co; ++c)
         {
@@ -353,13 +363,20 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             for (int r = 0; r < Kh; ++r)
                 for (int bidx = 0; bidx < row_bytes; ++bidx)
                 {
-                    const int8_t v = ws[(static_cast<size_t>(c) * Kh + r) * row_bytes + bidx];
-                    wp[(static_cast<size_t>(c) * Kh + r) * RD + bidx / 4] |= static_cast<uint32_t>(static_cast<uint8_t>(v)) << (8 * (bidx % 4));
-                    sum += v;
+                    // the weight minus the weights' zero point, whole or as floor(d / 2) and the rest
+                    const uint8_t raw = wsrc[(static_cast<size_t>(c) * Kh + r) * row_bytes + bidx];
+                    const int dv = static_cast<int>(static_cast<int8_t>(g.w_u8 ? raw ^ 0x80u : raw)) - zw_shift;
+                    const int first = stem_fits ? dv : dv >> 1;
+                    const size_t at = (static_cast<size_t>(c) * Kh + r) * RD + bidx / 4;
+                    wp[at] |= static_cast<uint32_t>(static_cast<uint8_t>(first)) << (8 * (bidx % 4));
+                    wp2[at] |= static_cast<uint32_t>(static_cast<uint8_t>(dv - first)) << (8 * (bidx % 4));
+                    sum += dv;
                 }
             corr[c] = static_cast<int32_t>(-static_cast<long long>(zx_shift) * sum);
         }
         if (int rc = Upload(reinterpret_cast<void**>(&p->w_dot4), wp.data(), wp.size() * sizeof(uint32_t))) return rc;
+        if (!stem_fits)
+            if (int rc = Upload(reinterpret_cast<void**>(&p->w_dot4b), wp2.data(), wp2.size() * sizeof(uint32_t))) return rc;
         if (int rc = Upload(reinterpret_cast<void**>(&p->corr), corr.data(), corr.size() * sizeof(int32_t))) return rc;
         p->xor_mask = g.in_u8 ? 0x80u : 0u;
         p->pad_word = static_cast<uint32_t>(zx_shift) & 0xffu;
@@ -368,7 +385,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             const std::vector<uint8_t> padbytes(16, static_cast<uint8_t>((p->pad_word ^ p->xor_mask) & 0xffu));
             if (int rc = Upload(reinterpret_cast<void**>(&p->pad16), padbytes.data(), padbytes.size())) return rc;
         }
-        if (Co == 32 || Co == 64)
+        if ((Co == 32 || Co == 64) && stem_fits)
         {
             // the same rows, end to end, as the K vector of the MFMA variant
             const int kp = (Kh * RD * 4 + 31) / 32 * 32;
@@ -382,6 +399,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         char buf[96];
         snprintf(buf, sizeof(buf), "smallci_dot4_lds %dx%dx%d stride %u, tile 32x16", Kh, Kw, Ci, d.stride_x);
         p->info = buf;
+        if (p->w_dot4b) p->info += ", weights minus their zero point as two int8 halves";
     }
     else
     {
@@ -758,7 +776,15 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
         if (nb > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
         const dim3 grid(static_cast<unsigned>(nb));
-        if (g.Kh == 3) hipLaunchKernelGGL((SmallCiConvKernel<3, 3>), grid, dim3(256), 0, stream, a);
+        a.wpack2 = p->w_dot4b;
+        if (p->w_dot4b)
+        {
+            if (g.Kh == 3) hipLaunchKernelGGL((SmallCiConvKernel<3, 3, true>), grid, dim3(256), 0, stream, a);
+            else if (g.Kh == 7) hipLaunchKernelGGL((SmallCiConvKernel<7, 6, true>), grid, dim3(256), 0, stream, a);
+            else if (g.Kh == 5) hipLaunchKernelGGL((SmallCiConvKernel<5, 5, true>), grid, dim3(256), 0, stream, a);
+            else hipLaunchKernelGGL((SmallCiConvKernel<1, 1, true>), grid, dim3(256), 0, stream, a);
+        }
+        else if (g.Kh == 3) hipLaunchKernelGGL((SmallCiConvKernel<3, 3>), grid, dim3(256), 0, stream, a);
         else if (g.Kh == 7) hipLaunchKernelGGL((SmallCiConvKernel<7, 6>), grid, dim3(256), 0, stream, a);
         else if (g.Kh == 5) hipLaunchKernelGGL((SmallCiConvKernel<5, 5>), grid, dim3(256), 0, stream, a);
         else hipLaunchKernelGGL((SmallCiConvKernel<1, 1>), grid, dim3(256), 0, stream, a);

@@ -8,7 +8,7 @@
 // per-channel constant (`corr`) that initialises the accumulators.  The depthwise kernel takes as "w" the difference
 // d = w - zw between a weight and the weights' zero point; where some d does not fit int8 (it lies in -255 .. 254) it is
 // the sum of two int8 halves, each in a packed array of its own (template W2), and costs a second v_dot4.  The stem
-// kernel needs symmetric int8 weights (offset 0).
+// kernel on v_dot4 does the same; its MFMA variant needs weights that fit one int8.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -223,6 +223,7 @@ struct SmallCiArgs
 {
     const uint8_t*  x;
     const uint32_t* wpack;    // [Co][KH][RD] dwords: row r of filter co as consecutive (kx, ci) bytes, zero padded
+    const uint32_t* wpack2;   // W2: the second halves, same layout
     ChanTab         ct;       // rows 2, 5, 6 on the fast path (accumulators start at zero), rows 0, 1 on the exact path
     const int32_t*  corr;     // [Co]
     uint8_t*        y;
@@ -372,7 +373,7 @@ __device__ __forceinline__ void StageSmallCiHalo(const SmallCiArgs& a, uint32_t*
     }
 }
 
-template <int KH, int RD>
+template <int KH, int RD, bool W2 = false>
 __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
 {
     constexpr int P = 2, TW = 16 * P, TH = 16;
@@ -414,6 +415,7 @@ __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
     const bool second = ox0 + 1 < a.Wo;
     uint8_t* yp = a.y + ((static_cast<long long>(n) * a.Ho + oy) * a.Wo + ox0) * a.Co;
     const uint32_t MI355X_CONST_AS* wc = AsConstant(a.wpack);
+    const uint32_t MI355X_CONST_AS* wc2 = AsConstant(W2 ? a.wpack2 : a.wpack);
     const float MI355X_CONST_AS* tab = AsConstant(a.ct.p);
     const int ts = a.ct.stride;
     for (int co = 0; co < a.Co; co += 16)
@@ -440,6 +442,12 @@ __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
                         const int wv = static_cast<int>(w[r * RD + i]);
 #pragma unroll
                         for (int p = 0; p < P; ++p) acc[p][u] = __builtin_amdgcn_sdot4(static_cast<int>(xr[p][r][i]), wv, acc[p][u], false);
+                        if constexpr (W2)
+                        {
+                            const int wv2 = static_cast<int>(wc2[(c + u) * (KH * RD) + r * RD + i]);
+#pragma unroll
+                            for (int p = 0; p < P; ++p) acc[p][u] = __builtin_amdgcn_sdot4(static_cast<int>(xr[p][r][i]), wv2, acc[p][u], false);
+                        }
                     }
             }
             const float4 fm = {tab[2 * ts + c], tab[2 * ts + c + 1], tab[2 * ts + c + 2], tab[2 * ts + c + 3]};

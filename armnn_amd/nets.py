@@ -82,8 +82,10 @@ class Network:
 
 
 class _Builder:
-    def __init__(self, name, seed, act_dtype):
-        self.name, self.seed, self.act_dtype = name, seed, act_dtype
+    def __init__(self, name, seed, act_dtype, weights="per_channel_s8"):
+        if weights not in ("per_channel_s8", "per_tensor_u8"):
+            raise ValueError(f"unknown weight quantization {weights!r}")
+        self.name, self.seed, self.act_dtype, self.weights = name, seed, act_dtype, weights
         self.tensors: Dict[str, TensorInfo] = {}
         self.layers: List[Layer] = []
         self._n = 0
@@ -91,6 +93,17 @@ class _Builder:
     def _next_seed(self):
         self._n += 1
         return self.seed * 1000 + self._n * 17
+
+    def _weights(self, s, wshape, ws, qdim):
+        """Synthetic weights and the scales the bias uses.  "per_channel_s8": QSymmS8, one scale per output channel.
+        "per_tensor_u8": QAsymmU8 with one scale and a zero point somewhere in 90..170, the quantization of older
+        uint8 models; the same draws, twice as wide, so that codes reach both ends of the range."""
+        if self.weights == "per_channel_s8":
+            return QTensor(TensorInfo(wshape, DataType.QSymmS8, tuple(ws), 0, qdim), synth.int8_weights(s + 1, wshape)), ws
+        zp = 90 + int(synth.uniform01(s + 4, 1, stream=5)[0] * 80.0)
+        one = np.asarray([np.float32(np.mean(ws) / 2.0)], np.float32)
+        codes = np.clip(2 * synth.int8_weights(s + 1, wshape).astype(np.int32) + zp, 0, 255).astype(np.uint8)
+        return QTensor(TensorInfo(wshape, DataType.QAsymmU8, tuple(one), zp, None), codes), one
 
     def tensor(self, name, shape, scale, offset, dtype=None):
         self.tensors[name] = TensorInfo(tuple(shape), dtype or self.act_dtype, (scale,), offset)
@@ -113,9 +126,9 @@ class _Builder:
         s = self._next_seed()
         u = 0.5 + synth.uniform01(s + 3, co, stream=3)
         ws = (u * G_TARGET / (30.0 * np.sqrt(taps) * r_in)).astype(np.float32)
-        wt = QTensor(TensorInfo(wshape, DataType.QSymmS8, tuple(ws), 0, qdim), synth.int8_weights(s + 1, wshape))
+        wt, ws = self._weights(s, wshape, ws, qdim)
         bs = (np.float32(xi.scale) * ws).astype(np.float32)
-        bt = QTensor(TensorInfo((co,), DataType.Signed32, tuple(bs), 0, 0), synth.int32_bias(s + 2, co))
+        bt = QTensor(TensorInfo((co,), DataType.Signed32, tuple(bs), 0, 0 if len(bs) > 1 else None), synth.int32_bias(s + 2, co))
         out = self.tensor(name + ":out", (1, ho, wo, co), out_scale, out_offset)
         params = dict(pad_top=pt, pad_left=pl, stride_x=stride, stride_y=stride, dilation_x=1, dilation_y=1,
                       depthwise=depthwise, _macs=ho * wo * co * taps)
@@ -128,9 +141,9 @@ class _Builder:
         s = self._next_seed()
         u = 0.5 + synth.uniform01(s + 3, o, stream=3)
         ws = (u * G_TARGET / (30.0 * np.sqrt(k) * r_in)).astype(np.float32)
-        wt = QTensor(TensorInfo((o, k), DataType.QSymmS8, tuple(ws), 0, 0), synth.int8_weights(s + 1, (o, k)))
+        wt, ws = self._weights(s, (o, k), ws, 0)
         bs = (np.float32(xi.scale) * ws).astype(np.float32)
-        bt = QTensor(TensorInfo((o,), DataType.Signed32, tuple(bs), 0, 0), synth.int32_bias(s + 2, o))
+        bt = QTensor(TensorInfo((o,), DataType.Signed32, tuple(bs), 0, 0 if len(bs) > 1 else None), synth.int32_bias(s + 2, o))
         out = self.tensor(name + ":out", (1, o), out_scale, out_offset)
         self.layers.append(Layer("fc", name, (x,), out, wt, bt, dict(transpose_weights=True, _macs=k * o)))
         return out
@@ -176,9 +189,10 @@ R_IMAGE = 0.58      # rms of uniform codes on [-1, 1]
 R_RELU = 1.4        # rms assumed for a ReLU/ReLU6 output whose pre-activation has std 2
 
 
-def mobilenet_v1(seed: int = 2025, resolution: int = 224, classes: int = 1001, width: float = 1.0) -> Network:
+def mobilenet_v1(seed: int = 2025, resolution: int = 224, classes: int = 1001, width: float = 1.0,
+                 weights: str = "per_channel_s8") -> Network:
     """MobileNetV1-1.0-224-style: stem 3x3/2 -> 32, 13 depthwise-separable blocks, avgpool, FC, softmax."""
-    b = _Builder(f"mobilenet_v1_{width}_{resolution}", seed, DataType.QAsymmU8)
+    b = _Builder(f"mobilenet_v1_{width}_{resolution}", seed, DataType.QAsymmU8, weights)
     x = b.tensor("input", (1, resolution, resolution, 3), float(np.float32(2.0 / 255.0)), 128)
     ch = lambda c: max(8, int(c * width))
     t = b.conv("stem", x, ch(32), 3, 2, RELU6_SCALE, 0, RELU6, R_IMAGE)

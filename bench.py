@@ -154,6 +154,9 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--net", default="mobilenet_v1", choices=["mobilenet_v1", "resnet50"])
+    ap.add_argument("--weights", default="per_channel_s8", choices=["per_channel_s8", "per_tensor_u8"],
+                    help="mobilenet_v1 only: per_tensor_u8 gives every layer QAsymmU8 weights with one scale and a zero point "
+                         "(the quantization of older uint8 models) instead of the headline workload's per-channel QSymmS8")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--fuse", action="store_true",
@@ -173,7 +176,7 @@ def main():
     from armnn_amd import nets, shim
     from armnn_amd.executor import DeviceNetwork
 
-    net = nets.mobilenet_v1() if args.net == "mobilenet_v1" else nets.resnet50()
+    net = nets.mobilenet_v1(weights=args.weights) if args.net == "mobilenet_v1" else nets.resnet50()
     batch = args.batch
     dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse, lanes=args.lanes)
     dn.upload_input(nets.synthetic_input(net, batch))
@@ -265,7 +268,7 @@ def main():
         "value": images_per_s, "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
-        "config": {"workload": f"{net.name} int8 (QAsymm activations, per-channel QSymmS8 weights), batch {batch}, "
+        "config": {"workload": f"{net.name} int8 (QAsymm activations, {'per-channel QSymmS8' if args.weights == 'per_channel_s8' or args.net != 'mobilenet_v1' else 'per-tensor QAsymmU8'} weights), batch {batch}, "
                                f"random-init, whole forward pass incl. avgpool/FC/softmax, input resident in HBM",
                    "batch": batch, "graph_replay": not args.no_graph, "fused_depthwise_pointwise": args.fuse, "lanes": args.lanes,
                    "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12},

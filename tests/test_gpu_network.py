@@ -183,3 +183,18 @@ def test_tflite_model_with_quantize_and_squeeze(port):
     from tests.test_tflite import quantize_squeeze_model
     net = tflite.parse(quantize_squeeze_model(), "qs")
     _layerwise(port, net, 2)
+
+
+def test_mobilenet_with_per_tensor_uint8_weights(port):
+    """Every layer's weights QAsymmU8 with one scale and a zero point: the stem and the depthwise layers multiply with the
+    weights minus their zero point in two int8 halves, the pointwise layers and the classifier sum their rows' activations."""
+    net = nets.mobilenet_v1(resolution=96, classes=50, weights="per_tensor_u8")
+    assert all(l.weights.info.dtype.name == "QAsymmU8" and l.weights.info.offset != 128 for l in net.layers if l.weights is not None)
+    _layerwise(port, net, 3)
+    dn = DeviceNetwork(net, 3, use_graph=False, fuse=False)
+    kinds = {l.name: p.algo()[1] for (l, _), p in zip(dn.steps, dn._step_plans) if p is not None}
+    dn.close()
+    print(kinds, flush=True)
+    assert "two int8 halves" in kinds["stem"] and "smallci_dot4" in kinds["stem"]
+    assert all("depthwise3x3_dot4" in k for n, k in kinds.items() if n.startswith("dw"))
+    assert all("weight zero point by row sums" in k for n, k in kinds.items() if n.startswith("pw") or n == "logits")

@@ -446,3 +446,34 @@ def test_depthwise_weight_255_above_its_zero_point_takes_the_general_kernel(port
     want = _oracle_conv(port, case)
     got = _gpu_conv(case, shim.ALGO_AUTO)
     assert lsb_diff(got.data, want.data)[0] <= 1
+
+
+_ZP_STEMS = [
+    ("u8_3x3_s2_rgb_two_halves", dict(n=2, h=33, w=35, ci=3, co=32, kh=3, kw=3, stride=(2, 2), w_dtype=DataType.QAsymmU8, w_offset=151, w_std=70.0), True),
+    ("u8_3x3_s2_rgb_fits", dict(n=2, h=32, w=32, ci=3, co=32, kh=3, kw=3, stride=(2, 2), w_dtype=DataType.QAsymmU8, w_offset=128, w_std=30.0), False),
+    ("u8_7x7_s2_rgb", dict(n=1, h=40, w=40, ci=3, co=64, kh=7, kw=7, stride=(2, 2), w_dtype=DataType.QAsymmU8, w_offset=60, w_std=70.0), True),
+    ("s8_5x5_grey", dict(n=3, h=21, w=19, ci=1, co=8, kh=5, kw=5, stride=(1, 1), w_dtype=DataType.QAsymmS8, w_offset=-50, w_std=70.0), True),
+    ("s8_1x1_rgba", dict(n=2, h=16, w=16, ci=4, co=16, kh=1, kw=1, stride=(1, 1), w_dtype=DataType.QAsymmS8, w_offset=9, w_std=20.0), False),
+]
+
+
+@pytest.mark.parametrize("in_u8", [False, True], ids=["s8_in", "u8_in"])
+@pytest.mark.parametrize("name,kw,halves", _ZP_STEMS, ids=[n for n, _, _ in _ZP_STEMS])
+def test_stem_weights_with_a_zero_point(port, name, kw, halves, in_u8):
+    """Convolutions with at most 4 input channels whose per-tensor weights have a zero point stay on the v_dot4 stem kernel."""
+    seed = 34000 + 5 * [n for n, _, _ in _ZP_STEMS].index(name) + int(in_u8)
+    case = cases.make_conv_case(name, seed, padding="same", per_axis=False, in_dtype=DataType.QAsymmU8 if in_u8 else DataType.QAsymmS8,
+                                in_offset=128 if in_u8 else -1, out_offset=0 if in_u8 else -128, act=(2, 6.0, 0.0), **kw)
+    fn, a, b = case.act
+    plan = shim.Conv2dPlan(case.x.info, case.w, case.b, case.out_info, activation=fn, act_a=a, act_b=b, algo=shim.ALGO_AUTO, **case.params)
+    algo, desc = plan.algo()
+    plan.destroy()
+    print(f"{name}: x={case.x.info.shape} zw={case.w.info.offset} kernel: {desc}", flush=True)
+    assert algo == shim.ALGO_DOT4
+    assert ("two int8 halves" in desc) == halves
+    want = _oracle_conv(port, case)
+    auto = _gpu_conv(case, shim.ALGO_AUTO)
+    mx, exact = lsb_diff(auto.data, want.data)
+    print(f"  max|d|={mx} exact={exact:.5f}", flush=True)
+    assert mx <= 1 and exact >= 0.99
+    np.testing.assert_array_equal(auto.data, _gpu_conv(case, shim.ALGO_DIRECT).data)
