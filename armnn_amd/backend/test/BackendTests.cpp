@@ -819,6 +819,27 @@ TEST_CASE("runtime: pointwise Convolution2d, per-tensor weights, QAsymmU8", "gpu
     CheckSingleLayer(MakeConv(QLayer::Conv, ActInfo({3, 14, 14, 64}, DataType::QAsymmU8, 0.0235f, 120), 128, 1, 1, 0.03f, 110, false, false, 102), 2, "conv1x1-u8");
 }
 
+namespace
+{
+// the same layer with per-tensor QAsymmU8 weights: every code moved up by the zero point
+QLayer WithUint8Weights(QLayer l, int zeroPoint)
+{
+    l.w = TensorInfo(l.w.GetShape(), DataType::QAsymmU8, l.wScales[0], zeroPoint, true);
+    for (auto& v : l.weights) v = static_cast<int8_t>(static_cast<uint8_t>(std::min(255, std::max(0, static_cast<int>(v) + zeroPoint))));
+    return l;
+}
+} // namespace
+
+TEST_CASE("runtime: per-tensor QAsymmU8 weights with a zero point: Convolution2d, DepthwiseConvolution2d, stem, FullyConnected", "gpu")
+{
+    const TensorInfo in = ActInfo({2, 21, 17, 32}, DataType::QAsymmU8, 0.0235f, 119);
+    CheckSingleLayer(WithUint8Weights(MakeConv(QLayer::Conv, in, 64, 3, 1, 0.03f, 7, true, false, 141), 93), 11, "conv3x3 zw=93");
+    CheckSingleLayer(WithUint8Weights(MakeConv(QLayer::Conv, in, 48, 1, 1, 0.03f, 7, false, false, 142), 160), 12, "conv1x1 zw=160");
+    CheckSingleLayer(WithUint8Weights(MakeConv(QLayer::Depthwise, in, 32, 3, 2, 0.03f, 7, true, false, 143), 93), 13, "depthwise zw=93");
+    CheckSingleLayer(WithUint8Weights(MakeConv(QLayer::Conv, ActInfo({2, 30, 30, 3}, DataType::QAsymmU8, 0.0078f, 128), 32, 3, 2, 0.0235f, 0, true, false, 144), 151), 14, "stem zw=151");
+    CheckSingleLayer(WithUint8Weights(MakeFc(ActInfo({5, 256}, DataType::QAsymmU8, 0.02f, 63), 100, 0.25f, 30, false, 145), 93), 15, "fc zw=93");
+}
+
 TEST_CASE("runtime: stem Convolution2d with 3 input channels", "gpu")
 {
     CheckSingleLayer(MakeConv(QLayer::Conv, ActInfo({2, 32, 32, 3}, DataType::QAsymmS8, 0.0078f, 0), 32, 3, 2, 0.0235f, -128, true, true, 103), 3, "stem");
