@@ -41,6 +41,7 @@ struct mi355x_conv2d_s
     int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 96 (= 128x64) / 128: the "igemm_tile" option at plan creation
     uint32_t xor_mask = 0, pad_word = 0;
     int zw_neg = 0;                // MFMA plans: minus the zero point of the stored int8 weights (0: symmetric)
+    int rowsum_bias = 0;           // ... and what the bytes between K and K_pad add to a row's sum of activations
     std::string info;
 
     ~mi355x_conv2d_s()
@@ -265,11 +266,12 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
                 dst[k] = g.w_u8 ? static_cast<int8_t>(static_cast<uint8_t>(src[k]) ^ 0x80u) : src[k];
                 sum += dst[k];
             }
-            // sum_k (x' - zx')(w - zw') = sum_k x'w - zx' sum_k w - zw' sum_k x' + K_pad zx' zw' over the padded row, whose bytes
-            // beyond K and outside the image are zx' against zero weights; the term with sum_k x' is the kernel's
-            corr[c] = static_cast<int32_t>(-static_cast<long long>(zx_shift) * sum + static_cast<long long>(zw_shift) * zx_shift * p->K_pad);
+            // sum_k (x' - zx')(w - zw') = sum_k x'w - zx' sum_k w - zw' sum_k x' + K zx' zw' over the K bytes of a row, of which
+            // those outside the image are zx'; the term with sum_k x' is the kernel's
+            corr[c] = static_cast<int32_t>(-static_cast<long long>(zx_shift) * sum + static_cast<long long>(zw_shift) * zx_shift * p->K);
         }
         p->zw_neg = -zw_shift;
+        p->rowsum_bias = (p->K_pad - p->K) * zx_shift;     // kernels that walk K_pad bytes meet zx' beyond K
         if (int rc = Upload(reinterpret_cast<void**>(&p->w_mfma), wp.data(), wp.size())) return rc;
         if (int rc = Upload(reinterpret_cast<void**>(&p->corr), corr.data(), corr.size() * sizeof(int32_t))) return rc;
         p->xor_mask = g.in_u8 ? 0x80808080u : 0u;
@@ -283,18 +285,16 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         FoldCorrIntoTable(p, corr, Co);
         ChoosePointwiseConfig(p);
         if (p->tile_override != 0) p->pw_bn = 0;     // a forced tile also forces the LDS-tiled implicit GEMM
-        if (p->zw_neg != 0) p->pw_bn = 0;            // only the implicit GEMM sums the activations a weight zero point needs
         if (int rc = PreparePointwise(p)) return rc;
         char buf[128];
-        if (p->zw_neg != 0)
-            snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 tiles 128x128|128x64|64x64 x%d K=%d, weight zero point by row sums", p->bk128 ? 128 : 64, p->K);
-        else if (p->pw_bn)
+        if (p->pw_bn)
             snprintf(buf, sizeof(buf), "pointwise_gemm_mfma_i8_32x32x32 weight-stationary slab %dxK=%d, chunk %d k-steps", p->pw_bn, p->K, p->pw_ks);
         else if (p->bk128 && (Ci % 128) == 0)
             snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 global_load_lds tiles 64x64..256x256 x128 K=%d", p->K);
         else
             snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 tiles 128x128|128x64|64x64 x%d K=%d", p->bk128 ? 128 : 64, p->K);
         p->info = buf;
+        if (p->zw_neg != 0) p->info += ", weight zero point by row sums";
     }
     else if (algo == MI355X_ALGO_DEPTHWISE && dw3_ok)
     {
@@ -471,7 +471,7 @@ void ChoosePointwiseConfig(mi355x_conv2d_s* p)
 template <int BN, int KS>
 int PreparePw(mi355x_conv2d_s* p)
 {
-    auto kernel = PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2)>;
+    auto kernel = p->zw_neg != 0 ? PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2), true> : PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2), false>;
     MI355X_HIP(hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024));
     int per_cu = 1, dev = 0, n_cu = 256;
     MI355X_HIP(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel, 256, PwSmemBytes<BN>(p->geom.Ci)));
@@ -518,9 +518,10 @@ int LaunchPw(const mi355x_conv2d_s* p, long long M, const void* x, void* y, hipS
     a.w_stride = p->K_pad;
     a.n_slabs = (g.Co + BN - 1) / BN;
     a.xor_mask = p->xor_mask;
+    a.zw_neg = p->zw_neg;
     a.rq = p->rq;
     const int smem = PwSmemBytes<BN>(g.Ci);
-    auto kernel = PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2)>;
+    auto kernel = p->zw_neg != 0 ? PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2), true> : PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2), false>;
     const int n_cu = p->pw_n_cu, cached_per_cu = p->pw_blocks_per_cu;      // queried once, when the plan was built
     // exactly one resident wave of blocks: every block walks its share of the row tiles
     const long long groups = ((M + 31) / 32 + 3) / 4;
@@ -588,6 +589,7 @@ int LaunchIgemmT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* 
     a.xor_mask = p->xor_mask;
     a.pad_word = p->pad_word;
     a.zw_neg = p->zw_neg;
+    a.rowsum_bias = p->rowsum_bias;
     a.rq = p->rq;
     const int nblocks = a.tiles_m * a.tiles_n;
     const int grid = (nblocks + 7) / 8 * 8;
@@ -600,7 +602,7 @@ int LaunchIgemmT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* 
     return 0;
 }
 
-template <int BM, int BN, int WM, int WN, int ST, bool U8>
+template <int BM, int BN, int WM, int WN, int ST, bool U8, bool AW>
 int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
 {
     const ConvGeom& g = p->geom;
@@ -626,15 +628,16 @@ int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, voi
     a.tiles_n = (g.Co + BN - 1) / BN;
     a.xor_mask = p->xor_mask;
     a.pad_word = p->pad_word;
-    a.zw_neg = 0;
+    a.zw_neg = p->zw_neg;
+    a.rowsum_bias = p->rowsum_bias;
     a.rq = p->rq;
     const int nblocks = a.tiles_m * a.tiles_n;
     const int grid = (nblocks + 7) / 8 * 8;
     constexpr int smem = IgemmLdsSmemBytes<BM, BN, ST>();
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmLdsKernel<BM, BN, WM, WN, ST, U8>),
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmLdsKernel<BM, BN, WM, WN, ST, U8, AW>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);
-    hipLaunchKernelGGL((IgemmLdsKernel<BM, BN, WM, WN, ST, U8>), dim3(grid), dim3(64 * WM * WN), smem, stream, a);
+    hipLaunchKernelGGL((IgemmLdsKernel<BM, BN, WM, WN, ST, U8, AW>), dim3(grid), dim3(64 * WM * WN), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;
 }
@@ -646,10 +649,16 @@ int LaunchIgemmLds(const mi355x_conv2d_s* p, int stages, uint32_t batch, const v
     if constexpr (3 * (BM + BN) * 128 <= 160 * 1024)
     {
         if (stages == 3)
-            return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 3, true>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 3, false>(p, batch, x, y, stream);
+        {
+            if (p->zw_neg != 0)
+                return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 3, true, true>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 3, false, true>(p, batch, x, y, stream);
+            return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 3, true, false>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 3, false, false>(p, batch, x, y, stream);
+        }
     }
 
-    return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 2, true>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 2, false>(p, batch, x, y, stream);
+    if (p->zw_neg != 0)
+        return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 2, true, true>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 2, false, true>(p, batch, x, y, stream);
+    return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 2, true, false>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 2, false, false>(p, batch, x, y, stream);
 }
 
 int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
@@ -721,7 +730,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const int tile = p->tile_override ? p->tile_override : big < 400 ? 64 : (huge >= 192 && g.Co >= 256) ? 512 : 128;
         // channel counts that are multiples of 128: k-tiles go from global memory straight into LDS
         const int lds_stages = GlobalOptions().igemm_lds;
-        if (lds_stages != 0 && bk128 && (g.Ci % 128) == 0 && p->zw_neg == 0)
+        if (lds_stages != 0 && bk128 && (g.Ci % 128) == 0)
         {
             if (tile == 64)
             {

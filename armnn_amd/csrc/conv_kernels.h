@@ -150,7 +150,8 @@ __global__ __launch_bounds__(256) void DepthwiseC4Kernel(ConvGeom g, Requant rq,
 //
 //   Weights with a zero point (template AW): w' = w - zw' with the stored int8 w, so
 //   sum (x' - zx')(w - zw') = sum x'w + corr[c] - zw' * S[m],  S[m] = sum_k x'[m][k] over the whole padded K row
-//   (bytes outside the image and beyond K are zx', which corr accounts for).  S[m] is summed with v_dot4 from the
+//   (bytes outside the image are zx', which corr accounts for; those beyond K, zx' as well, are taken off again as the
+//   constant `rowsum_bias`).  S[m] is summed with v_dot4 from the
 //   activation fragments a lane reads for the MFMA anyway -- the two lanes that hold the halves of a pixel's k-slice
 //   add up at the end -- and enters the accumulators just before they are requantized.
 //
@@ -178,6 +179,7 @@ struct IgemmArgs
     uint32_t xor_mask;      // 0x80808080 for uint8 input, else 0
     uint32_t pad_word;      // shifted input zero point replicated in 4 bytes
     int zw_neg;             // minus the zero point of the stored int8 weights (0: symmetric)
+    int rowsum_bias;        // (K_pad - K) * zx': what the bytes beyond K add to a row sum
     Requant rq;
 };
 
@@ -415,7 +417,7 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
     {
         // lanes l and l ^ 32 hold the two halves of every k-slice of pixel (l & 31)
 #pragma unroll
-        for (int tp = 0; tp < TP; ++tp) rowsum[tp] = (rowsum[tp] + __shfl_xor(rowsum[tp], 32)) * a.zw_neg;
+        for (int tp = 0; tp < TP; ++tp) rowsum[tp] = (rowsum[tp] + __shfl_xor(rowsum[tp], 32) - a.rowsum_bias) * a.zw_neg;
     }
 #pragma unroll
     for (int tc = 0; tc < TC; ++tc)

@@ -39,7 +39,8 @@ constexpr int VmcntImm(int n)
 }
 
 // WM x WN waves per block (4, 8 or 16), each with a (BM / WM) x (BN / WN) tile of the block tile.
-template <int BM, int BN, int WM, int WN, int ST, bool U8>
+// AW: the weights have a zero point; each pixel's activations are summed beside the products (see IgemmKernel).
+template <int BM, int BN, int WM, int WN, int ST, bool U8, bool AW = false>
 __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
 {
     static_assert(ST >= 2 && ST <= 8, "2 to 8 LDS stages");
@@ -166,6 +167,9 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
     const int frag_row = lane & 31;
     const int frag_half = lane >> 5;
     const int xm = static_cast<int>(a.xor_mask);
+    int rowsum[TP];
+#pragma unroll
+    for (int tp = 0; tp < TP; ++tp) rowsum[tp] = 0;
 
     auto compute = [&](int stage) {
         const uint8_t* As = smem + stage * STAGE;
@@ -181,6 +185,11 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
             {
                 fa[tp] = *reinterpret_cast<const v4i*>(As + (wm * WTM + tp * 32 + frag_row) * BK + slot);
                 if (U8) fa[tp] ^= xm;
+                if constexpr (AW)
+                {
+#pragma unroll
+                    for (int i = 0; i < 4; ++i) rowsum[tp] = __builtin_amdgcn_sdot4(fa[tp][i], 0x01010101, rowsum[tp], false);
+                }
             }
 #pragma unroll
             for (int tc = 0; tc < TC; ++tc)
@@ -223,6 +232,11 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
 
     // ---- epilogue: requantize, pack 4 channels per dword, stage the byte tile in LDS, coalesced write-out -----------
     uint8_t* Os = smem;
+    if constexpr (AW)
+    {
+#pragma unroll
+        for (int tp = 0; tp < TP; ++tp) rowsum[tp] = (rowsum[tp] + __shfl_xor(rowsum[tp], 32) - a.rowsum_bias) * a.zw_neg;
+    }
 #pragma unroll
     for (int tc = 0; tc < TC; ++tc)
     {
@@ -235,7 +249,8 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
             for (int tp = 0; tp < TP; ++tp)
             {
                 const v16i& c = acc[tc][tp];
-                const uint32_t out = Requant4Dev(c[4 * q + 0], c[4 * q + 1], c[4 * q + 2], c[4 * q + 3], f4, a.ct, tn * BN + cl, a.rq);
+                const int rt = AW ? rowsum[tp] : 0;
+                const uint32_t out = Requant4Dev(c[4 * q + 0] + rt, c[4 * q + 1] + rt, c[4 * q + 2] + rt, c[4 * q + 3] + rt, f4, a.ct, tn * BN + cl, a.rq);
                 const int pl = wm * WTM + tp * 32 + (lane & 31);
                 *reinterpret_cast<uint32_t*>(Os + pl * LDO + cl) = out;
             }

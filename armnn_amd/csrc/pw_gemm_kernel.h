@@ -36,6 +36,7 @@ struct PwArgs
     int w_stride;
     int n_slabs, gm;         // grid = n_slabs * gm blocks; block (slab, g) takes tile groups g, g+gm, ...
     uint32_t xor_mask;
+    int zw_neg;              // AW: minus the zero point of the stored int8 weights
     Requant rq;
 };
 
@@ -46,7 +47,9 @@ constexpr int PwSmemBytes(int K)
 }
 
 // KS = MFMA k-steps (of 32) per register chunk, K % (32 * KS) == 0;  NB = register chunks per wave (NB-1 in flight).
-template <int BN, int KS, int NB>
+// AW: the weights have a zero point zw'; a lane sums the activation bytes it feeds to the MFMAs (v_dot4 with ones), the two
+// lanes holding the halves of a row's k-slices add up, and -zw' times that sum joins the row's accumulators.
+template <int BN, int KS, int NB, bool AW = false>
 __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
 {
     constexpr int TC = BN / 32;
@@ -79,6 +82,7 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
     const int tile0 = g * 4 + wave;              // first tile of this wave
 
     v16i acc[TC];
+    int rowsum = 0;
 
     auto load_chunk = [&](v4i (&buf)[KS], int t, int ch) {
         // rows past the end re-read the last row (their results are never stored): no load depends on a branch
@@ -97,6 +101,12 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
         for (int ks = 0; ks < KS; ++ks)
         {
             const v4i av = buf[ks] ^ xm;
+            if constexpr (AW)
+            {
+                if (FIRST && ks == 0) rowsum = 0;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) rowsum = __builtin_amdgcn_sdot4(av[i], 0x01010101, rowsum, false);
+            }
 #pragma unroll
             for (int tc = 0; tc < TC; ++tc)
             {
@@ -108,6 +118,8 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
 
     auto epilogue = [&](int t) {
         const int lane_c = 4 * (lane >> 5);
+        int rt = 0;
+        if constexpr (AW) rt = (rowsum + __shfl_xor(rowsum, 32)) * a.zw_neg;
 #pragma unroll
         for (int tc = 0; tc < TC; ++tc)
         {
@@ -118,7 +130,7 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
                 const float4 fm = *reinterpret_cast<const float4*>(cst + cl);
                 const float4 fb = *reinterpret_cast<const float4*>(cst + BN + cl);
                 const float4 th = *reinterpret_cast<const float4*>(cst + 2 * BN + cl);
-                const uint32_t out = Requant4Dev(acc[tc][4 * q + 0], acc[tc][4 * q + 1], acc[tc][4 * q + 2], acc[tc][4 * q + 3],
+                const uint32_t out = Requant4Dev(acc[tc][4 * q + 0] + rt, acc[tc][4 * q + 1] + rt, acc[tc][4 * q + 2] + rt, acc[tc][4 * q + 3] + rt,
                                                  fm, fb, th, a.ct, a.corr, n0 + cl, a.rq);
                 *reinterpret_cast<uint32_t*>(ostage + frag_row * LDO + cl) = out;
             }
