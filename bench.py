@@ -5,7 +5,10 @@ A step is one forward pass of the whole network over one batch that is already r
 runs on the device through the C ABI; the pass is replayed as one HIP graph).  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 64] [--net mobilenet_v1|resnet50]
-                  [--no-cpu-baseline] [--layers]
+                  [--weights per_channel_s8|per_tensor_u8] [--no-cpu-baseline] [--layers]
+
+The headline workload is the default: per-channel QSymmS8 weights.  --weights per_tensor_u8 runs the same network with
+QAsymmU8 weights that have one scale and a zero point per layer, and says so in config.workload.
 
 Extra objects in the line:
   roofline      the kernel with the largest share of the step (HIP-event timed on the launch stream)
