@@ -680,12 +680,12 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const long long rows = static_cast<long long>(batch) * g.Ho * g.Wo;
         const bool unit = dd.kernel_h == 1 && dd.kernel_w == 1 && dd.stride_x == 1 && dd.stride_y == 1 && dd.pad_top == 0 &&
                           dd.pad_left == 0 && dd.out_h == dd.in_h && dd.out_w == dd.in_w;
-        if (unit && rows <= 4 && (g.Ci % 16) == 0 && p->tile_override == 0 && p->zw_neg == 0)
+        if (unit && rows <= 4 && (g.Ci % 16) == 0 && p->tile_override == 0)
         {
             // a handful of rows: stream the weights once, no tiles
             GemvArgs a;
             a.x = xin; a.w = p->w_mfma; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
-            a.M = static_cast<int>(rows); a.K = g.Ci; a.N = g.Co; a.w_stride = p->K_pad; a.xor_mask = p->xor_mask; a.rq = p->rq;
+            a.M = static_cast<int>(rows); a.K = g.Ci; a.N = g.Co; a.w_stride = p->K_pad; a.xor_mask = p->xor_mask; a.zw_neg = p->zw_neg; a.rq = p->rq;
             const dim3 grid(static_cast<unsigned>((g.Co + 15) / 16));
             switch (a.M)
             {
@@ -697,13 +697,13 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             MI355X_HIP(hipGetLastError());
             return 0;
         }
-        if (unit && rows <= 64 && (g.Ci % 16) == 0 && g.Ci >= 128 && p->tile_override == 0 && p->zw_neg == 0 && p->Co_pad >= (g.Co + 31) / 32 * 32 &&
+        if (unit && rows <= 64 && (g.Ci % 16) == 0 && g.Ci >= 128 && p->tile_override == 0 && p->Co_pad >= (g.Co + 31) / 32 * 32 &&
             (reinterpret_cast<uintptr_t>(y) & 3) == 0)
         {
             // a few dozen rows: 32x32 tiles with K split over the block's waves
             GemvArgs a;
             a.x = xin; a.w = p->w_mfma; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
-            a.M = static_cast<int>(rows); a.K = g.Ci; a.N = g.Co; a.w_stride = p->K_pad; a.xor_mask = p->xor_mask; a.rq = p->rq;
+            a.M = static_cast<int>(rows); a.K = g.Ci; a.N = g.Co; a.w_stride = p->K_pad; a.xor_mask = p->xor_mask; a.zw_neg = p->zw_neg; a.rq = p->rq;
             const dim3 grid(static_cast<unsigned>((g.Co + 31) / 32), static_cast<unsigned>((rows + 31) / 32));
             if (g.Ci <= 512) hipLaunchKernelGGL(SmallMGemmKernel<4>, grid, dim3(256), 0, stream, a);
             else hipLaunchKernelGGL(SmallMGemmKernel<8>, grid, dim3(256), 0, stream, a);

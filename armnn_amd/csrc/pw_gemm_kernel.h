@@ -244,6 +244,8 @@ struct GemvArgs
     uint8_t*       y;        // [M][N]
     int M, K, N, w_stride;
     uint32_t xor_mask;
+    int zw_neg;              // minus the zero point of the stored int8 weights; when not 0 every row's activations are summed
+                             // as well and zw_neg times that sum joins the row's accumulators
     Requant rq;
 };
 
@@ -256,11 +258,13 @@ __global__ __launch_bounds__(256) void GemvKernel(GemvArgs a)
     const int n0 = (static_cast<int>(blockIdx.x) * 4 + wave) * R;
     if (n0 >= a.N) return;
     const int xm = static_cast<int>(a.xor_mask);
-    int acc[R][MR];
+    int acc[R][MR], xs[MR];
 #pragma unroll
     for (int r = 0; r < R; ++r)
 #pragma unroll
         for (int m = 0; m < MR; ++m) acc[r][m] = 0;
+#pragma unroll
+    for (int m = 0; m < MR; ++m) xs[m] = 0;
     const int chunks = a.K >> 4;
     const int8_t* wrow = a.w + static_cast<long long>(n0) * a.w_stride;
 #pragma unroll 4
@@ -269,6 +273,13 @@ __global__ __launch_bounds__(256) void GemvKernel(GemvArgs a)
         v4i xv[MR];
 #pragma unroll
         for (int m = 0; m < MR; ++m) xv[m] = *reinterpret_cast<const v4i*>(a.x + static_cast<long long>(m) * a.K + j * 16) ^ xm;
+        if (a.zw_neg != 0)       // uniform
+        {
+#pragma unroll
+            for (int m = 0; m < MR; ++m)
+#pragma unroll
+                for (int d = 0; d < 4; ++d) xs[m] = __builtin_amdgcn_sdot4(xv[m][d], 0x01010101, xs[m], false);
+        }
 #pragma unroll
         for (int r = 0; r < R; ++r)
         {
@@ -277,6 +288,16 @@ __global__ __launch_bounds__(256) void GemvKernel(GemvArgs a)
             for (int m = 0; m < MR; ++m)
 #pragma unroll
                 for (int d = 0; d < 4; ++d) acc[r][m] = __builtin_amdgcn_sdot4(xv[m][d], wv[d], acc[r][m], false);
+        }
+    }
+    if (a.zw_neg != 0)
+    {
+#pragma unroll
+        for (int m = 0; m < MR; ++m)
+        {
+            xs[m] *= a.zw_neg;           // joins every channel's sum below, lane by lane
+#pragma unroll
+            for (int r = 0; r < R; ++r) acc[r][m] += xs[m];
         }
     }
 #pragma unroll
@@ -300,6 +321,7 @@ template <int UN>
 __global__ __launch_bounds__(256) void SmallMGemmKernel(GemvArgs a)
 {
     __shared__ int part[4][16][64];
+    __shared__ int rowpart[4][64];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
     const int n0 = static_cast<int>(blockIdx.x) * 32;
@@ -313,6 +335,7 @@ __global__ __launch_bounds__(256) void SmallMGemmKernel(GemvArgs a)
     const uint8_t* xp = a.x + static_cast<long long>(min(m0 + frag_row, a.M - 1)) * a.K;
     const int8_t* wp = a.w + static_cast<long long>(n0 + frag_row) * a.w_stride + frag_k;
     v16i acc = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0};
+    int xs = 0;
     for (int s0 = wave; s0 < steps; s0 += 4 * UN)
     {
         v4i xv[UN], wv[UN];
@@ -329,8 +352,16 @@ __global__ __launch_bounds__(256) void SmallMGemmKernel(GemvArgs a)
             const v4i zero = {0, 0, 0, 0};
             const v4i wu = (s0 + 4 * u < steps) ? wv[u] : zero;      // steps past the end (clamped above) add nothing
             acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wu, xv[u] ^ xm, acc, 0, 0, 0);
+            // the row's sum counts a lane's 16 bytes only where they are bytes of the row that no other step covers
+            if (a.zw_neg != 0 && s0 + 4 * u < steps && (s0 + 4 * u) * 32 + frag_k + 16 <= a.K)
+            {
+                const v4i xb = xv[u] ^ xm;
+#pragma unroll
+                for (int d = 0; d < 4; ++d) xs = __builtin_amdgcn_sdot4(xb[d], 0x01010101, xs, false);
+            }
         }
     }
+    rowpart[wave][lane] = xs;
 #pragma unroll
     for (int i = 0; i < 16; ++i) part[wave][i][lane] = acc[i];
     __syncthreads();
@@ -338,6 +369,15 @@ __global__ __launch_bounds__(256) void SmallMGemmKernel(GemvArgs a)
 #pragma unroll
     for (int i = 0; i < 4; ++i)
         v[i] = part[0][4 * wave + i][lane] + part[1][4 * wave + i][lane] + part[2][4 * wave + i][lane] + part[3][4 * wave + i][lane];
+    if (a.zw_neg != 0)
+    {
+        // the four waves split the k-steps and the two lanes of a row the halves of each step
+        int total = 0;
+#pragma unroll
+        for (int w = 0; w < 4; ++w) total += rowpart[w][frag_row] + rowpart[w][frag_row + 32];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) v[i] += total * a.zw_neg;
+    }
     // accumulator group g of the 32x32 tile: channels 8 g + 4 (lane / 32) + 0..3 of row lane % 32
     const int c = n0 + 8 * wave + 4 * (lane >> 5);
     const int row = m0 + frag_row;

@@ -384,12 +384,14 @@ def test_weights_with_a_zero_point_on_the_matrix_cores(port, name, kw, in_u8):
     np.testing.assert_array_equal(auto.data, _gpu_conv(case, shim.ALGO_DIRECT).data)
 
 
-@pytest.mark.parametrize("m", [1, 3, 40, 256])
+@pytest.mark.parametrize("m", [1, 3, 4, 40, 64, 256])
+@pytest.mark.parametrize("k", [512, 400], ids=["k512", "k400_half_last_step"])
 @pytest.mark.parametrize("w_dtype,w_offset", [(DataType.QAsymmU8, 93), (DataType.QAsymmS8, -30)])
-def test_fully_connected_weights_with_a_zero_point(port, m, w_dtype, w_offset):
-    case = cases.make_fc_case(f"fc_zp_m{m}", 32000 + m, m=m, k=512, o=320, in_dtype=DataType.QAsymmU8, in_offset=63, w_dtype=w_dtype,
+def test_fully_connected_weights_with_a_zero_point(port, m, k, w_dtype, w_offset):
+    """Rows from one (matrix-vector kernel) over a few dozen (32x32 tiles with K split over the waves) to the tiled GEMM."""
+    case = cases.make_fc_case(f"fc_zp_m{m}", 32000 + m + k, m=m, k=k, o=320, in_dtype=DataType.QAsymmU8, in_offset=63, w_dtype=w_dtype,
                               per_axis=False, w_offset=w_offset, out_offset=30)
-    print(f"fc m={m} {w_dtype.name} zw={w_offset}", flush=True)
+    print(f"fc m={m} k={k} {w_dtype.name} zw={w_offset}", flush=True)
     kw = dict(transpose_weights=case.transpose_weights)
     want = port.fully_connected(case.x, case.w, case.b, case.out_info, **kw)
     auto = shim.fully_connected(case.x, case.w, case.b, case.out_info, algo=shim.ALGO_AUTO, **kw)
