@@ -218,7 +218,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         }
     }
     const bool dw3_ok = dw_ok && zw_shift >= -128 && zw_shift <= 127 && zx_shift >= -128 && zx_shift <= 127 && dw3_halves && Kh == 3 &&
-                        Kw == 3 && (Co % 32) == 0 && d.dilation_x == 1 && d.dilation_y == 1 && d.stride_x == d.stride_y &&
+                        Kw == 3 && (Co % 16) == 0 && d.dilation_x == 1 && d.dilation_y == 1 && d.stride_x == d.stride_y &&
                         (d.stride_x == 1 || d.stride_x == 2);
     // stems: <= 4 input channels, rows of Kw*Ci bytes walked with v_dot4
     const int row_bytes = Kw * Ci;
@@ -299,8 +299,10 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     else if (algo == MI355X_ALGO_DEPTHWISE && dw3_ok)
     {
         // [1][3][3][C] -> per channel 4 dwords, dword r = { w[r][0], w[r][1], w[r][2], 0 }
-        std::vector<uint32_t> wp(static_cast<size_t>(Co) * 4, 0u), wp2(static_cast<size_t>(Co) * 4, 0u);
-        std::vector<int32_t> corr(Co, 0);
+        // the kernel works in blocks of 32 channels: its per-channel arrays are padded to whole blocks
+        const int C32 = (Co + 31) / 32 * 32;
+        std::vector<uint32_t> wp(static_cast<size_t>(C32) * 4, 0u), wp2(static_cast<size_t>(C32) * 4, 0u);
+        std::vector<int32_t> corr(C32, 0);
         for (int c = 0; c < Co; ++c)
         {
             long long sum = 0;
@@ -815,7 +817,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             const int opt_r = GlobalOptions().dw_rows;
             const int rows_per_thread = opt_r ? opt_r : ((g.Ho + 15) / 16 * 16 - g.Ho) * 4 <= g.Ho ? 2 : 1;
             const int th = 8 * rows_per_thread;
-            a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + th - 1) / th; a.cblocks = g.Co / 32;
+            a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + th - 1) / th; a.cblocks = (g.Co + 31) / 32;
             a.xor_mask = p->xor_mask; a.pad_word = p->pad_word; a.rq = p->rq;
             const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y * a.cblocks;
             if (nb > 0x7fffffffll - 8) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
@@ -919,7 +921,7 @@ int mi355x_conv2d_fusable(mi355x_conv2d_t dw, mi355x_conv2d_t pw)
     if (!dw || !pw) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
     const mi355x_conv2d_desc& a = dw->d;
     const mi355x_conv2d_desc& b = pw->d;
-    if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || !dw->dw_grp || dw->w_dot4b)
+    if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || !dw->dw_grp || dw->w_dot4b || (dw->d.out_c % 32) != 0)
         return SetError(MI355X_ERR_UNSUPPORTED, "first plan is not a 3x3 depthwise layer on the v_dot4 kernel");
     const bool pointwise = pw->algo == MI355X_ALGO_MFMA && !b.depthwise && b.kernel_h == 1 && b.kernel_w == 1 && b.stride_x == 1 &&
                            b.stride_y == 1 && b.pad_top == 0 && b.pad_left == 0 && b.out_h == b.in_h && b.out_w == b.in_w;

@@ -1,6 +1,9 @@
 // VALU kernels built on v_dot4_i32_i8 with LDS-staged halo tiles:
 //
-//   Depthwise3x3Kernel<S,R> DepthwiseConvolution2d 3x3, multiplier 1, stride S in {1,2}, channels % 32 == 0, R output rows per thread.
+//   Depthwise3x3Kernel<S,R> DepthwiseConvolution2d 3x3, multiplier 1, stride S in {1,2}, channels % 16 == 0, R output rows per thread.
+//                           (A block takes 32 channels; the last block of a tensor with 16 more stages padding for the missing
+//                           half, computes on it and stores nothing for it.  The packed weights, corr and the channel table are
+//                           padded to whole blocks.)
 //   SmallCiConvKernel<..>   Convolution2d with <= 4 input channels (network stems): too little K per tap for MFMA.
 //
 // Both bring the input to signed int8 while staging (uint8: x ^ 0x80) and fill out-of-image positions with the
@@ -91,7 +94,8 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
         const int col = pix % HC;
         const int row = pix / HC;
         const int iy = iy_org + row, ix = ix_org + col;
-        const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && static_cast<unsigned>(ix) < static_cast<unsigned>(a.W);
+        const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && static_cast<unsigned>(ix) < static_cast<unsigned>(a.W) &&
+                        cb * CB + half * 16 < a.C;
         const uint8_t* src = ok ? xn + (static_cast<long long>(iy) * a.W + ix) * a.C + half * 16 : a.pad16;
         st[k] = *reinterpret_cast<const v4i*>(src);
     }
@@ -199,7 +203,7 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
         for (int j = 0; j < P; ++j)
         {
             const int ox = tx * TW + xg * P + j;
-            if (ox < a.Wo)
+            if (ox < a.Wo && c < a.C)
             {
                 *reinterpret_cast<uint32_t*>(yrow + static_cast<long long>(ox) * a.C) =
                     Requant4Dev(acc[o][j][0], acc[o][j][1], acc[o][j][2], acc[o][j][3], f4, a.ct, c, a.rq);

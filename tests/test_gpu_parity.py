@@ -84,9 +84,12 @@ def test_algo_selection():
     assert shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()[0] == shim.ALGO_DOT4
     c = cases.make_conv_case("sel", 1, ci=3, co=15)
     assert shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()[0] == shim.ALGO_DIRECT
-    c = cases.make_conv_case("sel", 1, ci=16, depthwise=True)
+    c = cases.make_conv_case("sel", 1, ci=24, depthwise=True)
     a, info = shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()
     assert a == shim.ALGO_DEPTHWISE and "c4" in info
+    c = cases.make_conv_case("sel", 1, ci=16, depthwise=True)
+    a, info = shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()
+    assert a == shim.ALGO_DEPTHWISE and "dot4" in info
     c = cases.make_conv_case("sel", 1, ci=64, depthwise=True)
     a, info = shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()
     assert a == shim.ALGO_DEPTHWISE and "dot4" in info
@@ -473,6 +476,28 @@ def test_stem_weights_with_a_zero_point(port, name, kw, halves, in_u8):
     print(f"{name}: x={case.x.info.shape} zw={case.w.info.offset} kernel: {desc}", flush=True)
     assert algo == shim.ALGO_DOT4
     assert ("two int8 halves" in desc) == halves
+    want = _oracle_conv(port, case)
+    auto = _gpu_conv(case, shim.ALGO_AUTO)
+    mx, exact = lsb_diff(auto.data, want.data)
+    print(f"  max|d|={mx} exact={exact:.5f}", flush=True)
+    assert mx <= 1 and exact >= 0.99
+    np.testing.assert_array_equal(auto.data, _gpu_conv(case, shim.ALGO_DIRECT).data)
+
+
+@pytest.mark.parametrize("c", [16, 48, 80, 144])
+@pytest.mark.parametrize("stride", [1, 2])
+@pytest.mark.parametrize("w_kind", ["per_axis", "u8_zero_point"])
+def test_depthwise_channel_counts_that_are_odd_multiples_of_16(port, c, stride, w_kind):
+    """The 3x3 depthwise kernel works in blocks of 32 channels; a tensor with 16 more gets a last block that is half padding."""
+    kw = dict(per_axis=True) if w_kind == "per_axis" else dict(per_axis=False, w_dtype=DataType.QAsymmU8, w_offset=101, w_std=70.0)
+    case = cases.make_conv_case(f"dw_c{c}", 35000 + c + stride, n=3, h=19, w=21, ci=c, kh=3, kw=3, stride=(stride, stride), padding="same",
+                                depthwise=True, in_dtype=DataType.QAsymmU8, in_offset=121, out_offset=4, act=(2, 6.0, 0.0), **kw)
+    fn, a, b = case.act
+    plan = shim.Conv2dPlan(case.x.info, case.w, case.b, case.out_info, activation=fn, act_a=a, act_b=b, algo=shim.ALGO_AUTO, **case.params)
+    desc = plan.algo()[1]
+    plan.destroy()
+    print(f"c={c} stride={stride} {w_kind}: {desc}", flush=True)
+    assert "depthwise3x3_dot4" in desc
     want = _oracle_conv(port, case)
     auto = _gpu_conv(case, shim.ALGO_AUTO)
     mx, exact = lsb_diff(auto.data, want.data)
