@@ -73,6 +73,9 @@ def main(argv=None):
     ap.add_argument("--u8", action="store_true", help="QAsymmU8 activations (default QAsymmS8)")
     ap.add_argument("--wzp", type=int, default=None, metavar="ZERO_POINT",
                     help="per-tensor QAsymmU8 weights with this zero point (default: per-channel QSymmS8)")
+    ap.add_argument("--wspread", type=int, default=1, metavar="FACTOR",
+                    help="with --wzp: multiply the weight draws (std 30) by this before adding the zero point; 3 spreads the "
+                         "codes over the whole uint8 range, so that weight minus zero point no longer fits int8")
     ap.add_argument("--algo", type=int, default=0)
     ap.add_argument("--iters", type=int, default=50)
     ap.add_argument("--warmup", type=int, default=5)
@@ -97,7 +100,7 @@ def main(argv=None):
         if a.wzp is not None:
             ws = ws[:1]
             w = QTensor(TensorInfo((o, k), DataType.QAsymmU8, tuple(ws), a.wzp, None),
-                        np.clip(synth.int8_weights(2, (o, k)).astype(np.int32) + a.wzp, 0, 255).astype(np.uint8))
+                        np.clip(a.wspread * synth.int8_weights(2, (o, k)).astype(np.int32) + a.wzp, 0, 255).astype(np.uint8))
         b = QTensor(TensorInfo((o,), DataType.Signed32, tuple(np.float32(0.02) * ws), 0, 0 if a.wzp is None else None), synth.int32_bias(4, o))
         plan = shim.FullyConnectedPlan(xin, w, b, yout, algo=a.algo)
         batch, macs = m, m * k * o
@@ -118,7 +121,7 @@ def main(argv=None):
         if a.wzp is not None:
             ws = ws[:1]
             w = QTensor(TensorInfo(wshape, DataType.QAsymmU8, tuple(ws), a.wzp, None),
-                        np.clip(synth.int8_weights(2, wshape).astype(np.int32) + a.wzp, 0, 255).astype(np.uint8))
+                        np.clip(a.wspread * synth.int8_weights(2, wshape).astype(np.int32) + a.wzp, 0, 255).astype(np.uint8))
         b = QTensor(TensorInfo((co,), DataType.Signed32, tuple(np.float32(0.0235) * ws), 0, 0 if a.wzp is None else None), synth.int32_bias(4, co))
         plan = shim.Conv2dPlan(xin, w, b, yout, pad_top=pt, pad_left=pl, stride_x=a.stride, stride_y=a.stride,
                                depthwise=dw, activation=act[0], act_a=act[1], act_b=act[2], algo=a.algo)
