@@ -25,6 +25,7 @@ struct mi355x_conv2d_s
     int8_t*  w_mfma   = nullptr;   // [Co_pad][K_pad] signed, zero padded
     uint8_t* pad16    = nullptr;   // 16 bytes that turn into the padding value under the kernel's input xor
     int8_t*  w_stem   = nullptr;   // small-Ci conv on MFMA: [Co rounded up to 32][stem_kp]
+    int8_t*  w_stem2  = nullptr;   // ... the second halves of weight differences that need two
     int      stem_kp  = 0;
     uint32_t* dw_grp  = nullptr;   // depthwise 3x3: constants per group of 4 channels for the fused dw+pw kernel
     uint32_t* w_dot4  = nullptr;   // depthwise 3x3: [C][4] dwords; small-Ci conv: [Co][Kh][RD] dwords
@@ -51,6 +52,7 @@ struct mi355x_conv2d_s
         (void)hipFree(pad16);
         (void)hipFree(dw_grp);
         (void)hipFree(w_stem);
+        (void)hipFree(w_stem2);
         (void)hipFree(w_dot4);
         (void)hipFree(w_dot4b);
         (void)hipFree(chan);
@@ -387,7 +389,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             const std::vector<uint8_t> padbytes(16, static_cast<uint8_t>((p->pad_word ^ p->xor_mask) & 0xffu));
             if (int rc = Upload(reinterpret_cast<void**>(&p->pad16), padbytes.data(), padbytes.size())) return rc;
         }
-        if ((Co == 32 || Co == 64) && stem_fits)
+        if (Co == 32 || Co == 64)
         {
             // the same rows, end to end, as the K vector of the MFMA variant
             const int kp = (Kh * RD * 4 + 31) / 32 * 32;
@@ -395,6 +397,12 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             std::vector<int8_t> wm(static_cast<size_t>(rows) * kp, 0);
             for (int c = 0; c < Co; ++c) std::memcpy(wm.data() + static_cast<size_t>(c) * kp, wp.data() + static_cast<size_t>(c) * Kh * RD, static_cast<size_t>(Kh) * RD * 4);
             if (int rc = Upload(reinterpret_cast<void**>(&p->w_stem), wm.data(), wm.size())) return rc;
+            if (!stem_fits)
+            {
+                std::fill(wm.begin(), wm.end(), 0);
+                for (int c = 0; c < Co; ++c) std::memcpy(wm.data() + static_cast<size_t>(c) * kp, wp2.data() + static_cast<size_t>(c) * Kh * RD, static_cast<size_t>(Kh) * RD * 4);
+                if (int rc = Upload(reinterpret_cast<void**>(&p->w_stem2), wm.data(), wm.size())) return rc;
+            }
             p->stem_kp = kp;
         }
         FoldCorrIntoTable(p, corr, Co);
@@ -771,13 +779,20 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         if (a.lp > 288) return SetError(MI355X_ERR_UNSUPPORTED, "dot4 kernel: halo row of %d bytes does not fit", a.lp);
         if (static_cast<long long>(g.H) * g.W * g.Ci >= (1ll << 30)) return SetError(MI355X_ERR_UNSUPPORTED, "dot4 kernel: image too large for 32-bit offsets");
         a.rq = p->rq;
-        a.w_mfma = p->w_stem; a.kp = p->stem_kp;
+        a.w_mfma = p->w_stem; a.w_mfma2 = p->w_stem2; a.kp = p->stem_kp;
         if (p->w_stem && !GlobalOptions().stem_dot4 && (g.Kh == 3 || g.Kh == 7))
         {
             const long long nbm = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
             if (nbm > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
             const dim3 gridm(static_cast<unsigned>(nbm));
-            if (g.Kh == 3 && g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 1, 16>), gridm, dim3(256), 0, stream, a);
+            if (p->w_stem2)
+            {
+                if (g.Kh == 3 && g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 1, 16, true>), gridm, dim3(256), 0, stream, a);
+                else if (g.Kh == 3) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 2, 16, true>), gridm, dim3(256), 0, stream, a);
+                else if (g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 1, 16, true>), gridm, dim3(256), 0, stream, a);
+                else hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 2, 16, true>), gridm, dim3(256), 0, stream, a);
+            }
+            else if (g.Kh == 3 && g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 1, 16>), gridm, dim3(256), 0, stream, a);
             else if (g.Kh == 3) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 2, 16>), gridm, dim3(256), 0, stream, a);
             else if (g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 1, 16>), gridm, dim3(256), 0, stream, a);
             else hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 2, 16>), gridm, dim3(256), 0, stream, a);

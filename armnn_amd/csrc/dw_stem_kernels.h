@@ -11,7 +11,7 @@
 // per-channel constant (`corr`) that initialises the accumulators.  The depthwise kernel takes as "w" the difference
 // d = w - zw between a weight and the weights' zero point; where some d does not fit int8 (it lies in -255 .. 254) it is
 // the sum of two int8 halves, each in a packed array of its own (template W2), and costs a second v_dot4.  The stem
-// kernel on v_dot4 does the same; its MFMA variant needs weights that fit one int8.
+// kernels do the same, the MFMA variant with a second set of weight fragments and a second run of MFMAs over the same patches.
 #pragma once
 
 #include <hip/hip_runtime.h>
@@ -243,6 +243,7 @@ struct SmallCiArgs
                               // 16-byte loads (lp is then a multiple of 16)
     uint32_t nch_recip;       // ceil(2^32 / (lp / 16))
     const int8_t* w_mfma;     // MFMA variant: [Co rounded up to 32][kp] bytes, a filter's rows as RD dwords each, zero padded
+    const int8_t* w_mfma2;    // W2: the second halves, same layout
     int kp;                   // bytes per weight row of w_mfma (multiple of 32)
     Requant rq;
 };
@@ -484,7 +485,7 @@ __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
 // the padding), and 32 pixels x 32 output channels become ceil(KH*RD/8) MFMA steps instead of 32*KH*RD dot products per
 // pixel.  Both lanes of a pixel (lane, lane + 32) gather the pixel's rows from the LDS halo and keep the half of each
 // 32-byte k-step that the MFMA B operand assigns them.  A wave takes 4 of the tile's 16 rows; NT = output channels / 32.
-template <int KH, int RD, int NT, int TH>
+template <int KH, int RD, int NT, int TH, bool W2 = false>
 __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
 {
     constexpr int TW = 32;
@@ -517,6 +518,15 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
 #pragma unroll
         for (int t = 0; t < KST; ++t)
             wfrag[ct][t] = *reinterpret_cast<const v4i*>(a.w_mfma + static_cast<long long>(ct * 32 + px) * a.kp + t * 32 + half * 16);
+    v4i wfrag2[W2 ? NT : 1][W2 ? KST : 1];
+    if constexpr (W2)
+    {
+#pragma unroll
+        for (int ct = 0; ct < NT; ++ct)
+#pragma unroll
+            for (int t = 0; t < KST; ++t)
+                wfrag2[ct][t] = *reinterpret_cast<const v4i*>(a.w_mfma2 + static_cast<long long>(ct * 32 + px) * a.kp + t * 32 + half * 16);
+    }
     __syncthreads();
 
     const int ox = tx * TW + px;
@@ -557,6 +567,11 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
             v16i acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wfrag[ct][0], bfrag[0], zero, 0, 0, 0);
 #pragma unroll
             for (int t = 1; t < KST; ++t) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wfrag[ct][t], bfrag[t], acc, 0, 0, 0);
+            if constexpr (W2)
+            {
+#pragma unroll
+                for (int t = 0; t < KST; ++t) acc = __builtin_amdgcn_mfma_i32_32x32x32_i8(wfrag2[ct][t], bfrag[t], acc, 0, 0, 0);
+            }
             uint32_t o[4];
 #pragma unroll
             for (int qd = 0; qd < 4; ++qd)
