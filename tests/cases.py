@@ -157,6 +157,8 @@ def small_conv_cases():
                             in_scale=0.0235, out_scale=0.0235, out_offset=0, act=RELU6))
     c.append(make_conv_case("s8_wide_64x64", 117, h=6, w=6, ci=64, co=64, act=RELU6))
     c.append(make_conv_case("s8_1x1_k128_n96", 118, h=5, w=5, ci=128, co=96, kh=1, kw=1))
+    # K = 3*3*512 = 4608 taps: the longest accumulation of the ResNet-50 layers (fp32 summation order in the reference)
+    c.append(make_conv_case("s8_3x3_ci512_k4608", 119, h=5, w=4, ci=512, co=24, act=RELU))
     # weight-stationary pointwise GEMM kernel: several tiles per wave, ragged M, every chunk depth
     c.append(make_conv_case("pw_u8_k64_n128_m3200", 120, n=2, h=40, w=40, ci=64, co=128, kh=1, kw=1, in_dtype=U8, in_scale=0.0235,
                             in_offset=0, out_scale=0.0235, out_offset=0, act=RELU6))

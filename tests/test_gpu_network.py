@@ -66,6 +66,16 @@ def test_mobilenet_v1_batch2(port):
     _layerwise(port, nets.mobilenet_v1(), 2)
 
 
+def test_mobilenet_v1_batch1(port):
+    # batch 1 selects the matrix-vector classifier and the few-block tilings everywhere
+    _layerwise(port, nets.mobilenet_v1(), 1)
+
+
+def test_resnet50_224_batch1(port):
+    # full resolution against the CPU checker: what the batch-32 row-equality test below chains to
+    _layerwise(port, nets.resnet50(), 1)
+
+
 def test_mobilenet_v1_small_odd_resolution(port):
     # odd spatial sizes exercise the SAME-padding edges of every stride-2 layer
     _layerwise(port, nets.mobilenet_v1(resolution=97, classes=37), 3)

@@ -213,9 +213,10 @@ def test_config_c2_block(port):
     assert mx <= 1 and exact >= 0.999
 
 
-@pytest.mark.parametrize("m", [1, 256])
+@pytest.mark.parametrize("m", [1, 256, 2048])
 def test_config_c4_fc(port, m):
-    """Benchmark configuration C4: [M,4096] x [4096,4096] per-channel, fused requantize (output scale 1.0, zp 0)."""
+    """Benchmark configuration C4: [M,4096] x [4096,4096] per-channel, fused requantize (output scale 1.0, zp 0), at the
+    three row counts the configuration names; M = 2048 is the size the large GEMM tilings are selected and timed at."""
     c = cases.make_fc_case("C4", 20250104, m=m, k=4096, o=4096, in_offset=0, out_scale=1.0, out_offset=0)
     want = port.fully_connected(c.x, c.w, c.b, c.out_info)
     got = shim.fully_connected(c.x, c.w, c.b, c.out_info)
@@ -223,6 +224,19 @@ def test_config_c4_fc(port, m):
     sat = float(((got.data == 127) | (got.data == -128)).mean())
     print(f"C4 M={m}: max|d|={mx} exact={exact:.6f} saturated={sat:.4f}", flush=True)
     assert mx <= 1 and exact >= 0.995 and sat < 0.05
+    if m == 2048:
+        direct = shim.fully_connected(c.x, c.w, c.b, c.out_info, algo=shim.ALGO_DIRECT)
+        np.testing.assert_array_equal(got.data, direct.data)
+
+
+def test_c4_fc_8192_rows_equal_direct_kernel():
+    """M = 8192 selects the largest GEMM tiling; the rows are independent, so every row must carry the bytes the
+    one-thread-per-output kernel gives (which the M = 2048 case ties to the CPU checker)."""
+    c = cases.make_fc_case("C4big", 20250105, m=8192, k=4096, o=4096, in_offset=0, out_scale=1.0, out_offset=0)
+    got = shim.fully_connected(c.x, c.w, c.b, c.out_info)
+    direct = shim.fully_connected(c.x, c.w, c.b, c.out_info, algo=shim.ALGO_DIRECT)
+    np.testing.assert_array_equal(got.data, direct.data)
+    assert got.data.max() > got.data.min()
 
 
 def _random_conv_case(k):
