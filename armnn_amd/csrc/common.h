@@ -60,6 +60,7 @@ struct Requant
     int32_t  pk_bias;       // 128 for QAsymmS8 outputs, 0 for QAsymmU8
     uint32_t pk_xor;        // 0x80808080 or 0
     float    pk_lo_f, pk_hi_f;   // activation clamp in the biased domain
+    float    pk_lo_q, pk_hi_q;   // ... widened by a quarter code: the clamp the fast path applies before rounding
     int32_t  pk_full;       // the clamp is 0..255: the instruction's own saturation does it
 };
 
@@ -69,7 +70,7 @@ Requant MakeRequant(const mi355x_quant& out, int32_t activation, float a, float 
 struct Options
 {
     int exact_division_epilogue = 0;   // 1: every output takes the fp32 division (no reciprocal fast path)
-    int igemm_tile = 0;                // 0: automatic; 64, 96 (128x64) or 128: every MFMA plan created meanwhile uses that implicit-GEMM tile
+    int igemm_tile = 0;                // 0: automatic; 64, 96 (128x64), 128, 256, 512 (256x256), or 2256 / 2128 / 1256 (large-tile kernel): every MFMA plan created meanwhile uses that implicit-GEMM tile
     int igemm_lds = 2;                 // LDS stages of the direct-to-LDS implicit GEMM (2 or 3); 0: use the register-staged kernel
     int dw_rows = 0;                   // output rows per thread of the 3x3 depthwise kernel: 0 automatic, 1 or 2 forced
     int stem_dot4 = 0;                 // 1: small-Ci convolutions stay on the v_dot4 kernel (tests compare it with the MFMA one)

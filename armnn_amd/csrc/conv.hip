@@ -6,6 +6,7 @@
 #include "dwpw_kernel.h"
 #include "pw_gemm_kernel.h"
 #include "igemm_lds_kernel.h"
+#include "big_gemm.h"
 
 #include <cmath>
 #include <cstdlib>
@@ -284,6 +285,8 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             if (int rc = Upload(reinterpret_cast<void**>(&p->pad16), padbytes.data(), padbytes.size())) return rc;
         }
         p->tile_override = GlobalOptions().igemm_tile;
+        if (p->bk128 && (Ci % 128) == 0)
+            if (int rc = PrepareBigGemm()) return rc;
         FoldCorrIntoTable(p, corr, Co);
         ChoosePointwiseConfig(p);
         if (p->tile_override != 0) p->pw_bn = 0;     // a forced tile also forces the LDS-tiled implicit GEMM
@@ -652,6 +655,38 @@ int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, voi
     return 0;
 }
 
+// the large-tile kernel of big_gemm.hip (one wave per SIMD, accumulators in AGPRs)
+int LaunchBig(const mi355x_conv2d_s* p, int bm, int bn, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    const ConvGeom& g = p->geom;
+    IgemmArgs a;
+    a.x = static_cast<const uint8_t*>(x);
+    a.pad16 = p->pad16;
+    a.w = p->w_mfma;
+    a.ct = ChanTab{p->chan, p->Co_pad};
+    a.corr = p->corr;
+    a.y = static_cast<uint8_t*>(y);
+    const long long M = static_cast<long long>(batch) * g.Ho * g.Wo;
+    if (M > 0x7fffffffll / 2) return SetError(MI355X_ERR_UNSUPPORTED, "too many output pixels for one launch (%lld)", M);
+    if (p->Co_pad % bn != 0) return SetError(MI355X_ERR_UNSUPPORTED, "large-tile GEMM: %d padded channels are not whole %d-wide tiles", p->Co_pad, bn);
+    a.M = static_cast<int>(M);
+    a.H = g.H; a.W = g.W; a.Ci = g.Ci; a.Ho = g.Ho; a.Wo = g.Wo; a.Co = g.Co;
+    a.Kh = g.Kh; a.Kw = g.Kw;
+    a.pad_top = g.pad_top; a.pad_left = g.pad_left; a.stride_x = g.stride_x; a.stride_y = g.stride_y;
+    a.dil_x = g.dil_x; a.dil_y = g.dil_y;
+    a.K_pad = p->K_pad;
+    a.unit = (g.Kh == 1 && g.Kw == 1 && g.stride_x == 1 && g.stride_y == 1 && g.pad_top == 0 && g.pad_left == 0 && g.Ho == g.H &&
+              g.Wo == g.W) ? 1 : 0;
+    if (a.unit) { a.H = 1; a.W = a.M; a.Ho = 1; a.Wo = a.M; }      // one row of M pixels
+    a.tiles_m = 0; a.tiles_n = 0;                                  // the launcher fills them in
+    a.xor_mask = p->xor_mask;
+    a.pad_word = p->pad_word;
+    a.zw_neg = p->zw_neg;
+    a.rowsum_bias = p->rowsum_bias;
+    a.rq = p->rq;
+    return LaunchBigGemm(a, bm, bn, stream);
+}
+
 template <int BM, int BN, int WM, int WN>
 int LaunchIgemmLds(const mi355x_conv2d_s* p, int stages, uint32_t batch, const void* x, void* y, hipStream_t stream)
 {
@@ -742,6 +777,19 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const int lds_stages = GlobalOptions().igemm_lds;
         if (lds_stages != 0 && bk128 && (g.Ci % 128) == 0)
         {
+            // Launches that fill the device with 256-row tiles: one wave per SIMD with a 128 x 128 (or 128 x 64) wave tile.
+            // A CU's L1 delivers 30 to 45 bytes per clock from L2; only these tiles ask for less than that per MFMA clock.
+            if (p->tile_override == 0 || p->tile_override >= 1000)
+            {
+                const long long rows256 = (M + 255) / 256;
+                int bm = 0, bn = 0;
+                if (p->tile_override == 2256) { bm = 256; bn = 256; }
+                else if (p->tile_override == 2128) { bm = 256; bn = 128; }
+                else if (p->tile_override == 1256) { bm = 128; bn = 256; }
+                else if ((p->Co_pad % 256) == 0 && rows256 * (p->Co_pad / 256) >= 224) { bm = 256; bn = 256; }
+                else if (rows256 * (p->Co_pad / 128) >= 224) { bm = 256; bn = 128; }
+                if (bm != 0) return LaunchBig(p, bm, bn, batch, x, y, stream);
+            }
             if (tile == 64)
             {
                 // at most one block per CU: nothing else hides a k-tile's round trip, so keep two tiles on their way

@@ -68,7 +68,8 @@ __device__ __forceinline__ uint32_t Pack4(int q0, int q1, int q2, int q3)
 
 struct Fast4
 {
-    float4 m, b, t;
+    float4 m, b, t;      // rows 2, 3, 4: the fast path
+    float4 m0, b0;       // rows 0, 1: the exact path, fetched along so that entering it waits for nothing
 };
 
 __device__ __forceinline__ Fast4 LoadFast4(const ChanTab& ct, int c)
@@ -77,6 +78,8 @@ __device__ __forceinline__ Fast4 LoadFast4(const ChanTab& ct, int c)
     f.m = *reinterpret_cast<const float4*>(ct.p + 2 * ct.stride + c);
     f.b = *reinterpret_cast<const float4*>(ct.p + 3 * ct.stride + c);
     f.t = *reinterpret_cast<const float4*>(ct.p + 4 * ct.stride + c);
+    f.m0 = *reinterpret_cast<const float4*>(ct.p + c);
+    f.b0 = *reinterpret_cast<const float4*>(ct.p + ct.stride + c);
     return f;
 }
 
@@ -89,61 +92,82 @@ __device__ __forceinline__ Fast4 LoadFast4(const ChanTab& ct, int c)
         SLOW = !(fabsf(e_) <= __fmaf_rn(fabsf(r_), -kTieSlope, T));           \
     }
 
-// Four consecutive channels c..c+3 of one pixel -> packed dword.
-//   `corr` (may be null) is an integer added to the accumulator on the exact path only (rows 5/6, see ChanTab).
-// The fast path is branch-free (7 VALU instructions per value when the clamp is the whole byte range); the four flags are combined as wave masks, and
-// only when some lane of the wave has a flagged value does the wave enter the fix-up loop, which evaluates one
-// flagged value per lane and pass.
-__device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const float4& fm, const float4& fb,
-                                                const float4& thr, const ChanTab& ct, const int32_t* corr, int c,
-                                                const Requant& rq)
-{
-    float k0, k1, k2, k3;
-    bool s0, s1, s2, s3;
-    MI355X_FAST1(a0, fm.x, fb.x, thr.x, k0, s0)
-    MI355X_FAST1(a1, fm.y, fb.y, thr.y, k1, s1)
-    MI355X_FAST1(a2, fm.z, fb.z, thr.z, k2, s2)
-    MI355X_FAST1(a3, fm.w, fb.w, thr.w, k3, s3)
-    if (!rq.pk_full)      // wave-uniform: a clamp narrower than 0..255 (the conversion below saturates to that by itself)
-    {
-        k0 = __builtin_amdgcn_fmed3f(k0, rq.pk_lo_f, rq.pk_hi_f);
-        k1 = __builtin_amdgcn_fmed3f(k1, rq.pk_lo_f, rq.pk_hi_f);
-        k2 = __builtin_amdgcn_fmed3f(k2, rq.pk_lo_f, rq.pk_hi_f);
-        k3 = __builtin_amdgcn_fmed3f(k3, rq.pk_lo_f, rq.pk_hi_f);
+// r' is first clamped to a quarter code beyond the activation's range [LO, HI] (biased domain): whatever lies further out
+// ends at LO or HI on either path, its distance to an integer is then exactly 0.25, and it can never look like a tie.
+// K = rint(r'), U = |r' - K| + kTieSlope |r'|: the value needs the exact path when U exceeds its channel's threshold.
+#define MI355X_FAST1U(ACC, M, B, LO, HI, K, U)                                                        \
+    {                                                                                                 \
+        const float r_ = __builtin_amdgcn_fmed3f(__fmaf_rn(static_cast<float>(ACC), M, B), LO, HI);   \
+        K = __builtin_rintf(r_);                                                                      \
+        U = __fmaf_rn(fabsf(r_), kTieSlope, fabsf(__fsub_rn(r_, K)));                                 \
     }
-    // integral floats -> saturated unsigned bytes, one instruction per value, packed as it goes
+
+// Four consecutive channels c..c+3 of one pixel -> packed dword.
+// The fast path is branch-free, 7 VALU instructions per value plus a few per quad: the four tie measures are folded
+// with v_max3 / v_max and compared once against the smallest of the four thresholds (a smaller threshold only sends
+// more values to the exact path), so a quad costs one compare and one scalar branch.  r' is finite whenever a
+// threshold is non-negative (the host checks the constants and the accumulator range), so no NaN can hide in the
+// maxima; a channel without a fast path has threshold -1, which every measure exceeds.  When some lane of the wave has
+// a flagged value, the wave redoes that value's position of the quad with the reference's sequence on every lane (always
+// right, and cheaper than sorting out which lanes need it); LOAD_EXACT supplies rows 0 / 1 of the table and, for kernels
+// whose accumulators start at zero, the zero-point correction that only the exact path adds as an integer.
+template <typename LoadExact>
+__device__ __forceinline__ uint32_t Requant4Core(int a0, int a1, int a2, int a3, const float4& fm, const float4& fb,
+                                                 const float4& thr, const Requant& rq, LoadExact load_exact)
+{
+    float k0, k1, k2, k3, u0, u1, u2, u3;
+    MI355X_FAST1U(a0, fm.x, fb.x, rq.pk_lo_q, rq.pk_hi_q, k0, u0)
+    MI355X_FAST1U(a1, fm.y, fb.y, rq.pk_lo_q, rq.pk_hi_q, k1, u1)
+    MI355X_FAST1U(a2, fm.z, fb.z, rq.pk_lo_q, rq.pk_hi_q, k2, u2)
+    MI355X_FAST1U(a3, fm.w, fb.w, rq.pk_lo_q, rq.pk_hi_q, k3, u3)
+    const float umax = fmaxf(fmaxf(fmaxf(u0, u1), u2), u3);       // v_max3_f32 + v_max_f32
+    const float tmin = fminf(fminf(thr.x, thr.y), fminf(thr.z, thr.w));
+    // integral floats within [LO, HI] -> unsigned bytes, one instruction per value, packed as it goes
     uint32_t out = __builtin_amdgcn_cvt_pk_u8_f32(k0, 0, 0u);
     out = __builtin_amdgcn_cvt_pk_u8_f32(k1, 1, out);
     out = __builtin_amdgcn_cvt_pk_u8_f32(k2, 2, out);
     out = __builtin_amdgcn_cvt_pk_u8_f32(k3, 3, out);
-    const unsigned long long any = __builtin_amdgcn_ballot_w64(s0) | __builtin_amdgcn_ballot_w64(s1) |
-                                   __builtin_amdgcn_ballot_w64(s2) | __builtin_amdgcn_ballot_w64(s3);
-    if (__builtin_expect(any != 0, 0))
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(umax <= tmin)) != 0, 0))
     {
-        const float4 m = *reinterpret_cast<const float4*>(ct.p + c);
-        const float4 b = *reinterpret_cast<const float4*>(ct.p + ct.stride + c);
-        int4 cr = {0, 0, 0, 0};
-        if (corr) cr = *reinterpret_cast<const int4*>(corr + c);
-        unsigned fl = (s0 ? 1u : 0u) | (s1 ? 2u : 0u) | (s2 ? 4u : 0u) | (s3 ? 8u : 0u);
-        while (__builtin_amdgcn_ballot_w64(fl != 0) != 0)
-        {
-            const int which = __builtin_ctz(fl | 16u);     // 4 when the lane has nothing left
-            const int av = which == 0 ? a0 + cr.x : which == 1 ? a1 + cr.y : which == 2 ? a2 + cr.z : a3 + cr.w;
-            const float mv = which == 0 ? m.x : which == 1 ? m.y : which == 2 ? m.z : m.w;
-            const float bv = which == 0 ? b.x : which == 1 ? b.y : which == 2 ? b.z : b.w;
-            const uint32_t qe = static_cast<uint32_t>(RequantExactDev(av, mv, bv, rq) + rq.pk_bias) & 0xffu;
-            if (which < 4) out = (out & ~(0xffu << (8 * which))) | (qe << (8 * which));
-            fl &= fl - 1u;
-        }
+        float4 m, b;
+        int4 cr;
+        load_exact(m, b, cr);
+        // usually one value of the wave's 256 is flagged: only its position is redone (on every lane: the exact result is
+        // always the right one)
+        if (__builtin_amdgcn_ballot_w64(!(u0 <= tmin)) != 0)
+            out = (out & 0xffffff00u) | (static_cast<uint32_t>(RequantExactDev(a0 + cr.x, m.x, b.x, rq) + rq.pk_bias) & 0xffu);
+        if (__builtin_amdgcn_ballot_w64(!(u1 <= tmin)) != 0)
+            out = (out & 0xffff00ffu) | ((static_cast<uint32_t>(RequantExactDev(a1 + cr.y, m.y, b.y, rq) + rq.pk_bias) & 0xffu) << 8);
+        if (__builtin_amdgcn_ballot_w64(!(u2 <= tmin)) != 0)
+            out = (out & 0xff00ffffu) | ((static_cast<uint32_t>(RequantExactDev(a2 + cr.z, m.z, b.z, rq) + rq.pk_bias) & 0xffu) << 16);
+        if (__builtin_amdgcn_ballot_w64(!(u3 <= tmin)) != 0)
+            out = (out & 0x00ffffffu) | ((static_cast<uint32_t>(RequantExactDev(a3 + cr.w, m.w, b.w, rq) + rq.pk_bias) & 0xffu) << 24);
     }
     return out ^ rq.pk_xor;
 }
 
-// constants of rows 2,3,4 (accumulator already contains the zero-point correction)
-__device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const Fast4& f, const ChanTab& ct, int c,
+// `corr` (may be null) is an integer added to the accumulator on the exact path only (rows 5/6, see ChanTab).
+__device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const float4& fm, const float4& fb,
+                                                const float4& thr, const ChanTab& ct, const int32_t* corr, int c,
                                                 const Requant& rq)
 {
-    return Requant4Dev(a0, a1, a2, a3, f.m, f.b, f.t, ct, nullptr, c, rq);
+    return Requant4Core(a0, a1, a2, a3, fm, fb, thr, rq, [&](float4& m, float4& b, int4& cr) {
+        m = *reinterpret_cast<const float4*>(ct.p + c);
+        b = *reinterpret_cast<const float4*>(ct.p + ct.stride + c);
+        cr = int4{0, 0, 0, 0};
+        if (corr) cr = *reinterpret_cast<const int4*>(corr + c);
+    });
+}
+
+// constants of rows 2,3,4 (accumulator already contains the zero-point correction), exact-path rows fetched beforehand
+__device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const Fast4& f, const ChanTab&, int,
+                                                const Requant& rq)
+{
+    return Requant4Core(a0, a1, a2, a3, f.m, f.b, f.t, rq, [&](float4& m, float4& b, int4& cr) {
+        m = f.m0;
+        b = f.b0;
+        cr = int4{0, 0, 0, 0};
+    });
 }
 
 // one channel (scalar kernels)

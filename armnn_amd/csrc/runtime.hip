@@ -90,6 +90,8 @@ Requant MakeRequant(const mi355x_quant& out, int32_t activation, float a, float 
     rq.pk_xor  = rq.out_is_u8 ? 0u : 0x80808080u;
     rq.pk_lo_f = static_cast<float>(rq.act_lo + rq.pk_bias);
     rq.pk_hi_f = static_cast<float>(rq.act_hi + rq.pk_bias);
+    rq.pk_lo_q = rq.pk_lo_f - 0.25f;
+    rq.pk_hi_q = rq.pk_hi_f + 0.25f;
     rq.pk_full = (rq.act_lo + rq.pk_bias == 0 && rq.act_hi + rq.pk_bias == 255) ? 1 : 0;
     rq.fast_ok = !GlobalOptions().exact_division_epilogue && std::isnormal(rq.inv_scale) && std::isnormal(out.scale) && out.offset >= -255 && out.offset <= 255 &&
                  rq.act_lo <= rq.act_hi;
@@ -132,8 +134,9 @@ int mi355x_set_option(const char* name, int value)
     }
     if (std::strcmp(name, "igemm_tile") == 0)
     {
-        if (value != 0 && value != 64 && value != 96 && value != 128 && value != 256 && value != 512)
-            return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_tile must be 0, 64, 96, 128, 256 or 512");
+        // 2256, 2128, 1256: the large-tile kernel at 256x256, 256x128, 128x256
+        if (value != 0 && value != 64 && value != 96 && value != 128 && value != 256 && value != 512 && value != 2256 && value != 2128 && value != 1256)
+            return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_tile must be 0, 64, 96, 128, 256, 512, 2256, 2128 or 1256");
         GlobalOptions().igemm_tile = value;
         return 0;
     }

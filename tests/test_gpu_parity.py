@@ -162,6 +162,42 @@ def test_every_igemm_tiling_gives_the_same_bytes():
         shim.set_option("igemm_tile", 100)
 
 
+def test_large_tile_gemm_gives_the_same_bytes():
+    """The one-wave-per-SIMD kernel (256x256, 256x128 and 128x256 block tiles, accumulators in AGPRs) is chosen only for
+    launches that fill the device; here each tiling is forced on small problems -- ragged rows and channels, padding,
+    stride, dilation, uint8 activations, weights with a zero point, K of one to eighteen k-tiles -- against the direct kernel."""
+    S8, U8 = DataType.QAsymmS8, DataType.QAsymmU8
+    cs = [cases.make_conv_case("big_1x1_c256", 611, n=3, h=14, w=14, ci=256, co=512, kh=1, kw=1),
+          cases.make_conv_case("big_1x1_c128_co200", 612, n=2, h=13, w=11, ci=128, co=200, kh=1, kw=1, act=cases.RELU6),
+          cases.make_conv_case("big_3x3_c128_s2", 613, n=2, h=29, w=31, ci=128, co=256, stride=(2, 2)),
+          cases.make_conv_case("big_3x3_c128_u8_dil2", 614, n=2, h=19, w=23, ci=128, co=192, dilation=(2, 2), in_dtype=U8,
+                               in_offset=131, out_offset=-100),
+          cases.make_conv_case("big_3x3_c256_asym_pad", 615, n=1, h=17, w=20, ci=256, co=256, padding=(2, 0, 1, 3), act=cases.RELU),
+          cases.make_conv_case("big_1x1_c128_wzp_s8", 616, n=2, h=16, w=16, ci=128, co=256, kh=1, kw=1, w_dtype=S8, per_axis=False, w_offset=-7),
+          cases.make_conv_case("big_3x3_c128_wzp_u8", 617, n=1, h=15, w=18, ci=128, co=256, in_dtype=U8, in_offset=120, w_dtype=U8,
+                               per_axis=False, w_offset=93, out_offset=10)]
+    for c in cs:
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        for tile in (2256, 2128, 1256):
+            shim.set_option("igemm_tile", tile)
+            try:
+                got = _gpu_conv(c, shim.ALGO_MFMA)
+            finally:
+                shim.set_option("igemm_tile", 0)
+            print(f"{c.name} tile {tile}: {got.data.size} outputs", flush=True)
+            np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} tile {tile}")
+    # FullyConnected rows through the same kernels
+    f = cases.make_fc_case("big_fc", 618, m=300, k=1024, o=512)
+    want = shim.fully_connected(f.x, f.w, f.b, f.out_info, algo=shim.ALGO_DIRECT)
+    for tile in (2256, 2128, 1256):
+        shim.set_option("igemm_tile", tile)
+        try:
+            got = shim.fully_connected(f.x, f.w, f.b, f.out_info)
+        finally:
+            shim.set_option("igemm_tile", 0)
+        np.testing.assert_array_equal(got.data, want.data, err_msg=f"fc tile {tile}")
+
+
 def test_depthwise_rows_per_thread_variants_give_the_same_bytes():
     """The 3x3 depthwise kernel with one and with two output rows per thread (8- and 16-row tiles), forced on feature maps
     of every parity of height, against the plain depthwise kernel."""
