@@ -42,6 +42,7 @@ int Launch(IgemmArgs a, hipStream_t stream)
     xcd_rows = std::max(1, std::min(xcd_rows, a.tiles_m));
     const int grid = (nblocks + 7) / 8 * 8;
     constexpr int smem = BigGemmSmemBytes<BM, BN, ST>();
+    NoteKernel("BigGemmKernel<%d, %d, %d, %s, %s, %s>", BM, BN, ST, BoolName(U8), BoolName(AW), BoolName(a.unit != 0));
     if (a.unit) hipLaunchKernelGGL((BigGemmKernel<BM, BN, ST, U8, AW, true>), dim3(grid), dim3(256), smem, stream, a, xcd_rows);
     else hipLaunchKernelGGL((BigGemmKernel<BM, BN, ST, U8, AW, false>), dim3(grid), dim3(256), smem, stream, a, xcd_rows);
     MI355X_HIP(hipGetLastError());

@@ -17,6 +17,12 @@ namespace mi355x
 char* ErrorBuffer();
 int SetError(int code, const char* fmt, ...);
 
+// Records the name of the kernel the calling thread is about to launch, as a profiler would list it (without the
+// namespace and the argument list); mi355x_last_kernel() returns it.  Measurement support: lets a benchmark label its
+// per-layer timings with kernel symbols.
+void NoteKernel(const char* fmt, ...);
+inline const char* BoolName(bool b) { return b ? "true" : "false"; }
+
 inline int HipFail(hipError_t e, const char* what)
 {
     return SetError(static_cast<int>(e), "%s: %s", what, hipGetErrorString(e));

@@ -543,6 +543,7 @@ int LaunchPw(const mi355x_conv2d_s* p, long long M, const void* x, void* y, hipS
     if (gm < 8) gm = 8;
     if (gm > (groups + 7) / 8 * 8) gm = (groups + 7) / 8 * 8;
     a.gm = static_cast<int>(gm);
+    NoteKernel("PwGemmKernel<%d, %d, %d, %s>", BN, KS, KS <= 2 ? 4 : 2, BoolName(p->zw_neg != 0));
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(a.n_slabs * gm)), dim3(256), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;
@@ -610,6 +611,7 @@ int LaunchIgemmT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* 
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmKernel<BM, BN, WM, WN, D, BK, UT, AW>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);
+    NoteKernel("IgemmKernel<%d, %d, %d, %d, %d, %d, %s, %s>", BM, BN, WM, WN, D, BK, BoolName(UT), BoolName(AW));
     hipLaunchKernelGGL((IgemmKernel<BM, BN, WM, WN, D, BK, UT, AW>), dim3(grid), dim3(256), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;
@@ -650,6 +652,7 @@ int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, voi
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmLdsKernel<BM, BN, WM, WN, ST, U8, AW>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);
+    NoteKernel("IgemmLdsKernel<%d, %d, %d, %d, %d, %s, %s>", BM, BN, WM, WN, ST, BoolName(U8), BoolName(AW));
     hipLaunchKernelGGL((IgemmLdsKernel<BM, BN, WM, WN, ST, U8, AW>), dim3(grid), dim3(64 * WM * WN), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;
@@ -732,6 +735,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             a.x = xin; a.w = p->w_mfma; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
             a.M = static_cast<int>(rows); a.K = g.Ci; a.N = g.Co; a.w_stride = p->K_pad; a.xor_mask = p->xor_mask; a.zw_neg = p->zw_neg; a.rq = p->rq;
             const dim3 grid(static_cast<unsigned>((g.Co + 15) / 16));
+            NoteKernel("GemvKernel<%d>", a.M);
             switch (a.M)
             {
                 case 1: hipLaunchKernelGGL(GemvKernel<1>, grid, dim3(256), 0, stream, a); break;
@@ -750,6 +754,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             a.x = xin; a.w = p->w_mfma; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
             a.M = static_cast<int>(rows); a.K = g.Ci; a.N = g.Co; a.w_stride = p->K_pad; a.xor_mask = p->xor_mask; a.zw_neg = p->zw_neg; a.rq = p->rq;
             const dim3 grid(static_cast<unsigned>((g.Co + 31) / 32), static_cast<unsigned>((rows + 31) / 32));
+            NoteKernel("SmallMGemmKernel<%d>", g.Ci <= 512 ? 4 : 8);
             if (g.Ci <= 512) hipLaunchKernelGGL(SmallMGemmKernel<4>, grid, dim3(256), 0, stream, a);
             else hipLaunchKernelGGL(SmallMGemmKernel<8>, grid, dim3(256), 0, stream, a);
             MI355X_HIP(hipGetLastError());
@@ -833,6 +838,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             const long long nbm = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
             if (nbm > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
             const dim3 gridm(static_cast<unsigned>(nbm));
+            NoteKernel("SmallCiMfmaKernel<%d, %d, %d, 16, %s>", g.Kh, g.Kh == 3 ? 3 : 6, g.Co == 32 ? 1 : 2, BoolName(p->w_stem2 != nullptr));
             if (p->w_stem2)
             {
                 if (g.Kh == 3 && g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 1, 16, true>), gridm, dim3(256), 0, stream, a);
@@ -851,6 +857,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         if (nb > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
         const dim3 grid(static_cast<unsigned>(nb));
         a.wpack2 = p->w_dot4b;
+        NoteKernel("SmallCiConvKernel<%d, %d, %s>", g.Kh, p->row_dwords, BoolName(p->w_dot4b != nullptr));
         if (p->w_dot4b)
         {
             if (g.Kh == 3) hipLaunchKernelGGL((SmallCiConvKernel<3, 3, true>), grid, dim3(256), 0, stream, a);
@@ -888,6 +895,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             a.xcd_chunk = static_cast<int>((nb + 7) / 8);
             const dim3 grid(static_cast<unsigned>(a.xcd_chunk) * 8u);
             a.wpack2 = p->w_dot4b;
+            NoteKernel("Depthwise3x3Kernel<%d, %d, %s>", g.stride_x, rows_per_thread, BoolName(p->w_dot4b != nullptr));
             if (p->w_dot4b)
             {
                 if (g.stride_x == 1 && rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2, true>), grid, dim3(256), 0, stream, a);
@@ -906,6 +914,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             return SetError(MI355X_ERR_INVALID_ARGUMENT, "depthwise kernel needs 4-byte aligned tensors");
         const long long total4 = total / 4;
         const unsigned blocks = static_cast<unsigned>((total4 + 255) / 256);
+        NoteKernel("DepthwiseC4Kernel<%s, %s>", BoolName(g.in_u8), BoolName(g.w_u8));
         if (g.in_u8 && !g.w_u8)
             hipLaunchKernelGGL((DepthwiseC4Kernel<true, false>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, ChanTab{p->chan, p->Co_pad}, yout, total4);
         else if (!g.in_u8 && !g.w_u8)
@@ -920,6 +929,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
     default:
     {
         const unsigned blocks = static_cast<unsigned>((total + 255) / 256);
+        NoteKernel("ConvDirectKernel<%s>", BoolName(p->d.depthwise != 0));
         if (p->d.depthwise)
             hipLaunchKernelGGL((ConvDirectKernel<true>), dim3(blocks), dim3(256), 0, stream, g, p->rq, xin, p->w_direct, ChanTab{p->chan, p->Co_pad}, yout, total);
         else
@@ -954,6 +964,7 @@ int LaunchDwPw(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, uint32_t ba
     const int smem = DwPwSmemBytes<S, P>(g.Co);
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&DwPwKernel<S, P, D>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     MI355X_HIP(attr);
+    NoteKernel("DwPwKernel<%d, %d, %d>", S, P, D);
     hipLaunchKernelGGL((DwPwKernel<S, P, D>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(256), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;

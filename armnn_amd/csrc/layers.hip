@@ -468,6 +468,7 @@ int mi355x_activation_run(size_t n, const mi355x_quant* in_q, const mi355x_quant
     if (n == 0) return 0;
     if (!input_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "null tensor pointer");
     Requant rq = MakeRequant(*out_q, MI355X_ACT_NONE, 0.0f, 0.0f);
+    NoteKernel("ActivationKernel");
     hipLaunchKernelGGL(ActivationKernel, dim3(GridFor(n)), dim3(256), 0, ToHip(stream), MakeQIn(*in_q), rq, activation, a, b,
                        static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), n);
     MI355X_HIP(hipGetLastError());
@@ -498,17 +499,29 @@ int mi355x_pool2d_run(const mi355x_pool2d_desc* d, uint32_t batch, const void* i
     const bool global = p.Ho == 1 && p.Wo == 1 && p.pad_top == 0 && p.pad_left == 0 && p.pool_h == p.H && p.pool_w == p.W &&
                         p.H * p.W <= kGlobalPoolMaxTaps;
     if (vec4 && global)
+    {
+        NoteKernel("GlobalPoolKernel");
         hipLaunchKernelGGL(GlobalPoolKernel, dim3(static_cast<unsigned>(batch * ((p.C + 255) / 256))), dim3(256), 0, ToHip(stream), p,
                            MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev));
+    }
     else if (vec4 && p.pool_w <= 3 && p.pool_h <= 3)
+    {
+        NoteKernel("Pool2dC4Kernel<3>");
         hipLaunchKernelGGL(Pool2dC4Kernel<3>, dim3(static_cast<unsigned>((total / 4 + 255) / 256)), dim3(256), 0, ToHip(stream), p,
                            MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), total / 4);
+    }
     else if (vec4 && p.pool_w <= 8 && p.pool_h <= 8)
+    {
+        NoteKernel("Pool2dC4Kernel<8>");
         hipLaunchKernelGGL(Pool2dC4Kernel<8>, dim3(static_cast<unsigned>((total / 4 + 255) / 256)), dim3(256), 0, ToHip(stream), p,
                            MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), total / 4);
+    }
     else
+    {
+        NoteKernel("Pool2dKernel");
         hipLaunchKernelGGL(Pool2dKernel, dim3(static_cast<unsigned>((total + 255) / 256)), dim3(256), 0, ToHip(stream), p,
                            MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), total);
+    }
     MI355X_HIP(hipGetLastError());
     return 0;
 }
@@ -527,12 +540,18 @@ int mi355x_add_run(size_t n, const mi355x_quant* in0_q, const mi355x_quant* in1_
     const bool vec16 = (n % 16) == 0 && ((reinterpret_cast<uintptr_t>(input0_dev) | reinterpret_cast<uintptr_t>(input1_dev) |
                                            reinterpret_cast<uintptr_t>(output_dev)) & 15) == 0;
     if (vec16)
+    {
+        NoteKernel("AddVec16Kernel");
         hipLaunchKernelGGL(AddVec16Kernel, dim3(GridFor(n / 16)), dim3(256), 0, ToHip(stream), MakeQIn(*in0_q), MakeQIn(*in1_q), rq,
                            static_cast<const v4u*>(input0_dev), static_cast<const v4u*>(input1_dev), static_cast<v4u*>(output_dev), n / 16);
+    }
     else
+    {
+        NoteKernel("AddKernel");
         hipLaunchKernelGGL(AddKernel, dim3(GridFor(n)), dim3(256), 0, ToHip(stream), MakeQIn(*in0_q), MakeQIn(*in1_q), rq,
                            activation, a, b, static_cast<const uint8_t*>(input0_dev), static_cast<const uint8_t*>(input1_dev),
                            static_cast<uint8_t*>(output_dev), n);
+    }
     MI355X_HIP(hipGetLastError());
     return 0;
 }
@@ -548,11 +567,20 @@ int mi355x_softmax_run(uint32_t rows, uint32_t cols, float beta, const mi355x_qu
     const uint8_t* xin = static_cast<const uint8_t*>(input_dev);
     uint8_t* yout = static_cast<uint8_t*>(output_dev);
     if (cols <= 1024)
+    {
+        NoteKernel("SoftmaxRowKernel<4>");
         hipLaunchKernelGGL(SoftmaxRowKernel<4>, dim3(rows), dim3(256), 0, ToHip(stream), static_cast<int>(cols), beta, MakeQIn(*in_q), rq, xin, yout);
+    }
     else if (cols <= 2048)
+    {
+        NoteKernel("SoftmaxRowKernel<8>");
         hipLaunchKernelGGL(SoftmaxRowKernel<8>, dim3(rows), dim3(256), 0, ToHip(stream), static_cast<int>(cols), beta, MakeQIn(*in_q), rq, xin, yout);
+    }
     else
+    {
+        NoteKernel("SoftmaxKernel");
         hipLaunchKernelGGL(SoftmaxKernel, dim3(rows), dim3(64), 0, ToHip(stream), static_cast<int>(cols), beta, MakeQIn(*in_q), rq, xin, yout);
+    }
     MI355X_HIP(hipGetLastError());
     return 0;
 }
@@ -616,11 +644,20 @@ int mi355x_pad_run(const mi355x_pad_desc* d, const void* input_dev, void* output
     const uint8_t* xin = static_cast<const uint8_t*>(input_dev);
     uint8_t* yout = static_cast<uint8_t*>(output_dev);
     if (v == 16)
+    {
+        NoteKernel("PadKernel<16>");
         hipLaunchKernelGGL(PadKernel<16>, grid, dim3(256), 0, ToHip(stream), p, MakeQIn(d->input), rq, static_cast<uint32_t>(chunks), xin, yout);
+    }
     else if (v == 4)
+    {
+        NoteKernel("PadKernel<4>");
         hipLaunchKernelGGL(PadKernel<4>, grid, dim3(256), 0, ToHip(stream), p, MakeQIn(d->input), rq, static_cast<uint32_t>(chunks), xin, yout);
+    }
     else
+    {
+        NoteKernel("PadKernel<1>");
         hipLaunchKernelGGL(PadKernel<1>, grid, dim3(256), 0, ToHip(stream), p, MakeQIn(d->input), rq, static_cast<uint32_t>(chunks), xin, yout);
+    }
     MI355X_HIP(hipGetLastError());
     return 0;
 }

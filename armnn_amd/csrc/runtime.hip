@@ -22,6 +22,23 @@ int SetError(int code, const char* fmt, ...)
     return code;
 }
 
+namespace
+{
+char* KernelNameBuffer()
+{
+    static thread_local char buf[192] = {0};
+    return buf;
+}
+} // namespace
+
+void NoteKernel(const char* fmt, ...)
+{
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(KernelNameBuffer(), 192, fmt, ap);
+    va_end(ap);
+}
+
 int UploadNow(void* dst_dev, const void* src_host, size_t bytes)
 {
     // one stream per calling thread, so concurrent plan creations do not wait for each other
@@ -112,6 +129,8 @@ using namespace mi355x;
 extern "C" {
 
 const char* mi355x_last_error(void) { return ErrorBuffer(); }
+
+const char* mi355x_last_kernel(void) { return KernelNameBuffer(); }
 
 int mi355x_abi_version(void) { return MI355X_ABI_VERSION; }
 
@@ -287,6 +306,7 @@ int mi355x_fill_u8(void* dst_dev, uint8_t value, size_t bytes, mi355x_stream_t s
     if (!dst_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "dst is null");
     size_t blocks = (bytes + 255) / 256;
     if (blocks > 65535) blocks = 65535;
+    NoteKernel("FillU8Kernel");
     hipLaunchKernelGGL(FillU8Kernel, dim3(static_cast<unsigned>(blocks)), dim3(256), 0, ToHip(stream),
                        static_cast<uint8_t*>(dst_dev), value, bytes);
     MI355X_HIP(hipGetLastError());

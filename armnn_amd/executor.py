@@ -236,8 +236,9 @@ class DeviceNetwork:
         return self.download()
 
     def time_layers(self, iters: int = 20, warmup: int = 3):
-        """Device time in ms of one launch of every step, as launched by enqueue() (lane 0's slice of the batch when
-        the network runs in lanes), alone on the launch stream, timed with HIP events on that stream."""
+        """(layer, device time in ms of one launch, kernel name) of every step, as launched by enqueue() (lane 0's slice
+        of the batch when the network runs in lanes), alone on the launch stream, timed with HIP events on that stream.
+        The kernel name is what the library reports for the step's last launch (mi355x_last_kernel)."""
         e0, e1 = self.dev.event(), self.dev.event()
         out = []
         for l, fn in self.steps:
@@ -248,7 +249,8 @@ class DeviceNetwork:
                 fn(self.stream, 0, self.lanes)
             self.dev.event_record(e1, self.stream)
             self.dev.event_sync(e1)
-            out.append((l, self.dev.elapsed_ms(e0, e1) / iters))
+            kernel = self.lib.mi355x_last_kernel().decode(errors="replace")
+            out.append((l, self.dev.elapsed_ms(e0, e1) / iters, kernel))
         return out
 
     def close(self):

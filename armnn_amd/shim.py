@@ -21,7 +21,7 @@ ACT_NONE, ACT_RELU, ACT_BOUNDED_RELU = 0, 1, 2
 
 #: every symbol include/armnn_mi355x.h declares
 EXPORTS = [
-    "mi355x_last_error", "mi355x_abi_version", "mi355x_set_option", "mi355x_device_count", "mi355x_init", "mi355x_device_name",
+    "mi355x_last_error", "mi355x_last_kernel", "mi355x_abi_version", "mi355x_set_option", "mi355x_device_count", "mi355x_init", "mi355x_device_name",
     "mi355x_device_props", "mi355x_malloc", "mi355x_free", "mi355x_host_alloc", "mi355x_host_device_pointer", "mi355x_host_free",
     "mi355x_memcpy_h2d", "mi355x_memcpy_d2h", "mi355x_memcpy_d2d", "mi355x_memcpy_h2d_async", "mi355x_memcpy_d2h_async", "mi355x_fill_u8", "mi355x_stream_create",
     "mi355x_stream_destroy", "mi355x_stream_synchronize", "mi355x_device_synchronize", "mi355x_event_create",
@@ -93,6 +93,7 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
                                     f"(or __graft_entry__.build()); there is no fallback path")
         _lib = C.CDLL(path)
         _lib.mi355x_last_error.restype = C.c_char_p
+        _lib.mi355x_last_kernel.restype = C.c_char_p
         V = C.c_void_p
         sig = {
             "mi355x_malloc": [C.POINTER(V), C.c_size_t], "mi355x_free": [V],

@@ -5,13 +5,19 @@ A step is one forward pass of the whole network over one batch that is already r
 runs on the device through the C ABI; the pass is replayed as one HIP graph).  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 64] [--net mobilenet_v1|resnet50]
-                  [--weights per_channel_s8|per_tensor_u8] [--no-cpu-baseline] [--layers]
+                  [--weights per_channel_s8|per_tensor_u8] [--no-cpu-baseline] [--no-backend] [--layers]
 
 The headline workload is the default: per-channel QSymmS8 weights.  --weights per_tensor_u8 runs the same network with
 QAsymmU8 weights that have one scale and a zero point per layer, and says so in config.workload.
 
 Extra objects in the line:
-  roofline      the kernel with the largest share of the step (HIP-event timed on the launch stream)
+  roofline      the kernel SYMBOL with the largest summed time over one step: algorithmic work of all its launches over
+                their summed time (each launch HIP-event timed alone on the launch stream), `traffic` = the summed counter
+                bytes of those launches from the committed rocprofv3 summary (null when the profile was taken with other
+                kernels than run now); roofline_next holds the next two symbols
+  config.backend_path   the same network through IRuntime::EnqueueWorkload on the C++ backend (child process, wall clock,
+                host buffers in and out: pageable, and pinned buffers adopted with ImportInputs / ImportOutputs); its output
+                bytes are compared with the executor's
   groups        conv/FC ops vs the int8 MFMA peak and depthwise bytes vs the HBM peak over the whole net
   cpu_baseline  the reference's own CpuRef code (oracle/_ref, kind "reference") or the C restatement
                 (kind "port"), one thread, on a bounded sample of the same workload
@@ -31,74 +37,28 @@ INT8_MFMA_PEAK_OPS = 5.0e15      # MI355X dense int8, ops/s
 HBM_PEAK_BYTES = 8.0e12          # MI355X HBM3E, B/s
 RIDGE_OPS_PER_BYTE = INT8_MFMA_PEAK_OPS / HBM_PEAK_BYTES
 
-# HBM bytes per launch (read + written) of each MobileNetV1 layer, keyed by the images one launch covers (32 = one of
-# the two lanes of the default run), from two rocprofv3 --pmc passes (FETCH_SIZE, then WRITE_SIZE) over
-# `python3 bench.py --profile-pass --no-graph` (batch-64 entries: `--lanes 1`), each scaled by what the same counter
-# reads for the 64 MiB calibration copy of that pass (FETCH_SIZE counts 2 KiB units on this device: factor 1.999;
-# WRITE_SIZE 1 KiB units: factor 1.000).  Summary: profiles/mobilenet_v1_b64_hbm_traffic.md.
-MEASURED_HBM_TRAFFIC = {
-    ("mobilenet_v1_1.0_224", 32): {
-        "stem": 21485289,
-        "dw1": 25858383,
-        "pw1": 38751390,
-        "dw2": 32236845,
-        "pw2": 19656450,
-        "dw3": 25886017,
-        "pw3": 26132677,
-        "dw4": 16206570,
-        "pw4": 10235764,
-        "dw5": 13085401,
-        "pw5": 13540596,
-        "dw6": 8216572,
-        "pw6": 6180643,
-        "dw7": 6736907,
-        "pw7": 8934584,
-        "dw8": 6733324,
-        "pw8": 8931769,
-        "dw9": 6733708,
-        "pw9": 8932281,
-        "dw10": 6734988,
-        "pw10": 8931641,
-        "dw11": 6732557,
-        "pw11": 8932537,
-        "dw12": 4223300,
-        "pw12": 7106219,
-        "dw13": 3586967,
-        "pw13": 12327782,
-        "avgpool": 1687743,
-        "logits": 1453028,
-        "softmax": 127440
-    },
-    ("mobilenet_v1_1.0_224", 64): {
-        "dw1": 51482293,
-        "pw1": 77282791,
-        "dw2": 64298192,
-        "pw2": 38912815,
-        "dw3": 51513126,
-        "pw3": 51807254,
-        "dw4": 32217414,
-        "pw4": 19858707,
-        "dw5": 25869979,
-        "pw5": 26564936,
-        "dw6": 16205108,
-        "pw6": 10982215,
-        "dw7": 13107001,
-        "pw7": 15305224,
-        "dw8": 13106106,
-        "pw8": 15305736,
-        "dw9": 13104059,
-        "pw9": 15306376,
-        "dw10": 13104187,
-        "pw10": 15305608,
-        "dw11": 13104827,
-        "pw11": 15306120,
-        "dw12": 8241622,
-        "pw12": 9543656,
-        "dw13": 6807456,
-        "pw13": 15567723,
-        "softmax": 194497
-    },
+TRAFFIC_PROFILES = {
+    # (network name, images per launch) -> rocprofv3 counter summary written by `python -m armnn_amd.profile_summary traffic`
+    ("mobilenet_v1_1.0_224", 32): os.path.join(ROOT, "profiles", "mobilenet_v1_b64_hbm_traffic.md"),
 }
+
+
+def measured_traffic(net_name, launch_batch):
+    """{layer: (kernel name, HBM bytes read + written per launch)} from the committed counter summary of this workload
+    (FETCH_SIZE and WRITE_SIZE passes, each scaled by a calibration copy; the file says how it was made), or {}."""
+    path = TRAFFIC_PROFILES.get((net_name, launch_batch))
+    table = {}
+    if not path or not os.path.exists(path):
+        return table
+    with open(path) as f:
+        for line in f:
+            cells = [c.strip() for c in line.strip().strip("|").split("|")]
+            if len(cells) >= 5 and cells[1].startswith("`"):
+                try:
+                    table[cells[0]] = (cells[1].strip("`"), float(cells[4]) * 1e6)
+                except ValueError:
+                    pass
+    return table
 
 
 def layer_work(net, l, batch):
@@ -150,17 +110,43 @@ def cpu_baseline(net, seconds_budget=25.0):
             "sample": f"{images} image(s) of the same network at batch 1, {elapsed:.1f} s, 1 thread of {os.cpu_count()}"}
 
 
+def run_backend_child(net, batch, steps, warmup):
+    """The same network through the C++ backend (INetwork -> Optimize -> LoadNetwork -> IRuntime::EnqueueWorkload) in a
+    child process, started before this process has touched the GPU.  Returns (figures, output bytes) or (error, None)."""
+    import subprocess
+    import tempfile
+    import numpy as np
+    from armnn_amd import netfile, nets
+    exe = os.path.join(ROOT, "armnn_amd", "backend", "test", "bin", "backend_bench")
+    if not os.path.exists(exe):
+        return {"error": "armnn_amd/backend/test/bin/backend_bench is not built"}, None
+    with tempfile.TemporaryDirectory(prefix="mi355x_bench_") as tmp:
+        nf, fin, fout = (os.path.join(tmp, n) for n in ("net.bin", "input.bin", "output.bin"))
+        netfile.write_net(net, batch, nf)
+        np.ascontiguousarray(nets.synthetic_input(net, batch).data).tofile(fin)
+        try:
+            r = subprocess.run([exe, nf, fin, fout, str(steps), str(warmup)], capture_output=True, text=True, timeout=300)
+        except subprocess.TimeoutExpired:
+            return {"error": "backend_bench timed out"}, None
+        if r.returncode != 0:
+            return {"error": f"backend_bench exit {r.returncode}: {r.stderr.strip()[-300:]}"}, None
+        fig = json.loads(r.stdout.strip().splitlines()[-1])
+        with open(fout, "rb") as f:
+            return fig, f.read()
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--steps", type=int, default=3000, help="timed forward passes (the default keeps the timed region above a second)")
+    ap.add_argument("--warmup", type=int, default=100)
     ap.add_argument("--batch", type=int, default=64)
     ap.add_argument("--net", default="mobilenet_v1", choices=["mobilenet_v1", "resnet50"])
     ap.add_argument("--weights", default="per_channel_s8", choices=["per_channel_s8", "per_tensor_u8"],
                     help="mobilenet_v1 only: per_tensor_u8 gives every layer QAsymmU8 weights with one scale and a zero point "
                          "(the quantization of older uint8 models) instead of the headline workload's per-channel QSymmS8")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-backend", action="store_true", help="skip the run through the C++ backend (config.backend_path)")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--fuse", action="store_true",
                     help="run depthwise + pointwise pairs as one kernel (same bytes; slower than two launches at present)")
@@ -176,11 +162,19 @@ def main():
               "(the path shards by batch with no exchange step: one process per GPU would run the same plans on its slice).", file=sys.stderr)
         return 2
 
-    from armnn_amd import nets, shim
-    from armnn_amd.executor import DeviceNetwork
-
+    from armnn_amd import nets
     net = nets.mobilenet_v1(weights=args.weights) if args.net == "mobilenet_v1" else nets.resnet50()
     batch = args.batch
+
+    # ---- the product path north_star names: the backend behind IRuntime::EnqueueWorkload, in a child process that is
+    # started (and has ended) before anything here touches the GPU
+    backend, backend_out = (None, None)
+    if not args.no_backend and not args.profile_pass:
+        backend, backend_out = run_backend_child(net, batch, max(50, args.steps // 4), 20)
+
+    from armnn_amd import shim
+    from armnn_amd.executor import DeviceNetwork
+
     dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse, lanes=args.lanes)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev
@@ -193,10 +187,14 @@ def main():
         shim._chk(dn.lib.mi355x_fill_u8(a.ptr, 1, n, dn.stream))
         dev.stream_sync(dn.stream)
         shim._chk(dn.lib.mi355x_activation_run(n, C.byref(q), C.byref(q), shim.ACT_BOUNDED_RELU, 1000.0, -1000.0, a.ptr, b.ptr, dn.stream))
+        kernels = []
         for _, fn in dn.steps:
             fn(dn.stream, 0, args.lanes)                 # lane 0's launch of every layer, as the timed region launches it
+            kernels.append(dn.lib.mi355x_last_kernel().decode(errors="replace"))
         dev.stream_sync(dn.stream)
         print(json.dumps({"dispatch_order": ["fill (setup)", f"calibration copy {n} B in + {n} B out"] + [l.name for l, _ in dn.steps],
+                          "kernels": ["FillU8Kernel", "ActivationKernel"] + kernels,
+                          "algorithmic_bytes": [n, 2 * n] + [algorithmic_bytes(net, l, batch // args.lanes) for l, _ in dn.steps],
                           "batch": batch, "launch_batch": batch // args.lanes, "net": net.name}))
         dn.close()
         return 0
@@ -211,46 +209,73 @@ def main():
     t1 = time.perf_counter()
     ms_per_step = (t1 - t0) * 1e3 / args.steps
     images_per_s = batch * args.steps / (t1 - t0)
+    executor_out = dn.download().data.tobytes()
 
     # ---- per-kernel timing on the launch stream, for the roofline object ------------------------------------
     # (one launch = one layer over one lane's slice of the batch; in the timed region `lanes` such launches of a layer
     # run side by side on their own streams)
     launch_batch = batch // args.lanes
-    per_layer = dn.time_layers(iters=20, warmup=3)
+    per_layer = dn.time_layers(iters=50, warmup=10)
+    traffic = measured_traffic(net.name, launch_batch)
     rows = []
-    for l, ms in per_layer:
+    for l, ms, kernel in per_layer:
         kind, work = layer_work(net, l, launch_batch)
         peak = INT8_MFMA_PEAK_OPS if kind == "mfma" else HBM_PEAK_BYTES
-        row = {"layer": l.name, "op": l.op, "ms": ms, "bound": kind, "work": work, "frac": work / (ms * 1e-3) / peak}
+        row = {"layer": l.name, "op": l.op, "ms": ms, "bound": kind, "work": work, "frac": work / (ms * 1e-3) / peak, "kernel": kernel}
         if kind == "mfma":
             # the roof that binds a conv / FC layer depends on its arithmetic intensity: below the ridge
             # (peak ops / peak bytes = 625 ops/B) the HBM roof is the lower one
             nbytes = float(algorithmic_bytes(net, l, launch_batch))
             row["bytes"] = nbytes
+            row["ops"] = work
             row["binding"] = "mfma" if work / nbytes >= RIDGE_OPS_PER_BYTE else "hbm"
         else:
             row["bytes"] = work
+            row["ops"] = 0.0
             row["binding"] = "hbm"
+        # counter bytes of this layer's launch, only while the profile was taken with the kernel that runs now
+        t = traffic.get(l.name)
+        row["traffic"] = t[1] if t and t[0] == kernel else None
         rows.append(row)
     total_ms = sum(r["ms"] for r in rows)
-    dom = max(rows, key=lambda r: r["ms"])
     if args.layers:
         for r in rows:
             hbm = r["bytes"] / (r["ms"] * 1e-3) / HBM_PEAK_BYTES
             print(f"{r['layer']:>10s} {r['op']:>9s} {r['ms']*1e3:9.1f} us  {r['bound']:>4s} {100*r['frac']:6.2f}% of peak"
-                  f"   binding roof {r['binding']:>4s}, {100*hbm:5.1f}% of HBM peak on algorithmic bytes", file=sys.stderr)
+                  f"   binding roof {r['binding']:>4s}, {100*hbm:5.1f}% of HBM peak on algorithmic bytes   {r['kernel']}", file=sys.stderr)
         print(f"launches of {launch_batch} images; sum of one lane's launches {total_ms:.3f} ms; step of {args.lanes} lane(s) "
               f"{ms_per_step:.3f} ms", file=sys.stderr)
-    if dom["binding"] == "mfma":
-        roof = {"bound": "mfma", "achieved": dom["work"] / (dom["ms"] * 1e-3) / 1e12, "peak": INT8_MFMA_PEAK_OPS / 1e12,
-                "unit": "TOP/s"}
-    else:
-        roof = {"bound": "hbm", "achieved": dom["bytes"] / (dom["ms"] * 1e-3) / 1e9, "peak": HBM_PEAK_BYTES / 1e9,
-                "unit": "GB/s"}
-    roof["frac"] = roof["achieved"] / roof["peak"]
-    roof["traffic"] = MEASURED_HBM_TRAFFIC.get((net.name, launch_batch), {}).get(dom["layer"])
-    roof["kernel"] = (f"{dom['layer']} ({dom['op']}), one launch over {launch_batch} images: {dom['ms']*1e3:.1f} us of "
-                      f"{total_ms*1e3:.1f} us for all layers")
+
+    # ---- the dominant kernel: the symbol with the largest summed time over one step
+    by_kernel = {}
+    for r in rows:
+        by_kernel.setdefault(r["kernel"], []).append(r)
+
+    def kernel_roof(name):
+        sel = by_kernel[name]
+        t = sum(r["ms"] for r in sel) * 1e-3
+        ops, nbytes = sum(r["ops"] for r in sel), sum(r["bytes"] for r in sel)
+        mfma_bound = ops > 0 and ops / nbytes >= RIDGE_OPS_PER_BYTE
+        if mfma_bound:
+            roof = {"bound": "mfma", "achieved": ops / t / 1e12, "peak": INT8_MFMA_PEAK_OPS / 1e12, "unit": "TOP/s"}
+        else:
+            roof = {"bound": "hbm", "achieved": nbytes / t / 1e9, "peak": HBM_PEAK_BYTES / 1e9, "unit": "GB/s"}
+        roof["frac"] = roof["achieved"] / roof["peak"]
+        roof["traffic"] = sum(r["traffic"] for r in sel) if all(r["traffic"] is not None for r in sel) else None
+        roof["kernel"] = name
+        roof["launches_per_lane_pass"] = len(sel)
+        roof["layers"] = [r["layer"] for r in sel]
+        roof["avg_launch_us"] = t * 1e6 / len(sel)
+        roof["share_of_lane_pass"] = t * 1e3 / total_ms
+        roof["algorithmic_bytes"] = nbytes
+        if ops > 0:
+            roof["TOPS"] = ops / t / 1e12
+            roof["frac_of_int8_mfma_peak"] = ops / t / INT8_MFMA_PEAK_OPS
+        return roof
+
+    ranked = sorted(by_kernel, key=lambda k: -sum(r["ms"] for r in by_kernel[k]))
+    roof = kernel_roof(ranked[0])
+    runners_up = [kernel_roof(k) for k in ranked[1:3]]
 
     def group(ops, peak):
         sel = [r for r in rows if r["op"] in ops]
@@ -266,16 +291,29 @@ def main():
     if g_dw:
         groups["depthwise"] = {"ms": g_dw["ms"], "GBps": g_dw["achieved"] / 1e9, "frac_of_hbm_peak": g_dw["frac"]}
 
+    config = {"workload": f"{net.name} int8 (QAsymm activations, {'per-channel QSymmS8' if args.weights == 'per_channel_s8' or args.net != 'mobilenet_v1' else 'per-tensor QAsymmU8'} weights), batch {batch}, "
+                          f"random-init, whole forward pass incl. avgpool/FC/softmax, input resident in HBM, every layer through the C ABI, "
+                          f"one HIP graph replay per step",
+              "batch": batch, "graph_replay": not args.no_graph, "fused_depthwise_pointwise": args.fuse, "lanes": args.lanes,
+              "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12}
+    if backend is not None:
+        # the same network and input through the C++ backend: wall clock per IRuntime::EnqueueWorkload call, host buffers in
+        # and out (PCIe inclusive; never `value`)
+        bp = dict(backend)
+        if backend_out is not None:
+            bp["output_equals_executor"] = backend_out == executor_out
+            bp["images_per_sec_pageable_io"] = batch / (backend["ms_pageable"] * 1e-3)
+            bp["images_per_sec_adopted_pinned_io"] = batch / (backend["ms_pinned"] * 1e-3)
+            bp["path"] = "INetwork -> Optimize({Mi355x}) -> IRuntime::LoadNetwork -> IRuntime::EnqueueWorkload (armnn_amd/backend/test/BackendBench.cpp)"
+        config["backend_path"] = bp
+
     line = {
         "metric": "int8 images/sec MobileNetV1 b64 @1 GPU" if args.net == "mobilenet_v1" else f"int8 images/sec {args.net} b{batch} @1 GPU",
         "value": images_per_s, "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
-        "config": {"workload": f"{net.name} int8 (QAsymm activations, {'per-channel QSymmS8' if args.weights == 'per_channel_s8' or args.net != 'mobilenet_v1' else 'per-tensor QAsymmU8'} weights), batch {batch}, "
-                               f"random-init, whole forward pass incl. avgpool/FC/softmax, input resident in HBM",
-                   "batch": batch, "graph_replay": not args.no_graph, "fused_depthwise_pointwise": args.fuse, "lanes": args.lanes,
-                   "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12},
-        "roofline": roof, "groups": groups,
+        "config": config,
+        "roofline": roof, "roofline_next": runners_up, "groups": groups,
     }
     # what the device itself delivers on register-only MFMA chains and on a plain copy, next to the published peaks
     from armnn_amd import peaks

@@ -207,6 +207,11 @@ int mi355x_conv2d_run_fused(mi355x_conv2d_t depthwise, mi355x_conv2d_t pointwise
                             const void* input_dev, void* output_dev, mi355x_stream_t stream);
 /* which kernel a plan resolved to (mi355x_algo) and its tile configuration, for logs and tests */
 int mi355x_conv2d_algo(mi355x_conv2d_t plan, int32_t* algo, char* desc_buf, size_t desc_len);
+/* Name of the device kernel the calling thread's last *_run call launched, with its template arguments, as a profiler
+ * lists it (without namespace and argument list); "" before the first launch.  The reference reports what a workload
+ * resolved to through its profiler the same way (ARMNN_REPORT_PROFILING_WORKLOAD_DESC, src/armnn/Profiling.hpp:227-236;
+ * ClConvolution2dWorkload reports its ConvolutionMethod, src/backends/cl/workloads/ClConvolution2dWorkload.cpp:135-161). */
+const char* mi355x_last_kernel(void);
 
 /* ------------------------------------------------------------------------------------------------------
  * FullyConnected
