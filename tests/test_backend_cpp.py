@@ -16,7 +16,7 @@ BIN = os.path.join(BACKEND, "test", "bin")
 
 
 def _ensure_built():
-    need = [os.path.join(BIN, "backend_tests"), os.path.join(BIN, "dynamic_tests"),
+    need = [os.path.join(BIN, "backend_tests"), os.path.join(BIN, "dynamic_tests"), os.path.join(BIN, "backend_bench"),
             os.path.join(ROOT, "armnn_amd", "lib", "Amd_Mi355x_backend.so")]
     if all(os.path.exists(p) for p in need):
         return
@@ -54,6 +54,43 @@ def test_backend_networks_on_device():
 @pytest.mark.gpu
 def test_backend_dynamic_on_device():
     _run("dynamic_tests", "gpu", 300)
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("name,batch", [("resnet50", 32), ("mobilenet_v1", 64)])
+def test_benchmark_network_through_the_backend_equals_the_executor(tmp_path, name, batch):
+    """ResNet-50 at batch 32 (7x7 stem, max pooling, 16 residual adds with their ReLU folded in, 53 convolutions) and
+    MobileNetV1 at batch 64, from one network file: INetwork -> Optimize({Mi355x}) -> LoadNetwork -> EnqueueWorkload in
+    backend_bench gives the bytes the C-ABI executor gives (which the network tests tie to the CPU checker), with pageable
+    and with adopted pinned host buffers; no Activation layer survives optimization and no copy layer is inserted."""
+    import json
+
+    import numpy as np
+
+    from armnn_amd import netfile, nets
+    from armnn_amd.executor import DeviceNetwork
+
+    _ensure_built()
+    exe = os.path.join(BIN, "backend_bench")
+    assert os.path.exists(exe), "backend_bench is not built"
+    net = nets.resnet50() if name == "resnet50" else nets.mobilenet_v1()
+    x = nets.synthetic_input(net, batch, seed=11)
+    nf, fin, fout = (str(tmp_path / n) for n in ("net.bin", "input.bin", "output.bin"))
+    netfile.write_net(net, batch, nf)
+    np.ascontiguousarray(x.data).tofile(fin)
+    proc = subprocess.run([exe, nf, fin, fout, "20", "3"], capture_output=True, text=True, timeout=300)
+    assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
+    fig = json.loads(proc.stdout.strip().splitlines()[-1])
+    print(f"{name} b{batch} through EnqueueWorkload: {fig['ms_pageable']:.3f} ms pageable I/O = {batch / fig['ms_pageable'] * 1e3:.0f} images/s, "
+          f"{fig['ms_pinned']:.3f} ms adopted pinned I/O = {batch / fig['ms_pinned'] * 1e3:.0f} images/s; {fig}", flush=True)
+    assert fig["pinned_equals_pageable"] and fig["activation_layers_left"] == 0 and fig["memcopy_layers"] == 0
+    assert fig["add_layers"] == (16 if name == "resnet50" else 0)
+    dn = DeviceNetwork(net, batch, use_graph=False)
+    want = dn.run(x).data.tobytes()
+    dn.close()
+    with open(fout, "rb") as f:
+        got = f.read()
+    assert got == want, "the backend's output differs from the executor's"
 
 
 @pytest.mark.skipif(not os.path.isdir("/root/reference/include/armnn"), reason="needs an Arm NN source tree")
