@@ -92,7 +92,8 @@ class DeviceNetwork:
                 d = shim.Pool2dDesc(h, w, c, ho, wo, p["pool_w"], p["pool_h"], p["stride_x"], p["stride_y"], p["pad_left"],
                                     p["pad_right"], p["pad_top"], p["pad_bottom"], p["pool_type"], p["padding_method"],
                                     shim._quant(xin[0]), shim._quant(yout))
-                self.steps.append((l, self._pool_step(d, xb[0].ptr, yb.ptr, xin[0].num_elements, yout.num_elements)))
+                self.steps.append((l, self._pool_step(d, xb[0].ptr, yb.ptr, xin[0].num_elements, yout.num_elements, l.act,
+                                                      shim._quant(yout))))
                 self._step_plans.append(None)
             elif l.op == "add":
                 q0, q1, qo = shim._quant(xin[0]), shim._quant(xin[1]), shim._quant(yout)
@@ -150,10 +151,18 @@ class DeviceNetwork:
         batch = self.batch
         return lambda s, lane=0, lanes=1: plan.run(batch // lanes, x + lane * (nx // lanes), y + lane * (ny // lanes), s)
 
-    def _pool_step(self, d, x, y, nx, ny):
+    def _pool_step(self, d, x, y, nx, ny, act=(0, 0.0, 0.0), qo=None):
+        """Pooling, then -- when the layer carries a fused activation, as a parsed AVERAGE_POOL_2D / MAX_POOL_2D may
+        (src/armnnTfLiteParser/TfLiteParser.cpp ParsePool -> AddFusedActivationLayer) -- the activation in place on the
+        pooled tensor, in the output's own quantization."""
         batch, lib = self.batch, self.lib
-        return lambda s, lane=0, lanes=1: shim._chk(lib.mi355x_pool2d_run(C.byref(d), batch // lanes, x + lane * (nx // lanes),
-                                                                          y + lane * (ny // lanes), s))
+
+        def run(s, lane=0, lanes=1):
+            out = y + lane * (ny // lanes)
+            shim._chk(lib.mi355x_pool2d_run(C.byref(d), batch // lanes, x + lane * (nx // lanes), out, s))
+            if act[0] != 0:
+                shim._chk(lib.mi355x_activation_run(ny // lanes, C.byref(qo), C.byref(qo), act[0], act[1], act[2], out, out, s))
+        return run
 
     def _add_step(self, n, q0, q1, qo, act, x0, x1, y):
         lib = self.lib

@@ -188,6 +188,20 @@ def test_tflite_model_with_standalone_activations(port):
     _layerwise(port, net, 32)
 
 
+def test_tflite_pooling_with_fused_activations(port):
+    """The clamp of a fused RELU6 / RELU behind MAX_POOL_2D / AVERAGE_POOL_2D: with input scale 0.1 and offset -20 the
+    codes span -10.8 .. 14.7, so both bounds bite and a dropped activation changes most outputs."""
+    from armnn_amd import tflite
+    from tests.test_tflite import pool_activation_model
+    net = tflite.parse(pool_activation_model(), "poolact")
+    assert [l.act[0] for l in net.layers if l.op == "pool"] == [2, 1]
+    x = nets.synthetic_input(net, 4)
+    ref = netref.run_network(port, net, x, keep=True)
+    pooled = [l.output for l in net.layers if l.op == "pool"]
+    assert ref[pooled[0]].data.max() == -20 + 60 and ref[pooled[0]].data.min() == -20      # 6.0 and 0.0 in codes: both bounds bite
+    _layerwise(port, net, 4)
+
+
 def test_tflite_model_with_quantize_and_squeeze(port):
     from armnn_amd import tflite
     from tests.test_tflite import quantize_squeeze_model

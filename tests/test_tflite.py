@@ -12,6 +12,18 @@ from tests import tflite_writer as tw
 from tests.helpers import GOLDEN
 
 
+def pool_activation_model(seed=5):
+    """MAX_POOL_2D with a fused RELU6 and AVERAGE_POOL_2D with a fused RELU: the clamps must survive on the device."""
+    rng = np.random.default_rng(seed)
+    b = tw.ModelBuilder()
+    x = b.tensor("input", (1, 12, 12, 16), tw.INT8, 0.1, -20)
+    m = b.tensor("maxpool/out", (1, 6, 6, 16), tw.INT8, 0.1, -20)
+    b.op(tw.MAX_POOL_2D, [x], [m], tw.OPT_POOL, {0: ("b", tw.SAME), 1: ("i", 2), 2: ("i", 2), 3: ("i", 2), 4: ("i", 2), 5: ("b", tw.ACT_RELU6)})
+    a = b.tensor("avgpool/out", (1, 3, 3, 16), tw.INT8, 0.1, -20)
+    b.op(tw.AVERAGE_POOL_2D, [m], [a], tw.OPT_POOL, {0: ("b", tw.VALID), 1: ("i", 2), 2: ("i", 2), 3: ("i", 2), 4: ("i", 2), 5: ("b", tw.ACT_RELU)})
+    return b.finish([x], [a])
+
+
 def mock_model():
     return tflite.load(os.path.join(GOLDEN, "mock_model.tflite"))
 
