@@ -605,18 +605,28 @@ public:
     Status LoadNetwork(NetworkId& idOut, IOptimizedNetworkPtr network, std::string& error,
                        const INetworkProperties& properties = INetworkProperties(MemorySource::Undefined, MemorySource::Undefined))
     {
-        const NetworkId id = m_NextId++;
+        NetworkId id;
+        {
+            std::lock_guard<std::mutex> lock(m_NetworksMutex);
+            id = m_NextId++;
+        }
         idOut = id;
         for (auto& c : m_Contexts) c.second->BeforeLoadNetwork(id);
+        std::unique_ptr<LoadedNetwork> loaded;
         try
         {
-            m_Networks[id] = std::make_unique<LoadedNetwork>(std::move(network), properties);
+            // built outside the lock (plans are created and constants uploaded here); only the map is guarded, as
+            // RuntimeImpl::LoadNetwork does with m_Mutex (src/armnn/Runtime.cpp:153-200)
+            loaded = std::make_unique<LoadedNetwork>(std::move(network), properties);
         }
         catch (const Exception& e)
         {
             error = e.what();
-            m_Networks.erase(id);
             return Status::Failure;
+        }
+        {
+            std::lock_guard<std::mutex> lock(m_NetworksMutex);
+            m_Networks[id] = std::move(loaded);
         }
         for (auto& c : m_Contexts) c.second->AfterLoadNetwork(id);
         return Status::Success;
@@ -624,6 +634,7 @@ public:
 
     LoadedNetwork& Get(NetworkId id) const
     {
+        std::lock_guard<std::mutex> lock(m_NetworksMutex);
         auto it = m_Networks.find(id);
         if (it == m_Networks.end()) throw InvalidArgumentException("Unknown network id " + std::to_string(id));
         return *it->second;
@@ -651,7 +662,18 @@ public:
     Status Unload(NetworkId id)
     {
         for (auto& c : m_Contexts) c.second->BeforeUnloadNetwork(id);
-        const bool erased = m_Networks.erase(id) != 0;
+        std::unique_ptr<LoadedNetwork> gone;
+        {
+            std::lock_guard<std::mutex> lock(m_NetworksMutex);
+            auto it = m_Networks.find(id);
+            if (it != m_Networks.end())
+            {
+                gone = std::move(it->second);
+                m_Networks.erase(it);
+            }
+        }
+        const bool erased = gone != nullptr;
+        gone.reset();                           // the network's memory is released outside the lock
         for (auto& c : m_Contexts) c.second->AfterUnloadNetwork(id);
         return erased ? Status::Success : Status::Failure;
     }
@@ -660,6 +682,7 @@ public:
 private:
     std::map<BackendId, IBackendInternal::IBackendContextPtr> m_Contexts;
     std::map<NetworkId, std::unique_ptr<LoadedNetwork>> m_Networks;
+    mutable std::mutex m_NetworksMutex;         // guards m_Networks and m_NextId: networks may be loaded, run and unloaded from several threads
     BackendIdSet m_AllocatorsAdded, m_StrategiesAdded;
     NetworkId m_NextId = 0;
 };

@@ -8,6 +8,7 @@
 #include "igemm_lds_kernel.h"
 #include "big_gemm.h"
 
+#include <algorithm>
 #include <cmath>
 #include <cstdlib>
 #include <string>
@@ -41,6 +42,8 @@ struct mi355x_conv2d_s
     int pw_bn = 0, pw_ks = 0;      // pointwise GEMM kernel configuration (0: not applicable)
     bool bk128 = false;            // implicit GEMM walks K in 128-byte tiles
     int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 96 (= 128x64) / 128: the "igemm_tile" option at plan creation
+    int opt_igemm_lds = 2, opt_dw_rows = 0, opt_stem_dot4 = 0;     // the other process-wide options, as they stood at plan creation
+                                   // (launches read the plan, never the mutable globals: plans may run on any host thread)
     uint32_t xor_mask = 0, pad_word = 0;
     int zw_neg = 0;                // MFMA plans: minus the zero point of the stored int8 weights (0: symmetric)
     int rowsum_bias = 0;           // ... and what the bytes between K and K_pad add to a row's sum of activations
@@ -124,6 +127,9 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     }
 
     p->d = d;
+    p->opt_igemm_lds = GlobalOptions().igemm_lds;
+    p->opt_dw_rows = GlobalOptions().dw_rows;
+    p->opt_stem_dot4 = GlobalOptions().stem_dot4;
     const int Co = static_cast<int>(d.out_c), Ci = static_cast<int>(d.in_c);
     const int Kh = static_cast<int>(d.kernel_h), Kw = static_cast<int>(d.kernel_w);
     ConvGeom& g = p->geom;
@@ -138,6 +144,21 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     p->rq = MakeRequant(d.output, d.activation, d.activation_a, d.activation_b);
 
     p->K = d.depthwise ? Kh * Kw : Kh * Kw * Ci;
+    // Every kernel accumulates sum (x - zx)(w - zw) in 32 bits.  CpuRef accumulates in float and saturates at the end, so
+    // a sum that could wrap here is refused rather than computed wrongly: K * max|x - zx| * max|w - zw| must stay below 2^31.
+    {
+        const long long xmax = g.in_u8 ? std::max(std::abs(0 - g.zx), std::abs(255 - g.zx)) : std::max(std::abs(-128 - g.zx), std::abs(127 - g.zx));
+        const size_t nw = static_cast<size_t>(d.depthwise ? 1 : Co) * Kh * Kw * (d.depthwise ? Co : Ci);
+        const uint8_t* wb = static_cast<const uint8_t*>(weights_host);
+        long long wmax = 0;
+        for (size_t i = 0; i < nw; ++i)
+        {
+            const int wv = g.w_u8 ? static_cast<int>(wb[i]) : static_cast<int>(static_cast<int8_t>(wb[i]));
+            wmax = std::max<long long>(wmax, std::abs(wv - g.zw));
+        }
+        if (static_cast<long long>(p->K) * xmax * wmax >= (1ll << 31))
+            return SetError(MI355X_ERR_UNSUPPORTED, "%d taps of up to %lld x %lld could overflow the 32-bit accumulator", p->K, xmax, wmax);
+    }
     p->Co_pad = (Co + 127) / 128 * 128;
     // K is padded to the implicit GEMM's k-tile.  128-byte tiles pay when a row chunk is one whole cache line, i.e. when
     // 128 consecutive K bytes are contiguous in memory (input channels a multiple of 128) and K needs no extra padding
@@ -779,7 +800,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const long long huge = ((M + 255) / 256) * ((g.Co + 255) / 256);
         const int tile = p->tile_override ? p->tile_override : big < 400 ? 64 : (huge >= 192 && g.Co >= 256) ? 512 : 128;
         // channel counts that are multiples of 128: k-tiles go from global memory straight into LDS
-        const int lds_stages = GlobalOptions().igemm_lds;
+        const int lds_stages = p->opt_igemm_lds;
         if (lds_stages != 0 && bk128 && (g.Ci % 128) == 0)
         {
             // Launches that fill the device with 256-row tiles: one wave per SIMD with a 128 x 128 (or 128 x 64) wave tile.
@@ -833,7 +854,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         if (static_cast<long long>(g.H) * g.W * g.Ci >= (1ll << 30)) return SetError(MI355X_ERR_UNSUPPORTED, "dot4 kernel: image too large for 32-bit offsets");
         a.rq = p->rq;
         a.w_mfma = p->w_stem; a.w_mfma2 = p->w_stem2; a.kp = p->stem_kp;
-        if (p->w_stem && !GlobalOptions().stem_dot4 && (g.Kh == 3 || g.Kh == 7))
+        if (p->w_stem && !p->opt_stem_dot4 && (g.Kh == 3 || g.Kh == 7))
         {
             const long long nbm = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
             if (nbm > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
@@ -884,7 +905,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             a.pad_top = g.pad_top; a.pad_left = g.pad_left;
             const int tw = g.stride_x == 1 ? 16 : 8;
             // two output rows per thread (16-row tiles) unless that would leave much of a tile outside a small feature map
-            const int opt_r = GlobalOptions().dw_rows;
+            const int opt_r = p->opt_dw_rows;
             const int rows_per_thread = opt_r ? opt_r : ((g.Ho + 15) / 16 * 16 - g.Ho) * 4 <= g.Ho ? 2 : 1;
             const int th = 8 * rows_per_thread;
             a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + th - 1) / th; a.cblocks = (g.Co + 31) / 32;
