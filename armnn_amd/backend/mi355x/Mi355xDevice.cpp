@@ -43,6 +43,19 @@ int DeviceCount()
     return n;
 }
 
+namespace
+{
+std::atomic<bool> g_Assume{false};
+}
+
+void AssumeDevice(bool assume) { g_Assume.store(assume); }
+
+bool DeviceUsable()
+{
+    static const bool present = DeviceCount() > 0;
+    return present || g_Assume.load();
+}
+
 void EnsureDevice()
 {
     std::call_once(g_Once, [] {

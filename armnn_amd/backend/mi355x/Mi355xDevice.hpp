@@ -15,6 +15,13 @@ namespace mi355x
 {
 /// number of usable devices; 0 when there is none or the driver cannot be reached
 int DeviceCount();
+/// Whether layer support may answer "yes".  The runtime lists every dynamically loaded backend as usable even when its
+/// backend context could not be created (src/armnn/Runtime.cpp:684-687 against :501), so on a machine without the device
+/// the optimizer would still place layers here and LoadNetwork would fail; layer support therefore answers "no" for
+/// every layer while this is false, and Optimize({"Mi355x", "CpuRef"}) falls back.  True when a device is visible, or
+/// after AssumeDevice(true): for optimizing on a machine that lacks the device (and for host-only tests of the rules).
+bool DeviceUsable();
+void AssumeDevice(bool assume);
 /// selects device 0 on first use; throws BackendUnavailableException when there is no device
 void EnsureDevice();
 /// The stream workloads and tensor-handle copies are ordered on.  If the calling thread has lanes running (see below) they

@@ -1,4 +1,5 @@
 #include "Mi355xLayerSupport.hpp"
+#include "Mi355xDevice.hpp"
 
 #include <armnn/TypesUtils.hpp>
 #include <armnn/utility/PolymorphicDowncast.hpp>
@@ -207,6 +208,7 @@ bool Mi355xLayerSupport::IsLayerSupported(const LayerType& type, const std::vect
                                           const Optional<LstmInputParamsInfo>&, const Optional<QuantizedLstmInputParamsInfo>&,
                                           Optional<std::string&> reason) const
 {
+    if (!mi355x::DeviceUsable()) return No(reason, "no MI355X device is visible to this process");
     auto need = [&](size_t n) {
         if (infos.size() < n) throw InvalidArgumentException("Mi355xLayerSupport: too few TensorInfos for " + std::string(GetLayerTypeAsCString(type)));
     };

@@ -75,6 +75,13 @@ std::vector<uint8_t> RunOnRuntime(IRuntime& rt, const INetwork& net, const std::
 // ---------------------------------------------------------------------------------------------------------------------
 // cpu
 // ---------------------------------------------------------------------------------------------------------------------
+namespace
+{
+// The host-only cases test the rules of layer support and of the optimizer on machines without the device; layer support
+// itself answers "no" there unless told to assume one (Mi355xDevice.hpp).
+const bool g_AssumeDeviceForHostCases = (mi355x::AssumeDevice(true), true);
+} // namespace
+
 TEST_CASE("registry: Mi355x is registered by the static initializer", "cpu")
 {
     CHECK(BackendRegistryInstance().IsBackendRegistered(kMi355x));
@@ -775,6 +782,31 @@ TEST_CASE("runtime: without a device the backend is left out and nothing runs on
     QLayer l = MakeConv(QLayer::Conv, ActInfo({1, 8, 8, 16}, DataType::QAsymmS8, 0.05f, -3), 32, 3, 1, 0.1f, 5, true, true, 31);
     SingleLayerNet n(l);
     CHECK_THROWS_AS(Optimize(*n.net, {kMi355x}, rt->GetDeviceSpec()), InvalidArgumentException);
+    // A runtime that lists the backend all the same (Arm NN's own does so for every dynamically loaded backend) gets "no"
+    // with the reason for every layer, and the next backend of the preference list takes the layers.
+    FixedDeviceSpec both{kMi355x, testhost::Id()};
+    testhost::Register();
+    {
+        struct Restore { ~Restore() { mi355x::AssumeDevice(true); } } restore;
+        mi355x::AssumeDevice(false);
+        std::string why;
+        const TensorInfo info = ActInfo({1, 4, 4, 8}, DataType::QAsymmS8, 0.05f, -3);
+        const ActivationDescriptor relu(ActivationFunction::ReLu, 0.0f, 0.0f);
+        CHECK(!backend.GetLayerSupport()->IsLayerSupported(LayerType::Activation, {info, info}, relu, EmptyOptional(), EmptyOptional(),
+                                                           Optional<std::string&>(why)));
+        CHECK_MSG(why.find("no MI355X device") != std::string::npos, why);
+        INetworkPtr net = INetwork::Create();
+        IConnectableLayer* input = net->AddInputLayer(0, "input");
+        input->GetOutputSlot(0).SetTensorInfo(info);
+        IConnectableLayer* lin = net->AddActivationLayer(ActivationDescriptor(ActivationFunction::Linear, 1.0f, 0.0f), "identity");
+        input->GetOutputSlot(0).Connect(lin->GetInputSlot(0));
+        lin->GetOutputSlot(0).SetTensorInfo(info);
+        IConnectableLayer* out = net->AddOutputLayer(0, "output");
+        lin->GetOutputSlot(0).Connect(out->GetInputSlot(0));
+        IOptimizedNetworkPtr fallen = Optimize(*net, {kMi355x, testhost::Id()}, both);
+        for (const auto& layer : fallen->GetGraph().GetLayers()) CHECK(layer->GetBackendId() == testhost::Id());
+        CHECK_THROWS_AS(Optimize(*n.net, {kMi355x}, both), InvalidArgumentException);
+    }
     // workloads exist without a device, but executing one fails loudly
     FixedDeviceSpec pretend{kMi355x};
     IOptimizedNetworkPtr opt = Optimize(*n.net, {kMi355x}, pretend);

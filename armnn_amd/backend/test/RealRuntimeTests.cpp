@@ -15,7 +15,10 @@
 #include <armnn/backends/IBackendInternal.hpp>
 
 #include <cstdio>
+#include <algorithm>
 #include <cstdlib>
+#include <memory>
+#include <sstream>
 #include <string>
 #include <vector>
 
@@ -30,6 +33,8 @@ int g_failed = 0, g_checked = 0;
 int main(int argc, char** argv)
 {
     if (argc < 2) { std::fprintf(stderr, "usage: %s <dynamic backend directory>\n", argv[0]); return 2; }
+    std::setvbuf(stdout, nullptr, _IOLBF, 0);
+    if (argv[1][0] != '/') { std::fprintf(stderr, "the runtime only searches absolute paths (DynamicBackendUtils.cpp IsPathValid)\n"); return 2; }
     const BackendId mi("Mi355x");
     CHECK(!BackendRegistryInstance().IsBackendRegistered(mi));
     {
@@ -39,6 +44,7 @@ int main(int argc, char** argv)
 
         // ---- found, version accepted, registered under its own id
         CHECK(BackendRegistryInstance().IsBackendRegistered(mi));
+        if (!BackendRegistryInstance().IsBackendRegistered(mi)) { std::printf("the backend was not loaded from %s\n", argv[1]); return 1; }
         std::printf("registered backends: %s\n", BackendRegistryInstance().GetBackendIdsAsString().c_str());
         const BackendIdSet& supported = runtime->GetDeviceSpec().GetSupportedBackends();
         const bool listed = supported.count(mi) != 0;
@@ -93,44 +99,231 @@ int main(int argc, char** argv)
         CHECK(!handle.IsConvolution2dSupported(fin, fout, cd, fw, EmptyOptional(), Optional<std::string&>(reasonF)));
         CHECK(!reasonF.empty());                             // float convolutions are never ours, and we say why
 
-        // ---- Optimize with a fallback, then run: the bytes are CpuRef's either way of placing the layers
-        INetworkPtr net = INetwork::Create();
-        IConnectableLayer* input = net->AddInputLayer(0);
-        std::vector<int8_t> wdata(weights.GetNumElements(), 3);
-        std::vector<int32_t> bdata(32, 100);
-        cd.m_BiasEnabled = true;
-        IConnectableLayer* wl = net->AddConstantLayer(ConstTensor(weights, wdata.data()));
-        IConnectableLayer* bl = net->AddConstantLayer(ConstTensor(bias, bdata.data()));
-        IConnectableLayer* conv = net->AddConvolution2dLayer(cd, "conv");
-        IConnectableLayer* output = net->AddOutputLayer(0);
-        input->GetOutputSlot(0).SetTensorInfo(in);
-        wl->GetOutputSlot(0).SetTensorInfo(weights);
-        bl->GetOutputSlot(0).SetTensorInfo(bias);
-        conv->GetOutputSlot(0).SetTensorInfo(out);
-        input->GetOutputSlot(0).Connect(conv->GetInputSlot(0));
-        wl->GetOutputSlot(0).Connect(conv->GetInputSlot(1));
-        bl->GetOutputSlot(0).Connect(conv->GetInputSlot(2));
-        conv->GetOutputSlot(0).Connect(output->GetInputSlot(0));
-        std::vector<std::string> messages;
-        IOptimizedNetworkPtr opt = Optimize(*net, {mi, BackendId("CpuRef")}, runtime->GetDeviceSpec(), OptimizerOptionsOpaque(),
-                                            Optional<std::vector<std::string>&>(messages));
-        CHECK(opt != nullptr);
-        for (const std::string& m : messages) std::printf("optimizer: %s\n", m.c_str());
-        NetworkId id = 0;
-        std::string err;
-        const Status loaded = runtime->LoadNetwork(id, std::move(opt), err);
-        if (loaded != Status::Success) std::printf("LoadNetwork: %s\n", err.c_str());
-        CHECK(loaded == Status::Success);
-        if (loaded == Status::Success)
-        {
-            std::vector<int8_t> x(in.GetNumElements(), 7), y(out.GetNumElements(), 0);
-            TensorInfo cin = in;
+        // ---- Optimize with a fallback, then run.  Known answer first: constant data, one output checked by hand.
+        auto convNet = [&](const std::vector<int8_t>& wdata, const std::vector<int32_t>& bdata, const TensorInfo& out) {
+            INetworkPtr net = INetwork::Create();
+            IConnectableLayer* input = net->AddInputLayer(0);
+            Convolution2dDescriptor d = cd;
+            d.m_BiasEnabled = true;
+            IConnectableLayer* wl = net->AddConstantLayer(ConstTensor(weights, wdata.data()));
+            IConnectableLayer* bl = net->AddConstantLayer(ConstTensor(bias, bdata.data()));
+            IConnectableLayer* conv = net->AddConvolution2dLayer(d, "conv");
+            IConnectableLayer* output = net->AddOutputLayer(0);
+            input->GetOutputSlot(0).SetTensorInfo(in);
+            wl->GetOutputSlot(0).SetTensorInfo(weights);
+            bl->GetOutputSlot(0).SetTensorInfo(bias);
+            conv->GetOutputSlot(0).SetTensorInfo(out);
+            input->GetOutputSlot(0).Connect(conv->GetInputSlot(0));
+            wl->GetOutputSlot(0).Connect(conv->GetInputSlot(1));
+            bl->GetOutputSlot(0).Connect(conv->GetInputSlot(2));
+            conv->GetOutputSlot(0).Connect(output->GetInputSlot(0));
+            return net;
+        };
+        auto run = [&](INetwork& net, const std::vector<BackendId>& prefs, const TensorInfo& inInfo, const std::vector<int8_t>& x,
+                       const TensorInfo& outInfo, std::string& placement) {
+            std::vector<std::string> messages;
+            std::vector<int8_t> y(outInfo.GetNumElements(), 0);
+            IOptimizedNetworkPtr opt(nullptr, [](IOptimizedNetwork*) {});
+            try
+            {
+                opt = Optimize(net, prefs, runtime->GetDeviceSpec(), OptimizerOptionsOpaque(), Optional<std::vector<std::string>&>(messages));
+            }
+            catch (const Exception& e)
+            {
+                std::printf("Optimize: %s\n", e.what());
+            }
+            for (const std::string& m : messages) std::printf("optimizer: %s\n", m.c_str());
+            CHECK(opt != nullptr);
+            if (!opt) return y;
+            NetworkId id = 0;
+            std::string err;
+            const Status loaded = runtime->LoadNetwork(id, std::move(opt), err);
+            if (loaded != Status::Success) std::printf("LoadNetwork: %s\n", err.c_str());
+            CHECK(loaded == Status::Success);
+            if (loaded != Status::Success) return y;
+            TensorInfo cin = inInfo;
             cin.SetConstant(true);
-            CHECK(runtime->EnqueueWorkload(id, {{0, ConstTensor(cin, x.data())}}, {{0, Tensor(out, y.data())}}) == Status::Success);
+            runtime->GetProfiler(id)->EnableProfiling(true);
+            CHECK(runtime->EnqueueWorkload(id, {{0, ConstTensor(cin, x.data())}}, {{0, Tensor(outInfo, y.data())}}) == Status::Success);
+            std::ostringstream prof;
+            runtime->GetProfiler(id)->Print(prof);
+            placement = prof.str().find("Mi355x") != std::string::npos ? "Mi355x" : "CpuRef";
+            runtime->UnloadNetwork(id);
+            return y;
+        };
+        {
+            std::string where;
+            INetworkPtr net = convNet(std::vector<int8_t>(weights.GetNumElements(), 3), std::vector<int32_t>(32, 100), out);
+            const std::vector<int8_t> y = run(*net, {mi, BackendId("CpuRef")}, in, std::vector<int8_t>(in.GetNumElements(), 7), out, where);
             // centre pixel: 9 taps x 16 channels of (7 - (-3)) * 0.05 * 3 * 0.01 = 2.16, + 100 * 0.0005 = 2.21 -> 22 codes above -128
             CHECK(y[(4 * 8 + 4) * 32] == -128 + 22);
-            std::printf("EnqueueWorkload through the fallback placement: centre output code %d\n", static_cast<int>(y[(4 * 8 + 4) * 32]));
-            runtime->UnloadNetwork(id);
+            std::printf("constant convolution ran on %s: centre output code %d\n", where.c_str(), static_cast<int>(y[(4 * 8 + 4) * 32]));
+            CHECK((where == "Mi355x") == !unavailable);
+        }
+        // ---- random data: {Mi355x, CpuRef} against {CpuRef} alone.  On a machine with the device that is this backend's
+        //      integer-accumulating convolution against the reference implementation's float accumulation: within one
+        //      code everywhere (the tolerance of the reference's own quantized layer tests, TensorHelpers.hpp:24-31),
+        //      equal nearly everywhere.
+        auto compare = [&](const std::vector<int8_t>& got, const std::vector<int8_t>& want, const char* what, const std::string& where) {
+            size_t differing = 0;
+            int worst = 0, lo = 127, hi = -128;
+            for (size_t i = 0; i < got.size(); ++i)
+            {
+                differing += got[i] != want[i];
+                worst = std::max(worst, std::abs(static_cast<int>(got[i]) - static_cast<int>(want[i])));
+                lo = std::min<int>(lo, want[i]);
+                hi = std::max<int>(hi, want[i]);
+            }
+            std::printf("%s on %s against CpuRef: %zu of %zu bytes differ, max |difference| %d, codes span [%d, %d]\n", what, where.c_str(),
+                        differing, got.size(), worst, lo, hi);
+            CHECK(worst <= 1);
+            CHECK(differing * 100 <= got.size());
+            CHECK(hi - lo > 100);
+            if (unavailable) CHECK(differing == 0);
+        };
+        {
+            uint64_t state = 0x9E3779B97F4A7C15ull;
+            auto next = [&]() { state ^= state << 13; state ^= state >> 7; state ^= state << 17; return state; };
+            std::vector<int8_t> w(weights.GetNumElements()), x(in.GetNumElements());
+            std::vector<int32_t> b(32);
+            for (auto& v : w) v = static_cast<int8_t>(static_cast<int>(next() % 81) - 40);
+            for (auto& v : x) v = static_cast<int8_t>(static_cast<int>(next() % 256) - 128);
+            for (auto& v : b) v = static_cast<int32_t>(next() % 4001) - 2000;
+            const TensorInfo spread({1, 8, 8, 32}, DataType::QAsymmS8, 0.25f, 4);
+            std::string where, whereRef;
+            INetworkPtr net = convNet(w, b, spread);
+            const std::vector<int8_t> got = run(*net, {mi, BackendId("CpuRef")}, in, x, spread, where);
+            INetworkPtr net2 = convNet(w, b, spread);
+            const std::vector<int8_t> want = run(*net2, {BackendId("CpuRef")}, in, x, spread, whereRef);
+            compare(got, want, "random convolution", where);
+            CHECK(whereRef == "CpuRef");
+        }
+        // ---- a small MobileNet-shaped network with per-channel weight scales, fused activations to fold, a strided
+        //      depthwise layer, a pointwise layer, global average pooling and a fully connected layer
+        {
+            uint64_t state = 0xD1B54A32D192ED03ull;
+            auto next = [&]() { state ^= state << 13; state ^= state >> 7; state ^= state << 17; return state; };
+            auto scales = [&](unsigned int n, float base) {
+                std::vector<float> v(n);
+                for (auto& f : v) f = base * (0.5f + static_cast<float>(next() % 1000) / 1000.0f);
+                return v;
+            };
+            struct Held { std::vector<int8_t> w; std::vector<int32_t> b; };
+            std::vector<std::unique_ptr<Held>> held;
+            auto build = [&](int depth) {
+                state = 0xD1B54A32D192ED03ull;
+                held.clear();
+                INetworkPtr net = INetwork::Create();
+                const TensorInfo t0({2, 16, 16, 16}, DataType::QAsymmS8, 0.04f, -5);
+                IConnectableLayer* input = net->AddInputLayer(0);
+                input->GetOutputSlot(0).SetTensorInfo(t0);
+                IOutputSlot* cur = &input->GetOutputSlot(0);
+                TensorInfo curInfo = t0;
+                auto constants = [&](IConnectableLayer* layer, const TensorShape& wshape, unsigned int channels, unsigned int qdim, float wbase) {
+                    // CpuRef's FullyConnected wants weights of the input's type (RefLayerSupport.cpp IsFullyConnectedSupported):
+                    // one scale, QAsymmS8, there; per-channel QSymmS8 for the convolutions
+                    const bool perTensor = layer->GetType() == LayerType::FullyConnected;
+                    const std::vector<float> ws = perTensor ? std::vector<float>(channels, wbase) : scales(channels, wbase);
+                    TensorInfo wi = perTensor ? TensorInfo(wshape, DataType::QAsymmS8, wbase, 0) : TensorInfo(wshape, DataType::QSymmS8, ws, qdim);
+                    wi.SetConstant(true);
+                    std::vector<float> bs(channels);
+                    for (unsigned int c = 0; c < channels; ++c) bs[c] = ws[c] * curInfo.GetQuantizationScale();
+                    TensorInfo bi = perTensor ? TensorInfo({channels}, DataType::Signed32, bs[0], 0) : TensorInfo({channels}, DataType::Signed32, bs, 0);
+                    bi.SetConstant(true);
+                    held.emplace_back(new Held);
+                    Held& h = *held.back();
+                    h.w.resize(wi.GetNumElements());
+                    h.b.resize(channels);
+                    for (auto& v : h.w) v = static_cast<int8_t>(static_cast<int>(next() % 255) - 127);
+                    for (auto& v : h.b) v = static_cast<int32_t>(next() % 2001) - 1000;
+                    IConnectableLayer* wl = net->AddConstantLayer(ConstTensor(wi, h.w.data()));
+                    IConnectableLayer* bl = net->AddConstantLayer(ConstTensor(bi, h.b.data()));
+                    wl->GetOutputSlot(0).SetTensorInfo(wi);
+                    bl->GetOutputSlot(0).SetTensorInfo(bi);
+                    cur->Connect(layer->GetInputSlot(0));
+                    wl->GetOutputSlot(0).Connect(layer->GetInputSlot(1));
+                    bl->GetOutputSlot(0).Connect(layer->GetInputSlot(2));
+                };
+                auto finish = [&](IConnectableLayer* layer, const TensorInfo& info, int act) {
+                    layer->GetOutputSlot(0).SetTensorInfo(info);
+                    cur = &layer->GetOutputSlot(0);
+                    curInfo = info;
+                    if (act != 0)
+                    {
+                        const ActivationDescriptor ad(act == 1 ? ActivationFunction::ReLu : ActivationFunction::BoundedReLu, 6.0f, 0.0f);
+                        IConnectableLayer* a = net->AddActivationLayer(ad);
+                        cur->Connect(a->GetInputSlot(0));
+                        a->GetOutputSlot(0).SetTensorInfo(info);
+                        cur = &a->GetOutputSlot(0);
+                    }
+                };
+                Convolution2dDescriptor c1;
+                c1.m_PadLeft = c1.m_PadRight = c1.m_PadTop = c1.m_PadBottom = 1;
+                c1.m_StrideX = c1.m_StrideY = 1;
+                c1.m_BiasEnabled = true;
+                c1.m_DataLayout = DataLayout::NHWC;
+                IConnectableLayer* l1 = net->AddConvolution2dLayer(c1, "conv3x3");
+                constants(l1, {32, 3, 3, 16}, 32, 0, 0.004f);
+                finish(l1, TensorInfo({2, 16, 16, 32}, DataType::QAsymmS8, 6.0f / 255.0f, -128), 2);
+                DepthwiseConvolution2dDescriptor d2;
+                d2.m_PadLeft = d2.m_PadTop = 0;
+                d2.m_PadRight = d2.m_PadBottom = 1;
+                d2.m_StrideX = d2.m_StrideY = 2;
+                d2.m_BiasEnabled = true;
+                d2.m_DataLayout = DataLayout::NHWC;
+                IConnectableLayer* l2 = net->AddDepthwiseConvolution2dLayer(d2, "depthwise3x3s2");
+                constants(l2, {1, 3, 3, 32}, 32, 3, 0.01f);
+                finish(l2, TensorInfo({2, 8, 8, 32}, DataType::QAsymmS8, 0.03f, -128), 1);
+                Convolution2dDescriptor c3;
+                c3.m_StrideX = c3.m_StrideY = 1;
+                c3.m_BiasEnabled = true;
+                c3.m_DataLayout = DataLayout::NHWC;
+                IConnectableLayer* l3 = net->AddConvolution2dLayer(c3, "pointwise");
+                constants(l3, {64, 1, 1, 32}, 64, 0, 0.006f);
+                finish(l3, TensorInfo({2, 8, 8, 64}, DataType::QAsymmS8, 6.0f / 255.0f, -128), 2);
+                if (depth == 3)
+                {
+                    IConnectableLayer* output = net->AddOutputLayer(0);
+                    cur->Connect(output->GetInputSlot(0));
+                    return net;
+                }
+                Pooling2dDescriptor p4;
+                p4.m_PoolType = PoolingAlgorithm::Average;
+                p4.m_PoolWidth = p4.m_PoolHeight = 8;
+                p4.m_StrideX = p4.m_StrideY = 8;
+                p4.m_DataLayout = DataLayout::NHWC;
+                IConnectableLayer* l4 = net->AddPooling2dLayer(p4, "pool");
+                cur->Connect(l4->GetInputSlot(0));
+                finish(l4, TensorInfo({2, 1, 1, 64}, DataType::QAsymmS8, 6.0f / 255.0f, -128), 0);
+                IConnectableLayer* l5 = net->AddReshapeLayer(ReshapeDescriptor(TensorShape({2, 64})), "reshape");
+                cur->Connect(l5->GetInputSlot(0));
+                finish(l5, TensorInfo({2, 64}, DataType::QAsymmS8, 6.0f / 255.0f, -128), 0);
+                FullyConnectedDescriptor f6;
+                f6.m_BiasEnabled = true;
+                f6.m_TransposeWeightMatrix = true;
+                IConnectableLayer* l6 = net->AddFullyConnectedLayer(f6, "fc");
+                constants(l6, {10, 64}, 10, 0, 0.008f);
+                finish(l6, TensorInfo({2, 10}, DataType::QAsymmS8, 0.3f, 3), 0);
+                IConnectableLayer* output = net->AddOutputLayer(0);
+                cur->Connect(output->GetInputSlot(0));
+                return net;
+            };
+            const TensorInfo t0({2, 16, 16, 16}, DataType::QAsymmS8, 0.04f, -5);
+            std::vector<int8_t> x(t0.GetNumElements());
+            uint64_t xs = 88172645463325252ull;
+            for (auto& v : x) { xs ^= xs << 13; xs ^= xs >> 7; xs ^= xs << 17; v = static_cast<int8_t>(static_cast<int>(xs % 256) - 128); }
+            for (int depth : {3, 6})
+            {
+                const TensorInfo tout = depth == 3 ? TensorInfo({2, 8, 8, 64}, DataType::QAsymmS8, 6.0f / 255.0f, -128)
+                                                   : TensorInfo({2, 10}, DataType::QAsymmS8, 0.3f, 3);
+                std::string where, whereRef;
+                INetworkPtr a = build(depth);
+                const std::vector<int8_t> got = run(*a, {mi, BackendId("CpuRef")}, t0, x, tout, where);
+                INetworkPtr b = build(depth);
+                const std::vector<int8_t> want = run(*b, {BackendId("CpuRef")}, t0, x, tout, whereRef);
+                compare(got, want, depth == 3 ? "convolution + ReLU6, strided depthwise + ReLU, pointwise + ReLU6" : "the same, then pooling, reshape, fully connected",
+                        where);
+            }
         }
     }
     // ---- the runtime's destructor takes the dynamic backend out of the registry again

@@ -98,3 +98,49 @@ def test_backend_sources_compile_against_real_armnn_headers():
     """-fsyntax-only against the reference's own headers: the backend uses no name the real API lacks."""
     proc = subprocess.run(["make", "-C", BACKEND, "conformance"], capture_output=True, text=True, timeout=600)
     assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
+
+
+REAL = os.path.join(BIN, "real")
+
+
+def _real_runtime():
+    """Runs test/bin/real/real_runtime_tests: libarmnn.so built from an Arm NN source tree loads the backend, compiled
+    against that tree's headers, from a dynamic backend directory."""
+    exe = os.path.join(REAL, "real_runtime_tests")
+    if not os.path.exists(exe):
+        pytest.skip("the backend has not been built against an Arm NN source tree (make -C armnn_amd/backend real-armnn real-runtime)")
+    proc = subprocess.run([exe, os.path.join(REAL, "backends")], capture_output=True, text=True, timeout=300)
+    out = proc.stdout
+    print("\n".join(l for l in out.splitlines() if not l.startswith("optimizer:")))
+    print(proc.stderr[-2000:])
+    assert proc.returncode == 0, out[-4000:]
+    assert " 0 failed" in out and "registered backends: CpuRef, Mi355x" in out
+    return out
+
+
+def test_backend_in_the_real_runtime_host():
+    """The reference's own runtime finds Amd_Mi355x_backend.so by name, accepts its API version and registers Mi355x; the
+    backend's id, capabilities and layer support answer through the public handles; on a machine without the device
+    the backend context is unavailable, every layer is refused with the reason, Optimize({Mi355x, CpuRef}) places the
+    network on CpuRef and the runtime computes it; the runtime's destructor deregisters the backend."""
+    import shutil
+    if os.path.isdir("/root/reference/include/armnn") and os.path.exists(os.environ.get("ARMNN_BUILD", "/tmp/mi355x_armnn_build") + "/libarmnn.so") \
+            and shutil.which("make"):
+        proc = subprocess.run(["make", "-C", BACKEND, "real-runtime"], capture_output=True, text=True, timeout=900)
+        assert proc.returncode == 0, proc.stdout[-3000:] + proc.stderr[-3000:]
+    out = _real_runtime()
+    from armnn_amd import shim
+    if shim.Device.count() == 0:
+        assert "backend context unavailable" in out and "random convolution on CpuRef" in out
+        assert "IsConvolution2dSupported(QAsymmS8 NHWC 3x3): no" in out
+
+
+@pytest.mark.gpu
+def test_backend_in_the_real_runtime_on_device():
+    """The same executable where there is a device: the reference's runtime creates the backend context, the optimizer
+    places every layer on Mi355x, and the outputs are within one code of what the reference's CpuRef backend computes in
+    the same process (convolution, strided depthwise, pointwise, pooling, reshape, fully connected, folded activations)."""
+    out = _real_runtime()
+    assert "backend context created" in out
+    assert "random convolution on Mi355x against CpuRef" in out
+    assert "fully connected on Mi355x against CpuRef" in out
