@@ -127,6 +127,9 @@ public:
     /// layers with every producer before its consumers; throws GraphValidationException on a cycle or a dangling input
     std::vector<Layer*> TopologicalSort() const;
     const std::vector<std::unique_ptr<Layer>>& GetLayers() const { return m_Layers; }
+    /// `for (auto&& layer : graph)` as with the reference's Graph (src/armnn/Graph.hpp:169-186); elements act as Layer*
+    auto begin() const { return m_Layers.begin(); }
+    auto end() const { return m_Layers.end(); }
     size_t GetNumLayers() const { return m_Layers.size(); }
 private:
     std::vector<std::unique_ptr<Layer>> m_Layers;

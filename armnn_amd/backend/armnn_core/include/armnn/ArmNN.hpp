@@ -9,4 +9,5 @@
 #include "BackendOptions.hpp"
 #include "INetwork.hpp"
 #include "IRuntime.hpp"
+#include "Utils.hpp"
 #include <hostcore/BackendLifecycle.hpp>

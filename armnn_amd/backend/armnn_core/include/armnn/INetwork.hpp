@@ -129,6 +129,10 @@ private:
     ModelOptions m_ModelOptions;
 };
 
+/// The optimized graph, for tests and tools that count or inspect its layers (declared a friend of IOptimizedNetwork in
+/// include/armnn/INetwork.hpp:929 and defined by the test utilities, src/armnnTestUtils/TestUtils.cpp:49-52).
+Graph& GetGraphForTesting(IOptimizedNetwork* optNetPtr);
+
 /// Assign every layer to the first backend of `backendPreferences` that is available and supports it, let each
 /// backend substitute sub-graphs it can fuse, and return the result (src/armnn/Network.cpp:2026-2271).
 /// Throws InvalidArgumentException when a layer is supported by none of the preferred backends.

@@ -230,6 +230,7 @@ IOptimizedNetwork::~IOptimizedNetwork() = default;
 void IOptimizedNetwork::Destroy(IOptimizedNetwork* n) { delete n; }
 Graph& IOptimizedNetwork::GetGraph() { return *m_Graph; }
 const Graph& IOptimizedNetwork::GetGraph() const { return *m_Graph; }
+Graph& GetGraphForTesting(IOptimizedNetwork* optNetPtr) { return optNetPtr->GetGraph(); }
 size_t IOptimizedNetwork::GetNumInputs() const
 {
     size_t n = 0;

@@ -1,10 +1,12 @@
 // Minimal host core: IRuntime -- backend discovery, LoadNetwork (tensor handles, workloads, constants), and
 // EnqueueWorkload (src/armnn/Runtime.cpp:301-574, src/armnn/LoadedNetwork.cpp:82-360 and :845-1100).
 #include <algorithm>
+#include <atomic>
 #include <Layer.hpp>
 #include <Profiling.hpp>
 #include <armnn/BackendRegistry.hpp>
 #include <armnn/IRuntime.hpp>
+#include <armnn/Utils.hpp>
 #include <armnn/backends/DynamicBackend.hpp>
 #include <armnn/backends/IBackendInternal.hpp>
 #include <backendsCommon/TensorHandleFactoryRegistry.hpp>
@@ -19,6 +21,22 @@ namespace armnn
 {
 namespace
 {
+std::atomic<int> g_LogThreshold{static_cast<int>(LogSeverity::Warning)};
+std::atomic<bool> g_LogToStdout{false};
+} // namespace
+
+void ConfigureLogging(bool printToStandardOutput, bool, LogSeverity severity)
+{
+    g_LogToStdout.store(printToStandardOutput);
+    g_LogThreshold.store(static_cast<int>(severity));
+}
+bool LogsAt(LogSeverity severity) { return static_cast<int>(severity) >= g_LogThreshold.load(); }
+bool LogsToStandardOutput() { return g_LogToStdout.load(); }
+
+namespace
+{
+std::ostream& LogStream() { return LogsToStandardOutput() ? std::cout : std::cerr; }
+
 class DeviceSpec final : public IDeviceSpec
 {
 public:
@@ -115,7 +133,8 @@ public:
             slot.backend = BackendRegistryInstance().GetFactory(id)();
             if (slot.backend->SupportsTensorAllocatorAPI())
             {
-                slot.backend->RegisterTensorHandleFactories(m_Registry);
+                // the backend registers its tensor handle factories from CreateWorkloadFactory (LoadedNetwork.cpp:265-272
+                // calls nothing else)
                 slot.factory = slot.backend->CreateWorkloadFactory(m_Registry, m_Net->GetModelOptions());
                 slot.handleFactory = m_Registry.GetFactory(slot.backend->GetHandleFactoryPreferences().front());
             }
@@ -304,6 +323,9 @@ public:
         }
         {
             ARMNN_SCOPED_PROFILING_EVENT(BackendId(), "Execute");
+            // constant workloads are part of the queue that runs for every inference (LoadedNetwork.cpp:366-394): a backend
+            // that wants its constants uploaded once has to see to that itself
+            for (auto& w : m_Constants) w->Execute();
             for (auto& w : m_Workloads) w->Execute();
         }
         for (const auto& out : outputs)
@@ -471,8 +493,11 @@ private:
         {
             const Layer& owner = isOutput ? b.slot->GetOwningLayer() : b.slot->GetConnections().empty() ? *b.layer : b.slot->GetConnections().front()->GetOwningLayer();
             BackendSlot& bs = m_Backends.at(owner.GetBackendId());
-            if (!bs.handleFactory || (bs.handleFactory->GetImportFlags() & static_cast<MemorySourceFlags>(source)) == 0) return false;
-            b.imported = bs.handleFactory->CreateTensorHandle(b.slot->GetTensorInfo(), false);
+            if (!bs.handleFactory) return false;
+            // the factory the backend paired with its copying factory for imports (LoadedNetwork.cpp:433-447)
+            ITensorHandleFactory* importFactory = m_Registry.GetFactory(m_Registry.GetMatchingImportFactoryId(bs.handleFactory->GetId()));
+            if (!importFactory || (importFactory->GetImportFlags() & static_cast<MemorySourceFlags>(source)) == 0) return false;
+            b.imported = importFactory->CreateTensorHandle(b.slot->GetTensorInfo(), false);
             if (!b.imported) return false;
         }
         try
@@ -482,7 +507,7 @@ private:
         }
         catch (const MemoryImportException& e)
         {
-            std::cerr << "armnn: an error occurred attempting to import a tensor: " << e.what() << "\n";
+            if (LogsAt(LogSeverity::Error)) LogStream() << "armnn: an error occurred attempting to import a tensor: " << e.what() << "\n";
         }
         return b.adopted;
     }
@@ -570,7 +595,7 @@ public:
                     std::string err;
                     if (!backend->UseCustomMemoryAllocator(allocator->second, err))
                     {
-                        std::cerr << "armnn: the backend " << id << " reported an error when trying to use the provided custom allocator."
+                        if (LogsAt(LogSeverity::Warning)) LogStream() << "armnn: the backend " << id << " reported an error when trying to use the provided custom allocator."
                                   << " Backend won't be used. ErrorMsg: " << err << "\n";
                         continue;
                     }
@@ -588,7 +613,7 @@ public:
             }
             catch (const BackendUnavailableException& e)
             {
-                std::cerr << "armnn: backend " << id << " is unavailable and ignored: " << e.what() << "\n";
+                if (LogsAt(LogSeverity::Warning)) LogStream() << "armnn: backend " << id << " is unavailable and ignored: " << e.what() << "\n";
             }
         }
     }
@@ -652,7 +677,7 @@ public:
         catch (const RuntimeException& e)
         {
             // a failing workload ends the inference, not the process (LoadedNetwork.cpp:1088-1100)
-            std::cerr << "armnn: an error occurred attempting to execute a workload: " << e.what() << "\n";
+            if (LogsAt(LogSeverity::Error)) LogStream() << "armnn: an error occurred attempting to execute a workload: " << e.what() << "\n";
             return Status::Failure;
         }
         for (auto& c : m_Contexts) c.second->AfterEnqueueWorkload(id);

@@ -125,15 +125,31 @@ IBackendInternal::IWorkloadFactoryPtr Mi355xBackend::CreateWorkloadFactory(const
     return std::make_unique<Mi355xWorkloadFactory>(std::dynamic_pointer_cast<Mi355xMemoryManager>(memoryManager));
 }
 
-IBackendInternal::IWorkloadFactoryPtr Mi355xBackend::CreateWorkloadFactory(TensorHandleFactoryRegistry& registry) const
+namespace
 {
-    // handles made by the registered tensor handle factory and by the workload factory share one arena
-    if (auto* existing = dynamic_cast<Mi355xTensorHandleFactory*>(registry.GetFactory(Mi355xTensorHandleFactory::GetIdStatic())))
-        return std::make_unique<Mi355xWorkloadFactory>(existing->GetMemoryManager());
+// The registry as this backend leaves it: one memory manager, one tensor handle factory, paired with itself for imports --
+// the same factory makes the handles that adopt caller memory (RefBackend.cpp:34-48 and :190-203 pair likewise); without
+// the pairing LoadedNetwork finds no import factory (LoadedNetwork.cpp:433-447) and ImportInputs / ImportOutputs adopt
+// nothing.
+Mi355xTensorHandleFactory& EnsureFactories(TensorHandleFactoryRegistry& registry)
+{
+    if (auto* existing = dynamic_cast<Mi355xTensorHandleFactory*>(registry.GetFactory(Mi355xTensorHandleFactory::GetIdStatic()))) return *existing;
     auto memoryManager = std::make_shared<Mi355xMemoryManager>(mi355x::Lanes() == 1);
     registry.RegisterMemoryManager(memoryManager);
-    registry.RegisterFactory(std::make_unique<Mi355xTensorHandleFactory>(memoryManager));
-    return std::make_unique<Mi355xWorkloadFactory>(memoryManager);
+    auto factory = std::make_unique<Mi355xTensorHandleFactory>(memoryManager);
+    Mi355xTensorHandleFactory& made = *factory;
+    registry.RegisterCopyAndImportFactoryPair(Mi355xTensorHandleFactory::GetIdStatic(), Mi355xTensorHandleFactory::GetIdStatic());
+    registry.RegisterFactory(std::move(factory));
+    return made;
+}
+} // namespace
+
+// LoadedNetwork calls this without RegisterTensorHandleFactories (LoadedNetwork.cpp:265-272), the optimizer calls that
+// without this (Network.cpp CreateSupportedBackends): either leaves the registry complete.  Handles made by the registered
+// tensor handle factory and by the workload factory share one arena.
+IBackendInternal::IWorkloadFactoryPtr Mi355xBackend::CreateWorkloadFactory(TensorHandleFactoryRegistry& registry) const
+{
+    return std::make_unique<Mi355xWorkloadFactory>(EnsureFactories(registry).GetMemoryManager());
 }
 
 IBackendInternal::IBackendContextPtr Mi355xBackend::CreateBackendContext(const IRuntime::CreationOptions& options) const
@@ -154,10 +170,7 @@ std::vector<ITensorHandleFactory::FactoryId> Mi355xBackend::GetHandleFactoryPref
 
 void Mi355xBackend::RegisterTensorHandleFactories(TensorHandleFactoryRegistry& registry)
 {
-    if (registry.GetFactory(Mi355xTensorHandleFactory::GetIdStatic()) != nullptr) return;
-    auto memoryManager = std::make_shared<Mi355xMemoryManager>(mi355x::Lanes() == 1);
-    registry.RegisterMemoryManager(memoryManager);
-    registry.RegisterFactory(std::make_unique<Mi355xTensorHandleFactory>(memoryManager));
+    EnsureFactories(registry);
 }
 
 std::unique_ptr<ICustomAllocator> Mi355xBackend::GetDefaultAllocator() const

@@ -510,10 +510,15 @@ Mi355xConstantWorkload::Mi355xConstantWorkload(const ConstantQueueDescriptor& de
 
 void Mi355xConstantWorkload::Execute() const
 {
+    // The runtime keeps constant workloads in the queue it runs for every inference (LoadedNetwork.cpp:366-394 and the
+    // loop of LoadedNetwork::Execute); the data goes to the device the first time only, as with
+    // ClConstantWorkload (src/backends/cl/workloads/ClConstantWorkload.cpp:53-120).
+    if (m_RanOnce) return;
     ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xConstantWorkload_Execute");
     const void* src = m_Data.m_LayerOutput->Map(true);
     if (!src) throw NullPointerException("Mi355xConstantWorkload: layer has no data");
     m_Data.m_Outputs[0]->CopyInFrom(src);
     m_Data.m_LayerOutput->Unmap();
+    m_RanOnce = true;
 }
 } // namespace armnn

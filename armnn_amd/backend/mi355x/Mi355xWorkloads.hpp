@@ -156,5 +156,7 @@ class Mi355xConstantWorkload : public Mi355xBaseWorkload<ConstantQueueDescriptor
 public:
     Mi355xConstantWorkload(const ConstantQueueDescriptor& descriptor, const WorkloadInfo& info);
     void Execute() const override;
+private:
+    mutable bool m_RanOnce = false;
 };
 } // namespace armnn

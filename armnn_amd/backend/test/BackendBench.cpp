@@ -6,7 +6,10 @@
 // pageable host buffers (two host copies and the staging transfers) and with adopted pinned buffers (ImportInputs /
 // ImportOutputs, one transfer each way), the layer counts of the optimized graph, and whether both runs gave the same
 // bytes.  The output of the last run is written to the output file for the caller to compare.
+// Builds against this repository's host core and, unchanged, against an Arm NN source tree and its libarmnn.so (then
+// together with RealGraphAccess.cpp, which supplies the test utilities' GetGraphForTesting).
 #include <armnn/ArmNN.hpp>
+#include <Graph.hpp>
 #include <Layer.hpp>
 
 #include <armnn_mi355x.h>
@@ -26,7 +29,7 @@ namespace
 size_t Count(const Graph& g, LayerType t)
 {
     size_t n = 0;
-    for (const auto& l : g.GetLayers()) n += l->GetType() == t;
+    for (auto&& l : g) n += l->GetType() == t;
     return n;
 }
 } // namespace
@@ -49,10 +52,11 @@ int main(int argc, char** argv)
         const TensorInfo outInfo = nf.tensors.at(nf.output);
         if (input.size() != inInfo.GetNumBytes()) throw std::runtime_error("input file size does not match the network's input");
 
+        ConfigureLogging(true, false, LogSeverity::Error);
         IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
         INetworkPtr net = netfile::Build(nf);
         IOptimizedNetworkPtr opt = Optimize(*net, {BackendId("Mi355x")}, rt->GetDeviceSpec());
-        const Graph& og = opt->GetGraph();
+        const Graph& og = GetGraphForTesting(opt.get());
         const size_t nLayers = og.GetNumLayers(), nAct = Count(og, LayerType::Activation), nCopy = Count(og, LayerType::MemCopy),
                      nConv = Count(og, LayerType::Convolution2d), nDw = Count(og, LayerType::DepthwiseConvolution2d),
                      nAdd = Count(og, LayerType::ElementwiseBinary);
@@ -77,7 +81,8 @@ int main(int argc, char** argv)
         std::memcpy(pin, input.data(), input.size());
         const auto inIds = rt->ImportInputs(id, {{0, ConstTensor(constIn, pin)}}, MemorySource::Malloc);
         const auto outIds = rt->ImportOutputs(id, {{0, Tensor(outInfo, pout)}}, MemorySource::Malloc);
-        if (inIds.size() != 1 || outIds.size() != 1) throw std::runtime_error("pinned buffers were not adopted");
+        if (inIds.size() != 1 || outIds.size() != 1)
+            throw std::runtime_error("pinned buffers were not adopted: " + std::to_string(inIds.size()) + " of 1 inputs, " + std::to_string(outIds.size()) + " of 1 outputs");
         for (int i = 0; i < warmup; ++i)
             if (rt->EnqueueWorkload(id, {}, {}, inIds, outIds) != Status::Success) throw std::runtime_error("EnqueueWorkload failed");
         t0 = std::chrono::steady_clock::now();

@@ -110,16 +110,18 @@ def cpu_baseline(net, seconds_budget=25.0):
             "sample": f"{images} image(s) of the same network at batch 1, {elapsed:.1f} s, 1 thread of {os.cpu_count()}"}
 
 
-def run_backend_child(net, batch, steps, warmup):
+def run_backend_child(net, batch, steps, warmup, real=False):
     """The same network through the C++ backend (INetwork -> Optimize -> LoadNetwork -> IRuntime::EnqueueWorkload) in a
-    child process, started before this process has touched the GPU.  Returns (figures, output bytes) or (error, None)."""
+    child process, started before this process has touched the GPU.  Returns (figures, output bytes) or (error, None).
+    real=True runs the build of the same program against an Arm NN source tree and its own libarmnn.so
+    (armnn_amd/backend/test/bin/real/, made by `make -C armnn_amd/backend real-runtime`), if it is there."""
     import subprocess
     import tempfile
     import numpy as np
     from armnn_amd import netfile, nets
-    exe = os.path.join(ROOT, "armnn_amd", "backend", "test", "bin", "backend_bench")
+    exe = os.path.join(ROOT, "armnn_amd", "backend", "test", "bin", *(["real"] if real else []), "backend_bench")
     if not os.path.exists(exe):
-        return {"error": "armnn_amd/backend/test/bin/backend_bench is not built"}, None
+        return {"error": os.path.relpath(exe, ROOT) + " is not built"}, None
     with tempfile.TemporaryDirectory(prefix="mi355x_bench_") as tmp:
         nf, fin, fout = (os.path.join(tmp, n) for n in ("net.bin", "input.bin", "output.bin"))
         netfile.write_net(net, batch, nf)
@@ -169,8 +171,10 @@ def main():
     # ---- the product path north_star names: the backend behind IRuntime::EnqueueWorkload, in a child process that is
     # started (and has ended) before anything here touches the GPU
     backend, backend_out = (None, None)
+    real, real_out = (None, None)
     if not args.no_backend and not args.profile_pass:
         backend, backend_out = run_backend_child(net, batch, max(50, args.steps // 4), 20)
+        real, real_out = run_backend_child(net, batch, max(50, args.steps // 4), 20, real=True)
 
     from armnn_amd import shim
     from armnn_amd.executor import DeviceNetwork
@@ -305,6 +309,18 @@ def main():
             bp["images_per_sec_pageable_io"] = batch / (backend["ms_pageable"] * 1e-3)
             bp["images_per_sec_adopted_pinned_io"] = batch / (backend["ms_pinned"] * 1e-3)
             bp["path"] = "INetwork -> Optimize({Mi355x}) -> IRuntime::LoadNetwork -> IRuntime::EnqueueWorkload (armnn_amd/backend/test/BackendBench.cpp)"
+        if real is not None and real_out is not None:
+            # the same program built against the reference's source tree: the reference's own optimizer, loaded network and
+            # runtime drive the backend
+            bp["reference_runtime"] = {"ms_pageable": real["ms_pageable"], "ms_pinned": real["ms_pinned"],
+                                       "output_equals_executor": real_out == executor_out,
+                                       "images_per_sec_pageable_io": batch / (real["ms_pageable"] * 1e-3),
+                                       "images_per_sec_adopted_pinned_io": batch / (real["ms_pinned"] * 1e-3),
+                                       "optimized_layers": real["optimized_layers"], "activation_layers_left": real["activation_layers_left"],
+                                       "memcopy_layers": real["memcopy_layers"],
+                                       "path": "the same calls on libarmnn.so built from the reference's sources (armnn_amd/backend/test/bin/real/backend_bench)"}
+        elif real is not None:
+            bp["reference_runtime"] = real
         config["backend_path"] = bp
 
     line = {

@@ -57,12 +57,15 @@ def test_backend_dynamic_on_device():
 
 
 @pytest.mark.gpu
+@pytest.mark.parametrize("runtime", ["host_core", "reference_runtime"])
 @pytest.mark.parametrize("name,batch", [("resnet50", 32), ("mobilenet_v1", 64)])
-def test_benchmark_network_through_the_backend_equals_the_executor(tmp_path, name, batch):
+def test_benchmark_network_through_the_backend_equals_the_executor(tmp_path, name, batch, runtime):
     """ResNet-50 at batch 32 (7x7 stem, max pooling, 16 residual adds with their ReLU folded in, 53 convolutions) and
     MobileNetV1 at batch 64, from one network file: INetwork -> Optimize({Mi355x}) -> LoadNetwork -> EnqueueWorkload in
     backend_bench gives the bytes the C-ABI executor gives (which the network tests tie to the CPU checker), with pageable
-    and with adopted pinned host buffers; no Activation layer survives optimization and no copy layer is inserted."""
+    and with adopted pinned host buffers; no Activation layer survives optimization and no copy layer is inserted.
+    "reference_runtime" is the same program built against an Arm NN source tree and run on the libarmnn.so made from it:
+    the reference's optimizer, LoadedNetwork and Runtime around this backend."""
     import json
 
     import numpy as np
@@ -71,7 +74,9 @@ def test_benchmark_network_through_the_backend_equals_the_executor(tmp_path, nam
     from armnn_amd.executor import DeviceNetwork
 
     _ensure_built()
-    exe = os.path.join(BIN, "backend_bench")
+    exe = os.path.join(BIN, "backend_bench") if runtime == "host_core" else os.path.join(BIN, "real", "backend_bench")
+    if runtime == "reference_runtime" and not os.path.exists(exe):
+        pytest.skip("the backend has not been built against an Arm NN source tree (make -C armnn_amd/backend real-armnn real-runtime)")
     assert os.path.exists(exe), "backend_bench is not built"
     net = nets.resnet50() if name == "resnet50" else nets.mobilenet_v1()
     x = nets.synthetic_input(net, batch, seed=11)
@@ -81,7 +86,7 @@ def test_benchmark_network_through_the_backend_equals_the_executor(tmp_path, nam
     proc = subprocess.run([exe, nf, fin, fout, "20", "3"], capture_output=True, text=True, timeout=300)
     assert proc.returncode == 0, proc.stdout[-2000:] + proc.stderr[-2000:]
     fig = json.loads(proc.stdout.strip().splitlines()[-1])
-    print(f"{name} b{batch} through EnqueueWorkload: {fig['ms_pageable']:.3f} ms pageable I/O = {batch / fig['ms_pageable'] * 1e3:.0f} images/s, "
+    print(f"{name} b{batch} through EnqueueWorkload ({runtime}): {fig['ms_pageable']:.3f} ms pageable I/O = {batch / fig['ms_pageable'] * 1e3:.0f} images/s, "
           f"{fig['ms_pinned']:.3f} ms adopted pinned I/O = {batch / fig['ms_pinned'] * 1e3:.0f} images/s; {fig}", flush=True)
     assert fig["pinned_equals_pageable"] and fig["activation_layers_left"] == 0 and fig["memcopy_layers"] == 0
     assert fig["add_layers"] == (16 if name == "resnet50" else 0)
