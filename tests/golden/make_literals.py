@@ -103,6 +103,140 @@ for bias_enabled in (False, True):
     })
 
 # ---------------------------------------------------------------------------------------------------
+# The reference registers most layer tests once per data layout and permutes the NCHW-described data itself for the NHWC
+# variant (armnnUtils::Permute in the test implementations); both variants are written here the same way.
+def nhwc(a):
+    return np.transpose(np.asarray(a), (0, 2, 3, 1))
+
+
+def conv_pair(name, source, x, w, bias, e, q, params, b_scale, lo=0, hi=255, dtype=U8, exact=True):
+    """x (N,C,H,W), w (O,I,H,W), e (N,O,H,W) as real numbers; q = (scale, offset) shared by all three tensors.  `params`
+    names the padding before the first row and column; the padding after the last ones follows from the output's shape."""
+    scale, offset = q
+    qx, qw, qe = (quantize(v, scale, offset, lo, hi) for v in (x, w, e))
+    qb = t((len(bias),), S32, quantize(bias, b_scale, 0, -2**31, 2**31 - 1), (b_scale,), 0) if bias is not None else None
+    for layout in ("NCHW", "NHWC"):
+        f = (lambda a: a) if layout == "NCHW" else nhwc
+        cases.append({
+            "name": name + ("" if layout == "NCHW" else "Nhwc"), "source": source,
+            "op": "conv2d", "tolerance": 1, "exact_on_cpuref": exact,
+            "params": dict(params, depthwise=False, layout=layout),
+            "input": t(f(qx).shape, dtype, f(qx), (scale,), offset),
+            "weights": t(f(qw).shape, dtype, f(qw), (scale,), offset),
+            "bias": qb,
+            "output": t(f(qe).shape, dtype, f(qe), (scale,), offset),
+        })
+
+
+NO_PAD = {"pad_top": 0, "pad_left": 0, "stride_x": 1, "stride_y": 1, "dilation_x": 1, "dilation_y": 1}
+
+# SimpleConvolution2d3x3Uint8Test (registered with bias, both layouts): the 3x8x16 image of the 3x5 test, two 3x3 filters.
+ker33 = np.zeros((2, 3, 3, 3), dtype=np.float32)
+ker33[0, 0] = 1.0
+ker33[0, 0, 1, 1] = -1.0
+ker33[0, 2] = 2.0
+ker33[1, 1] = 1.0
+exp33 = np.zeros((1, 2, 6, 14), dtype=np.float32)
+exp33[0, 0, 0], exp33[0, 0, 1], exp33[0, 0, 2:] = -15.0, -16.0, -14.5
+exp33[0, 1, :, :3] = 3.0
+exp33[0, 1] += 2.0                      # Bias2 = {0, 2} through ApplyBias
+conv_pair("SimpleConvolution2d3x3Uint8Test", "src/backends/backendsCommon/test/layerTests/Conv2dTestImpl.cpp:38-63,842-918,3488-3497; "
+          "src/backends/reference/test/RefLayerTests.cpp:44,48",
+          img[None], ker33, [0.0, 2.0], exp33, (0.5, 50), NO_PAD, 0.25)
+
+# Dilation tests (Convolution2d3x3DilationTestCommon: every tensor scale 0.1 / offset 128, registered without bias).
+blob = np.zeros((1, 1, 10, 10), dtype=np.float32)
+blob[0, 0, 3:6, 4:7] = 1.0
+k19 = np.arange(1, 10, dtype=np.float32).reshape(1, 1, 3, 3)
+DIL3 = dict(NO_PAD, dilation_x=3, dilation_y=3)
+DIL_SRC = "src/backends/backendsCommon/test/layerTests/Conv2dTestImpl.cpp:1060-1142,%s; src/backends/reference/test/RefLayerTests.cpp:%s"
+conv_pair("Convolution2d3x3Dilation3x3Uint8Test", DIL_SRC % ("1150-1205", "91-98"), blob, k19, None,
+          np.array([[6, 5, 5, 5]] * 3 + [[3, 2, 2, 2]], dtype=np.float32).reshape(1, 1, 4, 4), (0.1, 128), DIL3, 0.01)
+conv_pair("Convolution2d2x3x3Dilation3x3Uint8Test", DIL_SRC % ("1208-1278", "124-131"), np.concatenate([blob, blob], axis=1),
+          np.concatenate([k19, k19], axis=1), None,
+          np.array([[12, 10, 10, 10]] * 3 + [[6, 4, 4, 4]], dtype=np.float32).reshape(1, 1, 4, 4), (0.1, 128), DIL3, 0.01)
+conv_pair("Convolution2d2x2Dilation2x2Padding2x2Stride3x3Uint8Test", DIL_SRC % ("1281-1347", "157-164"),
+          np.ones((1, 1, 10, 10), dtype=np.float32), np.array([1, 2, 3, 4], dtype=np.float32).reshape(1, 1, 2, 2), None,
+          np.array([[4, 7, 7, 3], [6, 10, 10, 4], [6, 10, 10, 4], [2, 3, 3, 1]], dtype=np.float32).reshape(1, 1, 4, 4), (0.1, 128),
+          {"pad_top": 1, "pad_left": 1, "stride_x": 3, "stride_y": 3, "dilation_x": 2, "dilation_y": 2}, 0.01)
+# The QAsymmS8 instances use the same scale 0.1 / offset 128: every value saturates at code 127 on the way in, and the
+# expected output saturates likewise.  Transcribed as the reference holds them.
+conv_pair("Convolution2d3x3Dilation3x3Int8Test", DIL_SRC % ("1150-1205", "83-90"), blob, k19, None,
+          np.array([[6, 5, 5, 5]] * 3 + [[3, 2, 2, 2]], dtype=np.float32).reshape(1, 1, 4, 4), (0.1, 128), DIL3, 0.01, -128, 127, S8)
+conv_pair("Convolution2d2x2Dilation2x2Padding2x2Stride3x3Int8Test", DIL_SRC % ("1281-1347", "149-156"),
+          np.ones((1, 1, 10, 10), dtype=np.float32), np.array([1, 2, 3, 4], dtype=np.float32).reshape(1, 1, 2, 2), None,
+          np.array([[4, 7, 7, 3], [6, 10, 10, 4], [6, 10, 10, 4], [2, 3, 3, 1]], dtype=np.float32).reshape(1, 1, 4, 4), (0.1, 128),
+          {"pad_top": 1, "pad_left": 1, "stride_x": 3, "stride_y": 3, "dilation_x": 2, "dilation_y": 2}, 0.01,
+          -128, 127, S8)
+
+# RefConvolution2dInt8Test (Convolution2dEndToEnd through INetwork/Optimize/IRuntime): registered with QSymmS8 tensors that
+# carry offset 10; the QSymmS8 decoder and encoder apply scale and offset exactly as the QAsymmS8 ones do
+# (src/backends/reference/workloads/Decoders.hpp, Encoders.hpp), so the case is held as QAsymmS8, the type this path takes.
+e2e_in = [1, 5, 2, 3, 5, 8, 7, 3, 6, 3, 3, 3, 9, 1, 9, 4, 1, 8, 1, 3, 6, 8, 1, 9, 2]
+e2e_out = [v + 1 for v in (65, 76, 91, 107, 99, 89, 116, 98, 118)]
+cases.append({
+    "name": "RefConvolution2dInt8Test",
+    "source": "src/backends/backendsCommon/test/Convolution2dEndToEndTestImpl.hpp:50-118; src/backends/reference/test/RefEndToEndTests.cpp:722-727",
+    "op": "conv2d", "tolerance": 1, "exact_on_cpuref": True,
+    "params": dict(NO_PAD, depthwise=False, layout="NHWC"),
+    "input": t((1, 5, 5, 1), S8, quantize(e2e_in, 1.0, 10, -128, 127), (1.0,), 10),
+    "weights": t((1, 3, 3, 1), S8, quantize([4, 5, 6, 0, 0, 0, 3, 2, 1], 1.0, 10, -128, 127), (1.0,), 10),
+    "bias": t((1,), S32, [1], (1.0,), 0),
+    "output": t((1, 3, 3, 1), S8, quantize(e2e_out, 1.0, 10, -128, 127), (1.0,), 10),
+})
+
+# DepthwiseConvolution2dUint8Test: 2 channels, depth multiplier 2, 5x3 kernel, stride (2, 1), padding top/bottom 1; all
+# tensors scale 0.5 / offset 50.  The kernel values are written filter by filter in the test but bound to a [1, 5, 3, 4]
+# TensorInfo unpermuted for CpuRef, and are transcribed in that flat order.
+dw_in = np.empty((1, 2, 8, 16), dtype=np.float32)
+dw_in[0, 0] = 0.5
+dw_in[0, 0, 1] = 0.0
+dw_in[0, 1] = 0.0
+dw_in[0, 1, :, 2] = 1.0
+dw_k_flat = [1, 1, 1, 1, -1, 1, 1, 1, 1, 1, 1, 1, 1, 1, 1] + [2] * 15 + [0, 0, 0, 0, -1, 0] + [0] * 9 + [0] * 7 + [1] + [0] * 7
+dw_exp = np.array(
+    [3] * 14 + [5] * 7 + [5.5] * 7 + [5.5] * 7 + [5] * 7 +
+    [2.5] * 7 + [3.5] * 7 + [4.5] * 7 + [6] * 7 + [6] * 14 +
+    [1, 3, 0, 0, 0, 0, 0] + [2, 4, 0, 0, 0, 0, 0] * 6 + [3, 5, 0, 0, 0, 0, 0] * 5, dtype=np.float32).reshape(1, 4, 6, 7)
+for bias_enabled in (True, False):
+    e = dw_exp.copy()
+    if bias_enabled:
+        e += np.array([0, 2, 1, -1], dtype=np.float32).reshape(1, 4, 1, 1)
+    for layout in ("NCHW", "NHWC"):
+        f = (lambda a: a) if layout == "NCHW" else nhwc
+        cases.append({
+            "name": ("" if bias_enabled else "Unbiased") + "DepthwiseConvolution2dUint8Test" + ("" if layout == "NCHW" else "Nhwc"),
+            "source": "src/backends/backendsCommon/test/layerTests/Conv2dTestImpl.cpp:2020-2237,3768-3777; "
+                      "src/backends/reference/test/RefLayerTests.cpp:294-310",
+            "op": "conv2d", "tolerance": 1, "exact_on_cpuref": True,
+            "params": {"pad_top": 1, "pad_left": 0, "stride_x": 2, "stride_y": 1,
+                       "dilation_x": 1, "dilation_y": 1, "depthwise": True, "layout": layout},
+            "input": t(f(dw_in).shape, U8, f(quantize(dw_in, 0.5, 50, 0, 255)), (0.5,), 50),
+            "weights": t((1, 5, 3, 4), U8, quantize(dw_k_flat, 0.5, 50, 0, 255), (0.5,), 50),
+            "bias": t((4,), S32, quantize([0, 2, 1, -1], 0.25, 0, -2**31, 2**31 - 1), (0.25,), 0) if bias_enabled else None,
+            "output": t(f(e).shape, U8, f(quantize(e, 0.5, 50, 0, 255)), (0.5,), 50),
+        })
+
+# DepthwiseConvolution2dDepthMul1Uint8Test: 2 channels of a 3x3 image under a 3x3 kernel, expected 0 (+ bias {0, 2}).
+dm1_in = np.array([1, 2, 1, 2, 1, 2, 1, 2, 1] * 2, dtype=np.float32).reshape(1, 2, 3, 3)
+dm1_k_flat = [1, 0, 1, 0, 0, 0, -1, 0, -1] * 2
+for bias_enabled in (True, False):
+    e = np.zeros((1, 2, 1, 1), dtype=np.float32) + (np.array([0, 2], dtype=np.float32).reshape(1, 2, 1, 1) if bias_enabled else 0)
+    for layout in ("NCHW", "NHWC"):
+        f = (lambda a: a) if layout == "NCHW" else nhwc
+        cases.append({
+            "name": ("" if bias_enabled else "Unbiased") + "DepthwiseConvolution2dDepthMul1Uint8Test" + ("" if layout == "NCHW" else "Nhwc"),
+            "source": "src/backends/backendsCommon/test/layerTests/Conv2dTestImpl.cpp:1848-2017,3779-3788; "
+                      "src/backends/reference/test/RefLayerTests.cpp:393-428",
+            "op": "conv2d", "tolerance": 1, "exact_on_cpuref": True,
+            "params": dict(NO_PAD, depthwise=True, layout=layout),
+            "input": t(f(dm1_in).shape, U8, f(quantize(dm1_in, 0.5, 50, 0, 255)), (0.5,), 50),
+            "weights": t((1, 3, 3, 2), U8, quantize(dm1_k_flat, 0.5, 50, 0, 255), (0.5,), 50),
+            "bias": t((2,), S32, quantize([0, 2], 0.25, 0, -2**31, 2**31 - 1), (0.25,), 0) if bias_enabled else None,
+            "output": t(f(e).shape, U8, f(quantize(e, 0.5, 50, 0, 255)), (0.5,), 50),
+        })
+
+# ---------------------------------------------------------------------------------------------------
 # TfLite-delegate vectors (expected values come from the TfLite integer kernels; tolerance 1 in the reference).
 cases.append({
     "name": "Conv2DPerChannelInt8Test",
