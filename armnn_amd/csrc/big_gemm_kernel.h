@@ -32,7 +32,7 @@ constexpr int BigGemmSmemBytes()
 {
     constexpr int stages = ST * (BM + BN) * 128;
     constexpr int out = BM * (BN + 16);
-    return (stages > out ? stages : out) + 5 * BN * 4;       // + the block's slice of the per-channel table
+    return (stages > out ? stages : out) + 4 * BN * 4;       // + the block's slice of the per-channel table
 }
 
 // 2 x 2 waves, wave tile (BM / 2) x (BN / 2).  Needs Ci % 128 == 0 (a k-tile is 128 bytes of one filter tap) and
@@ -247,19 +247,20 @@ __global__ __launch_bounds__(256) void BigGemmKernel(IgemmArgs a, int xcd_rows)
     constexpr int LAST = (KS - 1) & 1;           // fragment buffer of a tile's last k-step
     constexpr int PRE = NM / 4;                  // MFMAs of the last k-step issued ahead of the barrier
 
-    // ---- the block's slice of the per-channel table (rows 0 .. 4, BN channels) goes to LDS behind the stages: with one
-    // wave per SIMD nothing would hide the epilogue's table reads from global memory, one round trip per channel quad
+    // ---- the block's slice of the per-channel table (rows 2 .. 5: the fast path's bracket, BN channels) goes to LDS behind
+    // the stages: with one wave per SIMD nothing would hide the epilogue's table reads from global memory, one round trip
+    // per channel quad.  The rare exact path reads its two rows from global memory.
     constexpr int TAB = (ST * STAGE > BM * LDO ? ST * STAGE : BM * LDO);
     float* tab_lds = reinterpret_cast<float*>(smem + TAB);
     {
-        constexpr int N4 = 5 * BN / 4;                     // float4 pieces
+        constexpr int N4 = 4 * BN / 4;                     // float4 pieces
         v4i piece[(N4 + 255) / 256];
 #pragma unroll
         for (int i = 0; i < (N4 + 255) / 256; ++i)
         {
             const int e = i * 256 + tid;
             const int row = e / (BN / 4), col = e - row * (BN / 4);
-            if (e < N4) piece[i] = *reinterpret_cast<const v4i*>(a.ct.p + static_cast<long long>(row) * a.ct.stride + tn * BN + col * 4);
+            if (e < N4) piece[i] = *reinterpret_cast<const v4i*>(a.ct.p + static_cast<long long>(row + 2) * a.ct.stride + tn * BN + col * 4);
         }
         // ---- prologue: ST tiles requested behind the table reads (older requests complete first) ...
 #pragma unroll
@@ -356,18 +357,16 @@ __global__ __launch_bounds__(256) void BigGemmKernel(IgemmArgs a, int xcd_rows)
         for (int q = 0; q < 4; ++q)
         {
             const int cl = wn * WTN + tc * 32 + 8 * q + lane_c;
-            Fast4 f4;
-            f4.m0 = *reinterpret_cast<const float4*>(tab_lds + 0 * BN + cl);
-            f4.b0 = *reinterpret_cast<const float4*>(tab_lds + 1 * BN + cl);
-            f4.m = *reinterpret_cast<const float4*>(tab_lds + 2 * BN + cl);
-            f4.b = *reinterpret_cast<const float4*>(tab_lds + 3 * BN + cl);
-            f4.t = *reinterpret_cast<const float4*>(tab_lds + 4 * BN + cl);
+            const float4 mp = *reinterpret_cast<const float4*>(tab_lds + 0 * BN + cl);
+            const float4 bp = *reinterpret_cast<const float4*>(tab_lds + 1 * BN + cl);
+            const float4 mm = *reinterpret_cast<const float4*>(tab_lds + 2 * BN + cl);
+            const float4 bm = *reinterpret_cast<const float4*>(tab_lds + 3 * BN + cl);
 #pragma unroll
             for (int tp = 0; tp < TP; ++tp)
             {
                 const v16i& c = acc[tc][tp];
                 const int rt = AW ? rowsum[tp] : 0;
-                const uint32_t out = Requant4Dev(c[4 * q + 0] + rt, c[4 * q + 1] + rt, c[4 * q + 2] + rt, c[4 * q + 3] + rt, f4, a.ct, tn * BN + cl, a.rq);
+                const uint32_t out = Requant4Dev(c[4 * q + 0] + rt, c[4 * q + 1] + rt, c[4 * q + 2] + rt, c[4 * q + 3] + rt, mp, bp, mm, bm, a.ct, nullptr, tn * BN + cl, a.rq);
                 const int pl = wm * WTM + tp * 32 + (lane & 31);
                 *reinterpret_cast<uint32_t*>(Os + pl * LDO + cl) = out;
             }

@@ -66,7 +66,6 @@ struct Requant
     int32_t  pk_bias;       // 128 for QAsymmS8 outputs, 0 for QAsymmU8
     uint32_t pk_xor;        // 0x80808080 or 0
     float    pk_lo_f, pk_hi_f;   // activation clamp in the biased domain
-    float    pk_lo_q, pk_hi_q;   // ... widened by a quarter code: the clamp the fast path applies before rounding
     int32_t  pk_full;       // the clamp is 0..255: the instruction's own saturation does it
 };
 

@@ -34,11 +34,13 @@ struct mi355x_conv2d_s
     uint32_t* w_dot4b = nullptr;   // depthwise 3x3 / small-Ci conv whose weight differences need two int8 halves: the second halves
     int variant = 0;               // kernel variant within an algo (see RunPlan)
     int row_dwords = 0;            // small-Ci conv: dwords per filter row
-    float*   chan     = nullptr;   // [5][Co_pad] per-channel requantization constants (rows: see ChanTab)
+    float*   chan     = nullptr;   // [8][Co_pad] per-channel requantization constants (rows: see ChanTab)
     int32_t* corr     = nullptr;   // [Co_pad]  -zx' * sum_k w[c][k]
     int K = 0, K_pad = 0, Co_pad = 0;
     int pw_blocks_per_cu = 1, pw_n_cu = 256;     // weight-stationary kernel: blocks a CU holds at once, CUs of the device
     std::vector<float> chan_host;  // host copy, completed with the corr-folded rows once corr is known
+    std::vector<float> fast_fm, fast_fb;   // per channel: the unwidened fast-path constants and the constant half-width of the
+    std::vector<double> fast_cw;           // bracket (negative: no fast path), kept until the table is uploaded
     int pw_bn = 0, pw_ks = 0;      // pointwise GEMM kernel configuration (0: not applicable)
     bool bk128 = false;            // implicit GEMM walks K in 128-byte tiles
     int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 96 (= 128x64) / 128: the "igemm_tile" option at plan creation
@@ -72,6 +74,10 @@ struct mi355x_fc_s
 
 namespace
 {
+// unit roundoff of fp32 and the relative half-width of the requantization bracket (device_math.h)
+constexpr double kBracketUnit = 1.0 / 16777216.0;
+constexpr double kBracketRel = 16.0 / 16777216.0;
+
 
 void FoldCorrIntoTable(mi355x_conv2d_s* p, const std::vector<int32_t>& corr, int Co);
 void ChoosePointwiseConfig(mi355x_conv2d_s* p);
@@ -186,36 +192,46 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             }
         }
     }
-    // fast-path coefficients: r' = fma(float(acc), fm, fb) ~ f / s_out + offset, with the per-channel tie window
-    // inside which the value is recomputed exactly (device_math.h).  thr = -1 sends every value to the exact path.
+    // fast-path coefficients: the bracket r- < f / s_out + offset' < r+ of device_math.h, one FMA per side.  A channel
+    // whose constants do not qualify gets a bracket that never closes (bytes 255 and 0), so it always takes the exact path.
     {
         const int CP = p->Co_pad;
-        std::vector<float> tab(static_cast<size_t>(7) * CP, 0.0f);
+        std::vector<float> tab(static_cast<size_t>(8) * CP, 0.0f);
         const float inv = 1.0f / d.output.scale;
         // the fast path works 128 codes higher for signed outputs (Requant::pk_bias), so that is its offset
         const float zp_f = static_cast<float>(d.output.offset + (d.output.dtype == MI355X_QASYMM_U8 ? 0 : 128));
         const double max_acc = static_cast<double>(p->K) * 65025.0;
         const bool base_ok = !GlobalOptions().exact_division_epilogue && std::isnormal(inv) && std::isnormal(d.output.scale) &&
                              d.output.offset >= -255 && d.output.offset <= 255 && p->rq.fast_ok;
+        p->fast_fm.assign(CP, 0.0f);
+        p->fast_fb.assign(CP, 0.0f);
+        p->fast_cw.assign(CP, -1.0);
         for (int c = 0; c < CP; ++c)
         {
             tab[c] = mult[c];
             tab[CP + c] = biasf[c];
-            tab[4 * CP + c] = -1.0f;
-            tab[6 * CP + c] = -1.0f;
-            if (c >= Co || !base_ok) continue;
+            if (c >= Co) continue;                    // padding: both sides give byte 0, nothing is ever redone or stored
+            tab[3 * CP + c] = tab[6 * CP + c] = 255.0f;
+            if (!base_ok) continue;
             const float fm = mult[c] * inv;
             const float fb = biasf[c] * inv + zp_f;
-            const float bq = std::fabs(biasf[c]) * inv;
-            // constant part of the tie window (device_math.h): 1.5 * 2^-24 * (9 |offset| + 9 |biasf/s_out| + 64);
-            // the part proportional to |r'| is applied per value on the device
-            const float win = 1.5f * (9.0f * std::fabs(zp_f) + 9.0f * bq + 64.0f) * (1.0f / 16777216.0f);
-            const bool ok = std::isfinite(fm) && std::isfinite(fb) && std::isfinite(win) && win < 0.25f &&
+            const double bq = std::fabs(static_cast<double>(biasf[c])) * inv;
+            // constant half-width (device_math.h): 1.5 * 2^-24 * (14 |biasf/s_out| + 10 |offset'| + 64) + 2 e; the part
+            // proportional to the value is the factor 1 +- e on both constants
+            const double cw = 1.5 * kBracketUnit * (14.0 * bq + 10.0 * std::fabs(static_cast<double>(zp_f)) + 64.0) + 2.0 * kBracketRel;
+            const bool ok = std::isfinite(fm) && std::isfinite(fb) && std::isfinite(cw) && cw < 0.125 &&
                             max_acc * std::fabs(static_cast<double>(fm)) < 268435456.0;
             if (!ok) continue;
-            tab[2 * CP + c] = fm;
-            tab[3 * CP + c] = fb;
-            tab[4 * CP + c] = 0.5f - win;
+            tab[2 * CP + c] = static_cast<float>(static_cast<double>(fm) * (1.0 + kBracketRel));
+            tab[3 * CP + c] = static_cast<float>(static_cast<double>(fb) * (1.0 + kBracketRel) + cw);
+            tab[4 * CP + c] = static_cast<float>(static_cast<double>(fm) * (1.0 - kBracketRel));
+            tab[5 * CP + c] = static_cast<float>(static_cast<double>(fb) * (1.0 - kBracketRel) - cw);
+            // until a kernel folds its zero-point correction in, rows 6/7 never close either
+            tab[6 * CP + c] = 255.0f;
+            tab[7 * CP + c] = 0.0f;
+            p->fast_fm[c] = fm;
+            p->fast_fb[c] = fb;
+            p->fast_cw[c] = cw;
         }
         p->chan_host = tab;
     }
@@ -358,7 +374,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
         p->pad_word = zb | (zb << 8) | (zb << 16) | (zb << 24);
         p->variant = 1;
         {
-            // [C/4][8][4] dwords: weight rows 0..2, corr, fm, fb, thr (rows 2..4 of the channel table), 0
+            // [C/4][8][4] dwords: weight rows 0..2, corr, m+, b+, m-, b- (rows 2..5 of the channel table)
             const int CP = p->Co_pad;
             std::vector<uint32_t> grp(static_cast<size_t>(Co / 4) * 32, 0u);
             for (int c = 0; c < Co; ++c)
@@ -366,7 +382,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
                 uint32_t* gdst = grp.data() + static_cast<size_t>(c / 4) * 32 + (c % 4);
                 for (int r = 0; r < 3; ++r) gdst[r * 4] = wp[static_cast<size_t>(c) * 4 + r];
                 gdst[3 * 4] = static_cast<uint32_t>(corr[c]);
-                for (int r = 0; r < 3; ++r) std::memcpy(&gdst[(4 + r) * 4], &p->chan_host[static_cast<size_t>(2 + r) * CP + c], 4);
+                for (int r = 0; r < 4; ++r) std::memcpy(&gdst[(4 + r) * 4], &p->chan_host[static_cast<size_t>(2 + r) * CP + c], 4);
             }
             if (int rc = Upload(reinterpret_cast<void**>(&p->dw_grp), grp.data(), grp.size() * sizeof(uint32_t))) return rc;
             const std::vector<uint8_t> padbytes(16, static_cast<uint8_t>((zb ^ (g.in_u8 ? 0x80u : 0u)) & 0xffu));
@@ -455,26 +471,29 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     if (int rc = Upload(reinterpret_cast<void**>(&p->chan), p->chan_host.data(), p->chan_host.size() * sizeof(float))) return rc;
     p->chan_host.clear();
     p->chan_host.shrink_to_fit();
+    p->fast_fm = std::vector<float>();
+    p->fast_fb = std::vector<float>();
+    p->fast_cw = std::vector<double>();
     return 0;
 }
 
-// Rows 5/6 of the channel table: the fast-path constants with the zero-point correction folded in,
-//   fb' = fb + corr * fm,   window' = 2^-24 * (8192 + 11 (|biasf/s_out| + |corr * fm|))
-// (the accumulator then starts at zero and only the rare exact path adds corr as an integer).
+// Rows 6/7 of the channel table: the bracket with the zero-point correction folded in,
+//   bc+- = (fb + corr * fm) (1 +- e) +- (c + 1.5 * 2^-24 * 5 |corr * fm|)
+// (the accumulator then starts at zero and only the rare exact path adds corr as an integer; the wider constant covers
+// the roundings of corr * fm and of the two conversions of an accumulator beyond 2^24).
 void FoldCorrIntoTable(mi355x_conv2d_s* p, const std::vector<int32_t>& corr, int Co)
 {
     const int CP = p->Co_pad;
     std::vector<float>& tab = p->chan_host;
-    for (int c = 0; c < Co; ++c)
+    for (int c = 0; c < Co && c < static_cast<int>(p->fast_cw.size()); ++c)
     {
-        if (tab[4 * CP + c] < 0.0f) continue;         // fast path disabled for this channel
-        const float fm = tab[2 * CP + c];
-        const float cq = static_cast<float>(corr[c]) * fm;
-        const float fbc = tab[3 * CP + c] + cq;
-        const float win = (0.5f - tab[4 * CP + c]) + 1.5f * 7.0f * std::fabs(cq) * (1.0f / 16777216.0f);
-        if (!std::isfinite(fbc) || !(win < 0.25f) || std::fabs(static_cast<double>(corr[c])) >= 16777216.0) continue;
-        tab[5 * CP + c] = fbc;
-        tab[6 * CP + c] = 0.5f - win;
+        if (p->fast_cw[c] < 0.0) continue;            // fast path disabled for this channel
+        const double cq = static_cast<double>(corr[c]) * static_cast<double>(p->fast_fm[c]);
+        const double fbc = static_cast<double>(p->fast_fb[c]) + cq;
+        const double cw = p->fast_cw[c] + 1.5 * kBracketUnit * 5.0 * std::fabs(cq);
+        if (!std::isfinite(fbc) || !(cw < 0.125) || std::fabs(static_cast<double>(corr[c])) >= 16777216.0) continue;
+        tab[6 * CP + c] = static_cast<float>(fbc * (1.0 + kBracketRel) + cw);
+        tab[7 * CP + c] = static_cast<float>(fbc * (1.0 - kBracketRel) - cw);
     }
 }
 

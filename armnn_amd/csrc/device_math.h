@@ -31,14 +31,13 @@ __device__ __forceinline__ int RequantExactDev(int acc, float mult, float biasf,
     return QuantizeDev(__fadd_rn(__fmul_rn(static_cast<float>(acc), mult), biasf), rq);
 }
 
-// Per-channel constants, seven rows of `stride` floats, built on the host (conv.hip):
+// Per-channel constants, eight rows of `stride` floats, built on the host (conv.hip):
 //   row 0 mult   s_in * s_w[c]                      row 1 biasf  float(bias[c]) * s_b[c]
-//   row 2 fm     fl(mult * fl(1/s_out))             row 3 fb     fl(fl(biasf * fl(1/s_out)) + offset'),
-//                                                    offset' = offset + Requant::pk_bias (codes as unsigned bytes)
-//   row 4 thr    tie threshold for rows 2/3 (negative: the channel always takes the exact path)
-//   row 5 fbc    fb + corr * fm                     row 6 thrc   tie threshold for rows 2/5
-// Rows 5/6 serve kernels whose accumulators start at zero: the zero-point correction corr[c] is then part of the
-// fast-path constant, and only the exact path adds it to the accumulator as an integer.
+//   rows 2..5    m+, b+, m-, b-   the bracket of the fast path (below); b carries offset' = offset + Requant::pk_bias
+//                                 (codes as unsigned bytes)
+//   rows 6, 7    bc+, bc-         b+ and b- with corr * m+ / corr * m- added
+// Rows 6/7 serve kernels whose accumulators start at zero: the zero-point correction corr[c] is then part of the
+// fast-path constants, and only the exact path adds it to the accumulator as an integer.
 struct ChanTab
 {
     const float* p;
@@ -46,17 +45,21 @@ struct ChanTab
 };
 
 // Fast path with an exact fallback.
-//   r' = fma(float(acc), fm, fb) approximates  t = f/s_out + offset  (f = the reference's fp32 value).  Counting every
-//   rounding on both sides (three in the reference; the reciprocal, two coefficient products, the offset add and the
-//   fma on ours), each relative 2^-24 to a magnitude bounded through |r'|, one gets
-//       |r' - (fl(f/s_out) + offset)|  <=  2^-24 * (8 |r'| + 9 |offset| + 9 |biasf/s_out| + 7 |corr*fm|)
-//   (this includes the int32 -> fp32 conversion of accumulators beyond 2^24 on either path).
-//   The two can therefore round to different integers only when r' lies that close to a half-integer.  The test
-//       |r' - rint(r')|  <=  thr[c] - kTieSlope * |r'|,    thr[c] = 0.5 - 1.5 * 2^-24 * (9|offset| + 9|biasf/s_out| + 7|corr*fm| + 64)
-//   (1.5x margin on every term) passes everything else; values that fail it -- a few in 10^4 -- are recomputed with
-//   the reference's own sequence.  Results beyond the 8-bit range clamp alike on both paths.  Round-half-even
-//   (v_rndne) serves on the fast path: it differs from round-half-away only at exact ties, which fail the test.
-constexpr float kTieSlope = 12.0f / 16777216.0f;
+//   With rho = float(acc) * fm + fb in real arithmetic (fm = fl(mult * fl(1/s_out)), fb = fl(fl(biasf * fl(1/s_out)) + offset'))
+//   and t = fl(f / s_out) + offset' the reference's value before rounding (f = fl(fl(float(acc) * mult) + biasf)), counting
+//   every rounding on both sides (three in the reference, five in the constants) gives
+//       |t - rho|  <=  2^-24 * (5 |rho| + 10 |biasf / s_out| + 6 |offset'|),
+//   two more |rho| where a kernel converts an accumulator beyond 2^24 without its zero-point correction.
+//   The host widens that to a bracket r- < t < r+ that costs one FMA per side,
+//       r+ = fma(float(acc), m+, b+),   m+ = fm (1 + e),  b+ = fb (1 + e) + c
+//       r- = fma(float(acc), m-, b-),   m- = fm (1 - e),  b- = fb (1 - e) - c
+//   with e = 16 * 2^-24 and c a per-channel constant that also covers the roundings of m+-, b+- and of the FMA itself
+//   (conv.hip, 1.5x margin on every term; valid while -1 <= rho <= 257, and beyond that range both sides saturate).
+//   v_cvt_pk_u8_f32 rounds to nearest (ties to even) and saturates to 0..255, both monotone, so when r- and r+ convert
+//   to the same byte, t -- strictly between them -- rounds to that byte under any tie rule, the reference's half-away-
+//   from-zero included.  Values whose two bytes differ (about two in 10^4: r lies that close to a half-integer) are
+//   recomputed with the reference's own sequence.  A channel without a fast path has m+ = m- = 0, b+ = 255, b- = 0.
+//   The activation's clamp, where it is narrower than 0..255, is applied to both sides before converting.
 
 __device__ __forceinline__ uint32_t Pack4(int q0, int q1, int q2, int q3)
 {
@@ -68,90 +71,76 @@ __device__ __forceinline__ uint32_t Pack4(int q0, int q1, int q2, int q3)
 
 struct Fast4
 {
-    float4 m, b, t;      // rows 2, 3, 4: the fast path
-    float4 m0, b0;       // rows 0, 1: the exact path, fetched along so that entering it waits for nothing
+    float4 mp, bp, mm, bm;   // rows 2..5: the bracket (the rare exact path fetches rows 0 / 1 when it is entered)
 };
 
 __device__ __forceinline__ Fast4 LoadFast4(const ChanTab& ct, int c)
 {
     Fast4 f;
-    f.m = *reinterpret_cast<const float4*>(ct.p + 2 * ct.stride + c);
-    f.b = *reinterpret_cast<const float4*>(ct.p + 3 * ct.stride + c);
-    f.t = *reinterpret_cast<const float4*>(ct.p + 4 * ct.stride + c);
-    f.m0 = *reinterpret_cast<const float4*>(ct.p + c);
-    f.b0 = *reinterpret_cast<const float4*>(ct.p + ct.stride + c);
+    f.mp = *reinterpret_cast<const float4*>(ct.p + 2 * ct.stride + c);
+    f.bp = *reinterpret_cast<const float4*>(ct.p + 3 * ct.stride + c);
+    f.mm = *reinterpret_cast<const float4*>(ct.p + 4 * ct.stride + c);
+    f.bm = *reinterpret_cast<const float4*>(ct.p + 5 * ct.stride + c);
     return f;
 }
 
-// K = rint(r'), SLOW = the value needs the exact path ("not <=" also catches NaN)
-#define MI355X_FAST1(ACC, M, B, T, K, SLOW)                                   \
-    {                                                                         \
-        const float r_ = __fmaf_rn(static_cast<float>(ACC), M, B);            \
-        K = __builtin_rintf(r_);                                              \
-        const float e_ = __fsub_rn(r_, K);                                    \
-        SLOW = !(fabsf(e_) <= __fmaf_rn(fabsf(r_), -kTieSlope, T));           \
-    }
-
-// r' is first clamped to a quarter code beyond the activation's range [LO, HI] (biased domain): whatever lies further out
-// ends at LO or HI on either path, its distance to an integer is then exactly 0.25, and it can never look like a tie.
-// K = rint(r'), U = |r' - K| + kTieSlope |r'|: the value needs the exact path when U exceeds its channel's threshold.
-#define MI355X_FAST1U(ACC, M, B, LO, HI, K, U)                                                        \
-    {                                                                                                 \
-        const float r_ = __builtin_amdgcn_fmed3f(__fmaf_rn(static_cast<float>(ACC), M, B), LO, HI);   \
-        K = __builtin_rintf(r_);                                                                      \
-        U = __fmaf_rn(fabsf(r_), kTieSlope, fabsf(__fsub_rn(r_, K)));                                 \
-    }
-
 // Four consecutive channels c..c+3 of one pixel -> packed dword.
-// The fast path is branch-free, 7 VALU instructions per value plus a few per quad: the four tie measures are folded
-// with v_max3 / v_max and compared once against the smallest of the four thresholds (a smaller threshold only sends
-// more values to the exact path), so a quad costs one compare and one scalar branch.  r' is finite whenever a
-// threshold is non-negative (the host checks the constants and the accumulator range), so no NaN can hide in the
-// maxima; a channel without a fast path has threshold -1, which every measure exceeds.  When some lane of the wave has
-// a flagged value, the wave redoes that value's position of the quad with the reference's sequence on every lane (always
-// right, and cheaper than sorting out which lanes need it); LOAD_EXACT supplies rows 0 / 1 of the table and, for kernels
-// whose accumulators start at zero, the zero-point correction that only the exact path adds as an integer.
+// Five VALU instructions per value on the fast path (convert, two FMAs, two converting packs; two v_med3 more when the
+// activation clamps inside 0..255) and one compare and scalar branch per quad.  When some lane of the wave has a byte
+// that differs between the two sides, the wave redoes that position of the quad with the reference's sequence on every
+// lane (always right, and cheaper than sorting out which lanes need it); LOAD_EXACT supplies rows 0 / 1 of the table
+// and, for kernels whose accumulators start at zero, the zero-point correction that only the exact path adds as an
+// integer.  The constants are finite (the host checks them and the accumulator range), so no NaN reaches a conversion.
 template <typename LoadExact>
-__device__ __forceinline__ uint32_t Requant4Core(int a0, int a1, int a2, int a3, const float4& fm, const float4& fb,
-                                                 const float4& thr, const Requant& rq, LoadExact load_exact)
+__device__ __forceinline__ uint32_t Requant4Core(int a0, int a1, int a2, int a3, const float4& mp, const float4& bp,
+                                                 const float4& mm, const float4& bm, const Requant& rq, LoadExact load_exact)
 {
-    float k0, k1, k2, k3, u0, u1, u2, u3;
-    MI355X_FAST1U(a0, fm.x, fb.x, rq.pk_lo_q, rq.pk_hi_q, k0, u0)
-    MI355X_FAST1U(a1, fm.y, fb.y, rq.pk_lo_q, rq.pk_hi_q, k1, u1)
-    MI355X_FAST1U(a2, fm.z, fb.z, rq.pk_lo_q, rq.pk_hi_q, k2, u2)
-    MI355X_FAST1U(a3, fm.w, fb.w, rq.pk_lo_q, rq.pk_hi_q, k3, u3)
-    const float umax = fmaxf(fmaxf(fmaxf(u0, u1), u2), u3);       // v_max3_f32 + v_max_f32
-    const float tmin = fminf(fminf(thr.x, thr.y), fminf(thr.z, thr.w));
-    // integral floats within [LO, HI] -> unsigned bytes, one instruction per value, packed as it goes
-    uint32_t out = __builtin_amdgcn_cvt_pk_u8_f32(k0, 0, 0u);
-    out = __builtin_amdgcn_cvt_pk_u8_f32(k1, 1, out);
-    out = __builtin_amdgcn_cvt_pk_u8_f32(k2, 2, out);
-    out = __builtin_amdgcn_cvt_pk_u8_f32(k3, 3, out);
-    if (__builtin_expect(__builtin_amdgcn_ballot_w64(!(umax <= tmin)) != 0, 0))
+    const float f0 = static_cast<float>(a0), f1 = static_cast<float>(a1), f2 = static_cast<float>(a2), f3 = static_cast<float>(a3);
+    float p0 = __fmaf_rn(f0, mp.x, bp.x), p1 = __fmaf_rn(f1, mp.y, bp.y), p2 = __fmaf_rn(f2, mp.z, bp.z), p3 = __fmaf_rn(f3, mp.w, bp.w);
+    float q0 = __fmaf_rn(f0, mm.x, bm.x), q1 = __fmaf_rn(f1, mm.y, bm.y), q2 = __fmaf_rn(f2, mm.z, bm.z), q3 = __fmaf_rn(f3, mm.w, bm.w);
+    if (!rq.pk_full)
+    {
+        p0 = __builtin_amdgcn_fmed3f(p0, rq.pk_lo_f, rq.pk_hi_f); q0 = __builtin_amdgcn_fmed3f(q0, rq.pk_lo_f, rq.pk_hi_f);
+        p1 = __builtin_amdgcn_fmed3f(p1, rq.pk_lo_f, rq.pk_hi_f); q1 = __builtin_amdgcn_fmed3f(q1, rq.pk_lo_f, rq.pk_hi_f);
+        p2 = __builtin_amdgcn_fmed3f(p2, rq.pk_lo_f, rq.pk_hi_f); q2 = __builtin_amdgcn_fmed3f(q2, rq.pk_lo_f, rq.pk_hi_f);
+        p3 = __builtin_amdgcn_fmed3f(p3, rq.pk_lo_f, rq.pk_hi_f); q3 = __builtin_amdgcn_fmed3f(q3, rq.pk_lo_f, rq.pk_hi_f);
+    }
+    // round to nearest, saturate to 0..255 and pack, one instruction per value
+    uint32_t out = __builtin_amdgcn_cvt_pk_u8_f32(p0, 0, 0u);
+    out = __builtin_amdgcn_cvt_pk_u8_f32(p1, 1, out);
+    out = __builtin_amdgcn_cvt_pk_u8_f32(p2, 2, out);
+    out = __builtin_amdgcn_cvt_pk_u8_f32(p3, 3, out);
+    uint32_t low = __builtin_amdgcn_cvt_pk_u8_f32(q0, 0, 0u);
+    low = __builtin_amdgcn_cvt_pk_u8_f32(q1, 1, low);
+    low = __builtin_amdgcn_cvt_pk_u8_f32(q2, 2, low);
+    low = __builtin_amdgcn_cvt_pk_u8_f32(q3, 3, low);
+    const uint32_t differ = out ^ low;
+    if (__builtin_expect(__builtin_amdgcn_ballot_w64(differ != 0u) != 0, 0))
     {
         float4 m, b;
         int4 cr;
         load_exact(m, b, cr);
         // usually one value of the wave's 256 is flagged: only its position is redone (on every lane: the exact result is
         // always the right one)
-        if (__builtin_amdgcn_ballot_w64(!(u0 <= tmin)) != 0)
+        if (__builtin_amdgcn_ballot_w64((differ & 0x000000ffu) != 0u) != 0)
             out = (out & 0xffffff00u) | (static_cast<uint32_t>(RequantExactDev(a0 + cr.x, m.x, b.x, rq) + rq.pk_bias) & 0xffu);
-        if (__builtin_amdgcn_ballot_w64(!(u1 <= tmin)) != 0)
+        if (__builtin_amdgcn_ballot_w64((differ & 0x0000ff00u) != 0u) != 0)
             out = (out & 0xffff00ffu) | ((static_cast<uint32_t>(RequantExactDev(a1 + cr.y, m.y, b.y, rq) + rq.pk_bias) & 0xffu) << 8);
-        if (__builtin_amdgcn_ballot_w64(!(u2 <= tmin)) != 0)
+        if (__builtin_amdgcn_ballot_w64((differ & 0x00ff0000u) != 0u) != 0)
             out = (out & 0xff00ffffu) | ((static_cast<uint32_t>(RequantExactDev(a2 + cr.z, m.z, b.z, rq) + rq.pk_bias) & 0xffu) << 16);
-        if (__builtin_amdgcn_ballot_w64(!(u3 <= tmin)) != 0)
+        if (__builtin_amdgcn_ballot_w64((differ & 0xff000000u) != 0u) != 0)
             out = (out & 0x00ffffffu) | ((static_cast<uint32_t>(RequantExactDev(a3 + cr.w, m.w, b.w, rq) + rq.pk_bias) & 0xffu) << 24);
     }
     return out ^ rq.pk_xor;
 }
 
-// `corr` (may be null) is an integer added to the accumulator on the exact path only (rows 5/6, see ChanTab).
-__device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const float4& fm, const float4& fb,
-                                                const float4& thr, const ChanTab& ct, const int32_t* corr, int c,
+// Bracket constants given row by row (kernels that keep rows 2, 6, 4, 7 -- the corr-folded bracket -- in LDS or registers).
+// `corr` (may be null) is an integer added to the accumulator on the exact path only.
+__device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const float4& mp, const float4& bp,
+                                                const float4& mm, const float4& bm, const ChanTab& ct, const int32_t* corr, int c,
                                                 const Requant& rq)
 {
-    return Requant4Core(a0, a1, a2, a3, fm, fb, thr, rq, [&](float4& m, float4& b, int4& cr) {
+    return Requant4Core(a0, a1, a2, a3, mp, bp, mm, bm, rq, [&](float4& m, float4& b, int4& cr) {
         m = *reinterpret_cast<const float4*>(ct.p + c);
         b = *reinterpret_cast<const float4*>(ct.p + ct.stride + c);
         cr = int4{0, 0, 0, 0};
@@ -159,35 +148,34 @@ __device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, 
     });
 }
 
-// constants of rows 2,3,4 (accumulator already contains the zero-point correction), exact-path rows fetched beforehand
-__device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const Fast4& f, const ChanTab&, int,
+// constants of rows 2..5 (accumulator already contains the zero-point correction)
+__device__ __forceinline__ uint32_t Requant4Dev(int a0, int a1, int a2, int a3, const Fast4& f, const ChanTab& ct, int c,
                                                 const Requant& rq)
 {
-    return Requant4Core(a0, a1, a2, a3, f.m, f.b, f.t, rq, [&](float4& m, float4& b, int4& cr) {
-        m = f.m0;
-        b = f.b0;
-        cr = int4{0, 0, 0, 0};
-    });
+    return Requant4Dev(a0, a1, a2, a3, f.mp, f.bp, f.mm, f.bm, ct, nullptr, c, rq);
 }
 
-// one channel (scalar kernels)
+// one channel (scalar kernels): the same bracket, compared after rounding
+__device__ __forceinline__ int RequantBracket1(int acc, int exact_acc, float mp, float bp, float mm, float bm, float m0, float b0, const Requant& rq)
+{
+    const float f = static_cast<float>(acc);
+    const float kp = __builtin_rintf(__builtin_amdgcn_fmed3f(__fmaf_rn(f, mp, bp), rq.pk_lo_f, rq.pk_hi_f));
+    const float km = __builtin_rintf(__builtin_amdgcn_fmed3f(__fmaf_rn(f, mm, bm), rq.pk_lo_f, rq.pk_hi_f));
+    if (__builtin_expect(!(kp == km), 0)) return RequantExactDev(exact_acc, m0, b0, rq);
+    return static_cast<int>(kp) - rq.pk_bias;
+}
+
 __device__ __forceinline__ int Requant1Dev(int acc, const ChanTab& ct, int c, const Requant& rq)
 {
-    float k;
-    bool slow;
-    MI355X_FAST1(acc, ct.p[2 * ct.stride + c], ct.p[3 * ct.stride + c], ct.p[4 * ct.stride + c], k, slow)
-    if (__builtin_expect(slow, 0)) return RequantExactDev(acc, ct.p[c], ct.p[ct.stride + c], rq);
-    return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.pk_lo_f, rq.pk_hi_f)) - rq.pk_bias;
+    return RequantBracket1(acc, acc, ct.p[2 * ct.stride + c], ct.p[3 * ct.stride + c], ct.p[4 * ct.stride + c], ct.p[5 * ct.stride + c],
+                           ct.p[c], ct.p[ct.stride + c], rq);
 }
 
-// one channel, accumulator started at zero: rows 2/5/6 on the fast path, `corr[c]` joins the accumulator on the exact path
+// one channel, accumulator started at zero: rows 2/6/4/7 on the fast path, `corr[c]` joins the accumulator on the exact path
 __device__ __forceinline__ int Requant1FoldedDev(int acc, const ChanTab& ct, const int32_t* corr, int c, const Requant& rq)
 {
-    float k;
-    bool slow;
-    MI355X_FAST1(acc, ct.p[2 * ct.stride + c], ct.p[5 * ct.stride + c], ct.p[6 * ct.stride + c], k, slow)
-    if (__builtin_expect(slow, 0)) return RequantExactDev(acc + corr[c], ct.p[c], ct.p[ct.stride + c], rq);
-    return static_cast<int>(__builtin_amdgcn_fmed3f(k, rq.pk_lo_f, rq.pk_hi_f)) - rq.pk_bias;
+    return RequantBracket1(acc, acc + corr[c], ct.p[2 * ct.stride + c], ct.p[6 * ct.stride + c], ct.p[4 * ct.stride + c], ct.p[7 * ct.stride + c],
+                           ct.p[c], ct.p[ct.stride + c], rq);
 }
 
 // value already in float (pooling, add, ...): reciprocal fast path with the exact fallback near ties.

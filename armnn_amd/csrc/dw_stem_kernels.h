@@ -455,12 +455,13 @@ __global__ __launch_bounds__(256) void SmallCiConvKernel(SmallCiArgs a)
                         }
                     }
             }
-            const float4 fm = {tab[2 * ts + c], tab[2 * ts + c + 1], tab[2 * ts + c + 2], tab[2 * ts + c + 3]};
-            const float4 fb = {tab[5 * ts + c], tab[5 * ts + c + 1], tab[5 * ts + c + 2], tab[5 * ts + c + 3]};
-            const float4 th = {tab[6 * ts + c], tab[6 * ts + c + 1], tab[6 * ts + c + 2], tab[6 * ts + c + 3]};
+            const float4 mp = {tab[2 * ts + c], tab[2 * ts + c + 1], tab[2 * ts + c + 2], tab[2 * ts + c + 3]};
+            const float4 bp = {tab[6 * ts + c], tab[6 * ts + c + 1], tab[6 * ts + c + 2], tab[6 * ts + c + 3]};
+            const float4 mm = {tab[4 * ts + c], tab[4 * ts + c + 1], tab[4 * ts + c + 2], tab[4 * ts + c + 3]};
+            const float4 bm = {tab[7 * ts + c], tab[7 * ts + c + 1], tab[7 * ts + c + 2], tab[7 * ts + c + 3]};
 #pragma unroll
             for (int p = 0; p < P; ++p)
-                o[p][g4] = Requant4Dev(acc[p][0], acc[p][1], acc[p][2], acc[p][3], fm, fb, th, a.ct, a.corr, c, a.rq);
+                o[p][g4] = Requant4Dev(acc[p][0], acc[p][1], acc[p][2], acc[p][3], mp, bp, mm, bm, a.ct, a.corr, c, a.rq);
         }
         if (groups == 4 && a.vec16)
         {
@@ -493,7 +494,7 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
     constexpr int NDWP = KH * RD;                 // patch dwords per pixel
     constexpr int KST = (NDWP + 7) / 8;           // MFMA k-steps of 32 bytes
     __shared__ __attribute__((aligned(16))) uint32_t tile[SmallCiTile<KH, TH>::DWORDS];
-    __shared__ __attribute__((aligned(16))) float cst[3][NT * 32];
+    __shared__ __attribute__((aligned(16))) float cst[4][NT * 32];      // the corr-folded bracket: m+, bc+, m-, bc-
 
     int b = blockIdx.x;
     const int tx = b % a.tiles_x; b /= a.tiles_x;
@@ -503,10 +504,10 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
     const int S = a.stride;
     int iy_org, ix_org, mis;
     StageSmallCiHalo<KH, TH>(a, tile, tx, ty, n, tid, iy_org, ix_org, mis);
-    for (int i = tid; i < 3 * NT * 32; i += 256)
+    for (int i = tid; i < 4 * NT * 32; i += 256)
     {
         const int row = i / (NT * 32), c = i - row * (NT * 32);
-        cst[row][c] = a.ct.p[(row == 0 ? 2 : row == 1 ? 5 : 6) * a.ct.stride + c];
+        cst[row][c] = a.ct.p[(row == 0 ? 2 : row == 1 ? 6 : row == 2 ? 4 : 7) * a.ct.stride + c];
     }
 
     const int lane = tid & 63, wave = tid >> 6;
@@ -577,10 +578,11 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
             for (int qd = 0; qd < 4; ++qd)
             {
                 const int cl = ct * 32 + 8 * qd + 4 * half;
-                const float4 fm = *reinterpret_cast<const float4*>(&cst[0][cl]);
-                const float4 fb = *reinterpret_cast<const float4*>(&cst[1][cl]);
-                const float4 th = *reinterpret_cast<const float4*>(&cst[2][cl]);
-                o[qd] = Requant4Dev(acc[4 * qd + 0], acc[4 * qd + 1], acc[4 * qd + 2], acc[4 * qd + 3], fm, fb, th, a.ct, a.corr, cl, a.rq);
+                const float4 mp = *reinterpret_cast<const float4*>(&cst[0][cl]);
+                const float4 bp = *reinterpret_cast<const float4*>(&cst[1][cl]);
+                const float4 mm = *reinterpret_cast<const float4*>(&cst[2][cl]);
+                const float4 bm = *reinterpret_cast<const float4*>(&cst[3][cl]);
+                o[qd] = Requant4Dev(acc[4 * qd + 0], acc[4 * qd + 1], acc[4 * qd + 2], acc[4 * qd + 3], mp, bp, mm, bm, a.ct, a.corr, cl, a.rq);
             }
             // lane and lane + 32 hold interleaved 4-channel groups of one pixel; trading two dwords gives each of them
             // 16 contiguous channels (the low lane 0..15, the high lane 16..31) and one 16-byte store

@@ -31,7 +31,7 @@ struct DwPwArgs
     // depthwise stage
     const uint8_t*  x;
     const uint8_t*  pad16;      // 16 bytes that become the depthwise padding value under dw_xor
-    const uint32_t* dw_grp;     // [C/4][8][4] dwords per group of 4 channels: w row 0, w row 1, w row 2, corr, fm, fb, thr, 0
+    const uint32_t* dw_grp;     // [C/4][8][4] dwords per group of 4 channels: w row 0, w row 1, w row 2, corr, m+, b+, m-, b-
     ChanTab         dw_ct;      // exact-path constants of the depthwise layer
     int N, H, W, C, Ho, Wo;
     int pad_top, pad_left;
@@ -211,14 +211,15 @@ __global__ __launch_bounds__(256) void DwPwKernel(DwPwArgs a)
                 }
             }
         }
-        const float4 fm = *reinterpret_cast<const float4*>(gc + 4);
-        const float4 fb = *reinterpret_cast<const float4*>(gc + 5);
-        const float4 th = *reinterpret_cast<const float4*>(gc + 6);
+        const float4 mp = *reinterpret_cast<const float4*>(gc + 4);
+        const float4 bp = *reinterpret_cast<const float4*>(gc + 5);
+        const float4 mm = *reinterpret_cast<const float4*>(gc + 6);
+        const float4 bm = *reinterpret_cast<const float4*>(gc + 7);
         const int c = cb * 32 + c4 * 4;
 #pragma unroll
         for (int j = 0; j < P; ++j)
         {
-            const uint32_t q = Requant4Dev(acc[j][0], acc[j][1], acc[j][2], acc[j][3], fm, fb, th, a.dw_ct, nullptr, c, a.dw_rq);
+            const uint32_t q = Requant4Dev(acc[j][0], acc[j][1], acc[j][2], acc[j][3], mp, bp, mm, bm, a.dw_ct, nullptr, c, a.dw_rq);
             *reinterpret_cast<uint32_t*>(T + (row * TW + xg * P + j) * LDT + c) = q ^ mid;
         }
     };
@@ -304,11 +305,12 @@ __global__ __launch_bounds__(256) void DwPwKernel(DwPwArgs a)
                 {
                     const int cl = i * 32 + 8 * q + lane_c;
                     const int cg = ct * 32 + cl;
-                    const float4 fm = *reinterpret_cast<const float4*>(a.pw_ct.p + 2 * a.pw_ct.stride + cg);
-                    const float4 fb = *reinterpret_cast<const float4*>(a.pw_ct.p + 5 * a.pw_ct.stride + cg);
-                    const float4 th = *reinterpret_cast<const float4*>(a.pw_ct.p + 6 * a.pw_ct.stride + cg);
+                    const float4 mp = *reinterpret_cast<const float4*>(a.pw_ct.p + 2 * a.pw_ct.stride + cg);
+                    const float4 bp = *reinterpret_cast<const float4*>(a.pw_ct.p + 6 * a.pw_ct.stride + cg);
+                    const float4 mm = *reinterpret_cast<const float4*>(a.pw_ct.p + 4 * a.pw_ct.stride + cg);
+                    const float4 bm = *reinterpret_cast<const float4*>(a.pw_ct.p + 7 * a.pw_ct.stride + cg);
                     const v16i& v = acc[i][p];
-                    const uint32_t out = Requant4Dev(v[4 * q + 0], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3], fm, fb, th, a.pw_ct, a.pw_corr, cg, a.pw_rq);
+                    const uint32_t out = Requant4Dev(v[4 * q + 0], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3], mp, bp, mm, bm, a.pw_ct, a.pw_corr, cg, a.pw_rq);
                     *reinterpret_cast<uint32_t*>(ostage + frag_row * LDO + cl) = out;
                 }
             __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");

@@ -43,7 +43,7 @@ struct PwArgs
 template <int BN>
 constexpr int PwSmemBytes(int K)
 {
-    return BN * (K + 16) + 4 * 32 * (BN + 16) + 3 * BN * 4;
+    return BN * (K + 16) + 4 * 32 * (BN + 16) + 4 * BN * 4;
 }
 
 // KS = MFMA k-steps (of 32) per register chunk, K % (32 * KS) == 0;  NB = register chunks per wave (NB-1 in flight).
@@ -57,8 +57,8 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     const int LDW = a.K + 16;
     uint8_t* slab = smem;
-    float* cst = reinterpret_cast<float*>(smem + BN * LDW);                 // [3][BN]: fm, fb(folded), thr(folded)
-    uint8_t* ostage_all = smem + BN * LDW + 3 * BN * 4;
+    float* cst = reinterpret_cast<float*>(smem + BN * LDW);                 // [4][BN]: the corr-folded bracket m+, bc+, m-, bc-
+    uint8_t* ostage_all = smem + BN * LDW + 4 * BN * 4;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63;
@@ -127,11 +127,12 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
             for (int q = 0; q < 4; ++q)
             {
                 const int cl = tc * 32 + 8 * q + lane_c;
-                const float4 fm = *reinterpret_cast<const float4*>(cst + cl);
-                const float4 fb = *reinterpret_cast<const float4*>(cst + BN + cl);
-                const float4 th = *reinterpret_cast<const float4*>(cst + 2 * BN + cl);
+                const float4 mp = *reinterpret_cast<const float4*>(cst + cl);
+                const float4 bp = *reinterpret_cast<const float4*>(cst + BN + cl);
+                const float4 mm = *reinterpret_cast<const float4*>(cst + 2 * BN + cl);
+                const float4 bm = *reinterpret_cast<const float4*>(cst + 3 * BN + cl);
                 const uint32_t out = Requant4Dev(acc[tc][4 * q + 0] + rt, acc[tc][4 * q + 1] + rt, acc[tc][4 * q + 2] + rt, acc[tc][4 * q + 3] + rt,
-                                                 fm, fb, th, a.ct, a.corr, n0 + cl, a.rq);
+                                                 mp, bp, mm, bm, a.ct, a.corr, n0 + cl, a.rq);
                 *reinterpret_cast<uint32_t*>(ostage + frag_row * LDO + cl) = out;
             }
         }
@@ -194,10 +195,11 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
 #pragma unroll
             for (int i = 0; i < BN / 16; ++i) *reinterpret_cast<v4i*>(slab + ((tid >> 4) + 16 * i) * LDW + c * 16) = t[i];
         }
-        for (int i = tid; i < 3 * BN; i += 256)
+        for (int i = tid; i < 4 * BN; i += 256)
         {
+            // the corr-folded bracket: m+, bc+, m-, bc-
             const int row = i / BN, c = i - row * BN;
-            const int src_row = row == 0 ? 2 : row == 1 ? 5 : 6;
+            const int src_row = row == 0 ? 2 : row == 1 ? 6 : row == 2 ? 4 : 7;
             cst[i] = a.ct.p[src_row * a.ct.stride + n0 + c];
         }
     }
@@ -381,10 +383,11 @@ __global__ __launch_bounds__(256) void SmallMGemmKernel(GemvArgs a)
     // accumulator group g of the 32x32 tile: channels 8 g + 4 (lane / 32) + 0..3 of row lane % 32
     const int c = n0 + 8 * wave + 4 * (lane >> 5);
     const int row = m0 + frag_row;
-    const float4 fm = *reinterpret_cast<const float4*>(a.ct.p + 2 * a.ct.stride + c);
-    const float4 fb = *reinterpret_cast<const float4*>(a.ct.p + 5 * a.ct.stride + c);
-    const float4 th = *reinterpret_cast<const float4*>(a.ct.p + 6 * a.ct.stride + c);
-    const uint32_t out = Requant4Dev(v[0], v[1], v[2], v[3], fm, fb, th, a.ct, a.corr, c, a.rq);
+    const float4 mp = *reinterpret_cast<const float4*>(a.ct.p + 2 * a.ct.stride + c);
+    const float4 bp = *reinterpret_cast<const float4*>(a.ct.p + 6 * a.ct.stride + c);
+    const float4 mm = *reinterpret_cast<const float4*>(a.ct.p + 4 * a.ct.stride + c);
+    const float4 bm = *reinterpret_cast<const float4*>(a.ct.p + 7 * a.ct.stride + c);
+    const uint32_t out = Requant4Dev(v[0], v[1], v[2], v[3], mp, bp, mm, bm, a.ct, a.corr, c, a.rq);
     if (row < a.M)
     {
         uint8_t* dst = a.y + static_cast<long long>(row) * a.N + c;

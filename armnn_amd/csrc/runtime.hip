@@ -107,8 +107,6 @@ Requant MakeRequant(const mi355x_quant& out, int32_t activation, float a, float 
     rq.pk_xor  = rq.out_is_u8 ? 0u : 0x80808080u;
     rq.pk_lo_f = static_cast<float>(rq.act_lo + rq.pk_bias);
     rq.pk_hi_f = static_cast<float>(rq.act_hi + rq.pk_bias);
-    rq.pk_lo_q = rq.pk_lo_f - 0.25f;
-    rq.pk_hi_q = rq.pk_hi_f + 0.25f;
     rq.pk_full = (rq.act_lo + rq.pk_bias == 0 && rq.act_hi + rq.pk_bias == 255) ? 1 : 0;
     rq.fast_ok = !GlobalOptions().exact_division_epilogue && std::isnormal(rq.inv_scale) && std::isnormal(out.scale) && out.offset >= -255 && out.offset <= 255 &&
                  rq.act_lo <= rq.act_hi;

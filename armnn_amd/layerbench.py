@@ -77,8 +77,8 @@ def main(argv=None):
                     help="with --wzp: multiply the weight draws (std 30) by this before adding the zero point; 3 spreads the "
                          "codes over the whole uint8 range, so that weight minus zero point no longer fits int8")
     ap.add_argument("--algo", type=int, default=0)
-    ap.add_argument("--iters", type=int, default=50)
-    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--iters", type=int, default=500, help="timed launches; long enough for the clocks to settle")
+    ap.add_argument("--warmup", type=int, default=200)
     ap.add_argument("--opt", action="append", default=[], metavar="NAME=VALUE", help="mi355x_set_option before the plan is built")
     a = ap.parse_args(argv)
     for item in a.opt:
