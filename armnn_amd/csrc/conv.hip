@@ -7,6 +7,7 @@
 #include "pw_gemm_kernel.h"
 #include "igemm_lds_kernel.h"
 #include "big_gemm.h"
+#include "halo_conv_kernel.h"
 
 #include <algorithm>
 #include <cmath>
@@ -43,6 +44,7 @@ struct mi355x_conv2d_s
     std::vector<double> fast_cw;           // bracket (negative: no fast path), kept until the table is uploaded
     int pw_bn = 0, pw_ks = 0;      // pointwise GEMM kernel configuration (0: not applicable)
     bool bk128 = false;            // implicit GEMM walks K in 128-byte tiles
+    bool halo_ok = false;          // shape fits the resident-tile kernel (weights without a zero point are checked at launch)
     int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 96 (= 128x64) / 128: the "igemm_tile" option at plan creation
     int opt_igemm_lds = 2, opt_dw_rows = 0, opt_stem_dot4 = 0;     // the other process-wide options, as they stood at plan creation
                                    // (launches read the plan, never the mutable globals: plans may run on any host thread)
@@ -171,6 +173,11 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     // for it; otherwise 64.
     p->K_pad = (p->K + 63) / 64 * 64;
     p->bk128 = (d.in_c % 128) == 0 && (p->K % 128) == 0;
+    // small filter, stride 1, 64 / 128 / 256 input channels: the resident-tile kernel (halo_conv_kernel.h) walks K in
+    // 128-byte tiles, so K is padded to that
+    p->halo_ok = !d.depthwise && (d.in_c == 64 || d.in_c == 128 || d.in_c == 256) && d.kernel_h * d.kernel_w > 1 && d.kernel_h <= 3 &&
+                 d.kernel_w <= 3 && d.stride_x == 1 && d.stride_y == 1 && d.dilation_x == 1 && d.dilation_y == 1 && d.out_w <= 224;
+    if (p->halo_ok) p->K_pad = (p->K + 127) / 128 * 128;
 
     // ---- per-channel requantization constants, in fp32 exactly as the reference's decoders produce them ----
     std::vector<float> mult(p->Co_pad, 0.0f), biasf(p->Co_pad, 0.0f);
@@ -337,6 +344,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             snprintf(buf, sizeof(buf), "igemm_mfma_i8_32x32x32 tiles 128x128|128x64|64x64 x%d K=%d", p->bk128 ? 128 : 64, p->K);
         p->info = buf;
         if (p->zw_neg != 0) p->info += ", weight zero point by row sums";
+        else if (p->halo_ok) p->info += "; launches of 192 or more row tiles: input tile resident in LDS for all taps";
     }
     else if (algo == MI355X_ALGO_DEPTHWISE && dw3_ok)
     {
@@ -749,6 +757,79 @@ int LaunchIgemmLds(const mi355x_conv2d_s* p, int stages, uint32_t batch, const v
     return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 2, true, false>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 2, false, false>(p, batch, x, y, stream);
 }
 
+template <int CI, int WM, int WN, int TP, int ST, bool U8>
+int LaunchHaloT(const HaloArgs& a, int smem, hipStream_t stream)
+{
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&HaloConvKernel<CI, WM, WN, TP, ST, U8>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+    MI355X_HIP(attr);
+    NoteKernel("HaloConvKernel<%d, %d, %d, %d, %d, %s>", CI, WM, WN, TP, ST, BoolName(U8));
+    const int nblocks = a.tiles_m * a.tiles_n;
+    hipLaunchKernelGGL((HaloConvKernel<CI, WM, WN, TP, ST, U8>), dim3((nblocks + 7) / 8 * 8), dim3(256), smem, stream, a);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+template <int CI, int WM, int WN, int TP>
+int LaunchHaloC(HaloArgs& a, const mi355x_conv2d_s* p, uint32_t batch, hipStream_t stream)
+{
+    constexpr int BN = 32 * WN, MF = WM * TP;
+    const ConvGeom& g = p->geom;
+    // as many whole output rows as fit the block's pixel fragments and, with the weight stages, LDS
+    int R = std::min(g.Ho, (32 * MF) / g.Wo);
+    auto smem_of = [&](int rows, int st) {
+        const int hp = (rows + g.Kh - 1) * (g.Wo + g.Kw - 1);
+        return st == 3 ? HaloSmemBytes<CI, BN, MF, 3>(hp) : HaloSmemBytes<CI, BN, MF, 2>(hp);
+    };
+    while (R > 1 && smem_of(R, 2) > 160 * 1024) --R;
+    if (R < 1 || smem_of(R, 2) > 160 * 1024) return -1;
+    a.R = R;
+    a.tiles_y = (g.Ho + R - 1) / R;
+    a.tiles_m = static_cast<int>(batch) * a.tiles_y;
+    a.tiles_n = (g.Co + BN - 1) / BN;
+    a.WP = g.Wo + g.Kw - 1;
+    a.HP = (R + g.Kh - 1) * a.WP;
+    a.wo_magic = static_cast<uint32_t>((0x100000000ull + g.Wo - 1) / g.Wo);
+    a.wp_magic = static_cast<uint32_t>((0x100000000ull + a.WP - 1) / a.WP);
+    const long long blocks = static_cast<long long>(a.tiles_m) * a.tiles_n;
+    // a block is one long dependent chain (tile, k-loop, epilogue): with fewer blocks than CUs the implicit GEMM's smaller
+    // tiles finish sooner
+    if (blocks < 192 && p->tile_override != 3000) return -1;
+    // three weight stages unless two let every block of the launch be resident at once and three do not
+    auto resident = [&](int st) { return 256ll * std::min(4, (160 * 1024) / smem_of(R, st)); };
+    const bool three = smem_of(R, 3) <= 160 * 1024 && !(blocks > resident(3) && blocks <= resident(2));
+    const bool u8 = p->xor_mask != 0;
+    if (three) return u8 ? LaunchHaloT<CI, WM, WN, TP, 3, true>(a, smem_of(R, 3), stream) : LaunchHaloT<CI, WM, WN, TP, 3, false>(a, smem_of(R, 3), stream);
+    return u8 ? LaunchHaloT<CI, WM, WN, TP, 2, true>(a, smem_of(R, 2), stream) : LaunchHaloT<CI, WM, WN, TP, 2, false>(a, smem_of(R, 2), stream);
+}
+
+// Returns -1 when the shape does not fit after all (the caller then takes the implicit GEMM).
+int LaunchHalo(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    const ConvGeom& g = p->geom;
+    HaloArgs a;
+    a.x = static_cast<const uint8_t*>(x);
+    a.pad16 = p->pad16;
+    a.w = p->w_mfma;
+    a.ct = ChanTab{p->chan, p->Co_pad};
+    a.corr = p->corr;
+    a.y = static_cast<uint8_t*>(y);
+    a.H = g.H; a.W = g.W; a.Ho = g.Ho; a.Wo = g.Wo; a.Co = g.Co;
+    a.Kh = g.Kh; a.Kw = g.Kw;
+    a.pad_top = g.pad_top; a.pad_left = g.pad_left;
+    a.K_pad = p->K_pad;
+    a.xor_mask = p->xor_mask;
+    a.rq = p->rq;
+    const bool wide = g.Co > 64;
+    switch (g.Ci)
+    {
+    case 64: return wide ? LaunchHaloC<64, 1, 4, 7>(a, p, batch, stream) : LaunchHaloC<64, 2, 2, 4>(a, p, batch, stream);
+    case 128: return wide ? LaunchHaloC<128, 1, 4, 7>(a, p, batch, stream) : LaunchHaloC<128, 2, 2, 4>(a, p, batch, stream);
+    case 256: return wide ? LaunchHaloC<256, 1, 4, 7>(a, p, batch, stream) : LaunchHaloC<256, 2, 2, 4>(a, p, batch, stream);
+    default: return -1;
+    }
+}
+
 int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
 {
     if (!p) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
@@ -807,6 +888,12 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             if (p->pw_bn == 128) return LaunchPwKs<128>(p, Mrows, x, y, stream);
             if (p->pw_bn == 64) return LaunchPwKs<64>(p, Mrows, x, y, stream);
             return LaunchPwKs<32>(p, Mrows, x, y, stream);
+        }
+        // Small filters at stride 1 over 64 / 128 / 256 channels: the input tile stays in LDS for all taps
+        if (p->halo_ok && p->zw_neg == 0 && p->opt_igemm_lds != 0 && (p->tile_override == 0 || p->tile_override == 3000))
+        {
+            const int rc = LaunchHalo(p, batch, x, y, stream);
+            if (rc >= 0) return rc;
         }
         // Tile choice: the large tile has the best MFMA : LDS-traffic ratio, but a launch needs several blocks per CU
         // in flight to hide global-load latency, so problems that would yield few large tiles take 64x64 tiles

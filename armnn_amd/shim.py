@@ -142,6 +142,11 @@ def _quant(info: TensorInfo) -> Quant:
     return Quant(int(info.dtype), float(np.float32(info.scale)), int(info.offset))
 
 
+def last_kernel() -> str:
+    """Name of the device kernel the calling thread's last launch through the library used (mi355x_last_kernel)."""
+    return (load_library().mi355x_last_kernel() or b"").decode()
+
+
 def set_option(name: str, value: int):
     _chk(load_library().mi355x_set_option(name.encode(), int(value)))
 

@@ -162,6 +162,50 @@ def test_every_igemm_tiling_gives_the_same_bytes():
         shim.set_option("igemm_tile", 100)
 
 
+def test_resident_tile_convolution_gives_the_same_bytes():
+    """Small filters at stride 1 over 64, 128 or 256 input channels keep the input tile in LDS for all taps
+    (HaloConvKernel).  Against the direct kernel: every channel count, narrow and wide output-channel tiles with ragged
+    channel counts, 3x3 / 2x2 / 1x3 / 3x1 filters, SAME, VALID and asymmetric padding, widths that do and do not divide the
+    pixel fragments, a last tile with fewer rows, several images, uint8 activations, fused activations."""
+    U8 = DataType.QAsymmU8
+    cs = [cases.make_conv_case("halo_c64_56", 801, n=16, h=56, w=56, ci=64, co=64, act=cases.RELU6),
+          cases.make_conv_case("halo_c64_ragged", 802, n=3, h=23, w=19, ci=64, co=40, act=cases.RELU),
+          cases.make_conv_case("halo_c64_wide_co", 803, n=1, h=30, w=60, ci=64, co=200),
+          cases.make_conv_case("halo_c64_2x2_valid_u8", 804, n=2, h=17, w=33, ci=64, co=96, kh=2, kw=2, padding="valid", in_dtype=U8, in_offset=131,
+                               out_offset=-100),
+          cases.make_conv_case("halo_c128_28", 805, n=2, h=28, w=28, ci=128, co=128, act=cases.RELU),
+          cases.make_conv_case("halo_c128_1x3_asym", 806, n=1, h=9, w=41, ci=128, co=72, kh=1, kw=3, padding=(0, 0, 2, 0)),
+          cases.make_conv_case("halo_c128_3x1_u8", 807, n=2, h=20, w=14, ci=128, co=256, kh=3, kw=1, in_dtype=U8, in_offset=120, out_offset=10),
+          cases.make_conv_case("halo_c256_14", 808, n=3, h=14, w=14, ci=256, co=256, act=cases.RELU),
+          cases.make_conv_case("halo_c256_7_asym", 809, n=2, h=7, w=7, ci=256, co=48, padding=(2, 1, 0, 1)),
+          cases.make_conv_case("halo_c64_w224", 810, n=1, h=5, w=224, ci=64, co=64)]
+    for c in cs:
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        for tile in (0, 3000):
+            shim.set_option("igemm_tile", tile)
+            try:
+                got = _gpu_conv(c, shim.ALGO_MFMA)
+                kernel = shim.last_kernel()
+            finally:
+                shim.set_option("igemm_tile", 0)
+            # unforced, launches of fewer blocks than three quarters of the CUs stay on the implicit GEMM
+            assert tile == 0 or kernel.startswith("HaloConvKernel<"), kernel
+            np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} tile {tile} {kernel}")
+        print(f"{c.name}: {want.data.size} outputs, {kernel}", flush=True)
+    # 16 images of 56 x 56 make 224 blocks: the automatic choice
+    shim.conv2d(cs[0].x, cs[0].w, cs[0].b, cs[0].out_info, activation=cs[0].act[0], act_a=cs[0].act[1], act_b=cs[0].act[2], **cs[0].params)
+    assert shim.last_kernel().startswith("HaloConvKernel<"), shim.last_kernel()
+    # a forced implicit-GEMM tile keeps the same layers on the other kernels, which must agree as well
+    c = cs[0]
+    shim.set_option("igemm_tile", 128)
+    try:
+        got = _gpu_conv(c, shim.ALGO_MFMA)
+        assert not shim.last_kernel().startswith("HaloConvKernel<")
+    finally:
+        shim.set_option("igemm_tile", 0)
+    np.testing.assert_array_equal(got.data, _gpu_conv(c, shim.ALGO_DIRECT).data)
+
+
 def test_large_tile_gemm_gives_the_same_bytes():
     """The one-wave-per-SIMD kernel (256x256, 256x128 and 128x256 block tiles, accumulators in AGPRs) is chosen only for
     launches that fill the device; here each tiling is forced on small problems -- ragged rows and channels, padding,
