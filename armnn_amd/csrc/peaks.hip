@@ -33,6 +33,41 @@ __global__ __launch_bounds__(256) void MfmaPeakKernel(int iters, int* sink)
     if (t == 0x7fffffff) sink[0] = t;          // keeps the chains alive; practically never taken
 }
 
+// The same chains with operands whose bytes are either all small (as above) or spread over the whole int8 range, and
+// with the shader clock read at both ends: the matrix cores' power draw depends on how many operand bits toggle, and the
+// clock the device sustains follows it.  cyc[0] receives block 0's cycle count, cyc[1] its 100 MHz wall-clock ticks.
+__global__ __launch_bounds__(256) void MfmaDataKernel(int iters, int spread, int* sink, long long* cyc)
+{
+    const int lane = threadIdx.x;
+    const unsigned h = (static_cast<unsigned>(lane) + 1u) * 2654435761u;
+    v4i a = {lane, lane + 1, lane + 2, lane + 3};
+    v4i b = {lane ^ 5, lane ^ 9, lane ^ 17, lane ^ 33};
+    if (spread)
+    {
+        a = v4i{static_cast<int>(h), static_cast<int>(h * 40503u + 7u), static_cast<int>(h ^ 0x9e3779b9u), static_cast<int>(h * 2246822519u)};
+        b = v4i{static_cast<int>(h * 3266489917u), static_cast<int>(~h), static_cast<int>(h * 668265263u + 1u), static_cast<int>(h ^ 0x85ebca6bu)};
+    }
+    v16i c0 = {0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0, 0}, c1 = c0, c2 = c0, c3 = c0;
+    const long long t0 = __builtin_readcyclecounter(), w0 = wall_clock64();
+    for (int i = 0; i < iters; ++i)
+    {
+        c0 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c0, 0, 0, 0);
+        c1 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c1, 0, 0, 0);
+        c2 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c2, 0, 0, 0);
+        c3 = __builtin_amdgcn_mfma_i32_32x32x32_i8(a, b, c3, 0, 0, 0);
+    }
+    const v16i s = c0 + c1 + c2 + c3;
+    int t = 0;
+#pragma unroll
+    for (int i = 0; i < 16; ++i) t += s[i];
+    if (t == 0x7fffffff) sink[0] = t;
+    if (blockIdx.x == 0 && threadIdx.x == 0)
+    {
+        cyc[0] = __builtin_readcyclecounter() - t0;
+        cyc[1] = wall_clock64() - w0;
+    }
+}
+
 // four 16-byte loads in flight per thread, non-temporal both ways (the fastest of the variants tried on this device)
 // ops per wave and iteration: 8 MFMAs x 32*32*32 MACs x 2; 6 ds_read_b128 per iteration
 __global__ __launch_bounds__(256) void MfmaLdsFedKernel(int iters, int* sink)
@@ -139,6 +174,43 @@ int mi355x_peak_mfma_i8(int waves_per_simd, double* ops_per_s)
         else *ops_per_s = static_cast<double>(grid.x) * 4.0 * iters * 4.0 * 65536.0 / (ms * 1e-3);
     }
     (void)hipFree(sink);
+    return rc;
+}
+
+// Register-only int8 MFMA rate in ops/s, one wave per SIMD, with small operand bytes (spread = 0) or operand bytes over
+// the whole range (spread = 1), and the shader clock in GHz that block 0 saw meanwhile.
+int mi355x_peak_mfma_i8_data(int spread, double* ops_per_s, double* clock_ghz)
+{
+    if (!ops_per_s || !clock_ghz) return 1;
+    int dev = 0, n_cu = 0;
+    if (hipGetDevice(&dev) != hipSuccess) return 2;
+    if (hipDeviceGetAttribute(&n_cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 2;
+    int* sink = nullptr;
+    long long* cyc = nullptr;
+    if (hipMalloc(&sink, 64) != hipSuccess) return 2;
+    if (hipMalloc(&cyc, 16) != hipSuccess) { (void)hipFree(sink); return 2; }
+    Events ev;
+    const int iters = 40000;
+    const dim3 grid(static_cast<unsigned>(n_cu));
+    int rc = ev.ok ? 0 : 2;
+    if (rc == 0)
+    {
+        hipLaunchKernelGGL(MfmaDataKernel, grid, dim3(256), 0, nullptr, 4000, spread, sink, cyc);      // warm-up
+        (void)hipEventRecord(ev.e0, nullptr);
+        hipLaunchKernelGGL(MfmaDataKernel, grid, dim3(256), 0, nullptr, iters, spread, sink, cyc);
+        (void)hipEventRecord(ev.e1, nullptr);
+        float ms = 0.0f;
+        long long host[2] = {0, 0};
+        if (hipEventSynchronize(ev.e1) != hipSuccess || hipEventElapsedTime(&ms, ev.e0, ev.e1) != hipSuccess || ms <= 0.0f ||
+            hipMemcpy(host, cyc, sizeof(host), hipMemcpyDeviceToHost) != hipSuccess || host[1] <= 0) rc = 2;
+        else
+        {
+            *ops_per_s = static_cast<double>(grid.x) * 4.0 * iters * 4.0 * 65536.0 / (ms * 1e-3);
+            *clock_ghz = static_cast<double>(host[0]) / (static_cast<double>(host[1]) * 10.0);      // cycles per 10 ns tick
+        }
+    }
+    (void)hipFree(sink);
+    (void)hipFree(cyc);
     return rc;
 }
 

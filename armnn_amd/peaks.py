@@ -25,6 +25,15 @@ def measure(copy_bytes: int = 1 << 30) -> dict:
             raise RuntimeError(f"mi355x_peak_mfma_i8 failed ({rc})")
         best = max(best, v.value)
     out["mfma_i8_TOPs"] = best / 1e12
+    # register-only chains again, with small and with full-range operand bytes, and the clock the device held meanwhile
+    lib.mi355x_peak_mfma_i8_data.argtypes = [C.c_int, C.POINTER(C.c_double), C.POINTER(C.c_double)]
+    for spread, key in ((0, "small_operands"), (1, "full_range_operands")):
+        v, g = C.c_double(), C.c_double()
+        rc = lib.mi355x_peak_mfma_i8_data(spread, C.byref(v), C.byref(g))
+        if rc != 0:
+            raise RuntimeError(f"mi355x_peak_mfma_i8_data failed ({rc})")
+        out[f"mfma_i8_{key}_TOPs"] = v.value / 1e12
+        out[f"mfma_i8_{key}_clock_GHz"] = g.value
     lib.mi355x_peak_mfma_i8_lds_fed.argtypes = [C.POINTER(C.c_double)]
     v = C.c_double()
     rc = lib.mi355x_peak_mfma_i8_lds_fed(C.byref(v))
