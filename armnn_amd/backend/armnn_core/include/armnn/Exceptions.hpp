@@ -50,5 +50,6 @@ ARMNN_CORE_EXCEPTION(LayerValidationException, InvalidArgumentException);
 ARMNN_CORE_EXCEPTION(GraphValidationException, Exception);
 ARMNN_CORE_EXCEPTION(BadOptionalAccessException, Exception);
 ARMNN_CORE_EXCEPTION(FileNotFoundException, Exception);
+ARMNN_CORE_EXCEPTION(ParseException, Exception);
 #undef ARMNN_CORE_EXCEPTION
 } // namespace armnn
