@@ -1,11 +1,12 @@
 // Throughput of a network through the backend, the way an Arm NN application runs it:
 //   INetwork -> Optimize({"Mi355x"}) -> IRuntime::LoadNetwork -> IRuntime::EnqueueWorkload, host buffers in and out.
 // Usage:
-//   backend_bench <network file> <input bytes file> <output bytes file> [steps] [warmup]
+//   backend_bench <network file> <input bytes file> <output bytes file> [steps] [warmup] [backends, default Mi355x]
 // The network file comes from armnn_amd/netfile.py.  Prints one JSON line: milliseconds per EnqueueWorkload with
 // pageable host buffers (two host copies and the staging transfers) and with adopted pinned buffers (ImportInputs /
 // ImportOutputs, one transfer each way), the layer counts of the optimized graph, and whether both runs gave the same
-// bytes.  The output of the last run is written to the output file for the caller to compare.
+// bytes.  The output of the last run is written to the output file for the caller to compare.  With a backend list that
+// does not name Mi355x (CpuRef on the reference's runtime: the CPU baseline) only the pageable figure is measured.
 // Builds against this repository's host core and, unchanged, against an Arm NN source tree and its libarmnn.so (then
 // together with RealGraphAccess.cpp, which supplies the test utilities' GetGraphForTesting).
 #include <armnn/ArmNN.hpp>
@@ -19,6 +20,7 @@
 #include <cstring>
 #include <fstream>
 #include <iterator>
+#include <sstream>
 
 #include "NetFile.hpp"
 
@@ -43,6 +45,7 @@ int main(int argc, char** argv)
     }
     const int steps = argc > 4 ? std::atoi(argv[4]) : 200;
     const int warmup = argc > 5 ? std::atoi(argv[5]) : 10;
+    const std::string backendList = argc > 6 ? argv[6] : "Mi355x";
     try
     {
         const netfile::Net nf = netfile::Read(argv[1]);
@@ -55,7 +58,11 @@ int main(int argc, char** argv)
         ConfigureLogging(true, false, LogSeverity::Error);
         IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
         INetworkPtr net = netfile::Build(nf);
-        IOptimizedNetworkPtr opt = Optimize(*net, {BackendId("Mi355x")}, rt->GetDeviceSpec());
+        std::vector<BackendId> backends;
+        std::stringstream list(backendList);
+        for (std::string b; std::getline(list, b, ',');) backends.emplace_back(b);
+        const bool onDevice = backendList.find("Mi355x") != std::string::npos;
+        IOptimizedNetworkPtr opt = Optimize(*net, backends, rt->GetDeviceSpec());
         const Graph& og = GetGraphForTesting(opt.get());
         const size_t nLayers = og.GetNumLayers(), nAct = Count(og, LayerType::Activation), nCopy = Count(og, LayerType::MemCopy),
                      nConv = Count(og, LayerType::Convolution2d), nDw = Count(og, LayerType::DepthwiseConvolution2d),
@@ -76,6 +83,15 @@ int main(int argc, char** argv)
             if (rt->EnqueueWorkload(id, ins, outs) != Status::Success) throw std::runtime_error("EnqueueWorkload failed");
         const double msPageable = 1e3 * std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() / steps;
 
+        if (!onDevice)
+        {
+            std::ofstream fout(argv[3], std::ios::binary);
+            fout.write(reinterpret_cast<const char*>(pageable.data()), static_cast<std::streamsize>(pageable.size()));
+            rt->UnloadNetwork(id);
+            std::printf("{\"batch\": %u, \"steps\": %d, \"backends\": \"%s\", \"ms_pageable\": %.4f, \"optimized_layers\": %zu}\n", nf.batch, steps,
+                        backendList.c_str(), msPageable, nLayers);
+            return 0;
+        }
         void *pin = nullptr, *pout = nullptr;
         if (mi355x_host_alloc(&pin, input.size()) != 0 || mi355x_host_alloc(&pout, pageable.size()) != 0) throw std::runtime_error(mi355x_last_error());
         std::memcpy(pin, input.data(), input.size());

@@ -19,8 +19,9 @@ Extra objects in the line:
                 host buffers in and out: pageable, and pinned buffers adopted with ImportInputs / ImportOutputs); its output
                 bytes are compared with the executor's
   groups        conv/FC ops vs the int8 MFMA peak and depthwise bytes vs the HBM peak over the whole net
-  cpu_baseline  the reference's own CpuRef code (oracle/_ref, kind "reference") or the C restatement
-                (kind "port"), one thread, on a bounded sample of the same workload
+  cpu_baseline  the reference's CpuRef backend behind its own runtime where that build is there, else the reference's own
+                CpuRef functions (oracle/_ref) -- both kind "reference" -- or the C restatement (kind "port"); one thread, on a
+                bounded sample of the same workload
 """
 from __future__ import annotations
 
@@ -89,7 +90,44 @@ def algorithmic_bytes(net, l, batch):
     return n
 
 
+def cpu_baseline_reference_runtime(net, seconds_budget=25.0):
+    """The same network at batch 1 through IRuntime::EnqueueWorkload on the reference's own CpuRef backend: backend_bench
+    built against the reference's source tree and the libarmnn.so made from it (armnn_amd/backend/test/bin/real/).  None
+    when that build is not there."""
+    import subprocess
+    import tempfile
+    import numpy as np
+    from armnn_amd import netfile, nets
+    exe = os.path.join(ROOT, "armnn_amd", "backend", "test", "bin", "real", "backend_bench")
+    if not os.path.exists(exe):
+        return None
+    with tempfile.TemporaryDirectory(prefix="mi355x_cpuref_") as tmp:
+        nf, fin, fout = (os.path.join(tmp, n) for n in ("net.bin", "input.bin", "output.bin"))
+        netfile.write_net(net, 1, nf)
+        np.ascontiguousarray(nets.synthetic_input(net, 1, seed=100).data).tofile(fin)
+        images, elapsed = 0, 0.0
+        steps = 1
+        while True:
+            try:
+                r = subprocess.run([exe, nf, fin, fout, str(steps), "0", "CpuRef"], capture_output=True, text=True, timeout=600)
+            except subprocess.TimeoutExpired:
+                return None
+            if r.returncode != 0:
+                return None
+            ms = json.loads(r.stdout.strip().splitlines()[-1])["ms_pageable"]
+            images += steps
+            elapsed += steps * ms * 1e-3
+            if elapsed * (images + steps) / images > seconds_budget or images >= 8:
+                break
+    return {"value": images / elapsed, "unit": "images/sec", "cores": 1, "kind": "reference",
+            "sample": f"{images} image(s) of the same network at batch 1 through IRuntime::EnqueueWorkload on the reference's CpuRef backend "
+                      f"(libarmnn.so built from the reference), {elapsed:.1f} s, single-threaded backend on one of {os.cpu_count()} cores"}
+
+
 def cpu_baseline(net, seconds_budget=25.0):
+    real = cpu_baseline_reference_runtime(net, seconds_budget)
+    if real is not None:
+        return real
     from oracle import cpuref, netref
     from armnn_amd import nets
     kind = "reference" if cpuref.have("reference") else "port"
