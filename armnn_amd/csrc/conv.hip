@@ -4,6 +4,7 @@
 #include "conv_kernels.h"
 #include "dw_stem_kernels.h"
 #include "dwpw_kernel.h"
+#include "pwdw_kernel.h"
 #include "pw_gemm_kernel.h"
 #include "igemm_lds_kernel.h"
 #include "big_gemm.h"
@@ -1096,6 +1097,85 @@ int LaunchDwPw(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, uint32_t ba
     MI355X_HIP(hipGetLastError());
     return 0;
 }
+
+// ---- pointwise 1x1 followed by depthwise 3x3, whole images per block ---------------------------------------------------
+constexpr int kPwDwMF = 7;       // 224 pixel rows per block: one 14x14 image, four 7x7 images
+// Two LDS stages and eight waves: with a K of 256 .. 512 bytes the k-loop is bound by what a CU's vector L1 delivers, not
+// by round trips (four stages measured 4 % slower), and the requantization and depthwise phases, which are pure VALU
+// issue, want two waves per SIMD (four waves: 16.1 us against 12.3 us for 32 images of 14 x 14 x 512).
+constexpr int kPwDwStages = 2, kPwDwWaves = 8;
+
+
+struct PwDwShape
+{
+    int G = 0, HR = 0, HC = 0, pairs = 0, S = 0;
+};
+
+// 0 when the pair (1x1 convolution, 3x3 depthwise) can run as PwDwKernel; the shape the launch needs comes back in `sh`
+int PwDwCheck(const mi355x_conv2d_s* pw, const mi355x_conv2d_s* dw, PwDwShape* sh)
+{
+    const mi355x_conv2d_desc& a = pw->d;
+    const mi355x_conv2d_desc& b = dw->d;
+    const bool pointwise = pw->algo == MI355X_ALGO_MFMA && !a.depthwise && a.kernel_h == 1 && a.kernel_w == 1 && a.stride_x == 1 &&
+                           a.stride_y == 1 && a.pad_top == 0 && a.pad_left == 0 && a.out_h == a.in_h && a.out_w == a.in_w;
+    if (!pointwise) return SetError(MI355X_ERR_UNSUPPORTED, "first plan is not an unpadded 1x1 stride-1 convolution on the MFMA kernel");
+    if (pw->zw_neg != 0) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel needs pointwise weights without a zero point");
+    if ((a.in_c % 128) != 0 || pw->K_pad != static_cast<int>(a.in_c))     // rows are fetched 128 bytes at a time: none may end inside a tile
+        return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel needs the pointwise layer's input channels in whole 128-byte k-tiles");
+    if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || !dw->dw_grp || dw->w_dot4b)
+        return SetError(MI355X_ERR_UNSUPPORTED, "second plan is not a 3x3 depthwise layer on the v_dot4 kernel");
+    if (b.stride_x != b.stride_y || (b.stride_x != 1 && b.stride_x != 2))
+        return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel needs depthwise stride 1 or 2");
+    if (a.out_c != b.in_c || a.out_h != b.in_h || a.out_w != b.in_w) return SetError(MI355X_ERR_INVALID_ARGUMENT, "the layers' shapes do not chain");
+    if (a.output.dtype != b.input.dtype || a.output.scale != b.input.scale || a.output.offset != b.input.offset)
+        return SetError(MI355X_ERR_INVALID_ARGUMENT, "the first layer's output quantization is not the second layer's input quantization");
+    if ((a.out_c % kPwDwBN) != 0 || b.out_c != a.out_c) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel needs channels %% 64 == 0 and depth multiplier 1");
+    const int hw = static_cast<int>(a.out_h) * static_cast<int>(a.out_w);
+    if (hw > kPwDwMF * 32) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel holds whole images: %d pixels exceed %d", hw, kPwDwMF * 32);
+    PwDwShape s;
+    s.S = static_cast<int>(b.stride_x);
+    s.G = kPwDwMF * 32 / hw;
+    s.pairs = (static_cast<int>(b.out_w) + 1) / 2;
+    s.HR = (static_cast<int>(b.out_h) - 1) * s.S + 3;
+    s.HC = 2 * s.S * s.pairs + 2;
+    // the padded intermediate tile reuses the GEMM's stages: tiny images take fewer per block than the rows would allow
+    s.G = std::min(s.G, PwDwStageBytes<kPwDwMF, kPwDwStages>() / (s.HR * s.HC * kPwDwPitch));
+    if (s.G < 1) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel: the intermediate tile does not fit LDS");
+    if (sh) *sh = s;
+    return 0;
+}
+
+template <int S>
+int LaunchPwDwT(const PwDwArgs& a, hipStream_t stream)
+{
+    constexpr int smem = PwDwStageBytes<kPwDwMF, kPwDwStages>();
+    static_assert(smem <= 160 * 1024, "LDS of one CU");
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwDwKernel<kPwDwMF, kPwDwStages, S, kPwDwWaves>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    MI355X_HIP(attr);
+    NoteKernel("PwDwKernel<%d, %d, %d, %d>", kPwDwMF, kPwDwStages, S, kPwDwWaves);
+    hipLaunchKernelGGL((PwDwKernel<kPwDwMF, kPwDwStages, S, kPwDwWaves>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(64 * kPwDwWaves), smem,
+                       stream, a);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+int LaunchPwDw(const mi355x_conv2d_s* pw, const mi355x_conv2d_s* dw, const PwDwShape& sh, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    PwDwArgs a;
+    a.x = static_cast<const uint8_t*>(x); a.w = pw->w_mfma; a.K_pad = pw->K_pad; a.pw_ct = ChanTab{pw->chan, pw->Co_pad}; a.pw_corr = pw->corr;
+    a.pw_xor = pw->xor_mask; a.pw_rq = pw->rq;
+    a.N = static_cast<int>(batch); a.H = pw->geom.Ho; a.W = pw->geom.Wo; a.Ci = pw->geom.Ci; a.C = pw->geom.Co;
+    a.G = sh.G; a.tiles_n = a.C / kPwDwBN;
+    const long long nb = (static_cast<long long>(batch) + sh.G - 1) / sh.G * a.tiles_n;
+    if (nb > 0x7fffffffll - 8) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
+    a.total_blocks = static_cast<int>(nb); a.xcd_chunk = static_cast<int>((nb + 7) / 8);
+    a.dw_grp = dw->dw_grp; a.dw_ct = ChanTab{dw->chan, dw->Co_pad}; a.dw_rq = dw->rq; a.dw_xor = dw->xor_mask; a.dw_pad = dw->pad_word;
+    a.Ho = dw->geom.Ho; a.Wo = dw->geom.Wo; a.pad_top = dw->geom.pad_top; a.pad_left = dw->geom.pad_left;
+    a.HR = sh.HR; a.HC = sh.HC; a.pairs = sh.pairs;
+    a.y = static_cast<uint8_t*>(y);
+    return sh.S == 1 ? LaunchPwDwT<1>(a, stream) : LaunchPwDwT<2>(a, stream);
+}
 } // namespace
 
 extern "C" {
@@ -1120,6 +1200,8 @@ int mi355x_conv2d_run(mi355x_conv2d_t plan, uint32_t batch, const void* input_de
 int mi355x_conv2d_fusable(mi355x_conv2d_t dw, mi355x_conv2d_t pw)
 {
     if (!dw || !pw) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
+    // the other order -- 1x1 convolution first, depthwise second -- is the whole-image kernel
+    if (!dw->d.depthwise && pw->d.depthwise) return PwDwCheck(dw, pw, nullptr);
     const mi355x_conv2d_desc& a = dw->d;
     const mi355x_conv2d_desc& b = pw->d;
     if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || !dw->dw_grp || dw->w_dot4b || (dw->d.out_c % 32) != 0)
@@ -1146,6 +1228,12 @@ int mi355x_conv2d_run_fused(mi355x_conv2d_t dw, mi355x_conv2d_t pw, uint32_t bat
     if (!input_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "input / output pointer is null");
     if ((reinterpret_cast<uintptr_t>(input_dev) & 15) != 0 || (reinterpret_cast<uintptr_t>(output_dev) & 15) != 0)
         return SetError(MI355X_ERR_INVALID_ARGUMENT, "fused kernel needs 16-byte aligned tensors");
+    if (!dw->d.depthwise && pw->d.depthwise)
+    {
+        PwDwShape sh;
+        if (int rc = PwDwCheck(dw, pw, &sh)) return rc;
+        return LaunchPwDw(dw, pw, sh, batch, input_dev, output_dev, ToHip(stream));
+    }
     if (dw->d.stride_x == 2) return LaunchDwPw<2, 2>(dw, pw, batch, input_dev, output_dev, ToHip(stream));
     // stride 1: the wide tile (8 x 16 pixels) while it still yields two blocks per CU, else the narrow one (8 x 8)
     const long long wide = static_cast<long long>(batch) * ((dw->d.out_w + 15) / 16) * ((dw->d.out_h + 7) / 8);

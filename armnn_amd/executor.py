@@ -15,9 +15,10 @@ from .tensor import QTensor, numpy_dtype
 
 @dataclass
 class FusedPair:
-    """A depthwise layer and the pointwise convolution consuming it, launched as one kernel."""
+    """Two neighbouring layers -- depthwise + the pointwise convolution consuming it, or pointwise + the depthwise
+    consuming it -- launched as one kernel."""
     name: str
-    parts: Tuple                       # (depthwise Layer, pointwise Layer)
+    parts: Tuple                       # (first Layer, second Layer)
     op: str = "dwpw"
 
     @property
@@ -114,11 +115,12 @@ class DeviceNetwork:
             else:
                 raise ValueError(l.op)
         if fuse:
-            self._fuse_depthwise_pointwise()
+            self._fuse_pairs(("conv", "depthwise") if fuse == "pwdw" else ("depthwise", "conv"))
 
-    def _fuse_depthwise_pointwise(self):
-        """Replace (depthwise 3x3, 1x1 convolution) neighbours by one fused launch where the library accepts the pair
-        and nothing else reads the tensor between them."""
+    def _fuse_pairs(self, ops):
+        """Replace neighbours (depthwise 3x3, 1x1 convolution) -- or, with ops = ("conv", "depthwise"), (1x1 convolution,
+        depthwise 3x3) -- by one fused launch where the library accepts the pair and nothing else reads the tensor
+        between them."""
         net = self.net
         consumers: Dict[str, int] = {}
         for l in net.layers:
@@ -129,7 +131,7 @@ class DeviceNetwork:
         while k < len(self.steps):
             l, fn = self.steps[k]
             nxt = self.steps[k + 1][0] if k + 1 < len(self.steps) else None
-            if (l.op == "depthwise" and nxt is not None and nxt.op == "conv" and nxt.inputs[0] == l.output and
+            if (l.op == ops[0] and nxt is not None and nxt.op == ops[1] and nxt.inputs[0] == l.output and
                     consumers.get(l.output, 0) == 1 and l.output != net.output and
                     plan_of[id(l)].fusable_with(plan_of[id(nxt)])):
                 pdw, ppw = plan_of[id(l)], plan_of[id(nxt)]

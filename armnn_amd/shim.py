@@ -297,13 +297,14 @@ class Conv2dPlan:
     def run(self, batch: int, x_dev: int, y_dev: int, stream=None):
         _chk(self.lib.mi355x_conv2d_run(self.plan, batch, x_dev, y_dev, stream))
 
-    def fusable_with(self, pointwise: "Conv2dPlan") -> bool:
-        """True when this 3x3 depthwise plan and `pointwise` (the 1x1 convolution consuming it) can run as one kernel."""
-        return self.lib.mi355x_conv2d_fusable(self.plan, pointwise.plan) == 0
+    def fusable_with(self, second: "Conv2dPlan") -> bool:
+        """True when this plan and `second`, the layer consuming its output, can run as one kernel: 3x3 depthwise + 1x1
+        convolution, or 1x1 convolution + 3x3 depthwise over images of at most 224 pixels."""
+        return self.lib.mi355x_conv2d_fusable(self.plan, second.plan) == 0
 
-    def run_fused(self, pointwise: "Conv2dPlan", batch: int, x_dev: int, y_dev: int, stream=None):
-        """depthwise -> pointwise without the intermediate tensor; bytes equal run() + pointwise.run()."""
-        _chk(self.lib.mi355x_conv2d_run_fused(self.plan, pointwise.plan, batch, x_dev, y_dev, stream))
+    def run_fused(self, second: "Conv2dPlan", batch: int, x_dev: int, y_dev: int, stream=None):
+        """Both layers without the intermediate tensor; bytes equal run() + second.run()."""
+        _chk(self.lib.mi355x_conv2d_run_fused(self.plan, second.plan, batch, x_dev, y_dev, stream))
 
     def destroy(self):
         if self.plan:

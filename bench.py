@@ -67,11 +67,12 @@ def layer_work(net, l, batch):
     if l.op in ("conv", "fc"):
         return "mfma", 2.0 * l.macs_per_image * batch
     if l.op == "dwpw":
-        # fused depthwise + pointwise: the tensor between them never exists, so the unit's algorithmic bytes are its
-        # input, its output and both layers' constants; priced against HBM like the depthwise layer it absorbs
-        dw, pw = l.parts
-        nbytes = (net.tensors[dw.inputs[0]].num_elements + net.tensors[pw.output].num_elements) * batch
-        for part in (dw, pw):
+        # two layers fused (depthwise + pointwise, in either order): the tensor between them never exists, so the unit's
+        # algorithmic bytes are its input, its output and both layers' constants; priced against HBM like the depthwise
+        # layer it absorbs
+        first, second = l.parts
+        nbytes = (net.tensors[first.inputs[0]].num_elements + net.tensors[second.output].num_elements) * batch
+        for part in (first, second):
             nbytes += part.weights.info.num_elements + 8 * net.tensors[part.output].shape[-1]
         return "hbm", float(nbytes)
     nbytes = sum(net.tensors[i].num_elements for i in l.inputs) + net.tensors[l.output].num_elements
@@ -188,8 +189,9 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-backend", action="store_true", help="skip the run through the C++ backend (config.backend_path)")
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--fuse", action="store_true",
-                    help="run depthwise + pointwise pairs as one kernel (same bytes; slower than two launches at present)")
+    ap.add_argument("--fuse", nargs="?", const="dwpw", default="", choices=("dwpw", "pwdw"),
+                    help="run pairs of layers as one kernel (same bytes): 'dwpw' depthwise + the pointwise after it, 'pwdw' "
+                         "pointwise + the depthwise after it where whole images fit a block")
     ap.add_argument("--lanes", type=int, default=2,
                     help="split the batch into this many slices, each running the network on a stream of its own")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
@@ -336,7 +338,7 @@ def main():
     config = {"workload": f"{net.name} int8 (QAsymm activations, {'per-channel QSymmS8' if args.weights == 'per_channel_s8' or args.net != 'mobilenet_v1' else 'per-tensor QAsymmU8'} weights), batch {batch}, "
                           f"random-init, whole forward pass incl. avgpool/FC/softmax, input resident in HBM, every layer through the C ABI, "
                           f"one HIP graph replay per step",
-              "batch": batch, "graph_replay": not args.no_graph, "fused_depthwise_pointwise": args.fuse, "lanes": args.lanes,
+              "batch": batch, "graph_replay": not args.no_graph, "fused_pairs": args.fuse or None, "lanes": args.lanes,
               "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12}
     if backend is not None:
         # the same network and input through the C++ backend: wall clock per IRuntime::EnqueueWorkload call, host buffers in

@@ -201,9 +201,14 @@ int mi355x_conv2d_destroy(mi355x_conv2d_t plan);
  * (RefDepthwiseConvolution2dWorkload.cpp:38-62, then RefConvolution2dWorkload.cpp:38-58).
  * mi355x_conv2d_fusable returns 0 when the pair qualifies (3x3 depthwise with channels % 32 == 0, multiplier 1,
  * stride 1 or 2; pointwise with output channels % 64 == 0; chaining shapes and identical quantization of the shared
- * tensor), else MI355X_ERR_UNSUPPORTED / MI355X_ERR_INVALID_ARGUMENT with the reason in mi355x_last_error(). */
-int mi355x_conv2d_fusable(mi355x_conv2d_t depthwise, mi355x_conv2d_t pointwise);
-int mi355x_conv2d_run_fused(mi355x_conv2d_t depthwise, mi355x_conv2d_t pointwise, uint32_t batch,
+ * tensor), else MI355X_ERR_UNSUPPORTED / MI355X_ERR_INVALID_ARGUMENT with the reason in mi355x_last_error().
+ * The other order is accepted as well: first = the unpadded 1x1 stride-1 Convolution2d, second = the 3x3 depthwise layer
+ * that consumes it (stride 1 or 2, multiplier 1).  A block then computes whole images of the intermediate tensor for 64
+ * of its channels, keeps them on chip and runs the depthwise filter there; it qualifies when one image has at most 224
+ * pixels (14 x 14, 7 x 7 ...), the 1x1 layer's input channels are a multiple of 128, its weights have no zero point and
+ * the shared channel count is a multiple of 64.  Same contract: the bytes of the two layers run one after the other. */
+int mi355x_conv2d_fusable(mi355x_conv2d_t first, mi355x_conv2d_t second);
+int mi355x_conv2d_run_fused(mi355x_conv2d_t first, mi355x_conv2d_t second, uint32_t batch,
                             const void* input_dev, void* output_dev, mi355x_stream_t stream);
 /* which kernel a plan resolved to (mi355x_algo) and its tile configuration, for logs and tests */
 int mi355x_conv2d_algo(mi355x_conv2d_t plan, int32_t* algo, char* desc_buf, size_t desc_len);

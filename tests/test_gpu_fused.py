@@ -1,5 +1,6 @@
-"""Depthwise 3x3 + pointwise 1x1 as one kernel: bytes must equal the two layers run one after the other, and the pair
-must stay within 1 LSB of the oracle per layer (the second layer judged on the first layer's actual output)."""
+"""Depthwise 3x3 + pointwise 1x1 as one kernel, and pointwise 1x1 + the depthwise 3x3 after it as one kernel: bytes must
+equal the two layers run one after the other, and the pair must stay within 1 LSB of the oracle per layer (the second
+layer judged on the first layer's actual output)."""
 import numpy as np
 import pytest
 
@@ -96,3 +97,90 @@ def test_unfusable_pairs_are_refused():
         xd = shim.DeviceBuffer(dw.x.data.nbytes).upload(dw.x.data)
         yd = shim.DeviceBuffer(c3.out_info.num_elements)
         pdw.run_fused(_plan(c3), 1, xd.ptr, yd.ptr)
+
+
+# ---- the other order: 1x1 convolution, then the 3x3 depthwise that consumes it, whole images per block ------------------
+# (name, n, h, w, ci, c, depthwise stride, dtype, act after pw, act after dw)
+PW_DW = [
+    ("14x14_k512_c512_s1_s8", 3, 14, 14, 512, 512, 1, S8, cases.RELU6, cases.RELU6),
+    ("14x14_k256_c128_s2_u8", 2, 14, 14, 256, 128, 2, U8, cases.RELU6, cases.RELU),
+    ("7x7_k512_c128_s1_s8_last_block_has_one_image", 5, 7, 7, 512, 128, 1, S8, cases.RELU6, cases.RELU6),
+    ("7x7_k128_c64_s1_u8_four_images_one_block", 4, 7, 7, 128, 64, 1, U8, (0, 0.0, 0.0), cases.RELU6),
+    ("9x11_k128_c64_s2_s8_odd_sizes", 2, 9, 11, 128, 64, 2, S8, cases.RELU, (0, 0.0, 0.0)),
+    ("6x5_k384_c192_s1_u8", 7, 6, 5, 384, 192, 1, U8, cases.RELU6, cases.RELU6),
+    ("1x1_k128_c64_s1_s8", 9, 1, 1, 128, 64, 1, S8, cases.RELU6, cases.RELU6),
+    ("14x16_k128_c64_s1_s8_exactly_224_rows", 2, 14, 16, 128, 64, 1, S8, cases.RELU6, cases.RELU6),
+]
+
+
+def _make_pw_dw(name, n, h, w, ci, c, stride, dt, act_pw, act_dw):
+    zp_in = 3 if dt == U8 else -128
+    zp_mid = 7 if dt == U8 else -121
+    pw = cases.make_conv_case(name + "_pw", 700 + ci, n=n, h=h, w=w, ci=ci, co=c, kh=1, kw=1, in_dtype=dt, in_scale=0.0235,
+                              in_offset=zp_in, out_scale=0.04, out_offset=zp_mid, act=act_pw)
+    dw = cases.make_conv_case(name + "_dw", 701 + c, n=n, h=h, w=w, ci=c, depthwise=True, stride=(stride, stride), in_dtype=dt,
+                              in_scale=0.04, in_offset=zp_mid, out_scale=0.0235, out_offset=zp_in, act=act_dw,
+                              w_scale_range=(0.01, 0.05))
+    return pw, dw
+
+
+@pytest.mark.parametrize("pair", PW_DW, ids=[p[0] for p in PW_DW])
+def test_pointwise_then_depthwise_fused_equals_two_layers(port, pair):
+    print("pair", pair, flush=True)
+    shim.Device()
+    pw, dw = _make_pw_dw(*pair)
+    ppw, pdw = _plan(pw), _plan(dw)
+    assert ppw.fusable_with(pdw), shim.load_library().mi355x_last_error().decode()
+    n = pw.x.info.shape[0]
+    xd = shim.DeviceBuffer(pw.x.data.nbytes).upload(pw.x.data)
+    mid = shim.DeviceBuffer(pw.out_info.num_elements)
+    y2 = shim.DeviceBuffer(dw.out_info.num_elements)
+    yf = shim.DeviceBuffer(dw.out_info.num_elements)
+    ppw.run(n, xd.ptr, mid.ptr)
+    pdw.run(n, mid.ptr, y2.ptr)
+    ppw.run_fused(pdw, n, xd.ptr, yf.ptr)
+    assert shim.last_kernel().startswith("PwDwKernel")
+    mid_h = mid.download(pw.out_info.shape, numpy_dtype(pw.out_info.dtype))
+    two = y2.download(dw.out_info.shape, numpy_dtype(dw.out_info.dtype))
+    fused = yf.download(dw.out_info.shape, numpy_dtype(dw.out_info.dtype))
+    np.testing.assert_array_equal(fused, two)
+    assert len(np.unique(fused)) > 8
+    # the padding the depthwise layer sees is its input zero point: border outputs against the oracle on the device's own
+    # intermediate tensor, like every other output
+    dw.x = QTensor(dw.x.info, mid_h)
+    fn, a, b = dw.act
+    want = port.conv2d(dw.x, dw.w, dw.b, dw.out_info, **dw.params)
+    if fn:
+        want = port.activation(want, dw.out_info, fn, a, b)
+    mx, exact = lsb_diff(fused, want.data)
+    print(f"  fused vs oracle on the device's intermediate: max|d|={mx} exact={exact:.5f}", flush=True)
+    assert mx <= 1 and exact >= 0.99
+    fn, a, b = pw.act
+    want_mid = port.conv2d(pw.x, pw.w, pw.b, pw.out_info, **pw.params)
+    if fn:
+        want_mid = port.activation(want_mid, pw.out_info, fn, a, b)
+    mx, exact = lsb_diff(mid_h, want_mid.data)
+    assert mx <= 1 and exact >= 0.99
+
+
+def test_pointwise_then_depthwise_pairs_outside_the_kernels_shape_are_refused():
+    shim.Device()
+    lib = shim.load_library()
+    # 15 x 15 = 225 pixels: one image no longer fits the block's 224 rows
+    pw, dw = _make_pw_dw("big", 1, 15, 15, 128, 64, 1, S8, cases.RELU6, cases.RELU6)
+    assert not _plan(pw).fusable_with(_plan(dw))
+    assert "whole images" in lib.mi355x_last_error().decode()
+    # 96 channels are not whole 64-channel blocks
+    pw, dw = _make_pw_dw("c96", 1, 7, 7, 128, 96, 1, S8, cases.RELU6, cases.RELU6)
+    assert not _plan(pw).fusable_with(_plan(dw))
+    # 64 input channels: no whole 128-byte k-tile
+    pw, dw = _make_pw_dw("k64", 1, 7, 7, 64, 64, 1, S8, cases.RELU6, cases.RELU6)
+    assert not _plan(pw).fusable_with(_plan(dw))
+    # the shared tensor's quantization differs
+    pw, dw = _make_pw_dw("q", 1, 7, 7, 128, 64, 1, S8, cases.RELU6, cases.RELU6)
+    other = cases.make_conv_case("q_dw2", 3, n=1, h=7, w=7, ci=64, depthwise=True, in_scale=0.05, in_offset=-121)
+    assert not _plan(pw).fusable_with(_plan(other))
+    with pytest.raises(shim.ShimError):
+        xd = shim.DeviceBuffer(pw.x.data.nbytes).upload(pw.x.data)
+        yd = shim.DeviceBuffer(other.out_info.num_elements)
+        _plan(pw).run_fused(_plan(other), 1, xd.ptr, yd.ptr)

@@ -39,6 +39,14 @@ def _layerwise(port, net, batch):
     df.close()
     print(f"{net.name} b{batch}: {n_fused} fused depthwise+pointwise pairs", flush=True)
     np.testing.assert_array_equal(fused.data, eager.data)
+    # pointwise + the depthwise after it as one kernel, where whole images fit a block (graph replay with two lanes too)
+    for kw in ({"use_graph": False}, {"use_graph": True, "lanes": 2 if batch % 2 == 0 else 1}):
+        df = DeviceNetwork(net, batch, fuse="pwdw", **kw)
+        n_fused = sum(1 for l, _ in df.steps if l.op == "dwpw")
+        fused = df.run(x)
+        df.close()
+        print(f"{net.name} b{batch}: {n_fused} fused pointwise+depthwise pairs {kw}", flush=True)
+        np.testing.assert_array_equal(fused.data, eager.data)
     dg = DeviceNetwork(net, batch, use_graph=True, fuse=False)
     g1 = dg.run(x)
     dg.enqueue()
