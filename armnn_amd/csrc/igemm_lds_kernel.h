@@ -171,34 +171,74 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
 #pragma unroll
     for (int tp = 0; tp < TP; ++tp) rowsum[tp] = 0;
 
+    // Fragment reads run ahead of the MFMAs that use them: a block that has a CU to itself has one wave per SIMD, and
+    // nothing else hides a ds_read's latency between dependent read -> MFMA pairs.  Small wave tiles fetch the whole
+    // k-tile's fragments first (32 VGPRs per fragment column); larger ones keep one k-step in flight.
+    constexpr int KS = BK / 32;
+    constexpr bool ALL_AHEAD = TP * TC <= 2;
     auto compute = [&](int stage) {
         const uint8_t* As = smem + stage * STAGE;
         const uint8_t* Bs = As + BM * BK;
-#pragma unroll
-        for (int ks = 0; ks < BK / 32; ++ks)
-        {
+        auto read_a = [&](int ks, int tp) {
             // chunk ks*2 + half of row r sits at slot chunk ^ ((r >> 1) & 7); fragment rows start at multiples of 32
             const int slot = ((ks * 2 + frag_half) ^ ((frag_row >> 1) & 7)) * 16;
-            v4i fa[TP], fw[TC];
-#pragma unroll
-            for (int tp = 0; tp < TP; ++tp)
+            v4i f = *reinterpret_cast<const v4i*>(As + (wm * WTM + tp * 32 + frag_row) * BK + slot);
+            if (U8) f ^= xm;
+            return f;
+        };
+        auto read_w = [&](int ks, int tc) {
+            const int slot = ((ks * 2 + frag_half) ^ ((frag_row >> 1) & 7)) * 16;
+            return *reinterpret_cast<const v4i*>(Bs + (wn * WTN + tc * 32 + frag_row) * BK + slot);
+        };
+        auto multiply = [&](const v4i (&fa)[TP], const v4i (&fw)[TC]) {
+            if constexpr (AW)
             {
-                fa[tp] = *reinterpret_cast<const v4i*>(As + (wm * WTM + tp * 32 + frag_row) * BK + slot);
-                if (U8) fa[tp] ^= xm;
-                if constexpr (AW)
-                {
+#pragma unroll
+                for (int tp = 0; tp < TP; ++tp)
 #pragma unroll
                     for (int i = 0; i < 4; ++i) rowsum[tp] = __builtin_amdgcn_sdot4(fa[tp][i], 0x01010101, rowsum[tp], false);
-                }
             }
-#pragma unroll
-            for (int tc = 0; tc < TC; ++tc)
-                fw[tc] = *reinterpret_cast<const v4i*>(Bs + (wn * WTN + tc * 32 + frag_row) * BK + slot);
 #pragma unroll
             for (int tc = 0; tc < TC; ++tc)
 #pragma unroll
                 for (int tp = 0; tp < TP; ++tp)
                     acc[tc][tp] = __builtin_amdgcn_mfma_i32_32x32x32_i8(fw[tc], fa[tp], acc[tc][tp], 0, 0, 0);
+        };
+        if constexpr (ALL_AHEAD)
+        {
+            v4i fa[KS][TP], fw[KS][TC];
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+            {
+#pragma unroll
+                for (int tp = 0; tp < TP; ++tp) fa[ks][tp] = read_a(ks, tp);
+#pragma unroll
+                for (int tc = 0; tc < TC; ++tc) fw[ks][tc] = read_w(ks, tc);
+            }
+            __builtin_amdgcn_sched_barrier(0);      // the scheduler would otherwise sink every read to just before its MFMA
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks) multiply(fa[ks], fw[ks]);
+        }
+        else
+        {
+            v4i fa[2][TP], fw[2][TC];
+#pragma unroll
+            for (int tp = 0; tp < TP; ++tp) fa[0][tp] = read_a(0, tp);
+#pragma unroll
+            for (int tc = 0; tc < TC; ++tc) fw[0][tc] = read_w(0, tc);
+#pragma unroll
+            for (int ks = 0; ks < KS; ++ks)
+            {
+                if (ks + 1 < KS)
+                {
+#pragma unroll
+                    for (int tp = 0; tp < TP; ++tp) fa[(ks + 1) & 1][tp] = read_a(ks + 1, tp);
+#pragma unroll
+                    for (int tc = 0; tc < TC; ++tc) fw[(ks + 1) & 1][tc] = read_w(ks + 1, tc);
+                }
+                __builtin_amdgcn_sched_barrier(0);  // keep the next k-step's reads ahead of this k-step's MFMAs
+                multiply(fa[ks & 1], fw[ks & 1]);
+            }
         }
     };
 

@@ -162,6 +162,43 @@ def test_every_igemm_tiling_gives_the_same_bytes():
         shim.set_option("igemm_tile", 100)
 
 
+def test_k_split_over_wave_groups_gives_the_same_bytes():
+    """Launches of at most one 64x64 block per CU with K >= 2048 split K over two or four groups of waves inside the
+    block (IgemmKSplitKernel).  Forced on small and ragged problems -- fewer k-tiles than groups, k-tile counts that do not
+    divide by the group count, channel counts that are no multiple of 16, uint8 activations, stride 2 -- and taken
+    automatically for the shapes it is meant for; every result against the direct kernel."""
+    U8 = DataType.QAsymmU8
+    cs = [cases.make_conv_case("ks_3x3_c512_7", 821, n=3, h=7, w=7, ci=512, co=128, act=cases.RELU6),                  # 36 k-tiles
+          cases.make_conv_case("ks_3x3_c256_14_u8", 822, n=2, h=14, w=14, ci=256, co=192, in_dtype=U8, in_offset=131, out_offset=-100),
+          cases.make_conv_case("ks_1x1_c1024", 823, n=5, h=7, w=5, ci=1024, co=100, kh=1, kw=1),                       # Co % 16 != 0
+          cases.make_conv_case("ks_3x3_c128_one_tile_per_tap", 824, n=1, h=9, w=9, ci=128, co=64, in_dtype=U8, in_offset=3),   # 9 k-tiles
+          cases.make_conv_case("ks_1x1_c384", 825, n=2, h=6, w=6, ci=384, co=64, kh=1, kw=1),                          # 3 k-tiles < 4 groups
+          cases.make_conv_case("ks_1x1_c128", 826, n=1, h=5, w=5, ci=128, co=70, kh=1, kw=1, in_dtype=U8, in_offset=200),     # 1 k-tile
+          cases.make_conv_case("ks_3x3_c640_s2", 827, n=4, h=13, w=14, ci=640, co=64, stride=(2, 2), act=cases.RELU)]
+    for c in cs:
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        for tile in (2064, 4064):
+            shim.set_option("igemm_tile", tile)
+            try:
+                got = _gpu_conv(c, shim.ALGO_MFMA)
+                kernel = shim.last_kernel()
+            finally:
+                shim.set_option("igemm_tile", 0)
+            print(f"{c.name} tile {tile}: {got.data.size} outputs, {kernel}", flush=True)
+            assert kernel.startswith("IgemmKSplitKernel<%d" % (tile // 1000)), kernel
+            np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} tile {tile}")
+    # the automatic choice: ResNet-50's 3x3 layers of the last two stages at 16 images, FullyConnected-like 1x1 with K = 2048
+    auto = [(cases.make_conv_case("ks_auto_7x7_c512", 831, n=16, h=7, w=7, ci=512, co=512, act=cases.RELU), 4),
+            (cases.make_conv_case("ks_auto_14x14_c256", 832, n=16, h=14, w=14, ci=256, co=256, act=cases.RELU), 2),
+            (cases.make_conv_case("ks_auto_7x7_c2048_1x1", 833, n=16, h=7, w=7, ci=2048, co=512, kh=1, kw=1, act=cases.RELU), 4)]
+    for c, groups in auto:
+        got = _gpu_conv(c, shim.ALGO_AUTO)
+        kernel = shim.last_kernel()
+        print(f"{c.name}: {kernel}", flush=True)
+        assert kernel.startswith("IgemmKSplitKernel<%d" % groups), kernel
+        np.testing.assert_array_equal(got.data, _gpu_conv(c, shim.ALGO_DIRECT).data, err_msg=c.name)
+
+
 def test_resident_tile_convolution_gives_the_same_bytes():
     """Small filters at stride 1 over 64, 128 or 256 input channels keep the input tile in LDS for all taps
     (HaloConvKernel).  Against the direct kernel: every channel count, narrow and wide output-channel tiles with ragged
