@@ -846,7 +846,7 @@ int LaunchHaloC(HaloArgs& a, const mi355x_conv2d_s* p, uint32_t batch, hipStream
     const long long blocks = static_cast<long long>(a.tiles_m) * a.tiles_n;
     // a block is one long dependent chain (tile, k-loop, epilogue): with fewer blocks than CUs the implicit GEMM's smaller
     // tiles finish sooner
-    if (blocks < 192 && p->tile_override != 3000) return -1;
+    if (blocks < 192 && !(p->tile_override == 3000 || p->tile_override == 3001)) return -1;
     // three weight stages unless two let every block of the launch be resident at once and three do not
     auto resident = [&](int st) { return 256ll * std::min(4, (160 * 1024) / smem_of(R, st)); };
     const bool three = smem_of(R, 3) <= 160 * 1024 && !(blocks > resident(3) && blocks <= resident(2));
@@ -875,7 +875,14 @@ int LaunchHalo(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y,
     const bool wide = g.Co > 64;
     switch (g.Ci)
     {
-    case 64: return wide ? LaunchHaloC<64, 1, 4, 7>(a, p, batch, stream) : LaunchHaloC<64, 2, 2, 4>(a, p, batch, stream);
+    case 64:
+    {
+        // narrow output: half-height tiles (128 pixels) while the full ones would leave at most one block per CU
+        const int r4 = std::max(1, std::min(g.Ho, 256 / std::max(1, g.Wo)));
+        const long long blocks4 = static_cast<long long>(batch) * ((g.Ho + r4 - 1) / r4);
+        if (!wide && g.Wo <= 128 && (p->tile_override == 3001 || (p->tile_override == 0 && blocks4 <= 256))) return LaunchHaloC<64, 2, 2, 2>(a, p, batch, stream);
+        return wide ? LaunchHaloC<64, 1, 4, 7>(a, p, batch, stream) : LaunchHaloC<64, 2, 2, 4>(a, p, batch, stream);
+    }
     case 128: return wide ? LaunchHaloC<128, 1, 4, 7>(a, p, batch, stream) : LaunchHaloC<128, 2, 2, 4>(a, p, batch, stream);
     case 256: return wide ? LaunchHaloC<256, 1, 4, 7>(a, p, batch, stream) : LaunchHaloC<256, 2, 2, 4>(a, p, batch, stream);
     default: return -1;
@@ -942,7 +949,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             return LaunchPwKs<32>(p, Mrows, x, y, stream);
         }
         // Small filters at stride 1 over 64 / 128 / 256 channels: the input tile stays in LDS for all taps
-        if (p->halo_ok && p->zw_neg == 0 && p->opt_igemm_lds != 0 && (p->tile_override == 0 || p->tile_override == 3000))
+        if (p->halo_ok && p->zw_neg == 0 && p->opt_igemm_lds != 0 && (p->tile_override == 0 || (p->tile_override == 3000 || p->tile_override == 3001)))
         {
             const int rc = LaunchHalo(p, batch, x, y, stream);
             if (rc >= 0) return rc;

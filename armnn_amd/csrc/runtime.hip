@@ -152,11 +152,11 @@ int mi355x_set_option(const char* name, int value)
     if (std::strcmp(name, "igemm_tile") == 0)
     {
         // 2256, 2128, 1256: the large-tile kernel at 256x256, 256x128, 128x256; 2064 / 4064: 64x64 tiles with K split over 2 / 4
-        // groups of waves; 3000: the resident-tile kernel where its shape
+        // groups of waves; 3000 / 3001: the resident-tile kernel (3001: half-height tiles for narrow outputs) where its shape
         // rules allow it (any other forced tile keeps a convolution off that kernel)
         if (value != 0 && value != 64 && value != 96 && value != 128 && value != 256 && value != 512 && value != 2256 && value != 2128 && value != 1256 &&
-            value != 3000 && value != 4064 && value != 2064)
-            return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_tile must be 0, 64, 96, 128, 256, 512, 2256, 2128, 1256, 3000, 2064 or 4064");
+            value != 3000 && value != 3001 && value != 4064 && value != 2064)
+            return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_tile must be 0, 64, 96, 128, 256, 512, 2256, 2128, 1256, 3000, 3001, 2064 or 4064");
         GlobalOptions().igemm_tile = value;
         return 0;
     }

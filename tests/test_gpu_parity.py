@@ -218,7 +218,7 @@ def test_resident_tile_convolution_gives_the_same_bytes():
           cases.make_conv_case("halo_c64_w224", 810, n=1, h=5, w=224, ci=64, co=64)]
     for c in cs:
         want = _gpu_conv(c, shim.ALGO_DIRECT)
-        for tile in (0, 3000):
+        for tile in (0, 3000, 3001):               # 3001: half-height tiles where the output has at most 64 channels
             shim.set_option("igemm_tile", tile)
             try:
                 got = _gpu_conv(c, shim.ALGO_MFMA)
@@ -227,6 +227,8 @@ def test_resident_tile_convolution_gives_the_same_bytes():
                 shim.set_option("igemm_tile", 0)
             # unforced, launches of fewer blocks than three quarters of the CUs stay on the implicit GEMM
             assert tile == 0 or kernel.startswith("HaloConvKernel<"), kernel
+            if tile == 3001 and c.w.info.shape[-1] == 64 and c.out_info.shape[-1] <= 64 and c.out_info.shape[2] <= 128:
+                assert kernel.startswith("HaloConvKernel<64, 2, 2, 2,"), kernel
             np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} tile {tile} {kernel}")
         print(f"{c.name}: {want.data.size} outputs, {kernel}", flush=True)
     # 16 images of 56 x 56 make 224 blocks: the automatic choice
