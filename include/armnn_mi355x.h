@@ -100,7 +100,10 @@ int  mi355x_abi_version(void);
  *   (identical bytes; lets tests compare the two).
  *   "igemm_tile" = 0 | 64 | 96 | 128 | 256 | 512: plans created while it is set run on the LDS-tiled implicit-GEMM
  *   kernel with 64x64, 128x64, 128x128, 256x128 or 256x256 tiles instead of the automatic choice (the two largest only
- *   where the direct-to-LDS kernel applies; identical bytes; tests and tuning).
+ *   where the direct-to-LDS kernel applies; identical bytes; tests and tuning).  Further values force the other MFMA
+ *   kernels where their shape rules allow them: 2256 | 2128 | 1256 the large-tile GEMM at 256x256, 256x128, 128x256;
+ *   2064 | 4064 64x64 tiles with K split over 2 or 4 groups of waves inside the block; 3000 | 3001 the convolution that
+ *   keeps its input tile resident in on-chip memory (3001: half-height tiles).
  *   "igemm_lds" = 2 | 3 | 0: LDS stages of the implicit-GEMM kernel that loads its k-tiles from global memory straight
  *   into LDS (input channels a multiple of 128); 0 selects the register-staged kernel instead (identical bytes).
  *   "dw_rows" = 0 | 1 | 2: output rows per thread of the 3x3 depthwise kernel (0: chosen from the feature-map height;
