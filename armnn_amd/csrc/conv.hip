@@ -699,6 +699,20 @@ int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, voi
     const int nblocks = a.tiles_m * a.tiles_n;
     const int grid = (nblocks + 7) / 8 * 8;
     constexpr int smem = IgemmLdsSmemBytes<BM, BN, ST>();
+    if constexpr (BM == 64 && BN == 64 && !AW)
+    {
+        // pointwise layers and FullyConnected below 2 GiB per tensor: addresses without per-load vector arithmetic
+        if (a.unit && static_cast<long long>(a.M) * a.Ci < (1ll << 31) && static_cast<long long>(p->Co_pad) * a.K_pad < (1ll << 31) && a.Ci == a.K_pad)
+        {
+            static const hipError_t uattr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmLdsKernel<BM, BN, WM, WN, ST, U8, false, true>),
+                                                                hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+            MI355X_HIP(uattr);
+            NoteKernel("IgemmLdsKernel<%d, %d, %d, %d, %d, %s, false, true>", BM, BN, WM, WN, ST, BoolName(U8));
+            hipLaunchKernelGGL((IgemmLdsKernel<BM, BN, WM, WN, ST, U8, false, true>), dim3(grid), dim3(64 * WM * WN), smem, stream, a);
+            MI355X_HIP(hipGetLastError());
+            return 0;
+        }
+    }
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmLdsKernel<BM, BN, WM, WN, ST, U8, AW>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);

@@ -40,7 +40,10 @@ constexpr int VmcntImm(int n)
 
 // WM x WN waves per block (4, 8 or 16), each with a (BM / WM) x (BN / WN) tile of the block tile.
 // AW: the weights have a zero point; each pixel's activations are summed beside the products (see IgemmKernel).
-template <int BM, int BN, int WM, int WN, int ST, bool U8, bool AW = false>
+// UNIT: the launch is a 1x1 stride-1 unpadded convolution or a FullyConnected layer (a.unit) whose tensors are below
+// 2 GiB: output row m reads input row m, there is no padding and no tap walk, and every load address is a wave-uniform
+// base (advanced by 128 bytes per k-tile) plus a 32-bit lane offset fixed for the kernel -- no vector arithmetic per load.
+template <int BM, int BN, int WM, int WN, int ST, bool U8, bool AW = false, bool UNIT = false>
 __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
 {
     static_assert(ST >= 2 && ST <= 8, "2 to 8 LDS stages");
@@ -112,10 +115,34 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
     static_assert((BM / NW) % 16 == 0 && (BN / NW) % 16 == 0, "a wave's first row is a multiple of 16");
     const int8_t* wrow = a.w + static_cast<long long>(tn * BN + wave * (BN / NW) + lrow) * a.K_pad;
     int ci = 0, kx = 0, ky = 0;                  // tap walk, identical in every thread
+    // UNIT: lane offsets from the tensors' first bytes (rows past the end re-read row 0; their results are not stored)
+    uint32_t aoff[RA], boff[RB];
+    if constexpr (UNIT)
+    {
+#pragma unroll
+        for (int j = 0; j < RA; ++j)
+        {
+            const int m = tm * BM + wave * (BM / NW) + j * 8 + lrow;
+            aoff[j] = static_cast<uint32_t>(m < a.M ? m : 0) * static_cast<uint32_t>(a.Ci) + ((j & 1) ? lchunk_odd : lchunk_even) * 16;
+        }
+#pragma unroll
+        for (int j = 0; j < RB; ++j)
+            boff[j] = static_cast<uint32_t>(tn * BN + wave * (BN / NW) + j * 8 + lrow) * static_cast<uint32_t>(a.K_pad) + ((j & 1) ? lchunk_odd : lchunk_even) * 16;
+    }
 
     auto load_tile = [&](int kt, int stage) {
         uint8_t* As = smem + stage * STAGE + wave * (BM / NW) * BK;
         uint8_t* Bs = smem + stage * STAGE + BM * BK + wave * (BN / NW) * BK;
+        if constexpr (UNIT)
+        {
+            const uint8_t* abase = a.x + kt * BK;
+            const int8_t* bbase = a.w + kt * BK;
+#pragma unroll
+            for (int j = 0; j < RA; ++j) __builtin_amdgcn_global_load_lds((GlobalPtr)(abase + aoff[j]), (LdsPtr)(As + j * 8 * BK), 16, 0, 0);
+#pragma unroll
+            for (int j = 0; j < RB; ++j) __builtin_amdgcn_global_load_lds((GlobalPtr)(bbase + boff[j]), (LdsPtr)(Bs + j * 8 * BK), 16, 0, 0);
+            return;
+        }
         const int dy = ky * a.dil_y, dx = kx * a.dil_x;
         const long long tap_off = (static_cast<long long>(dy) * a.W + dx) * a.Ci + ci;
 #pragma unroll
