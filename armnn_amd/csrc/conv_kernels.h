@@ -457,7 +457,7 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
                 if (m < a.M)
                 {
                     const v4i v = *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16);
-                    *reinterpret_cast<v4i*>(a.y + static_cast<long long>(m) * a.Co + c0) = v;
+                    StoreOut16(a.y + static_cast<long long>(m) * a.Co + c0, v);
                 }
             }
         }

@@ -61,6 +61,27 @@ struct ChanTab
 //   recomputed with the reference's own sequence.  A channel without a fast path has m+ = m- = 0, b+ = 255, b- = 0.
 //   The activation's clamp, where it is narrower than 0..255, is applied to both sides before converting.
 
+// Stores of layer outputs.  An ordinary store leaves its line dirty in the XCD's L2 until the end-of-kernel write-back,
+// which then moves the whole output tensor (up to the 32 MB the eight L2s hold) after the last wave has finished, with
+// nothing to overlap it.  With the sc1 bit (agent scope) the L2 writes the line through as the store is issued, so the
+// write-back runs beside the rest of the kernel and the data is where the next kernel -- whose blocks run on any XCD --
+// reads it from.  (The nt bit instead also helps a kernel timed alone but makes the next layer slower.)  Only for stores
+// that cover whole lines per instruction: the depthwise kernel's 32-byte pieces and the pooling kernel's dwords, written
+// through one by one, are slower than ordinary stores that L2 merges.
+#ifndef MI355X_STORE_THROUGH
+#define MI355X_STORE_THROUGH 1
+#endif
+typedef int StoreVec4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ void StoreOut16(void* p, const StoreVec4& v)
+{
+#if MI355X_STORE_THROUGH
+    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+#else
+    *reinterpret_cast<StoreVec4*>(p) = v;
+#endif
+}
+
 __device__ __forceinline__ uint32_t Pack4(int q0, int q1, int q2, int q3)
 {
     // four codes -> one dword (byte 0 = q0), three v_perm_b32

@@ -205,6 +205,7 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
             const int ox = tx * TW + xg * P + j;
             if (ox < a.Wo && c < a.C)
             {
+                // an ordinary store: these 32-byte pieces of a line are merged in L2 (written through one by one they are slower)
                 *reinterpret_cast<uint32_t*>(yrow + static_cast<long long>(ox) * a.C) =
                     Requant4Dev(acc[o][j][0], acc[o][j][1], acc[o][j][2], acc[o][j][3], f4, a.ct, c, a.rq);
             }
@@ -591,7 +592,7 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
             const uint4 v = half ? uint4{r0, o[2], r1, o[3]} : uint4{o[0], r0, o[1], r1};
             if (ox < a.Wo)
             {
-                if (a.vec16) *reinterpret_cast<uint4*>(yp + ct * 32 + 16 * half) = v;
+                if (a.vec16) StoreOut16(yp + ct * 32 + 16 * half, StoreVec4{static_cast<int>(v.x), static_cast<int>(v.y), static_cast<int>(v.z), static_cast<int>(v.w)});
                 else
                 {
                     uint32_t* dst = reinterpret_cast<uint32_t*>(yp + ct * 32 + 16 * half);

@@ -271,7 +271,7 @@ __global__ __launch_bounds__(256) void HaloConvKernel(HaloArgs a)
         if (c0 < a.Co)
         {
             for (int r = orow; r < mt; r += ROWS_PER_PASS)
-                *reinterpret_cast<v4i*>(yt + static_cast<long long>(r) * a.Co + c0) = *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16);
+                StoreOut16(yt + static_cast<long long>(r) * a.Co + c0, *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16));
         }
     }
     else

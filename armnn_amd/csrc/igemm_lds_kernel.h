@@ -338,7 +338,7 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
             {
                 const int m = tm * BM + r;
                 if (m < a.M)
-                    *reinterpret_cast<v4i*>(a.y + static_cast<long long>(m) * a.Co + c0) = *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16);
+                    StoreOut16(a.y + static_cast<long long>(m) * a.Co + c0, *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16));
             }
         }
     }

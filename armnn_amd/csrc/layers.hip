@@ -295,7 +295,7 @@ __global__ __launch_bounds__(256) void AddVec16Kernel(QIn q0, QIn q1, Requant rq
             Dequant4Dev(b[d], q1, vb);
             o[d] = QuantizePack4Dev(__fadd_rn(va[0], vb[0]), __fadd_rn(va[1], vb[1]), __fadd_rn(va[2], vb[2]), __fadd_rn(va[3], vb[3]), rq);
         }
-        y[i] = o;
+        StoreOut16(y + i, StoreVec4{static_cast<int>(o[0]), static_cast<int>(o[1]), static_cast<int>(o[2]), static_cast<int>(o[3])});
     }
 }
 

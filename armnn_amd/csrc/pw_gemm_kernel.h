@@ -151,8 +151,11 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
                 const int row = t * 32 + r;
                 const int c0 = n0 + cc * 16;
                 if (row < a.M && c0 < a.N)
-                    *reinterpret_cast<v4i*>(a.y + static_cast<long long>(row) * a.N + c0) =
-                        *reinterpret_cast<const v4i*>(ostage + r * LDO + cc * 16);
+                {
+                    const v4i ov = *reinterpret_cast<const v4i*>(ostage + r * LDO + cc * 16);
+                    uint8_t* dst = a.y + static_cast<long long>(row) * a.N + c0;
+                    StoreOut16(dst, ov);
+                }
             }
         }
         else
