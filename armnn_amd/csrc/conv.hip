@@ -48,7 +48,7 @@ struct mi355x_conv2d_s
     bool bk128 = false;            // implicit GEMM walks K in 128-byte tiles
     bool halo_ok = false;          // shape fits the resident-tile kernel (weights without a zero point are checked at launch)
     int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 96 (= 128x64) / 128: the "igemm_tile" option at plan creation
-    int opt_igemm_lds = 2, opt_dw_rows = 0, opt_stem_dot4 = 0;     // the other process-wide options, as they stood at plan creation
+    int opt_igemm_lds = 2, opt_dw_rows = 0, opt_dw_cb = 0, opt_stem_dot4 = 0;     // the other process-wide options, as they stood at plan creation
                                    // (launches read the plan, never the mutable globals: plans may run on any host thread)
     uint32_t xor_mask = 0, pad_word = 0;
     int zw_neg = 0;                // MFMA plans: minus the zero point of the stored int8 weights (0: symmetric)
@@ -139,6 +139,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     p->d = d;
     p->opt_igemm_lds = GlobalOptions().igemm_lds;
     p->opt_dw_rows = GlobalOptions().dw_rows;
+    p->opt_dw_cb = GlobalOptions().dw_cb;
     p->opt_stem_dot4 = GlobalOptions().stem_dot4;
     const int Co = static_cast<int>(d.out_c), Ci = static_cast<int>(d.in_c);
     const int Kh = static_cast<int>(d.kernel_h), Kw = static_cast<int>(d.kernel_w);
@@ -1091,12 +1092,21 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             a.x = xin; a.pad16 = p->pad16; a.wpack = p->w_dot4; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
             a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.C = g.Co; a.Ho = g.Ho; a.Wo = g.Wo;
             a.pad_top = g.pad_top; a.pad_left = g.pad_left;
-            const int tw = g.stride_x == 1 ? 16 : 8;
-            // two output rows per thread (16-row tiles) unless that would leave much of a tile outside a small feature map
+            // 128 channels per block where the channel count allows: every pixel a block reads or writes is a whole line
+            // -- for the large feature maps (56 x 56 x 128: 13.2 -> 12.7 us at stride 1, 7.3 -> 6.6 us at stride 2, 32 images)
+            // and for those so small that a 16-pixel-wide tile is mostly outside the image (7 x 7 x 1024: 5.1 -> 4.5 us); in
+            // between (28 x 28, 14 x 14) the 32-channel blocks with their larger tiles and smaller halo are as fast or faster
+            const bool wide = (g.Co % 128) == 0 && p->opt_dw_cb != 32 && (g.H * g.W >= 2500 || (g.Ho <= 8 && g.Wo <= 8));
+            const int tw = wide ? (g.stride_x == 1 ? 8 : 4) : (g.stride_x == 1 ? 16 : 8);
+            const int th1 = wide ? 4 : 8;            // tile rows with one output row per thread
+            // two output rows per thread unless that would leave much of a tile outside a small feature map (or, with the
+            // small tiles of the 128-channel blocks, fewer than four blocks per CU)
             const int opt_r = p->opt_dw_rows;
-            const int rows_per_thread = opt_r ? opt_r : ((g.Ho + 15) / 16 * 16 - g.Ho) * 4 <= g.Ho ? 2 : 1;
-            const int th = 8 * rows_per_thread;
-            a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + th - 1) / th; a.cblocks = (g.Co + 31) / 32;
+            int rows_per_thread = opt_r ? opt_r : ((g.Ho + 2 * th1 - 1) / (2 * th1) * (2 * th1) - g.Ho) * 4 <= g.Ho ? 2 : 1;
+            if (wide && !opt_r && static_cast<long long>(batch) * ((g.Wo + tw - 1) / tw) * ((g.Ho + 2 * th1 - 1) / (2 * th1)) * (g.Co / 128) < 1024)
+                rows_per_thread = 1;
+            const int th = th1 * rows_per_thread;
+            a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + th - 1) / th; a.cblocks = wide ? g.Co / 128 : (g.Co + 31) / 32;
             a.xor_mask = p->xor_mask; a.pad_word = p->pad_word; a.rq = p->rq;
             const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y * a.cblocks;
             if (nb > 0x7fffffffll - 8) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
@@ -1104,18 +1114,29 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             a.xcd_chunk = static_cast<int>((nb + 7) / 8);
             const dim3 grid(static_cast<unsigned>(a.xcd_chunk) * 8u);
             a.wpack2 = p->w_dot4b;
-            NoteKernel("Depthwise3x3Kernel<%d, %d, %s>", g.stride_x, rows_per_thread, BoolName(p->w_dot4b != nullptr));
-            if (p->w_dot4b)
+            const bool w2 = p->w_dot4b != nullptr;
+            if (wide) NoteKernel("Depthwise3x3Kernel<%d, %d, %s, 128>", g.stride_x, rows_per_thread, BoolName(w2));
+            else NoteKernel("Depthwise3x3Kernel<%d, %d, %s>", g.stride_x, rows_per_thread, BoolName(w2));
+            const int variant = (g.stride_x == 1 ? 0 : 4) + (rows_per_thread == 2 ? 0 : 2) + (w2 ? 1 : 0);
+            switch (variant + (wide ? 8 : 0))
             {
-                if (g.stride_x == 1 && rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2, true>), grid, dim3(256), 0, stream, a);
-                else if (g.stride_x == 1) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1, true>), grid, dim3(256), 0, stream, a);
-                else if (rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<2, 2, true>), grid, dim3(256), 0, stream, a);
-                else hipLaunchKernelGGL((Depthwise3x3Kernel<2, 1, true>), grid, dim3(256), 0, stream, a);
+            case 0: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2, false>), grid, dim3(256), 0, stream, a); break;
+            case 1: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2, true>), grid, dim3(256), 0, stream, a); break;
+            case 2: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1, false>), grid, dim3(256), 0, stream, a); break;
+            case 3: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1, true>), grid, dim3(256), 0, stream, a); break;
+            case 4: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 2, false>), grid, dim3(256), 0, stream, a); break;
+            case 5: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 2, true>), grid, dim3(256), 0, stream, a); break;
+            case 6: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 1, false>), grid, dim3(256), 0, stream, a); break;
+            case 7: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 1, true>), grid, dim3(256), 0, stream, a); break;
+            case 8: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2, false, 128>), grid, dim3(256), 0, stream, a); break;
+            case 9: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2, true, 128>), grid, dim3(256), 0, stream, a); break;
+            case 10: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1, false, 128>), grid, dim3(256), 0, stream, a); break;
+            case 11: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1, true, 128>), grid, dim3(256), 0, stream, a); break;
+            case 12: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 2, false, 128>), grid, dim3(256), 0, stream, a); break;
+            case 13: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 2, true, 128>), grid, dim3(256), 0, stream, a); break;
+            case 14: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 1, false, 128>), grid, dim3(256), 0, stream, a); break;
+            default: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 1, true, 128>), grid, dim3(256), 0, stream, a); break;
             }
-            else if (g.stride_x == 1 && rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2>), grid, dim3(256), 0, stream, a);
-            else if (g.stride_x == 1) hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1>), grid, dim3(256), 0, stream, a);
-            else if (rows_per_thread == 2) hipLaunchKernelGGL((Depthwise3x3Kernel<2, 2>), grid, dim3(256), 0, stream, a);
-            else hipLaunchKernelGGL((Depthwise3x3Kernel<2, 1>), grid, dim3(256), 0, stream, a);
             MI355X_HIP(hipGetLastError());
             return 0;
         }

@@ -82,6 +82,15 @@ __device__ __forceinline__ void StoreOut16(void* p, const StoreVec4& v)
 #endif
 }
 
+__device__ __forceinline__ void StoreOut4(void* p, uint32_t v)
+{
+#if MI355X_STORE_THROUGH
+    asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
+#else
+    *reinterpret_cast<uint32_t*>(p) = v;
+#endif
+}
+
 __device__ __forceinline__ uint32_t Pack4(int q0, int q1, int q2, int q3)
 {
     // four codes -> one dword (byte 0 = q0), three v_perm_b32

@@ -56,16 +56,26 @@ __device__ __forceinline__ int XcdContiguousWorkItem(int block, int chunk)
 // through one v_dot4 per channel and output row that the input row belongs to.  With R = 2 the rows two outputs share
 // are read and transposed once, and the per-thread set-up (staging, constants, addresses) is spread over twice the
 // outputs; R = 1 keeps more blocks in flight for small feature maps.
-template <int S, int R, bool W2 = false>
+//
+// CB = 128 (channel counts that are multiples of 128): a block takes 128 channels of a tile of 4 R rows x 2 P pixels, 32
+// lanes per pixel.  Every pixel it loads or stores is then one whole 128-byte line instead of a quarter of one, and its
+// stores can be written through L2 (StoreOut4); the smaller tile costs more halo (1.56 x instead of 1.27 x at stride 1).
+template <int S, int R, bool W2 = false, int CB = 32>
 __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
 {
-    constexpr int CB = 32, TH = 8 * R, XG = 4;
+    static_assert(CB == 32 || CB == 128, "32 or 128 channels per block");
+    constexpr int LPC = CB / 4;                  // lanes per pixel
+    constexpr int XG = CB == 32 ? 4 : 2;         // thread columns
+    constexpr int TH = (256 / (LPC * XG)) * R;   // 8 R or 4 R output rows per tile
+    constexpr int CPP = CB / 16;                 // 16-byte staging chunks per pixel
     constexpr int P = S == 1 ? 4 : 2;            // outputs per thread and row
     constexpr int TW = P * XG;                   // outputs per tile row
     constexpr int HR = TH * S + 2;               // halo rows held in LDS
     constexpr int HC = TW * S + 2;               // halo columns
     constexpr int IR = (R - 1) * S + 3;          // input rows a thread walks
-    constexpr int PITCH = 48;                    // bytes per pixel in LDS: 32 used; 48 spreads dword reads over banks
+    // bytes per pixel in LDS.  CB = 32: 48 spreads the dword reads of a wave's eight pixels over the banks; CB = 128: the 32
+    // lanes of a pixel read 128 contiguous bytes
+    constexpr int PITCH = CB == 32 ? 48 : 128;
     __shared__ __attribute__((aligned(16))) uint8_t tile[HR * HC * PITCH];
 
     int b = XcdContiguousWorkItem(blockIdx.x, a.xcd_chunk);
@@ -83,33 +93,33 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
     const int xm = static_cast<int>(a.xor_mask);
     // all of a thread's staging loads are issued before the first is used; a chunk outside the image reads 16 prepared
     // bytes that become the padding value under the xor, so no load sits in a divergent branch
-    constexpr int NST = (HR * HC * 2 + 255) / 256;
+    constexpr int NST = (HR * HC * CPP + 255) / 256;
     v4i st[NST];
 #pragma unroll
     for (int k = 0; k < NST; ++k)
     {
-        const int i = min(tid + k * 256, HR * HC * 2 - 1);
-        const int half = i & 1;
-        const int pix = i >> 1;
+        const int i = min(tid + k * 256, HR * HC * CPP - 1);
+        const int part = i % CPP;
+        const int pix = i / CPP;
         const int col = pix % HC;
         const int row = pix / HC;
         const int iy = iy_org + row, ix = ix_org + col;
         const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && static_cast<unsigned>(ix) < static_cast<unsigned>(a.W) &&
-                        cb * CB + half * 16 < a.C;
-        const uint8_t* src = ok ? xn + (static_cast<long long>(iy) * a.W + ix) * a.C + half * 16 : a.pad16;
+                        cb * CB + part * 16 < a.C;
+        const uint8_t* src = ok ? xn + (static_cast<long long>(iy) * a.W + ix) * a.C + part * 16 : a.pad16;
         st[k] = *reinterpret_cast<const v4i*>(src);
     }
 #pragma unroll
     for (int k = 0; k < NST; ++k)
     {
         const int i = tid + k * 256;
-        if (i < HR * HC * 2) *reinterpret_cast<v4i*>(tile + (i >> 1) * PITCH + (i & 1) * 16) = st[k] ^ xm;
+        if (i < HR * HC * CPP) *reinterpret_cast<v4i*>(tile + (i / CPP) * PITCH + (i % CPP) * 16) = st[k] ^ xm;
     }
 
     // ---- per-thread constants ---------------------------------------------------------------------------------
-    const int c4 = tid & 7;
-    const int xg = (tid >> 3) & 3;
-    const int row = (tid >> 5) * R;              // first of this thread's output rows within the tile
+    const int c4 = tid % LPC;
+    const int xg = (tid / LPC) % XG;
+    const int row = (tid / (LPC * XG)) * R;      // first of this thread's output rows within the tile
     const int c = cb * CB + c4 * 4;
     uint32_t wA[3][4], wB[3][4];
 #pragma unroll
@@ -205,9 +215,11 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
             const int ox = tx * TW + xg * P + j;
             if (ox < a.Wo && c < a.C)
             {
-                // an ordinary store: these 32-byte pieces of a line are merged in L2 (written through one by one they are slower)
-                *reinterpret_cast<uint32_t*>(yrow + static_cast<long long>(ox) * a.C) =
-                    Requant4Dev(acc[o][j][0], acc[o][j][1], acc[o][j][2], acc[o][j][3], f4, a.ct, c, a.rq);
+                const uint32_t q = Requant4Dev(acc[o][j][0], acc[o][j][1], acc[o][j][2], acc[o][j][3], f4, a.ct, c, a.rq);
+                // CB = 32: an ordinary store, these 32-byte pieces of a line are merged in L2 (written through one by one they
+                // are slower); CB = 128: half a wave stores a whole line
+                if constexpr (CB == 128) StoreOut4(yrow + static_cast<long long>(ox) * a.C, q);
+                else *reinterpret_cast<uint32_t*>(yrow + static_cast<long long>(ox) * a.C) = q;
             }
         }
     }

@@ -143,6 +143,12 @@ int mi355x_set_option(const char* name, int value)
         GlobalOptions().dw_rows = value;
         return 0;
     }
+    if (std::strcmp(name, "dw_cb") == 0)
+    {
+        if (value != 0 && value != 32) return SetError(MI355X_ERR_INVALID_ARGUMENT, "dw_cb must be 0 or 32");
+        GlobalOptions().dw_cb = value;
+        return 0;
+    }
     if (std::strcmp(name, "igemm_lds") == 0)
     {
         if (value != 0 && value != 2 && value != 3) return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_lds must be 0, 2 or 3");

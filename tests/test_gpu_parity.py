@@ -300,6 +300,36 @@ def test_depthwise_rows_per_thread_variants_give_the_same_bytes():
             np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} rows {rows}")
 
 
+def test_depthwise_128_channel_blocks_give_the_same_bytes():
+    """Channel counts that are multiples of 128 run the 3x3 depthwise kernel with 128 channels per block (whole lines per
+    pixel) on large feature maps and on maps of at most 8 x 8: ragged sizes, both strides, one and two rows per thread,
+    uint8 activations, weights with a zero point (two int8 halves), against the 32-channel blocks and the plain kernel."""
+    U8 = DataType.QAsymmU8
+    cs = [cases.make_conv_case("dw128_s1_57x53", 711, n=2, h=57, w=53, ci=128, depthwise=True, act=cases.RELU6),
+          cases.make_conv_case("dw128_s2_57x53_u8", 712, n=2, h=57, w=53, ci=256, depthwise=True, stride=(2, 2), in_dtype=U8, in_offset=140, out_offset=5),
+          cases.make_conv_case("dw128_s1_7x7", 713, n=3, h=7, w=7, ci=256, depthwise=True, act=cases.RELU),
+          cases.make_conv_case("dw128_s2_8x5", 714, n=2, h=8, w=5, ci=128, depthwise=True, stride=(2, 2)),
+          cases.make_conv_case("dw128_s1_64x50_zero_point_weights", 715, n=1, h=64, w=50, ci=128, depthwise=True, per_axis=False, w_std=60.0,
+                               w_dtype=U8, w_offset=93, in_dtype=U8, in_offset=120, out_offset=3, act=cases.RELU6)]
+    for c in cs:
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        for cb in (0, 32):
+            for rows in (0, 1, 2):
+                shim.set_option("dw_cb", cb)
+                shim.set_option("dw_rows", rows)
+                try:
+                    got = _gpu_conv(c, shim.ALGO_DEPTHWISE)
+                    kernel = shim.last_kernel()
+                finally:
+                    shim.set_option("dw_cb", 0)
+                    shim.set_option("dw_rows", 0)
+                print(f"{c.name} blocks {cb or 'auto'} rows {rows}: {kernel}", flush=True)
+                assert kernel.startswith("Depthwise3x3Kernel<") and kernel.endswith(", 128>") == (cb == 0), kernel
+                np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} blocks {cb} rows {rows}")
+    with pytest.raises(shim.ShimError):
+        shim.set_option("dw_cb", 64)
+
+
 def test_config_c1_full_size(port):
     """Benchmark configuration C1: 1x56x56x64 -> 64, 3x3 SAME, per-channel, ReLU6; expected code range [-128, -8]."""
     c = cases.make_conv_case("C1", 20250101, h=56, w=56, ci=64, co=64, act=cases.RELU6)
