@@ -1115,8 +1115,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             const dim3 grid(static_cast<unsigned>(a.xcd_chunk) * 8u);
             a.wpack2 = p->w_dot4b;
             const bool w2 = p->w_dot4b != nullptr;
-            if (wide) NoteKernel("Depthwise3x3Kernel<%d, %d, %s, 128>", g.stride_x, rows_per_thread, BoolName(w2));
-            else NoteKernel("Depthwise3x3Kernel<%d, %d, %s>", g.stride_x, rows_per_thread, BoolName(w2));
+            NoteKernel("Depthwise3x3Kernel<%d, %d, %s, %d>", g.stride_x, rows_per_thread, BoolName(w2), wide ? 128 : 32);
             const int variant = (g.stride_x == 1 ? 0 : 4) + (rows_per_thread == 2 ? 0 : 2) + (w2 ? 1 : 0);
             switch (variant + (wide ? 8 : 0))
             {
