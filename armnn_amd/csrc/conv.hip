@@ -1045,11 +1045,26 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         a.w_mfma = p->w_stem; a.w_mfma2 = p->w_stem2; a.kp = p->stem_kp;
         if (p->w_stem && !p->opt_stem_dot4 && (g.Kh == 3 || g.Kh == 7))
         {
-            const long long nbm = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
+            long long nbm = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
             if (nbm > 0x7fffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
+            // 8-row tiles while the 16-row ones would give a CU fewer than three blocks: a block is one dependent chain of
+            // staging, gather, MFMA and requantization, and with one or two per CU nothing runs beside it
+            const bool th8 = !p->w_stem2 && nbm < 768;
+            if (th8)
+            {
+                a.tiles_y = (g.Ho + 7) / 8;
+                nbm = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
+            }
             const dim3 gridm(static_cast<unsigned>(nbm));
-            NoteKernel("SmallCiMfmaKernel<%d, %d, %d, 16, %s>", g.Kh, g.Kh == 3 ? 3 : 6, g.Co == 32 ? 1 : 2, BoolName(p->w_stem2 != nullptr));
-            if (p->w_stem2)
+            NoteKernel("SmallCiMfmaKernel<%d, %d, %d, %d, %s>", g.Kh, g.Kh == 3 ? 3 : 6, g.Co == 32 ? 1 : 2, th8 ? 8 : 16, BoolName(p->w_stem2 != nullptr));
+            if (th8)
+            {
+                if (g.Kh == 3 && g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 1, 8>), gridm, dim3(256), 0, stream, a);
+                else if (g.Kh == 3) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 2, 8>), gridm, dim3(256), 0, stream, a);
+                else if (g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 1, 8>), gridm, dim3(256), 0, stream, a);
+                else hipLaunchKernelGGL((SmallCiMfmaKernel<7, 6, 2, 8>), gridm, dim3(256), 0, stream, a);
+            }
+            else if (p->w_stem2)
             {
                 if (g.Kh == 3 && g.Co == 32) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 1, 16, true>), gridm, dim3(256), 0, stream, a);
                 else if (g.Kh == 3) hipLaunchKernelGGL((SmallCiMfmaKernel<3, 3, 2, 16, true>), gridm, dim3(256), 0, stream, a);

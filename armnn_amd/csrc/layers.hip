@@ -229,6 +229,89 @@ __global__ __launch_bounds__(256) void Pool2dC4Kernel(PoolArgs p, QIn qin, Requa
     *reinterpret_cast<uint32_t*>(y + idx * 4) = QuantizePack4Dev(res[0], res[1], res[2], res[3], rq);
 }
 
+// Max pooling over windows of at most WB x WB taps, sixteen channels per thread: 16-byte loads, and the maximum taken on
+// pairs of bytes at a time (v_pk_max_u16 on the even and on the odd bytes of a dword; int8 codes are first mapped to
+// unsigned order by flipping the sign bit).  The window arithmetic is spent once per sixteen outputs instead of once per
+// four.  The largest code is the largest value (dequantization is strictly increasing); it is dequantized and requantized
+// like every pooling result.
+template <int WB>
+__global__ __launch_bounds__(256) void MaxPool2dC16Kernel(PoolArgs p, QIn qin, Requant rq, const uint8_t* __restrict__ x,
+                                                          uint8_t* __restrict__ y, long long total16)
+{
+    typedef unsigned short us2 __attribute__((ext_vector_type(2)));
+    const long long idx = static_cast<long long>(blockIdx.x) * 256 + threadIdx.x;
+    if (idx >= total16) return;
+    const int C16 = p.C >> 4;
+    const int c = static_cast<int>(idx % C16) * 16;
+    long long pix = idx / C16;
+    const int ox = static_cast<int>(pix % p.Wo);
+    pix /= p.Wo;
+    const int oy = static_cast<int>(pix % p.Ho);
+    const long long n = pix / p.Ho;
+
+    int hstart = oy * p.stride_y - p.pad_top;
+    int hend = min(hstart + p.pool_h, p.H + p.pad_bottom);
+    hstart = min(max(hstart, 0), p.H);
+    hend = min(max(hend, 0), p.H);
+    int wstart = ox * p.stride_x - p.pad_left;
+    int wend = min(wstart + p.pool_w, p.W + p.pad_right);
+    const bool empty = hend <= 0 || hstart > p.H || wend <= 0 || wstart > p.W;
+    wstart = min(max(wstart, 0), p.W);
+    wend = min(max(wend, 0), p.W);
+    us2 blo[4], bhi[4];
+#pragma unroll
+    for (int d = 0; d < 4; ++d) { blo[d] = us2{0, 0}; bhi[d] = us2{0, 0}; }
+    bool any = false;
+    if (!empty)
+    {
+        const uint8_t* xn = x + n * p.H * p.W * p.C + c;
+        v4u raw[WB * WB];
+        const long long first = (static_cast<long long>(min(hstart, p.H - 1)) * p.W + min(wstart, p.W - 1)) * p.C;
+#pragma unroll
+        for (int dy = 0; dy < WB; ++dy)
+#pragma unroll
+            for (int dx = 0; dx < WB; ++dx)
+            {
+                const bool in = hstart + dy < hend && wstart + dx < wend;
+                raw[dy * WB + dx] = *reinterpret_cast<const v4u*>(xn + (in ? (static_cast<long long>(hstart + dy) * p.W + wstart + dx) * p.C : first));
+            }
+        const uint32_t flip = qin.is_u8 ? 0u : 0x80808080u;
+#pragma unroll
+        for (int dy = 0; dy < WB; ++dy)
+#pragma unroll
+            for (int dx = 0; dx < WB; ++dx)
+            {
+                if (hstart + dy < hend && wstart + dx < wend)
+                {
+                    any = true;
+#pragma unroll
+                    for (int d = 0; d < 4; ++d)
+                    {
+                        const uint32_t w = raw[dy * WB + dx][d] ^ flip;
+                        const uint32_t lo = w & 0x00ff00ffu, hi = (w >> 8) & 0x00ff00ffu;
+                        blo[d] = __builtin_elementwise_max(blo[d], __builtin_bit_cast(us2, lo));
+                        bhi[d] = __builtin_elementwise_max(bhi[d], __builtin_bit_cast(us2, hi));
+                    }
+                }
+            }
+    }
+    v4u out;
+    const int unflip = qin.is_u8 ? 0 : 128;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+    {
+        const int code[4] = {static_cast<int>(blo[d].x) - unflip, static_cast<int>(bhi[d].x) - unflip, static_cast<int>(blo[d].y) - unflip,
+                             static_cast<int>(bhi[d].y) - unflip};
+        float res[4];
+#pragma unroll
+        // a window wholly outside the padded extent gives 0.0 ("nothing to pool"), one that only covers padding the lowest value
+        for (int ch = 0; ch < 4; ++ch)
+            res[ch] = any ? __fmul_rn(static_cast<float>(code[ch] - qin.offset), qin.scale) : empty ? 0.0f : -FLT_MAX;
+        out[d] = QuantizePack4Dev(res[0], res[1], res[2], res[3], rq);
+    }
+    *reinterpret_cast<v4u*>(y + idx * 16) = out;
+}
+
 // The window is the whole image (global pooling): a block owns 256 channels of one image.  All threads fetch the
 // image's taps as dwords into LDS at once; then thread c walks channel c's taps in the reference's order (row by row),
 // so the fp32 sum is the reference's sum.  `taps` = H * W, at most kGlobalPoolMaxTaps.
@@ -503,6 +586,13 @@ int mi355x_pool2d_run(const mi355x_pool2d_desc* d, uint32_t batch, const void* i
         NoteKernel("GlobalPoolKernel");
         hipLaunchKernelGGL(GlobalPoolKernel, dim3(static_cast<unsigned>(batch * ((p.C + 255) / 256))), dim3(256), 0, ToHip(stream), p,
                            MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev));
+    }
+    else if (p.is_max && (p.C % 16) == 0 && p.pool_w <= 3 && p.pool_h <= 3 && (reinterpret_cast<uintptr_t>(input_dev) & 15) == 0 &&
+             (reinterpret_cast<uintptr_t>(output_dev) & 15) == 0)
+    {
+        NoteKernel("MaxPool2dC16Kernel<3>");
+        hipLaunchKernelGGL(MaxPool2dC16Kernel<3>, dim3(static_cast<unsigned>((total / 16 + 255) / 256)), dim3(256), 0, ToHip(stream), p,
+                           MakeQIn(d->input), rq, static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), total / 16);
     }
     else if (vec4 && p.pool_w <= 3 && p.pool_h <= 3)
     {

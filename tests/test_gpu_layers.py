@@ -19,9 +19,12 @@ def _rand(seed, shape, dtype, scale, offset):
 
 
 POOLS = [
-    # (name, shape, pool_type, pw, ph, sx, sy, pads l r t b)  -- channel counts hit the 4-channel and the scalar kernel
+    # (name, shape, pool_type, pw, ph, sx, sy, pads l r t b)  -- channel counts hit the 16-channel max kernel, the 4-channel and the scalar kernel
     ("max3x3s2_c64", (2, 23, 21, 64), cpuref.POOL_MAX, 3, 3, 2, 2, (1, 1, 1, 1)),
     ("max3x3s2_c5", (1, 11, 13, 5), cpuref.POOL_MAX, 3, 3, 2, 2, (1, 1, 1, 1)),
+    ("max3x3s1_c16_pad", (1, 6, 7, 16), cpuref.POOL_MAX, 3, 3, 1, 1, (1, 1, 1, 1)),
+    ("max2x2s2_c32", (3, 9, 8, 32), cpuref.POOL_MAX, 2, 2, 2, 2, (0, 1, 0, 1)),
+    ("max3x2s3_c48_window_in_the_padding", (2, 5, 4, 48), cpuref.POOL_MAX, 3, 2, 3, 3, (3, 3, 2, 2)),
     ("avg7x7_global_c1024", (3, 7, 7, 1024), cpuref.POOL_AVERAGE, 7, 7, 1, 1, (0, 0, 0, 0)),
     ("max14x14_global_c300", (2, 14, 14, 300), cpuref.POOL_MAX, 14, 14, 1, 1, (0, 0, 0, 0)),
     ("avg3x5_global_c8", (5, 5, 3, 8), cpuref.POOL_AVERAGE, 3, 5, 2, 2, (0, 0, 0, 0)),
