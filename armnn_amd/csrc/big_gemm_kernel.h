@@ -378,6 +378,7 @@ __global__ __launch_bounds__(256) void BigGemmKernel(IgemmArgs a, int xcd_rows)
     const int oc = tid % CHUNKS;
     const int orow = tid / CHUNKS;
     const int c0 = tn * BN + oc * 16;
+    const OutPtr outp = MakeOutPtr(a.y, static_cast<long long>(a.M) * a.Co);
     if ((a.Co & 15) == 0)
     {
         if (c0 < a.Co)
@@ -387,7 +388,7 @@ __global__ __launch_bounds__(256) void BigGemmKernel(IgemmArgs a, int xcd_rows)
             {
                 const int m = tm * BM + r;
                 if (m < a.M)
-                    StoreOut16(a.y + static_cast<long long>(m) * a.Co + c0, *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16));
+                    StoreOut16(outp, static_cast<long long>(m) * a.Co + c0, *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16));
             }
         }
     }

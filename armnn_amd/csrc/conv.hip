@@ -78,6 +78,16 @@ struct mi355x_fc_s
 
 namespace
 {
+// An Addition waiting to be fused into the next launch of this thread (mi355x_conv2d_run_add): the launchers whose
+// kernels can do it take it and mark it taken; otherwise the caller runs the Addition as a launch of its own.
+struct PendingAdd
+{
+    const uint8_t* other = nullptr;
+    AddFuse fuse{};
+    bool taken = false;
+};
+thread_local PendingAdd* t_pending_add = nullptr;
+
 // unit roundoff of fp32 and the relative half-width of the requantization bracket (device_math.h)
 constexpr double kBracketUnit = 1.0 / 16777216.0;
 constexpr double kBracketRel = 16.0 / 16777216.0;
@@ -584,6 +594,13 @@ int LaunchPw(const mi355x_conv2d_s* p, long long M, const void* x, void* y, hipS
     a.xor_mask = p->xor_mask;
     a.zw_neg = p->zw_neg;
     a.rq = p->rq;
+    a.res = nullptr;
+    if (t_pending_add && (g.Co & 15) == 0)
+    {
+        a.res = t_pending_add->other;
+        a.add = t_pending_add->fuse;
+        t_pending_add->taken = true;
+    }
     const int smem = PwSmemBytes<BN>(g.Ci);
     auto kernel = p->zw_neg != 0 ? PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2), true> : PwGemmKernel<BN, KS, (KS <= 2 ? 4 : 2), false>;
     const int n_cu = p->pw_n_cu, cached_per_cu = p->pw_blocks_per_cu;      // queried once, when the plan was built
@@ -697,6 +714,12 @@ int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, voi
     a.zw_neg = p->zw_neg;
     a.rowsum_bias = p->rowsum_bias;
     a.rq = p->rq;
+    if (t_pending_add && (g.Co & 15) == 0)
+    {
+        a.res = t_pending_add->other;
+        a.add = t_pending_add->fuse;
+        t_pending_add->taken = true;
+    }
     const int nblocks = a.tiles_m * a.tiles_n;
     const int grid = (nblocks + 7) / 8 * 8;
     constexpr int smem = IgemmLdsSmemBytes<BM, BN, ST>();
@@ -1311,6 +1334,30 @@ int mi355x_conv2d_create(const mi355x_conv2d_desc* desc, const void* weights_hos
 int mi355x_conv2d_run(mi355x_conv2d_t plan, uint32_t batch, const void* input_dev, void* output_dev, mi355x_stream_t stream)
 {
     return RunPlan(plan, batch, input_dev, output_dev, ToHip(stream));
+}
+
+int mi355x_conv2d_run_add(mi355x_conv2d_t plan, uint32_t batch, const void* input_dev, const void* other_dev, const mi355x_quant* other_quant,
+                          const mi355x_quant* sum_quant, int32_t activation, float a, float b, void* output_dev, mi355x_stream_t stream)
+{
+    if (!plan) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
+    if (!other_quant || !sum_quant) return SetError(MI355X_ERR_INVALID_ARGUMENT, "quantization of the Addition is null");
+    if (activation < MI355X_ACT_NONE || activation > MI355X_ACT_BOUNDED_RELU) return SetError(MI355X_ERR_UNSUPPORTED, "activation %d", activation);
+    if (batch == 0) return 0;
+    if (!other_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "other input / output pointer is null");
+    if (other_dev == output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "the Addition's other input may not be the output buffer");
+    PendingAdd pending;
+    pending.other = static_cast<const uint8_t*>(other_dev);
+    pending.fuse.qa = MakeQIn(plan->d.output);
+    pending.fuse.qr = MakeQIn(*other_quant);
+    pending.fuse.rq = MakeRequant(*sum_quant, activation, a, b);
+    const bool aligned = (reinterpret_cast<uintptr_t>(other_dev) & 15) == 0 && (reinterpret_cast<uintptr_t>(output_dev) & 15) == 0;
+    t_pending_add = aligned ? &pending : nullptr;
+    const int rc = RunPlan(plan, batch, input_dev, output_dev, ToHip(stream));
+    t_pending_add = nullptr;
+    if (rc != 0 || pending.taken) return rc;
+    // the kernel this launch resolved to writes its tiles some other way: the Addition runs behind it, in place
+    const size_t n = static_cast<size_t>(batch) * plan->d.out_h * plan->d.out_w * plan->d.out_c;
+    return mi355x_add_run(n, &plan->d.output, other_quant, sum_quant, activation, a, b, output_dev, other_dev, output_dev, stream);
 }
 
 int mi355x_conv2d_fusable(mi355x_conv2d_t dw, mi355x_conv2d_t pw)

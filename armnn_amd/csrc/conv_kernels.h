@@ -181,6 +181,8 @@ struct IgemmArgs
     int zw_neg;             // minus the zero point of the stored int8 weights (0: symmetric)
     int rowsum_bias;        // (K_pad - K) * zx': what the bytes beyond K add to a row sum
     Requant rq;
+    const uint8_t* res = nullptr;   // direct-to-LDS kernel: the other input of an Addition fused into the write-out ([M][Co]), or null
+    AddFuse add;
 };
 
 // K is walked in tiles of BK bytes per GEMM row.  BK = 128 makes every row chunk a whole 128-byte cache line: with 64-byte
@@ -446,6 +448,7 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
     const int oc = tid % CHUNKS;
     const int orow = tid / CHUNKS;
     const int c0 = tn * BN + oc * 16;
+    const OutPtr outp = MakeOutPtr(a.y, static_cast<long long>(a.M) * a.Co);
     if ((a.Co & 15) == 0)
     {
         if (c0 < a.Co)
@@ -457,7 +460,7 @@ __global__ __launch_bounds__(256) void IgemmKernel(IgemmArgs a)
                 if (m < a.M)
                 {
                     const v4i v = *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16);
-                    StoreOut16(a.y + static_cast<long long>(m) * a.Co + c0, v);
+                    StoreOut16(outp, static_cast<long long>(m) * a.Co + c0, v);
                 }
             }
         }

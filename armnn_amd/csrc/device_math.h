@@ -66,29 +66,47 @@ struct ChanTab
 // nothing to overlap it.  With the sc1 bit (agent scope) the L2 writes the line through as the store is issued, so the
 // write-back runs beside the rest of the kernel and the data is where the next kernel -- whose blocks run on any XCD --
 // reads it from.  (The nt bit instead also helps a kernel timed alone but makes the next layer slower.)  Only for stores
-// that cover whole lines per instruction: the depthwise kernel's 32-byte pieces and the pooling kernel's dwords, written
-// through one by one, are slower than ordinary stores that L2 merges.
+// that cover whole lines per instruction: the 32-channel depthwise blocks' 32-byte pieces and the pooling kernel's dwords,
+// written through one by one, are slower than ordinary stores that L2 merges.
+//   The bit is set through the buffer-store builtins (their cache-policy argument), which the compiler knows as vector
+// memory instructions; a hand-written store instruction in inline assembly is invisible to its hazard and wait-count
+// bookkeeping and produced wrong bytes now and then.  A buffer store takes a wave-uniform base and an unsigned 32-bit
+// byte offset, so tensors of 4 GiB and more fall back to ordinary stores.
 #ifndef MI355X_STORE_THROUGH
 #define MI355X_STORE_THROUGH 1
 #endif
 typedef int StoreVec4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ void StoreOut16(void* p, const StoreVec4& v)
+struct OutPtr
 {
-#if MI355X_STORE_THROUGH
-    asm volatile("global_store_dwordx4 %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-#else
-    *reinterpret_cast<StoreVec4*>(p) = v;
-#endif
+    __amdgpu_buffer_rsrc_t rsrc;
+    uint8_t* base;
+    bool through;
+};
+
+// `base` must be the same in every lane of the wave (a kernel argument, or derived from block-uniform values)
+__device__ __forceinline__ OutPtr MakeOutPtr(uint8_t* base, long long bytes)
+{
+    OutPtr o;
+    o.base = base;
+    o.through = MI355X_STORE_THROUGH != 0 && bytes > 0 && bytes <= 0xffffffffll;
+    o.rsrc = __builtin_amdgcn_make_buffer_rsrc(base, 0, -1, 0x00020000);
+    return o;
 }
 
-__device__ __forceinline__ void StoreOut4(void* p, uint32_t v)
+constexpr int kStoreAuxSc1 = 16;     // cache-policy operand of the buffer-store builtins: bit 4 = sc1
+
+__device__ __forceinline__ void StoreOut16(const OutPtr& o, long long offset, const StoreVec4& v)
 {
-#if MI355X_STORE_THROUGH
-    asm volatile("global_store_dword %0, %1, off sc1" ::"v"(p), "v"(v) : "memory");
-#else
-    *reinterpret_cast<uint32_t*>(p) = v;
-#endif
+    typedef unsigned int U4 __attribute__((ext_vector_type(4)));
+    if (o.through) __builtin_amdgcn_raw_buffer_store_b128(__builtin_bit_cast(U4, v), o.rsrc, static_cast<int>(offset), 0, kStoreAuxSc1);
+    else *reinterpret_cast<StoreVec4*>(o.base + offset) = v;
+}
+
+__device__ __forceinline__ void StoreOut4(const OutPtr& o, long long offset, uint32_t v)
+{
+    if (o.through) __builtin_amdgcn_raw_buffer_store_b32(v, o.rsrc, static_cast<int>(offset), 0, kStoreAuxSc1);
+    else *reinterpret_cast<uint32_t*>(o.base + offset) = v;
 }
 
 __device__ __forceinline__ uint32_t Pack4(int q0, int q1, int q2, int q3)
@@ -250,6 +268,65 @@ __device__ __forceinline__ uint32_t QuantizePack4Dev(float f0, float f1, float f
                 out = (out & ~(0xffu << (8 * i))) | ((static_cast<uint32_t>(QuantizeDev(f[i], rq) + rq.pk_bias) & 0xffu) << (8 * i));
     }
     return out ^ rq.pk_xor;
+}
+
+struct QIn
+{
+    float scale;
+    int   offset;
+    int   is_u8;
+};
+
+__device__ __forceinline__ float DequantDev(uint8_t code, const QIn& q)
+{
+    const int v = q.is_u8 ? static_cast<int>(code) : static_cast<int>(static_cast<int8_t>(code));
+    return __fmul_rn(static_cast<float>(v - q.offset), q.scale);   // armnn::Dequantize, TypesUtils.cpp:47-56
+}
+
+// The four codes of a dword -> float values: signed codes are made unsigned with one xor for the dword (offset moves by
+// 128 with them), then v_cvt_f32_ubyteN converts byte N directly; value - offset is an exact small integer either way,
+// so the single multiplication rounds exactly as in armnn::Dequantize.
+__device__ __forceinline__ void Dequant4Dev(uint32_t w, const QIn& q, float (&v)[4])
+{
+    const uint32_t u = q.is_u8 ? w : (w ^ 0x80808080u);
+    const float off = static_cast<float>(q.is_u8 ? q.offset : q.offset + 128);
+    v[0] = __fmul_rn(__fsub_rn(static_cast<float>(u & 0xffu), off), q.scale);
+    v[1] = __fmul_rn(__fsub_rn(static_cast<float>((u >> 8) & 0xffu), off), q.scale);
+    v[2] = __fmul_rn(__fsub_rn(static_cast<float>((u >> 16) & 0xffu), off), q.scale);
+    v[3] = __fmul_rn(__fsub_rn(static_cast<float>(u >> 24), off), q.scale);
+}
+
+inline QIn MakeQIn(const mi355x_quant& q)
+{
+    QIn r;
+    r.scale = q.scale;
+    r.offset = q.offset;
+    r.is_u8 = q.dtype == MI355X_QASYMM_U8;
+    return r;
+}
+
+// The Addition that follows a convolution, run inside the convolution's write-out: `own` are sixteen finished output
+// codes of the convolution (quantization qa), `other` the sixteen codes of the Addition's other input (qr); the sum is
+// formed and quantized exactly as the Addition layer does it (dequantize both, one fp32 add, quantize with the
+// Addition's output quantization and its fused activation), so the bytes are those of the two layers run apart.
+struct AddFuse
+{
+    QIn qa, qr;
+    Requant rq;
+};
+
+__device__ __forceinline__ StoreVec4 AddResidual16(const StoreVec4& own, const StoreVec4& other, const AddFuse& f)
+{
+    StoreVec4 o;
+#pragma unroll
+    for (int d = 0; d < 4; ++d)
+    {
+        float va[4], vb[4];
+        Dequant4Dev(static_cast<uint32_t>(own[d]), f.qa, va);
+        Dequant4Dev(static_cast<uint32_t>(other[d]), f.qr, vb);
+        o[d] = static_cast<int>(QuantizePack4Dev(__fadd_rn(va[0], vb[0]), __fadd_rn(va[1], vb[1]), __fadd_rn(va[2], vb[2]), __fadd_rn(va[3], vb[3]), f.rq));
+    }
+    return o;
 }
 
 } // namespace mi355x

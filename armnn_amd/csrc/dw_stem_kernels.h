@@ -203,6 +203,7 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
 
     // ---- epilogue ------------------------------------------------------------------------------------------------
     const Fast4 f4 = LoadFast4(a.ct, c);
+    const OutPtr outp = MakeOutPtr(a.y, static_cast<long long>(a.N) * a.Ho * a.Wo * a.C);
 #pragma unroll
     for (int o = 0; o < R; ++o)
     {
@@ -218,7 +219,7 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
                 const uint32_t q = Requant4Dev(acc[o][j][0], acc[o][j][1], acc[o][j][2], acc[o][j][3], f4, a.ct, c, a.rq);
                 // CB = 32: an ordinary store, these 32-byte pieces of a line are merged in L2 (written through one by one they
                 // are slower); CB = 128: half a wave stores a whole line
-                if constexpr (CB == 128) StoreOut4(yrow + static_cast<long long>(ox) * a.C, q);
+                if constexpr (CB == 128) StoreOut4(outp, (yrow - a.y) + static_cast<long long>(ox) * a.C, q);
                 else *reinterpret_cast<uint32_t*>(yrow + static_cast<long long>(ox) * a.C) = q;
             }
         }
@@ -574,6 +575,7 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
             for (int j = 0; j < 4; ++j) bfrag[t][j] = static_cast<int>(half ? flat[8 * t + 4 + j] : flat[8 * t + j]);
 
         uint8_t* yp = a.y + ((static_cast<long long>(n) * a.Ho + oy) * a.Wo + ox) * a.Co;
+        const OutPtr outp = MakeOutPtr(a.y, static_cast<long long>(a.N) * a.Ho * a.Wo * a.Co);
 #pragma unroll
         for (int ct = 0; ct < NT; ++ct)
         {
@@ -604,7 +606,7 @@ __global__ __launch_bounds__(256) void SmallCiMfmaKernel(SmallCiArgs a)
             const uint4 v = half ? uint4{r0, o[2], r1, o[3]} : uint4{o[0], r0, o[1], r1};
             if (ox < a.Wo)
             {
-                if (a.vec16) StoreOut16(yp + ct * 32 + 16 * half, StoreVec4{static_cast<int>(v.x), static_cast<int>(v.y), static_cast<int>(v.z), static_cast<int>(v.w)});
+                if (a.vec16) StoreOut16(outp, (yp - a.y) + ct * 32 + 16 * half, StoreVec4{static_cast<int>(v.x), static_cast<int>(v.y), static_cast<int>(v.z), static_cast<int>(v.w)});
                 else
                 {
                     uint32_t* dst = reinterpret_cast<uint32_t*>(yp + ct * 32 + 16 * half);

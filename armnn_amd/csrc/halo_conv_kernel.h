@@ -266,12 +266,13 @@ __global__ __launch_bounds__(256) void HaloConvKernel(HaloArgs a)
     const int orow = tid / CHUNKS;
     const int c0 = tn * BN + oc * 16;
     uint8_t* yt = a.y + (static_cast<long long>(n) * a.Ho + y0) * a.Wo * a.Co;     // the tile's rows are contiguous in the output
+    const OutPtr outp = MakeOutPtr(yt, static_cast<long long>(mt) * a.Co);
     if ((a.Co & 15) == 0)
     {
         if (c0 < a.Co)
         {
             for (int r = orow; r < mt; r += ROWS_PER_PASS)
-                StoreOut16(yt + static_cast<long long>(r) * a.Co + c0, *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16));
+                StoreOut16(outp, static_cast<long long>(r) * a.Co + c0, *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16));
         }
     }
     else

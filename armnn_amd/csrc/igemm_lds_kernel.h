@@ -329,6 +329,7 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
     const int oc = tid % CHUNKS;
     const int orow = tid / CHUNKS;
     const int c0 = tn * BN + oc * 16;
+    const OutPtr outp = MakeOutPtr(a.y, static_cast<long long>(a.M) * a.Co);
     if ((a.Co & 15) == 0)
     {
         if (c0 < a.Co)
@@ -338,7 +339,11 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
             {
                 const int m = tm * BM + r;
                 if (m < a.M)
-                    StoreOut16(a.y + static_cast<long long>(m) * a.Co + c0, *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16));
+                {
+                    v4i ov = *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16);
+                    if (a.res) ov = AddResidual16(ov, *reinterpret_cast<const v4i*>(a.res + static_cast<long long>(m) * a.Co + c0), a.add);
+                    StoreOut16(outp, static_cast<long long>(m) * a.Co + c0, ov);
+                }
             }
         }
     }

@@ -16,32 +16,6 @@ typedef unsigned int v4u __attribute__((ext_vector_type(4)));
 namespace
 {
 
-struct QIn
-{
-    float scale;
-    int   offset;
-    int   is_u8;
-};
-
-__device__ __forceinline__ float DequantDev(uint8_t code, const QIn& q)
-{
-    const int v = q.is_u8 ? static_cast<int>(code) : static_cast<int>(static_cast<int8_t>(code));
-    return __fmul_rn(static_cast<float>(v - q.offset), q.scale);   // armnn::Dequantize, TypesUtils.cpp:47-56
-}
-
-// The four codes of a dword -> float values: signed codes are made unsigned with one xor for the dword (offset moves by
-// 128 with them), then v_cvt_f32_ubyteN converts byte N directly; value - offset is an exact small integer either way,
-// so the single multiplication rounds exactly as in armnn::Dequantize.
-__device__ __forceinline__ void Dequant4Dev(uint32_t w, const QIn& q, float (&v)[4])
-{
-    const uint32_t u = q.is_u8 ? w : (w ^ 0x80808080u);
-    const float off = static_cast<float>(q.is_u8 ? q.offset : q.offset + 128);
-    v[0] = __fmul_rn(__fsub_rn(static_cast<float>(u & 0xffu), off), q.scale);
-    v[1] = __fmul_rn(__fsub_rn(static_cast<float>((u >> 8) & 0xffu), off), q.scale);
-    v[2] = __fmul_rn(__fsub_rn(static_cast<float>((u >> 16) & 0xffu), off), q.scale);
-    v[3] = __fmul_rn(__fsub_rn(static_cast<float>(u >> 24), off), q.scale);
-}
-
 __device__ __forceinline__ float ActivationDev(float in, int fn, float a, float b)
 {
     if (fn == MI355X_ACT_RELU) return fmaxf(0.0f, in);
@@ -49,14 +23,6 @@ __device__ __forceinline__ float ActivationDev(float in, int fn, float a, float 
     return in;
 }
 
-QIn MakeQIn(const mi355x_quant& q)
-{
-    QIn r;
-    r.scale = q.scale;
-    r.offset = q.offset;
-    r.is_u8 = q.dtype == MI355X_QASYMM_U8;
-    return r;
-}
 
 // A per-element function of one 8-bit code: build the 256-entry table once per block, then stream.
 __global__ __launch_bounds__(256) void ActivationKernel(QIn qin, Requant rq, int fn, float a, float b,
@@ -364,6 +330,7 @@ __global__ __launch_bounds__(256) void GlobalPoolKernel(PoolArgs p, QIn qin, Req
 __global__ __launch_bounds__(256) void AddVec16Kernel(QIn q0, QIn q1, Requant rq, const v4u* __restrict__ x0,
                                                       const v4u* __restrict__ x1, v4u* __restrict__ y, size_t n16)
 {
+    const OutPtr outp = MakeOutPtr(reinterpret_cast<uint8_t*>(y), static_cast<long long>(n16) * 16);
     size_t i = static_cast<size_t>(blockIdx.x) * 256 + threadIdx.x;
     const size_t stride = static_cast<size_t>(gridDim.x) * 256;
     for (; i < n16; i += stride)
@@ -378,7 +345,7 @@ __global__ __launch_bounds__(256) void AddVec16Kernel(QIn q0, QIn q1, Requant rq
             Dequant4Dev(b[d], q1, vb);
             o[d] = QuantizePack4Dev(__fadd_rn(va[0], vb[0]), __fadd_rn(va[1], vb[1]), __fadd_rn(va[2], vb[2]), __fadd_rn(va[3], vb[3]), rq);
         }
-        StoreOut16(y + i, StoreVec4{static_cast<int>(o[0]), static_cast<int>(o[1]), static_cast<int>(o[2]), static_cast<int>(o[3])});
+        StoreOut16(outp, static_cast<long long>(i) * 16, StoreVec4{static_cast<int>(o[0]), static_cast<int>(o[1]), static_cast<int>(o[2]), static_cast<int>(o[3])});
     }
 }
 

@@ -37,6 +37,8 @@ struct PwArgs
     int n_slabs, gm;         // grid = n_slabs * gm blocks; block (slab, g) takes tile groups g, g+gm, ...
     uint32_t xor_mask;
     int zw_neg;              // AW: minus the zero point of the stored int8 weights
+    const uint8_t* res;      // the other input of an Addition fused into the write-out ([M][N]), or null
+    AddFuse add;
     Requant rq;
 };
 
@@ -74,6 +76,7 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
 
     uint8_t* ostage = ostage_all + wave * 32 * LDO;
     const int n_tiles = (a.M + 31) >> 5;
+    const OutPtr outp = MakeOutPtr(a.y, static_cast<long long>(a.M) * a.N);
     const int nch = a.K / (32 * KS);
     const int frag_row = lane & 31;
     const int frag_k = (lane >> 5) * 16;
@@ -152,9 +155,9 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
                 const int c0 = n0 + cc * 16;
                 if (row < a.M && c0 < a.N)
                 {
-                    const v4i ov = *reinterpret_cast<const v4i*>(ostage + r * LDO + cc * 16);
-                    uint8_t* dst = a.y + static_cast<long long>(row) * a.N + c0;
-                    StoreOut16(dst, ov);
+                    v4i ov = *reinterpret_cast<const v4i*>(ostage + r * LDO + cc * 16);
+                    if (a.res) ov = AddResidual16(ov, *reinterpret_cast<const v4i*>(a.res + static_cast<long long>(row) * a.N + c0), a.add);
+                    StoreOut16(outp, static_cast<long long>(row) * a.N + c0, ov);
                 }
             }
         }

@@ -15,15 +15,15 @@ from .tensor import QTensor, numpy_dtype
 
 @dataclass
 class FusedPair:
-    """Two neighbouring layers -- depthwise + the pointwise convolution consuming it, or pointwise + the depthwise
-    consuming it -- launched as one kernel."""
+    """Two neighbouring layers -- depthwise + the pointwise convolution consuming it, pointwise + the depthwise consuming
+    it, or a convolution + the Addition consuming it (op "convadd") -- launched as one kernel."""
     name: str
     parts: Tuple                       # (first Layer, second Layer)
     op: str = "dwpw"
 
     @property
     def inputs(self):
-        return self.parts[0].inputs
+        return tuple(self.parts[0].inputs) + tuple(i for i in self.parts[1].inputs if i != self.parts[0].output)
 
     @property
     def output(self):
@@ -36,7 +36,7 @@ class FusedPair:
 
 class DeviceNetwork:
     def __init__(self, net: Network, batch: int, algo_overrides: Optional[Dict[str, int]] = None, use_graph: bool = True,
-                 fuse: bool = False, lanes: int = 1):
+                 fuse: bool = False, lanes: int = 1, fuse_add: bool = True):
         """lanes > 1 splits the batch into that many contiguous slices; each slice runs the whole network on a stream of
         its own (the same plans, pointers offset to the slice), so one slice's kernels fill the ramp-up, tail and
         launch gaps of the others. Results do not depend on the split: every image is computed independently."""
@@ -114,8 +114,11 @@ class DeviceNetwork:
                 self._step_plans.append(None)
             else:
                 raise ValueError(l.op)
-        if fuse:
+        self._plan_of = {id(l): pl for (l, _), pl in zip(self.steps, self._step_plans)}
+        if fuse in ("dwpw", "pwdw", True):
             self._fuse_pairs(("conv", "depthwise") if fuse == "pwdw" else ("depthwise", "conv"))
+        if fuse_add:
+            self._fuse_additions()
 
     def _fuse_pairs(self, ops):
         """Replace neighbours (depthwise 3x3, 1x1 convolution) -- or, with ops = ("conv", "depthwise"), (1x1 convolution,
@@ -126,7 +129,7 @@ class DeviceNetwork:
         for l in net.layers:
             for i in l.inputs:
                 consumers[i] = consumers.get(i, 0) + 1
-        plan_of = {id(l): pl for (l, _), pl in zip(self.steps, self._step_plans)}
+        plan_of = self._plan_of
         fused, k = [], 0
         while k < len(self.steps):
             l, fn = self.steps[k]
@@ -141,6 +144,38 @@ class DeviceNetwork:
                 fused.append((FusedPair(f"{l.name}+{nxt.name}", (l, nxt)),
                               (lambda pdw, ppw, x, y, nx, ny: lambda s, lane=0, lanes=1: pdw.run_fused(
                                   ppw, batch // lanes, x + lane * (nx // lanes), y + lane * (ny // lanes), s))(pdw, ppw, x, y, nx, ny)))
+                k += 2
+            else:
+                fused.append((l, fn))
+                k += 1
+        self.steps = fused
+
+    def _fuse_additions(self):
+        """A convolution whose output only feeds the Addition launched right behind it (the last convolution of a residual
+        block) runs that Addition inside its own write-out (Conv2dPlan.run_add): same bytes, one launch and one round trip
+        of the tensor less.  The Addition's other input was produced earlier, so launch order is unchanged."""
+        net = self.net
+        consumers: Dict[str, int] = {}
+        for l in net.layers:
+            for i in l.inputs:
+                consumers[i] = consumers.get(i, 0) + 1
+        plan_of = self._plan_of
+        fused, k = [], 0
+        while k < len(self.steps):
+            l, fn = self.steps[k]
+            nxt = self.steps[k + 1][0] if k + 1 < len(self.steps) else None
+            if (l.op == "conv" and nxt is not None and nxt.op == "add" and l.output in nxt.inputs and nxt.inputs[0] != nxt.inputs[1] and
+                    consumers.get(l.output, 0) == 1 and l.output != net.output and isinstance(plan_of.get(id(l)), shim.Conv2dPlan)):
+                plan = plan_of[id(l)]
+                other = nxt.inputs[1] if nxt.inputs[0] == l.output else nxt.inputs[0]
+                x, o, y = self.buffers[l.inputs[0]].ptr, self.buffers[other].ptr, self.buffers[nxt.output].ptr
+                nx, ny = net.info(l.inputs[0], self.batch).num_elements, net.info(nxt.output, self.batch).num_elements
+                oi, si = net.info(other, self.batch), net.info(nxt.output, self.batch)
+                batch, act = self.batch, nxt.act
+                fused.append((FusedPair(f"{l.name}+{nxt.name}", (l, nxt), op="convadd"),
+                              (lambda plan, x, o, y, nx, ny, oi, si, act: lambda s, lane=0, lanes=1: plan.run_add(
+                                  batch // lanes, x + lane * (nx // lanes), o + lane * (ny // lanes), oi, si, y + lane * (ny // lanes),
+                                  activation=act[0], act_a=act[1], act_b=act[2], stream=s))(plan, x, o, y, nx, ny, oi, si, act)))
                 k += 2
             else:
                 fused.append((l, fn))

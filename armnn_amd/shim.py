@@ -28,7 +28,7 @@ EXPORTS = [
     "mi355x_event_destroy", "mi355x_event_record", "mi355x_stream_wait_event", "mi355x_event_synchronize", "mi355x_event_elapsed_ms",
     "mi355x_graph_capture_begin", "mi355x_graph_capture_end", "mi355x_graph_launch", "mi355x_graph_destroy",
     "mi355x_conv2d_create", "mi355x_conv2d_run", "mi355x_conv2d_destroy", "mi355x_conv2d_algo",
-    "mi355x_conv2d_fusable", "mi355x_conv2d_run_fused",
+    "mi355x_conv2d_fusable", "mi355x_conv2d_run_fused", "mi355x_conv2d_run_add",
     "mi355x_fc_create", "mi355x_fc_run", "mi355x_fc_destroy", "mi355x_fc_algo",
     "mi355x_activation_run", "mi355x_pool2d_run", "mi355x_add_run", "mi355x_softmax_run", "mi355x_pad_run",
 ]
@@ -112,6 +112,7 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
             "mi355x_conv2d_run": [V, C.c_uint32, V, V, V], "mi355x_conv2d_destroy": [V],
             "mi355x_conv2d_algo": [V, C.POINTER(C.c_int32), C.c_char_p, C.c_size_t],
             "mi355x_conv2d_fusable": [V, V], "mi355x_conv2d_run_fused": [V, V, C.c_uint32, V, V, V],
+            "mi355x_conv2d_run_add": [V, C.c_uint32, V, V, C.POINTER(Quant), C.POINTER(Quant), C.c_int32, C.c_float, C.c_float, V, V],
             "mi355x_fc_create": [C.POINTER(FcDesc), V, C.POINTER(ConstQuant), V, C.POINTER(ConstQuant), C.POINTER(V)],
             "mi355x_fc_run": [V, C.c_uint32, V, V, V], "mi355x_fc_destroy": [V],
             "mi355x_fc_algo": [V, C.POINTER(C.c_int32), C.c_char_p, C.c_size_t],
@@ -305,6 +306,14 @@ class Conv2dPlan:
     def run_fused(self, second: "Conv2dPlan", batch: int, x_dev: int, y_dev: int, stream=None):
         """Both layers without the intermediate tensor; bytes equal run() + second.run()."""
         _chk(self.lib.mi355x_conv2d_run_fused(self.plan, second.plan, batch, x_dev, y_dev, stream))
+
+    def run_add(self, batch: int, x_dev: int, other_dev: int, other_info: TensorInfo, sum_info: TensorInfo, y_dev: int,
+                activation=ACT_NONE, act_a=0.0, act_b=0.0, stream=None):
+        """This convolution and the Addition consuming it in one launch where the kernel can; bytes equal run() followed
+        by the Addition (the other input in `other_dev`, the sum quantized as `sum_info`, then the activation)."""
+        qo, qs = _quant(other_info), _quant(sum_info)
+        _chk(self.lib.mi355x_conv2d_run_add(self.plan, batch, x_dev, other_dev, C.byref(qo), C.byref(qs), activation, act_a, act_b,
+                                            y_dev, stream))
 
     def destroy(self):
         if self.plan:

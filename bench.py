@@ -66,6 +66,8 @@ def layer_work(net, l, batch):
     """(kind, algorithmic work per launch): conv/fc -> ops = 2*MACs; others -> bytes, each tensor once."""
     if l.op in ("conv", "fc"):
         return "mfma", 2.0 * l.macs_per_image * batch
+    if l.op == "convadd":                      # a convolution with the Addition behind it in its write-out
+        return "mfma", 2.0 * l.parts[0].macs_per_image * batch
     if l.op == "dwpw":
         # two layers fused (depthwise + pointwise, in either order): the tensor between them never exists, so the unit's
         # algorithmic bytes are its input, its output and both layers' constants; priced against HBM like the depthwise
@@ -192,6 +194,8 @@ def main():
     ap.add_argument("--fuse", nargs="?", const="dwpw", default="", choices=("dwpw", "pwdw"),
                     help="run pairs of layers as one kernel (same bytes): 'dwpw' depthwise + the pointwise after it, 'pwdw' "
                          "pointwise + the depthwise after it where whole images fit a block")
+    ap.add_argument("--no-fuse-add", action="store_true",
+                    help="launch a residual Addition on its own instead of inside the convolution that feeds it")
     ap.add_argument("--lanes", type=int, default=2,
                     help="split the batch into this many slices, each running the network on a stream of its own")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
@@ -219,7 +223,7 @@ def main():
     from armnn_amd import shim
     from armnn_amd.executor import DeviceNetwork
 
-    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse, lanes=args.lanes)
+    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev
 
@@ -327,7 +331,7 @@ def main():
         w = sum(r["work"] for r in sel)
         return {"ms": t * 1e3, "achieved": w / t, "frac": w / t / peak} if t > 0 else None
 
-    g_conv = group(("conv", "fc"), INT8_MFMA_PEAK_OPS)
+    g_conv = group(("conv", "fc", "convadd"), INT8_MFMA_PEAK_OPS)
     g_dw = group(("depthwise", "dwpw"), HBM_PEAK_BYTES)
     groups = {
         "conv_fc": {"ms": g_conv["ms"], "TOPS": g_conv["achieved"] / 1e12, "frac_of_int8_mfma_peak": g_conv["frac"]},
@@ -338,7 +342,7 @@ def main():
     config = {"workload": f"{net.name} int8 (QAsymm activations, {'per-channel QSymmS8' if args.weights == 'per_channel_s8' or args.net != 'mobilenet_v1' else 'per-tensor QAsymmU8'} weights), batch {batch}, "
                           f"random-init, whole forward pass incl. avgpool/FC/softmax, input resident in HBM, every layer through the C ABI, "
                           f"one HIP graph replay per step",
-              "batch": batch, "graph_replay": not args.no_graph, "fused_pairs": args.fuse or None, "lanes": args.lanes,
+              "batch": batch, "graph_replay": not args.no_graph, "fused_pairs": args.fuse or None, "additions_inside_convolutions": not args.no_fuse_add, "lanes": args.lanes,
               "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12}
     if backend is not None:
         # the same network and input through the C++ backend: wall clock per IRuntime::EnqueueWorkload call, host buffers in

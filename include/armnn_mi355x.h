@@ -199,6 +199,16 @@ int mi355x_conv2d_create(const mi355x_conv2d_desc* desc,
 int mi355x_conv2d_run(mi355x_conv2d_t plan, uint32_t batch, const void* input_dev, void* output_dev,
                       mi355x_stream_t stream);
 int mi355x_conv2d_destroy(mi355x_conv2d_t plan);
+/* A Convolution2d and the Addition that consumes its output (a residual connection), run as one launch where the kernel
+ * the plan resolves to can do it (the matrix-core kernels with 16-byte row stores), else as the convolution followed by
+ * the Addition in place.  other_dev / other_quant: the Addition's other input, same shape as the convolution's output;
+ * sum_quant, activation, a, b: the Addition's output quantization and the activation fused into it.  The convolution's
+ * own output codes are formed first and then added exactly as the Addition layer adds (dequantize both inputs, one
+ * fp32 addition, quantize), so the bytes are those of mi355x_conv2d_run followed by mi355x_add_run -- in the reference
+ * these are two workloads in sequence (RefConvolution2dWorkload.cpp:38-58, then RefElementwiseBinaryWorkload.cpp:27-107). */
+int mi355x_conv2d_run_add(mi355x_conv2d_t plan, uint32_t batch, const void* input_dev, const void* other_dev,
+                          const mi355x_quant* other_quant, const mi355x_quant* sum_quant, int32_t activation, float a, float b,
+                          void* output_dev, mi355x_stream_t stream);
 /* A 3x3 depthwise plan and the plan of the unpadded 1x1 stride-1 Convolution2d that consumes its output, run as one
  * kernel: the depthwise result is requantized to its own int8 codes in on-chip memory and fed to the pointwise GEMM
  * there, so the intermediate tensor is never written.  The bytes produced equal mi355x_conv2d_run(depthwise) followed

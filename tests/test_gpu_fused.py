@@ -5,7 +5,7 @@ import numpy as np
 import pytest
 
 from armnn_amd import shim
-from armnn_amd.tensor import DataType, QTensor, numpy_dtype
+from armnn_amd.tensor import DataType, QTensor, TensorInfo, numpy_dtype
 from tests import cases
 from tests.helpers import lsb_diff
 
@@ -184,3 +184,55 @@ def test_pointwise_then_depthwise_pairs_outside_the_kernels_shape_are_refused():
         xd = shim.DeviceBuffer(pw.x.data.nbytes).upload(pw.x.data)
         yd = shim.DeviceBuffer(other.out_info.num_elements)
         _plan(pw).run_fused(_plan(other), 1, xd.ptr, yd.ptr)
+
+
+# ---- a convolution and the Addition that consumes it (residual connection) as one launch ------------------------------------
+# (name, n, h, w, ci, co, kernel, stride, dtype, activation of the Addition, kernel the launch should resolve to or None)
+CONV_ADD = [
+    ("pointwise_k64_co256_s8_relu", 2, 56, 56, 64, 256, 1, 1, S8, cases.RELU, "PwGemmKernel"),
+    ("pointwise_k128_co512_u8", 3, 28, 28, 128, 512, 1, 1, U8, (0, 0.0, 0.0), "PwGemmKernel"),
+    ("pointwise_k256_co1024_s8_relu", 2, 14, 14, 256, 1024, 1, 1, S8, cases.RELU, "IgemmLdsKernel"),
+    ("projection_k256_co512_stride2_u8_relu6", 2, 56, 56, 256, 512, 1, 2, U8, cases.RELU6, "IgemmLdsKernel"),
+    ("pointwise_k512_co2048_ragged_rows_s8", 3, 7, 7, 512, 2048, 1, 1, S8, cases.RELU, "IgemmLdsKernel"),
+    ("conv3x3_c64_falls_back_to_two_launches", 2, 20, 20, 64, 64, 3, 1, S8, cases.RELU, None),
+    ("pointwise_co40_not_whole_chunks_falls_back", 1, 9, 9, 128, 40, 1, 1, U8, cases.RELU, None),
+]
+
+
+@pytest.mark.parametrize("cfg", CONV_ADD, ids=[c[0] for c in CONV_ADD])
+def test_convolution_with_fused_addition_equals_two_layers(port, cfg):
+    name, n, h, w, ci, co, k, stride, dt, act, kernel = cfg
+    print("conv+add", cfg, flush=True)
+    shim.Device()
+    zp = 3 if dt == U8 else -120
+    c = cases.make_conv_case(name, 1300 + co, n=n, h=h, w=w, ci=ci, co=co, kh=k, kw=k, stride=(stride, stride), in_dtype=dt, in_scale=0.0235,
+                             in_offset=zp, out_scale=0.06, out_offset=zp + 90)
+    plan = _plan(c)
+    rng = np.random.default_rng(77)
+    lo, hi = (0, 255) if dt == U8 else (-128, 127)
+    other_info = TensorInfo(c.out_info.shape, dt, (0.043,), zp + 60)
+    other = QTensor(other_info, rng.integers(lo, hi + 1, size=c.out_info.shape).astype(numpy_dtype(dt)))
+    sum_info = TensorInfo(c.out_info.shape, dt, (0.09,), zp + 5)
+    xd = shim.DeviceBuffer(c.x.data.nbytes).upload(c.x.data)
+    od = shim.DeviceBuffer(other.data.nbytes).upload(other.data)
+    mid = shim.DeviceBuffer(c.out_info.num_elements)
+    yf = shim.DeviceBuffer(c.out_info.num_elements)
+    plan.run(n, xd.ptr, mid.ptr)
+    conv_out = QTensor(c.out_info, mid.download(c.out_info.shape, numpy_dtype(dt)))
+    fn, a, b = act
+    two = shim.add(conv_out, other, sum_info, activation=fn, act_a=a, act_b=b)
+    plan.run_add(n, xd.ptr, od.ptr, other_info, sum_info, yf.ptr, activation=fn, act_a=a, act_b=b)
+    last = shim.last_kernel()
+    fused = yf.download(c.out_info.shape, numpy_dtype(dt))
+    print(f"  {last}; distinct codes {len(np.unique(fused))}", flush=True)
+    if kernel is None:
+        assert last.startswith("Add"), last               # the Addition ran as a launch of its own
+    else:
+        assert last.startswith(kernel), last
+    np.testing.assert_array_equal(fused, two.data)
+    assert len(np.unique(fused)) > 8
+    # and the Addition itself against the oracle, on the device's convolution output
+    want = port.add(conv_out, other, sum_info)
+    if fn:
+        want = port.activation(want, sum_info, fn, a, b)
+    np.testing.assert_array_equal(fused, want.data)

@@ -16,7 +16,7 @@ def _layerwise(port, net, batch):
     independently of drift upstream.  Returns the end-to-end device output as well."""
     x = nets.synthetic_input(net, batch)
     ref = netref.run_network(port, net, x, keep=True)
-    dn = DeviceNetwork(net, batch, use_graph=False, fuse=False)
+    dn = DeviceNetwork(net, batch, use_graph=False, fuse=False, fuse_add=False)
     worst = 0
     for l, fn in dn.steps:
         for name in l.inputs:
@@ -47,6 +47,15 @@ def _layerwise(port, net, batch):
         df.close()
         print(f"{net.name} b{batch}: {n_fused} fused pointwise+depthwise pairs {kw}", flush=True)
         np.testing.assert_array_equal(fused.data, eager.data)
+    # residual Additions inside the write-out of the convolution that feeds them (the default): same bytes
+    da = DeviceNetwork(net, batch, use_graph=False, fuse_add=True)
+    n_add = sum(1 for l, _ in da.steps if l.op == "convadd")
+    with_add = da.run(x)
+    da.close()
+    print(f"{net.name} b{batch}: {n_add} Additions fused into convolutions", flush=True)
+    n_layers = sum(1 for l in net.layers if l.op == "add")
+    assert n_add <= n_layers and (n_add == n_layers or not net.name.startswith("resnet"))     # every residual block of ResNet fuses
+    np.testing.assert_array_equal(with_add.data, eager.data)
     dg = DeviceNetwork(net, batch, use_graph=True, fuse=False)
     g1 = dg.run(x)
     dg.enqueue()
@@ -117,6 +126,11 @@ def _rows_equal_small_batch_runs(net, batch, picks, lanes):
 
 def test_mobilenet_v1_batch64_rows_equal_batch2_runs():
     _rows_equal_small_batch_runs(nets.mobilenet_v1(), 64, (0, 31, 62), lanes=2)
+
+
+def test_mobilenet_v1_batch64_in_one_lane_rows_equal_batch2_runs():
+    # 64 images per launch: the largest launches of the benchmark (persistent blocks walk the most tiles here)
+    _rows_equal_small_batch_runs(nets.mobilenet_v1(), 64, (0, 20, 42, 62), lanes=1)
 
 
 def test_resnet50_batch32_rows_equal_batch2_runs():

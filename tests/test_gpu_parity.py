@@ -330,6 +330,28 @@ def test_depthwise_128_channel_blocks_give_the_same_bytes():
         shim.set_option("dw_cb", 64)
 
 
+def test_launches_of_tens_of_megabytes_equal_the_plain_kernel():
+    """The benchmark networks' largest launches (64 and 32 images of the early MobileNetV1 / ResNet-50 layers: outputs of
+    13 to 51 MB, thousands of blocks, persistent blocks walking many tiles) against the plain one-thread-per-output kernel.
+    Small cases cannot show a store that goes wrong once in a million."""
+    U8 = DataType.QAsymmU8
+    cs = [cases.make_conv_case("big_pw_32_64_n64", 901, n=64, h=112, w=112, ci=32, co=64, kh=1, kw=1, in_dtype=U8, in_offset=0, out_offset=0, act=cases.RELU6),
+          cases.make_conv_case("big_pw_64_128_n32", 902, n=32, h=56, w=56, ci=64, co=128, kh=1, kw=1, in_dtype=U8, in_offset=0, out_offset=0, act=cases.RELU6),
+          cases.make_conv_case("big_pw_128_128_n64", 903, n=64, h=56, w=56, ci=128, co=128, kh=1, kw=1, act=cases.RELU6),
+          cases.make_conv_case("big_pw_256_256_n32", 904, n=32, h=28, w=28, ci=256, co=256, kh=1, kw=1, act=cases.RELU6),
+          cases.make_conv_case("big_stem_n32", 905, n=32, h=224, w=224, ci=3, co=32, stride=(2, 2), in_dtype=U8, in_offset=128, out_offset=0, act=cases.RELU6),
+          cases.make_conv_case("big_c1_n64", 906, n=64, h=56, w=56, ci=64, co=64, act=cases.RELU6),
+          cases.make_conv_case("big_dw_128_n32", 907, n=32, h=56, w=56, ci=128, depthwise=True, in_dtype=U8, in_offset=0, out_offset=0, act=cases.RELU6),
+          cases.make_conv_case("big_dw_128_s2_n32", 908, n=32, h=56, w=56, ci=128, depthwise=True, stride=(2, 2), act=cases.RELU6)]
+    for c in cs:
+        got = _gpu_conv(c, shim.ALGO_AUTO)
+        kernel = shim.last_kernel()
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        bad = int((got.data != want.data).sum())
+        print(f"{c.name}: {got.data.size} outputs, {kernel}, {bad} differ", flush=True)
+        assert bad == 0, f"{c.name} {kernel}: {bad} of {got.data.size} bytes differ"
+
+
 def test_config_c1_full_size(port):
     """Benchmark configuration C1: 1x56x56x64 -> 64, 3x3 SAME, per-channel, ReLU6; expected code range [-128, -8]."""
     c = cases.make_conv_case("C1", 20250101, h=56, w=56, ci=64, co=64, act=cases.RELU6)
