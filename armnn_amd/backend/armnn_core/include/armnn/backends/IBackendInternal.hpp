@@ -51,15 +51,17 @@ public:
         IgnoreUnused(tensorHandleFactoryRegistry);
         return IWorkloadFactoryPtr{};
     }
+    // A backend that is handed model options of its own must override the overloads that take them: the defaults answer
+    // with nothing then (IBackendInternal.cpp:24-58, 88-102).
     virtual IWorkloadFactoryPtr CreateWorkloadFactory(const IMemoryManagerSharedPtr& memoryManager, const ModelOptions& modelOptions) const
     {
-        IgnoreUnused(modelOptions);
+        if (NamesThisBackend(modelOptions)) return IWorkloadFactoryPtr{};
         return CreateWorkloadFactory(memoryManager);
     }
     virtual IWorkloadFactoryPtr CreateWorkloadFactory(TensorHandleFactoryRegistry& tensorHandleFactoryRegistry,
                                                       const ModelOptions& modelOptions) const
     {
-        IgnoreUnused(modelOptions);
+        if (NamesThisBackend(modelOptions)) return IWorkloadFactoryPtr{};
         return CreateWorkloadFactory(tensorHandleFactoryRegistry);
     }
     virtual IWorkloadFactoryPtr CreateWorkloadFactory(TensorHandleFactoryRegistry& tensorHandleFactoryRegistry,
@@ -78,7 +80,7 @@ public:
     virtual ILayerSupportSharedPtr GetLayerSupport() const = 0;
     virtual ILayerSupportSharedPtr GetLayerSupport(const ModelOptions& modelOptions) const
     {
-        IgnoreUnused(modelOptions);
+        if (NamesThisBackend(modelOptions)) return ILayerSupportSharedPtr{};
         return GetLayerSupport();
     }
     virtual OptimizationViews OptimizeSubgraphView(const SubgraphView& subgraph) const;
@@ -114,6 +116,13 @@ public:
         throw armnn::Exception("GetDefaultAllocator: Function has not been implemented in backend.");
     }
     virtual unsigned int GetNumberOfCacheFiles() const { return 0; }
+private:
+    bool NamesThisBackend(const ModelOptions& modelOptions) const
+    {
+        for (const BackendOptions& group : modelOptions)
+            if (group.GetBackendId() == GetId()) return true;
+        return false;
+    }
 };
 using IBackendInternalUniquePtr = std::unique_ptr<IBackendInternal>;
 } // namespace armnn

@@ -5,6 +5,7 @@
 #include "Mi355xLayerSupport.hpp"
 #include "Mi355xTensorHandle.hpp"
 #include "Mi355xWorkloadFactory.hpp"
+#include "Mi355xWorkloads.hpp"
 
 #include <Layer.hpp>
 #include <armnn/BackendOptions.hpp>
@@ -152,6 +153,17 @@ IBackendInternal::IWorkloadFactoryPtr Mi355xBackend::CreateWorkloadFactory(Tenso
     return std::make_unique<Mi355xWorkloadFactory>(EnsureFactories(registry).GetMemoryManager());
 }
 
+IBackendInternal::IWorkloadFactoryPtr Mi355xBackend::CreateWorkloadFactory(const IBackendInternal::IMemoryManagerSharedPtr& memoryManager,
+                                                                           const ModelOptions&) const
+{
+    return CreateWorkloadFactory(memoryManager);
+}
+IBackendInternal::IWorkloadFactoryPtr Mi355xBackend::CreateWorkloadFactory(TensorHandleFactoryRegistry& registry, const ModelOptions&) const
+{
+    return CreateWorkloadFactory(registry);
+}
+IBackendInternal::ILayerSupportSharedPtr Mi355xBackend::GetLayerSupport(const ModelOptions&) const { return GetLayerSupport(); }
+
 IBackendInternal::IBackendContextPtr Mi355xBackend::CreateBackendContext(const IRuntime::CreationOptions& options) const
 {
     return std::make_unique<Mi355xBackendContext>(options);
@@ -225,6 +237,8 @@ BackendCapabilities Mi355xBackend::GetCapabilities() const
 //   kernels apply in their epilogue.  With different quantizations the Activation layer re-quantizes and stays a layer
 //   of its own.  The replacement layer carries the ActivationDescriptor as its additional-info object, as the Neon and
 //   CL backends do (src/backends/aclCommon/ArmComputeSubgraphUtils.hpp:60-109).
+// * A Convolution2d without an activation whose output goes to one Addition of this backend and nowhere else is marked
+//   (Mi355xFeedsOnlyAnAddition): the two workloads may then run as one launch (Mi355xAdditionWorkload).
 // * A constant Pad of height and width in front of a Convolution2d, DepthwiseConvolution2d or Pooling2d moves into that
 //   layer's own padding when the padded value is the layer's neutral element, as CpuRef does
 //   (src/backends/reference/RefBackend.cpp:72-184 with the rules of src/armnn/optimizations/FoldPadIntoLayer2d.hpp:21-145).
@@ -234,6 +248,11 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
     const SubgraphView::IConnectableLayers& layers = subgraph.GetIConnectableLayers();
     std::set<const IConnectableLayer*> members(layers.begin(), layers.end());
     std::set<const IConnectableLayer*> consumed;
+    // BackendOptions("Mi355x", {{"FuseAdditions", false}}) among the network's model options keeps every Addition a launch of its own
+    bool fuseAdditions = true;
+    ParseOptions(modelOptions, Mi355xBackendId(), [&](const std::string& name, const BackendOptions::Var& value) {
+        if (name == "FuseAdditions" && value.IsBool()) fuseAdditions = value.AsBool();
+    });
 
     for (IConnectableLayer* il : layers)
     {
@@ -278,7 +297,18 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
                     act = next;
             }
         }
-        if (!pad && !act) continue;
+        // a Convolution2d whose only consumer is an Addition of this backend: its workload may run inside that Addition's
+        bool residual = false;
+        if (fuseAdditions && type == LayerType::Convolution2d && !act && base->GetAdditionalInformation<ActivationDescriptor>() == nullptr &&
+            base->GetOutputSlot(0).GetNumConnections() == 1)
+        {
+            Layer* next = &base->GetOutputSlot(0).GetConnections()[0]->GetOwningLayer();
+            if (next->GetType() == LayerType::ElementwiseBinary && members.count(next) &&
+                static_cast<const ElementwiseBinaryDescriptor&>(next->GetParameters()).m_Operation == BinaryOperation::Add &&
+                next->GetInputSlot(0).GetConnectedOutputSlot() != next->GetInputSlot(1).GetConnectedOutputSlot())
+                residual = true;
+        }
+        if (!pad && !act && !residual) continue;
 
         std::string name = base->GetName();
         if (pad) name = std::string("folded-") + pad->GetName() + "-into-" + name;
@@ -304,6 +334,8 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
                 std::make_shared<ActivationDescriptor>(static_cast<const ActivationDescriptor&>(act->GetParameters())));
         else if (auto carried = base->GetAdditionalInformation<ActivationDescriptor>())
             PolymorphicDowncast<Layer*>(replacement)->SetAdditionalInfoForObject(carried);
+        else if (residual)
+            PolymorphicDowncast<Layer*>(replacement)->SetAdditionalInfoForObject(std::make_shared<ActivationDescriptor>(Mi355xFeedsOnlyAnAddition()));
 
         SubgraphView::IConnectableLayers replaced;
         SubgraphView::IInputSlots ins;

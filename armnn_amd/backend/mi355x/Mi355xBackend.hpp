@@ -17,6 +17,14 @@ public:
     IBackendInternal::IMemoryManagerUniquePtr CreateMemoryManager() const override;
     IBackendInternal::IWorkloadFactoryPtr CreateWorkloadFactory(const IBackendInternal::IMemoryManagerSharedPtr& memoryManager = nullptr) const override;
     IBackendInternal::IWorkloadFactoryPtr CreateWorkloadFactory(TensorHandleFactoryRegistry& tensorHandleFactoryRegistry) const override;
+    /// The backend reads its model options ("FuseAdditions") when it optimizes a network; factories and layer support do
+    /// not depend on them.  The overloads exist because the defaults answer with nothing once the options name the backend
+    /// (IBackendInternal.cpp:24-58, 88-102).
+    IBackendInternal::IWorkloadFactoryPtr CreateWorkloadFactory(const IBackendInternal::IMemoryManagerSharedPtr& memoryManager,
+                                                                const ModelOptions& modelOptions) const override;
+    IBackendInternal::IWorkloadFactoryPtr CreateWorkloadFactory(TensorHandleFactoryRegistry& tensorHandleFactoryRegistry,
+                                                                const ModelOptions& modelOptions) const override;
+    IBackendInternal::ILayerSupportSharedPtr GetLayerSupport(const ModelOptions& modelOptions) const override;
     /// throws BackendUnavailableException when the process sees no MI355X; the runtime then leaves the backend out
     IBackendInternal::IBackendContextPtr CreateBackendContext(const IRuntime::CreationOptions&) const override;
     IBackendInternal::ILayerSupportSharedPtr GetLayerSupport() const override;

@@ -6,11 +6,51 @@
 #include <armnn/backends/MemCopyWorkload.hpp>
 #include <armnn/utility/PolymorphicDowncast.hpp>
 
+#include <mutex>
+#include <thread>
+
 namespace armnn
 {
 namespace
 {
 const BackendId s_Id{Mi355xBackendId()};
+
+// The Convolution2d workload created last, while no workload that writes device tensors has been created since: the
+// candidate an Addition created next may take over (Mi355xAdditionWorkload::TakeOver).  A network's workloads are created in
+// execution order by one thread; the thread is recorded so that networks loading at the same time at worst lose a
+// pairing.  The entry is dropped when the workload is destroyed.
+struct Candidate
+{
+    std::mutex mutex;
+    Mi355xConvolution2dWorkload* convolution = nullptr;
+    std::thread::id thread;
+};
+Candidate& TheCandidate()
+{
+    static Candidate c;
+    return c;
+}
+Mi355xConvolution2dWorkload* TakeCandidate()
+{
+    Candidate& c = TheCandidate();
+    std::lock_guard<std::mutex> lock(c.mutex);
+    Mi355xConvolution2dWorkload* w = c.thread == std::this_thread::get_id() ? c.convolution : nullptr;
+    c.convolution = nullptr;
+    return w;
+}
+
+// deleter-side hook: a candidate that is destroyed before anything took it
+class CandidateConvolution final : public Mi355xConvolution2dWorkload
+{
+public:
+    using Mi355xConvolution2dWorkload::Mi355xConvolution2dWorkload;
+    ~CandidateConvolution() override
+    {
+        Candidate& c = TheCandidate();
+        std::lock_guard<std::mutex> lock(c.mutex);
+        if (c.convolution == this) c.convolution = nullptr;
+    }
+};
 }
 
 Mi355xWorkloadFactory::Mi355xWorkloadFactory(const std::shared_ptr<Mi355xMemoryManager>& memoryManager) : m_MemoryManager(memoryManager) {}
@@ -34,10 +74,22 @@ std::unique_ptr<ITensorHandle> Mi355xWorkloadFactory::CreateTensorHandle(const T
 
 std::unique_ptr<IWorkload> Mi355xWorkloadFactory::CreateWorkload(LayerType type, const QueueDescriptor& descriptor, const WorkloadInfo& info) const
 {
+    // constants write no tensor another workload's operand could share an address with: they leave the candidate alone
+    Mi355xConvolution2dWorkload* candidate = type == LayerType::Constant ? nullptr : TakeCandidate();
     switch (type)
     {
         case LayerType::Convolution2d:
-            return std::make_unique<Mi355xConvolution2dWorkload>(*PolymorphicDowncast<const Convolution2dQueueDescriptor*>(&descriptor), info);
+        {
+            auto w = std::make_unique<CandidateConvolution>(*PolymorphicDowncast<const Convolution2dQueueDescriptor*>(&descriptor), info);
+            if (w->FeedsOnlyAnAddition())
+            {
+                Candidate& c = TheCandidate();
+                std::lock_guard<std::mutex> lock(c.mutex);
+                c.convolution = w.get();
+                c.thread = std::this_thread::get_id();
+            }
+            return w;
+        }
         case LayerType::DepthwiseConvolution2d:
             return std::make_unique<Mi355xDepthwiseConvolution2dWorkload>(*PolymorphicDowncast<const DepthwiseConvolution2dQueueDescriptor*>(&descriptor), info);
         case LayerType::FullyConnected:
@@ -53,7 +105,11 @@ std::unique_ptr<IWorkload> Mi355xWorkloadFactory::CreateWorkload(LayerType type,
         case LayerType::Softmax:
             return std::make_unique<Mi355xSoftmaxWorkload>(*PolymorphicDowncast<const SoftmaxQueueDescriptor*>(&descriptor), info);
         case LayerType::ElementwiseBinary:
-            return std::make_unique<Mi355xAdditionWorkload>(*PolymorphicDowncast<const ElementwiseBinaryQueueDescriptor*>(&descriptor), info);
+        {
+            auto w = std::make_unique<Mi355xAdditionWorkload>(*PolymorphicDowncast<const ElementwiseBinaryQueueDescriptor*>(&descriptor), info);
+            w->TakeOver(candidate);
+            return w;
+        }
         case LayerType::Reshape:
             return std::make_unique<Mi355xReshapeWorkload>(*PolymorphicDowncast<const ReshapeQueueDescriptor*>(&descriptor), info);
         case LayerType::Constant:

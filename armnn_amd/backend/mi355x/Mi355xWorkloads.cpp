@@ -9,6 +9,7 @@
 #include <armnn/utility/PolymorphicDowncast.hpp>
 
 #include <algorithm>
+#include <atomic>
 #include <cstring>
 
 namespace armnn
@@ -106,9 +107,21 @@ Mi355xFusedActivation Mi355xFusedActivation::From(const ActivationDescriptor* d)
     {
         case ActivationFunction::ReLu: f.function = MI355X_ACT_RELU; break;
         case ActivationFunction::BoundedReLu: f.function = MI355X_ACT_BOUNDED_RELU; f.a = d->m_A; f.b = d->m_B; break;
+        case ActivationFunction::Linear:
+            if (d->m_A == 1.0f && d->m_B == 0.0f) { f.feedsOnlyAnAddition = true; break; }
+            throw InvalidArgumentException("Mi355x: only ReLu / BoundedReLu can be fused into a layer");
         default: throw InvalidArgumentException("Mi355x: only ReLu / BoundedReLu can be fused into a layer");
     }
     return f;
+}
+
+ActivationDescriptor Mi355xFeedsOnlyAnAddition()
+{
+    ActivationDescriptor d;
+    d.m_Function = ActivationFunction::Linear;
+    d.m_A = 1.0f;
+    d.m_B = 0.0f;
+    return d;
 }
 
 // ---- Convolution2d ---------------------------------------------------------------------------------------------------
@@ -117,7 +130,7 @@ Mi355xConvolution2dWorkload::Mi355xConvolution2dWorkload(const Convolution2dQueu
 {
     ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xConvolution2dWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
     if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xConvolution2dWorkload: NHWC only");
-    Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());   // validates early
+    m_FeedsOnlyAnAddition = Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>()).feedsOnlyAnAddition;   // validates early
 }
 
 Mi355xConvolution2dWorkload::~Mi355xConvolution2dWorkload()
@@ -162,16 +175,57 @@ void Mi355xConvolution2dWorkload::BuildPlan() const
 
 void Mi355xConvolution2dWorkload::Execute() const
 {
+    if (m_RunsInsideTheAddition) return;
     ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xConvolution2dWorkload_Execute");
+    Run(Out(m_Data.m_Outputs[0]));
+}
+
+void Mi355xConvolution2dWorkload::Run(void* y) const
+{
     std::call_once(m_Once, [this] { BuildPlan(); });
     if (!m_Plan) throw RuntimeException("Mi355xConvolution2dWorkload: no device plan (its creation failed earlier)");
     const TensorInfo& in = m_Info.m_InputTensorInfos[0];
     const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
     const uint32_t batch = in.GetShape()[0];
     const void* x = In(m_Data.m_Inputs[0]);
-    void* y = Out(m_Data.m_Outputs[0]);
     ForEachLane(batch, [&](const Lane& l) {
         mi355x::Check(mi355x_conv2d_run(m_Plan, batch / l.count, l.Of(x, in), l.Of(y, out), l.stream), "mi355x_conv2d_run");
+    });
+}
+
+void Mi355xConvolution2dWorkload::ExecuteWithAddition(const ITensorHandle* other, const TensorInfo& otherInfo, ITensorHandle* sum,
+                                                      const TensorInfo& sumInfo, const Mi355xFusedActivation& activation) const
+{
+    std::call_once(m_Once, [this] { BuildPlan(); });
+    if (!m_Plan) throw RuntimeException("Mi355xConvolution2dWorkload: no device plan (its creation failed earlier)");
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const uint32_t batch = in.GetShape()[0];
+    const mi355x_quant qOther = mi355x::ToQuant(otherInfo);
+    const mi355x_quant qSum = mi355x::ToQuant(sumInfo);
+    const mi355x_quant qOwn = mi355x::ToQuant(out);
+    const unsigned char* x = static_cast<const unsigned char*>(In(m_Data.m_Inputs[0]));
+    const void* r = In(other);
+    unsigned char* y = static_cast<unsigned char*>(Out(sum));
+    // The sum's tensor began its life after the convolution's input ended its own, so a memory manager that shares
+    // addresses may have put the one where the other is.  One launch that reads and writes the same range would race:
+    // then the convolution writes its own output first (that tensor lives until the Addition has run).
+    const bool overlap = x < y + sumInfo.GetNumBytes() && y < x + in.GetNumBytes();
+    if (overlap)
+    {
+        void* own = Out(m_Data.m_Outputs[0]);
+        ForEachLane(batch, [&](const Lane& l) {
+            mi355x::Check(mi355x_conv2d_run(m_Plan, batch / l.count, l.Of(static_cast<const void*>(x), in), l.Of(own, out), l.stream), "mi355x_conv2d_run");
+            mi355x::Check(mi355x_add_run(out.GetNumElements() / l.count, &qOwn, &qOther, &qSum, activation.function, activation.a, activation.b,
+                                         l.Of(static_cast<const void*>(own), out), l.Of(r, otherInfo), l.Of(static_cast<void*>(y), sumInfo), l.stream),
+                          "mi355x_add_run");
+        });
+        return;
+    }
+    ForEachLane(batch, [&](const Lane& l) {
+        mi355x::Check(mi355x_conv2d_run_add(m_Plan, batch / l.count, l.Of(static_cast<const void*>(x), in), l.Of(r, otherInfo), &qOther, &qSum,
+                                            activation.function, activation.a, activation.b, l.Of(static_cast<void*>(y), sumInfo), l.stream),
+                      "mi355x_conv2d_run_add");
     });
 }
 
@@ -462,10 +516,42 @@ Mi355xAdditionWorkload::Mi355xAdditionWorkload(const ElementwiseBinaryQueueDescr
     Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
 }
 
+namespace
+{
+std::atomic<unsigned long long> g_PairsFormed{0};
+}
+unsigned long long Mi355xAdditionWorkload::PairsFormed() { return g_PairsFormed.load(); }
+
+bool Mi355xAdditionWorkload::TakeOver(Mi355xConvolution2dWorkload* convolution)
+{
+    if (!convolution || m_Convolution || !convolution->FeedsOnlyAnAddition() || convolution->RunsInsideTheAddition()) return false;
+    const ITensorHandle* produced = convolution->GetOutputHandle();
+    if (!produced || m_Data.m_Inputs[0] == m_Data.m_Inputs[1]) return false;
+    unsigned int own;
+    if (m_Data.m_Inputs[0] == produced) own = 0;
+    else if (m_Data.m_Inputs[1] == produced) own = 1;
+    else return false;
+    // no broadcast: both inputs have the shape of the sum
+    if (m_Info.m_InputTensorInfos[0].GetShape() != m_Info.m_OutputTensorInfos[0].GetShape() ||
+        m_Info.m_InputTensorInfos[1].GetShape() != m_Info.m_OutputTensorInfos[0].GetShape())
+        return false;
+    m_OtherInput = 1 - own;
+    m_Convolution = convolution;
+    convolution->LeaveExecutionToTheAddition();
+    g_PairsFormed.fetch_add(1);
+    return true;
+}
+
 void Mi355xAdditionWorkload::Execute() const
 {
     ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xAdditionWorkload_Execute");
     const Mi355xFusedActivation act = Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
+    if (m_Convolution)
+    {
+        m_Convolution->ExecuteWithAddition(m_Data.m_Inputs[m_OtherInput], m_Info.m_InputTensorInfos[m_OtherInput], m_Data.m_Outputs[0],
+                                           m_Info.m_OutputTensorInfos[0], act);
+        return;
+    }
     const mi355x_quant q0 = mi355x::ToQuant(m_Info.m_InputTensorInfos[0]);
     const mi355x_quant q1 = mi355x::ToQuant(m_Info.m_InputTensorInfos[1]);
     const mi355x_quant qo = mi355x::ToQuant(m_Info.m_OutputTensorInfos[0]);

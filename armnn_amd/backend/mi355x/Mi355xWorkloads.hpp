@@ -19,8 +19,14 @@ struct Mi355xFusedActivation
 {
     int32_t function = MI355X_ACT_NONE;
     float a = 0.0f, b = 0.0f;
+    /// the descriptor was Mi355xFeedsOnlyAnAddition()
+    bool feedsOnlyAnAddition = false;
     static Mi355xFusedActivation From(const ActivationDescriptor* descriptor);
 };
+
+/// The additional-info object of a Convolution2d whose output goes to one Addition of this backend and nowhere else:
+/// Linear with slope 1 and offset 0, the identity, so a reader that applies it changes nothing.
+ActivationDescriptor Mi355xFeedsOnlyAnAddition();
 
 /// Every workload here reads its tensor handles when it executes, so the runtime may swap a handle for one that adopted
 /// caller memory (pre-imported inputs and outputs; RefBaseWorkload, src/backends/reference/workloads/RefBaseWorkload.hpp:13-35).
@@ -43,9 +49,22 @@ public:
     void Execute() const override;
     /// kernel the plan resolved to; empty before the first Execute()
     std::string GetKernelDescription() const;
+    /// the layer was marked Mi355xFeedsOnlyAnAddition()
+    bool FeedsOnlyAnAddition() const { return m_FeedsOnlyAnAddition; }
+    const ITensorHandle* GetOutputHandle() const { return m_Data.m_Outputs[0]; }
+    /// From now on Execute() does nothing: the Addition that consumes this convolution calls ExecuteWithAddition() in its
+    /// own Execute().
+    void LeaveExecutionToTheAddition() { m_RunsInsideTheAddition = true; }
+    bool RunsInsideTheAddition() const { return m_RunsInsideTheAddition; }
+    /// convolution and Addition as one launch per lane: sum = activation(convolution(input) + other)
+    void ExecuteWithAddition(const ITensorHandle* other, const TensorInfo& otherInfo, ITensorHandle* sum, const TensorInfo& sumInfo,
+                             const Mi355xFusedActivation& activation) const;
 private:
     void BuildPlan() const;
+    void Run(void* y) const;
     WorkloadInfo m_Info;
+    bool m_FeedsOnlyAnAddition = false;
+    bool m_RunsInsideTheAddition = false;
     mutable mi355x_conv2d_t m_Plan = nullptr;
     mutable std::once_flag m_Once;
 };
@@ -136,8 +155,20 @@ class Mi355xAdditionWorkload : public Mi355xBaseWorkload<ElementwiseBinaryQueueD
 public:
     Mi355xAdditionWorkload(const ElementwiseBinaryQueueDescriptor& descriptor, const WorkloadInfo& info);
     void Execute() const override;
+    /// `convolution` is the workload created directly before this one.  If it produces one of this Addition's inputs and
+    /// nothing else reads that tensor, it leaves its execution to this workload, which then runs both as one launch.
+    /// Nothing ran between the two, so every tensor the convolution reads is still intact when this workload executes;
+    /// only this Addition's own output may have taken the place of the convolution's input, which Execute() checks.
+    /// Returns whether the pair was formed.  The convolution must outlive every Execute() of this workload (both belong
+    /// to one loaded network).
+    bool TakeOver(Mi355xConvolution2dWorkload* convolution);
+    bool RunsAConvolution() const { return m_Convolution != nullptr; }
+    /// how many pairs this process has formed so far (for tests and benchmarks)
+    static unsigned long long PairsFormed();
 private:
     WorkloadInfo m_Info;
+    const Mi355xConvolution2dWorkload* m_Convolution = nullptr;
+    unsigned int m_OtherInput = 0;
 };
 
 /// counterpart of RefReshapeWorkload (RefReshapeWorkload.cpp:14-31): a device-to-device copy

@@ -23,6 +23,7 @@
 #include <sstream>
 
 #include "NetFile.hpp"
+#include "../mi355x/Mi355xWorkloads.hpp"
 
 using namespace armnn;
 
@@ -114,8 +115,8 @@ int main(int argc, char** argv)
         mi355x_host_free(pout);
         std::printf("{\"batch\": %u, \"steps\": %d, \"ms_pageable\": %.4f, \"ms_pinned\": %.4f, \"pinned_equals_pageable\": %s, "
                     "\"optimized_layers\": %zu, \"activation_layers_left\": %zu, \"memcopy_layers\": %zu, \"conv_layers\": %zu, "
-                    "\"depthwise_layers\": %zu, \"add_layers\": %zu}\n",
-                    nf.batch, steps, msPageable, msPinned, same ? "true" : "false", nLayers, nAct, nCopy, nConv, nDw, nAdd);
+                    "\"depthwise_layers\": %zu, \"add_layers\": %zu, \"additions_running_a_convolution\": %llu}\n",
+                    nf.batch, steps, msPageable, msPinned, same ? "true" : "false", nLayers, nAct, nCopy, nConv, nDw, nAdd, Mi355xAdditionWorkload::PairsFormed());
         return same ? 0 : 1;
     }
     catch (const std::exception& e)

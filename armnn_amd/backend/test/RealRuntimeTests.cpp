@@ -119,6 +119,8 @@ int main(int argc, char** argv)
             conv->GetOutputSlot(0).Connect(output->GetInputSlot(0));
             return net;
         };
+        std::string lastProfile;
+        OptimizerOptionsOpaque optimizerOptions;
         auto run = [&](INetwork& net, const std::vector<BackendId>& prefs, const TensorInfo& inInfo, const std::vector<int8_t>& x,
                        const TensorInfo& outInfo, std::string& placement) {
             std::vector<std::string> messages;
@@ -126,7 +128,7 @@ int main(int argc, char** argv)
             IOptimizedNetworkPtr opt(nullptr, [](IOptimizedNetwork*) {});
             try
             {
-                opt = Optimize(net, prefs, runtime->GetDeviceSpec(), OptimizerOptionsOpaque(), Optional<std::vector<std::string>&>(messages));
+                opt = Optimize(net, prefs, runtime->GetDeviceSpec(), optimizerOptions, Optional<std::vector<std::string>&>(messages));
             }
             catch (const Exception& e)
             {
@@ -147,7 +149,8 @@ int main(int argc, char** argv)
             CHECK(runtime->EnqueueWorkload(id, {{0, ConstTensor(cin, x.data())}}, {{0, Tensor(outInfo, y.data())}}) == Status::Success);
             std::ostringstream prof;
             runtime->GetProfiler(id)->Print(prof);
-            placement = prof.str().find("Mi355x") != std::string::npos ? "Mi355x" : "CpuRef";
+            lastProfile = prof.str();
+            placement = lastProfile.find("Mi355x") != std::string::npos ? "Mi355x" : "CpuRef";
             runtime->UnloadNetwork(id);
             return y;
         };
@@ -287,6 +290,21 @@ int main(int argc, char** argv)
                     cur->Connect(output->GetInputSlot(0));
                     return net;
                 }
+                if (depth == 4)
+                {
+                    // a residual connection: a 1x1 convolution of the trunk, added to the trunk, then ReLU
+                    IOutputSlot* trunk = cur;
+                    IConnectableLayer* l4 = net->AddConvolution2dLayer(c3, "branch");
+                    constants(l4, {64, 1, 1, 64}, 64, 0, 0.005f);
+                    finish(l4, TensorInfo({2, 8, 8, 64}, DataType::QAsymmS8, 0.05f, 3), 0);
+                    IConnectableLayer* add = net->AddElementwiseBinaryLayer(ElementwiseBinaryDescriptor(BinaryOperation::Add), "add");
+                    cur->Connect(add->GetInputSlot(0));
+                    trunk->Connect(add->GetInputSlot(1));
+                    finish(add, TensorInfo({2, 8, 8, 64}, DataType::QAsymmS8, 0.04f, -128), 1);
+                    IConnectableLayer* output = net->AddOutputLayer(0);
+                    cur->Connect(output->GetInputSlot(0));
+                    return net;
+                }
                 Pooling2dDescriptor p4;
                 p4.m_PoolType = PoolingAlgorithm::Average;
                 p4.m_PoolWidth = p4.m_PoolHeight = 8;
@@ -323,6 +341,38 @@ int main(int argc, char** argv)
                 const std::vector<int8_t> want = run(*b, {BackendId("CpuRef")}, t0, x, tout, whereRef);
                 compare(got, want, depth == 3 ? "convolution + ReLU6, strided depthwise + ReLU, pointwise + ReLU6" : "the same, then pooling, reshape, fully connected",
                         where);
+            }
+            // ---- a residual connection.  The backend's Addition workload runs the convolution that feeds it inside its
+            //      own launch; with BackendOptions("Mi355x", {{"FuseAdditions", false}}) among the model options the two stay
+            //      apart.  Same bytes either way, and one convolution workload fewer executes on its own.
+            {
+                auto executed = [&] {
+                    size_t n = 0;
+                    for (size_t at = lastProfile.find("Mi355xConvolution2dWorkload_Execute"); at != std::string::npos;
+                         at = lastProfile.find("Mi355xConvolution2dWorkload_Execute", at + 1))
+                        ++n;
+                    return n;
+                };
+                const TensorInfo tout({2, 8, 8, 64}, DataType::QAsymmS8, 0.04f, -128);
+                std::string where, whereApart, whereRef;
+                INetworkPtr a = build(4);
+                const std::vector<int8_t> got = run(*a, {mi, BackendId("CpuRef")}, t0, x, tout, where);
+                const size_t together = executed();
+                optimizerOptions.AddModelOption(BackendOptions("Mi355x", {{"FuseAdditions", false}}));
+                INetworkPtr b = build(4);
+                const std::vector<int8_t> apart = run(*b, {mi, BackendId("CpuRef")}, t0, x, tout, whereApart);
+                const size_t alone = executed();
+                optimizerOptions = OptimizerOptionsOpaque();
+                INetworkPtr c = build(4);
+                const std::vector<int8_t> want = run(*c, {BackendId("CpuRef")}, t0, x, tout, whereRef);
+                compare(got, want, "convolution, depthwise, pointwise, then a 1x1 convolution added to its own input + ReLU", where);
+                CHECK(got == apart);
+                if (!unavailable)
+                {
+                    std::printf("convolution workloads executing on their own: %zu with the Addition taking one over, %zu apart\n", together, alone);
+                    CHECK(alone > 0);
+                    CHECK(together + (alone / 3) == alone);      // each workload appears the same number of times in the printed profile
+                }
             }
         }
     }

@@ -90,6 +90,8 @@ def test_benchmark_network_through_the_backend_equals_the_executor(tmp_path, nam
           f"{fig['ms_pinned']:.3f} ms adopted pinned I/O = {batch / fig['ms_pinned'] * 1e3:.0f} images/s; {fig}", flush=True)
     assert fig["pinned_equals_pageable"] and fig["activation_layers_left"] == 0 and fig["memcopy_layers"] == 0
     assert fig["add_layers"] == (16 if name == "resnet50" else 0)
+    # every residual Addition of ResNet-50 runs the convolution in front of it inside its own launch
+    assert fig["additions_running_a_convolution"] == fig["add_layers"]
     dn = DeviceNetwork(net, batch, use_graph=False)
     want = dn.run(x).data.tobytes()
     dn.close()
