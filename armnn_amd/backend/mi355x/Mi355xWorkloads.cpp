@@ -32,6 +32,8 @@ void* Out(ITensorHandle* h)
     return d.GetDevicePointer();
 }
 
+std::atomic<unsigned long long> g_PairsFormed{0}, g_PairsRunApart{0};
+
 // One slice of a batch and the stream it runs on.
 struct Lane
 {
@@ -213,6 +215,7 @@ void Mi355xConvolution2dWorkload::ExecuteWithAddition(const ITensorHandle* other
     const bool overlap = x < y + sumInfo.GetNumBytes() && y < x + in.GetNumBytes();
     if (overlap)
     {
+        g_PairsRunApart.fetch_add(1);
         void* own = Out(m_Data.m_Outputs[0]);
         ForEachLane(batch, [&](const Lane& l) {
             mi355x::Check(mi355x_conv2d_run(m_Plan, batch / l.count, l.Of(static_cast<const void*>(x), in), l.Of(own, out), l.stream), "mi355x_conv2d_run");
@@ -516,11 +519,8 @@ Mi355xAdditionWorkload::Mi355xAdditionWorkload(const ElementwiseBinaryQueueDescr
     Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
 }
 
-namespace
-{
-std::atomic<unsigned long long> g_PairsFormed{0};
-}
 unsigned long long Mi355xAdditionWorkload::PairsFormed() { return g_PairsFormed.load(); }
+unsigned long long Mi355xAdditionWorkload::PairsRunApart() { return g_PairsRunApart.load(); }
 
 bool Mi355xAdditionWorkload::TakeOver(Mi355xConvolution2dWorkload* convolution)
 {

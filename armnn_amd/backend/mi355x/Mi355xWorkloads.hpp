@@ -163,8 +163,10 @@ public:
     /// to one loaded network).
     bool TakeOver(Mi355xConvolution2dWorkload* convolution);
     bool RunsAConvolution() const { return m_Convolution != nullptr; }
-    /// how many pairs this process has formed so far (for tests and benchmarks)
+    /// how many pairs this process has formed so far, and how many executions of a pair ran as two launches because the
+    /// sum had been placed over the convolution's input (for tests and benchmarks)
     static unsigned long long PairsFormed();
+    static unsigned long long PairsRunApart();
 private:
     WorkloadInfo m_Info;
     const Mi355xConvolution2dWorkload* m_Convolution = nullptr;

@@ -12,6 +12,7 @@
 #include "../mi355x/Mi355xDevice.hpp"
 #include "../mi355x/Mi355xLayerSupport.hpp"
 #include "../mi355x/Mi355xMemoryManager.hpp"
+#include "../mi355x/Mi355xWorkloads.hpp"
 #include "../mi355x/Mi355xTensorHandle.hpp"
 #include "../mi355x/Mi355xWorkloadFactory.hpp"
 
@@ -404,6 +405,41 @@ const Layer* ConvolutionNamed(const Graph& g, const std::string& name)
         if (l->GetType() == LayerType::Convolution2d && l->GetNameStr() == name) return l.get();
     return nullptr;
 }
+
+// input (64 channels) -> 3x3 conv to 256 channels + ReLU6 -> 1x1 conv back to 64 channels -+-> Addition + ReLU -> output
+//   \------------------------------------------------------------------------------------+
+// The 1x1 convolution's input is four times the sum and dies where the sum is born: an arena that shares addresses puts
+// the sum there.
+struct NarrowingResidualBlock
+{
+    TensorInfo in, sum;
+    QLayer first, last;
+    explicit NarrowingResidualBlock(unsigned int batch)
+    {
+        in = ActInfo({batch, 16, 16, 64}, DataType::QAsymmS8, 0.05f, -3);
+        first = MakeConv(QLayer::Conv, in, 256, 3, 1, 0.04f, -128, true, true, 41);
+        last = MakeConv(QLayer::Conv, first.out, 64, 1, 1, 0.09f, 5, false, true, 42);
+        sum = TensorInfo(last.out.GetShape(), DataType::QAsymmS8, 0.06f, -128);
+    }
+    INetworkPtr Build() const
+    {
+        INetworkPtr net = INetwork::Create();
+        IConnectableLayer* input = net->AddInputLayer(0, "input");
+        input->GetOutputSlot(0).SetTensorInfo(in);
+        IOutputSlot& a = AddToNetwork(*net, input->GetOutputSlot(0), first, "first");
+        IOutputSlot& b = AddToNetwork(*net, a, last, "last");
+        IConnectableLayer* add = net->AddElementwiseBinaryLayer(ElementwiseBinaryDescriptor(BinaryOperation::Add), "add");
+        input->GetOutputSlot(0).Connect(add->GetInputSlot(0));
+        b.Connect(add->GetInputSlot(1));
+        add->GetOutputSlot(0).SetTensorInfo(sum);
+        IConnectableLayer* relu = net->AddActivationLayer(ActivationDescriptor(ActivationFunction::ReLu, 0.0f, 0.0f), "relu");
+        add->GetOutputSlot(0).Connect(relu->GetInputSlot(0));
+        relu->GetOutputSlot(0).SetTensorInfo(sum);
+        IConnectableLayer* out = net->AddOutputLayer(0, "output");
+        relu->GetOutputSlot(0).Connect(out->GetInputSlot(0));
+        return net;
+    }
+};
 
 bool MarkedForAnAddition(const Layer* l)
 {
@@ -1729,6 +1765,52 @@ TEST_CASE("runtime: an Addition runs the convolution that feeds it in one launch
         const std::vector<uint8_t> c = OracleRun(block.shortcut, input);
         const Diff d = Compare(results[1], OracleAddRelu(block.last.out, b, block.shortcut.out, c, block.sum), DataType::QAsymmS8);
         std::printf("    residual block vs oracle: max |diff| %d, exact %.5f\n", d.maxAbs, 1.0 - static_cast<double>(d.mismatches) / static_cast<double>(d.n));
+        CHECK(d.maxAbs <= 2);
+        CHECK(d.mismatches * 1000 <= d.n);
+    }
+    mi355x::SetLanes(lanesBefore);
+}
+
+TEST_CASE("runtime: an Addition whose sum was placed over the convolution's input runs the pair as two launches, same bytes", "gpu")
+{
+    const unsigned int lanesBefore = mi355x::Lanes();
+    mi355x::SetLanes(1);                                   // one stream: the arena shares addresses
+    {
+        NarrowingResidualBlock block(4);
+        const std::vector<uint8_t> input = RandomActivations(block.in, 92);
+        TensorInfo constIn = block.in;
+        constIn.SetConstant(true);
+        std::vector<uint8_t> results[2];
+        unsigned long long pairs[2] = {0, 0}, apart[2] = {0, 0};
+        for (int fused = 0; fused < 2; ++fused)
+        {
+            const unsigned long long pairsBefore = Mi355xAdditionWorkload::PairsFormed(), apartBefore = Mi355xAdditionWorkload::PairsRunApart();
+            IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+            INetworkPtr net = block.Build();
+            OptimizerOptionsOpaque options;
+            options.AddModelOption(BackendOptions("Mi355x", {{"FuseAdditions", fused == 1}}));
+            IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, rt->GetDeviceSpec(), options);
+            NetworkId id = -1;
+            std::string err;
+            REQUIRE(rt->LoadNetwork(id, std::move(opt), err) == Status::Success);
+            results[fused].assign(block.sum.GetNumBytes(), 0);
+            InputTensors ins{{0, ConstTensor(constIn, input.data())}};
+            OutputTensors outs{{0, Tensor(block.sum, results[fused].data())}};
+            REQUIRE(rt->EnqueueWorkload(id, ins, outs) == Status::Success);
+            rt->UnloadNetwork(id);
+            pairs[fused] = Mi355xAdditionWorkload::PairsFormed() - pairsBefore;
+            apart[fused] = Mi355xAdditionWorkload::PairsRunApart() - apartBefore;
+        }
+        std::printf("    pairs formed %llu, executions that ran as two launches %llu\n", pairs[1], apart[1]);
+        CHECK(pairs[0] == 0);
+        CHECK(pairs[1] == 1);
+        CHECK(apart[0] == 0);
+        CHECK(apart[1] == 1);                              // first fit puts the sum at the start of the dead 256-channel tensor
+        CHECK(results[0] == results[1]);
+        const std::vector<uint8_t> a = OracleRun(block.first, input);
+        const std::vector<uint8_t> b = OracleRun(block.last, a);
+        const Diff d = Compare(results[1], OracleAddRelu(block.in, input, block.last.out, b, block.sum), DataType::QAsymmS8);
+        std::printf("    narrowing residual block vs oracle: max |diff| %d, exact %.5f\n", d.maxAbs, 1.0 - static_cast<double>(d.mismatches) / static_cast<double>(d.n));
         CHECK(d.maxAbs <= 2);
         CHECK(d.mismatches * 1000 <= d.n);
     }
