@@ -1131,10 +1131,9 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.C = g.Co; a.Ho = g.Ho; a.Wo = g.Wo;
             a.pad_top = g.pad_top; a.pad_left = g.pad_left;
             // 128 channels per block where the channel count allows: every pixel a block reads or writes is a whole line
-            // -- for the large feature maps (56 x 56 x 128: 13.2 -> 12.7 us at stride 1, 7.3 -> 6.6 us at stride 2, 32 images)
-            // and for those so small that a 16-pixel-wide tile is mostly outside the image (7 x 7 x 1024: 5.1 -> 4.5 us); in
-            // between (28 x 28, 14 x 14) the 32-channel blocks with their larger tiles and smaller halo are as fast or faster
-            const bool wide = (g.Co % 128) == 0 && p->opt_dw_cb != 32 && (g.H * g.W >= 2500 || (g.Ho <= 8 && g.Wo <= 8));
+            // (32 images: 56 x 56 x 128 13.1 -> 11.6 us at stride 1, 7.3 -> 6.4 us at stride 2; 28 x 28 x 256 8.1 -> 7.7 us;
+            // 7 x 7 x 1024, where a 16-pixel-wide tile is mostly outside the image, 5.1 -> 4.0 us; 14 x 14 x 512 on par)
+            const bool wide = (g.Co % 128) == 0 && p->opt_dw_cb != 32;
             const int tw = wide ? (g.stride_x == 1 ? 8 : 4) : (g.stride_x == 1 ? 16 : 8);
             const int th1 = wide ? 4 : 8;            // tile rows with one output row per thread
             // two output rows per thread unless that would leave much of a tile outside a small feature map (or, with the

@@ -103,12 +103,6 @@ __device__ __forceinline__ void StoreOut16(const OutPtr& o, long long offset, co
     else *reinterpret_cast<StoreVec4*>(o.base + offset) = v;
 }
 
-__device__ __forceinline__ void StoreOut4(const OutPtr& o, long long offset, uint32_t v)
-{
-    if (o.through) __builtin_amdgcn_raw_buffer_store_b32(v, o.rsrc, static_cast<int>(offset), 0, kStoreAuxSc1);
-    else *reinterpret_cast<uint32_t*>(o.base + offset) = v;
-}
-
 __device__ __forceinline__ uint32_t Pack4(int q0, int q1, int q2, int q3)
 {
     // four codes -> one dword (byte 0 = q0), three v_perm_b32

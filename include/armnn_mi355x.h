@@ -108,8 +108,8 @@ int  mi355x_abi_version(void);
  *   into LDS (input channels a multiple of 128); 0 selects the register-staged kernel instead (identical bytes).
  *   "dw_rows" = 0 | 1 | 2: output rows per thread of the 3x3 depthwise kernel (0: chosen from the feature-map height;
  *   identical bytes).
- *   "dw_cb" = 0 | 32: channels per block of the 3x3 depthwise kernel (0: 128 where the channel count and the feature
- *   map make that the faster choice, else 32; 32: always 32; identical bytes).
+ *   "dw_cb" = 0 | 32: channels per block of the 3x3 depthwise kernel (0: 128 where the channel count is a multiple of
+ *   128, else 32; 32: always 32; identical bytes).
  * Unknown names and values outside these return MI355X_ERR_INVALID_ARGUMENT. */
 int  mi355x_set_option(const char* name, int value);
 int  mi355x_device_count(int* count);                 /* 0 devices is success with *count == 0 */

@@ -302,13 +302,16 @@ def test_depthwise_rows_per_thread_variants_give_the_same_bytes():
 
 def test_depthwise_128_channel_blocks_give_the_same_bytes():
     """Channel counts that are multiples of 128 run the 3x3 depthwise kernel with 128 channels per block (whole lines per
-    pixel) on large feature maps and on maps of at most 8 x 8: ragged sizes, both strides, one and two rows per thread,
-    uint8 activations, weights with a zero point (two int8 halves), against the 32-channel blocks and the plain kernel."""
+    pixel): large, mid-sized and tiny feature maps of ragged sizes, both strides, one and two rows per thread, uint8
+    activations, weights with a zero point (two int8 halves), against the 32-channel blocks and the plain kernel."""
     U8 = DataType.QAsymmU8
     cs = [cases.make_conv_case("dw128_s1_57x53", 711, n=2, h=57, w=53, ci=128, depthwise=True, act=cases.RELU6),
           cases.make_conv_case("dw128_s2_57x53_u8", 712, n=2, h=57, w=53, ci=256, depthwise=True, stride=(2, 2), in_dtype=U8, in_offset=140, out_offset=5),
           cases.make_conv_case("dw128_s1_7x7", 713, n=3, h=7, w=7, ci=256, depthwise=True, act=cases.RELU),
           cases.make_conv_case("dw128_s2_8x5", 714, n=2, h=8, w=5, ci=128, depthwise=True, stride=(2, 2)),
+          cases.make_conv_case("dw128_s1_29x27", 716, n=3, h=29, w=27, ci=256, depthwise=True, act=cases.RELU6),
+          cases.make_conv_case("dw128_s2_29x27", 717, n=3, h=29, w=27, ci=128, depthwise=True, stride=(2, 2), act=cases.RELU),
+          cases.make_conv_case("dw128_s1_15x13_u8", 718, n=5, h=15, w=13, ci=512, depthwise=True, in_dtype=U8, in_offset=131, out_offset=2),
           cases.make_conv_case("dw128_s1_64x50_zero_point_weights", 715, n=1, h=64, w=50, ci=128, depthwise=True, per_axis=False, w_std=60.0,
                                w_dtype=U8, w_offset=93, in_dtype=U8, in_offset=120, out_offset=3, act=cases.RELU6)]
     for c in cs:
