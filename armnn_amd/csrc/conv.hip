@@ -1134,16 +1134,19 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             // (32 images: 56 x 56 x 128 13.1 -> 11.6 us at stride 1, 7.3 -> 6.4 us at stride 2; 28 x 28 x 256 8.1 -> 7.7 us;
             // 7 x 7 x 1024, where a 16-pixel-wide tile is mostly outside the image, 5.1 -> 4.0 us; 14 x 14 x 512 on par)
             const bool wide = (g.Co % 128) == 0 && p->opt_dw_cb != 32;
+            // 64 per block for the other multiples of 64 (32 images: 112 x 112 x 64 at stride 2 10.0 -> 9.4 us, 56 x 56 x 64 7.7 -> 7.5 us, 28 x 28 x 192 6.8 -> 6.5 us)
+            const bool mid = !wide && (g.Co % 64) == 0 && p->opt_dw_cb != 32;
+            const int cbw = wide ? 128 : mid ? 64 : 32;
             const int tw = wide ? (g.stride_x == 1 ? 8 : 4) : (g.stride_x == 1 ? 16 : 8);
-            const int th1 = wide ? 4 : 8;            // tile rows with one output row per thread
+            const int th1 = cbw == 32 ? 8 : 4;       // tile rows with one output row per thread
             // two output rows per thread unless that would leave much of a tile outside a small feature map (or, with the
-            // small tiles of the 128-channel blocks, fewer than four blocks per CU)
+            // small tiles of the 64- and 128-channel blocks, fewer than two blocks per CU)
             const int opt_r = p->opt_dw_rows;
             int rows_per_thread = opt_r ? opt_r : ((g.Ho + 2 * th1 - 1) / (2 * th1) * (2 * th1) - g.Ho) * 4 <= g.Ho ? 2 : 1;
-            if (wide && !opt_r && static_cast<long long>(batch) * ((g.Wo + tw - 1) / tw) * ((g.Ho + 2 * th1 - 1) / (2 * th1)) * (g.Co / 128) < 1024)
+            if (cbw != 32 && !opt_r && static_cast<long long>(batch) * ((g.Wo + tw - 1) / tw) * ((g.Ho + 2 * th1 - 1) / (2 * th1)) * (g.Co / cbw) < 512)
                 rows_per_thread = 1;
             const int th = th1 * rows_per_thread;
-            a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + th - 1) / th; a.cblocks = wide ? g.Co / 128 : (g.Co + 31) / 32;
+            a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + th - 1) / th; a.cblocks = (g.Co + cbw - 1) / cbw;
             a.xor_mask = p->xor_mask; a.pad_word = p->pad_word; a.rq = p->rq;
             const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y * a.cblocks;
             if (nb > 0x7fffffffll - 8) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
@@ -1152,10 +1155,18 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             const dim3 grid(static_cast<unsigned>(a.xcd_chunk) * 8u);
             a.wpack2 = p->w_dot4b;
             const bool w2 = p->w_dot4b != nullptr;
-            NoteKernel("Depthwise3x3Kernel<%d, %d, %s, %d>", g.stride_x, rows_per_thread, BoolName(w2), wide ? 128 : 32);
+            NoteKernel("Depthwise3x3Kernel<%d, %d, %s, %d>", g.stride_x, rows_per_thread, BoolName(w2), cbw);
             const int variant = (g.stride_x == 1 ? 0 : 4) + (rows_per_thread == 2 ? 0 : 2) + (w2 ? 1 : 0);
-            switch (variant + (wide ? 8 : 0))
+            switch (variant + (wide ? 8 : mid ? 16 : 0))
             {
+            case 16: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2, false, 64>), grid, dim3(256), 0, stream, a); break;
+            case 17: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2, true, 64>), grid, dim3(256), 0, stream, a); break;
+            case 18: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1, false, 64>), grid, dim3(256), 0, stream, a); break;
+            case 19: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1, true, 64>), grid, dim3(256), 0, stream, a); break;
+            case 20: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 2, false, 64>), grid, dim3(256), 0, stream, a); break;
+            case 21: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 2, true, 64>), grid, dim3(256), 0, stream, a); break;
+            case 22: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 1, false, 64>), grid, dim3(256), 0, stream, a); break;
+            case 23: hipLaunchKernelGGL((Depthwise3x3Kernel<2, 1, true, 64>), grid, dim3(256), 0, stream, a); break;
             case 0: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2, false>), grid, dim3(256), 0, stream, a); break;
             case 1: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 2, true>), grid, dim3(256), 0, stream, a); break;
             case 2: hipLaunchKernelGGL((Depthwise3x3Kernel<1, 1, false>), grid, dim3(256), 0, stream, a); break;

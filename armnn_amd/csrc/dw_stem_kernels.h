@@ -57,6 +57,8 @@ __device__ __forceinline__ int XcdContiguousWorkItem(int block, int chunk)
 // are read and transposed once, and the per-thread set-up (staging, constants, addresses) is spread over twice the
 // outputs; R = 1 keeps more blocks in flight for small feature maps.
 //
+// CB = 64 (channel counts that are odd multiples of 64): 64 channels of a tile of 4 R rows x 4 P pixels, 16 lanes per
+// pixel; with 64 channels in all a tile row is then one contiguous run of memory.
 // CB = 128 (channel counts that are multiples of 128): a block takes 128 channels of a tile of 4 R rows x 2 P pixels, 32
 // lanes per pixel.  Every pixel it loads or stores is then one whole 128-byte line instead of a quarter of one; the
 // smaller tile costs more halo (1.56 x instead of 1.27 x at stride 1).  The stores are ordinary ones: dwords written
@@ -64,19 +66,19 @@ __device__ __forceinline__ int XcdContiguousWorkItem(int block, int chunk)
 template <int S, int R, bool W2 = false, int CB = 32>
 __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
 {
-    static_assert(CB == 32 || CB == 128, "32 or 128 channels per block");
+    static_assert(CB == 32 || CB == 64 || CB == 128, "32, 64 or 128 channels per block");
     constexpr int LPC = CB / 4;                  // lanes per pixel
-    constexpr int XG = CB == 32 ? 4 : 2;         // thread columns
-    constexpr int TH = (256 / (LPC * XG)) * R;   // 8 R or 4 R output rows per tile
+    constexpr int XG = CB == 128 ? 2 : 4;        // thread columns
+    constexpr int TH = (256 / (LPC * XG)) * R;   // 8 R (CB = 32) or 4 R output rows per tile
     constexpr int CPP = CB / 16;                 // 16-byte staging chunks per pixel
     constexpr int P = S == 1 ? 4 : 2;            // outputs per thread and row
     constexpr int TW = P * XG;                   // outputs per tile row
     constexpr int HR = TH * S + 2;               // halo rows held in LDS
     constexpr int HC = TW * S + 2;               // halo columns
     constexpr int IR = (R - 1) * S + 3;          // input rows a thread walks
-    // bytes per pixel in LDS.  CB = 32: 48 spreads the dword reads of a wave's eight pixels over the banks; CB = 128: the 32
-    // lanes of a pixel read 128 contiguous bytes
-    constexpr int PITCH = CB == 32 ? 48 : 128;
+    // bytes per pixel in LDS.  CB = 32: 48 spreads the dword reads of a wave's eight pixels over the banks; CB = 64: 80 does
+    // the same for the four pixels (P S pixels apart) a wave reads; CB = 128: the 32 lanes of a pixel read 128 contiguous bytes
+    constexpr int PITCH = CB == 32 ? 48 : CB == 64 ? 80 : 128;
     __shared__ __attribute__((aligned(16))) uint8_t tile[HR * HC * PITCH];
 
     int b = XcdContiguousWorkItem(blockIdx.x, a.xcd_chunk);

@@ -300,10 +300,11 @@ def test_depthwise_rows_per_thread_variants_give_the_same_bytes():
             np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} rows {rows}")
 
 
-def test_depthwise_128_channel_blocks_give_the_same_bytes():
+def test_depthwise_64_and_128_channel_blocks_give_the_same_bytes():
     """Channel counts that are multiples of 128 run the 3x3 depthwise kernel with 128 channels per block (whole lines per
-    pixel): large, mid-sized and tiny feature maps of ragged sizes, both strides, one and two rows per thread, uint8
-    activations, weights with a zero point (two int8 halves), against the 32-channel blocks and the plain kernel."""
+    pixel), the other multiples of 64 with 64: large, mid-sized and tiny feature maps of ragged sizes, both strides, one
+    and two rows per thread, uint8 activations, weights with a zero point (two int8 halves), against the 32-channel
+    blocks and the plain kernel."""
     U8 = DataType.QAsymmU8
     cs = [cases.make_conv_case("dw128_s1_57x53", 711, n=2, h=57, w=53, ci=128, depthwise=True, act=cases.RELU6),
           cases.make_conv_case("dw128_s2_57x53_u8", 712, n=2, h=57, w=53, ci=256, depthwise=True, stride=(2, 2), in_dtype=U8, in_offset=140, out_offset=5),
@@ -312,6 +313,11 @@ def test_depthwise_128_channel_blocks_give_the_same_bytes():
           cases.make_conv_case("dw128_s1_29x27", 716, n=3, h=29, w=27, ci=256, depthwise=True, act=cases.RELU6),
           cases.make_conv_case("dw128_s2_29x27", 717, n=3, h=29, w=27, ci=128, depthwise=True, stride=(2, 2), act=cases.RELU),
           cases.make_conv_case("dw128_s1_15x13_u8", 718, n=5, h=15, w=13, ci=512, depthwise=True, in_dtype=U8, in_offset=131, out_offset=2),
+          cases.make_conv_case("dw64_s2_113x59", 719, n=2, h=113, w=59, ci=64, depthwise=True, stride=(2, 2), act=cases.RELU6),
+          cases.make_conv_case("dw64_s1_37x41_u8", 720, n=2, h=37, w=41, ci=192, depthwise=True, in_dtype=U8, in_offset=99, out_offset=-7, act=cases.RELU),
+          cases.make_conv_case("dw64_s1_6x9", 721, n=3, h=6, w=9, ci=64, depthwise=True),
+          cases.make_conv_case("dw64_s2_30x30_zero_point_weights", 722, n=1, h=30, w=30, ci=320, depthwise=True, stride=(2, 2), per_axis=False, w_std=60.0,
+                               w_dtype=U8, w_offset=101, in_dtype=U8, in_offset=120, out_offset=3, act=cases.RELU6),
           cases.make_conv_case("dw128_s1_64x50_zero_point_weights", 715, n=1, h=64, w=50, ci=128, depthwise=True, per_axis=False, w_std=60.0,
                                w_dtype=U8, w_offset=93, in_dtype=U8, in_offset=120, out_offset=3, act=cases.RELU6)]
     for c in cs:
@@ -327,7 +333,9 @@ def test_depthwise_128_channel_blocks_give_the_same_bytes():
                     shim.set_option("dw_cb", 0)
                     shim.set_option("dw_rows", 0)
                 print(f"{c.name} blocks {cb or 'auto'} rows {rows}: {kernel}", flush=True)
-                assert kernel.startswith("Depthwise3x3Kernel<") and kernel.endswith(", 128>") == (cb == 0), kernel
+                channels = c.x.info.shape[3]
+                blocks = 32 if cb == 32 else 128 if channels % 128 == 0 else 64
+                assert kernel.startswith("Depthwise3x3Kernel<") and kernel.endswith(f", {blocks}>"), kernel
                 np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} blocks {cb} rows {rows}")
     with pytest.raises(shim.ShimError):
         shim.set_option("dw_cb", 64)
