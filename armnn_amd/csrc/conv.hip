@@ -409,7 +409,14 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             const std::vector<uint8_t> padbytes(16, static_cast<uint8_t>((zb ^ (g.in_u8 ? 0x80u : 0u)) & 0xffu));
             if (int rc = Upload(reinterpret_cast<void**>(&p->pad16), padbytes.data(), padbytes.size())) return rc;
         }
-        p->info = d.stride_x == 1 ? "depthwise3x3_dot4_lds stride 1, tile 8x16x32" : "depthwise3x3_dot4_lds stride 2, tile 8x8x32";
+        {
+            // rows x pixels x channels of a block's tile with one output row per thread (twice the rows with two)
+            const int cbw = p->opt_dw_cb == 32 ? 32 : (Co % 128) == 0 ? 128 : (Co % 64) == 0 ? 64 : 32;
+            const int pixels = (cbw == 128 ? 2 : 4) * (d.stride_x == 1 ? 4 : 2);
+            char buf[96];
+            std::snprintf(buf, sizeof(buf), "depthwise3x3_dot4_lds stride %d, tile %dx%dx%d", static_cast<int>(d.stride_x), cbw == 32 ? 8 : 4, pixels, cbw);
+            p->info = buf;
+        }
         if (p->w_dot4b) p->info += ", weights minus their zero point as two int8 halves";
     }
     else if (algo == MI355X_ALGO_DEPTHWISE)

@@ -196,8 +196,9 @@ def main():
                          "pointwise + the depthwise after it where whole images fit a block")
     ap.add_argument("--no-fuse-add", action="store_true",
                     help="launch a residual Addition on its own instead of inside the convolution that feeds it")
-    ap.add_argument("--lanes", type=int, default=2,
-                    help="split the batch into this many slices, each running the network on a stream of its own")
+    ap.add_argument("--lanes", type=int, default=0,
+                    help="split the batch into this many slices, each running the network on a stream of its own "
+                         "(default: 2 for batches of at least 16 images that halve, else 1)")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
     ap.add_argument("--profile-pass", action="store_true",
                     help="for rocprofv3 --pmc: one 64 MiB calibration copy (1 B read + 1 B written per element), then ONE "
@@ -223,6 +224,8 @@ def main():
     from armnn_amd import shim
     from armnn_amd.executor import DeviceNetwork
 
+    if args.lanes == 0:
+        args.lanes = 2 if batch >= 16 and batch % 2 == 0 else 1
     dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev
@@ -368,7 +371,7 @@ def main():
         config["backend_path"] = bp
 
     line = {
-        "metric": "int8 images/sec MobileNetV1 b64 @1 GPU" if args.net == "mobilenet_v1" else f"int8 images/sec {args.net} b{batch} @1 GPU",
+        "metric": f"int8 images/sec MobileNetV1 b{batch} @1 GPU" if args.net == "mobilenet_v1" else f"int8 images/sec {args.net} b{batch} @1 GPU",
         "value": images_per_s, "unit": "images/sec", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "int8", "data": "synthetic",
