@@ -299,6 +299,27 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
 
     // ---- epilogue: requantize, pack 4 channels per dword, stage the byte tile in LDS, coalesced write-out -----------
     uint8_t* Os = smem;
+    constexpr int CHUNKS = BN / 16;
+    constexpr int ROWS_PER_PASS = NT / CHUNKS;
+    constexpr int NP = (BM + ROWS_PER_PASS - 1) / ROWS_PER_PASS;   // 16-byte pieces a thread writes
+    const int oc = tid % CHUNKS;
+    const int orow = tid / CHUNKS;
+    const int c0 = tn * BN + oc * 16;
+    // The other input of an Addition that runs in this write-out: every piece a thread will need is requested here, before
+    // the requantization, from clamped addresses (no load waits inside a divergent branch).  Tiles of more than four
+    // pieces per thread request them after the requantization instead, when the accumulators' registers are free.
+    constexpr bool EARLY = NP <= 4;
+    const bool fuse = a.res != nullptr && (a.Co & 15) == 0;
+    v4i other[NP] = {};
+    auto load_other = [&]() {
+#pragma unroll
+        for (int i = 0; i < NP; ++i)
+        {
+            const int m = min(tm * BM + min(orow + i * ROWS_PER_PASS, BM - 1), a.M - 1);
+            other[i] = *reinterpret_cast<const v4i*>(a.res + static_cast<long long>(m) * a.Co + min(c0, a.Co - 16));
+        }
+    };
+    if (EARLY && fuse) load_other();
     if constexpr (AW)
     {
 #pragma unroll
@@ -324,24 +345,21 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
         }
     }
     __syncthreads();
-    constexpr int CHUNKS = BN / 16;
-    constexpr int ROWS_PER_PASS = NT / CHUNKS;
-    const int oc = tid % CHUNKS;
-    const int orow = tid / CHUNKS;
-    const int c0 = tn * BN + oc * 16;
+    if (!EARLY && fuse) load_other();
     const OutPtr outp = MakeOutPtr(a.y, static_cast<long long>(a.M) * a.Co);
     if ((a.Co & 15) == 0)
     {
         if (c0 < a.Co)
         {
 #pragma unroll
-            for (int r = orow; r < BM; r += ROWS_PER_PASS)
+            for (int i = 0; i < NP; ++i)
             {
+                const int r = orow + i * ROWS_PER_PASS;
                 const int m = tm * BM + r;
-                if (m < a.M)
+                if (r < BM && m < a.M)
                 {
                     v4i ov = *reinterpret_cast<const v4i*>(Os + r * LDO + oc * 16);
-                    if (a.res) ov = AddResidual16(ov, *reinterpret_cast<const v4i*>(a.res + static_cast<long long>(m) * a.Co + c0), a.add);
+                    if (fuse) ov = AddResidual16(ov, other[i], a.add);
                     StoreOut16(outp, static_cast<long long>(m) * a.Co + c0, ov);
                 }
             }

@@ -145,7 +145,33 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
         constexpr int CH = BN / 16;                 // 16-byte chunks per row
-        if ((a.N & 15) == 0)
+        if ((a.N & 15) == 0 && a.res)
+        {
+            // the Addition's other input: all of a tile's loads are issued before the first is used (clamped addresses, so
+            // none sits in a divergent branch and waits there)
+            constexpr int NJ = 32 * CH / 64;
+            v4i other[NJ];
+#pragma unroll
+            for (int i = 0; i < NJ; ++i)
+            {
+                const int j = lane + 64 * i;
+                const int row = min(t * 32 + j / CH, a.M - 1);
+                const int c0 = min(n0 + (j % CH) * 16, a.N - 16);
+                other[i] = *reinterpret_cast<const v4i*>(a.res + static_cast<long long>(row) * a.N + c0);
+            }
+#pragma unroll
+            for (int i = 0; i < NJ; ++i)
+            {
+                const int j = lane + 64 * i;
+                const int r = j / CH, cc = j % CH;
+                const int row = t * 32 + r;
+                const int c0 = n0 + cc * 16;
+                if (row < a.M && c0 < a.N)
+                    StoreOut16(outp, static_cast<long long>(row) * a.N + c0,
+                               AddResidual16(*reinterpret_cast<const v4i*>(ostage + r * LDO + cc * 16), other[i], a.add));
+            }
+        }
+        else if ((a.N & 15) == 0)
         {
 #pragma unroll
             for (int j = lane; j < 32 * CH; j += 64)
@@ -154,11 +180,7 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
                 const int row = t * 32 + r;
                 const int c0 = n0 + cc * 16;
                 if (row < a.M && c0 < a.N)
-                {
-                    v4i ov = *reinterpret_cast<const v4i*>(ostage + r * LDO + cc * 16);
-                    if (a.res) ov = AddResidual16(ov, *reinterpret_cast<const v4i*>(a.res + static_cast<long long>(row) * a.N + c0), a.add);
-                    StoreOut16(outp, static_cast<long long>(row) * a.N + c0, ov);
-                }
+                    StoreOut16(outp, static_cast<long long>(row) * a.N + c0, *reinterpret_cast<const v4i*>(ostage + r * LDO + cc * 16));
             }
         }
         else
