@@ -66,7 +66,7 @@ struct ChanTab
 // nothing to overlap it.  With the sc1 bit (agent scope) the L2 writes the line through as the store is issued, so the
 // write-back runs beside the rest of the kernel and the data is where the next kernel -- whose blocks run on any XCD --
 // reads it from.  (The nt bit instead also helps a kernel timed alone but makes the next layer slower.)  Only for stores
-// that cover whole lines per instruction: the 32-channel depthwise blocks' 32-byte pieces and the pooling kernel's dwords,
+// of 16 bytes per lane that cover whole lines per instruction: the depthwise blocks' and the pooling kernel's dwords,
 // written through one by one, are slower than ordinary stores that L2 merges.
 //   The bit is set through the buffer-store builtins (their cache-policy argument), which the compiler knows as vector
 // memory instructions; a hand-written store instruction in inline assembly is invisible to its hazard and wait-count
