@@ -108,16 +108,44 @@ int main(int argc, char** argv)
         const double msPinned = 1e3 * std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() / steps;
         const bool same = std::memcmp(pout, pageable.data(), pageable.size()) == 0;
 
+        // input and output resident on the device (adopted device memory): what one inference costs without the bus
+        double msDevice = 0.0;
+        bool deviceSame = true;
+        void *din = nullptr, *dout = nullptr;
+        {
+            if (mi355x_malloc(&din, input.size()) != 0 || mi355x_malloc(&dout, pageable.size()) != 0) throw std::runtime_error(mi355x_last_error());
+            if (mi355x_memcpy_h2d(din, input.data(), input.size(), nullptr) != 0 || mi355x_device_synchronize() != 0) throw std::runtime_error(mi355x_last_error());
+            const auto dinIds = rt->ImportInputs(id, {{0, ConstTensor(constIn, din)}}, MemorySource::Malloc);
+            const auto doutIds = rt->ImportOutputs(id, {{0, Tensor(outInfo, dout)}}, MemorySource::Malloc);
+            if (dinIds.size() == 1 && doutIds.size() == 1)
+            {
+                for (int i = 0; i < warmup; ++i)
+                    if (rt->EnqueueWorkload(id, {}, {}, dinIds, doutIds) != Status::Success) throw std::runtime_error("EnqueueWorkload failed");
+                mi355x_device_synchronize();
+                t0 = std::chrono::steady_clock::now();
+                for (int i = 0; i < steps; ++i)
+                    if (rt->EnqueueWorkload(id, {}, {}, dinIds, doutIds) != Status::Success) throw std::runtime_error("EnqueueWorkload failed");
+                mi355x_device_synchronize();
+                msDevice = 1e3 * std::chrono::duration<double>(std::chrono::steady_clock::now() - t0).count() / steps;
+                std::vector<uint8_t> back(pageable.size());
+                if (mi355x_memcpy_d2h(back.data(), dout, back.size(), nullptr) != 0 || mi355x_device_synchronize() != 0) throw std::runtime_error(mi355x_last_error());
+                deviceSame = back == pageable;
+            }
+            mi355x_device_synchronize();
+        }
+
         std::ofstream fout(argv[3], std::ios::binary);
         fout.write(static_cast<const char*>(pout), static_cast<std::streamsize>(pageable.size()));
         rt->UnloadNetwork(id);
         mi355x_host_free(pin);
         mi355x_host_free(pout);
-        std::printf("{\"batch\": %u, \"steps\": %d, \"ms_pageable\": %.4f, \"ms_pinned\": %.4f, \"pinned_equals_pageable\": %s, "
+        mi355x_free(din);
+        mi355x_free(dout);
+        std::printf("{\"batch\": %u, \"steps\": %d, \"ms_pageable\": %.4f, \"ms_pinned\": %.4f, \"ms_device_resident\": %.4f, \"pinned_equals_pageable\": %s, "
                     "\"optimized_layers\": %zu, \"activation_layers_left\": %zu, \"memcopy_layers\": %zu, \"conv_layers\": %zu, "
                     "\"depthwise_layers\": %zu, \"add_layers\": %zu, \"additions_running_a_convolution\": %llu}\n",
-                    nf.batch, steps, msPageable, msPinned, same ? "true" : "false", nLayers, nAct, nCopy, nConv, nDw, nAdd, Mi355xAdditionWorkload::PairsFormed());
-        return same ? 0 : 1;
+                    nf.batch, steps, msPageable, msPinned, msDevice, (same && deviceSame) ? "true" : "false", nLayers, nAct, nCopy, nConv, nDw, nAdd, Mi355xAdditionWorkload::PairsFormed());
+        return (same && deviceSame) ? 0 : 1;
     }
     catch (const std::exception& e)
     {

@@ -355,11 +355,14 @@ def main():
             bp["output_equals_executor"] = backend_out == executor_out
             bp["images_per_sec_pageable_io"] = batch / (backend["ms_pageable"] * 1e-3)
             bp["images_per_sec_adopted_pinned_io"] = batch / (backend["ms_pinned"] * 1e-3)
+            if backend.get("ms_device_resident"):
+                bp["images_per_sec_device_resident_io"] = batch / (backend["ms_device_resident"] * 1e-3)
             bp["path"] = "INetwork -> Optimize({Mi355x}) -> IRuntime::LoadNetwork -> IRuntime::EnqueueWorkload (armnn_amd/backend/test/BackendBench.cpp)"
         if real is not None and real_out is not None:
             # the same program built against the reference's source tree: the reference's own optimizer, loaded network and
             # runtime drive the backend
             bp["reference_runtime"] = {"ms_pageable": real["ms_pageable"], "ms_pinned": real["ms_pinned"],
+                                       "ms_device_resident": real.get("ms_device_resident"),
                                        "output_equals_executor": real_out == executor_out,
                                        "images_per_sec_pageable_io": batch / (real["ms_pageable"] * 1e-3),
                                        "images_per_sec_adopted_pinned_io": batch / (real["ms_pinned"] * 1e-3),
