@@ -239,6 +239,8 @@ BackendCapabilities Mi355xBackend::GetCapabilities() const
 //   CL backends do (src/backends/aclCommon/ArmComputeSubgraphUtils.hpp:60-109).
 // * A Convolution2d without an activation whose output goes to one Addition of this backend and nowhere else is marked
 //   (Mi355xFeedsOnlyAnAddition): the two workloads may then run as one launch (Mi355xAdditionWorkload).
+// * A Reshape that only flattens the dimensions behind the batch, in front of a FullyConnected, is dropped: the
+//   FullyConnected reads the unflattened tensor (same bytes in the same order).
 // * A constant Pad of height and width in front of a Convolution2d, DepthwiseConvolution2d or Pooling2d moves into that
 //   layer's own padding when the padded value is the layer's neutral element, as CpuRef does
 //   (src/backends/reference/RefBackend.cpp:72-184 with the rules of src/armnn/optimizations/FoldPadIntoLayer2d.hpp:21-145).
@@ -284,6 +286,26 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
             }
         }
 
+        // the Reshape in front of a FullyConnected, if it only flattens what follows the batch: FullyConnected takes the
+        // unflattened tensor as it is (FullyConnectedLayer.cpp:64-80 infers {shape[0], outputs} from any input;
+        // WorkloadData.cpp:1036-1098 admits 2 or 4 dimensions), and the copy the Reshape workload would make goes away
+        Layer* flat = nullptr;
+        if (type == LayerType::FullyConnected)
+        {
+            OutputSlot* source = base->GetInputSlot(0).GetConnectedOutputSlot();
+            Layer* producer = source ? &source->GetOwningLayer() : nullptr;
+            if (producer && producer->GetType() == LayerType::Reshape && members.count(producer) && !consumed.count(producer) &&
+                source->GetNumConnections() == 1 && producer->GetInputSlot(0).GetConnectedOutputSlot() != nullptr)
+            {
+                const TensorInfo& before = producer->GetInputSlot(0).GetConnectedOutputSlot()->GetTensorInfo();
+                const TensorInfo& after = source->GetTensorInfo();
+                if ((before.GetNumDimensions() == 2 || before.GetNumDimensions() == 4) && after.GetNumDimensions() == 2 &&
+                    before.GetShape()[0] == after.GetShape()[0] && before.GetNumElements() == after.GetNumElements() &&
+                    SameQuantization(before, after))
+                    flat = producer;
+            }
+        }
+
         // the Activation behind the layer, if it is a clamp in the layer's own output quantization
         Layer* act = nullptr;
         if (Fusable(*base) && base->GetAdditionalInformation<ActivationDescriptor>() == nullptr && base->GetOutputSlot(0).GetNumConnections() == 1)
@@ -308,10 +330,11 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
                 next->GetInputSlot(0).GetConnectedOutputSlot() != next->GetInputSlot(1).GetConnectedOutputSlot())
                 residual = true;
         }
-        if (!pad && !act && !residual) continue;
+        if (!pad && !act && !residual && !flat) continue;
 
         std::string name = base->GetName();
         if (pad) name = std::string("folded-") + pad->GetName() + "-into-" + name;
+        if (flat) name = std::string("folded-") + flat->GetName() + "-into-" + name;
         if (act) name = std::string("fused-") + act->GetName() + "-into-" + name;
         INetwork& net = views.GetINetworkRef();
         IConnectableLayer* replacement = nullptr;
@@ -339,15 +362,16 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
 
         SubgraphView::IConnectableLayers replaced;
         SubgraphView::IInputSlots ins;
-        if (pad) replaced.push_back(pad);
+        Layer* front = pad ? pad : flat;
+        if (front) replaced.push_back(front);
         replaced.push_back(base);
         if (act) replaced.push_back(act);
-        ins.push_back(pad ? &pad->GetInputSlot(0) : &base->GetInputSlot(0));
+        ins.push_back(front ? &front->GetInputSlot(0) : &base->GetInputSlot(0));
         for (unsigned int i = 1; i < base->GetNumInputSlots(); ++i) ins.push_back(&base->GetInputSlot(i));
         SubgraphView::IOutputSlots outs{&last->GetOutputSlot(0)};
         SubgraphView substitutable(std::move(replaced), std::move(ins), std::move(outs));
         views.AddSubstitution({std::move(substitutable), SubgraphView(replacement)});
-        for (Layer* l : {pad, base, act})
+        for (Layer* l : {pad, flat, base, act})
             if (l) consumed.insert(l);
     }
 

@@ -495,6 +495,67 @@ TEST_CASE("optimize: a convolution that feeds one Addition and nothing else is m
 
 namespace
 {
+// input [n, 2, 2, 16] -> Reshape -> FullyConnected (64 -> 10) + ReLU6 -> output
+INetworkPtr ReshapeFcNet(const TensorShape& reshaped, bool reshapedAlsoAnOutput)
+{
+    INetworkPtr net = INetwork::Create();
+    const TensorInfo in = ActInfo({2, 2, 2, 16}, DataType::QAsymmS8, 0.05f, -3);
+    TensorInfo flat = in;
+    flat.SetShape(reshaped);
+    QLayer fc = MakeFc(flat, 10, 0.1f, -128, true, 17);
+    fc.relu6 = true;
+    IConnectableLayer* input = net->AddInputLayer(0, "input");
+    input->GetOutputSlot(0).SetTensorInfo(in);
+    IConnectableLayer* reshape = net->AddReshapeLayer(ReshapeDescriptor(reshaped), "reshape");
+    input->GetOutputSlot(0).Connect(reshape->GetInputSlot(0));
+    reshape->GetOutputSlot(0).SetTensorInfo(flat);
+    IOutputSlot& out = AddToNetwork(*net, reshape->GetOutputSlot(0), fc, "fc");
+    IConnectableLayer* output = net->AddOutputLayer(0, "output");
+    out.Connect(output->GetInputSlot(0));
+    if (reshapedAlsoAnOutput)
+    {
+        IConnectableLayer* out2 = net->AddOutputLayer(1, "output2");
+        reshape->GetOutputSlot(0).Connect(out2->GetInputSlot(0));
+    }
+    return net;
+}
+} // namespace
+
+TEST_CASE("optimize: a Reshape that only flattens what follows the batch goes into the FullyConnected behind it", "cpu")
+{
+    FixedDeviceSpec spec{kMi355x};
+    {
+        INetworkPtr net = ReshapeFcNet(TensorShape({2, 64}), false);
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, spec);
+        const Graph& g = opt->GetGraph();
+        CHECK(CountLayers(g, LayerType::Reshape) == 0);
+        CHECK(CountLayers(g, LayerType::Activation) == 0);
+        CHECK(CountLayers(g, LayerType::FullyConnected) == 1);
+        const Layer* fc = FindLayer(g, "folded-reshape-into-fc");
+        REQUIRE(fc != nullptr);
+        CHECK(fc->GetType() == LayerType::FullyConnected);
+        CHECK(fc->In(0).GetConnectedOutputSlot()->GetOwningLayer().GetType() == LayerType::Input);
+        CHECK(fc->In(0).GetConnectedOutputSlot()->GetTensorInfo().GetNumDimensions() == 4);
+        CHECK(fc->In(1).GetConnectedOutputSlot()->GetOwningLayer().GetType() == LayerType::Constant);
+        CHECK(fc->Out(0).GetTensorInfo().GetShape() == TensorShape({2, 10}));
+        auto ad = fc->GetAdditionalInformation<ActivationDescriptor>();
+        REQUIRE(ad != nullptr);
+        CHECK(ad->m_Function == ActivationFunction::BoundedReLu);
+    }
+    {
+        INetworkPtr net = ReshapeFcNet(TensorShape({1, 128}), false);      // the batch dimension changes: rows would differ
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, spec);
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Reshape) == 1);
+    }
+    {
+        INetworkPtr net = ReshapeFcNet(TensorShape({2, 64}), true);        // the flattened tensor is wanted as well
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, spec);
+        CHECK(CountLayers(opt->GetGraph(), LayerType::Reshape) == 1);
+    }
+}
+
+namespace
+{
 using PadList = std::vector<std::pair<unsigned int, unsigned int>>;
 
 TensorInfo Padded(const TensorInfo& in, const PadList& pads)
