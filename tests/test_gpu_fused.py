@@ -236,3 +236,37 @@ def test_convolution_with_fused_addition_equals_two_layers(port, cfg):
     if fn:
         want = port.activation(want, sum_info, fn, a, b)
     np.testing.assert_array_equal(fused, want.data)
+
+
+@pytest.mark.parametrize("tile", [96, 128, 256, 512])
+def test_fused_addition_in_the_large_tiles_equals_two_layers(tile):
+    """The implicit-GEMM kernel forced to 128x64, 128x128, 256x128 and 256x256 tiles (a thread then writes two to sixteen
+    16-byte pieces of the output; with more than four it requests the Addition's other input after the requantization
+    instead of before it): same bytes as the convolution followed by the Addition, ragged last row tile included."""
+    print("conv+add tile", tile, flush=True)
+    shim.Device()
+    c = cases.make_conv_case(f"pointwise_k256_co512_tile{tile}", 1900 + tile, n=2, h=33, w=31, ci=256, co=512, kh=1, kw=1, in_dtype=S8, in_scale=0.0235,
+                             in_offset=-7, out_scale=0.06, out_offset=11)
+    shim.set_option("igemm_tile", tile)
+    try:
+        plan = _plan(c)
+    finally:
+        shim.set_option("igemm_tile", 0)
+    n = c.x.info.shape[0]
+    rng = np.random.default_rng(78)
+    other_info = TensorInfo(c.out_info.shape, S8, (0.043,), -20)
+    other = QTensor(other_info, rng.integers(-128, 128, size=c.out_info.shape).astype(np.int8))
+    sum_info = TensorInfo(c.out_info.shape, S8, (0.09,), -128)
+    xd = shim.DeviceBuffer(c.x.data.nbytes).upload(c.x.data)
+    od = shim.DeviceBuffer(other.data.nbytes).upload(other.data)
+    mid = shim.DeviceBuffer(c.out_info.num_elements)
+    yf = shim.DeviceBuffer(c.out_info.num_elements)
+    plan.run(n, xd.ptr, mid.ptr)
+    conv_out = QTensor(c.out_info, mid.download(c.out_info.shape, np.int8))
+    fn, a, b = cases.RELU
+    two = shim.add(conv_out, other, sum_info, activation=fn, act_a=a, act_b=b)
+    plan.run_add(n, xd.ptr, od.ptr, other_info, sum_info, yf.ptr, activation=fn, act_a=a, act_b=b)
+    last = shim.last_kernel()
+    print(f"  {last}", flush=True)
+    assert last.startswith("IgemmLdsKernel<"), last
+    np.testing.assert_array_equal(yf.download(c.out_info.shape, np.int8), two.data)
