@@ -39,7 +39,7 @@ Mi355xConvolution2dWorkload* TakeCandidate()
     return w;
 }
 
-// deleter-side hook: a candidate that is destroyed before anything took it
+// the convolution workload the factory hands out: its destructor withdraws it as the candidate, should it still be one
 class CandidateConvolution final : public Mi355xConvolution2dWorkload
 {
 public:
