@@ -170,6 +170,8 @@ void Mi355xConvolution2dWorkload::BuildPlan() const
                                        bias ? reinterpret_cast<const int32_t*>(bias->data.data()) : nullptr,
                                        bias ? &bias->quant : nullptr, &m_Plan),
                   "mi355x_conv2d_create");
+    // the batch runs as this many slices side by side (Execute() asks the same question for every launch)
+    mi355x::Check(mi355x_conv2d_set_concurrency(m_Plan, mi355x::LanesFor(in.GetShape()[0])), "mi355x_conv2d_set_concurrency");
     WorkloadInfo details = m_Info;
     details.m_ConvolutionMethod = Optional<std::string>(Describe(m_Plan));
     ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xConvolution2dWorkload_Plan", m_Data.m_Parameters, details, this->GetGuid());

@@ -47,6 +47,7 @@ struct mi355x_conv2d_s
     int pw_bn = 0, pw_ks = 0;      // pointwise GEMM kernel configuration (0: not applicable)
     bool bk128 = false;            // implicit GEMM walks K in 128-byte tiles
     bool halo_ok = false;          // shape fits the resident-tile kernel (weights without a zero point are checked at launch)
+    unsigned concurrency = 1;      // launches of the plan's network that run side by side (mi355x_conv2d_set_concurrency)
     int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 96 (= 128x64) / 128: the "igemm_tile" option at plan creation
     int opt_igemm_lds = 2, opt_dw_rows = 0, opt_dw_cb = 0, opt_stem_dot4 = 0;     // the other process-wide options, as they stood at plan creation
                                    // (launches read the plan, never the mutable globals: plans may run on any host thread)
@@ -854,9 +855,13 @@ int LaunchIgemmLds(const mi355x_conv2d_s* p, int stages, uint32_t batch, const v
     return u8 ? LaunchIgemmLdsT<BM, BN, WM, WN, 2, true, false>(p, batch, x, y, stream) : LaunchIgemmLdsT<BM, BN, WM, WN, 2, false, false>(p, batch, x, y, stream);
 }
 
+// set around a call of LaunchHalo that only asks whether the kernel would take the launch
+thread_local bool t_halo_probe = false;
+
 template <int CI, int WM, int WN, int TP, int ST, bool U8>
 int LaunchHaloT(const HaloArgs& a, int smem, hipStream_t stream)
 {
+    if (t_halo_probe) return 0;
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&HaloConvKernel<CI, WM, WN, TP, ST, U8>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     MI355X_HIP(attr);
@@ -994,10 +999,25 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             return LaunchPwKs<32>(p, Mrows, x, y, stream);
         }
         // Small filters at stride 1 over 64 / 128 / 256 channels: the input tile stays in LDS for all taps
+        // -- unless the launch shares the device with another lane's launches: a block of that kernel holds a whole input
+        // tile in LDS, few of them fit a CU, and beside a neighbour the implicit GEMM with 128 x 64 tiles is the faster
+        // choice (ResNet-50 b32 in two lanes: 13.7 us per step for its three 3 x 3 x 64 layers; alone the kernel below
+        // wins).  Measured for the 64-channel form only.
+        const bool shared_device = p->concurrency > 1 && p->tile_override == 0;
+        bool gemm_instead = false;
         if (p->halo_ok && p->zw_neg == 0 && p->opt_igemm_lds != 0 && (p->tile_override == 0 || (p->tile_override == 3000 || p->tile_override == 3001)))
         {
-            const int rc = LaunchHalo(p, batch, x, y, stream);
-            if (rc >= 0) return rc;
+            if (shared_device && g.Ci == 64)
+            {
+                t_halo_probe = true;
+                gemm_instead = LaunchHalo(p, batch, x, y, stream) >= 0;
+                t_halo_probe = false;
+            }
+            if (!gemm_instead)
+            {
+                const int rc = LaunchHalo(p, batch, x, y, stream);
+                if (rc >= 0) return rc;
+            }
         }
         // Tile choice: the large tile has the best MFMA : LDS-traffic ratio, but a launch needs several blocks per CU
         // in flight to hide global-load latency, so problems that would yield few large tiles take 64x64 tiles
@@ -1008,7 +1028,9 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         const bool bk128 = p->bk128;
         // 256x256 tiles (16 waves) halve the operand traffic per output once they alone fill three quarters of the CUs
         const long long huge = ((M + 255) / 256) * ((g.Co + 255) / 256);
-        const int tile = p->tile_override ? p->tile_override : big < 400 ? 64 : (huge >= 192 && g.Co >= 256) ? 512 : 128;
+        const int tile = p->tile_override ? p->tile_override
+                       : gemm_instead ? 96
+                       : big < 400 ? 64 : (huge >= 192 && g.Co >= 256) ? 512 : 128;
         // channel counts that are multiples of 128: k-tiles go from global memory straight into LDS
         const int lds_stages = p->opt_igemm_lds;
         if (lds_stages != 0 && bk128 && (g.Ci % 128) == 0)
@@ -1033,7 +1055,9 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
                 // rate.  K split over groups of waves inside the block: 17.4 -> 13.5 us for 7 x 7 x 512 -> 512, 3 x 3, 16 images.
                 const long long blocks64 = ((M + 63) / 64) * ((g.Co + 63) / 64);
                 if (blocks64 <= 128) return LaunchIgemmKSplit(p, 4, batch, x, y, stream);
-                if (blocks64 <= 256) return LaunchIgemmKSplit(p, 2, batch, x, y, stream);
+                // two groups: only when the launch has the device to itself (beside another lane's launches the plain
+                // 64 x 64 blocks of 256 threads co-run better: ResNet-50 b32 in two lanes, 6.3 us per step for five layers)
+                if (blocks64 <= 256 && !shared_device) return LaunchIgemmKSplit(p, 2, batch, x, y, stream);
             }
             if (tile == 64)
             {
@@ -1425,6 +1449,14 @@ int mi355x_conv2d_run_fused(mi355x_conv2d_t dw, mi355x_conv2d_t pw, uint32_t bat
 int mi355x_conv2d_destroy(mi355x_conv2d_t plan)
 {
     delete plan;
+    return 0;
+}
+
+int mi355x_conv2d_set_concurrency(mi355x_conv2d_t plan, uint32_t lanes)
+{
+    if (!plan) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan is null");
+    if (lanes == 0) return SetError(MI355X_ERR_INVALID_ARGUMENT, "the number of lanes must be at least 1");
+    plan->concurrency = lanes;
     return 0;
 }
 

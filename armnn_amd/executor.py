@@ -76,6 +76,7 @@ class DeviceNetwork:
                 p = {k: v for k, v in l.params.items() if not k.startswith("_")}
                 plan = shim.Conv2dPlan(xin[0], l.weights, l.bias, yout, activation=l.act[0], act_a=l.act[1],
                                        act_b=l.act[2], algo=algo_overrides.get(l.name, shim.ALGO_AUTO), **p)
+                plan.set_concurrency(lanes)
                 self.plans.append(plan)
                 self.steps.append((l, self._conv_step(plan, xb[0].ptr, yb.ptr, xin[0].num_elements, yout.num_elements)))
                 self._step_plans.append(plan)

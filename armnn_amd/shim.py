@@ -28,7 +28,7 @@ EXPORTS = [
     "mi355x_event_destroy", "mi355x_event_record", "mi355x_stream_wait_event", "mi355x_event_synchronize", "mi355x_event_elapsed_ms",
     "mi355x_graph_capture_begin", "mi355x_graph_capture_end", "mi355x_graph_launch", "mi355x_graph_destroy",
     "mi355x_conv2d_create", "mi355x_conv2d_run", "mi355x_conv2d_destroy", "mi355x_conv2d_algo",
-    "mi355x_conv2d_fusable", "mi355x_conv2d_run_fused", "mi355x_conv2d_run_add",
+    "mi355x_conv2d_fusable", "mi355x_conv2d_run_fused", "mi355x_conv2d_run_add", "mi355x_conv2d_set_concurrency",
     "mi355x_fc_create", "mi355x_fc_run", "mi355x_fc_destroy", "mi355x_fc_algo",
     "mi355x_activation_run", "mi355x_pool2d_run", "mi355x_add_run", "mi355x_softmax_run", "mi355x_pad_run",
 ]
@@ -113,6 +113,7 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
             "mi355x_conv2d_algo": [V, C.POINTER(C.c_int32), C.c_char_p, C.c_size_t],
             "mi355x_conv2d_fusable": [V, V], "mi355x_conv2d_run_fused": [V, V, C.c_uint32, V, V, V],
             "mi355x_conv2d_run_add": [V, C.c_uint32, V, V, C.POINTER(Quant), C.POINTER(Quant), C.c_int32, C.c_float, C.c_float, V, V],
+            "mi355x_conv2d_set_concurrency": [V, C.c_uint32],
             "mi355x_fc_create": [C.POINTER(FcDesc), V, C.POINTER(ConstQuant), V, C.POINTER(ConstQuant), C.POINTER(V)],
             "mi355x_fc_run": [V, C.c_uint32, V, V, V], "mi355x_fc_destroy": [V],
             "mi355x_fc_algo": [V, C.POINTER(C.c_int32), C.c_char_p, C.c_size_t],
@@ -307,6 +308,10 @@ class Conv2dPlan:
         """Both layers without the intermediate tensor; bytes equal run() + second.run()."""
         _chk(self.lib.mi355x_conv2d_run_fused(self.plan, second.plan, batch, x_dev, y_dev, stream))
 
+    def set_concurrency(self, lanes: int):
+        """Tell the plan that `lanes` launches of its network run side by side (kernels with small blocks are preferred then)."""
+        _chk(self.lib.mi355x_conv2d_set_concurrency(self.plan, int(lanes)))
+
     def run_add(self, batch: int, x_dev: int, other_dev: int, other_info: TensorInfo, sum_info: TensorInfo, y_dev: int,
                 activation=ACT_NONE, act_a=0.0, act_b=0.0, stream=None):
         """This convolution and the Addition consuming it in one launch where the kernel can; bytes equal run() followed
@@ -370,9 +375,11 @@ class FullyConnectedPlan:
 
 
 # ---- one-call helpers: upload, run, download (tests and the smoke check) -------------------------------------
-def conv2d(x: QTensor, w: QTensor, b: Optional[QTensor], out_info: TensorInfo, **kw) -> QTensor:
+def conv2d(x: QTensor, w: QTensor, b: Optional[QTensor], out_info: TensorInfo, concurrency: int = 1, **kw) -> QTensor:
     Device()
     plan = Conv2dPlan(x.info, w, b, out_info, **kw)
+    if concurrency != 1:
+        plan.set_concurrency(concurrency)
     xd = DeviceBuffer(x.data.nbytes).upload(x.data)
     y = QTensor(out_info)
     yd = DeviceBuffer(y.data.nbytes)

@@ -199,6 +199,11 @@ int mi355x_conv2d_create(const mi355x_conv2d_desc* desc,
 int mi355x_conv2d_run(mi355x_conv2d_t plan, uint32_t batch, const void* input_dev, void* output_dev,
                       mi355x_stream_t stream);
 int mi355x_conv2d_destroy(mi355x_conv2d_t plan);
+/* How many launches of the network this plan belongs to run side by side on the device (a batch split into lanes on
+ * streams of their own); 1 after creation.  With more than one the plan prefers kernels whose blocks are small and
+ * many, which share a CU with a neighbour's blocks better than the kernels that are fastest alone (identical bytes
+ * either way).  No counterpart in the reference, whose workloads run one after the other on the calling thread. */
+int mi355x_conv2d_set_concurrency(mi355x_conv2d_t plan, uint32_t lanes);
 /* A Convolution2d and the Addition that consumes its output (a residual connection), run as one launch where the kernel
  * the plan resolves to can do it (the matrix-core kernels with 16-byte row stores), else as the convolution followed by
  * the Addition in place.  other_dev / other_quant: the Addition's other input, same shape as the convolution's output;

@@ -300,6 +300,33 @@ def test_depthwise_rows_per_thread_variants_give_the_same_bytes():
             np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} rows {rows}")
 
 
+def test_plans_told_that_they_share_the_device_pick_small_blocks_and_give_the_same_bytes():
+    """mi355x_conv2d_set_concurrency(plan, 2): the 3x3 convolution over 64 channels leaves the kernel that keeps its input
+    tile in LDS for the implicit GEMM with 128x64 tiles, and the 3x3 convolution over 256 channels at 14x14 leaves the
+    K split over two wave groups for plain 64x64 blocks; the four-group split of the smallest launches stays.  Same
+    bytes as alone, and as the direct kernel."""
+    picks = [(cases.make_conv_case("shared_3x3_c64_56", 841, n=16, h=56, w=56, ci=64, co=64, act=cases.RELU), "HaloConvKernel<64", "IgemmKernel<128, 64"),
+             (cases.make_conv_case("shared_3x3_c256_14", 842, n=16, h=14, w=14, ci=256, co=256, act=cases.RELU), "IgemmKSplitKernel<2", "IgemmLdsKernel<64, 64"),
+             (cases.make_conv_case("shared_3x3_c512_7", 843, n=16, h=7, w=7, ci=512, co=512, act=cases.RELU), "IgemmKSplitKernel<4", "IgemmKSplitKernel<4"),
+             (cases.make_conv_case("shared_3x3_c64_small", 844, n=1, h=20, w=20, ci=64, co=64, act=cases.RELU6), None, None)]
+    for c, alone_kernel, shared_kernel in picks:
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        fn, a, b = c.act
+        alone = shim.conv2d(c.x, c.w, c.b, c.out_info, activation=fn, act_a=a, act_b=b, **c.params)
+        k1 = shim.last_kernel()
+        shared = shim.conv2d(c.x, c.w, c.b, c.out_info, concurrency=2, activation=fn, act_a=a, act_b=b, **c.params)
+        k2 = shim.last_kernel()
+        print(f"{c.name}: alone {k1}; sharing the device {k2}", flush=True)
+        if alone_kernel is None:
+            assert k1 == k2, (k1, k2)             # where the resident-tile kernel would not run anyway, nothing changes
+        else:
+            assert k1.startswith(alone_kernel) and k2.startswith(shared_kernel), (k1, k2)
+        np.testing.assert_array_equal(alone.data, want.data, err_msg=c.name)
+        np.testing.assert_array_equal(shared.data, want.data, err_msg=c.name)
+    with pytest.raises(shim.ShimError):
+        shim.Conv2dPlan(picks[3][0].x.info, picks[3][0].w, picks[3][0].b, picks[3][0].out_info, **picks[3][0].params).set_concurrency(0)
+
+
 def test_depthwise_64_and_128_channel_blocks_give_the_same_bytes():
     """Channel counts that are multiples of 128 run the 3x3 depthwise kernel with 128 channels per block (whole lines per
     pixel), the other multiples of 64 with 64: large, mid-sized and tiny feature maps of ragged sizes, both strides, one
