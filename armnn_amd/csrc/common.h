@@ -78,6 +78,7 @@ struct Options
     int igemm_tile = 0;                // 0: automatic; 64, 96 (128x64), 128, 256, 512 (256x256), or 2256 / 2128 / 1256 (large-tile kernel), 2064 / 4064 (64x64 with K split over 2 / 4 wave groups), or 3000 (resident-tile kernel): every MFMA plan created meanwhile uses that implicit-GEMM tile
     int igemm_lds = 2;                 // LDS stages of the direct-to-LDS implicit GEMM (2 or 3); 0: use the register-staged kernel
     int dw_rows = 0;                   // output rows per thread of the 3x3 depthwise kernel: 0 automatic, 1 or 2 forced
+    int pw_slab = 0;                   // output channels per slab of the weight-stationary pointwise kernel: 0 automatic, 32 / 64 / 128 forced
     int dw_cb = 0;                     // channels per block of the 3x3 depthwise kernel: 0 automatic (128 where the count allows), 32 forced
     int stem_dot4 = 0;                 // 1: small-Ci convolutions stay on the v_dot4 kernel (tests compare it with the MFMA one)
 };

@@ -542,6 +542,9 @@ void ChoosePointwiseConfig(mi355x_conv2d_s* p)
     if (N > 64 && PwSmemBytes<128>(K) <= budget) bn = 128;
     else if (N > 32 && PwSmemBytes<64>(K) <= budget) bn = 64;
     else if (PwSmemBytes<32>(K) <= budget) bn = 32;
+    // the "pw_slab" option: a narrower slab than the automatic one (never wider than the layer's output)
+    const int forced = GlobalOptions().pw_slab;
+    if (forced != 0 && forced <= bn && PwSmemBytes<32>(K) <= budget) bn = forced;
     if (bn == 0) return;
     const int steps = K / 32;
     p->pw_bn = bn;

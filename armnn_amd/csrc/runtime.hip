@@ -143,6 +143,12 @@ int mi355x_set_option(const char* name, int value)
         GlobalOptions().dw_rows = value;
         return 0;
     }
+    if (std::strcmp(name, "pw_slab") == 0)
+    {
+        if (value != 0 && value != 32 && value != 64 && value != 128) return SetError(MI355X_ERR_INVALID_ARGUMENT, "pw_slab must be 0, 32, 64 or 128");
+        GlobalOptions().pw_slab = value;
+        return 0;
+    }
     if (std::strcmp(name, "dw_cb") == 0)
     {
         if (value != 0 && value != 32) return SetError(MI355X_ERR_INVALID_ARGUMENT, "dw_cb must be 0 or 32");

@@ -108,6 +108,9 @@ int  mi355x_abi_version(void);
  *   into LDS (input channels a multiple of 128); 0 selects the register-staged kernel instead (identical bytes).
  *   "dw_rows" = 0 | 1 | 2: output rows per thread of the 3x3 depthwise kernel (0: chosen from the feature-map height;
  *   identical bytes).
+ *   "pw_slab" = 0 | 32 | 64 | 128: output channels per weight slab of the weight-stationary kernel for 1x1 convolutions
+ *   with at most 128 input channels (0: the widest that fits the layer; a value wider than that is ignored; identical
+ *   bytes; tests and tuning).
  *   "dw_cb" = 0 | 32: channels per block of the 3x3 depthwise kernel (0: 128 where the channel count is a multiple of
  *   128, else 32; 32: always 32; identical bytes).
  * Unknown names and values outside these return MI355X_ERR_INVALID_ARGUMENT. */

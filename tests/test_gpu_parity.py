@@ -300,6 +300,33 @@ def test_depthwise_rows_per_thread_variants_give_the_same_bytes():
             np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} rows {rows}")
 
 
+def test_pointwise_slab_widths_give_the_same_bytes():
+    """The weight-stationary kernel for 1x1 convolutions with at most 128 input channels, forced to 32-, 64- and
+    128-channel weight slabs ("pw_slab"): ragged row counts, uint8 activations, an output width that is no multiple of
+    the slab; a value wider than the layer allows is ignored; against the direct kernel."""
+    U8 = DataType.QAsymmU8
+    cs = [cases.make_conv_case("slab_k64_co256", 851, n=2, h=31, w=29, ci=64, co=256, kh=1, kw=1, act=cases.RELU),
+          cases.make_conv_case("slab_k32_co64_u8", 852, n=3, h=17, w=19, ci=32, co=64, kh=1, kw=1, in_dtype=U8, in_offset=128, act=cases.RELU6),
+          cases.make_conv_case("slab_k128_co200", 853, n=1, h=23, w=23, ci=128, co=200, kh=1, kw=1)]
+    for c in cs:
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        seen = set()
+        for slab in (0, 32, 64, 128):
+            shim.set_option("pw_slab", slab)
+            try:
+                got = _gpu_conv(c, shim.ALGO_AUTO)
+                kernel = shim.last_kernel()
+            finally:
+                shim.set_option("pw_slab", 0)
+            print(f"{c.name} slab {slab}: {kernel}", flush=True)
+            assert kernel.startswith("PwGemmKernel<"), kernel
+            seen.add(kernel)
+            np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} slab {slab}")
+        assert len(seen) >= 2, seen
+    with pytest.raises(shim.ShimError):
+        shim.set_option("pw_slab", 48)
+
+
 def test_plans_told_that_they_share_the_device_pick_small_blocks_and_give_the_same_bytes():
     """mi355x_conv2d_set_concurrency(plan, 2): the 3x3 convolution over 64 channels leaves the kernel that keeps its input
     tile in LDS for the implicit GEMM with 128x64 tiles, and the 3x3 convolution over 256 channels at 14x14 leaves the
