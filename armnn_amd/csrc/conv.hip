@@ -1010,7 +1010,9 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
         bool gemm_instead = false;
         if (p->halo_ok && p->zw_neg == 0 && p->opt_igemm_lds != 0 && (p->tile_override == 0 || (p->tile_override == 3000 || p->tile_override == 3001)))
         {
-            if (shared_device && g.Ci == 64)
+            // ... and only where the 128 x 64 tiles still give every CU a block
+            const long long gemm_blocks = ((static_cast<long long>(batch) * g.Ho * g.Wo + 127) / 128) * ((g.Co + 63) / 64);
+            if (shared_device && g.Ci == 64 && gemm_blocks >= 256)
             {
                 t_halo_probe = true;
                 gemm_instead = LaunchHalo(p, batch, x, y, stream) >= 0;
