@@ -10,6 +10,7 @@
 #include "igemm_lds_kernel.h"
 #include "big_gemm.h"
 #include "halo_conv_kernel.h"
+#include "plan.h"
 
 #include <algorithm>
 #include <cmath>
@@ -18,58 +19,6 @@
 #include <vector>
 
 using namespace mi355x;
-
-struct mi355x_conv2d_s
-{
-    mi355x_conv2d_desc d{};
-    int32_t algo = MI355X_ALGO_DIRECT;
-    ConvGeom geom{};
-    Requant rq{};
-    // device constants
-    uint8_t* w_direct = nullptr;   // [Kh][Kw][Ci][Co] / depthwise [Kh][Kw][Co], raw codes
-    int8_t*  w_mfma   = nullptr;   // [Co_pad][K_pad] signed, zero padded
-    uint8_t* pad16    = nullptr;   // 16 bytes that turn into the padding value under the kernel's input xor
-    int8_t*  w_stem   = nullptr;   // small-Ci conv on MFMA: [Co rounded up to 32][stem_kp]
-    int8_t*  w_stem2  = nullptr;   // ... the second halves of weight differences that need two
-    int      stem_kp  = 0;
-    uint32_t* dw_grp  = nullptr;   // depthwise 3x3: constants per group of 4 channels for the fused dw+pw kernel
-    uint32_t* w_dot4  = nullptr;   // depthwise 3x3: [C][4] dwords; small-Ci conv: [Co][Kh][RD] dwords
-    uint32_t* w_dot4b = nullptr;   // depthwise 3x3 / small-Ci conv whose weight differences need two int8 halves: the second halves
-    int variant = 0;               // kernel variant within an algo (see RunPlan)
-    int row_dwords = 0;            // small-Ci conv: dwords per filter row
-    float*   chan     = nullptr;   // [8][Co_pad] per-channel requantization constants (rows: see ChanTab)
-    int32_t* corr     = nullptr;   // [Co_pad]  -zx' * sum_k w[c][k]
-    int K = 0, K_pad = 0, Co_pad = 0;
-    int pw_blocks_per_cu = 1, pw_n_cu = 256;     // weight-stationary kernel: blocks a CU holds at once, CUs of the device
-    std::vector<float> chan_host;  // host copy, completed with the corr-folded rows once corr is known
-    std::vector<float> fast_fm, fast_fb;   // per channel: the unwidened fast-path constants and the constant half-width of the
-    std::vector<double> fast_cw;           // bracket (negative: no fast path), kept until the table is uploaded
-    int pw_bn = 0, pw_ks = 0;      // pointwise GEMM kernel configuration (0: not applicable)
-    bool bk128 = false;            // implicit GEMM walks K in 128-byte tiles
-    bool halo_ok = false;          // shape fits the resident-tile kernel (weights without a zero point are checked at launch)
-    unsigned concurrency = 1;      // launches of the plan's network that run side by side (mi355x_conv2d_set_concurrency)
-    int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 96 (= 128x64) / 128: the "igemm_tile" option at plan creation
-    int opt_igemm_lds = 2, opt_dw_rows = 0, opt_dw_cb = 0, opt_stem_dot4 = 0;     // the other process-wide options, as they stood at plan creation
-                                   // (launches read the plan, never the mutable globals: plans may run on any host thread)
-    uint32_t xor_mask = 0, pad_word = 0;
-    int zw_neg = 0;                // MFMA plans: minus the zero point of the stored int8 weights (0: symmetric)
-    int rowsum_bias = 0;           // ... and what the bytes between K and K_pad add to a row's sum of activations
-    std::string info;
-
-    ~mi355x_conv2d_s()
-    {
-        (void)hipFree(w_direct);
-        (void)hipFree(w_mfma);
-        (void)hipFree(pad16);
-        (void)hipFree(dw_grp);
-        (void)hipFree(w_stem);
-        (void)hipFree(w_stem2);
-        (void)hipFree(w_dot4);
-        (void)hipFree(w_dot4b);
-        (void)hipFree(chan);
-        (void)hipFree(corr);
-    }
-};
 
 struct mi355x_fc_s
 {
@@ -699,32 +648,10 @@ int LaunchIgemmT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* 
 template <int BM, int BN, int WM, int WN, int ST, bool U8, bool AW>
 int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
 {
-    const ConvGeom& g = p->geom;
     IgemmArgs a;
-    a.x = static_cast<const uint8_t*>(x);
-    a.pad16 = p->pad16;
-    a.w = p->w_mfma;
-    a.ct = ChanTab{p->chan, p->Co_pad};
-    a.corr = p->corr;
-    a.y = static_cast<uint8_t*>(y);
-    const long long M = static_cast<long long>(batch) * g.Ho * g.Wo;
-    if (M > 0x7fffffffll / 2) return SetError(MI355X_ERR_UNSUPPORTED, "too many output pixels for one launch (%lld)", M);
-    a.M = static_cast<int>(M);
-    a.H = g.H; a.W = g.W; a.Ci = g.Ci; a.Ho = g.Ho; a.Wo = g.Wo; a.Co = g.Co;
-    a.Kh = g.Kh; a.Kw = g.Kw;
-    a.pad_top = g.pad_top; a.pad_left = g.pad_left; a.stride_x = g.stride_x; a.stride_y = g.stride_y;
-    a.dil_x = g.dil_x; a.dil_y = g.dil_y;
-    a.K_pad = p->K_pad;
-    a.unit = (g.Kh == 1 && g.Kw == 1 && g.stride_x == 1 && g.stride_y == 1 && g.pad_top == 0 && g.pad_left == 0 && g.Ho == g.H &&
-              g.Wo == g.W) ? 1 : 0;
-    if (a.unit) { a.H = 1; a.W = a.M; a.Ho = 1; a.Wo = a.M; }      // one row of M pixels
-    a.tiles_m = static_cast<int>((M + BM - 1) / BM);
-    a.tiles_n = (g.Co + BN - 1) / BN;
-    a.xor_mask = p->xor_mask;
-    a.pad_word = p->pad_word;
-    a.zw_neg = p->zw_neg;
-    a.rowsum_bias = p->rowsum_bias;
-    a.rq = p->rq;
+    bool unit_fast = false;
+    if (const int rc = FillIgemmLdsArgs(p, BM, BN, batch, x, y, &a, &unit_fast)) return rc;
+    const ConvGeom& g = p->geom;
     if (t_pending_add && (g.Co & 15) == 0)
     {
         a.res = t_pending_add->other;
@@ -737,7 +664,7 @@ int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, voi
     if constexpr (BM == 64 && BN == 64 && !AW)
     {
         // pointwise layers and FullyConnected below 2 GiB per tensor: addresses without per-load vector arithmetic
-        if (a.unit && static_cast<long long>(a.M) * a.Ci < (1ll << 31) && static_cast<long long>(p->Co_pad) * a.K_pad < (1ll << 31) && a.Ci == a.K_pad)
+        if (unit_fast)
         {
             static const hipError_t uattr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmLdsKernel<BM, BN, WM, WN, ST, U8, false, true>),
                                                                 hipFuncAttributeMaxDynamicSharedMemorySize, smem);
@@ -1163,33 +1090,10 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 3) != 0)
                 return SetError(MI355X_ERR_INVALID_ARGUMENT, "depthwise 3x3 kernel needs a 16-byte aligned input and 4-byte aligned output");
             Dw3x3Args a;
-            a.x = xin; a.pad16 = p->pad16; a.wpack = p->w_dot4; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = yout;
-            a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.C = g.Co; a.Ho = g.Ho; a.Wo = g.Wo;
-            a.pad_top = g.pad_top; a.pad_left = g.pad_left;
-            // 128 channels per block where the channel count allows: every pixel a block reads or writes is a whole line
-            // (32 images: 56 x 56 x 128 13.1 -> 11.6 us at stride 1, 7.3 -> 6.4 us at stride 2; 28 x 28 x 256 8.1 -> 7.7 us;
-            // 7 x 7 x 1024, where a 16-pixel-wide tile is mostly outside the image, 5.1 -> 4.0 us; 14 x 14 x 512 on par)
-            const bool wide = (g.Co % 128) == 0 && p->opt_dw_cb != 32;
-            // 64 per block for the other multiples of 64 (32 images: 112 x 112 x 64 at stride 2 10.0 -> 9.4 us, 56 x 56 x 64 7.7 -> 7.5 us, 28 x 28 x 192 6.8 -> 6.5 us)
-            const bool mid = !wide && (g.Co % 64) == 0 && p->opt_dw_cb != 32;
-            const int cbw = wide ? 128 : mid ? 64 : 32;
-            const int tw = wide ? (g.stride_x == 1 ? 8 : 4) : (g.stride_x == 1 ? 16 : 8);
-            const int th1 = cbw == 32 ? 8 : 4;       // tile rows with one output row per thread
-            // two output rows per thread unless that would leave much of a tile outside a small feature map (or, with the
-            // small tiles of the 64- and 128-channel blocks, fewer than two blocks per CU)
-            const int opt_r = p->opt_dw_rows;
-            int rows_per_thread = opt_r ? opt_r : ((g.Ho + 2 * th1 - 1) / (2 * th1) * (2 * th1) - g.Ho) * 4 <= g.Ho ? 2 : 1;
-            if (cbw != 32 && !opt_r && static_cast<long long>(batch) * ((g.Wo + tw - 1) / tw) * ((g.Ho + 2 * th1 - 1) / (2 * th1)) * (g.Co / cbw) < 512)
-                rows_per_thread = 1;
-            const int th = th1 * rows_per_thread;
-            a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + th - 1) / th; a.cblocks = (g.Co + cbw - 1) / cbw;
-            a.xor_mask = p->xor_mask; a.pad_word = p->pad_word; a.rq = p->rq;
-            const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y * a.cblocks;
-            if (nb > 0x7fffffffll - 8) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
-            a.total_blocks = static_cast<int>(nb);
-            a.xcd_chunk = static_cast<int>((nb + 7) / 8);
+            int rows_per_thread = 1, cbw = 32;
+            if (const int rc = FillDw3x3Args(p, batch, x, y, &a, &rows_per_thread, &cbw)) return rc;
+            const bool wide = cbw == 128, mid = cbw == 64;
             const dim3 grid(static_cast<unsigned>(a.xcd_chunk) * 8u);
-            a.wpack2 = p->w_dot4b;
             const bool w2 = p->w_dot4b != nullptr;
             NoteKernel("Depthwise3x3Kernel<%d, %d, %s, %d>", g.stride_x, rows_per_thread, BoolName(w2), cbw);
             const int variant = (g.stride_x == 1 ? 0 : 4) + (rows_per_thread == 2 ? 0 : 2) + (w2 ? 1 : 0);
@@ -1362,6 +1266,80 @@ int LaunchPwDw(const mi355x_conv2d_s* pw, const mi355x_conv2d_s* dw, const PwDwS
     return sh.S == 1 ? LaunchPwDwT<1>(a, stream) : LaunchPwDwT<2>(a, stream);
 }
 } // namespace
+
+namespace mi355x
+{
+int FillIgemmLdsArgs(const mi355x_conv2d_s* p, int bm, int bn, uint32_t batch, const void* x, void* y, IgemmArgs* out, bool* unit_fast)
+{
+    const ConvGeom& g = p->geom;
+    IgemmArgs a;
+    a.x = static_cast<const uint8_t*>(x);
+    a.pad16 = p->pad16;
+    a.w = p->w_mfma;
+    a.ct = ChanTab{p->chan, p->Co_pad};
+    a.corr = p->corr;
+    a.y = static_cast<uint8_t*>(y);
+    const long long M = static_cast<long long>(batch) * g.Ho * g.Wo;
+    if (M > 0x7fffffffll / 2) return SetError(MI355X_ERR_UNSUPPORTED, "too many output pixels for one launch (%lld)", M);
+    a.M = static_cast<int>(M);
+    a.H = g.H; a.W = g.W; a.Ci = g.Ci; a.Ho = g.Ho; a.Wo = g.Wo; a.Co = g.Co;
+    a.Kh = g.Kh; a.Kw = g.Kw;
+    a.pad_top = g.pad_top; a.pad_left = g.pad_left; a.stride_x = g.stride_x; a.stride_y = g.stride_y;
+    a.dil_x = g.dil_x; a.dil_y = g.dil_y;
+    a.K_pad = p->K_pad;
+    a.unit = (g.Kh == 1 && g.Kw == 1 && g.stride_x == 1 && g.stride_y == 1 && g.pad_top == 0 && g.pad_left == 0 && g.Ho == g.H &&
+              g.Wo == g.W) ? 1 : 0;
+    if (a.unit) { a.H = 1; a.W = a.M; a.Ho = 1; a.Wo = a.M; }      // one row of M pixels
+    a.tiles_m = static_cast<int>((M + bm - 1) / bm);
+    a.tiles_n = (g.Co + bn - 1) / bn;
+    a.xor_mask = p->xor_mask;
+    a.pad_word = p->pad_word;
+    a.zw_neg = p->zw_neg;
+    a.rowsum_bias = p->rowsum_bias;
+    a.rq = p->rq;
+    // pointwise layers and FullyConnected below 2 GiB per tensor: addresses without per-load vector arithmetic
+    *unit_fast = a.unit && static_cast<long long>(a.M) * a.Ci < (1ll << 31) && static_cast<long long>(p->Co_pad) * a.K_pad < (1ll << 31) &&
+                 a.Ci == a.K_pad;
+    *out = a;
+    return 0;
+}
+
+int FillDw3x3Args(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, Dw3x3Args* out, int* rows_out, int* cbw_out)
+{
+    const ConvGeom& g = p->geom;
+    Dw3x3Args a;
+    a.x = static_cast<const uint8_t*>(x); a.pad16 = p->pad16; a.wpack = p->w_dot4; a.ct = ChanTab{p->chan, p->Co_pad}; a.corr = p->corr; a.y = static_cast<uint8_t*>(y);
+    a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.C = g.Co; a.Ho = g.Ho; a.Wo = g.Wo;
+    a.pad_top = g.pad_top; a.pad_left = g.pad_left;
+    // 128 channels per block where the channel count allows: every pixel a block reads or writes is a whole line
+    // (32 images: 56 x 56 x 128 13.1 -> 11.6 us at stride 1, 7.3 -> 6.4 us at stride 2; 28 x 28 x 256 8.1 -> 7.7 us;
+    // 7 x 7 x 1024, where a 16-pixel-wide tile is mostly outside the image, 5.1 -> 4.0 us; 14 x 14 x 512 on par)
+    const bool wide = (g.Co % 128) == 0 && p->opt_dw_cb != 32;
+    // 64 per block for the other multiples of 64 (32 images: 112 x 112 x 64 at stride 2 10.0 -> 9.4 us, 56 x 56 x 64 7.7 -> 7.5 us, 28 x 28 x 192 6.8 -> 6.5 us)
+    const bool mid = !wide && (g.Co % 64) == 0 && p->opt_dw_cb != 32;
+    const int cbw = wide ? 128 : mid ? 64 : 32;
+    const int tw = wide ? (g.stride_x == 1 ? 8 : 4) : (g.stride_x == 1 ? 16 : 8);
+    const int th1 = cbw == 32 ? 8 : 4;       // tile rows with one output row per thread
+    // two output rows per thread unless that would leave much of a tile outside a small feature map (or, with the
+    // small tiles of the 64- and 128-channel blocks, fewer than two blocks per CU)
+    const int opt_r = p->opt_dw_rows;
+    int rows_per_thread = opt_r ? opt_r : ((g.Ho + 2 * th1 - 1) / (2 * th1) * (2 * th1) - g.Ho) * 4 <= g.Ho ? 2 : 1;
+    if (cbw != 32 && !opt_r && static_cast<long long>(batch) * ((g.Wo + tw - 1) / tw) * ((g.Ho + 2 * th1 - 1) / (2 * th1)) * (g.Co / cbw) < 512)
+        rows_per_thread = 1;
+    const int th = th1 * rows_per_thread;
+    a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + th - 1) / th; a.cblocks = (g.Co + cbw - 1) / cbw;
+    a.xor_mask = p->xor_mask; a.pad_word = p->pad_word; a.rq = p->rq;
+    const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y * a.cblocks;
+    if (nb > 0x7fffffffll - 8) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
+    a.total_blocks = static_cast<int>(nb);
+    a.xcd_chunk = static_cast<int>((nb + 7) / 8);
+    a.wpack2 = p->w_dot4b;
+    *out = a;
+    *rows_out = rows_per_thread;
+    *cbw_out = cbw;
+    return 0;
+}
+} // namespace mi355x
 
 extern "C" {
 

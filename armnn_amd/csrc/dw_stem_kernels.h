@@ -63,26 +63,40 @@ __device__ __forceinline__ int XcdContiguousWorkItem(int block, int chunk)
 // lanes per pixel.  Every pixel it loads or stores is then one whole 128-byte line instead of a quarter of one; the
 // smaller tile costs more halo (1.56 x instead of 1.27 x at stride 1).  The stores are ordinary ones: dwords written
 // through L2 one by one (buffer stores with sc1) made a MobileNetV1 step 1.2 % slower.
-template <int S, int R, bool W2 = false, int CB = 32>
-__global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
+template <int S, int R, int CB>
+struct Dw3x3Tile
 {
-    static_assert(CB == 32 || CB == 64 || CB == 128, "32, 64 or 128 channels per block");
-    constexpr int LPC = CB / 4;                  // lanes per pixel
-    constexpr int XG = CB == 128 ? 2 : 4;        // thread columns
-    constexpr int TH = (256 / (LPC * XG)) * R;   // 8 R (CB = 32) or 4 R output rows per tile
-    constexpr int CPP = CB / 16;                 // 16-byte staging chunks per pixel
-    constexpr int P = S == 1 ? 4 : 2;            // outputs per thread and row
-    constexpr int TW = P * XG;                   // outputs per tile row
-    constexpr int HR = TH * S + 2;               // halo rows held in LDS
-    constexpr int HC = TW * S + 2;               // halo columns
-    constexpr int IR = (R - 1) * S + 3;          // input rows a thread walks
+    static constexpr int LPC = CB / 4;                  // lanes per pixel
+    static constexpr int XG = CB == 128 ? 2 : 4;        // thread columns
+    static constexpr int TH = (256 / (LPC * XG)) * R;   // 8 R (CB = 32) or 4 R output rows per tile
+    static constexpr int P = S == 1 ? 4 : 2;            // outputs per thread and row
+    static constexpr int TW = P * XG;                   // outputs per tile row
+    static constexpr int HR = TH * S + 2;               // halo rows held in LDS
+    static constexpr int HC = TW * S + 2;               // halo columns
     // bytes per pixel in LDS.  CB = 32: 48 spreads the dword reads of a wave's eight pixels over the banks; CB = 64: 80 does
     // the same for the four pixels (P S pixels apart) a wave reads; CB = 128: the 32 lanes of a pixel read 128 contiguous bytes
-    constexpr int PITCH = CB == 32 ? 48 : CB == 64 ? 80 : 128;
-    __shared__ __attribute__((aligned(16))) uint8_t tile[HR * HC * PITCH];
+    static constexpr int PITCH = CB == 32 ? 48 : CB == 64 ? 80 : 128;
+    static constexpr int SMEM = HR * HC * PITCH;
+};
 
-    int b = XcdContiguousWorkItem(blockIdx.x, a.xcd_chunk);
-    if ((static_cast<int>(blockIdx.x) >> 3) >= a.xcd_chunk || b >= a.total_blocks) return;
+// The work of one block (256 threads) on work item `b` (channel block fastest, then tile column, tile row, image); `tile`
+// is the block's Dw3x3Tile<S, R, CB>::SMEM bytes of LDS.  THROUGH: the output dwords are written through L2 as they are
+// issued (buffer stores with sc1; tensors below 4 GiB), for callers that hand the output to other blocks of the same launch.
+struct NoBlockHook
+{
+    __device__ __forceinline__ void operator()() const {}
+};
+
+// `after_loads()` is called by every thread once the block's last global load has been issued (before its stores).
+template <int S, int R, bool W2, int CB, bool THROUGH, typename Hook = NoBlockHook>
+__device__ __forceinline__ void Depthwise3x3Block(const Dw3x3Args& a, int b, uint8_t* const tile, Hook after_loads = Hook())
+{
+    static_assert(CB == 32 || CB == 64 || CB == 128, "32, 64 or 128 channels per block");
+    using G = Dw3x3Tile<S, R, CB>;
+    constexpr int LPC = G::LPC, XG = G::XG, TH = G::TH, P = G::P, TW = G::TW, HR = G::HR, HC = G::HC, PITCH = G::PITCH;
+    constexpr int CPP = CB / 16;                 // 16-byte staging chunks per pixel
+    constexpr int IR = (R - 1) * S + 3;          // input rows a thread walks
+
     const int cb = b % a.cblocks; b /= a.cblocks;
     const int tx = b % a.tiles_x; b /= a.tiles_x;
     const int ty = b % a.tiles_y;
@@ -206,6 +220,8 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
 
     // ---- epilogue ------------------------------------------------------------------------------------------------
     const Fast4 f4 = LoadFast4(a.ct, c);
+    after_loads();
+    [[maybe_unused]] const __amdgpu_buffer_rsrc_t yrsrc = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, -1, 0x00020000);
 #pragma unroll
     for (int o = 0; o < R; ++o)
     {
@@ -219,11 +235,23 @@ __global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
             if (ox < a.Wo && c < a.C)
             {
                 const uint32_t q = Requant4Dev(acc[o][j][0], acc[o][j][1], acc[o][j][2], acc[o][j][3], f4, a.ct, c, a.rq);
-                // an ordinary store: the pieces of a line are merged in L2 (written through one by one they are slower)
-                *reinterpret_cast<uint32_t*>(yrow + static_cast<long long>(ox) * a.C) = q;
+                if constexpr (THROUGH)
+                    __builtin_amdgcn_raw_buffer_store_b32(q, yrsrc, static_cast<int>(yrow - a.y) + ox * a.C, 0, kStoreAuxSc1);
+                else
+                    // an ordinary store: the pieces of a line are merged in L2 (written through one by one they are slower)
+                    *reinterpret_cast<uint32_t*>(yrow + static_cast<long long>(ox) * a.C) = q;
             }
         }
     }
+}
+
+template <int S, int R, bool W2 = false, int CB = 32>
+__global__ __launch_bounds__(256) void Depthwise3x3Kernel(Dw3x3Args a)
+{
+    __shared__ __attribute__((aligned(16))) uint8_t tile[Dw3x3Tile<S, R, CB>::SMEM];
+    const int b = XcdContiguousWorkItem(blockIdx.x, a.xcd_chunk);
+    if ((static_cast<int>(blockIdx.x) >> 3) >= a.xcd_chunk || b >= a.total_blocks) return;
+    Depthwise3x3Block<S, R, W2, CB, false>(a, b, tile);
 }
 
 // ---------------------------------------------------------------------------------------------------------------

@@ -43,8 +43,19 @@ constexpr int VmcntImm(int n)
 // UNIT: the launch is a 1x1 stride-1 unpadded convolution or a FullyConnected layer (a.unit) whose tensors are below
 // 2 GiB: output row m reads input row m, there is no padding and no tap walk, and every load address is a wave-uniform
 // base (advanced by 128 bytes per k-tile) plus a 32-bit lane offset fixed for the kernel -- no vector arithmetic per load.
-template <int BM, int BN, int WM, int WN, int ST, bool U8, bool AW = false, bool UNIT = false>
-__global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
+// The work of one block on output tile `tile` (row-block major: tile = tm * tiles_n + tn); `smem` is the block's
+// IgemmLdsSmemBytes<BM, BN, ST>() bytes of LDS.  Ends with the tile's stores issued (not waited for) and LDS still in
+// use by the write-out: a caller that runs another tile afterwards puts a block barrier in between.
+// `after_loads()` is called by every thread once the tile's last global load has been issued (before the write-out's
+// stores; a fused Addition with more than four pieces per thread still loads its other input afterwards): a persistent
+// caller starts the memory operations of its own bookkeeping there, behind the tile's loads.
+struct NoTileHook
+{
+    __device__ __forceinline__ void operator()() const {}
+};
+
+template <int BM, int BN, int WM, int WN, int ST, bool U8, bool AW = false, bool UNIT = false, typename Hook = NoTileHook>
+__device__ __forceinline__ void IgemmLdsTile(const IgemmArgs& a, const int tile, uint8_t* const smem, Hook after_loads = Hook())
 {
     static_assert(ST >= 2 && ST <= 8, "2 to 8 LDS stages");
     static_assert((ST - 2) * (BM + BN) / (8 * WM * WN) < 64, "outstanding loads must fit the vmcnt counter");
@@ -62,12 +73,6 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
     typedef __attribute__((address_space(3))) void* LdsPtr;
     typedef const __attribute__((address_space(1))) void* GlobalPtr;
 
-    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];   // IgemmLdsSmemBytes<BM, BN, ST>()
-
-    const int nblocks = a.tiles_m * a.tiles_n;
-    const int per_xcd = (nblocks + 7) >> 3;
-    const int tile = static_cast<int>(blockIdx.x & 7) * per_xcd + static_cast<int>(blockIdx.x >> 3);
-    if (tile >= nblocks) return;
     const int tn = tile % a.tiles_n;
     const int tm = tile / a.tiles_n;
 
@@ -90,7 +95,7 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
     {
         const int m = tm * BM + wave * (BM / NW) + j * 8 + lrow;
         mvalid[j] = m < a.M;
-        const int mm = mvalid[j] ? m : 0;
+        const int mm = min(m, a.M - 1);          // rows past the end re-read the last row (never stored)
         int n, oy, ox;
         if (a.unit)
         {
@@ -115,7 +120,7 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
     static_assert((BM / NW) % 16 == 0 && (BN / NW) % 16 == 0, "a wave's first row is a multiple of 16");
     const int8_t* wrow = a.w + static_cast<long long>(tn * BN + wave * (BN / NW) + lrow) * a.K_pad;
     int ci = 0, kx = 0, ky = 0;                  // tap walk, identical in every thread
-    // UNIT: lane offsets from the tensors' first bytes (rows past the end re-read row 0; their results are not stored)
+    // UNIT: lane offsets from the tensors' first bytes (rows past the end re-read the last row; their results are not stored)
     uint32_t aoff[RA], boff[RB];
     if constexpr (UNIT)
     {
@@ -123,7 +128,7 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
         for (int j = 0; j < RA; ++j)
         {
             const int m = tm * BM + wave * (BM / NW) + j * 8 + lrow;
-            aoff[j] = static_cast<uint32_t>(m < a.M ? m : 0) * static_cast<uint32_t>(a.Ci) + ((j & 1) ? lchunk_odd : lchunk_even) * 16;
+            aoff[j] = static_cast<uint32_t>(min(m, a.M - 1)) * static_cast<uint32_t>(a.Ci) + ((j & 1) ? lchunk_odd : lchunk_even) * 16;
         }
 #pragma unroll
         for (int j = 0; j < RB; ++j)
@@ -345,6 +350,7 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
         }
     }
     __syncthreads();
+    after_loads();
     if (!EARLY && fuse) load_other();
     const OutPtr outp = MakeOutPtr(a.y, static_cast<long long>(a.M) * a.Co);
     if ((a.Co & 15) == 0)
@@ -378,6 +384,19 @@ __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
             }
         }
     }
+}
+
+// One tile per block; consecutive block ids are dealt round-robin to the 8 XCDs, so XCD x takes the contiguous range of
+// tiles [x * per_xcd, (x + 1) * per_xcd): the column tiles of a row block share an L2.
+template <int BM, int BN, int WM, int WN, int ST, bool U8, bool AW = false, bool UNIT = false>
+__global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
+{
+    extern __shared__ __attribute__((aligned(16))) uint8_t smem[];   // IgemmLdsSmemBytes<BM, BN, ST>()
+    const int nblocks = a.tiles_m * a.tiles_n;
+    const int per_xcd = (nblocks + 7) >> 3;
+    const int tile = static_cast<int>(blockIdx.x & 7) * per_xcd + static_cast<int>(blockIdx.x >> 3);
+    if (tile >= nblocks) return;
+    IgemmLdsTile<BM, BN, WM, WN, ST, U8, AW, UNIT>(a, tile, smem);
 }
 
 } // namespace mi355x

@@ -137,6 +137,20 @@ int mi355x_set_option(const char* name, int value)
     if (!name) return SetError(MI355X_ERR_INVALID_ARGUMENT, "option name is null");
     if (std::strcmp(name, "exact_division_epilogue") == 0) { GlobalOptions().exact_division_epilogue = value != 0; return 0; }
     if (std::strcmp(name, "stem_dot4") == 0) { GlobalOptions().stem_dot4 = value != 0; return 0; }
+    if (std::strcmp(name, "chain_stages") == 0)
+    {
+        if (value < 2 || value > 4) return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain_stages must be 2, 3 or 4");
+        GlobalOptions().chain_stages = value;
+        return 0;
+    }
+    if (std::strcmp(name, "chain_defer_signal") == 0) { GlobalOptions().chain_defer_signal = value != 0; return 0; }
+    if (std::strcmp(name, "chain_panel") == 0) { GlobalOptions().chain_panel = value != 0; return 0; }
+    if (std::strcmp(name, "chain_blocks_per_cu") == 0)
+    {
+        if (value < 0 || value > 16) return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain_blocks_per_cu must be 0 .. 16");
+        GlobalOptions().chain_blocks_per_cu = value;
+        return 0;
+    }
     if (std::strcmp(name, "dw_rows") == 0)
     {
         if (value < 0 || value > 2) return SetError(MI355X_ERR_INVALID_ARGUMENT, "dw_rows must be 0, 1 or 2");

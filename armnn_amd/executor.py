@@ -34,10 +34,33 @@ class FusedPair:
         return self.parts[0].macs_per_image + self.parts[1].macs_per_image
 
 
+@dataclass
+class ChainedRun:
+    """Consecutive convolution layers executed by one persistent launch (shim.LayerChain) over the whole batch."""
+    name: str
+    parts: Tuple                       # the Layers, in order
+    op: str = "chain"
+
+    @property
+    def inputs(self):
+        return tuple(self.parts[0].inputs)
+
+    @property
+    def output(self):
+        return self.parts[-1].output
+
+    @property
+    def macs_per_image(self):
+        return sum(p.macs_per_image for p in self.parts)
+
+
 class DeviceNetwork:
     def __init__(self, net: Network, batch: int, algo_overrides: Optional[Dict[str, int]] = None, use_graph: bool = True,
-                 fuse: bool = False, lanes: int = 1, fuse_add: bool = True):
-        """lanes > 1 splits the batch into that many contiguous slices; each slice runs the whole network on a stream of
+                 fuse: bool = False, lanes: int = 1, fuse_add: bool = True, chain: bool = False, lanes_after_chain: bool = False):
+        """chain: runs of consecutive layers the library accepts (mi355x_chain_accepts) become one persistent launch over
+        the whole batch; with lanes > 1 the lanes join in front of such a run and, if lanes_after_chain, fork again behind it
+        (else the rest of the network runs on one stream).
+        lanes > 1 splits the batch into that many contiguous slices; each slice runs the whole network on a stream of
         its own (the same plans, pointers offset to the slice), so one slice's kernels fill the ramp-up, tail and
         launch gaps of the others. Results do not depend on the split: every image is computed independently."""
         if lanes < 1 or batch % lanes != 0:
@@ -48,12 +71,12 @@ class DeviceNetwork:
         self.lib = shim.load_library()
         self.stream = self.dev.stream()
         self.side_streams = [self.dev.stream() for _ in range(lanes - 1)]
-        self.fork_event = self.dev.event() if lanes > 1 else None
-        self.join_events = [self.dev.event() for _ in range(lanes - 1)]
         self.buffers: Dict[str, shim.DeviceBuffer] = {}
         self.steps: List = []          # (layer, callable(stream))
         self._step_plans: List = []    # plan of each step (None for plan-less layers), parallel to self.steps
         self.plans = []
+        self.chains: List = []
+        self.lanes_after_chain = lanes_after_chain
         self.graph = None
         self.use_graph = use_graph
         algo_overrides = algo_overrides or {}
@@ -120,6 +143,45 @@ class DeviceNetwork:
             self._fuse_pairs(("conv", "depthwise") if fuse == "pwdw" else ("depthwise", "conv"))
         if fuse_add:
             self._fuse_additions()
+        if chain:
+            self._build_chains()
+
+    def _build_chains(self, min_layers: int = 2):
+        """Replace every maximal run of consecutive steps that are plain convolution / depthwise layers accepted by the
+        library, each reading the output of the one before, by one chain step."""
+        plan_of = self._plan_of
+        batch = self.batch
+
+        def eligible(step):
+            l = step[0]
+            return (getattr(l, "op", None) in ("conv", "depthwise") and isinstance(plan_of.get(id(l)), shim.Conv2dPlan) and
+                    shim.LayerChain.accepts(plan_of[id(l)], batch))
+
+        out, k = [], 0
+        while k < len(self.steps):
+            if not eligible(self.steps[k]):
+                out.append(self.steps[k])
+                k += 1
+                continue
+            run = [self.steps[k]]
+            while (k + len(run) < len(self.steps) and eligible(self.steps[k + len(run)]) and
+                   self.steps[k + len(run)][0].inputs[0] == run[-1][0].output):
+                run.append(self.steps[k + len(run)])
+            if len(run) < min_layers:
+                out.append(self.steps[k])
+                k += 1
+                continue
+            layers = [st[0] for st in run]
+            ch = shim.LayerChain([plan_of[id(l)] for l in layers], batch, self.buffers[layers[0].inputs[0]].ptr,
+                                 [self.buffers[l.output].ptr for l in layers])
+            self.chains.append(ch)
+
+            def fn(s, lane=0, lanes=1, ch=ch):
+                ch.run(s)
+            fn.whole_batch = True
+            out.append((ChainedRun("chain(" + layers[0].name + ".." + layers[-1].name + ")", tuple(layers)), fn))
+            k += len(run)
+        self.steps = out
 
     def _fuse_pairs(self, ops):
         """Replace neighbours (depthwise 3x3, 1x1 convolution) -- or, with ops = ("conv", "depthwise"), (1x1 convolution,
@@ -240,22 +302,56 @@ class DeviceNetwork:
         self.buffers[self.net.input].upload(x.data, self.stream)
 
     def _enqueue_lanes(self):
-        """Every lane's chain of launches: lane 0 on self.stream, the others on streams forked from it and joined back."""
+        """Every lane's chain of launches: lane 0 on self.stream, the others on streams forked from it and joined back.
+        A step that works on the whole batch (a layer chain) runs on self.stream with the lanes joined in front of it."""
         if self.lanes == 1:
             for _, fn in self.steps:
                 fn(self.stream)
             return
-        self.dev.event_record(self.fork_event, self.stream)
-        for side in self.side_streams:
-            self.dev.stream_wait_event(side, self.fork_event)
+        forked = False
+        single_from_here = False
+
+        def fork():
+            ev = self._sync_event()
+            self.dev.event_record(ev, self.stream)
+            for side in self.side_streams:
+                self.dev.stream_wait_event(side, ev)
+
+        def join():
+            for side in self.side_streams:
+                ev = self._sync_event()
+                self.dev.event_record(ev, side)
+                self.dev.stream_wait_event(self.stream, ev)
+
+        self._sync_next = 0
         # lanes interleaved layer by layer, so launches next to each other in submission order can overlap
         for _, fn in self.steps:
+            if getattr(fn, "whole_batch", False) or single_from_here:
+                if forked:
+                    join()
+                    forked = False
+                fn(self.stream, 0, 1)
+                if getattr(fn, "whole_batch", False) and not self.lanes_after_chain:
+                    single_from_here = True
+                continue
+            if not forked:
+                fork()
+                forked = True
             fn(self.stream, 0, self.lanes)
             for k, side in enumerate(self.side_streams, start=1):
                 fn(side, k, self.lanes)
-        for k, side in enumerate(self.side_streams, start=1):
-            self.dev.event_record(self.join_events[k - 1], side)
-            self.dev.stream_wait_event(self.stream, self.join_events[k - 1])
+        if forked:
+            join()
+
+    def _sync_event(self):
+        """Events for forks and joins, one per use within a forward pass (a captured graph keeps them)."""
+        if not hasattr(self, "_sync_events"):
+            self._sync_events, self._sync_next = [], 0
+        if self._sync_next == len(self._sync_events):
+            self._sync_events.append(self.dev.event())
+        ev = self._sync_events[self._sync_next]
+        self._sync_next += 1
+        return ev
 
     def enqueue(self):
         """One forward pass on self.stream (asynchronous)."""
@@ -304,6 +400,9 @@ class DeviceNetwork:
         if self.graph is not None:
             self.dev.graph_destroy(self.graph)
             self.graph = None
+        for ch in self.chains:
+            ch.destroy()
+        self.chains = []
         for p in self.plans:
             p.destroy()
         for b in set(self.buffers.values()):

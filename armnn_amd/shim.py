@@ -7,7 +7,7 @@ from __future__ import annotations
 
 import ctypes as C
 import os
-from typing import Optional
+from typing import Optional, Sequence
 
 import numpy as np
 
@@ -29,6 +29,7 @@ EXPORTS = [
     "mi355x_graph_capture_begin", "mi355x_graph_capture_end", "mi355x_graph_launch", "mi355x_graph_destroy",
     "mi355x_conv2d_create", "mi355x_conv2d_run", "mi355x_conv2d_destroy", "mi355x_conv2d_algo",
     "mi355x_conv2d_fusable", "mi355x_conv2d_run_fused", "mi355x_conv2d_run_add", "mi355x_conv2d_set_concurrency",
+    "mi355x_chain_accepts", "mi355x_chain_create", "mi355x_chain_run", "mi355x_chain_status", "mi355x_chain_info", "mi355x_chain_run_stamped", "mi355x_chain_destroy",
     "mi355x_fc_create", "mi355x_fc_run", "mi355x_fc_destroy", "mi355x_fc_algo",
     "mi355x_activation_run", "mi355x_pool2d_run", "mi355x_add_run", "mi355x_softmax_run", "mi355x_pad_run",
 ]
@@ -114,6 +115,11 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
             "mi355x_conv2d_fusable": [V, V], "mi355x_conv2d_run_fused": [V, V, C.c_uint32, V, V, V],
             "mi355x_conv2d_run_add": [V, C.c_uint32, V, V, C.POINTER(Quant), C.POINTER(Quant), C.c_int32, C.c_float, C.c_float, V, V],
             "mi355x_conv2d_set_concurrency": [V, C.c_uint32],
+            "mi355x_chain_accepts": [V, C.c_uint32],
+            "mi355x_chain_create": [C.c_uint32, C.POINTER(V), C.c_uint32, V, C.POINTER(V), C.POINTER(V)],
+            "mi355x_chain_run": [V, V], "mi355x_chain_status": [V, C.POINTER(C.c_uint32)],
+            "mi355x_chain_info": [V, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)], "mi355x_chain_destroy": [V],
+            "mi355x_chain_run_stamped": [V, V, C.POINTER(C.c_uint64)],
             "mi355x_fc_create": [C.POINTER(FcDesc), V, C.POINTER(ConstQuant), V, C.POINTER(ConstQuant), C.POINTER(V)],
             "mi355x_fc_run": [V, C.c_uint32, V, V, V], "mi355x_fc_destroy": [V],
             "mi355x_fc_algo": [V, C.POINTER(C.c_int32), C.c_char_p, C.c_size_t],
@@ -324,6 +330,57 @@ class Conv2dPlan:
         if self.plan:
             self.lib.mi355x_conv2d_destroy(self.plan)
             self.plan = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class LayerChain:
+    """mi355x_chain_*: consecutive convolution plans (plans[k] reads plans[k - 1]'s output) as one persistent launch.
+    Addresses are bound here; the bytes written to every output equal those of running the plans one by one."""
+
+    def __init__(self, plans: Sequence["Conv2dPlan"], batch: int, x_dev: int, outputs_dev: Sequence[int]):
+        self.lib = load_library()
+        self.plans = list(plans)                  # the chain refers to them: keep them alive
+        n = len(self.plans)
+        pa = (C.c_void_p * n)(*[p.plan for p in self.plans])
+        oa = (C.c_void_p * n)(*outputs_dev)
+        chain = C.c_void_p()
+        _chk(self.lib.mi355x_chain_create(n, pa, batch, x_dev, oa, C.byref(chain)))
+        self.chain = chain.value
+
+    @staticmethod
+    def accepts(plan: "Conv2dPlan", batch: int) -> bool:
+        return load_library().mi355x_chain_accepts(plan.plan, batch) == 0
+
+    def run(self, stream=None):
+        _chk(self.lib.mi355x_chain_run(self.chain, stream))
+
+    def gave_up(self) -> int:
+        """Blocks whose bounded wait ran out in a launch since the last call (0 in normal operation); call after synchronizing."""
+        n = C.c_uint32()
+        _chk(self.lib.mi355x_chain_status(self.chain, C.byref(n)))
+        return n.value
+
+    def run_stamped(self, stream=None):
+        """One launch with per-phase cycle sums over all blocks: dict of cycles per phase and tile counts."""
+        sums = (C.c_uint64 * 8)()
+        _chk(self.lib.mi355x_chain_run_stamped(self.chain, stream, sums))
+        names = ("pop", "wait", "mfma_tiles", "dw_tiles", "drain", "n_mfma_tiles", "n_dw_tiles", "n_waited")
+        return dict(zip(names, [int(v) for v in sums]))
+
+    def info(self):
+        items, blocks = C.c_uint32(), C.c_uint32()
+        _chk(self.lib.mi355x_chain_info(self.chain, C.byref(items), C.byref(blocks)))
+        return items.value, blocks.value
+
+    def destroy(self):
+        if self.chain:
+            self.lib.mi355x_chain_destroy(self.chain)
+            self.chain = None
 
     def __del__(self):
         try:

@@ -5,7 +5,7 @@ A step is one forward pass of the whole network over one batch that is already r
 runs on the device through the C ABI; the pass is replayed as one HIP graph).  Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 64] [--net mobilenet_v1|resnet50]
-                  [--weights per_channel_s8|per_tensor_u8] [--no-cpu-baseline] [--no-backend] [--layers]
+                  [--weights per_channel_s8|per_tensor_u8] [--no-cpu-baseline] [--no-backend] [--layers] [--chain]
 
 The headline workload is the default: per-channel QSymmS8 weights.  --weights per_tensor_u8 runs the same network with
 QAsymmU8 weights that have one scale and a zero point per layer, and says so in config.workload.
@@ -22,6 +22,9 @@ Extra objects in the line:
   cpu_baseline  the reference's CpuRef backend behind its own runtime where that build is there, else the reference's own
                 CpuRef functions (oracle/_ref) -- both kind "reference" -- or the C restatement (kind "port"); one thread, on a
                 bounded sample of the same workload
+  parity        the timed device network run once more, outside the timed region, on the images the cpu_baseline leg
+                computed: max |difference| in codes and exact-match fraction against the CPU checker, end to end, for the
+                network's output and for the logits in front of the softmax
 """
 from __future__ import annotations
 
@@ -68,6 +71,10 @@ def layer_work(net, l, batch):
         return "mfma", 2.0 * l.macs_per_image * batch
     if l.op == "convadd":                      # a convolution with the Addition behind it in its write-out
         return "mfma", 2.0 * l.parts[0].macs_per_image * batch
+    if l.op == "chain":
+        # a run of layers in one persistent launch: every layer's tensors are still written and read, so the launch's
+        # algorithmic bytes are the sum of its layers'; priced against HBM like the depthwise layers in it
+        return "hbm", float(sum(algorithmic_bytes(net, part, batch) for part in l.parts))
     if l.op == "dwpw":
         # two layers fused (depthwise + pointwise, in either order): the tensor between them never exists, so the unit's
         # algorithmic bytes are its input, its output and both layers' constants; priced against HBM like the depthwise
@@ -122,7 +129,10 @@ def cpu_baseline_reference_runtime(net, seconds_budget=25.0):
             elapsed += steps * ms * 1e-3
             if elapsed * (images + steps) / images > seconds_budget or images >= 8:
                 break
-    return {"value": images / elapsed, "unit": "images/sec", "cores": 1, "kind": "reference",
+        info = net.info(net.output, 1)
+        from armnn_amd.tensor import numpy_dtype
+        outputs = [(100, {net.output: np.fromfile(fout, dtype=numpy_dtype(info.dtype)).reshape(info.shape)})]
+    return {"_outputs": outputs, "value": images / elapsed, "unit": "images/sec", "cores": 1, "kind": "reference",
             "sample": f"{images} image(s) of the same network at batch 1 through IRuntime::EnqueueWorkload on the reference's CpuRef backend "
                       f"(libarmnn.so built from the reference), {elapsed:.1f} s, single-threaded backend on one of {os.cpu_count()} cores"}
 
@@ -139,16 +149,42 @@ def cpu_baseline(net, seconds_budget=25.0):
     orc = cpuref.Oracle(kind)
     os.environ["OMP_NUM_THREADS"] = "1"
     images, elapsed = 0, 0.0
+    outputs = []
+    keep = {net.output, net.layers[-1].inputs[0]}       # the network's output and what the last layer reads (the logits)
     while True:
         x = nets.synthetic_input(net, 1, seed=100 + images)
         t0 = time.perf_counter()
-        netref.run_network(orc, net, x, fast=False)      # literal single-thread loop nest, as CpuRef runs it
+        vals = netref.run_network(orc, net, x, fast=False, keep=True)      # literal single-thread loop nest, as CpuRef runs it
         elapsed += time.perf_counter() - t0
+        outputs.append((100 + images, {k: vals[k].data for k in keep}))
         images += 1
         if elapsed * (images + 1) / images > seconds_budget or images >= 8:
             break
-    return {"value": images / elapsed, "unit": "images/sec", "cores": 1, "kind": kind,
+    return {"_outputs": outputs, "value": images / elapsed, "unit": "images/sec", "cores": 1, "kind": kind,
             "sample": f"{images} image(s) of the same network at batch 1, {elapsed:.1f} s, 1 thread of {os.cpu_count()}"}
+
+
+def parity_against_checker(net, dn, batch, checked):
+    """The timed device network (same plans, same graph) run once more on a batch whose first images are the ones the CPU
+    baseline computed, outside the timed region; the CPU side is the checker only.  End to end: differences of the layers
+    add up along the network, so max_abs_lsb here is not the per-layer bound the tests assert (<= 1 per layer on
+    identical inputs, armnnTestUtils/TensorHelpers.hpp:24-31 is the reference's own tolerance rule)."""
+    import numpy as np
+    from armnn_amd import nets
+    x = nets.synthetic_input(net, batch)
+    for k, (seed, _) in enumerate(checked[:batch]):
+        x.data[k] = nets.synthetic_input(net, 1, seed=seed).data[0]
+    dn.upload_input(x)
+    dn.enqueue()
+    out = {"images": min(len(checked), batch), "against": "CPU checker outputs of the cpu_baseline leg, end to end"}
+    for name in checked[0][1]:
+        got = dn.download(name).data
+        d = np.concatenate([np.abs(got[k].astype(np.int32) - ref[name][0].astype(np.int32)).ravel() for k, (_, ref) in enumerate(checked[:batch])])
+        key = "output" if name == net.output else "logits"
+        out[key] = {"tensor": name, "max_abs_lsb": int(d.max()), "exact_fraction": float((d == 0).mean()), "within_1_lsb_fraction": float((d <= 1).mean())}
+    if "output" in out:
+        out["max_abs_lsb"], out["exact_fraction"] = out["output"]["max_abs_lsb"], out["output"]["exact_fraction"]
+    return out
 
 
 def run_backend_child(net, batch, steps, warmup, real=False):
@@ -199,6 +235,9 @@ def main():
     ap.add_argument("--lanes", type=int, default=0,
                     help="split the batch into this many slices, each running the network on a stream of its own "
                          "(default: 2 for batches of at least 16 images that halve, else 1)")
+    ap.add_argument("--chain", action="store_true",
+                    help="runs of consecutive layers the library accepts (3x3 depthwise over multiples of 128 channels, 1x1 convolutions "
+                         "over more than 128 input channels) as one persistent launch over the whole batch (same bytes)")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
     ap.add_argument("--profile-pass", action="store_true",
                     help="for rocprofv3 --pmc: one 64 MiB calibration copy (1 B read + 1 B written per element), then ONE "
@@ -226,7 +265,7 @@ def main():
 
     if args.lanes == 0:
         args.lanes = 2 if batch >= 16 and batch % 2 == 0 else 1
-    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add)
+    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add, chain=args.chain)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev
 
@@ -270,13 +309,14 @@ def main():
     traffic = measured_traffic(net.name, launch_batch)
     rows = []
     for l, ms, kernel in per_layer:
-        kind, work = layer_work(net, l, launch_batch)
+        images = batch if l.op == "chain" else launch_batch        # a layer chain runs the whole batch in one launch
+        kind, work = layer_work(net, l, images)
         peak = INT8_MFMA_PEAK_OPS if kind == "mfma" else HBM_PEAK_BYTES
         row = {"layer": l.name, "op": l.op, "ms": ms, "bound": kind, "work": work, "frac": work / (ms * 1e-3) / peak, "kernel": kernel}
         if kind == "mfma":
             # the roof that binds a conv / FC layer depends on its arithmetic intensity: below the ridge
             # (peak ops / peak bytes = 625 ops/B) the HBM roof is the lower one
-            nbytes = float(algorithmic_bytes(net, l, launch_batch))
+            nbytes = float(algorithmic_bytes(net, l, images))
             row["bytes"] = nbytes
             row["ops"] = work
             row["binding"] = "mfma" if work / nbytes >= RIDGE_OPS_PER_BYTE else "hbm"
@@ -319,6 +359,8 @@ def main():
         roof["avg_launch_us"] = t * 1e6 / len(sel)
         roof["share_of_lane_pass"] = t * 1e3 / total_ms
         roof["algorithmic_bytes"] = nbytes
+        roof["timing"] = ("HIP events around repeated launches of each layer alone on the stream, same buffers every time: every tensor of a "
+                          "launch fits the 256 MB last-level cache, so fractions of the HBM roof are upper bounds on what HBM itself sees")
         if ops > 0:
             roof["TOPS"] = ops / t / 1e12
             roof["frac_of_int8_mfma_peak"] = ops / t / INT8_MFMA_PEAK_OPS
@@ -346,6 +388,7 @@ def main():
                           f"random-init, whole forward pass incl. avgpool/FC/softmax, input resident in HBM, every layer through the C ABI, "
                           f"one HIP graph replay per step",
               "batch": batch, "graph_replay": not args.no_graph, "fused_pairs": args.fuse or None, "additions_inside_convolutions": not args.no_fuse_add, "lanes": args.lanes,
+              "layer_chains": [l.name for l, _ in dn.steps if l.op == "chain"] or None,
               "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12}
     if backend is not None:
         # the same network and input through the C++ backend: wall clock per IRuntime::EnqueueWorkload call, host buffers in
@@ -385,7 +428,11 @@ def main():
     from armnn_amd import peaks
     line["measured_peaks"] = peaks.measure()
     if not args.no_cpu_baseline:
-        line["cpu_baseline"] = cpu_baseline(net)
+        base = cpu_baseline(net)
+        checked = base.pop("_outputs", [])
+        line["cpu_baseline"] = base
+        if checked:
+            line["parity"] = parity_against_checker(net, dn, batch, checked)
     dn.close()
     print(json.dumps(line))
     return 0

@@ -113,6 +113,14 @@ int  mi355x_abi_version(void);
  *   bytes; tests and tuning).
  *   "dw_cb" = 0 | 32: channels per block of the 3x3 depthwise kernel (0: 128 where the channel count is a multiple of
  *   128, else 32; 32: always 32; identical bytes).
+ *   "chain_stages" = 2 | 3 | 4: LDS stages of the matrix-core tiles inside a layer chain; "chain_blocks_per_cu" = 0 .. 16:
+ *   persistent blocks per CU of a layer chain (0: as many as fit); "chain_panel" = 0 | 1: 1x1 convolutions with 256 or 512
+ *   input channels and at least 96 row blocks run as one work item per 64 output rows with the activation panel resident
+ *   in on-chip memory; "chain_defer_signal" = 0 | 1: a tile is counted as finished behind the next tile's loads instead of
+ *   after a wait for its stores.  All four are read by mi355x_chain_create and give identical bytes; they exist for
+ *   tests and tuning (the defaults are the fastest measured).
+ *   Every option except "exact_division_epilogue" is a test and tuning hook: the numeric codes of "igemm_tile" name
+ *   kernels of this library's current build and are no stable interface.
  * Unknown names and values outside these return MI355X_ERR_INVALID_ARGUMENT. */
 int  mi355x_set_option(const char* name, int value);
 int  mi355x_device_count(int* count);                 /* 0 devices is success with *count == 0 */
@@ -233,6 +241,42 @@ int mi355x_conv2d_run_add(mi355x_conv2d_t plan, uint32_t batch, const void* inpu
 int mi355x_conv2d_fusable(mi355x_conv2d_t first, mi355x_conv2d_t second);
 int mi355x_conv2d_run_fused(mi355x_conv2d_t first, mi355x_conv2d_t second, uint32_t batch,
                             const void* input_dev, void* output_dev, mi355x_stream_t stream);
+/* A run of consecutive layers as one persistent launch ("chain").  plans[k] reads the output of plans[k - 1] (plans[0]
+ * reads input_dev) and writes outputs_dev[k]; all for `batch` images.  One kernel executes the whole run: its blocks draw
+ * (layer, tile) work items in layer order, and a tile starts as soon as the images it reads are complete in the layer
+ * before -- there is no kernel boundary and no device-wide barrier between the layers, so tiles of neighbouring layers
+ * overlap on every CU.  The tiles are those of mi355x_conv2d_run's kernels: the bytes written to every outputs_dev[k]
+ * equal the bytes of running the plans one after the other with mi355x_conv2d_run -- in the reference the workloads of a
+ * network run in sequence on the calling thread (LoadedNetwork::Execute, src/armnn/LoadedNetwork.cpp:845-1100, each
+ * RefDepthwiseConvolution2dWorkload.cpp:38-62 / RefConvolution2dWorkload.cpp:38-58).
+ *   Accepted members (mi355x_chain_accepts: 0, else MI355X_ERR_UNSUPPORTED with the reason): 3x3 depthwise plans of
+ * multiplier 1, stride 1 or 2, a channel count that is a multiple of 128 and weights that fit one int8 each; unpadded 1x1
+ * stride-1 Convolution2d plans with more than 128 input channels that are a multiple of 128, output channels a multiple of
+ * 16 and weights without a zero point.  Tensors stay below 2 GiB.
+ *   The addresses are bound at creation (a captured graph replays them).  input_dev and all outputs must not overlap each
+ * other: every tensor of the run is written once per launch and read by other blocks as soon as an image is complete.
+ * Outputs are 128-byte aligned, the input 16-byte aligned.  The chain owns a few KB of device memory (work queue head and
+ * one counter per layer and image), so two launches of ONE chain object must not run at the same time; launches of
+ * different chain objects may.  The plans must outlive the chain.
+ *   mi355x_chain_status waits for nothing: call it after synchronizing the stream.  *gave_up is the number of blocks
+ * whose bounded wait for a producer ran out (2 s; never in normal operation): if it is not 0 the outputs of that launch
+ * are invalid; the call clears the condition. */
+typedef struct mi355x_chain_s* mi355x_chain_t;
+int mi355x_chain_accepts(mi355x_conv2d_t plan, uint32_t batch);
+int mi355x_chain_create(uint32_t n_layers, const mi355x_conv2d_t* plans, uint32_t batch, const void* input_dev,
+                        void* const* outputs_dev, mi355x_chain_t* chain);
+int mi355x_chain_run(mi355x_chain_t chain, mi355x_stream_t stream);
+int mi355x_chain_status(mi355x_chain_t chain, uint32_t* gave_up);
+/* work items (tiles) of one launch and the number of persistent blocks it uses */
+int mi355x_chain_info(mi355x_chain_t chain, uint32_t* work_items, uint32_t* blocks);
+/* Measurement support (not for graph capture: allocates, synchronizes the stream and uses the default stream for the
+ * read-back): one launch of the chain whose blocks add up shader-clock cycles per phase; sums[0..4] = cycles, summed over
+ * all blocks, spent taking an item from the queue, waiting for producers, inside matrix-core tiles, inside depthwise
+ * tiles, and waiting for the tile's stores plus the hand-over; sums[5], sums[6] = matrix-core and depthwise tiles run,
+ * sums[7] = tiles that found their producer unfinished.  The reference's counterpart is its per-workload profiler
+ * (src/armnn/Profiling.hpp:227-236). */
+int mi355x_chain_run_stamped(mi355x_chain_t chain, mi355x_stream_t stream, uint64_t* sums);
+int mi355x_chain_destroy(mi355x_chain_t chain);
 /* which kernel a plan resolved to (mi355x_algo) and its tile configuration, for logs and tests */
 int mi355x_conv2d_algo(mi355x_conv2d_t plan, int32_t* algo, char* desc_buf, size_t desc_len);
 /* Name of the device kernel the calling thread's last *_run call launched, with its template arguments, as a profiler
