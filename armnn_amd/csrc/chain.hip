@@ -3,10 +3,22 @@
 #include "plan.h"
 
 #include <algorithm>
+#include <mutex>
 #include <string>
 #include <vector>
 
 using namespace mi355x;
+
+// mi355x_chain_run_noalloc: the memory mi355x_chain_create would allocate (layer records, per-image tile counts, queue heads
+// and counters), as one file-scope device array.  Every GPU the library runs on holds its own copy until the process
+// ends.  In host code the array's name is only a stand-in: its address on the current device comes from
+// hipGetSymbolAddress, once per device, and only that pointer is handed to kernels and copies.
+constexpr uint32_t kNoallocMaxLayers = 32, kNoallocMaxBatch = 64;
+constexpr size_t kNoallocSyncBytes = (static_cast<size_t>(kChainCounterSlot) + kNoallocMaxLayers * kNoallocMaxBatch) * kChainSlot * 4;   // 264 320
+constexpr size_t kNoallocNeedBytes = static_cast<size_t>(kNoallocMaxLayers) * kNoallocMaxBatch * 4;                                        //   8 192
+constexpr size_t kNoallocLayerBytes = static_cast<size_t>(kNoallocMaxLayers) * sizeof(ChainLayer);
+constexpr size_t kNoallocBytes = kNoallocSyncBytes + kNoallocNeedBytes + kNoallocLayerBytes;
+static __device__ __align__(256) unsigned char scratch[kNoallocBytes];
 
 struct mi355x_chain_s
 {
@@ -123,25 +135,13 @@ int ChainOccupancy(int smem, int* blocks_per_cu)
     return 0;
 }
 
-} // namespace
-
-extern "C" {
-
-int mi355x_chain_accepts(mi355x_conv2d_t plan, uint32_t batch)
+// Everything mi355x_chain_create and mi355x_chain_run_noalloc derive from the caller's arguments: layer records, queue
+// sizes, the per-image tile counts, LDS size and grid.  Fills `c` (no device memory is touched) and `need_out`.
+int DescribeRun(uint32_t n_layers, const mi355x_conv2d_t* plans, uint32_t batch, const void* input_dev, void* const* outputs_dev,
+                mi355x_chain_s* c, std::vector<uint32_t>* need_out)
 {
-    ChainLayer L;
-    // addresses do not matter for the answer
-    return Describe(plan, batch, nullptr, nullptr, &L);
-}
-
-int mi355x_chain_create(uint32_t n_layers, const mi355x_conv2d_t* plans, uint32_t batch, const void* input_dev, void* const* outputs_dev,
-                        mi355x_chain_t* chain)
-{
-    if (!chain) return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain pointer is null");
-    *chain = nullptr;
     if (n_layers == 0 || !plans || !outputs_dev || !input_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain: no layers / null pointers");
     if (batch == 0 || batch > 65535) return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain: batch must be 1 .. 65535");
-    auto c = new mi355x_chain_s;
     c->batch = static_cast<int>(batch);
     c->layers.resize(n_layers);
     struct Range { uintptr_t lo, hi; };
@@ -152,21 +152,20 @@ int mi355x_chain_create(uint32_t n_layers, const mi355x_conv2d_t* plans, uint32_
         const mi355x_conv2d_s* p = plans[k];
         void* y = outputs_dev[k];
         const void* x = k == 0 ? input_dev : outputs_dev[k - 1];
-        if (!p || !y) { delete c; return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain: layer %u has a null plan or output", k); }
+        if (!p || !y) { return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain: layer %u has a null plan or output", k); }
         if ((reinterpret_cast<uintptr_t>(x) & 15) != 0 || (reinterpret_cast<uintptr_t>(y) & 127) != 0)
         {
-            delete c;
             return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain: layer %u needs a 16-byte aligned input and a 128-byte aligned output", k);
         }
         ChainLayer& L = c->layers[k];
-        if (const int rc = Describe(p, batch, x, y, &L)) { delete c; return rc; }
+        if (const int rc = Describe(p, batch, x, y, &L)) { return rc; }
         const ConvGeom& g = p->geom;
         if (k > 0)
         {
             const ConvGeom& q = plans[k - 1]->geom;
-            if (q.Ho != g.H || q.Wo != g.W || q.Co != g.Ci) { delete c; return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain: layer %u does not consume layer %u's output shape", k, k - 1); }
+            if (q.Ho != g.H || q.Wo != g.W || q.Co != g.Ci) { return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain: layer %u does not consume layer %u's output shape", k, k - 1); }
             const mi355x_quant& a = plans[k - 1]->d.output; const mi355x_quant& b = p->d.input;
-            if (a.dtype != b.dtype || a.scale != b.scale || a.offset != b.offset) { delete c; return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain: layer %u reads another quantization than layer %u writes", k, k - 1); }
+            if (a.dtype != b.dtype || a.scale != b.scale || a.offset != b.offset) { return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain: layer %u reads another quantization than layer %u writes", k, k - 1); }
         }
         L.src = static_cast<int>(k) - 1;
         // queue q takes the layer's groups q, q + 8, ...: their items follow those of the layers before
@@ -177,7 +176,7 @@ int mi355x_chain_create(uint32_t n_layers, const mi355x_conv2d_t* plans, uint32_
             c->qtotal[q] += (n_groups > q ? (n_groups - q + kChainQueues - 1) / kChainQueues : 0) * L.group;
         }
         items += L.n_items;
-        if (items > 0x3fffffffll) { delete c; return SetError(MI355X_ERR_UNSUPPORTED, "chain: too many work items"); }
+        if (items > 0x3fffffffll) { return SetError(MI355X_ERR_UNSUPPORTED, "chain: too many work items"); }
         if (k == 0) ranges.push_back(Range{reinterpret_cast<uintptr_t>(x), reinterpret_cast<uintptr_t>(x) + static_cast<uintptr_t>(batch) * g.H * g.W * g.Ci});
         ranges.push_back(Range{reinterpret_cast<uintptr_t>(y), reinterpret_cast<uintptr_t>(y) + static_cast<uintptr_t>(batch) * g.Ho * g.Wo * g.Co});
     }
@@ -186,13 +185,13 @@ int mi355x_chain_create(uint32_t n_layers, const mi355x_conv2d_t* plans, uint32_
         for (size_t j = i + 1; j < ranges.size(); ++j)
             if (ranges[i].lo < ranges[j].hi && ranges[j].lo < ranges[i].hi)
             {
-                delete c;
-                return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain: tensors %zu and %zu of the run overlap (0 = the input, k = output of layer k - 1)", i, j);
+                    return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain: tensors %zu and %zu of the run overlap (0 = the input, k = output of layer k - 1)", i, j);
             }
     c->total_items = static_cast<int>(items);
 
     // tiles of layer l that touch image n
-    std::vector<uint32_t> need(static_cast<size_t>(n_layers) * batch, 0u);
+    std::vector<uint32_t>& need = *need_out;
+    need.assign(static_cast<size_t>(n_layers) * batch, 0u);
     for (uint32_t k = 0; k < n_layers; ++k)
     {
         const ChainLayer& L = c->layers[k];
@@ -217,18 +216,40 @@ int mi355x_chain_create(uint32_t n_layers, const mi355x_conv2d_t* plans, uint32_
             c->smem = std::max(c->smem, L.variant == 2 ? GemmPanelSmemBytes<kChainPanelStages, 2>(L.tiles_n * 64) : GemmPanelSmemBytes<kChainPanelStages, 4>(L.tiles_n * 64));
     int per_cu = 0;
     int rc = c->stages == 3 ? ChainOccupancy<3>(c->smem, &per_cu) : c->stages == 4 ? ChainOccupancy<4>(c->smem, &per_cu) : ChainOccupancy<2>(c->smem, &per_cu);
-    if (rc) { delete c; return rc; }
-    if (per_cu < 1) { delete c; return SetError(MI355X_ERR_UNSUPPORTED, "chain: the kernel does not fit a CU"); }
+    if (rc) { return rc; }
+    if (per_cu < 1) { return SetError(MI355X_ERR_UNSUPPORTED, "chain: the kernel does not fit a CU"); }
     int dev = 0, cus = 0;
     if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 1)
     {
-        delete c;
         return SetError(MI355X_ERR_NO_DEVICE, "chain: cannot read the device's CU count");
     }
     if (opt.chain_blocks_per_cu > 0) per_cu = std::min(per_cu, opt.chain_blocks_per_cu);
     // at least one block per queue; never more blocks than the device holds at once
     c->grid = std::max(kChainQueues, std::min(c->total_items, per_cu * cus));
 
+    return 0;
+}
+
+} // namespace
+
+extern "C" {
+
+int mi355x_chain_accepts(mi355x_conv2d_t plan, uint32_t batch)
+{
+    ChainLayer L;
+    // addresses do not matter for the answer
+    return Describe(plan, batch, nullptr, nullptr, &L);
+}
+
+int mi355x_chain_create(uint32_t n_layers, const mi355x_conv2d_t* plans, uint32_t batch, const void* input_dev, void* const* outputs_dev,
+                        mi355x_chain_t* chain)
+{
+    if (!chain) return SetError(MI355X_ERR_INVALID_ARGUMENT, "chain pointer is null");
+    *chain = nullptr;
+    auto c = new mi355x_chain_s;
+    std::vector<uint32_t> need;
+    int rc = DescribeRun(n_layers, plans, batch, input_dev, outputs_dev, c, &need);
+    if (rc) { delete c; return rc; }
     const size_t sync_words = (static_cast<size_t>(kChainCounterSlot) + need.size()) * kChainSlot;
     const std::vector<uint32_t> zeros(sync_words, 0u);
     if (hipMalloc(reinterpret_cast<void**>(&c->d_layers), c->layers.size() * sizeof(ChainLayer)) != hipSuccess ||
@@ -252,6 +273,53 @@ int mi355x_chain_run(mi355x_chain_t chain, mi355x_stream_t stream)
     if (chain->stages == 3) return LaunchChain<3>(chain, ToHip(stream));
     if (chain->stages == 4) return LaunchChain<4>(chain, ToHip(stream));
     return LaunchChain<2>(chain, ToHip(stream));
+}
+
+int mi355x_chain_run_noalloc(uint32_t n_layers, const mi355x_conv2d_t* plans, uint32_t batch, const void* input_dev, void* const* outputs_dev,
+                             mi355x_stream_t stream)
+{
+    if (n_layers > kNoallocMaxLayers || batch > kNoallocMaxBatch)
+        return SetError(MI355X_ERR_UNSUPPORTED, "chain without allocation: at most %u layers and %u images (got %u and %u); use mi355x_chain_create",
+                        kNoallocMaxLayers, kNoallocMaxBatch, n_layers, batch);
+    // the array's address on the current device, looked up once per device
+    constexpr int kMaxDevices = 64;
+    static std::mutex mutex;
+    static unsigned char* base_of[kMaxDevices] = {};
+    int dev = 0;
+    MI355X_HIP(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kMaxDevices) return SetError(MI355X_ERR_UNSUPPORTED, "chain without allocation: device index %d", dev);
+    unsigned char* base = nullptr;
+    {
+        std::lock_guard<std::mutex> lock(mutex);
+        if (!base_of[dev])
+        {
+            void* p = nullptr;
+            MI355X_HIP(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+            base_of[dev] = static_cast<unsigned char*>(p);
+        }
+        base = base_of[dev];
+    }
+    // the description lives in the calling thread's own storage, which keeps its capacity from call to call
+    thread_local mi355x_chain_s host;
+    thread_local std::vector<uint32_t> need;
+    host.layers.clear();
+    host.total_items = 0;
+    for (int q = 0; q < kChainQueues; ++q) host.qtotal[q] = 0;
+    if (const int rc = DescribeRun(n_layers, plans, batch, input_dev, outputs_dev, &host, &need)) return rc;
+    host.d_sync = reinterpret_cast<uint32_t*>(base);
+    host.d_need = reinterpret_cast<uint32_t*>(base + kNoallocSyncBytes);
+    host.d_layers = reinterpret_cast<ChainLayer*>(base + kNoallocSyncBytes + kNoallocNeedBytes);
+    hipStream_t s = ToHip(stream);
+    // The array keeps what the call before left there.  Queue heads and counters must start at zero (a launch leaves them so,
+    // but one that gave up, or a larger run before, may not have): a fill kernel, which a captured graph can hold.
+    const size_t sync_bytes = (static_cast<size_t>(kChainCounterSlot) + need.size()) * kChainSlot * 4;
+    int rc = mi355x_fill_u8(host.d_sync, 0, sync_bytes, stream);
+    if (!rc) rc = hipMemcpyAsync(host.d_need, need.data(), need.size() * 4, hipMemcpyHostToDevice, s) == hipSuccess ? 0 : SetError(MI355X_ERR_INVALID_ARGUMENT, "chain without allocation: copy of the tile counts failed");
+    if (!rc) rc = hipMemcpyAsync(host.d_layers, host.layers.data(), host.layers.size() * sizeof(ChainLayer), hipMemcpyHostToDevice, s) == hipSuccess ? 0 : SetError(MI355X_ERR_INVALID_ARGUMENT, "chain without allocation: copy of the layer records failed");
+    if (!rc) rc = host.stages == 3 ? LaunchChain<3>(&host, s) : host.stages == 4 ? LaunchChain<4>(&host, s) : LaunchChain<2>(&host, s);
+    // the thread-local object must not free the static array
+    host.d_sync = nullptr; host.d_need = nullptr; host.d_layers = nullptr;
+    return rc;
 }
 
 int mi355x_chain_status(mi355x_chain_t chain, uint32_t* gave_up)

@@ -29,7 +29,7 @@ EXPORTS = [
     "mi355x_graph_capture_begin", "mi355x_graph_capture_end", "mi355x_graph_launch", "mi355x_graph_destroy",
     "mi355x_conv2d_create", "mi355x_conv2d_run", "mi355x_conv2d_destroy", "mi355x_conv2d_algo",
     "mi355x_conv2d_fusable", "mi355x_conv2d_run_fused", "mi355x_conv2d_run_add", "mi355x_conv2d_set_concurrency",
-    "mi355x_chain_accepts", "mi355x_chain_create", "mi355x_chain_run", "mi355x_chain_status", "mi355x_chain_info", "mi355x_chain_run_stamped", "mi355x_chain_destroy",
+    "mi355x_chain_accepts", "mi355x_chain_create", "mi355x_chain_run", "mi355x_chain_status", "mi355x_chain_info", "mi355x_chain_run_stamped", "mi355x_chain_run_noalloc", "mi355x_chain_destroy",
     "mi355x_fc_create", "mi355x_fc_run", "mi355x_fc_destroy", "mi355x_fc_algo",
     "mi355x_activation_run", "mi355x_pool2d_run", "mi355x_add_run", "mi355x_softmax_run", "mi355x_pad_run",
 ]
@@ -120,6 +120,7 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
             "mi355x_chain_run": [V, V], "mi355x_chain_status": [V, C.POINTER(C.c_uint32)],
             "mi355x_chain_info": [V, C.POINTER(C.c_uint32), C.POINTER(C.c_uint32)], "mi355x_chain_destroy": [V],
             "mi355x_chain_run_stamped": [V, V, C.POINTER(C.c_uint64)],
+            "mi355x_chain_run_noalloc": [C.c_uint32, C.POINTER(V), C.c_uint32, V, C.POINTER(V), V],
             "mi355x_fc_create": [C.POINTER(FcDesc), V, C.POINTER(ConstQuant), V, C.POINTER(ConstQuant), C.POINTER(V)],
             "mi355x_fc_run": [V, C.c_uint32, V, V, V], "mi355x_fc_destroy": [V],
             "mi355x_fc_algo": [V, C.POINTER(C.c_int32), C.c_char_p, C.c_size_t],
@@ -351,6 +352,15 @@ class LayerChain:
         chain = C.c_void_p()
         _chk(self.lib.mi355x_chain_create(n, pa, batch, x_dev, oa, C.byref(chain)))
         self.chain = chain.value
+
+    @staticmethod
+    def run_noalloc(plans: Sequence["Conv2dPlan"], batch: int, x_dev: int, outputs_dev: Sequence[int], stream=None):
+        """mi355x_chain_run_noalloc: the same run without a chain object and without any device allocation (at most 32
+        layers and 64 images); calls on one GPU share one device array and must not overlap."""
+        n = len(plans)
+        pa = (C.c_void_p * n)(*[p.plan for p in plans])
+        oa = (C.c_void_p * n)(*outputs_dev)
+        _chk(load_library().mi355x_chain_run_noalloc(n, pa, batch, x_dev, oa, stream))
 
     @staticmethod
     def accepts(plan: "Conv2dPlan", batch: int) -> bool:

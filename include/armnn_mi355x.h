@@ -266,6 +266,18 @@ int mi355x_chain_accepts(mi355x_conv2d_t plan, uint32_t batch);
 int mi355x_chain_create(uint32_t n_layers, const mi355x_conv2d_t* plans, uint32_t batch, const void* input_dev,
                         void* const* outputs_dev, mi355x_chain_t* chain);
 int mi355x_chain_run(mi355x_chain_t chain, mi355x_stream_t stream);
+/* The same run as mi355x_chain_create + mi355x_chain_run in one call that allocates nothing: the layer records, the work
+ * queue heads and the per-image counters live in a device array that is part of the library (about 300 KB on every GPU
+ * the library runs on, held until the process ends).  It has no counterpart in the reference; it is for callers that
+ * cannot allocate device memory where they launch: code under graph capture, tight serving loops, harnesses that forbid
+ * hipMalloc.  Limits: at most 32 layers and 64 images, else MI355X_ERR_UNSUPPORTED (use mi355x_chain_create).  Same
+ * members, same rules for the tensors, same bytes.  All calls on one GPU share the one array: two calls whose launches
+ * could run at the same time on that GPU race (order them on one stream or with events); the array keeps the last call's
+ * contents, and each call first sets what must start at zero with a fill kernel.  The two small host-to-device copies of
+ * the call read the calling thread's own buffers; wait for the stream before the same thread calls again with other
+ * arguments.  mi355x_chain_status does not apply: synchronize and compare, or use the chain object where a report is needed. */
+int mi355x_chain_run_noalloc(uint32_t n_layers, const mi355x_conv2d_t* plans, uint32_t batch, const void* input_dev,
+                             void* const* outputs_dev, mi355x_stream_t stream);
 int mi355x_chain_status(mi355x_chain_t chain, uint32_t* gave_up);
 /* work items (tiles) of one launch and the number of persistent blocks it uses */
 int mi355x_chain_info(mi355x_chain_t chain, uint32_t* work_items, uint32_t* blocks);
