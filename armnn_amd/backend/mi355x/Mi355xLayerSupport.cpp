@@ -68,6 +68,16 @@ bool CheckConstants(const TensorInfo& weights, const Optional<TensorInfo>& biase
     }
     return true;
 }
+
+// The device kernels accumulate sum (x - zx)(w - zw) exactly in 32 bits and refuse a plan whose taps could overflow that
+// (mi355x_conv2d_create: K * max|x - zx| * max|w - zw| < 2^31, with the true zero points and weights).  Layer support sees
+// neither, so it applies the bound that holds for any of them: K * 255 * 255 < 2^31, i.e. K <= 33 025 taps per output.
+// A layer beyond that goes to the next backend at optimization time instead of failing at the first inference.
+bool CheckTaps(unsigned long long taps, Optional<std::string&> reason)
+{
+    if (taps * 255ull * 255ull >= (1ull << 31)) return No(reason, "more than 33 025 taps per output could overflow the 32-bit accumulator");
+    return true;
+}
 } // namespace
 
 bool Mi355xLayerSupport::IsConvolution2dSupported(const TensorInfo& input, const TensorInfo& output, const Convolution2dDescriptor& d,
@@ -80,6 +90,7 @@ bool Mi355xLayerSupport::IsConvolution2dSupported(const TensorInfo& input, const
     if (weights.GetShape()[0] != output.GetShape()[3]) return No(reason, "weights [O,H,W,I]: O differs from the output channels");
     if (input.GetShape()[0] != output.GetShape()[0]) return No(reason, "batch sizes differ");
     if (d.m_StrideX == 0 || d.m_StrideY == 0 || d.m_DilationX == 0 || d.m_DilationY == 0) return No(reason, "zero stride or dilation");
+    if (!CheckTaps(static_cast<unsigned long long>(weights.GetShape()[1]) * weights.GetShape()[2] * weights.GetShape()[3], reason)) return false;
     return CheckConstants(weights, biases, d.m_BiasEnabled, output.GetShape()[3], 0, reason);
 }
 
@@ -110,6 +121,7 @@ bool Mi355xLayerSupport::IsFullyConnectedSupported(const TensorInfo& input, cons
     const unsigned int wo = d.m_TransposeWeightMatrix ? weights.GetShape()[0] : weights.GetShape()[1];
     if (wk != k || wo != o) return No(reason, "weights shape does not match input width / output width");
     if (output.GetShape()[0] != input.GetShape()[0]) return No(reason, "batch sizes differ");
+    if (!CheckTaps(k, reason)) return false;
     return CheckConstants(weights, biases, d.m_BiasEnabled, o, d.m_TransposeWeightMatrix ? 0 : 1, reason);
 }
 

@@ -6,8 +6,8 @@
 #include <armnn/backends/MemCopyWorkload.hpp>
 #include <armnn/utility/PolymorphicDowncast.hpp>
 
+#include <functional>
 #include <mutex>
-#include <thread>
 
 namespace armnn
 {
@@ -15,46 +15,44 @@ namespace
 {
 const BackendId s_Id{Mi355xBackendId()};
 
-// The Convolution2d workload created last, while no workload that writes device tensors has been created since: the
-// candidate an Addition created next may take over (Mi355xAdditionWorkload::TakeOver).  A network's workloads are created in
-// execution order by one thread; the thread is recorded so that networks loading at the same time at worst lose a
-// pairing.  The entry is dropped when the workload is destroyed.
-struct Candidate
+}
+
+struct Mi355xWorkloadFactory::Candidate
 {
     std::mutex mutex;
     Mi355xConvolution2dWorkload* convolution = nullptr;
-    std::thread::id thread;
+    Mi355xConvolution2dWorkload* Take()
+    {
+        std::lock_guard<std::mutex> lock(mutex);
+        Mi355xConvolution2dWorkload* w = convolution;
+        convolution = nullptr;
+        return w;
+    }
 };
-Candidate& TheCandidate()
-{
-    static Candidate c;
-    return c;
-}
-Mi355xConvolution2dWorkload* TakeCandidate()
-{
-    Candidate& c = TheCandidate();
-    std::lock_guard<std::mutex> lock(c.mutex);
-    Mi355xConvolution2dWorkload* w = c.thread == std::this_thread::get_id() ? c.convolution : nullptr;
-    c.convolution = nullptr;
-    return w;
-}
 
-// the convolution workload the factory hands out: its destructor withdraws it as the candidate, should it still be one
+namespace
+{
+// the convolution workload the factory hands out: its destructor withdraws it as its factory's candidate, should it still be one
 class CandidateConvolution final : public Mi355xConvolution2dWorkload
 {
 public:
-    using Mi355xConvolution2dWorkload::Mi355xConvolution2dWorkload;
-    ~CandidateConvolution() override
+    template <typename C>
+    CandidateConvolution(const Convolution2dQueueDescriptor& d, const WorkloadInfo& info, std::shared_ptr<C> slot)
+        : Mi355xConvolution2dWorkload(d, info), m_Withdraw([slot](Mi355xConvolution2dWorkload* self) {
+              std::lock_guard<std::mutex> lock(slot->mutex);
+              if (slot->convolution == self) slot->convolution = nullptr;
+          })
     {
-        Candidate& c = TheCandidate();
-        std::lock_guard<std::mutex> lock(c.mutex);
-        if (c.convolution == this) c.convolution = nullptr;
     }
+    ~CandidateConvolution() override { m_Withdraw(this); }
+private:
+    std::function<void(Mi355xConvolution2dWorkload*)> m_Withdraw;
 };
 }
 
-Mi355xWorkloadFactory::Mi355xWorkloadFactory(const std::shared_ptr<Mi355xMemoryManager>& memoryManager) : m_MemoryManager(memoryManager) {}
-Mi355xWorkloadFactory::Mi355xWorkloadFactory() : m_MemoryManager(new Mi355xMemoryManager()) {}
+Mi355xWorkloadFactory::Mi355xWorkloadFactory(const std::shared_ptr<Mi355xMemoryManager>& memoryManager)
+    : m_MemoryManager(memoryManager), m_Candidate(std::make_shared<Candidate>()) {}
+Mi355xWorkloadFactory::Mi355xWorkloadFactory() : m_MemoryManager(new Mi355xMemoryManager()), m_Candidate(std::make_shared<Candidate>()) {}
 
 const BackendId& Mi355xWorkloadFactory::GetBackendId() const { return s_Id; }
 
@@ -75,18 +73,16 @@ std::unique_ptr<ITensorHandle> Mi355xWorkloadFactory::CreateTensorHandle(const T
 std::unique_ptr<IWorkload> Mi355xWorkloadFactory::CreateWorkload(LayerType type, const QueueDescriptor& descriptor, const WorkloadInfo& info) const
 {
     // constants write no tensor another workload's operand could share an address with: they leave the candidate alone
-    Mi355xConvolution2dWorkload* candidate = type == LayerType::Constant ? nullptr : TakeCandidate();
+    Mi355xConvolution2dWorkload* candidate = type == LayerType::Constant ? nullptr : m_Candidate->Take();
     switch (type)
     {
         case LayerType::Convolution2d:
         {
-            auto w = std::make_unique<CandidateConvolution>(*PolymorphicDowncast<const Convolution2dQueueDescriptor*>(&descriptor), info);
+            auto w = std::make_unique<CandidateConvolution>(*PolymorphicDowncast<const Convolution2dQueueDescriptor*>(&descriptor), info, m_Candidate);
             if (w->FeedsOnlyAnAddition())
             {
-                Candidate& c = TheCandidate();
-                std::lock_guard<std::mutex> lock(c.mutex);
-                c.convolution = w.get();
-                c.thread = std::this_thread::get_id();
+                std::lock_guard<std::mutex> lock(m_Candidate->mutex);
+                m_Candidate->convolution = w.get();
             }
             return w;
         }

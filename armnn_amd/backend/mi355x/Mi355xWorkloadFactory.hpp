@@ -23,5 +23,11 @@ public:
     std::unique_ptr<IWorkload> CreateWorkload(LayerType type, const QueueDescriptor& descriptor, const WorkloadInfo& info) const override;
 private:
     mutable std::shared_ptr<Mi355xMemoryManager> m_MemoryManager;
+    /// The Convolution2d workload THIS factory created last, while it has created no other workload that writes device
+    /// tensors since: the one an Addition created next may take over (Mi355xAdditionWorkload::TakeOver).  A loaded network
+    /// has a factory of its own and creates its workloads in execution order, so pairs never cross networks, whatever else
+    /// the process loads meanwhile.  Shared with the convolution workload, which withdraws itself when it is destroyed.
+    struct Candidate;
+    std::shared_ptr<Candidate> m_Candidate;
 };
 } // namespace armnn

@@ -133,6 +133,28 @@ TEST_CASE("layer support: the accepted envelope and the reasons outside it", "cp
     u8out.SetDataType(DataType::QAsymmU8);
     CHECK(!ls.IsLayerSupported(LayerType::Convolution2d, {l.in, u8out, l.w, l.b}, d, EmptyOptional(), EmptyOptional(), reason));
 
+    // more taps per output than a 32-bit accumulator is sure to hold (33 025): answered here, so that the optimizer falls
+    // back instead of the plan being refused at the first inference.  Only shapes are looked at.
+    {
+        TensorInfo wideIn({1, 1, 1, 40000}, DataType::QAsymmS8, 0.05f, -3);
+        TensorInfo wideW({8, 1, 1, 40000}, DataType::QSymmS8, 0.01f, 0);
+        wideW.SetConstant(true);
+        TensorInfo wideOut({1, 1, 1, 8}, DataType::QAsymmS8, 0.1f, 5);
+        Convolution2dDescriptor plain;
+        plain.m_DataLayout = DataLayout::NHWC;
+        CHECK(!ls.IsLayerSupported(LayerType::Convolution2d, {wideIn, wideOut, wideW}, plain, EmptyOptional(), EmptyOptional(), reason));
+        CHECK(why.find("33 025 taps") != std::string::npos);
+        TensorInfo okIn({1, 1, 1, 33025}, DataType::QAsymmS8, 0.05f, -3), okW({8, 1, 1, 33025}, DataType::QSymmS8, 0.01f, 0);
+        okW.SetConstant(true);
+        CHECK(ls.IsLayerSupported(LayerType::Convolution2d, {okIn, wideOut, okW}, plain, EmptyOptional(), EmptyOptional(), reason));
+        TensorInfo fcIn({2, 40000}, DataType::QAsymmS8, 0.05f, -3), fcW({40000, 8}, DataType::QSymmS8, 0.01f, 0), fcOut({2, 8}, DataType::QAsymmS8, 0.1f, 5);
+        fcW.SetConstant(true);
+        FullyConnectedDescriptor fd;
+        fd.m_BiasEnabled = false;
+        CHECK(!ls.IsLayerSupported(LayerType::FullyConnected, {fcIn, fcOut, fcW}, fd, EmptyOptional(), EmptyOptional(), reason));
+        CHECK(why.find("33 025 taps") != std::string::npos);
+    }
+
     // depthwise: [1,H,W,O] weights quantized along dimension 3
     QLayer dw = MakeConv(QLayer::Depthwise, in, 16, 3, 2, 0.1f, 5, false, true, 2);
     DepthwiseConvolution2dDescriptor dd;
@@ -1876,6 +1898,57 @@ TEST_CASE("runtime: an Addition whose sum was placed over the convolution's inpu
         CHECK(d.mismatches * 1000 <= d.n);
     }
     mi355x::SetLanes(lanesBefore);
+}
+
+TEST_CASE("runtime: two networks loaded side by side pair their own convolutions and Additions, and survive each other's unloading", "gpu")
+{
+    // every loaded network has a workload factory of its own, and a pairing never leaves its factory: load A, load B, run
+    // both interleaved, unload A, run B again
+    ResidualBlock blockA(4);
+    NarrowingResidualBlock blockB(2);
+    const std::vector<uint8_t> inA = RandomActivations(blockA.in, 191), inB = RandomActivations(blockB.in, 192);
+    TensorInfo constA = blockA.in, constB = blockB.in;
+    constA.SetConstant(true);
+    constB.SetConstant(true);
+    auto runAlone = [&](INetworkPtr net, const TensorInfo& cin, const std::vector<uint8_t>& in, const TensorInfo& out) {
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        OptimizerOptionsOpaque options;
+        options.AddModelOption(BackendOptions("Mi355x", {{"FuseAdditions", false}}));
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, rt->GetDeviceSpec(), options);
+        NetworkId id = -1;
+        std::string err;
+        REQUIRE(rt->LoadNetwork(id, std::move(opt), err) == Status::Success);
+        std::vector<uint8_t> result(out.GetNumBytes(), 0);
+        REQUIRE(rt->EnqueueWorkload(id, InputTensors{{0, ConstTensor(cin, in.data())}}, OutputTensors{{0, Tensor(out, result.data())}}) == Status::Success);
+        return result;
+    };
+    const std::vector<uint8_t> wantA = runAlone(blockA.Build(), constA, inA, blockA.sum);
+    const std::vector<uint8_t> wantB = runAlone(blockB.Build(), constB, inB, blockB.sum);
+
+    const unsigned long long pairsBefore = Mi355xAdditionWorkload::PairsFormed();
+    IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+    NetworkId idA = -1, idB = -1;
+    std::string err;
+    {
+        INetworkPtr netA = blockA.Build(), netB = blockB.Build();
+        IOptimizedNetworkPtr optA = Optimize(*netA, {kMi355x}, rt->GetDeviceSpec(), OptimizerOptionsOpaque());
+        IOptimizedNetworkPtr optB = Optimize(*netB, {kMi355x}, rt->GetDeviceSpec(), OptimizerOptionsOpaque());
+        REQUIRE(rt->LoadNetwork(idA, std::move(optA), err) == Status::Success);
+        REQUIRE(rt->LoadNetwork(idB, std::move(optB), err) == Status::Success);
+    }
+    CHECK(Mi355xAdditionWorkload::PairsFormed() - pairsBefore == 2);
+    std::vector<uint8_t> gotA(blockA.sum.GetNumBytes(), 0), gotB(blockB.sum.GetNumBytes(), 0);
+    for (int pass = 0; pass < 2; ++pass)
+    {
+        REQUIRE(rt->EnqueueWorkload(idA, InputTensors{{0, ConstTensor(constA, inA.data())}}, OutputTensors{{0, Tensor(blockA.sum, gotA.data())}}) == Status::Success);
+        REQUIRE(rt->EnqueueWorkload(idB, InputTensors{{0, ConstTensor(constB, inB.data())}}, OutputTensors{{0, Tensor(blockB.sum, gotB.data())}}) == Status::Success);
+        CHECK(gotA == wantA);
+        CHECK(gotB == wantB);
+    }
+    REQUIRE(rt->UnloadNetwork(idA) == Status::Success);
+    std::fill(gotB.begin(), gotB.end(), 0);
+    REQUIRE(rt->EnqueueWorkload(idB, InputTensors{{0, ConstTensor(constB, inB.data())}}, OutputTensors{{0, Tensor(blockB.sum, gotB.data())}}) == Status::Success);
+    CHECK(gotB == wantB);
 }
 
 TEST_CASE("runtime: a layer the device lacks runs on the next backend and the copies preserve the data", "gpu")

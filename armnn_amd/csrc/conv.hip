@@ -978,7 +978,9 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
                 else if (p->tile_override == 1256) { bm = 128; bn = 256; }
                 else if ((p->Co_pad % 256) == 0 && rows256 * (p->Co_pad / 256) >= 224) { bm = 256; bn = 256; }
                 else if (rows256 * (p->Co_pad / 128) >= 224) { bm = 256; bn = 128; }
-                if (bm != 0) return LaunchBig(p, bm, bn, batch, x, y, stream);
+                // the large-tile kernel walks a filter's taps through a 32-bit mask per row: filters of more than 32 taps
+                // (6 x 6, 7 x 7 ...) stay on the tiles below, also when a test forces the large tile
+                if (bm != 0 && (unit || g.Kh * g.Kw <= 32)) return LaunchBig(p, bm, bn, batch, x, y, stream);
             }
             if ((tile == 4064 || tile == 2064) && p->zw_neg == 0) return LaunchIgemmKSplit(p, tile == 4064 ? 4 : 2, batch, x, y, stream);
             if (tile == 64 && p->tile_override == 0 && p->zw_neg == 0 && p->K_pad >= 16 * 128)
@@ -1368,7 +1370,15 @@ int mi355x_conv2d_run_add(mi355x_conv2d_t plan, uint32_t batch, const void* inpu
     if (activation < MI355X_ACT_NONE || activation > MI355X_ACT_BOUNDED_RELU) return SetError(MI355X_ERR_UNSUPPORTED, "activation %d", activation);
     if (batch == 0) return 0;
     if (!other_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "other input / output pointer is null");
-    if (other_dev == output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "the Addition's other input may not be the output buffer");
+    if (!input_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "input pointer is null");
+    {
+        // one launch reads the input and the other operand while it writes the sum: the sum may share bytes with neither
+        const uintptr_t n_out = static_cast<uintptr_t>(batch) * plan->d.out_h * plan->d.out_w * plan->d.out_c;
+        const uintptr_t n_in = static_cast<uintptr_t>(batch) * plan->d.in_h * plan->d.in_w * plan->d.in_c;
+        const uintptr_t y0 = reinterpret_cast<uintptr_t>(output_dev), x0 = reinterpret_cast<uintptr_t>(input_dev), o0 = reinterpret_cast<uintptr_t>(other_dev);
+        if (y0 < o0 + n_out && o0 < y0 + n_out) return SetError(MI355X_ERR_INVALID_ARGUMENT, "the Addition's other input may not overlap the output buffer");
+        if (y0 < x0 + n_in && x0 < y0 + n_out) return SetError(MI355X_ERR_INVALID_ARGUMENT, "the convolution's input may not overlap the output buffer");
+    }
     PendingAdd pending;
     pending.other = static_cast<const uint8_t*>(other_dev);
     pending.fuse.qa = MakeQIn(plan->d.output);

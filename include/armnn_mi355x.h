@@ -202,7 +202,11 @@ typedef struct {
 /* weights_host / bias_host are read once and may be released after the call returns.
  * Weight scales index the OUTPUT channel (quantization dim 0 for conv, 3 for depthwise); bias scales index
  * the output channel; with n_scales == 1 the single scale applies to all channels.  bias quantization is
- * NOT assumed to equal input_scale * weight_scale. */
+ * NOT assumed to equal input_scale * weight_scale.
+ * Limit: the kernels accumulate sum (x - zx)(w - zw) exactly in 32 bits; a plan whose K taps per output could overflow
+ * that (K * max|x - zx| * max|w - zw| >= 2^31 with the given zero points and weights; never below K = 33 026) is refused
+ * with MI355X_ERR_UNSUPPORTED.  The same holds for mi355x_fc_create with K = input features.
+ * Filters of more than 32 taps over a multiple of 128 channels never run on the 256-row tiles (they take smaller ones). */
 int mi355x_conv2d_create(const mi355x_conv2d_desc* desc,
                          const void* weights_host, const mi355x_const_quant* weights_quant,
                          const int32_t* bias_host, const mi355x_const_quant* bias_quant,
@@ -221,7 +225,9 @@ int mi355x_conv2d_set_concurrency(mi355x_conv2d_t plan, uint32_t lanes);
  * sum_quant, activation, a, b: the Addition's output quantization and the activation fused into it.  The convolution's
  * own output codes are formed first and then added exactly as the Addition layer adds (dequantize both inputs, one
  * fp32 addition, quantize), so the bytes are those of mi355x_conv2d_run followed by mi355x_add_run -- in the reference
- * these are two workloads in sequence (RefConvolution2dWorkload.cpp:38-58, then RefElementwiseBinaryWorkload.cpp:27-107). */
+ * these are two workloads in sequence (RefConvolution2dWorkload.cpp:38-58, then RefElementwiseBinaryWorkload.cpp:27-107).
+ * output_dev may share no byte with input_dev or other_dev (one launch reads both while it writes the sum): overlapping
+ * buffers are refused with MI355X_ERR_INVALID_ARGUMENT. */
 int mi355x_conv2d_run_add(mi355x_conv2d_t plan, uint32_t batch, const void* input_dev, const void* other_dev,
                           const mi355x_quant* other_quant, const mi355x_quant* sum_quant, int32_t activation, float a, float b,
                           void* output_dev, mi355x_stream_t stream);

@@ -88,6 +88,11 @@ def test_mobilenet_v1_batch1(port):
     _layerwise(port, nets.mobilenet_v1(), 1)
 
 
+def test_resnet50_224_batch2(port):
+    # what the batch-32 property test compares its rows with
+    _layerwise(port, nets.resnet50(), 2)
+
+
 def test_resnet50_224_batch1(port):
     # full resolution against the CPU checker: what the batch-32 row-equality test below chains to
     _layerwise(port, nets.resnet50(), 1)

@@ -281,6 +281,69 @@ def test_large_tile_gemm_gives_the_same_bytes():
         np.testing.assert_array_equal(got.data, want.data, err_msg=f"fc tile {tile}")
 
 
+def test_filters_of_more_than_32_taps_stay_off_the_large_tile_kernel():
+    """The large-tile kernel walks at most 32 taps; a 7 x 7 or 6 x 6 convolution over a multiple of 128 channels must run
+    on the other tiles -- when a test forces the large tile and when a launch that fills the device would choose it."""
+    small = cases.make_conv_case("taps49_c128", 641, n=2, h=15, w=17, ci=128, co=256, kh=7, kw=7, act=cases.RELU)
+    six = cases.make_conv_case("taps36_c256", 642, n=1, h=12, w=12, ci=256, co=128, kh=6, kw=6, padding=(2, 3, 2, 3))
+    for c in (small, six):
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        for tile in (2256, 2128, 0):
+            shim.set_option("igemm_tile", tile)
+            try:
+                got = _gpu_conv(c, shim.ALGO_MFMA)
+                kernel = shim.last_kernel()
+            finally:
+                shim.set_option("igemm_tile", 0)
+            assert not kernel.startswith("BigGemmKernel"), kernel
+            np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} tile {tile} {kernel}")
+    # 8 x 60 x 60 rows over 256 channels: 226 tiles of 256 x 128, which a filter of up to 32 taps would run on the large tile
+    big = cases.make_conv_case("taps49_c128_fills_device", 643, n=8, h=60, w=60, ci=128, co=256, kh=7, kw=7, act=cases.RELU6)
+    got = _gpu_conv(big, shim.ALGO_AUTO)
+    kernel = shim.last_kernel()
+    print(f"{big.name}: {kernel}", flush=True)
+    assert not kernel.startswith("BigGemmKernel"), kernel
+    np.testing.assert_array_equal(got.data, _gpu_conv(big, shim.ALGO_DIRECT).data)
+    same = cases.make_conv_case("taps9_c128_fills_device", 644, n=8, h=120, w=120, ci=128, co=256, stride=(2, 2), act=cases.RELU6)
+    _gpu_conv(same, shim.ALGO_AUTO)
+    assert shim.last_kernel().startswith("BigGemmKernel"), shim.last_kernel()
+
+
+def test_specialised_kernels_equal_the_exact_division():
+    """Every specialised kernel is otherwise compared with the direct kernel, which shares the bracket constants.  Here each
+    one runs layers whose bias term is hundreds of codes and whose offsets are far from zero -- wide brackets, saturation on
+    both sides -- against the same kernel with the fp32 division of armnn::Quantize forced for every output."""
+    U8, S8 = DataType.QAsymmU8, DataType.QAsymmS8
+    big_bias = dict(in_scale=0.5, w_scale_range=(0.01, 0.03), out_scale=0.04)          # |bias * s_in * s_w / s_out| up to some hundreds
+    runs = [
+        (cases.make_conv_case("xd_ksplit", 901, n=2, h=7, w=7, ci=512, co=128, out_offset=100, **big_bias), 4064, None),
+        (cases.make_conv_case("xd_ksplit2_u8", 902, n=2, h=14, w=14, ci=256, co=192, in_dtype=U8, in_offset=131, out_dtype=U8, out_offset=250, **big_bias), 2064, None),
+        (cases.make_conv_case("xd_halo", 903, n=4, h=23, w=19, ci=64, co=64, out_offset=-100, act=cases.RELU, **big_bias), 3000, None),
+        (cases.make_conv_case("xd_big", 904, n=2, h=29, w=31, ci=128, co=256, stride=(2, 2), out_offset=60, **big_bias), 2256, None),
+        (cases.make_conv_case("xd_big_1x1", 905, n=3, h=14, w=14, ci=256, co=512, kh=1, kw=1, out_offset=-77, act=cases.RELU6, **big_bias), 2128, None),
+        (cases.make_conv_case("xd_lds64", 906, n=3, h=14, w=14, ci=512, co=512, kh=1, kw=1, in_dtype=U8, in_offset=3, out_dtype=U8, out_offset=5, **big_bias), 64, None),
+        (cases.make_conv_case("xd_dw128", 907, n=3, h=14, w=14, ci=256, depthwise=True, in_dtype=U8, in_offset=128, out_dtype=U8, out_offset=200,
+                              in_scale=0.5, w_scale_range=(0.01, 0.05), out_scale=0.05), 0, shim.ALGO_DEPTHWISE),
+        (cases.make_conv_case("xd_dw64_s2", 908, n=2, h=29, w=31, ci=192, depthwise=True, stride=(2, 2), out_offset=-120, in_scale=0.5,
+                              w_scale_range=(0.01, 0.05), out_scale=0.05, act=cases.RELU), 0, shim.ALGO_DEPTHWISE),
+    ]
+    for c, tile, algo in runs:
+        got = {}
+        for exact in (0, 1):
+            shim.set_option("igemm_tile", tile)
+            shim.set_option("exact_division_epilogue", exact)
+            try:
+                got[exact] = _gpu_conv(c, algo if algo is not None else shim.ALGO_MFMA)
+                kernel = shim.last_kernel()
+            finally:
+                shim.set_option("igemm_tile", 0)
+                shim.set_option("exact_division_epilogue", 0)
+        codes = np.unique(got[1].data)
+        print(f"{c.name}: {kernel}, {len(codes)} distinct codes from {codes.min()} to {codes.max()}", flush=True)
+        assert len(codes) > 20, c.name                       # not saturated to a handful of values
+        np.testing.assert_array_equal(got[0].data, got[1].data, err_msg=f"{c.name} {kernel}")
+
+
 def test_depthwise_rows_per_thread_variants_give_the_same_bytes():
     """The 3x3 depthwise kernel with one and with two output rows per thread (8- and 16-row tiles), forced on feature maps
     of every parity of height, against the plain depthwise kernel."""
@@ -525,7 +588,7 @@ def test_random_convolutions(port, chunk):
         auto = _gpu_conv(case, shim.ALGO_AUTO)
         mx, exact = lsb_diff(auto.data, want.data)
         assert mx <= 1, (k, mx)
-        assert exact >= 0.98 or auto.data.size < 200, (k, exact)
+        assert exact >= 0.995 or auto.data.size < 200, (k, exact)
         direct = _gpu_conv(case, shim.ALGO_DIRECT)
         np.testing.assert_array_equal(auto.data, direct.data, err_msg=f"random case {k}")
 
@@ -567,7 +630,7 @@ def test_random_draws_from_the_specialised_kernels_shapes(port, chunk):
         auto = _gpu_conv(case, shim.ALGO_AUTO)
         mx, exact = lsb_diff(auto.data, want.data)
         assert mx <= 1, (k, mx)
-        assert exact >= 0.98, (k, exact)
+        assert exact >= 0.995, (k, exact)
         direct = _gpu_conv(case, shim.ALGO_DIRECT)
         np.testing.assert_array_equal(auto.data, direct.data, err_msg=f"fast-path case {k}")
 
@@ -593,7 +656,7 @@ def test_random_fully_connected(port, chunk):
         auto = shim.fully_connected(case.x, case.w, case.b, case.out_info, algo=shim.ALGO_AUTO, **kw)
         mx, exact = lsb_diff(auto.data, want.data)
         assert mx <= 1, (k, mx)
-        assert exact >= 0.98 or auto.data.size < 200, (k, exact)
+        assert exact >= 0.995 or auto.data.size < 200, (k, exact)
         direct = shim.fully_connected(case.x, case.w, case.b, case.out_info, algo=shim.ALGO_DIRECT, **kw)
         np.testing.assert_array_equal(auto.data, direct.data, err_msg=f"fc case {k}")
 
