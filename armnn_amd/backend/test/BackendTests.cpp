@@ -142,16 +142,16 @@ TEST_CASE("layer support: the accepted envelope and the reasons outside it", "cp
         TensorInfo wideOut({1, 1, 1, 8}, DataType::QAsymmS8, 0.1f, 5);
         Convolution2dDescriptor plain;
         plain.m_DataLayout = DataLayout::NHWC;
-        CHECK(!ls.IsLayerSupported(LayerType::Convolution2d, {wideIn, wideOut, wideW}, plain, EmptyOptional(), EmptyOptional(), reason));
+        CHECK(!ls.IsLayerSupported(LayerType::Convolution2d, {wideIn, wideOut, wideW, TensorInfo()}, plain, EmptyOptional(), EmptyOptional(), reason));
         CHECK(why.find("33 025 taps") != std::string::npos);
         TensorInfo okIn({1, 1, 1, 33025}, DataType::QAsymmS8, 0.05f, -3), okW({8, 1, 1, 33025}, DataType::QSymmS8, 0.01f, 0);
         okW.SetConstant(true);
-        CHECK(ls.IsLayerSupported(LayerType::Convolution2d, {okIn, wideOut, okW}, plain, EmptyOptional(), EmptyOptional(), reason));
+        CHECK(ls.IsLayerSupported(LayerType::Convolution2d, {okIn, wideOut, okW, TensorInfo()}, plain, EmptyOptional(), EmptyOptional(), reason));
         TensorInfo fcIn({2, 40000}, DataType::QAsymmS8, 0.05f, -3), fcW({40000, 8}, DataType::QSymmS8, 0.01f, 0), fcOut({2, 8}, DataType::QAsymmS8, 0.1f, 5);
         fcW.SetConstant(true);
         FullyConnectedDescriptor fd;
         fd.m_BiasEnabled = false;
-        CHECK(!ls.IsLayerSupported(LayerType::FullyConnected, {fcIn, fcOut, fcW}, fd, EmptyOptional(), EmptyOptional(), reason));
+        CHECK(!ls.IsLayerSupported(LayerType::FullyConnected, {fcIn, fcOut, fcW, TensorInfo()}, fd, EmptyOptional(), EmptyOptional(), reason));
         CHECK(why.find("33 025 taps") != std::string::npos);
     }
 
