@@ -4,6 +4,7 @@
 #include "conv_kernels.h"
 #include "dw_stem_kernels.h"
 #include "dwpw_kernel.h"
+#include "dwpw_panel_kernel.h"
 #include "pwdw_kernel.h"
 #include "igemm_ksplit_kernel.h"
 #include "pw_gemm_kernel.h"
@@ -1189,6 +1190,90 @@ int LaunchDwPw(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, uint32_t ba
     return 0;
 }
 
+// ---- depthwise 3x3 stride 1 + pointwise over 256 / 512 channels: one block per 8 x 8 tile over all channels ---------------
+// KT = channels between the layers / 128, NQ = output channels / 256; 0 when the pair does not fit that kernel
+bool DwPwPanelShape(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, int* kt, int* nq)
+{
+    const mi355x_conv2d_desc& a = dw->d;
+    if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || dw->w_dot4b || a.stride_x != 1 || a.stride_y != 1) return false;
+    if (a.out_c != a.in_c || (a.out_c != 256 && a.out_c != 512)) return false;
+    if (pw->zw_neg != 0 || pw->K_pad != static_cast<int>(a.out_c) || !pw->bk128 || !pw->w_mfma || pw->pw_bn != 0) return false;
+    if (pw->d.out_c != 256 && pw->d.out_c != 512) return false;
+    if (static_cast<long long>(a.in_h) * a.in_w * a.in_c >= (1ll << 31)) return false;
+    *kt = static_cast<int>(a.out_c) / 128;
+    *nq = static_cast<int>(pw->d.out_c) / 256;
+    return true;
+}
+
+template <int KT, int NQ>
+int LaunchDwPwPanelT(const DwPwPanelArgs& a, hipStream_t stream)
+{
+    constexpr int smem = DwPwPanelGeom<KT, NQ>::SMEM;
+    static_assert(smem <= 156 * 1024, "LDS of one CU");
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&DwPwPanelKernel<KT, NQ>), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    MI355X_HIP(attr);
+    NoteKernel("DwPwPanelKernel<%d, %d>", KT, NQ);
+    hipLaunchKernelGGL((DwPwPanelKernel<KT, NQ>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(512), smem, stream, a);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+int LaunchDwPwPanel(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, int kt, int nq, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    const ConvGeom& g = dw->geom;
+    DwPwPanelArgs a;
+    a.x = static_cast<const uint8_t*>(x); a.pad16 = dw->pad16; a.wpack = dw->w_dot4; a.dw_ct = ChanTab{dw->chan, dw->Co_pad}; a.dw_corr = dw->corr;
+    a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.C = g.Co; a.Ho = g.Ho; a.Wo = g.Wo;
+    a.pad_top = g.pad_top; a.pad_left = g.pad_left;
+    a.tiles_x = (g.Wo + 7) / 8; a.tiles_y = (g.Ho + 7) / 8;
+    const long long nb = static_cast<long long>(batch) * a.tiles_x * a.tiles_y;
+    if (nb > 0x7fffffffll - 8) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
+    a.total_tiles = static_cast<int>(nb); a.xcd_chunk = static_cast<int>((nb + 7) / 8);
+    a.dw_xor = dw->xor_mask; a.dw_rq = dw->rq;
+    a.w = pw->w_mfma; a.K_pad = pw->K_pad; a.pw_ct = ChanTab{pw->chan, pw->Co_pad}; a.pw_corr = pw->corr;
+    a.y = static_cast<uint8_t*>(y); a.Co = pw->geom.Co; a.mid_xor = pw->xor_mask; a.pw_rq = pw->rq;
+#ifdef MI355X_DWPW_STAMPS
+    // measurement build: the first 40 launches record wave 0's shader-clock stamps per block and print the average durations
+    // between consecutive stamps, over all blocks
+    static unsigned long long* d_stamps = nullptr;
+    static int launches = 0;
+    a.stamps = nullptr;
+    if (launches < 40)
+    {
+        if (!d_stamps) MI355X_HIP(hipMalloc(reinterpret_cast<void**>(&d_stamps), 65536 * 16 * 8));
+        a.stamps = a.total_tiles <= 65536 - 8 ? d_stamps : nullptr;
+    }
+    int rc = kt == 2 ? (nq == 1 ? LaunchDwPwPanelT<2, 1>(a, stream) : LaunchDwPwPanelT<2, 2>(a, stream))
+                     : (nq == 1 ? LaunchDwPwPanelT<4, 1>(a, stream) : LaunchDwPwPanelT<4, 2>(a, stream));
+    if (a.stamps && rc == 0 && ++launches == 40)
+    {
+        MI355X_HIP(hipStreamSynchronize(stream));
+        const int nblk = a.xcd_chunk * 8;
+        std::vector<unsigned long long> h(static_cast<size_t>(nblk) * 16);
+        MI355X_HIP(hipMemcpy(h.data(), d_stamps, h.size() * 8, hipMemcpyDeviceToHost));
+        const int ns = 3 + 3 * kt + 1;
+        std::vector<double> sum(ns, 0.0);
+        int used = 0;
+        unsigned long long tmin = ~0ull, tmax = 0;
+        for (int b = 0; b < a.total_tiles; ++b)
+        {
+            const unsigned long long* s = &h[static_cast<size_t>(b) * 16];
+            if (s[0] == 0) continue;
+            ++used;
+            for (int i = 1; i < ns; ++i) sum[i] += static_cast<double>(s[i] - s[i - 1]);
+            tmin = std::min(tmin, s[0]); tmax = std::max(tmax, s[ns - 1]);
+        }
+        std::fprintf(stderr, "DwPwPanelKernel<%d, %d> stamps over %d blocks (cycles): prologue %.0f", kt, nq, used, sum[1] / used);
+        for (int k = 0; k < kt; ++k) std::fprintf(stderr, " | dw%d %.0f wait %.0f gemm %.0f", k, sum[2 + 3 * k] / used, sum[3 + 3 * k] / used, sum[4 + 3 * k] / used);
+        std::fprintf(stderr, " | requant %.0f stores %.0f | first start to last end %llu\n", sum[2 + 3 * kt] / used, sum[3 + 3 * kt] / used, tmax - tmin);
+    }
+    return rc;
+#else
+    if (kt == 2) return nq == 1 ? LaunchDwPwPanelT<2, 1>(a, stream) : LaunchDwPwPanelT<2, 2>(a, stream);
+    return nq == 1 ? LaunchDwPwPanelT<4, 1>(a, stream) : LaunchDwPwPanelT<4, 2>(a, stream);
+#endif
+}
+
 // ---- pointwise 1x1 followed by depthwise 3x3, whole images per block ---------------------------------------------------
 constexpr int kPwDwMF = 7;       // 224 pixel rows per block: one 14x14 image, four 7x7 images
 // Two LDS stages and eight waves: with a K of 256 .. 512 bytes the k-loop is bound by what a CU's vector L1 delivers, not
@@ -1417,6 +1502,19 @@ int mi355x_conv2d_fusable(mi355x_conv2d_t dw, mi355x_conv2d_t pw)
     return 0;
 }
 
+int mi355x_conv2d_fusion_pays(mi355x_conv2d_t first, mi355x_conv2d_t second, uint32_t batch)
+{
+    if (!first || !second || batch == 0) return 0;
+    if (!first->d.depthwise || second->d.depthwise) return 0;
+    int kt = 0, nq = 0;
+    if (GlobalOptions().dwpw_panel == 0 || !DwPwPanelShape(first, second, &kt, &nq)) return 0;
+    if (mi355x_conv2d_fusable(first, second) != 0) return 0;
+    // a block takes a CU to itself: below about a hundred tiles per launch most of the device would idle (measured on
+    // MobileNetV1: a gain at 32 images per launch, a loss at 16)
+    const long long tiles = static_cast<long long>(batch) * ((first->d.out_w + 7) / 8) * ((first->d.out_h + 7) / 8);
+    return tiles >= 100 ? 1 : 0;
+}
+
 int mi355x_conv2d_run_fused(mi355x_conv2d_t dw, mi355x_conv2d_t pw, uint32_t batch, const void* input_dev, void* output_dev,
                             mi355x_stream_t stream)
 {
@@ -1430,6 +1528,10 @@ int mi355x_conv2d_run_fused(mi355x_conv2d_t dw, mi355x_conv2d_t pw, uint32_t bat
         PwDwShape sh;
         if (int rc = PwDwCheck(dw, pw, &sh)) return rc;
         return LaunchPwDw(dw, pw, sh, batch, input_dev, output_dev, ToHip(stream));
+    }
+    {
+        int kt = 0, nq = 0;
+        if (GlobalOptions().dwpw_panel != 0 && DwPwPanelShape(dw, pw, &kt, &nq)) return LaunchDwPwPanel(dw, pw, kt, nq, batch, input_dev, output_dev, ToHip(stream));
     }
     if (dw->d.stride_x == 2) return LaunchDwPw<2, 2>(dw, pw, batch, input_dev, output_dev, ToHip(stream));
     // stride 1: the wide tile (8 x 16 pixels) while it still yields two blocks per CU, else the narrow one (8 x 8)

@@ -56,7 +56,8 @@ class ChainedRun:
 
 class DeviceNetwork:
     def __init__(self, net: Network, batch: int, algo_overrides: Optional[Dict[str, int]] = None, use_graph: bool = True,
-                 fuse: bool = False, lanes: int = 1, fuse_add: bool = True, chain: bool = False, lanes_after_chain: bool = False):
+                 fuse: bool = False, lanes: int = 1, fuse_add: bool = True, chain: bool = False, lanes_after_chain: bool = False,
+                 join_for_fused: bool = False):
         """chain: runs of consecutive layers the library accepts (mi355x_chain_accepts) become one persistent launch over
         the whole batch; with lanes > 1 the lanes join in front of such a run and, if lanes_after_chain, fork again behind it
         (else the rest of the network runs on one stream).
@@ -77,6 +78,7 @@ class DeviceNetwork:
         self.plans = []
         self.chains: List = []
         self.lanes_after_chain = lanes_after_chain
+        self.join_for_fused = join_for_fused      # fused pairs run on the whole batch: the lanes join in front of the first one
         self.graph = None
         self.use_graph = use_graph
         algo_overrides = algo_overrides or {}
@@ -141,6 +143,9 @@ class DeviceNetwork:
         self._plan_of = {id(l): pl for (l, _), pl in zip(self.steps, self._step_plans)}
         if fuse in ("dwpw", "pwdw", True):
             self._fuse_pairs(("conv", "depthwise") if fuse == "pwdw" else ("depthwise", "conv"))
+        elif fuse == "auto":
+            # only the pairs the library recommends as one launch at the batch a launch sees
+            self._fuse_pairs(("depthwise", "conv"), only_where_it_pays=True)
         if fuse_add:
             self._fuse_additions()
         if chain:
@@ -183,7 +188,7 @@ class DeviceNetwork:
             k += len(run)
         self.steps = out
 
-    def _fuse_pairs(self, ops):
+    def _fuse_pairs(self, ops, only_where_it_pays=False):
         """Replace neighbours (depthwise 3x3, 1x1 convolution) -- or, with ops = ("conv", "depthwise"), (1x1 convolution,
         depthwise 3x3) -- by one fused launch where the library accepts the pair and nothing else reads the tensor
         between them."""
@@ -199,14 +204,19 @@ class DeviceNetwork:
             nxt = self.steps[k + 1][0] if k + 1 < len(self.steps) else None
             if (l.op == ops[0] and nxt is not None and nxt.op == ops[1] and nxt.inputs[0] == l.output and
                     consumers.get(l.output, 0) == 1 and l.output != net.output and
-                    plan_of[id(l)].fusable_with(plan_of[id(nxt)])):
+                    plan_of[id(l)].fusable_with(plan_of[id(nxt)]) and
+                    (not only_where_it_pays or plan_of[id(l)].fusion_pays(plan_of[id(nxt)], self.batch if self.join_for_fused else self.batch // self.lanes))):
                 pdw, ppw = plan_of[id(l)], plan_of[id(nxt)]
                 x, y = self.buffers[l.inputs[0]].ptr, self.buffers[nxt.output].ptr
                 nx, ny = net.info(l.inputs[0], self.batch).num_elements, net.info(nxt.output, self.batch).num_elements
                 batch = self.batch
-                fused.append((FusedPair(f"{l.name}+{nxt.name}", (l, nxt)),
-                              (lambda pdw, ppw, x, y, nx, ny: lambda s, lane=0, lanes=1: pdw.run_fused(
-                                  ppw, batch // lanes, x + lane * (nx // lanes), y + lane * (ny // lanes), s))(pdw, ppw, x, y, nx, ny)))
+                if self.join_for_fused and self.lanes > 1:
+                    fn2 = (lambda pdw, ppw, x, y: lambda s, lane=0, lanes=1: pdw.run_fused(ppw, batch, x, y, s))(pdw, ppw, x, y)
+                    fn2.whole_batch = True
+                else:
+                    fn2 = (lambda pdw, ppw, x, y, nx, ny: lambda s, lane=0, lanes=1: pdw.run_fused(
+                        ppw, batch // lanes, x + lane * (nx // lanes), y + lane * (ny // lanes), s))(pdw, ppw, x, y, nx, ny)
+                fused.append((FusedPair(f"{l.name}+{nxt.name}", (l, nxt)), fn2))
                 k += 2
             else:
                 fused.append((l, fn))

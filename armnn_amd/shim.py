@@ -28,7 +28,7 @@ EXPORTS = [
     "mi355x_event_destroy", "mi355x_event_record", "mi355x_stream_wait_event", "mi355x_event_synchronize", "mi355x_event_elapsed_ms",
     "mi355x_graph_capture_begin", "mi355x_graph_capture_end", "mi355x_graph_launch", "mi355x_graph_destroy",
     "mi355x_conv2d_create", "mi355x_conv2d_run", "mi355x_conv2d_destroy", "mi355x_conv2d_algo",
-    "mi355x_conv2d_fusable", "mi355x_conv2d_run_fused", "mi355x_conv2d_run_add", "mi355x_conv2d_set_concurrency",
+    "mi355x_conv2d_fusable", "mi355x_conv2d_fusion_pays", "mi355x_conv2d_run_fused", "mi355x_conv2d_run_add", "mi355x_conv2d_set_concurrency",
     "mi355x_chain_accepts", "mi355x_chain_create", "mi355x_chain_run", "mi355x_chain_status", "mi355x_chain_info", "mi355x_chain_run_stamped", "mi355x_chain_run_noalloc", "mi355x_chain_destroy",
     "mi355x_fc_create", "mi355x_fc_run", "mi355x_fc_destroy", "mi355x_fc_algo",
     "mi355x_activation_run", "mi355x_pool2d_run", "mi355x_add_run", "mi355x_softmax_run", "mi355x_pad_run",
@@ -112,7 +112,7 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
             "mi355x_conv2d_create": [C.POINTER(Conv2dDesc), V, C.POINTER(ConstQuant), V, C.POINTER(ConstQuant), C.POINTER(V)],
             "mi355x_conv2d_run": [V, C.c_uint32, V, V, V], "mi355x_conv2d_destroy": [V],
             "mi355x_conv2d_algo": [V, C.POINTER(C.c_int32), C.c_char_p, C.c_size_t],
-            "mi355x_conv2d_fusable": [V, V], "mi355x_conv2d_run_fused": [V, V, C.c_uint32, V, V, V],
+            "mi355x_conv2d_fusable": [V, V], "mi355x_conv2d_fusion_pays": [V, V, C.c_uint32], "mi355x_conv2d_run_fused": [V, V, C.c_uint32, V, V, V],
             "mi355x_conv2d_run_add": [V, C.c_uint32, V, V, C.POINTER(Quant), C.POINTER(Quant), C.c_int32, C.c_float, C.c_float, V, V],
             "mi355x_conv2d_set_concurrency": [V, C.c_uint32],
             "mi355x_chain_accepts": [V, C.c_uint32],
@@ -310,6 +310,10 @@ class Conv2dPlan:
         """True when this plan and `second`, the layer consuming its output, can run as one kernel: 3x3 depthwise + 1x1
         convolution, or 1x1 convolution + 3x3 depthwise over images of at most 224 pixels."""
         return self.lib.mi355x_conv2d_fusable(self.plan, second.plan) == 0
+
+    def fusion_pays(self, second: "Conv2dPlan", batch: int) -> bool:
+        """True when the library recommends running this plan and `second` as one launch at this batch."""
+        return self.lib.mi355x_conv2d_fusion_pays(self.plan, second.plan, batch) == 1
 
     def run_fused(self, second: "Conv2dPlan", batch: int, x_dev: int, y_dev: int, stream=None):
         """Both layers without the intermediate tensor; bytes equal run() + second.run()."""

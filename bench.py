@@ -227,9 +227,10 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-backend", action="store_true", help="skip the run through the C++ backend (config.backend_path)")
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--fuse", nargs="?", const="dwpw", default="", choices=("dwpw", "pwdw"),
-                    help="run pairs of layers as one kernel (same bytes): 'dwpw' depthwise + the pointwise after it, 'pwdw' "
-                         "pointwise + the depthwise after it where whole images fit a block")
+    ap.add_argument("--fuse", default="auto", choices=("auto", "none", "dwpw", "pwdw"),
+                    help="pairs of layers as one kernel (same bytes): 'auto' the depthwise + pointwise pairs the library recommends at "
+                         "the batch a launch sees (mi355x_conv2d_fusion_pays), 'none' every layer a launch of its own, 'dwpw' every "
+                         "depthwise + pointwise pair the fused kernels accept, 'pwdw' pointwise + the depthwise after it where whole images fit a block")
     ap.add_argument("--no-fuse-add", action="store_true",
                     help="launch a residual Addition on its own instead of inside the convolution that feeds it")
     ap.add_argument("--lanes", type=int, default=0,
@@ -265,7 +266,7 @@ def main():
 
     if args.lanes == 0:
         args.lanes = 2 if batch >= 16 and batch % 2 == 0 else 1
-    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse=args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add, chain=args.chain)
+    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse="" if args.fuse == "none" else args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add, chain=args.chain)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev
 
@@ -377,17 +378,27 @@ def main():
         return {"ms": t * 1e3, "achieved": w / t, "frac": w / t / peak} if t > 0 else None
 
     g_conv = group(("conv", "fc", "convadd"), INT8_MFMA_PEAK_OPS)
-    g_dw = group(("depthwise", "dwpw"), HBM_PEAK_BYTES)
+    g_dw = group(("depthwise",), HBM_PEAK_BYTES)
     groups = {
         "conv_fc": {"ms": g_conv["ms"], "TOPS": g_conv["achieved"] / 1e12, "frac_of_int8_mfma_peak": g_conv["frac"]},
     }
     if g_dw:
         groups["depthwise"] = {"ms": g_dw["ms"], "GBps": g_dw["achieved"] / 1e9, "frac_of_hbm_peak": g_dw["frac"]}
+    fused_rows = [r for r in rows if r["op"] == "dwpw"]
+    if fused_rows:
+        # depthwise + pointwise pairs that ran as one launch belong to neither group above: their time buys both the pointwise
+        # layer's ops and the pair's bytes (input, output, constants; the tensor between the layers never exists)
+        t = sum(r["ms"] for r in fused_rows) * 1e-3
+        by_name = {l.name: l for l, _, _ in per_layer}
+        ops = sum(2.0 * by_name[r["layer"]].parts[1].macs_per_image * launch_batch for r in fused_rows)
+        nbytes = sum(r["work"] for r in fused_rows)
+        groups["fused_depthwise_pointwise"] = {"ms": t * 1e3, "launches": len(fused_rows), "TOPS": ops / t / 1e12, "frac_of_int8_mfma_peak": ops / t / INT8_MFMA_PEAK_OPS,
+                                               "GBps": nbytes / t / 1e9, "frac_of_hbm_peak": nbytes / t / HBM_PEAK_BYTES}
 
     config = {"workload": f"{net.name} int8 (QAsymm activations, {'per-channel QSymmS8' if args.weights == 'per_channel_s8' or args.net != 'mobilenet_v1' else 'per-tensor QAsymmU8'} weights), batch {batch}, "
                           f"random-init, whole forward pass incl. avgpool/FC/softmax, input resident in HBM, every layer through the C ABI, "
                           f"one HIP graph replay per step",
-              "batch": batch, "graph_replay": not args.no_graph, "fused_pairs": args.fuse or None, "additions_inside_convolutions": not args.no_fuse_add, "lanes": args.lanes,
+              "batch": batch, "graph_replay": not args.no_graph, "fused_pairs": [l.name for l, _ in dn.steps if l.op == "dwpw"] or None, "additions_inside_convolutions": not args.no_fuse_add, "lanes": args.lanes,
               "layer_chains": [l.name for l, _ in dn.steps if l.op == "chain"] or None,
               "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12}
     if backend is not None:

@@ -113,6 +113,9 @@ int  mi355x_abi_version(void);
  *   bytes; tests and tuning).
  *   "dw_cb" = 0 | 32: channels per block of the 3x3 depthwise kernel (0: 128 where the channel count is a multiple of
  *   128, else 32; 32: always 32; identical bytes).
+ *   "dwpw_panel" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a stride-1 depthwise layer of 256 or 512
+ *   channels and a pointwise layer of 256 or 512 output channels on the kernel that gives a block an 8 x 8 pixel tile over
+ *   all channels (identical bytes; lets tests compare it with the older fused kernel).
  *   "chain_stages" = 2 | 3 | 4: LDS stages of the matrix-core tiles inside a layer chain; "chain_blocks_per_cu" = 0 .. 16:
  *   persistent blocks per CU of a layer chain (0: as many as fit); "chain_panel" = 0 | 1: 1x1 convolutions with 256 or 512
  *   input channels and at least 96 row blocks run as one work item per 64 output rows with the activation panel resident
@@ -245,6 +248,11 @@ int mi355x_conv2d_run_add(mi355x_conv2d_t plan, uint32_t batch, const void* inpu
  * pixels (14 x 14, 7 x 7 ...), the 1x1 layer's input channels are a multiple of 128, its weights have no zero point and
  * the shared channel count is a multiple of 64.  Same contract: the bytes of the two layers run one after the other. */
 int mi355x_conv2d_fusable(mi355x_conv2d_t first, mi355x_conv2d_t second);
+/* 1 when running the pair as one launch is what the library recommends at this batch (today: a stride-1 depthwise layer
+ * over 256 or 512 channels and the pointwise layer of 256 or 512 output channels behind it, which run on the kernel that
+ * gives a block an 8 x 8 pixel tile over all channels), else 0; never an error.  No counterpart in the reference, which
+ * has no fused workloads on CpuRef. */
+int mi355x_conv2d_fusion_pays(mi355x_conv2d_t first, mi355x_conv2d_t second, uint32_t batch);
 int mi355x_conv2d_run_fused(mi355x_conv2d_t first, mi355x_conv2d_t second, uint32_t batch,
                             const void* input_dev, void* output_dev, mi355x_stream_t stream);
 /* A run of consecutive layers as one persistent launch ("chain").  plans[k] reads the output of plans[k - 1] (plans[0]

@@ -25,6 +25,16 @@ PAIRS = [
 ]
 
 
+# pairs the one-block-per-tile-over-all-channels kernel takes: stride 1, 256 or 512 channels in between, 256 or 512 out
+PANEL_PAIRS = [
+    ("panel_c512_co512_u8_14", 5, 14, 14, 512, 512, 1, U8, cases.RELU6, cases.RELU6),      # the MobileNetV1 pairs dw7+pw7 ... dw11+pw11
+    ("panel_c256_co256_u8_28", 3, 28, 28, 256, 256, 1, U8, cases.RELU6, cases.RELU6),      # dw5+pw5
+    ("panel_c256_co512_s8_ragged", 2, 13, 9, 256, 512, 1, S8, cases.RELU, (0, 0.0, 0.0)),
+    ("panel_c512_co256_s8_tiny", 1, 3, 5, 512, 256, 1, S8, (0, 0.0, 0.0), cases.RELU6),
+    ("panel_c512_co512_s8_17x23", 2, 17, 23, 512, 512, 1, S8, cases.RELU6, cases.RELU),
+]
+
+
 def _make(name, n, h, w, c, co, stride, dt, act_dw, act_pw):
     zp_in = 120 if dt == U8 else -8
     zp_mid = 0 if dt == U8 else -128
@@ -42,7 +52,28 @@ def _plan(c):
     return shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, activation=fn, act_a=a, act_b=b, **c.params)
 
 
-@pytest.mark.parametrize("pair", PAIRS, ids=[p[0] for p in PAIRS])
+@pytest.mark.parametrize("pair", PANEL_PAIRS, ids=[p[0] for p in PANEL_PAIRS])
+def test_panel_kernel_is_taken_and_equals_the_older_fused_kernel(pair):
+    shim.Device()
+    dw, pw = _make(*pair)
+    pdw, ppw = _plan(dw), _plan(pw)
+    n = dw.x.info.shape[0]
+    xd = shim.DeviceBuffer(dw.x.data.nbytes).upload(dw.x.data)
+    ya, yb = shim.DeviceBuffer(pw.out_info.num_elements), shim.DeviceBuffer(pw.out_info.num_elements)
+    pdw.run_fused(ppw, n, xd.ptr, ya.ptr)
+    assert shim.last_kernel().startswith("DwPwPanelKernel<"), shim.last_kernel()
+    shim.set_option("dwpw_panel", 0)
+    try:
+        pdw.run_fused(ppw, n, xd.ptr, yb.ptr)
+        assert shim.last_kernel().startswith("DwPwKernel<"), shim.last_kernel()
+    finally:
+        shim.set_option("dwpw_panel", 1)
+    a = ya.download(pw.out_info.shape, numpy_dtype(pw.out_info.dtype))
+    b = yb.download(pw.out_info.shape, numpy_dtype(pw.out_info.dtype))
+    np.testing.assert_array_equal(a, b)
+
+
+@pytest.mark.parametrize("pair", PAIRS + PANEL_PAIRS, ids=[p[0] for p in PAIRS + PANEL_PAIRS])
 def test_fused_equals_two_layers(port, pair):
     print("pair", pair, flush=True)
     shim.Device()
