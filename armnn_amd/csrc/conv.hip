@@ -99,6 +99,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
 
     p->d = d;
     p->opt_igemm_lds = GlobalOptions().igemm_lds;
+    p->opt_xcd_cols = GlobalOptions().igemm_xcd_cols;
     p->opt_dw_rows = GlobalOptions().dw_rows;
     p->opt_dw_cb = GlobalOptions().dw_cb;
     p->opt_stem_dot4 = GlobalOptions().stem_dot4;
@@ -659,8 +660,12 @@ int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, voi
         a.add = t_pending_add->fuse;
         t_pending_add->taken = true;
     }
-    const int nblocks = a.tiles_m * a.tiles_n;
-    const int grid = (nblocks + 7) / 8 * 8;
+    // XCD groups over the output channels where the weights outweigh a quarter of the activations a launch reads ("igemm_xcd_cols":
+    // 0 that rule, 1 never, 2 wherever the column tiles halve)
+    const long long w_bytes = static_cast<long long>(p->Co_pad) * a.K_pad, x_bytes = static_cast<long long>(a.M) * a.K_pad;
+    const int split = p->opt_xcd_cols;
+    if ((a.tiles_n & 1) == 0 && a.tiles_m >= 4 && (split == 2 || (split == 0 && 4 * w_bytes > x_bytes))) a.xcd_cols = 2;
+    const int grid = 8 * IgemmLdsBlocksPerXcd(a.tiles_m, a.tiles_n, a.xcd_cols);
     constexpr int smem = IgemmLdsSmemBytes<BM, BN, ST>();
     if constexpr (BM == 64 && BN == 64 && !AW)
     {

@@ -176,6 +176,9 @@ struct IgemmArgs
     int K_pad;
     int unit;               // 1x1 kernel, stride 1, no padding: H = 1, W = M describe the input as one row of pixels
     int tiles_m, tiles_n;
+    int xcd_cols = 1;       // direct-to-LDS kernel: XCD groups over the output channels (1: every XCD takes a range of row blocks over all
+                            // column tiles and so reads every weight; 2: XCDs 0-3 take the lower half of the column tiles, 4-7 the
+                            // upper half, each over a quarter of the row blocks: half the weights per XCD, every activation row twice)
     uint32_t xor_mask;      // 0x80808080 for uint8 input, else 0
     uint32_t pad_word;      // shifted input zero point replicated in 4 bytes
     int zw_neg;             // minus the zero point of the stored int8 weights (0: symmetric)

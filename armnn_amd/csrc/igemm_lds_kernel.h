@@ -386,16 +386,38 @@ __device__ __forceinline__ void IgemmLdsTile(const IgemmArgs& a, const int tile,
     }
 }
 
-// One tile per block; consecutive block ids are dealt round-robin to the 8 XCDs, so XCD x takes the contiguous range of
-// tiles [x * per_xcd, (x + 1) * per_xcd): the column tiles of a row block share an L2.
+// One tile per block; consecutive block ids are dealt round-robin to the 8 XCDs, each with an L2 of its own.
+//   xcd_cols == 1: XCD x takes the contiguous range of tiles [x * per_xcd, (x + 1) * per_xcd) in row-block-major order: the
+//   column tiles of a row block share an L2, an activation row is fetched by one XCD, every XCD fetches all weights.
+//   xcd_cols == 2 (even tiles_n): XCD x takes column half x >> 2 and the (x & 3)-th quarter of the row blocks: a weight is
+//   fetched by four XCDs instead of eight, an activation row by two instead of one -- less traffic where the weights
+//   outweigh a quarter of the activations.  The grid is 8 * IgemmLdsBlocksPerXcd() blocks either way.
+__host__ __device__ inline int IgemmLdsBlocksPerXcd(int tiles_m, int tiles_n, int xcd_cols)
+{
+    if (xcd_cols == 2) return ((tiles_m + 3) / 4) * (tiles_n / 2);
+    return (tiles_m * tiles_n + 7) / 8;
+}
+
 template <int BM, int BN, int WM, int WN, int ST, bool U8, bool AW = false, bool UNIT = false>
 __global__ __launch_bounds__(64 * WM * WN) void IgemmLdsKernel(IgemmArgs a)
 {
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];   // IgemmLdsSmemBytes<BM, BN, ST>()
-    const int nblocks = a.tiles_m * a.tiles_n;
-    const int per_xcd = (nblocks + 7) >> 3;
-    const int tile = static_cast<int>(blockIdx.x & 7) * per_xcd + static_cast<int>(blockIdx.x >> 3);
-    if (tile >= nblocks) return;
+    const int x = static_cast<int>(blockIdx.x & 7), i = static_cast<int>(blockIdx.x >> 3);
+    int tile;
+    if (a.xcd_cols == 2)
+    {
+        const int half = a.tiles_n >> 1, rows_per = (a.tiles_m + 3) >> 2;
+        const int tm = (x & 3) * rows_per + i / half;
+        if (i >= rows_per * half || tm >= a.tiles_m) return;
+        tile = tm * a.tiles_n + (x >> 2) * half + i % half;
+    }
+    else
+    {
+        const int nblocks = a.tiles_m * a.tiles_n;
+        const int per_xcd = (nblocks + 7) >> 3;
+        tile = x * per_xcd + i;
+        if (i >= per_xcd || tile >= nblocks) return;
+    }
     IgemmLdsTile<BM, BN, WM, WN, ST, U8, AW, UNIT>(a, tile, smem);
 }
 

@@ -143,6 +143,12 @@ int mi355x_set_option(const char* name, int value)
         GlobalOptions().chain_stages = value;
         return 0;
     }
+    if (std::strcmp(name, "igemm_xcd_cols") == 0)
+    {
+        if (value < 0 || value > 2) return SetError(MI355X_ERR_INVALID_ARGUMENT, "igemm_xcd_cols must be 0, 1 or 2");
+        GlobalOptions().igemm_xcd_cols = value;
+        return 0;
+    }
     if (std::strcmp(name, "dwpw_panel") == 0) { GlobalOptions().dwpw_panel = value != 0; return 0; }
     if (std::strcmp(name, "chain_defer_signal") == 0) { GlobalOptions().chain_defer_signal = value != 0; return 0; }
     if (std::strcmp(name, "chain_panel") == 0) { GlobalOptions().chain_panel = value != 0; return 0; }

@@ -239,6 +239,8 @@ def main():
     ap.add_argument("--chain", action="store_true",
                     help="runs of consecutive layers the library accepts (3x3 depthwise over multiples of 128 channels, 1x1 convolutions "
                          "over more than 128 input channels) as one persistent launch over the whole batch (same bytes)")
+    ap.add_argument("--option", action="append", default=[], metavar="NAME=VALUE",
+                    help="mi355x_set_option before any plan is created (tests and tuning), e.g. igemm_xcd_cols=1")
     ap.add_argument("--layers", action="store_true", help="print the per-layer table to stderr")
     ap.add_argument("--profile-pass", action="store_true",
                     help="for rocprofv3 --pmc: one 64 MiB calibration copy (1 B read + 1 B written per element), then ONE "
@@ -264,6 +266,9 @@ def main():
     from armnn_amd import shim
     from armnn_amd.executor import DeviceNetwork
 
+    for opt in args.option:
+        name, _, value = opt.partition("=")
+        shim.set_option(name, int(value))
     if args.lanes == 0:
         args.lanes = 2 if batch >= 16 and batch % 2 == 0 else 1
     dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse="" if args.fuse == "none" else args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add, chain=args.chain)

@@ -113,6 +113,10 @@ int  mi355x_abi_version(void);
  *   bytes; tests and tuning).
  *   "dw_cb" = 0 | 32: channels per block of the 3x3 depthwise kernel (0: 128 where the channel count is a multiple of
  *   128, else 32; 32: always 32; identical bytes).
+ *   "igemm_xcd_cols" = 0 | 1 | 2: how the direct-to-LDS implicit GEMM deals its tiles to the 8 XCDs (each has an L2 of its
+ *   own): 1 every XCD takes a range of row blocks over all output channels (each fetches every weight), 2 XCDs 0-3 take
+ *   the lower half of the output channels and XCDs 4-7 the upper half (half the weights per XCD, every activation row
+ *   fetched twice), 0 chooses 2 where the weights outweigh a quarter of the activations of a launch.  Identical bytes.
  *   "dwpw_panel" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a stride-1 depthwise layer of 256 or 512
  *   channels and a pointwise layer of 256 or 512 output channels on the kernel that gives a block an 8 x 8 pixel tile over
  *   all channels (identical bytes; lets tests compare it with the older fused kernel).

@@ -162,6 +162,30 @@ def test_every_igemm_tiling_gives_the_same_bytes():
         shim.set_option("igemm_tile", 100)
 
 
+def test_xcd_groups_over_the_output_channels_give_the_same_bytes():
+    """The direct-to-LDS implicit GEMM with its tiles dealt to the XCDs by row range only, and by channel half x row quarter:
+    forced both ways on ragged problems (odd and even numbers of column tiles, fewer row blocks than XCD groups, 3x3 and 1x1)."""
+    cs = [cases.make_conv_case("xcd_1x1_c512_co1024", 851, n=6, h=7, w=7, ci=512, co=1024, kh=1, kw=1, in_dtype=DataType.QAsymmU8, in_offset=9, act=cases.RELU6),
+          cases.make_conv_case("xcd_1x1_c256_co200", 852, n=3, h=14, w=14, ci=256, co=200, kh=1, kw=1),
+          cases.make_conv_case("xcd_3x3_c128_co192", 853, n=2, h=13, w=11, ci=128, co=192, act=cases.RELU),
+          cases.make_conv_case("xcd_1x1_c128_few_rows", 854, n=1, h=9, w=9, ci=128, co=512, kh=1, kw=1),
+          cases.make_conv_case("xcd_1x1_c1024_co1024", 855, n=32, h=7, w=7, ci=1024, co=1024, kh=1, kw=1, in_dtype=DataType.QAsymmU8, in_offset=0, act=cases.RELU6)]
+    for c in cs:
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        for cols in (1, 2, 0):
+            for tile in (64, 128):
+                shim.set_option("igemm_xcd_cols", cols)
+                shim.set_option("igemm_tile", tile)
+                try:
+                    got = _gpu_conv(c, shim.ALGO_MFMA)
+                    kernel = shim.last_kernel()
+                finally:
+                    shim.set_option("igemm_xcd_cols", 0)
+                    shim.set_option("igemm_tile", 0)
+                assert kernel.startswith("IgemmLdsKernel<"), kernel
+                np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} xcd_cols {cols} tile {tile}")
+
+
 def test_k_split_over_wave_groups_gives_the_same_bytes():
     """Launches of at most one 64x64 block per CU with K >= 2048 split K over two or four groups of waves inside the
     block (IgemmKSplitKernel).  Forced on small and ragged problems -- fewer k-tiles than groups, k-tile counts that do not
