@@ -80,6 +80,7 @@ struct Options
     int dw_rows = 0;                   // output rows per thread of the 3x3 depthwise kernel: 0 automatic, 1 or 2 forced
     int pw_slab = 0;                   // output channels per slab of the weight-stationary pointwise kernel: 0 automatic, 32 / 64 / 128 forced
     int dw_cb = 0;                     // channels per block of the 3x3 depthwise kernel: 0 automatic (128 where the count allows), 32 forced
+    int dw_mfma = 1;                   // 3x3 depthwise: 1 on the matrix cores (tile chosen from the feature map), 0 on the VALU kernel, 7 / 8 / 14 / 16 that tile edge where the stride allows it
     int stem_dot4 = 0;                 // 1: small-Ci convolutions stay on the v_dot4 kernel (tests compare it with the MFMA one)
     int igemm_xcd_cols = 0;            // direct-to-LDS implicit GEMM: 0 split the XCDs over the output channels where the weights are heavy, 1 never, 2 wherever possible
     int dwpw_panel = 1;                // 0: fused depthwise + pointwise launches never take the one-block-per-tile-over-all-channels kernel

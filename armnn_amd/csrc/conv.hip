@@ -3,6 +3,7 @@
 #include "common.h"
 #include "conv_kernels.h"
 #include "dw_stem_kernels.h"
+#include "dw_mfma_kernel.h"
 #include "dwpw_kernel.h"
 #include "dwpw_panel_kernel.h"
 #include "pwdw_kernel.h"
@@ -62,6 +63,8 @@ int ValidateQuant(const mi355x_quant& q, const char* what)
 }
 
 // `weights` in the reference layout: conv [Co][Kh][Kw][Ci]; depthwise [1][Kh][Kw][Co].
+int ChooseDwMfmaTile(int stride, int Ho, int Wo, int forced);
+
 int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355x_const_quant* wq,
               const int32_t* bias_host, const mi355x_const_quant* bq, mi355x_conv2d_s* p)
 {
@@ -102,6 +105,7 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
     p->opt_xcd_cols = GlobalOptions().igemm_xcd_cols;
     p->opt_dw_rows = GlobalOptions().dw_rows;
     p->opt_dw_cb = GlobalOptions().dw_cb;
+    p->opt_dw_mfma = GlobalOptions().dw_mfma;
     p->opt_stem_dot4 = GlobalOptions().stem_dot4;
     const int Co = static_cast<int>(d.out_c), Ci = static_cast<int>(d.in_c);
     const int Kh = static_cast<int>(d.kernel_h), Kw = static_cast<int>(d.kernel_w);
@@ -366,7 +370,12 @@ int BuildPlan(const mi355x_conv2d_desc& d, const void* weights_host, const mi355
             const int cbw = p->opt_dw_cb == 32 ? 32 : (Co % 128) == 0 ? 128 : (Co % 64) == 0 ? 64 : 32;
             const int pixels = (cbw == 128 ? 2 : 4) * (d.stride_x == 1 ? 4 : 2);
             char buf[96];
-            std::snprintf(buf, sizeof(buf), "depthwise3x3_dot4_lds stride %d, tile %dx%dx%d", static_cast<int>(d.stride_x), cbw == 32 ? 8 : 4, pixels, cbw);
+            if (p->opt_dw_mfma != 0)
+            {
+                std::snprintf(buf, sizeof(buf), "depthwise3x3_mfma16x16x64_lds stride %d", static_cast<int>(d.stride_x));
+            }
+            else
+                std::snprintf(buf, sizeof(buf), "depthwise3x3_dot4_lds stride %d, tile %dx%dx%d", static_cast<int>(d.stride_x), cbw == 32 ? 8 : 4, pixels, cbw);
             p->info = buf;
         }
         if (p->w_dot4b) p->info += ", weights minus their zero point as two int8 halves";
@@ -684,7 +693,7 @@ int LaunchIgemmLdsT(const mi355x_conv2d_s* p, uint32_t batch, const void* x, voi
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&IgemmLdsKernel<BM, BN, WM, WN, ST, U8, AW>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);
-    NoteKernel("IgemmLdsKernel<%d, %d, %d, %d, %d, %s, %s>", BM, BN, WM, WN, ST, BoolName(U8), BoolName(AW));
+    NoteKernel("IgemmLdsKernel<%d, %d, %d, %d, %d, %s, %s, false>", BM, BN, WM, WN, ST, BoolName(U8), BoolName(AW));
     hipLaunchKernelGGL((IgemmLdsKernel<BM, BN, WM, WN, ST, U8, AW>), dim3(grid), dim3(64 * WM * WN), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;
@@ -873,6 +882,120 @@ int LaunchHalo(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y,
     case 256: return wide ? LaunchHaloC<256, 1, 4, 7>(a, p, batch, stream) : LaunchHaloC<256, 2, 2, 4>(a, p, batch, stream);
     default: return -1;
     }
+}
+
+// ---- 3x3 depthwise on the matrix cores -------------------------------------------------------------------------------
+// Tile height (outputs) for an Ho x Wo map: 16 or 14 (16 columns) or 8 or 7 (8 columns) at stride 1, 8 or 7 at stride 2
+// (the halo of a 16-column tile at stride 2 would not fit LDS).  The one that leaves the least padded work, ties to the
+// earlier entry.
+int ChooseDwMfmaTile(int stride, int Ho, int Wo, int forced)
+{
+    static const int kS1[] = {16, 14, 7, 8}, kS2[] = {7, 8};
+    const int* menu = stride == 1 ? kS1 : kS2;
+    const int count = stride == 1 ? 4 : 2;
+    int best = menu[0];
+    long long best_cost = -1;
+    for (int i = 0; i < count; ++i)
+    {
+        const int th = menu[i], tw = th >= 14 ? 16 : 8;
+        if (forced == th) return th;
+        const long long cost = static_cast<long long>((Ho + th - 1) / th) * ((Wo + tw - 1) / tw) * ((th * tw + 15) / 16) * 16;
+        if (best_cost < 0 || cost < best_cost) { best_cost = cost; best = th; }
+    }
+    return best;
+}
+
+int DeviceCuCount()
+{
+    static const int n = []() {
+        int dev = 0, cus = 0;
+        if (hipGetDevice(&dev) != hipSuccess || hipDeviceGetAttribute(&cus, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cus < 8) return 256;
+        return cus;
+    }();
+    return n;
+}
+
+template <int S, bool W2, int CB, int T>
+int LaunchDwMfmaT(const Dw3x3Args& a, hipStream_t stream)
+{
+    constexpr int TW = T >= 14 ? 16 : 8;
+    using G = DwMfmaTile<S, CB, T, TW>;
+    constexpr int smem = G::SMEM;
+    const auto kernel = &DepthwiseMfmaKernel<S, W2, CB, T, TW>;
+    // blocks that fit a CU at once (LDS, registers), asked once per kernel
+    static const int per_cu = [&]() {
+        int n = 0;
+        if (smem > 48 * 1024 && hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess) return 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, G::NT, smem) != hipSuccess) return 0;
+        return n;
+    }();
+    if (per_cu <= 0) { (void)hipGetLastError(); return SetError(MI355X_ERR_UNSUPPORTED, "depthwise kernel: no block fits a CU"); }
+    // As many blocks per XCD as run at once; each walks its share of the XCD's items with the next item's loads in flight.
+    // A stride between a block's items that is a multiple of the channel blocks keeps its weights in registers.
+    int per_xcd = per_cu * (DeviceCuCount() / 8);
+    if (per_xcd >= a.xcd_chunk) per_xcd = a.xcd_chunk;
+    else if (per_xcd > a.cblocks) per_xcd -= per_xcd % a.cblocks;
+    NoteKernel("DepthwiseMfmaKernel<%d, %s, %d, %d, %d>", S, BoolName(W2), CB, T, TW);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(per_xcd) * 8u), dim3(G::NT), smem, stream, a);
+    return 0;
+}
+
+template <int S, bool W2, int CB>
+int LaunchDwMfmaTile(int tile, const Dw3x3Args& a, hipStream_t stream)
+{
+    if (tile == 7) return LaunchDwMfmaT<S, W2, CB, 7>(a, stream);
+    return LaunchDwMfmaT<S, W2, CB, 8>(a, stream);
+}
+
+template <int S, bool W2>
+int LaunchDwMfmaCb(int cbw, int tile, const Dw3x3Args& a, hipStream_t stream)
+{
+    if constexpr (S == 1)
+    {
+        if (tile == 16) return LaunchDwMfmaT<S, W2, 32, 16>(a, stream);
+        if (tile == 14) return LaunchDwMfmaT<S, W2, 32, 14>(a, stream);
+    }
+    if (cbw == 64) return LaunchDwMfmaTile<S, W2, 64>(tile, a, stream);
+    return LaunchDwMfmaTile<S, W2, 32>(tile, a, stream);
+}
+
+// Whether the matrix-core kernel takes this launch (else the VALU kernel does): tensors it can address with 32-bit offsets
+// within an image, 16-byte aligned, and an item count its reciprocal decoding is exact for.
+bool DwMfmaTakes(const mi355x_conv2d_s* p, uint32_t batch, const void* x, const void* y)
+{
+    const ConvGeom& g = p->geom;
+    if (p->opt_dw_mfma == 0) return false;
+    if (((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) != 0) return false;
+    if (static_cast<long long>(g.Ho) * g.Wo * g.Co >= 0x40000000ll || static_cast<long long>(g.H) * g.W * g.Co >= 0x40000000ll) return false;
+    // items at the smallest tile and channel block, times the largest divisor, stays below 2^32
+    const long long items = static_cast<long long>(batch) * ((g.Ho + 6) / 7) * ((g.Wo + 7) / 8) * ((g.Co + 31) / 32);
+    const long long divisor = std::max<long long>({(g.Ho + 6) / 7, (g.Wo + 7) / 8, (g.Co + 31) / 32});
+    return items < 0x7fffffffll - 8 && items * divisor < 0xffffffffll;
+}
+
+// `a`: as filled for the VALU kernel; the tiling is replaced.
+int LaunchDwMfma(const mi355x_conv2d_s* p, Dw3x3Args a, hipStream_t stream)
+{
+    const ConvGeom& g = p->geom;
+    const int tile = ChooseDwMfmaTile(g.stride_x, g.Ho, g.Wo, p->opt_dw_mfma);
+    const int tw = tile >= 14 ? 16 : 8;
+    // 64 channels per block (one wave per group of 16) where the count allows; the 16-column tiles take 32 (two waves per
+    // group): with 64 their halo buffers would leave two blocks per CU
+    const int cbw = tw == 16 || (g.Co % 64) != 0 || p->opt_dw_cb == 32 ? 32 : 64;
+    a.cblocks = (g.Co + cbw - 1) / cbw;
+    a.tiles_x = (g.Wo + tw - 1) / tw; a.tiles_y = (g.Ho + tile - 1) / tile;
+    const long long nb = static_cast<long long>(a.N) * a.tiles_x * a.tiles_y * a.cblocks;
+    a.total_blocks = static_cast<int>(nb);
+    a.xcd_chunk = static_cast<int>((nb + 7) / 8);
+    const auto rcp = [](int d) { return d <= 1 ? 0u : static_cast<uint32_t>((0x100000000ull + static_cast<unsigned>(d) - 1) / static_cast<unsigned>(d)); };
+    a.rcp_cblocks = rcp(a.cblocks); a.rcp_tiles_x = rcp(a.tiles_x); a.rcp_tiles_y = rcp(a.tiles_y);
+    const bool w2 = p->w_dot4b != nullptr;
+    int rc;
+    if (g.stride_x == 1) rc = w2 ? LaunchDwMfmaCb<1, true>(cbw, tile, a, stream) : LaunchDwMfmaCb<1, false>(cbw, tile, a, stream);
+    else rc = w2 ? LaunchDwMfmaCb<2, true>(cbw, tile, a, stream) : LaunchDwMfmaCb<2, false>(cbw, tile, a, stream);
+    if (rc != 0) return rc;
+    MI355X_HIP(hipGetLastError());
+    return 0;
 }
 
 int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hipStream_t stream)
@@ -1100,6 +1223,7 @@ int RunPlan(const mi355x_conv2d_s* p, uint32_t batch, const void* x, void* y, hi
             Dw3x3Args a;
             int rows_per_thread = 1, cbw = 32;
             if (const int rc = FillDw3x3Args(p, batch, x, y, &a, &rows_per_thread, &cbw)) return rc;
+            if (DwMfmaTakes(p, batch, x, y)) return LaunchDwMfma(p, a, stream);
             const bool wide = cbw == 128, mid = cbw == 64;
             const dim3 grid(static_cast<unsigned>(a.xcd_chunk) * 8u);
             const bool w2 = p->w_dot4b != nullptr;

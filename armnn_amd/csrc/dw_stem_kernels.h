@@ -37,6 +37,7 @@ struct Dw3x3Args
     int tiles_x, tiles_y, cblocks;
     int total_blocks, xcd_chunk;   // work items, and ceil(work items / 8): the grid is 8 * xcd_chunk blocks
     uint32_t xor_mask, pad_word;
+    uint32_t rcp_cblocks, rcp_tiles_x, rcp_tiles_y;   // matrix-core kernel: ceil(2^32 / d) of the three divisors (unused where d = 1)
     Requant rq;
 };
 

@@ -4,11 +4,12 @@
 //   The intermediate tensor never leaves the CU, and it is produced in exactly the pieces the GEMM consumes: the
 //   depthwise layer's channel block kt (128 channels) of the 64 pixels IS k-tile kt of the GEMM's activation operand.
 //   The kernel alternates, once per k-tile, between
-//     a depthwise phase   all 512 threads run the v_dot4 arithmetic of Depthwise3x3Block on channel block kt (thread = one
-//                         tile row, 4 pixels, 4 channels), requantize with the depthwise layer's own constants and write
-//                         the codes -- the bytes the separate layer would have stored, shifted to int8 where they are
-//                         uint8 -- into k-tile kt of the activation panel in LDS (the xor-swizzled image the MFMA
-//                         fragment reads expect), and
+//     a depthwise phase   the eight waves run the matrix-core arithmetic of DepthwiseMfmaKernel on channel block kt (wave =
+//                         16 channels, four groups of 16 pixels: three v_mfma_i32_16x16x64_i8 per group over diagonal weight
+//                         operands; a third of the VALU work of the v_dot4 formulation, which bounded this phase),
+//                         requantize with the depthwise layer's own constants and write the codes -- the bytes the
+//                         separate layer would have stored, shifted to int8 where they are uint8 -- into k-tile kt of the
+//                         activation panel in LDS (the xor-swizzled image the MFMA fragment reads expect), and
 //     a GEMM phase        all eight waves multiply k-tile kt into accumulators for ALL output channels: wave (wm, wq) keeps
 //                         the 32 pixel rows wm x 64 NQ channels wq of the output in 32 NQ registers for the whole kernel.
 //   What keeps the phases short is that nothing in them waits for memory: the weights of k-tile kt (64 KB for 512 output
@@ -67,13 +68,17 @@ struct DwPwPanelGeom
     static constexpr int NCOL = 256 * NQ;             // output channels
     static constexpr int NT = 4 * NQ;                 // 64-channel weight tiles per k-tile
     static constexpr int HR = 10, HC = 10;            // halo of an 8 x 8 tile
-    static constexpr int HALO = HR * HC * 128;
+    static constexpr int HPITCH = 144;                // bytes per halo pixel in LDS: 128 + 16, so that the 16-byte reads of 8
+                                                      // neighbouring pixels fall on different bank quads
+    static constexpr int HROWP = 1664;                // bytes per halo row: >= 10 pixels and 128 mod 256, so that the reads of
+                                                      // the pixel group's second row take the quads the first row's leave free
+    static constexpr int HALO = HR * HROWP;
     static constexpr int LDO = NCOL + 16;
     static constexpr int PANEL = KT * 64 * 128;
     static constexpr int TAB = 4 * NCOL * 4;
     static constexpr int RING = NT * 64 * 128;
     static constexpr int OUT = 64 * LDO;
-    static constexpr int WORK = 2 * HALO + RING > OUT ? 2 * HALO + RING : OUT;   // halo buffers + weight ring; the output staging reuses them
+    static constexpr int WORK = HALO + RING > OUT ? HALO + RING : OUT;   // halo buffer + weight ring; the output staging reuses them
     static constexpr int SMEM = PANEL + TAB + WORK;
 };
 
@@ -82,15 +87,15 @@ template <int KT, int NQ>
 __global__ __launch_bounds__(512) void DwPwPanelKernel(DwPwPanelArgs a)
 {
     using G = DwPwPanelGeom<KT, NQ>;
-    constexpr int NCOL = G::NCOL, NT = G::NT, HC = G::HC, HALO = G::HALO, LDO = G::LDO;
+    constexpr int NCOL = G::NCOL, NT = G::NT, HC = G::HC, HALO = G::HALO, LDO = G::LDO, HPITCH = G::HPITCH, HROWP = G::HROWP;
     constexpr int NTHR = 512;
     typedef __attribute__((address_space(3))) void* LdsPtr;
     typedef const __attribute__((address_space(1))) void* GlobalPtr;
     extern __shared__ __attribute__((aligned(16))) uint8_t smem[];
     uint8_t* const panel = smem;                                           // [KT][64 pixels][128 B]
     float* const tab = reinterpret_cast<float*>(smem + G::PANEL);          // [4][NCOL]: m+, b+ (corr folded in), m-, b- (corr folded in)
-    uint8_t* const halo = smem + G::PANEL + G::TAB;                        // [2][10 x 10 pixels][128 B]
-    uint8_t* const ring = halo + 2 * HALO;                                 // [NT][64 channels][128 B]
+    uint8_t* const halo = smem + G::PANEL + G::TAB;                        // [10 rows of HROWP bytes][10 pixels of HPITCH bytes]
+    uint8_t* const ring = halo + HALO;                                 // [NT][64 channels][128 B]
     uint8_t* const Os = halo;                                              // [64][LDO], after the last GEMM phase
 
     int b = XcdContiguousWorkItem(blockIdx.x, a.xcd_chunk);
@@ -109,10 +114,20 @@ __global__ __launch_bounds__(512) void DwPwPanelKernel(DwPwPanelArgs a)
 #endif
     DWPW_STAMP();
 
-    // ---- depthwise roles: thread = tile row (= wave), 4 pixels, 4 channels of the current 128-channel block ------------
-    const int c4 = tid & 31;
-    const int xg = (tid >> 5) & 1;
-    const int row = wave;
+    // ---- depthwise roles: wave = 16 channels of the current 128-channel block; lane (j, g): pixel j of a group of 16 (two
+    // tile rows) and tap slot g as an MFMA operand, channel quad g of pixel j as a result
+    const int dj = lane & 15, dg = lane >> 4;
+    const int drj = dj >> 3, dcj = dj & 7;
+    int dtap[3], dwrow[3], dwshift[3];
+#pragma unroll
+    for (int m = 0; m < 3; ++m)
+    {
+        const int t = 4 * m + dg;
+        const int tc = min(t, 8);                      // slots past the ninth tap read the ninth; their weights are zero
+        dtap[m] = (drj + tc / 3) * HROWP + (dcj + tc % 3) * HPITCH + wave * 16;
+        dwrow[m] = tc / 3;
+        dwshift[m] = t < 9 ? 8 * (tc % 3) : 24;        // shift 24: the zero byte of a packed filter row
+    }
     // ---- staging of a halo: 800 chunks of 16 bytes, at most two per thread; only the channel block moves from phase to phase
     const int iy_org = ty * 8 - a.pad_top;
     const int ix_org = tx * 8 - a.pad_left;
@@ -134,9 +149,16 @@ __global__ __launch_bounds__(512) void DwPwPanelKernel(DwPwPanelArgs a)
 #pragma unroll
         for (int k = 0; k < 2; ++k) h[k] = *reinterpret_cast<const v4i*>(hok[k] ? hsrc[k] + kt * 128 : a.pad16);
     };
-    auto store_halo = [&](int buf, const v4i (&h)[2]) {
-        *reinterpret_cast<v4i*>(halo + buf * HALO + tid * 16) = h[0] ^ dxm;
-        if (tid + NTHR < 800) *reinterpret_cast<v4i*>(halo + buf * HALO + (tid + NTHR) * 16) = h[1] ^ dxm;
+    int hlds[2];
+#pragma unroll
+    for (int k = 0; k < 2; ++k)
+    {
+        const int i = min(tid + k * NTHR, 799);
+        hlds[k] = ((i >> 3) / HC) * HROWP + ((i >> 3) % HC) * HPITCH + (i & 7) * 16;
+    }
+    auto store_halo = [&](const v4i (&h)[2]) {
+        *reinterpret_cast<v4i*>(halo + hlds[0]) = h[0] ^ dxm;
+        if (tid + NTHR < 800) *reinterpret_cast<v4i*>(halo + hlds[1]) = h[1] ^ dxm;
     };
 
     // ---- GEMM roles: wave (wm, wq) owns pixel rows [32 wm, 32 wm + 32) x output channels [64 NQ wq, 64 NQ (wq + 1)) ----------
@@ -172,7 +194,7 @@ __global__ __launch_bounds__(512) void DwPwPanelKernel(DwPwPanelArgs a)
 #pragma unroll
         for (int i = 0; i < TABV; ++i)
             if (tid + i * NTHR < NCOL) *reinterpret_cast<float4*>(tab + (tid + i * NTHR) * 4) = tv[i];
-        store_halo(0, h0);
+        store_halo(h0);
     }
     __syncthreads();
     DWPW_STAMP();
@@ -187,69 +209,48 @@ __global__ __launch_bounds__(512) void DwPwPanelKernel(DwPwPanelArgs a)
     for (int kt = 0; kt < KT; ++kt)
     {
         // ---- requests of this phase, in the order they will be needed: constants, next halo, weights ----------------------
-        const int c = kt * 128 + c4 * 4;
-        uint32_t wA[3][4];
-#pragma unroll
-        for (int ch = 0; ch < 4; ++ch)
-        {
-            const uint4 w4 = *reinterpret_cast<const uint4*>(a.wpack + (c + ch) * 4);
-            wA[0][ch] = w4.x; wA[1][ch] = w4.y; wA[2][ch] = w4.z;
-        }
-        const v4i corr4 = *reinterpret_cast<const v4i*>(a.dw_corr + c);
-        const Fast4 f4 = LoadFast4(a.dw_ct, c);
+        const int c0 = kt * 128 + wave * 16;
+        const uint4 w4 = *reinterpret_cast<const uint4*>(a.wpack + (c0 + dj) * 4);
+        const int cq = c0 + 4 * dg;                        // the four channels this lane requantizes
+        const v4i corr4 = *reinterpret_cast<const v4i*>(a.dw_corr + cq);
+        const Fast4 f4 = LoadFast4(a.dw_ct, cq);
         v4i hn[2];
         if (kt + 1 < KT) load_halo(kt + 1, hn);
         load_weights(kt);
 
         // ---- depthwise phase: channel block kt of the 8 x 8 tile --------------------------------------------------------
-        int dacc[4][4];
-#pragma unroll
-        for (int j = 0; j < 4; ++j)
-#pragma unroll
-            for (int ch = 0; ch < 4; ++ch) dacc[j][ch] = corr4[ch];
-        const uint8_t* hb = halo + (kt & 1) * HALO;
-#pragma unroll
-        for (int ir = 0; ir < 3; ++ir)
+        // weight operands: byte dj of the lane's 16 is w[tap][c0 + dj], the others are zero
+        v4i wa[3];
         {
-            const uint8_t* base = hb + ((row + ir) * HC + xg * 4) * 128 + c4 * 4;
-            uint32_t px[6];
+            const int dw = dj >> 2, sh = 8 * (dj & 3);
 #pragma unroll
-            for (int j = 0; j < 6; ++j) px[j] = *reinterpret_cast<const uint32_t*>(base + j * 128);
-            uint32_t lo[3], hi[3];
-#pragma unroll
-            for (int q = 0; q < 3; ++q)
+            for (int m = 0; m < 3; ++m)
             {
-                lo[q] = __builtin_amdgcn_perm(px[2 * q + 1], px[2 * q], 0x05010400u);
-                hi[q] = __builtin_amdgcn_perm(px[2 * q + 1], px[2 * q], 0x07030602u);
-            }
-#pragma unroll
-            for (int g = 0; g < 2; ++g)
-            {
-                uint32_t chv[4];
-                chv[0] = __builtin_amdgcn_perm(lo[g + 1], lo[g], 0x05040100u);
-                chv[1] = __builtin_amdgcn_perm(lo[g + 1], lo[g], 0x07060302u);
-                chv[2] = __builtin_amdgcn_perm(hi[g + 1], hi[g], 0x05040100u);
-                chv[3] = __builtin_amdgcn_perm(hi[g + 1], hi[g], 0x07060302u);
-#pragma unroll
-                for (int ch = 0; ch < 4; ++ch)
-                {
-                    dacc[2 * g][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wA[ir][ch]), dacc[2 * g][ch], false);
-                    dacc[2 * g + 1][ch] = __builtin_amdgcn_sdot4(static_cast<int>(chv[ch]), static_cast<int>(wA[ir][ch] << 8), dacc[2 * g + 1][ch], false);
-                }
+                const uint32_t ra = dwrow[m] == 0 ? w4.x : dwrow[m] == 1 ? w4.y : w4.z;
+                const int ba = static_cast<int>(((ra >> dwshift[m]) & 0xffu) << sh);
+                wa[m] = v4i{dw == 0 ? ba : 0, dw == 1 ? ba : 0, dw == 2 ? ba : 0, dw == 3 ? ba : 0};
             }
         }
-        // the codes of pixel r = 8 row + 4 xg + j, channels c .. c + 3: chunk (c4 >> 2) of panel row r, at its swizzled slot
+        const uint8_t* hb = halo;
 #pragma unroll
-        for (int j = 0; j < 4; ++j)
+        for (int u = 0; u < 4; ++u)
         {
-            const uint32_t q = Requant4Dev(dacc[j][0], dacc[j][1], dacc[j][2], dacc[j][3], f4, a.dw_ct, c, a.dw_rq) ^ a.mid_xor;
-            const int r = 8 * row + 4 * xg + j;
-            *reinterpret_cast<uint32_t*>(panel + kt * 8192 + r * 128 + (((c4 >> 2) ^ ((r >> 1) & 7)) * 16) + (c4 & 3) * 4) = q;
+            const v4i b0 = *reinterpret_cast<const v4i*>(hb + dtap[0] + u * 2 * HROWP);
+            const v4i b1 = *reinterpret_cast<const v4i*>(hb + dtap[1] + u * 2 * HROWP);
+            const v4i b2 = *reinterpret_cast<const v4i*>(hb + dtap[2] + u * 2 * HROWP);
+            v4i dacc = corr4;
+            dacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wa[0], b0, dacc, 0, 0, 0);
+            dacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wa[1], b1, dacc, 0, 0, 0);
+            dacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wa[2], b2, dacc, 0, 0, 0);
+            // the codes of pixel r = 16 u + dj, channels cq .. cq + 3: chunk `wave` of panel row r, at its swizzled slot
+            const uint32_t q = Requant4Dev(dacc[0], dacc[1], dacc[2], dacc[3], f4, a.dw_ct, cq, a.dw_rq) ^ a.mid_xor;
+            const int r = 16 * u + dj;
+            *reinterpret_cast<uint32_t*>(panel + kt * 8192 + r * 128 + ((wave ^ ((r >> 1) & 7)) * 16) + dg * 4) = q;
         }
-        if (kt + 1 < KT) store_halo((kt + 1) & 1, hn);
         DWPW_STAMP();
-        __builtin_amdgcn_s_waitcnt(VmcntImm(0));          // this wave's share of the weights has landed
-        __syncthreads();                                   // k-tile kt of the panel, all weight tiles and the next halo are in LDS
+        __builtin_amdgcn_s_waitcnt(VmcntImm(0));          // this wave's share of the weights (and of the next halo) has landed
+        __syncthreads();                                   // k-tile kt of the panel and all weight tiles are in LDS; the halo has been read
+        if (kt + 1 < KT) store_halo(hn);                   // (the barrier behind the GEMM phase orders it before the next phase's reads)
         DWPW_STAMP();
 
         // ---- GEMM phase: k-tile kt into every accumulator ------------------------------------------------------------------
@@ -271,7 +272,7 @@ __global__ __launch_bounds__(512) void DwPwPanelKernel(DwPwPanelArgs a)
                 }
             }
         }
-        __syncthreads();                                   // the ring may be refilled, the halo buffer of this phase overwritten
+        __syncthreads();                                   // the ring may be refilled; the next halo is in LDS
         DWPW_STAMP();
     }
 

@@ -41,7 +41,7 @@ struct mi355x_conv2d_s
     unsigned concurrency = 1;      // launches of the plan's network that run side by side (mi355x_conv2d_set_concurrency)
     int tile_override = 0;         // 0: choose the MFMA tile per launch; 64 / 96 (= 128x64) / 128: the "igemm_tile" option at plan creation
     int opt_xcd_cols = 0;
-    int opt_igemm_lds = 2, opt_dw_rows = 0, opt_dw_cb = 0, opt_stem_dot4 = 0;     // the other process-wide options, as they stood at plan creation
+    int opt_igemm_lds = 2, opt_dw_rows = 0, opt_dw_cb = 0, opt_dw_mfma = 1, opt_stem_dot4 = 0;     // the other process-wide options, as they stood at plan creation
                                    // (launches read the plan, never the mutable globals: plans may run on any host thread)
     uint32_t xor_mask = 0, pad_word = 0;
     int zw_neg = 0;                // MFMA plans: minus the zero point of the stored int8 weights (0: symmetric)

@@ -170,6 +170,12 @@ int mi355x_set_option(const char* name, int value)
         GlobalOptions().pw_slab = value;
         return 0;
     }
+    if (std::strcmp(name, "dw_mfma") == 0)
+    {
+        if (value != 0 && value != 1 && value != 7 && value != 8 && value != 14 && value != 16) return SetError(MI355X_ERR_INVALID_ARGUMENT, "dw_mfma must be 0, 1, 7, 8, 14 or 16");
+        GlobalOptions().dw_mfma = value;
+        return 0;
+    }
     if (std::strcmp(name, "dw_cb") == 0)
     {
         if (value != 0 && value != 32) return SetError(MI355X_ERR_INVALID_ARGUMENT, "dw_cb must be 0 or 32");

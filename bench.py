@@ -270,7 +270,11 @@ def main():
         name, _, value = opt.partition("=")
         shim.set_option(name, int(value))
     if args.lanes == 0:
-        args.lanes = 2 if batch >= 16 and batch % 2 == 0 else 1
+        # Two lanes overlap the tails of one lane's launches with the other's; the 3x3 depthwise kernel sizes its grid to
+        # the whole device and walks its items itself, and two of those side by side get in each other's way
+        # (MobileNetV1, 64 images: 0.330 ms in one lane, 0.336 in two; ResNet-50, 32 images: 0.864 and 0.725).
+        depthwise = any(l.op == "depthwise" for l in net.layers)
+        args.lanes = 2 if batch >= 16 and batch % 2 == 0 and not depthwise else 1
     dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse="" if args.fuse == "none" else args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add, chain=args.chain)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev

@@ -247,5 +247,5 @@ def test_mobilenet_with_per_tensor_uint8_weights(port):
     dn.close()
     print(kinds, flush=True)
     assert "two int8 halves" in kinds["stem"] and "smallci_dot4" in kinds["stem"]
-    assert all("depthwise3x3_dot4" in k for n, k in kinds.items() if n.startswith("dw"))
+    assert all("depthwise3x3_mfma" in k for n, k in kinds.items() if n.startswith("dw"))
     assert all("weight zero point by row sums" in k for n, k in kinds.items() if n.startswith("pw") or n == "logits")

@@ -89,10 +89,10 @@ def test_algo_selection():
     assert a == shim.ALGO_DEPTHWISE and "c4" in info
     c = cases.make_conv_case("sel", 1, ci=16, depthwise=True)
     a, info = shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()
-    assert a == shim.ALGO_DEPTHWISE and "dot4" in info
+    assert a == shim.ALGO_DEPTHWISE and "depthwise3x3" in info
     c = cases.make_conv_case("sel", 1, ci=64, depthwise=True)
     a, info = shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, **c.params).algo()
-    assert a == shim.ALGO_DEPTHWISE and "dot4" in info
+    assert a == shim.ALGO_DEPTHWISE and "depthwise3x3" in info
     with pytest.raises(shim.ShimError):
         c = cases.make_conv_case("sel", 1, ci=3, co=16)
         shim.Conv2dPlan(c.x.info, c.w, c.b, c.out_info, algo=shim.ALGO_MFMA, **c.params)
@@ -379,10 +379,12 @@ def test_depthwise_rows_per_thread_variants_give_the_same_bytes():
         want = _gpu_conv(c, shim.ALGO_DIRECT)
         for rows in (0, 1, 2):
             shim.set_option("dw_rows", rows)
+            shim.set_option("dw_mfma", 0)
             try:
                 got = _gpu_conv(c, shim.ALGO_DEPTHWISE)
             finally:
                 shim.set_option("dw_rows", 0)
+                shim.set_option("dw_mfma", 1)
             print(f"{c.name} rows {rows}", flush=True)
             np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} rows {rows}")
 
@@ -446,8 +448,70 @@ def test_depthwise_64_and_128_channel_blocks_give_the_same_bytes():
     pixel), the other multiples of 64 with 64: large, mid-sized and tiny feature maps of ragged sizes, both strides, one
     and two rows per thread, uint8 activations, weights with a zero point (two int8 halves), against the 32-channel
     blocks and the plain kernel."""
+    for c in _depthwise_block_cases():
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        for cb in (0, 32):
+            for rows in (0, 1, 2):
+                shim.set_option("dw_cb", cb)
+                shim.set_option("dw_rows", rows)
+                shim.set_option("dw_mfma", 0)
+                try:
+                    got = _gpu_conv(c, shim.ALGO_DEPTHWISE)
+                    kernel = shim.last_kernel()
+                finally:
+                    shim.set_option("dw_cb", 0)
+                    shim.set_option("dw_rows", 0)
+                    shim.set_option("dw_mfma", 1)
+                print(f"{c.name} blocks {cb or 'auto'} rows {rows}: {kernel}", flush=True)
+                channels = c.x.info.shape[3]
+                blocks = 32 if cb == 32 else 128 if channels % 128 == 0 else 64
+                assert kernel.startswith("Depthwise3x3Kernel<") and kernel.endswith(f", {blocks}>"), kernel
+                np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} blocks {cb} rows {rows}")
+
+
+def test_depthwise_on_the_matrix_cores_gives_the_same_bytes():
+    """The 3x3 depthwise kernel that computes on the matrix cores (sixteen channels x sixteen pixels x four taps per
+    instruction), with the tile chosen from the feature map and with every tile edge forced, 32-, 64- and 128-channel
+    blocks: ragged feature maps of both strides, uint8 activations, weights as two int8 halves; against the VALU kernel
+    and the plain kernel."""
+    more = [cases.make_conv_case("dwm_s1_112x112x32", 731, n=2, h=112, w=112, ci=32, depthwise=True, act=cases.RELU6),
+            cases.make_conv_case("dwm_s1_14x14x512", 732, n=3, h=14, w=14, ci=512, depthwise=True, act=cases.RELU6),
+            cases.make_conv_case("dwm_s2_14x14x48_u8", 733, n=2, h=14, w=14, ci=48, depthwise=True, stride=(2, 2), in_dtype=DataType.QAsymmU8, in_offset=77, out_offset=9),
+            cases.make_conv_case("dwm_s1_28x28x16", 734, n=2, h=28, w=28, ci=16, depthwise=True, act=cases.RELU),
+            cases.make_conv_case("dwm_s1_1x1x32", 735, n=2, h=1, w=1, ci=32, depthwise=True),
+            cases.make_conv_case("dwm_s1_33x17x80", 736, n=1, h=33, w=17, ci=80, depthwise=True, act=cases.RELU6)]
+    seen = set()
+    for c in _depthwise_block_cases() + more:
+        want = _gpu_conv(c, shim.ALGO_DIRECT)
+        shim.set_option("dw_mfma", 0)
+        try:
+            valu = _gpu_conv(c, shim.ALGO_DEPTHWISE)
+            assert shim.last_kernel().startswith("Depthwise3x3Kernel<"), shim.last_kernel()
+        finally:
+            shim.set_option("dw_mfma", 1)
+        np.testing.assert_array_equal(valu.data, want.data, err_msg=c.name)
+        for tile in (1, 7, 8, 14, 16):
+            for cb in (0, 32):
+                shim.set_option("dw_mfma", tile)
+                shim.set_option("dw_cb", cb)
+                try:
+                    got = _gpu_conv(c, shim.ALGO_DEPTHWISE)
+                    kernel = shim.last_kernel()
+                finally:
+                    shim.set_option("dw_mfma", 1)
+                    shim.set_option("dw_cb", 0)
+                print(f"{c.name} tile {tile} blocks {cb or 'auto'}: {kernel}", flush=True)
+                assert kernel.startswith("DepthwiseMfmaKernel<"), kernel
+                seen.add(kernel)
+                np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} tile {tile} blocks {cb}: {kernel}")
+    assert len(seen) >= 12, sorted(seen)
+    with pytest.raises(shim.ShimError):
+        shim.set_option("dw_mfma", 9)
+
+
+def _depthwise_block_cases():
     U8 = DataType.QAsymmU8
-    cs = [cases.make_conv_case("dw128_s1_57x53", 711, n=2, h=57, w=53, ci=128, depthwise=True, act=cases.RELU6),
+    return [cases.make_conv_case("dw128_s1_57x53", 711, n=2, h=57, w=53, ci=128, depthwise=True, act=cases.RELU6),
           cases.make_conv_case("dw128_s2_57x53_u8", 712, n=2, h=57, w=53, ci=256, depthwise=True, stride=(2, 2), in_dtype=U8, in_offset=140, out_offset=5),
           cases.make_conv_case("dw128_s1_7x7", 713, n=3, h=7, w=7, ci=256, depthwise=True, act=cases.RELU),
           cases.make_conv_case("dw128_s2_8x5", 714, n=2, h=8, w=5, ci=128, depthwise=True, stride=(2, 2)),
@@ -461,23 +525,6 @@ def test_depthwise_64_and_128_channel_blocks_give_the_same_bytes():
                                w_dtype=U8, w_offset=101, in_dtype=U8, in_offset=120, out_offset=3, act=cases.RELU6),
           cases.make_conv_case("dw128_s1_64x50_zero_point_weights", 715, n=1, h=64, w=50, ci=128, depthwise=True, per_axis=False, w_std=60.0,
                                w_dtype=U8, w_offset=93, in_dtype=U8, in_offset=120, out_offset=3, act=cases.RELU6)]
-    for c in cs:
-        want = _gpu_conv(c, shim.ALGO_DIRECT)
-        for cb in (0, 32):
-            for rows in (0, 1, 2):
-                shim.set_option("dw_cb", cb)
-                shim.set_option("dw_rows", rows)
-                try:
-                    got = _gpu_conv(c, shim.ALGO_DEPTHWISE)
-                    kernel = shim.last_kernel()
-                finally:
-                    shim.set_option("dw_cb", 0)
-                    shim.set_option("dw_rows", 0)
-                print(f"{c.name} blocks {cb or 'auto'} rows {rows}: {kernel}", flush=True)
-                channels = c.x.info.shape[3]
-                blocks = 32 if cb == 32 else 128 if channels % 128 == 0 else 64
-                assert kernel.startswith("Depthwise3x3Kernel<") and kernel.endswith(f", {blocks}>"), kernel
-                np.testing.assert_array_equal(got.data, want.data, err_msg=f"{c.name} blocks {cb} rows {rows}")
     with pytest.raises(shim.ShimError):
         shim.set_option("dw_cb", 64)
 
@@ -766,7 +813,7 @@ def test_depthwise_weights_with_a_zero_point(port, name, kw, halves, in_u8):
     algo, desc = plan.algo()
     plan.destroy()
     print(f"{name}: x={case.x.info.shape} zw={case.w.info.offset} kernel: {desc}", flush=True)
-    assert "depthwise3x3_dot4" in desc
+    assert "depthwise3x3_mfma" in desc
     if halves is not None:
         assert ("two int8 halves" in desc) == halves
     want = _oracle_conv(port, case)
@@ -834,7 +881,7 @@ def test_depthwise_channel_counts_that_are_odd_multiples_of_16(port, c, stride, 
     desc = plan.algo()[1]
     plan.destroy()
     print(f"c={c} stride={stride} {w_kind}: {desc}", flush=True)
-    assert "depthwise3x3_dot4" in desc
+    assert "depthwise3x3_mfma" in desc
     want = _oracle_conv(port, case)
     auto = _gpu_conv(case, shim.ALGO_AUTO)
     mx, exact = lsb_diff(auto.data, want.data)
