@@ -83,6 +83,7 @@ struct Options
     int dw_mfma = 1;                   // 3x3 depthwise: 1 on the matrix cores (tile chosen from the feature map), 0 on the VALU kernel, 7 / 8 / 14 / 16 that tile edge where the stride allows it
     int stem_dot4 = 0;                 // 1: small-Ci convolutions stay on the v_dot4 kernel (tests compare it with the MFMA one)
     int igemm_xcd_cols = 0;            // direct-to-LDS implicit GEMM: 0 split the XCDs over the output channels where the weights are heavy, 1 never, 2 wherever possible
+    int dwpw_stream = 1;               // 0: fused depthwise + pointwise launches never take the persistent kernel for 32 / 64 / 128 channels between the layers
     int dwpw_panel = 1;                // 0: fused depthwise + pointwise launches never take the one-block-per-tile-over-all-channels kernel
     int chain_stages = 2;              // LDS stages of the matrix-core tiles inside a layer chain (2, 3 or 4), read at mi355x_chain_create
     int chain_defer_signal = 0;        // 1: layer chains count a tile as finished behind the next tile's loads (no wait for its stores)

@@ -6,6 +6,7 @@
 #include "dw_mfma_kernel.h"
 #include "dwpw_kernel.h"
 #include "dwpw_panel_kernel.h"
+#include "dwpw_stream_kernel.h"
 #include "pwdw_kernel.h"
 #include "igemm_ksplit_kernel.h"
 #include "pw_gemm_kernel.h"
@@ -1319,6 +1320,63 @@ int LaunchDwPw(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, uint32_t ba
     return 0;
 }
 
+// ---- depthwise 3x3 + pointwise for the wide, shallow front layers: persistent blocks, pointwise weights resident in LDS -----
+// which: 1 = stride 1, 32 -> 64 channels; 2 = stride 2, 64 -> 128; 3 = stride 1, 128 -> 128; 0 when the pair does not fit
+int DwPwStreamShape(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw)
+{
+    const mi355x_conv2d_desc& a = dw->d;
+    if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || dw->w_dot4b || a.stride_x != a.stride_y || a.out_c != a.in_c) return 0;
+    if (pw->zw_neg != 0 || !pw->w_mfma || pw->K_pad < static_cast<int>(a.out_c)) return 0;
+    if (static_cast<long long>(a.in_h) * a.in_w * a.in_c >= (1ll << 30) || static_cast<long long>(a.out_h) * a.out_w * pw->d.out_c >= (1ll << 30)) return 0;
+    if (a.stride_x == 1 && a.out_c == 32 && pw->d.out_c == 64) return 1;
+    if (a.stride_x == 2 && a.out_c == 64 && pw->d.out_c == 128) return 2;
+    if (a.stride_x == 1 && a.out_c == 128 && pw->d.out_c == 128) return 3;
+    return 0;
+}
+
+template <int S, int C, int NO, int TH, int TW>
+int LaunchDwPwStreamT(DwPwStreamArgs a, const ConvGeom& g, hipStream_t stream)
+{
+    using G = DwPwStreamGeom<S, C, NO, TH, TW>;
+    constexpr int smem = G::SMEM;
+    static_assert(smem <= 156 * 1024, "LDS of one CU");
+    const auto kernel = &DwPwStreamKernel<S, C, NO, TH, TW>;
+    static const int per_cu = [&]() {
+        int n = 0;
+        if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess) return 0;
+        if (hipOccupancyMaxActiveBlocksPerMultiprocessor(&n, kernel, G::NT, smem) != hipSuccess) return 0;
+        return n;
+    }();
+    if (per_cu <= 0) { (void)hipGetLastError(); return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel: no block fits a CU"); }
+    a.tiles_x = (g.Wo + TW - 1) / TW; a.tiles_y = (g.Ho + TH - 1) / TH;
+    const long long items = static_cast<long long>(a.N) * a.tiles_x * a.tiles_y;
+    if (items > 0x7fffffffll - 8 || items * std::max(a.tiles_x, a.tiles_y) >= 0xffffffffll) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
+    a.total_items = static_cast<int>(items); a.xcd_chunk = static_cast<int>((items + 7) / 8);
+    const auto rcp = [](int d) { return d <= 1 ? 0u : static_cast<uint32_t>((0x100000000ull + static_cast<unsigned>(d) - 1) / static_cast<unsigned>(d)); };
+    a.rcp_tiles_x = rcp(a.tiles_x); a.rcp_tiles_y = rcp(a.tiles_y);
+    const int per_xcd = std::min(a.xcd_chunk, per_cu * (DeviceCuCount() / 8));
+    NoteKernel("DwPwStreamKernel<%d, %d, %d, %d, %d>", S, C, NO, TH, TW);
+    hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(per_xcd) * 8u), dim3(G::NT), smem, stream, a);
+    MI355X_HIP(hipGetLastError());
+    return 0;
+}
+
+int LaunchDwPwStream(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, int which, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    const ConvGeom& g = dw->geom;
+    DwPwStreamArgs a;
+    a.x = static_cast<const uint8_t*>(x); a.pad16 = dw->pad16; a.wpack = dw->w_dot4; a.dw_ct = ChanTab{dw->chan, dw->Co_pad}; a.dw_corr = dw->corr;
+    a.N = static_cast<int>(batch); a.H = g.H; a.W = g.W; a.Ho = g.Ho; a.Wo = g.Wo;
+    a.pad_top = g.pad_top; a.pad_left = g.pad_left;
+    a.dw_xor = dw->xor_mask; a.dw_rq = dw->rq;
+    a.w = pw->w_mfma; a.w_stride = pw->K_pad; a.pw_ct = ChanTab{pw->chan, pw->Co_pad}; a.pw_corr = pw->corr;
+    a.y = static_cast<uint8_t*>(y);
+    a.mid_xor = pw->xor_mask; a.pw_rq = pw->rq;
+    if (which == 1) return LaunchDwPwStreamT<1, 32, 64, 16, 16>(a, g, stream);
+    if (which == 2) return LaunchDwPwStreamT<2, 64, 128, 8, 8>(a, g, stream);
+    return LaunchDwPwStreamT<1, 128, 128, 8, 8>(a, g, stream);
+}
+
 // ---- depthwise 3x3 stride 1 + pointwise over 256 / 512 channels: one block per 8 x 8 tile over all channels ---------------
 // KT = channels between the layers / 128, NQ = output channels / 256; 0 when the pair does not fit that kernel
 bool DwPwPanelShape(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, int* kt, int* nq)
@@ -1635,6 +1693,12 @@ int mi355x_conv2d_fusion_pays(mi355x_conv2d_t first, mi355x_conv2d_t second, uin
 {
     if (!first || !second || batch == 0) return 0;
     if (!first->d.depthwise || second->d.depthwise) return 0;
+    if (GlobalOptions().dwpw_stream != 0 && DwPwStreamShape(first, second) != 0 && mi355x_conv2d_fusable(first, second) == 0)
+    {
+        // persistent blocks: a few items each are needed to overlap anything
+        const long long items = static_cast<long long>(batch) * ((first->d.out_w + 7) / 8) * ((first->d.out_h + 7) / 8);
+        return items >= 2048 ? 1 : 0;
+    }
     int kt = 0, nq = 0;
     if (GlobalOptions().dwpw_panel == 0 || !DwPwPanelShape(first, second, &kt, &nq)) return 0;
     if (mi355x_conv2d_fusable(first, second) != 0) return 0;
@@ -1658,6 +1722,8 @@ int mi355x_conv2d_run_fused(mi355x_conv2d_t dw, mi355x_conv2d_t pw, uint32_t bat
         if (int rc = PwDwCheck(dw, pw, &sh)) return rc;
         return LaunchPwDw(dw, pw, sh, batch, input_dev, output_dev, ToHip(stream));
     }
+    if (GlobalOptions().dwpw_stream != 0)
+        if (const int which = DwPwStreamShape(dw, pw)) return LaunchDwPwStream(dw, pw, which, batch, input_dev, output_dev, ToHip(stream));
     {
         int kt = 0, nq = 0;
         if (GlobalOptions().dwpw_panel != 0 && DwPwPanelShape(dw, pw, &kt, &nq)) return LaunchDwPwPanel(dw, pw, kt, nq, batch, input_dev, output_dev, ToHip(stream));

@@ -111,12 +111,18 @@ int  mi355x_abi_version(void);
  *   "pw_slab" = 0 | 32 | 64 | 128: output channels per weight slab of the weight-stationary kernel for 1x1 convolutions
  *   with at most 128 input channels (0: the widest that fits the layer; a value wider than that is ignored; identical
  *   bytes; tests and tuning).
- *   "dw_cb" = 0 | 32: channels per block of the 3x3 depthwise kernel (0: 128 where the channel count is a multiple of
- *   128, else 32; 32: always 32; identical bytes).
+ *   "dw_cb" = 0 | 32: channels per block of the 3x3 depthwise kernels (0: as many as the channel count and the kernel
+ *   allow: 64 on the matrix cores, 128 on the VALU kernel; 32: always 32; identical bytes).
+ *   "dw_mfma" = 1 | 0 | 7 | 8 | 14 | 16: 3x3 depthwise layers (multiplier 1, channels a multiple of 16) compute on the
+ *   matrix cores (1, with the tile chosen from the feature map; 7, 8, 14 or 16: that tile height where the stride allows
+ *   it) or on the VALU kernel (0).  Identical bytes.
  *   "igemm_xcd_cols" = 0 | 1 | 2: how the direct-to-LDS implicit GEMM deals its tiles to the 8 XCDs (each has an L2 of its
  *   own): 1 every XCD takes a range of row blocks over all output channels (each fetches every weight), 2 XCDs 0-3 take
  *   the lower half of the output channels and XCDs 4-7 the upper half (half the weights per XCD, every activation row
  *   fetched twice), 0 chooses 2 where the weights outweigh a quarter of the activations of a launch.  Identical bytes.
+ *   "dwpw_stream" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a depthwise layer of 32, 64 (stride 2) or
+ *   128 channels and the pointwise layer behind it (64, 128, 128 output channels) on the persistent kernel that keeps the
+ *   pointwise weights in on-chip memory (identical bytes; lets tests compare it with the older fused kernel).
  *   "dwpw_panel" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a stride-1 depthwise layer of 256 or 512
  *   channels and a pointwise layer of 256 or 512 output channels on the kernel that gives a block an 8 x 8 pixel tile over
  *   all channels (identical bytes; lets tests compare it with the older fused kernel).

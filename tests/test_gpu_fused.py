@@ -35,6 +35,41 @@ PANEL_PAIRS = [
 ]
 
 
+# pairs the persistent kernel with resident pointwise weights takes (32 -> 64, 64 -> 128 at stride 2, 128 -> 128): enough
+# images that a block walks several items, ragged maps, both activation types
+STREAM_PAIRS = [
+    ("stream_c32_co64_u8_112", 12, 112, 112, 32, 64, 1, U8, cases.RELU6, cases.RELU6),      # MobileNetV1 dw1+pw1
+    ("stream_c64_co128_u8_112_s2", 12, 112, 112, 64, 128, 2, U8, cases.RELU6, cases.RELU6),  # dw2+pw2
+    ("stream_c128_co128_u8_56", 12, 56, 56, 128, 128, 1, U8, cases.RELU6, cases.RELU6),      # dw3+pw3
+    ("stream_c32_co64_s8_ragged", 30, 50, 35, 32, 64, 1, S8, cases.RELU, (0, 0.0, 0.0)),
+    ("stream_c64_co128_s8_ragged_s2", 25, 45, 51, 64, 128, 2, S8, (0, 0.0, 0.0), cases.RELU6),
+    ("stream_c128_co128_s8_ragged", 40, 13, 29, 128, 128, 1, S8, cases.RELU6, cases.RELU),
+    ("stream_c32_co64_s8_tiny", 1, 3, 5, 32, 64, 1, S8, cases.RELU6, cases.RELU6),
+]
+
+
+@pytest.mark.parametrize("pair", STREAM_PAIRS + PAIRS[:3], ids=[p[0] for p in STREAM_PAIRS + PAIRS[:3]])
+def test_stream_kernel_is_taken_and_equals_the_older_fused_kernel(pair):
+    shim.Device()
+    dw, pw = _make(*pair)
+    pdw, ppw = _plan(dw), _plan(pw)
+    n = dw.x.info.shape[0]
+    xd = shim.DeviceBuffer(dw.x.data.nbytes).upload(dw.x.data)
+    ya, yb = shim.DeviceBuffer(pw.out_info.num_elements), shim.DeviceBuffer(pw.out_info.num_elements)
+    pdw.run_fused(ppw, n, xd.ptr, ya.ptr)
+    assert shim.last_kernel().startswith("DwPwStreamKernel<"), shim.last_kernel()
+    shim.set_option("dwpw_stream", 0)
+    try:
+        pdw.run_fused(ppw, n, xd.ptr, yb.ptr)
+        assert shim.last_kernel().startswith("DwPwKernel<"), shim.last_kernel()
+    finally:
+        shim.set_option("dwpw_stream", 1)
+    a = ya.download(pw.out_info.shape, numpy_dtype(pw.out_info.dtype))
+    b = yb.download(pw.out_info.shape, numpy_dtype(pw.out_info.dtype))
+    assert len(np.unique(a)) > 8
+    np.testing.assert_array_equal(a, b)
+
+
 def _make(name, n, h, w, c, co, stride, dt, act_dw, act_pw):
     zp_in = 120 if dt == U8 else -8
     zp_mid = 0 if dt == U8 else -128
@@ -73,7 +108,7 @@ def test_panel_kernel_is_taken_and_equals_the_older_fused_kernel(pair):
     np.testing.assert_array_equal(a, b)
 
 
-@pytest.mark.parametrize("pair", PAIRS + PANEL_PAIRS, ids=[p[0] for p in PAIRS + PANEL_PAIRS])
+@pytest.mark.parametrize("pair", PAIRS + PANEL_PAIRS + STREAM_PAIRS[3:], ids=[p[0] for p in PAIRS + PANEL_PAIRS + STREAM_PAIRS[3:]])
 def test_fused_equals_two_layers(port, pair):
     print("pair", pair, flush=True)
     shim.Device()
