@@ -1321,7 +1321,8 @@ int LaunchDwPw(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, uint32_t ba
 }
 
 // ---- depthwise 3x3 + pointwise for the wide, shallow front layers: persistent blocks, pointwise weights resident in LDS -----
-// which: 1 = stride 1, 32 -> 64 channels; 2 = stride 2, 64 -> 128; 3 = stride 1, 128 -> 128; 0 when the pair does not fit
+// which: 1 = stride 1, 32 -> 64 channels; 2 = stride 2, 64 -> 128; 3 = stride 1, 128 -> 128; 4 = stride 2, 128 -> 256 (eight
+// waves: its weights and halo leave room for one block per CU); 0 when the pair does not fit
 int DwPwStreamShape(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw)
 {
     const mi355x_conv2d_desc& a = dw->d;
@@ -1331,16 +1332,17 @@ int DwPwStreamShape(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw)
     if (a.stride_x == 1 && a.out_c == 32 && pw->d.out_c == 64) return 1;
     if (a.stride_x == 2 && a.out_c == 64 && pw->d.out_c == 128) return 2;
     if (a.stride_x == 1 && a.out_c == 128 && pw->d.out_c == 128) return 3;
+    if (a.stride_x == 2 && a.out_c == 128 && pw->d.out_c == 256) return 4;
     return 0;
 }
 
-template <int S, int C, int NO, int TH, int TW>
+template <int S, int C, int NO, int TH, int TW, int NWAVES = 4>
 int LaunchDwPwStreamT(DwPwStreamArgs a, const ConvGeom& g, hipStream_t stream)
 {
-    using G = DwPwStreamGeom<S, C, NO, TH, TW>;
+    using G = DwPwStreamGeom<S, C, NO, TH, TW, NWAVES>;
     constexpr int smem = G::SMEM;
     static_assert(smem <= 156 * 1024, "LDS of one CU");
-    const auto kernel = &DwPwStreamKernel<S, C, NO, TH, TW>;
+    const auto kernel = &DwPwStreamKernel<S, C, NO, TH, TW, NWAVES>;
     static const int per_cu = [&]() {
         int n = 0;
         if (hipFuncSetAttribute(reinterpret_cast<const void*>(kernel), hipFuncAttributeMaxDynamicSharedMemorySize, smem) != hipSuccess) return 0;
@@ -1355,7 +1357,7 @@ int LaunchDwPwStreamT(DwPwStreamArgs a, const ConvGeom& g, hipStream_t stream)
     const auto rcp = [](int d) { return d <= 1 ? 0u : static_cast<uint32_t>((0x100000000ull + static_cast<unsigned>(d) - 1) / static_cast<unsigned>(d)); };
     a.rcp_tiles_x = rcp(a.tiles_x); a.rcp_tiles_y = rcp(a.tiles_y);
     const int per_xcd = std::min(a.xcd_chunk, per_cu * (DeviceCuCount() / 8));
-    NoteKernel("DwPwStreamKernel<%d, %d, %d, %d, %d>", S, C, NO, TH, TW);
+    NoteKernel("DwPwStreamKernel<%d, %d, %d, %d, %d, %d>", S, C, NO, TH, TW, NWAVES);
     hipLaunchKernelGGL(kernel, dim3(static_cast<unsigned>(per_xcd) * 8u), dim3(G::NT), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;
@@ -1374,6 +1376,7 @@ int LaunchDwPwStream(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, int w
     a.mid_xor = pw->xor_mask; a.pw_rq = pw->rq;
     if (which == 1) return LaunchDwPwStreamT<1, 32, 64, 16, 16>(a, g, stream);
     if (which == 2) return LaunchDwPwStreamT<2, 64, 128, 8, 8>(a, g, stream);
+    if (which == 4) return LaunchDwPwStreamT<2, 128, 256, 8, 8, 8>(a, g, stream);
     return LaunchDwPwStreamT<1, 128, 128, 8, 8>(a, g, stream);
 }
 
@@ -1697,7 +1700,7 @@ int mi355x_conv2d_fusion_pays(mi355x_conv2d_t first, mi355x_conv2d_t second, uin
     {
         // persistent blocks: a few items each are needed to overlap anything
         const long long items = static_cast<long long>(batch) * ((first->d.out_w + 7) / 8) * ((first->d.out_h + 7) / 8);
-        return items >= 2048 ? 1 : 0;
+        return items >= 1024 ? 1 : 0;
     }
     int kt = 0, nq = 0;
     if (GlobalOptions().dwpw_panel == 0 || !DwPwPanelShape(first, second, &kt, &nq)) return 0;

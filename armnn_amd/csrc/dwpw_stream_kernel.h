@@ -1,11 +1,12 @@
 // Depthwise 3x3 (stride 1 or 2) + the pointwise 1x1 convolution that consumes it as ONE kernel, for the wide, shallow
-// layers at the front of a MobileNet: 32, 64 or 128 channels between the layers, 64 or 128 output channels.
+// layers at the front of a MobileNet: 32, 64 or 128 channels between the layers, 64, 128 or 256 output channels.
 //
 // Run apart, these layers are bound by memory: the tensor between them is written once and read once (112 x 112 x 32 at 64
 // images: 26 MB each way, next to 26 MB in and 51 MB out).  Here it never leaves the CU.
-//   * A block of four waves is persistent: it keeps the pointwise weights (at most 128 x 128 bytes) and the pointwise
+//   * A block of four (or eight) waves is persistent: it keeps the pointwise weights (at most 256 x 128 bytes) and the pointwise
 //     layer's requantization rows in LDS for its whole life and walks items -- TH x TW output pixels of one image over ALL
-//     channels -- with the next item's input halo in flight (in registers) while the current one is computed.
+//     channels -- with the next item's input halo in flight (in registers) while the current one is computed.  Two barriers
+//     per item: halo staged / panel complete.
 //   * Depthwise phase: the matrix-core arithmetic of DepthwiseMfmaKernel (16 channels x 16 pixels x 4 taps per
 //     v_mfma_i32_16x16x64_i8 over diagonal weight operands kept in registers), requantized with the depthwise layer's own
 //     constants; the codes -- the bytes the separate layer would have stored, shifted to int8 where they are uint8 -- go
@@ -56,14 +57,15 @@ struct DwPwStreamArgs
     Requant        pw_rq;
 };
 
-// S: depthwise stride; C: channels between the layers; NO: output channels; TH x TW: output pixels per item
-template <int S, int C, int NO, int TH, int TW>
+// S: depthwise stride; C: channels between the layers; NO: output channels; TH x TW: output pixels per item; NWAVES: 4 or
+// 8 waves per block (8 where the weights and the halo leave room for one block per CU only)
+template <int S, int C, int NO, int TH, int TW, int NWAVES = 4>
 struct DwPwStreamGeom
 {
     static_assert(C == 32 || C == 64 || C == 128, "channels between the layers");
-    static_assert(NO == 64 || NO == 128, "output channels");
+    static_assert(NO == 64 || NO == 128 || NO == 256, "output channels");
     static_assert(TW == 8 || TW == 16, "a group of 16 pixels is one or two whole tile rows");
-    static constexpr int NT = 256, NW = 4;
+    static constexpr int NW = NWAVES, NT = 64 * NW;
     static constexpr int NCG = C / 16;
     static constexpr int P = TH * TW;                     // pixels per item
     static_assert(P % 64 == 0, "whole 32-pixel MFMA tiles, two per wave at least");
@@ -77,7 +79,7 @@ struct DwPwStreamGeom
     static constexpr int PITCH = C + 16;
     static constexpr int ROWP_RAW = HC * PITCH;
     static constexpr int ROWP = (TW == 8 && S == 1) ? ((ROWP_RAW + 127) / 256 * 256 + 128) : ROWP_RAW;
-    static constexpr int HALO = HR * ROWP;                // one of the two halo buffers
+    static constexpr int HALO = HR * ROWP;                // the halo buffer
     static constexpr int KP = C + 16;                     // bytes per panel row and per weight row in LDS
     static constexpr int PANEL = P * KP;
     static constexpr int WTS = NO * KP;
@@ -91,13 +93,20 @@ struct DwPwStreamGeom
     static constexpr int LDO = SC + 16;
     static constexpr int OUT = NW * 64 * LDO;
     static constexpr int QUADS = 64 * (SC / 16) / 64;     // 16-byte stores per lane and item
-    static constexpr int SMEM = 2 * HALO + PANEL + WTS + TAB + OUT;
+    static constexpr int SMEM = HALO + PANEL + WTS + TAB + OUT;
+    // Blocks per CU that LDS allows; the register budget follows it (a few spilled registers cost less than the third block
+    // gains: 112 x 112 x 32 -> 64 at 64 images 29.5 us with two blocks, 24.4 with three).
+    static constexpr int BLOCKS = 160 * 1024 / SMEM >= 3 ? 3 : 160 * 1024 / SMEM >= 2 ? 2 : 1;
+    static constexpr int WAVES_PER_SIMD = BLOCKS * NW / 4;
 };
 
-template <int S, int C, int NO, int TH, int TW>
-__global__ __launch_bounds__(256) void DwPwStreamKernel(DwPwStreamArgs a)
+template <int S, int C, int NO, int TH, int TW, int NWAVES = 4>
+__global__ __launch_bounds__(64 * NWAVES)
+__attribute__((amdgpu_waves_per_eu(DwPwStreamGeom<S, C, NO, TH, TW, NWAVES>::WAVES_PER_SIMD, DwPwStreamGeom<S, C, NO, TH, TW, NWAVES>::WAVES_PER_SIMD)))
+void DwPwStreamKernel(DwPwStreamArgs a)
 {
-    using G = DwPwStreamGeom<S, C, NO, TH, TW>;
+    using G = DwPwStreamGeom<S, C, NO, TH, TW, NWAVES>;
+    constexpr int NW = G::NW;
     constexpr int NT = G::NT, NCG = G::NCG, HR = G::HR, HC = G::HC, PITCH = G::PITCH, ROWP = G::ROWP, HALO = G::HALO;
     constexpr int CGW = G::CGW, WPC = G::WPC, UNITS = G::UNITS, KP = G::KP, MTW = G::MTW, NTW = G::NTW, LDO = G::LDO, QUADS = G::QUADS;
     constexpr int RPG = 16 / TW;
@@ -106,7 +115,7 @@ __global__ __launch_bounds__(256) void DwPwStreamKernel(DwPwStreamArgs a)
     constexpr int NST = (NCH + NT - 1) / NT;
     extern __shared__ __attribute__((aligned(16))) uint8_t dwpw_stream_lds[];
     uint8_t* const lds = dwpw_stream_lds;
-    constexpr int PANEL0 = 2 * HALO, WTS0 = PANEL0 + G::PANEL, TAB0 = WTS0 + G::WTS, OUT0 = TAB0 + G::TAB;
+    constexpr int PANEL0 = HALO, WTS0 = PANEL0 + G::PANEL, TAB0 = WTS0 + G::WTS, OUT0 = TAB0 + G::TAB;
 
     const int tid = threadIdx.x;
     const int lane = tid & 63, wave = tid >> 6;
@@ -179,8 +188,8 @@ __global__ __launch_bounds__(256) void DwPwStreamKernel(DwPwStreamArgs a)
     // ---- depthwise roles: lane (j, g): pixel j of a group of 16 and tap slot g as an operand, channel quad g as a result --
     const int j = lane & 15, g = lane >> 4;
     const int rj = j / TW, cj = j % TW;
-    const int cg0 = NCG > 4 ? wave * CGW : wave % NCG;
-    const int pg0 = NCG > 4 ? 0 : wave / NCG;
+    const int cg0 = NCG > NW ? wave * CGW : wave % NCG;
+    const int pg0 = NCG > NW ? 0 : wave / NCG;
     int lds_tap[3];
     v4i wa[CGW][3], corr4[CGW];
     Fast4 f4[CGW];
@@ -224,20 +233,16 @@ __global__ __launch_bounds__(256) void DwPwStreamKernel(DwPwStreamArgs a)
     // the wave's output area [64 pixels][LDO]; lane writes dwords at (pixel frag_row of tile mt, channels 8 q + 4 frag_half of tile nt)
     const int out_area = OUT0 + wave * 64 * LDO;
     const int out_write = out_area + frag_row * LDO + 4 * frag_half;
-    // 16-byte pieces of that area: piece id = k 64 + lane -> (pixel id / (SC / 16), part id % (SC / 16))
+    // 16-byte pieces of that area: piece id = k 64 + lane -> (pixel id / PPP, part id % PPP).  64 / PPP pixels per store
+    // instruction are whole tile rows, so a lane keeps its column and part; only the row moves with k.
     constexpr int PPP = G::SC / 16;
-    int out_read[QUADS], y_lane[QUADS], y_col[QUADS];
-#pragma unroll
-    for (int k = 0; k < QUADS; ++k)
-    {
-        const int id = k * 64 + lane;
-        const int sr = id / PPP, part = id % PPP;
-        const int px = m0 * 32 + sr;
-        const int row = px / TW, col = px % TW;
-        out_read[k] = out_area + sr * LDO + part * 16;
-        y_lane[k] = (row * a.Wo + col) * NO + n0 * 32 + part * 16;
-        y_col[k] = col;
-    }
+    constexpr int RPS = 64 / PPP / TW;                     // tile rows per store instruction
+    static_assert((64 / PPP) % TW == 0, "whole tile rows per store instruction");
+    const int sr0 = lane / PPP, part0 = lane % PPP;
+    const int y_col = (m0 * 32 + sr0) % TW;
+    const int out_read = out_area + sr0 * LDO + part0 * 16;
+    const int y_lane = (((m0 * 32 + sr0) / TW) * a.Wo + y_col) * NO + n0 * 32 + part0 * 16;
+    const int y_step = RPS * a.Wo * NO;
     const int image_bytes = a.Ho * a.Wo * NO;
 
     int out_base = 0, out_n = -1, out_cols = 0;
@@ -246,8 +251,8 @@ __global__ __launch_bounds__(256) void DwPwStreamKernel(DwPwStreamArgs a)
 #pragma unroll
         for (int k = 0; k < QUADS; ++k)
         {
-            const v4i v = *reinterpret_cast<const v4i*>(lds + out_read[k]);
-            const int yo = y_col[k] < out_cols ? out_base + y_lane[k] : static_cast<int>(0x80000000u);
+            const v4i v = *reinterpret_cast<const v4i*>(lds + out_read + k * (64 / PPP) * LDO);
+            const int yo = y_col < out_cols ? out_base + y_lane + k * y_step : static_cast<int>(0x80000000u);
             __builtin_amdgcn_raw_buffer_store_b128(v, yrsrc, yo, 0, 0);
         }
     };
@@ -314,10 +319,10 @@ __global__ __launch_bounds__(256) void DwPwStreamKernel(DwPwStreamArgs a)
     };
 
     issue(item);
-    int buf = 0;
     while (true)
     {
-        commit(buf * HALO);
+        // (one halo buffer: its readers, the depthwise phase of the item before, all passed that item's second barrier)
+        commit(0);
         // all waves are done with the item before (its panel has been multiplied) and this item's halo is in LDS; on the first
         // pass the barrier also orders the resident weights and table rows before their first use
         __syncthreads();
@@ -327,12 +332,11 @@ __global__ __launch_bounds__(256) void DwPwStreamKernel(DwPwStreamArgs a)
         const int next = item + step;
         const bool more = next < item_end;
         if (more) issue(next);
-        depthwise(buf * HALO);
+        depthwise(0);
         __syncthreads();                                   // the panel is complete
         pointwise(item);
         if (!more) break;
         item = next;
-        buf ^= 1;
     }
     store_outputs();
 }

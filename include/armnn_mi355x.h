@@ -121,7 +121,7 @@ int  mi355x_abi_version(void);
  *   the lower half of the output channels and XCDs 4-7 the upper half (half the weights per XCD, every activation row
  *   fetched twice), 0 chooses 2 where the weights outweigh a quarter of the activations of a launch.  Identical bytes.
  *   "dwpw_stream" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a depthwise layer of 32, 64 (stride 2) or
- *   128 channels and the pointwise layer behind it (64, 128, 128 output channels) on the persistent kernel that keeps the
+ *   128 channels and the pointwise layer behind it (64, 128, 128 / 256 output channels) on the persistent kernel that keeps the
  *   pointwise weights in on-chip memory (identical bytes; lets tests compare it with the older fused kernel).
  *   "dwpw_panel" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a stride-1 depthwise layer of 256 or 512
  *   channels and a pointwise layer of 256 or 512 output channels on the kernel that gives a block an 8 x 8 pixel tile over

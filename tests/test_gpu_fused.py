@@ -35,12 +35,15 @@ PANEL_PAIRS = [
 ]
 
 
-# pairs the persistent kernel with resident pointwise weights takes (32 -> 64, 64 -> 128 at stride 2, 128 -> 128): enough
+# pairs the persistent kernel with resident pointwise weights takes (32 -> 64, 64 -> 128 at stride 2, 128 -> 128, 128 -> 256
+# at stride 2): enough
 # images that a block walks several items, ragged maps, both activation types
 STREAM_PAIRS = [
     ("stream_c32_co64_u8_112", 12, 112, 112, 32, 64, 1, U8, cases.RELU6, cases.RELU6),      # MobileNetV1 dw1+pw1
     ("stream_c64_co128_u8_112_s2", 12, 112, 112, 64, 128, 2, U8, cases.RELU6, cases.RELU6),  # dw2+pw2
     ("stream_c128_co128_u8_56", 12, 56, 56, 128, 128, 1, U8, cases.RELU6, cases.RELU6),      # dw3+pw3
+    ("stream_c128_co256_u8_56_s2", 20, 56, 56, 128, 256, 2, U8, cases.RELU6, cases.RELU6),   # dw4+pw4
+    ("stream_c128_co256_s8_ragged_s2", 30, 23, 31, 128, 256, 2, S8, cases.RELU, cases.RELU6),
     ("stream_c32_co64_s8_ragged", 30, 50, 35, 32, 64, 1, S8, cases.RELU, (0, 0.0, 0.0)),
     ("stream_c64_co128_s8_ragged_s2", 25, 45, 51, 64, 128, 2, S8, (0, 0.0, 0.0), cases.RELU6),
     ("stream_c128_co128_s8_ragged", 40, 13, 29, 128, 128, 1, S8, cases.RELU6, cases.RELU),
@@ -48,7 +51,7 @@ STREAM_PAIRS = [
 ]
 
 
-@pytest.mark.parametrize("pair", STREAM_PAIRS + PAIRS[:3], ids=[p[0] for p in STREAM_PAIRS + PAIRS[:3]])
+@pytest.mark.parametrize("pair", STREAM_PAIRS + PAIRS[:4], ids=[p[0] for p in STREAM_PAIRS + PAIRS[:4]])
 def test_stream_kernel_is_taken_and_equals_the_older_fused_kernel(pair):
     shim.Device()
     dw, pw = _make(*pair)
@@ -108,7 +111,7 @@ def test_panel_kernel_is_taken_and_equals_the_older_fused_kernel(pair):
     np.testing.assert_array_equal(a, b)
 
 
-@pytest.mark.parametrize("pair", PAIRS + PANEL_PAIRS + STREAM_PAIRS[3:], ids=[p[0] for p in PAIRS + PANEL_PAIRS + STREAM_PAIRS[3:]])
+@pytest.mark.parametrize("pair", PAIRS + PANEL_PAIRS + STREAM_PAIRS[4:], ids=[p[0] for p in PAIRS + PANEL_PAIRS + STREAM_PAIRS[4:]])
 def test_fused_equals_two_layers(port, pair):
     print("pair", pair, flush=True)
     shim.Device()
