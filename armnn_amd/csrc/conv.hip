@@ -1385,8 +1385,10 @@ int LaunchDwPwStream(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, int w
 bool DwPwPanelShape(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, int* kt, int* nq)
 {
     const mi355x_conv2d_desc& a = dw->d;
-    if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || dw->w_dot4b || a.stride_x != 1 || a.stride_y != 1) return false;
+    if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || dw->w_dot4b || a.stride_x != a.stride_y || a.stride_x > 2) return false;
     if (a.out_c != a.in_c || (a.out_c != 256 && a.out_c != 512)) return false;
+    // stride 2 (a 17 x 17 halo per 128 channels): built for 256 -> 512 channels
+    if (a.stride_x == 2 && (a.out_c != 256 || pw->d.out_c != 512)) return false;
     if (pw->zw_neg != 0 || pw->K_pad != static_cast<int>(a.out_c) || !pw->bk128 || !pw->w_mfma || pw->pw_bn != 0) return false;
     if (pw->d.out_c != 256 && pw->d.out_c != 512) return false;
     if (static_cast<long long>(a.in_h) * a.in_w * a.in_c >= (1ll << 31)) return false;
@@ -1395,15 +1397,16 @@ bool DwPwPanelShape(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, int* k
     return true;
 }
 
-template <int KT, int NQ>
+template <int KT, int NQ, int S = 1>
 int LaunchDwPwPanelT(const DwPwPanelArgs& a, hipStream_t stream)
 {
-    constexpr int smem = DwPwPanelGeom<KT, NQ>::SMEM;
+    constexpr int smem = DwPwPanelGeom<KT, NQ, S>::SMEM;
     static_assert(smem <= 156 * 1024, "LDS of one CU");
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&DwPwPanelKernel<KT, NQ>), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&DwPwPanelKernel<KT, NQ, S>), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);
-    NoteKernel("DwPwPanelKernel<%d, %d>", KT, NQ);
-    hipLaunchKernelGGL((DwPwPanelKernel<KT, NQ>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(512), smem, stream, a);
+    if (S == 1) NoteKernel("DwPwPanelKernel<%d, %d>", KT, NQ);
+    else NoteKernel("DwPwPanelKernel<%d, %d, %d>", KT, NQ, S);
+    hipLaunchKernelGGL((DwPwPanelKernel<KT, NQ, S>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(512), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;
 }
@@ -1433,8 +1436,9 @@ int LaunchDwPwPanel(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, int kt
         if (!d_stamps) MI355X_HIP(hipMalloc(reinterpret_cast<void**>(&d_stamps), 65536 * 16 * 8));
         a.stamps = a.total_tiles <= 65536 - 8 ? d_stamps : nullptr;
     }
-    int rc = kt == 2 ? (nq == 1 ? LaunchDwPwPanelT<2, 1>(a, stream) : LaunchDwPwPanelT<2, 2>(a, stream))
-                     : (nq == 1 ? LaunchDwPwPanelT<4, 1>(a, stream) : LaunchDwPwPanelT<4, 2>(a, stream));
+    int rc = dw->d.stride_x == 2 ? LaunchDwPwPanelT<2, 2, 2>(a, stream)
+             : kt == 2 ? (nq == 1 ? LaunchDwPwPanelT<2, 1>(a, stream) : LaunchDwPwPanelT<2, 2>(a, stream))
+                       : (nq == 1 ? LaunchDwPwPanelT<4, 1>(a, stream) : LaunchDwPwPanelT<4, 2>(a, stream));
     if (a.stamps && rc == 0 && ++launches == 40)
     {
         MI355X_HIP(hipStreamSynchronize(stream));
@@ -1459,6 +1463,7 @@ int LaunchDwPwPanel(const mi355x_conv2d_s* dw, const mi355x_conv2d_s* pw, int kt
     }
     return rc;
 #else
+    if (dw->d.stride_x == 2) return LaunchDwPwPanelT<2, 2, 2>(a, stream);
     if (kt == 2) return nq == 1 ? LaunchDwPwPanelT<2, 1>(a, stream) : LaunchDwPwPanelT<2, 2>(a, stream);
     return nq == 1 ? LaunchDwPwPanelT<4, 1>(a, stream) : LaunchDwPwPanelT<4, 2>(a, stream);
 #endif

@@ -1,4 +1,4 @@
-// Depthwise 3x3 (stride 1) + the pointwise 1x1 convolution that consumes it as ONE kernel, for 256 or 512 channels between
+// Depthwise 3x3 (stride 1 or 2) + the pointwise 1x1 convolution that consumes it as ONE kernel, for 256 or 512 channels between
 // them: a block of eight waves owns an 8 x 8 pixel tile of one image over ALL channels, and a CU holds one block.
 //
 //   The intermediate tensor never leaves the CU, and it is produced in exactly the pieces the GEMM consumes: the
@@ -36,7 +36,7 @@ namespace mi355x
 
 struct DwPwPanelArgs
 {
-    // depthwise 3x3, stride 1, multiplier 1, C % 128 == 0
+    // depthwise 3x3, multiplier 1, C % 128 == 0
     const uint8_t*  x;
     const uint8_t*  pad16;      // 16 bytes that become the depthwise padding value under dw_xor
     const uint32_t* wpack;      // [C][4] dwords, rows of the 3x3 filter per channel (Dw3x3Args::wpack)
@@ -62,16 +62,17 @@ struct DwPwPanelArgs
 #endif
 };
 
-template <int KT, int NQ>
+template <int KT, int NQ, int S = 1>
 struct DwPwPanelGeom
 {
     static constexpr int NCOL = 256 * NQ;             // output channels
     static constexpr int NT = 4 * NQ;                 // 64-channel weight tiles per k-tile
-    static constexpr int HR = 10, HC = 10;            // halo of an 8 x 8 tile
+    static constexpr int HR = 7 * S + 3, HC = 7 * S + 3;   // halo of an 8 x 8 tile of outputs: 10 x 10 or 17 x 17 input pixels
+    static constexpr int NCHUNK = HR * HC * 8;        // 16-byte pieces of a halo (128 channels per pixel)
     static constexpr int HPITCH = 144;                // bytes per halo pixel in LDS: 128 + 16, so that the 16-byte reads of 8
-                                                      // neighbouring pixels fall on different bank quads
-    static constexpr int HROWP = 1664;                // bytes per halo row: >= 10 pixels and 128 mod 256, so that the reads of
-                                                      // the pixel group's second row take the quads the first row's leave free
+                                                      // neighbouring pixels fall on different bank quads (stride 1)
+    static constexpr int HROWP = S == 1 ? 1664 : HC * HPITCH;   // bytes per halo row; at stride 1 >= 10 pixels and 128 mod 256, so that
+                                                      // the reads of the pixel group's second row take the quads the first row's leave free
     static constexpr int HALO = HR * HROWP;
     static constexpr int LDO = NCOL + 16;
     static constexpr int PANEL = KT * 64 * 128;
@@ -82,11 +83,12 @@ struct DwPwPanelGeom
     static constexpr int SMEM = PANEL + TAB + WORK;
 };
 
-// KT = C / 128 (2 or 4), NQ = Co / 256 (1 or 2).  512 threads.
-template <int KT, int NQ>
+// KT = C / 128 (2 or 4), NQ = Co / 256 (1 or 2), S = depthwise stride.  512 threads.
+template <int KT, int NQ, int S = 1>
 __global__ __launch_bounds__(512) void DwPwPanelKernel(DwPwPanelArgs a)
 {
-    using G = DwPwPanelGeom<KT, NQ>;
+    using G = DwPwPanelGeom<KT, NQ, S>;
+    constexpr int NCHUNK = G::NCHUNK, NHS = (G::NCHUNK + 511) / 512;     // halo pieces, and pieces per thread
     constexpr int NCOL = G::NCOL, NT = G::NT, HC = G::HC, HALO = G::HALO, LDO = G::LDO, HPITCH = G::HPITCH, HROWP = G::HROWP;
     constexpr int NTHR = 512;
     typedef __attribute__((address_space(3))) void* LdsPtr;
@@ -124,41 +126,35 @@ __global__ __launch_bounds__(512) void DwPwPanelKernel(DwPwPanelArgs a)
     {
         const int t = 4 * m + dg;
         const int tc = min(t, 8);                      // slots past the ninth tap read the ninth; their weights are zero
-        dtap[m] = (drj + tc / 3) * HROWP + (dcj + tc % 3) * HPITCH + wave * 16;
+        dtap[m] = (drj * S + tc / 3) * HROWP + (dcj * S + tc % 3) * HPITCH + wave * 16;
         dwrow[m] = tc / 3;
         dwshift[m] = t < 9 ? 8 * (tc % 3) : 24;        // shift 24: the zero byte of a packed filter row
     }
-    // ---- staging of a halo: 800 chunks of 16 bytes, at most two per thread; only the channel block moves from phase to phase
-    const int iy_org = ty * 8 - a.pad_top;
-    const int ix_org = tx * 8 - a.pad_left;
+    // ---- staging of a halo: NCHUNK pieces of 16 bytes, NHS per thread at most; only the channel block moves from phase to phase
+    const int iy_org = ty * 8 * S - a.pad_top;
+    const int ix_org = tx * 8 * S - a.pad_left;
     const uint8_t* const xn = a.x + static_cast<long long>(n) * a.H * a.W * a.C;
     const int dxm = static_cast<int>(a.dw_xor);
-    const uint8_t* hsrc[2];
-    bool hok[2];
+    int hoff[NHS], hlds[NHS];                              // offset within the image (-1: outside, reads the padding), place in LDS (-1: none)
 #pragma unroll
-    for (int k = 0; k < 2; ++k)
+    for (int k = 0; k < NHS; ++k)
     {
-        const int i = min(tid + k * NTHR, 799);
+        const int i = min(tid + k * NTHR, NCHUNK - 1);
         const int part = i & 7, pix = i >> 3;
         const int col = pix % HC, hrow = pix / HC;
         const int iy = iy_org + hrow, ix = ix_org + col;
-        hok[k] = static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && static_cast<unsigned>(ix) < static_cast<unsigned>(a.W);
-        hsrc[k] = xn + (static_cast<long long>(iy) * a.W + ix) * a.C + part * 16;
+        const bool ok = static_cast<unsigned>(iy) < static_cast<unsigned>(a.H) && static_cast<unsigned>(ix) < static_cast<unsigned>(a.W);
+        hoff[k] = ok ? (iy * a.W + ix) * a.C + part * 16 : -1;
+        hlds[k] = tid + k * NTHR < NCHUNK ? hrow * HROWP + col * HPITCH + part * 16 : -1;
     }
-    auto load_halo = [&](int kt, v4i (&h)[2]) {
+    auto load_halo = [&](int kt, v4i (&h)[NHS]) {
 #pragma unroll
-        for (int k = 0; k < 2; ++k) h[k] = *reinterpret_cast<const v4i*>(hok[k] ? hsrc[k] + kt * 128 : a.pad16);
+        for (int k = 0; k < NHS; ++k) h[k] = *reinterpret_cast<const v4i*>(hoff[k] >= 0 ? xn + hoff[k] + kt * 128 : a.pad16);
     };
-    int hlds[2];
+    auto store_halo = [&](const v4i (&h)[NHS]) {
 #pragma unroll
-    for (int k = 0; k < 2; ++k)
-    {
-        const int i = min(tid + k * NTHR, 799);
-        hlds[k] = ((i >> 3) / HC) * HROWP + ((i >> 3) % HC) * HPITCH + (i & 7) * 16;
-    }
-    auto store_halo = [&](const v4i (&h)[2]) {
-        *reinterpret_cast<v4i*>(halo + hlds[0]) = h[0] ^ dxm;
-        if (tid + NTHR < 800) *reinterpret_cast<v4i*>(halo + hlds[1]) = h[1] ^ dxm;
+        for (int k = 0; k < NHS; ++k)
+            if (hlds[k] >= 0) *reinterpret_cast<v4i*>(halo + hlds[k]) = h[k] ^ dxm;
     };
 
     // ---- GEMM roles: wave (wm, wq) owns pixel rows [32 wm, 32 wm + 32) x output channels [64 NQ wq, 64 NQ (wq + 1)) ----------
@@ -189,7 +185,7 @@ __global__ __launch_bounds__(512) void DwPwPanelKernel(DwPwPanelArgs a)
             const int src_row = r == 0 ? 2 : r == 1 ? 6 : r == 2 ? 4 : 7;
             tv[i] = *reinterpret_cast<const float4*>(a.pw_ct.p + src_row * a.pw_ct.stride + col4 * 4);
         }
-        v4i h0[2];
+        v4i h0[NHS];
         load_halo(0, h0);
 #pragma unroll
         for (int i = 0; i < TABV; ++i)
@@ -214,7 +210,7 @@ __global__ __launch_bounds__(512) void DwPwPanelKernel(DwPwPanelArgs a)
         const int cq = c0 + 4 * dg;                        // the four channels this lane requantizes
         const v4i corr4 = *reinterpret_cast<const v4i*>(a.dw_corr + cq);
         const Fast4 f4 = LoadFast4(a.dw_ct, cq);
-        v4i hn[2];
+        v4i hn[NHS];
         if (kt + 1 < KT) load_halo(kt + 1, hn);
         load_weights(kt);
 
@@ -235,9 +231,9 @@ __global__ __launch_bounds__(512) void DwPwPanelKernel(DwPwPanelArgs a)
 #pragma unroll
         for (int u = 0; u < 4; ++u)
         {
-            const v4i b0 = *reinterpret_cast<const v4i*>(hb + dtap[0] + u * 2 * HROWP);
-            const v4i b1 = *reinterpret_cast<const v4i*>(hb + dtap[1] + u * 2 * HROWP);
-            const v4i b2 = *reinterpret_cast<const v4i*>(hb + dtap[2] + u * 2 * HROWP);
+            const v4i b0 = *reinterpret_cast<const v4i*>(hb + dtap[0] + u * 2 * S * HROWP);
+            const v4i b1 = *reinterpret_cast<const v4i*>(hb + dtap[1] + u * 2 * S * HROWP);
+            const v4i b2 = *reinterpret_cast<const v4i*>(hb + dtap[2] + u * 2 * S * HROWP);
             v4i dacc = corr4;
             dacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wa[0], b0, dacc, 0, 0, 0);
             dacc = __builtin_amdgcn_mfma_i32_16x16x64_i8(wa[1], b1, dacc, 0, 0, 0);

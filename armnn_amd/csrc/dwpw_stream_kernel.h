@@ -62,7 +62,7 @@ struct DwPwStreamArgs
 template <int S, int C, int NO, int TH, int TW, int NWAVES = 4>
 struct DwPwStreamGeom
 {
-    static_assert(C == 32 || C == 64 || C == 128, "channels between the layers");
+    static_assert(C == 32 || C == 64 || C == 128 || C == 256, "channels between the layers");
     static_assert(NO == 64 || NO == 128 || NO == 256, "output channels");
     static_assert(TW == 8 || TW == 16, "a group of 16 pixels is one or two whole tile rows");
     static constexpr int NW = NWAVES, NT = 64 * NW;

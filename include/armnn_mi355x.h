@@ -123,7 +123,7 @@ int  mi355x_abi_version(void);
  *   "dwpw_stream" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a depthwise layer of 32, 64 (stride 2) or
  *   128 channels and the pointwise layer behind it (64, 128, 128 / 256 output channels) on the persistent kernel that keeps the
  *   pointwise weights in on-chip memory (identical bytes; lets tests compare it with the older fused kernel).
- *   "dwpw_panel" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a stride-1 depthwise layer of 256 or 512
+ *   "dwpw_panel" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a depthwise layer of 256 or 512
  *   channels and a pointwise layer of 256 or 512 output channels on the kernel that gives a block an 8 x 8 pixel tile over
  *   all channels (identical bytes; lets tests compare it with the older fused kernel).
  *   "chain_stages" = 2 | 3 | 4: LDS stages of the matrix-core tiles inside a layer chain; "chain_blocks_per_cu" = 0 .. 16:
@@ -258,10 +258,13 @@ int mi355x_conv2d_run_add(mi355x_conv2d_t plan, uint32_t batch, const void* inpu
  * pixels (14 x 14, 7 x 7 ...), the 1x1 layer's input channels are a multiple of 128, its weights have no zero point and
  * the shared channel count is a multiple of 64.  Same contract: the bytes of the two layers run one after the other. */
 int mi355x_conv2d_fusable(mi355x_conv2d_t first, mi355x_conv2d_t second);
-/* 1 when running the pair as one launch is what the library recommends at this batch (today: a stride-1 depthwise layer
- * over 256 or 512 channels and the pointwise layer of 256 or 512 output channels behind it, which run on the kernel that
- * gives a block an 8 x 8 pixel tile over all channels), else 0; never an error.  No counterpart in the reference, which
- * has no fused workloads on CpuRef. */
+/* 1 when running the pair as one launch is what the library recommends at this batch, else 0; never an error.  Today:
+ * a depthwise layer over 32, 64 (stride 2) or 128 channels and the pointwise layer behind it (64, 128, 128 or -- at stride
+ * 2 -- 256 output channels) in launches of at least 1024 tiles of 8 x 8 output pixels, which run on the persistent kernel
+ * that keeps the pointwise weights on chip; and a depthwise layer over 256 or 512 channels (stride 1, or stride 2 from 256
+ * to 512 channels) and the pointwise layer of 256 or 512 output channels behind it in launches of at least 100 such tiles,
+ * which run on the kernel that gives a block an 8 x 8 pixel tile over all channels.  No counterpart in the reference,
+ * which has no fused workloads on CpuRef. */
 int mi355x_conv2d_fusion_pays(mi355x_conv2d_t first, mi355x_conv2d_t second, uint32_t batch);
 int mi355x_conv2d_run_fused(mi355x_conv2d_t first, mi355x_conv2d_t second, uint32_t batch,
                             const void* input_dev, void* output_dev, mi355x_stream_t stream);

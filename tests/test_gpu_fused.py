@@ -25,13 +25,16 @@ PAIRS = [
 ]
 
 
-# pairs the one-block-per-tile-over-all-channels kernel takes: stride 1, 256 or 512 channels in between, 256 or 512 out
+# pairs the one-block-per-tile-over-all-channels kernel takes: 256 or 512 channels in between, 256 or 512 out, stride 1 (or
+# stride 2 from 256 to 512 channels)
 PANEL_PAIRS = [
     ("panel_c512_co512_u8_14", 5, 14, 14, 512, 512, 1, U8, cases.RELU6, cases.RELU6),      # the MobileNetV1 pairs dw7+pw7 ... dw11+pw11
     ("panel_c256_co256_u8_28", 3, 28, 28, 256, 256, 1, U8, cases.RELU6, cases.RELU6),      # dw5+pw5
     ("panel_c256_co512_s8_ragged", 2, 13, 9, 256, 512, 1, S8, cases.RELU, (0, 0.0, 0.0)),
     ("panel_c512_co256_s8_tiny", 1, 3, 5, 512, 256, 1, S8, (0, 0.0, 0.0), cases.RELU6),
     ("panel_c512_co512_s8_17x23", 2, 17, 23, 512, 512, 1, S8, cases.RELU6, cases.RELU),
+    ("panel_c256_co512_u8_28_s2", 5, 28, 28, 256, 512, 2, U8, cases.RELU6, cases.RELU6),   # dw6+pw6
+    ("panel_c256_co512_s8_ragged_s2", 3, 19, 25, 256, 512, 2, S8, cases.RELU, cases.RELU6),
 ]
 
 
