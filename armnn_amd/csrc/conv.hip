@@ -1404,8 +1404,7 @@ int LaunchDwPwPanelT(const DwPwPanelArgs& a, hipStream_t stream)
     static_assert(smem <= 156 * 1024, "LDS of one CU");
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&DwPwPanelKernel<KT, NQ, S>), hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);
-    if (S == 1) NoteKernel("DwPwPanelKernel<%d, %d>", KT, NQ);
-    else NoteKernel("DwPwPanelKernel<%d, %d, %d>", KT, NQ, S);
+    NoteKernel("DwPwPanelKernel<%d, %d, %d>", KT, NQ, S);
     hipLaunchKernelGGL((DwPwPanelKernel<KT, NQ, S>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(512), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;

@@ -43,7 +43,8 @@ RIDGE_OPS_PER_BYTE = INT8_MFMA_PEAK_OPS / HBM_PEAK_BYTES
 
 TRAFFIC_PROFILES = {
     # (network name, images per launch) -> rocprofv3 counter summary written by `python -m armnn_amd.profile_summary traffic`
-    ("mobilenet_v1_1.0_224", 32): os.path.join(ROOT, "profiles", "mobilenet_v1_b64_hbm_traffic.md"),
+    ("mobilenet_v1_1.0_224", 64): os.path.join(ROOT, "profiles", "mobilenet_v1_b64_hbm_traffic.md"),
+    ("resnet50_224", 16): os.path.join(ROOT, "profiles", "resnet50_b32_hbm_traffic.md"),
 }
 
 
