@@ -239,6 +239,9 @@ BackendCapabilities Mi355xBackend::GetCapabilities() const
 //   CL backends do (src/backends/aclCommon/ArmComputeSubgraphUtils.hpp:60-109).
 // * A Convolution2d without an activation whose output goes to one Addition of this backend and nowhere else is marked
 //   (Mi355xFeedsOnlyAnAddition): the two workloads may then run as one launch (Mi355xAdditionWorkload).
+// * A DepthwiseConvolution2d whose output goes to one unpadded 1x1 stride-1 Convolution2d of this backend and nowhere else
+//   is marked (Mi355xLayerNote, which also carries the fused activation): the two workloads may then run as one launch
+//   (Mi355xConvolution2dWorkload::TakeOver).
 // * A Reshape that only flattens the dimensions behind the batch, in front of a FullyConnected, is dropped: the
 //   FullyConnected reads the unflattened tensor (same bytes in the same order).
 // * A constant Pad of height and width in front of a Convolution2d, DepthwiseConvolution2d or Pooling2d moves into that
@@ -252,8 +255,11 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
     std::set<const IConnectableLayer*> consumed;
     // BackendOptions("Mi355x", {{"FuseAdditions", false}}) among the network's model options keeps every Addition a launch of its own
     bool fuseAdditions = true;
+    // ... {{"FuseDepthwisePointwise", false}} keeps every depthwise layer and the 1x1 convolution behind it two launches
+    bool fuseDepthwisePointwise = true;
     ParseOptions(modelOptions, Mi355xBackendId(), [&](const std::string& name, const BackendOptions::Var& value) {
         if (name == "FuseAdditions" && value.IsBool()) fuseAdditions = value.AsBool();
+        if (name == "FuseDepthwisePointwise" && value.IsBool()) fuseDepthwisePointwise = value.AsBool();
     });
 
     for (IConnectableLayer* il : layers)
@@ -330,7 +336,32 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
                 next->GetInputSlot(0).GetConnectedOutputSlot() != next->GetInputSlot(1).GetConnectedOutputSlot())
                 residual = true;
         }
-        if (!pad && !act && !residual && !flat) continue;
+        // a DepthwiseConvolution2d (with the Activation fused into it, if any) whose only consumer is an unpadded 1x1 stride-1
+        // Convolution2d of this backend: the two workloads may run as one launch (Mi355xConvolution2dWorkload::TakeOver)
+        bool pointwiseNext = false;
+        if (fuseDepthwisePointwise && type == LayerType::DepthwiseConvolution2d)
+        {
+            Layer* lastOfThis = act ? act : base;
+            if (lastOfThis->GetOutputSlot(0).GetNumConnections() == 1)
+            {
+                InputSlot* to = lastOfThis->GetOutputSlot(0).GetConnections()[0];
+                Layer* next = &to->GetOwningLayer();
+                if (next->GetType() == LayerType::Convolution2d && members.count(next) && to->GetSlotIndex() == 0)
+                {
+                    const auto& nd = static_cast<const Convolution2dDescriptor&>(next->GetParameters());
+                    const OutputSlot* weights = next->GetInputSlot(1).GetConnectedOutputSlot();
+                    pointwiseNext = weights != nullptr && weights->GetTensorInfo().GetNumDimensions() == 4 &&
+                                    weights->GetTensorInfo().GetShape()[1] == 1 && weights->GetTensorInfo().GetShape()[2] == 1 &&
+                                    nd.m_StrideX == 1 && nd.m_StrideY == 1 && nd.m_PadLeft == 0 && nd.m_PadRight == 0 && nd.m_PadTop == 0 &&
+                                    nd.m_PadBottom == 0 && nd.m_DataLayout == DataLayout::NHWC;
+                }
+            }
+            // (a layer that already carries the mark needs no second replacement)
+            if (pointwiseNext && !pad && !act)
+                if (const Mi355xLayerNote* note = Mi355xLayerNote::From(base->GetAdditionalInformation<ActivationDescriptor>().get()))
+                    if (note->onlyConsumerIsAPointwiseConvolution) pointwiseNext = false;
+        }
+        if (!pad && !act && !residual && !flat && !pointwiseNext) continue;
 
         std::string name = base->GetName();
         if (pad) name = std::string("folded-") + pad->GetName() + "-into-" + name;
@@ -352,7 +383,13 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
         }
         Layer* last = act ? act : base;
         replacement->GetOutputSlot(0).SetTensorInfo(last->GetOutputSlot(0).GetTensorInfo());
-        if (act)
+        if (pointwiseNext)
+        {
+            auto carried = base->GetAdditionalInformation<ActivationDescriptor>();
+            PolymorphicDowncast<Layer*>(replacement)->SetAdditionalInfoForObject(
+                Mi355xLayerNote::Make(act ? &static_cast<const ActivationDescriptor&>(act->GetParameters()) : carried.get(), true));
+        }
+        else if (act)
             PolymorphicDowncast<Layer*>(replacement)->SetAdditionalInfoForObject(
                 std::make_shared<ActivationDescriptor>(static_cast<const ActivationDescriptor&>(act->GetParameters())));
         else if (auto carried = base->GetAdditionalInformation<ActivationDescriptor>())

@@ -28,6 +28,15 @@ struct Mi355xWorkloadFactory::Candidate
         convolution = nullptr;
         return w;
     }
+    // the depthwise workload created last, while it is marked as feeding one pointwise convolution only
+    Mi355xDepthwiseConvolution2dWorkload* depthwise = nullptr;
+    Mi355xDepthwiseConvolution2dWorkload* TakeDepthwise()
+    {
+        std::lock_guard<std::mutex> lock(mutex);
+        Mi355xDepthwiseConvolution2dWorkload* w = depthwise;
+        depthwise = nullptr;
+        return w;
+    }
 };
 
 namespace
@@ -47,6 +56,23 @@ public:
     ~CandidateConvolution() override { m_Withdraw(this); }
 private:
     std::function<void(Mi355xConvolution2dWorkload*)> m_Withdraw;
+};
+
+// the same for the depthwise workload
+class CandidateDepthwise final : public Mi355xDepthwiseConvolution2dWorkload
+{
+public:
+    template <typename C>
+    CandidateDepthwise(const DepthwiseConvolution2dQueueDescriptor& d, const WorkloadInfo& info, std::shared_ptr<C> slot)
+        : Mi355xDepthwiseConvolution2dWorkload(d, info), m_Withdraw([slot](Mi355xDepthwiseConvolution2dWorkload* self) {
+              std::lock_guard<std::mutex> lock(slot->mutex);
+              if (slot->depthwise == self) slot->depthwise = nullptr;
+          })
+    {
+    }
+    ~CandidateDepthwise() override { m_Withdraw(this); }
+private:
+    std::function<void(Mi355xDepthwiseConvolution2dWorkload*)> m_Withdraw;
 };
 }
 
@@ -74,11 +100,14 @@ std::unique_ptr<IWorkload> Mi355xWorkloadFactory::CreateWorkload(LayerType type,
 {
     // constants write no tensor another workload's operand could share an address with: they leave the candidate alone
     Mi355xConvolution2dWorkload* candidate = type == LayerType::Constant ? nullptr : m_Candidate->Take();
+    Mi355xDepthwiseConvolution2dWorkload* depthwise = type == LayerType::Constant ? nullptr : m_Candidate->TakeDepthwise();
     switch (type)
     {
         case LayerType::Convolution2d:
         {
             auto w = std::make_unique<CandidateConvolution>(*PolymorphicDowncast<const Convolution2dQueueDescriptor*>(&descriptor), info, m_Candidate);
+            // the depthwise layer created just before, marked as feeding only this kind of convolution: the two run as a pair
+            w->TakeOver(depthwise);
             if (w->FeedsOnlyAnAddition())
             {
                 std::lock_guard<std::mutex> lock(m_Candidate->mutex);
@@ -87,7 +116,15 @@ std::unique_ptr<IWorkload> Mi355xWorkloadFactory::CreateWorkload(LayerType type,
             return w;
         }
         case LayerType::DepthwiseConvolution2d:
-            return std::make_unique<Mi355xDepthwiseConvolution2dWorkload>(*PolymorphicDowncast<const DepthwiseConvolution2dQueueDescriptor*>(&descriptor), info);
+        {
+            auto w = std::make_unique<CandidateDepthwise>(*PolymorphicDowncast<const DepthwiseConvolution2dQueueDescriptor*>(&descriptor), info, m_Candidate);
+            if (w->OnlyConsumerIsAPointwiseConvolution())
+            {
+                std::lock_guard<std::mutex> lock(m_Candidate->mutex);
+                m_Candidate->depthwise = w.get();
+            }
+            return w;
+        }
         case LayerType::FullyConnected:
             return std::make_unique<Mi355xFullyConnectedWorkload>(*PolymorphicDowncast<const FullyConnectedQueueDescriptor*>(&descriptor), info);
         case LayerType::Activation:

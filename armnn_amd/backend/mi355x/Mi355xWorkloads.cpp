@@ -10,6 +10,8 @@
 
 #include <algorithm>
 #include <atomic>
+#include <mutex>
+#include <set>
 #include <cstring>
 
 namespace armnn
@@ -126,6 +128,39 @@ ActivationDescriptor Mi355xFeedsOnlyAnAddition()
     return d;
 }
 
+// ---- the note on a depthwise layer ---------------------------------------------------------------------------------------
+namespace
+{
+std::mutex g_NotesMutex;
+std::set<const void*> g_Notes;
+std::atomic<unsigned long long> g_DepthwisePairsFormed{0}, g_DepthwisePairsRunFused{0}, g_DepthwisePairsRunApart{0};
+}
+
+std::shared_ptr<void> Mi355xLayerNote::Make(const ActivationDescriptor* activation, bool onlyConsumerIsAPointwiseConvolution)
+{
+    auto* note = new Mi355xLayerNote;
+    note->activation = activation ? *activation : Mi355xFeedsOnlyAnAddition();
+    note->onlyConsumerIsAPointwiseConvolution = onlyConsumerIsAPointwiseConvolution;
+    {
+        std::lock_guard<std::mutex> lock(g_NotesMutex);
+        g_Notes.insert(note);
+    }
+    return std::shared_ptr<void>(note, [](void* p) {
+        {
+            std::lock_guard<std::mutex> lock(g_NotesMutex);
+            g_Notes.erase(p);
+        }
+        delete static_cast<Mi355xLayerNote*>(p);
+    });
+}
+
+const Mi355xLayerNote* Mi355xLayerNote::From(const void* additionalInfo)
+{
+    if (!additionalInfo) return nullptr;
+    std::lock_guard<std::mutex> lock(g_NotesMutex);
+    return g_Notes.count(additionalInfo) ? static_cast<const Mi355xLayerNote*>(additionalInfo) : nullptr;
+}
+
 // ---- Convolution2d ---------------------------------------------------------------------------------------------------
 Mi355xConvolution2dWorkload::Mi355xConvolution2dWorkload(const Convolution2dQueueDescriptor& descriptor, const WorkloadInfo& info)
     : Mi355xBaseWorkload<Convolution2dQueueDescriptor>(descriptor, info), m_Info(info)
@@ -137,7 +172,25 @@ Mi355xConvolution2dWorkload::Mi355xConvolution2dWorkload(const Convolution2dQueu
 
 Mi355xConvolution2dWorkload::~Mi355xConvolution2dWorkload()
 {
+    if (m_Depthwise) m_Depthwise->ForgetPointwise();
     if (m_Plan) mi355x_conv2d_destroy(m_Plan);
+}
+
+unsigned long long Mi355xConvolution2dWorkload::DepthwisePairsFormed() { return g_DepthwisePairsFormed.load(); }
+unsigned long long Mi355xConvolution2dWorkload::DepthwisePairsRunFused() { return g_DepthwisePairsRunFused.load(); }
+unsigned long long Mi355xConvolution2dWorkload::DepthwisePairsRunApart() { return g_DepthwisePairsRunApart.load(); }
+
+bool Mi355xConvolution2dWorkload::TakeOver(Mi355xDepthwiseConvolution2dWorkload* depthwise)
+{
+    if (!depthwise || m_Depthwise || m_FeedsOnlyAnAddition || !depthwise->OnlyConsumerIsAPointwiseConvolution()) return false;
+    if (depthwise->GetOutputHandle() == nullptr || depthwise->GetOutputHandle() != m_Data.m_Inputs[0]) return false;
+    const Convolution2dDescriptor& p = m_Data.m_Parameters;
+    const TensorShape& w = m_Info.m_InputTensorInfos[1].GetShape();
+    if (w[1] != 1 || w[2] != 1 || p.m_StrideX != 1 || p.m_StrideY != 1 || p.m_PadLeft || p.m_PadRight || p.m_PadTop || p.m_PadBottom) return false;
+    m_Depthwise = depthwise;
+    depthwise->LeaveExecutionTo(this);
+    g_DepthwisePairsFormed.fetch_add(1);
+    return true;
 }
 
 void Mi355xConvolution2dWorkload::BuildPlan() const
@@ -181,6 +234,37 @@ void Mi355xConvolution2dWorkload::Execute() const
 {
     if (m_RunsInsideTheAddition) return;
     ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xConvolution2dWorkload_Execute");
+    if (m_Depthwise)
+    {
+        // the pair: the depthwise layer in front of this convolution has left its execution to this workload
+        std::call_once(m_Once, [this] { BuildPlan(); });
+        if (!m_Plan) throw RuntimeException("Mi355xConvolution2dWorkload: no device plan (its creation failed earlier)");
+        const mi355x_conv2d_t first = m_Depthwise->Plan();
+        const TensorInfo& in = m_Depthwise->GetInputInfo();
+        const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+        const uint32_t batch = in.GetShape()[0];
+        if (m_FusePair < 0)
+            m_FusePair = mi355x_conv2d_fusable(first, m_Plan) == 0 &&
+                         mi355x_conv2d_fusion_pays(first, m_Plan, batch / mi355x::LanesFor(batch)) == 1 ? 1 : 0;
+        const unsigned char* x = static_cast<const unsigned char*>(In(m_Depthwise->GetInputHandle()));
+        unsigned char* y = static_cast<unsigned char*>(Out(m_Data.m_Outputs[0]));
+        // The pair's output began its life after the pair's input ended its own, so a memory manager that shares addresses may
+        // have put the one where the other is; one launch that reads and writes the same range would race.  The fused
+        // kernels also want 16-byte aligned tensors.
+        const bool overlap = x < y + out.GetNumBytes() && y < x + in.GetNumBytes();
+        const bool aligned = ((reinterpret_cast<uintptr_t>(x) | reinterpret_cast<uintptr_t>(y)) & 15) == 0;
+        if (m_FusePair == 1 && !overlap && aligned)
+        {
+            g_DepthwisePairsRunFused.fetch_add(1);
+            ForEachLane(batch, [&](const Lane& l) {
+                mi355x::Check(mi355x_conv2d_run_fused(first, m_Plan, batch / l.count, l.Of(static_cast<const void*>(x), in),
+                                                      l.Of(static_cast<void*>(y), out), l.stream), "mi355x_conv2d_run_fused");
+            });
+            return;
+        }
+        g_DepthwisePairsRunApart.fetch_add(1);
+        m_Depthwise->Run();
+    }
     Run(Out(m_Data.m_Outputs[0]));
 }
 
@@ -250,11 +334,20 @@ Mi355xDepthwiseConvolution2dWorkload::Mi355xDepthwiseConvolution2dWorkload(const
     ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xDepthwiseConvolution2dWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
     if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xDepthwiseConvolution2dWorkload: NHWC only");
     Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>());
+    if (const Mi355xLayerNote* note = Mi355xLayerNote::From(m_Data.m_AdditionalInfoObject)) m_OnlyConsumerIsAPointwise = note->onlyConsumerIsAPointwiseConvolution;
 }
 
 Mi355xDepthwiseConvolution2dWorkload::~Mi355xDepthwiseConvolution2dWorkload()
 {
+    if (m_Pointwise) m_Pointwise->ForgetDepthwise();
     if (m_Plan) mi355x_conv2d_destroy(m_Plan);
+}
+
+mi355x_conv2d_t Mi355xDepthwiseConvolution2dWorkload::Plan() const
+{
+    std::call_once(m_Once, [this] { BuildPlan(); });
+    if (!m_Plan) throw RuntimeException("Mi355xDepthwiseConvolution2dWorkload: no device plan (its creation failed earlier)");
+    return m_Plan;
 }
 
 void Mi355xDepthwiseConvolution2dWorkload::BuildPlan() const
@@ -294,9 +387,14 @@ void Mi355xDepthwiseConvolution2dWorkload::BuildPlan() const
 
 void Mi355xDepthwiseConvolution2dWorkload::Execute() const
 {
+    if (m_Pointwise) return;              // the pointwise convolution behind this layer runs the pair
     ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xDepthwiseConvolution2dWorkload_Execute");
-    std::call_once(m_Once, [this] { BuildPlan(); });
-    if (!m_Plan) throw RuntimeException("Mi355xDepthwiseConvolution2dWorkload: no device plan (its creation failed earlier)");
+    Run();
+}
+
+void Mi355xDepthwiseConvolution2dWorkload::Run() const
+{
+    Plan();
     const TensorInfo& in = m_Info.m_InputTensorInfos[0];
     const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
     const uint32_t batch = in.GetShape()[0];

@@ -28,6 +28,22 @@ struct Mi355xFusedActivation
 /// Linear with slope 1 and offset 0, the identity, so a reader that applies it changes nothing.
 ActivationDescriptor Mi355xFeedsOnlyAnAddition();
 
+/// The additional-info object this backend's optimizer attaches to a DepthwiseConvolution2d whose output goes to one 1x1
+/// Convolution2d of this backend and nowhere else: the fused activation (first member, so a reader that takes the object
+/// for an ActivationDescriptor, as every workload does, reads exactly that) plus the mark.  Objects of this type are kept
+/// in a registry while they live, so a workload can tell them from a plain ActivationDescriptor without touching memory
+/// behind one.
+struct Mi355xLayerNote
+{
+    ActivationDescriptor activation;
+    bool onlyConsumerIsAPointwiseConvolution = false;
+
+    /// a note as a layer's additional-info object; `activation` null: the identity (Mi355xFeedsOnlyAnAddition's descriptor)
+    static std::shared_ptr<void> Make(const ActivationDescriptor* activation, bool onlyConsumerIsAPointwiseConvolution);
+    /// the note behind a queue descriptor's additional-info pointer, or null if that is something else
+    static const Mi355xLayerNote* From(const void* additionalInfo);
+};
+
 /// Every workload here reads its tensor handles when it executes, so the runtime may swap a handle for one that adopted
 /// caller memory (pre-imported inputs and outputs; RefBaseWorkload, src/backends/reference/workloads/RefBaseWorkload.hpp:13-35).
 template <typename QueueDescriptor>
@@ -56,6 +72,18 @@ public:
     /// own Execute().
     void LeaveExecutionToTheAddition() { m_RunsInsideTheAddition = true; }
     bool RunsInsideTheAddition() const { return m_RunsInsideTheAddition; }
+    /// `depthwise` was created just before this workload.  If it is marked as feeding one pointwise convolution only, writes
+    /// the tensor this workload reads, and this is an unpadded 1x1 stride-1 convolution that no Addition runs, the two become a
+    /// pair: the depthwise workload's Execute() does nothing from now on and this workload's Execute() runs both -- as one
+    /// launch per lane where the device library recommends it for the two plans (mi355x_conv2d_fusion_pays) and the pair's
+    /// output does not share memory with the pair's input, else one after the other.
+    bool TakeOver(class Mi355xDepthwiseConvolution2dWorkload* depthwise);
+    /// the depthwise workload of the pair is going away
+    void ForgetDepthwise() { m_Depthwise = nullptr; }
+    /// pairs formed / executions as one launch / executions as two launches since the process started (tests, benchmarks)
+    static unsigned long long DepthwisePairsFormed();
+    static unsigned long long DepthwisePairsRunFused();
+    static unsigned long long DepthwisePairsRunApart();
     /// convolution and Addition as one launch per lane: sum = activation(convolution(input) + other)
     void ExecuteWithAddition(const ITensorHandle* other, const TensorInfo& otherInfo, ITensorHandle* sum, const TensorInfo& sumInfo,
                              const Mi355xFusedActivation& activation) const;
@@ -65,6 +93,8 @@ private:
     WorkloadInfo m_Info;
     bool m_FeedsOnlyAnAddition = false;
     bool m_RunsInsideTheAddition = false;
+    class Mi355xDepthwiseConvolution2dWorkload* m_Depthwise = nullptr;
+    mutable int m_FusePair = -1;          // -1 not decided yet, 0 the pair runs as two launches, 1 as one
     mutable mi355x_conv2d_t m_Plan = nullptr;
     mutable std::once_flag m_Once;
 };
@@ -76,9 +106,24 @@ public:
     Mi355xDepthwiseConvolution2dWorkload(const DepthwiseConvolution2dQueueDescriptor& descriptor, const WorkloadInfo& info);
     ~Mi355xDepthwiseConvolution2dWorkload() override;
     void Execute() const override;
+    /// the layer was marked: its output goes to one 1x1 Convolution2d of this backend and nowhere else
+    bool OnlyConsumerIsAPointwiseConvolution() const { return m_OnlyConsumerIsAPointwise; }
+    const ITensorHandle* GetOutputHandle() const { return m_Data.m_Outputs[0]; }
+    const ITensorHandle* GetInputHandle() const { return m_Data.m_Inputs[0]; }
+    const TensorInfo& GetInputInfo() const { return m_Info.m_InputTensorInfos[0]; }
+    /// From now on Execute() does nothing: `pointwise`, the convolution that consumes this layer, runs it (see its TakeOver()).
+    void LeaveExecutionTo(Mi355xConvolution2dWorkload* pointwise) { m_Pointwise = pointwise; }
+    /// the convolution of the pair is going away: this workload runs itself again
+    void ForgetPointwise() { m_Pointwise = nullptr; }
+    /// the layer itself, whoever executes it
+    void Run() const;
+    /// the device plan (built on first use)
+    mi355x_conv2d_t Plan() const;
 private:
     void BuildPlan() const;
     WorkloadInfo m_Info;
+    bool m_OnlyConsumerIsAPointwise = false;
+    Mi355xConvolution2dWorkload* m_Pointwise = nullptr;
     mutable mi355x_conv2d_t m_Plan = nullptr;
     mutable std::once_flag m_Once;
 };
