@@ -23,12 +23,6 @@
 
 using namespace mi355x;
 
-struct mi355x_fc_s
-{
-    mi355x_conv2d_s* conv = nullptr;
-    ~mi355x_fc_s() { delete conv; }
-};
-
 namespace
 {
 // An Addition waiting to be fused into the next launch of this thread (mi355x_conv2d_run_add): the launchers whose

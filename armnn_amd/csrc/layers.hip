@@ -3,6 +3,7 @@
 // (dequantize -> float op -> armnn::Quantize) element for element.
 #include "common.h"
 #include "device_math.h"
+#include "pool_softmax_items.h"
 
 #include <algorithm>
 #include <cfloat>
@@ -35,14 +36,6 @@ __global__ __launch_bounds__(256) void ActivationKernel(QIn qin, Requant rq, int
     const size_t stride = static_cast<size_t>(gridDim.x) * 256;
     for (; i < n; i += stride) y[i] = lut[x[i]];
 }
-
-struct PoolArgs
-{
-    int H, W, C, Ho, Wo;
-    int pool_w, pool_h, stride_x, stride_y;
-    int pad_left, pad_right, pad_top, pad_bottom;
-    int is_max, exclude;
-};
 
 // One thread per output element; same window clamping and divisor rules as Pooling2d.cpp:186-300.
 __global__ __launch_bounds__(256) void Pool2dKernel(PoolArgs p, QIn qin, Requant rq, const uint8_t* __restrict__ x,
@@ -278,52 +271,12 @@ __global__ __launch_bounds__(256) void MaxPool2dC16Kernel(PoolArgs p, QIn qin, R
     *reinterpret_cast<v4u*>(y + idx * 16) = out;
 }
 
-// The window is the whole image (global pooling): a block owns 256 channels of one image.  All threads fetch the
-// image's taps as dwords into LDS at once; then thread c walks channel c's taps in the reference's order (row by row),
-// so the fp32 sum is the reference's sum.  `taps` = H * W, at most kGlobalPoolMaxTaps.
-constexpr int kGlobalPoolMaxTaps = 196;
+// The window is the whole image (global pooling): a block owns 256 channels of one image (GlobalPoolItem).
 __global__ __launch_bounds__(256) void GlobalPoolKernel(PoolArgs p, QIn qin, Requant rq, const uint8_t* __restrict__ x,
                                                         uint8_t* __restrict__ y)
 {
     __shared__ uint32_t raw[kGlobalPoolMaxTaps * 64];
-    const int taps = p.H * p.W;
-    const int groups = (p.C + 255) >> 8;
-    const long long n = blockIdx.x / groups;
-    const int c0 = static_cast<int>(blockIdx.x % groups) * 256;
-    const int quads = min(64, (p.C - c0) >> 2);
-    const uint8_t* xn = x + n * taps * p.C + c0;
-    for (int i = threadIdx.x; i < taps * 64; i += 256)
-    {
-        const int tap = i >> 6, q = i & 63;
-        if (q < quads) raw[i] = *reinterpret_cast<const uint32_t*>(xn + static_cast<long long>(tap) * p.C + q * 4);
-    }
-    __syncthreads();
-    const int c = threadIdx.x;
-    if (c0 + c >= p.C) return;
-    const uint8_t* col = reinterpret_cast<const uint8_t*>(raw) + c;
-    float res;
-    if (p.is_max)
-    {
-        int best = INT_MIN;
-        for (int t = 0; t < taps; ++t)
-        {
-            const int code = qin.is_u8 ? static_cast<int>(col[t * 256]) : static_cast<int>(static_cast<int8_t>(col[t * 256]));
-            best = max(best, code);
-        }
-        res = __fmul_rn(static_cast<float>(best - qin.offset), qin.scale);
-    }
-    else
-    {
-        float sum = 0.0f;
-#pragma unroll 7
-        for (int t = 0; t < taps; ++t)
-        {
-            const int code = qin.is_u8 ? static_cast<int>(col[t * 256]) : static_cast<int>(static_cast<int8_t>(col[t * 256]));
-            sum = __fadd_rn(sum, __fmul_rn(static_cast<float>(code - qin.offset), qin.scale));
-        }
-        res = __fdiv_rn(sum, static_cast<float>(taps));
-    }
-    y[n * p.C + c0 + c] = static_cast<uint8_t>(QuantizeFastDev(res, rq));
+    GlobalPoolItem<false>(p, qin, rq, x, y, static_cast<int>(blockIdx.x), raw);
 }
 
 // 16 elements per thread, 16-byte loads and stores
@@ -384,44 +337,13 @@ __global__ __launch_bounds__(64) void SoftmaxKernel(int cols, float beta, QIn qi
     }
 }
 
-// One block per row, the row held in registers (cols <= 256 * V): one pass over memory, one exp per element.
+// One block per row, the row held in registers (cols <= 256 * V): SoftmaxRowItem.
 template <int V>
 __global__ __launch_bounds__(256) void SoftmaxRowKernel(int cols, float beta, QIn qin, Requant rq,
                                                          const uint8_t* __restrict__ x, uint8_t* __restrict__ y)
 {
     __shared__ float red[8];
-    const uint8_t* xr = x + static_cast<long long>(blockIdx.x) * cols;
-    uint8_t* yr = y + static_cast<long long>(blockIdx.x) * cols;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    uint8_t raw[V];
-#pragma unroll
-    for (int k = 0; k < V; ++k) raw[k] = xr[min(tid + 256 * k, cols - 1)];
-    float v[V];
-    float mx = -FLT_MAX;
-#pragma unroll
-    for (int k = 0; k < V; ++k)
-    {
-        v[k] = DequantDev(raw[k], qin);
-        if (tid + 256 * k < cols) mx = fmaxf(mx, v[k]);
-    }
-    for (int o = 32; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o));
-    if (lane == 0) red[wave] = mx;
-    __syncthreads();
-    mx = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    float sum = 0.0f;
-#pragma unroll
-    for (int k = 0; k < V; ++k)
-    {
-        v[k] = tid + 256 * k < cols ? expf(__fmul_rn(__fsub_rn(v[k], mx), beta)) : 0.0f;
-        sum += v[k];
-    }
-    for (int o = 32; o > 0; o >>= 1) sum += __shfl_xor(sum, o);
-    if (lane == 0) red[4 + wave] = sum;
-    __syncthreads();
-    sum = (red[4] + red[5]) + (red[6] + red[7]);
-#pragma unroll
-    for (int k = 0; k < V; ++k)
-        if (tid + 256 * k < cols) yr[tid + 256 * k] = static_cast<uint8_t>(QuantizeDev(__fdiv_rn(v[k], sum), rq));
+    SoftmaxRowItem<V>(cols, beta, qin, rq, x + static_cast<long long>(blockIdx.x) * cols, y + static_cast<long long>(blockIdx.x) * cols, red);
 }
 
 // Constant padding.  The host merges every unpadded dimension into the one outside it, so a row of the canonical

@@ -63,6 +63,13 @@ struct mi355x_conv2d_s
     }
 };
 
+// The plan object behind mi355x_fc_t: a 1x1 convolution over a 1x1 image with k input channels.
+struct mi355x_fc_s
+{
+    mi355x_conv2d_s* conv = nullptr;
+    ~mi355x_fc_s() { delete conv; }
+};
+
 namespace mi355x
 {
 

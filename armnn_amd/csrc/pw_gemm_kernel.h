@@ -347,15 +347,14 @@ __global__ __launch_bounds__(256) void GemvKernel(GemvArgs a)
 // fill LDS-tiled blocks.  A block owns 32 rows x 32 channels; its four waves split K (wave w takes the 32-byte
 // k-steps w, w+4, ...), each issues the loads of UN steps at once and feeds them to v_mfma_i32_32x32x32_i8, and the
 // four partial tiles meet in LDS, where wave g requantizes accumulator group g.  K must be a multiple of 16.
-template <int UN>
-__global__ __launch_bounds__(256) void SmallMGemmKernel(GemvArgs a)
+// As a device function of a 256-thread block (tile at rows m0.., channels n0..; `part`: 4 x 16 x 64 ints of LDS, `rowpart`:
+// 4 x 64; a barrier must separate two calls).  THROUGH: outputs are written through L2 as they are stored, for a caller
+// that hands them to other blocks of the same launch (a.y + a.M * a.N below 4 GiB from a.y).
+template <int UN, bool THROUGH>
+__device__ __forceinline__ void SmallMGemmTile(const GemvArgs& a, int n0, int m0, int (*part)[16][64], int (*rowpart)[64])
 {
-    __shared__ int part[4][16][64];
-    __shared__ int rowpart[4][64];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const int n0 = static_cast<int>(blockIdx.x) * 32;
-    const int m0 = static_cast<int>(blockIdx.y) * 32;
     const int frag_row = lane & 31;
     const int frag_k = (lane >> 5) * 16;
     const int xm = static_cast<int>(a.xor_mask);
@@ -416,7 +415,44 @@ __global__ __launch_bounds__(256) void SmallMGemmKernel(GemvArgs a)
     const float4 mm = *reinterpret_cast<const float4*>(a.ct.p + 4 * a.ct.stride + c);
     const float4 bm = *reinterpret_cast<const float4*>(a.ct.p + 7 * a.ct.stride + c);
     const uint32_t out = Requant4Dev(v[0], v[1], v[2], v[3], mp, bp, mm, bm, a.ct, a.corr, c, a.rq);
-    if (row < a.M)
+    if constexpr (THROUGH)
+    {
+        // Bytes written through one by one are slow, and rows of N bytes start anywhere: the tile meets in LDS (in `part`,
+        // once every wave has read its sums) and leaves as the dwords of the output's own 4-byte grid, with single bytes
+        // only where a dword is shared with a neighbouring tile or row.  a.y must be 4-byte aligned.
+        __syncthreads();
+        uint8_t* stage = reinterpret_cast<uint8_t*>(part);
+        *reinterpret_cast<uint32_t*>(stage + frag_row * 32 + (c - n0)) = out;
+        __syncthreads();
+        const __amdgpu_buffer_rsrc_t rsrc = __builtin_amdgcn_make_buffer_rsrc(a.y, 0, a.M * a.N, 0x00020000);
+        const int r = threadIdx.x >> 3, seg = threadIdx.x & 7;
+        if (m0 + r < a.M)
+        {
+            const int len = min(32, a.N - n0);
+            const int first = (m0 + r) * a.N + n0;            // byte offset of the row's piece
+#pragma unroll
+            for (int e = 0; e < 2; ++e)
+            {
+                if (e == 1 && seg != 0) break;
+                const int word = (first >> 2) + (e == 0 ? seg : 8);
+                const int lo = word * 4 - first;               // position of the dword's first byte within the piece: -3 .. 32
+                if (lo >= 0 && lo + 4 <= len)
+                {
+                    const uint8_t* sb = stage + r * 32 + lo;
+                    const uint32_t v = static_cast<uint32_t>(sb[0]) | (static_cast<uint32_t>(sb[1]) << 8) | (static_cast<uint32_t>(sb[2]) << 16) |
+                                       (static_cast<uint32_t>(sb[3]) << 24);
+                    __builtin_amdgcn_raw_buffer_store_b32(v, rsrc, word * 4, 0, kStoreAuxSc1);
+                }
+                else
+                {
+#pragma unroll
+                    for (int k = 0; k < 4; ++k)
+                        if (lo + k >= 0 && lo + k < len) __builtin_amdgcn_raw_buffer_store_b8(stage[r * 32 + lo + k], rsrc, word * 4 + k, 0, kStoreAuxSc1);
+                }
+            }
+        }
+    }
+    else if (row < a.M)
     {
         uint8_t* dst = a.y + static_cast<long long>(row) * a.N + c;
         if ((a.N & 3) == 0 && c + 3 < a.N) *reinterpret_cast<uint32_t*>(dst) = out;
@@ -427,6 +463,14 @@ __global__ __launch_bounds__(256) void SmallMGemmKernel(GemvArgs a)
                 if (c + i < a.N) dst[i] = static_cast<uint8_t>(out >> (8 * i));
         }
     }
+}
+
+template <int UN>
+__global__ __launch_bounds__(256) void SmallMGemmKernel(GemvArgs a)
+{
+    __shared__ int part[4][16][64];
+    __shared__ int rowpart[4][64];
+    SmallMGemmTile<UN, false>(a, static_cast<int>(blockIdx.x) * 32, static_cast<int>(blockIdx.y) * 32, part, rowpart);
 }
 
 } // namespace mi355x

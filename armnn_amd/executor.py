@@ -54,11 +54,34 @@ class ChainedRun:
         return sum(p.macs_per_image for p in self.parts)
 
 
+@dataclass
+class FusedTail:
+    """Global pooling, the FullyConnected layer behind it and the Softmax behind that, executed by one launch
+    (shim.ClassifierTail); all three tensors are still written."""
+    name: str
+    parts: Tuple                       # (pooling Layer, FullyConnected Layer, Softmax Layer)
+    op: str = "tail"
+
+    @property
+    def inputs(self):
+        return tuple(self.parts[0].inputs)
+
+    @property
+    def output(self):
+        return self.parts[-1].output
+
+    @property
+    def macs_per_image(self):
+        return self.parts[1].macs_per_image
+
+
 class DeviceNetwork:
     def __init__(self, net: Network, batch: int, algo_overrides: Optional[Dict[str, int]] = None, use_graph: bool = True,
                  fuse: bool = False, lanes: int = 1, fuse_add: bool = True, chain: bool = False, lanes_after_chain: bool = False,
-                 join_for_fused: bool = False):
-        """chain: runs of consecutive layers the library accepts (mi355x_chain_accepts) become one persistent launch over
+                 join_for_fused: bool = False, fuse_tail: bool = False):
+        """fuse_tail: global pooling -> FullyConnected -> Softmax at the end of the network as one launch (same bytes; measured
+        slower than the three launches on MI355X, so off by default).
+        chain: runs of consecutive layers the library accepts (mi355x_chain_accepts) become one persistent launch over
         the whole batch; with lanes > 1 the lanes join in front of such a run and, if lanes_after_chain, fork again behind it
         (else the rest of the network runs on one stream).
         lanes > 1 splits the batch into that many contiguous slices; each slice runs the whole network on a stream of
@@ -77,6 +100,8 @@ class DeviceNetwork:
         self._step_plans: List = []    # plan of each step (None for plan-less layers), parallel to self.steps
         self.plans = []
         self.chains: List = []
+        self.tails: List = []
+        self._pool_descs = {}
         self.lanes_after_chain = lanes_after_chain
         self.join_for_fused = join_for_fused      # fused pairs run on the whole batch: the lanes join in front of the first one
         self.graph = None
@@ -119,6 +144,7 @@ class DeviceNetwork:
                 d = shim.Pool2dDesc(h, w, c, ho, wo, p["pool_w"], p["pool_h"], p["stride_x"], p["stride_y"], p["pad_left"],
                                     p["pad_right"], p["pad_top"], p["pad_bottom"], p["pool_type"], p["padding_method"],
                                     shim._quant(xin[0]), shim._quant(yout))
+                self._pool_descs[id(l)] = d
                 self.steps.append((l, self._pool_step(d, xb[0].ptr, yb.ptr, xin[0].num_elements, yout.num_elements, l.act,
                                                       shim._quant(yout))))
                 self._step_plans.append(None)
@@ -150,6 +176,44 @@ class DeviceNetwork:
             self._fuse_additions()
         if chain:
             self._build_chains()
+        if fuse_tail:
+            self._fuse_tail()
+
+    def _fuse_tail(self):
+        """Pooling over the whole image -> FullyConnected -> Softmax, launched one behind the other, become one launch where
+        the library takes the three (mi355x_tail_create); each lane gets an object of its own, because launches of one
+        object must not overlap."""
+        net, batch, lanes = self.net, self.batch, self.lanes
+        rows = batch // lanes
+        k = 0
+        while k + 2 < len(self.steps):
+            (lp, _), (lf, _), (ls, _) = self.steps[k:k + 3]
+            if not (getattr(lp, "op", None) == "pool" and getattr(lf, "op", None) == "fc" and getattr(ls, "op", None) == "softmax" and
+                    lp.act[0] == 0 and self.buffers[lf.inputs[0]] is self.buffers[lp.output] and ls.inputs[0] == lf.output):
+                k += 1
+                continue
+            fc_plan = self._plan_of[id(lf)]
+            cols = net.info(lf.output, batch).shape[-1]
+            chans = net.info(lp.output, batch).shape[-1]
+            if (rows * cols) % 4 != 0:
+                k += 1
+                continue
+            try:
+                tails = [shim.ClassifierTail(self._pool_descs[id(lp)], fc_plan, ls.params["beta"], net.info(ls.output, batch))
+                         for _ in range(lanes)]
+            except shim.ShimError:
+                k += 1
+                continue
+            self.tails.extend(tails)
+            x, pooled = self.buffers[lp.inputs[0]].ptr, self.buffers[lp.output].ptr
+            logits, y = self.buffers[lf.output].ptr, self.buffers[ls.output].ptr
+            nx = net.info(lp.inputs[0], batch).num_elements
+
+            def fn(s, lane=0, lanes=1, tails=tails, x=x, pooled=pooled, logits=logits, y=y, nx=nx, chans=chans, cols=cols):
+                r = batch // lanes
+                tails[lane].run(r, x + lane * (nx // lanes), pooled + lane * r * chans, logits + lane * r * cols, y + lane * r * cols, s)
+            self.steps[k:k + 3] = [(FusedTail(f"{lp.name}+{lf.name}+{ls.name}", (lp, lf, ls)), fn)]
+            k += 1
 
     def _build_chains(self, min_layers: int = 2):
         """Replace every maximal run of consecutive steps that are plain convolution / depthwise layers accepted by the
@@ -413,6 +477,9 @@ class DeviceNetwork:
         for ch in self.chains:
             ch.destroy()
         self.chains = []
+        for t in self.tails:
+            t.destroy()
+        self.tails = []
         for p in self.plans:
             p.destroy()
         for b in set(self.buffers.values()):

@@ -32,6 +32,7 @@ EXPORTS = [
     "mi355x_chain_accepts", "mi355x_chain_create", "mi355x_chain_run", "mi355x_chain_status", "mi355x_chain_info", "mi355x_chain_run_stamped", "mi355x_chain_run_noalloc", "mi355x_chain_destroy",
     "mi355x_fc_create", "mi355x_fc_run", "mi355x_fc_destroy", "mi355x_fc_algo",
     "mi355x_activation_run", "mi355x_pool2d_run", "mi355x_add_run", "mi355x_softmax_run", "mi355x_pad_run",
+    "mi355x_tail_create", "mi355x_tail_run", "mi355x_tail_status", "mi355x_tail_set_wait_limit", "mi355x_tail_destroy",
 ]
 
 
@@ -130,6 +131,9 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
                                C.c_float, V, V, V, V],
             "mi355x_softmax_run": [C.c_uint32, C.c_uint32, C.c_float, C.POINTER(Quant), C.POINTER(Quant), V, V, V],
             "mi355x_pad_run": [C.POINTER(PadDesc), V, V, V],
+            "mi355x_tail_create": [C.POINTER(Pool2dDesc), V, C.c_float, C.POINTER(Quant), C.POINTER(V)],
+            "mi355x_tail_run": [V, C.c_uint32, V, V, V, V, V], "mi355x_tail_status": [V, C.POINTER(C.c_uint32)],
+            "mi355x_tail_set_wait_limit": [V, C.c_uint64], "mi355x_tail_destroy": [V],
             "mi355x_device_count": [C.POINTER(C.c_int)], "mi355x_init": [C.c_int],
             "mi355x_set_option": [C.c_char_p, C.c_int],
             "mi355x_device_name": [C.c_char_p, C.c_size_t],
@@ -437,6 +441,43 @@ class FullyConnectedPlan:
         if self.plan:
             self.lib.mi355x_fc_destroy(self.plan)
             self.plan = None
+
+    def __del__(self):
+        try:
+            self.destroy()
+        except Exception:
+            pass
+
+
+class ClassifierTail:
+    """mi355x_tail_create / run / status / destroy: global pooling -> FullyConnected -> Softmax as one launch.  Raises
+    ShimError (unsupported) for what the library runs as three calls only."""
+
+    def __init__(self, pool_desc: "Pool2dDesc", fc: FullyConnectedPlan, beta: float, out_info: TensorInfo):
+        self.lib = load_library()
+        self.fc = fc                      # must outlive the object
+        self._desc = pool_desc
+        qo = _quant(out_info)
+        tail = C.c_void_p()
+        _chk(self.lib.mi355x_tail_create(C.byref(pool_desc), fc.plan, beta, C.byref(qo), C.byref(tail)))
+        self.tail = tail.value
+
+    def run(self, batch: int, x_dev: int, pooled_dev: int, logits_dev: int, y_dev: int, stream=None):
+        _chk(self.lib.mi355x_tail_run(self.tail, batch, x_dev, pooled_dev, logits_dev, y_dev, stream))
+
+    def gave_up(self) -> int:
+        """waits that ran out in runs since the last call (after the stream has been synchronized)"""
+        n = C.c_uint32()
+        _chk(self.lib.mi355x_tail_status(self.tail, C.byref(n)))
+        return n.value
+
+    def set_wait_limit(self, microseconds: int):
+        _chk(self.lib.mi355x_tail_set_wait_limit(self.tail, microseconds))
+
+    def destroy(self):
+        if self.tail:
+            self.lib.mi355x_tail_destroy(self.tail)
+            self.tail = None
 
     def __del__(self):
         try:

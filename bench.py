@@ -72,7 +72,7 @@ def layer_work(net, l, batch):
         return "mfma", 2.0 * l.macs_per_image * batch
     if l.op == "convadd":                      # a convolution with the Addition behind it in its write-out
         return "mfma", 2.0 * l.parts[0].macs_per_image * batch
-    if l.op == "chain":
+    if l.op in ("chain", "tail"):
         # a run of layers in one persistent launch: every layer's tensors are still written and read, so the launch's
         # algorithmic bytes are the sum of its layers'; priced against HBM like the depthwise layers in it
         return "hbm", float(sum(algorithmic_bytes(net, part, batch) for part in l.parts))
@@ -232,6 +232,7 @@ def main():
                     help="pairs of layers as one kernel (same bytes): 'auto' the depthwise + pointwise pairs the library recommends at "
                          "the batch a launch sees (mi355x_conv2d_fusion_pays), 'none' every layer a launch of its own, 'dwpw' every "
                          "depthwise + pointwise pair the fused kernels accept, 'pwdw' pointwise + the depthwise after it where whole images fit a block")
+    ap.add_argument("--fuse-tail", action="store_true", help="pooling, FullyConnected and Softmax at the end of the network as one launch instead of three (same bytes, measured slower)")
     ap.add_argument("--no-fuse-add", action="store_true",
                     help="launch a residual Addition on its own instead of inside the convolution that feeds it")
     ap.add_argument("--lanes", type=int, default=0,
@@ -276,7 +277,7 @@ def main():
         # (MobileNetV1, 64 images: 0.330 ms in one lane, 0.336 in two; ResNet-50, 32 images: 0.864 and 0.725).
         depthwise = any(l.op == "depthwise" for l in net.layers)
         args.lanes = 2 if batch >= 16 and batch % 2 == 0 and not depthwise else 1
-    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse="" if args.fuse == "none" else args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add, chain=args.chain)
+    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse="" if args.fuse == "none" else args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add, chain=args.chain, fuse_tail=args.fuse_tail)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev
 
@@ -410,6 +411,7 @@ def main():
                           f"one HIP graph replay per step",
               "batch": batch, "graph_replay": not args.no_graph, "fused_pairs": [l.name for l, _ in dn.steps if l.op == "dwpw"] or None, "additions_inside_convolutions": not args.no_fuse_add, "lanes": args.lanes,
               "layer_chains": [l.name for l, _ in dn.steps if l.op == "chain"] or None,
+              "tail_in_one_launch": any(l.op == "tail" for l, _ in dn.steps),
               "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12}
     if backend is not None:
         # the same network and input through the C++ backend: wall clock per IRuntime::EnqueueWorkload call, host buffers in

@@ -386,6 +386,31 @@ int mi355x_softmax_run(uint32_t rows, uint32_t cols, float beta, const mi355x_qu
                        const mi355x_quant* out_q, const void* input_dev, void* output_dev,
                        mi355x_stream_t stream);
 
+/* The tail of a classifier as ONE launch: global pooling (the window is the whole unpadded image, at most 196 pixels,
+ * channels % 4 == 0) -> FullyConnected (a matrix-core plan: k % 16 == 0, k >= 128, at most 2048 outputs) -> Softmax over
+ * each row of logits.  Every stage computes exactly what mi355x_pool2d_run, mi355x_fc_run and mi355x_softmax_run compute
+ * (Pooling2d.cpp:142-303, FullyConnected.cpp:13-65, Softmax.cpp:16-69) and writes the same bytes to pooled_dev
+ * [batch][channels], logits_dev [batch][out_features] and output_dev [batch][out_features]; the stages hand over inside the
+ * kernel through two counters in a few hundred bytes of device memory the object owns, so two launches of ONE object must
+ * not run at the same time (launches of different objects may).  `fc` must outlive the object; its input quantization
+ * must be the pooling's output quantization, its output quantization is the Softmax's input quantization.  The four
+ * tensors must not overlap; pooled_dev 16-byte, input_dev and logits_dev 4-byte aligned; at most 1024 rows per launch.
+ * What the object does not take (MI355X_ERR_UNSUPPORTED) runs as the three calls.  On an MI355X the one launch takes
+ * about 16 us for 64 rows of 1024 channels against about 13 us for the three calls back to back (each hand-over inside the
+ * kernel costs what a kernel boundary costs: stores written through, a counter, a poll, reads that miss), so the callers
+ * here launch the three; the entry point is for callers whose cost is the number of launches.
+ *   Every wait inside the kernel is bounded (2 s by default; mi355x_tail_set_wait_limit, for tests of the give-up path);
+ * mi355x_tail_status waits for nothing (call it after synchronizing the stream): *gave_up is the number of waits that ran
+ * out in runs since the last call, and a run that gave up leaves its outputs undefined. */
+typedef struct mi355x_tail_s* mi355x_tail_t;
+int mi355x_tail_create(const mi355x_pool2d_desc* pool, mi355x_fc_t fc, float beta, const mi355x_quant* output_quant,
+                       mi355x_tail_t* tail);
+int mi355x_tail_run(mi355x_tail_t tail, uint32_t batch, const void* input_dev, void* pooled_dev, void* logits_dev,
+                    void* output_dev, mi355x_stream_t stream);
+int mi355x_tail_status(mi355x_tail_t tail, uint32_t* gave_up);
+int mi355x_tail_set_wait_limit(mi355x_tail_t tail, uint64_t microseconds);
+int mi355x_tail_destroy(mi355x_tail_t tail);
+
 /* Pad with a constant, rank 1..4: Pad() (workloads/Pad.cpp:39-236) as RefPadWorkload::Execute calls it
  * (workloads/RefPadWorkload.cpp:18-40).  Fields mirror armnn::PadDescriptor (include/armnn/Descriptors.hpp:1196-1229):
  * pad_before[d] / pad_after[d] are m_PadList[d].first / .second.  pad_value is the stored code of the padding
