@@ -1654,9 +1654,7 @@ int mi355x_conv2d_run_add(mi355x_conv2d_t plan, uint32_t batch, const void* inpu
     }
     PendingAdd pending;
     pending.other = static_cast<const uint8_t*>(other_dev);
-    pending.fuse.qa = MakeQIn(plan->d.output);
-    pending.fuse.qr = MakeQIn(*other_quant);
-    pending.fuse.rq = MakeRequant(*sum_quant, activation, a, b);
+    pending.fuse = MakeAddFuse(plan->d.output, *other_quant, *sum_quant, activation, a, b);
     const bool aligned = (reinterpret_cast<uintptr_t>(other_dev) & 15) == 0 && (reinterpret_cast<uintptr_t>(output_dev) & 15) == 0;
     t_pending_add = aligned ? &pending : nullptr;
     const int rc = RunPlan(plan, batch, input_dev, output_dev, ToHip(stream));

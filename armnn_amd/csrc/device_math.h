@@ -3,6 +3,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <cmath>
+
 #include "common.h"
 
 namespace mi355x
@@ -299,27 +301,95 @@ inline QIn MakeQIn(const mi355x_quant& q)
     return r;
 }
 
-// The Addition that follows a convolution, run inside the convolution's write-out: `own` are sixteen finished output
-// codes of the convolution (quantization qa), `other` the sixteen codes of the Addition's other input (qr); the sum is
-// formed and quantized exactly as the Addition layer does it (dequantize both, one fp32 add, quantize with the
-// Addition's output quantization and its fused activation), so the bytes are those of the two layers run apart.
+// An Addition of two quantized tensors: dequantize both, one fp32 add, quantize with the Addition's output quantization and
+// its fused activation (RefElementwiseBinaryWorkload.cpp:27-107 over Decoder / Encoder).  Used by the Addition layer's
+// kernel and, inside a convolution's write-out, for the Addition that follows the convolution (`own`: the convolution's
+// finished output codes with quantization qa, `other`: the Addition's other input with qr) -- so the bytes are those of
+// the two layers run apart.
+//   The reference's sequence costs 14 vector instructions per value (two dequantizations of three, the add, a quantization
+//   with its own tie test).  The value before rounding is, in exact arithmetic, a linear function of the two codes,
+//     T = ua ka + ub kb + k0,   ka = sa / so, kb = sr / so, k0 = offset_out + pk_bias - oa ka - or kb   (ua, ub: codes as 0..255),
+//   and the reference's own fp32 value P' (its four roundings: two products, the sum, the division) lies within
+//   3.01 * 2^-24 * 255 (ka + kb) of T.  t+ = fma(ua, ka, fma(ub, kb, k0 + c)) and t- = t+ - 2c, with c above that distance plus
+//   the roundings of the constants, of the two FMAs and of the subtraction (for |T| <= 512: 2^-24 (1533 ka + 1278 kb + 2048)
+//   in all; c = 1.5 x that), enclose P'; beyond |T| = 512 all three saturate alike.  When t- and t+ convert to the same byte
+//   (v_cvt_pk_u8_f32: round to nearest, saturate; monotone), P' -- strictly between them -- rounds to that byte under any
+//   tie rule.  Otherwise (a few values in 10^4) that value is redone with the reference's sequence.  Seven instructions
+//   per value on the fast path, nine when the activation clamps inside 0..255.
 struct AddFuse
 {
     QIn qa, qr;
     Requant rq;
+    float ka, kb, k0p, two_c;
+    int bracket_ok;
 };
+
+inline AddFuse MakeAddFuse(const mi355x_quant& a, const mi355x_quant& r, const mi355x_quant& out, int32_t activation, float act_a, float act_b)
+{
+    AddFuse f;
+    f.qa = MakeQIn(a);
+    f.qr = MakeQIn(r);
+    f.rq = MakeRequant(out, activation, act_a, act_b);
+    const double so = static_cast<double>(out.scale);
+    const double ka = static_cast<double>(a.scale) / so, kb = static_cast<double>(r.scale) / so;
+    const double oa = f.qa.is_u8 ? a.offset : a.offset + 128, ob = f.qr.is_u8 ? r.offset : r.offset + 128;
+    const double k0 = static_cast<double>(out.offset) + f.rq.pk_bias - oa * ka - ob * kb;
+    const double c = 1.5 * (1533.0 * ka + 1278.0 * kb + 2048.0) / 16777216.0;
+    f.ka = static_cast<float>(ka);
+    f.kb = static_cast<float>(kb);
+    f.k0p = static_cast<float>(k0 + c);
+    f.two_c = nextafterf(static_cast<float>(2.0 * c), 1.0e30f);
+    f.bracket_ok = f.rq.fast_ok && std::isnormal(f.ka) && std::isnormal(f.kb) && ka < 1024.0 && kb < 1024.0 && std::fabs(k0) < 1048576.0 &&
+                   oa >= 0.0 && oa <= 255.0 && ob >= 0.0 && ob <= 255.0;     // offsets inside the type's range: |code - offset| <= 255
+    return f;
+}
+
+// four codes of each input (dwords wa, wb) -> packed dword of the four sums' codes
+__device__ __forceinline__ uint32_t AddQuantize4Dev(uint32_t wa, uint32_t wb, const AddFuse& f)
+{
+    if (!f.bracket_ok)
+    {
+        float va[4], vb[4];
+        Dequant4Dev(wa, f.qa, va);
+        Dequant4Dev(wb, f.qr, vb);
+        return QuantizePack4Dev(__fadd_rn(va[0], vb[0]), __fadd_rn(va[1], vb[1]), __fadd_rn(va[2], vb[2]), __fadd_rn(va[3], vb[3]), f.rq);
+    }
+    const uint32_t ua = f.qa.is_u8 ? wa : (wa ^ 0x80808080u), ub = f.qr.is_u8 ? wb : (wb ^ 0x80808080u);
+    const float af[4] = {static_cast<float>(ua & 0xffu), static_cast<float>((ua >> 8) & 0xffu), static_cast<float>((ua >> 16) & 0xffu), static_cast<float>(ua >> 24)};
+    const float bf[4] = {static_cast<float>(ub & 0xffu), static_cast<float>((ub >> 8) & 0xffu), static_cast<float>((ub >> 16) & 0xffu), static_cast<float>(ub >> 24)};
+    uint32_t out = 0u, low = 0u;
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+    {
+        float p = __fmaf_rn(af[i], f.ka, __fmaf_rn(bf[i], f.kb, f.k0p));
+        float m = __fsub_rn(p, f.two_c);
+        if (!f.rq.pk_full)
+        {
+            p = __builtin_amdgcn_fmed3f(p, f.rq.pk_lo_f, f.rq.pk_hi_f);
+            m = __builtin_amdgcn_fmed3f(m, f.rq.pk_lo_f, f.rq.pk_hi_f);
+        }
+        out = __builtin_amdgcn_cvt_pk_u8_f32(p, i, out);
+        low = __builtin_amdgcn_cvt_pk_u8_f32(m, i, low);
+    }
+    const uint32_t differ = out ^ low;
+    if (__builtin_expect(differ != 0u, 0))
+    {
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+            if ((differ >> (8 * i)) & 0xffu)
+            {
+                const float s = __fadd_rn(DequantDev(static_cast<uint8_t>(wa >> (8 * i)), f.qa), DequantDev(static_cast<uint8_t>(wb >> (8 * i)), f.qr));
+                out = (out & ~(0xffu << (8 * i))) | ((static_cast<uint32_t>(QuantizeDev(s, f.rq) + f.rq.pk_bias) & 0xffu) << (8 * i));
+            }
+    }
+    return out ^ f.rq.pk_xor;
+}
 
 __device__ __forceinline__ StoreVec4 AddResidual16(const StoreVec4& own, const StoreVec4& other, const AddFuse& f)
 {
     StoreVec4 o;
 #pragma unroll
-    for (int d = 0; d < 4; ++d)
-    {
-        float va[4], vb[4];
-        Dequant4Dev(static_cast<uint32_t>(own[d]), f.qa, va);
-        Dequant4Dev(static_cast<uint32_t>(other[d]), f.qr, vb);
-        o[d] = static_cast<int>(QuantizePack4Dev(__fadd_rn(va[0], vb[0]), __fadd_rn(va[1], vb[1]), __fadd_rn(va[2], vb[2]), __fadd_rn(va[3], vb[3]), f.rq));
-    }
+    for (int d = 0; d < 4; ++d) o[d] = static_cast<int>(AddQuantize4Dev(static_cast<uint32_t>(own[d]), static_cast<uint32_t>(other[d]), f));
     return o;
 }
 

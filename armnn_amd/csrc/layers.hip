@@ -280,7 +280,7 @@ __global__ __launch_bounds__(256) void GlobalPoolKernel(PoolArgs p, QIn qin, Req
 }
 
 // 16 elements per thread, 16-byte loads and stores
-__global__ __launch_bounds__(256) void AddVec16Kernel(QIn q0, QIn q1, Requant rq, const v4u* __restrict__ x0,
+__global__ __launch_bounds__(256) void AddVec16Kernel(AddFuse f, const v4u* __restrict__ x0,
                                                       const v4u* __restrict__ x1, v4u* __restrict__ y, size_t n16)
 {
     const OutPtr outp = MakeOutPtr(reinterpret_cast<uint8_t*>(y), static_cast<long long>(n16) * 16);
@@ -291,13 +291,7 @@ __global__ __launch_bounds__(256) void AddVec16Kernel(QIn q0, QIn q1, Requant rq
         const v4u a = x0[i], b = x1[i];
         v4u o;
 #pragma unroll
-        for (int d = 0; d < 4; ++d)
-        {
-            float va[4], vb[4];
-            Dequant4Dev(a[d], q0, va);
-            Dequant4Dev(b[d], q1, vb);
-            o[d] = QuantizePack4Dev(__fadd_rn(va[0], vb[0]), __fadd_rn(va[1], vb[1]), __fadd_rn(va[2], vb[2]), __fadd_rn(va[3], vb[3]), rq);
-        }
+        for (int d = 0; d < 4; ++d) o[d] = AddQuantize4Dev(a[d], b[d], f);
         StoreOut16(outp, static_cast<long long>(i) * 16, StoreVec4{static_cast<int>(o[0]), static_cast<int>(o[1]), static_cast<int>(o[2]), static_cast<int>(o[3])});
     }
 }
@@ -521,7 +515,7 @@ int mi355x_add_run(size_t n, const mi355x_quant* in0_q, const mi355x_quant* in1_
     if (vec16)
     {
         NoteKernel("AddVec16Kernel");
-        hipLaunchKernelGGL(AddVec16Kernel, dim3(GridFor(n / 16)), dim3(256), 0, ToHip(stream), MakeQIn(*in0_q), MakeQIn(*in1_q), rq,
+        hipLaunchKernelGGL(AddVec16Kernel, dim3(GridFor(n / 16)), dim3(256), 0, ToHip(stream), MakeAddFuse(*in0_q, *in1_q, *out_q, activation, a, b),
                            static_cast<const v4u*>(input0_dev), static_cast<const v4u*>(input1_dev), static_cast<v4u*>(output_dev), n / 16);
     }
     else

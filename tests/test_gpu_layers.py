@@ -70,6 +70,39 @@ def test_add(port, dtype, shape, act):
     np.testing.assert_array_equal(got.data, want.data)
 
 
+ADD_QUANTS = [
+    # (name, dtype, (scale, offset) of input 0, of input 1, of the output, activation)
+    ("resnet_like_relu", S8, (0.0235, -128), (0.1, -128), (0.1, -128), (1, 0.0, 0.0)),
+    ("generic", S8, (0.05, 3), (0.03, -7), (0.06, 10), (0, 0.0, 0.0)),
+    ("halves_all_ties", U8, (0.02, 128), (0.02, 128), (0.04, 128), (0, 0.0, 0.0)),
+    ("unit_scales", S8, (1.0, 0), (1.0, 0), (1.0, 0), (0, 0.0, 0.0)),
+    ("mostly_saturating", S8, (0.3, 5), (0.001, -100), (0.01, 0), (0, 0.0, 0.0)),
+    ("bounded_relu_inside_the_range", U8, (0.031, 7), (0.047, 201), (0.05, 10), (2, 6.0, 0.0)),
+    ("thirds", S8, (0.1, -3), (0.2, 4), (0.3, -1), (0, 0.0, 0.0)),
+    ("quarters_and_eighths", U8, (0.125, 0), (0.25, 255), (0.5, 100), (1, 0.0, 0.0)),
+    ("tiny_output_scale", S8, (0.004, 17), (0.006, -50), (0.0009, -128), (0, 0.0, 0.0)),
+]
+
+
+@pytest.mark.parametrize("cfg", ADD_QUANTS, ids=[c[0] for c in ADD_QUANTS])
+def test_add_of_every_pair_of_codes(port, cfg):
+    """All 256 x 256 pairs of input codes: the Addition's fast path (a two-sided bracket around the reference's fp32 value)
+    and its fallback together give the reference's byte everywhere, ties included."""
+    name, dtype, (sa, oa), (sb, ob), (so, oo), act = cfg
+    lo = 0 if dtype == U8 else -128
+    codes = np.arange(256, dtype=np.int64) + lo
+    a = QTensor(TensorInfo((256, 256), dtype, (sa,), oa), np.repeat(codes, 256).reshape(256, 256))
+    b = QTensor(TensorInfo((256, 256), dtype, (sb,), ob), np.tile(codes, 256).reshape(256, 256))
+    oi = TensorInfo((256, 256), dtype, (so,), oo)
+    want = port.add(a, b, oi)
+    if act[0]:
+        want = port.activation(want, oi, *act)
+    got = shim.add(a, b, oi, activation=act[0], act_a=act[1], act_b=act[2])
+    assert shim.last_kernel() == "AddVec16Kernel"
+    np.testing.assert_array_equal(got.data, want.data)
+    print(name, "distinct output codes:", len(np.unique(got.data)), flush=True)
+
+
 @pytest.mark.parametrize("dtype", [S8, U8])
 @pytest.mark.parametrize("cols", [10, 1001, 1500, 3000])
 def test_softmax(port, dtype, cols):
