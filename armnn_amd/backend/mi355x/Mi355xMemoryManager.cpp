@@ -45,6 +45,18 @@ size_t Mi355xMemoryManager::Reserve(size_t bytes)
 void Mi355xMemoryManager::Retire(size_t offset, size_t bytes)
 {
     if (!m_Share) return;
+    // A range becomes free one retirement late.  The runtime ends a tensor's lifetime behind its last consumer and starts
+    // the next layer's output before it retires anything else, so the output of the layer BEHIND that consumer never lies
+    // over the retired tensor: a depthwise layer's input and the output of the pointwise convolution that follows do not
+    // overlap, and the convolution workload can run the pair as one launch.
+    std::swap(offset, m_PendingOffset);
+    std::swap(bytes, m_PendingBytes);
+    if (bytes == kNothingPending) return;
+    Free(offset, bytes);
+}
+
+void Mi355xMemoryManager::Free(size_t offset, size_t bytes)
+{
     size_t len = Granules(bytes ? bytes : 1);
     auto next = m_Free.lower_bound(offset);
     if (next != m_Free.begin())

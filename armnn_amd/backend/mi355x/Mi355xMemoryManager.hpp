@@ -24,7 +24,7 @@ public:
 
     /// start of a lifetime: returns the offset of a free range of `bytes` (first fit, 256-byte granules)
     size_t Reserve(size_t bytes);
-    /// end of a lifetime: the range may be handed out again
+    /// end of a lifetime: the range may be handed out again once the NEXT lifetime has ended (see the definition)
     void Retire(size_t offset, size_t bytes);
     /// device address of `offset`; throws MemoryValidationException before Acquire()
     void* Resolve(size_t offset) const;
@@ -37,6 +37,9 @@ public:
 
 private:
     static size_t Granules(size_t bytes) { return (bytes + 255) / 256 * 256; }
+    void Free(size_t offset, size_t bytes);
+    static constexpr size_t kNothingPending = ~static_cast<size_t>(0);
+    size_t m_PendingOffset = 0, m_PendingBytes = kNothingPending;     // the range retired last, not yet free
     const bool m_Share;
     std::map<size_t, size_t> m_Free;     // offset -> length of free ranges below the high-water mark
     size_t m_HighWater = 0;

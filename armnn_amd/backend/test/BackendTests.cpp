@@ -271,32 +271,53 @@ TEST_CASE("queue descriptors: Validate enforces the quantized conv rules", "cpu"
     CHECK_THROWS_AS(fq.Validate(fbad), InvalidArgumentException);
 }
 
-TEST_CASE("arena planner: lifetimes that do not overlap share addresses", "cpu")
+TEST_CASE("arena planner: lifetimes that do not overlap share addresses, one retirement late", "cpu")
 {
     Mi355xMemoryManager mm;
     const size_t a = mm.Reserve(1000);      // 1024
     const size_t b = mm.Reserve(5000);      // 5120
     CHECK(a == 0);
     CHECK(b == 1024);
-    mm.Retire(a, 1000);
-    const size_t c = mm.Reserve(512);       // fits in a's hole
-    CHECK(c == 0);
-    const size_t d = mm.Reserve(512);       // second half of a's hole
-    CHECK(d == 512);
-    mm.Retire(b, 5000);
-    mm.Retire(c, 512);
-    mm.Retire(d, 512);                      // everything free again and coalesced
-    const size_t e = mm.Reserve(6144);
-    CHECK(e == 0);
-    CHECK(mm.ArenaBytes() == 6144);
-    const size_t f = mm.Reserve(100);       // grows past the end
-    CHECK(f == 6144);
-    mm.Retire(f, 100);
-    const size_t g = mm.Reserve(300);       // the free tail is extended, not left behind
-    CHECK(g == 6144);
+    mm.Retire(a, 1000);                     // a's range is free once the next range has been retired
+    const size_t c = mm.Reserve(512);
+    CHECK(c == 6144);
+    mm.Retire(c, 512);                      // now a's hole is free, c's is pending
+    const size_t d = mm.Reserve(512);       // first half of a's hole
+    CHECK(d == 0);
+    const size_t e = mm.Reserve(512);       // second half
+    CHECK(e == 512);
+    mm.Retire(b, 5000);                     // frees c
+    mm.Retire(d, 512);                      // frees b
+    mm.Retire(e, 512);                      // frees d
+    mm.Retire(0, 0);                        // (a lifetime of nothing) frees e: everything free again and coalesced
+    const size_t f = mm.Reserve(6144 + 512);
+    CHECK(f == 0);
     CHECK(mm.ArenaBytes() == 6144 + 512);
+    const size_t g = mm.Reserve(100);       // grows past the end
+    CHECK(g == 6144 + 512);
+    mm.Retire(g, 100);
+    mm.Retire(f, 6144 + 512);               // frees g's granule at the end
+    const size_t h = mm.Reserve(300);       // the free tail is extended, not left behind
+    CHECK(h == 6144 + 512);
+    CHECK(mm.ArenaBytes() == 6144 + 512 + 512);
     CHECK(mm.ReservedTotal() > mm.ArenaBytes());
     CHECK_THROWS_AS(mm.Resolve(0), MemoryValidationException);   // nothing acquired yet
+}
+
+TEST_CASE("arena planner: the output of the layer behind a tensor's last consumer never lies over that tensor", "cpu")
+{
+    // the order in which a runtime walks a chain x -> depthwise -> t -> pointwise -> y -> next -> z: a layer's output begins
+    // before the layer's inputs end
+    Mi355xMemoryManager mm;
+    const size_t x = mm.Reserve(4096);
+    const size_t t = mm.Reserve(4096);      // depthwise: its output begins ...
+    mm.Retire(x, 4096);                     // ... then its input ends
+    const size_t y = mm.Reserve(4096);      // pointwise: reads t; a fused launch reads x and writes y
+    CHECK(y != x);
+    CHECK(y != t);
+    mm.Retire(t, 4096);
+    const size_t z = mm.Reserve(4096);      // the layer after: x's range is free by now
+    CHECK(z == x);
 }
 
 TEST_CASE("tensor handle: lifecycle errors are reported, not ignored", "cpu")
@@ -1933,7 +1954,9 @@ TEST_CASE("runtime: a 1x1 convolution runs the depthwise layer in front of it in
             CHECK(formed[0] == 0);
             CHECK(formed[1] == 2);
             CHECK(fused[1] + apart[1] == 4);               // two pairs, two inferences
-            if (lanes == 2) CHECK(fused[1] == 2);          // separate memory per tensor: nothing overlaps, the first pair runs as one launch
+            // in lanes every tensor has memory of its own; on one stream the arena frees a range one retirement late, so that a
+            // pair's output never lies over its input: either way the first pair runs as one launch
+            CHECK(fused[1] == 2);
             CHECK(results[0] == results[1]);
             const std::vector<uint8_t> a = OracleRun(blocks.dw1, input);
             const std::vector<uint8_t> b = OracleRun(blocks.pw1, a);
@@ -1977,7 +2000,11 @@ TEST_CASE("runtime: a depthwise layer whose output is read by a second consumer 
 TEST_CASE("runtime: an Addition whose sum was placed over the convolution's input runs the pair as two launches, same bytes", "gpu")
 {
     const unsigned int lanesBefore = mi355x::Lanes();
-    mi355x::SetLanes(1);                                   // one stream: the arena shares addresses
+    mi355x::SetLanes(1);
+    // The backend's own arena frees a range one retirement late, which keeps a pair's output off the pair's input; a runtime
+    // that plans the memory itself makes no such promise: with a packing strategy the sum lands on the dead 256-channel
+    // tensor the last convolution reads.
+    const INetworkProperties external(MemorySource::Undefined, MemorySource::Undefined, false, ProfilingDetailsMethod::Undefined, true);
     {
         NarrowingResidualBlock block(4);
         const std::vector<uint8_t> input = RandomActivations(block.in, 92);
@@ -1988,14 +2015,16 @@ TEST_CASE("runtime: an Addition whose sum was placed over the convolution's inpu
         for (int fused = 0; fused < 2; ++fused)
         {
             const unsigned long long pairsBefore = Mi355xAdditionWorkload::PairsFormed(), apartBefore = Mi355xAdditionWorkload::PairsRunApart();
-            IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+            IRuntime::CreationOptions creation;
+            creation.m_MemoryOptimizerStrategyMap[kMi355x] = std::make_shared<testhost::PackingStrategy>();
+            IRuntimePtr rt = IRuntime::Create(creation);
             INetworkPtr net = block.Build();
             OptimizerOptionsOpaque options;
             options.AddModelOption(BackendOptions("Mi355x", {{"FuseAdditions", fused == 1}}));
             IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, rt->GetDeviceSpec(), options);
             NetworkId id = -1;
             std::string err;
-            REQUIRE(rt->LoadNetwork(id, std::move(opt), err) == Status::Success);
+            REQUIRE(rt->LoadNetwork(id, std::move(opt), err, external) == Status::Success);
             results[fused].assign(block.sum.GetNumBytes(), 0);
             InputTensors ins{{0, ConstTensor(constIn, input.data())}};
             OutputTensors outs{{0, Tensor(block.sum, results[fused].data())}};
@@ -2008,12 +2037,28 @@ TEST_CASE("runtime: an Addition whose sum was placed over the convolution's inpu
         CHECK(pairs[0] == 0);
         CHECK(pairs[1] == 1);
         CHECK(apart[0] == 0);
-        CHECK(apart[1] == 1);                              // first fit puts the sum at the start of the dead 256-channel tensor
+        CHECK(apart[1] == 1);                              // the strategy puts the sum at the start of the dead 256-channel tensor
         CHECK(results[0] == results[1]);
         const std::vector<uint8_t> a = OracleRun(block.first, input);
         const std::vector<uint8_t> b = OracleRun(block.last, a);
         const Diff d = Compare(results[1], OracleAddRelu(block.in, input, block.last.out, b, block.sum), DataType::QAsymmS8);
         std::printf("    narrowing residual block vs oracle: max |diff| %d, exact %.5f\n", d.maxAbs, 1.0 - static_cast<double>(d.mismatches) / static_cast<double>(d.n));
+        CHECK(d.maxAbs <= 2);
+        CHECK(d.mismatches * 1000 <= d.n);
+    }
+    // the same network in the backend's own arena, one stream: the pair runs as one launch
+    {
+        NarrowingResidualBlock block(4);
+        const std::vector<uint8_t> input = RandomActivations(block.in, 92);
+        const unsigned long long pairsBefore = Mi355xAdditionWorkload::PairsFormed(), apartBefore = Mi355xAdditionWorkload::PairsRunApart();
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        INetworkPtr net = block.Build();
+        const std::vector<uint8_t> got = RunOnRuntime(*rt, *net, {kMi355x}, block.in, input, block.sum);
+        CHECK(Mi355xAdditionWorkload::PairsFormed() - pairsBefore == 1);
+        CHECK(Mi355xAdditionWorkload::PairsRunApart() - apartBefore == 0);
+        const std::vector<uint8_t> a = OracleRun(block.first, input);
+        const std::vector<uint8_t> b = OracleRun(block.last, a);
+        const Diff d = Compare(got, OracleAddRelu(block.in, input, block.last.out, b, block.sum), DataType::QAsymmS8);
         CHECK(d.maxAbs <= 2);
         CHECK(d.mismatches * 1000 <= d.n);
     }

@@ -188,11 +188,12 @@ def parity_against_checker(net, dn, batch, checked):
     return out
 
 
-def run_backend_child(net, batch, steps, warmup, real=False):
+def run_backend_child(net, batch, steps, warmup, real=False, lanes=0):
     """The same network through the C++ backend (INetwork -> Optimize -> LoadNetwork -> IRuntime::EnqueueWorkload) in a
     child process, started before this process has touched the GPU.  Returns (figures, output bytes) or (error, None).
     real=True runs the build of the same program against an Arm NN source tree and its own libarmnn.so
-    (armnn_amd/backend/test/bin/real/, made by `make -C armnn_amd/backend real-runtime`), if it is there."""
+    (armnn_amd/backend/test/bin/real/, made by `make -C armnn_amd/backend real-runtime`), if it is there.
+    lanes > 0 sets the backend's lane count for the child (environment variable MI355X_LANES, which the backend reads once)."""
     import subprocess
     import tempfile
     import numpy as np
@@ -205,12 +206,17 @@ def run_backend_child(net, batch, steps, warmup, real=False):
         netfile.write_net(net, batch, nf)
         np.ascontiguousarray(nets.synthetic_input(net, batch).data).tofile(fin)
         try:
-            r = subprocess.run([exe, nf, fin, fout, str(steps), str(warmup)], capture_output=True, text=True, timeout=300)
+            env = dict(os.environ)
+            if lanes > 0:
+                env["MI355X_LANES"] = str(lanes)
+            r = subprocess.run([exe, nf, fin, fout, str(steps), str(warmup)], capture_output=True, text=True, timeout=300, env=env)
         except subprocess.TimeoutExpired:
             return {"error": "backend_bench timed out"}, None
         if r.returncode != 0:
             return {"error": f"backend_bench exit {r.returncode}: {r.stderr.strip()[-300:]}"}, None
         fig = json.loads(r.stdout.strip().splitlines()[-1])
+        if lanes > 0:
+            fig["lanes"] = lanes
         with open(fout, "rb") as f:
             return fig, f.read()
 
@@ -259,11 +265,19 @@ def main():
 
     # ---- the product path north_star names: the backend behind IRuntime::EnqueueWorkload, in a child process that is
     # started (and has ended) before anything here touches the GPU
+    if args.lanes == 0:
+        # Two lanes overlap the tails of one lane's launches with the other's; the 3x3 depthwise kernel sizes its grid to
+        # the whole device and walks its items itself, and two of those side by side get in each other's way
+        # (MobileNetV1, 64 images: 0.330 ms in one lane, 0.336 in two; ResNet-50, 32 images: 0.864 and 0.725).
+        depthwise = any(l.op == "depthwise" for l in net.layers)
+        args.lanes = 2 if batch >= 16 and batch % 2 == 0 and not depthwise else 1
     backend, backend_out = (None, None)
     real, real_out = (None, None)
     if not args.no_backend and not args.profile_pass:
-        backend, backend_out = run_backend_child(net, batch, max(50, args.steps // 4), 20)
-        real, real_out = run_backend_child(net, batch, max(50, args.steps // 4), 20, real=True)
+        # (the backend with the executor's lane count: through EnqueueWorkload MobileNetV1 b64 takes 0.306 ms in one lane
+        # against 0.327 in two with input and output resident)
+        backend, backend_out = run_backend_child(net, batch, max(50, args.steps // 4), 20, lanes=args.lanes)
+        real, real_out = run_backend_child(net, batch, max(50, args.steps // 4), 20, real=True, lanes=args.lanes)
 
     from armnn_amd import shim
     from armnn_amd.executor import DeviceNetwork
@@ -271,12 +285,6 @@ def main():
     for opt in args.option:
         name, _, value = opt.partition("=")
         shim.set_option(name, int(value))
-    if args.lanes == 0:
-        # Two lanes overlap the tails of one lane's launches with the other's; the 3x3 depthwise kernel sizes its grid to
-        # the whole device and walks its items itself, and two of those side by side get in each other's way
-        # (MobileNetV1, 64 images: 0.330 ms in one lane, 0.336 in two; ResNet-50, 32 images: 0.864 and 0.725).
-        depthwise = any(l.op == "depthwise" for l in net.layers)
-        args.lanes = 2 if batch >= 16 and batch % 2 == 0 and not depthwise else 1
     dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse="" if args.fuse == "none" else args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add, chain=args.chain, fuse_tail=args.fuse_tail)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev
