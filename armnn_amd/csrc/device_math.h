@@ -344,7 +344,9 @@ inline AddFuse MakeAddFuse(const mi355x_quant& a, const mi355x_quant& r, const m
     return f;
 }
 
-// four codes of each input (dwords wa, wb) -> packed dword of the four sums' codes
+// four codes of each input (dwords wa, wb) -> packed dword of the four sums' codes.  CLAMP = false: the caller knows that the
+// activation's clamp is the type's own range (rq.pk_full), which the conversion already applies.
+template <bool CLAMP = true>
 __device__ __forceinline__ uint32_t AddQuantize4Dev(uint32_t wa, uint32_t wb, const AddFuse& f)
 {
     if (!f.bracket_ok)
@@ -363,7 +365,7 @@ __device__ __forceinline__ uint32_t AddQuantize4Dev(uint32_t wa, uint32_t wb, co
     {
         float p = __fmaf_rn(af[i], f.ka, __fmaf_rn(bf[i], f.kb, f.k0p));
         float m = __fsub_rn(p, f.two_c);
-        if (!f.rq.pk_full)
+        if constexpr (CLAMP)
         {
             p = __builtin_amdgcn_fmed3f(p, f.rq.pk_lo_f, f.rq.pk_hi_f);
             m = __builtin_amdgcn_fmed3f(m, f.rq.pk_lo_f, f.rq.pk_hi_f);
@@ -389,7 +391,7 @@ __device__ __forceinline__ StoreVec4 AddResidual16(const StoreVec4& own, const S
 {
     StoreVec4 o;
 #pragma unroll
-    for (int d = 0; d < 4; ++d) o[d] = static_cast<int>(AddQuantize4Dev(static_cast<uint32_t>(own[d]), static_cast<uint32_t>(other[d]), f));
+    for (int d = 0; d < 4; ++d) o[d] = static_cast<int>(AddQuantize4Dev<true>(static_cast<uint32_t>(own[d]), static_cast<uint32_t>(other[d]), f));
     return o;
 }
 

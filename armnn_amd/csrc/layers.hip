@@ -280,6 +280,7 @@ __global__ __launch_bounds__(256) void GlobalPoolKernel(PoolArgs p, QIn qin, Req
 }
 
 // 16 elements per thread, 16-byte loads and stores
+template <bool CLAMP>
 __global__ __launch_bounds__(256) void AddVec16Kernel(AddFuse f, const v4u* __restrict__ x0,
                                                       const v4u* __restrict__ x1, v4u* __restrict__ y, size_t n16)
 {
@@ -291,7 +292,7 @@ __global__ __launch_bounds__(256) void AddVec16Kernel(AddFuse f, const v4u* __re
         const v4u a = x0[i], b = x1[i];
         v4u o;
 #pragma unroll
-        for (int d = 0; d < 4; ++d) o[d] = AddQuantize4Dev(a[d], b[d], f);
+        for (int d = 0; d < 4; ++d) o[d] = AddQuantize4Dev<CLAMP>(a[d], b[d], f);
         StoreOut16(outp, static_cast<long long>(i) * 16, StoreVec4{static_cast<int>(o[0]), static_cast<int>(o[1]), static_cast<int>(o[2]), static_cast<int>(o[3])});
     }
 }
@@ -515,8 +516,13 @@ int mi355x_add_run(size_t n, const mi355x_quant* in0_q, const mi355x_quant* in1_
     if (vec16)
     {
         NoteKernel("AddVec16Kernel");
-        hipLaunchKernelGGL(AddVec16Kernel, dim3(GridFor(n / 16)), dim3(256), 0, ToHip(stream), MakeAddFuse(*in0_q, *in1_q, *out_q, activation, a, b),
-                           static_cast<const v4u*>(input0_dev), static_cast<const v4u*>(input1_dev), static_cast<v4u*>(output_dev), n / 16);
+        const AddFuse f = MakeAddFuse(*in0_q, *in1_q, *out_q, activation, a, b);
+        if (f.rq.pk_full)
+            hipLaunchKernelGGL(AddVec16Kernel<false>, dim3(GridFor(n / 16)), dim3(256), 0, ToHip(stream), f,
+                               static_cast<const v4u*>(input0_dev), static_cast<const v4u*>(input1_dev), static_cast<v4u*>(output_dev), n / 16);
+        else
+            hipLaunchKernelGGL(AddVec16Kernel<true>, dim3(GridFor(n / 16)), dim3(256), 0, ToHip(stream), f,
+                               static_cast<const v4u*>(input0_dev), static_cast<const v4u*>(input1_dev), static_cast<v4u*>(output_dev), n / 16);
     }
     else
     {

@@ -4,6 +4,9 @@
   python -m armnn_amd.layerbench dw   --n 64 --h 112 --w 112 --c 32 --stride 1
   python -m armnn_amd.layerbench fc   --m 2048 --k 4096 --o 4096
   python -m armnn_amd.layerbench pad  --n 64 --h 112 --w 112 --c 64        (one row and column on every side)
+  python -m armnn_amd.layerbench add  --n 16 --h 56 --w 56 --c 256         (Addition of two tensors with a fused ReLU)
+  python -m armnn_amd.layerbench tail --n 64 --h 7 --w 7 --c 1024 --o 1001 (global average pooling -> FullyConnected ->
+                                                                            Softmax: three launches and one launch)
 
 Prints one JSON line: kernel chosen, average launch time (HIP events on the launch stream), algorithmic
 ops and bytes, and the fraction of the int8 MFMA peak (5.0 POP/s) or of the HBM peak (8 TB/s).
@@ -57,9 +60,77 @@ def _pad(dev, a, adt, zp):
     return 0
 
 
+def _timed(dev, stream, run, a):
+    for _ in range(a.warmup):
+        run()
+    e0, e1 = dev.event(), dev.event()
+    dev.event_record(e0, stream)
+    for _ in range(a.iters):
+        run()
+    dev.event_record(e1, stream)
+    dev.event_sync(e1)
+    return dev.elapsed_ms(e0, e1) / a.iters
+
+
+def _add(dev, a, adt, zp):
+    """Addition of two NHWC tensors (quantizations of a ResNet-50 residual block: convolution output + block input -> sum,
+    ReLU fused): two bytes read and one written per element."""
+    import ctypes as C
+    lo = 0 if a.u8 else -128
+    shape = (a.n, a.h, a.w, a.c)
+    s0, s1, so = a.scales
+    q0, q1, qo = TensorInfo(shape, adt, (s0,), lo), TensorInfo(shape, adt, (s1,), lo), TensorInfo(shape, adt, (so,), lo)
+    lib = shim.load_library()
+    n = q0.num_elements
+    x0 = shim.DeviceBuffer(n).upload(synth.uniform_int(1, shape, 0, 255, np.uint8))
+    x1 = shim.DeviceBuffer(n).upload(synth.uniform_int(2, shape, 0, 255, np.uint8))
+    y = shim.DeviceBuffer(n)
+    stream = dev.stream()
+    a0, a1, ao = shim._quant(q0), shim._quant(q1), shim._quant(qo)
+    run = lambda: shim._chk(lib.mi355x_add_run(n, C.byref(a0), C.byref(a1), C.byref(ao), shim.ACT_RELU, 0.0, 0.0, x0.ptr, x1.ptr, y.ptr, stream))
+    ms = _timed(dev, stream, run, a)
+    print(json.dumps({"layer": f"add N={a.n} {a.h}x{a.w}x{a.c} + ReLU, scales {s0} + {s1} -> {so}", "kernel": shim.last_kernel(), "us": ms * 1e3, "elements": n,
+                      "GBps": 3 * n / (ms * 1e-3) / 1e9, "frac_hbm_peak": 3 * n / (ms * 1e-3) / HBM_PEAK, "bytes": 3 * n}))
+    return 0
+
+
+def _tail(dev, a, adt, zp):
+    """Global average pooling -> FullyConnected -> Softmax over a.n images of a.h x a.w x a.c with a.o classes: the three
+    launches one behind the other, and the one launch of mi355x_tail_run (same bytes)."""
+    import ctypes as C
+    lo = 0 if a.u8 else -128
+    lib = shim.load_library()
+    xin = TensorInfo((a.n, a.h, a.w, a.c), adt, (0.0235,), lo)
+    pooled = TensorInfo((a.n, a.c), adt, (0.0235,), lo)
+    logits = TensorInfo((a.n, a.o), adt, (0.1,), lo + 70)
+    probs = TensorInfo((a.n, a.o), adt, (1.0 / 256,), lo)
+    ws = synth.scales(3, a.o)
+    w = QTensor(TensorInfo((a.o, a.c), DataType.QSymmS8, tuple(ws), 0, 0), synth.int8_weights(2, (a.o, a.c)))
+    b = QTensor(TensorInfo((a.o,), DataType.Signed32, tuple(np.float32(0.0235) * ws), 0, 0), synth.int32_bias(4, a.o))
+    fc = shim.FullyConnectedPlan(pooled, w, b, logits)
+    d = shim.Pool2dDesc(a.h, a.w, a.c, 1, 1, a.w, a.h, 1, 1, 0, 0, 0, 0, 1, 1, shim._quant(xin), shim._quant(pooled))
+    tail = shim.ClassifierTail(d, fc, 1.0, probs)
+    xd = shim.DeviceBuffer(xin.num_elements).upload(synth.uniform_int(1, xin.shape, 0, 255, np.uint8))
+    pd, ld, yd = shim.DeviceBuffer(pooled.num_elements), shim.DeviceBuffer(logits.num_elements), shim.DeviceBuffer(probs.num_elements)
+    stream = dev.stream()
+    qi, qo = shim._quant(logits), shim._quant(probs)
+
+    def three():
+        shim._chk(lib.mi355x_pool2d_run(C.byref(d), a.n, xd.ptr, pd.ptr, stream))
+        fc.run(a.n, pd.ptr, ld.ptr, stream)
+        shim._chk(lib.mi355x_softmax_run(a.n, a.o, 1.0, C.byref(qi), C.byref(qo), ld.ptr, yd.ptr, stream))
+
+    ms3 = _timed(dev, stream, three, a)
+    ms1 = _timed(dev, stream, lambda: tail.run(a.n, xd.ptr, pd.ptr, ld.ptr, yd.ptr, stream), a)
+    kernel = shim.last_kernel()
+    print(json.dumps({"layer": f"tail N={a.n} {a.h}x{a.w}x{a.c} -> {a.o}", "three_launches_us": ms3 * 1e3, "one_launch_us": ms1 * 1e3,
+                      "kernel": kernel, "waits_given_up": tail.gave_up()}))
+    return 0
+
+
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("op", choices=["conv", "dw", "fc", "pad"])
+    ap.add_argument("op", choices=["conv", "dw", "fc", "pad", "add", "tail"])
     ap.add_argument("--n", type=int, default=64)
     ap.add_argument("--h", type=int, default=56)
     ap.add_argument("--w", type=int, default=56)
@@ -76,6 +147,8 @@ def main(argv=None):
     ap.add_argument("--wspread", type=int, default=1, metavar="FACTOR",
                     help="with --wzp: multiply the weight draws (std 30) by this before adding the zero point; 3 spreads the "
                          "codes over the whole uint8 range, so that weight minus zero point no longer fits int8")
+    ap.add_argument("--scales", type=float, nargs=3, default=(0.0235, 0.1, 0.1), metavar=("IN0", "IN1", "OUT"),
+                    help="add: the three quantization scales (the default, 0.0235 + 0.1 -> 0.1, makes one sum in 200 an exact tie)")
     ap.add_argument("--algo", type=int, default=0)
     ap.add_argument("--iters", type=int, default=500, help="timed launches; long enough for the clocks to settle")
     ap.add_argument("--warmup", type=int, default=200)
@@ -90,6 +163,10 @@ def main(argv=None):
     zp = 128 if a.u8 else -3
     if a.op == "pad":
         return _pad(dev, a, adt, zp)
+    if a.op == "add":
+        return _add(dev, a, adt, zp)
+    if a.op == "tail":
+        return _tail(dev, a, adt, zp)
     act = (shim.ACT_BOUNDED_RELU, 6.0, 0.0)
     if a.op == "fc":
         k, o, m = a.k if a.k > 3 else 4096, a.o, a.m
