@@ -5,6 +5,9 @@
   python -m armnn_amd.layerbench fc   --m 2048 --k 4096 --o 4096
   python -m armnn_amd.layerbench pad  --n 64 --h 112 --w 112 --c 64        (one row and column on every side)
   python -m armnn_amd.layerbench add  --n 16 --h 56 --w 56 --c 256         (Addition of two tensors with a fused ReLU)
+  python -m armnn_amd.layerbench dwpw --n 64 --h 14 --w 14 --c 512 --co 512 --stride 1
+                                                                           (3x3 depthwise + the 1x1 convolution behind it, as
+                                                                            one launch: mi355x_conv2d_run_fused)
   python -m armnn_amd.layerbench tail --n 64 --h 7 --w 7 --c 1024 --o 1001 (global average pooling -> FullyConnected ->
                                                                             Softmax: three launches and one launch)
 
@@ -94,6 +97,39 @@ def _add(dev, a, adt, zp):
     return 0
 
 
+def _dwpw(dev, a, adt, zp):
+    """3x3 depthwise (ReLU6) + 1x1 convolution (ReLU6) over uint8-style activations, as MobileNetV1 has them, run as one
+    launch; algorithmic bytes: input + output + both layers' constants (the tensor between them never exists)."""
+    lo = 0 if a.u8 else -128
+    ho, pt = _same(a.h, 3, a.stride)
+    wo, pl = _same(a.w, 3, a.stride)
+    xin = TensorInfo((a.n, a.h, a.w, a.c), adt, (0.0235,), lo)
+    mid = TensorInfo((a.n, ho, wo, a.c), adt, (0.0235,), lo)
+    yout = TensorInfo((a.n, ho, wo, a.co), adt, (0.0235,), lo)
+    wsd = synth.scales(3, a.c) / np.float32(1.0)
+    wd = QTensor(TensorInfo((1, 3, 3, a.c), DataType.QSymmS8, tuple(wsd), 0, 3), synth.int8_weights(2, (1, 3, 3, a.c)))
+    bd = QTensor(TensorInfo((a.c,), DataType.Signed32, tuple(np.float32(0.0235) * wsd), 0, 0), synth.int32_bias(4, a.c))
+    wsp = synth.scales(5, a.co) / np.float32(np.sqrt(a.c) / 3.0)
+    wp = QTensor(TensorInfo((a.co, 1, 1, a.c), DataType.QSymmS8, tuple(wsp), 0, 0), synth.int8_weights(6, (a.co, 1, 1, a.c)))
+    bp = QTensor(TensorInfo((a.co,), DataType.Signed32, tuple(np.float32(0.0235) * wsp), 0, 0), synth.int32_bias(7, a.co))
+    act = (shim.ACT_BOUNDED_RELU, 6.0, 0.0)
+    pdw = shim.Conv2dPlan(xin, wd, bd, mid, pad_top=pt, pad_left=pl, stride_x=a.stride, stride_y=a.stride, depthwise=True,
+                          activation=act[0], act_a=act[1], act_b=act[2])
+    ppw = shim.Conv2dPlan(mid, wp, bp, yout, activation=act[0], act_a=act[1], act_b=act[2])
+    if not pdw.fusable_with(ppw):
+        raise SystemExit("the pair is not fusable: " + shim.load_library().mi355x_last_error().decode())
+    xd = shim.DeviceBuffer(xin.num_elements).upload(synth.uniform_int(1, xin.shape, 0, 255, np.uint8))
+    yd = shim.DeviceBuffer(yout.num_elements)
+    stream = dev.stream()
+    ms = _timed(dev, stream, lambda: pdw.run_fused(ppw, a.n, xd.ptr, yd.ptr, stream), a)
+    nbytes = xin.num_elements + yout.num_elements + 9 * a.c + 8 * a.c + a.c * a.co + 8 * a.co
+    ops = 2.0 * a.n * ho * wo * a.co * a.c
+    print(json.dumps({"layer": f"dw3x3 s{a.stride} + pw N={a.n} {a.h}x{a.w}x{a.c}->{a.co}", "kernel": shim.last_kernel(), "us": ms * 1e3,
+                      "GBps": nbytes / (ms * 1e-3) / 1e9, "frac_hbm_peak": nbytes / (ms * 1e-3) / HBM_PEAK, "bytes": nbytes,
+                      "pointwise_TOPS": ops / (ms * 1e-3) / 1e12, "recommended_by_the_library": bool(pdw.fusion_pays(ppw, a.n))}))
+    return 0
+
+
 def _tail(dev, a, adt, zp):
     """Global average pooling -> FullyConnected -> Softmax over a.n images of a.h x a.w x a.c with a.o classes: the three
     launches one behind the other, and the one launch of mi355x_tail_run (same bytes)."""
@@ -130,7 +166,7 @@ def _tail(dev, a, adt, zp):
 
 def main(argv=None):
     ap = argparse.ArgumentParser()
-    ap.add_argument("op", choices=["conv", "dw", "fc", "pad", "add", "tail"])
+    ap.add_argument("op", choices=["conv", "dw", "fc", "pad", "add", "tail", "dwpw"])
     ap.add_argument("--n", type=int, default=64)
     ap.add_argument("--h", type=int, default=56)
     ap.add_argument("--w", type=int, default=56)
@@ -167,6 +203,8 @@ def main(argv=None):
         return _add(dev, a, adt, zp)
     if a.op == "tail":
         return _tail(dev, a, adt, zp)
+    if a.op == "dwpw":
+        return _dwpw(dev, a, adt, zp)
     act = (shim.ACT_BOUNDED_RELU, 6.0, 0.0)
     if a.op == "fc":
         k, o, m = a.k if a.k > 3 else 4096, a.o, a.m
