@@ -1769,7 +1769,7 @@ TEST_CASE("runtime: two host threads, each with a runtime and a network of its o
             IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
             INetworkPtr net = m.Build();
             for (int i = 0; i < 4; ++i)
-                if (RunOnRuntime(*rt, *net, {kMi355x}, m.in, in, m.probs, 3) != want) problems[which] = "bytes differ in round " + std::to_string(i);
+                if (RunOnRuntime(*rt, *net, {kMi355x}, m.in, in, m.probs, 3) != want) problems[which] = "bytes differ in pass " + std::to_string(i);
         }
         catch (const std::exception& e) { problems[which] = e.what(); }
     };
