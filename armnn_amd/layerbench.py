@@ -76,8 +76,8 @@ def _timed(dev, stream, run, a):
 
 
 def _add(dev, a, adt, zp):
-    """Addition of two NHWC tensors (quantizations of a ResNet-50 residual block: convolution output + block input -> sum,
-    ReLU fused): two bytes read and one written per element."""
+    """Addition of two NHWC tensors with a fused ReLU, quantization scales from --scales: two bytes read and one written per
+    element."""
     import ctypes as C
     lo = 0 if a.u8 else -128
     shape = (a.n, a.h, a.w, a.c)
