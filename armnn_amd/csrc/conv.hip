@@ -1691,6 +1691,14 @@ int mi355x_conv2d_fusable(mi355x_conv2d_t dw, mi355x_conv2d_t pw)
 int mi355x_conv2d_fusion_pays(mi355x_conv2d_t first, mi355x_conv2d_t second, uint32_t batch)
 {
     if (!first || !second || batch == 0) return 0;
+    if (!first->d.depthwise && second->d.depthwise)
+    {
+        // 1x1 convolution + the depthwise layer behind it, whole images per block: measured on maps of 7 x 7 with 64 images
+        // per launch (512 -> 1024 channels: 12.5 us against 13.9 us as two launches); larger maps gain more as the second
+        // half of a depthwise + pointwise pair
+        if (GlobalOptions().pwdw_auto == 0 || PwDwCheck(first, second, nullptr) != 0) return 0;
+        return first->d.out_h <= 7 && first->d.out_w <= 7 && batch >= 64 ? 1 : 0;
+    }
     if (!first->d.depthwise || second->d.depthwise) return 0;
     if (GlobalOptions().dwpw_stream != 0 && DwPwStreamShape(first, second) != 0 && mi355x_conv2d_fusable(first, second) == 0)
     {

@@ -172,6 +172,8 @@ class DeviceNetwork:
         elif fuse == "auto":
             # only the pairs the library recommends as one launch at the batch a launch sees
             self._fuse_pairs(("depthwise", "conv"), only_where_it_pays=True)
+            # ... and, among the layers still on their own, 1x1 convolution + the depthwise layer behind it where recommended
+            self._fuse_pairs(("conv", "depthwise"), only_where_it_pays=True)
         if fuse_add:
             self._fuse_additions()
         if chain:

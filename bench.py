@@ -409,7 +409,7 @@ def main():
         # layer's ops and the pair's bytes (input, output, constants; the tensor between the layers never exists)
         t = sum(r["ms"] for r in fused_rows) * 1e-3
         by_name = {l.name: l for l, _, _ in per_layer}
-        ops = sum(2.0 * by_name[r["layer"]].parts[1].macs_per_image * launch_batch for r in fused_rows)
+        ops = sum(2.0 * next(part for part in by_name[r["layer"]].parts if part.op == "conv").macs_per_image * launch_batch for r in fused_rows)
         nbytes = sum(r["work"] for r in fused_rows)
         groups["fused_depthwise_pointwise"] = {"ms": t * 1e3, "launches": len(fused_rows), "TOPS": ops / t / 1e12, "frac_of_int8_mfma_peak": ops / t / INT8_MFMA_PEAK_OPS,
                                                "GBps": nbytes / t / 1e9, "frac_of_hbm_peak": nbytes / t / HBM_PEAK_BYTES}

@@ -123,6 +123,8 @@ int  mi355x_abi_version(void);
  *   "dwpw_stream" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a depthwise layer of 32, 64 (stride 2) or
  *   128 channels and the pointwise layer behind it (64, 128, 128 / 256 output channels) on the persistent kernel that keeps the
  *   pointwise weights in on-chip memory (identical bytes; lets tests compare it with the older fused kernel).
+ *   "pwdw_auto" = 1 | 0: mi355x_conv2d_fusion_pays may (1) or may not (0) recommend a 1x1 convolution + the depthwise layer
+ *   behind it (tests and tuning).
  *   "dwpw_panel" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a depthwise layer of 256 or 512
  *   channels and a pointwise layer of 256 or 512 output channels on the kernel that gives a block an 8 x 8 pixel tile over
  *   all channels (identical bytes; lets tests compare it with the older fused kernel).
@@ -263,8 +265,9 @@ int mi355x_conv2d_fusable(mi355x_conv2d_t first, mi355x_conv2d_t second);
  * 2 -- 256 output channels) in launches of at least 1024 tiles of 8 x 8 output pixels, which run on the persistent kernel
  * that keeps the pointwise weights on chip; and a depthwise layer over 256 or 512 channels (stride 1, or stride 2 from 256
  * to 512 channels) and the pointwise layer of 256 or 512 output channels behind it in launches of at least 100 such tiles,
- * which run on the kernel that gives a block an 8 x 8 pixel tile over all channels.  No counterpart in the reference,
- * which has no fused workloads on CpuRef. */
+ * which run on the kernel that gives a block an 8 x 8 pixel tile over all channels; and, in the other order, a 1x1
+ * convolution and the depthwise layer behind it on maps of at most 7 x 7 pixels in launches of at least 64 images (option
+ * "pwdw_auto" = 0 turns this one off).  No counterpart in the reference, which has no fused workloads on CpuRef. */
 int mi355x_conv2d_fusion_pays(mi355x_conv2d_t first, mi355x_conv2d_t second, uint32_t batch);
 int mi355x_conv2d_run_fused(mi355x_conv2d_t first, mi355x_conv2d_t second, uint32_t batch,
                             const void* input_dev, void* output_dev, mi355x_stream_t stream);

@@ -133,6 +133,26 @@ def test_mobilenet_v1_batch64_rows_equal_batch2_runs():
     _rows_equal_small_batch_runs(nets.mobilenet_v1(), 64, (0, 31, 62), lanes=2)
 
 
+def test_mobilenet_v1_batch64_as_the_benchmark_runs_it_rows_equal_batch2_runs():
+    """bench.py's configuration: one lane, the pairs the library recommends as one launch each (eleven depthwise + pointwise
+    pairs on the fused kernels, and pw12 + dw13 in the other order), replayed as a graph."""
+    net = nets.mobilenet_v1()
+    x = nets.synthetic_input(net, 64)
+    big = DeviceNetwork(net, 64, use_graph=True, lanes=1, fuse="auto")
+    names = [l.name for l, _ in big.steps]
+    assert names == (["stem"] + [f"dw{i}+pw{i}" for i in range(1, 12)] + ["dw12", "pw12+dw13", "pw13", "avgpool", "logits", "softmax"]), names
+    y = big.run(x)
+    for _ in range(2):                                    # replays give the same bytes
+        big.enqueue()
+        np.testing.assert_array_equal(big.download().data, y.data)
+    big.close()
+    small = DeviceNetwork(net, 2, use_graph=False)
+    for i in (0, 17, 40, 62):
+        yi = small.run(QTensor(net.info(net.input, 2), np.ascontiguousarray(x.data[i:i + 2])))
+        np.testing.assert_array_equal(yi.data, y.data[i:i + 2], err_msg=f"images {i},{i + 1} of 64")
+    small.close()
+
+
 def test_mobilenet_v1_batch64_in_one_lane_rows_equal_batch2_runs():
     # 64 images per launch: the largest launches of the benchmark (persistent blocks walk the most tiles here)
     _rows_equal_small_batch_runs(nets.mobilenet_v1(), 64, (0, 20, 42, 62), lanes=1)
