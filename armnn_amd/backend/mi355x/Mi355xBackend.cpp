@@ -242,6 +242,8 @@ BackendCapabilities Mi355xBackend::GetCapabilities() const
 // * A DepthwiseConvolution2d whose output goes to one unpadded 1x1 stride-1 Convolution2d of this backend and nowhere else
 //   is marked (Mi355xLayerNote, which also carries the fused activation): the two workloads may then run as one launch
 //   (Mi355xConvolution2dWorkload::TakeOver).
+// * An unpadded 1x1 stride-1 Convolution2d whose output goes to one Pooling2d of this backend over the whole unpadded image
+//   and nowhere else is marked the same way: the two workloads may then run as one launch (Mi355xPooling2dWorkload::TakeOver).
 // * A Reshape that only flattens the dimensions behind the batch, in front of a FullyConnected, is dropped: the
 //   FullyConnected reads the unflattened tensor (same bytes in the same order).
 // * A constant Pad of height and width in front of a Convolution2d, DepthwiseConvolution2d or Pooling2d moves into that
@@ -257,9 +259,12 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
     bool fuseAdditions = true;
     // ... {{"FuseDepthwisePointwise", false}} keeps every depthwise layer and the 1x1 convolution behind it two launches
     bool fuseDepthwisePointwise = true;
+    // ... {{"FuseConvolutionPooling", false}} keeps every 1x1 convolution and the pooling over its whole image two launches
+    bool fuseConvolutionPooling = true;
     ParseOptions(modelOptions, Mi355xBackendId(), [&](const std::string& name, const BackendOptions::Var& value) {
         if (name == "FuseAdditions" && value.IsBool()) fuseAdditions = value.AsBool();
         if (name == "FuseDepthwisePointwise" && value.IsBool()) fuseDepthwisePointwise = value.AsBool();
+        if (name == "FuseConvolutionPooling" && value.IsBool()) fuseConvolutionPooling = value.AsBool();
     });
 
     for (IConnectableLayer* il : layers)
@@ -361,7 +366,38 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
                 if (const Mi355xLayerNote* note = Mi355xLayerNote::From(base->GetAdditionalInformation<ActivationDescriptor>().get()))
                     if (note->onlyConsumerIsAPointwiseConvolution) pointwiseNext = false;
         }
-        if (!pad && !act && !residual && !flat && !pointwiseNext) continue;
+        // an unpadded 1x1 stride-1 Convolution2d (with the Activation fused into it, if any) whose only consumer is a Pooling2d
+        // of this backend over the whole unpadded image: the two workloads may run as one launch
+        // (Mi355xPooling2dWorkload::TakeOver)
+        bool poolingNext = false;
+        if (fuseConvolutionPooling && type == LayerType::Convolution2d && !residual && !pad)
+        {
+            Layer* lastOfThis = act ? act : base;
+            const OutputSlot* weights = base->GetInputSlot(1).GetConnectedOutputSlot();
+            const bool pointwise = weights != nullptr && weights->GetTensorInfo().GetNumDimensions() == 4 &&
+                                   weights->GetTensorInfo().GetShape()[1] == 1 && weights->GetTensorInfo().GetShape()[2] == 1 &&
+                                   conv.m_StrideX == 1 && conv.m_StrideY == 1 && conv.m_PadLeft == 0 && conv.m_PadRight == 0 &&
+                                   conv.m_PadTop == 0 && conv.m_PadBottom == 0 && conv.m_DataLayout == DataLayout::NHWC;
+            if (pointwise && lastOfThis->GetOutputSlot(0).GetNumConnections() == 1)
+            {
+                Layer* next = &lastOfThis->GetOutputSlot(0).GetConnections()[0]->GetOwningLayer();
+                if (next->GetType() == LayerType::Pooling2d && members.count(next))
+                {
+                    const auto& pd = static_cast<const Pooling2dDescriptor&>(next->GetParameters());
+                    const TensorInfo& image = lastOfThis->GetOutputSlot(0).GetTensorInfo();
+                    const TensorInfo& pooled = next->GetOutputSlot(0).GetTensorInfo();
+                    poolingNext = pd.m_DataLayout == DataLayout::NHWC && image.GetNumDimensions() == 4 && pooled.GetNumDimensions() == 4 &&
+                                  pd.m_PoolHeight == image.GetShape()[1] && pd.m_PoolWidth == image.GetShape()[2] &&
+                                  pooled.GetShape()[1] == 1 && pooled.GetShape()[2] == 1 && pd.m_PadLeft == 0 && pd.m_PadRight == 0 &&
+                                  pd.m_PadTop == 0 && pd.m_PadBottom == 0 &&
+                                  (pd.m_PoolType == PoolingAlgorithm::Max || pd.m_PoolType == PoolingAlgorithm::Average);
+                }
+            }
+            if (poolingNext && !act)
+                if (const Mi355xLayerNote* note = Mi355xLayerNote::From(base->GetAdditionalInformation<ActivationDescriptor>().get()))
+                    if (note->onlyConsumerIsAGlobalPooling) poolingNext = false;
+        }
+        if (!pad && !act && !residual && !flat && !pointwiseNext && !poolingNext) continue;
 
         std::string name = base->GetName();
         if (pad) name = std::string("folded-") + pad->GetName() + "-into-" + name;
@@ -383,11 +419,12 @@ OptimizationViews Mi355xBackend::OptimizeSubgraphView(const SubgraphView& subgra
         }
         Layer* last = act ? act : base;
         replacement->GetOutputSlot(0).SetTensorInfo(last->GetOutputSlot(0).GetTensorInfo());
-        if (pointwiseNext)
+        if (pointwiseNext || poolingNext)
         {
             auto carried = base->GetAdditionalInformation<ActivationDescriptor>();
             PolymorphicDowncast<Layer*>(replacement)->SetAdditionalInfoForObject(
-                Mi355xLayerNote::Make(act ? &static_cast<const ActivationDescriptor&>(act->GetParameters()) : carried.get(), true));
+                Mi355xLayerNote::Make(act ? &static_cast<const ActivationDescriptor&>(act->GetParameters()) : carried.get(), pointwiseNext,
+                                      poolingNext));
         }
         else if (act)
             PolymorphicDowncast<Layer*>(replacement)->SetAdditionalInfoForObject(

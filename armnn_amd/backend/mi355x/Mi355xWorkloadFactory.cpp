@@ -108,7 +108,7 @@ std::unique_ptr<IWorkload> Mi355xWorkloadFactory::CreateWorkload(LayerType type,
             auto w = std::make_unique<CandidateConvolution>(*PolymorphicDowncast<const Convolution2dQueueDescriptor*>(&descriptor), info, m_Candidate);
             // the depthwise layer created just before, marked as feeding only this kind of convolution: the two run as a pair
             w->TakeOver(depthwise);
-            if (w->FeedsOnlyAnAddition())
+            if (w->FeedsOnlyAnAddition() || w->OnlyConsumerIsAGlobalPooling())
             {
                 std::lock_guard<std::mutex> lock(m_Candidate->mutex);
                 m_Candidate->convolution = w.get();
@@ -130,7 +130,11 @@ std::unique_ptr<IWorkload> Mi355xWorkloadFactory::CreateWorkload(LayerType type,
         case LayerType::Activation:
             return std::make_unique<Mi355xActivationWorkload>(*PolymorphicDowncast<const ActivationQueueDescriptor*>(&descriptor), info);
         case LayerType::Pooling2d:
-            return std::make_unique<Mi355xPooling2dWorkload>(*PolymorphicDowncast<const Pooling2dQueueDescriptor*>(&descriptor), info);
+        {
+            auto w = std::make_unique<Mi355xPooling2dWorkload>(*PolymorphicDowncast<const Pooling2dQueueDescriptor*>(&descriptor), info);
+            w->TakeOver(candidate);
+            return w;
+        }
         case LayerType::Mean:
             return std::make_unique<Mi355xMeanWorkload>(*PolymorphicDowncast<const MeanQueueDescriptor*>(&descriptor), info);
         case LayerType::Pad:

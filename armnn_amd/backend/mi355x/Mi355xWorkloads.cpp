@@ -134,13 +134,16 @@ namespace
 std::mutex g_NotesMutex;
 std::set<const void*> g_Notes;
 std::atomic<unsigned long long> g_DepthwisePairsFormed{0}, g_DepthwisePairsRunFused{0}, g_DepthwisePairsRunApart{0};
+std::atomic<unsigned long long> g_PoolingPairsFormed{0}, g_PoolingPairsRunFused{0}, g_PoolingPairsRunApart{0};
 }
 
-std::shared_ptr<void> Mi355xLayerNote::Make(const ActivationDescriptor* activation, bool onlyConsumerIsAPointwiseConvolution)
+std::shared_ptr<void> Mi355xLayerNote::Make(const ActivationDescriptor* activation, bool onlyConsumerIsAPointwiseConvolution,
+                                            bool onlyConsumerIsAGlobalPooling)
 {
     auto* note = new Mi355xLayerNote;
     note->activation = activation ? *activation : Mi355xFeedsOnlyAnAddition();
     note->onlyConsumerIsAPointwiseConvolution = onlyConsumerIsAPointwiseConvolution;
+    note->onlyConsumerIsAGlobalPooling = onlyConsumerIsAGlobalPooling;
     {
         std::lock_guard<std::mutex> lock(g_NotesMutex);
         g_Notes.insert(note);
@@ -168,6 +171,13 @@ Mi355xConvolution2dWorkload::Mi355xConvolution2dWorkload(const Convolution2dQueu
     ARMNN_REPORT_PROFILING_WORKLOAD_DESC("Mi355xConvolution2dWorkload_Construct", descriptor.m_Parameters, info, this->GetGuid());
     if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xConvolution2dWorkload: NHWC only");
     m_FeedsOnlyAnAddition = Mi355xFusedActivation::From(m_Data.GetAdditionalInformation<ActivationDescriptor>()).feedsOnlyAnAddition;   // validates early
+    if (const Mi355xLayerNote* note = Mi355xLayerNote::From(m_Data.m_AdditionalInfoObject))
+        if (note->onlyConsumerIsAGlobalPooling)
+        {
+            // a note without an activation carries the identity, which is also how a plain descriptor marks "feeds an Addition"
+            m_OnlyConsumerIsAGlobalPooling = true;
+            m_FeedsOnlyAnAddition = false;
+        }
 }
 
 Mi355xConvolution2dWorkload::~Mi355xConvolution2dWorkload()
@@ -232,8 +242,45 @@ void Mi355xConvolution2dWorkload::BuildPlan() const
 
 void Mi355xConvolution2dWorkload::Execute() const
 {
-    if (m_RunsInsideTheAddition) return;
+    if (m_RunsInsideTheAddition || m_RunsInsideThePooling) return;
     ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xConvolution2dWorkload_Execute");
+    ExecuteOwn();
+}
+
+bool Mi355xConvolution2dWorkload::ExecuteWithPooling(const mi355x_pool2d_desc& pool, ITensorHandle* pooled, const TensorInfo& pooledInfo) const
+{
+    // (no profiling event of its own: the pooling workload's event covers the pair, as an Addition's covers its convolution)
+    std::call_once(m_Once, [this] { BuildPlan(); });
+    if (!m_Plan) throw RuntimeException("Mi355xConvolution2dWorkload: no device plan (its creation failed earlier)");
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const uint32_t batch = in.GetShape()[0];
+    if (m_FusePool < 0)
+        m_FusePool = mi355x_conv2d_pool_fusable(m_Plan, &pool) == 0 &&
+                     mi355x_conv2d_pool_fusion_pays(m_Plan, &pool, batch / mi355x::LanesFor(batch)) == 1 ? 1 : 0;
+    const unsigned char* x = static_cast<const unsigned char*>(In(m_Data.m_Inputs[0]));
+    unsigned char* y = static_cast<unsigned char*>(Out(pooled));
+    // as with the other pairs: the pooled tensor may have been placed where the convolution's input lies
+    const bool overlap = x < y + pooledInfo.GetNumBytes() && y < x + in.GetNumBytes();
+    const bool aligned = (reinterpret_cast<uintptr_t>(x) & 15) == 0;
+    if (m_FusePool != 1 || overlap || !aligned)
+    {
+        g_PoolingPairsRunApart.fetch_add(1);
+        ExecuteOwn();
+        return false;
+    }
+    // the depthwise layer in front of this convolution, if it left its execution to this workload, runs first as it is:
+    // the pair (depthwise, this convolution) as one launch would write the tensor the pooling then had to read again
+    if (m_Depthwise) m_Depthwise->Run();
+    g_PoolingPairsRunFused.fetch_add(1);
+    ForEachLane(batch, [&](const Lane& l) {
+        mi355x::Check(mi355x_conv2d_run_pooled(m_Plan, &pool, batch / l.count, l.Of(static_cast<const void*>(x), in),
+                                               l.Of(static_cast<void*>(y), pooledInfo), l.stream), "mi355x_conv2d_run_pooled");
+    });
+    return true;
+}
+
+void Mi355xConvolution2dWorkload::ExecuteOwn() const
+{
     if (m_Depthwise)
     {
         // the pair: the depthwise layer in front of this convolution has left its execution to this workload
@@ -496,9 +543,22 @@ Mi355xPooling2dWorkload::Mi355xPooling2dWorkload(const Pooling2dQueueDescriptor&
     if (m_Data.m_Parameters.m_DataLayout != DataLayout::NHWC) throw InvalidArgumentException("Mi355xPooling2dWorkload: NHWC only");
 }
 
-void Mi355xPooling2dWorkload::Execute() const
+unsigned long long Mi355xPooling2dWorkload::PairsFormed() { return g_PoolingPairsFormed.load(); }
+unsigned long long Mi355xPooling2dWorkload::PairsRunFused() { return g_PoolingPairsRunFused.load(); }
+unsigned long long Mi355xPooling2dWorkload::PairsRunApart() { return g_PoolingPairsRunApart.load(); }
+
+bool Mi355xPooling2dWorkload::TakeOver(Mi355xConvolution2dWorkload* convolution)
 {
-    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xPooling2dWorkload_Execute");
+    if (!convolution || m_Convolution || !convolution->OnlyConsumerIsAGlobalPooling()) return false;
+    if (!convolution->GetOutputHandle() || convolution->GetOutputHandle() != m_Data.m_Inputs[0]) return false;
+    m_Convolution = convolution;
+    convolution->LeaveExecutionToThePooling();
+    g_PoolingPairsFormed.fetch_add(1);
+    return true;
+}
+
+mi355x_pool2d_desc Mi355xPooling2dWorkload::Describe() const
+{
     const TensorInfo& in = m_Info.m_InputTensorInfos[0];
     const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
     const Pooling2dDescriptor& p = m_Data.m_Parameters;
@@ -511,6 +571,17 @@ void Mi355xPooling2dWorkload::Execute() const
     d.padding_method = p.m_PaddingMethod == PaddingMethod::IgnoreValue ? 0 : 1;
     d.input = mi355x::ToQuant(in);
     d.output = mi355x::ToQuant(out);
+    return d;
+}
+
+void Mi355xPooling2dWorkload::Execute() const
+{
+    ARMNN_SCOPED_PROFILING_EVENT_MI355X_NAME_GUID("Mi355xPooling2dWorkload_Execute");
+    const TensorInfo& in = m_Info.m_InputTensorInfos[0];
+    const TensorInfo& out = m_Info.m_OutputTensorInfos[0];
+    const mi355x_pool2d_desc d = Describe();
+    // the convolution in front has left its execution to this workload: both as one launch, or the convolution first
+    if (m_Convolution && m_Convolution->ExecuteWithPooling(d, m_Data.m_Outputs[0], out)) return;
     const void* x = In(m_Data.m_Inputs[0]);
     void* y = Out(m_Data.m_Outputs[0]);
     ForEachLane(in.GetShape()[0], [&](const Lane& l) {

@@ -37,9 +37,12 @@ struct Mi355xLayerNote
 {
     ActivationDescriptor activation;
     bool onlyConsumerIsAPointwiseConvolution = false;
+    /// on an unpadded 1x1 stride-1 Convolution2d: its output goes to one Pooling2d over the whole image and nowhere else
+    bool onlyConsumerIsAGlobalPooling = false;
 
     /// a note as a layer's additional-info object; `activation` null: the identity (Mi355xFeedsOnlyAnAddition's descriptor)
-    static std::shared_ptr<void> Make(const ActivationDescriptor* activation, bool onlyConsumerIsAPointwiseConvolution);
+    static std::shared_ptr<void> Make(const ActivationDescriptor* activation, bool onlyConsumerIsAPointwiseConvolution,
+                                      bool onlyConsumerIsAGlobalPooling = false);
     /// the note behind a queue descriptor's additional-info pointer, or null if that is something else
     static const Mi355xLayerNote* From(const void* additionalInfo);
 };
@@ -84,15 +87,29 @@ public:
     static unsigned long long DepthwisePairsFormed();
     static unsigned long long DepthwisePairsRunFused();
     static unsigned long long DepthwisePairsRunApart();
+    /// the layer was marked: its output goes to one Pooling2d over the whole image and nowhere else
+    bool OnlyConsumerIsAGlobalPooling() const { return m_OnlyConsumerIsAGlobalPooling; }
+    /// From now on Execute() does nothing: the Pooling2d that consumes this convolution calls ExecuteWithPooling() in its
+    /// own Execute().
+    void LeaveExecutionToThePooling() { m_RunsInsideThePooling = true; }
+    /// This convolution and the pooling `pool` of its output as one launch per lane, writing `pooled` only -- where the device
+    /// library takes and recommends the pair (mi355x_conv2d_pool_fusable, mi355x_conv2d_pool_fusion_pays), the input is
+    /// 16-byte aligned and `pooled` shares no memory with it: returns true.  Otherwise executes this convolution as
+    /// Execute() would have and returns false: the pooling is left to the caller.
+    bool ExecuteWithPooling(const mi355x_pool2d_desc& pool, ITensorHandle* pooled, const TensorInfo& pooledInfo) const;
     /// convolution and Addition as one launch per lane: sum = activation(convolution(input) + other)
     void ExecuteWithAddition(const ITensorHandle* other, const TensorInfo& otherInfo, ITensorHandle* sum, const TensorInfo& sumInfo,
                              const Mi355xFusedActivation& activation) const;
 private:
     void BuildPlan() const;
     void Run(void* y) const;
+    void ExecuteOwn() const;
     WorkloadInfo m_Info;
     bool m_FeedsOnlyAnAddition = false;
     bool m_RunsInsideTheAddition = false;
+    bool m_OnlyConsumerIsAGlobalPooling = false;
+    bool m_RunsInsideThePooling = false;
+    mutable int m_FusePool = -1;          // -1 not decided yet, 0 convolution and pooling run as two launches, 1 as one
     class Mi355xDepthwiseConvolution2dWorkload* m_Depthwise = nullptr;
     mutable int m_FusePair = -1;          // -1 not decided yet, 0 the pair runs as two launches, 1 as one
     mutable mi355x_conv2d_t m_Plan = nullptr;
@@ -158,8 +175,20 @@ class Mi355xPooling2dWorkload : public Mi355xBaseWorkload<Pooling2dQueueDescript
 public:
     Mi355xPooling2dWorkload(const Pooling2dQueueDescriptor& descriptor, const WorkloadInfo& info);
     void Execute() const override;
+    /// `convolution` is the workload created directly before this one.  If it is marked as feeding one pooling over the whole
+    /// image only and writes the tensor this workload reads, it leaves its execution to this workload, whose Execute() then
+    /// runs both (Mi355xConvolution2dWorkload::ExecuteWithPooling).  Returns whether the pair was formed.  The convolution
+    /// must outlive every Execute() of this workload (both belong to one loaded network).
+    bool TakeOver(Mi355xConvolution2dWorkload* convolution);
+    bool RunsAConvolution() const { return m_Convolution != nullptr; }
+    /// pairs formed / executions as one launch / executions as two launches since the process started (tests, benchmarks)
+    static unsigned long long PairsFormed();
+    static unsigned long long PairsRunFused();
+    static unsigned long long PairsRunApart();
 private:
+    mi355x_pool2d_desc Describe() const;
     WorkloadInfo m_Info;
+    const Mi355xConvolution2dWorkload* m_Convolution = nullptr;
 };
 
 /// counterpart of RefMeanWorkload (RefMeanWorkload.cpp:26-42) for the mean over height and width of an NHWC tensor: the

@@ -1455,8 +1455,10 @@ TEST_CASE("profiling: every workload of a profiled network reports its device ti
             if (meas.m_Name == "Device time") { hasDevice = true; deviceUs += meas.m_Value; CHECK(meas.m_Value > 0.0); CHECK(meas.m_Value < 5000.0); }
         CHECK(hasDevice);
     }
-    CHECK(workloads == 6);                     // stem, 2 x (depthwise + pointwise: the depthwise workload leaves its execution to the
-                                               // convolution behind it, whose event covers both), pool, fc, softmax; the activations are fused
+    CHECK(workloads == 5);                     // stem, depthwise + pointwise (the depthwise workload leaves its execution to the
+                                               // convolution behind it, whose event covers both), pool (the second depthwise +
+                                               // pointwise pair leaves its execution to the pooling over the whole image behind
+                                               // it), fc, softmax; the activations are fused
     std::ostringstream json;
     profiler->Print(json);
     const std::string j = json.str();
@@ -1995,6 +1997,177 @@ TEST_CASE("runtime: a depthwise layer whose output is read by a second consumer 
     const Diff d1 = Compare(out2, a, DataType::QAsymmU8);
     CHECK(d1.maxAbs <= 1);
     CHECK(d1.mismatches * 100 <= d1.n);
+}
+
+// Input -> 1x1 convolution (ReLu6 fused by the backend's own rewrite) -> pooling over the whole image [-> second output]
+struct PointwiseThenGlobalPooling
+{
+    TensorInfo in, pooled;
+    QLayer pw;
+    Pooling2dDescriptor pd;
+    PointwiseThenGlobalPooling(unsigned int batch, unsigned int side, unsigned int ci, unsigned int co, DataType type, PoolingAlgorithm algo)
+    {
+        in = ActInfo({batch, side, side, ci}, type, 0.0235f, type == DataType::QAsymmU8 ? 128 : 0);
+        pw = MakeConv(QLayer::Conv, in, co, 1, 1, 0.04f, type == DataType::QAsymmU8 ? 0 : -128, true, true, 61);
+        pooled = ActInfo({batch, 1, 1, co}, type, 0.03f, type == DataType::QAsymmU8 ? 2 : -126);
+        pd.m_DataLayout = DataLayout::NHWC;
+        pd.m_PoolType = algo;
+        pd.m_PoolWidth = pd.m_PoolHeight = side;
+        pd.m_StrideX = pd.m_StrideY = 1;
+    }
+    INetworkPtr Build(bool convolutionAlsoAnOutput = false) const
+    {
+        INetworkPtr net = INetwork::Create();
+        IConnectableLayer* input = net->AddInputLayer(0, "input");
+        input->GetOutputSlot(0).SetTensorInfo(in);
+        IOutputSlot& a = AddToNetwork(*net, input->GetOutputSlot(0), pw, "pw");
+        IConnectableLayer* pool = net->AddPooling2dLayer(pd, "pool");
+        a.Connect(pool->GetInputSlot(0));
+        pool->GetOutputSlot(0).SetTensorInfo(pooled);
+        IConnectableLayer* out = net->AddOutputLayer(0, "output");
+        pool->GetOutputSlot(0).Connect(out->GetInputSlot(0));
+        if (convolutionAlsoAnOutput)
+        {
+            IConnectableLayer* out2 = net->AddOutputLayer(1, "output2");
+            a.Connect(out2->GetInputSlot(0));
+        }
+        return net;
+    }
+};
+
+TEST_CASE("runtime: a pooling over the whole image runs the 1x1 convolution in front of it in one launch and gives the bytes of the two layers run apart", "gpu")
+{
+    const unsigned int lanesBefore = mi355x::Lanes();
+    for (DataType type : {DataType::QAsymmU8, DataType::QAsymmS8})
+        for (PoolingAlgorithm algo : {PoolingAlgorithm::Average, PoolingAlgorithm::Max})
+            for (unsigned int lanes : {2u, 1u})
+            {
+                mi355x::SetLanes(lanes);
+                // 16 images of 7 x 7, 128 -> 1024 channels: four images x 64 channels per block, 64 blocks per launch in one lane
+                // and 32 in each of two (the library recommends one launch from 32 on)
+                PointwiseThenGlobalPooling pair(16, 7, 128, 1024, type, algo);
+                const std::vector<uint8_t> input = RandomActivations(pair.in, 95);
+                TensorInfo constIn = pair.in;
+                constIn.SetConstant(true);
+                std::vector<uint8_t> results[2];
+                unsigned long long formed[2], fused[2], apart[2];
+                for (int on = 0; on < 2; ++on)
+                {
+                    const unsigned long long f0 = Mi355xPooling2dWorkload::PairsFormed(), r0 = Mi355xPooling2dWorkload::PairsRunFused(),
+                                             a0 = Mi355xPooling2dWorkload::PairsRunApart();
+                    IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+                    INetworkPtr net = pair.Build();
+                    OptimizerOptionsOpaque options;
+                    options.AddModelOption(BackendOptions("Mi355x", {{"FuseConvolutionPooling", on == 1}}));
+                    IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, rt->GetDeviceSpec(), options);
+                    NetworkId id = -1;
+                    std::string err;
+                    REQUIRE(rt->LoadNetwork(id, std::move(opt), err) == Status::Success);
+                    results[on].assign(pair.pooled.GetNumBytes(), 0);
+                    for (int pass = 0; pass < 2; ++pass)
+                    {
+                        InputTensors ins{{0, ConstTensor(constIn, input.data())}};
+                        OutputTensors outs{{0, Tensor(pair.pooled, results[on].data())}};
+                        REQUIRE(rt->EnqueueWorkload(id, ins, outs) == Status::Success);
+                    }
+                    rt->UnloadNetwork(id);
+                    formed[on] = Mi355xPooling2dWorkload::PairsFormed() - f0;
+                    fused[on] = Mi355xPooling2dWorkload::PairsRunFused() - r0;
+                    apart[on] = Mi355xPooling2dWorkload::PairsRunApart() - a0;
+                }
+                CHECK(formed[0] == 0);
+                CHECK(formed[1] == 1);
+                CHECK(fused[1] == 2);                        // one pair, two inferences
+                CHECK(apart[1] == 0);
+                CHECK(results[0] == results[1]);
+                const std::vector<uint8_t> a = OracleRun(pair.pw, input);
+                const std::vector<uint8_t> b = OraclePool(pair.pw.out, a, pair.pd, pair.pooled);
+                const Diff diff = Compare(results[1], b, type);
+                std::printf("    %s, %s, lanes %u: convolution + pooling vs oracle: max |diff| %d, exact %.5f\n", type == DataType::QAsymmU8 ? "uint8" : "int8",
+                            algo == PoolingAlgorithm::Max ? "max" : "average", lanes, diff.maxAbs,
+                            1.0 - static_cast<double>(diff.mismatches) / static_cast<double>(diff.n));
+                CHECK(diff.maxAbs <= 1);
+                CHECK(diff.mismatches * 50 <= diff.n);
+            }
+    mi355x::SetLanes(lanesBefore);
+}
+
+TEST_CASE("runtime: a 1x1 convolution whose output is read by a second consumer, or pooled in small windows, stays a launch of its own", "gpu")
+{
+    {
+        PointwiseThenGlobalPooling pair(16, 7, 128, 1024, DataType::QAsymmU8, PoolingAlgorithm::Average);
+        const std::vector<uint8_t> input = RandomActivations(pair.in, 96);
+        TensorInfo constIn = pair.in;
+        constIn.SetConstant(true);
+        const unsigned long long f0 = Mi355xPooling2dWorkload::PairsFormed();
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        INetworkPtr net = pair.Build(true);
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, rt->GetDeviceSpec(), OptimizerOptionsOpaque());
+        NetworkId id = -1;
+        std::string err;
+        REQUIRE(rt->LoadNetwork(id, std::move(opt), err) == Status::Success);
+        std::vector<uint8_t> out(pair.pooled.GetNumBytes(), 0), out2(pair.pw.out.GetNumBytes(), 0);
+        InputTensors ins{{0, ConstTensor(constIn, input.data())}};
+        OutputTensors outs{{0, Tensor(pair.pooled, out.data())}, {1, Tensor(pair.pw.out, out2.data())}};
+        REQUIRE(rt->EnqueueWorkload(id, ins, outs) == Status::Success);
+        rt->UnloadNetwork(id);
+        CHECK(Mi355xPooling2dWorkload::PairsFormed() - f0 == 0);
+        // the convolution's tensor exists and the pooling read it
+        CHECK(out == OraclePool(pair.pw.out, out2, pair.pd, pair.pooled));
+        const Diff d1 = Compare(out2, OracleRun(pair.pw, input), DataType::QAsymmU8);
+        CHECK(d1.maxAbs <= 1);
+    }
+    {
+        // 3 x 3 windows at stride 2 over an 8 x 8 image: not the whole image
+        PointwiseThenGlobalPooling pair(4, 8, 128, 64, DataType::QAsymmS8, PoolingAlgorithm::Max);
+        pair.pd.m_PoolWidth = pair.pd.m_PoolHeight = 3;
+        pair.pd.m_StrideX = pair.pd.m_StrideY = 2;
+        pair.pooled = ActInfo({4, 3, 3, 64}, DataType::QAsymmS8, 0.04f, -128);
+        const std::vector<uint8_t> input = RandomActivations(pair.in, 97);
+        TensorInfo constIn = pair.in;
+        constIn.SetConstant(true);
+        const unsigned long long f0 = Mi355xPooling2dWorkload::PairsFormed();
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        INetworkPtr net = pair.Build();
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, rt->GetDeviceSpec(), OptimizerOptionsOpaque());
+        NetworkId id = -1;
+        std::string err;
+        REQUIRE(rt->LoadNetwork(id, std::move(opt), err) == Status::Success);
+        std::vector<uint8_t> out(pair.pooled.GetNumBytes(), 0);
+        InputTensors ins{{0, ConstTensor(constIn, input.data())}};
+        OutputTensors outs{{0, Tensor(pair.pooled, out.data())}};
+        REQUIRE(rt->EnqueueWorkload(id, ins, outs) == Status::Success);
+        rt->UnloadNetwork(id);
+        CHECK(Mi355xPooling2dWorkload::PairsFormed() - f0 == 0);
+        const Diff d = Compare(out, OraclePool(pair.pw.out, OracleRun(pair.pw, input), pair.pd, pair.pooled), DataType::QAsymmS8);
+        CHECK(d.maxAbs <= 1);
+    }
+    {
+        // two images: one block row of 16 blocks per launch, fewer than the library recommends as one launch -- the pair is
+        // formed and runs as two launches
+        PointwiseThenGlobalPooling pair(2, 7, 128, 1024, DataType::QAsymmU8, PoolingAlgorithm::Average);
+        const std::vector<uint8_t> input = RandomActivations(pair.in, 98);
+        TensorInfo constIn = pair.in;
+        constIn.SetConstant(true);
+        const unsigned long long f0 = Mi355xPooling2dWorkload::PairsFormed(), r0 = Mi355xPooling2dWorkload::PairsRunFused(),
+                                 a0 = Mi355xPooling2dWorkload::PairsRunApart();
+        IRuntimePtr rt = IRuntime::Create(IRuntime::CreationOptions());
+        INetworkPtr net = pair.Build();
+        IOptimizedNetworkPtr opt = Optimize(*net, {kMi355x}, rt->GetDeviceSpec(), OptimizerOptionsOpaque());
+        NetworkId id = -1;
+        std::string err;
+        REQUIRE(rt->LoadNetwork(id, std::move(opt), err) == Status::Success);
+        std::vector<uint8_t> out(pair.pooled.GetNumBytes(), 0);
+        InputTensors ins{{0, ConstTensor(constIn, input.data())}};
+        OutputTensors outs{{0, Tensor(pair.pooled, out.data())}};
+        REQUIRE(rt->EnqueueWorkload(id, ins, outs) == Status::Success);
+        rt->UnloadNetwork(id);
+        CHECK(Mi355xPooling2dWorkload::PairsFormed() - f0 == 1);
+        CHECK(Mi355xPooling2dWorkload::PairsRunFused() - r0 == 0);
+        CHECK(Mi355xPooling2dWorkload::PairsRunApart() - a0 == 1);
+        const Diff d = Compare(out, OraclePool(pair.pw.out, OracleRun(pair.pw, input), pair.pd, pair.pooled), DataType::QAsymmU8);
+        CHECK(d.maxAbs <= 1);
+    }
 }
 
 TEST_CASE("runtime: an Addition whose sum was placed over the convolution's input runs the pair as two launches, same bytes", "gpu")

@@ -8,6 +8,7 @@
 #include "dwpw_panel_kernel.h"
 #include "dwpw_stream_kernel.h"
 #include "pwdw_kernel.h"
+#include "pool_softmax_items.h"
 #include "igemm_ksplit_kernel.h"
 #include "pw_gemm_kernel.h"
 #include "igemm_lds_kernel.h"
@@ -1476,16 +1477,24 @@ struct PwDwShape
 };
 
 // 0 when the pair (1x1 convolution, 3x3 depthwise) can run as PwDwKernel; the shape the launch needs comes back in `sh`
-int PwDwCheck(const mi355x_conv2d_s* pw, const mi355x_conv2d_s* dw, PwDwShape* sh)
+// 0 when `pw` can be the first stage of PwDwKernel
+int PwStageCheck(const mi355x_conv2d_s* pw)
 {
     const mi355x_conv2d_desc& a = pw->d;
-    const mi355x_conv2d_desc& b = dw->d;
     const bool pointwise = pw->algo == MI355X_ALGO_MFMA && !a.depthwise && a.kernel_h == 1 && a.kernel_w == 1 && a.stride_x == 1 &&
                            a.stride_y == 1 && a.pad_top == 0 && a.pad_left == 0 && a.out_h == a.in_h && a.out_w == a.in_w;
     if (!pointwise) return SetError(MI355X_ERR_UNSUPPORTED, "first plan is not an unpadded 1x1 stride-1 convolution on the MFMA kernel");
     if (pw->zw_neg != 0) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel needs pointwise weights without a zero point");
     if ((a.in_c % 128) != 0 || pw->K_pad != static_cast<int>(a.in_c))     // rows are fetched 128 bytes at a time: none may end inside a tile
         return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel needs the pointwise layer's input channels in whole 128-byte k-tiles");
+    return 0;
+}
+
+int PwDwCheck(const mi355x_conv2d_s* pw, const mi355x_conv2d_s* dw, PwDwShape* sh)
+{
+    const mi355x_conv2d_desc& a = pw->d;
+    const mi355x_conv2d_desc& b = dw->d;
+    if (int rc = PwStageCheck(pw)) return rc;
     if (dw->algo != MI355X_ALGO_DEPTHWISE || dw->variant != 1 || !dw->dw_grp || dw->w_dot4b)
         return SetError(MI355X_ERR_UNSUPPORTED, "second plan is not a 3x3 depthwise layer on the v_dot4 kernel");
     if (b.stride_x != b.stride_y || (b.stride_x != 1 && b.stride_x != 2))
@@ -1524,21 +1533,73 @@ int LaunchPwDwT(const PwDwArgs& a, hipStream_t stream)
     return 0;
 }
 
-int LaunchPwDw(const mi355x_conv2d_s* pw, const mi355x_conv2d_s* dw, const PwDwShape& sh, uint32_t batch, const void* x, void* y, hipStream_t stream)
+// the 1x1 stage's arguments and the grid for G images per block
+int FillPwStage(const mi355x_conv2d_s* pw, int G, uint32_t batch, const void* x, PwDwArgs* out)
 {
-    PwDwArgs a;
+    PwDwArgs a{};
     a.x = static_cast<const uint8_t*>(x); a.w = pw->w_mfma; a.K_pad = pw->K_pad; a.pw_ct = ChanTab{pw->chan, pw->Co_pad}; a.pw_corr = pw->corr;
     a.pw_xor = pw->xor_mask; a.pw_rq = pw->rq;
     a.N = static_cast<int>(batch); a.H = pw->geom.Ho; a.W = pw->geom.Wo; a.Ci = pw->geom.Ci; a.C = pw->geom.Co;
-    a.G = sh.G; a.tiles_n = a.C / kPwDwBN;
-    const long long nb = (static_cast<long long>(batch) + sh.G - 1) / sh.G * a.tiles_n;
+    a.G = G; a.tiles_n = a.C / kPwDwBN;
+    const long long nb = (static_cast<long long>(batch) + G - 1) / G * a.tiles_n;
     if (nb > 0x7fffffffll - 8) return SetError(MI355X_ERR_UNSUPPORTED, "grid too large");
     a.total_blocks = static_cast<int>(nb); a.xcd_chunk = static_cast<int>((nb + 7) / 8);
+    *out = a;
+    return 0;
+}
+
+int LaunchPwDw(const mi355x_conv2d_s* pw, const mi355x_conv2d_s* dw, const PwDwShape& sh, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    PwDwArgs a;
+    if (int rc = FillPwStage(pw, sh.G, batch, x, &a)) return rc;
     a.dw_grp = dw->dw_grp; a.dw_ct = ChanTab{dw->chan, dw->Co_pad}; a.dw_rq = dw->rq; a.dw_xor = dw->xor_mask; a.dw_pad = dw->pad_word;
     a.Ho = dw->geom.Ho; a.Wo = dw->geom.Wo; a.pad_top = dw->geom.pad_top; a.pad_left = dw->geom.pad_left;
     a.HR = sh.HR; a.HC = sh.HC; a.pairs = sh.pairs;
     a.y = static_cast<uint8_t*>(y);
     return sh.S == 1 ? LaunchPwDwT<1>(a, stream) : LaunchPwDwT<2>(a, stream);
+}
+
+// 0 when the pair (1x1 convolution, pooling over the whole image) can run as PwDwKernel<.., POOL>; G: images per block
+int PwPoolCheck(const mi355x_conv2d_s* pw, const mi355x_pool2d_desc* pool, int* G)
+{
+    if (int rc = PwStageCheck(pw)) return rc;
+    const mi355x_conv2d_desc& a = pw->d;
+    if (pool->pool_type != 0 && pool->pool_type != 1) return SetError(MI355X_ERR_UNSUPPORTED, "Unsupported pooling algorithm %d", pool->pool_type);
+    if (pool->in_h != a.out_h || pool->in_w != a.out_w || pool->channels != a.out_c)
+        return SetError(MI355X_ERR_INVALID_ARGUMENT, "the layers' shapes do not chain");
+    const bool global = pool->out_h == 1 && pool->out_w == 1 && pool->pool_h == pool->in_h && pool->pool_w == pool->in_w && pool->pad_left == 0 &&
+                        pool->pad_right == 0 && pool->pad_top == 0 && pool->pad_bottom == 0;
+    if (!global) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel needs a pooling window that is the whole unpadded image");
+    if (a.output.dtype != pool->input.dtype || a.output.scale != pool->input.scale || a.output.offset != pool->input.offset)
+        return SetError(MI355X_ERR_INVALID_ARGUMENT, "the convolution's output quantization is not the pooling's input quantization");
+    if (!IsActivationDtype(pool->output.dtype)) return SetError(MI355X_ERR_UNSUPPORTED, "pooling output: data type %d is not QAsymmS8/QAsymmU8", pool->output.dtype);
+    if (!(pool->output.scale > 0.0f) || !std::isfinite(pool->output.scale))
+        return SetError(MI355X_ERR_INVALID_ARGUMENT, "pooling output: scale must be positive and finite");
+    if ((a.out_c % kPwDwBN) != 0) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel needs channels %% 64 == 0");
+    const int hw = static_cast<int>(a.out_h) * static_cast<int>(a.out_w);
+    if (hw > kGlobalPoolMaxTaps) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel holds whole images: %d pixels exceed %d", hw, kGlobalPoolMaxTaps);
+    if (G) *G = kPwDwMF * 32 / hw;
+    return 0;
+}
+
+int LaunchPwPool(const mi355x_conv2d_s* pw, const mi355x_pool2d_desc* pool, int G, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    PwDwArgs a;
+    if (int rc = FillPwStage(pw, G, batch, x, &a)) return rc;
+    a.pool_in = MakeQIn(pool->input);
+    a.pool_rq = MakeRequant(pool->output, MI355X_ACT_NONE, 0.0f, 0.0f);
+    a.pool_is_max = pool->pool_type == 0;
+    a.y = static_cast<uint8_t*>(y);
+    constexpr int smem = PwDwStageBytes<kPwDwMF, kPwDwStages>();
+    static_assert(kPwDwMF * 32 * kPwDwPitch <= smem, "the intermediate tile reuses the GEMM's stages");
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwDwKernel<kPwDwMF, kPwDwStages, 1, kPwDwWaves, true>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    MI355X_HIP(attr);
+    NoteKernel("PwDwKernel<%d, %d, 1, %d, pool>", kPwDwMF, kPwDwStages, kPwDwWaves);
+    hipLaunchKernelGGL((PwDwKernel<kPwDwMF, kPwDwStages, 1, kPwDwWaves, true>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(64 * kPwDwWaves),
+                       smem, stream, a);
+    MI355X_HIP(hipGetLastError());
+    return 0;
 }
 } // namespace
 
@@ -1741,6 +1802,35 @@ int mi355x_conv2d_run_fused(mi355x_conv2d_t dw, mi355x_conv2d_t pw, uint32_t bat
     if (wide >= 512 && DwPwSmemBytes<1, 4>(static_cast<int>(dw->d.out_c)) <= 160 * 1024)
         return LaunchDwPw<1, 4>(dw, pw, batch, input_dev, output_dev, ToHip(stream));
     return LaunchDwPw<1, 2>(dw, pw, batch, input_dev, output_dev, ToHip(stream));
+}
+
+int mi355x_conv2d_pool_fusable(mi355x_conv2d_t conv, const mi355x_pool2d_desc* pool)
+{
+    if (!conv || !pool) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan / pooling descriptor is null");
+    return PwPoolCheck(conv, pool, nullptr);
+}
+
+int mi355x_conv2d_pool_fusion_pays(mi355x_conv2d_t conv, const mi355x_pool2d_desc* pool, uint32_t batch)
+{
+    if (!conv || !pool || batch == 0 || GlobalOptions().pwpool_auto == 0) return 0;
+    int G = 0;
+    if (PwPoolCheck(conv, pool, &G) != 0) return 0;
+    // a block per (G images, 64 channels).  Measured on 7 x 7 x 1024 -> 1024 with 8 .. 128 images per launch (32 .. 512
+    // blocks): the one launch is 1.2 us (8 images) to 11 us (128 images) shorter than the two; not measured below that
+    const long long blocks = (static_cast<long long>(batch) + G - 1) / G * (conv->d.out_c / kPwDwBN);
+    return blocks >= 32 ? 1 : 0;
+}
+
+int mi355x_conv2d_run_pooled(mi355x_conv2d_t conv, const mi355x_pool2d_desc* pool, uint32_t batch, const void* input_dev, void* output_dev,
+                             mi355x_stream_t stream)
+{
+    if (!conv || !pool) return SetError(MI355X_ERR_INVALID_ARGUMENT, "plan / pooling descriptor is null");
+    int G = 0;
+    if (int rc = PwPoolCheck(conv, pool, &G)) return rc;
+    if (batch == 0) return 0;
+    if (!input_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "input / output pointer is null");
+    if ((reinterpret_cast<uintptr_t>(input_dev) & 15) != 0) return SetError(MI355X_ERR_INVALID_ARGUMENT, "fused kernel needs a 16-byte aligned input");
+    return LaunchPwPool(conv, pool, G, batch, input_dev, output_dev, ToHip(stream));
 }
 
 int mi355x_conv2d_destroy(mi355x_conv2d_t plan)

@@ -20,6 +20,8 @@
 
 #include <hip/hip_runtime.h>
 
+#include <climits>
+
 #include "common.h"
 #include "conv_kernels.h"
 #include "device_math.h"
@@ -52,7 +54,11 @@ struct PwDwArgs
     int Ho, Wo, pad_top, pad_left;
     int HR, HC;                 // halo tile: (Ho - 1) * S + 3 rows, 2 * S * pairs + 2 columns
     int pairs;                  // (Wo + 1) / 2 output pixel pairs per row
-    uint8_t*        y;          // [N][Ho][Wo][C]
+    uint8_t*        y;          // [N][Ho][Wo][C]; with global pooling as the second stage [N][C]
+    // global pooling as the second stage (POOL) in place of the depthwise layer
+    QIn             pool_in;    // the intermediate tensor's quantization as the pooling reads it
+    Requant         pool_rq;
+    int             pool_is_max;
 };
 
 constexpr int kPwDwBN = 64;
@@ -85,8 +91,11 @@ __device__ __forceinline__ void WaitVmcntAtMost(int n)
     else __builtin_amdgcn_s_waitcnt(VmcntImm(0));
 }
 
-// MF: 32-pixel fragments per block; ST: LDS stages of the GEMM; S: depthwise stride (1 or 2); NW: waves (4 or 8)
-template <int MF, int ST, int S, int NW>
+// MF: 32-pixel fragments per block; ST: LDS stages of the GEMM; S: depthwise stride (1 or 2); NW: waves (4 or 8).
+// POOL: the second stage is a pooling whose window is the whole image instead of the depthwise layer: T holds the
+// images' pixels back to back without a border, and thread (image, channel) walks its column in the order of
+// GlobalPoolItem, so the pooled bytes are those of the two layers run one after the other (Pooling2d.cpp:186-300).
+template <int MF, int ST, int S, int NW, bool POOL = false>
 __global__ __launch_bounds__(64 * NW) void PwDwKernel(PwDwArgs a)
 {
     constexpr int BK = 128, BN = kPwDwBN, BM = MF * 32, PITCH = kPwDwPitch;
@@ -192,12 +201,17 @@ __global__ __launch_bounds__(64 * NW) void PwDwKernel(PwDwArgs a)
 
     // ---- depthwise constants of this thread's 4 channels, requested before the GEMM's tiles ---------------------------
     const int c4 = tid & 15;
-    const v4i* gc = reinterpret_cast<const v4i*>(a.dw_grp + (tn * (BN / 4) + c4) * 32);
-    const v4i w0 = gc[0], w1 = gc[1], w2 = gc[2], corr4 = gc[3];
-    const float4 dmp = *reinterpret_cast<const float4*>(gc + 4);
-    const float4 dbp = *reinterpret_cast<const float4*>(gc + 5);
-    const float4 dmm = *reinterpret_cast<const float4*>(gc + 6);
-    const float4 dbm = *reinterpret_cast<const float4*>(gc + 7);
+    v4i w0 = {}, w1 = {}, w2 = {}, corr4 = {};
+    float4 dmp = {}, dbp = {}, dmm = {}, dbm = {};
+    if constexpr (!POOL)
+    {
+        const v4i* gc = reinterpret_cast<const v4i*>(a.dw_grp + (tn * (BN / 4) + c4) * 32);
+        w0 = gc[0]; w1 = gc[1]; w2 = gc[2]; corr4 = gc[3];
+        dmp = *reinterpret_cast<const float4*>(gc + 4);
+        dbp = *reinterpret_cast<const float4*>(gc + 5);
+        dmm = *reinterpret_cast<const float4*>(gc + 6);
+        dbm = *reinterpret_cast<const float4*>(gc + 7);
+    }
 
     const int nk = a.K_pad / BK;
 #pragma unroll
@@ -224,12 +238,13 @@ __global__ __launch_bounds__(64 * NW) void PwDwKernel(PwDwArgs a)
 
     // ---- phase B: T <- padding value, then the requantized 1x1 outputs ---------------------------------------------------
     uint8_t* T = smem;
-    const int cells = a.G * a.HR * a.HC;
+    if constexpr (!POOL)
     {
+        const int cells = a.G * a.HR * a.HC;
         const v4i padv = {static_cast<int>(a.dw_pad), static_cast<int>(a.dw_pad), static_cast<int>(a.dw_pad), static_cast<int>(a.dw_pad)};
         for (int i = tid; i < cells * (PITCH / 16); i += 64 * NW) *reinterpret_cast<v4i*>(T + i * 16) = padv;
+        __syncthreads();
     }
-    __syncthreads();
 #pragma unroll
     for (int tp = 0; tp < TP; ++tp)
     {
@@ -237,11 +252,16 @@ __global__ __launch_bounds__(64 * NW) void PwDwKernel(PwDwArgs a)
         const int ml = f * 32 + frag_row;
         if (f < MF && ml < rows)
         {
-            const int g = ml / HW, p = ml - g * HW;
-            const int iy = p / a.W, ix = p - iy * a.W;
-            const int hy = iy + a.pad_top, hx = ix + a.pad_left;
-            const bool inside = hy < a.HR && hx < a.HC;
-            uint8_t* cell = T + ((g * a.HR + hy) * a.HC + hx) * PITCH + tc * 32 + lane_c;
+            bool inside = true;
+            uint8_t* cell = T + ml * PITCH + tc * 32 + lane_c;         // POOL: pixel rows as they come
+            if constexpr (!POOL)
+            {
+                const int g = ml / HW, p = ml - g * HW;
+                const int iy = p / a.W, ix = p - iy * a.W;
+                const int hy = iy + a.pad_top, hx = ix + a.pad_left;
+                inside = hy < a.HR && hx < a.HC;
+                cell = T + ((g * a.HR + hy) * a.HC + hx) * PITCH + tc * 32 + lane_c;
+            }
 #pragma unroll
             for (int q = 0; q < 4; ++q)
             {
@@ -249,11 +269,45 @@ __global__ __launch_bounds__(64 * NW) void PwDwKernel(PwDwArgs a)
                 const Fast4 f4 = LoadFast4(a.pw_ct, cg);
                 const v16i& v = acc[tp];
                 const uint32_t out = Requant4Dev(v[4 * q + 0], v[4 * q + 1], v[4 * q + 2], v[4 * q + 3], f4, a.pw_ct, cg, a.pw_rq);
-                if (inside) *reinterpret_cast<uint32_t*>(cell + 8 * q) = out ^ a.dw_xor;
+                if (inside) *reinterpret_cast<uint32_t*>(cell + 8 * q) = POOL ? out : out ^ a.dw_xor;
             }
         }
     }
     __syncthreads();
+
+    // ---- phase C, pooling: thread (image, channel) walks its column of T ------------------------------------------------
+    if constexpr (POOL)
+    {
+        for (int it = tid; it < images * BN; it += 64 * NW)
+        {
+            const int g = it / BN, c = it - g * BN;
+            const uint8_t* col = T + g * HW * PITCH + c;
+            float res;
+            if (a.pool_is_max)
+            {
+                int best = INT_MIN;
+                for (int t = 0; t < HW; ++t)
+                {
+                    const int code = a.pool_in.is_u8 ? static_cast<int>(col[t * PITCH]) : static_cast<int>(static_cast<int8_t>(col[t * PITCH]));
+                    best = max(best, code);
+                }
+                res = __fmul_rn(static_cast<float>(best - a.pool_in.offset), a.pool_in.scale);
+            }
+            else
+            {
+                float sum = 0.0f;
+#pragma unroll 7
+                for (int t = 0; t < HW; ++t)
+                {
+                    const int code = a.pool_in.is_u8 ? static_cast<int>(col[t * PITCH]) : static_cast<int>(static_cast<int8_t>(col[t * PITCH]));
+                    sum = __fadd_rn(sum, __fmul_rn(static_cast<float>(code - a.pool_in.offset), a.pool_in.scale));
+                }
+                res = __fdiv_rn(sum, static_cast<float>(HW));
+            }
+            a.y[static_cast<long long>(n0 + g) * a.C + tn * BN + c] = static_cast<uint8_t>(QuantizeFastDev(res, a.pool_rq));
+        }
+        return;
+    }
 
     // ---- phase C: depthwise 3x3 over T ---------------------------------------------------------------------------------
     constexpr int NPX = S == 1 ? 4 : 6;

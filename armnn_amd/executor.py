@@ -16,7 +16,8 @@ from .tensor import QTensor, numpy_dtype
 @dataclass
 class FusedPair:
     """Two neighbouring layers -- depthwise + the pointwise convolution consuming it, pointwise + the depthwise consuming
-    it, or a convolution + the Addition consuming it (op "convadd") -- launched as one kernel."""
+    it, a convolution + the Addition consuming it (op "convadd"), or a 1x1 convolution + the pooling over its whole output
+    image (op "convpool") -- launched as one kernel."""
     name: str
     parts: Tuple                       # (first Layer, second Layer)
     op: str = "dwpw"
@@ -78,8 +79,11 @@ class FusedTail:
 class DeviceNetwork:
     def __init__(self, net: Network, batch: int, algo_overrides: Optional[Dict[str, int]] = None, use_graph: bool = True,
                  fuse: bool = False, lanes: int = 1, fuse_add: bool = True, chain: bool = False, lanes_after_chain: bool = False,
-                 join_for_fused: bool = False, fuse_tail: bool = False):
-        """fuse_tail: global pooling -> FullyConnected -> Softmax at the end of the network as one launch (same bytes; measured
+                 join_for_fused: bool = False, fuse_tail: bool = False, fuse_pool: Optional[bool] = None):
+        """fuse_pool: a 1x1 convolution and the pooling over its whole output image as one launch (Conv2dPlan.run_pooled; same
+        bytes, the convolution's output tensor is not written): True wherever the library takes the pair, None (default) where
+        it also recommends it and fuse == "auto", False never.
+        fuse_tail: global pooling -> FullyConnected -> Softmax at the end of the network as one launch (same bytes; measured
         slower than the three launches on MI355X, so off by default).
         chain: runs of consecutive layers the library accepts (mi355x_chain_accepts) become one persistent launch over
         the whole batch; with lanes > 1 the lanes join in front of such a run and, if lanes_after_chain, fork again behind it
@@ -180,6 +184,38 @@ class DeviceNetwork:
             self._build_chains()
         if fuse_tail:
             self._fuse_tail()
+        if fuse_pool or (fuse_pool is None and fuse == "auto"):
+            self._fuse_conv_pool(only_where_it_pays=not fuse_pool)
+
+    def _fuse_conv_pool(self, only_where_it_pays):
+        """A 1x1 convolution whose output only feeds the pooling launched right behind it, where the library runs the two
+        as one kernel (mi355x_conv2d_pool_fusable): the step writes the pooled tensor only."""
+        net = self.net
+        consumers: Dict[str, int] = {}
+        for l in net.layers:
+            for i in l.inputs:
+                consumers[i] = consumers.get(i, 0) + 1
+        fused, k = [], 0
+        while k < len(self.steps):
+            l, fn = self.steps[k]
+            nxt = self.steps[k + 1][0] if k + 1 < len(self.steps) else None
+            plan = self._plan_of.get(id(l)) if getattr(l, "op", None) == "conv" else None
+            d = self._pool_descs.get(id(nxt)) if getattr(nxt, "op", None) == "pool" else None
+            rows = self.batch // self.lanes
+            if (isinstance(plan, shim.Conv2dPlan) and d is not None and nxt.inputs[0] == l.output and nxt.act[0] == 0 and
+                    consumers.get(l.output, 0) == 1 and l.output != net.output and plan.pool_fusable(d) and
+                    (not only_where_it_pays or plan.pool_fusion_pays(d, rows))):
+                x, y = self.buffers[l.inputs[0]].ptr, self.buffers[nxt.output].ptr
+                nx, ny = net.info(l.inputs[0], self.batch).num_elements, net.info(nxt.output, self.batch).num_elements
+                batch = self.batch
+                fused.append((FusedPair(f"{l.name}+{nxt.name}", (l, nxt), op="convpool"),
+                              (lambda plan, d, x, y, nx, ny: lambda s, lane=0, lanes=1: plan.run_pooled(
+                                  d, batch // lanes, x + lane * (nx // lanes), y + lane * (ny // lanes), s))(plan, d, x, y, nx, ny)))
+                k += 2
+            else:
+                fused.append((l, fn))
+                k += 1
+        self.steps = fused
 
     def _fuse_tail(self):
         """Pooling over the whole image -> FullyConnected -> Softmax, launched one behind the other, become one launch where

@@ -28,7 +28,8 @@ EXPORTS = [
     "mi355x_event_destroy", "mi355x_event_record", "mi355x_stream_wait_event", "mi355x_event_synchronize", "mi355x_event_elapsed_ms",
     "mi355x_graph_capture_begin", "mi355x_graph_capture_end", "mi355x_graph_launch", "mi355x_graph_destroy",
     "mi355x_conv2d_create", "mi355x_conv2d_run", "mi355x_conv2d_destroy", "mi355x_conv2d_algo",
-    "mi355x_conv2d_fusable", "mi355x_conv2d_fusion_pays", "mi355x_conv2d_run_fused", "mi355x_conv2d_run_add", "mi355x_conv2d_set_concurrency",
+    "mi355x_conv2d_fusable", "mi355x_conv2d_fusion_pays", "mi355x_conv2d_run_fused", "mi355x_conv2d_pool_fusable",
+    "mi355x_conv2d_pool_fusion_pays", "mi355x_conv2d_run_pooled", "mi355x_conv2d_run_add", "mi355x_conv2d_set_concurrency",
     "mi355x_chain_accepts", "mi355x_chain_create", "mi355x_chain_run", "mi355x_chain_status", "mi355x_chain_info", "mi355x_chain_run_stamped", "mi355x_chain_run_noalloc", "mi355x_chain_destroy",
     "mi355x_fc_create", "mi355x_fc_run", "mi355x_fc_destroy", "mi355x_fc_algo",
     "mi355x_activation_run", "mi355x_pool2d_run", "mi355x_add_run", "mi355x_softmax_run", "mi355x_pad_run",
@@ -127,6 +128,8 @@ def load_library(path: str = LIB_PATH) -> C.CDLL:
             "mi355x_fc_algo": [V, C.POINTER(C.c_int32), C.c_char_p, C.c_size_t],
             "mi355x_activation_run": [C.c_size_t, C.POINTER(Quant), C.POINTER(Quant), C.c_int32, C.c_float, C.c_float, V, V, V],
             "mi355x_pool2d_run": [C.POINTER(Pool2dDesc), C.c_uint32, V, V, V],
+            "mi355x_conv2d_pool_fusable": [V, C.POINTER(Pool2dDesc)], "mi355x_conv2d_pool_fusion_pays": [V, C.POINTER(Pool2dDesc), C.c_uint32],
+            "mi355x_conv2d_run_pooled": [V, C.POINTER(Pool2dDesc), C.c_uint32, V, V, V],
             "mi355x_add_run": [C.c_size_t, C.POINTER(Quant), C.POINTER(Quant), C.POINTER(Quant), C.c_int32, C.c_float,
                                C.c_float, V, V, V, V],
             "mi355x_softmax_run": [C.c_uint32, C.c_uint32, C.c_float, C.POINTER(Quant), C.POINTER(Quant), V, V, V],
@@ -322,6 +325,19 @@ class Conv2dPlan:
     def run_fused(self, second: "Conv2dPlan", batch: int, x_dev: int, y_dev: int, stream=None):
         """Both layers without the intermediate tensor; bytes equal run() + second.run()."""
         _chk(self.lib.mi355x_conv2d_run_fused(self.plan, second.plan, batch, x_dev, y_dev, stream))
+
+    def pool_fusable(self, pool: "Pool2dDesc") -> bool:
+        """True when this plan (an unpadded 1x1 convolution) and the pooling over its whole output image can run as one kernel."""
+        return self.lib.mi355x_conv2d_pool_fusable(self.plan, C.byref(pool)) == 0
+
+    def pool_fusion_pays(self, pool: "Pool2dDesc", batch: int) -> bool:
+        """True when the library recommends that one launch at this batch."""
+        return self.lib.mi355x_conv2d_pool_fusion_pays(self.plan, C.byref(pool), batch) == 1
+
+    def run_pooled(self, pool: "Pool2dDesc", batch: int, x_dev: int, y_dev: int, stream=None):
+        """The convolution and the pooling behind it; only the pooled tensor [batch][channels] is written, with the bytes
+        of run() followed by mi355x_pool2d_run."""
+        _chk(self.lib.mi355x_conv2d_run_pooled(self.plan, C.byref(pool), batch, x_dev, y_dev, stream))
 
     def set_concurrency(self, lanes: int):
         """Tell the plan that `lanes` launches of its network run side by side (kernels with small blocks are preferred then)."""

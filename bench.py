@@ -70,7 +70,7 @@ def layer_work(net, l, batch):
     """(kind, algorithmic work per launch): conv/fc -> ops = 2*MACs; others -> bytes, each tensor once."""
     if l.op in ("conv", "fc"):
         return "mfma", 2.0 * l.macs_per_image * batch
-    if l.op == "convadd":                      # a convolution with the Addition behind it in its write-out
+    if l.op in ("convadd", "convpool"):        # a convolution with the Addition / the global pooling behind it in its write-out
         return "mfma", 2.0 * l.parts[0].macs_per_image * batch
     if l.op in ("chain", "tail"):
         # a run of layers in one persistent launch: every layer's tensors are still written and read, so the launch's
@@ -396,7 +396,7 @@ def main():
         w = sum(r["work"] for r in sel)
         return {"ms": t * 1e3, "achieved": w / t, "frac": w / t / peak} if t > 0 else None
 
-    g_conv = group(("conv", "fc", "convadd"), INT8_MFMA_PEAK_OPS)
+    g_conv = group(("conv", "fc", "convadd", "convpool"), INT8_MFMA_PEAK_OPS)
     g_dw = group(("depthwise",), HBM_PEAK_BYTES)
     groups = {
         "conv_fc": {"ms": g_conv["ms"], "TOPS": g_conv["achieved"] / 1e12, "frac_of_int8_mfma_peak": g_conv["frac"]},
@@ -420,6 +420,7 @@ def main():
               "batch": batch, "graph_replay": not args.no_graph, "fused_pairs": [l.name for l, _ in dn.steps if l.op == "dwpw"] or None, "additions_inside_convolutions": not args.no_fuse_add, "lanes": args.lanes,
               "layer_chains": [l.name for l, _ in dn.steps if l.op == "chain"] or None,
               "tail_in_one_launch": any(l.op == "tail" for l, _ in dn.steps),
+              "convolution_and_global_pooling_in_one_launch": [l.name for l, _ in dn.steps if l.op == "convpool"] or None,
               "total_TOPS": 2.0 * net.macs_per_image() * batch / (ms_per_step * 1e-3) / 1e12}
     if backend is not None:
         # the same network and input through the C++ backend: wall clock per IRuntime::EnqueueWorkload call, host buffers in

@@ -125,6 +125,8 @@ int  mi355x_abi_version(void);
  *   pointwise weights in on-chip memory (identical bytes; lets tests compare it with the older fused kernel).
  *   "pwdw_auto" = 1 | 0: mi355x_conv2d_fusion_pays may (1) or may not (0) recommend a 1x1 convolution + the depthwise layer
  *   behind it (tests and tuning).
+ *   "pwpool_auto" = 1 | 0: mi355x_conv2d_pool_fusion_pays may (1) or may not (0) recommend a 1x1 convolution + the global
+ *   pooling behind it (tests and tuning).
  *   "dwpw_panel" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a depthwise layer of 256 or 512
  *   channels and a pointwise layer of 256 or 512 output channels on the kernel that gives a block an 8 x 8 pixel tile over
  *   all channels (identical bytes; lets tests compare it with the older fused kernel).
@@ -377,6 +379,22 @@ typedef struct {
 } mi355x_pool2d_desc;
 int mi355x_pool2d_run(const mi355x_pool2d_desc* desc, uint32_t batch, const void* input_dev, void* output_dev,
                       mi355x_stream_t stream);
+/* An unpadded 1x1 stride-1 Convolution2d and the Pooling2d over its whole output image (Max or Average, no padding,
+ * one output pixel) as one launch: a block computes whole images of the convolution's output for 64 of its channels,
+ * keeps them on chip and pools them there in the order of Pooling2d.cpp:186-300, so output_dev [batch][channels] holds
+ * the bytes of mi355x_conv2d_run followed by mi355x_pool2d_run -- two workloads in sequence in the reference
+ * (RefConvolution2dWorkload.cpp:38-58, then RefPooling2dWorkload.cpp:18-36) -- and the convolution's output tensor is
+ * never written: the caller must have no other reader of it.  mi355x_conv2d_pool_fusable returns 0 when the pair
+ * qualifies: a matrix-core plan whose input channels are a multiple of 128 and whose weights have no zero point, output
+ * channels % 64 == 0, an image of at most 196 pixels, the pooling's input quantization equal to the convolution's
+ * output quantization; else MI355X_ERR_UNSUPPORTED / MI355X_ERR_INVALID_ARGUMENT with the reason in mi355x_last_error().
+ * mi355x_conv2d_pool_fusion_pays: 1 when the library recommends the one launch at this batch (at least 32 blocks of
+ * whole images x 64 channels; option "pwpool_auto" = 0 turns the recommendation off), else 0; never an error.
+ * input_dev 16-byte aligned. */
+int mi355x_conv2d_pool_fusable(mi355x_conv2d_t conv, const mi355x_pool2d_desc* pool);
+int mi355x_conv2d_pool_fusion_pays(mi355x_conv2d_t conv, const mi355x_pool2d_desc* pool, uint32_t batch);
+int mi355x_conv2d_run_pooled(mi355x_conv2d_t conv, const mi355x_pool2d_desc* pool, uint32_t batch, const void* input_dev,
+                             void* output_dev, mi355x_stream_t stream);
 
 /* ElementwiseBinary Add of two equally-shaped tensors (dequantize, add, requantize) with an optional fused
  * ReLu / BoundedReLu: RefElementwiseBinaryWorkload (workloads/RefElementwiseBinaryWorkload.cpp:27-107). */

@@ -1,6 +1,8 @@
 """Depthwise 3x3 + pointwise 1x1 as one kernel, and pointwise 1x1 + the depthwise 3x3 after it as one kernel: bytes must
 equal the two layers run one after the other, and the pair must stay within 1 LSB of the oracle per layer (the second
 layer judged on the first layer's actual output)."""
+import ctypes as C
+
 import numpy as np
 import pytest
 
@@ -256,6 +258,99 @@ def test_pointwise_then_depthwise_pairs_outside_the_kernels_shape_are_refused():
         xd = shim.DeviceBuffer(pw.x.data.nbytes).upload(pw.x.data)
         yd = shim.DeviceBuffer(other.out_info.num_elements)
         _plan(pw).run_fused(_plan(other), 1, xd.ptr, yd.ptr)
+
+
+# ---- a 1x1 convolution and the pooling over its whole output image as one launch ----------------------------------------
+# (name, n, h, w, ci, c, dtype, act after the convolution, pool type (0 max, 1 average), pooled scale, pooled offset)
+PW_POOL = [
+    ("7x7_k1024_c1024_s8_avg_as_mobilenet_ends", 6, 7, 7, 1024, 1024, S8, cases.RELU6, 1, 0.0235, -128),
+    ("7x7_k512_c128_u8_avg_last_block_has_one_image", 5, 7, 7, 512, 128, U8, cases.RELU6, 1, 0.03, 2),
+    ("7x7_k128_c64_s8_max", 4, 7, 7, 128, 64, S8, (0, 0.0, 0.0), 0, 0.04, -121),
+    ("14x14_k256_c128_u8_avg_one_image_per_block", 3, 14, 14, 256, 128, U8, cases.RELU, 1, 0.02, 0),
+    ("4x5_k128_c192_s8_avg_eleven_images_per_block", 13, 4, 5, 128, 192, S8, cases.RELU6, 1, 0.05, -100),
+    ("1x1_k128_c64_u8_max", 9, 1, 1, 128, 64, U8, cases.RELU6, 0, 0.04, 7),
+    ("10x10_k384_c64_s8_avg_wider_output_scale", 3, 10, 10, 384, 64, S8, (0, 0.0, 0.0), 1, 0.01, 5),
+]
+
+
+def _make_pw_pool(name, n, h, w, ci, c, dt, act_pw, pool_type, pooled_scale, pooled_offset):
+    zp_in = 3 if dt == U8 else -128
+    zp_mid = 7 if dt == U8 else -121
+    pw = cases.make_conv_case(name + "_pw", 900 + ci, n=n, h=h, w=w, ci=ci, co=c, kh=1, kw=1, in_dtype=dt, in_scale=0.0235,
+                              in_offset=zp_in, out_scale=0.04, out_offset=zp_mid, act=act_pw)
+    pooled = TensorInfo((n, 1, 1, c), dt, pooled_scale, pooled_offset)
+    d = shim.Pool2dDesc(h, w, c, 1, 1, w, h, 1, 1, 0, 0, 0, 0, pool_type, 1, shim._quant(pw.out_info), shim._quant(pooled))
+    return pw, pooled, d
+
+
+@pytest.mark.parametrize("cfg", PW_POOL, ids=[c[0] for c in PW_POOL])
+def test_pointwise_then_global_pooling_fused_equals_two_layers(port, cfg):
+    print("pair", cfg, flush=True)
+    shim.Device()
+    lib = shim.load_library()
+    pw, pooled, d = _make_pw_pool(*cfg)
+    ppw = _plan(pw)
+    assert ppw.pool_fusable(d), lib.mi355x_last_error().decode()
+    n, h, w, _ = pw.x.info.shape
+    xd = shim.DeviceBuffer(pw.x.data.nbytes).upload(pw.x.data)
+    mid = shim.DeviceBuffer(pw.out_info.num_elements)
+    y2 = shim.DeviceBuffer(pooled.num_elements)
+    yf = shim.DeviceBuffer(pooled.num_elements + 64)
+    shim._chk(lib.mi355x_fill_u8(yf.ptr, 0x5A, pooled.num_elements + 64, None))
+    ppw.run(n, xd.ptr, mid.ptr)
+    shim._chk(lib.mi355x_pool2d_run(C.byref(d), n, mid.ptr, y2.ptr, None))
+    ppw.run_pooled(d, n, xd.ptr, yf.ptr)
+    assert shim.last_kernel().startswith("PwDwKernel") and "pool" in shim.last_kernel()
+    two = y2.download(pooled.shape, numpy_dtype(pooled.dtype))
+    got = yf.download((pooled.num_elements + 64,), np.uint8)
+    fused = got[:pooled.num_elements].view(numpy_dtype(pooled.dtype)).reshape(pooled.shape)
+    np.testing.assert_array_equal(fused, two)
+    assert (got[pooled.num_elements:] == 0x5A).all()         # nothing written behind the pooled tensor
+    assert len(np.unique(fused)) > 4
+    # against the oracle's pooling of the device's own intermediate tensor
+    mid_h = mid.download(pw.out_info.shape, numpy_dtype(pw.out_info.dtype))
+    want = port.pooling2d(QTensor(pw.out_info, mid_h), pooled, pool_type=d.pool_type, pool_w=w, pool_h=h, stride_x=1, stride_y=1)
+    mx, exact = lsb_diff(fused, want.data)
+    print(f"  fused vs oracle on the device's intermediate: max|d|={mx} exact={exact:.5f}", flush=True)
+    assert mx <= 1 and exact >= 0.99
+
+
+def test_pointwise_then_pooling_pairs_outside_the_kernels_shape_are_refused():
+    shim.Device()
+    lib = shim.load_library()
+    pw, pooled, d = _make_pw_pool("ok", 2, 7, 7, 128, 64, S8, cases.RELU6, 1, 0.04, -121)
+    plan = _plan(pw)
+    assert plan.pool_fusable(d)
+    assert not plan.pool_fusion_pays(d, 2)                   # one block: two launches are no slower
+    xd = shim.DeviceBuffer(pw.x.data.nbytes).upload(pw.x.data)
+    yd = shim.DeviceBuffer(pooled.num_elements)
+
+    def changed(**kw):
+        e = shim.Pool2dDesc.from_buffer_copy(d)
+        for k, v in kw.items():
+            setattr(e, k, v)
+        return e
+    for e, why in ((changed(pool_w=3, pool_h=3, out_h=5, out_w=5), "whole"),        # a window smaller than the image
+                   (changed(pad_left=1), "whole"),
+                   (changed(channels=128), "chain"),
+                   (changed(pool_type=2), "pooling algorithm"),
+                   (changed(input=shim.Quant(int(S8), 0.05, -121)), "quantization")):
+        assert not plan.pool_fusable(e)
+        assert why in lib.mi355x_last_error().decode(), lib.mi355x_last_error().decode()
+        with pytest.raises(shim.ShimError):
+            plan.run_pooled(e, 2, xd.ptr, yd.ptr)
+    # 15 x 15 = 225 pixels exceed what a block holds; 96 channels are not whole 64-channel blocks; 64 input channels are no
+    # whole k-tile; a 3x3 convolution is not pointwise
+    for args in (("big", 1, 15, 15, 128, 64), ("c96", 1, 7, 7, 128, 96), ("k64", 1, 7, 7, 64, 64)):
+        pw2, _, d2 = _make_pw_pool(*args, S8, cases.RELU6, 1, 0.04, -121)
+        assert not _plan(pw2).pool_fusable(d2), args
+    c3 = cases.make_conv_case("c3", 7, n=1, h=7, w=7, ci=128, co=64, in_scale=0.0235, in_offset=-128, out_scale=0.04, out_offset=-121)
+    assert not _plan(c3).pool_fusable(d)
+    # a misaligned input pointer
+    with pytest.raises(shim.ShimError):
+        plan.run_pooled(d, 1, xd.ptr + 4, yd.ptr)
+    # an empty batch is no work and no error
+    plan.run_pooled(d, 0, xd.ptr, yd.ptr)
 
 
 # ---- a convolution and the Addition that consumes it (residual connection) as one launch ------------------------------------
