@@ -1526,7 +1526,7 @@ int LaunchPwDwT(const PwDwArgs& a, hipStream_t stream)
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwDwKernel<kPwDwMF, kPwDwStages, S, kPwDwWaves>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);
-    NoteKernel("PwDwKernel<%d, %d, %d, %d>", kPwDwMF, kPwDwStages, S, kPwDwWaves);
+    NoteKernel("PwDwKernel<%d, %d, %d, %d, false>", kPwDwMF, kPwDwStages, S, kPwDwWaves);
     hipLaunchKernelGGL((PwDwKernel<kPwDwMF, kPwDwStages, S, kPwDwWaves>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(64 * kPwDwWaves), smem,
                        stream, a);
     MI355X_HIP(hipGetLastError());
@@ -1595,7 +1595,7 @@ int LaunchPwPool(const mi355x_conv2d_s* pw, const mi355x_pool2d_desc* pool, int 
     static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwDwKernel<kPwDwMF, kPwDwStages, 1, kPwDwWaves, true>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);
-    NoteKernel("PwDwKernel<%d, %d, 1, %d, pool>", kPwDwMF, kPwDwStages, kPwDwWaves);
+    NoteKernel("PwDwKernel<%d, %d, 1, %d, true>", kPwDwMF, kPwDwStages, kPwDwWaves);
     hipLaunchKernelGGL((PwDwKernel<kPwDwMF, kPwDwStages, 1, kPwDwWaves, true>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(64 * kPwDwWaves),
                        smem, stream, a);
     MI355X_HIP(hipGetLastError());
