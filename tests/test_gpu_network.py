@@ -154,6 +154,28 @@ def test_mobilenet_v1_batch64_as_the_benchmark_runs_it_rows_equal_batch2_runs():
     small.close()
 
 
+@pytest.mark.parametrize("batch,lanes,forced", [(64, 2, None), (8, 1, None), (6, 2, True), (1, 1, True), (2, 1, None)])
+def test_mobilenet_v1_last_convolution_with_the_pooling_behind_it_gives_the_bytes_of_the_layers_run_apart(batch, lanes, forced):
+    """fuse_pool None: where the library recommends it (from 32 blocks of four 7 x 7 images x 64 channels per launch on);
+    True: wherever it takes the pair.  Both the pooled tensor and the network's output must be those of the unfused run."""
+    net = nets.mobilenet_v1()
+    x = nets.synthetic_input(net, batch, seed=5)
+    apart = DeviceNetwork(net, batch, use_graph=False, lanes=1)
+    want = apart.run(x).data.copy()
+    want_pooled = apart.download("avgpool:out").data.copy()
+    apart.close()
+    dn = DeviceNetwork(net, batch, use_graph=True, lanes=lanes, fuse="auto", fuse_pool=forced)
+    names = [l.name for l, _ in dn.steps]
+    if forced or batch // lanes >= 8:
+        assert "pw13+avgpool" in names and "avgpool" not in names, names
+    else:
+        assert "pw13+avgpool" not in names and "avgpool" in names, names
+    for replay in range(2):
+        np.testing.assert_array_equal(dn.run(x).data, want, err_msg=f"replay {replay}")
+    np.testing.assert_array_equal(dn.download("avgpool:out").data, want_pooled)
+    dn.close()
+
+
 def test_mobilenet_v1_batch64_in_one_lane_rows_equal_batch2_runs():
     # 64 images per launch: the largest launches of the benchmark (persistent blocks walk the most tiles here)
     _rows_equal_small_batch_runs(nets.mobilenet_v1(), 64, (0, 20, 42, 62), lanes=1)
