@@ -1830,6 +1830,13 @@ int mi355x_conv2d_run_pooled(mi355x_conv2d_t conv, const mi355x_pool2d_desc* poo
     if (batch == 0) return 0;
     if (!input_dev || !output_dev) return SetError(MI355X_ERR_INVALID_ARGUMENT, "input / output pointer is null");
     if ((reinterpret_cast<uintptr_t>(input_dev) & 15) != 0) return SetError(MI355X_ERR_INVALID_ARGUMENT, "fused kernel needs a 16-byte aligned input");
+    {
+        // one launch reads the input while it writes the pooled tensor
+        const uintptr_t x0 = reinterpret_cast<uintptr_t>(input_dev), y0 = reinterpret_cast<uintptr_t>(output_dev);
+        const uintptr_t n_in = static_cast<uintptr_t>(batch) * conv->d.in_h * conv->d.in_w * conv->d.in_c;
+        const uintptr_t n_out = static_cast<uintptr_t>(batch) * conv->d.out_c;
+        if (y0 < x0 + n_in && x0 < y0 + n_out) return SetError(MI355X_ERR_INVALID_ARGUMENT, "the convolution's input may not overlap the pooled output");
+    }
     return LaunchPwPool(conv, pool, G, batch, input_dev, output_dev, ToHip(stream));
 }
 

@@ -279,6 +279,46 @@ __global__ __launch_bounds__(256) void GlobalPoolKernel(PoolArgs p, QIn qin, Req
     GlobalPoolItem<false>(p, qin, rq, x, y, static_cast<int>(blockIdx.x), raw);
 }
 
+// The same pooling for images of at most MAXT pixels: a thread owns one channel of one image and asks for all of its taps
+// before it uses the first, so the launch waits for memory once; the taps are then summed in GlobalPoolItem's order with
+// GlobalPoolItem's arithmetic (same bytes).  Any channel count, no alignment rule.
+template <int MAXT>
+__global__ __launch_bounds__(64) void GlobalPoolSmallKernel(PoolArgs p, QIn qin, Requant rq, const uint8_t* __restrict__ x,
+                                                            uint8_t* __restrict__ y, long long total)
+{
+    const long long i = static_cast<long long>(blockIdx.x) * 64 + threadIdx.x;
+    if (i >= total) return;
+    const int taps = p.H * p.W;
+    const long long n = i / p.C;
+    const int c = static_cast<int>(i - n * p.C);
+    const uint8_t* src = x + n * taps * p.C + c;
+    uint8_t v[MAXT];
+#pragma unroll
+    for (int t = 0; t < MAXT; ++t) v[t] = t < taps ? src[static_cast<long long>(t) * p.C] : 0;
+    float res;
+    if (p.is_max)
+    {
+        int best = INT_MIN;
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t)
+            if (t < taps) best = max(best, qin.is_u8 ? static_cast<int>(v[t]) : static_cast<int>(static_cast<int8_t>(v[t])));
+        res = __fmul_rn(static_cast<float>(best - qin.offset), qin.scale);
+    }
+    else
+    {
+        float sum = 0.0f;
+#pragma unroll
+        for (int t = 0; t < MAXT; ++t)
+            if (t < taps)
+            {
+                const int code = qin.is_u8 ? static_cast<int>(v[t]) : static_cast<int>(static_cast<int8_t>(v[t]));
+                sum = __fadd_rn(sum, __fmul_rn(static_cast<float>(code - qin.offset), qin.scale));
+            }
+        res = __fdiv_rn(sum, static_cast<float>(taps));
+    }
+    y[i] = static_cast<uint8_t>(QuantizeFastDev(res, rq));
+}
+
 // 16 elements per thread, 16-byte loads and stores
 template <bool CLAMP>
 __global__ __launch_bounds__(256) void AddVec16Kernel(AddFuse f, const v4u* __restrict__ x0,
@@ -465,7 +505,14 @@ int mi355x_pool2d_run(const mi355x_pool2d_desc* d, uint32_t batch, const void* i
     const bool vec4 = (p.C % 4) == 0 && (reinterpret_cast<uintptr_t>(input_dev) & 3) == 0 && (reinterpret_cast<uintptr_t>(output_dev) & 3) == 0;
     const bool global = p.Ho == 1 && p.Wo == 1 && p.pad_top == 0 && p.pad_left == 0 && p.pool_h == p.H && p.pool_w == p.W &&
                         p.H * p.W <= kGlobalPoolMaxTaps;
-    if (vec4 && global)
+    if (global && p.H * p.W <= 64 && GlobalOptions().pool_small != 0)
+    {
+        NoteKernel("GlobalPoolSmallKernel<64>");
+        const long long n = static_cast<long long>(batch) * p.C;
+        hipLaunchKernelGGL(GlobalPoolSmallKernel<64>, dim3(static_cast<unsigned>((n + 63) / 64)), dim3(64), 0, ToHip(stream), p, MakeQIn(d->input), rq,
+                           static_cast<const uint8_t*>(input_dev), static_cast<uint8_t*>(output_dev), n);
+    }
+    else if (vec4 && global)
     {
         NoteKernel("GlobalPoolKernel");
         hipLaunchKernelGGL(GlobalPoolKernel, dim3(static_cast<unsigned>(batch * ((p.C + 255) / 256))), dim3(256), 0, ToHip(stream), p,

@@ -125,6 +125,9 @@ int  mi355x_abi_version(void);
  *   pointwise weights in on-chip memory (identical bytes; lets tests compare it with the older fused kernel).
  *   "pwdw_auto" = 1 | 0: mi355x_conv2d_fusion_pays may (1) or may not (0) recommend a 1x1 convolution + the depthwise layer
  *   behind it (tests and tuning).
+ *   "pool_small" = 1 | 0: a pooling over a whole image of at most 64 pixels runs on the kernel that gives a thread one
+ *   channel and requests all its taps at once (1), or on the kernel that stages the image in on-chip memory (0).  Identical
+ *   bytes.
  *   "pwpool_auto" = 1 | 0: mi355x_conv2d_pool_fusion_pays may (1) or may not (0) recommend a 1x1 convolution + the global
  *   pooling behind it (tests and tuning).
  *   "dwpw_panel" = 1 | 0: mi355x_conv2d_run_fused may (1) or may not (0) run a depthwise layer of 256 or 512
@@ -390,7 +393,8 @@ int mi355x_pool2d_run(const mi355x_pool2d_desc* desc, uint32_t batch, const void
  * output quantization; else MI355X_ERR_UNSUPPORTED / MI355X_ERR_INVALID_ARGUMENT with the reason in mi355x_last_error().
  * mi355x_conv2d_pool_fusion_pays: 1 when the library recommends the one launch at this batch (at least 32 blocks of
  * whole images x 64 channels; option "pwpool_auto" = 0 turns the recommendation off), else 0; never an error.
- * input_dev 16-byte aligned. */
+ * input_dev 16-byte aligned; output_dev may share no byte with input_dev (one launch reads the one while it writes the
+ * other: MI355X_ERR_INVALID_ARGUMENT). */
 int mi355x_conv2d_pool_fusable(mi355x_conv2d_t conv, const mi355x_pool2d_desc* pool);
 int mi355x_conv2d_pool_fusion_pays(mi355x_conv2d_t conv, const mi355x_pool2d_desc* pool, uint32_t batch);
 int mi355x_conv2d_run_pooled(mi355x_conv2d_t conv, const mi355x_pool2d_desc* pool, uint32_t batch, const void* input_dev,

@@ -349,6 +349,11 @@ def test_pointwise_then_pooling_pairs_outside_the_kernels_shape_are_refused():
     # a misaligned input pointer
     with pytest.raises(shim.ShimError):
         plan.run_pooled(d, 1, xd.ptr + 4, yd.ptr)
+    # the pooled tensor inside the input's range: one launch would read what it writes
+    with pytest.raises(shim.ShimError):
+        plan.run_pooled(d, 2, xd.ptr, xd.ptr + 2 * 7 * 7 * 128 - 64)
+    assert "overlap" in lib.mi355x_last_error().decode()
+    plan.run_pooled(d, 2, xd.ptr, yd.ptr)
     # an empty batch is no work and no error
     plan.run_pooled(d, 0, xd.ptr, yd.ptr)
 

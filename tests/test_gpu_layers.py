@@ -28,6 +28,10 @@ POOLS = [
     ("avg7x7_global_c1024", (3, 7, 7, 1024), cpuref.POOL_AVERAGE, 7, 7, 1, 1, (0, 0, 0, 0)),
     ("max14x14_global_c300", (2, 14, 14, 300), cpuref.POOL_MAX, 14, 14, 1, 1, (0, 0, 0, 0)),
     ("avg3x5_global_c8", (5, 5, 3, 8), cpuref.POOL_AVERAGE, 3, 5, 2, 2, (0, 0, 0, 0)),
+    ("max7x7_global_c1001_odd_channels", (4, 7, 7, 1001), cpuref.POOL_MAX, 7, 7, 1, 1, (0, 0, 0, 0)),
+    ("avg8x8_global_c2048_64_taps", (16, 8, 8, 2048), cpuref.POOL_AVERAGE, 8, 8, 1, 1, (0, 0, 0, 0)),
+    ("avg1x1_global_c7", (3, 1, 1, 7), cpuref.POOL_AVERAGE, 1, 1, 1, 1, (0, 0, 0, 0)),
+    ("avg13x5_global_c40_65_taps", (2, 5, 13, 40), cpuref.POOL_AVERAGE, 13, 5, 1, 1, (0, 0, 0, 0)),
     ("avg3x2_pad_c12", (1, 9, 10, 12), cpuref.POOL_AVERAGE, 3, 2, 2, 1, (1, 1, 1, 0)),
     ("avg2x2_c8", (2, 8, 8, 8), cpuref.POOL_AVERAGE, 2, 2, 2, 2, (0, 0, 0, 0)),
     ("max9x9_big_window_c8", (1, 12, 12, 8), cpuref.POOL_MAX, 9, 9, 3, 3, (4, 4, 4, 4)),
@@ -52,6 +56,16 @@ def test_pooling(port, cfg, method, dtype):
     want = port.pooling2d(x, oi, **kw)
     got = shim.pooling2d(x, oi, **kw)
     np.testing.assert_array_equal(got.data, want.data)
+    if ph == h and pw == w and (pl, pr, pt, pb) == (0, 0, 0, 0) and h * w <= 64:
+        # a whole small image: the kernel that requests a channel's taps at once ran; the LDS-staged kernel gives the same
+        assert shim.last_kernel().startswith("GlobalPoolSmallKernel")
+        shim.set_option("pool_small", 0)
+        try:
+            staged = shim.pooling2d(x, oi, **kw)
+            assert not shim.last_kernel().startswith("GlobalPoolSmallKernel")
+        finally:
+            shim.set_option("pool_small", 1)
+        np.testing.assert_array_equal(staged.data, want.data)
 
 
 @pytest.mark.parametrize("dtype", [S8, U8])
