@@ -1,5 +1,6 @@
 """Runs a nets.Network on the device through the C ABI: one plan per layer, all activations resident in HBM,
-the whole forward pass optionally captured into a HIP graph and replayed with one launch."""
+the whole forward pass launched kernel by kernel or captured into a HIP graph and replayed with one launch
+(DeviceNetwork.choose_submission measures which is faster for the network and batch at hand)."""
 from __future__ import annotations
 
 import ctypes as C
@@ -475,6 +476,28 @@ class DeviceNetwork:
             self.dev.graph_launch(self.graph, self.stream)
         else:
             self._enqueue_lanes()
+
+    def choose_submission(self, passes: int = 40, rounds: int = 2):
+        """Times `passes` forward passes launched kernel by kernel and the same number of replays of the captured graph,
+        alternated `rounds` times, and keeps the faster way for enqueue() (self.use_graph).  A replay costs the host one call,
+        so it wins where the host cannot launch as fast as the device computes (a few images per pass); at tens of images
+        per pass the device is the limit, and there kernels launched one by one on the stream finish a few percent sooner
+        than the same kernels as nodes of a graph.  Returns {"eager_ms", "graph_ms"}: the best pass time of either way."""
+        import time
+        best = {False: float("inf"), True: float("inf")}
+        for _ in range(rounds):
+            for mode in (False, True):
+                self.use_graph = mode
+                self.enqueue()                         # first use captures the graph
+                self.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(passes):
+                    self.enqueue()
+                self.synchronize()
+                best[mode] = min(best[mode], (time.perf_counter() - t0) * 1e3 / passes)
+        self.use_graph = best[True] < best[False]
+        self.submission = {"eager_ms": best[False], "graph_ms": best[True]}
+        return self.submission
 
     def synchronize(self):
         self.dev.stream_sync(self.stream)

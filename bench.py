@@ -233,7 +233,10 @@ def main():
                          "(the quantization of older uint8 models) instead of the headline workload's per-channel QSymmS8")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-backend", action="store_true", help="skip the run through the C++ backend (config.backend_path)")
-    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--no-graph", action="store_true", help="launch every pass kernel by kernel (same as --submission eager)")
+    ap.add_argument("--submission", default="auto", choices=("auto", "graph", "eager"),
+                    help="how a forward pass reaches the device: one replay of the captured HIP graph, kernel by kernel on the stream, or "
+                         "(auto) whichever of the two is faster in a trial of 2 x 40 passes each before the warm-up steps")
     ap.add_argument("--fuse", default="auto", choices=("auto", "none", "dwpw", "pwdw"),
                     help="pairs of layers as one kernel (same bytes): 'auto' the depthwise + pointwise pairs the library recommends at "
                          "the batch a launch sees (mi355x_conv2d_fusion_pays), 'none' every layer a launch of its own, 'dwpw' every "
@@ -285,7 +288,9 @@ def main():
     for opt in args.option:
         name, _, value = opt.partition("=")
         shim.set_option(name, int(value))
-    dn = DeviceNetwork(net, batch, use_graph=not args.no_graph, fuse="" if args.fuse == "none" else args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add, chain=args.chain, fuse_tail=args.fuse_tail)
+    if args.no_graph:
+        args.submission = "eager"
+    dn = DeviceNetwork(net, batch, use_graph=args.submission != "eager", fuse="" if args.fuse == "none" else args.fuse, lanes=args.lanes, fuse_add=not args.no_fuse_add, chain=args.chain, fuse_tail=args.fuse_tail)
     dn.upload_input(nets.synthetic_input(net, batch))
     dev = dn.dev
 
@@ -308,6 +313,9 @@ def main():
                           "batch": batch, "launch_batch": batch // args.lanes, "net": net.name}))
         dn.close()
         return 0
+
+    # ---- set-up: which way of submitting a pass is faster here (like a plan's choice of kernel, made once, before the warm-up)
+    submission = dn.choose_submission() if args.submission == "auto" else None
 
     for _ in range(args.warmup):
         dn.enqueue()
@@ -416,8 +424,8 @@ def main():
 
     config = {"workload": f"{net.name} int8 (QAsymm activations, {'per-channel QSymmS8' if args.weights == 'per_channel_s8' or args.net != 'mobilenet_v1' else 'per-tensor QAsymmU8'} weights), batch {batch}, "
                           f"random-init, whole forward pass incl. avgpool/FC/softmax, input resident in HBM, every layer through the C ABI, "
-                          f"one HIP graph replay per step",
-              "batch": batch, "graph_replay": not args.no_graph, "fused_pairs": [l.name for l, _ in dn.steps if l.op == "dwpw"] or None, "additions_inside_convolutions": not args.no_fuse_add, "lanes": args.lanes,
+                          + ("one HIP graph replay per step" if dn.use_graph else "the kernels of a step launched one by one on the stream"),
+              "batch": batch, "graph_replay": bool(dn.use_graph), "submission_trial": submission, "fused_pairs": [l.name for l, _ in dn.steps if l.op == "dwpw"] or None, "additions_inside_convolutions": not args.no_fuse_add, "lanes": args.lanes,
               "layer_chains": [l.name for l, _ in dn.steps if l.op == "chain"] or None,
               "tail_in_one_launch": any(l.op == "tail" for l, _ in dn.steps),
               "convolution_and_global_pooling_in_one_launch": [l.name for l, _ in dn.steps if l.op == "convpool"] or None,

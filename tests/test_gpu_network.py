@@ -176,6 +176,21 @@ def test_mobilenet_v1_last_convolution_with_the_pooling_behind_it_gives_the_byte
     dn.close()
 
 
+@pytest.mark.parametrize("which,batch,lanes", [("mobilenet", 8, 1), ("resnet", 4, 2)])
+def test_the_measured_choice_between_launching_and_replaying_changes_no_byte(which, batch, lanes):
+    net = nets.mobilenet_v1(resolution=96, classes=50) if which == "mobilenet" else nets.resnet50(resolution=64)
+    x = nets.synthetic_input(net, batch, seed=9)
+    dn = DeviceNetwork(net, batch, use_graph=False, lanes=lanes, fuse="auto")
+    want = dn.run(x).data.copy()
+    trial = dn.choose_submission(passes=10, rounds=2)
+    assert set(trial) == {"eager_ms", "graph_ms"} and all(0.0 < v < 50.0 for v in trial.values()), trial
+    assert dn.use_graph == (trial["graph_ms"] < trial["eager_ms"])
+    np.testing.assert_array_equal(dn.run(x).data, want)
+    dn.use_graph = not dn.use_graph                      # the other way gives the same bytes
+    np.testing.assert_array_equal(dn.run(x).data, want)
+    dn.close()
+
+
 def test_mobilenet_v1_batch64_in_one_lane_rows_equal_batch2_runs():
     # 64 images per launch: the largest launches of the benchmark (persistent blocks walk the most tiles here)
     _rows_equal_small_batch_runs(nets.mobilenet_v1(), 64, (0, 20, 42, 62), lanes=1)
