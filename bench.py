@@ -2,10 +2,13 @@
 """Benchmark: int8 images/sec of the MobileNetV1-1.0-224-style network at batch 64 on one MI355X.
 
 A step is one forward pass of the whole network over one batch that is already resident in HBM (every layer
-runs on the device through the C ABI; the pass is replayed as one HIP graph).  Prints ONE JSON line.
+runs on the device through the C ABI; the pass reaches the device as one replay of a captured HIP graph or kernel by
+kernel on the stream, whichever a trial before the warm-up steps finds faster: --submission, config.submission_trial).
+Prints ONE JSON line.
 
   python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 64] [--net mobilenet_v1|resnet50]
                   [--weights per_channel_s8|per_tensor_u8] [--no-cpu-baseline] [--no-backend] [--layers] [--chain]
+                  [--submission auto|graph|eager]
 
 The headline workload is the default: per-channel QSymmS8 weights.  --weights per_tensor_u8 runs the same network with
 QAsymmU8 weights that have one scale and a zero point per layer, and says so in config.workload.
