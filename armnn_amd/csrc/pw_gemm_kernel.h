@@ -121,6 +121,23 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
 
     auto epilogue = [&](int t) {
         const int lane_c = 4 * (lane >> 5);
+        constexpr int CH = BN / 16;                 // 16-byte chunks per row
+        constexpr int NJ = 32 * CH / 64;
+        // The Addition's other input: all of a tile's pieces are requested here, ahead of the requantization whose
+        // arithmetic they then travel behind, from clamped addresses (so none sits in a divergent branch and waits there).
+        const bool fuse = (a.N & 15) == 0 && a.res != nullptr;
+        v4i other[NJ] = {};
+        if (fuse)
+        {
+#pragma unroll
+            for (int i = 0; i < NJ; ++i)
+            {
+                const int j = lane + 64 * i;
+                const int row = min(t * 32 + j / CH, a.M - 1);
+                const int c0 = min(n0 + (j % CH) * 16, a.N - 16);
+                other[i] = *reinterpret_cast<const v4i*>(a.res + static_cast<long long>(row) * a.N + c0);
+            }
+        }
         int rt = 0;
         if constexpr (AW) rt = (rowsum + __shfl_xor(rowsum, 32)) * a.zw_neg;
 #pragma unroll
@@ -144,21 +161,8 @@ __global__ __launch_bounds__(256) void PwGemmKernel(PwArgs a)
         __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
         __builtin_amdgcn_wave_barrier();
         __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
-        constexpr int CH = BN / 16;                 // 16-byte chunks per row
-        if ((a.N & 15) == 0 && a.res)
+        if (fuse)
         {
-            // the Addition's other input: all of a tile's loads are issued before the first is used (clamped addresses, so
-            // none sits in a divergent branch and waits there)
-            constexpr int NJ = 32 * CH / 64;
-            v4i other[NJ];
-#pragma unroll
-            for (int i = 0; i < NJ; ++i)
-            {
-                const int j = lane + 64 * i;
-                const int row = min(t * 32 + j / CH, a.M - 1);
-                const int c0 = min(n0 + (j % CH) * 16, a.N - 16);
-                other[i] = *reinterpret_cast<const v4i*>(a.res + static_cast<long long>(row) * a.N + c0);
-            }
 #pragma unroll
             for (int i = 0; i < NJ; ++i)
             {
