@@ -32,6 +32,7 @@ struct mi355x_conv2d_s
     int32_t* corr     = nullptr;   // [Co_pad]  -zx' * sum_k w[c][k]
     int K = 0, K_pad = 0, Co_pad = 0;
     int pw_blocks_per_cu = 1, pw_n_cu = 256;     // weight-stationary kernel: blocks a CU holds at once, CUs of the device
+    int pw_blocks_per_cu_64 = 0;                 // ... with 64-channel slabs, where the plan's own slab is 128 (0: not prepared)
     std::vector<float> chan_host;  // host copy, completed with the corr-folded rows once corr is known
     std::vector<float> fast_fm, fast_fb;   // per channel: the unwidened fast-path constants and the constant half-width of the
     std::vector<double> fast_cw;           // bracket (negative: no fast path), kept until the table is uploaded

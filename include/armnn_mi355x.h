@@ -109,8 +109,8 @@ int  mi355x_abi_version(void);
  *   "dw_rows" = 0 | 1 | 2: output rows per thread of the 3x3 depthwise kernel (0: chosen from the feature-map height;
  *   identical bytes).
  *   "pw_slab" = 0 | 32 | 64 | 128: output channels per weight slab of the weight-stationary kernel for 1x1 convolutions
- *   with at most 128 input channels (0: the widest that fits the layer; a value wider than that is ignored; identical
- *   bytes; tests and tuning).
+ *   with at most 128 input channels (0: 128 with 128 input channels and more than 64 outputs, else 64 or 32 by the layer's
+ *   width; a value wider than the layer is ignored; identical bytes; tests and tuning).
  *   "dw_cb" = 0 | 32: channels per block of the 3x3 depthwise kernels (0: as many as the channel count and the kernel
  *   allow: 64 on the matrix cores, 128 on the VALU kernel; 32: always 32; identical bytes).
  *   "dw_mfma" = 1 | 0 | 7 | 8 | 14 | 16: 3x3 depthwise layers (multiplier 1, channels a multiple of 16) compute on the

@@ -419,11 +419,14 @@ def test_pointwise_slab_widths_give_the_same_bytes():
 def test_plans_told_that_they_share_the_device_pick_small_blocks_and_give_the_same_bytes():
     """mi355x_conv2d_set_concurrency(plan, 2): the 3x3 convolution over 64 channels leaves the kernel that keeps its input
     tile in LDS for the implicit GEMM with 128x64 tiles, and the 3x3 convolution over 256 channels at 14x14 leaves the
-    K split over two wave groups for plain 64x64 blocks; the four-group split of the smallest launches stays.  Same
-    bytes as alone, and as the direct kernel."""
+    K split over two wave groups for plain 64x64 blocks; the four-group split of the smallest launches stays; a 1x1
+    convolution over 128 channels takes 64-channel weight slabs instead of 128-channel ones (over 64 channels it has them
+    anyway).  Same bytes as alone, and as the direct kernel."""
     picks = [(cases.make_conv_case("shared_3x3_c64_56", 841, n=16, h=56, w=56, ci=64, co=64, act=cases.RELU), "HaloConvKernel<64", "IgemmKernel<128, 64"),
              (cases.make_conv_case("shared_3x3_c256_14", 842, n=16, h=14, w=14, ci=256, co=256, act=cases.RELU), "IgemmKSplitKernel<2", "IgemmLdsKernel<64, 64"),
              (cases.make_conv_case("shared_3x3_c512_7", 843, n=16, h=7, w=7, ci=512, co=512, act=cases.RELU), "IgemmKSplitKernel<4", "IgemmKSplitKernel<4"),
+             (cases.make_conv_case("shared_1x1_k128_co512", 845, n=3, h=28, w=28, ci=128, co=512, kh=1, kw=1, act=cases.RELU), "PwGemmKernel<128, 4", "PwGemmKernel<64, 4"),
+             (cases.make_conv_case("shared_1x1_k64_co256", 846, n=2, h=56, w=56, ci=64, co=256, kh=1, kw=1), "PwGemmKernel<64, 2", "PwGemmKernel<64, 2"),
              (cases.make_conv_case("shared_3x3_c64_small", 844, n=1, h=20, w=20, ci=64, co=64, act=cases.RELU6), None, None)]
     for c, alone_kernel, shared_kernel in picks:
         want = _gpu_conv(c, shim.ALGO_DIRECT)
@@ -440,7 +443,7 @@ def test_plans_told_that_they_share_the_device_pick_small_blocks_and_give_the_sa
         np.testing.assert_array_equal(alone.data, want.data, err_msg=c.name)
         np.testing.assert_array_equal(shared.data, want.data, err_msg=c.name)
     with pytest.raises(shim.ShimError):
-        shim.Conv2dPlan(picks[3][0].x.info, picks[3][0].w, picks[3][0].b, picks[3][0].out_info, **picks[3][0].params).set_concurrency(0)
+        shim.Conv2dPlan(picks[-1][0].x.info, picks[-1][0].w, picks[-1][0].b, picks[-1][0].out_info, **picks[-1][0].params).set_concurrency(0)
 
 
 def test_depthwise_64_and_128_channel_blocks_give_the_same_bytes():
