@@ -85,6 +85,7 @@ struct Options
     int igemm_xcd_cols = 0;            // direct-to-LDS implicit GEMM: 0 split the XCDs over the output channels where the weights are heavy, 1 never, 2 wherever possible
     int dwpw_stream = 1;               // 0: fused depthwise + pointwise launches never take the persistent kernel for 32 / 64 / 128 channels between the layers
     int pwdw_auto = 1;                 // 1: mi355x_conv2d_fusion_pays may recommend a 1x1 convolution + the depthwise layer behind it (7 x 7 maps)
+    int pwdw_mf = 0;                   // 32-pixel fragments per block of the whole-image kernels (1x1 convolution + depthwise / + pooling): 0 automatic, 2, 4 or 7 forced
     int pool_small = 1;                // 0: pooling over a whole image of at most 64 pixels runs on the LDS-staged kernel (tests compare the two)
     int pwpool_auto = 1;               // 1: mi355x_conv2d_pool_fusion_pays may recommend a 1x1 convolution + the global pooling behind it
     int dwpw_panel = 1;                // 0: fused depthwise + pointwise launches never take the one-block-per-tile-over-all-channels kernel

@@ -1486,8 +1486,26 @@ constexpr int kPwDwStages = 2, kPwDwWaves = 8;
 
 struct PwDwShape
 {
-    int G = 0, HR = 0, HC = 0, pairs = 0, S = 0;
+    int G = 0, HR = 0, HC = 0, pairs = 0, S = 0, MF = 0;
 };
+
+constexpr int PwDwWavesFor(int mf) { return mf == 2 ? 4 : kPwDwWaves; }
+constexpr int PwDwSmemFor(int mf) { return kPwDwStages * (mf * 32 + 64) * 128; }
+
+// 32-pixel fragments per block for images of `hw` pixels: 7, 4 or 2 (two: four waves).  A block's phases run one after
+// the other, so blocks that start together stream, requantize and write together; two smaller blocks per CU overlap
+// each other's phases at the price of streaming the 64 channels' weights twice.  Measured on MobileNetV1's 7 x 7 layers
+// at 64 images (step, alternated three times): with the pooling as second stage 0.2607 ms at 7 fragments, 0.2589 at 4;
+// with the depthwise layer as second stage 4 fragments cost 0.5 us; 2 fragments lose 3 us for both.  At 128 images, where
+// the large blocks already come two to a CU, the small ones lose 6 us; at 8 images they gain 3.  `blocks7`: blocks of the
+// launch at 7 fragments.
+int PwDwFragmentsFor(int hw, bool pooling, long long blocks7)
+{
+    const int forced = GlobalOptions().pwdw_mf;
+    if ((forced == 2 || forced == 4) && hw <= forced * 32) return forced;
+    if (forced == 0 && pooling && 2 * hw <= 4 * 32 && blocks7 <= 256) return 4;
+    return kPwDwMF;
+}
 
 // 0 when the pair (1x1 convolution, 3x3 depthwise) can run as PwDwKernel; the shape the launch needs comes back in `sh`
 // 0 when `pw` can be the first stage of PwDwKernel
@@ -1520,28 +1538,28 @@ int PwDwCheck(const mi355x_conv2d_s* pw, const mi355x_conv2d_s* dw, PwDwShape* s
     if (hw > kPwDwMF * 32) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel holds whole images: %d pixels exceed %d", hw, kPwDwMF * 32);
     PwDwShape s;
     s.S = static_cast<int>(b.stride_x);
-    s.G = kPwDwMF * 32 / hw;
+    s.MF = PwDwFragmentsFor(hw, false, 0);
+    s.G = s.MF * 32 / hw;
     s.pairs = (static_cast<int>(b.out_w) + 1) / 2;
     s.HR = (static_cast<int>(b.out_h) - 1) * s.S + 3;
     s.HC = 2 * s.S * s.pairs + 2;
     // the padded intermediate tile reuses the GEMM's stages: tiny images take fewer per block than the rows would allow
-    s.G = std::min(s.G, PwDwStageBytes<kPwDwMF, kPwDwStages>() / (s.HR * s.HC * kPwDwPitch));
+    s.G = std::min(s.G, PwDwSmemFor(s.MF) / (s.HR * s.HC * kPwDwPitch));
     if (s.G < 1) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel: the intermediate tile does not fit LDS");
     if (sh) *sh = s;
     return 0;
 }
 
-template <int S>
+template <int MF, int S>
 int LaunchPwDwT(const PwDwArgs& a, hipStream_t stream)
 {
-    constexpr int smem = PwDwStageBytes<kPwDwMF, kPwDwStages>();
-    static_assert(smem <= 160 * 1024, "LDS of one CU");
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwDwKernel<kPwDwMF, kPwDwStages, S, kPwDwWaves>),
+    constexpr int smem = PwDwStageBytes<MF, kPwDwStages>(), NW = PwDwWavesFor(MF);
+    static_assert(smem <= 160 * 1024 && smem == PwDwSmemFor(MF), "LDS of one CU");
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwDwKernel<MF, kPwDwStages, S, NW>),
                                                        hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     MI355X_HIP(attr);
-    NoteKernel("PwDwKernel<%d, %d, %d, %d, false>", kPwDwMF, kPwDwStages, S, kPwDwWaves);
-    hipLaunchKernelGGL((PwDwKernel<kPwDwMF, kPwDwStages, S, kPwDwWaves>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(64 * kPwDwWaves), smem,
-                       stream, a);
+    NoteKernel("PwDwKernel<%d, %d, %d, %d, false>", MF, kPwDwStages, S, NW);
+    hipLaunchKernelGGL((PwDwKernel<MF, kPwDwStages, S, NW>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(64 * NW), smem, stream, a);
     MI355X_HIP(hipGetLastError());
     return 0;
 }
@@ -1569,7 +1587,9 @@ int LaunchPwDw(const mi355x_conv2d_s* pw, const mi355x_conv2d_s* dw, const PwDwS
     a.Ho = dw->geom.Ho; a.Wo = dw->geom.Wo; a.pad_top = dw->geom.pad_top; a.pad_left = dw->geom.pad_left;
     a.HR = sh.HR; a.HC = sh.HC; a.pairs = sh.pairs;
     a.y = static_cast<uint8_t*>(y);
-    return sh.S == 1 ? LaunchPwDwT<1>(a, stream) : LaunchPwDwT<2>(a, stream);
+    if (sh.MF == 2) return sh.S == 1 ? LaunchPwDwT<2, 1>(a, stream) : LaunchPwDwT<2, 2>(a, stream);
+    if (sh.MF == 4) return sh.S == 1 ? LaunchPwDwT<4, 1>(a, stream) : LaunchPwDwT<4, 2>(a, stream);
+    return sh.S == 1 ? LaunchPwDwT<kPwDwMF, 1>(a, stream) : LaunchPwDwT<kPwDwMF, 2>(a, stream);
 }
 
 // 0 when the pair (1x1 convolution, pooling over the whole image) can run as PwDwKernel<.., POOL>; G: images per block
@@ -1591,28 +1611,38 @@ int PwPoolCheck(const mi355x_conv2d_s* pw, const mi355x_pool2d_desc* pool, int* 
     if ((a.out_c % kPwDwBN) != 0) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel needs channels %% 64 == 0");
     const int hw = static_cast<int>(a.out_h) * static_cast<int>(a.out_w);
     if (hw > kGlobalPoolMaxTaps) return SetError(MI355X_ERR_UNSUPPORTED, "fused kernel holds whole images: %d pixels exceed %d", hw, kGlobalPoolMaxTaps);
-    if (G) *G = kPwDwMF * 32 / hw;
+    if (G) *G = kPwDwMF * 32 / hw;             // images per block of 7 fragments
+    return 0;
+}
+
+template <int MF>
+int LaunchPwPoolT(const mi355x_conv2d_s* pw, const mi355x_pool2d_desc* pool, uint32_t batch, const void* x, void* y, hipStream_t stream)
+{
+    const int hw = static_cast<int>(pw->d.out_h) * static_cast<int>(pw->d.out_w);
+    PwDwArgs a;
+    if (int rc = FillPwStage(pw, MF * 32 / hw, batch, x, &a)) return rc;
+    a.pool_in = MakeQIn(pool->input);
+    a.pool_rq = MakeRequant(pool->output, MI355X_ACT_NONE, 0.0f, 0.0f);
+    a.pool_is_max = pool->pool_type == 0;
+    a.y = static_cast<uint8_t*>(y);
+    constexpr int smem = PwDwStageBytes<MF, kPwDwStages>(), NW = PwDwWavesFor(MF);
+    static_assert(MF * 32 * kPwDwPitch <= smem, "the intermediate tile reuses the GEMM's stages");
+    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwDwKernel<MF, kPwDwStages, 1, NW, true>),
+                                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    MI355X_HIP(attr);
+    NoteKernel("PwDwKernel<%d, %d, 1, %d, true>", MF, kPwDwStages, NW);
+    hipLaunchKernelGGL((PwDwKernel<MF, kPwDwStages, 1, NW, true>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(64 * NW), smem, stream, a);
+    MI355X_HIP(hipGetLastError());
     return 0;
 }
 
 int LaunchPwPool(const mi355x_conv2d_s* pw, const mi355x_pool2d_desc* pool, int G, uint32_t batch, const void* x, void* y, hipStream_t stream)
 {
-    PwDwArgs a;
-    if (int rc = FillPwStage(pw, G, batch, x, &a)) return rc;
-    a.pool_in = MakeQIn(pool->input);
-    a.pool_rq = MakeRequant(pool->output, MI355X_ACT_NONE, 0.0f, 0.0f);
-    a.pool_is_max = pool->pool_type == 0;
-    a.y = static_cast<uint8_t*>(y);
-    constexpr int smem = PwDwStageBytes<kPwDwMF, kPwDwStages>();
-    static_assert(kPwDwMF * 32 * kPwDwPitch <= smem, "the intermediate tile reuses the GEMM's stages");
-    static const hipError_t attr = hipFuncSetAttribute(reinterpret_cast<const void*>(&PwDwKernel<kPwDwMF, kPwDwStages, 1, kPwDwWaves, true>),
-                                                       hipFuncAttributeMaxDynamicSharedMemorySize, smem);
-    MI355X_HIP(attr);
-    NoteKernel("PwDwKernel<%d, %d, 1, %d, true>", kPwDwMF, kPwDwStages, kPwDwWaves);
-    hipLaunchKernelGGL((PwDwKernel<kPwDwMF, kPwDwStages, 1, kPwDwWaves, true>), dim3(static_cast<unsigned>(a.xcd_chunk) * 8u), dim3(64 * kPwDwWaves),
-                       smem, stream, a);
-    MI355X_HIP(hipGetLastError());
-    return 0;
+    const int hw = static_cast<int>(pw->d.out_h) * static_cast<int>(pw->d.out_w);
+    const int mf = PwDwFragmentsFor(hw, true, (static_cast<long long>(batch) + G - 1) / G * (pw->d.out_c / kPwDwBN));
+    if (mf == 2) return LaunchPwPoolT<2>(pw, pool, batch, x, y, stream);
+    if (mf == 4) return LaunchPwPoolT<4>(pw, pool, batch, x, y, stream);
+    return LaunchPwPoolT<kPwDwMF>(pw, pool, batch, x, y, stream);
 }
 } // namespace
 

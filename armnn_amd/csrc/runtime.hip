@@ -151,6 +151,12 @@ int mi355x_set_option(const char* name, int value)
     }
     if (std::strcmp(name, "dwpw_stream") == 0) { GlobalOptions().dwpw_stream = value != 0; return 0; }
     if (std::strcmp(name, "pwdw_auto") == 0) { GlobalOptions().pwdw_auto = value != 0; return 0; }
+    if (std::strcmp(name, "pwdw_mf") == 0)
+    {
+        if (value != 0 && value != 2 && value != 4 && value != 7) return SetError(MI355X_ERR_INVALID_ARGUMENT, "pwdw_mf must be 0, 2, 4 or 7");
+        GlobalOptions().pwdw_mf = value;
+        return 0;
+    }
     if (std::strcmp(name, "pool_small") == 0) { GlobalOptions().pool_small = value != 0; return 0; }
     if (std::strcmp(name, "pwpool_auto") == 0) { GlobalOptions().pwpool_auto = value != 0; return 0; }
     if (std::strcmp(name, "dwpw_panel") == 0) { GlobalOptions().dwpw_panel = value != 0; return 0; }

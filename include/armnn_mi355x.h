@@ -125,6 +125,9 @@ int  mi355x_abi_version(void);
  *   pointwise weights in on-chip memory (identical bytes; lets tests compare it with the older fused kernel).
  *   "pwdw_auto" = 1 | 0: mi355x_conv2d_fusion_pays may (1) or may not (0) recommend a 1x1 convolution + the depthwise layer
  *   behind it (tests and tuning).
+ *   "pwdw_mf" = 0 | 2 | 4 | 7: rows per block, in units of 32 pixels, of the kernels that keep whole images of a 1x1
+ *   convolution's output on chip for the depthwise layer or the global pooling behind it (0: 7 with the depthwise layer, 4
+ *   with the pooling where two images fit; a value too small for one image is ignored; identical bytes; tests and tuning).
  *   "pool_small" = 1 | 0: a pooling over a whole image of at most 64 pixels runs on the kernel that gives a thread one
  *   channel and requests all its taps at once (1), or on the kernel that stages the image in on-chip memory (0).  Identical
  *   bytes.

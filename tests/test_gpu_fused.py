@@ -214,6 +214,17 @@ def test_pointwise_then_depthwise_fused_equals_two_layers(port, pair):
     pdw.run(n, mid.ptr, y2.ptr)
     ppw.run_fused(pdw, n, xd.ptr, yf.ptr)
     assert shim.last_kernel().startswith("PwDwKernel")
+    first = yf.download(dw.out_info.shape, numpy_dtype(dw.out_info.dtype))
+    _, h, w, _ = pw.x.info.shape
+    for mf in (2, 4):                                        # smaller blocks, where an image fits them, give the same bytes
+        shim.set_option("pwdw_mf", mf)
+        try:
+            ppw.run_fused(pdw, n, xd.ptr, yf.ptr)
+            kernel = shim.last_kernel()
+        finally:
+            shim.set_option("pwdw_mf", 0)
+        assert kernel.startswith(f"PwDwKernel<{mf}," if h * w <= mf * 32 else "PwDwKernel<7,"), kernel
+        np.testing.assert_array_equal(yf.download(dw.out_info.shape, numpy_dtype(dw.out_info.dtype)), first, err_msg=f"{mf} fragments per block")
     mid_h = mid.download(pw.out_info.shape, numpy_dtype(pw.out_info.dtype))
     two = y2.download(dw.out_info.shape, numpy_dtype(dw.out_info.dtype))
     fused = yf.download(dw.out_info.shape, numpy_dtype(dw.out_info.dtype))
@@ -301,6 +312,18 @@ def test_pointwise_then_global_pooling_fused_equals_two_layers(port, cfg):
     shim._chk(lib.mi355x_pool2d_run(C.byref(d), n, mid.ptr, y2.ptr, None))
     ppw.run_pooled(d, n, xd.ptr, yf.ptr)
     assert shim.last_kernel().startswith("PwDwKernel") and shim.last_kernel().endswith("true>")
+    first = yf.download((pooled.num_elements + 64,), np.uint8)
+    for mf in (2, 4, 7):                                     # every block size the kernel comes in gives the same bytes
+        shim.set_option("pwdw_mf", mf)
+        try:
+            shim._chk(lib.mi355x_fill_u8(yf.ptr, 0x5A, pooled.num_elements + 64, None))
+            ppw.run_pooled(d, n, xd.ptr, yf.ptr)
+            kernel = shim.last_kernel()
+        finally:
+            shim.set_option("pwdw_mf", 0)
+        if h * w <= mf * 32:
+            assert kernel.startswith(f"PwDwKernel<{mf},"), kernel
+        np.testing.assert_array_equal(yf.download((pooled.num_elements + 64,), np.uint8), first, err_msg=f"{mf} fragments per block")
     two = y2.download(pooled.shape, numpy_dtype(pooled.dtype))
     got = yf.download((pooled.num_elements + 64,), np.uint8)
     fused = got[:pooled.num_elements].view(numpy_dtype(pooled.dtype)).reshape(pooled.shape)
